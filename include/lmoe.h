@@ -1,0 +1,130 @@
+/*
+ * lmoe.h -- C ABI of liblmoe_hip.so: MI355X (gfx950) chunked linear-attention kernels.
+ *
+ * This is the drop-in boundary for the one hot path the reference
+ * (OpenSparseLLMs/Linear-MoE) delegates to flash-linear-attention ("fla"):
+ * the reference's token mixers bind python callables at import time and call them in
+ * forward(); a maintainer binds this library with ctypes instead.
+ * Every entry point below names the reference call site it serves.
+ *
+ * Conventions
+ *  - plain C types only; the caller owns all memory (device pointers unless stated);
+ *    the library never allocates or frees device memory and keeps no pointer after return;
+ *  - every function returns 0 on success, a negative value for an invalid argument
+ *    (nothing was launched) or a positive hipError_t; lmoe_last_error() gives the text
+ *    (thread-local);
+ *  - all work is enqueued asynchronously on the `stream` argument (a hipStream_t passed
+ *    as void*); no host synchronisation, no use of the default stream;
+ *  - results are deterministic (no atomics): re-execution by activation recompute gives
+ *    bit-identical outputs.
+ */
+#ifndef LMOE_H_
+#define LMOE_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LMOE_BF16 0
+#define LMOE_F32 1
+
+#define LMOE_GATE_NONE 0   /* no decay (basic linear attention)                  */
+#define LMOE_GATE_SCALAR 1 /* one log-decay per token and head   g: [B,T,H]      */
+#define LMOE_GATE_VECTOR 2 /* one log-decay per token, head, key channel [B,T,H,K] */
+
+#define LMOE_CHUNK 64
+
+/* A tensor addressed as x[b][t][h][d]: element offset b*sb + t*st + h*sh + d.
+ * Both fla layouts ([B,H,T,D] "head first" and [B,T,H,D]) and transposed views are
+ * described without a copy.  The last dimension is contiguous; ptr and all strides must
+ * keep 16-byte alignment for tensors with a last dimension (q,k,v,o,w,...). */
+typedef struct lmoe_tensor {
+  void* ptr;
+  int64_t sb, st, sh;
+} lmoe_tensor;
+
+/* One problem instance.  Fields an entry point does not use may be zero / NULL. */
+typedef struct lmoe_args {
+  int32_t dtype;      /* LMOE_BF16 | LMOE_F32: q,k,v,o,do,dq,dk,dv and the saved intermediates */
+  int32_t g_dtype;    /* element type of g    */
+  int32_t beta_dtype; /* element type of beta */
+  int32_t gate;       /* LMOE_GATE_*          */
+  int32_t B, T, H, K, V;
+  int32_t N;          /* number of sequences: B, or len(cu_seqlens)-1 when packed (then B == 1) */
+  int32_t NT;         /* total number of 64-token chunks over all sequences                    */
+  float scale;
+  /* packed variable-length input (all NULL for dense input) -- device int32 arrays */
+  const int32_t* cu_seqlens; /* [N+1] token offsets                                   */
+  const int32_t* chunk_map;  /* [NT][2] (sequence index, chunk index inside sequence) */
+  const int32_t* seq_chunk0; /* [N+1] index of the first chunk of each sequence       */
+  /* inputs */
+  lmoe_tensor q, k, v; /* [B,T,H,K], [B,T,H,K], [B,T,H,V]                              */
+  lmoe_tensor g;       /* [B,T,H] or [B,T,H,K]; log-space decay; ptr NULL = no decay   */
+  lmoe_tensor beta;    /* [B,T,H] (gated delta rule only)                              */
+  const float* h0;     /* [N,H,K,V] fp32 initial state or NULL                         */
+  /* outputs */
+  lmoe_tensor o;       /* [B,T,H,V]                                                    */
+  float* ht;           /* [N,H,K,V] fp32 final state or NULL                           */
+  /* intermediates written by *_fwd and read by *_bwd (caller-allocated, element type = dtype) */
+  void* hs;            /* [NT,H,K,V]  state at the start of every chunk                */
+  lmoe_tensor vnew;    /* [B,T,H,V]   delta-rule pseudo values (gated delta rule)      */
+  lmoe_tensor w;       /* [B,T,H,K]   WY factor w (gated delta rule)                   */
+  lmoe_tensor u;       /* [B,T,H,V]   WY factor u (gated delta rule; forward only)     */
+  void* tinv;          /* [NT,H,64,64] (I + L)^-1 per chunk (gated delta rule)         */
+  void* amat;          /* [NT,H,64,64] intra-chunk attention matrix (chunk_gla)        */
+  /* backward inputs */
+  lmoe_tensor d_o;     /* [B,T,H,V] gradient of o                                      */
+  const float* dht;    /* [N,H,K,V] fp32 gradient of the final state or NULL           */
+  /* backward outputs */
+  lmoe_tensor dq, dk, dv; /* same shapes as q,k,v, element type = dtype                */
+  lmoe_tensor dg;      /* fp32, shape of g                                             */
+  lmoe_tensor dbeta;   /* fp32, shape of beta                                          */
+  float* dh0;          /* [N,H,K,V] fp32 or NULL                                       */
+  /* backward workspace (caller-allocated, element type = dtype) */
+  void* dhs;           /* [NT,H,K,V] gradient w.r.t. the state at the END of every chunk */
+  lmoe_tensor dvnew;   /* [B,T,H,V]                                                    */
+} lmoe_args;
+
+/* Library version (major*10000 + minor*100 + patch). */
+int lmoe_version(void);
+/* Text of the last error on the calling thread ("" if none). */
+const char* lmoe_last_error(void);
+
+/* chunk_simple_gla: S_t = e^{g_t} S_{t-1} + k_t^T v_t, o_t = scale q_t S_t, g scalar per
+ * token-head (gate = SCALAR) or absent (gate = NONE).
+ * Replaces fla.ops.simple_gla.chunk_simple_gla reached from the reference through
+ *   linear_moe/sequence_modeling/retention/retention.py:91                (chunk_retention)
+ *   linear_moe/sequence_modeling/basic_linear_attention/basic_linear_attention.py:133 (chunk_linear_attn)
+ *   linear_moe/sequence_modeling/lightning_attention/lightning_attention.py:121-123 (lightning_attn2)
+ * fwd uses q,k,v,g,h0 -> o,ht,hs.  bwd uses q,k,v,g,hs,d_o,dht -> dq,dk,dv,dg,dh0 (+ dhs). */
+int lmoe_chunk_simple_gla_fwd(const lmoe_args* a, void* stream);
+int lmoe_chunk_simple_gla_bwd(const lmoe_args* a, void* stream);
+
+/* chunk_gla: S_t = diag(e^{g_t}) S_{t-1} + k_t^T v_t, g_t in R^K (gate = VECTOR).
+ * Replaces fla.ops.gla.chunk_gla called at
+ *   linear_moe/sequence_modeling/gla/gla.py:94 and linear_moe/sequence_modeling/hgrn2/hgrn2.py:76.
+ * fwd uses q,k,v,g,h0 -> o,ht,hs,amat.  bwd uses those + d_o,dht -> dq,dk,dv,dg,dh0 (+ dhs). */
+int lmoe_chunk_gla_fwd(const lmoe_args* a, void* stream);
+int lmoe_chunk_gla_bwd(const lmoe_args* a, void* stream);
+
+/* chunk_gated_delta_rule: S~_t = e^{g_t} S_{t-1}; S_t = S~_t + k_t^T beta_t (v_t - k_t S~_t);
+ * o_t = scale q_t S_t.
+ * Replaces fla.ops.gated_delta_rule.chunk_gated_delta_rule called at
+ *   linear_moe/sequence_modeling/gated_deltanet/gated_deltanet.py:112.
+ * fwd uses q,k,v,g,beta,h0 -> o,ht,hs,vnew,w,u,tinv.
+ * bwd uses q,k,v,g,beta,hs,vnew,w,tinv,d_o,dht -> dq,dk,dv,dg,dbeta,dh0 (+ dhs, dvnew). */
+int lmoe_chunk_gated_delta_rule_fwd(const lmoe_args* a, void* stream);
+int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream);
+
+/* Toolkit self-test: C[64][64] (fp32) = A[64][kd] * B[64][kd]^T through the same tile
+ * loaders, MFMA fragments and accumulator stores the kernels use; Ct gets the transpose
+ * via the transposed store path.  dtype selects the operand type; kd in {64, 128}.
+ * No counterpart in the reference (test support). */
+int lmoe_selftest_gemm(int32_t dtype, int32_t kd, const void* A, const void* B, float* C, float* Ct, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LMOE_H_ */

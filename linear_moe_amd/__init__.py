@@ -1,0 +1,10 @@
+"""MI355X-native chunked linear-attention ops behind flash-linear-attention's call signatures.
+
+Drop-in for the ``fla.ops`` callables the reference's token mixers import
+(``linear_moe/sequence_modeling/{gla,retention,gated_deltanet,basic_linear_attention}``).
+All compute runs in hand-written HIP kernels (``csrc/``) reached through the C ABI of
+``liblmoe_hip.so`` (``include/lmoe.h``); there is no fallback path.
+"""
+from .simple_gla import chunk_simple_gla  # noqa: F401
+
+__all__ = ["chunk_simple_gla"]

@@ -1,0 +1,130 @@
+"""Host-side plumbing shared by the chunk ops: argument validation, stride descriptors,
+the chunk table of packed (cu_seqlens) input and the ``lmoe_args`` block of the C ABI.
+
+Argument meaning follows flash-linear-attention's chunk ops as the reference calls them
+(``linear_moe/sequence_modeling/gla/gla.py:94``, ``.../retention/retention.py:91``,
+``.../gated_deltanet/gated_deltanet.py:112``): ``head_first=True`` means ``[B,H,T,D]``,
+otherwise ``[B,T,H,D]``; ``scale=None`` means ``K ** -0.5``; states are fp32 ``[N,H,K,V]``.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import Args, Tensor4, CHUNK
+
+_DT = {torch.bfloat16: _lib.LMOE_BF16, torch.float32: _lib.LMOE_F32}
+
+
+def _check_inputs(q, k, v, head_first: bool, cu_seqlens) -> Tuple[int, int, int, int, int]:
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise ValueError("q, k, v must be 4-dimensional")
+    if not (q.is_cuda and k.is_cuda and v.is_cuda):
+        raise RuntimeError("linear_moe_amd ops run on the GPU only (HIP kernels; there is no CPU path)")
+    if q.dtype not in _DT or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise ValueError(f"q, k, v must share dtype bfloat16 or float32, got {q.dtype}, {k.dtype}, {v.dtype}")
+    if q.shape != k.shape or q.shape[:3] != v.shape[:3]:
+        raise ValueError(f"shape mismatch: q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}")
+    if head_first:
+        B, H, T, K = q.shape
+    else:
+        B, T, H, K = q.shape
+    V = v.shape[-1]
+    if K not in (64, 128) or V not in (64, 128):
+        raise ValueError(f"head dims K={K}, V={V} unsupported: K and V must be 64 or 128")
+    if cu_seqlens is not None:
+        if head_first:
+            raise ValueError("cu_seqlens requires head_first=False ([1, T, H, D] packed input)")
+        if B != 1:
+            raise ValueError(f"cu_seqlens requires batch size 1 (packed input), got B={B}")
+    return B, T, H, K, V
+
+
+def _desc(x: Optional[torch.Tensor], head_first: bool) -> Tensor4:
+    """Stride descriptor of a [B,H,T,(D)] or [B,T,H,(D)] tensor."""
+    if x is None:
+        return Tensor4(None, 0, 0, 0)
+    if head_first:
+        sb, sh, st = x.stride(0), x.stride(1), x.stride(2)
+    else:
+        sb, st, sh = x.stride(0), x.stride(1), x.stride(2)
+    return Tensor4(x.data_ptr(), sb, st, sh)
+
+
+def _aligned(x: torch.Tensor) -> torch.Tensor:
+    """Return x (or a contiguous copy) such that rows are 16-byte aligned and last dim contiguous."""
+    if x.dim() == 4:
+        vec = 16 // x.element_size()
+        ok = x.stride(3) == 1 and x.data_ptr() % 16 == 0 and all(x.stride(i) % vec == 0 for i in range(3))
+        return x if ok else x.contiguous()
+    return x
+
+
+class SeqPlan:
+    """Chunk bookkeeping of one call: number of sequences / chunks and, for packed input,
+    the device tables the kernels index with."""
+
+    def __init__(self, B: int, T: int, cu_seqlens: Optional[torch.Tensor], device):
+        self.cu = None
+        self.chunk_map = None
+        self.seq_chunk0 = None
+        if cu_seqlens is None:
+            self.N = B
+            self.NT = B * ((T + CHUNK - 1) // CHUNK)
+            return
+        cu_host = cu_seqlens.detach().to("cpu", torch.int64)
+        if cu_host.dim() != 1 or cu_host.numel() < 2:
+            raise ValueError("cu_seqlens must be a 1-D tensor of N+1 offsets")
+        lens = cu_host[1:] - cu_host[:-1]
+        if int(cu_host[0]) != 0 or int(cu_host[-1]) != T or bool((lens < 0).any()):
+            raise ValueError("cu_seqlens must start at 0, be non-decreasing and end at T")
+        self.N = int(lens.numel())
+        nch = (lens + CHUNK - 1) // CHUNK
+        c0 = torch.zeros(self.N + 1, dtype=torch.int64)
+        c0[1:] = torch.cumsum(nch, 0)
+        self.NT = int(c0[-1])
+        seq_of = torch.repeat_interleave(torch.arange(self.N), nch)
+        local = torch.arange(self.NT) - c0[:-1][seq_of]
+        cmap = torch.stack([seq_of, local], 1).to(torch.int32).contiguous()
+        self.cu = cu_host.to(torch.int32).to(device)
+        self.chunk_map = cmap.to(device)
+        self.seq_chunk0 = c0.to(torch.int32).to(device)
+
+
+def _state_check(x: Optional[torch.Tensor], N, H, K, V, name: str) -> Optional[torch.Tensor]:
+    if x is None:
+        return None
+    if tuple(x.shape) != (N, H, K, V):
+        raise ValueError(f"{name} must have shape [N,H,K,V] = {(N, H, K, V)}, got {tuple(x.shape)}")
+    return x.detach().to(torch.float32).contiguous()
+
+
+def base_args(q, k, v, head_first: bool, scale: Optional[float], plan: SeqPlan, dims) -> Args:
+    B, T, H, K, V = dims
+    a = Args()
+    a.dtype = _DT[q.dtype]
+    a.B, a.T, a.H, a.K, a.V = B, T, H, K, V
+    a.N, a.NT = plan.N, plan.NT
+    a.scale = float(K ** -0.5 if scale is None else scale)
+    if plan.cu is not None:
+        a.cu_seqlens = plan.cu.data_ptr()
+        a.chunk_map = plan.chunk_map.data_ptr()
+        a.seq_chunk0 = plan.seq_chunk0.data_ptr()
+    a.q, a.k, a.v = _desc(q, head_first), _desc(k, head_first), _desc(v, head_first)
+    return a
+
+
+def token_major(B: int, T: int, H: int, D: int, dtype, device) -> torch.Tensor:
+    """Internal per-token buffer [B, T, H, D] (time-first, contiguous)."""
+    return torch.empty(B, T, H, D, dtype=dtype, device=device)
+
+
+def stream_ptr() -> C.c_void_p:
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def ptr(x: Optional[torch.Tensor]):
+    return None if x is None else x.data_ptr()

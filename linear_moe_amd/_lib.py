@@ -1,0 +1,82 @@
+"""ctypes binding of ``liblmoe_hip.so`` (C ABI declared in ``include/lmoe.h``).
+
+The library is the only compute path of this package: when it is missing every op raises
+``RuntimeError`` -- there is no eager or CPU fallback.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "liblmoe_hip.so")
+
+LMOE_BF16, LMOE_F32 = 0, 1
+GATE_NONE, GATE_SCALAR, GATE_VECTOR = 0, 1, 2
+CHUNK = 64
+
+
+class Tensor4(C.Structure):
+    """``lmoe_tensor``: x[b][t][h][d] at ptr + b*sb + t*st + h*sh + d (element strides)."""
+    _fields_ = [("ptr", C.c_void_p), ("sb", C.c_int64), ("st", C.c_int64), ("sh", C.c_int64)]
+
+
+class Args(C.Structure):
+    """``lmoe_args`` -- field order must match include/lmoe.h."""
+    _fields_ = [
+        ("dtype", C.c_int32), ("g_dtype", C.c_int32), ("beta_dtype", C.c_int32), ("gate", C.c_int32),
+        ("B", C.c_int32), ("T", C.c_int32), ("H", C.c_int32), ("K", C.c_int32), ("V", C.c_int32),
+        ("N", C.c_int32), ("NT", C.c_int32), ("scale", C.c_float),
+        ("cu_seqlens", C.c_void_p), ("chunk_map", C.c_void_p), ("seq_chunk0", C.c_void_p),
+        ("q", Tensor4), ("k", Tensor4), ("v", Tensor4), ("g", Tensor4), ("beta", Tensor4),
+        ("h0", C.c_void_p),
+        ("o", Tensor4), ("ht", C.c_void_p),
+        ("hs", C.c_void_p), ("vnew", Tensor4), ("w", Tensor4), ("u", Tensor4),
+        ("tinv", C.c_void_p), ("amat", C.c_void_p),
+        ("d_o", Tensor4), ("dht", C.c_void_p),
+        ("dq", Tensor4), ("dk", Tensor4), ("dv", Tensor4), ("dg", Tensor4), ("dbeta", Tensor4),
+        ("dh0", C.c_void_p),
+        ("dhs", C.c_void_p), ("dvnew", Tensor4),
+    ]
+
+
+ENTRY_POINTS = (
+    "lmoe_version", "lmoe_last_error",
+    "lmoe_chunk_simple_gla_fwd", "lmoe_chunk_simple_gla_bwd",
+    "lmoe_chunk_gla_fwd", "lmoe_chunk_gla_bwd",
+    "lmoe_chunk_gated_delta_rule_fwd", "lmoe_chunk_gated_delta_rule_bwd",
+    "lmoe_selftest_gemm",
+)
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    """Load the HIP library (once).  Raises RuntimeError when it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `make -C {os.path.join(_HERE, 'csrc')}` "
+            "(or __graft_entry__.build()).  This package has no fallback path.")
+    lib = C.CDLL(LIB_PATH)
+    lib.lmoe_version.restype = C.c_int
+    lib.lmoe_last_error.restype = C.c_char_p
+    for name in ENTRY_POINTS[2:8]:
+        fn = getattr(lib, name)
+        fn.argtypes = [C.POINTER(Args), C.c_void_p]
+        fn.restype = C.c_int
+    lib.lmoe_selftest_gemm.argtypes = [C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                       C.c_void_p]
+    lib.lmoe_selftest_gemm.restype = C.c_int
+    _lib = lib
+    return lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load().lmoe_last_error().decode()
+        if rc < 0:
+            raise ValueError(f"{what}: {msg} (code {rc})")
+        raise RuntimeError(f"{what}: {msg} (hipError {rc})")

@@ -1,0 +1,77 @@
+// C ABI of liblmoe_hip.so (declared in include/lmoe.h): argument validation and kernel dispatch.
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "../../include/lmoe.h"
+#include "lmoe_launch.hpp"
+
+namespace {
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_common(const lmoe_args* a, const char* op) {
+  if (!a) return fail(-1, "%s: null argument block", op);
+  if (a->dtype != LMOE_BF16 && a->dtype != LMOE_F32) return fail(-2, "%s: dtype must be LMOE_BF16 or LMOE_F32", op);
+  if (!((a->K == 64 || a->K == 128) && (a->V == 64 || a->V == 128)))
+    return fail(-3, "%s: head dims K=%d V=%d unsupported (K, V must be 64 or 128)", op, a->K, a->V);
+  if (a->B < 0 || a->T < 0 || a->H <= 0 || a->N < 0 || a->NT < 0) return fail(-4, "%s: negative dimension", op);
+  if (a->cu_seqlens && (a->B != 1 || !a->chunk_map || !a->seq_chunk0))
+    return fail(-5, "%s: packed input needs B == 1, chunk_map and seq_chunk0", op);
+  if (!a->cu_seqlens && a->N != a->B) return fail(-6, "%s: dense input needs N == B", op);
+  if (!a->q.ptr || !a->k.ptr || !a->v.ptr) return fail(-7, "%s: q, k, v must not be null", op);
+  if (a->H > 65535 || a->N > 65535) return fail(-8, "%s: H and N must be <= 65535", op);
+  return 0;
+}
+
+int launched(const char* op) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail((int)e, "%s: launch failed: %s", op, hipGetErrorString(e));
+  return 0;
+}
+}  // namespace
+
+extern "C" {
+
+int lmoe_version(void) { return 100; }
+const char* lmoe_last_error(void) { return g_err; }
+
+int lmoe_chunk_simple_gla_fwd(const lmoe_args* a, void* stream) {
+  const char* op = "lmoe_chunk_simple_gla_fwd";
+  if (int r = check_common(a, op)) return r;
+  if (a->gate == LMOE_GATE_VECTOR) return fail(-10, "%s: vector gates belong to lmoe_chunk_gla_fwd", op);
+  if (!a->o.ptr || !a->hs) return fail(-11, "%s: o and hs must not be null", op);
+  if (a->NT == 0 || a->N == 0) return 0;
+  lmoe::launch_scalar_fwd(*a, false, (hipStream_t)stream);
+  return launched(op);
+}
+
+int lmoe_chunk_simple_gla_bwd(const lmoe_args* a, void* stream) {
+  return fail(-100, "lmoe_chunk_simple_gla_bwd: not built yet");
+}
+int lmoe_chunk_gla_fwd(const lmoe_args* a, void* stream) { return fail(-100, "lmoe_chunk_gla_fwd: not built yet"); }
+int lmoe_chunk_gla_bwd(const lmoe_args* a, void* stream) { return fail(-100, "lmoe_chunk_gla_bwd: not built yet"); }
+int lmoe_chunk_gated_delta_rule_fwd(const lmoe_args* a, void* stream) {
+  return fail(-100, "lmoe_chunk_gated_delta_rule_fwd: not built yet");
+}
+int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream) {
+  return fail(-100, "lmoe_chunk_gated_delta_rule_bwd: not built yet");
+}
+
+int lmoe_selftest_gemm(int32_t dtype, int32_t kd, const void* A, const void* B, float* C, float* Ct, void* stream) {
+  if (!A || !B || !C || !Ct) return fail(-1, "lmoe_selftest_gemm: null pointer");
+  if ((dtype != LMOE_BF16 && dtype != LMOE_F32) || (kd != 64 && kd != 128))
+    return fail(-2, "lmoe_selftest_gemm: dtype/kd unsupported");
+  lmoe::launch_selftest(dtype, kd, A, B, C, Ct, (hipStream_t)stream);
+  return launched("lmoe_selftest_gemm");
+}
+
+}  // extern "C"

@@ -1,0 +1,233 @@
+// Device toolkit shared by all chunk kernels (gfx950 / CDNA4, wave64).
+//
+// Conventions used by every kernel in this directory:
+//  * a work-group is 256 threads = 4 wavefronts; a chunk is 64 tokens;
+//  * every LDS tile is stored "contraction-contiguous": element (r, c) at
+//    tile[r * ld + c] where c runs along the index the next MFMA contracts
+//    over.  A product X * Y^T with X:[M x Kd], Y:[N x Kd] therefore needs both
+//    operands as row-major tiles, and one helper (gemm_nt) serves every
+//    product; operands that are needed in both orientations are written to
+//    LDS twice (once transposed) while they are still in registers;
+//  * MFMA shape: v_mfma_f32_16x16x32_bf16 for bf16 operands and
+//    8 x v_mfma_f32_16x16x4_f32 for fp32 operands, behind the same fragment
+//    layout (lane l holds row l%16, contraction elements 8*(l/16) .. +7);
+//  * accumulator layout of one 16x16 block: lane l holds rows 4*(l/16)+i
+//    (i = 0..3) of column l%16.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace lmoe {
+
+typedef __bf16 bf16;
+typedef bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int CH = 64;        // chunk length (tokens)
+constexpr int NTHR = 256;     // threads per work-group
+constexpr int LPAD = 8;       // LDS row padding in elements (16 B for bf16, 32 B for fp32)
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
+__device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
+
+// ------------------------------------------------------------------------- //
+// element traits
+// ------------------------------------------------------------------------- //
+template <typename T> struct ET;
+
+template <> struct ET<bf16> {
+  static constexpr int VEC = 8;                       // elements per 16-byte vector
+  typedef bf16x8 vec;
+  typedef bf16x8 frag;
+  static __device__ __forceinline__ vec zero() { vec z; for (int i = 0; i < 8; ++i) z[i] = (bf16)0.0f; return z; }
+  static __device__ __forceinline__ float to_f(bf16 x) { return (float)x; }
+  static __device__ __forceinline__ bf16 from_f(float x) { return (bf16)x; }
+  static __device__ __forceinline__ frag load_frag(const bf16* p) { return *(const bf16x8*)p; }
+  static __device__ __forceinline__ void mma(f32x4& c, const frag& a, const frag& b) {
+    c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+
+struct f32frag { f32x4 lo, hi; };
+
+template <> struct ET<float> {
+  static constexpr int VEC = 4;
+  typedef f32x4 vec;
+  typedef f32frag frag;
+  static __device__ __forceinline__ vec zero() { vec z = {0.f, 0.f, 0.f, 0.f}; return z; }
+  static __device__ __forceinline__ float to_f(float x) { return x; }
+  static __device__ __forceinline__ float from_f(float x) { return x; }
+  static __device__ __forceinline__ frag load_frag(const float* p) {
+    frag f; f.lo = *(const f32x4*)p; f.hi = *(const f32x4*)(p + 4); return f;
+  }
+  static __device__ __forceinline__ void mma(f32x4& c, const frag& a, const frag& b) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) c = __builtin_amdgcn_mfma_f32_16x16x4f32(a.lo[i], b.lo[i], c, 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) c = __builtin_amdgcn_mfma_f32_16x16x4f32(a.hi[i], b.hi[i], c, 0, 0, 0);
+  }
+};
+
+// ------------------------------------------------------------------------- //
+// gemm_nt: acc[mi][ni] += A[arow0 + 16 mi + r][k] * B[brow0 + 16 ni + c][k], k in [k0, k1)
+// (k0, k1 multiples of 32).  A, B: LDS tiles with leading dimensions lda, ldb.
+// ------------------------------------------------------------------------- //
+template <typename T, int MB, int NB>
+__device__ __forceinline__ void gemm_nt(f32x4 (&acc)[MB][NB], const T* A, int lda, int arow0,
+                                        const T* B, int ldb, int brow0, int k0, int k1) {
+  const int l = lane_id();
+  const int r = l & 15, kg = (l >> 4) * 8;
+  for (int kk = k0; kk < k1; kk += 32) {
+    typename ET<T>::frag a[MB], b[NB];
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi) a[mi] = ET<T>::load_frag(A + (arow0 + 16 * mi + r) * lda + kk + kg);
+#pragma unroll
+    for (int ni = 0; ni < NB; ++ni) b[ni] = ET<T>::load_frag(B + (brow0 + 16 * ni + r) * ldb + kk + kg);
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) ET<T>::mma(acc[mi][ni], a[mi], b[ni]);
+  }
+}
+
+template <int MB, int NB>
+__device__ __forceinline__ void acc_zero(f32x4 (&acc)[MB][NB]) {
+#pragma unroll
+  for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < NB; ++ni) acc[mi][ni] = f32x4{0.f, 0.f, 0.f, 0.f};
+}
+
+// row / column of accumulator element i of block (mi, ni)
+__device__ __forceinline__ int acc_row(int mi, int i) { return 16 * mi + 4 * (lane_id() >> 4) + i; }
+__device__ __forceinline__ int acc_col(int ni) { return 16 * ni + (lane_id() & 15); }
+
+// store one 16x16 accumulator block to an LDS tile as tile[row][col] (row = M index)
+template <typename T>
+__device__ __forceinline__ void acc_to_lds(const f32x4& a, T* tile, int ld, int row0, int col0) {
+  const int l = lane_id();
+  const int r = row0 + 4 * (l >> 4), c = col0 + (l & 15);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) tile[(r + i) * ld + c] = ET<T>::from_f(a[i]);
+}
+// store transposed: tile[col][row] -- the lane's 4 values are contiguous
+template <typename T>
+__device__ __forceinline__ void acc_to_lds_t(const f32x4& a, T* tile, int ld, int row0, int col0) {
+  const int l = lane_id();
+  const int r = row0 + 4 * (l >> 4), c = col0 + (l & 15);
+  T* p = tile + c * ld + r;
+  if constexpr (sizeof(T) == 2) {
+    bf16x4 v; v[0] = (bf16)a[0]; v[1] = (bf16)a[1]; v[2] = (bf16)a[2]; v[3] = (bf16)a[3];
+    *(bf16x4*)p = v;
+  } else {
+    *(f32x4*)p = a;
+  }
+}
+
+// ------------------------------------------------------------------------- //
+// cooperative global <-> LDS tile movement (all 256 threads)
+//   a tile is ROWS x COLS elements, source rows `row_stride` elements apart;
+//   rows >= nvalid read as zero / are not written.
+// ------------------------------------------------------------------------- //
+template <typename T, int ROWS, int COLS> struct TileIO {
+  static constexpr int VEC = ET<T>::VEC;
+  static constexpr int VPR = COLS / VEC;                 // vectors per row
+  static constexpr int NVEC = ROWS * VPR;                // vectors in the tile
+  static constexpr int PASSES = (NVEC + NTHR - 1) / NTHR;
+  typedef typename ET<T>::vec vec;
+  struct Regs { vec v[PASSES]; };
+
+  static __device__ __forceinline__ void coords(int p, int& row, int& col) {
+    const int idx = p * NTHR + threadIdx.x;
+    row = idx / VPR; col = (idx % VPR) * VEC;
+  }
+  static __device__ __forceinline__ void load(Regs& r, const T* __restrict__ src, int64_t row_stride, int nvalid) {
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      int row, col; coords(p, row, col);
+      if (row < ROWS && row < nvalid) r.v[p] = *(const vec*)(src + (int64_t)row * row_stride + col);
+      else r.v[p] = ET<T>::zero();
+    }
+  }
+  // tile[row][col] = x
+  static __device__ __forceinline__ void store_lds(const Regs& r, T* tile, int ld) {
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      int row, col; coords(p, row, col);
+      if (row < ROWS) *(vec*)(tile + row * ld + col) = r.v[p];
+    }
+  }
+  // tile[row][col] = x * rs[row]
+  static __device__ __forceinline__ void store_lds_scaled(const Regs& r, T* tile, int ld, const float* rs) {
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      int row, col; coords(p, row, col);
+      if (row < ROWS) {
+        const float s = rs[row];
+        vec o;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) o[i] = ET<T>::from_f(ET<T>::to_f(r.v[p][i]) * s);
+        *(vec*)(tile + row * ld + col) = o;
+      }
+    }
+  }
+  // tileT[col][row] = x * (rs ? rs[row] : 1)
+  static __device__ __forceinline__ void store_lds_t(const Regs& r, T* tileT, int ldT, const float* rs) {
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      int row, col; coords(p, row, col);
+      if (row < ROWS) {
+        const float s = rs ? rs[row] : 1.0f;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) tileT[(col + i) * ldT + row] = ET<T>::from_f(ET<T>::to_f(r.v[p][i]) * s);
+      }
+    }
+  }
+  // global[row][col] = tile[row][col]
+  static __device__ __forceinline__ void lds_to_global(const T* tile, int ld, T* __restrict__ dst, int64_t row_stride, int nvalid) {
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      int row, col; coords(p, row, col);
+      if (row < ROWS && row < nvalid) *(vec*)(dst + (int64_t)row * row_stride + col) = *(const vec*)(tile + row * ld + col);
+    }
+  }
+};
+
+// ------------------------------------------------------------------------- //
+// gates
+// ------------------------------------------------------------------------- //
+// scalar gate / beta value for one token; dtype: 0 = bf16, 1 = fp32; null pointer = 0
+__device__ __forceinline__ float load_scalar(const void* p, int dtype, int64_t idx) {
+  if (p == nullptr) return 0.f;
+  return dtype == 1 ? ((const float*)p)[idx] : (float)((const bf16*)p)[idx];
+}
+
+// inclusive prefix sum across the 64 lanes of a wavefront
+__device__ __forceinline__ float wave_incl_scan(float x) {
+  const int l = lane_id();
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    float y = __shfl_up(x, d, 64);
+    if (l >= d) x += y;
+  }
+  return x;
+}
+// inclusive suffix sum (reverse cumulative sum) across the 64 lanes
+__device__ __forceinline__ float wave_rev_scan(float x) {
+  const int l = lane_id();
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    float y = __shfl_down(x, d, 64);
+    if (l + d < 64) x += y;
+  }
+  return x;
+}
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) x += __shfl_xor(x, d, 64);
+  return x;
+}
+
+}  // namespace lmoe

@@ -1,0 +1,199 @@
+// Forward kernels for scalar-gated chunks (chunk_simple_gla and chunk_gated_delta_rule):
+//   k_state_fwd : sequential pass over the chunks of one (sequence, head, V-slice); keeps the
+//                 state S[K x BV] in fp32 MFMA accumulators, writes the state at the start of
+//                 every chunk (hs) and, for the delta rule, v_new = u - w S.
+//   k_out_fwd   : chunk-parallel output  o = scale [ e^{b_i} q_i S + ((q k^T) . Gamma) v' ].
+// Math: S' = e^{b_C} S + (k . e^{b_C - b})^T v',  Gamma_ij = e^{b_i - b_j} [i >= j].
+#pragma once
+#include "lmoe_seq.hpp"
+
+namespace lmoe {
+
+// ------------------------------------------------------------------------- //
+// state pass (forward)
+//   grid = (V / BV, H, N), block = 256
+//   wave w owns state rows [w*K/4, (w+1)*K/4) x BV columns
+// ------------------------------------------------------------------------- //
+template <typename T, int K, int V, int BV, bool GDN>
+__global__ __launch_bounds__(NTHR) void k_state_fwd(const lmoe_args a) {
+  constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDU = BV + LPAD;
+  constexpr int MB = K / 64, NB = BV / 16;
+  __shared__ __attribute__((aligned(16))) T s_kT[K * LDC];            // (k e^{b_C-b})^T  [K][64]
+  __shared__ __attribute__((aligned(16))) T s_vT[BV * LDC];           // v'^T             [BV][64]
+  __shared__ __attribute__((aligned(16))) T s_w[GDN ? CH * LDK : 8];  // w                [64][K]
+  __shared__ __attribute__((aligned(16))) T s_hT[GDN ? BV * LDK : 8]; // S^T              [BV][K]
+  __shared__ __attribute__((aligned(16))) T s_u[GDN ? CH * LDU : 8];  // u                [64][BV]
+  __shared__ float s_b[64], s_ed[64];
+
+  const int v0 = blockIdx.x * BV, h = blockIdx.y, n = blockIdx.z;
+  const SeqInfo sq = seq_info(a, n);
+  const int wv = wave_id(), l = lane_id();
+  const int krow0 = wv * (K / 4);
+
+  f32x4 S[MB][NB];
+  acc_zero(S);
+  if (a.h0) {
+    const float* h0 = a.h0 + ((int64_t)n * a.H + h) * K * V;
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          S[mi][ni][i] = h0[(int64_t)(krow0 + acc_row(mi, i)) * V + v0 + acc_col(ni)];
+  }
+
+  typedef TileIO<T, CH, K> IOK;
+  typedef TileIO<T, CH, BV> IOV;
+
+  for (int c = 0; c < sq.nchunks; ++c) {
+    const int tok = sq.tok0 + c * CH;
+    const int len = min(CH, sq.len - c * CH);
+    chunk_gate_cumsum(a, sq.b, tok, len, h, s_b, nullptr, s_ed);
+
+    typename IOK::Regs rk;
+    IOK::load(rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, len);
+    IOK::store_lds_t(rk, s_kT, LDC, s_ed);
+    if constexpr (GDN) {
+      typename IOK::Regs rw;
+      IOK::load(rw, row_ptr<T>(a.w, sq.b, tok, h), a.w.st, len);
+      IOK::store_lds(rw, s_w, LDK);
+      typename IOV::Regs ru;
+      IOV::load(ru, row_ptr<T>(a.u, sq.b, tok, h) + v0, a.u.st, len);
+      IOV::store_lds(ru, s_u, LDU);
+    } else {
+      typename IOV::Regs rv;
+      IOV::load(rv, row_ptr<T>(a.v, sq.b, tok, h) + v0, a.v.st, len);
+      IOV::store_lds_t(rv, s_vT, LDC, nullptr);
+    }
+    // state at chunk start -> hs (and LDS copy for the delta rule)
+    {
+      T* hs = (T*)a.hs + ((int64_t)(sq.chunk0 + c) * a.H + h) * K * V;
+#pragma unroll
+      for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            hs[(int64_t)(krow0 + acc_row(mi, i)) * V + v0 + acc_col(ni)] = ET<T>::from_f(S[mi][ni][i]);
+          if constexpr (GDN) acc_to_lds_t<T>(S[mi][ni], s_hT, LDK, krow0 + 16 * mi, 16 * ni);
+        }
+    }
+    __syncthreads();
+    if constexpr (GDN) {
+      // v_new = u - w S  (rows 16*wv .. +15 of the chunk)
+      f32x4 vn[1][NB];
+      acc_zero(vn);
+      gemm_nt<T, 1, NB>(vn, s_w, LDK, 16 * wv, s_hT, LDK, 0, 0, K);
+      T* vdst = row_ptr<T>(a.vnew, sq.b, tok, h) + v0;
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) {
+        f32x4 x;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
+          x[i] = ET<T>::to_f(s_u[r * LDU + cc]) - vn[0][ni][i];
+          // round once to the storage type so that the state update and the output kernel
+          // see the same v_new
+          x[i] = ET<T>::to_f(ET<T>::from_f(x[i]));
+          if (r < len) vdst[(int64_t)r * a.vnew.st + cc] = ET<T>::from_f(x[i]);
+        }
+        acc_to_lds_t<T>(x, s_vT, LDC, 16 * wv, 16 * ni);
+      }
+      __syncthreads();
+    }
+    // S = e^{b_C} S + k_d^T v'
+    const float dec = expf(s_b[63]);
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) S[mi][ni] *= dec;
+    gemm_nt<T, MB, NB>(S, s_kT, LDC, krow0, s_vT, LDC, 0, 0, CH);
+    __syncthreads();
+  }
+
+  if (a.ht) {
+    float* ht = a.ht + ((int64_t)n * a.H + h) * K * V;
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          ht[(int64_t)(krow0 + acc_row(mi, i)) * V + v0 + acc_col(ni)] = S[mi][ni][i];
+  }
+}
+
+// ------------------------------------------------------------------------- //
+// output (forward), chunk-parallel
+//   grid = (NT, H, V / BV), block = 256; wave w owns chunk rows 16w .. 16w+15
+// ------------------------------------------------------------------------- //
+template <typename T, int K, int V, int BV, bool GDN>
+__global__ __launch_bounds__(NTHR) void k_out_fwd(const lmoe_args a) {
+  constexpr int LDK = K + LPAD, LDC = CH + LPAD;
+  constexpr int NB = BV / 16;
+  __shared__ __attribute__((aligned(16))) T s_q[CH * LDK];
+  __shared__ __attribute__((aligned(16))) T s_k[CH * LDK];
+  __shared__ __attribute__((aligned(16))) T s_vT[BV * LDC];
+  __shared__ __attribute__((aligned(16))) T s_hT[BV * LDK];
+  __shared__ __attribute__((aligned(16))) T s_P[CH * LDC];
+  __shared__ float s_b[64], s_eb[64];
+
+  const int cid = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * BV;
+  const ChunkInfo ci = chunk_info(a, cid);
+  const int wv = wave_id(), l = lane_id();
+  chunk_gate_cumsum(a, ci.b, ci.tok, ci.len, h, s_b, s_eb, nullptr);
+
+  typedef TileIO<T, CH, K> IOK;
+  typedef TileIO<T, CH, BV> IOV;
+  typedef TileIO<T, K, BV> IOH;
+  {
+    typename IOK::Regs rq, rk;
+    IOK::load(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
+    IOK::load(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
+    const lmoe_tensor& vs = GDN ? a.vnew : a.v;
+    typename IOV::Regs rv;
+    IOV::load(rv, row_ptr<T>(vs, ci.b, ci.tok, h) + v0, vs.st, ci.len);
+    typename IOH::Regs rh;
+    IOH::load(rh, (const T*)a.hs + ((int64_t)cid * a.H + h) * K * V + v0, V, K);
+    IOK::store_lds(rq, s_q, LDK);
+    IOK::store_lds(rk, s_k, LDK);
+    IOV::store_lds_t(rv, s_vT, LDC, nullptr);
+    IOH::store_lds_t(rh, s_hT, LDK, nullptr);
+  }
+  __syncthreads();
+  {
+    f32x4 s[1][4];
+    acc_zero(s);
+    gemm_nt<T, 1, 4>(s, s_q, LDK, 16 * wv, s_k, LDK, 0, 0, K);
+#pragma unroll
+    for (int nj = 0; nj < 4; ++nj) {
+      f32x4 p;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * nj + (l & 15);
+        p[i] = (r >= cc) ? s[0][nj][i] * expf(s_b[r] - s_b[cc]) : 0.f;
+      }
+      acc_to_lds<T>(p, s_P, LDC, 16 * wv, 16 * nj);
+    }
+  }
+  __syncthreads();
+  f32x4 o[1][NB];
+  acc_zero(o);
+  gemm_nt<T, 1, NB>(o, s_q, LDK, 16 * wv, s_hT, LDK, 0, 0, K);
+#pragma unroll
+  for (int ni = 0; ni < NB; ++ni)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[0][ni][i] *= s_eb[16 * wv + 4 * (l >> 4) + i];
+  gemm_nt<T, 1, NB>(o, s_P, LDC, 16 * wv, s_vT, LDC, 0, 0, CH);
+  T* od = row_ptr<T>(a.o, ci.b, ci.tok, h) + v0;
+#pragma unroll
+  for (int ni = 0; ni < NB; ++ni)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
+      if (r < ci.len) od[(int64_t)r * a.o.st + cc] = ET<T>::from_f(o[0][ni][i] * a.scale);
+    }
+}
+
+}  // namespace lmoe

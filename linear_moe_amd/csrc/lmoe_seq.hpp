@@ -1,0 +1,90 @@
+// Sequence / chunk addressing shared by all kernels: maps a sequence index or a global
+// chunk index to token ranges, for dense [B,T,...] input and for packed variable-length
+// input (cu_seqlens).  Chunks never straddle a sequence boundary; the last chunk of a
+// sequence may be partial.
+#pragma once
+#include "../../include/lmoe.h"
+#include "lmoe_common.hpp"
+
+namespace lmoe {
+
+struct SeqInfo {
+  int b;        // batch row holding the sequence
+  int tok0;     // first token of the sequence inside that batch row
+  int len;      // number of tokens
+  int chunk0;   // global index of the sequence's first chunk
+  int nchunks;  // ceil(len / 64)
+};
+
+__device__ __forceinline__ SeqInfo seq_info(const lmoe_args& a, int n) {
+  SeqInfo s;
+  if (a.cu_seqlens) {
+    s.b = 0; s.tok0 = a.cu_seqlens[n]; s.len = a.cu_seqlens[n + 1] - s.tok0;
+    s.chunk0 = a.seq_chunk0[n];
+  } else {
+    s.b = n; s.tok0 = 0; s.len = a.T;
+    s.chunk0 = n * ((a.T + CH - 1) / CH);
+  }
+  s.nchunks = (s.len + CH - 1) / CH;
+  return s;
+}
+
+struct ChunkInfo {
+  int n;       // sequence
+  int b;       // batch row
+  int tok;     // first token of the chunk inside the batch row
+  int len;     // valid tokens in this chunk (1..64)
+  int last;    // 1 if this is the last chunk of its sequence
+};
+
+__device__ __forceinline__ ChunkInfo chunk_info(const lmoe_args& a, int cid) {
+  ChunkInfo c;
+  int lc, slen;
+  if (a.cu_seqlens) {
+    c.n = a.chunk_map[2 * cid]; lc = a.chunk_map[2 * cid + 1];
+    c.b = 0;
+    const int t0 = a.cu_seqlens[c.n];
+    slen = a.cu_seqlens[c.n + 1] - t0;
+    c.tok = t0 + lc * CH;
+  } else {
+    const int nts = (a.T + CH - 1) / CH;
+    c.n = cid / nts; lc = cid % nts;
+    c.b = c.n; slen = a.T;
+    c.tok = lc * CH;
+  }
+  const int rem = slen - lc * CH;
+  c.len = rem < CH ? rem : CH;
+  c.last = rem <= CH;
+  return c;
+}
+
+// pointer to row (b, tok, h) of a strided tensor with element type T
+template <typename T>
+__device__ __forceinline__ T* row_ptr(const lmoe_tensor& x, int b, int tok, int h) {
+  return (T*)x.ptr + (int64_t)b * x.sb + (int64_t)tok * x.st + (int64_t)h * x.sh;
+}
+__device__ __forceinline__ int64_t row_off(const lmoe_tensor& x, int b, int tok, int h) {
+  return (int64_t)b * x.sb + (int64_t)tok * x.st + (int64_t)h * x.sh;
+}
+
+// Load the chunk's 64 scalar log-decays, form the inclusive cumulative sum b_j in fp32 and
+// leave in LDS: sb[j] = b_j, seb[j] = e^{b_j}, sed[j] = e^{b_63 - b_j} (seb / sed may be null).
+// Tokens past the end of the chunk contribute 0.  All exponents are <= 0 for g <= 0.
+// Must be called by all threads of the work-group; ends with a barrier.
+__device__ __forceinline__ void chunk_gate_cumsum(const lmoe_args& a, int b, int tok, int len, int h,
+                                                  float* sb, float* seb, float* sed) {
+  if (threadIdx.x < 64) {
+    const int j = threadIdx.x;
+    float g = 0.f;
+    if (a.gate != LMOE_GATE_NONE && a.g.ptr != nullptr && j < len)
+      g = load_scalar(a.g.ptr, a.g_dtype, row_off(a.g, b, tok + j, h));
+    const float x = wave_incl_scan(g);
+    const float xl = __shfl(x, 63, 64);
+    sb[j] = x;
+    if (seb) seb[j] = expf(x);
+    if (sed) sed[j] = expf(xl - x);
+  }
+  __syncthreads();
+}
+
+}  // namespace lmoe

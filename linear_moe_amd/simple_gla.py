@@ -1,0 +1,99 @@
+"""``chunk_simple_gla`` on MI355X: S_t = e^{g_t} S_{t-1} + k_t^T v_t, o_t = scale q_t S_t.
+
+Keeps flash-linear-attention's call signature; it is the op behind the reference's
+``chunk_retention`` (``linear_moe/sequence_modeling/retention/retention.py:91``),
+``chunk_linear_attn`` (``.../basic_linear_attention/basic_linear_attention.py:133``) and
+``lightning_attn2`` (``.../lightning_attention/lightning_attention.py:121-123``).
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._host import (SeqPlan, _aligned, _check_inputs, _desc, _state_check, base_args, ptr, stream_ptr)
+
+
+class _ChunkSimpleGLA(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first):
+        lib = _lib.load()
+        dims = _check_inputs(q, k, v, head_first, cu_seqlens)
+        B, T, H, K, V = dims
+        q, k, v = _aligned(q), _aligned(k), _aligned(v)
+        plan = SeqPlan(B, T, cu_seqlens, q.device)
+        if g is not None:
+            want = (B, H, T) if head_first else (B, T, H)
+            if tuple(g.shape) != want:
+                raise ValueError(f"g must have shape {want}, got {tuple(g.shape)}")
+            if g.dtype not in (torch.float32, torch.bfloat16):
+                g = g.float()
+        h0 = _state_check(initial_state, plan.N, H, K, V, "initial_state")
+        a = base_args(q, k, v, head_first, scale, plan, dims)
+        a.gate = _lib.GATE_NONE if g is None else _lib.GATE_SCALAR
+        if g is not None:
+            a.g = _desc(g, head_first)
+            a.g_dtype = _lib.LMOE_F32 if g.dtype == torch.float32 else _lib.LMOE_BF16
+        a.h0 = ptr(h0)
+        o = torch.empty_like(v)
+        ht = torch.empty(plan.N, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
+        hs = torch.empty(max(plan.NT, 1), H, K, V, dtype=q.dtype, device=q.device)
+        a.o = _desc(o, head_first)
+        a.ht = ptr(ht)
+        a.hs = hs.data_ptr()
+        _lib.check(lib.lmoe_chunk_simple_gla_fwd(C.byref(a), stream_ptr()), "chunk_simple_gla forward")
+        ctx.save_for_backward(q, k, v, g, h0, hs)
+        ctx.plan, ctx.dims, ctx.head_first, ctx.scale = plan, dims, head_first, scale
+        ctx.has_h0 = initial_state is not None
+        return o, ht
+
+    @staticmethod
+    def backward(ctx, do, dht):
+        lib = _lib.load()
+        q, k, v, g, h0, hs = ctx.saved_tensors
+        plan, dims, head_first = ctx.plan, ctx.dims, ctx.head_first
+        B, T, H, K, V = dims
+        do = _aligned(do)
+        a = base_args(q, k, v, head_first, ctx.scale, plan, dims)
+        a.gate = _lib.GATE_NONE if g is None else _lib.GATE_SCALAR
+        if g is not None:
+            a.g = _desc(g, head_first)
+            a.g_dtype = _lib.LMOE_F32 if g.dtype == torch.float32 else _lib.LMOE_BF16
+        a.h0 = ptr(h0)
+        a.hs = hs.data_ptr()
+        a.d_o = _desc(do, head_first)
+        dht = None if dht is None else dht.float().contiguous()
+        a.dht = ptr(dht)
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        a.dq, a.dk, a.dv = _desc(dq, head_first), _desc(dk, head_first), _desc(dv, head_first)
+        dg = None
+        if g is not None:
+            dg = torch.empty(g.shape, dtype=torch.float32, device=q.device)
+            a.dg = _desc(dg, head_first)
+        dh0 = torch.empty_like(h0) if ctx.has_h0 else None
+        a.dh0 = ptr(dh0)
+        dhs = torch.empty_like(hs)
+        a.dhs = dhs.data_ptr()
+        _lib.check(lib.lmoe_chunk_simple_gla_bwd(C.byref(a), stream_ptr()), "chunk_simple_gla backward")
+        if dg is not None and dg.dtype != g.dtype:
+            dg = dg.to(g.dtype)
+        return dq, dk, dv, dg, None, dh0, None, None, None
+
+
+def chunk_simple_gla(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    g: Optional[torch.Tensor] = None,
+    scale: Optional[float] = None,
+    initial_state: Optional[torch.Tensor] = None,
+    output_final_state: bool = False,
+    cu_seqlens: Optional[torch.Tensor] = None,
+    head_first: bool = True,
+) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """q, k: ``[B,H,T,K]``, v: ``[B,H,T,V]`` (``[B,T,H,*]`` with ``head_first=False``);
+    g: ``[B,H,T]`` log-space decay or None.  Returns ``(o, final_state)`` with ``o`` shaped like
+    ``v`` and ``final_state`` fp32 ``[N,H,K,V]`` or None."""
+    return _ChunkSimpleGLA.apply(q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first)

@@ -1,0 +1,243 @@
+"""CPU oracle: token-by-token recurrences for the chunked linear-attention path.
+
+TEST INFRASTRUCTURE ONLY.  Nothing in the shipped package imports this file; it
+is the checker used by ``tests/``, by ``__graft_entry__.smoke()`` and by the
+``cpu_baseline`` leg of ``bench.py``.
+
+The reference (OpenSparseLLMs/Linear-MoE) does not hold this arithmetic itself:
+its token mixers call the third-party package flash-linear-attention ("fla",
+pinned snapshot 2025-03-03 by ``examples/linear_moe_qwen2/run_pretrain_qwen.sh:8``;
+the submodule directory is empty in the checkout).  The functions below restate
+fla's published ``naive_recurrent_*`` recurrences, anchored on the reference's
+call sites:
+
+* ``linear_moe/sequence_modeling/gated_deltanet/gated_deltanet.py:112``
+  ``chunk_gated_delta_rule(q, k, v, g, beta, head_first=False)``
+* ``linear_moe/sequence_modeling/gla/gla.py:94``  ``chunk_gla(q, k, v, gk)``
+* ``linear_moe/sequence_modeling/retention/retention.py:91`` ``chunk_retention(q, k, v)``
+* ``linear_moe/sequence_modeling/basic_linear_attention/basic_linear_attention.py:133``
+  ``chunk_linear_attn(q, k, v, normalize=...)``
+* ``linear_moe/sequence_modeling/lightning_attention/lightning_attention.py:121-123``
+  ``lightning_attn2(q, k, v, slope)``
+
+Parity status: the reference ships no test, golden vector or fixture for this
+path, so these recurrences are pinned by mathematics instead (closed forms,
+special cases that reduce to ``tril(QK^T)V``, hand-unrolled tiny cases, linearity
+and state hand-off invariants, finite-difference gradients, and the independent
+``transformers`` torch routine for the gated delta rule) in
+``tests/test_oracle_pins.py``.  What only an import of fla could pin -- its
+exact low-precision rounding points and the epsilon of ``normalize=True`` --
+is "parity unpinned" and documented as such in the tests.
+
+All functions are differentiable through ``torch.autograd`` and compute in the
+dtype given by ``dtype`` (float64 by default).
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+
+Tensor = torch.Tensor
+
+
+def _to_head_first(x: Tensor, head_first: bool) -> Tensor:
+    # [B,T,H,...] -> [B,H,T,...]
+    return x if head_first else x.transpose(1, 2)
+
+
+def _seq_ranges(cu_seqlens, B: int, T: int):
+    if cu_seqlens is None:
+        return None
+    cu = [int(c) for c in cu_seqlens]
+    return list(zip(cu[:-1], cu[1:]))
+
+
+def _run_varlen(core, tensors, initial_state, output_final_state, cu_seqlens):
+    """Apply ``core`` (head-first dense op on [1,H,T,..]) to every packed sequence."""
+    outs, finals = [], []
+    for n, (s, e) in enumerate(_seq_ranges(cu_seqlens, 1, 0)):
+        sl = [None if t is None else t[:, :, s:e] for t in tensors]
+        h0 = None if initial_state is None else initial_state[n:n + 1]
+        o, ht = core(*sl, h0)
+        outs.append(o)
+        finals.append(ht)
+    o = torch.cat(outs, dim=2)
+    ht = torch.cat(finals, dim=0) if output_final_state else None
+    return o, ht
+
+
+# --------------------------------------------------------------------------- #
+# simple_gla: S_t = e^{g_t} S_{t-1} + k_t^T v_t ; o_t = scale q_t S_t
+# (g scalar per token and head; g=None means no decay)
+# --------------------------------------------------------------------------- #
+def naive_recurrent_simple_gla(
+    q: Tensor, k: Tensor, v: Tensor, g: Optional[Tensor] = None,
+    scale: Optional[float] = None, initial_state: Optional[Tensor] = None,
+    output_final_state: bool = False, cu_seqlens=None, head_first: bool = True,
+    dtype=torch.float64,
+) -> Tuple[Tensor, Optional[Tensor]]:
+    out_dtype = v.dtype
+    q, k, v = (_to_head_first(x, head_first).to(dtype) for x in (q, k, v))
+    g = None if g is None else _to_head_first(g, head_first).to(dtype)
+    K = q.shape[-1]
+    scale = K ** -0.5 if scale is None else scale
+    h0 = None if initial_state is None else initial_state.to(dtype)
+
+    def core(q, k, v, g, h0):
+        B, H, T, _ = q.shape
+        V = v.shape[-1]
+        S = q.new_zeros(B, H, K, V) if h0 is None else h0
+        o = []
+        for t in range(T):
+            if g is not None:
+                S = S * g[:, :, t].exp()[..., None, None]
+            S = S + k[:, :, t, :, None] * v[:, :, t, None, :]
+            o.append(torch.einsum('bhk,bhkv->bhv', q[:, :, t], S) * scale)
+        o = torch.stack(o, dim=2) if T > 0 else q.new_zeros(B, H, 0, V)
+        return o, S
+
+    if cu_seqlens is not None:
+        o, ht = _run_varlen(core, (q, k, v, g), h0, output_final_state, cu_seqlens)
+    else:
+        o, ht = core(q, k, v, g, h0)
+        ht = ht if output_final_state else None
+    o = _to_head_first(o, head_first)  # transpose back when time-first
+    return o, ht
+
+
+# --------------------------------------------------------------------------- #
+# gla: S_t = diag(e^{g_t}) S_{t-1} + k_t^T v_t ; o_t = scale q_t S_t  (g_t in R^K)
+# --------------------------------------------------------------------------- #
+def naive_recurrent_gla(
+    q: Tensor, k: Tensor, v: Tensor, g: Tensor,
+    scale: Optional[float] = None, initial_state: Optional[Tensor] = None,
+    output_final_state: bool = False, cu_seqlens=None, head_first: bool = True,
+    dtype=torch.float64,
+) -> Tuple[Tensor, Optional[Tensor]]:
+    q, k, v, g = (_to_head_first(x, head_first).to(dtype) for x in (q, k, v, g))
+    K = q.shape[-1]
+    scale = K ** -0.5 if scale is None else scale
+    h0 = None if initial_state is None else initial_state.to(dtype)
+
+    def core(q, k, v, g, h0):
+        B, H, T, _ = q.shape
+        V = v.shape[-1]
+        S = q.new_zeros(B, H, K, V) if h0 is None else h0
+        o = []
+        for t in range(T):
+            S = S * g[:, :, t].exp()[..., None]
+            S = S + k[:, :, t, :, None] * v[:, :, t, None, :]
+            o.append(torch.einsum('bhk,bhkv->bhv', q[:, :, t], S) * scale)
+        o = torch.stack(o, dim=2) if T > 0 else q.new_zeros(B, H, 0, V)
+        return o, S
+
+    if cu_seqlens is not None:
+        o, ht = _run_varlen(core, (q, k, v, g), h0, output_final_state, cu_seqlens)
+    else:
+        o, ht = core(q, k, v, g, h0)
+        ht = ht if output_final_state else None
+    return _to_head_first(o, head_first), ht
+
+
+# --------------------------------------------------------------------------- #
+# gated delta rule:
+#   S~_t = e^{g_t} S_{t-1};  r_t = v_t - k_t S~_t;  S_t = S~_t + k_t^T (beta_t r_t)
+#   o_t = scale q_t S_t
+# --------------------------------------------------------------------------- #
+def naive_recurrent_gated_delta_rule(
+    q: Tensor, k: Tensor, v: Tensor, g: Optional[Tensor], beta: Tensor,
+    scale: Optional[float] = None, initial_state: Optional[Tensor] = None,
+    output_final_state: bool = False, cu_seqlens=None, head_first: bool = False,
+    use_qk_l2norm_in_kernel: bool = False, dtype=torch.float64,
+) -> Tuple[Tensor, Optional[Tensor]]:
+    q, k, v, beta = (_to_head_first(x, head_first).to(dtype) for x in (q, k, v, beta))
+    g = None if g is None else _to_head_first(g, head_first).to(dtype)
+    if use_qk_l2norm_in_kernel:
+        # linear_moe/model/common_modules/l2norm.py:22-45 (eps 1e-6 inside the rsqrt)
+        q = q * torch.rsqrt((q * q).sum(-1, keepdim=True) + 1e-6)
+        k = k * torch.rsqrt((k * k).sum(-1, keepdim=True) + 1e-6)
+    K = q.shape[-1]
+    scale = K ** -0.5 if scale is None else scale
+    h0 = None if initial_state is None else initial_state.to(dtype)
+
+    def core(q, k, v, g, beta, h0):
+        B, H, T, _ = q.shape
+        V = v.shape[-1]
+        S = q.new_zeros(B, H, K, V) if h0 is None else h0
+        o = []
+        for t in range(T):
+            if g is not None:
+                S = S * g[:, :, t].exp()[..., None, None]
+            r = v[:, :, t] - torch.einsum('bhk,bhkv->bhv', k[:, :, t], S)
+            S = S + k[:, :, t, :, None] * (beta[:, :, t, None] * r)[:, :, None, :]
+            o.append(torch.einsum('bhk,bhkv->bhv', q[:, :, t], S) * scale)
+        o = torch.stack(o, dim=2) if T > 0 else q.new_zeros(B, H, 0, V)
+        return o, S
+
+    if cu_seqlens is not None:
+        o, ht = _run_varlen(core, (q, k, v, g, beta), h0, output_final_state, cu_seqlens)
+    else:
+        o, ht = core(q, k, v, g, beta, h0)
+        ht = ht if output_final_state else None
+    return _to_head_first(o, head_first), ht
+
+
+# --------------------------------------------------------------------------- #
+# adaptors the reference's modules call (same recurrences, fixed gates)
+# --------------------------------------------------------------------------- #
+def retention_log_decay(H: int, dtype=torch.float64) -> Tensor:
+    """g_h = log(1 - 2^(-5-h)) -- the per-head decay chunk_retention applies."""
+    h = torch.arange(H, dtype=dtype)
+    return torch.log1p(-torch.pow(torch.tensor(2.0, dtype=dtype), -5.0 - h))
+
+
+def naive_retention(q, k, v, scale=None, initial_state=None, output_final_state=False,
+                    cu_seqlens=None, head_first=True, dtype=torch.float64):
+    H = q.shape[1] if head_first else q.shape[2]
+    T = q.shape[2] if head_first else q.shape[1]
+    gh = retention_log_decay(H, dtype)
+    g = gh[None, :, None].expand(q.shape[0], H, T) if head_first else gh[None, None, :].expand(q.shape[0], T, H)
+    return naive_recurrent_simple_gla(q, k, v, g, scale, initial_state, output_final_state,
+                                      cu_seqlens, head_first, dtype)
+
+
+def naive_linear_attn(q, k, v, scale=None, initial_state=None, output_final_state=False,
+                      normalize=True, head_first=True, dtype=torch.float64, eps=1e-10):
+    """chunk_linear_attn: simple_gla with g=None; normalize divides o by q . cumsum(k) + eps.
+
+    The eps value is recalled from fla (not checkable offline): parity unpinned for
+    normalize=True; the reference's default path is normalize=False
+    (linear_moe/arguments.py:533-536).
+    """
+    o, ht = naive_recurrent_simple_gla(q, k, v, None, scale, initial_state, output_final_state,
+                                       None, head_first, dtype)
+    if normalize:
+        qh, kh = (_to_head_first(x, head_first).to(dtype) for x in (q, k))
+        z = (qh * kh.cumsum(2)).sum(-1, keepdim=True) + eps
+        o = _to_head_first(_to_head_first(o, head_first) / z, head_first)
+    return o, ht
+
+
+def lightning_slopes(H: int, dtype=torch.float64) -> Tensor:
+    """ALiBi-style slopes, linear_moe/sequence_modeling/lightning_attention/lightning_attention.py:79-105."""
+    def pow2(n):
+        start = 2 ** (-(2 ** -(math.log2(n) - 3)))
+        return [start * start ** i for i in range(n)]
+
+    def slopes(n):
+        if math.log2(n).is_integer():
+            return pow2(n)
+        c = 2 ** math.floor(math.log2(n))
+        return pow2(c) + slopes(2 * c)[0::2][: n - c]
+
+    return torch.tensor(slopes(H), dtype=dtype)
+
+
+def naive_lightning_attn2(q, k, v, s, dtype=torch.float64):
+    """o_i = sum_{j<=i} e^{-s_h (i-j)} (q_i . k_j) v_j  (head-first, no scale)."""
+    B, H, T, _ = q.shape
+    g = (-s.reshape(1, H, 1).to(dtype)).expand(B, H, T)
+    o, _ = naive_recurrent_simple_gla(q, k, v, g, 1.0, None, False, None, True, dtype)
+    return o
