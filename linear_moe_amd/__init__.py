@@ -5,6 +5,7 @@ Drop-in for the ``fla.ops`` callables the reference's token mixers import
 All compute runs in hand-written HIP kernels (``csrc/``) reached through the C ABI of
 ``liblmoe_hip.so`` (``include/lmoe.h``); there is no fallback path.
 """
+from .gated_delta_rule import chunk_gated_delta_rule  # noqa: F401
 from .simple_gla import chunk_simple_gla  # noqa: F401
 
-__all__ = ["chunk_simple_gla"]
+__all__ = ["chunk_simple_gla", "chunk_gated_delta_rule"]

@@ -60,7 +60,16 @@ int lmoe_chunk_simple_gla_bwd(const lmoe_args* a, void* stream) {
 int lmoe_chunk_gla_fwd(const lmoe_args* a, void* stream) { return fail(-100, "lmoe_chunk_gla_fwd: not built yet"); }
 int lmoe_chunk_gla_bwd(const lmoe_args* a, void* stream) { return fail(-100, "lmoe_chunk_gla_bwd: not built yet"); }
 int lmoe_chunk_gated_delta_rule_fwd(const lmoe_args* a, void* stream) {
-  return fail(-100, "lmoe_chunk_gated_delta_rule_fwd: not built yet");
+  const char* op = "lmoe_chunk_gated_delta_rule_fwd";
+  if (int r = check_common(a, op)) return r;
+  if (a->gate == LMOE_GATE_VECTOR) return fail(-10, "%s: the gate is one scalar per token and head", op);
+  if (!a->beta.ptr) return fail(-12, "%s: beta must not be null", op);
+  if (!a->o.ptr || !a->hs || !a->vnew.ptr || !a->w.ptr || !a->u.ptr || !a->tinv)
+    return fail(-11, "%s: o, hs, vnew, w, u and tinv must not be null", op);
+  if (a->NT == 0 || a->N == 0) return 0;
+  lmoe::launch_gdn_wy_fwd(*a, (hipStream_t)stream);
+  lmoe::launch_scalar_fwd(*a, true, (hipStream_t)stream);
+  return launched(op);
 }
 int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream) {
   return fail(-100, "lmoe_chunk_gated_delta_rule_bwd: not built yet");

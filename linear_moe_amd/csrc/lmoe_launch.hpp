@@ -6,5 +6,7 @@
 namespace lmoe {
 // simple_gla / gated delta rule forward: state pass + output (gdn = false: plain values)
 void launch_scalar_fwd(const lmoe_args& a, bool gdn, hipStream_t st);
+// gated delta rule: chunk-parallel WY preparation (w, u, Tinv)
+void launch_gdn_wy_fwd(const lmoe_args& a, hipStream_t st);
 void launch_selftest(int dtype, int kd, const void* A, const void* B, float* C, float* Ct, hipStream_t st);
 }  // namespace lmoe

@@ -1,0 +1,124 @@
+"""``chunk_gated_delta_rule`` on MI355X.
+
+  S~_t = e^{g_t} S_{t-1};  S_t = S~_t + k_t^T beta_t (v_t - k_t S~_t);  o_t = scale q_t S_t
+
+Keeps flash-linear-attention's call signature as the reference uses it at
+``linear_moe/sequence_modeling/gated_deltanet/gated_deltanet.py:112``:
+``chunk_gated_delta_rule(q, k, v, g, beta, head_first=False)`` with q, k, v ``[B,T,H,D]`` and
+g, beta ``[B,T,H]``.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._host import (SeqPlan, _aligned, _check_inputs, _desc, _state_check, base_args, ptr, stream_ptr)
+
+
+def _scalar_dt(x: torch.Tensor) -> int:
+    return _lib.LMOE_F32 if x.dtype == torch.float32 else _lib.LMOE_BF16
+
+
+class _ChunkGatedDeltaRule(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, head_first):
+        lib = _lib.load()
+        dims = _check_inputs(q, k, v, head_first, cu_seqlens)
+        B, T, H, K, V = dims
+        q, k, v = _aligned(q), _aligned(k), _aligned(v)
+        plan = SeqPlan(B, T, cu_seqlens, q.device)
+        want = (B, H, T) if head_first else (B, T, H)
+        if beta is None or tuple(beta.shape) != want:
+            raise ValueError(f"beta must have shape {want}")
+        if g is not None and tuple(g.shape) != want:
+            raise ValueError(f"g must have shape {want}, got {tuple(g.shape)}")
+        if g is not None and g.dtype not in (torch.float32, torch.bfloat16):
+            g = g.float()
+        if beta.dtype not in (torch.float32, torch.bfloat16):
+            beta = beta.float()
+        h0 = _state_check(initial_state, plan.N, H, K, V, "initial_state")
+        a = base_args(q, k, v, head_first, scale, plan, dims)
+        a.gate = _lib.GATE_NONE if g is None else _lib.GATE_SCALAR
+        if g is not None:
+            a.g, a.g_dtype = _desc(g, head_first), _scalar_dt(g)
+        a.beta, a.beta_dtype = _desc(beta, head_first), _scalar_dt(beta)
+        a.h0 = ptr(h0)
+        dev, dt = q.device, q.dtype
+        o = torch.empty_like(v)
+        ht = torch.empty(plan.N, H, K, V, dtype=torch.float32, device=dev) if output_final_state else None
+        hs = torch.empty(max(plan.NT, 1), H, K, V, dtype=dt, device=dev)
+        tinv = torch.empty(max(plan.NT, 1), H, 64, 64, dtype=dt, device=dev)
+        w = torch.empty(B, T, H, K, dtype=dt, device=dev)
+        u = torch.empty(B, T, H, V, dtype=dt, device=dev)
+        vnew = torch.empty(B, T, H, V, dtype=dt, device=dev)
+        a.o, a.ht, a.hs, a.tinv = _desc(o, head_first), ptr(ht), hs.data_ptr(), tinv.data_ptr()
+        a.w, a.u, a.vnew = _desc(w, False), _desc(u, False), _desc(vnew, False)
+        _lib.check(lib.lmoe_chunk_gated_delta_rule_fwd(C.byref(a), stream_ptr()), "chunk_gated_delta_rule forward")
+        ctx.save_for_backward(q, k, v, g, beta, h0, hs, tinv, w, vnew)
+        ctx.plan, ctx.dims, ctx.head_first, ctx.scale = plan, dims, head_first, scale
+        ctx.has_h0 = initial_state is not None
+        return o, ht
+
+    @staticmethod
+    def backward(ctx, do, dht):
+        lib = _lib.load()
+        q, k, v, g, beta, h0, hs, tinv, w, vnew = ctx.saved_tensors
+        plan, dims, head_first = ctx.plan, ctx.dims, ctx.head_first
+        B, T, H, K, V = dims
+        do = _aligned(do)
+        a = base_args(q, k, v, head_first, ctx.scale, plan, dims)
+        a.gate = _lib.GATE_NONE if g is None else _lib.GATE_SCALAR
+        if g is not None:
+            a.g, a.g_dtype = _desc(g, head_first), _scalar_dt(g)
+        a.beta, a.beta_dtype = _desc(beta, head_first), _scalar_dt(beta)
+        a.h0, a.hs, a.tinv = ptr(h0), hs.data_ptr(), tinv.data_ptr()
+        a.w, a.vnew = _desc(w, False), _desc(vnew, False)
+        a.d_o = _desc(do, head_first)
+        dht = None if dht is None else dht.float().contiguous()
+        a.dht = ptr(dht)
+        dev, dt = q.device, q.dtype
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        a.dq, a.dk, a.dv = _desc(dq, head_first), _desc(dk, head_first), _desc(dv, head_first)
+        dg = torch.empty(beta.shape, dtype=torch.float32, device=dev)
+        dbeta = torch.empty(beta.shape, dtype=torch.float32, device=dev)
+        a.dg, a.dbeta = _desc(dg, head_first), _desc(dbeta, head_first)
+        dh0 = torch.empty_like(h0) if ctx.has_h0 else None
+        a.dh0 = ptr(dh0)
+        dhs = torch.empty_like(hs)
+        dvnew = torch.empty(B, T, H, V, dtype=dt, device=dev)
+        a.dhs, a.dvnew = dhs.data_ptr(), _desc(dvnew, False)
+        _lib.check(lib.lmoe_chunk_gated_delta_rule_bwd(C.byref(a), stream_ptr()), "chunk_gated_delta_rule backward")
+        dg = None if g is None else dg.to(g.dtype)
+        return dq, dk, dv, dg, dbeta.to(beta.dtype), None, dh0, None, None, None
+
+
+def chunk_gated_delta_rule(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    g: torch.Tensor,
+    beta: torch.Tensor,
+    scale: Optional[float] = None,
+    initial_state: Optional[torch.Tensor] = None,
+    output_final_state: bool = False,
+    cu_seqlens: Optional[torch.Tensor] = None,
+    head_first: bool = False,
+    use_qk_l2norm_in_kernel: bool = False,
+) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """q, k: ``[B,T,H,K]``, v: ``[B,T,H,V]``, g (log-space decay) and beta: ``[B,T,H]``
+    (``[B,H,T,*]`` with ``head_first=True``).  Returns ``(o, final_state)``."""
+    if use_qk_l2norm_in_kernel:
+        q = _l2norm(q)
+        k = _l2norm(k)
+    return _ChunkGatedDeltaRule.apply(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens,
+                                      head_first)
+
+
+def _l2norm(x: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
+    """x * rsqrt(sum x^2 + eps) in fp32 (linear_moe/model/common_modules/l2norm.py:22-45);
+    differentiable torch ops, placed in front of the HIP op."""
+    xf = x.float()
+    return (xf * torch.rsqrt((xf * xf).sum(-1, keepdim=True) + eps)).to(x.dtype)

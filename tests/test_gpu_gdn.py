@@ -1,0 +1,75 @@
+"""GPU parity of chunk_gated_delta_rule (HIP, through the C ABI) against the token-recurrence oracle."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import naive
+from tests.util import TOL, gen, max_abs_rel
+
+pytestmark = pytest.mark.gpu
+
+
+def gdn_inputs(seed, B, T, H, K, V, dtype, head_first=False, strong_gate=False):
+    """Inputs with the laws of the contract's gated-delta-rule configs."""
+    shp = (B, H, T) if head_first else (B, T, H)
+    q = F.normalize(gen(seed, *shp, K), dim=-1).to(dtype)
+    k = F.normalize(gen(seed + 1, *shp, K), dim=-1).to(dtype)
+    v = gen(seed + 2, *shp, V, dtype=dtype)
+    beta = torch.sigmoid(gen(seed + 3, *shp)).to(dtype)
+    gh = torch.Generator().manual_seed(seed + 4)
+    if strong_gate:   # g = -exp(A_h) softplus(x + dt_bias_h), A_h ~ U(log 1, log 16)
+        A = torch.rand(H, generator=gh) * torch.log(torch.tensor(16.0))
+        dtb = torch.randn(H, generator=gh) * 0.1
+    else:             # the reference's init: small decays
+        A = torch.log(torch.rand(H, generator=gh) * 15 + 1)
+        dtb = torch.full((H,), -4.0)
+    x = gen(seed + 5, *shp)
+    hdim = 1 if head_first else 2
+    sh = [1, 1, 1]
+    sh[hdim] = H
+    g = -torch.exp(A).view(sh) * F.softplus(x + dtb.view(sh))
+    return q, k, v, g.float(), beta
+
+
+CASES = [
+    # B, T, H, K, V, h0, head_first, strong
+    (2, 200, 3, 128, 128, True, False, False),
+    (1, 256, 2, 128, 128, False, False, True),
+    (2, 130, 2, 64, 128, True, True, True),
+    (1, 64, 2, 128, 64, True, False, False),
+    (1, 5, 1, 64, 64, False, False, True),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", CASES)
+def test_gdn_fwd(cuda, dtype, case):
+    from linear_moe_amd import chunk_gated_delta_rule
+    B, T, H, K, V, use_h0, head_first, strong = case
+    q, k, v, g, beta = gdn_inputs(100, B, T, H, K, V, dtype, head_first, strong)
+    h0 = gen(114, B, H, K, V) * 0.1 if use_h0 else None
+    ref_o, ref_ht = naive.naive_recurrent_gated_delta_rule(q, k, v, g, beta, None, h0, True, None, head_first)
+    dev = lambda x: None if x is None else x.to(cuda)
+    o, ht = chunk_gated_delta_rule(dev(q), dev(k), dev(v), dev(g), dev(beta), None, dev(h0), True, None, head_first)
+    torch.cuda.synchronize()
+    assert o.dtype == dtype and o.shape == v.shape
+    tol = TOL[dtype]
+    assert max_abs_rel(o.cpu(), ref_o) < tol
+    assert max_abs_rel(ht.cpu(), ref_ht) < tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gdn_fwd_varlen(cuda, dtype):
+    from linear_moe_amd import chunk_gated_delta_rule
+    lens = [1, 64, 135, 70]
+    cu = torch.tensor([0, 1, 65, 200, 270], dtype=torch.int32)
+    T, H, K, V = sum(lens), 2, 128, 128
+    q, k, v, g, beta = gdn_inputs(200, 1, T, H, K, V, dtype, False, True)
+    h0 = gen(214, len(lens), H, K, V) * 0.1
+    ref_o, ref_ht = naive.naive_recurrent_gated_delta_rule(q, k, v, g, beta, None, h0, True, cu, False)
+    dev = lambda x: x.to(cuda)
+    o, ht = chunk_gated_delta_rule(dev(q), dev(k), dev(v), dev(g), dev(beta), None, dev(h0), True, dev(cu), False)
+    torch.cuda.synchronize()
+    tol = TOL[dtype]
+    assert max_abs_rel(o.cpu(), ref_o) < tol
+    assert max_abs_rel(ht.cpu(), ref_ht) < tol
