@@ -84,7 +84,8 @@ typedef struct lmoe_args {
   float* dh0;          /* [N,H,K,V] fp32 or NULL                                       */
   /* backward workspace (caller-allocated, element type = dtype) */
   void* dhs;           /* [NT,H,K,V] gradient w.r.t. the state at the END of every chunk */
-  lmoe_tensor dvnew;   /* [B,T,H,V]                                                    */
+  lmoe_tensor dvnew;   /* [B,T,H,V]   gradient of vnew (gated delta rule)              */
+  lmoe_tensor dw;      /* [B,T,H,K]   gradient of w    (gated delta rule)              */
 } lmoe_args;
 
 /* Library version (major*10000 + minor*100 + patch). */
@@ -114,7 +115,7 @@ int lmoe_chunk_gla_bwd(const lmoe_args* a, void* stream);
  * Replaces fla.ops.gated_delta_rule.chunk_gated_delta_rule called at
  *   linear_moe/sequence_modeling/gated_deltanet/gated_deltanet.py:112.
  * fwd uses q,k,v,g,beta,h0 -> o,ht,hs,vnew,w,u,tinv.
- * bwd uses q,k,v,g,beta,hs,vnew,w,tinv,d_o,dht -> dq,dk,dv,dg,dbeta,dh0 (+ dhs, dvnew). */
+ * bwd uses q,k,v,g,beta,hs,vnew,w,tinv,d_o,dht -> dq,dk,dv,dg,dbeta,dh0 (+ dhs, dvnew, dw). */
 int lmoe_chunk_gated_delta_rule_fwd(const lmoe_args* a, void* stream);
 int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream);
 

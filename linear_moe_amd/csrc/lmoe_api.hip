@@ -55,7 +55,15 @@ int lmoe_chunk_simple_gla_fwd(const lmoe_args* a, void* stream) {
 }
 
 int lmoe_chunk_simple_gla_bwd(const lmoe_args* a, void* stream) {
-  return fail(-100, "lmoe_chunk_simple_gla_bwd: not built yet");
+  const char* op = "lmoe_chunk_simple_gla_bwd";
+  if (int r = check_common(a, op)) return r;
+  if (a->gate == LMOE_GATE_VECTOR) return fail(-10, "%s: vector gates belong to lmoe_chunk_gla_bwd", op);
+  if (!a->hs || !a->dhs || !a->d_o.ptr || !a->dq.ptr || !a->dk.ptr || !a->dv.ptr)
+    return fail(-11, "%s: hs, dhs, d_o, dq, dk and dv must not be null", op);
+  if (a->gate == LMOE_GATE_SCALAR && !a->dg.ptr) return fail(-13, "%s: dg must not be null for a gated call", op);
+  if (a->NT == 0 || a->N == 0) return 0;
+  lmoe::launch_scalar_bwd(*a, false, (hipStream_t)stream);
+  return launched(op);
 }
 int lmoe_chunk_gla_fwd(const lmoe_args* a, void* stream) { return fail(-100, "lmoe_chunk_gla_fwd: not built yet"); }
 int lmoe_chunk_gla_bwd(const lmoe_args* a, void* stream) { return fail(-100, "lmoe_chunk_gla_bwd: not built yet"); }
@@ -72,7 +80,18 @@ int lmoe_chunk_gated_delta_rule_fwd(const lmoe_args* a, void* stream) {
   return launched(op);
 }
 int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream) {
-  return fail(-100, "lmoe_chunk_gated_delta_rule_bwd: not built yet");
+  const char* op = "lmoe_chunk_gated_delta_rule_bwd";
+  if (int r = check_common(a, op)) return r;
+  if (a->gate == LMOE_GATE_VECTOR) return fail(-10, "%s: the gate is one scalar per token and head", op);
+  if (!a->beta.ptr) return fail(-12, "%s: beta must not be null", op);
+  if (!a->hs || !a->dhs || !a->vnew.ptr || !a->w.ptr || !a->tinv || !a->dvnew.ptr || !a->dw.ptr)
+    return fail(-11, "%s: hs, dhs, vnew, w, tinv, dvnew and dw must not be null", op);
+  if (!a->d_o.ptr || !a->dq.ptr || !a->dk.ptr || !a->dv.ptr || !a->dg.ptr || !a->dbeta.ptr)
+    return fail(-13, "%s: d_o, dq, dk, dv, dg and dbeta must not be null", op);
+  if (a->NT == 0 || a->N == 0) return 0;
+  lmoe::launch_scalar_bwd(*a, true, (hipStream_t)stream);
+  lmoe::launch_gdn_wy_bwd(*a, (hipStream_t)stream);
+  return launched(op);
 }
 
 int lmoe_selftest_gemm(int32_t dtype, int32_t kd, const void* A, const void* B, float* C, float* Ct, void* stream) {

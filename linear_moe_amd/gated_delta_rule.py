@@ -89,7 +89,8 @@ class _ChunkGatedDeltaRule(torch.autograd.Function):
         a.dh0 = ptr(dh0)
         dhs = torch.empty_like(hs)
         dvnew = torch.empty(B, T, H, V, dtype=dt, device=dev)
-        a.dhs, a.dvnew = dhs.data_ptr(), _desc(dvnew, False)
+        dw = torch.empty(B, T, H, K, dtype=dt, device=dev)
+        a.dhs, a.dvnew, a.dw = dhs.data_ptr(), _desc(dvnew, False), _desc(dw, False)
         _lib.check(lib.lmoe_chunk_gated_delta_rule_bwd(C.byref(a), stream_ptr()), "chunk_gated_delta_rule backward")
         dg = None if g is None else dg.to(g.dtype)
         return dq, dk, dv, dg, dbeta.to(beta.dtype), None, dh0, None, None, None

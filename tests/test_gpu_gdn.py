@@ -73,3 +73,47 @@ def test_gdn_fwd_varlen(cuda, dtype):
     tol = TOL[dtype]
     assert max_abs_rel(o.cpu(), ref_o) < tol
     assert max_abs_rel(ht.cpu(), ref_ht) < tol
+
+
+BWD_CASES = [
+    # B, T, H, K, V, h0, head_first, strong
+    (2, 200, 2, 128, 128, True, False, False),
+    (1, 256, 2, 128, 128, False, False, True),
+    (1, 130, 2, 64, 128, True, True, True),
+    (1, 3, 1, 64, 64, True, False, False),
+]
+
+
+def _gdn_bwd_check(cuda, dtype, ins, do, dht, cu, head_first):
+    from linear_moe_amd import chunk_gated_delta_rule
+    from tests.util import oracle_grads
+    fn = lambda q, k, v, g, beta, h0: naive.naive_recurrent_gated_delta_rule(
+        q, k, v, g, beta, None, h0, True, cu, head_first)
+    _, _, ref = oracle_grads(fn, ins, do, dht)
+    dev = {n: (None if x is None else x.to(cuda).requires_grad_(True)) for n, x in ins.items()}
+    o, ht = chunk_gated_delta_rule(dev['q'], dev['k'], dev['v'], dev['g'], dev['beta'], None, dev['h0'], True,
+                                   None if cu is None else cu.to(cuda), head_first)
+    ((o * do.to(cuda)).sum() + (ht * dht.to(cuda)).sum()).backward()
+    torch.cuda.synchronize()
+    for n, r in ref.items():
+        err = max_abs_rel(dev[n].grad.cpu(), r)
+        assert err < TOL[dtype], (n, err)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", BWD_CASES)
+def test_gdn_bwd(cuda, dtype, case):
+    B, T, H, K, V, use_h0, head_first, strong = case
+    q, k, v, g, beta = gdn_inputs(300, B, T, H, K, V, dtype, head_first, strong)
+    ins = dict(q=q, k=k, v=v, g=g, beta=beta, h0=gen(314, B, H, K, V) * 0.1 if use_h0 else None)
+    shp = (B, H, T) if head_first else (B, T, H)
+    _gdn_bwd_check(cuda, dtype, ins, gen(315, *shp, V, dtype=dtype), gen(316, B, H, K, V), None, head_first)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gdn_bwd_varlen(cuda, dtype):
+    cu = torch.tensor([0, 1, 65, 200, 270], dtype=torch.int32)
+    T, H, K, V, N = 270, 2, 128, 128, 4
+    q, k, v, g, beta = gdn_inputs(400, 1, T, H, K, V, dtype, False, True)
+    ins = dict(q=q, k=k, v=v, g=g, beta=beta, h0=gen(414, N, H, K, V) * 0.1)
+    _gdn_bwd_check(cuda, dtype, ins, gen(415, 1, T, H, V, dtype=dtype), gen(416, N, H, K, V), cu, False)

@@ -75,3 +75,54 @@ def test_simple_gla_fwd_varlen(cuda, dtype):
     tol = TOL[dtype]
     assert max_abs_rel(o.cpu(), ref_o) < tol
     assert max_abs_rel(ht.cpu(), ref_ht) < tol
+
+
+BWD_CASES = [
+    # B, H, T, K, V, gate, h0, head_first
+    (2, 3, 200, 128, 128, True, True, True),
+    (2, 2, 130, 64, 128, True, True, False),
+    (1, 2, 256, 128, 64, False, False, True),
+    (1, 1, 3, 64, 64, True, True, True),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", BWD_CASES)
+def test_simple_gla_bwd(cuda, dtype, case):
+    from linear_moe_amd import chunk_simple_gla
+    from tests.util import oracle_grads
+    B, H, T, K, V, gate, use_h0, head_first = case
+    shp = (B, H, T) if head_first else (B, T, H)
+    ins = dict(q=gen(30, *shp, K, dtype=dtype), k=gen(31, *shp, K, dtype=dtype), v=gen(32, *shp, V, dtype=dtype),
+               g=torch.nn.functional.logsigmoid(gen(33, *shp)) if gate else None,
+               h0=gen(34, B, H, K, V) * 0.5 if use_h0 else None)
+    do, dht = gen(35, *shp, V, dtype=dtype), gen(36, B, H, K, V)
+    fn = lambda q, k, v, g, h0: naive.naive_recurrent_simple_gla(q, k, v, g, None, h0, True, None, head_first)
+    _, _, ref = oracle_grads(fn, ins, do, dht)
+    dev = {n: (None if x is None else x.to(cuda).requires_grad_(True)) for n, x in ins.items()}
+    o, ht = chunk_simple_gla(dev['q'], dev['k'], dev['v'], dev['g'], None, dev['h0'], True, None, head_first)
+    ((o * do.to(cuda)).sum() + (ht * dht.to(cuda)).sum()).backward()
+    torch.cuda.synchronize()
+    tol = TOL[dtype]
+    for n, r in ref.items():
+        assert max_abs_rel(dev[n].grad.cpu(), r) < tol, n
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_simple_gla_bwd_varlen(cuda, dtype):
+    from linear_moe_amd import chunk_simple_gla
+    from tests.util import oracle_grads
+    cu = torch.tensor([0, 1, 65, 200, 270], dtype=torch.int32)
+    T, H, K, V, N = 270, 2, 64, 128, 4
+    ins = dict(q=gen(40, 1, T, H, K, dtype=dtype), k=gen(41, 1, T, H, K, dtype=dtype),
+               v=gen(42, 1, T, H, V, dtype=dtype), g=torch.nn.functional.logsigmoid(gen(43, 1, T, H)),
+               h0=gen(44, N, H, K, V) * 0.5)
+    do, dht = gen(45, 1, T, H, V, dtype=dtype), gen(46, N, H, K, V)
+    fn = lambda q, k, v, g, h0: naive.naive_recurrent_simple_gla(q, k, v, g, None, h0, True, cu, False)
+    _, _, ref = oracle_grads(fn, ins, do, dht)
+    dev = {n: x.to(cuda).requires_grad_(True) for n, x in ins.items()}
+    o, ht = chunk_simple_gla(dev['q'], dev['k'], dev['v'], dev['g'], None, dev['h0'], True, cu.to(cuda), False)
+    ((o * do.to(cuda)).sum() + (ht * dht.to(cuda)).sum()).backward()
+    torch.cuda.synchronize()
+    for n, r in ref.items():
+        assert max_abs_rel(dev[n].grad.cpu(), r) < TOL[dtype], n

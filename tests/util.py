@@ -21,3 +21,15 @@ def gen(seed: int, *shape, dtype=torch.float32):
 
 
 TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2}
+
+
+def oracle_grads(fn, inputs, do, dht):
+    """Gradients of sum(o*do) + sum(ht*dht) through an oracle function, in float64.
+    ``inputs``: dict name -> tensor or None; returns (o, ht, dict name -> grad)."""
+    leaves = {k: v.detach().double().requires_grad_(True) for k, v in inputs.items() if v is not None}
+    o, ht = fn(**{k: leaves.get(k) for k in inputs})
+    loss = (o * do.double()).sum()
+    if dht is not None:
+        loss = loss + (ht * dht.double()).sum()
+    grads = torch.autograd.grad(loss, list(leaves.values()))
+    return o.detach(), ht.detach(), dict(zip(leaves.keys(), grads))
