@@ -1,0 +1,195 @@
+#!/usr/bin/env python3
+"""Headline benchmark: chunk_gated_delta_rule forward + backward on one MI355X.
+
+Workload (BASELINE.json configs[3], the one the metric is quoted on): B=4, H=16, T=8192,
+K=V=128, bf16; q,k ~ N(0,1) L2-normalised, v ~ N(0,1), beta = sigmoid(N(0,1)),
+g = -exp(A_h) softplus(x + dt_bias_h), dO ~ N(0,1).  A "step" is one forward + one backward of
+the op over that batch with all inputs resident in HBM.
+
+Prints ONE JSON line: tokens/s of the whole step, the roofline record of the dominant kernel
+(timed live with HIP events on the launch stream through ``lmoe_launch_stage``) and the CPU
+baseline (the chunked torch restatement in ``oracle/`` timed on this host's cores).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_MFMA_BF16 = 2.5e15   # dense bf16 MFMA, FLOP/s (MI355X published)
+PEAK_HBM = 8.0e12         # B/s
+CH = 64
+
+STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_state_fwd", 2: "k_out_fwd", 3: "k_bwd_dv", 4: "k_state_bwd",
+               5: "k_bwd_dqk", 6: "k_gdn_wy_bwd"}
+
+
+def gdn_inputs(B, T, H, K, V, seed, dtype, device):
+    """Contract laws of the gated-delta-rule configs (CPU generator, then copied to the GPU)."""
+    import torch
+    import torch.nn.functional as F
+    g_ = torch.Generator().manual_seed(seed)
+    rn = lambda *s: torch.randn(*s, generator=g_, dtype=torch.float32)
+    q = F.normalize(rn(B, T, H, K), dim=-1)
+    k = F.normalize(rn(B, T, H, K), dim=-1)
+    v = rn(B, T, H, V)
+    beta = torch.sigmoid(rn(B, T, H))
+    A = torch.rand(H, generator=g_) * math.log(16.0)          # A_h ~ U(log 1, log 16)
+    dt_bias = rn(H) * 0.1
+    g = -torch.exp(A)[None, None, :] * F.softplus(rn(B, T, H) + dt_bias[None, None, :])
+    do = rn(B, T, H, V)
+    dev = lambda x, dt: x.to(dt).to(device)
+    return dict(q=dev(q, dtype), k=dev(k, dtype), v=dev(v, dtype), g=dev(g, torch.float32),
+                beta=dev(beta, dtype), do=dev(do, dtype))
+
+
+def stage_model(stage, K, V, s=2):
+    """Algorithmic (flops, bytes) of one kernel per chunk and head: every product counted on full
+    64-token tiles, multiply-add = 2 flops; every input read once and every output written once."""
+    c = CH
+    kv, ck, cv, cc = K * V, c * K, c * V, c * c
+    if stage == 0:   # k k^T, triangular inverse, w, u
+        return 2 * cc * K + (2 / 3) * c ** 3 + 2 * cc * K + 2 * cc * V, 2 * (ck + cv) * s + cc * s + c * (4 + s)
+    if stage == 1:   # w S, k_d^T v_new
+        return 4 * c * kv, (2 * ck + cv) * s + cv * s + kv * s + 4 * c
+    if stage == 2:   # q k^T, q S, P v_new
+        return 2 * cc * K + 2 * c * kv + 2 * cc * V, (2 * ck + cv + kv) * s + cv * s + 4 * c
+    if stage == 3:   # q k^T, P^T do
+        return 2 * cc * K + 2 * cc * V, (2 * ck + cv) * s + cv * s + 4 * c
+    if stage == 4:   # k_d dS', q^T do, w^T dv_new
+        return 6 * c * kv, (3 * ck + 2 * cv) * s + (cv + kv) * s + 4 * c
+    if stage == 5:   # do v^T, do S^T, v dS'^T, dv_new S^T, dP k, dP^T q
+        return 2 * cc * V + 6 * c * kv + 4 * cc * K, (3 * cv + 2 * kv + 2 * ck) * s + 3 * ck * s + 8 * c
+    if stage == 6:   # dT, Tinv^T du, Tinv^T dw, two 64^3 products, dM k, dM^T k_b
+        return (2 * cc * (K + V) + 2 * cc * V + 2 * cc * K + 4 * c ** 3 + 4 * cc * K,
+                (2 * cv + 3 * ck + cc) * s + (ck + cv) * s + c * (12 + s))
+    raise ValueError(stage)
+
+
+def time_stages(call, lib, reps):
+    """Average duration (seconds) of every kernel, measured with events on the launch stream."""
+    import torch
+    from linear_moe_amd import _lib
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    out = {}
+    for stage in range(7):
+        a = call.fwd_args if stage <= 2 else call.bwd_args
+        for _ in range(2):
+            _lib.check(lib.lmoe_launch_stage(C.byref(a), call.OP, stage, st), "stage")
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            lib.lmoe_launch_stage(C.byref(a), call.OP, stage, st)
+        e1.record()
+        e1.synchronize()
+        out[stage] = e0.elapsed_time(e1) * 1e-3 / reps
+    return out
+
+
+def cpu_baseline(B, T, H, K, V, seed):
+    """The chunked torch restatement (oracle/chunked.py), forward + manual backward, fp32, on the
+    host cores: one pass over the full workload after a short warm-up."""
+    import torch
+    from oracle import chunked
+    x = gdn_inputs(B, T, H, K, V, seed, torch.float32, "cpu")
+    hf = {n: t.transpose(1, 2).contiguous() for n, t in x.items()}
+    small = {n: t[:1, :2, :256].contiguous() for n, t in hf.items()}
+    chunked.chunk_fwd_bwd("gdn", small["q"], small["k"], small["v"], small["g"], small["beta"], None, None,
+                          small["do"], None)
+    t0 = time.perf_counter()
+    with torch.no_grad():
+        chunked.chunk_fwd_bwd("gdn", hf["q"], hf["k"], hf["v"], hf["g"], hf["beta"], None, None, hf["do"], None)
+    dt = time.perf_counter() - t0
+    return {"value": B * T / dt, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"full workload once (B={B}, T={T}, H={H}, K=V={K}), fp32 chunked torch port, {dt:.2f} s"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--stage-reps", type=int, default=20)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the op shards over batch and heads without "
+              "communication); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from linear_moe_amd import _lib
+    from linear_moe_amd.gated_delta_rule import GDNCall
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    B, T, H, K, V, seed = 4, 8192, 16, 128, 128, 1004
+    x = gdn_inputs(B, T, H, K, V, seed, torch.bfloat16, dev)
+
+    call = GDNCall(keep=True)
+
+    def step():
+        call.forward(x["q"], x["k"], x["v"], x["g"], x["beta"], None, None, False, None, False)
+        call.backward(x["do"], None)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+
+    tokens = B * T
+    # whole-op algorithmic work per token and head (SURVEY 8d model): fwd 6CK+4CV+6KV+(2/3)C^2, x3
+    f_tok = 3 * (6 * CH * K + 4 * CH * V + 6 * K * V + (2 / 3) * CH * CH)
+    b_tok = (6 * K + 5 * V) * 2 + 3 * 2 + 12
+    flops, bytes_ = f_tok * tokens * H, b_tok * tokens * H
+
+    stages = time_stages(call, lib, args.stage_reps)
+    dom = max(stages, key=stages.get)
+    f_c, b_c = stage_model(dom, K, V)
+    units = (B * T // CH) * H
+    ai = f_c / b_c
+    if ai >= PEAK_MFMA_BF16 / PEAK_HBM:
+        roof = {"bound": "mfma", "achieved": f_c * units / stages[dom] / 1e12, "peak": PEAK_MFMA_BF16 / 1e12,
+                "unit": "TFLOP/s"}
+    else:
+        roof = {"bound": "hbm", "achieved": b_c * units / stages[dom] / 1e9, "peak": PEAK_HBM / 1e9, "unit": "GB/s"}
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["traffic"] = None
+    roof["kernel"] = STAGE_NAMES[dom]
+    roof["kernel_us"] = stages[dom] * 1e6
+    roof["flops_per_launch"] = f_c * units
+    roof["bytes_per_launch"] = b_c * units
+
+    rec = {
+        "metric": "chunk GDN fwd+bwd tokens/s @T=8k,H=16,D=128 bf16; % bf16 MFMA peak",
+        "value": tokens / dt, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "chunk_gated_delta_rule fwd+bwd B=4 H=16 T=8192 K=V=128 (BASELINE configs[3])",
+                   "B": B, "T": T, "H": H, "K": K, "V": V, "chunk": CH},
+        "mfma_frac": flops / dt / PEAK_MFMA_BF16, "hbm_frac_algorithmic": bytes_ / dt / PEAK_HBM,
+        "tflops": flops / dt / 1e12,
+        "kernels_us": {STAGE_NAMES[s]: round(t * 1e6, 1) for s, t in stages.items()},
+        "kernels_sum_ms": sum(stages.values()) * 1e3,
+        "roofline": roof,
+    }
+    if not args.no_cpu:
+        rec["cpu_baseline"] = cpu_baseline(B, T, H, K, V, seed)
+    print(json.dumps(rec))
+
+
+if __name__ == "__main__":
+    main()

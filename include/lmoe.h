@@ -119,6 +119,18 @@ int lmoe_chunk_gla_bwd(const lmoe_args* a, void* stream);
 int lmoe_chunk_gated_delta_rule_fwd(const lmoe_args* a, void* stream);
 int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream);
 
+/* Launch ONE kernel of an op's pipeline (profiling support: lets a harness time each kernel
+ * with events on its own stream).  `a` must be the fully populated argument block of the
+ * op's fwd (stages 0-2, 7) or bwd (stages 3-6) entry point, with the intermediates of the
+ * earlier stages already in place.  Stages: 0 gated-delta-rule WY preparation, 1 forward state
+ * pass, 2 output, 3 dv / local dv_new, 4 reverse state pass, 5 dq dk and gate gradient,
+ * 6 gated-delta-rule WY backward, 7 chunk_gla intra-chunk matrix.
+ * No counterpart in the reference (measurement support). */
+#define LMOE_OP_SIMPLE_GLA 0
+#define LMOE_OP_GLA 1
+#define LMOE_OP_GATED_DELTA_RULE 2
+int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* stream);
+
 /* Toolkit self-test: C[64][64] (fp32) = A[64][kd] * B[64][kd]^T through the same tile
  * loaders, MFMA fragments and accumulator stores the kernels use; Ct gets the transpose
  * via the transposed store path.  dtype selects the operand type; kd in {64, 128}.

@@ -45,7 +45,7 @@ ENTRY_POINTS = (
     "lmoe_chunk_simple_gla_fwd", "lmoe_chunk_simple_gla_bwd",
     "lmoe_chunk_gla_fwd", "lmoe_chunk_gla_bwd",
     "lmoe_chunk_gated_delta_rule_fwd", "lmoe_chunk_gated_delta_rule_bwd",
-    "lmoe_selftest_gemm",
+    "lmoe_launch_stage", "lmoe_selftest_gemm",
 )
 
 _lib = None
@@ -67,6 +67,8 @@ def load() -> C.CDLL:
         fn = getattr(lib, name)
         fn.argtypes = [C.POINTER(Args), C.c_void_p]
         fn.restype = C.c_int
+    lib.lmoe_launch_stage.argtypes = [C.POINTER(Args), C.c_int32, C.c_int32, C.c_void_p]
+    lib.lmoe_launch_stage.restype = C.c_int
     lib.lmoe_selftest_gemm.argtypes = [C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                        C.c_void_p]
     lib.lmoe_selftest_gemm.restype = C.c_int

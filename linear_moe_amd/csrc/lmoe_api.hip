@@ -50,7 +50,8 @@ int lmoe_chunk_simple_gla_fwd(const lmoe_args* a, void* stream) {
   if (a->gate == LMOE_GATE_VECTOR) return fail(-10, "%s: vector gates belong to lmoe_chunk_gla_fwd", op);
   if (!a->o.ptr || !a->hs) return fail(-11, "%s: o and hs must not be null", op);
   if (a->NT == 0 || a->N == 0) return 0;
-  lmoe::launch_scalar_fwd(*a, false, (hipStream_t)stream);
+  lmoe::launch_state_fwd(*a, false, (hipStream_t)stream);
+  lmoe::launch_out_fwd(*a, false, (hipStream_t)stream);
   return launched(op);
 }
 
@@ -62,7 +63,9 @@ int lmoe_chunk_simple_gla_bwd(const lmoe_args* a, void* stream) {
     return fail(-11, "%s: hs, dhs, d_o, dq, dk and dv must not be null", op);
   if (a->gate == LMOE_GATE_SCALAR && !a->dg.ptr) return fail(-13, "%s: dg must not be null for a gated call", op);
   if (a->NT == 0 || a->N == 0) return 0;
-  lmoe::launch_scalar_bwd(*a, false, (hipStream_t)stream);
+  lmoe::launch_state_bwd(*a, false, (hipStream_t)stream);
+  lmoe::launch_bwd_dv(*a, false, (hipStream_t)stream);
+  lmoe::launch_bwd_dqk(*a, false, (hipStream_t)stream);
   return launched(op);
 }
 int lmoe_chunk_gla_fwd(const lmoe_args* a, void* stream) { return fail(-100, "lmoe_chunk_gla_fwd: not built yet"); }
@@ -76,7 +79,8 @@ int lmoe_chunk_gated_delta_rule_fwd(const lmoe_args* a, void* stream) {
     return fail(-11, "%s: o, hs, vnew, w, u and tinv must not be null", op);
   if (a->NT == 0 || a->N == 0) return 0;
   lmoe::launch_gdn_wy_fwd(*a, (hipStream_t)stream);
-  lmoe::launch_scalar_fwd(*a, true, (hipStream_t)stream);
+  lmoe::launch_state_fwd(*a, true, (hipStream_t)stream);
+  lmoe::launch_out_fwd(*a, true, (hipStream_t)stream);
   return launched(op);
 }
 int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream) {
@@ -89,9 +93,36 @@ int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream) {
   if (!a->d_o.ptr || !a->dq.ptr || !a->dk.ptr || !a->dv.ptr || !a->dg.ptr || !a->dbeta.ptr)
     return fail(-13, "%s: d_o, dq, dk, dv, dg and dbeta must not be null", op);
   if (a->NT == 0 || a->N == 0) return 0;
-  lmoe::launch_scalar_bwd(*a, true, (hipStream_t)stream);
+  lmoe::launch_bwd_dv(*a, true, (hipStream_t)stream);
+  lmoe::launch_state_bwd(*a, true, (hipStream_t)stream);
+  lmoe::launch_bwd_dqk(*a, true, (hipStream_t)stream);
   lmoe::launch_gdn_wy_bwd(*a, (hipStream_t)stream);
   return launched(op);
+}
+
+int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* stream) {
+  const char* nm = "lmoe_launch_stage";
+  if (int r = check_common(a, nm)) return r;
+  if (a->NT == 0 || a->N == 0) return 0;
+  hipStream_t st = (hipStream_t)stream;
+  const bool gdn = op == LMOE_OP_GATED_DELTA_RULE;
+  if (op == LMOE_OP_SIMPLE_GLA || gdn) {
+    switch (stage) {
+      case lmoe::ST_GDN_WY_FWD: if (!gdn) return fail(-20, "%s: stage not part of this op", nm);
+        lmoe::launch_gdn_wy_fwd(*a, st); break;
+      case lmoe::ST_STATE_FWD: lmoe::launch_state_fwd(*a, gdn, st); break;
+      case lmoe::ST_OUT_FWD: lmoe::launch_out_fwd(*a, gdn, st); break;
+      case lmoe::ST_DV: lmoe::launch_bwd_dv(*a, gdn, st); break;
+      case lmoe::ST_STATE_BWD: lmoe::launch_state_bwd(*a, gdn, st); break;
+      case lmoe::ST_DQK: lmoe::launch_bwd_dqk(*a, gdn, st); break;
+      case lmoe::ST_GDN_WY_BWD: if (!gdn) return fail(-20, "%s: stage not part of this op", nm);
+        lmoe::launch_gdn_wy_bwd(*a, st); break;
+      default: return fail(-20, "%s: stage %d not part of this op", nm, stage);
+    }
+  } else {
+    return fail(-21, "%s: unknown op %d", nm, op);
+  }
+  return launched(nm);
 }
 
 int lmoe_selftest_gemm(int32_t dtype, int32_t kd, const void* A, const void* B, float* C, float* Ct, void* stream) {

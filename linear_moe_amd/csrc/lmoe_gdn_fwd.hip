@@ -4,18 +4,11 @@
 
 namespace lmoe {
 
-template <typename T>
-static void launch_gdn_wy_fwd_t(const lmoe_args& a, hipStream_t st) {
-  const dim3 grid(a.NT, a.H), block(NTHR);
-  if (a.K == 64 && a.V == 64) hipLaunchKernelGGL((k_gdn_wy_fwd<T, 64, 64>), grid, block, 0, st, a);
-  else if (a.K == 64 && a.V == 128) hipLaunchKernelGGL((k_gdn_wy_fwd<T, 64, 128>), grid, block, 0, st, a);
-  else if (a.K == 128 && a.V == 64) hipLaunchKernelGGL((k_gdn_wy_fwd<T, 128, 64>), grid, block, 0, st, a);
-  else hipLaunchKernelGGL((k_gdn_wy_fwd<T, 128, 128>), grid, block, 0, st, a);
-}
-
-void launch_gdn_wy_fwd(const lmoe_args& a, hipStream_t st) {
-  if (a.dtype == LMOE_BF16) launch_gdn_wy_fwd_t<bf16>(a, st);
-  else launch_gdn_wy_fwd_t<float>(a, st);
-}
+template <typename T, int K, int V> struct GdnWyFwd {
+  static void run(const lmoe_args& a, hipStream_t st) {
+    hipLaunchKernelGGL((k_gdn_wy_fwd<T, K, V>), dim3(a.NT, a.H), dim3(NTHR), 0, st, a);
+  }
+};
+void launch_gdn_wy_fwd(const lmoe_args& a, hipStream_t st) { dispatch<GdnWyFwd>(a, st); }
 
 }  // namespace lmoe

@@ -1,16 +1,42 @@
-// Host-side launch functions, one translation unit per kernel family.
+// Host-side launch functions, one translation unit per kernel family, and the
+// (dtype, K, V) dispatcher they share.
 #pragma once
 #include <hip/hip_runtime.h>
 #include "../../include/lmoe.h"
 
 namespace lmoe {
-// simple_gla / gated delta rule forward: state pass + output (gdn = false: plain values)
-void launch_scalar_fwd(const lmoe_args& a, bool gdn, hipStream_t st);
-// gated delta rule: chunk-parallel WY preparation (w, u, Tinv)
+
+// Stages of the three ops (argument of lmoe_launch_stage; declared in include/lmoe.h)
+enum Stage {
+  ST_GDN_WY_FWD = 0,   // gated delta rule: w, u, Tinv                   (chunk-parallel)
+  ST_STATE_FWD = 1,    // sequential state pass: hs (, vnew), ht
+  ST_OUT_FWD = 2,      // output o                                       (chunk-parallel)
+  ST_DV = 3,           // dv (simple_gla / gla) or local part of dv_new  (chunk-parallel)
+  ST_STATE_BWD = 4,    // reverse sequential state pass: dhs (, dv_new), dh0
+  ST_DQK = 5,          // dq, dk, gate gradient (, dw)                   (chunk-parallel)
+  ST_GDN_WY_BWD = 6,   // gated delta rule: backward through w, u        (chunk-parallel)
+  ST_GLA_INTRA_FWD = 7 // chunk_gla: intra-chunk attention matrix        (chunk-parallel)
+};
+
+// F<T, K, V>::run(a, st) for the runtime (dtype, K, V) of the problem
+template <template <typename, int, int> class F>
+inline void dispatch(const lmoe_args& a, hipStream_t st) {
+  typedef __bf16 bf16_t;
+#define LMOE_KV(T)                                                   \
+  if (a.K == 64 && a.V == 64) F<T, 64, 64>::run(a, st);              \
+  else if (a.K == 64 && a.V == 128) F<T, 64, 128>::run(a, st);       \
+  else if (a.K == 128 && a.V == 64) F<T, 128, 64>::run(a, st);       \
+  else F<T, 128, 128>::run(a, st);
+  if (a.dtype == LMOE_BF16) { LMOE_KV(bf16_t) } else { LMOE_KV(float) }
+#undef LMOE_KV
+}
+
+void launch_state_fwd(const lmoe_args& a, bool gdn, hipStream_t st);
+void launch_out_fwd(const lmoe_args& a, bool gdn, hipStream_t st);
 void launch_gdn_wy_fwd(const lmoe_args& a, hipStream_t st);
-// simple_gla / gated delta rule backward: dv (local), reverse state pass, dq/dk/gate gradient
-void launch_scalar_bwd(const lmoe_args& a, bool gdn, hipStream_t st);
-// gated delta rule: backward through the WY factors (finishes dk, dv, dbeta, dg)
+void launch_bwd_dv(const lmoe_args& a, bool local, hipStream_t st);
+void launch_state_bwd(const lmoe_args& a, bool gdn, hipStream_t st);
+void launch_bwd_dqk(const lmoe_args& a, bool gdn, hipStream_t st);
 void launch_gdn_wy_bwd(const lmoe_args& a, hipStream_t st);
 void launch_selftest(int dtype, int kd, const void* A, const void* B, float* C, float* Ct, hipStream_t st);
 }  // namespace lmoe

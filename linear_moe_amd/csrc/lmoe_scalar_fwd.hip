@@ -4,28 +4,34 @@
 
 namespace lmoe {
 
-template <typename T, int K, int V, bool GDN>
-static void launch_scalar_fwd_t(const lmoe_args& a, hipStream_t st) {
-  constexpr int BVS = 32;                                   // V-slice of the sequential state pass
-  constexpr int BVO = (sizeof(T) == 4 && V == 128) ? 64 : V; // V-slice of the output kernel
-  hipLaunchKernelGGL((k_state_fwd<T, K, V, BVS, GDN>), dim3(V / BVS, a.H, a.N), dim3(NTHR), 0, st, a);
-  hipLaunchKernelGGL((k_out_fwd<T, K, V, BVO, GDN>), dim3(a.NT, a.H, V / BVO), dim3(NTHR), 0, st, a);
-}
+// V-slice of the sequential state pass and of the output kernel
+template <typename T, int V> struct FwdTiles {
+  static constexpr int BVS = 32;
+  static constexpr int BVO = (sizeof(T) == 4 && V == 128) ? 64 : V;
+};
 
-template <typename T, bool GDN>
-static void launch_scalar_fwd_kv(const lmoe_args& a, hipStream_t st) {
-  if (a.K == 64 && a.V == 64) launch_scalar_fwd_t<T, 64, 64, GDN>(a, st);
-  else if (a.K == 64 && a.V == 128) launch_scalar_fwd_t<T, 64, 128, GDN>(a, st);
-  else if (a.K == 128 && a.V == 64) launch_scalar_fwd_t<T, 128, 64, GDN>(a, st);
-  else launch_scalar_fwd_t<T, 128, 128, GDN>(a, st);
-}
+template <bool GDN> struct StateFwd {
+  template <typename T, int K, int V> struct F {
+    static void run(const lmoe_args& a, hipStream_t st) {
+      constexpr int BV = FwdTiles<T, V>::BVS;
+      hipLaunchKernelGGL((k_state_fwd<T, K, V, BV, GDN>), dim3(V / BV, a.H, a.N), dim3(NTHR), 0, st, a);
+    }
+  };
+};
+template <bool GDN> struct OutFwd {
+  template <typename T, int K, int V> struct F {
+    static void run(const lmoe_args& a, hipStream_t st) {
+      constexpr int BV = FwdTiles<T, V>::BVO;
+      hipLaunchKernelGGL((k_out_fwd<T, K, V, BV, GDN>), dim3(a.NT, a.H, V / BV), dim3(NTHR), 0, st, a);
+    }
+  };
+};
 
-void launch_scalar_fwd(const lmoe_args& a, bool gdn, hipStream_t st) {
-  if (a.dtype == LMOE_BF16) {
-    if (gdn) launch_scalar_fwd_kv<bf16, true>(a, st); else launch_scalar_fwd_kv<bf16, false>(a, st);
-  } else {
-    if (gdn) launch_scalar_fwd_kv<float, true>(a, st); else launch_scalar_fwd_kv<float, false>(a, st);
-  }
+void launch_state_fwd(const lmoe_args& a, bool gdn, hipStream_t st) {
+  if (gdn) dispatch<StateFwd<true>::F>(a, st); else dispatch<StateFwd<false>::F>(a, st);
+}
+void launch_out_fwd(const lmoe_args& a, bool gdn, hipStream_t st) {
+  if (gdn) dispatch<OutFwd<true>::F>(a, st); else dispatch<OutFwd<false>::F>(a, st);
 }
 
 // C = A B^T over one 64 x KD tile pair, through the loaders / fragments / stores of the toolkit

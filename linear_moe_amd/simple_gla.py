@@ -16,9 +16,19 @@ from . import _lib
 from ._host import (SeqPlan, _aligned, _check_inputs, _desc, _state_check, base_args, ptr, stream_ptr)
 
 
-class _ChunkSimpleGLA(torch.autograd.Function):
-    @staticmethod
-    def forward(ctx, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first):
+class SimpleGLACall:
+    """One call of the op: owns the argument blocks and every buffer the kernels touch
+    (shared by the autograd function and the benchmark harness)."""
+
+    OP = 0  # LMOE_OP_SIMPLE_GLA
+
+    def __init__(self, keep: bool = False):
+        # keep=True (benchmark harness) also pins outputs and gradients so that the argument
+        # blocks stay valid for lmoe_launch_stage; the autograd path must not (reference cycle)
+        self.keep = keep
+
+    def forward(self, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first):
+        ctx = self
         lib = _lib.load()
         dims = _check_inputs(q, k, v, head_first, cu_seqlens)
         B, T, H, K, V = dims
@@ -44,15 +54,16 @@ class _ChunkSimpleGLA(torch.autograd.Function):
         a.ht = ptr(ht)
         a.hs = hs.data_ptr()
         _lib.check(lib.lmoe_chunk_simple_gla_fwd(C.byref(a), stream_ptr()), "chunk_simple_gla forward")
-        ctx.save_for_backward(q, k, v, g, h0, hs)
+        ctx.saved = (q, k, v, g, h0, hs)
+        ctx.fwd_args, ctx.fwd_keep = a, ((o, ht) if self.keep else None)
         ctx.plan, ctx.dims, ctx.head_first, ctx.scale = plan, dims, head_first, scale
         ctx.has_h0 = initial_state is not None
         return o, ht
 
-    @staticmethod
-    def backward(ctx, do, dht):
+    def backward(self, do, dht):
+        ctx = self
         lib = _lib.load()
-        q, k, v, g, h0, hs = ctx.saved_tensors
+        q, k, v, g, h0, hs = ctx.saved
         plan, dims, head_first = ctx.plan, ctx.dims, ctx.head_first
         B, T, H, K, V = dims
         do = _aligned(do)
@@ -77,8 +88,24 @@ class _ChunkSimpleGLA(torch.autograd.Function):
         dhs = torch.empty_like(hs)
         a.dhs = dhs.data_ptr()
         _lib.check(lib.lmoe_chunk_simple_gla_bwd(C.byref(a), stream_ptr()), "chunk_simple_gla backward")
+        ctx.bwd_args = a
+        ctx.bwd_keep = (do, dht, dq, dk, dv, dg, dh0, dhs) if self.keep else None
         if dg is not None and dg.dtype != g.dtype:
             dg = dg.to(g.dtype)
+        return dq, dk, dv, dg, dh0
+
+
+class _ChunkSimpleGLA(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first):
+        call = SimpleGLACall()
+        o, ht = call.forward(q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first)
+        ctx.call = call
+        return o, ht
+
+    @staticmethod
+    def backward(ctx, do, dht):
+        dq, dk, dv, dg, dh0 = ctx.call.backward(do, dht)
         return dq, dk, dv, dg, None, dh0, None, None, None
 
 
