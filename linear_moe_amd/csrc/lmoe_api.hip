@@ -68,8 +68,38 @@ int lmoe_chunk_simple_gla_bwd(const lmoe_args* a, void* stream) {
   lmoe::launch_bwd_dqk(*a, false, (hipStream_t)stream);
   return launched(op);
 }
-int lmoe_chunk_gla_fwd(const lmoe_args* a, void* stream) { return fail(-100, "lmoe_chunk_gla_fwd: not built yet"); }
-int lmoe_chunk_gla_bwd(const lmoe_args* a, void* stream) { return fail(-100, "lmoe_chunk_gla_bwd: not built yet"); }
+static int check_gla(const lmoe_args* a, const char* op) {
+  if (int r = check_common(a, op)) return r;
+  if (a->gate != LMOE_GATE_VECTOR || !a->g.ptr) return fail(-10, "%s: needs a vector gate g [B,T,H,K]", op);
+  if (a->dtype == LMOE_F32 && a->g_dtype != LMOE_F32) return fail(-14, "%s: fp32 q/k/v need an fp32 gate", op);
+  if (!a->hs || !a->amat) return fail(-11, "%s: hs and amat must not be null", op);
+  return 0;
+}
+
+int lmoe_chunk_gla_fwd(const lmoe_args* a, void* stream) {
+  const char* op = "lmoe_chunk_gla_fwd";
+  if (int r = check_gla(a, op)) return r;
+  if (!a->o.ptr) return fail(-11, "%s: o must not be null", op);
+  if (a->NT == 0 || a->N == 0) return 0;
+  hipStream_t st = (hipStream_t)stream;
+  lmoe::launch_gla(*a, lmoe::ST_GLA_INTRA_FWD, st);
+  lmoe::launch_gla(*a, lmoe::ST_STATE_FWD, st);
+  lmoe::launch_gla(*a, lmoe::ST_OUT_FWD, st);
+  return launched(op);
+}
+
+int lmoe_chunk_gla_bwd(const lmoe_args* a, void* stream) {
+  const char* op = "lmoe_chunk_gla_bwd";
+  if (int r = check_gla(a, op)) return r;
+  if (!a->dhs || !a->d_o.ptr || !a->dq.ptr || !a->dk.ptr || !a->dv.ptr || !a->dg.ptr)
+    return fail(-11, "%s: dhs, d_o, dq, dk, dv and dg must not be null", op);
+  if (a->NT == 0 || a->N == 0) return 0;
+  hipStream_t st = (hipStream_t)stream;
+  lmoe::launch_gla(*a, lmoe::ST_STATE_BWD, st);
+  lmoe::launch_gla(*a, lmoe::ST_DV, st);
+  lmoe::launch_gla(*a, lmoe::ST_DQK, st);
+  return launched(op);
+}
 int lmoe_chunk_gated_delta_rule_fwd(const lmoe_args* a, void* stream) {
   const char* op = "lmoe_chunk_gated_delta_rule_fwd";
   if (int r = check_common(a, op)) return r;
@@ -119,6 +149,12 @@ int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* strea
         lmoe::launch_gdn_wy_bwd(*a, st); break;
       default: return fail(-20, "%s: stage %d not part of this op", nm, stage);
     }
+  } else if (op == LMOE_OP_GLA) {
+    if (int r = check_gla(a, nm)) return r;
+    if (stage != lmoe::ST_GLA_INTRA_FWD && stage != lmoe::ST_STATE_FWD && stage != lmoe::ST_OUT_FWD &&
+        stage != lmoe::ST_STATE_BWD && stage != lmoe::ST_DV && stage != lmoe::ST_DQK)
+      return fail(-20, "%s: stage %d not part of this op", nm, stage);
+    lmoe::launch_gla(*a, stage, st);
   } else {
     return fail(-21, "%s: unknown op %d", nm, op);
   }

@@ -70,6 +70,12 @@ template <> struct ET<float> {
   }
 };
 
+// e^x for the pairwise decay factors: library expf on the fp32 path (keeps 1e-5 parity),
+// the hardware exp2 path for bf16 operands
+template <typename T> __device__ __forceinline__ float texp(float x) {
+  if constexpr (sizeof(T) == 4) return expf(x); else return __expf(x);
+}
+
 // ------------------------------------------------------------------------- //
 // gemm_nt: acc[mi][ni] += A[arow0 + 16 mi + r][k] * B[brow0 + 16 ni + c][k], k in [k0, k1)
 // (k0, k1 multiples of 32).  A, B: LDS tiles with leading dimensions lda, ldb.
@@ -182,6 +188,44 @@ template <typename T, int ROWS, int COLS> struct TileIO {
         const float s = rs ? rs[row] : 1.0f;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) tileT[(col + i) * ldT + row] = ET<T>::from_f(ET<T>::to_f(r.v[p][i]) * s);
+      }
+    }
+  }
+  // fp32 tile[row][col] = (float) x
+  static __device__ __forceinline__ void store_lds_f32(const Regs& r, float* tile, int ld) {
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      int row, col; coords(p, row, col);
+      if (row < ROWS) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) tile[row * ld + col + i] = ET<T>::to_f(r.v[p][i]);
+      }
+    }
+  }
+  // tile[row][col] = x * f(row, col)           (f: fp32 factor per element)
+  template <typename F>
+  static __device__ __forceinline__ void store_lds_elem(const Regs& r, T* tile, int ld, F f) {
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      int row, col; coords(p, row, col);
+      if (row < ROWS) {
+        vec o;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) o[i] = ET<T>::from_f(ET<T>::to_f(r.v[p][i]) * f(row, col + i));
+        *(vec*)(tile + row * ld + col) = o;
+      }
+    }
+  }
+  // tileT[col][row] = x * f(row, col)
+  template <typename F>
+  static __device__ __forceinline__ void store_lds_t_elem(const Regs& r, T* tileT, int ldT, F f) {
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      int row, col; coords(p, row, col);
+      if (row < ROWS) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i)
+          tileT[(col + i) * ldT + row] = ET<T>::from_f(ET<T>::to_f(r.v[p][i]) * f(row, col + i));
       }
     }
   }

@@ -1,0 +1,52 @@
+// Instantiation and launch of the chunk_gla kernels.
+#include "lmoe_launch.hpp"
+#include "lmoe_gla.hpp"
+
+namespace lmoe {
+
+template <typename T, int V> struct GlaTiles {
+  static constexpr int BVS = 32;                                      // sequential passes
+  static constexpr int BVO = (sizeof(T) == 4 && V == 128) ? 64 : V;   // output / dv kernels
+  static constexpr int BVH = sizeof(T) == 4 ? 32 : 64;                // V-slice loop of dq/dk/dg
+};
+
+template <typename T, typename GT, int K, int V>
+static void launch_gla_t(const lmoe_args& a, int stage, hipStream_t st) {
+  typedef GlaTiles<T, V> Tl;
+  const dim3 block(NTHR);
+  switch (stage) {
+    case ST_GLA_INTRA_FWD:
+      hipLaunchKernelGGL((k_gla_intra_fwd<T, GT, K>), dim3(a.NT, a.H), block, 0, st, a); break;
+    case ST_STATE_FWD:
+      hipLaunchKernelGGL((k_gla_state_fwd<T, GT, K, V, Tl::BVS>), dim3(V / Tl::BVS, a.H, a.N), block, 0, st, a); break;
+    case ST_OUT_FWD:
+      hipLaunchKernelGGL((k_gla_out_fwd<T, GT, K, V, Tl::BVO>), dim3(a.NT, a.H, V / Tl::BVO), block, 0, st, a); break;
+    case ST_STATE_BWD:
+      hipLaunchKernelGGL((k_gla_state_bwd<T, GT, K, V, Tl::BVS>), dim3(V / Tl::BVS, a.H, a.N), block, 0, st, a); break;
+    case ST_DV:
+      hipLaunchKernelGGL((k_gla_bwd_dv<T, GT, K, V, Tl::BVO>), dim3(a.NT, a.H, V / Tl::BVO), block, 0, st, a); break;
+    case ST_DQK:
+      hipLaunchKernelGGL((k_gla_bwd_dqkg<T, GT, K, V, Tl::BVH>), dim3(a.NT, a.H), block, 0, st, a); break;
+    default: break;
+  }
+}
+
+template <typename T, typename GT>
+static void launch_gla_kv(const lmoe_args& a, int stage, hipStream_t st) {
+  if (a.K == 64 && a.V == 64) launch_gla_t<T, GT, 64, 64>(a, stage, st);
+  else if (a.K == 64 && a.V == 128) launch_gla_t<T, GT, 64, 128>(a, stage, st);
+  else if (a.K == 128 && a.V == 64) launch_gla_t<T, GT, 128, 64>(a, stage, st);
+  else launch_gla_t<T, GT, 128, 128>(a, stage, st);
+}
+
+// (dtype, g_dtype) must be (bf16, bf16), (bf16, f32) or (f32, f32): checked by the caller
+void launch_gla(const lmoe_args& a, int stage, hipStream_t st) {
+  if (a.dtype == LMOE_BF16) {
+    if (a.g_dtype == LMOE_BF16) launch_gla_kv<bf16, bf16>(a, stage, st);
+    else launch_gla_kv<bf16, float>(a, stage, st);
+  } else {
+    launch_gla_kv<float, float>(a, stage, st);
+  }
+}
+
+}  // namespace lmoe

@@ -1,0 +1,433 @@
+// chunk_gla kernels: per-channel log-decays g_t in R^K.
+// Per chunk: b = inclusive cumsum of g over tokens (fp32, [64 x K]);
+//   A_ij  = sum_k q_ik k_jk e^{b_ik - b_jk}   (i >= j)     exponent formed per pair: always <= 0
+//   o     = scale [ (q . e^{b}) S + A v ]
+//   S'    = diag(e^{b_C}) S + (k . e^{b_C - b})^T v
+// Backward (dS' = gradient w.r.t. the state at chunk end, dA = scale do v^T masked i >= j):
+//   dv    = scale A^T do + (k . e^{b_C - b}) dS'
+//   dS    = diag(e^{b_C}) dS' + scale (q . e^{b})^T do
+//   dq_ik = scale e^{b_ik} (do S^T)_ik + sum_{j<=i} dA_ij k_jk e^{b_ik - b_jk}
+//   dk_jk = e^{b_Ck - b_jk} (v dS'^T)_jk + sum_{i>=j} dA_ij q_ik e^{b_ik - b_jk}
+//   db_ik = q_ik dq_ik - k_ik dk_ik (+ on the last row: sum_j (dk_d . k_d)_jk + e^{b_Ck} sum_v S_kv dS'_kv)
+//   dg    = reverse cumsum of db over the chunk's tokens
+// The pairwise-exponent sums (A, and the intra-chunk parts of dq, dk) run on the vector ALU in
+// fp32; every other product runs on MFMA through gemm_nt.
+#pragma once
+#include "lmoe_seq.hpp"
+
+namespace lmoe {
+
+// g tile of the chunk -> fp32 LDS tile s_b[64][K+1] holding the inclusive cumsum over tokens.
+// All threads; ends with a barrier.
+template <typename GT, int K>
+__device__ __forceinline__ void gla_gate_tile(const lmoe_args& a, int b, int tok, int len, int h, float* s_b) {
+  constexpr int LDB = K + 1;
+  typedef TileIO<GT, CH, K> IOG;
+  typename IOG::Regs rg;
+  IOG::load(rg, row_ptr<GT>(a.g, b, tok, h), a.g.st, len);
+  IOG::store_lds_f32(rg, s_b, LDB);
+  __syncthreads();
+  if (threadIdx.x < K) {
+    float acc = 0.f;
+    for (int r = 0; r < CH; ++r) {
+      acc += s_b[r * LDB + threadIdx.x];
+      s_b[r * LDB + threadIdx.x] = acc;
+    }
+  }
+  __syncthreads();
+}
+
+// ------------------------------------------------------------------------- //
+// A (intra-chunk attention matrix), grid = (NT, H)
+// ------------------------------------------------------------------------- //
+template <typename T, typename GT, int K>
+__global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
+  constexpr int LDB = K + 1;
+  __shared__ float s_b[CH * LDB], s_q[CH * LDB], s_k[CH * LDB];
+  const int cid = blockIdx.x, h = blockIdx.y;
+  const ChunkInfo ci = chunk_info(a, cid);
+  typedef TileIO<T, CH, K> IOK;
+  {
+    typename IOK::Regs rq, rk;
+    IOK::load(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
+    IOK::load(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
+    IOK::store_lds_f32(rq, s_q, LDB);
+    IOK::store_lds_f32(rk, s_k, LDB);
+  }
+  gla_gate_tile<GT, K>(a, ci.b, ci.tok, ci.len, h, s_b);
+  T* am = (T*)a.amat + ((int64_t)cid * a.H + h) * CH * CH;
+  const int j = threadIdx.x & 63, i0 = threadIdx.x >> 6;
+  for (int r = 0; r < 16; ++r) {
+    const int i = i0 + 4 * r;
+    float s = 0.f;
+    if (i >= j) {
+      const float* qi = s_q + i * LDB; const float* bi = s_b + i * LDB;
+      const float* kj = s_k + j * LDB; const float* bj = s_b + j * LDB;
+#pragma unroll 4
+      for (int kk = 0; kk < K; ++kk) s += qi[kk] * kj[kk] * texp<T>(bi[kk] - bj[kk]);
+    }
+    am[i * CH + j] = ET<T>::from_f(s);
+  }
+}
+
+// ------------------------------------------------------------------------- //
+// forward state pass, grid = (V / BV, H, N)
+// ------------------------------------------------------------------------- //
+template <typename T, typename GT, int K, int V, int BV>
+__global__ __launch_bounds__(NTHR) void k_gla_state_fwd(const lmoe_args a) {
+  constexpr int LDB = K + 1, LDC = CH + LPAD;
+  constexpr int MB = K / 64, NB = BV / 16;
+  __shared__ float s_b[CH * LDB];
+  __shared__ __attribute__((aligned(16))) T s_kT[K * LDC];
+  __shared__ __attribute__((aligned(16))) T s_vT[BV * LDC];
+  const int v0 = blockIdx.x * BV, h = blockIdx.y, n = blockIdx.z;
+  const SeqInfo sq = seq_info(a, n);
+  const int wv = wave_id();
+  const int krow0 = wv * (K / 4);
+  f32x4 S[MB][NB];
+  acc_zero(S);
+  if (a.h0) {
+    const float* h0 = a.h0 + ((int64_t)n * a.H + h) * K * V;
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) S[mi][ni][i] = h0[(int64_t)(krow0 + acc_row(mi, i)) * V + v0 + acc_col(ni)];
+  }
+  typedef TileIO<T, CH, K> IOK;
+  typedef TileIO<T, CH, BV> IOV;
+  for (int c = 0; c < sq.nchunks; ++c) {
+    const int tok = sq.tok0 + c * CH;
+    const int len = min(CH, sq.len - c * CH);
+    gla_gate_tile<GT, K>(a, sq.b, tok, len, h, s_b);
+    typename IOK::Regs rk;
+    IOK::load(rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, len);
+    IOK::store_lds_t_elem(rk, s_kT, LDC, [&](int r, int cc) { return texp<T>(s_b[63 * LDB + cc] - s_b[r * LDB + cc]); });
+    typename IOV::Regs rv;
+    IOV::load(rv, row_ptr<T>(a.v, sq.b, tok, h) + v0, a.v.st, len);
+    IOV::store_lds_t(rv, s_vT, LDC, nullptr);
+    T* hs = (T*)a.hs + ((int64_t)(sq.chunk0 + c) * a.H + h) * K * V;
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int kr = krow0 + acc_row(mi, i);
+          hs[(int64_t)kr * V + v0 + acc_col(ni)] = ET<T>::from_f(S[mi][ni][i]);
+          S[mi][ni][i] *= texp<T>(s_b[63 * LDB + kr]);
+        }
+    __syncthreads();
+    gemm_nt<T, MB, NB>(S, s_kT, LDC, krow0, s_vT, LDC, 0, 0, CH);
+    __syncthreads();
+  }
+  if (a.ht) {
+    float* ht = a.ht + ((int64_t)n * a.H + h) * K * V;
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ht[(int64_t)(krow0 + acc_row(mi, i)) * V + v0 + acc_col(ni)] = S[mi][ni][i];
+  }
+}
+
+// ------------------------------------------------------------------------- //
+// output, grid = (NT, H, V / BV)
+// ------------------------------------------------------------------------- //
+template <typename T, typename GT, int K, int V, int BV>
+__global__ __launch_bounds__(NTHR) void k_gla_out_fwd(const lmoe_args a) {
+  constexpr int LDB = K + 1, LDK = K + LPAD, LDC = CH + LPAD;
+  constexpr int NB = BV / 16;
+  __shared__ float s_b[CH * LDB];
+  __shared__ __attribute__((aligned(16))) T s_q[CH * LDK];
+  __shared__ __attribute__((aligned(16))) T s_hT[BV * LDK];
+  __shared__ __attribute__((aligned(16))) T s_P[CH * LDC];
+  __shared__ __attribute__((aligned(16))) T s_vT[BV * LDC];
+  const int cid = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * BV;
+  const ChunkInfo ci = chunk_info(a, cid);
+  const int wv = wave_id(), l = lane_id();
+  gla_gate_tile<GT, K>(a, ci.b, ci.tok, ci.len, h, s_b);
+  typedef TileIO<T, CH, K> IOK;
+  typedef TileIO<T, CH, BV> IOV;
+  typedef TileIO<T, K, BV> IOH;
+  typedef TileIO<T, CH, CH> IOA;
+  {
+    typename IOK::Regs rq;
+    IOK::load(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
+    IOK::store_lds_elem(rq, s_q, LDK, [&](int r, int cc) { return texp<T>(s_b[r * LDB + cc]); });
+    typename IOV::Regs rv;
+    IOV::load(rv, row_ptr<T>(a.v, ci.b, ci.tok, h) + v0, a.v.st, ci.len);
+    IOV::store_lds_t(rv, s_vT, LDC, nullptr);
+    typename IOH::Regs rh;
+    IOH::load(rh, (const T*)a.hs + ((int64_t)cid * a.H + h) * K * V + v0, V, K);
+    IOH::store_lds_t(rh, s_hT, LDK, nullptr);
+    typename IOA::Regs ra;
+    IOA::load(ra, (const T*)a.amat + ((int64_t)cid * a.H + h) * CH * CH, CH, CH);
+    IOA::store_lds(ra, s_P, LDC);
+  }
+  __syncthreads();
+  f32x4 o[1][NB];
+  acc_zero(o);
+  gemm_nt<T, 1, NB>(o, s_q, LDK, 16 * wv, s_hT, LDK, 0, 0, K);
+  gemm_nt<T, 1, NB>(o, s_P, LDC, 16 * wv, s_vT, LDC, 0, 0, CH);
+  T* od = row_ptr<T>(a.o, ci.b, ci.tok, h) + v0;
+#pragma unroll
+  for (int ni = 0; ni < NB; ++ni)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
+      if (r < ci.len) od[(int64_t)r * a.o.st + cc] = ET<T>::from_f(o[0][ni][i] * a.scale);
+    }
+}
+
+// ------------------------------------------------------------------------- //
+// reverse state pass, grid = (V / BV, H, N)
+// ------------------------------------------------------------------------- //
+template <typename T, typename GT, int K, int V, int BV>
+__global__ __launch_bounds__(NTHR) void k_gla_state_bwd(const lmoe_args a) {
+  constexpr int LDB = K + 1, LDC = CH + LPAD;
+  constexpr int MB = K / 64, NB = BV / 16;
+  __shared__ float s_b[CH * LDB];
+  __shared__ __attribute__((aligned(16))) T s_qT[K * LDC];
+  __shared__ __attribute__((aligned(16))) T s_doT[BV * LDC];
+  const int v0 = blockIdx.x * BV, h = blockIdx.y, n = blockIdx.z;
+  const SeqInfo sq = seq_info(a, n);
+  const int wv = wave_id();
+  const int krow0 = wv * (K / 4);
+  f32x4 dS[MB][NB];
+  acc_zero(dS);
+  if (a.dht) {
+    const float* p = a.dht + ((int64_t)n * a.H + h) * K * V;
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dS[mi][ni][i] = p[(int64_t)(krow0 + acc_row(mi, i)) * V + v0 + acc_col(ni)];
+  }
+  typedef TileIO<T, CH, K> IOK;
+  typedef TileIO<T, CH, BV> IOV;
+  const float scale = a.scale;
+  for (int c = sq.nchunks - 1; c >= 0; --c) {
+    const int tok = sq.tok0 + c * CH;
+    const int len = min(CH, sq.len - c * CH);
+    gla_gate_tile<GT, K>(a, sq.b, tok, len, h, s_b);
+    typename IOK::Regs rq;
+    IOK::load(rq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, len);
+    IOK::store_lds_t_elem(rq, s_qT, LDC, [&](int r, int cc) { return scale * texp<T>(s_b[r * LDB + cc]); });
+    typename IOV::Regs rd;
+    IOV::load(rd, row_ptr<T>(a.d_o, sq.b, tok, h) + v0, a.d_o.st, len);
+    IOV::store_lds_t(rd, s_doT, LDC, nullptr);
+    T* dhs = (T*)a.dhs + ((int64_t)(sq.chunk0 + c) * a.H + h) * K * V;
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int kr = krow0 + acc_row(mi, i);
+          dhs[(int64_t)kr * V + v0 + acc_col(ni)] = ET<T>::from_f(dS[mi][ni][i]);
+          dS[mi][ni][i] *= texp<T>(s_b[63 * LDB + kr]);
+        }
+    __syncthreads();
+    gemm_nt<T, MB, NB>(dS, s_qT, LDC, krow0, s_doT, LDC, 0, 0, CH);
+    __syncthreads();
+  }
+  if (a.dh0) {
+    float* p = a.dh0 + ((int64_t)n * a.H + h) * K * V;
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) p[(int64_t)(krow0 + acc_row(mi, i)) * V + v0 + acc_col(ni)] = dS[mi][ni][i];
+  }
+}
+
+// ------------------------------------------------------------------------- //
+// dv = scale A^T do + (k . e^{b_C - b}) dS',  grid = (NT, H, V / BV)
+// ------------------------------------------------------------------------- //
+template <typename T, typename GT, int K, int V, int BV>
+__global__ __launch_bounds__(NTHR) void k_gla_bwd_dv(const lmoe_args a) {
+  constexpr int LDB = K + 1, LDK = K + LPAD, LDC = CH + LPAD;
+  constexpr int NB = BV / 16;
+  __shared__ float s_b[CH * LDB];
+  __shared__ __attribute__((aligned(16))) T s_kd[CH * LDK];
+  __shared__ __attribute__((aligned(16))) T s_dhT[BV * LDK];
+  __shared__ __attribute__((aligned(16))) T s_PT[CH * LDC];
+  __shared__ __attribute__((aligned(16))) T s_doT[BV * LDC];
+  const int cid = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * BV;
+  const ChunkInfo ci = chunk_info(a, cid);
+  const int wv = wave_id(), l = lane_id();
+  gla_gate_tile<GT, K>(a, ci.b, ci.tok, ci.len, h, s_b);
+  typedef TileIO<T, CH, K> IOK;
+  typedef TileIO<T, CH, BV> IOV;
+  typedef TileIO<T, K, BV> IOH;
+  typedef TileIO<T, CH, CH> IOA;
+  {
+    typename IOK::Regs rk;
+    IOK::load(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
+    IOK::store_lds_elem(rk, s_kd, LDK, [&](int r, int cc) { return texp<T>(s_b[63 * LDB + cc] - s_b[r * LDB + cc]); });
+    typename IOV::Regs rd;
+    IOV::load(rd, row_ptr<T>(a.d_o, ci.b, ci.tok, h) + v0, a.d_o.st, ci.len);
+    IOV::store_lds_t(rd, s_doT, LDC, nullptr);
+    typename IOH::Regs rh;
+    IOH::load(rh, (const T*)a.dhs + ((int64_t)cid * a.H + h) * K * V + v0, V, K);
+    IOH::store_lds_t(rh, s_dhT, LDK, nullptr);
+    typename IOA::Regs ra;
+    IOA::load(ra, (const T*)a.amat + ((int64_t)cid * a.H + h) * CH * CH, CH, CH);
+    IOA::store_lds_t(ra, s_PT, LDC, nullptr);
+  }
+  __syncthreads();
+  f32x4 dv[1][NB];
+  acc_zero(dv);
+  gemm_nt<T, 1, NB>(dv, s_PT, LDC, 16 * wv, s_doT, LDC, 0, 0, CH);
+#pragma unroll
+  for (int ni = 0; ni < NB; ++ni) dv[0][ni] *= a.scale;
+  gemm_nt<T, 1, NB>(dv, s_kd, LDK, 16 * wv, s_dhT, LDK, 0, 0, K);
+  T* dd = row_ptr<T>(a.dv, ci.b, ci.tok, h) + v0;
+#pragma unroll
+  for (int ni = 0; ni < NB; ++ni)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
+      if (r < ci.len) dd[(int64_t)r * a.dv.st + cc] = ET<T>::from_f(dv[0][ni][i]);
+    }
+}
+
+// ------------------------------------------------------------------------- //
+// dq, dk, dg, grid = (NT, H)
+// ------------------------------------------------------------------------- //
+template <typename T, typename GT, int K, int V, int BVH>
+__global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
+  constexpr int LDV = BVH + LPAD, LDB = K + 1, LDP = CH + 1;
+  constexpr int NBK = K / 16;
+  // phase A (element type T): do, v, S, dS' slices.  phase B (fp32): dA, q, k, b tiles
+  constexpr int A_DO = 0, A_V = A_DO + CH * LDV, A_H = A_V + CH * LDV, A_DH = A_H + K * LDV, A_END = A_DH + K * LDV;
+  constexpr int B_DP = 0, B_Q = B_DP + CH * LDP, B_K = B_Q + CH * LDB, B_B = B_K + CH * LDB, B_END = B_B + CH * LDB;
+  constexpr int NBYTES = (A_END * (int)sizeof(T) > B_END * 4) ? A_END * (int)sizeof(T) : B_END * 4;
+  __shared__ __attribute__((aligned(16))) unsigned char smem_raw[NBYTES];
+  __shared__ float s_hdh[K], s_kk[4 * K];
+  T* smT = (T*)smem_raw;
+  float* smF = (float*)smem_raw;
+
+  const int cid = blockIdx.x, h = blockIdx.y;
+  const ChunkInfo ci = chunk_info(a, cid);
+  const int wv = wave_id(), l = lane_id();
+  typedef TileIO<T, CH, BVH> IOV;
+  typedef TileIO<T, K, BVH> IOH;
+  typedef TileIO<T, CH, K> IOK;
+
+  f32x4 dP[1][4], dqi[1][NBK], dkd[1][NBK];
+  acc_zero(dP); acc_zero(dqi); acc_zero(dkd);
+  float hdh[IOH::PASSES];
+#pragma unroll
+  for (int p = 0; p < IOH::PASSES; ++p) hdh[p] = 0.f;
+  for (int vv = 0; vv < V; vv += BVH) {
+    {
+      typename IOV::Regs rd, rv;
+      IOV::load(rd, row_ptr<T>(a.d_o, ci.b, ci.tok, h) + vv, a.d_o.st, ci.len);
+      IOV::load(rv, row_ptr<T>(a.v, ci.b, ci.tok, h) + vv, a.v.st, ci.len);
+      typename IOH::Regs rh, rdh;
+      IOH::load(rh, (const T*)a.hs + ((int64_t)cid * a.H + h) * K * V + vv, V, K);
+      IOH::load(rdh, (const T*)a.dhs + ((int64_t)cid * a.H + h) * K * V + vv, V, K);
+#pragma unroll
+      for (int p = 0; p < IOH::PASSES; ++p)
+#pragma unroll
+        for (int i = 0; i < IOH::VEC; ++i) hdh[p] += ET<T>::to_f(rh.v[p][i]) * ET<T>::to_f(rdh.v[p][i]);
+      IOV::store_lds(rd, smT + A_DO, LDV);
+      IOV::store_lds(rv, smT + A_V, LDV);
+      IOH::store_lds(rh, smT + A_H, LDV);
+      IOH::store_lds(rdh, smT + A_DH, LDV);
+    }
+    __syncthreads();
+    gemm_nt<T, 1, 4>(dP, smT + A_DO, LDV, 16 * wv, smT + A_V, LDV, 0, 0, BVH);
+    gemm_nt<T, 1, NBK>(dqi, smT + A_DO, LDV, 16 * wv, smT + A_H, LDV, 0, 0, BVH);
+    gemm_nt<T, 1, NBK>(dkd, smT + A_V, LDV, 16 * wv, smT + A_DH, LDV, 0, 0, BVH);
+    __syncthreads();
+  }
+  // per state row k: sum_v S_kv dS'_kv  (the IOH::VPR adjacent threads of a pass share a row)
+#pragma unroll
+  for (int p = 0; p < IOH::PASSES; ++p) {
+    float x = hdh[p];
+#pragma unroll
+    for (int d = 1; d < IOH::VPR; d <<= 1) x += __shfl_xor(x, d, 64);
+    int row, col; IOH::coords(p, row, col);
+    if (col == 0 && row < K) s_hdh[row] = x;
+  }
+  // phase B tiles (fp32)
+  {
+#pragma unroll
+    for (int nj = 0; nj < 4; ++nj)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * nj + (l & 15);
+        smF[B_DP + r * LDP + cc] = (r >= cc) ? a.scale * dP[0][nj][i] : 0.f;
+      }
+    typename IOK::Regs rq, rk;
+    IOK::load(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
+    IOK::load(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
+    IOK::store_lds_f32(rq, smF + B_Q, LDB);
+    IOK::store_lds_f32(rk, smF + B_K, LDB);
+  }
+  gla_gate_tile<GT, K>(a, ci.b, ci.tok, ci.len, h, smF + B_B);   // barriers inside
+  const float* sP = smF + B_DP; const float* sQ = smF + B_Q; const float* sK = smF + B_K; const float* sB = smF + B_B;
+  T* dqd = row_ptr<T>(a.dq, ci.b, ci.tok, h);
+  T* dkd_g = row_ptr<T>(a.dk, ci.b, ci.tok, h);
+  float kkp[NBK];                      // per column: sum over this lane's rows of (dk_d . k_d)
+  float dbv[NBK][4];
+#pragma unroll
+  for (int ni = 0; ni < NBK; ++ni) {
+    const int cc = 16 * ni + (l & 15);
+    const float bC = sB[63 * LDB + cc];
+    kkp[ni] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = 16 * wv + 4 * (l >> 4) + i;
+      const float br = sB[r * LDB + cc];
+      float sq_ = 0.f, sk_ = 0.f;
+      for (int j = 0; j <= r; ++j) sq_ += sP[r * LDP + j] * sK[j * LDB + cc] * texp<T>(br - sB[j * LDB + cc]);
+      for (int ii = r; ii < CH; ++ii) sk_ += sP[ii * LDP + r] * sQ[ii * LDB + cc] * texp<T>(sB[ii * LDB + cc] - br);
+      const float qv = sQ[r * LDB + cc], kv = sK[r * LDB + cc];
+      const float ed = texp<T>(bC - br);
+      const float dqv = a.scale * texp<T>(br) * dqi[0][ni][i] + sq_;
+      const float dkdv = dkd[0][ni][i] * ed;
+      const float dkv = dkdv + sk_;
+      kkp[ni] += kv * dkdv;
+      dbv[ni][i] = qv * dqv - kv * dkv;
+      if (r < ci.len) {
+        dqd[(int64_t)r * a.dq.st + cc] = ET<T>::from_f(dqv);
+        dkd_g[(int64_t)r * a.dk.st + cc] = ET<T>::from_f(dkv);
+      }
+    }
+    // sum over the 4 row groups of the wave
+    kkp[ni] += __shfl_xor(kkp[ni], 16, 64);
+    kkp[ni] += __shfl_xor(kkp[ni], 32, 64);
+    if (l < 16) s_kk[wv * K + cc] = kkp[ni];
+  }
+  __syncthreads();   // all reads of the q tile are done: reuse it for db
+  float* sDB = smF + B_Q;
+#pragma unroll
+  for (int ni = 0; ni < NBK; ++ni)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
+      sDB[r * LDB + cc] = dbv[ni][i];
+    }
+  __syncthreads();
+  if (threadIdx.x < K) {
+    const int cc = threadIdx.x;
+    const float last = s_kk[cc] + s_kk[K + cc] + s_kk[2 * K + cc] + s_kk[3 * K + cc] +
+                       texp<T>(sB[63 * LDB + cc]) * s_hdh[cc];
+    float* dg = (float*)a.dg.ptr + row_off(a.dg, ci.b, ci.tok, h);
+    float acc = last;   // rows past the end of a partial chunk have zero db
+    for (int r = ci.len - 1; r >= 0; --r) {
+      acc += sDB[r * LDB + cc];
+      dg[(int64_t)r * a.dg.st + cc] = acc;
+    }
+  }
+}
+
+}  // namespace lmoe
