@@ -1,0 +1,113 @@
+"""CPU-only checks of the host side: the C ABI library loads and exports what include/lmoe.h
+declares, the ctypes mirror of lmoe_args has the C layout, the chunk tables of packed input are
+right, and invalid calls are rejected before anything is launched."""
+import ctypes as C
+import os
+import re
+import subprocess
+import tempfile
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "lmoe.h")
+
+
+def declared_functions():
+    src = open(HEADER).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    return re.findall(r"^\s*(?:const\s+char\s*\*|int)\s+(lmoe_\w+)\s*\(", src, flags=re.M)
+
+
+def test_library_exports_every_declared_symbol():
+    from linear_moe_amd import _lib
+    lib = _lib.load()
+    names = declared_functions()
+    assert set(names) == set(_lib.ENTRY_POINTS), (names, _lib.ENTRY_POINTS)
+    for n in names:
+        assert getattr(lib, n) is not None
+    assert lib.lmoe_version() >= 100
+
+
+def test_ctypes_struct_matches_c_layout():
+    from linear_moe_amd import _lib
+    fields = [f[0] for f in _lib.Args._fields_]
+    prog = ['#include <stdio.h>', '#include <stddef.h>', f'#include "{HEADER}"', 'int main(void){',
+            'printf("%zu\\n", sizeof(lmoe_args));']
+    prog += [f'printf("%zu\\n", offsetof(lmoe_args, {f}));' for f in fields]
+    prog += ['return 0;}']
+    with tempfile.TemporaryDirectory() as d:
+        src, exe = os.path.join(d, "t.c"), os.path.join(d, "t")
+        open(src, "w").write("\n".join(prog))
+        subprocess.check_call(["gcc", "-o", exe, src])
+        out = [int(x) for x in subprocess.check_output([exe]).split()]
+    assert out[0] == C.sizeof(_lib.Args)
+    for f, off in zip(fields, out[1:]):
+        assert getattr(_lib.Args, f).offset == off, f
+
+
+def test_invalid_arguments_are_rejected_without_a_launch():
+    from linear_moe_amd import _lib
+    lib = _lib.load()
+    for name in _lib.ENTRY_POINTS[2:8]:
+        assert getattr(lib, name)(None, None) == -1
+        assert b"null argument block" in lib.lmoe_last_error()
+    a = _lib.Args()
+    a.dtype, a.K, a.V, a.H = 7, 64, 64, 1
+    assert lib.lmoe_chunk_simple_gla_fwd(C.byref(a), None) == -2
+    a.dtype, a.K = _lib.LMOE_BF16, 48
+    assert lib.lmoe_chunk_simple_gla_fwd(C.byref(a), None) == -3
+    assert b"K=48" in lib.lmoe_last_error()
+    a.K, a.B, a.N = 64, 2, 1                       # dense input must have N == B
+    assert lib.lmoe_chunk_gla_fwd(C.byref(a), None) == -6
+    a.N = 2                                        # q, k, v null
+    assert lib.lmoe_chunk_gated_delta_rule_fwd(C.byref(a), None) == -7
+    with pytest.raises(ValueError):
+        _lib.check(-7, "x")
+    assert lib.lmoe_selftest_gemm(0, 64, None, None, None, None, None) == -1
+
+
+def test_seq_plan_tables():
+    from linear_moe_amd._host import SeqPlan
+    p = SeqPlan(3, 130, None, "cpu")
+    assert (p.N, p.NT) == (3, 9) and p.cu is None
+    cu = torch.tensor([0, 1, 65, 200, 270, 270], dtype=torch.int64)
+    p = SeqPlan(1, 270, cu, "cpu")
+    assert p.N == 5 and p.NT == 1 + 1 + 3 + 2 + 0
+    assert p.seq_chunk0.tolist() == [0, 1, 2, 5, 7, 7]
+    assert p.chunk_map.tolist() == [[0, 0], [1, 0], [2, 0], [2, 1], [2, 2], [3, 0], [3, 1]]
+    assert p.cu.dtype == torch.int32
+    for bad in ([1, 5, 270], [0, 50, 40, 270], [0, 100]):
+        with pytest.raises(ValueError):
+            SeqPlan(1, 270, torch.tensor(bad), "cpu")
+
+
+def test_python_layer_validates_before_launch():
+    import linear_moe_amd as L
+    q = torch.zeros(1, 2, 8, 64)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        L.chunk_simple_gla(q, q, q)
+    from linear_moe_amd._host import _check_inputs
+    qc = torch.zeros(1, 2, 8, 64, device="meta")
+
+    class Fake:  # shape / dtype / is_cuda carrier: validation must not touch data
+        def __init__(self, t, dt=torch.bfloat16):
+            self.shape, self.dtype, self.is_cuda, self._t = t.shape, dt, True, t
+
+        def dim(self):
+            return self._t.dim()
+
+    f = Fake(qc)
+    assert _check_inputs(f, f, f, True, None) == (1, 8, 2, 64, 64)
+    with pytest.raises(ValueError, match="unsupported"):
+        g = Fake(torch.zeros(1, 2, 8, 48, device="meta"))
+        _check_inputs(g, g, g, True, None)
+    with pytest.raises(ValueError, match="head_first=False"):
+        _check_inputs(f, f, f, True, torch.tensor([0, 8]))
+    with pytest.raises(ValueError, match="batch size 1"):
+        g = Fake(torch.zeros(2, 8, 2, 64, device="meta"))
+        _check_inputs(g, g, g, False, torch.tensor([0, 8]))
+    with pytest.raises(ValueError, match="dtype"):
+        g = Fake(qc, torch.float16)
+        _check_inputs(g, g, g, True, None)

@@ -1,0 +1,269 @@
+"""Pins of the CPU oracle (oracle/naive.py, oracle/chunked.py).
+
+The reference ships no test or golden vector for this path (its arithmetic lives in the absent
+flash-linear-attention submodule), so the oracle is pinned by what the mathematics fixes:
+closed forms, special cases that reduce to library routines, hand-unrolled tiny cases,
+invariants, finite differences, and the independent torch routines shipped with
+``transformers`` for the gated delta rule.  Each check is chosen so that a plausible slip (a
+dropped decay, a transposed operand, an off-by-one in the gate's position) breaks it.
+"""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import chunked, naive
+
+D = torch.float64
+
+
+def rnd(seed, *shape):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed), dtype=D)
+
+
+# ----------------------------- closed forms -------------------------------- #
+def test_simple_gla_no_gate_is_masked_attention():
+    q, k, v = rnd(1, 2, 3, 37, 8), rnd(2, 2, 3, 37, 8), rnd(3, 2, 3, 37, 5)
+    o, ht = naive.naive_recurrent_simple_gla(q, k, v, None, 0.3, None, True)
+    ref = 0.3 * torch.tril(q @ k.transpose(-1, -2)) @ v
+    assert torch.allclose(o, ref, atol=1e-12)
+    assert torch.allclose(ht, k.transpose(-1, -2) @ v, atol=1e-12)
+
+
+def test_default_scale_is_rsqrt_k():
+    q, k, v = rnd(1, 1, 1, 9, 16), rnd(2, 1, 1, 9, 16), rnd(3, 1, 1, 9, 4)
+    o, _ = naive.naive_recurrent_simple_gla(q, k, v)
+    assert torch.allclose(o, 0.25 * torch.tril(q @ k.transpose(-1, -2)) @ v, atol=1e-12)
+
+
+def test_retention_closed_form():
+    B, H, T = 1, 4, 50
+    q, k, v = rnd(4, B, H, T, 8), rnd(5, B, H, T, 8), rnd(6, B, H, T, 6)
+    o, _ = naive.naive_retention(q, k, v, scale=1.0)
+    gam = 1 - torch.pow(torch.tensor(2.0, dtype=D), -5.0 - torch.arange(H, dtype=D))
+    idx = torch.arange(T)
+    dist = (idx[:, None] - idx[None, :]).clamp_min(0).to(D)
+    Dm = torch.tril(gam[:, None, None] ** dist)
+    ref = ((q @ k.transpose(-1, -2)) * Dm[None]) @ v
+    assert torch.allclose(o, ref, atol=1e-12)
+    # value of the first head's decay: 1 - 2^-5
+    assert math.isclose(math.exp(naive.retention_log_decay(4)[0].item()), 1 - 2 ** -5, rel_tol=1e-14)
+
+
+def test_lightning_slopes_and_closed_form():
+    s8 = naive.lightning_slopes(8)
+    assert torch.allclose(s8, torch.tensor([2.0 ** -(i + 1) for i in range(8)], dtype=D))
+    s16 = naive.lightning_slopes(16)
+    assert torch.allclose(s16, torch.tensor([2.0 ** (-(i + 1) / 2) for i in range(16)], dtype=D))
+    assert len(naive.lightning_slopes(12)) == 12          # non power of two: interleaved completion
+    B, H, T = 1, 8, 20
+    q, k, v = rnd(7, B, H, T, 4), rnd(8, B, H, T, 4), rnd(9, B, H, T, 4)
+    o = naive.naive_lightning_attn2(q, k, v, s8.reshape(H, 1, 1))
+    idx = torch.arange(T)
+    dist = (idx[:, None] - idx[None, :]).clamp_min(0).to(D)
+    Dm = torch.tril(torch.exp(-s8[:, None, None] * dist))
+    assert torch.allclose(o, ((q @ k.transpose(-1, -2)) * Dm[None]) @ v, atol=1e-12)
+
+
+def test_scalars_by_hand():
+    # K = V = 1, T = 3, everything written out
+    q = torch.tensor([2.0, -1.0, 0.5], dtype=D).view(1, 1, 3, 1)
+    k = torch.tensor([1.0, 3.0, -2.0], dtype=D).view(1, 1, 3, 1)
+    v = torch.tensor([0.5, 1.0, 4.0], dtype=D).view(1, 1, 3, 1)
+    g = torch.tensor([-0.1, -0.2, -0.3], dtype=D).view(1, 1, 3)
+    h0 = torch.tensor([[[[0.7]]]], dtype=D)
+    e = math.exp
+    s1 = e(-0.1) * 0.7 + 1.0 * 0.5
+    s2 = e(-0.2) * s1 + 3.0 * 1.0
+    s3 = e(-0.3) * s2 + (-2.0) * 4.0
+    o, ht = naive.naive_recurrent_simple_gla(q, k, v, g, 1.0, h0, True)
+    assert torch.allclose(o.flatten(), torch.tensor([2 * s1, -s2, 0.5 * s3], dtype=D), atol=1e-14)
+    assert math.isclose(ht.item(), s3, rel_tol=1e-14)
+    # gated delta rule on the same numbers, beta = (0.5, 1, 0.25)
+    beta = torch.tensor([0.5, 1.0, 0.25], dtype=D).view(1, 1, 3)
+    t1 = e(-0.1) * 0.7
+    d1 = t1 + 1.0 * 0.5 * (0.5 - 1.0 * t1)
+    t2 = e(-0.2) * d1
+    d2 = t2 + 3.0 * 1.0 * (1.0 - 3.0 * t2)
+    t3 = e(-0.3) * d2
+    d3 = t3 + (-2.0) * 0.25 * (4.0 - (-2.0) * t3)
+    o, ht = naive.naive_recurrent_gated_delta_rule(q, k, v, g, beta, 1.0, h0, True, head_first=True)
+    assert torch.allclose(o.flatten(), torch.tensor([2 * d1, -d2, 0.5 * d3], dtype=D), atol=1e-14)
+    assert math.isclose(ht.item(), d3, rel_tol=1e-14)
+
+
+def test_gla_channel_constant_gate_equals_simple_gla():
+    q, k, v = rnd(10, 2, 2, 33, 8), rnd(11, 2, 2, 33, 8), rnd(12, 2, 2, 33, 6)
+    g = F.logsigmoid(rnd(13, 2, 2, 33))
+    h0 = rnd(14, 2, 2, 8, 6)
+    o1, h1 = naive.naive_recurrent_simple_gla(q, k, v, g, None, h0, True)
+    o2, h2 = naive.naive_recurrent_gla(q, k, v, g[..., None].expand(-1, -1, -1, 8), None, h0, True)
+    assert torch.allclose(o1, o2, atol=1e-12) and torch.allclose(h1, h2, atol=1e-12)
+
+
+def test_gla_per_channel_decay_closed_form():
+    # o_t = scale sum_{s<=t} sum_k q_tk k_sk exp(sum_{s<r<=t} g_rk) v_s
+    B, H, T, K, V = 1, 1, 6, 3, 2
+    q, k, v = rnd(15, B, H, T, K), rnd(16, B, H, T, K), rnd(17, B, H, T, V)
+    g = F.logsigmoid(rnd(18, B, H, T, K))
+    o, _ = naive.naive_recurrent_gla(q, k, v, g, 1.0)
+    cs = g.cumsum(2)
+    ref = torch.zeros(B, H, T, V, dtype=D)
+    for t in range(T):
+        for s in range(t + 1):
+            wgt = (q[0, 0, t] * k[0, 0, s] * torch.exp(cs[0, 0, t] - cs[0, 0, s])).sum()
+            ref[0, 0, t] += wgt * v[0, 0, s]
+    assert torch.allclose(o, ref, atol=1e-12)
+
+
+def test_gdn_beta_zero_only_decays_initial_state():
+    B, H, T, K, V = 1, 2, 20, 4, 3
+    q, k, v = rnd(19, B, T, H, K), rnd(20, B, T, H, K), rnd(21, B, T, H, V)
+    g = F.logsigmoid(rnd(22, B, T, H))
+    h0 = rnd(23, B, H, K, V)
+    o, ht = naive.naive_recurrent_gated_delta_rule(q, k, v, g, torch.zeros(B, T, H, dtype=D), 1.0, h0, True)
+    dec = torch.exp(g.cumsum(1))                                    # [B,T,H]
+    ref = torch.einsum('bthk,bhkv->bthv', q, h0) * dec[..., None]
+    assert torch.allclose(o, ref, atol=1e-12)
+    assert torch.allclose(ht, h0 * dec[:, -1, :, None, None], atol=1e-12)
+
+
+def test_gdn_orthonormal_keys_store_values_exactly():
+    # distinct orthonormal keys, beta = 1, no decay: the state maps k_i to v_i
+    K = V = T = 8
+    k = torch.linalg.qr(rnd(24, K, K))[0].view(1, T, 1, K)
+    v = rnd(25, 1, T, 1, V)
+    z = torch.zeros(1, T, 1, dtype=D)
+    o, ht = naive.naive_recurrent_gated_delta_rule(k, k, v, z, torch.ones(1, T, 1, dtype=D), 1.0, None, True)
+    assert torch.allclose(torch.einsum('bthk,bhkv->bthv', k, ht), v, atol=1e-12)
+    assert torch.allclose(o, v, atol=1e-12)          # querying with k_t right after writing v_t
+
+
+def test_gdn_matches_transformers_torch_routines():
+    tr = pytest.importorskip("transformers.models.qwen3_next.modeling_qwen3_next")
+    B, T, H, K, V = 2, 150, 3, 16, 24
+    q = F.normalize(rnd(26, B, T, H, K), dim=-1)
+    k = F.normalize(rnd(27, B, T, H, K), dim=-1)
+    v, beta = rnd(28, B, T, H, V), torch.sigmoid(rnd(29, B, T, H))
+    g = -torch.rand(B, T, H, generator=torch.Generator().manual_seed(30), dtype=D)
+    h0 = rnd(31, B, H, K, V) * 0.3
+    o, ht = naive.naive_recurrent_gated_delta_rule(q, k, v, g, beta, None, h0, True)
+    f = lambda x: x.float()
+    o1, h1 = tr.torch_recurrent_gated_delta_rule(f(q), f(k), f(v), f(g), f(beta), f(h0), True)
+    o2, h2 = tr.torch_chunk_gated_delta_rule(f(q), f(k), f(v), f(g), f(beta), 64, f(h0), True)
+    for oo, hh in ((o1, h1), (o2, h2)):
+        assert (oo.double() - o).abs().max() < 2e-5 * o.abs().max().clamp_min(1)
+        assert (hh.double() - ht).abs().max() < 2e-5 * ht.abs().max().clamp_min(1)
+
+
+# ------------------------------- invariants -------------------------------- #
+def _ops():
+    B, H, T, K, V = 2, 2, 90, 8, 6
+    q, k, v = rnd(40, B, H, T, K), rnd(41, B, H, T, K), rnd(42, B, H, T, V)
+    gs, gv = F.logsigmoid(rnd(43, B, H, T)), F.logsigmoid(rnd(44, B, H, T, K))
+    beta = torch.sigmoid(rnd(45, B, H, T))
+    kn = F.normalize(k, dim=-1)
+    return {
+        'simple_gla': lambda q_, k_, v_, h0, sl: naive.naive_recurrent_simple_gla(q_, k_, v_, gs[:, :, sl], None, h0, True),
+        'gla': lambda q_, k_, v_, h0, sl: naive.naive_recurrent_gla(q_, k_, v_, gv[:, :, sl], None, h0, True),
+        'gdn': lambda q_, k_, v_, h0, sl: naive.naive_recurrent_gated_delta_rule(
+            q_, F.normalize(k_, dim=-1), v_, gs[:, :, sl], beta[:, :, sl], None, h0, True, head_first=True),
+    }, (q, k, v)
+
+
+@pytest.mark.parametrize("op", ['simple_gla', 'gla', 'gdn'])
+def test_state_handoff_and_linearity(op):
+    ops, (q, k, v) = _ops()
+    f = ops[op]
+    T, T1 = q.shape[2], 37
+    full = slice(0, T)
+    o, ht = f(q, k, v, None, full)
+    o1, h1 = f(q[:, :, :T1], k[:, :, :T1], v[:, :, :T1], None, slice(0, T1))
+    o2, h2 = f(q[:, :, T1:], k[:, :, T1:], v[:, :, T1:], h1, slice(T1, T))
+    assert torch.allclose(torch.cat([o1, o2], 2), o, atol=1e-11)
+    assert torch.allclose(h2, ht, atol=1e-11)
+    # linear in v (zero initial state)
+    oa, _ = f(q, k, 2.5 * v, None, full)
+    assert torch.allclose(oa, 2.5 * o, atol=1e-10)
+
+
+def test_varlen_equals_per_sequence_and_time_first_equals_head_first():
+    T, H, K, V = 60, 2, 8, 6
+    cu = torch.tensor([0, 7, 8, 40, 60])
+    q, k, v = rnd(50, 1, T, H, K), F.normalize(rnd(51, 1, T, H, K), dim=-1), rnd(52, 1, T, H, V)
+    g, beta = F.logsigmoid(rnd(53, 1, T, H)), torch.sigmoid(rnd(54, 1, T, H))
+    h0 = rnd(55, 4, H, K, V)
+    o, ht = naive.naive_recurrent_gated_delta_rule(q, k, v, g, beta, None, h0, True, cu)
+    for n in range(4):
+        s, e = int(cu[n]), int(cu[n + 1])
+        on, hn = naive.naive_recurrent_gated_delta_rule(q[:, s:e], k[:, s:e], v[:, s:e], g[:, s:e], beta[:, s:e],
+                                                        None, h0[n:n + 1], True)
+        assert torch.allclose(o[:, s:e], on, atol=1e-12) and torch.allclose(ht[n:n + 1], hn, atol=1e-12)
+    tp = lambda x: x.transpose(1, 2)
+    oh, hh = naive.naive_recurrent_gated_delta_rule(tp(q), tp(k), tp(v), tp(g), tp(beta), None, h0[:1], True,
+                                                    head_first=True)
+    ot, ht_ = naive.naive_recurrent_gated_delta_rule(q, k, v, g, beta, None, h0[:1], True)
+    assert torch.allclose(tp(oh), ot, atol=1e-12) and torch.allclose(hh, ht_, atol=1e-12)
+
+
+# ---------------------- gradients: finite differences ---------------------- #
+@pytest.mark.parametrize("op", ['simple_gla', 'gla', 'gdn'])
+def test_oracle_gradcheck(op):
+    B, H, T, K, V = 1, 1, 5, 3, 2
+    q, k, v = rnd(60, B, H, T, K), rnd(61, B, H, T, K), rnd(62, B, H, T, V)
+    h0 = rnd(63, B, H, K, V)
+    if op == 'simple_gla':
+        g = F.logsigmoid(rnd(64, B, H, T))
+        f = lambda q, k, v, g, h0: naive.naive_recurrent_simple_gla(q, k, v, g, None, h0, True)
+        args = (q, k, v, g, h0)
+    elif op == 'gla':
+        g = F.logsigmoid(rnd(64, B, H, T, K))
+        f = lambda q, k, v, g, h0: naive.naive_recurrent_gla(q, k, v, g, None, h0, True)
+        args = (q, k, v, g, h0)
+    else:
+        g, beta = F.logsigmoid(rnd(64, B, H, T)), torch.sigmoid(rnd(65, B, H, T))
+        f = lambda q, k, v, g, beta, h0: naive.naive_recurrent_gated_delta_rule(q, k, v, g, beta, None, h0, True,
+                                                                              head_first=True)
+        args = (q, k, v, g, beta, h0)
+    args = tuple(a.clone().requires_grad_(True) for a in args)
+    assert torch.autograd.gradcheck(f, args, eps=1e-6, atol=1e-6)
+
+
+# ------------------ chunked restatement vs token recurrence ---------------- #
+@pytest.mark.parametrize("op", ['simple_gla', 'gla', 'gdn'])
+@pytest.mark.parametrize("C", [16, 32, 64])
+def test_chunked_matches_naive_and_autograd(op, C):
+    B, H, T, K, V = 2, 2, 150, 8, 12
+    q, k, v = rnd(70, B, H, T, K), rnd(71, B, H, T, K), rnd(72, B, H, T, V)
+    if op == 'gdn':
+        q, k = F.normalize(q, dim=-1), F.normalize(k, dim=-1)
+    g = F.logsigmoid(rnd(73, B, H, T, K)) if op == 'gla' else F.logsigmoid(rnd(73, B, H, T))
+    beta = torch.sigmoid(rnd(74, B, H, T)) if op == 'gdn' else None
+    h0, do, dht = rnd(75, B, H, K, V) * 0.3, rnd(76, B, H, T, V), rnd(77, B, H, K, V)
+    leaves = [x.clone().requires_grad_(True) for x in (q, k, v, g, h0)] + ([beta.clone().requires_grad_(True)] if op == 'gdn' else [])
+    if op == 'simple_gla':
+        o, ht = naive.naive_recurrent_simple_gla(*leaves[:4], None, leaves[4], True)
+    elif op == 'gla':
+        o, ht = naive.naive_recurrent_gla(*leaves[:4], None, leaves[4], True)
+    else:
+        o, ht = naive.naive_recurrent_gated_delta_rule(*leaves[:4], leaves[5], None, leaves[4], True, head_first=True)
+    grads = torch.autograd.grad((o * do).sum() + (ht * dht).sum(), leaves)
+    o2, ht2, (dq, dk, dv, dg, dbeta, dh0) = chunked.chunk_fwd_bwd(op, q, k, v, g, beta, None, h0, do, dht, C=C, dtype=D)
+    assert torch.allclose(o2, o, atol=1e-10) and torch.allclose(ht2, ht, atol=1e-10)
+    mine = [dq, dk, dv, dg, dh0] + ([dbeta] if op == 'gdn' else [])
+    for a, b in zip(grads, mine):
+        assert torch.allclose(a, b, atol=1e-9 * max(1.0, a.abs().max().item()))
+
+
+def test_gate_gradient_identity():
+    # dg_t = sum_{s>=t} (q_s.dq_s - k_s.dk_s) + <S_T, dht>   (simple_gla)
+    B, H, T, K, V = 1, 2, 40, 4, 3
+    q, k, v = (x.requires_grad_(True) for x in (rnd(80, B, H, T, K), rnd(81, B, H, T, K), rnd(82, B, H, T, V)))
+    g = F.logsigmoid(rnd(83, B, H, T)).requires_grad_(True)
+    do, dht = rnd(84, B, H, T, V), rnd(85, B, H, K, V)
+    o, ht = naive.naive_recurrent_simple_gla(q, k, v, g, None, None, True)
+    dq, dk, dg = torch.autograd.grad((o * do).sum() + (ht * dht).sum(), (q, k, g))
+    x = (q * dq).sum(-1) - (k * dk).sum(-1)
+    ref = x.flip(2).cumsum(2).flip(2) + (ht * dht).sum((-1, -2))[..., None]
+    assert torch.allclose(dg, ref, atol=1e-10)
