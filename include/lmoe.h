@@ -131,11 +131,12 @@ int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream);
 #define LMOE_OP_GATED_DELTA_RULE 2
 int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* stream);
 
-/* Toolkit self-test: C[64][64] (fp32) = A[64][kd] * B[64][kd]^T through the same tile
- * loaders, MFMA fragments and accumulator stores the kernels use; Ct gets the transpose
- * via the transposed store path.  dtype selects the operand type; kd in {64, 128}.
+/* Toolkit self-test over one pair of 64 x kd tiles A, B (element type by dtype, kd in {64,128}),
+ * through the same tile loaders, MFMA fragments and accumulator stores the kernels use:
+ * C[64][64] (fp32) = A B^T (contraction along tile columns), G[kd][kd] (fp32) = A^T B
+ * (contraction along tile rows: the transposed-fragment path).
  * No counterpart in the reference (test support). */
-int lmoe_selftest_gemm(int32_t dtype, int32_t kd, const void* A, const void* B, float* C, float* Ct, void* stream);
+int lmoe_selftest_gemm(int32_t dtype, int32_t kd, const void* A, const void* B, float* C, float* G, void* stream);
 
 #ifdef __cplusplus
 }

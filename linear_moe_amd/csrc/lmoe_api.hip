@@ -161,11 +161,11 @@ int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* strea
   return launched(nm);
 }
 
-int lmoe_selftest_gemm(int32_t dtype, int32_t kd, const void* A, const void* B, float* C, float* Ct, void* stream) {
-  if (!A || !B || !C || !Ct) return fail(-1, "lmoe_selftest_gemm: null pointer");
+int lmoe_selftest_gemm(int32_t dtype, int32_t kd, const void* A, const void* B, float* C, float* G, void* stream) {
+  if (!A || !B || !C || !G) return fail(-1, "lmoe_selftest_gemm: null pointer");
   if ((dtype != LMOE_BF16 && dtype != LMOE_F32) || (kd != 64 && kd != 128))
     return fail(-2, "lmoe_selftest_gemm: dtype/kd unsupported");
-  lmoe::launch_selftest(dtype, kd, A, B, C, Ct, (hipStream_t)stream);
+  lmoe::launch_selftest(dtype, kd, A, B, C, G, (hipStream_t)stream);
   return launched("lmoe_selftest_gemm");
 }
 

@@ -29,6 +29,15 @@ constexpr int CH = 64;        // chunk length (tokens)
 constexpr int NTHR = 256;     // threads per work-group
 constexpr int LPAD = 8;       // LDS row padding in elements (16 B for bf16, 32 B for fp32)
 
+// Work-group barrier that orders LDS traffic only: waits for this wave's outstanding LDS
+// operations, not for its global loads, so register prefetches issued before the barrier stay
+// in flight across it (__syncthreads() would drain them).
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
 __device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
 
@@ -45,6 +54,19 @@ template <> struct ET<bf16> {
   static __device__ __forceinline__ float to_f(bf16 x) { return (float)x; }
   static __device__ __forceinline__ bf16 from_f(float x) { return (bf16)x; }
   static __device__ __forceinline__ frag load_frag(const bf16* p) { return *(const bf16x8*)p; }
+  // Fragment of an operand stored with the contraction index along the ROWS of the tile:
+  // lane (c = l%16, g = l/16) receives tile[k0 + 8g + i][n0 + c], i = 0..7, through two
+  // ds_read_b64_tr_b16: inside each group of 16 lanes, lane s points at the 4 elements
+  // tile[row + s/4][n0 + 4 (s%4) ..] and receives element (s%4) of the lanes 4j + s/4, j = 0..3,
+  // i.e. the four rows row..row+3 of its own column.
+  static __device__ __forceinline__ frag load_frag_t(const bf16* tile, int ld, int k0, int n0) {
+    const int l = threadIdx.x & 63, s = l & 15;
+    const bf16* p = tile + (k0 + 8 * (l >> 4) + (s >> 2)) * ld + n0 + 4 * (s & 3);
+    typedef __attribute__((address_space(3))) bf16x4 lds_b4;
+    const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_b4*)p);
+    const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_b4*)(p + 4 * ld));
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  }
   static __device__ __forceinline__ void mma(f32x4& c, const frag& a, const frag& b) {
     c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
   }
@@ -61,6 +83,15 @@ template <> struct ET<float> {
   static __device__ __forceinline__ float from_f(float x) { return x; }
   static __device__ __forceinline__ frag load_frag(const float* p) {
     frag f; f.lo = *(const f32x4*)p; f.hi = *(const f32x4*)(p + 4); return f;
+  }
+  // contraction index along the rows of the tile: plain strided reads (fp32 is the parity path)
+  static __device__ __forceinline__ frag load_frag_t(const float* tile, int ld, int k0, int n0) {
+    const int l = threadIdx.x & 63;
+    const float* p = tile + (k0 + 8 * (l >> 4)) * ld + n0 + (l & 15);
+    frag f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { f.lo[i] = p[i * ld]; f.hi[i] = p[(i + 4) * ld]; }
+    return f;
   }
   static __device__ __forceinline__ void mma(f32x4& c, const frag& a, const frag& b) {
 #pragma unroll
@@ -91,6 +122,33 @@ __device__ __forceinline__ void gemm_nt(f32x4 (&acc)[MB][NB], const T* A, int ld
     for (int mi = 0; mi < MB; ++mi) a[mi] = ET<T>::load_frag(A + (arow0 + 16 * mi + r) * lda + kk + kg);
 #pragma unroll
     for (int ni = 0; ni < NB; ++ni) b[ni] = ET<T>::load_frag(B + (brow0 + 16 * ni + r) * ldb + kk + kg);
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) ET<T>::mma(acc[mi][ni], a[mi], b[ni]);
+  }
+}
+
+// gemm: like gemm_nt, but either operand may be stored with the contraction index along the
+// rows of its tile (AT / BT = true):  AT = false: A[a0 + m][k]   AT = true: A[k][a0 + m]
+//                                     BT = false: B[b0 + n][k]   BT = true: B[k][b0 + n]
+template <typename T, int MB, int NB, bool AT, bool BT>
+__device__ __forceinline__ void gemm(f32x4 (&acc)[MB][NB], const T* A, int lda, int a0,
+                                     const T* B, int ldb, int b0, int k0, int k1) {
+  const int l = lane_id();
+  const int r = l & 15, kg = (l >> 4) * 8;
+  for (int kk = k0; kk < k1; kk += 32) {
+    typename ET<T>::frag a[MB], b[NB];
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi) {
+      if constexpr (AT) a[mi] = ET<T>::load_frag_t(A, lda, kk, a0 + 16 * mi);
+      else a[mi] = ET<T>::load_frag(A + (a0 + 16 * mi + r) * lda + kk + kg);
+    }
+#pragma unroll
+    for (int ni = 0; ni < NB; ++ni) {
+      if constexpr (BT) b[ni] = ET<T>::load_frag_t(B, ldb, kk, b0 + 16 * ni);
+      else b[ni] = ET<T>::load_frag(B + (b0 + 16 * ni + r) * ldb + kk + kg);
+    }
 #pragma unroll
     for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
@@ -129,6 +187,29 @@ __device__ __forceinline__ void acc_to_lds_t(const f32x4& a, T* tile, int ld, in
     *(bf16x4*)p = v;
   } else {
     *(f32x4*)p = a;
+  }
+}
+
+// Store the 16-row strip a wave holds in accumulators (NB*16 columns) to global memory with
+// 16-byte vector stores, through a wave-private LDS staging area stg[16][NB*16 + LPAD].
+// gdst points at row 0 / column 0 of the strip; rows >= nvalid are not written.  Only the
+// calling wave touches stg, so no work-group barrier is involved.
+template <typename T, int NB>
+__device__ __forceinline__ void store_strip(const f32x4 (&acc)[1][NB], T* stg, T* __restrict__ gdst,
+                                            int64_t row_stride, int nvalid, float mul) {
+  constexpr int W = NB * 16, LD = W + LPAD, VEC = ET<T>::VEC, VPR = W / VEC;
+  const int l = lane_id();
+#pragma unroll
+  for (int ni = 0; ni < NB; ++ni)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) stg[(4 * (l >> 4) + i) * LD + 16 * ni + (l & 15)] = ET<T>::from_f(acc[0][ni][i] * mul);
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+  for (int idx = l; idx < 16 * VPR; idx += 64) {
+    const int r = idx / VPR, c = (idx % VPR) * VEC;
+    if (r < nvalid) *(typename ET<T>::vec*)(gdst + (int64_t)r * row_stride + c) = *(const typename ET<T>::vec*)(stg + r * LD + c);
   }
 }
 
@@ -246,6 +327,15 @@ template <typename T, int ROWS, int COLS> struct TileIO {
 __device__ __forceinline__ float load_scalar(const void* p, int dtype, int64_t idx) {
   if (p == nullptr) return 0.f;
   return dtype == 1 ? ((const float*)p)[idx] : (float)((const bf16*)p)[idx];
+}
+
+// Two-step variant for prefetching: fetch the raw bits now, convert when the value is used, so
+// that no wait on the load is placed right behind the issue of a batch of prefetches.
+__device__ __forceinline__ uint32_t load_scalar_raw(const void* p, int dtype, int64_t idx) {
+  return dtype == 1 ? ((const uint32_t*)p)[idx] : (uint32_t)((const uint16_t*)p)[idx];
+}
+__device__ __forceinline__ float scalar_from_raw(uint32_t raw, int dtype) {
+  return __uint_as_float(dtype == 1 ? raw : raw << 16);
 }
 
 // inclusive prefix sum across the 64 lanes of a wavefront

@@ -125,75 +125,95 @@ __global__ __launch_bounds__(NTHR) void k_state_fwd(const lmoe_args a) {
 }
 
 // ------------------------------------------------------------------------- //
-// output (forward), chunk-parallel
-//   grid = (NT, H, V / BV), block = 256; wave w owns chunk rows 16w .. 16w+15
+// output (forward), chunk-parallel, persistent
+//   grid = min(NT*H, 2 per CU), block = 256; one work item = one (chunk, head), full V;
+//   wave w owns chunk rows 16w .. 16w+15.
+//   The tiles of the next item are fetched into registers while the current one is computed
+//   (barriers order LDS traffic only, so the loads stay in flight).
+//   LDS: q, k, S stored as loaded; P^T overlays k once q k^T is done, v' overlays S once q S is
+//   done; products that contract over tile rows use transposed fragments.
 // ------------------------------------------------------------------------- //
-template <typename T, int K, int V, int BV, bool GDN>
-__global__ __launch_bounds__(NTHR) void k_out_fwd(const lmoe_args a) {
-  constexpr int LDK = K + LPAD, LDC = CH + LPAD;
-  constexpr int NB = BV / 16;
-  __shared__ __attribute__((aligned(16))) T s_q[CH * LDK];
-  __shared__ __attribute__((aligned(16))) T s_k[CH * LDK];
-  __shared__ __attribute__((aligned(16))) T s_vT[BV * LDC];
-  __shared__ __attribute__((aligned(16))) T s_hT[BV * LDK];
-  __shared__ __attribute__((aligned(16))) T s_P[CH * LDC];
+template <typename T, int K, int V, bool GDN>
+__global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_out_fwd(const lmoe_args a) {
+  constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDV = V + LPAD;
+  constexpr int NB = V / 16;
+  constexpr int H_EL = K * LDV > CH * LDV ? K * LDV : CH * LDV;
+  constexpr int Q_EL = CH * LDK > 4 * 16 * LDV ? CH * LDK : 4 * 16 * LDV;   // also the store staging area
+  __shared__ __attribute__((aligned(16))) T s_q[Q_EL];
+  __shared__ __attribute__((aligned(16))) T s_k[CH * LDK];      // later: P^T [64][LDC]
+  __shared__ __attribute__((aligned(16))) T s_h[H_EL];          // later: v' [64][LDV]
   __shared__ float s_b[64], s_eb[64];
+  static_assert(CH * LDC <= CH * LDK, "P^T must fit into the k tile");
+  T* s_PT = s_k;
+  T* s_v = s_h;
 
-  const int cid = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * BV;
-  const ChunkInfo ci = chunk_info(a, cid);
   const int wv = wave_id(), l = lane_id();
-  chunk_gate_cumsum(a, ci.b, ci.tok, ci.len, h, s_b, s_eb, nullptr);
-
   typedef TileIO<T, CH, K> IOK;
-  typedef TileIO<T, CH, BV> IOV;
-  typedef TileIO<T, K, BV> IOH;
-  {
-    typename IOK::Regs rq, rk;
+  typedef TileIO<T, CH, V> IOV;
+  typedef TileIO<T, K, V> IOH;
+  const lmoe_tensor& vs = GDN ? a.vnew : a.v;
+  const int nitems = a.NT * a.H;
+  typename IOK::Regs rq, rk;
+  typename IOV::Regs rv;
+  typename IOH::Regs rh;
+  uint32_t graw = 0;
+  auto issue = [&](int it) {
+    const int cid = it / a.H, h = it % a.H;
+    const ChunkInfo ci = chunk_info(a, cid);
     IOK::load(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
     IOK::load(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
-    const lmoe_tensor& vs = GDN ? a.vnew : a.v;
-    typename IOV::Regs rv;
-    IOV::load(rv, row_ptr<T>(vs, ci.b, ci.tok, h) + v0, vs.st, ci.len);
-    typename IOH::Regs rh;
-    IOH::load(rh, (const T*)a.hs + ((int64_t)cid * a.H + h) * K * V + v0, V, K);
+    IOH::load(rh, (const T*)a.hs + ((int64_t)cid * a.H + h) * K * V, V, K);
+    graw = gate_prefetch(a, ci.b, ci.tok, ci.len, h);
+  };
+  auto issue_v = [&](int it) {
+    const int cid = it / a.H, h = it % a.H;
+    const ChunkInfo ci = chunk_info(a, cid);
+    IOV::load(rv, row_ptr<T>(vs, ci.b, ci.tok, h), vs.st, ci.len);
+  };
+  int it = blockIdx.x;
+  if (it < nitems) { issue(it); issue_v(it); }
+  for (; it < nitems; it += gridDim.x) {
+    const int cid = it / a.H, h = it % a.H;
+    const ChunkInfo ci = chunk_info(a, cid);
+    const int nxt = it + gridDim.x;
+    gate_finish(a, graw, s_b, s_eb, nullptr);
     IOK::store_lds(rq, s_q, LDK);
     IOK::store_lds(rk, s_k, LDK);
-    IOV::store_lds_t(rv, s_vT, LDC, nullptr);
-    IOH::store_lds_t(rh, s_hT, LDK, nullptr);
-  }
-  __syncthreads();
-  {
+    IOH::store_lds(rh, s_h, LDV);
+    lds_barrier();
+    if (nxt < nitems) issue(nxt);
     f32x4 s[1][4];
     acc_zero(s);
-    gemm_nt<T, 1, 4>(s, s_q, LDK, 16 * wv, s_k, LDK, 0, 0, K);
+    gemm<T, 1, 4, false, false>(s, s_q, LDK, 16 * wv, s_k, LDK, 0, 0, K);
+    f32x4 o[1][NB];
+    acc_zero(o);
+    gemm<T, 1, NB, false, true>(o, s_q, LDK, 16 * wv, s_h, LDV, 0, 0, K);
+    lds_barrier();            // every wave is done reading k and S: P^T and v' may overlay them
+    IOV::store_lds(rv, s_v, LDV);
+    if (nxt < nitems) issue_v(nxt);
 #pragma unroll
     for (int nj = 0; nj < 4; ++nj) {
       f32x4 p;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * nj + (l & 15);
-        p[i] = (r >= cc) ? s[0][nj][i] * expf(s_b[r] - s_b[cc]) : 0.f;
+        p[i] = (r >= cc) ? s[0][nj][i] * texp<T>(s_b[r] - s_b[cc]) : 0.f;
       }
-      acc_to_lds<T>(p, s_P, LDC, 16 * wv, 16 * nj);
+      acc_to_lds_t<T>(p, s_PT, LDC, 16 * wv, 16 * nj);     // s_PT[j][i]
     }
+#pragma unroll
+    for (int ni = 0; ni < NB; ++ni)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[0][ni][i] *= s_eb[16 * wv + 4 * (l >> 4) + i];
+    lds_barrier();
+    // o += P v' : A = P^T stored [j][i] (contraction j along rows), B = v' stored [j][v]
+    gemm<T, 1, NB, true, true>(o, s_PT, LDC, 16 * wv, s_v, LDV, 0, 0, CH);
+    // stage through a wave-private slice of the q tile: q was last read before the second
+    // barrier of this iteration (as the A operand of the first two products)
+    store_strip<T, NB>(o, s_q + wv * 16 * LDV, row_ptr<T>(a.o, ci.b, ci.tok + 16 * wv, h), a.o.st,
+                       ci.len - 16 * wv, a.scale);
+    lds_barrier();
   }
-  __syncthreads();
-  f32x4 o[1][NB];
-  acc_zero(o);
-  gemm_nt<T, 1, NB>(o, s_q, LDK, 16 * wv, s_hT, LDK, 0, 0, K);
-#pragma unroll
-  for (int ni = 0; ni < NB; ++ni)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) o[0][ni][i] *= s_eb[16 * wv + 4 * (l >> 4) + i];
-  gemm_nt<T, 1, NB>(o, s_P, LDC, 16 * wv, s_vT, LDC, 0, 0, CH);
-  T* od = row_ptr<T>(a.o, ci.b, ci.tok, h) + v0;
-#pragma unroll
-  for (int ni = 0; ni < NB; ++ni)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
-      if (r < ci.len) od[(int64_t)r * a.o.st + cc] = ET<T>::from_f(o[0][ni][i] * a.scale);
-    }
 }
 
 }  // namespace lmoe

@@ -87,4 +87,36 @@ __device__ __forceinline__ void chunk_gate_cumsum(const lmoe_args& a, int b, int
   __syncthreads();
 }
 
+// Split form of chunk_gate_cumsum for software-pipelined kernels: gate_prefetch issues the loads
+// of a chunk's log-decays (lanes 0..63 of wave 0 hold one token each, raw bits), gate_finish
+// turns them into the LDS arrays later.  Neither contains a barrier.
+__device__ __forceinline__ uint32_t gate_prefetch(const lmoe_args& a, int b, int tok, int len, int h) {
+  uint32_t raw = 0;
+  if (threadIdx.x < 64 && a.gate != LMOE_GATE_NONE && a.g.ptr != nullptr && (int)threadIdx.x < len)
+    raw = load_scalar_raw(a.g.ptr, a.g_dtype, row_off(a.g, b, tok + threadIdx.x, h));
+  return raw;
+}
+__device__ __forceinline__ void gate_finish(const lmoe_args& a, uint32_t raw, float* sb, float* seb, float* sed) {
+  if (threadIdx.x < 64) {
+    const int j = threadIdx.x;
+    const float x = wave_incl_scan(scalar_from_raw(raw, a.g_dtype));
+    const float xl = __shfl(x, 63, 64);
+    if (sb) sb[j] = x;
+    if (seb) seb[j] = expf(x);
+    if (sed) sed[j] = expf(xl - x);
+  }
+}
+
+// number of work-groups of a persistent chunk-parallel kernel: `per_cu` per compute unit
+inline int persistent_grid(int nitems, int per_cu) {
+  static int ncu = 0;
+  if (ncu == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    ncu = n;
+  }
+  const int g = ncu * per_cu;
+  return nitems < g ? nitems : g;
+}
+
 }  // namespace lmoe
