@@ -5,7 +5,7 @@
 namespace lmoe {
 
 template <typename T, int V> struct BwdTiles {
-  static constexpr int BVS = 32;                                      // V-slice of the sequential pass
+  static constexpr int BVS = sizeof(T) == 4 ? 16 : 32;                // V-slice of the sequential pass
   static constexpr int BVD = (sizeof(T) == 4 && V == 128) ? 64 : V;   // V-slice of k_bwd_dv
   static constexpr int BVH = sizeof(T) == 4 ? 32 : 64;                // V-slice loop of k_bwd_dqk
 };
@@ -22,7 +22,8 @@ template <bool GDN> struct StateBwd {
   template <typename T, int K, int V> struct F {
     static void run(const lmoe_args& a, hipStream_t st) {
       constexpr int BV = BwdTiles<T, V>::BVS;
-      hipLaunchKernelGGL((k_state_bwd<T, K, V, BV, GDN>), dim3(V / BV, a.H, a.N), dim3(NTHR), 0, st, a);
+      const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BV);
+      hipLaunchKernelGGL((k_state_bwd<T, K, V, BV, GDN>), dim3(grid), dim3(NTHR), 0, st, a);
     }
   };
 };

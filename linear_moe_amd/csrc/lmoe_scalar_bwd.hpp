@@ -18,54 +18,53 @@ namespace lmoe {
 
 // ------------------------------------------------------------------------- //
 // dv' = scale P^T do + (k . e_d) dS'        grid = (NT, H, V / BV)
+// (dhs holds dS'^T: [V][K])
 // ------------------------------------------------------------------------- //
 template <typename T, int K, int V, int BV, bool LOCAL>
 __global__ __launch_bounds__(NTHR) void k_bwd_dv(const lmoe_args a) {
-  constexpr int LDK = K + LPAD, LDC = CH + LPAD;
+  constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDV = BV + LPAD;
   constexpr int NB = BV / 16;
   __shared__ __attribute__((aligned(16))) T s_q[CH * LDK];
   __shared__ __attribute__((aligned(16))) T s_k[CH * LDK];
-  __shared__ __attribute__((aligned(16))) T s_doT[BV * LDC];
+  __shared__ __attribute__((aligned(16))) T s_do[CH * LDV];
   __shared__ __attribute__((aligned(16))) T s_dhT[LOCAL ? 8 : BV * LDK];
   __shared__ __attribute__((aligned(16))) T s_PT[CH * LDC];
+  __shared__ __attribute__((aligned(16))) T s_stg[4 * 16 * LDV];
   __shared__ float s_b[64], s_ed[64];
 
   const int cid = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * BV;
   const ChunkInfo ci = chunk_info(a, cid);
   const int wv = wave_id(), l = lane_id();
-  chunk_gate_cumsum(a, ci.b, ci.tok, ci.len, h, s_b, nullptr, s_ed);
-
   typedef TileIO<T, CH, K> IOK;
   typedef TileIO<T, CH, BV> IOV;
-  typedef TileIO<T, K, BV> IOH;
+  typedef TileIO<T, BV, K> IOH;
   {
     typename IOK::Regs rq, rk;
     IOK::load(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
     IOK::load(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
     typename IOV::Regs rd;
     IOV::load(rd, row_ptr<T>(a.d_o, ci.b, ci.tok, h) + v0, a.d_o.st, ci.len);
+    typename IOH::Regs rh;
+    if constexpr (!LOCAL) IOH::load(rh, (const T*)a.dhs + (((int64_t)cid * a.H + h) * V + v0) * K, K, BV);
+    chunk_gate_cumsum(a, ci.b, ci.tok, ci.len, h, s_b, nullptr, s_ed);
     IOK::store_lds(rq, s_q, LDK);
     IOK::store_lds(rk, s_k, LDK);
-    IOV::store_lds_t(rd, s_doT, LDC, nullptr);
-    if constexpr (!LOCAL) {
-      typename IOH::Regs rh;
-      IOH::load(rh, (const T*)a.dhs + ((int64_t)cid * a.H + h) * K * V + v0, V, K);
-      IOH::store_lds_t(rh, s_dhT, LDK, nullptr);
-    }
+    IOV::store_lds(rd, s_do, LDV);
+    if constexpr (!LOCAL) IOH::store_lds(rh, s_dhT, LDK);
   }
   __syncthreads();
   {
     // P^T stored as s_PT[j][i]; wave w computes rows i = 16w.. of P and writes them transposed
     f32x4 s[1][4];
     acc_zero(s);
-    gemm_nt<T, 1, 4>(s, s_q, LDK, 16 * wv, s_k, LDK, 0, 0, K);
+    gemm<T, 1, 4, false, false>(s, s_q, LDK, 16 * wv, s_k, LDK, 0, 0, K);
 #pragma unroll
     for (int nj = 0; nj < 4; ++nj) {
       f32x4 p;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * nj + (l & 15);
-        p[i] = (r >= cc) ? s[0][nj][i] * expf(s_b[r] - s_b[cc]) : 0.f;
+        p[i] = (r >= cc) ? s[0][nj][i] * texp<T>(s_b[r] - s_b[cc]) : 0.f;
       }
       acc_to_lds_t<T>(p, s_PT, LDC, 16 * wv, 16 * nj);
     }
@@ -73,46 +72,51 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dv(const lmoe_args a) {
   __syncthreads();
   f32x4 dv[1][NB];
   acc_zero(dv);
-  gemm_nt<T, 1, NB>(dv, s_PT, LDC, 16 * wv, s_doT, LDC, 0, 0, CH);
+  gemm<T, 1, NB, false, true>(dv, s_PT, LDC, 16 * wv, s_do, LDV, 0, 0, CH);
 #pragma unroll
   for (int ni = 0; ni < NB; ++ni) dv[0][ni] *= a.scale;
   if constexpr (!LOCAL) {
     f32x4 t[1][NB];
     acc_zero(t);
-    gemm_nt<T, 1, NB>(t, s_k, LDK, 16 * wv, s_dhT, LDK, 0, 0, K);
+    gemm<T, 1, NB, false, false>(t, s_k, LDK, 16 * wv, s_dhT, LDK, 0, 0, K);
 #pragma unroll
     for (int ni = 0; ni < NB; ++ni)
 #pragma unroll
       for (int i = 0; i < 4; ++i) dv[0][ni][i] += t[0][ni][i] * s_ed[16 * wv + 4 * (l >> 4) + i];
   }
   const lmoe_tensor& dst = LOCAL ? a.dvnew : a.dv;
-  T* dd = row_ptr<T>(dst, ci.b, ci.tok, h) + v0;
-#pragma unroll
-  for (int ni = 0; ni < NB; ++ni)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
-      if (r < ci.len) dd[(int64_t)r * dst.st + cc] = ET<T>::from_f(dv[0][ni][i]);
-    }
+  store_strip<T, NB>(dv, s_stg + wv * 16 * LDV, row_ptr<T>(dst, ci.b, ci.tok + 16 * wv, h) + v0, dst.st,
+                     ci.len - 16 * wv, 1.0f);
 }
 
 // ------------------------------------------------------------------------- //
-// reverse state pass        grid = (V / BV, H, N)
+// reverse state pass, software-pipelined (mirror of k_state_fwd)
+//   grid = ceil(N*H / 8) * 8 * (V / BV) work-groups (1-D); V-slices of one (sequence, head)
+//   share an XCD.  dS slice [K x BV] lives in fp32 MFMA accumulators.
+//   Chain per chunk:  dS' -> LDS | barrier | dv_new = dv_loc + (k e_d) dS' -> LDS | barrier |
+//                     dS = e^{b_C} dS' + (scale q e_b)^T do - w^T dv_new.
+//   dhs (layout [V][K]) and dv_new leave through LDS with 16-byte stores; the operands of the
+//   next chunk are prefetched into registers and staged into the other LDS buffer.
 // ------------------------------------------------------------------------- //
 template <typename T, int K, int V, int BV, bool GDN>
 __global__ __launch_bounds__(NTHR) void k_state_bwd(const lmoe_args a) {
   constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDU = BV + LPAD;
   constexpr int MB = K / 64, NB = BV / 16;
-  __shared__ __attribute__((aligned(16))) T s_qT[K * LDC];             // (scale q e_b)^T  [K][64]
-  __shared__ __attribute__((aligned(16))) T s_doT[BV * LDC];           // do^T             [BV][64]
-  __shared__ __attribute__((aligned(16))) T s_kd[GDN ? CH * LDK : 8];  // k e_d            [64][K]
-  __shared__ __attribute__((aligned(16))) T s_wT[GDN ? K * LDC : 8];   // w^T              [K][64]
-  __shared__ __attribute__((aligned(16))) T s_dvl[GDN ? CH * LDU : 8]; // dv_loc           [64][BV]
-  __shared__ __attribute__((aligned(16))) T s_dST[GDN ? BV * LDK : 8]; // dS'^T            [BV][K]
-  __shared__ __attribute__((aligned(16))) T s_dvT[GDN ? BV * LDC : 8]; // -dv_new^T        [BV][64]
-  __shared__ float s_b[64], s_eb[64], s_ed[64], s_qs[64];
+  constexpr int NBUF = sizeof(T) == 2 ? 2 : 1;
+  __shared__ __attribute__((aligned(16))) T s_qs[NBUF][CH * LDK];            // scale q e_b    [64][K]
+  __shared__ __attribute__((aligned(16))) T s_do[NBUF][CH * LDU];            // do             [64][BV]
+  __shared__ __attribute__((aligned(16))) T s_kd[NBUF][GDN ? CH * LDK : 8];  // k e_d          [64][K]
+  __shared__ __attribute__((aligned(16))) T s_w[NBUF][GDN ? CH * LDK : 8];   // w              [64][K]
+  __shared__ __attribute__((aligned(16))) T s_dvl[NBUF][GDN ? CH * LDU : 8]; // dv_loc         [64][BV]
+  __shared__ __attribute__((aligned(16))) T s_dST[BV * LDK];                 // dS'^T          [BV][K]
+  __shared__ __attribute__((aligned(16))) T s_dvT[GDN ? BV * LDC : 8];       // -dv_new^T      [BV][64]
+  __shared__ __attribute__((aligned(16))) T s_stg[GDN ? 4 * 16 * LDU : 8];
 
-  const int v0 = blockIdx.x * BV, h = blockIdx.y, n = blockIdx.z;
+  constexpr int NVS = V / BV;
+  const int xcd = blockIdx.x & 7, jj = blockIdx.x >> 3;
+  const int vsl = jj % NVS, pair = (jj / NVS) * 8 + xcd;
+  if (pair >= a.N * a.H) return;
+  const int v0 = vsl * BV, h = pair % a.H, n = pair / a.H;
   const SeqInfo sq = seq_info(a, n);
   const int wv = wave_id(), l = lane_id();
   const int krow0 = wv * (K / 4);
@@ -131,73 +135,103 @@ __global__ __launch_bounds__(NTHR) void k_state_bwd(const lmoe_args a) {
   }
   typedef TileIO<T, CH, K> IOK;
   typedef TileIO<T, CH, BV> IOV;
+  typedef TileIO<T, BV, K> IOHT;
+  typename IOK::Regs rq, rk, rw;
+  typename IOV::Regs rd, rl;
+  uint32_t graw = 0;
+  const bool gated = a.gate != LMOE_GATE_NONE && a.g.ptr != nullptr;
+  const float scale = a.scale;
 
-  for (int c = sq.nchunks - 1; c >= 0; --c) {
+  auto issue = [&](int c) {
     const int tok = sq.tok0 + c * CH;
     const int len = min(CH, sq.len - c * CH);
-    chunk_gate_cumsum(a, sq.b, tok, len, h, s_b, s_eb, s_ed);
-    if (threadIdx.x < 64) s_qs[threadIdx.x] = a.scale * s_eb[threadIdx.x];
-    __syncthreads();
-    {
-      typename IOK::Regs rq;
-      IOK::load(rq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, len);
-      IOK::store_lds_t(rq, s_qT, LDC, s_qs);
-      typename IOV::Regs rd;
-      IOV::load(rd, row_ptr<T>(a.d_o, sq.b, tok, h) + v0, a.d_o.st, len);
-      IOV::store_lds_t(rd, s_doT, LDC, nullptr);
+    IOK::load(rq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, len);
+    IOV::load(rd, row_ptr<T>(a.d_o, sq.b, tok, h) + v0, a.d_o.st, len);
+    if constexpr (GDN) {
+      IOK::load(rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, len);
+      IOK::load(rw, row_ptr<T>(a.w, sq.b, tok, h), a.w.st, len);
+      IOV::load(rl, row_ptr<T>(a.dvnew, sq.b, tok, h) + v0, a.dvnew.st, len);
+    }
+    graw = 0;
+    if (gated && l < len) graw = load_scalar_raw(a.g.ptr, a.g_dtype, row_off(a.g, sq.b, tok + l, h));
+  };
+  auto stage = [&](int buf) -> float {
+    const float x = wave_incl_scan(scalar_from_raw(graw, a.g_dtype));
+    const float xl = __shfl(x, 63, 64);
+    const float qs = scale * expf(x);                     // lane j: scale e^{b_j}
+    const float ed = expf(xl - x);                        // lane j: e^{b_C - b_j}
+#pragma unroll
+    for (int p = 0; p < IOK::PASSES; ++p) {
+      int row, col; IOK::coords(p, row, col);
+      const float sq_ = __shfl(qs, row, 64);
+      typename IOK::vec o;
+#pragma unroll
+      for (int i = 0; i < IOK::VEC; ++i) o[i] = ET<T>::from_f(ET<T>::to_f(rq.v[p][i]) * sq_);
+      *(typename IOK::vec*)(&s_qs[buf][row * LDK + col]) = o;
       if constexpr (GDN) {
-        typename IOK::Regs rk, rw;
-        IOK::load(rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, len);
-        IOK::store_lds_scaled(rk, s_kd, LDK, s_ed);
-        IOK::load(rw, row_ptr<T>(a.w, sq.b, tok, h), a.w.st, len);
-        IOK::store_lds_t(rw, s_wT, LDC, nullptr);
-        typename IOV::Regs rl;
-        IOV::load(rl, row_ptr<T>(a.dvnew, sq.b, tok, h) + v0, a.dvnew.st, len);
-        IOV::store_lds(rl, s_dvl, LDU);
+        const float se = __shfl(ed, row, 64);
+#pragma unroll
+        for (int i = 0; i < IOK::VEC; ++i) o[i] = ET<T>::from_f(ET<T>::to_f(rk.v[p][i]) * se);
+        *(typename IOK::vec*)(&s_kd[buf][row * LDK + col]) = o;
       }
     }
-    {
-      T* dhs = (T*)a.dhs + ((int64_t)(sq.chunk0 + c) * a.H + h) * K * V;
-#pragma unroll
-      for (int mi = 0; mi < MB; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < NB; ++ni) {
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-            dhs[(int64_t)(krow0 + acc_row(mi, i)) * V + v0 + acc_col(ni)] = ET<T>::from_f(dS[mi][ni][i]);
-          if constexpr (GDN) acc_to_lds_t<T>(dS[mi][ni], s_dST, LDK, krow0 + 16 * mi, 16 * ni);
-        }
+    IOV::store_lds(rd, s_do[buf], LDU);
+    if constexpr (GDN) {
+      IOK::store_lds(rw, s_w[buf], LDK);
+      IOV::store_lds(rl, s_dvl[buf], LDU);
     }
-    __syncthreads();
+    return expf(xl);
+  };
+
+  float dec_cur = 1.f;
+  if (sq.nchunks > 0) {
+    issue(sq.nchunks - 1);
+    dec_cur = stage(0);
+    if (sq.nchunks > 1) issue(sq.nchunks - 2);
+  }
+  for (int c = sq.nchunks - 1, it = 0; c >= 0; --c, ++it) {
+    const int cur = NBUF == 2 ? (it & 1) : 0;
+    const int tok = sq.tok0 + c * CH;
+    const int len = min(CH, sq.len - c * CH);
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) acc_to_lds_t<T>(dS[mi][ni], s_dST, LDK, krow0 + 16 * mi, 16 * ni);
+    lds_barrier();
+    IOHT::lds_to_global(s_dST, LDK, (T*)a.dhs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
+    f32x4 t[1][NB];
+    acc_zero(t);
     if constexpr (GDN) {
       // dv_new = dv_loc + k_d dS'   (rows 16 wv .. of the chunk)
-      f32x4 t[1][NB];
-      acc_zero(t);
-      gemm_nt<T, 1, NB>(t, s_kd, LDK, 16 * wv, s_dST, LDK, 0, 0, K);
-      T* vd = row_ptr<T>(a.dvnew, sq.b, tok, h) + v0;
+      gemm<T, 1, NB, false, false>(t, s_kd[cur], LDK, 16 * wv, s_dST, LDK, 0, 0, K);
 #pragma unroll
       for (int ni = 0; ni < NB; ++ni) {
         f32x4 x;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
-          float y = ET<T>::to_f(s_dvl[r * LDU + cc]) + t[0][ni][i];
-          y = ET<T>::to_f(ET<T>::from_f(y));
-          if (r < len) vd[(int64_t)r * a.dvnew.st + cc] = ET<T>::from_f(y);
-          x[i] = -y;
+          t[0][ni][i] = ET<T>::to_f(ET<T>::from_f(ET<T>::to_f(s_dvl[cur][r * LDU + cc]) + t[0][ni][i]));
+          x[i] = -t[0][ni][i];
         }
         acc_to_lds_t<T>(x, s_dvT, LDC, 16 * wv, 16 * ni);
       }
-      __syncthreads();
+      lds_barrier();
     }
-    const float dec = expf(s_b[63]);
 #pragma unroll
     for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
-      for (int ni = 0; ni < NB; ++ni) dS[mi][ni] *= dec;
-    gemm_nt<T, MB, NB>(dS, s_qT, LDC, krow0, s_doT, LDC, 0, 0, CH);
-    if constexpr (GDN) gemm_nt<T, MB, NB>(dS, s_wT, LDC, krow0, s_dvT, LDC, 0, 0, CH);
-    __syncthreads();
+      for (int ni = 0; ni < NB; ++ni) dS[mi][ni] *= dec_cur;
+    gemm<T, MB, NB, true, true>(dS, s_qs[cur], LDK, krow0, s_do[cur], LDU, 0, 0, CH);
+    if constexpr (GDN) {
+      gemm<T, MB, NB, true, false>(dS, s_w[cur], LDK, krow0, s_dvT, LDC, 0, 0, CH);
+      store_strip<T, NB>(t, s_stg + wv * 16 * LDU, row_ptr<T>(a.dvnew, sq.b, tok + 16 * wv, h) + v0, a.dvnew.st,
+                         len - 16 * wv, 1.0f);
+    }
+    if (c > 0) {
+      if constexpr (NBUF == 1) lds_barrier();
+      dec_cur = stage(NBUF == 2 ? (cur ^ 1) : 0);
+      if (c > 1) issue(c - 2);
+    }
   }
   if (a.dh0) {
     float* p = a.dh0 + ((int64_t)n * a.H + h) * K * V;
@@ -215,18 +249,19 @@ __global__ __launch_bounds__(NTHR) void k_state_bwd(const lmoe_args a) {
 // dq, dk, gate gradient        grid = (NT, H)
 //   phase A: loop over V-slices of width BVH accumulating
 //              dP = do v'^T, dq_i = do S^T, dk_d = v' dS'^T (, dw = dv_new S^T)
+//            (hs, dhs hold S^T, dS'^T: [V][K]; the slice tiles are [BVH][K])
 //   phase B: dq = scale e_b dq_i + (scale dP . Gamma) k ; dk = e_d dk_d + (scale dP . Gamma)^T q
+//            with one LDS copy of (scale dP . Gamma)^T and q, k stored as loaded
 // ------------------------------------------------------------------------- //
 template <typename T, int K, int V, int BVH, bool GDN>
 __global__ __launch_bounds__(NTHR) void k_bwd_dqk(const lmoe_args a) {
-  constexpr int LDV = BVH + LPAD, LDC = CH + LPAD;
+  constexpr int LDV = BVH + LPAD, LDC = CH + LPAD, LDK = K + LPAD;
   constexpr int NBK = K / 16;
   // phase A tiles
-  constexpr int A_DO = 0, A_V = A_DO + CH * LDV, A_H = A_V + CH * LDV, A_DH = A_H + K * LDV,
-                A_DVN = A_DH + K * LDV, A_END = A_DVN + (GDN ? CH * LDV : 0);
+  constexpr int A_DO = 0, A_V = A_DO + CH * LDV, A_H = A_V + CH * LDV, A_DH = A_H + BVH * LDK,
+                A_DVN = A_DH + BVH * LDK, A_END = A_DVN + (GDN ? CH * LDV : 0);
   // phase B tiles
-  constexpr int B_DP = 0, B_DPT = B_DP + CH * LDC, B_KT = B_DPT + CH * LDC, B_QT = B_KT + K * LDC,
-                B_END = B_QT + K * LDC;
+  constexpr int B_DPT = 0, B_K = B_DPT + CH * LDC, B_Q = B_K + CH * LDK, B_END = B_Q + CH * LDK;
   constexpr int NELEM = A_END > B_END ? A_END : B_END;
   __shared__ __attribute__((aligned(16))) T smem[NELEM];
   __shared__ float s_b[64], s_eb[64], s_ed[64], s_db[64], s_red[8];
@@ -237,7 +272,7 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dqk(const lmoe_args a) {
   chunk_gate_cumsum(a, ci.b, ci.tok, ci.len, h, s_b, s_eb, s_ed);
 
   typedef TileIO<T, CH, BVH> IOV;
-  typedef TileIO<T, K, BVH> IOH;
+  typedef TileIO<T, BVH, K> IOH;
   typedef TileIO<T, CH, K> IOK;
   const lmoe_tensor& vs = GDN ? a.vnew : a.v;
 
@@ -250,16 +285,16 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dqk(const lmoe_args a) {
       IOV::load(rd, row_ptr<T>(a.d_o, ci.b, ci.tok, h) + vv, a.d_o.st, ci.len);
       IOV::load(rv, row_ptr<T>(vs, ci.b, ci.tok, h) + vv, vs.st, ci.len);
       typename IOH::Regs rh, rdh;
-      IOH::load(rh, (const T*)a.hs + ((int64_t)cid * a.H + h) * K * V + vv, V, K);
-      IOH::load(rdh, (const T*)a.dhs + ((int64_t)cid * a.H + h) * K * V + vv, V, K);
+      IOH::load(rh, (const T*)a.hs + (((int64_t)cid * a.H + h) * V + vv) * K, K, BVH);
+      IOH::load(rdh, (const T*)a.dhs + (((int64_t)cid * a.H + h) * V + vv) * K, K, BVH);
 #pragma unroll
       for (int p = 0; p < IOH::PASSES; ++p)
 #pragma unroll
         for (int i = 0; i < IOH::VEC; ++i) hdh += ET<T>::to_f(rh.v[p][i]) * ET<T>::to_f(rdh.v[p][i]);
       IOV::store_lds(rd, smem + A_DO, LDV);
       IOV::store_lds(rv, smem + A_V, LDV);
-      IOH::store_lds(rh, smem + A_H, LDV);
-      IOH::store_lds(rdh, smem + A_DH, LDV);
+      IOH::store_lds(rh, smem + A_H, LDK);
+      IOH::store_lds(rdh, smem + A_DH, LDK);
       if constexpr (GDN) {
         typename IOV::Regs rn;
         IOV::load(rn, row_ptr<T>(a.dvnew, ci.b, ci.tok, h) + vv, a.dvnew.st, ci.len);
@@ -267,10 +302,10 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dqk(const lmoe_args a) {
       }
     }
     __syncthreads();
-    gemm_nt<T, 1, 4>(dP, smem + A_DO, LDV, 16 * wv, smem + A_V, LDV, 0, 0, BVH);
-    gemm_nt<T, 1, NBK>(dqi, smem + A_DO, LDV, 16 * wv, smem + A_H, LDV, 0, 0, BVH);
-    gemm_nt<T, 1, NBK>(dkd, smem + A_V, LDV, 16 * wv, smem + A_DH, LDV, 0, 0, BVH);
-    if constexpr (GDN) gemm_nt<T, 1, NBK>(dw, smem + A_DVN, LDV, 16 * wv, smem + A_H, LDV, 0, 0, BVH);
+    gemm<T, 1, 4, false, false>(dP, smem + A_DO, LDV, 16 * wv, smem + A_V, LDV, 0, 0, BVH);
+    gemm<T, 1, NBK, false, true>(dqi, smem + A_DO, LDV, 16 * wv, smem + A_H, LDK, 0, 0, BVH);
+    gemm<T, 1, NBK, false, true>(dkd, smem + A_V, LDV, 16 * wv, smem + A_DH, LDK, 0, 0, BVH);
+    if constexpr (GDN) gemm<T, 1, NBK, false, true>(dw, smem + A_DVN, LDV, 16 * wv, smem + A_H, LDK, 0, 0, BVH);
     __syncthreads();
   }
   // block reduction of <S, dS'>
@@ -284,45 +319,40 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dqk(const lmoe_args a) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * nj + (l & 15);
-        p[i] = (r >= cc) ? a.scale * dP[0][nj][i] * expf(s_b[r] - s_b[cc]) : 0.f;
+        p[i] = (r >= cc) ? a.scale * dP[0][nj][i] * texp<T>(s_b[r] - s_b[cc]) : 0.f;
       }
-      acc_to_lds<T>(p, smem + B_DP, LDC, 16 * wv, 16 * nj);
-      acc_to_lds_t<T>(p, smem + B_DPT, LDC, 16 * wv, 16 * nj);
+      acc_to_lds_t<T>(p, smem + B_DPT, LDC, 16 * wv, 16 * nj);      // [j][i]
     }
     typename IOK::Regs rq, rk;
     IOK::load(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
     IOK::load(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
-    IOK::store_lds_t(rq, smem + B_QT, LDC, nullptr);
-    IOK::store_lds_t(rk, smem + B_KT, LDC, nullptr);
+    IOK::store_lds(rq, smem + B_Q, LDK);
+    IOK::store_lds(rk, smem + B_K, LDK);
   }
   __syncthreads();
   f32x4 dq[1][NBK], dk[1][NBK];
   acc_zero(dq); acc_zero(dk);
-  gemm_nt<T, 1, NBK>(dq, smem + B_DP, LDC, 16 * wv, smem + B_KT, LDC, 0, 0, CH);
-  gemm_nt<T, 1, NBK>(dk, smem + B_DPT, LDC, 16 * wv, smem + B_QT, LDC, 0, 0, CH);
-  // combine, store, and form db_i = q_i.dq_i - k_i.dk_i ; kk = sum_j (dk_d . k_d)_j
+  // dq_intra[i][c] = sum_j dPG[i][j] k[j][c] : A = dPG^T stored [j][i] (contraction along rows)
+  gemm<T, 1, NBK, true, true>(dq, smem + B_DPT, LDC, 16 * wv, smem + B_K, LDK, 0, 0, CH);
+  // dk_intra[j][c] = sum_i dPG[i][j] q[i][c] : A = dPG^T rows j (contraction along columns)
+  gemm<T, 1, NBK, false, true>(dk, smem + B_DPT, LDC, 16 * wv, smem + B_Q, LDK, 0, 0, CH);
+  // combine and form db_i = q_i.dq_i - k_i.dk_i ; kk = sum_j (dk_d . k_d)_j
   float dbp[4] = {0.f, 0.f, 0.f, 0.f};
   float kk = 0.f;
-  T* dqd = row_ptr<T>(a.dq, ci.b, ci.tok, h);
-  T* dkd_ = row_ptr<T>(a.dk, ci.b, ci.tok, h);
-  T* dwd = GDN ? row_ptr<T>(a.dw, ci.b, ci.tok, h) : nullptr;
 #pragma unroll
   for (int ni = 0; ni < NBK; ++ni)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
-      const float qv = ET<T>::to_f(smem[B_QT + cc * LDC + r]);
-      const float kv = ET<T>::to_f(smem[B_KT + cc * LDC + r]);
+      const float qv = ET<T>::to_f(smem[B_Q + r * LDK + cc]);
+      const float kv = ET<T>::to_f(smem[B_K + r * LDK + cc]);
       const float dqv = a.scale * s_eb[r] * dqi[0][ni][i] + dq[0][ni][i];
       const float dkdv = s_ed[r] * dkd[0][ni][i];
       const float dkv = dkdv + dk[0][ni][i];
       dbp[i] += qv * dqv - kv * dkv;
       kk += kv * dkdv;
-      if (r < ci.len) {
-        dqd[(int64_t)r * a.dq.st + cc] = ET<T>::from_f(dqv);
-        dkd_[(int64_t)r * a.dk.st + cc] = ET<T>::from_f(dkv);
-        if constexpr (GDN) dwd[(int64_t)r * a.dw.st + cc] = ET<T>::from_f(-dw[0][ni][i]);
-      }
+      dq[0][ni][i] = dqv;
+      dk[0][ni][i] = dkv;
     }
   // reduce db over the 16 lanes that share a row group, kk over the whole block
 #pragma unroll
@@ -336,7 +366,17 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dqk(const lmoe_args a) {
   }
   kk = wave_sum(kk);
   if (l == 0) s_red[4 + wv] = kk;
-  __syncthreads();
+  __syncthreads();     // q, k tiles are dead from here: wave-private slices become store staging
+  {
+    T* stg = smem + B_K + wv * 16 * LDK;    // this wave's 16 rows of the k tile, then of the q tile
+    store_strip<T, NBK>(dq, stg, row_ptr<T>(a.dq, ci.b, ci.tok + 16 * wv, h), a.dq.st, ci.len - 16 * wv, 1.0f);
+    T* stg2 = smem + B_Q + wv * 16 * LDK;
+    store_strip<T, NBK>(dk, stg2, row_ptr<T>(a.dk, ci.b, ci.tok + 16 * wv, h), a.dk.st, ci.len - 16 * wv, 1.0f);
+    if constexpr (GDN) {
+      // dw = -dv_new S^T ; staging reuses the first slice again (same wave, program order)
+      store_strip<T, NBK>(dw, stg, row_ptr<T>(a.dw, ci.b, ci.tok + 16 * wv, h), a.dw.st, ci.len - 16 * wv, -1.0f);
+    }
+  }
   if (threadIdx.x < 64) {
     const int j = threadIdx.x;
     float x = s_db[j];

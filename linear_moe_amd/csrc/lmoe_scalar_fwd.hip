@@ -14,7 +14,8 @@ template <bool GDN> struct StateFwd {
   template <typename T, int K, int V> struct F {
     static void run(const lmoe_args& a, hipStream_t st) {
       constexpr int BV = FwdTiles<T, V>::BVS;
-      hipLaunchKernelGGL((k_state_fwd<T, K, V, BV, GDN>), dim3(V / BV, a.H, a.N), dim3(NTHR), 0, st, a);
+      const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BV);
+      hipLaunchKernelGGL((k_state_fwd<T, K, V, BV, GDN>), dim3(grid), dim3(NTHR), 0, st, a);
     }
   };
 };

@@ -10,22 +10,35 @@
 namespace lmoe {
 
 // ------------------------------------------------------------------------- //
-// state pass (forward)
-//   grid = (V / BV, H, N), block = 256
-//   wave w owns state rows [w*K/4, (w+1)*K/4) x BV columns
+// state pass (forward), software-pipelined
+//   grid = ceil(N*H / 8) * 8 * (V / BV) work-groups (1-D), block = 256.
+//   Work-group -> (sequence, head, V-slice): the V-slices of one (sequence, head) get ids that
+//   are congruent mod 8, i.e. run on the same XCD and share k, w through its L2.
+//   wave w owns state rows [w*K/4, (w+1)*K/4) x BV columns (fp32 MFMA accumulators).
+//   Per chunk, on the dependency chain of S:   S -> LDS (element type T)  | barrier |
+//   v_new = u - w S -> LDS | barrier | S = e^{b_C} S + (k e_d)^T v_new.
+//   Off the chain: the operands of chunk c+1 sit in registers while chunk c is computed and go
+//   to the other LDS buffer at the end of the step, the loads of chunk c+2 are issued right
+//   after; hs (layout [V][K]) and v_new are written with 16-byte stores from LDS.
+//   Every wave forms the gate cumsum of a chunk for itself (lane j = token j).
 // ------------------------------------------------------------------------- //
 template <typename T, int K, int V, int BV, bool GDN>
 __global__ __launch_bounds__(NTHR) void k_state_fwd(const lmoe_args a) {
   constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDU = BV + LPAD;
   constexpr int MB = K / 64, NB = BV / 16;
-  __shared__ __attribute__((aligned(16))) T s_kT[K * LDC];            // (k e^{b_C-b})^T  [K][64]
-  __shared__ __attribute__((aligned(16))) T s_vT[BV * LDC];           // v'^T             [BV][64]
-  __shared__ __attribute__((aligned(16))) T s_w[GDN ? CH * LDK : 8];  // w                [64][K]
-  __shared__ __attribute__((aligned(16))) T s_hT[GDN ? BV * LDK : 8]; // S^T              [BV][K]
-  __shared__ __attribute__((aligned(16))) T s_u[GDN ? CH * LDU : 8];  // u                [64][BV]
-  __shared__ float s_b[64], s_ed[64];
+  constexpr int NBUF = sizeof(T) == 2 ? 2 : 1;
+  __shared__ __attribute__((aligned(16))) T s_kd[NBUF][CH * LDK];             // k e^{b_C-b}   [64][K]
+  __shared__ __attribute__((aligned(16))) T s_w[NBUF][GDN ? CH * LDK : 8];    // w             [64][K]
+  __shared__ __attribute__((aligned(16))) T s_u[NBUF][CH * LDU];              // u or v        [64][BV]
+  __shared__ __attribute__((aligned(16))) T s_hT[BV * LDK];                   // S^T           [BV][K]
+  __shared__ __attribute__((aligned(16))) T s_vT[GDN ? BV * LDC : 8];         // v_new^T       [BV][64]
+  __shared__ __attribute__((aligned(16))) T s_stg[GDN ? 4 * 16 * LDU : 8];    // v_new store staging
 
-  const int v0 = blockIdx.x * BV, h = blockIdx.y, n = blockIdx.z;
+  constexpr int NVS = V / BV;
+  const int xcd = blockIdx.x & 7, jj = blockIdx.x >> 3;
+  const int vsl = jj % NVS, pair = (jj / NVS) * 8 + xcd;
+  if (pair >= a.N * a.H) return;
+  const int v0 = vsl * BV, h = pair % a.H, n = pair / a.H;
   const SeqInfo sq = seq_info(a, n);
   const int wv = wave_id(), l = lane_id();
   const int krow0 = wv * (K / 4);
@@ -45,71 +58,96 @@ __global__ __launch_bounds__(NTHR) void k_state_fwd(const lmoe_args a) {
 
   typedef TileIO<T, CH, K> IOK;
   typedef TileIO<T, CH, BV> IOV;
+  typedef TileIO<T, BV, K> IOHT;
+  typename IOK::Regs rk, rw;
+  typename IOV::Regs ru;
+  uint32_t graw = 0;
+  const lmoe_tensor& us = GDN ? a.u : a.v;
+  const bool gated = a.gate != LMOE_GATE_NONE && a.g.ptr != nullptr;
 
-  for (int c = 0; c < sq.nchunks; ++c) {
+  auto issue = [&](int c) {
     const int tok = sq.tok0 + c * CH;
     const int len = min(CH, sq.len - c * CH);
-    chunk_gate_cumsum(a, sq.b, tok, len, h, s_b, nullptr, s_ed);
-
-    typename IOK::Regs rk;
     IOK::load(rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, len);
-    IOK::store_lds_t(rk, s_kT, LDC, s_ed);
-    if constexpr (GDN) {
-      typename IOK::Regs rw;
-      IOK::load(rw, row_ptr<T>(a.w, sq.b, tok, h), a.w.st, len);
-      IOK::store_lds(rw, s_w, LDK);
-      typename IOV::Regs ru;
-      IOV::load(ru, row_ptr<T>(a.u, sq.b, tok, h) + v0, a.u.st, len);
-      IOV::store_lds(ru, s_u, LDU);
-    } else {
-      typename IOV::Regs rv;
-      IOV::load(rv, row_ptr<T>(a.v, sq.b, tok, h) + v0, a.v.st, len);
-      IOV::store_lds_t(rv, s_vT, LDC, nullptr);
+    if constexpr (GDN) IOK::load(rw, row_ptr<T>(a.w, sq.b, tok, h), a.w.st, len);
+    IOV::load(ru, row_ptr<T>(us, sq.b, tok, h) + v0, us.st, len);
+    graw = 0;
+    if (gated && l < len) graw = load_scalar_raw(a.g.ptr, a.g_dtype, row_off(a.g, sq.b, tok + l, h));
+  };
+  // registers -> LDS buffer `buf`; returns e^{b_C} of that chunk
+  auto stage = [&](int buf) -> float {
+    const float x = wave_incl_scan(scalar_from_raw(graw, a.g_dtype));
+    const float xl = __shfl(x, 63, 64);
+    const float ed = expf(xl - x);                        // lane j: e^{b_C - b_j}
+#pragma unroll
+    for (int p = 0; p < IOK::PASSES; ++p) {
+      int row, col; IOK::coords(p, row, col);
+      const float sc = __shfl(ed, row, 64);
+      typename IOK::vec o;
+#pragma unroll
+      for (int i = 0; i < IOK::VEC; ++i) o[i] = ET<T>::from_f(ET<T>::to_f(rk.v[p][i]) * sc);
+      *(typename IOK::vec*)(&s_kd[buf][row * LDK + col]) = o;
     }
-    // state at chunk start -> hs (and LDS copy for the delta rule)
-    {
-      T* hs = (T*)a.hs + ((int64_t)(sq.chunk0 + c) * a.H + h) * K * V;
+    if constexpr (GDN) IOK::store_lds(rw, s_w[buf], LDK);
+    IOV::store_lds(ru, s_u[buf], LDU);
+    return expf(xl);
+  };
+
+  float dec_cur = 1.f;
+  if (sq.nchunks > 0) {
+    issue(0);
+    dec_cur = stage(0);
+    if (sq.nchunks > 1) issue(1);
+  }
+  for (int c = 0; c < sq.nchunks; ++c) {
+    const int cur = NBUF == 2 ? (c & 1) : 0;
+    const int tok = sq.tok0 + c * CH;
+    const int len = min(CH, sq.len - c * CH);
+    // S (state at chunk start) -> LDS as S^T
 #pragma unroll
-      for (int mi = 0; mi < MB; ++mi)
+    for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < NB; ++ni) {
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-            hs[(int64_t)(krow0 + acc_row(mi, i)) * V + v0 + acc_col(ni)] = ET<T>::from_f(S[mi][ni][i]);
-          if constexpr (GDN) acc_to_lds_t<T>(S[mi][ni], s_hT, LDK, krow0 + 16 * mi, 16 * ni);
-        }
-    }
-    __syncthreads();
+      for (int ni = 0; ni < NB; ++ni) acc_to_lds_t<T>(S[mi][ni], s_hT, LDK, krow0 + 16 * mi, 16 * ni);
+    lds_barrier();
+    // hs[chunk][h][v0 .. v0+BV][K] <- S^T   (off the dependency chain)
+    IOHT::lds_to_global(s_hT, LDK, (T*)a.hs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
     if constexpr (GDN) {
       // v_new = u - w S  (rows 16*wv .. +15 of the chunk)
       f32x4 vn[1][NB];
       acc_zero(vn);
-      gemm_nt<T, 1, NB>(vn, s_w, LDK, 16 * wv, s_hT, LDK, 0, 0, K);
-      T* vdst = row_ptr<T>(a.vnew, sq.b, tok, h) + v0;
+      gemm<T, 1, NB, false, false>(vn, s_w[cur], LDK, 16 * wv, s_hT, LDK, 0, 0, K);
 #pragma unroll
       for (int ni = 0; ni < NB; ++ni) {
-        f32x4 x;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
-          x[i] = ET<T>::to_f(s_u[r * LDU + cc]) - vn[0][ni][i];
-          // round once to the storage type so that the state update and the output kernel
-          // see the same v_new
-          x[i] = ET<T>::to_f(ET<T>::from_f(x[i]));
-          if (r < len) vdst[(int64_t)r * a.vnew.st + cc] = ET<T>::from_f(x[i]);
+          // round once to the storage type so that the state update and the output kernel see
+          // the same v_new
+          vn[0][ni][i] = ET<T>::to_f(ET<T>::from_f(ET<T>::to_f(s_u[cur][r * LDU + cc]) - vn[0][ni][i]));
         }
-        acc_to_lds_t<T>(x, s_vT, LDC, 16 * wv, 16 * ni);
+        acc_to_lds_t<T>(vn[0][ni], s_vT, LDC, 16 * wv, 16 * ni);
       }
-      __syncthreads();
+      lds_barrier();
+#pragma unroll
+      for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) S[mi][ni] *= dec_cur;
+      gemm<T, MB, NB, true, false>(S, s_kd[cur], LDK, krow0, s_vT, LDC, 0, 0, CH);
+      store_strip<T, NB>(vn, s_stg + wv * 16 * LDU, row_ptr<T>(a.vnew, sq.b, tok + 16 * wv, h) + v0, a.vnew.st,
+                         len - 16 * wv, 1.0f);
+    } else {
+#pragma unroll
+      for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) S[mi][ni] *= dec_cur;
+      gemm<T, MB, NB, true, true>(S, s_kd[cur], LDK, krow0, s_u[cur], LDU, 0, 0, CH);
     }
-    // S = e^{b_C} S + k_d^T v'
-    const float dec = expf(s_b[63]);
-#pragma unroll
-    for (int mi = 0; mi < MB; ++mi)
-#pragma unroll
-      for (int ni = 0; ni < NB; ++ni) S[mi][ni] *= dec;
-    gemm_nt<T, MB, NB>(S, s_kT, LDC, krow0, s_vT, LDC, 0, 0, CH);
-    __syncthreads();
+    // stage the next chunk (its loads were issued one step ago) and fetch the one after
+    if (c + 1 < sq.nchunks) {
+      if constexpr (NBUF == 1) lds_barrier();       // single buffer: wait until it has been read
+      dec_cur = stage(NBUF == 2 ? (cur ^ 1) : 0);
+      if (c + 2 < sq.nchunks) issue(c + 2);
+    }
   }
 
   if (a.ht) {
@@ -130,14 +168,14 @@ __global__ __launch_bounds__(NTHR) void k_state_fwd(const lmoe_args a) {
 //   wave w owns chunk rows 16w .. 16w+15.
 //   The tiles of the next item are fetched into registers while the current one is computed
 //   (barriers order LDS traffic only, so the loads stay in flight).
-//   LDS: q, k, S stored as loaded; P^T overlays k once q k^T is done, v' overlays S once q S is
+//   LDS: q, k, S^T stored as loaded (hs holds S^T, [V][K]); P^T overlays k once q k^T is done, v' overlays S once q S is
 //   done; products that contract over tile rows use transposed fragments.
 // ------------------------------------------------------------------------- //
 template <typename T, int K, int V, bool GDN>
 __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_out_fwd(const lmoe_args a) {
   constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDV = V + LPAD;
   constexpr int NB = V / 16;
-  constexpr int H_EL = K * LDV > CH * LDV ? K * LDV : CH * LDV;
+  constexpr int H_EL = V * LDK > CH * LDV ? V * LDK : CH * LDV;
   constexpr int Q_EL = CH * LDK > 4 * 16 * LDV ? CH * LDK : 4 * 16 * LDV;   // also the store staging area
   __shared__ __attribute__((aligned(16))) T s_q[Q_EL];
   __shared__ __attribute__((aligned(16))) T s_k[CH * LDK];      // later: P^T [64][LDC]
@@ -150,7 +188,7 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_out_fwd(cons
   const int wv = wave_id(), l = lane_id();
   typedef TileIO<T, CH, K> IOK;
   typedef TileIO<T, CH, V> IOV;
-  typedef TileIO<T, K, V> IOH;
+  typedef TileIO<T, V, K> IOH;        // hs holds S^T: [V][K]
   const lmoe_tensor& vs = GDN ? a.vnew : a.v;
   const int nitems = a.NT * a.H;
   typename IOK::Regs rq, rk;
@@ -162,7 +200,7 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_out_fwd(cons
     const ChunkInfo ci = chunk_info(a, cid);
     IOK::load(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
     IOK::load(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
-    IOH::load(rh, (const T*)a.hs + ((int64_t)cid * a.H + h) * K * V, V, K);
+    IOH::load(rh, (const T*)a.hs + ((int64_t)cid * a.H + h) * K * V, K, V);
     graw = gate_prefetch(a, ci.b, ci.tok, ci.len, h);
   };
   auto issue_v = [&](int it) {
@@ -179,7 +217,7 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_out_fwd(cons
     gate_finish(a, graw, s_b, s_eb, nullptr);
     IOK::store_lds(rq, s_q, LDK);
     IOK::store_lds(rk, s_k, LDK);
-    IOH::store_lds(rh, s_h, LDV);
+    IOH::store_lds(rh, s_h, LDK);
     lds_barrier();
     if (nxt < nitems) issue(nxt);
     f32x4 s[1][4];
@@ -187,7 +225,7 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_out_fwd(cons
     gemm<T, 1, 4, false, false>(s, s_q, LDK, 16 * wv, s_k, LDK, 0, 0, K);
     f32x4 o[1][NB];
     acc_zero(o);
-    gemm<T, 1, NB, false, true>(o, s_q, LDK, 16 * wv, s_h, LDV, 0, 0, K);
+    gemm<T, 1, NB, false, false>(o, s_q, LDK, 16 * wv, s_h, LDK, 0, 0, K);
     lds_barrier();            // every wave is done reading k and S: P^T and v' may overlay them
     IOV::store_lds(rv, s_v, LDV);
     if (nxt < nitems) issue_v(nxt);
