@@ -193,23 +193,38 @@ __device__ __forceinline__ void acc_to_lds_t(const f32x4& a, T* tile, int ld, in
 // Store the 16-row strip a wave holds in accumulators (NB*16 columns) to global memory with
 // 16-byte vector stores, through a wave-private LDS staging area stg[16][NB*16 + LPAD].
 // gdst points at row 0 / column 0 of the strip; rows >= nvalid are not written.  Only the
-// calling wave touches stg, so no work-group barrier is involved.
-template <typename T, int NB>
+// calling wave touches stg, so no work-group barrier is involved.  With ADD the strip is added
+// to what the destination already holds (read with the same 16-byte vectors).
+template <typename T, int NB, bool ADD = false>
 __device__ __forceinline__ void store_strip(const f32x4 (&acc)[1][NB], T* stg, T* __restrict__ gdst,
                                             int64_t row_stride, int nvalid, float mul) {
   constexpr int W = NB * 16, LD = W + LPAD, VEC = ET<T>::VEC, VPR = W / VEC;
+  typedef typename ET<T>::vec vec;
   const int l = lane_id();
 #pragma unroll
   for (int ni = 0; ni < NB; ++ni)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) stg[(4 * (l >> 4) + i) * LD + 16 * ni + (l & 15)] = ET<T>::from_f(acc[0][ni][i] * mul);
+    for (int i = 0; i < 4; ++i) {
+      stg[(4 * (l >> 4) + i) * LD + 16 * ni + (l & 15)] = ET<T>::from_f(acc[0][ni][i] * mul);
+    }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
   for (int idx = l; idx < 16 * VPR; idx += 64) {
     const int r = idx / VPR, c = (idx % VPR) * VEC;
-    if (r < nvalid) *(typename ET<T>::vec*)(gdst + (int64_t)r * row_stride + c) = *(const typename ET<T>::vec*)(stg + r * LD + c);
+    if (r < nvalid) {
+      T* g = gdst + (int64_t)r * row_stride + c;
+      if constexpr (ADD) {
+        vec o = *(const vec*)g;
+        const vec x = *(const vec*)(stg + r * LD + c);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) o[i] = ET<T>::from_f(ET<T>::to_f(o[i]) + ET<T>::to_f(x[i]));
+        *(vec*)g = o;
+      } else {
+        *(vec*)g = *(const vec*)(stg + r * LD + c);
+      }
+    }
   }
 }
 
