@@ -57,98 +57,81 @@ __device__ __forceinline__ void tri_inverse_64(const float* sL, int ldl, float* 
 }
 
 template <typename T, int K, int V>
-__global__ __launch_bounds__(NTHR) void k_gdn_wy_fwd(const lmoe_args a) {
-  constexpr int LDK = K + LPAD, LDC = CH + LPAD;
+__global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(const lmoe_args a) {
+  constexpr int LDK = K + LPAD, LDV = V + LPAD, LDC = CH + LPAD;
+  constexpr int NBK = K / 16, NBV = V / 16;
+  // k (raw, for k k^T), then overwritten in place by k beta e^{b}; v beta; both stored [64][D]
   __shared__ __attribute__((aligned(16))) T s_k[CH * LDK];
-  __shared__ __attribute__((aligned(16))) T s_kbgT[K * LDC];
-  __shared__ __attribute__((aligned(16))) T s_vbT[V * LDC];
-  __shared__ __attribute__((aligned(16))) float s_L[CH * LDC];
+  __shared__ __attribute__((aligned(16))) T s_vb[CH * LDV];
+  __shared__ __attribute__((aligned(16))) float s_L[CH * LDC];   // L, later Tinv in element type T
   __shared__ __attribute__((aligned(16))) float s_X[CH * LDC];
-  // Tinv as an MFMA operand: fp32 reuses s_X in place, bf16 gets its own copy
-  __shared__ __attribute__((aligned(16))) T s_Tm_own[sizeof(T) == 4 ? 8 : CH * LDC];
-  T* s_Tm = sizeof(T) == 4 ? (T*)s_X : s_Tm_own;
   __shared__ float s_Y[3 * 256];
   __shared__ float s_b[64], s_eb[64], s_beta[64], s_beb[64];
+  // Tinv as an MFMA operand: fp32 uses s_X in place, bf16 a copy in the (dead) L tile
+  T* s_Tm = sizeof(T) == 4 ? (T*)s_X : (T*)s_L;
 
   const int cid = blockIdx.x, h = blockIdx.y;
   const ChunkInfo ci = chunk_info(a, cid);
   const int wv = wave_id(), l = lane_id();
+  typedef TileIO<T, CH, K> IOK;
+  typedef TileIO<T, CH, V> IOV;
+  typename IOK::Regs rk;
+  typename IOV::Regs rv;
+  IOK::load(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
+  IOV::load(rv, row_ptr<T>(a.v, ci.b, ci.tok, h), a.v.st, ci.len);
   if (threadIdx.x >= 64 && threadIdx.x < 128) {
     const int j = threadIdx.x - 64;
     s_beta[j] = j < ci.len ? load_scalar(a.beta.ptr, a.beta_dtype, row_off(a.beta, ci.b, ci.tok + j, h)) : 0.f;
   }
-  chunk_gate_cumsum(a, ci.b, ci.tok, ci.len, h, s_b, s_eb, nullptr);
+  chunk_gate_cumsum(a, ci.b, ci.tok, ci.len, h, s_b, s_eb, nullptr);    // barrier inside
   if (threadIdx.x < 64) s_beb[threadIdx.x] = s_beta[threadIdx.x] * s_eb[threadIdx.x];
-  __syncthreads();
-
-  typedef TileIO<T, CH, K> IOK;
-  typedef TileIO<T, CH, V> IOV;
-  {
-    typename IOK::Regs rk;
-    IOK::load(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
-    typename IOV::Regs rv;
-    IOV::load(rv, row_ptr<T>(a.v, ci.b, ci.tok, h), a.v.st, ci.len);
-    IOK::store_lds(rk, s_k, LDK);
-    IOK::store_lds_t(rk, s_kbgT, LDC, s_beb);
-    IOV::store_lds_t(rv, s_vbT, LDC, s_beta);
-  }
+  IOK::store_lds(rk, s_k, LDK);
+  IOV::store_lds_scaled(rv, s_vb, LDV, s_beta);
   __syncthreads();
   {
     f32x4 m[1][4];
     acc_zero(m);
-    gemm_nt<T, 1, 4>(m, s_k, LDK, 16 * wv, s_k, LDK, 0, 0, K);
+    gemm<T, 1, 4, false, false>(m, s_k, LDK, 16 * wv, s_k, LDK, 0, 0, K);
 #pragma unroll
     for (int nj = 0; nj < 4; ++nj) {
       f32x4 p;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * nj + (l & 15);
-        p[i] = (r > cc) ? s_beta[r] * m[0][nj][i] * expf(s_b[r] - s_b[cc]) : 0.f;
+        p[i] = (r > cc) ? s_beta[r] * m[0][nj][i] * texp<T>(s_b[r] - s_b[cc]) : 0.f;
       }
       acc_to_lds<float>(p, s_L, LDC, 16 * wv, 16 * nj);
     }
   }
   __syncthreads();
-  tri_inverse_64(s_L, LDC, s_X, LDC, s_Y);
-  // Tinv -> element type T (LDS operand + global copy for the backward)
+  // k is dead as an operand of k k^T: scale it in place to k beta e^{b} (from the registers)
+  IOK::store_lds_scaled(rk, s_k, LDK, s_beb);
+  tri_inverse_64(s_L, LDC, s_X, LDC, s_Y);       // barriers inside; s_L is dead afterwards
   {
     T* tg = (T*)a.tinv + ((int64_t)cid * a.H + h) * CH * CH;
-    for (int idx = threadIdx.x; idx < CH * CH; idx += NTHR) {
-      const int r = idx >> 6, c = idx & 63;
-      const T x = ET<T>::from_f(s_X[r * LDC + c]);
-      if constexpr (sizeof(T) != 4) s_Tm[r * LDC + c] = x;
-      tg[idx] = x;
+    for (int idx = threadIdx.x; idx < CH * CH / 4; idx += NTHR) {
+      const int r = idx >> 4, c = (idx & 15) * 4;
+      const f32x4 x = *(const f32x4*)(s_X + r * LDC + c);
+      if constexpr (sizeof(T) == 2) {
+        bf16x4 y; y[0] = (bf16)x[0]; y[1] = (bf16)x[1]; y[2] = (bf16)x[2]; y[3] = (bf16)x[3];
+        *(bf16x4*)(s_Tm + r * LDC + c) = y;
+        *(bf16x4*)(tg + r * CH + c) = y;
+      } else {
+        *(f32x4*)(tg + r * CH + c) = x;
+      }
     }
   }
   __syncthreads();
-  {
-    constexpr int NBK = K / 16;
-    f32x4 w[1][NBK];
-    acc_zero(w);
-    gemm_nt<T, 1, NBK>(w, s_Tm, LDC, 16 * wv, s_kbgT, LDC, 0, 0, CH);
-    T* wd = row_ptr<T>(a.w, ci.b, ci.tok, h);
-#pragma unroll
-    for (int ni = 0; ni < NBK; ++ni)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
-        if (r < ci.len) wd[(int64_t)r * a.w.st + cc] = ET<T>::from_f(w[0][ni][i]);
-      }
-  }
-  {
-    constexpr int NBV = V / 16;
-    f32x4 u[1][NBV];
-    acc_zero(u);
-    gemm_nt<T, 1, NBV>(u, s_Tm, LDC, 16 * wv, s_vbT, LDC, 0, 0, CH);
-    T* ud = row_ptr<T>(a.u, ci.b, ci.tok, h);
-#pragma unroll
-    for (int ni = 0; ni < NBV; ++ni)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
-        if (r < ci.len) ud[(int64_t)r * a.u.st + cc] = ET<T>::from_f(u[0][ni][i]);
-      }
-  }
+  // w = Tinv (k beta e^{b}),  u = Tinv (v beta): contraction over the rows of the [64][D] tiles
+  f32x4 w[1][NBK];
+  acc_zero(w);
+  gemm<T, 1, NBK, false, true>(w, s_Tm, LDC, 16 * wv, s_k, LDK, 0, 0, CH);
+  f32x4 u[1][NBV];
+  acc_zero(u);
+  gemm<T, 1, NBV, false, true>(u, s_Tm, LDC, 16 * wv, s_vb, LDV, 0, 0, CH);
+  __syncthreads();   // k, v tiles are dead: wave-private slices of them stage the stores
+  store_strip<T, NBK>(w, s_k + wv * 16 * LDK, row_ptr<T>(a.w, ci.b, ci.tok + 16 * wv, h), a.w.st, ci.len - 16 * wv, 1.0f);
+  store_strip<T, NBV>(u, s_vb + wv * 16 * LDV, row_ptr<T>(a.u, ci.b, ci.tok + 16 * wv, h), a.u.st, ci.len - 16 * wv, 1.0f);
 }
 
 }  // namespace lmoe
