@@ -31,7 +31,8 @@ template <bool GDN> struct BwdDqk {
   template <typename T, int K, int V> struct F {
     static void run(const lmoe_args& a, hipStream_t st) {
       constexpr int BVH = BwdTiles<T, V>::BVH;
-      hipLaunchKernelGGL((k_bwd_dqk<T, K, V, BVH, GDN>), dim3(a.NT, a.H), dim3(NTHR), 0, st, a);
+      const int grid = persistent_grid(a.NT * a.H, 1);
+      hipLaunchKernelGGL((k_bwd_dqk<T, K, V, BVH, GDN>), dim3(grid), dim3(NTHR), 0, st, a);
     }
   };
 };

@@ -246,12 +246,14 @@ __global__ __launch_bounds__(NTHR) void k_state_bwd(const lmoe_args a) {
 }
 
 // ------------------------------------------------------------------------- //
-// dq, dk, gate gradient        grid = (NT, H)
+// dq, dk, gate gradient        persistent: grid = min(NT*H, 2 per CU), one item = (chunk, head)
 //   phase A: loop over V-slices of width BVH accumulating
 //              dP = do v'^T, dq_i = do S^T, dk_d = v' dS'^T (, dw = dv_new S^T)
 //            (hs, dhs hold S^T, dS'^T: [V][K]; the slice tiles are [BVH][K])
 //   phase B: dq = scale e_b dq_i + (scale dP . Gamma) k ; dk = e_d dk_d + (scale dP . Gamma)^T q
 //            with one LDS copy of (scale dP . Gamma)^T and q, k stored as loaded
+//   The loads of the next slice / of q, k / of the next item's first slice are in flight while
+//   the current step computes (barriers order LDS traffic only).
 // ------------------------------------------------------------------------- //
 template <typename T, int K, int V, int BVH, bool GDN>
 __global__ __launch_bounds__(NTHR) void k_bwd_dqk(const lmoe_args a) {
@@ -266,27 +268,43 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dqk(const lmoe_args a) {
   __shared__ __attribute__((aligned(16))) T smem[NELEM];
   __shared__ float s_b[64], s_eb[64], s_ed[64], s_db[64], s_red[8];
 
-  const int cid = blockIdx.x, h = blockIdx.y;
-  const ChunkInfo ci = chunk_info(a, cid);
   const int wv = wave_id(), l = lane_id();
-  chunk_gate_cumsum(a, ci.b, ci.tok, ci.len, h, s_b, s_eb, s_ed);
-
   typedef TileIO<T, CH, BVH> IOV;
   typedef TileIO<T, BVH, K> IOH;
   typedef TileIO<T, CH, K> IOK;
   const lmoe_tensor& vs = GDN ? a.vnew : a.v;
+  const int nitems = a.NT * a.H;
 
-  f32x4 dP[1][4], dqi[1][NBK], dkd[1][NBK], dw[1][GDN ? NBK : 1];
-  acc_zero(dP); acc_zero(dqi); acc_zero(dkd); acc_zero(dw);
-  float hdh = 0.f;   // partial <S, dS'>
-  for (int vv = 0; vv < V; vv += BVH) {
-    {
-      typename IOV::Regs rd, rv;
-      IOV::load(rd, row_ptr<T>(a.d_o, ci.b, ci.tok, h) + vv, a.d_o.st, ci.len);
-      IOV::load(rv, row_ptr<T>(vs, ci.b, ci.tok, h) + vv, vs.st, ci.len);
-      typename IOH::Regs rh, rdh;
-      IOH::load(rh, (const T*)a.hs + (((int64_t)cid * a.H + h) * V + vv) * K, K, BVH);
-      IOH::load(rdh, (const T*)a.dhs + (((int64_t)cid * a.H + h) * V + vv) * K, K, BVH);
+  typename IOV::Regs rd, rv, rn;
+  typename IOH::Regs rh, rdh;
+  typename IOK::Regs rq, rk;
+  uint32_t graw = 0;
+  auto issueA = [&](int it, int vv) {
+    const int cid = it / a.H, h = it % a.H;
+    const ChunkInfo ci = chunk_info(a, cid);
+    IOV::load(rd, row_ptr<T>(a.d_o, ci.b, ci.tok, h) + vv, a.d_o.st, ci.len);
+    IOV::load(rv, row_ptr<T>(vs, ci.b, ci.tok, h) + vv, vs.st, ci.len);
+    IOH::load(rh, (const T*)a.hs + (((int64_t)cid * a.H + h) * V + vv) * K, K, BVH);
+    IOH::load(rdh, (const T*)a.dhs + (((int64_t)cid * a.H + h) * V + vv) * K, K, BVH);
+    if constexpr (GDN) IOV::load(rn, row_ptr<T>(a.dvnew, ci.b, ci.tok, h) + vv, a.dvnew.st, ci.len);
+  };
+  auto issueQK = [&](int it) {
+    const int cid = it / a.H, h = it % a.H;
+    const ChunkInfo ci = chunk_info(a, cid);
+    IOK::load(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
+    IOK::load(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
+    graw = gate_prefetch(a, ci.b, ci.tok, ci.len, h);
+  };
+
+  int it = blockIdx.x;
+  if (it < nitems) issueA(it, 0);
+  for (; it < nitems; it += gridDim.x) {
+    const int cid = it / a.H, h = it % a.H;
+    const ChunkInfo ci = chunk_info(a, cid);
+    f32x4 dP[1][4], dqi[1][NBK], dkd[1][NBK], dw[1][GDN ? NBK : 1];
+    acc_zero(dP); acc_zero(dqi); acc_zero(dkd); acc_zero(dw);
+    float hdh = 0.f;   // partial <S, dS'>
+    for (int vv = 0; vv < V; vv += BVH) {
 #pragma unroll
       for (int p = 0; p < IOH::PASSES; ++p)
 #pragma unroll
@@ -295,24 +313,24 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dqk(const lmoe_args a) {
       IOV::store_lds(rv, smem + A_V, LDV);
       IOH::store_lds(rh, smem + A_H, LDK);
       IOH::store_lds(rdh, smem + A_DH, LDK);
-      if constexpr (GDN) {
-        typename IOV::Regs rn;
-        IOV::load(rn, row_ptr<T>(a.dvnew, ci.b, ci.tok, h) + vv, a.dvnew.st, ci.len);
-        IOV::store_lds(rn, smem + A_DVN, LDV);
-      }
+      if constexpr (GDN) IOV::store_lds(rn, smem + A_DVN, LDV);
+      lds_barrier();
+      if (vv + BVH < V) issueA(it, vv + BVH); else issueQK(it);
+      gemm<T, 1, 4, false, false>(dP, smem + A_DO, LDV, 16 * wv, smem + A_V, LDV, 0, 0, BVH);
+      gemm<T, 1, NBK, false, true>(dqi, smem + A_DO, LDV, 16 * wv, smem + A_H, LDK, 0, 0, BVH);
+      gemm<T, 1, NBK, false, true>(dkd, smem + A_V, LDV, 16 * wv, smem + A_DH, LDK, 0, 0, BVH);
+      if constexpr (GDN) gemm<T, 1, NBK, false, true>(dw, smem + A_DVN, LDV, 16 * wv, smem + A_H, LDK, 0, 0, BVH);
+      lds_barrier();
     }
-    __syncthreads();
-    gemm<T, 1, 4, false, false>(dP, smem + A_DO, LDV, 16 * wv, smem + A_V, LDV, 0, 0, BVH);
-    gemm<T, 1, NBK, false, true>(dqi, smem + A_DO, LDV, 16 * wv, smem + A_H, LDK, 0, 0, BVH);
-    gemm<T, 1, NBK, false, true>(dkd, smem + A_V, LDV, 16 * wv, smem + A_DH, LDK, 0, 0, BVH);
-    if constexpr (GDN) gemm<T, 1, NBK, false, true>(dw, smem + A_DVN, LDV, 16 * wv, smem + A_H, LDK, 0, 0, BVH);
-    __syncthreads();
-  }
-  // block reduction of <S, dS'>
-  hdh = wave_sum(hdh);
-  if (l == 0) s_red[wv] = hdh;
-  // phase B operands
-  {
+    // block reduction of <S, dS'>
+    hdh = wave_sum(hdh);
+    if (l == 0) s_red[wv] = hdh;
+    // phase B operands
+    gate_finish(a, graw, s_b, s_eb, s_ed);
+    IOK::store_lds(rq, smem + B_Q, LDK);
+    IOK::store_lds(rk, smem + B_K, LDK);
+    lds_barrier();
+    if (it + gridDim.x < nitems) issueA(it + gridDim.x, 0);
 #pragma unroll
     for (int nj = 0; nj < 4; ++nj) {
       f32x4 p;
@@ -323,70 +341,66 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dqk(const lmoe_args a) {
       }
       acc_to_lds_t<T>(p, smem + B_DPT, LDC, 16 * wv, 16 * nj);      // [j][i]
     }
-    typename IOK::Regs rq, rk;
-    IOK::load(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
-    IOK::load(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
-    IOK::store_lds(rq, smem + B_Q, LDK);
-    IOK::store_lds(rk, smem + B_K, LDK);
-  }
-  __syncthreads();
-  f32x4 dq[1][NBK], dk[1][NBK];
-  acc_zero(dq); acc_zero(dk);
-  // dq_intra[i][c] = sum_j dPG[i][j] k[j][c] : A = dPG^T stored [j][i] (contraction along rows)
-  gemm<T, 1, NBK, true, true>(dq, smem + B_DPT, LDC, 16 * wv, smem + B_K, LDK, 0, 0, CH);
-  // dk_intra[j][c] = sum_i dPG[i][j] q[i][c] : A = dPG^T rows j (contraction along columns)
-  gemm<T, 1, NBK, false, true>(dk, smem + B_DPT, LDC, 16 * wv, smem + B_Q, LDK, 0, 0, CH);
-  // combine and form db_i = q_i.dq_i - k_i.dk_i ; kk = sum_j (dk_d . k_d)_j
-  float dbp[4] = {0.f, 0.f, 0.f, 0.f};
-  float kk = 0.f;
+    lds_barrier();
+    f32x4 dq[1][NBK], dk[1][NBK];
+    acc_zero(dq); acc_zero(dk);
+    // dq_intra[i][c] = sum_j dPG[i][j] k[j][c] : A = dPG^T stored [j][i] (contraction along rows)
+    gemm<T, 1, NBK, true, true>(dq, smem + B_DPT, LDC, 16 * wv, smem + B_K, LDK, 0, 0, CH);
+    // dk_intra[j][c] = sum_i dPG[i][j] q[i][c] : A = dPG^T rows j (contraction along columns)
+    gemm<T, 1, NBK, false, true>(dk, smem + B_DPT, LDC, 16 * wv, smem + B_Q, LDK, 0, 0, CH);
+    // combine and form db_i = q_i.dq_i - k_i.dk_i ; kk = sum_j (dk_d . k_d)_j
+    float dbp[4] = {0.f, 0.f, 0.f, 0.f};
+    float kk = 0.f;
 #pragma unroll
-  for (int ni = 0; ni < NBK; ++ni)
+    for (int ni = 0; ni < NBK; ++ni)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
+        const float qv = ET<T>::to_f(smem[B_Q + r * LDK + cc]);
+        const float kv = ET<T>::to_f(smem[B_K + r * LDK + cc]);
+        const float dqv = a.scale * s_eb[r] * dqi[0][ni][i] + dq[0][ni][i];
+        const float dkdv = s_ed[r] * dkd[0][ni][i];
+        const float dkv = dkdv + dk[0][ni][i];
+        dbp[i] += qv * dqv - kv * dkv;
+        kk += kv * dkdv;
+        dq[0][ni][i] = dqv;
+        dk[0][ni][i] = dkv;
+      }
+    // reduce db over the 16 lanes that share a row group, kk over the whole block
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
-      const float qv = ET<T>::to_f(smem[B_Q + r * LDK + cc]);
-      const float kv = ET<T>::to_f(smem[B_K + r * LDK + cc]);
-      const float dqv = a.scale * s_eb[r] * dqi[0][ni][i] + dq[0][ni][i];
-      const float dkdv = s_ed[r] * dkd[0][ni][i];
-      const float dkv = dkdv + dk[0][ni][i];
-      dbp[i] += qv * dqv - kv * dkv;
-      kk += kv * dkdv;
-      dq[0][ni][i] = dqv;
-      dk[0][ni][i] = dkv;
+#pragma unroll
+      for (int d = 1; d < 16; d <<= 1) dbp[i] += __shfl_xor(dbp[i], d, 64);
     }
-  // reduce db over the 16 lanes that share a row group, kk over the whole block
+    if ((l & 15) == 0) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-#pragma unroll
-    for (int d = 1; d < 16; d <<= 1) dbp[i] += __shfl_xor(dbp[i], d, 64);
-  }
-  if ((l & 15) == 0) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) s_db[16 * wv + 4 * (l >> 4) + i] = dbp[i];
-  }
-  kk = wave_sum(kk);
-  if (l == 0) s_red[4 + wv] = kk;
-  __syncthreads();     // q, k tiles are dead from here: wave-private slices become store staging
-  {
-    T* stg = smem + B_K + wv * 16 * LDK;    // this wave's 16 rows of the k tile, then of the q tile
-    store_strip<T, NBK>(dq, stg, row_ptr<T>(a.dq, ci.b, ci.tok + 16 * wv, h), a.dq.st, ci.len - 16 * wv, 1.0f);
-    T* stg2 = smem + B_Q + wv * 16 * LDK;
-    store_strip<T, NBK>(dk, stg2, row_ptr<T>(a.dk, ci.b, ci.tok + 16 * wv, h), a.dk.st, ci.len - 16 * wv, 1.0f);
-    if constexpr (GDN) {
-      // dw = -dv_new S^T ; staging reuses the first slice again (same wave, program order)
-      store_strip<T, NBK>(dw, stg, row_ptr<T>(a.dw, ci.b, ci.tok + 16 * wv, h), a.dw.st, ci.len - 16 * wv, -1.0f);
+      for (int i = 0; i < 4; ++i) s_db[16 * wv + 4 * (l >> 4) + i] = dbp[i];
     }
-  }
-  if (threadIdx.x < 64) {
-    const int j = threadIdx.x;
-    float x = s_db[j];
-    // last-row term; rows past the end of a partial chunk carry zero q, k, so the term may sit
-    // on the last valid row without changing the reverse cumulative sum
-    const float hsum = s_red[0] + s_red[1] + s_red[2] + s_red[3];
-    const float ksum = s_red[4] + s_red[5] + s_red[6] + s_red[7];
-    if (j == ci.len - 1) x += ksum + expf(s_b[63]) * hsum;
-    if constexpr (!GDN) x = wave_rev_scan(x);   // dg; the delta rule finishes db in its WY backward
-    if (a.dg.ptr && j < ci.len) ((float*)a.dg.ptr)[row_off(a.dg, ci.b, ci.tok + j, h)] = x;
+    kk = wave_sum(kk);
+    if (l == 0) s_red[4 + wv] = kk;
+    lds_barrier();     // q, k tiles are dead from here: wave-private slices become store staging
+    {
+      T* stg = smem + B_K + wv * 16 * LDK;    // this wave's 16 rows of the k tile, then of the q tile
+      store_strip<T, NBK>(dq, stg, row_ptr<T>(a.dq, ci.b, ci.tok + 16 * wv, h), a.dq.st, ci.len - 16 * wv, 1.0f);
+      T* stg2 = smem + B_Q + wv * 16 * LDK;
+      store_strip<T, NBK>(dk, stg2, row_ptr<T>(a.dk, ci.b, ci.tok + 16 * wv, h), a.dk.st, ci.len - 16 * wv, 1.0f);
+      if constexpr (GDN) {
+        // dw = -dv_new S^T ; staging reuses the first slice again (same wave, program order)
+        store_strip<T, NBK>(dw, stg, row_ptr<T>(a.dw, ci.b, ci.tok + 16 * wv, h), a.dw.st, ci.len - 16 * wv, -1.0f);
+      }
+    }
+    if (threadIdx.x < 64) {
+      const int j = threadIdx.x;
+      float x = s_db[j];
+      // last-row term; rows past the end of a partial chunk carry zero q, k, so the term may sit
+      // on the last valid row without changing the reverse cumulative sum
+      const float hsum = s_red[0] + s_red[1] + s_red[2] + s_red[3];
+      const float ksum = s_red[4] + s_red[5] + s_red[6] + s_red[7];
+      if (j == ci.len - 1) x += ksum + expf(s_b[63]) * hsum;
+      if constexpr (!GDN) x = wave_rev_scan(x);   // dg; the delta rule finishes db in its WY backward
+      if (a.dg.ptr && j < ci.len) ((float*)a.dg.ptr)[row_off(a.dg, ci.b, ci.tok + j, h)] = x;
+    }
+    lds_barrier();     // staging and the gate arrays are reused by the next item
   }
 }
 
