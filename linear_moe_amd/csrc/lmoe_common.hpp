@@ -245,13 +245,35 @@ template <typename T, int ROWS, int COLS> struct TileIO {
     const int idx = p * NTHR + threadIdx.x;
     row = idx / VPR; col = (idx % VPR) * VEC;
   }
-  static __device__ __forceinline__ void load(Regs& r, const T* __restrict__ src, int64_t row_stride, int nvalid) {
+  // Branch-free loads: rows >= nvalid (nvalid >= 1) re-read the last valid row, so that no load
+  // sits behind a branch and the compiler can count outstanding loads exactly (prefetches stay in
+  // flight across barriers).  mask() then zeroes the rows >= nvalid; software-pipelined kernels
+  // call load_nomask() when they issue a prefetch and mask() when they consume it.
+  static __device__ __forceinline__ void load_nomask(Regs& r, const T* __restrict__ src, int64_t row_stride, int nvalid) {
+    const int last = (nvalid < ROWS ? nvalid : ROWS) - 1;
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
       int row, col; coords(p, row, col);
-      if (row < ROWS && row < nvalid) r.v[p] = *(const vec*)(src + (int64_t)row * row_stride + col);
-      else r.v[p] = ET<T>::zero();
+      row = row < last ? row : last;
+      r.v[p] = *(const vec*)(src + (int64_t)row * row_stride + col);
     }
+  }
+  static __device__ __forceinline__ void mask(Regs& r, int nvalid) {
+    if (nvalid >= ROWS) return;                 // uniform: full tiles (the common case) skip it
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      int row, col; coords(p, row, col);
+      const bool ok = row < nvalid;
+      u32x4 w = __builtin_bit_cast(u32x4, r.v[p]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) w[i] = ok ? w[i] : 0u;
+      r.v[p] = __builtin_bit_cast(vec, w);
+    }
+  }
+  static __device__ __forceinline__ void load(Regs& r, const T* __restrict__ src, int64_t row_stride, int nvalid) {
+    load_nomask(r, src, row_stride, nvalid);
+    mask(r, nvalid);
   }
   // tile[row][col] = x
   static __device__ __forceinline__ void store_lds(const Regs& r, T* tile, int ld) {

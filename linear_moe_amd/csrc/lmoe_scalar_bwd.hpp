@@ -136,27 +136,40 @@ __global__ __launch_bounds__(NTHR) void k_state_bwd(const lmoe_args a) {
   typedef TileIO<T, CH, K> IOK;
   typedef TileIO<T, CH, BV> IOV;
   typedef TileIO<T, BV, K> IOHT;
-  typename IOK::Regs rq, rk, rw;
-  typename IOV::Regs rd, rl;
-  uint32_t graw = 0;
+  // PF chunks of operands are in flight in registers (ring of PF sets, statically indexed);
+  // prefetches are always issued with a clamped chunk index (see k_state_fwd)
+  constexpr int PF = 2;
+  struct Pre { typename IOK::Regs rq, rk, rw; typename IOV::Regs rd, rl; uint32_t graw; int len; };
+  Pre pre[PF];
   const bool gated = a.gate != LMOE_GATE_NONE && a.g.ptr != nullptr;
+  const void* gptr = gated ? a.g.ptr : a.k.ptr;
   const float scale = a.scale;
 
-  auto issue = [&](int c) {
+  auto issue = [&](Pre& P, int c) {
+    c = max(c, 0);
     const int tok = sq.tok0 + c * CH;
     const int len = min(CH, sq.len - c * CH);
-    IOK::load(rq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, len);
-    IOV::load(rd, row_ptr<T>(a.d_o, sq.b, tok, h) + v0, a.d_o.st, len);
+    IOK::load_nomask(P.rq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, len);
+    IOV::load_nomask(P.rd, row_ptr<T>(a.d_o, sq.b, tok, h) + v0, a.d_o.st, len);
     if constexpr (GDN) {
-      IOK::load(rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, len);
-      IOK::load(rw, row_ptr<T>(a.w, sq.b, tok, h), a.w.st, len);
-      IOV::load(rl, row_ptr<T>(a.dvnew, sq.b, tok, h) + v0, a.dvnew.st, len);
+      IOK::load_nomask(P.rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, len);
+      IOK::load_nomask(P.rw, row_ptr<T>(a.w, sq.b, tok, h), a.w.st, len);
+      IOV::load_nomask(P.rl, row_ptr<T>(a.dvnew, sq.b, tok, h) + v0, a.dvnew.st, len);
     }
-    graw = 0;
-    if (gated && l < len) graw = load_scalar_raw(a.g.ptr, a.g_dtype, row_off(a.g, sq.b, tok + l, h));
+    P.len = len;
+    P.graw = load_scalar_raw(gptr, a.g_dtype, gated ? row_off(a.g, sq.b, tok + min(l, len - 1), h) : 0);
   };
-  auto stage = [&](int buf) -> float {
-    const float x = wave_incl_scan(scalar_from_raw(graw, a.g_dtype));
+  auto stage = [&](Pre& P, int buf) -> float {
+    IOK::mask(P.rq, P.len);
+    IOV::mask(P.rd, P.len);
+    if constexpr (GDN) {
+      IOK::mask(P.rk, P.len);
+      IOK::mask(P.rw, P.len);
+      IOV::mask(P.rl, P.len);
+    }
+    typename IOK::Regs& rq = P.rq; typename IOK::Regs& rk = P.rk; typename IOK::Regs& rw = P.rw;
+    typename IOV::Regs& rd = P.rd; typename IOV::Regs& rl = P.rl;
+    const float x = wave_incl_scan((gated && l < P.len) ? scalar_from_raw(P.graw, a.g_dtype) : 0.f);
     const float xl = __shfl(x, 63, 64);
     const float qs = scale * expf(x);                     // lane j: scale e^{b_j}
     const float ed = expf(xl - x);                        // lane j: e^{b_C - b_j}
@@ -185,11 +198,17 @@ __global__ __launch_bounds__(NTHR) void k_state_bwd(const lmoe_args a) {
 
   float dec_cur = 1.f;
   if (sq.nchunks > 0) {
-    issue(sq.nchunks - 1);
-    dec_cur = stage(0);
-    if (sq.nchunks > 1) issue(sq.nchunks - 2);
+#pragma unroll
+    for (int j = 0; j < PF; ++j) issue(pre[j], sq.nchunks - 1 - j);
+    dec_cur = stage(pre[0], 0);
+    issue(pre[0], sq.nchunks - 1 - PF);
   }
-  for (int c = sq.nchunks - 1, it = 0; c >= 0; --c, ++it) {
+  for (int it0 = 0; it0 < sq.nchunks; it0 += PF) {
+#pragma unroll
+   for (int j = 0; j < PF; ++j) {
+    const int it = it0 + j;
+    if (it >= sq.nchunks) break;
+    const int c = sq.nchunks - 1 - it;
     const int cur = NBUF == 2 ? (it & 1) : 0;
     const int tok = sq.tok0 + c * CH;
     const int len = min(CH, sq.len - c * CH);
@@ -229,9 +248,10 @@ __global__ __launch_bounds__(NTHR) void k_state_bwd(const lmoe_args a) {
     }
     if (c > 0) {
       if constexpr (NBUF == 1) lds_barrier();
-      dec_cur = stage(NBUF == 2 ? (cur ^ 1) : 0);
-      if (c > 1) issue(c - 2);
+      dec_cur = stage(pre[(j + 1) % PF], NBUF == 2 ? (cur ^ 1) : 0);
+      issue(pre[(j + 1) % PF], c - 1 - PF);
     }
+   }
   }
   if (a.dh0) {
     float* p = a.dh0 + ((int64_t)n * a.H + h) * K * V;
@@ -282,20 +302,21 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dqk(const lmoe_args a) {
   auto issueA = [&](int it, int vv) {
     const int cid = it / a.H, h = it % a.H;
     const ChunkInfo ci = chunk_info(a, cid);
-    IOV::load(rd, row_ptr<T>(a.d_o, ci.b, ci.tok, h) + vv, a.d_o.st, ci.len);
-    IOV::load(rv, row_ptr<T>(vs, ci.b, ci.tok, h) + vv, vs.st, ci.len);
-    IOH::load(rh, (const T*)a.hs + (((int64_t)cid * a.H + h) * V + vv) * K, K, BVH);
-    IOH::load(rdh, (const T*)a.dhs + (((int64_t)cid * a.H + h) * V + vv) * K, K, BVH);
-    if constexpr (GDN) IOV::load(rn, row_ptr<T>(a.dvnew, ci.b, ci.tok, h) + vv, a.dvnew.st, ci.len);
+    IOV::load_nomask(rd, row_ptr<T>(a.d_o, ci.b, ci.tok, h) + vv, a.d_o.st, ci.len);
+    IOV::load_nomask(rv, row_ptr<T>(vs, ci.b, ci.tok, h) + vv, vs.st, ci.len);
+    IOH::load_nomask(rh, (const T*)a.hs + (((int64_t)cid * a.H + h) * V + vv) * K, K, BVH);
+    IOH::load_nomask(rdh, (const T*)a.dhs + (((int64_t)cid * a.H + h) * V + vv) * K, K, BVH);
+    if constexpr (GDN) IOV::load_nomask(rn, row_ptr<T>(a.dvnew, ci.b, ci.tok, h) + vv, a.dvnew.st, ci.len);
   };
   auto issueQK = [&](int it) {
     const int cid = it / a.H, h = it % a.H;
     const ChunkInfo ci = chunk_info(a, cid);
-    IOK::load(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
-    IOK::load(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
+    IOK::load_nomask(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
+    IOK::load_nomask(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
     graw = gate_prefetch(a, ci.b, ci.tok, ci.len, h);
   };
 
+  // prefetches are always issued (item index clamped): see k_state_fwd
   int it = blockIdx.x;
   if (it < nitems) issueA(it, 0);
   for (; it < nitems; it += gridDim.x) {
@@ -309,11 +330,16 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dqk(const lmoe_args a) {
       for (int p = 0; p < IOH::PASSES; ++p)
 #pragma unroll
         for (int i = 0; i < IOH::VEC; ++i) hdh += ET<T>::to_f(rh.v[p][i]) * ET<T>::to_f(rdh.v[p][i]);
+      IOV::mask(rd, ci.len);
+      IOV::mask(rv, ci.len);
       IOV::store_lds(rd, smem + A_DO, LDV);
       IOV::store_lds(rv, smem + A_V, LDV);
       IOH::store_lds(rh, smem + A_H, LDK);
       IOH::store_lds(rdh, smem + A_DH, LDK);
-      if constexpr (GDN) IOV::store_lds(rn, smem + A_DVN, LDV);
+      if constexpr (GDN) {
+        IOV::mask(rn, ci.len);
+        IOV::store_lds(rn, smem + A_DVN, LDV);
+      }
       lds_barrier();
       if (vv + BVH < V) issueA(it, vv + BVH); else issueQK(it);
       gemm<T, 1, 4, false, false>(dP, smem + A_DO, LDV, 16 * wv, smem + A_V, LDV, 0, 0, BVH);
@@ -326,11 +352,13 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dqk(const lmoe_args a) {
     hdh = wave_sum(hdh);
     if (l == 0) s_red[wv] = hdh;
     // phase B operands
-    gate_finish(a, graw, s_b, s_eb, s_ed);
+    gate_finish(a, graw, ci.len, s_b, s_eb, s_ed);
+    IOK::mask(rq, ci.len);
+    IOK::mask(rk, ci.len);
     IOK::store_lds(rq, smem + B_Q, LDK);
     IOK::store_lds(rk, smem + B_K, LDK);
     lds_barrier();
-    if (it + gridDim.x < nitems) issueA(it + gridDim.x, 0);
+    issueA(min(it + (int)gridDim.x, nitems - 1), 0);
 #pragma unroll
     for (int nj = 0; nj < 4; ++nj) {
       f32x4 p;

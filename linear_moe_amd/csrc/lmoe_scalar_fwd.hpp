@@ -17,9 +17,9 @@ namespace lmoe {
 //   wave w owns state rows [w*K/4, (w+1)*K/4) x BV columns (fp32 MFMA accumulators).
 //   Per chunk, on the dependency chain of S:   S -> LDS (element type T)  | barrier |
 //   v_new = u - w S -> LDS | barrier | S = e^{b_C} S + (k e_d)^T v_new.
-//   Off the chain: the operands of chunk c+1 sit in registers while chunk c is computed and go
-//   to the other LDS buffer at the end of the step, the loads of chunk c+2 are issued right
-//   after; hs (layout [V][K]) and v_new are written with 16-byte stores from LDS.
+//   Off the chain: the operands of the next three chunks are in flight in registers; at the end
+//   of a step the next chunk goes to the other LDS buffer and its register set is refilled;
+//   hs (layout [V][K]) and v_new are written with 16-byte stores from LDS.
 //   Every wave forms the gate cumsum of a chunk for itself (lane j = token j).
 // ------------------------------------------------------------------------- //
 template <typename T, int K, int V, int BV, bool GDN>
@@ -59,24 +59,33 @@ __global__ __launch_bounds__(NTHR) void k_state_fwd(const lmoe_args a) {
   typedef TileIO<T, CH, K> IOK;
   typedef TileIO<T, CH, BV> IOV;
   typedef TileIO<T, BV, K> IOHT;
-  typename IOK::Regs rk, rw;
-  typename IOV::Regs ru;
-  uint32_t graw = 0;
+  // PF chunks of operands are in flight in registers (ring of PF sets, statically indexed)
+  constexpr int PF = 3;
+  struct Pre { typename IOK::Regs rk, rw; typename IOV::Regs ru; uint32_t graw; int len; };
+  Pre pre[PF];
   const lmoe_tensor& us = GDN ? a.u : a.v;
   const bool gated = a.gate != LMOE_GATE_NONE && a.g.ptr != nullptr;
 
-  auto issue = [&](int c) {
+  // Always issued (chunk index clamped to the last chunk; the few surplus loads at the end of a
+  // sequence are never consumed): a prefetch that is skipped on some path would force the
+  // compiler to drain all outstanding loads at every consumer.
+  const void* gptr = gated ? a.g.ptr : a.k.ptr;
+  auto issue = [&](Pre& P, int c) {
+    c = min(c, sq.nchunks - 1);
     const int tok = sq.tok0 + c * CH;
     const int len = min(CH, sq.len - c * CH);
-    IOK::load(rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, len);
-    if constexpr (GDN) IOK::load(rw, row_ptr<T>(a.w, sq.b, tok, h), a.w.st, len);
-    IOV::load(ru, row_ptr<T>(us, sq.b, tok, h) + v0, us.st, len);
-    graw = 0;
-    if (gated && l < len) graw = load_scalar_raw(a.g.ptr, a.g_dtype, row_off(a.g, sq.b, tok + l, h));
+    IOK::load_nomask(P.rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, len);
+    if constexpr (GDN) IOK::load_nomask(P.rw, row_ptr<T>(a.w, sq.b, tok, h), a.w.st, len);
+    IOV::load_nomask(P.ru, row_ptr<T>(us, sq.b, tok, h) + v0, us.st, len);
+    P.len = len;
+    P.graw = load_scalar_raw(gptr, a.g_dtype, gated ? row_off(a.g, sq.b, tok + min(l, len - 1), h) : 0);
   };
   // registers -> LDS buffer `buf`; returns e^{b_C} of that chunk
-  auto stage = [&](int buf) -> float {
-    const float x = wave_incl_scan(scalar_from_raw(graw, a.g_dtype));
+  auto stage = [&](Pre& P, int buf) -> float {
+    IOK::mask(P.rk, P.len);
+    if constexpr (GDN) IOK::mask(P.rw, P.len);
+    IOV::mask(P.ru, P.len);
+    const float x = wave_incl_scan((gated && l < P.len) ? scalar_from_raw(P.graw, a.g_dtype) : 0.f);
     const float xl = __shfl(x, 63, 64);
     const float ed = expf(xl - x);                        // lane j: e^{b_C - b_j}
 #pragma unroll
@@ -85,68 +94,74 @@ __global__ __launch_bounds__(NTHR) void k_state_fwd(const lmoe_args a) {
       const float sc = __shfl(ed, row, 64);
       typename IOK::vec o;
 #pragma unroll
-      for (int i = 0; i < IOK::VEC; ++i) o[i] = ET<T>::from_f(ET<T>::to_f(rk.v[p][i]) * sc);
+      for (int i = 0; i < IOK::VEC; ++i) o[i] = ET<T>::from_f(ET<T>::to_f(P.rk.v[p][i]) * sc);
       *(typename IOK::vec*)(&s_kd[buf][row * LDK + col]) = o;
     }
-    if constexpr (GDN) IOK::store_lds(rw, s_w[buf], LDK);
-    IOV::store_lds(ru, s_u[buf], LDU);
+    if constexpr (GDN) IOK::store_lds(P.rw, s_w[buf], LDK);
+    IOV::store_lds(P.ru, s_u[buf], LDU);
     return expf(xl);
   };
 
   float dec_cur = 1.f;
   if (sq.nchunks > 0) {
-    issue(0);
-    dec_cur = stage(0);
-    if (sq.nchunks > 1) issue(1);
+#pragma unroll
+    for (int j = 0; j < PF; ++j) issue(pre[j], j);
+    dec_cur = stage(pre[0], 0);
+    issue(pre[0], PF);
   }
-  for (int c = 0; c < sq.nchunks; ++c) {
-    const int cur = NBUF == 2 ? (c & 1) : 0;
-    const int tok = sq.tok0 + c * CH;
-    const int len = min(CH, sq.len - c * CH);
-    // S (state at chunk start) -> LDS as S^T
+  for (int c0 = 0; c0 < sq.nchunks; c0 += PF) {
 #pragma unroll
-    for (int mi = 0; mi < MB; ++mi)
+    for (int j = 0; j < PF; ++j) {
+      const int c = c0 + j;
+      if (c >= sq.nchunks) break;
+      const int cur = NBUF == 2 ? (c & 1) : 0;
+      const int tok = sq.tok0 + c * CH;
+      const int len = min(CH, sq.len - c * CH);
+      // S (state at chunk start) -> LDS as S^T
 #pragma unroll
-      for (int ni = 0; ni < NB; ++ni) acc_to_lds_t<T>(S[mi][ni], s_hT, LDK, krow0 + 16 * mi, 16 * ni);
-    lds_barrier();
-    // hs[chunk][h][v0 .. v0+BV][K] <- S^T   (off the dependency chain)
-    IOHT::lds_to_global(s_hT, LDK, (T*)a.hs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
-    if constexpr (GDN) {
-      // v_new = u - w S  (rows 16*wv .. +15 of the chunk)
-      f32x4 vn[1][NB];
-      acc_zero(vn);
-      gemm<T, 1, NB, false, false>(vn, s_w[cur], LDK, 16 * wv, s_hT, LDK, 0, 0, K);
+      for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
-      for (int ni = 0; ni < NB; ++ni) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
-          // round once to the storage type so that the state update and the output kernel see
-          // the same v_new
-          vn[0][ni][i] = ET<T>::to_f(ET<T>::from_f(ET<T>::to_f(s_u[cur][r * LDU + cc]) - vn[0][ni][i]));
-        }
-        acc_to_lds_t<T>(vn[0][ni], s_vT, LDC, 16 * wv, 16 * ni);
-      }
+        for (int ni = 0; ni < NB; ++ni) acc_to_lds_t<T>(S[mi][ni], s_hT, LDK, krow0 + 16 * mi, 16 * ni);
       lds_barrier();
+      // hs[chunk][h][v0 .. v0+BV][K] <- S^T   (off the dependency chain)
+      IOHT::lds_to_global(s_hT, LDK, (T*)a.hs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
+      if constexpr (GDN) {
+        // v_new = u - w S  (rows 16*wv .. +15 of the chunk)
+        f32x4 vn[1][NB];
+        acc_zero(vn);
+        gemm<T, 1, NB, false, false>(vn, s_w[cur], LDK, 16 * wv, s_hT, LDK, 0, 0, K);
 #pragma unroll
-      for (int mi = 0; mi < MB; ++mi)
+        for (int ni = 0; ni < NB; ++ni) {
 #pragma unroll
-        for (int ni = 0; ni < NB; ++ni) S[mi][ni] *= dec_cur;
-      gemm<T, MB, NB, true, false>(S, s_kd[cur], LDK, krow0, s_vT, LDC, 0, 0, CH);
-      store_strip<T, NB>(vn, s_stg + wv * 16 * LDU, row_ptr<T>(a.vnew, sq.b, tok + 16 * wv, h) + v0, a.vnew.st,
-                         len - 16 * wv, 1.0f);
-    } else {
+          for (int i = 0; i < 4; ++i) {
+            const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
+            // round once to the storage type so that the state update and the output kernel see
+            // the same v_new
+            vn[0][ni][i] = ET<T>::to_f(ET<T>::from_f(ET<T>::to_f(s_u[cur][r * LDU + cc]) - vn[0][ni][i]));
+          }
+          acc_to_lds_t<T>(vn[0][ni], s_vT, LDC, 16 * wv, 16 * ni);
+        }
+        lds_barrier();
 #pragma unroll
-      for (int mi = 0; mi < MB; ++mi)
+        for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < NB; ++ni) S[mi][ni] *= dec_cur;
-      gemm<T, MB, NB, true, true>(S, s_kd[cur], LDK, krow0, s_u[cur], LDU, 0, 0, CH);
-    }
-    // stage the next chunk (its loads were issued one step ago) and fetch the one after
-    if (c + 1 < sq.nchunks) {
-      if constexpr (NBUF == 1) lds_barrier();       // single buffer: wait until it has been read
-      dec_cur = stage(NBUF == 2 ? (cur ^ 1) : 0);
-      if (c + 2 < sq.nchunks) issue(c + 2);
+          for (int ni = 0; ni < NB; ++ni) S[mi][ni] *= dec_cur;
+        gemm<T, MB, NB, true, false>(S, s_kd[cur], LDK, krow0, s_vT, LDC, 0, 0, CH);
+        store_strip<T, NB>(vn, s_stg + wv * 16 * LDU, row_ptr<T>(a.vnew, sq.b, tok + 16 * wv, h) + v0, a.vnew.st,
+                           len - 16 * wv, 1.0f);
+      } else {
+#pragma unroll
+        for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+          for (int ni = 0; ni < NB; ++ni) S[mi][ni] *= dec_cur;
+        gemm<T, MB, NB, true, true>(S, s_kd[cur], LDK, krow0, s_u[cur], LDU, 0, 0, CH);
+      }
+      // stage the next chunk (its loads were issued PF steps ago) and refill its register set
+      if (c + 1 < sq.nchunks) {
+        if constexpr (NBUF == 1) lds_barrier();       // single buffer: wait until it has been read
+        dec_cur = stage(pre[(j + 1) % PF], NBUF == 2 ? (cur ^ 1) : 0);
+        issue(pre[(j + 1) % PF], c + 1 + PF);
+      }
     }
   }
 
@@ -198,28 +213,31 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_out_fwd(cons
   auto issue = [&](int it) {
     const int cid = it / a.H, h = it % a.H;
     const ChunkInfo ci = chunk_info(a, cid);
-    IOK::load(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
-    IOK::load(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
-    IOH::load(rh, (const T*)a.hs + ((int64_t)cid * a.H + h) * K * V, K, V);
+    IOK::load_nomask(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
+    IOK::load_nomask(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
+    IOH::load_nomask(rh, (const T*)a.hs + ((int64_t)cid * a.H + h) * K * V, K, V);
     graw = gate_prefetch(a, ci.b, ci.tok, ci.len, h);
   };
   auto issue_v = [&](int it) {
     const int cid = it / a.H, h = it % a.H;
     const ChunkInfo ci = chunk_info(a, cid);
-    IOV::load(rv, row_ptr<T>(vs, ci.b, ci.tok, h), vs.st, ci.len);
+    IOV::load_nomask(rv, row_ptr<T>(vs, ci.b, ci.tok, h), vs.st, ci.len);
   };
+  // prefetches are always issued (item index clamped): see k_state_fwd
   int it = blockIdx.x;
   if (it < nitems) { issue(it); issue_v(it); }
   for (; it < nitems; it += gridDim.x) {
     const int cid = it / a.H, h = it % a.H;
     const ChunkInfo ci = chunk_info(a, cid);
-    const int nxt = it + gridDim.x;
-    gate_finish(a, graw, s_b, s_eb, nullptr);
+    const int nxt = min(it + (int)gridDim.x, nitems - 1);
+    gate_finish(a, graw, ci.len, s_b, s_eb, nullptr);
+    IOK::mask(rq, ci.len);
+    IOK::mask(rk, ci.len);
     IOK::store_lds(rq, s_q, LDK);
     IOK::store_lds(rk, s_k, LDK);
     IOH::store_lds(rh, s_h, LDK);
     lds_barrier();
-    if (nxt < nitems) issue(nxt);
+    issue(nxt);
     f32x4 s[1][4];
     acc_zero(s);
     gemm<T, 1, 4, false, false>(s, s_q, LDK, 16 * wv, s_k, LDK, 0, 0, K);
@@ -227,8 +245,9 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_out_fwd(cons
     acc_zero(o);
     gemm<T, 1, NB, false, false>(o, s_q, LDK, 16 * wv, s_h, LDK, 0, 0, K);
     lds_barrier();            // every wave is done reading k and S: P^T and v' may overlay them
+    IOV::mask(rv, ci.len);
     IOV::store_lds(rv, s_v, LDV);
-    if (nxt < nitems) issue_v(nxt);
+    issue_v(nxt);
 #pragma unroll
     for (int nj = 0; nj < 4; ++nj) {
       f32x4 p;

@@ -91,15 +91,16 @@ __device__ __forceinline__ void chunk_gate_cumsum(const lmoe_args& a, int b, int
 // of a chunk's log-decays (lanes 0..63 of wave 0 hold one token each, raw bits), gate_finish
 // turns them into the LDS arrays later.  Neither contains a barrier.
 __device__ __forceinline__ uint32_t gate_prefetch(const lmoe_args& a, int b, int tok, int len, int h) {
-  uint32_t raw = 0;
-  if (threadIdx.x < 64 && a.gate != LMOE_GATE_NONE && a.g.ptr != nullptr && (int)threadIdx.x < len)
-    raw = load_scalar_raw(a.g.ptr, a.g_dtype, row_off(a.g, b, tok + threadIdx.x, h));
-  return raw;
+  // branch-free: an ungated call reads a dummy word of k, tokens past the end re-read the last one
+  const bool gated = a.gate != LMOE_GATE_NONE && a.g.ptr != nullptr;
+  const int j = min((int)(threadIdx.x & 63), len - 1);
+  return load_scalar_raw(gated ? a.g.ptr : a.k.ptr, a.g_dtype, gated ? row_off(a.g, b, tok + j, h) : 0);
 }
-__device__ __forceinline__ void gate_finish(const lmoe_args& a, uint32_t raw, float* sb, float* seb, float* sed) {
+__device__ __forceinline__ void gate_finish(const lmoe_args& a, uint32_t raw, int len, float* sb, float* seb, float* sed) {
   if (threadIdx.x < 64) {
     const int j = threadIdx.x;
-    const float x = wave_incl_scan(scalar_from_raw(raw, a.g_dtype));
+    const bool gated = a.gate != LMOE_GATE_NONE && a.g.ptr != nullptr;
+    const float x = wave_incl_scan((gated && j < len) ? scalar_from_raw(raw, a.g_dtype) : 0.f);
     const float xl = __shfl(x, 63, 64);
     if (sb) sb[j] = x;
     if (seb) seb[j] = expf(x);
