@@ -241,8 +241,10 @@ template <typename T, int ROWS, int COLS> struct TileIO {
   typedef typename ET<T>::vec vec;
   struct Regs { vec v[PASSES]; };
 
+  // thread index inside a team of 256: work-groups of 512 threads use two teams (waves 0-3 and
+  // 4-7) that each move whole tiles
   static __device__ __forceinline__ void coords(int p, int& row, int& col) {
-    const int idx = p * NTHR + threadIdx.x;
+    const int idx = p * NTHR + (threadIdx.x & (NTHR - 1));
     row = idx / VPR; col = (idx % VPR) * VEC;
   }
   // Branch-free loads: rows >= nvalid (nvalid >= 1) re-read the last valid row, so that no load

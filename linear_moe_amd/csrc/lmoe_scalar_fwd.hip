@@ -6,7 +6,7 @@ namespace lmoe {
 
 // V-slice of the sequential state pass and of the output kernel
 template <typename T, int V> struct FwdTiles {
-  static constexpr int BVS = 32;
+  static constexpr int BVS = sizeof(T) == 4 ? 16 : 32;
   static constexpr int BVO = V == 128 ? 64 : V;
 };
 
@@ -15,7 +15,7 @@ template <bool GDN> struct StateFwd {
     static void run(const lmoe_args& a, hipStream_t st) {
       constexpr int BV = FwdTiles<T, V>::BVS;
       const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BV);
-      hipLaunchKernelGGL((k_state_fwd<T, K, V, BV, GDN>), dim3(grid), dim3(NTHR), 0, st, a);
+      hipLaunchKernelGGL((k_state_fwd<T, K, V, BV, GDN>), dim3(grid), dim3(2 * NTHR), 0, st, a);
     }
   };
 };
