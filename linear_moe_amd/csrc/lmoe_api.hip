@@ -123,7 +123,6 @@ int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream) {
   if (!a->d_o.ptr || !a->dq.ptr || !a->dk.ptr || !a->dv.ptr || !a->dg.ptr || !a->dbeta.ptr)
     return fail(-13, "%s: d_o, dq, dk, dv, dg and dbeta must not be null", op);
   if (a->NT == 0 || a->N == 0) return 0;
-  lmoe::launch_bwd_dv(*a, true, (hipStream_t)stream);
   lmoe::launch_state_bwd(*a, true, (hipStream_t)stream);
   lmoe::launch_bwd_dqk(*a, true, (hipStream_t)stream);
   lmoe::launch_gdn_wy_bwd(*a, (hipStream_t)stream);
@@ -142,7 +141,8 @@ int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* strea
         lmoe::launch_gdn_wy_fwd(*a, st); break;
       case lmoe::ST_STATE_FWD: lmoe::launch_state_fwd(*a, gdn, st); break;
       case lmoe::ST_OUT_FWD: lmoe::launch_out_fwd(*a, gdn, st); break;
-      case lmoe::ST_DV: lmoe::launch_bwd_dv(*a, gdn, st); break;
+      case lmoe::ST_DV: if (gdn) return fail(-20, "%s: the delta rule forms dv inside its state pass", nm);
+        lmoe::launch_bwd_dv(*a, false, st); break;
       case lmoe::ST_STATE_BWD: lmoe::launch_state_bwd(*a, gdn, st); break;
       case lmoe::ST_DQK: lmoe::launch_bwd_dqk(*a, gdn, st); break;
       case lmoe::ST_GDN_WY_BWD: if (!gdn) return fail(-20, "%s: stage not part of this op", nm);

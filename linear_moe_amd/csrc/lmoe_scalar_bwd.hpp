@@ -3,9 +3,10 @@
 // Gamma_ij = e^{b_i - b_j} [i >= j], P = (q k^T) . Gamma, S = state at chunk start,
 // dS' = gradient w.r.t. the state at chunk end, v' = v (simple_gla) or v_new (delta rule).
 //
-//   k_bwd_dv    : chunk-parallel   dv' = scale P^T do (+ (k . e_d) dS'  unless LOCAL)
+//   k_bwd_dv    : chunk-parallel   dv = scale P^T do + (k . e_d) dS'     (simple_gla only)
 //   k_state_bwd : reverse sequential pass over the chunks of one (sequence, head, V-slice):
-//                 writes dS' of every chunk (dhs); delta rule: dv_new = dv_loc + (k . e_d) dS';
+//                 writes dS' of every chunk (dhs); delta rule: dv_new = dv_loc + (k . e_d) dS'
+//                 with dv_loc = scale P^T do formed in the same kernel;
 //                 dS = e^{b_C} dS' + scale (q . e_b)^T do  (- w^T dv_new)
 //   k_bwd_dqk   : chunk-parallel   dq, dk (delta rule: the part of dk that does not go through
 //                 the WY factors, and dw = -dv_new S^T), gate gradient
@@ -90,27 +91,43 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dv(const lmoe_args a) {
 }
 
 // ------------------------------------------------------------------------- //
-// reverse state pass, software-pipelined (mirror of k_state_fwd)
+// reverse state pass: producer / consumer work-group of 512 threads (mirror of k_state_fwd)
 //   grid = ceil(N*H / 8) * 8 * (V / BV) work-groups (1-D); V-slices of one (sequence, head)
-//   share an XCD.  dS slice [K x BV] lives in fp32 MFMA accumulators.
-//   Chain per chunk:  dS' -> LDS | barrier | dv_new = dv_loc + (k e_d) dS' -> LDS | barrier |
-//                     dS = e^{b_C} dS' + (scale q e_b)^T do - w^T dv_new.
-//   dhs (layout [V][K]) and dv_new leave through LDS with 16-byte stores; the operands of the
-//   next chunk are prefetched into registers and staged into the other LDS buffer.
+//   share an XCD.  dS slice [K x BV] lives in fp32 MFMA accumulators of waves 0-3 (consumers):
+//        dS' -> LDS | B1 | dv_new = dv_loc + e_d (k dS') -> LDS | B2 |
+//        dS = e^{b_C} dS' + q^T (scale e_b do) - w^T dv_new
+//   Waves 4-7 (producers) keep the next chunks' q, k, w, do in flight, stage them unscaled, write
+//   dhs (layout [V][K]) and, for the delta rule, compute the local part of dv_new for the next
+//   step themselves:  dv_loc = scale ((q k^T) . Gamma)^T do  (each producer wave: 16 rows of it,
+//   P^T through a wave-private LDS strip), so no separate dv kernel runs for that op.
 // ------------------------------------------------------------------------- //
+template <typename T> __device__ __forceinline__ void scale_frag(typename ET<T>::frag& f, const float* s8) {
+  const f32x4 s0 = *(const f32x4*)s8, s1 = *(const f32x4*)(s8 + 4);
+  if constexpr (sizeof(T) == 2) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { f[i] = (bf16)((float)f[i] * s0[i]); f[i + 4] = (bf16)((float)f[i + 4] * s1[i]); }
+  } else {
+    f.lo *= s0; f.hi *= s1;
+  }
+}
+
 template <typename T, int K, int V, int BV, bool GDN>
-__global__ __launch_bounds__(NTHR) void k_state_bwd(const lmoe_args a) {
+__global__ __launch_bounds__(2 * NTHR) void k_state_bwd(const lmoe_args a) {
   constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDU = BV + LPAD;
   constexpr int MB = K / 64, NB = BV / 16;
+  // bf16: two operand buffers; fp32 (the parity path) has LDS for one and pays extra barriers
   constexpr int NBUF = sizeof(T) == 2 ? 2 : 1;
-  __shared__ __attribute__((aligned(16))) T s_qs[NBUF][CH * LDK];            // scale q e_b    [64][K]
-  __shared__ __attribute__((aligned(16))) T s_do[NBUF][CH * LDU];            // do             [64][BV]
-  __shared__ __attribute__((aligned(16))) T s_kd[NBUF][GDN ? CH * LDK : 8];  // k e_d          [64][K]
-  __shared__ __attribute__((aligned(16))) T s_w[NBUF][GDN ? CH * LDK : 8];   // w              [64][K]
-  __shared__ __attribute__((aligned(16))) T s_dvl[NBUF][GDN ? CH * LDU : 8]; // dv_loc         [64][BV]
-  __shared__ __attribute__((aligned(16))) T s_dST[BV * LDK];                 // dS'^T          [BV][K]
-  __shared__ __attribute__((aligned(16))) T s_dvT[GDN ? BV * LDC : 8];       // -dv_new^T      [BV][64]
-  __shared__ __attribute__((aligned(16))) T s_stg[GDN ? 4 * 16 * LDU : 8];
+  __shared__ __attribute__((aligned(16))) T s_q[NBUF][CH * LDK];             // q       [64][K]
+  __shared__ __attribute__((aligned(16))) T s_do[NBUF][CH * LDU];            // do      [64][BV]
+  __shared__ __attribute__((aligned(16))) T s_k[NBUF][GDN ? CH * LDK : 8];   // k       [64][K]
+  __shared__ __attribute__((aligned(16))) T s_w[NBUF][GDN ? CH * LDK : 8];   // w       [64][K]
+  __shared__ __attribute__((aligned(16))) T s_dvl[NBUF][GDN ? CH * LDU : 8]; // dv_loc  [64][BV]
+  __shared__ __attribute__((aligned(16))) T s_dST[BV * LDK];                 // dS'^T   [BV][K]
+  __shared__ __attribute__((aligned(16))) T s_dvT[GDN ? BV * LDC : 8];       // -dv_new^T [BV][64]
+  __shared__ __attribute__((aligned(16))) T s_pt[GDN ? 4 * 16 * LDC : 8];    // producers: P^T strips
+  __shared__ __attribute__((aligned(16))) T s_stg[GDN ? 4 * 16 * LDU : 8];   // consumers: dv_new store
+  __shared__ __attribute__((aligned(16))) float s_b[NBUF][64], s_qs[NBUF][64], s_ed[NBUF][64];
+  __shared__ float s_dec[NBUF];
 
   constexpr int NVS = V / BV;
   const int xcd = blockIdx.x & 7, jj = blockIdx.x >> 3;
@@ -118,9 +135,129 @@ __global__ __launch_bounds__(NTHR) void k_state_bwd(const lmoe_args a) {
   if (pair >= a.N * a.H) return;
   const int v0 = vsl * BV, h = pair % a.H, n = pair / a.H;
   const SeqInfo sq = seq_info(a, n);
-  const int wv = wave_id(), l = lane_id();
-  const int krow0 = wv * (K / 4);
+  const int l = lane_id();
+  const bool producer = threadIdx.x >= NTHR;
+  if (sq.nchunks == 0) {
+    if (a.dh0 && !producer) {
+      for (int idx = threadIdx.x; idx < K * BV; idx += NTHR) {
+        const int r = idx / BV, c = v0 + idx % BV;
+        const int64_t o = ((int64_t)n * a.H + h) * K * V + (int64_t)r * V + c;
+        a.dh0[o] = a.dht ? a.dht[o] : 0.f;
+      }
+    }
+    return;
+  }
+  typedef TileIO<T, CH, K> IOK;
+  typedef TileIO<T, CH, BV> IOV;
+  typedef TileIO<T, BV, K> IOHT;
 
+  if (producer) {
+    // ------------------------------- producers -------------------------------------------
+    constexpr int PF = 2;
+    struct Pre { typename IOK::Regs rq, rk, rw; typename IOV::Regs rd; uint32_t graw; int len; };
+    Pre pre[PF];
+    const int pw = wave_id() - 4;
+    const bool gated = a.gate != LMOE_GATE_NONE && a.g.ptr != nullptr;
+    const void* gptr = gated ? a.g.ptr : a.k.ptr;
+    const float scale = a.scale;
+    // always issued, chunk index clamped (see k_state_fwd)
+    auto issue = [&](Pre& P, int c) {
+      c = max(c, 0);
+      const int tok = sq.tok0 + c * CH;
+      const int len = min(CH, sq.len - c * CH);
+      IOK::load_nomask(P.rq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, len);
+      IOV::load_nomask(P.rd, row_ptr<T>(a.d_o, sq.b, tok, h) + v0, a.d_o.st, len);
+      if constexpr (GDN) {
+        IOK::load_nomask(P.rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, len);
+        IOK::load_nomask(P.rw, row_ptr<T>(a.w, sq.b, tok, h), a.w.st, len);
+      }
+      P.len = len;
+      P.graw = load_scalar_raw(gptr, a.g_dtype, gated ? row_off(a.g, sq.b, tok + min(l, len - 1), h) : 0);
+    };
+    auto stage = [&](Pre& P, int buf) {
+      IOK::mask(P.rq, P.len);
+      IOV::mask(P.rd, P.len);
+      IOK::store_lds(P.rq, s_q[buf], LDK);
+      IOV::store_lds(P.rd, s_do[buf], LDU);
+      if constexpr (GDN) {
+        IOK::mask(P.rk, P.len);
+        IOK::mask(P.rw, P.len);
+        IOK::store_lds(P.rk, s_k[buf], LDK);
+        IOK::store_lds(P.rw, s_w[buf], LDK);
+      }
+      if (pw == 0) {
+        const float x = wave_incl_scan((gated && l < P.len) ? scalar_from_raw(P.graw, a.g_dtype) : 0.f);
+        const float xl = __shfl(x, 63, 64);
+        s_b[buf][l] = x;
+        s_qs[buf][l] = scale * expf(x);
+        s_ed[buf][l] = expf(xl - x);
+        if (l == 0) s_dec[buf] = expf(xl);
+      }
+    };
+    // local part of dv_new of the chunk staged in `buf`: rows 16 pw .. 16 pw + 15
+    auto dv_local = [&](int buf) {
+      if constexpr (GDN) {
+        T* pt = s_pt + pw * 16 * LDC;
+        f32x4 p[1][4];
+        acc_zero(p);
+        gemm<T, 1, 4, false, false>(p, s_k[buf], LDK, 16 * pw, s_q[buf], LDK, 0, 0, K);   // p[j][i] = k_j . q_i
+#pragma unroll
+        for (int ni = 0; ni < 4; ++ni) {
+          f32x4 x;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int j = 16 * pw + 4 * (l >> 4) + e, i = 16 * ni + (l & 15);
+            x[e] = (i >= j) ? p[0][ni][e] * texp<T>(s_b[buf][i] - s_b[buf][j]) : 0.f;
+          }
+          acc_to_lds<T>(x, pt, LDC, 0, 16 * ni);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        f32x4 d[1][NB];
+        acc_zero(d);
+        gemm<T, 1, NB, false, true>(d, pt, LDC, 0, s_do[buf], LDU, 0, 0, CH);
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) {
+          d[0][ni] *= scale;
+          acc_to_lds<T>(d[0][ni], s_dvl[buf], LDU, 16 * pw, 16 * ni);
+        }
+      }
+    };
+#pragma unroll
+    for (int j = 0; j < PF; ++j) issue(pre[j], sq.nchunks - 1 - j);
+    stage(pre[0], 0);
+    issue(pre[0], sq.nchunks - 1 - PF);
+    lds_barrier();                                   // P0: the first chunk's tiles are complete
+    dv_local(0);
+    for (int it0 = 0; it0 < sq.nchunks; it0 += PF) {
+#pragma unroll
+      for (int j = 0; j < PF; ++j) {
+        const int it = it0 + j;
+        if (it >= sq.nchunks) break;
+        const int c = sq.nchunks - 1 - it;
+        const int nb = NBUF == 2 ? ((it + 1) & 1) : 0;
+        lds_barrier();                                                                   // B1
+        IOHT::lds_to_global(s_dST, LDK, (T*)a.dhs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
+        if constexpr (NBUF == 2) {
+          if (c > 0) stage(pre[(j + 1) % PF], nb);
+        }
+        lds_barrier();                                                                   // B2
+        if constexpr (NBUF == 1) {
+          lds_barrier();                                                                 // B3: buffer read
+          if (c > 0) stage(pre[(j + 1) % PF], 0);
+          lds_barrier();                                                                 // B4: tiles complete
+        }
+        if (c > 0) dv_local(nb);
+        issue(pre[(j + 1) % PF], c - 1 - PF);
+      }
+    }
+    return;
+  }
+
+  // --------------------------------- consumers -------------------------------------------
+  const int wv = wave_id();
+  const int krow0 = wv * (K / 4);
   f32x4 dS[MB][NB];
   acc_zero(dS);
   if (a.dht) {
@@ -133,81 +270,8 @@ __global__ __launch_bounds__(NTHR) void k_state_bwd(const lmoe_args a) {
         for (int i = 0; i < 4; ++i)
           dS[mi][ni][i] = p[(int64_t)(krow0 + acc_row(mi, i)) * V + v0 + acc_col(ni)];
   }
-  typedef TileIO<T, CH, K> IOK;
-  typedef TileIO<T, CH, BV> IOV;
-  typedef TileIO<T, BV, K> IOHT;
-  // PF chunks of operands are in flight in registers (ring of PF sets, statically indexed);
-  // prefetches are always issued with a clamped chunk index (see k_state_fwd)
-  constexpr int PF = 2;
-  struct Pre { typename IOK::Regs rq, rk, rw; typename IOV::Regs rd, rl; uint32_t graw; int len; };
-  Pre pre[PF];
-  const bool gated = a.gate != LMOE_GATE_NONE && a.g.ptr != nullptr;
-  const void* gptr = gated ? a.g.ptr : a.k.ptr;
-  const float scale = a.scale;
-
-  auto issue = [&](Pre& P, int c) {
-    c = max(c, 0);
-    const int tok = sq.tok0 + c * CH;
-    const int len = min(CH, sq.len - c * CH);
-    IOK::load_nomask(P.rq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, len);
-    IOV::load_nomask(P.rd, row_ptr<T>(a.d_o, sq.b, tok, h) + v0, a.d_o.st, len);
-    if constexpr (GDN) {
-      IOK::load_nomask(P.rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, len);
-      IOK::load_nomask(P.rw, row_ptr<T>(a.w, sq.b, tok, h), a.w.st, len);
-      IOV::load_nomask(P.rl, row_ptr<T>(a.dvnew, sq.b, tok, h) + v0, a.dvnew.st, len);
-    }
-    P.len = len;
-    P.graw = load_scalar_raw(gptr, a.g_dtype, gated ? row_off(a.g, sq.b, tok + min(l, len - 1), h) : 0);
-  };
-  auto stage = [&](Pre& P, int buf) -> float {
-    IOK::mask(P.rq, P.len);
-    IOV::mask(P.rd, P.len);
-    if constexpr (GDN) {
-      IOK::mask(P.rk, P.len);
-      IOK::mask(P.rw, P.len);
-      IOV::mask(P.rl, P.len);
-    }
-    typename IOK::Regs& rq = P.rq; typename IOK::Regs& rk = P.rk; typename IOK::Regs& rw = P.rw;
-    typename IOV::Regs& rd = P.rd; typename IOV::Regs& rl = P.rl;
-    const float x = wave_incl_scan((gated && l < P.len) ? scalar_from_raw(P.graw, a.g_dtype) : 0.f);
-    const float xl = __shfl(x, 63, 64);
-    const float qs = scale * expf(x);                     // lane j: scale e^{b_j}
-    const float ed = expf(xl - x);                        // lane j: e^{b_C - b_j}
-#pragma unroll
-    for (int p = 0; p < IOK::PASSES; ++p) {
-      int row, col; IOK::coords(p, row, col);
-      const float sq_ = __shfl(qs, row, 64);
-      typename IOK::vec o;
-#pragma unroll
-      for (int i = 0; i < IOK::VEC; ++i) o[i] = ET<T>::from_f(ET<T>::to_f(rq.v[p][i]) * sq_);
-      *(typename IOK::vec*)(&s_qs[buf][row * LDK + col]) = o;
-      if constexpr (GDN) {
-        const float se = __shfl(ed, row, 64);
-#pragma unroll
-        for (int i = 0; i < IOK::VEC; ++i) o[i] = ET<T>::from_f(ET<T>::to_f(rk.v[p][i]) * se);
-        *(typename IOK::vec*)(&s_kd[buf][row * LDK + col]) = o;
-      }
-    }
-    IOV::store_lds(rd, s_do[buf], LDU);
-    if constexpr (GDN) {
-      IOK::store_lds(rw, s_w[buf], LDK);
-      IOV::store_lds(rl, s_dvl[buf], LDU);
-    }
-    return expf(xl);
-  };
-
-  float dec_cur = 1.f;
-  if (sq.nchunks > 0) {
-#pragma unroll
-    for (int j = 0; j < PF; ++j) issue(pre[j], sq.nchunks - 1 - j);
-    dec_cur = stage(pre[0], 0);
-    issue(pre[0], sq.nchunks - 1 - PF);
-  }
-  for (int it0 = 0; it0 < sq.nchunks; it0 += PF) {
-#pragma unroll
-   for (int j = 0; j < PF; ++j) {
-    const int it = it0 + j;
-    if (it >= sq.nchunks) break;
+  lds_barrier();                                     // P0
+  for (int it = 0; it < sq.nchunks; ++it) {
     const int c = sq.nchunks - 1 - it;
     const int cur = NBUF == 2 ? (it & 1) : 0;
     const int tok = sq.tok0 + c * CH;
@@ -216,42 +280,54 @@ __global__ __launch_bounds__(NTHR) void k_state_bwd(const lmoe_args a) {
     for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
       for (int ni = 0; ni < NB; ++ni) acc_to_lds_t<T>(dS[mi][ni], s_dST, LDK, krow0 + 16 * mi, 16 * ni);
-    lds_barrier();
-    IOHT::lds_to_global(s_dST, LDK, (T*)a.dhs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
+    lds_barrier();                                                                       // B1
+    const float dec = s_dec[cur];
     f32x4 t[1][NB];
     acc_zero(t);
     if constexpr (GDN) {
-      // dv_new = dv_loc + k_d dS'   (rows 16 wv .. of the chunk)
-      gemm<T, 1, NB, false, false>(t, s_kd[cur], LDK, 16 * wv, s_dST, LDK, 0, 0, K);
+      // dv_new = dv_loc + e_d (k dS')   (rows 16 wv .. of the chunk)
+      gemm<T, 1, NB, false, false>(t, s_k[cur], LDK, 16 * wv, s_dST, LDK, 0, 0, K);
 #pragma unroll
       for (int ni = 0; ni < NB; ++ni) {
         f32x4 x;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
-          t[0][ni][i] = ET<T>::to_f(ET<T>::from_f(ET<T>::to_f(s_dvl[cur][r * LDU + cc]) + t[0][ni][i]));
+          t[0][ni][i] = ET<T>::to_f(ET<T>::from_f(ET<T>::to_f(s_dvl[cur][r * LDU + cc]) + s_ed[cur][r] * t[0][ni][i]));
           x[i] = -t[0][ni][i];
         }
         acc_to_lds_t<T>(x, s_dvT, LDC, 16 * wv, 16 * ni);
       }
-      lds_barrier();
     }
+    lds_barrier();                                                                       // B2
 #pragma unroll
     for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
-      for (int ni = 0; ni < NB; ++ni) dS[mi][ni] *= dec_cur;
-    gemm<T, MB, NB, true, true>(dS, s_qs[cur], LDK, krow0, s_do[cur], LDU, 0, 0, CH);
+      for (int ni = 0; ni < NB; ++ni) dS[mi][ni] *= dec;
+    // dS += q^T (scale e_b do): the row scaling is applied to the do fragments in registers
+    for (int kk = 0; kk < CH; kk += 32) {
+      typename ET<T>::frag af[MB], bf[NB];
+#pragma unroll
+      for (int mi = 0; mi < MB; ++mi) af[mi] = ET<T>::load_frag_t(s_q[cur], LDK, kk, krow0 + 16 * mi);
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) {
+        bf[ni] = ET<T>::load_frag_t(s_do[cur], LDU, kk, 16 * ni);
+        scale_frag<T>(bf[ni], &s_qs[cur][kk + 8 * (l >> 4)]);
+      }
+#pragma unroll
+      for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) ET<T>::mma(dS[mi][ni], af[mi], bf[ni]);
+    }
     if constexpr (GDN) {
       gemm<T, MB, NB, true, false>(dS, s_w[cur], LDK, krow0, s_dvT, LDC, 0, 0, CH);
       store_strip<T, NB>(t, s_stg + wv * 16 * LDU, row_ptr<T>(a.dvnew, sq.b, tok + 16 * wv, h) + v0, a.dvnew.st,
                          len - 16 * wv, 1.0f);
     }
-    if (c > 0) {
-      if constexpr (NBUF == 1) lds_barrier();
-      dec_cur = stage(pre[(j + 1) % PF], NBUF == 2 ? (cur ^ 1) : 0);
-      issue(pre[(j + 1) % PF], c - 1 - PF);
+    if constexpr (NBUF == 1) {
+      lds_barrier();                                                                     // B3
+      lds_barrier();                                                                     // B4
     }
-   }
   }
   if (a.dh0) {
     float* p = a.dh0 + ((int64_t)n * a.H + h) * K * V;
