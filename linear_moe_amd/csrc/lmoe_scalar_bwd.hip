@@ -23,7 +23,7 @@ template <bool GDN> struct StateBwd {
     static void run(const lmoe_args& a, hipStream_t st) {
       constexpr int BV = BwdTiles<T, V>::BVS;
       const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BV);
-      hipLaunchKernelGGL((k_state_bwd<T, K, V, BV, GDN>), dim3(grid), dim3(2 * NTHR), 0, st, a);
+      hipLaunchKernelGGL((k_state_bwd<T, K, V, BV, GDN>), dim3(grid), dim3((GDN ? 3 : 2) * NTHR), 0, st, a);
     }
   };
 };

@@ -96,10 +96,11 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dv(const lmoe_args a) {
 //   share an XCD.  dS slice [K x BV] lives in fp32 MFMA accumulators of waves 0-3 (consumers):
 //        dS' -> LDS | B1 | dv_new = dv_loc + e_d (k dS') -> LDS | B2 |
 //        dS = e^{b_C} dS' + q^T (scale e_b do) - w^T dv_new
-//   Waves 4-7 (producers) keep the next chunks' q, k, w, do in flight, stage them unscaled, write
-//   dhs (layout [V][K]) and, for the delta rule, compute the local part of dv_new for the next
-//   step themselves:  dv_loc = scale ((q k^T) . Gamma)^T do  (each producer wave: 16 rows of it,
-//   P^T through a wave-private LDS strip), so no separate dv kernel runs for that op.
+//   Waves 4-7 (loaders) keep the next chunks' q, k, w, do in flight, stage them unscaled and write
+//   dhs (layout [V][K]).  For the delta rule waves 8-11 compute the local part of dv_new of the
+//   next step from the staged tiles:  dv_loc = scale ((q k^T) . Gamma)^T do  (each wave 16 rows of
+//   it, P^T through a wave-private LDS strip), so no separate dv kernel runs for that op.
+//   All teams meet at the same barriers; three waves per SIMD hide each other's latencies.
 // ------------------------------------------------------------------------- //
 template <typename T> __device__ __forceinline__ void scale_frag(typename ET<T>::frag& f, const float* s8) {
   const f32x4 s0 = *(const f32x4*)s8, s1 = *(const f32x4*)(s8 + 4);
@@ -112,7 +113,7 @@ template <typename T> __device__ __forceinline__ void scale_frag(typename ET<T>:
 }
 
 template <typename T, int K, int V, int BV, bool GDN>
-__global__ __launch_bounds__(2 * NTHR) void k_state_bwd(const lmoe_args a) {
+__global__ __launch_bounds__((GDN ? 3 : 2) * NTHR) void k_state_bwd(const lmoe_args a) {
   constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDU = BV + LPAD;
   constexpr int MB = K / 64, NB = BV / 16;
   // bf16: two operand buffers; fp32 (the parity path) has LDS for one and pays extra barriers
@@ -136,9 +137,10 @@ __global__ __launch_bounds__(2 * NTHR) void k_state_bwd(const lmoe_args a) {
   const int v0 = vsl * BV, h = pair % a.H, n = pair / a.H;
   const SeqInfo sq = seq_info(a, n);
   const int l = lane_id();
-  const bool producer = threadIdx.x >= NTHR;
+  const int team = threadIdx.x / NTHR;      // 0: consumers, 1: loaders, 2: local dv (delta rule)
+  const bool producer = team == 1;
   if (sq.nchunks == 0) {
-    if (a.dh0 && !producer) {
+    if (a.dh0 && team == 0) {
       for (int idx = threadIdx.x; idx < K * BV; idx += NTHR) {
         const int r = idx / BV, c = v0 + idx % BV;
         const int64_t o = ((int64_t)n * a.H + h) * K * V + (int64_t)r * V + c;
@@ -194,6 +196,40 @@ __global__ __launch_bounds__(2 * NTHR) void k_state_bwd(const lmoe_args a) {
         if (l == 0) s_dec[buf] = expf(xl);
       }
     };
+#pragma unroll
+    for (int j = 0; j < PF; ++j) issue(pre[j], sq.nchunks - 1 - j);
+    stage(pre[0], 0);
+    issue(pre[0], sq.nchunks - 1 - PF);
+    lds_barrier();                                   // P0: the first chunk's tiles are complete
+    if constexpr (GDN) lds_barrier();                // P1: its local dv is complete
+    for (int it0 = 0; it0 < sq.nchunks; it0 += PF) {
+#pragma unroll
+      for (int j = 0; j < PF; ++j) {
+        const int it = it0 + j;
+        if (it >= sq.nchunks) break;
+        const int c = sq.nchunks - 1 - it;
+        const int nb = NBUF == 2 ? ((it + 1) & 1) : 0;
+        lds_barrier();                                                                   // B1
+        IOHT::lds_to_global(s_dST, LDK, (T*)a.dhs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
+        if constexpr (NBUF == 2) {
+          if (c > 0) stage(pre[(j + 1) % PF], nb);
+        }
+        lds_barrier();                                                                   // B2
+        if constexpr (NBUF == 1) {
+          lds_barrier();                                                                 // B3: buffer read
+          if (c > 0) stage(pre[(j + 1) % PF], 0);
+          lds_barrier();                                                                 // B4: tiles complete
+        }
+        issue(pre[(j + 1) % PF], c - 1 - PF);
+      }
+    }
+    return;
+  }
+
+  if (team == 2) {
+    // ------------------------------- local dv (delta rule) -------------------------------
+    const int pw = wave_id() - 8;
+    const float scale = a.scale;
     // local part of dv_new of the chunk staged in `buf`: rows 16 pw .. 16 pw + 15
     auto dv_local = [&](int buf) {
       if constexpr (GDN) {
@@ -224,33 +260,19 @@ __global__ __launch_bounds__(2 * NTHR) void k_state_bwd(const lmoe_args a) {
         }
       }
     };
-#pragma unroll
-    for (int j = 0; j < PF; ++j) issue(pre[j], sq.nchunks - 1 - j);
-    stage(pre[0], 0);
-    issue(pre[0], sq.nchunks - 1 - PF);
-    lds_barrier();                                   // P0: the first chunk's tiles are complete
+    lds_barrier();                                   // P0
     dv_local(0);
-    for (int it0 = 0; it0 < sq.nchunks; it0 += PF) {
-#pragma unroll
-      for (int j = 0; j < PF; ++j) {
-        const int it = it0 + j;
-        if (it >= sq.nchunks) break;
-        const int c = sq.nchunks - 1 - it;
-        const int nb = NBUF == 2 ? ((it + 1) & 1) : 0;
-        lds_barrier();                                                                   // B1
-        IOHT::lds_to_global(s_dST, LDK, (T*)a.dhs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
-        if constexpr (NBUF == 2) {
-          if (c > 0) stage(pre[(j + 1) % PF], nb);
-        }
-        lds_barrier();                                                                   // B2
-        if constexpr (NBUF == 1) {
-          lds_barrier();                                                                 // B3: buffer read
-          if (c > 0) stage(pre[(j + 1) % PF], 0);
-          lds_barrier();                                                                 // B4: tiles complete
-        }
-        if (c > 0) dv_local(nb);
-        issue(pre[(j + 1) % PF], c - 1 - PF);
+    lds_barrier();                                   // P1
+    for (int it = 0; it < sq.nchunks; ++it) {
+      const int c = sq.nchunks - 1 - it;
+      const int nb = NBUF == 2 ? ((it + 1) & 1) : 0;
+      lds_barrier();                                                                     // B1
+      lds_barrier();                                                                     // B2
+      if constexpr (NBUF == 1) {
+        lds_barrier();                                                                   // B3
+        lds_barrier();                                                                   // B4
       }
+      if (c > 0) dv_local(nb);
     }
     return;
   }
@@ -271,6 +293,7 @@ __global__ __launch_bounds__(2 * NTHR) void k_state_bwd(const lmoe_args a) {
           dS[mi][ni][i] = p[(int64_t)(krow0 + acc_row(mi, i)) * V + v0 + acc_col(ni)];
   }
   lds_barrier();                                     // P0
+  if constexpr (GDN) lds_barrier();                  // P1
   for (int it = 0; it < sq.nchunks; ++it) {
     const int c = sq.nchunks - 1 - it;
     const int cur = NBUF == 2 ? (it & 1) : 0;
