@@ -79,7 +79,7 @@ def time_stages(call, lib, reps):
     from linear_moe_amd import _lib
     st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     out = {}
-    for stage in (0, 1, 2, 4, 5, 6):      # stage 3 (separate dv kernel) is not part of this op
+    for stage in (0, 1, 4, 5, 6):      # stages 2, 3 (separate output / dv kernels) are not part of this op
         a = call.fwd_args if stage <= 2 else call.bwd_args
         for _ in range(2):
             _lib.check(lib.lmoe_launch_stage(C.byref(a), call.OP, stage, st), "stage")

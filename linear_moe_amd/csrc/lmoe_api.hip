@@ -51,7 +51,6 @@ int lmoe_chunk_simple_gla_fwd(const lmoe_args* a, void* stream) {
   if (!a->o.ptr || !a->hs) return fail(-11, "%s: o and hs must not be null", op);
   if (a->NT == 0 || a->N == 0) return 0;
   lmoe::launch_state_fwd(*a, false, (hipStream_t)stream);
-  lmoe::launch_out_fwd(*a, false, (hipStream_t)stream);
   return launched(op);
 }
 
@@ -110,7 +109,6 @@ int lmoe_chunk_gated_delta_rule_fwd(const lmoe_args* a, void* stream) {
   if (a->NT == 0 || a->N == 0) return 0;
   lmoe::launch_gdn_wy_fwd(*a, (hipStream_t)stream);
   lmoe::launch_state_fwd(*a, true, (hipStream_t)stream);
-  lmoe::launch_out_fwd(*a, true, (hipStream_t)stream);
   return launched(op);
 }
 int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream) {
@@ -140,7 +138,6 @@ int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* strea
       case lmoe::ST_GDN_WY_FWD: if (!gdn) return fail(-20, "%s: stage not part of this op", nm);
         lmoe::launch_gdn_wy_fwd(*a, st); break;
       case lmoe::ST_STATE_FWD: lmoe::launch_state_fwd(*a, gdn, st); break;
-      case lmoe::ST_OUT_FWD: lmoe::launch_out_fwd(*a, gdn, st); break;
       case lmoe::ST_DV: if (gdn) return fail(-20, "%s: the delta rule forms dv inside its state pass", nm);
         lmoe::launch_bwd_dv(*a, false, st); break;
       case lmoe::ST_STATE_BWD: lmoe::launch_state_bwd(*a, gdn, st); break;

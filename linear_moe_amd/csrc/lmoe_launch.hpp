@@ -9,8 +9,8 @@ namespace lmoe {
 // Stages of the three ops (argument of lmoe_launch_stage; declared in include/lmoe.h)
 enum Stage {
   ST_GDN_WY_FWD = 0,   // gated delta rule: w, u, Tinv                   (chunk-parallel)
-  ST_STATE_FWD = 1,    // sequential state pass: hs (, vnew), ht
-  ST_OUT_FWD = 2,      // output o                                       (chunk-parallel)
+  ST_STATE_FWD = 1,    // sequential state pass: hs (, vnew), ht; scalar gates: also the output o
+  ST_OUT_FWD = 2,      // chunk_gla: output o                            (chunk-parallel)
   ST_DV = 3,           // dv (simple_gla / gla) or local part of dv_new  (chunk-parallel)
   ST_STATE_BWD = 4,    // reverse sequential state pass: dhs (, dv_new), dh0
   ST_DQK = 5,          // dq, dk, gate gradient (, dw)                   (chunk-parallel)
@@ -32,7 +32,6 @@ inline void dispatch(const lmoe_args& a, hipStream_t st) {
 }
 
 void launch_state_fwd(const lmoe_args& a, bool gdn, hipStream_t st);
-void launch_out_fwd(const lmoe_args& a, bool gdn, hipStream_t st);
 void launch_gdn_wy_fwd(const lmoe_args& a, hipStream_t st);
 void launch_bwd_dv(const lmoe_args& a, bool local, hipStream_t st);
 void launch_state_bwd(const lmoe_args& a, bool gdn, hipStream_t st);

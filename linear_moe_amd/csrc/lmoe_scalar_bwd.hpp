@@ -14,6 +14,7 @@
 //                 and, for simple_gla, dg = reverse cumsum of db.
 #pragma once
 #include "lmoe_seq.hpp"
+#include "lmoe_scalar_fwd.hpp"   // scale_frag
 
 namespace lmoe {
 
@@ -102,16 +103,6 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dv(const lmoe_args a) {
 //   it, P^T through a wave-private LDS strip), so no separate dv kernel runs for that op.
 //   All teams meet at the same barriers; three waves per SIMD hide each other's latencies.
 // ------------------------------------------------------------------------- //
-template <typename T> __device__ __forceinline__ void scale_frag(typename ET<T>::frag& f, const float* s8) {
-  const f32x4 s0 = *(const f32x4*)s8, s1 = *(const f32x4*)(s8 + 4);
-  if constexpr (sizeof(T) == 2) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) { f[i] = (bf16)((float)f[i] * s0[i]); f[i + 4] = (bf16)((float)f[i + 4] * s1[i]); }
-  } else {
-    f.lo *= s0; f.hi *= s1;
-  }
-}
-
 template <typename T, int K, int V, int BV, bool GDN>
 __global__ __launch_bounds__((GDN ? 3 : 2) * NTHR) void k_state_bwd(const lmoe_args a) {
   constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDU = BV + LPAD;

@@ -4,10 +4,9 @@
 
 namespace lmoe {
 
-// V-slice of the sequential state pass and of the output kernel
+// V-slice of the sequential state pass
 template <typename T, int V> struct FwdTiles {
   static constexpr int BVS = sizeof(T) == 4 ? 16 : 32;
-  static constexpr int BVO = V == 128 ? 64 : V;
 };
 
 template <bool GDN> struct StateFwd {
@@ -15,26 +14,13 @@ template <bool GDN> struct StateFwd {
     static void run(const lmoe_args& a, hipStream_t st) {
       constexpr int BV = FwdTiles<T, V>::BVS;
       const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BV);
-      hipLaunchKernelGGL((k_state_fwd<T, K, V, BV, GDN>), dim3(grid), dim3(2 * NTHR), 0, st, a);
+      hipLaunchKernelGGL((k_state_fwd<T, K, V, BV, GDN>), dim3(grid), dim3(3 * NTHR), 0, st, a);
     }
   };
 };
-template <bool GDN> struct OutFwd {
-  template <typename T, int K, int V> struct F {
-    static void run(const lmoe_args& a, hipStream_t st) {
-      const int grid = persistent_grid(a.NT * a.H, sizeof(T) == 2 ? 2 : 1);
-      hipLaunchKernelGGL((k_out_fwd<T, K, V, GDN>), dim3(grid), dim3(NTHR), 0, st, a);
-    }
-  };
-};
-
 void launch_state_fwd(const lmoe_args& a, bool gdn, hipStream_t st) {
   if (gdn) dispatch<StateFwd<true>::F>(a, st); else dispatch<StateFwd<false>::F>(a, st);
 }
-void launch_out_fwd(const lmoe_args& a, bool gdn, hipStream_t st) {
-  if (gdn) dispatch<OutFwd<true>::F>(a, st); else dispatch<OutFwd<false>::F>(a, st);
-}
-
 // C = A B^T (64 x 64, contraction along the tile columns) and G = A^T B (KD x KD, contraction
 // along the tile rows, i.e. the transposed-fragment path) over one pair of 64 x KD tiles,
 // through the loaders / fragments / accumulator stores of the toolkit
