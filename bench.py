@@ -27,8 +27,15 @@ PEAK_MFMA_BF16 = 2.5e15   # dense bf16 MFMA, FLOP/s (MI355X published)
 PEAK_HBM = 8.0e12         # B/s
 CH = 64
 
-STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_state_fwd", 2: "k_out_fwd", 3: "k_bwd_dv", 4: "k_state_bwd",
-               5: "k_bwd_dqk", 6: "k_gdn_wy_bwd"}
+STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_state_fwd", 4: "k_state_bwd", 5: "k_bwd_dqk", 6: "k_gdn_wy_bwd"}
+
+# HBM bytes per launch on this workload, from two rocprofv3 --pmc runs of this file (FETCH_SIZE, then
+# WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for the 256 MiB device
+# copy that main() issues first (FETCH_SIZE reads half of the bytes fetched, WRITE_SIZE all of the
+# bytes written).  Summary and commands: profiles/gdn_fwd_bwd_cfg4_hbm_traffic.md.
+CALIB_COPY_BYTES = 256 << 20
+MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 649013210, "k_state_fwd": 1091391848, "k_state_bwd": 956576801,
+                    "k_bwd_dqk": 1646585149, "k_gdn_wy_bwd": 1121118387}
 
 
 def gdn_inputs(B, T, H, K, V, seed, dtype, device):
@@ -51,23 +58,19 @@ def gdn_inputs(B, T, H, K, V, seed, dtype, device):
 
 
 def stage_model(stage, K, V, s=2):
-    """Algorithmic (flops, bytes) of one kernel per chunk and head: every product counted on full
-    64-token tiles, multiply-add = 2 flops; every input read once and every output written once."""
+    """Algorithmic (flops, bytes) of one kernel per chunk and head: every product counted once on
+    full 64-token tiles, multiply-add = 2 flops; every input read once, every output written once."""
     c = CH
     kv, ck, cv, cc = K * V, c * K, c * V, c * c
-    if stage == 0:   # k k^T, triangular inverse, w, u
-        return 2 * cc * K + (2 / 3) * c ** 3 + 2 * cc * K + 2 * cc * V, 2 * (ck + cv) * s + cc * s + c * (4 + s)
-    if stage == 1:   # w S, k_d^T v_new
-        return 4 * c * kv, (2 * ck + cv) * s + cv * s + kv * s + 4 * c
-    if stage == 2:   # q k^T, q S, P v_new
-        return 2 * cc * K + 2 * c * kv + 2 * cc * V, (2 * ck + cv + kv) * s + cv * s + 4 * c
-    if stage == 3:   # q k^T, P^T do
-        return 2 * cc * K + 2 * cc * V, (2 * ck + cv) * s + cv * s + 4 * c
-    if stage == 4:   # k_d dS', q^T do, w^T dv_new
-        return 6 * c * kv, (3 * ck + 2 * cv) * s + (cv + kv) * s + 4 * c
-    if stage == 5:   # do v^T, do S^T, v dS'^T, dv_new S^T, dP k, dP^T q
+    if stage == 0:   # k k^T, triangular inverse, w, u | r k,v  w w,u,Tinv
+        return 4 * cc * K + 2 * cc * V + (2 / 3) * c ** 3, 2 * (ck + cv) * s + cc * s + c * (4 + s)
+    if stage == 1:   # w S, k^T v_new, q k^T, q S, P v_new | r q,k,w,u  w v_new,hs,o
+        return 6 * c * kv + 2 * cc * K + 2 * cc * V, (3 * ck + cv) * s + (2 * cv + kv) * s + 4 * c
+    if stage == 4:   # k dS', q^T do, w^T dv_new, q k^T, P^T do | r q,k,w,do  w dv_new,dhs
+        return 6 * c * kv + 2 * cc * K + 2 * cc * V, (3 * ck + cv) * s + (cv + kv) * s + 4 * c
+    if stage == 5:   # do v^T, do S^T, v dS'^T, dv_new S^T, dP k, dP^T q | r do,v_new,dv_new,hs,dhs,q,k  w dq,dk,dw
         return 2 * cc * V + 6 * c * kv + 4 * cc * K, (3 * cv + 2 * kv + 2 * ck) * s + 3 * ck * s + 8 * c
-    if stage == 6:   # dT, Tinv^T du, Tinv^T dw, two 64^3 products, dM k, dM^T k_b
+    if stage == 6:   # dT, Tinv^T du, Tinv^T dw, two 64^3 products, dM k, dM^T k_b | r du,dw,k,v,Tinv,dk  w dk,dv
         return (2 * cc * (K + V) + 2 * cc * V + 2 * cc * K + 4 * c ** 3 + 4 * cc * K,
                 (2 * cv + 3 * ck + cc) * s + (ck + cv) * s + c * (12 + s))
     raise ValueError(stage)
@@ -93,9 +96,9 @@ def time_stages(call, lib, reps):
     return out
 
 
-def cpu_baseline(B, T, H, K, V, seed):
+def cpu_baseline(B, T, H, K, V, seed, min_seconds=10.0):
     """The chunked torch restatement (oracle/chunked.py), forward + manual backward, fp32, on the
-    host cores: one pass over the full workload after a short warm-up."""
+    host cores: whole passes over the full workload until at least ``min_seconds`` have elapsed."""
     import torch
     from oracle import chunked
     x = gdn_inputs(B, T, H, K, V, seed, torch.float32, "cpu")
@@ -103,12 +106,17 @@ def cpu_baseline(B, T, H, K, V, seed):
     small = {n: t[:1, :2, :256].contiguous() for n, t in hf.items()}
     chunked.chunk_fwd_bwd("gdn", small["q"], small["k"], small["v"], small["g"], small["beta"], None, None,
                           small["do"], None)
-    t0 = time.perf_counter()
+    passes, t0 = 0, time.perf_counter()
     with torch.no_grad():
-        chunked.chunk_fwd_bwd("gdn", hf["q"], hf["k"], hf["v"], hf["g"], hf["beta"], None, None, hf["do"], None)
-    dt = time.perf_counter() - t0
-    return {"value": B * T / dt, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"full workload once (B={B}, T={T}, H={H}, K=V={K}), fp32 chunked torch port, {dt:.2f} s"}
+        while True:
+            chunked.chunk_fwd_bwd("gdn", hf["q"], hf["k"], hf["v"], hf["g"], hf["beta"], None, None, hf["do"], None)
+            passes += 1
+            dt = time.perf_counter() - t0
+            if dt >= min_seconds or passes >= 20:
+                break
+    return {"value": passes * B * T / dt, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{passes} passes over the full workload (B={B}, T={T}, H={H}, K=V={K}), fp32 chunked "
+                      f"torch port, {dt:.1f} s"}
 
 
 def main():
@@ -134,6 +142,13 @@ def main():
     dev = torch.device("cuda:0")
     B, T, H, K, V, seed = 4, 8192, 16, 128, 128, 1004
     x = gdn_inputs(B, T, H, K, V, seed, torch.bfloat16, dev)
+
+    # known-size device copy: the yardstick for the FETCH_SIZE / WRITE_SIZE counters under rocprofv3
+    src = torch.empty(CALIB_COPY_BYTES, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
 
     call = GDNCall(keep=True)
 
@@ -167,7 +182,7 @@ def main():
     else:
         roof = {"bound": "hbm", "achieved": b_c * units / stages[dom] / 1e9, "peak": PEAK_HBM / 1e9, "unit": "GB/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = None
+    roof["traffic"] = MEASURED_TRAFFIC.get(STAGE_NAMES[dom])
     roof["kernel"] = STAGE_NAMES[dom]
     roof["kernel_us"] = stages[dom] * 1e6
     roof["flops_per_launch"] = f_c * units

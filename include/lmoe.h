@@ -4,7 +4,7 @@
  * This is the drop-in boundary for the one hot path the reference
  * (OpenSparseLLMs/Linear-MoE) delegates to flash-linear-attention ("fla"):
  * the reference's token mixers bind python callables at import time and call them in
- * forward(); a maintainer binds this library with ctypes instead (see INTEGRATION.md).
+ * forward(); a maintainer binds this library with ctypes instead.
  * Every entry point below names the reference call site it serves.
  *
  * Conventions
@@ -68,7 +68,8 @@ typedef struct lmoe_args {
   lmoe_tensor o;       /* [B,T,H,V]                                                    */
   float* ht;           /* [N,H,K,V] fp32 final state or NULL                           */
   /* intermediates written by *_fwd and read by *_bwd (caller-allocated, element type = dtype) */
-  void* hs;            /* [NT,H,K,V]  state at the start of every chunk                */
+  void* hs;            /* state at the start of every chunk: [NT,H,V,K] (transposed) for
+                          simple_gla and the gated delta rule, [NT,H,K,V] for chunk_gla    */
   lmoe_tensor vnew;    /* [B,T,H,V]   delta-rule pseudo values (gated delta rule)      */
   lmoe_tensor w;       /* [B,T,H,K]   WY factor w (gated delta rule)                   */
   lmoe_tensor u;       /* [B,T,H,V]   WY factor u (gated delta rule; forward only)     */
@@ -83,7 +84,7 @@ typedef struct lmoe_args {
   lmoe_tensor dbeta;   /* fp32, shape of beta                                          */
   float* dh0;          /* [N,H,K,V] fp32 or NULL                                       */
   /* backward workspace (caller-allocated, element type = dtype) */
-  void* dhs;           /* [NT,H,K,V] gradient w.r.t. the state at the END of every chunk */
+  void* dhs;           /* gradient w.r.t. the state at the END of every chunk, laid out as hs */
   lmoe_tensor dvnew;   /* [B,T,H,V]   gradient of vnew (gated delta rule)              */
   lmoe_tensor dw;      /* [B,T,H,K]   gradient of w    (gated delta rule)              */
 } lmoe_args;
@@ -92,6 +93,16 @@ typedef struct lmoe_args {
 int lmoe_version(void);
 /* Text of the last error on the calling thread ("" if none). */
 const char* lmoe_last_error(void);
+
+/* Bytes of caller-allocated intermediates of one call: part 0 = what *_fwd writes for *_bwd
+ * (hs, and per op amat / vnew, w, u, tinv), part 1 = the backward workspace (dhs, and dvnew, dw
+ * for the gated delta rule).  Each buffer is still passed through its own lmoe_args field; this
+ * is the sum a caller that carves them out of one arena must reserve (every buffer's size is a
+ * multiple of 256 bytes for the supported K, V).  Negative for an invalid op / dtype / part.
+ * Stands where fla sizes its saved tensors inside its autograd functions (no single call site
+ * in the reference; the ops are reached from the files named below). */
+int64_t lmoe_workspace_bytes(int32_t op, int32_t dtype, int32_t part, int32_t B, int32_t T, int32_t H, int32_t K,
+                             int32_t V, int32_t NT);
 
 /* chunk_simple_gla: S_t = e^{g_t} S_{t-1} + k_t^T v_t, o_t = scale q_t S_t, g scalar per
  * token-head (gate = SCALAR) or absent (gate = NONE).

@@ -44,6 +44,24 @@ extern "C" {
 int lmoe_version(void) { return 100; }
 const char* lmoe_last_error(void) { return g_err; }
 
+int64_t lmoe_workspace_bytes(int32_t op, int32_t dtype, int32_t part, int32_t B, int32_t T, int32_t H, int32_t K,
+                             int32_t V, int32_t NT) {
+  const char* nm = "lmoe_workspace_bytes";
+  if (dtype != LMOE_BF16 && dtype != LMOE_F32) return fail(-2, "%s: dtype must be LMOE_BF16 or LMOE_F32", nm);
+  if (op != LMOE_OP_SIMPLE_GLA && op != LMOE_OP_GLA && op != LMOE_OP_GATED_DELTA_RULE)
+    return fail(-21, "%s: unknown op %d", nm, op);
+  if (part != 0 && part != 1) return fail(-22, "%s: part must be 0 (saved by fwd) or 1 (bwd workspace)", nm);
+  if (B < 0 || T < 0 || H <= 0 || K <= 0 || V <= 0 || NT < 0) return fail(-4, "%s: negative dimension", nm);
+  const int64_t s = dtype == LMOE_BF16 ? 2 : 4;
+  const int64_t states = (int64_t)NT * H * K * V, tiles = (int64_t)NT * H * LMOE_CHUNK * LMOE_CHUNK;
+  const int64_t rows_k = (int64_t)B * T * H * K, rows_v = (int64_t)B * T * H * V;
+  int64_t n = states;                                                    // hs | dhs
+  if (op == LMOE_OP_GLA && part == 0) n += tiles;                        // amat
+  if (op == LMOE_OP_GATED_DELTA_RULE) n += part == 0 ? 2 * rows_v + rows_k + tiles   // vnew, u, w, tinv
+                                                     : rows_v + rows_k;              // dvnew, dw
+  return n * s;
+}
+
 int lmoe_chunk_simple_gla_fwd(const lmoe_args* a, void* stream) {
   const char* op = "lmoe_chunk_simple_gla_fwd";
   if (int r = check_common(a, op)) return r;

@@ -17,7 +17,7 @@ HEADER = os.path.join(ROOT, "include", "lmoe.h")
 def declared_functions():
     src = open(HEADER).read()
     src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
-    return re.findall(r"^\s*(?:const\s+char\s*\*|int)\s+(lmoe_\w+)\s*\(", src, flags=re.M)
+    return re.findall(r"^\s*(?:const\s+char\s*\*|int64_t|int)\s+(lmoe_\w+)\s*\(", src, flags=re.M)
 
 
 def test_library_exports_every_declared_symbol():
@@ -66,6 +66,23 @@ def test_invalid_arguments_are_rejected_without_a_launch():
     with pytest.raises(ValueError):
         _lib.check(-7, "x")
     assert lib.lmoe_selftest_gemm(0, 64, None, None, None, None, None) == -1
+
+
+def test_workspace_bytes_matches_the_buffers_the_host_layer_allocates():
+    from linear_moe_amd import _lib
+    lib = _lib.load()
+    B, T, H, K, V = 2, 200, 3, 64, 128
+    NT = B * ((T + 63) // 64)
+    for dtype, s in ((_lib.LMOE_BF16, 2), (_lib.LMOE_F32, 4)):
+        states, tiles, rk, rv = NT * H * K * V, NT * H * 64 * 64, B * T * H * K, B * T * H * V
+        want = {(0, 0): states, (0, 1): states, (1, 0): states + tiles, (1, 1): states,
+                (2, 0): states + tiles + rk + 2 * rv, (2, 1): states + rk + rv}
+        for (op, part), n in want.items():
+            assert lib.lmoe_workspace_bytes(op, dtype, part, B, T, H, K, V, NT) == n * s
+    assert lib.lmoe_workspace_bytes(5, 0, 0, B, T, H, K, V, NT) == -21
+    assert lib.lmoe_workspace_bytes(0, 9, 0, B, T, H, K, V, NT) == -2
+    assert lib.lmoe_workspace_bytes(0, 0, 2, B, T, H, K, V, NT) == -22
+    assert lib.lmoe_workspace_bytes(0, 0, 0, B, -1, H, K, V, NT) == -4
 
 
 def test_seq_plan_tables():
