@@ -1,10 +1,11 @@
 """MI355X-native chunked linear-attention ops behind flash-linear-attention's call signatures.
 
 Drop-in for the ``fla.ops`` callables the reference's token mixers import
-(``linear_moe/sequence_modeling/{gla,retention,gated_deltanet,basic_linear_attention}``).
+(``linear_moe/sequence_modeling/{gla,retention,gated_deltanet,deltanet,basic_linear_attention}``).
 All compute runs in hand-written HIP kernels (``csrc/``) reached through the C ABI of
 ``liblmoe_hip.so`` (``include/lmoe.h``); there is no fallback path.
 """
+from .delta_rule import chunk_delta_rule  # noqa: F401
 from .gated_delta_rule import chunk_gated_delta_rule  # noqa: F401
 from .gla import chunk_gla  # noqa: F401
 from .lightning import lightning_attn2, lightning_attn2_no_decay  # noqa: F401
@@ -12,5 +13,5 @@ from .linear_attn import chunk_linear_attn  # noqa: F401
 from .retention import chunk_retention  # noqa: F401
 from .simple_gla import chunk_simple_gla  # noqa: F401
 
-__all__ = ["chunk_simple_gla", "chunk_gla", "chunk_gated_delta_rule", "chunk_retention", "chunk_linear_attn",
+__all__ = ["chunk_simple_gla", "chunk_gla", "chunk_gated_delta_rule", "chunk_delta_rule", "chunk_retention", "chunk_linear_attn",
            "lightning_attn2", "lightning_attn2_no_decay"]

@@ -117,3 +117,27 @@ def test_gdn_bwd_varlen(cuda, dtype):
     q, k, v, g, beta = gdn_inputs(400, 1, T, H, K, V, dtype, False, True)
     ins = dict(q=q, k=k, v=v, g=g, beta=beta, h0=gen(414, N, H, K, V) * 0.1)
     _gdn_bwd_check(cuda, dtype, ins, gen(415, 1, T, H, V, dtype=dtype), gen(416, N, H, K, V), cu, False)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", [(2, 200, 2, 128, 128, True), (1, 70, 2, 64, 128, False)])
+def test_delta_rule_fwd_bwd(cuda, dtype, case):
+    """chunk_delta_rule as the reference calls it (deltanet.py:127-130): head-first, positional chunk size."""
+    from linear_moe_amd import chunk_delta_rule
+    from tests.util import oracle_grads
+    B, T, H, K, V, use_h0 = case
+    q, k, v, _, beta = gdn_inputs(500, B, T, H, K, V, dtype, True, False)
+    ins = dict(q=q, k=k, v=v, beta=beta, h0=gen(514, B, H, K, V) * 0.1 if use_h0 else None)
+    do, dht = gen(515, B, H, T, V, dtype=dtype), gen(516, B, H, K, V)
+    fn = lambda q, k, v, beta, h0: naive.naive_recurrent_gated_delta_rule(q, k, v, None, beta, None, h0, True, None, True)
+    ref_o, ref_ht, ref = oracle_grads(fn, ins, do, dht)
+    dev = {n: (None if x is None else x.to(cuda).requires_grad_(True)) for n, x in ins.items()}
+    o, ht = chunk_delta_rule(dev['q'], dev['k'], dev['v'], dev['beta'], 32, initial_state=dev['h0'],
+                             output_final_state=True)
+    ((o * do.to(cuda)).sum() + (ht * dht.to(cuda)).sum()).backward()
+    torch.cuda.synchronize()
+    tol = TOL[dtype]
+    assert max_abs_rel(o.detach().cpu(), ref_o) < tol and max_abs_rel(ht.detach().cpu(), ref_ht) < tol
+    for n, r in ref.items():
+        err = max_abs_rel(dev[n].grad.cpu(), r)
+        assert err < tol, (n, err)

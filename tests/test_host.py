@@ -5,6 +5,7 @@ import ctypes as C
 import os
 import re
 import subprocess
+import sys
 import tempfile
 
 import pytest
@@ -128,3 +129,28 @@ def test_python_layer_validates_before_launch():
     with pytest.raises(ValueError, match="dtype"):
         g = Fake(qc, torch.float16)
         _check_inputs(g, g, g, True, None)
+
+
+def test_fla_shim_resolves_every_name_the_reference_imports():
+    """A fresh interpreter with only the shim directory on its path (as the reference's launcher sets
+    PYTHONPATH=$FLA_PATH) finds every operator name of the reference's import lines."""
+    shim = os.path.join(ROOT, "linear_moe_amd", "fla_shim")
+    code = (
+        "from fla.ops.gla import chunk_gla, fused_chunk_gla, fused_recurrent_gla\n"
+        "from fla.ops.gated_delta_rule import chunk_gated_delta_rule, fused_recurrent_gated_delta_rule\n"
+        "from fla.ops.delta_rule import chunk_delta_rule, fused_chunk_delta_rule, fused_recurrent_delta_rule\n"
+        "from fla.ops.linear_attn import chunk_linear_attn, fused_chunk_linear_attn, fused_recurrent_linear_attn\n"
+        "from fla.ops.retention import (chunk_retention, fused_chunk_retention, fused_recurrent_retention,\n"
+        "                               parallel_retention)\n"
+        "from fla.ops.simple_gla import chunk_simple_gla\n"
+        "from fla.modules.l2norm import l2_norm\n"
+        "from lightning_attn.ops.triton import lightning_attn2, lightning_attn2_no_decay\n"
+        "import linear_moe_amd, torch\n"
+        "assert chunk_gated_delta_rule is linear_moe_amd.chunk_gated_delta_rule\n"
+        "x = torch.tensor([[3.0, 4.0]])\n"
+        "assert torch.allclose(l2_norm(x), x / 5.0, atol=1e-6)\n"
+        "print('ok')\n")
+    env = {k: v for k, v in os.environ.items() if k != "PYTHONPATH"}
+    env["PYTHONPATH"] = shim
+    out = subprocess.check_output([sys.executable, "-c", code], env=env, cwd=tempfile.gettempdir())
+    assert out.strip() == b"ok"
