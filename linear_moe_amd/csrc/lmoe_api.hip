@@ -57,7 +57,7 @@ int64_t lmoe_workspace_bytes(int32_t op, int32_t dtype, int32_t part, int32_t B,
   const int64_t rows_k = (int64_t)B * T * H * K, rows_v = (int64_t)B * T * H * V;
   int64_t n = states;                                                    // hs | dhs
   if (op == LMOE_OP_GLA && part == 0) n += tiles;                        // amat
-  if (op == LMOE_OP_GATED_DELTA_RULE) n += part == 0 ? 2 * rows_v + rows_k + tiles   // vnew, u, w, tinv
+  if (op == LMOE_OP_GATED_DELTA_RULE) n += part == 0 ? 2 * rows_v + rows_k + 3 * tiles   // vnew, u, w, tinv, pmat
                                                      : rows_v + rows_k;              // dvnew, dw
   return n * s;
 }
@@ -68,7 +68,7 @@ int lmoe_chunk_simple_gla_fwd(const lmoe_args* a, void* stream) {
   if (a->gate == LMOE_GATE_VECTOR) return fail(-10, "%s: vector gates belong to lmoe_chunk_gla_fwd", op);
   if (!a->o.ptr || !a->hs) return fail(-11, "%s: o and hs must not be null", op);
   if (a->NT == 0 || a->N == 0) return 0;
-  lmoe::launch_state_fwd(*a, false, (hipStream_t)stream);
+  lmoe::launch_state_fwd(*a, (hipStream_t)stream);
   return launched(op);
 }
 
@@ -80,7 +80,7 @@ int lmoe_chunk_simple_gla_bwd(const lmoe_args* a, void* stream) {
     return fail(-11, "%s: hs, dhs, d_o, dq, dk and dv must not be null", op);
   if (a->gate == LMOE_GATE_SCALAR && !a->dg.ptr) return fail(-13, "%s: dg must not be null for a gated call", op);
   if (a->NT == 0 || a->N == 0) return 0;
-  lmoe::launch_state_bwd(*a, false, (hipStream_t)stream);
+  lmoe::launch_state_bwd(*a, (hipStream_t)stream);
   lmoe::launch_bwd_dv(*a, false, (hipStream_t)stream);
   lmoe::launch_bwd_dqk(*a, false, (hipStream_t)stream);
   return launched(op);
@@ -122,11 +122,11 @@ int lmoe_chunk_gated_delta_rule_fwd(const lmoe_args* a, void* stream) {
   if (int r = check_common(a, op)) return r;
   if (a->gate == LMOE_GATE_VECTOR) return fail(-10, "%s: the gate is one scalar per token and head", op);
   if (!a->beta.ptr) return fail(-12, "%s: beta must not be null", op);
-  if (!a->o.ptr || !a->hs || !a->vnew.ptr || !a->w.ptr || !a->u.ptr || !a->tinv)
-    return fail(-11, "%s: o, hs, vnew, w, u and tinv must not be null", op);
+  if (!a->o.ptr || !a->hs || !a->vnew.ptr || !a->w.ptr || !a->u.ptr || !a->tinv || !a->pmat)
+    return fail(-11, "%s: o, hs, vnew, w, u, tinv and pmat must not be null", op);
   if (a->NT == 0 || a->N == 0) return 0;
   lmoe::launch_gdn_wy_fwd(*a, (hipStream_t)stream);
-  lmoe::launch_state_fwd(*a, true, (hipStream_t)stream);
+  lmoe::launch_gdn_state_fwd(*a, (hipStream_t)stream);
   return launched(op);
 }
 int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream) {
@@ -134,12 +134,12 @@ int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream) {
   if (int r = check_common(a, op)) return r;
   if (a->gate == LMOE_GATE_VECTOR) return fail(-10, "%s: the gate is one scalar per token and head", op);
   if (!a->beta.ptr) return fail(-12, "%s: beta must not be null", op);
-  if (!a->hs || !a->dhs || !a->vnew.ptr || !a->w.ptr || !a->tinv || !a->dvnew.ptr || !a->dw.ptr)
-    return fail(-11, "%s: hs, dhs, vnew, w, tinv, dvnew and dw must not be null", op);
+  if (!a->hs || !a->dhs || !a->vnew.ptr || !a->w.ptr || !a->tinv || !a->pmat || !a->dvnew.ptr || !a->dw.ptr)
+    return fail(-11, "%s: hs, dhs, vnew, w, tinv, pmat, dvnew and dw must not be null", op);
   if (!a->d_o.ptr || !a->dq.ptr || !a->dk.ptr || !a->dv.ptr || !a->dg.ptr || !a->dbeta.ptr)
     return fail(-13, "%s: d_o, dq, dk, dv, dg and dbeta must not be null", op);
   if (a->NT == 0 || a->N == 0) return 0;
-  lmoe::launch_state_bwd(*a, true, (hipStream_t)stream);
+  lmoe::launch_gdn_state_bwd(*a, (hipStream_t)stream);
   lmoe::launch_bwd_dqk(*a, true, (hipStream_t)stream);
   lmoe::launch_gdn_wy_bwd(*a, (hipStream_t)stream);
   return launched(op);
@@ -154,11 +154,26 @@ int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* strea
   if (op == LMOE_OP_SIMPLE_GLA || gdn) {
     switch (stage) {
       case lmoe::ST_GDN_WY_FWD: if (!gdn) return fail(-20, "%s: stage not part of this op", nm);
+        if (!a->pmat) return fail(-11, "%s: pmat must not be null", nm);
         lmoe::launch_gdn_wy_fwd(*a, st); break;
-      case lmoe::ST_STATE_FWD: lmoe::launch_state_fwd(*a, gdn, st); break;
+      case lmoe::ST_STATE_FWD:
+        if (gdn) {
+          if (!a->pmat) return fail(-11, "%s: pmat must not be null", nm);
+          lmoe::launch_gdn_state_fwd(*a, st);
+        } else {
+          lmoe::launch_state_fwd(*a, st);
+        }
+        break;
       case lmoe::ST_DV: if (gdn) return fail(-20, "%s: the delta rule forms dv inside its state pass", nm);
         lmoe::launch_bwd_dv(*a, false, st); break;
-      case lmoe::ST_STATE_BWD: lmoe::launch_state_bwd(*a, gdn, st); break;
+      case lmoe::ST_STATE_BWD:
+        if (gdn) {
+          if (!a->pmat) return fail(-11, "%s: pmat must not be null", nm);
+          lmoe::launch_gdn_state_bwd(*a, st);
+        } else {
+          lmoe::launch_state_bwd(*a, st);
+        }
+        break;
       case lmoe::ST_DQK: lmoe::launch_bwd_dqk(*a, gdn, st); break;
       case lmoe::ST_GDN_WY_BWD: if (!gdn) return fail(-20, "%s: stage not part of this op", nm);
         lmoe::launch_gdn_wy_bwd(*a, st); break;

@@ -38,6 +38,14 @@ __device__ __forceinline__ void lds_barrier() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
+// s_waitcnt vmcnt(0): every global load / store this wave has issued so far has completed (the
+// scheduling barriers keep later loads behind it and earlier ones in front of it)
+__device__ __forceinline__ void wait_all_loads() {
+  __builtin_amdgcn_sched_barrier(0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  __builtin_amdgcn_sched_barrier(0);
+}
+
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
 __device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
 
@@ -227,6 +235,55 @@ __device__ __forceinline__ void store_strip(const f32x4 (&acc)[1][NB], T* stg, T
     }
   }
 }
+
+// ------------------------------------------------------------------------- //
+// fragments held in registers
+// ------------------------------------------------------------------------- //
+// multiply the 8 contraction elements a lane holds by s8[0..7]
+template <typename T> __device__ __forceinline__ void scale_frag8(typename ET<T>::frag& f, const float* s8) {
+  const f32x4 s0 = *(const f32x4*)s8, s1 = *(const f32x4*)(s8 + 4);
+  if constexpr (sizeof(T) == 2) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { f[i] = (bf16)((float)f[i] * s0[i]); f[i + 4] = (bf16)((float)f[i + 4] * s1[i]); }
+  } else {
+    f.lo *= s0; f.hi *= s1;
+  }
+}
+
+__device__ __forceinline__ void frag_keep_if(bf16x8& f, bool ok) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  u32x4 w = __builtin_bit_cast(u32x4, f);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = ok ? w[i] : 0u;
+  f = __builtin_bit_cast(bf16x8, w);
+}
+__device__ __forceinline__ void frag_keep_if(f32frag& f, bool ok) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { f.lo[i] = ok ? f.lo[i] : 0.f; f.hi[i] = ok ? f.hi[i] : 0.f; }
+}
+
+// MFMA A-fragments of one 16-row strip of a row-major matrix with D columns, loaded straight from
+// global memory: lane (r = l%16, g = l/16) holds, for contraction step j, the 8 elements
+// [row0 + r][32 j + 8 g ..].  Rows beyond `last` re-read row `last` (branch-free, so a prefetch
+// stays in flight); mask() zeroes the rows >= nvalid when the strip is consumed.
+template <typename T, int D> struct RowFrags {
+  static constexpr int KS = D / 32;
+  typename ET<T>::frag f[KS];
+  __device__ __forceinline__ void load(const T* __restrict__ base, int64_t row_stride, int row0, int last) {
+    const int l = threadIdx.x & 63;
+    int r = row0 + (l & 15);
+    r = r < last ? r : last;
+    const T* p = base + (int64_t)r * row_stride + 8 * (l >> 4);
+#pragma unroll
+    for (int j = 0; j < KS; ++j) f[j] = ET<T>::load_frag(p + 32 * j);
+  }
+  __device__ __forceinline__ void mask(int row0, int nvalid) {
+    if (row0 + 16 <= nvalid) return;            // uniform: full strips (the common case) skip it
+    const bool ok = row0 + (lane_id() & 15) < nvalid;
+#pragma unroll
+    for (int j = 0; j < KS; ++j) frag_keep_if(f[j], ok);
+  }
+};
 
 // ------------------------------------------------------------------------- //
 // cooperative global <-> LDS tile movement (all 256 threads)

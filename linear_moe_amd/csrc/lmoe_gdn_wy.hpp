@@ -2,7 +2,9 @@
 //   L = strictlower( diag(beta) (k k^T) . Gamma ),  Gamma_ij = e^{b_i - b_j}
 //   Tinv = (I + L)^-1            (unit lower triangular, fp32)
 //   w = Tinv (k . beta e^{b}),   u = Tinv (v . beta)
-// grid = (NT, H), block = 256.  Writes w, u and Tinv (element type T).
+// and the intra-chunk attention matrix the two sequential passes consume,
+//   P = (q k^T) . Gamma  (lower triangle incl. the diagonal), stored as P and as P^T.
+// grid = (NT, H), block = 256.  Writes w, u, Tinv and P, P^T (element type T).
 #pragma once
 #include "lmoe_seq.hpp"
 
@@ -75,8 +77,12 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
   const int wv = wave_id(), l = lane_id();
   typedef TileIO<T, CH, K> IOK;
   typedef TileIO<T, CH, V> IOV;
+  typedef TileIO<T, CH, CH> IO64;
   typename IOK::Regs rk;
   typename IOV::Regs rv;
+  // q enters only as the A operand of q k^T: each wave takes its 16 rows straight into fragments
+  RowFrags<T, K> fq;
+  fq.load(row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, 16 * wv, ci.len - 1);
   IOK::load(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
   IOV::load(rv, row_ptr<T>(a.v, ci.b, ci.tok, h), a.v.st, ci.len);
   if (threadIdx.x >= 64 && threadIdx.x < 128) {
@@ -103,9 +109,44 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
       acc_to_lds<float>(p, s_L, LDC, 16 * wv, 16 * nj);
     }
   }
-  __syncthreads();
-  // k is dead as an operand of k k^T: scale it in place to k beta e^{b} (from the registers)
+  {
+    // P = (q k^T) . Gamma -> global as P and P^T, staged through the (still unused) X tile
+    T* s_P = (T*)s_X;
+    T* pg = (T*)a.pmat + ((int64_t)cid * a.H + h) * 2 * CH * CH;
+    f32x4 pm[1][4];
+    acc_zero(pm);
+    fq.mask(16 * wv, ci.len);
+#pragma unroll
+    for (int ks = 0; ks < K / 32; ++ks)
+#pragma unroll
+      for (int nj = 0; nj < 4; ++nj)
+        ET<T>::mma(pm[0][nj], fq.f[ks], ET<T>::load_frag(s_k + (16 * nj + (l & 15)) * LDK + 32 * ks + 8 * (l >> 4)));
+#pragma unroll
+    for (int nj = 0; nj < 4; ++nj) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * nj + (l & 15);
+        pm[0][nj][i] = (r >= cc) ? pm[0][nj][i] * texp<T>(s_b[r] - s_b[cc]) : 0.f;
+      }
+      acc_to_lds<T>(pm[0][nj], s_P, LDC, 16 * wv, 16 * nj);
+      if constexpr (sizeof(T) == 2) acc_to_lds_t<T>(pm[0][nj], s_P + CH * LDC, LDC, 16 * wv, 16 * nj);
+    }
+    __syncthreads();
+    IO64::lds_to_global(s_P, LDC, pg, CH, CH);
+    if constexpr (sizeof(T) == 2) {
+      IO64::lds_to_global(s_P + CH * LDC, LDC, pg + CH * CH, CH, CH);
+    } else {
+      // an fp32 tile fills the X tile: the transpose takes a second round
+      __syncthreads();
+#pragma unroll
+      for (int nj = 0; nj < 4; ++nj) acc_to_lds_t<T>(pm[0][nj], s_P, LDC, 16 * wv, 16 * nj);
+      __syncthreads();
+      IO64::lds_to_global(s_P, LDC, pg + CH * CH, CH, CH);
+    }
+  }
+  // k is dead as an operand of k k^T and q k^T: scale it in place to k beta e^{b} (from the registers)
   IOK::store_lds_scaled(rk, s_k, LDK, s_beb);
+  __syncthreads();   // L is complete, the P staging has been read: the inverse may overwrite X
   tri_inverse_64(s_L, LDC, s_X, LDC, s_Y);       // barriers inside; s_L is dead afterwards
   {
     T* tg = (T*)a.tinv + ((int64_t)cid * a.H + h) * CH * CH;

@@ -8,7 +8,7 @@ namespace lmoe {
 
 // Stages of the three ops (argument of lmoe_launch_stage; declared in include/lmoe.h)
 enum Stage {
-  ST_GDN_WY_FWD = 0,   // gated delta rule: w, u, Tinv                   (chunk-parallel)
+  ST_GDN_WY_FWD = 0,   // gated delta rule: w, u, Tinv, P                (chunk-parallel)
   ST_STATE_FWD = 1,    // sequential state pass: hs (, vnew), ht; scalar gates: also the output o
   ST_OUT_FWD = 2,      // chunk_gla: output o                            (chunk-parallel)
   ST_DV = 3,           // dv (simple_gla / gla) or local part of dv_new  (chunk-parallel)
@@ -31,10 +31,12 @@ inline void dispatch(const lmoe_args& a, hipStream_t st) {
 #undef LMOE_KV
 }
 
-void launch_state_fwd(const lmoe_args& a, bool gdn, hipStream_t st);
+void launch_state_fwd(const lmoe_args& a, hipStream_t st);        // chunk_simple_gla
+void launch_gdn_state_fwd(const lmoe_args& a, hipStream_t st);    // gated delta rule
+void launch_gdn_state_bwd(const lmoe_args& a, hipStream_t st);
 void launch_gdn_wy_fwd(const lmoe_args& a, hipStream_t st);
 void launch_bwd_dv(const lmoe_args& a, bool local, hipStream_t st);
-void launch_state_bwd(const lmoe_args& a, bool gdn, hipStream_t st);
+void launch_state_bwd(const lmoe_args& a, hipStream_t st);        // chunk_simple_gla
 void launch_bwd_dqk(const lmoe_args& a, bool gdn, hipStream_t st);
 void launch_gdn_wy_bwd(const lmoe_args& a, hipStream_t st);
 // chunk_gla: one kernel of the pipeline (stage = ST_GLA_INTRA_FWD, ST_STATE_FWD, ST_OUT_FWD,

@@ -40,9 +40,7 @@ template <bool GDN> struct BwdDqk {
 void launch_bwd_dv(const lmoe_args& a, bool local, hipStream_t st) {
   if (local) dispatch<BwdDv<true>::F>(a, st); else dispatch<BwdDv<false>::F>(a, st);
 }
-void launch_state_bwd(const lmoe_args& a, bool gdn, hipStream_t st) {
-  if (gdn) dispatch<StateBwd<true>::F>(a, st); else dispatch<StateBwd<false>::F>(a, st);
-}
+void launch_state_bwd(const lmoe_args& a, hipStream_t st) { dispatch<StateBwd<false>::F>(a, st); }
 void launch_bwd_dqk(const lmoe_args& a, bool gdn, hipStream_t st) {
   if (gdn) dispatch<BwdDqk<true>::F>(a, st); else dispatch<BwdDqk<false>::F>(a, st);
 }

@@ -18,9 +18,7 @@ template <bool GDN> struct StateFwd {
     }
   };
 };
-void launch_state_fwd(const lmoe_args& a, bool gdn, hipStream_t st) {
-  if (gdn) dispatch<StateFwd<true>::F>(a, st); else dispatch<StateFwd<false>::F>(a, st);
-}
+void launch_state_fwd(const lmoe_args& a, hipStream_t st) { dispatch<StateFwd<false>::F>(a, st); }
 // C = A B^T (64 x 64, contraction along the tile columns) and G = A^T B (KD x KD, contraction
 // along the tile rows, i.e. the transposed-fragment path) over one pair of 64 x KD tiles,
 // through the loaders / fragments / accumulator stores of the toolkit
