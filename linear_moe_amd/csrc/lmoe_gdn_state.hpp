@@ -6,15 +6,18 @@
 //   with P = (q k^T) . Gamma (written by k_gdn_wy_fwd as P and P^T), e_b = e^{b}, e_d = e^{b_C - b}.
 //
 // Both kernels keep the per-chunk work of the dependency chain as small as it can be made:
-//   * work-group = 2 teams of 4 waves.  Team 0 (consumers) owns the state slice [K x BV] in fp32
-//     MFMA accumulators (wave w: rows [w K/4, (w+1) K/4)) and, for the products whose rows are
-//     tokens, rows 16 w .. 16 w + 15 of the chunk.  Team 1 (loaders) stages the tiles that are
-//     contracted along their rows (they need the transposing LDS read) and the gate vectors two
-//     chunks ahead, and writes the state checkpoints (hs / dhs, layout [V][K]).
-//   * operands that are contracted along their columns and used by one wave only (w, q, P rows in
-//     the forward; k, P^T rows in the backward) never touch LDS: every consumer wave loads its own
-//     16-row strip as MFMA A-fragments straight from global memory, a few chunks ahead
-//     (RowFrags), so the LDS pipe carries only what several waves share.
+//   * work-group = 2 teams of 4 waves that meet at two barriers per chunk (B1, B2).
+//     Team 0 (consumers) owns the state slice [K x BV] in fp32 MFMA accumulators (wave w: rows
+//     [w K/4, (w+1) K/4)) and, for the products whose rows are tokens, rows 16 w .. 16 w + 15 of
+//     the chunk.  It touches LDS and the matrix cores only: a wave that issues global loads or
+//     stores stalls at the issue whenever the vector memory pipe of the CU is busy, and on this
+//     wave every such stall lengthens the chain.
+//     Team 1 (loaders) owns all global traffic: it keeps the operand tiles of the next chunks in
+//     flight in registers (whole 128-byte lines per row), stages them into single LDS buffers in
+//     the half-step before they are needed, and writes the state checkpoints (hs / dhs, layout
+//     [V][K]) and the chunk's results from LDS.
+//   * the intra-chunk matrix P is not formed here: the chunk-parallel WY preparation writes it
+//     once per (chunk, head) instead of once per V-slice.
 //   * grid = ceil(N*H / 8) * 8 * (V / BV) work-groups (1-D): the V-slices of one (sequence, head)
 //     get ids congruent mod 8, i.e. run on the same XCD and share k, w, q, P through its L2.
 #pragma once
@@ -26,27 +29,47 @@ namespace lmoe {
 // V-slice / prefetch shape of the sequential passes per element type
 template <typename T> struct GdnStateCfg {
   static constexpr int BV = sizeof(T) == 2 ? 32 : 16;    // V columns per work-group
-  static constexpr int PF = sizeof(T) == 2 ? 3 : 1;      // consumer-side prefetch depth (chunks)
-  static constexpr int LPF = 3;                          // loader-side prefetch depth (chunks)
+  static constexpr int LPF = sizeof(T) == 2 ? 2 : 1;     // chunks a loader keeps in flight per ring
 };
+
+// Runs step(slot, i) for i = 0 .. n-1 with slot = i % L as a compile-time constant (L = 1 or 2).
+// Whole groups of L steps run without an exit in between: an early exit inside a group would be
+// one more path to the loop header, on which the compiler could count only the loads of the
+// first step as issued and would drain the prefetch ring on every trip.
+template <int L, typename F> __device__ __forceinline__ void ring_loop(int n, F&& step) {
+  static_assert(L == 1 || L == 2, "rings of one or two register sets");
+  int i = 0;
+  for (; i + L <= n; i += L) {
+    step(std::integral_constant<int, 0>(), i);
+    if constexpr (L == 2) step(std::integral_constant<int, 1>(), i + 1);
+  }
+  if constexpr (L == 2) {
+    if (i < n) step(std::integral_constant<int, 0>(), i);
+  }
+}
 
 // ------------------------------------------------------------------------- //
 // forward
+//   loaders, chunk c:  B1 | stage k(c), P(c); store hs(c), o(c-1), v_new(c-1); prefetch k, P |
+//                      B2 | stage w, q, u, gates of chunk c+1; prefetch w, q, u, g
+//   consumers, chunk c: S -> LDS | B1 | w S, q S, v_new -> LDS | B2 | S update, P v_new, o -> LDS
 // ------------------------------------------------------------------------- //
 template <typename T, int K, int V, int BV>
 __global__ __launch_bounds__(2 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
   constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDU = BV + LPAD;
   constexpr int MB = K / 64, NB = BV / 16, KS = K / 32;
-  constexpr int PF = GdnStateCfg<T>::PF, LPF = GdnStateCfg<T>::LPF;
-  static_assert(LPF == 3 && PF <= 3, "the chunk loops are written out for rings of three");
-  __shared__ __attribute__((aligned(16))) T s_k[2][CH * LDK];       // k             [64][K]
-  __shared__ __attribute__((aligned(16))) T s_u[2][CH * LDU];       // u             [64][BV]
+  constexpr int LPF = GdnStateCfg<T>::LPF;
+  __shared__ __attribute__((aligned(16))) T s_k[CH * LDK];          // k             [64][K]
+  __shared__ __attribute__((aligned(16))) T s_w[CH * LDK];          // w             [64][K]
+  __shared__ __attribute__((aligned(16))) T s_q[CH * LDK];          // q             [64][K]
+  __shared__ __attribute__((aligned(16))) T s_p[CH * LDC];          // P             [64][64]
+  __shared__ __attribute__((aligned(16))) T s_u[CH * LDU];          // u             [64][BV]
   __shared__ __attribute__((aligned(16))) T s_hT[BV * LDK];         // S^T           [BV][K]
   __shared__ __attribute__((aligned(16))) T s_vT[BV * LDC];         // v_new^T       [BV][64]
-  __shared__ __attribute__((aligned(16))) T s_stg[4 * 16 * LDU];    // v_new store strips
-  __shared__ __attribute__((aligned(16))) T s_ost[4 * 16 * LDU];    // o store strips
+  __shared__ __attribute__((aligned(16))) T s_vn[CH * LDU];         // v_new         [64][BV] (to be stored)
+  __shared__ __attribute__((aligned(16))) T s_o[CH * LDU];          // o             [64][BV] (to be stored)
   __shared__ __attribute__((aligned(16))) float s_eb[2][64], s_ed[2][64];
-  __shared__ float s_dec[2];                                        // e^{b_C} per buffer
+  __shared__ float s_dec[2];                                        // e^{b_C}; gate arrays: buffer c & 1
 
   constexpr int NVS = V / BV;
   const int xcd = blockIdx.x & 7, jj = blockIdx.x >> 3;
@@ -69,31 +92,49 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
   }
   typedef TileIO<T, CH, K> IOK;
   typedef TileIO<T, CH, BV> IOV;
+  typedef TileIO<T, CH, CH> IOP;
   typedef TileIO<T, BV, K> IOHT;
 
   if (team == 1) {
     // --------------------------------- loaders -------------------------------------------
-    struct Pre { typename IOK::Regs rk; typename IOV::Regs ru; uint32_t graw; int len; };
-    Pre pre[LPF];
+    // two rings of register sets: A = what phase 2 of the chunk's own step reads (k, P),
+    // B = what phase 1 reads (w, q, u, gates), staged during phase 2 of the step before
+    struct PreA { typename IOK::Regs rk; typename IOP::Regs rp; int len; };
+    struct PreB { typename IOK::Regs rw, rq; typename IOV::Regs ru; uint32_t graw; int len; };
+    PreA pa[LPF];
+    PreB pb[LPF];
     const bool gated = a.gate != LMOE_GATE_NONE && a.g.ptr != nullptr;
     const void* gptr = gated ? a.g.ptr : a.k.ptr;
     // Always issued (chunk index clamped to the last chunk; the surplus loads at the end of a
     // sequence are never consumed): a prefetch that is skipped on some path would make the
     // compiler drain all outstanding loads at every consumer of a register set.
-    auto issue = [&](Pre& P, int c) {
+    auto issue_a = [&](PreA& P, int c) {
       c = min(c, sq.nchunks - 1);
       const int tok = sq.tok0 + c * CH;
-      const int len = min(CH, sq.len - c * CH);
-      IOK::load_nomask(P.rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, len);
-      IOV::load_nomask(P.ru, row_ptr<T>(a.u, sq.b, tok, h) + v0, a.u.st, len);
-      P.len = len;
-      P.graw = load_scalar_raw(gptr, a.g_dtype, gated ? row_off(a.g, sq.b, tok + min(l, len - 1), h) : 0);
+      P.len = min(CH, sq.len - c * CH);
+      IOK::load_nomask(P.rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, P.len);
+      IOP::load_nomask(P.rp, (const T*)a.pmat + ((int64_t)(sq.chunk0 + c) * a.H + h) * 2 * CH * CH, CH, CH);
     };
-    auto stage = [&](Pre& P, int buf) {
+    auto issue_b = [&](PreB& P, int c) {
+      c = min(c, sq.nchunks - 1);
+      const int tok = sq.tok0 + c * CH;
+      P.len = min(CH, sq.len - c * CH);
+      IOK::load_nomask(P.rw, row_ptr<T>(a.w, sq.b, tok, h), a.w.st, P.len);
+      IOK::load_nomask(P.rq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, P.len);
+      IOV::load_nomask(P.ru, row_ptr<T>(a.u, sq.b, tok, h) + v0, a.u.st, P.len);
+      P.graw = load_scalar_raw(gptr, a.g_dtype, gated ? row_off(a.g, sq.b, tok + min(l, P.len - 1), h) : 0);
+    };
+    auto stage_a = [&](PreA& P) {
       IOK::mask(P.rk, P.len);
+      IOK::store_lds(P.rk, s_k, LDK);
+      IOP::store_lds(P.rp, s_p, LDC);       // rows and columns past the end are zero as written
+    };
+    auto stage_b = [&](PreB& P, int buf) {
+      IOK::mask(P.rw, P.len);
       IOV::mask(P.ru, P.len);
-      IOK::store_lds(P.rk, s_k[buf], LDK);
-      IOV::store_lds(P.ru, s_u[buf], LDU);
+      IOK::store_lds(P.rw, s_w, LDK);
+      IOK::store_lds(P.rq, s_q, LDK);       // rows past the end only reach output rows that are not stored
+      IOV::store_lds(P.ru, s_u, LDU);
       if (wave_id() == 4) {
         const float x = wave_incl_scan((gated && l < P.len) ? scalar_from_raw(P.graw, a.g_dtype) : 0.f);
         const float xl = __shfl(x, 63, 64);
@@ -102,29 +143,34 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
         if (l == 0) s_dec[buf] = expf(xl);
       }
     };
+    // o and v_new of chunk c: LDS -> global
+    auto store_results = [&](int c) {
+      const int tok = sq.tok0 + c * CH;
+      const int len = min(CH, sq.len - c * CH);
+      IOV::lds_to_global(s_vn, LDU, row_ptr<T>(a.vnew, sq.b, tok, h) + v0, a.vnew.st, len);
+      IOV::lds_to_global(s_o, LDU, row_ptr<T>(a.o, sq.b, tok, h) + v0, a.o.st, len);
+    };
 #pragma unroll
-    for (int j = 0; j < LPF; ++j) issue(pre[j], j);
-    stage(pre[0], 0);
-    issue(pre[0], LPF);
+    for (int j = 0; j < LPF; ++j) { issue_b(pb[j], j); issue_a(pa[j], j); }
+    stage_b(pb[0], 0);
+    issue_b(pb[0], LPF);
+    // the first loads may be ordered freely by the compiler; were they still pending at the loop
+    // header, its wait-count analysis would carry that order into every iteration
     wait_all_loads();
-    auto step = [&](auto slot, const int c) {
-      constexpr int j = decltype(slot)::value;
+    ring_loop<LPF>(sq.nchunks, [&](auto slot, const int c) {
+      constexpr int j = decltype(slot)::value, jn = (j + 1) % LPF;
       lds_barrier();                                                                     // B1
+      stage_a(pa[j]);
       // hs[chunk][h][v0 .. v0+BV][K] <- S^T
       IOHT::lds_to_global(s_hT, LDK, (T*)a.hs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
-      if (c + 1 < sq.nchunks) stage(pre[(j + 1) % LPF], (c + 1) & 1);
+      if (c > 0) store_results(c - 1);
+      issue_a(pa[j], c + LPF);
       lds_barrier();                                                                     // B2
-      issue(pre[(j + 1) % LPF], c + 1 + LPF);
-    };
-    // whole groups of LPF chunks without an exit in between (see the consumers)
-    int c0 = 0;
-    for (; c0 + LPF <= sq.nchunks; c0 += LPF) {
-      step(std::integral_constant<int, 0>(), c0);
-      step(std::integral_constant<int, 1>(), c0 + 1);
-      step(std::integral_constant<int, 2>(), c0 + 2);
-    }
-    if (c0 < sq.nchunks) step(std::integral_constant<int, 0>(), c0);
-    if (c0 + 1 < sq.nchunks) step(std::integral_constant<int, 1>(), c0 + 1);
+      if (c + 1 < sq.nchunks) stage_b(pb[jn], (c + 1) & 1);
+      issue_b(pb[jn], c + 1 + LPF);
+    });
+    lds_barrier();                                                                       // results of the last chunk
+    store_results(sq.nchunks - 1);
     return;
   }
 
@@ -132,6 +178,7 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
   const int wv = wave_id();
   const int krow0 = wv * (K / 4);
   const int fr = l & 15, fg = 8 * (l >> 4);          // fragment row / contraction offset of this lane
+  const float scale = a.scale;
   f32x4 S[MB][NB];
   acc_zero(S);
   if (a.h0) {
@@ -144,109 +191,74 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
         for (int i = 0; i < 4; ++i)
           S[mi][ni][i] = h0[(int64_t)(krow0 + acc_row(mi, i)) * V + v0 + acc_col(ni)];
   }
-  // this wave's strips of w, q (rows of the chunk) and P, kept PF chunks ahead in registers
-  RowFrags<T, K> fw[PF], fq[PF];
-  RowFrags<T, CH> fp[PF];
-  auto issue = [&](RowFrags<T, K>& W, RowFrags<T, K>& Q, RowFrags<T, CH>& P, int c) {
-    c = min(c, sq.nchunks - 1);
-    const int tok = sq.tok0 + c * CH;
-    const int last = min(CH, sq.len - c * CH) - 1;
-    W.load(row_ptr<T>(a.w, sq.b, tok, h), a.w.st, 16 * wv, last);
-    Q.load(row_ptr<T>(a.q, sq.b, tok, h), a.q.st, 16 * wv, last);
-    P.load((const T*)a.pmat + ((int64_t)(sq.chunk0 + c) * a.H + h) * 2 * CH * CH, CH, 16 * wv, CH - 1);
-  };
+  for (int c = 0; c < sq.nchunks; ++c) {
+    const int cur = c & 1;
+    // S (state at chunk start) -> LDS as S^T
 #pragma unroll
-  for (int j = 0; j < PF; ++j) issue(fw[j], fq[j], fp[j], j);
-  // The compiler may order these first loads freely; were they still pending at the loop header,
-  // its wait-count analysis would merge that order into every iteration (a full drain per trip).
-  wait_all_loads();
-
-  // one chunk; `slot` (compile-time) names the register set that holds its strips
-  auto step = [&](auto slot, const int c) {
-    {
-      constexpr int j = decltype(slot)::value;
-      const int cur = c & 1;
-      const int tok = sq.tok0 + c * CH;
-      const int len = min(CH, sq.len - c * CH);
-      // S (state at chunk start) -> LDS as S^T
+    for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
-      for (int mi = 0; mi < MB; ++mi)
+      for (int ni = 0; ni < NB; ++ni) acc_to_lds_t<T>(S[mi][ni], s_hT, LDK, krow0 + 16 * mi, 16 * ni);
+    lds_barrier();                                                                       // B1
+    // w S and q S over the same S^T fragments (rows 16 wv .. of the chunk)
+    f32x4 vn[1][NB], o[1][NB];
+    acc_zero(vn);
+    acc_zero(o);
 #pragma unroll
-        for (int ni = 0; ni < NB; ++ni) acc_to_lds_t<T>(S[mi][ni], s_hT, LDK, krow0 + 16 * mi, 16 * ni);
-      lds_barrier();                                                                     // B1
-      // w S and q S over the same S^T fragments (rows 16 wv .. of the chunk)
-      f32x4 vn[1][NB], o[1][NB];
-      acc_zero(vn);
-      acc_zero(o);
-      fw[j].mask(16 * wv, len);
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        typename ET<T>::frag bS[NB];
-#pragma unroll
-        for (int ni = 0; ni < NB; ++ni) bS[ni] = ET<T>::load_frag(s_hT + (16 * ni + fr) * LDK + 32 * ks + fg);
-#pragma unroll
-        for (int ni = 0; ni < NB; ++ni) {
-          ET<T>::mma(vn[0][ni], fw[j].f[ks], bS[ni]);
-          ET<T>::mma(o[0][ni], fq[j].f[ks], bS[ni]);
-        }
-      }
+    for (int ks = 0; ks < KS; ++ks) {
+      const typename ET<T>::frag aw = ET<T>::load_frag(s_w + (16 * wv + fr) * LDK + 32 * ks + fg);
+      const typename ET<T>::frag aq = ET<T>::load_frag(s_q + (16 * wv + fr) * LDK + 32 * ks + fg);
 #pragma unroll
       for (int ni = 0; ni < NB; ++ni) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
-          // v_new = u - w S, rounded once to the storage type so that the state update, the
-          // output and the backward see the same values
-          vn[0][ni][i] = ET<T>::to_f(ET<T>::from_f(ET<T>::to_f(s_u[cur][r * LDU + cc]) - vn[0][ni][i]));
-          o[0][ni][i] *= s_eb[cur][r];
-        }
-        acc_to_lds_t<T>(vn[0][ni], s_vT, LDC, 16 * wv, 16 * ni);
+        const typename ET<T>::frag bS = ET<T>::load_frag(s_hT + (16 * ni + fr) * LDK + 32 * ks + fg);
+        ET<T>::mma(vn[0][ni], aw, bS);
+        ET<T>::mma(o[0][ni], aq, bS);
       }
-      const float dec = s_dec[cur];
-      lds_barrier();                                                                     // B2
+    }
+#pragma unroll
+    for (int ni = 0; ni < NB; ++ni) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
+        // v_new = u - w S, rounded once to the storage type so that the state update, the
+        // output and the backward see the same values
+        vn[0][ni][i] = ET<T>::to_f(ET<T>::from_f(ET<T>::to_f(s_u[r * LDU + cc]) - vn[0][ni][i]));
+        o[0][ni][i] *= s_eb[cur][r];
+      }
+      acc_to_lds_t<T>(vn[0][ni], s_vT, LDC, 16 * wv, 16 * ni);
+    }
+    const float dec = s_dec[cur];
+    lds_barrier();                                                                       // B2
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) S[mi][ni] *= dec;
+    // o += P v_new ;  S += k^T (e_d v_new)   over the same v_new^T fragments
+#pragma unroll
+    for (int ks = 0; ks < CH / 32; ++ks) {
+      typename ET<T>::frag af[MB], bv[NB];
+      const typename ET<T>::frag ap = ET<T>::load_frag(s_p + (16 * wv + fr) * LDC + 32 * ks + fg);
+#pragma unroll
+      for (int mi = 0; mi < MB; ++mi) af[mi] = ET<T>::load_frag_t(s_k, LDK, 32 * ks, krow0 + 16 * mi);
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) {
+        bv[ni] = ET<T>::load_frag(s_vT + (16 * ni + fr) * LDC + 32 * ks + fg);
+        ET<T>::mma(o[0][ni], ap, bv[ni]);
+        scale_frag8<T>(bv[ni], &s_ed[cur][32 * ks + fg]);
+      }
 #pragma unroll
       for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < NB; ++ni) S[mi][ni] *= dec;
-      // o += P v_new ;  S += k^T (e_d v_new)   over the same v_new^T fragments
-#pragma unroll
-      for (int ks = 0; ks < CH / 32; ++ks) {
-        typename ET<T>::frag af[MB], bv[NB];
-#pragma unroll
-        for (int mi = 0; mi < MB; ++mi) af[mi] = ET<T>::load_frag_t(s_k[cur], LDK, 32 * ks, krow0 + 16 * mi);
-#pragma unroll
-        for (int ni = 0; ni < NB; ++ni) {
-          bv[ni] = ET<T>::load_frag(s_vT + (16 * ni + fr) * LDC + 32 * ks + fg);
-          ET<T>::mma(o[0][ni], fp[j].f[ks], bv[ni]);
-          scale_frag8<T>(bv[ni], &s_ed[cur][32 * ks + fg]);
-        }
-#pragma unroll
-        for (int mi = 0; mi < MB; ++mi)
-#pragma unroll
-          for (int ni = 0; ni < NB; ++ni) ET<T>::mma(S[mi][ni], af[mi], bv[ni]);
-      }
-      issue(fw[j], fq[j], fp[j], c + PF);
-      store_strip<T, NB>(vn, s_stg + wv * 16 * LDU, row_ptr<T>(a.vnew, sq.b, tok + 16 * wv, h) + v0, a.vnew.st,
-                         len - 16 * wv, 1.0f);
-      store_strip<T, NB>(o, s_ost + wv * 16 * LDU, row_ptr<T>(a.o, sq.b, tok + 16 * wv, h) + v0, a.o.st,
-                         len - 16 * wv, a.scale);
+        for (int ni = 0; ni < NB; ++ni) ET<T>::mma(S[mi][ni], af[mi], bv[ni]);
     }
-  };
-  // Whole groups of PF chunks run without an exit between the chunks: an early exit inside the
-  // group would be one more path to the loop header, on which the compiler could count only the
-  // loads of the first chunk as issued and would drain the prefetch ring on every trip.
-  int c0 = 0;
-  for (; c0 + PF <= sq.nchunks; c0 += PF) {
-    step(std::integral_constant<int, 0>(), c0);
-    if constexpr (PF > 1) step(std::integral_constant<int, 1 % PF>(), c0 + 1);
-    if constexpr (PF > 2) step(std::integral_constant<int, 2 % PF>(), c0 + 2);
-  }
-  if constexpr (PF > 1) {
-    if (c0 < sq.nchunks) step(std::integral_constant<int, 0>(), c0);
-    if constexpr (PF > 2) {
-      if (c0 + 1 < sq.nchunks) step(std::integral_constant<int, 1 % PF>(), c0 + 1);
+#pragma unroll
+    for (int ni = 0; ni < NB; ++ni) {
+      // results for the loaders (they store the previous chunk's during phase 1, hence not earlier)
+      o[0][ni] *= scale;
+      acc_to_lds<T>(o[0][ni], s_o, LDU, 16 * wv, 16 * ni);
+      acc_to_lds<T>(vn[0][ni], s_vn, LDU, 16 * wv, 16 * ni);
     }
   }
+  lds_barrier();                                                                         // results of the last chunk
   if (a.ht) {
     float* ht = a.ht + ((int64_t)n * a.H + h) * K * V;
 #pragma unroll
@@ -260,25 +272,26 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
 }
 
 // ------------------------------------------------------------------------- //
-// backward (reverse order over the chunks)
+// backward (reverse order over the chunks; it = 0 is the last chunk)
+//   loaders, chunk c:  B1 | stage q(c), w(c); store dhs(c), dv_new(c+1); prefetch q, w |
+//                      B2 | stage k, P^T, do, gates of chunk c-1; prefetch k, P^T, do, g
+//   consumers, chunk c: dS' -> LDS | B1 | k dS', P^T do, dv_new -> LDS | B2 | dS update
 // ------------------------------------------------------------------------- //
 template <typename T, int K, int V, int BV>
 __global__ __launch_bounds__(2 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
   constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDU = BV + LPAD;
   constexpr int MB = K / 64, NB = BV / 16, KS = K / 32;
-  constexpr int PF = GdnStateCfg<T>::PF, LPF = GdnStateCfg<T>::LPF;
-  static_assert(LPF == 3 && PF <= 3, "the chunk loops are written out for rings of three");
-  // two operand buffers; fp32 tiles with K = 128 (the parity path) leave LDS for one and pay a
-  // third barrier per chunk
-  constexpr int NBUF = (sizeof(T) == 4 && K == 128) ? 1 : 2;
-  __shared__ __attribute__((aligned(16))) T s_q[NBUF][CH * LDK];    // q        [64][K]
-  __shared__ __attribute__((aligned(16))) T s_w[NBUF][CH * LDK];    // w        [64][K]
-  __shared__ __attribute__((aligned(16))) T s_do[NBUF][CH * LDU];   // do       [64][BV]
-  __shared__ __attribute__((aligned(16))) T s_dST[BV * LDK];        // dS'^T    [BV][K]
+  constexpr int LPF = GdnStateCfg<T>::LPF;
+  __shared__ __attribute__((aligned(16))) T s_q[CH * LDK];          // q         [64][K]
+  __shared__ __attribute__((aligned(16))) T s_w[CH * LDK];          // w         [64][K]
+  __shared__ __attribute__((aligned(16))) T s_k[CH * LDK];          // k         [64][K]
+  __shared__ __attribute__((aligned(16))) T s_pt[CH * LDC];         // P^T       [64][64]
+  __shared__ __attribute__((aligned(16))) T s_do[CH * LDU];         // do        [64][BV]
+  __shared__ __attribute__((aligned(16))) T s_dST[BV * LDK];        // dS'^T     [BV][K]
   __shared__ __attribute__((aligned(16))) T s_dvT[BV * LDC];        // -dv_new^T [BV][64]
-  __shared__ __attribute__((aligned(16))) T s_stg[4 * 16 * LDU];    // dv_new store strips
-  __shared__ __attribute__((aligned(16))) float s_qs[NBUF][64], s_ed[NBUF][64];
-  __shared__ float s_dec[NBUF];
+  __shared__ __attribute__((aligned(16))) T s_dvn[CH * LDU];        // dv_new    [64][BV] (to be stored)
+  __shared__ __attribute__((aligned(16))) float s_qs[2][64], s_ed[2][64];
+  __shared__ float s_dec[2];                                        // gate arrays: buffer it & 1
 
   constexpr int NVS = V / BV;
   const int xcd = blockIdx.x & 7, jj = blockIdx.x >> 3;
@@ -300,33 +313,49 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
   }
   typedef TileIO<T, CH, K> IOK;
   typedef TileIO<T, CH, BV> IOV;
+  typedef TileIO<T, CH, CH> IOP;
   typedef TileIO<T, BV, K> IOHT;
 
   if (team == 1) {
     // --------------------------------- loaders -------------------------------------------
-    struct Pre { typename IOK::Regs rq, rw; typename IOV::Regs rd; uint32_t graw; int len; };
-    Pre pre[LPF];
+    // ring A = what phase 2 of the chunk's own step reads (q, w), ring B = what phase 1 reads
+    // (k, P^T, do, gates), staged during phase 2 of the step before
+    struct PreA { typename IOK::Regs rq, rw; int len; };
+    struct PreB { typename IOK::Regs rk; typename IOP::Regs rp; typename IOV::Regs rd; uint32_t graw; int len; };
+    PreA pa[LPF];
+    PreB pb[LPF];
     const bool gated = a.gate != LMOE_GATE_NONE && a.g.ptr != nullptr;
     const void* gptr = gated ? a.g.ptr : a.k.ptr;
     const float scale = a.scale;
-    // always issued, chunk index clamped (see k_gdn_state_fwd)
-    auto issue = [&](Pre& P, int c) {
-      c = max(c, 0);
+    // always issued, chunk index clamped (see k_gdn_state_fwd); `it` counts chunks from the end
+    auto issue_a = [&](PreA& P, int it) {
+      const int c = max(sq.nchunks - 1 - it, 0);
       const int tok = sq.tok0 + c * CH;
-      const int len = min(CH, sq.len - c * CH);
-      IOK::load_nomask(P.rq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, len);
-      IOK::load_nomask(P.rw, row_ptr<T>(a.w, sq.b, tok, h), a.w.st, len);
-      IOV::load_nomask(P.rd, row_ptr<T>(a.d_o, sq.b, tok, h) + v0, a.d_o.st, len);
-      P.len = len;
-      P.graw = load_scalar_raw(gptr, a.g_dtype, gated ? row_off(a.g, sq.b, tok + min(l, len - 1), h) : 0);
+      P.len = min(CH, sq.len - c * CH);
+      IOK::load_nomask(P.rq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, P.len);
+      IOK::load_nomask(P.rw, row_ptr<T>(a.w, sq.b, tok, h), a.w.st, P.len);
     };
-    auto stage = [&](Pre& P, int buf) {
+    auto issue_b = [&](PreB& P, int it) {
+      const int c = max(sq.nchunks - 1 - it, 0);
+      const int tok = sq.tok0 + c * CH;
+      P.len = min(CH, sq.len - c * CH);
+      IOK::load_nomask(P.rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, P.len);
+      IOP::load_nomask(P.rp, (const T*)a.pmat + (((int64_t)(sq.chunk0 + c) * a.H + h) * 2 + 1) * CH * CH, CH, CH);
+      IOV::load_nomask(P.rd, row_ptr<T>(a.d_o, sq.b, tok, h) + v0, a.d_o.st, P.len);
+      P.graw = load_scalar_raw(gptr, a.g_dtype, gated ? row_off(a.g, sq.b, tok + min(l, P.len - 1), h) : 0);
+    };
+    auto stage_a = [&](PreA& P) {
       IOK::mask(P.rq, P.len);
       IOK::mask(P.rw, P.len);
+      IOK::store_lds(P.rq, s_q, LDK);
+      IOK::store_lds(P.rw, s_w, LDK);
+    };
+    auto stage_b = [&](PreB& P, int buf) {
+      IOK::mask(P.rk, P.len);
       IOV::mask(P.rd, P.len);
-      IOK::store_lds(P.rq, s_q[buf], LDK);
-      IOK::store_lds(P.rw, s_w[buf], LDK);
-      IOV::store_lds(P.rd, s_do[buf], LDU);
+      IOK::store_lds(P.rk, s_k, LDK);
+      IOP::store_lds(P.rp, s_pt, LDC);      // rows and columns past the end are zero as written
+      IOV::store_lds(P.rd, s_do, LDU);
       if (wave_id() == 4) {
         const float x = wave_incl_scan((gated && l < P.len) ? scalar_from_raw(P.graw, a.g_dtype) : 0.f);
         const float xl = __shfl(x, 63, 64);
@@ -335,35 +364,30 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
         if (l == 0) s_dec[buf] = expf(xl);
       }
     };
+    auto store_results = [&](int c) {
+      const int tok = sq.tok0 + c * CH;
+      const int len = min(CH, sq.len - c * CH);
+      IOV::lds_to_global(s_dvn, LDU, row_ptr<T>(a.dvnew, sq.b, tok, h) + v0, a.dvnew.st, len);
+    };
 #pragma unroll
-    for (int j = 0; j < LPF; ++j) issue(pre[j], sq.nchunks - 1 - j);
-    stage(pre[0], 0);
-    issue(pre[0], sq.nchunks - 1 - LPF);
-    wait_all_loads();
-    auto step = [&](auto slot, const int it) {
-      constexpr int j = decltype(slot)::value;
+    for (int j = 0; j < LPF; ++j) { issue_b(pb[j], j); issue_a(pa[j], j); }
+    stage_b(pb[0], 0);
+    issue_b(pb[0], LPF);
+    wait_all_loads();   // see k_gdn_state_fwd
+    ring_loop<LPF>(sq.nchunks, [&](auto slot, const int it) {
+      constexpr int j = decltype(slot)::value, jn = (j + 1) % LPF;
       const int c = sq.nchunks - 1 - it;
       lds_barrier();                                                                     // B1
+      stage_a(pa[j]);
       IOHT::lds_to_global(s_dST, LDK, (T*)a.dhs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
-      if constexpr (NBUF == 2) {
-        if (c > 0) stage(pre[(j + 1) % LPF], (it + 1) & 1);
-      }
+      if (it > 0) store_results(c + 1);
+      issue_a(pa[j], it + LPF);
       lds_barrier();                                                                     // B2
-      if constexpr (NBUF == 1) {
-        lds_barrier();                                                                   // B3: buffer read
-        if (c > 0) stage(pre[(j + 1) % LPF], 0);
-      }
-      issue(pre[(j + 1) % LPF], c - 1 - LPF);
-    };
-    // whole groups of LPF chunks without an exit in between (see k_gdn_state_fwd)
-    int it0 = 0;
-    for (; it0 + LPF <= sq.nchunks; it0 += LPF) {
-      step(std::integral_constant<int, 0>(), it0);
-      step(std::integral_constant<int, 1>(), it0 + 1);
-      step(std::integral_constant<int, 2>(), it0 + 2);
-    }
-    if (it0 < sq.nchunks) step(std::integral_constant<int, 0>(), it0);
-    if (it0 + 1 < sq.nchunks) step(std::integral_constant<int, 1>(), it0 + 1);
+      if (c > 0) stage_b(pb[jn], (it + 1) & 1);
+      issue_b(pb[jn], it + 1 + LPF);
+    });
+    lds_barrier();                                                                       // dv_new of chunk 0
+    store_results(0);
     return;
   }
 
@@ -384,113 +408,80 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
         for (int i = 0; i < 4; ++i)
           dS[mi][ni][i] = p[(int64_t)(krow0 + acc_row(mi, i)) * V + v0 + acc_col(ni)];
   }
-  // this wave's strips of k (rows of the chunk) and P^T, kept PF chunks ahead in registers
-  RowFrags<T, K> fk[PF];
-  RowFrags<T, CH> fpt[PF];
-  auto issue = [&](RowFrags<T, K>& Kf, RowFrags<T, CH>& Pt, int c) {
-    c = max(c, 0);
-    const int tok = sq.tok0 + c * CH;
-    const int last = min(CH, sq.len - c * CH) - 1;
-    Kf.load(row_ptr<T>(a.k, sq.b, tok, h), a.k.st, 16 * wv, last);
-    Pt.load((const T*)a.pmat + (((int64_t)(sq.chunk0 + c) * a.H + h) * 2 + 1) * CH * CH, CH, 16 * wv, CH - 1);
-  };
+  for (int it = 0; it < sq.nchunks; ++it) {
+    const int cur = it & 1;
 #pragma unroll
-  for (int j = 0; j < PF; ++j) issue(fk[j], fpt[j], sq.nchunks - 1 - j);
-  wait_all_loads();   // see k_gdn_state_fwd
-
-  // one chunk (the it-th from the end); `slot` (compile-time) names its register set
-  auto step = [&](auto slot, const int it) {
-    {
-      constexpr int j = decltype(slot)::value;
-      const int c = sq.nchunks - 1 - it;
-      const int cur = NBUF == 2 ? (it & 1) : 0;
-      const int tok = sq.tok0 + c * CH;
-      const int len = min(CH, sq.len - c * CH);
+    for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
-      for (int mi = 0; mi < MB; ++mi)
+      for (int ni = 0; ni < NB; ++ni) acc_to_lds_t<T>(dS[mi][ni], s_dST, LDK, krow0 + 16 * mi, 16 * ni);
+    lds_barrier();                                                                       // B1
+    // t = k dS'  and  dv_loc = P^T do   (rows 16 wv .. of the chunk)
+    f32x4 t[1][NB], dvl[1][NB];
+    acc_zero(t);
+    acc_zero(dvl);
 #pragma unroll
-        for (int ni = 0; ni < NB; ++ni) acc_to_lds_t<T>(dS[mi][ni], s_dST, LDK, krow0 + 16 * mi, 16 * ni);
-      lds_barrier();                                                                     // B1
-      // t = k dS'  and  dv_loc = P^T do   (rows 16 wv .. of the chunk)
-      f32x4 t[1][NB], dvl[1][NB];
-      acc_zero(t);
-      acc_zero(dvl);
-      fk[j].mask(16 * wv, len);
+    for (int ks = 0; ks < KS; ++ks) {
+      const typename ET<T>::frag ak = ET<T>::load_frag(s_k + (16 * wv + fr) * LDK + 32 * ks + fg);
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
+      for (int ni = 0; ni < NB; ++ni)
+        ET<T>::mma(t[0][ni], ak, ET<T>::load_frag(s_dST + (16 * ni + fr) * LDK + 32 * ks + fg));
+    }
+    typename ET<T>::frag bdo[CH / 32][NB];
 #pragma unroll
-        for (int ni = 0; ni < NB; ++ni) {
-          const typename ET<T>::frag bD = ET<T>::load_frag(s_dST + (16 * ni + fr) * LDK + 32 * ks + fg);
-          ET<T>::mma(t[0][ni], fk[j].f[ks], bD);
-        }
-      }
-      typename ET<T>::frag bdo[CH / 32][NB];
-#pragma unroll
-      for (int ks = 0; ks < CH / 32; ++ks)
-#pragma unroll
-        for (int ni = 0; ni < NB; ++ni) {
-          bdo[ks][ni] = ET<T>::load_frag_t(s_do[cur], LDU, 32 * ks, 16 * ni);
-          ET<T>::mma(dvl[0][ni], fpt[j].f[ks], bdo[ks][ni]);
-        }
+    for (int ks = 0; ks < CH / 32; ++ks) {
+      const typename ET<T>::frag ap = ET<T>::load_frag(s_pt + (16 * wv + fr) * LDC + 32 * ks + fg);
 #pragma unroll
       for (int ni = 0; ni < NB; ++ni) {
-        f32x4 x;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int r = 16 * wv + 4 * (l >> 4) + i;
-          // dv_new, rounded once to the storage type (the WY backward reads the stored values)
-          t[0][ni][i] = ET<T>::to_f(ET<T>::from_f(scale * dvl[0][ni][i] + s_ed[cur][r] * t[0][ni][i]));
-          x[i] = -t[0][ni][i];
-        }
-        acc_to_lds_t<T>(x, s_dvT, LDC, 16 * wv, 16 * ni);
+        bdo[ks][ni] = ET<T>::load_frag_t(s_do, LDU, 32 * ks, 16 * ni);
+        ET<T>::mma(dvl[0][ni], ap, bdo[ks][ni]);
       }
-      const float dec = s_dec[cur];
-      lds_barrier();                                                                     // B2
+    }
+#pragma unroll
+    for (int ks = 0; ks < CH / 32; ++ks)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) scale_frag8<T>(bdo[ks][ni], &s_qs[cur][32 * ks + fg]);
+#pragma unroll
+    for (int ni = 0; ni < NB; ++ni) {
+      f32x4 x;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = 16 * wv + 4 * (l >> 4) + i;
+        // dv_new, rounded once to the storage type (the WY backward reads the stored values)
+        t[0][ni][i] = ET<T>::to_f(ET<T>::from_f(scale * dvl[0][ni][i] + s_ed[cur][r] * t[0][ni][i]));
+        x[i] = -t[0][ni][i];
+      }
+      acc_to_lds_t<T>(x, s_dvT, LDC, 16 * wv, 16 * ni);
+    }
+    const float dec = s_dec[cur];
+    lds_barrier();                                                                       // B2
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) dS[mi][ni] *= dec;
+    // dS += q^T (scale e_b do) - w^T dv_new
+#pragma unroll
+    for (int ks = 0; ks < CH / 32; ++ks) {
+      typename ET<T>::frag aq[MB], aw[MB], bn[NB];
+#pragma unroll
+      for (int mi = 0; mi < MB; ++mi) {
+        aq[mi] = ET<T>::load_frag_t(s_q, LDK, 32 * ks, krow0 + 16 * mi);
+        aw[mi] = ET<T>::load_frag_t(s_w, LDK, 32 * ks, krow0 + 16 * mi);
+      }
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) bn[ni] = ET<T>::load_frag(s_dvT + (16 * ni + fr) * LDC + 32 * ks + fg);
 #pragma unroll
       for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < NB; ++ni) dS[mi][ni] *= dec;
-      // dS += q^T (scale e_b do) - w^T dv_new
-#pragma unroll
-      for (int ks = 0; ks < CH / 32; ++ks) {
-        typename ET<T>::frag aq[MB], aw[MB], bn[NB];
-#pragma unroll
-        for (int mi = 0; mi < MB; ++mi) {
-          aq[mi] = ET<T>::load_frag_t(s_q[cur], LDK, 32 * ks, krow0 + 16 * mi);
-          aw[mi] = ET<T>::load_frag_t(s_w[cur], LDK, 32 * ks, krow0 + 16 * mi);
-        }
-#pragma unroll
         for (int ni = 0; ni < NB; ++ni) {
-          scale_frag8<T>(bdo[ks][ni], &s_qs[cur][32 * ks + fg]);
-          bn[ni] = ET<T>::load_frag(s_dvT + (16 * ni + fr) * LDC + 32 * ks + fg);
+          ET<T>::mma(dS[mi][ni], aq[mi], bdo[ks][ni]);
+          ET<T>::mma(dS[mi][ni], aw[mi], bn[ni]);
         }
-#pragma unroll
-        for (int mi = 0; mi < MB; ++mi)
-#pragma unroll
-          for (int ni = 0; ni < NB; ++ni) {
-            ET<T>::mma(dS[mi][ni], aq[mi], bdo[ks][ni]);
-            ET<T>::mma(dS[mi][ni], aw[mi], bn[ni]);
-          }
-      }
-      if constexpr (NBUF == 1) lds_barrier();                                            // B3
-      issue(fk[j], fpt[j], c - PF);
-      store_strip<T, NB>(t, s_stg + wv * 16 * LDU, row_ptr<T>(a.dvnew, sq.b, tok + 16 * wv, h) + v0, a.dvnew.st,
-                         len - 16 * wv, 1.0f);
     }
-  };
-  // whole groups of PF chunks without an exit in between (see k_gdn_state_fwd)
-  int it0 = 0;
-  for (; it0 + PF <= sq.nchunks; it0 += PF) {
-    step(std::integral_constant<int, 0>(), it0);
-    if constexpr (PF > 1) step(std::integral_constant<int, 1 % PF>(), it0 + 1);
-    if constexpr (PF > 2) step(std::integral_constant<int, 2 % PF>(), it0 + 2);
+    // dv_new for the loaders (they store the previous chunk's during phase 1, hence not earlier)
+#pragma unroll
+    for (int ni = 0; ni < NB; ++ni) acc_to_lds<T>(t[0][ni], s_dvn, LDU, 16 * wv, 16 * ni);
   }
-  if constexpr (PF > 1) {
-    if (it0 < sq.nchunks) step(std::integral_constant<int, 0>(), it0);
-    if constexpr (PF > 2) {
-      if (it0 + 1 < sq.nchunks) step(std::integral_constant<int, 1 % PF>(), it0 + 1);
-    }
-  }
+  lds_barrier();                                                                         // dv_new of chunk 0
   if (a.dh0) {
     float* p = a.dh0 + ((int64_t)n * a.H + h) * K * V;
 #pragma unroll
