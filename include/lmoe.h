@@ -77,6 +77,8 @@ typedef struct lmoe_args {
   void* amat;          /* [NT,H,64,64] intra-chunk attention matrix (chunk_gla)        */
   void* pmat;          /* [NT,H,2,64,64] P = (q k^T) . Gamma and its transpose per chunk
                           (gated delta rule; written by the WY preparation)             */
+  float* gcum;         /* [NT,H,2,64] fp32 e^{b_j} and e^{b_C - b_j}, b = cumulative log-decay
+                          inside the chunk (gated delta rule; written by the WY preparation) */
   /* backward inputs */
   lmoe_tensor d_o;     /* [B,T,H,V] gradient of o                                      */
   const float* dht;    /* [N,H,K,V] fp32 gradient of the final state or NULL           */
@@ -97,7 +99,7 @@ int lmoe_version(void);
 const char* lmoe_last_error(void);
 
 /* Bytes of caller-allocated intermediates of one call: part 0 = what *_fwd writes for *_bwd
- * (hs, and per op amat / vnew, w, u, tinv, pmat), part 1 = the backward workspace (dhs, and dvnew, dw
+ * (hs, and per op amat / vnew, w, u, tinv, pmat, gcum), part 1 = the backward workspace (dhs, and dvnew, dw
  * for the gated delta rule).  Each buffer is still passed through its own lmoe_args field; this
  * is the sum a caller that carves them out of one arena must reserve (every buffer's size is a
  * multiple of 256 bytes for the supported K, V).  Negative for an invalid op / dtype / part.
@@ -127,8 +129,8 @@ int lmoe_chunk_gla_bwd(const lmoe_args* a, void* stream);
  * o_t = scale q_t S_t.
  * Replaces fla.ops.gated_delta_rule.chunk_gated_delta_rule called at
  *   linear_moe/sequence_modeling/gated_deltanet/gated_deltanet.py:112.
- * fwd uses q,k,v,g,beta,h0 -> o,ht,hs,vnew,w,u,tinv,pmat.
- * bwd uses q,k,v,g,beta,hs,vnew,w,tinv,pmat,d_o,dht -> dq,dk,dv,dg,dbeta,dh0 (+ dhs, dvnew, dw). */
+ * fwd uses q,k,v,g,beta,h0 -> o,ht,hs,vnew,w,u,tinv,pmat,gcum.
+ * bwd uses q,k,v,g,beta,hs,vnew,w,tinv,pmat,gcum,d_o,dht -> dq,dk,dv,dg,dbeta,dh0 (+ dhs, dvnew, dw). */
 int lmoe_chunk_gated_delta_rule_fwd(const lmoe_args* a, void* stream);
 int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream);
 

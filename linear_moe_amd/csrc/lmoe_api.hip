@@ -59,7 +59,9 @@ int64_t lmoe_workspace_bytes(int32_t op, int32_t dtype, int32_t part, int32_t B,
   if (op == LMOE_OP_GLA && part == 0) n += tiles;                        // amat
   if (op == LMOE_OP_GATED_DELTA_RULE) n += part == 0 ? 2 * rows_v + rows_k + 3 * tiles   // vnew, u, w, tinv, pmat
                                                      : rows_v + rows_k;              // dvnew, dw
-  return n * s;
+  int64_t bytes = n * s;
+  if (op == LMOE_OP_GATED_DELTA_RULE && part == 0) bytes += (int64_t)NT * H * 2 * LMOE_CHUNK * 4;   // gcum (fp32)
+  return bytes;
 }
 
 int lmoe_chunk_simple_gla_fwd(const lmoe_args* a, void* stream) {
@@ -122,8 +124,8 @@ int lmoe_chunk_gated_delta_rule_fwd(const lmoe_args* a, void* stream) {
   if (int r = check_common(a, op)) return r;
   if (a->gate == LMOE_GATE_VECTOR) return fail(-10, "%s: the gate is one scalar per token and head", op);
   if (!a->beta.ptr) return fail(-12, "%s: beta must not be null", op);
-  if (!a->o.ptr || !a->hs || !a->vnew.ptr || !a->w.ptr || !a->u.ptr || !a->tinv || !a->pmat)
-    return fail(-11, "%s: o, hs, vnew, w, u, tinv and pmat must not be null", op);
+  if (!a->o.ptr || !a->hs || !a->vnew.ptr || !a->w.ptr || !a->u.ptr || !a->tinv || !a->pmat || !a->gcum)
+    return fail(-11, "%s: o, hs, vnew, w, u, tinv, pmat and gcum must not be null", op);
   if (a->NT == 0 || a->N == 0) return 0;
   lmoe::launch_gdn_wy_fwd(*a, (hipStream_t)stream);
   lmoe::launch_gdn_state_fwd(*a, (hipStream_t)stream);
@@ -134,8 +136,8 @@ int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream) {
   if (int r = check_common(a, op)) return r;
   if (a->gate == LMOE_GATE_VECTOR) return fail(-10, "%s: the gate is one scalar per token and head", op);
   if (!a->beta.ptr) return fail(-12, "%s: beta must not be null", op);
-  if (!a->hs || !a->dhs || !a->vnew.ptr || !a->w.ptr || !a->tinv || !a->pmat || !a->dvnew.ptr || !a->dw.ptr)
-    return fail(-11, "%s: hs, dhs, vnew, w, tinv, pmat, dvnew and dw must not be null", op);
+  if (!a->hs || !a->dhs || !a->vnew.ptr || !a->w.ptr || !a->tinv || !a->pmat || !a->gcum || !a->dvnew.ptr || !a->dw.ptr)
+    return fail(-11, "%s: hs, dhs, vnew, w, tinv, pmat, gcum, dvnew and dw must not be null", op);
   if (!a->d_o.ptr || !a->dq.ptr || !a->dk.ptr || !a->dv.ptr || !a->dg.ptr || !a->dbeta.ptr)
     return fail(-13, "%s: d_o, dq, dk, dv, dg and dbeta must not be null", op);
   if (a->NT == 0 || a->N == 0) return 0;
@@ -154,11 +156,11 @@ int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* strea
   if (op == LMOE_OP_SIMPLE_GLA || gdn) {
     switch (stage) {
       case lmoe::ST_GDN_WY_FWD: if (!gdn) return fail(-20, "%s: stage not part of this op", nm);
-        if (!a->pmat) return fail(-11, "%s: pmat must not be null", nm);
+        if (!a->pmat || !a->gcum) return fail(-11, "%s: pmat and gcum must not be null", nm);
         lmoe::launch_gdn_wy_fwd(*a, st); break;
       case lmoe::ST_STATE_FWD:
         if (gdn) {
-          if (!a->pmat) return fail(-11, "%s: pmat must not be null", nm);
+          if (!a->pmat || !a->gcum) return fail(-11, "%s: pmat and gcum must not be null", nm);
           lmoe::launch_gdn_state_fwd(*a, st);
         } else {
           lmoe::launch_state_fwd(*a, st);
@@ -168,7 +170,7 @@ int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* strea
         lmoe::launch_bwd_dv(*a, false, st); break;
       case lmoe::ST_STATE_BWD:
         if (gdn) {
-          if (!a->pmat) return fail(-11, "%s: pmat must not be null", nm);
+          if (!a->pmat || !a->gcum) return fail(-11, "%s: pmat and gcum must not be null", nm);
           lmoe::launch_gdn_state_bwd(*a, st);
         } else {
           lmoe::launch_state_bwd(*a, st);

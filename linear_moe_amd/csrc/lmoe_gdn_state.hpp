@@ -51,7 +51,7 @@ template <int L, typename F> __device__ __forceinline__ void ring_loop(int n, F&
 // ------------------------------------------------------------------------- //
 // forward
 //   loaders, chunk c:  B1 | stage k(c), P(c); store hs(c), o(c-1), v_new(c-1); prefetch k, P |
-//                      B2 | stage w, q, u, gates of chunk c+1; prefetch w, q, u, g
+//                      B2 | stage w, q, u, decay table of chunk c+1; prefetch them
 //   consumers, chunk c: S -> LDS | B1 | w S, q S, v_new -> LDS | B2 | S update, P v_new, o -> LDS
 // ------------------------------------------------------------------------- //
 template <typename T, int K, int V, int BV>
@@ -100,11 +100,9 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
     // two rings of register sets: A = what phase 2 of the chunk's own step reads (k, P),
     // B = what phase 1 reads (w, q, u, gates), staged during phase 2 of the step before
     struct PreA { typename IOK::Regs rk; typename IOP::Regs rp; int len; };
-    struct PreB { typename IOK::Regs rw, rq; typename IOV::Regs ru; uint32_t graw; int len; };
+    struct PreB { typename IOK::Regs rw, rq; typename IOV::Regs ru; float eb, ed; int len; };
     PreA pa[LPF];
     PreB pb[LPF];
-    const bool gated = a.gate != LMOE_GATE_NONE && a.g.ptr != nullptr;
-    const void* gptr = gated ? a.g.ptr : a.k.ptr;
     // Always issued (chunk index clamped to the last chunk; the surplus loads at the end of a
     // sequence are never consumed): a prefetch that is skipped on some path would make the
     // compiler drain all outstanding loads at every consumer of a register set.
@@ -122,7 +120,9 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
       IOK::load_nomask(P.rw, row_ptr<T>(a.w, sq.b, tok, h), a.w.st, P.len);
       IOK::load_nomask(P.rq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, P.len);
       IOV::load_nomask(P.ru, row_ptr<T>(a.u, sq.b, tok, h) + v0, a.u.st, P.len);
-      P.graw = load_scalar_raw(gptr, a.g_dtype, gated ? row_off(a.g, sq.b, tok + min(l, P.len - 1), h) : 0);
+      const float* gc = a.gcum + ((int64_t)(sq.chunk0 + c) * a.H + h) * 2 * CH;
+      P.eb = gc[l];
+      P.ed = gc[CH + l];
     };
     auto stage_a = [&](PreA& P) {
       IOK::mask(P.rk, P.len);
@@ -136,11 +136,9 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
       IOK::store_lds(P.rq, s_q, LDK);       // rows past the end only reach output rows that are not stored
       IOV::store_lds(P.ru, s_u, LDU);
       if (wave_id() == 4) {
-        const float x = wave_incl_scan((gated && l < P.len) ? scalar_from_raw(P.graw, a.g_dtype) : 0.f);
-        const float xl = __shfl(x, 63, 64);
-        s_eb[buf][l] = expf(x);
-        s_ed[buf][l] = expf(xl - x);
-        if (l == 0) s_dec[buf] = expf(xl);
+        s_eb[buf][l] = P.eb;
+        s_ed[buf][l] = P.ed;
+        if (l == 63) s_dec[buf] = P.eb;
       }
     };
     // o and v_new of chunk c: LDS -> global
@@ -274,7 +272,7 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
 // ------------------------------------------------------------------------- //
 // backward (reverse order over the chunks; it = 0 is the last chunk)
 //   loaders, chunk c:  B1 | stage q(c), w(c); store dhs(c), dv_new(c+1); prefetch q, w |
-//                      B2 | stage k, P^T, do, gates of chunk c-1; prefetch k, P^T, do, g
+//                      B2 | stage k, P^T, do, decay table of chunk c-1; prefetch them
 //   consumers, chunk c: dS' -> LDS | B1 | k dS', P^T do, dv_new -> LDS | B2 | dS update
 // ------------------------------------------------------------------------- //
 template <typename T, int K, int V, int BV>
@@ -321,11 +319,9 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
     // ring A = what phase 2 of the chunk's own step reads (q, w), ring B = what phase 1 reads
     // (k, P^T, do, gates), staged during phase 2 of the step before
     struct PreA { typename IOK::Regs rq, rw; int len; };
-    struct PreB { typename IOK::Regs rk; typename IOP::Regs rp; typename IOV::Regs rd; uint32_t graw; int len; };
+    struct PreB { typename IOK::Regs rk; typename IOP::Regs rp; typename IOV::Regs rd; float eb, ed; int len; };
     PreA pa[LPF];
     PreB pb[LPF];
-    const bool gated = a.gate != LMOE_GATE_NONE && a.g.ptr != nullptr;
-    const void* gptr = gated ? a.g.ptr : a.k.ptr;
     const float scale = a.scale;
     // always issued, chunk index clamped (see k_gdn_state_fwd); `it` counts chunks from the end
     auto issue_a = [&](PreA& P, int it) {
@@ -342,7 +338,9 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
       IOK::load_nomask(P.rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, P.len);
       IOP::load_nomask(P.rp, (const T*)a.pmat + (((int64_t)(sq.chunk0 + c) * a.H + h) * 2 + 1) * CH * CH, CH, CH);
       IOV::load_nomask(P.rd, row_ptr<T>(a.d_o, sq.b, tok, h) + v0, a.d_o.st, P.len);
-      P.graw = load_scalar_raw(gptr, a.g_dtype, gated ? row_off(a.g, sq.b, tok + min(l, P.len - 1), h) : 0);
+      const float* gc = a.gcum + ((int64_t)(sq.chunk0 + c) * a.H + h) * 2 * CH;
+      P.eb = gc[l];
+      P.ed = gc[CH + l];
     };
     auto stage_a = [&](PreA& P) {
       IOK::mask(P.rq, P.len);
@@ -357,11 +355,9 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
       IOP::store_lds(P.rp, s_pt, LDC);      // rows and columns past the end are zero as written
       IOV::store_lds(P.rd, s_do, LDU);
       if (wave_id() == 4) {
-        const float x = wave_incl_scan((gated && l < P.len) ? scalar_from_raw(P.graw, a.g_dtype) : 0.f);
-        const float xl = __shfl(x, 63, 64);
-        s_qs[buf][l] = scale * expf(x);
-        s_ed[buf][l] = expf(xl - x);
-        if (l == 0) s_dec[buf] = expf(xl);
+        s_qs[buf][l] = scale * P.eb;
+        s_ed[buf][l] = P.ed;
+        if (l == 63) s_dec[buf] = P.eb;
       }
     };
     auto store_results = [&](int c) {

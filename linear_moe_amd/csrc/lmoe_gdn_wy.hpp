@@ -4,7 +4,8 @@
 //   w = Tinv (k . beta e^{b}),   u = Tinv (v . beta)
 // and the intra-chunk attention matrix the two sequential passes consume,
 //   P = (q k^T) . Gamma  (lower triangle incl. the diagonal), stored as P and as P^T.
-// grid = (NT, H), block = 256.  Writes w, u, Tinv and P, P^T (element type T).
+// grid = (NT, H), block = 256.  Writes w, u, Tinv and P, P^T (element type T) and the chunk's
+// decay table e^{b}, e^{b_C - b} (fp32).
 #pragma once
 #include "lmoe_seq.hpp"
 
@@ -90,7 +91,13 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
     s_beta[j] = j < ci.len ? load_scalar(a.beta.ptr, a.beta_dtype, row_off(a.beta, ci.b, ci.tok + j, h)) : 0.f;
   }
   chunk_gate_cumsum(a, ci.b, ci.tok, ci.len, h, s_b, s_eb, nullptr);    // barrier inside
-  if (threadIdx.x < 64) s_beb[threadIdx.x] = s_beta[threadIdx.x] * s_eb[threadIdx.x];
+  if (threadIdx.x < 64) {
+    s_beb[threadIdx.x] = s_beta[threadIdx.x] * s_eb[threadIdx.x];
+    // decay table of the chunk for the sequential passes: e^{b_j}, e^{b_C - b_j}
+    float* gc = a.gcum + ((int64_t)cid * a.H + h) * 2 * CH;
+    gc[threadIdx.x] = s_eb[threadIdx.x];
+    gc[CH + threadIdx.x] = expf(s_b[CH - 1] - s_b[threadIdx.x]);
+  }
   IOK::store_lds(rk, s_k, LDK);
   IOV::store_lds_scaled(rv, s_vb, LDV, s_beta);
   __syncthreads();
