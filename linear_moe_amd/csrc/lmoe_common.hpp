@@ -406,6 +406,23 @@ template <typename T, int ROWS, int COLS> struct TileIO {
       }
     }
   }
+  // registers <- tile[row][col]  /  global[row][col] <- registers (rows < nvalid): the two halves of
+  // lds_to_global for callers that must leave the tile before the stores are issued
+  static __device__ __forceinline__ void load_lds(Regs& r, const T* tile, int ld) {
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      int row, col; coords(p, row, col);
+      row = row < ROWS ? row : ROWS - 1;
+      r.v[p] = *(const vec*)(tile + row * ld + col);
+    }
+  }
+  static __device__ __forceinline__ void store_global(const Regs& r, T* __restrict__ dst, int64_t row_stride, int nvalid) {
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      int row, col; coords(p, row, col);
+      if (row < ROWS && row < nvalid) *(vec*)(dst + (int64_t)row * row_stride + col) = r.v[p];
+    }
+  }
   // global[row][col] = tile[row][col]
   static __device__ __forceinline__ void lds_to_global(const T* tile, int ld, T* __restrict__ dst, int64_t row_stride, int nvalid) {
 #pragma unroll

@@ -6,16 +6,19 @@
 //   with P = (q k^T) . Gamma (written by k_gdn_wy_fwd as P and P^T), e_b = e^{b}, e_d = e^{b_C - b}.
 //
 // Both kernels keep the per-chunk work of the dependency chain as small as it can be made:
-//   * work-group = 2 teams of 4 waves that meet at two barriers per chunk (B1, B2).
+//   * work-group = 3 teams of 4 waves that meet at two barriers per chunk (B1, B2).
 //     Team 0 (consumers) owns the state slice [K x BV] in fp32 MFMA accumulators (wave w: rows
 //     [w K/4, (w+1) K/4)) and, for the products whose rows are tokens, rows 16 w .. 16 w + 15 of
 //     the chunk.  It touches LDS and the matrix cores only: a wave that issues global loads or
 //     stores stalls at the issue whenever the vector memory pipe of the CU is busy, and on this
 //     wave every such stall lengthens the chain.
-//     Team 1 (loaders) owns all global traffic: it keeps the operand tiles of the next chunks in
-//     flight in registers (whole 128-byte lines per row), stages them into single LDS buffers in
-//     the half-step before they are needed, and writes the state checkpoints (hs / dhs, layout
-//     [V][K]) and the chunk's results from LDS.
+//     Teams 1 and 2 (loaders) own all global traffic: they keep the operand tiles of the next
+//     chunks in flight in registers (whole 128-byte lines per row) and stage them into single
+//     LDS buffers in the half-step before they are needed.  Team 1 has the tiles phase 2 reads
+//     and writes the state checkpoints (hs / dhs, layout [V][K]) and the chunk's results, which
+//     it lifts out of LDS during phase 1 and stores during phase 2; team 2 has the tiles phase 1
+//     reads: it stages during phase 2 and issues its loads during phase 1, so that in both
+//     half-steps one team fills LDS while the other waits on the memory pipe.
 //   * the intra-chunk matrix P is not formed here: the chunk-parallel WY preparation writes it
 //     once per (chunk, head) instead of once per V-slice.
 //   * grid = ceil(N*H / 8) * 8 * (V / BV) work-groups (1-D): the V-slices of one (sequence, head)
@@ -50,12 +53,13 @@ template <int L, typename F> __device__ __forceinline__ void ring_loop(int n, F&
 
 // ------------------------------------------------------------------------- //
 // forward
-//   loaders, chunk c:  B1 | stage k(c), P(c); store hs(c), o(c-1), v_new(c-1); prefetch k, P |
-//                      B2 | stage w, q, u, decay table of chunk c+1; prefetch them
+//   team 1, chunk c:   B1 | stage k(c), P(c); lift S^T(c), o(c-1), v_new(c-1) out of LDS |
+//                      B2 | store hs(c), o(c-1), v_new(c-1); prefetch k, P
+//   team 2, chunk c:   B1 | prefetch w, q, u, decay table | B2 | stage those of chunk c+1
 //   consumers, chunk c: S -> LDS | B1 | w S, q S, v_new -> LDS | B2 | S update, P v_new, o -> LDS
 // ------------------------------------------------------------------------- //
 template <typename T, int K, int V, int BV>
-__global__ __launch_bounds__(2 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
+__global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
   constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDU = BV + LPAD;
   constexpr int MB = K / 64, NB = BV / 16, KS = K / 32;
   constexpr int LPF = GdnStateCfg<T>::LPF;
@@ -96,13 +100,9 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
   typedef TileIO<T, BV, K> IOHT;
 
   if (team == 1) {
-    // --------------------------------- loaders -------------------------------------------
-    // two rings of register sets: A = what phase 2 of the chunk's own step reads (k, P),
-    // B = what phase 1 reads (w, q, u, gates), staged during phase 2 of the step before
+    // ------------------------- loaders, ring A (k, P) and all stores ----------------------
     struct PreA { typename IOK::Regs rk; typename IOP::Regs rp; int len; };
-    struct PreB { typename IOK::Regs rw, rq; typename IOV::Regs ru; float eb, ed; int len; };
     PreA pa[LPF];
-    PreB pb[LPF];
     // Always issued (chunk index clamped to the last chunk; the surplus loads at the end of a
     // sequence are never consumed): a prefetch that is skipped on some path would make the
     // compiler drain all outstanding loads at every consumer of a register set.
@@ -113,6 +113,50 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
       IOK::load_nomask(P.rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, P.len);
       IOP::load_nomask(P.rp, (const T*)a.pmat + ((int64_t)(sq.chunk0 + c) * a.H + h) * 2 * CH * CH, CH, CH);
     };
+    auto stage_a = [&](PreA& P) {
+      IOK::mask(P.rk, P.len);
+      IOK::store_lds(P.rk, s_k, LDK);
+      IOP::store_lds(P.rp, s_p, LDC);       // rows and columns past the end are zero as written
+    };
+    // o and v_new of chunk c: registers -> global
+    auto store_results = [&](const typename IOV::Regs& rvn, const typename IOV::Regs& ro, int c) {
+      const int tok = sq.tok0 + c * CH;
+      const int len = min(CH, sq.len - c * CH);
+      IOV::store_global(rvn, row_ptr<T>(a.vnew, sq.b, tok, h) + v0, a.vnew.st, len);
+      IOV::store_global(ro, row_ptr<T>(a.o, sq.b, tok, h) + v0, a.o.st, len);
+    };
+#pragma unroll
+    for (int j = 0; j < LPF; ++j) issue_a(pa[j], j);
+    // the first loads may be ordered freely by the compiler; were they still pending at the loop
+    // header, its wait-count analysis would carry that order into every iteration
+    wait_all_loads();
+    typename IOHT::Regs rh;
+    typename IOV::Regs rvn, ro;
+    ring_loop<LPF>(sq.nchunks, [&](auto slot, const int c) {
+      constexpr int j = decltype(slot)::value;
+      lds_barrier();                                                                     // B1
+      stage_a(pa[j]);
+      // S^T and the previous chunk's results leave LDS now (the consumers rewrite them after B2)
+      IOHT::load_lds(rh, s_hT, LDK);
+      IOV::load_lds(rvn, s_vn, LDU);
+      IOV::load_lds(ro, s_o, LDU);
+      lds_barrier();                                                                     // B2
+      // hs[chunk][h][v0 .. v0+BV][K] <- S^T
+      IOHT::store_global(rh, (T*)a.hs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
+      if (c > 0) store_results(rvn, ro, c - 1);
+      issue_a(pa[j], c + LPF);
+    });
+    lds_barrier();                                                                       // results of the last chunk
+    IOV::load_lds(rvn, s_vn, LDU);
+    IOV::load_lds(ro, s_o, LDU);
+    store_results(rvn, ro, sq.nchunks - 1);
+    return;
+  }
+  if (team == 2) {
+    // ------------------------- loaders, ring B (w, q, u, decay table) ---------------------
+    // staged during phase 2 of the step before the one that reads them in phase 1
+    struct PreB { typename IOK::Regs rw, rq; typename IOV::Regs ru; float eb, ed; int len; };
+    PreB pb[LPF];
     auto issue_b = [&](PreB& P, int c) {
       c = min(c, sq.nchunks - 1);
       const int tok = sq.tok0 + c * CH;
@@ -124,51 +168,30 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
       P.eb = gc[l];
       P.ed = gc[CH + l];
     };
-    auto stage_a = [&](PreA& P) {
-      IOK::mask(P.rk, P.len);
-      IOK::store_lds(P.rk, s_k, LDK);
-      IOP::store_lds(P.rp, s_p, LDC);       // rows and columns past the end are zero as written
-    };
     auto stage_b = [&](PreB& P, int buf) {
       IOK::mask(P.rw, P.len);
       IOV::mask(P.ru, P.len);
       IOK::store_lds(P.rw, s_w, LDK);
       IOK::store_lds(P.rq, s_q, LDK);       // rows past the end only reach output rows that are not stored
       IOV::store_lds(P.ru, s_u, LDU);
-      if (wave_id() == 4) {
+      if (wave_id() == 8) {
         s_eb[buf][l] = P.eb;
         s_ed[buf][l] = P.ed;
         if (l == 63) s_dec[buf] = P.eb;
       }
     };
-    // o and v_new of chunk c: LDS -> global
-    auto store_results = [&](int c) {
-      const int tok = sq.tok0 + c * CH;
-      const int len = min(CH, sq.len - c * CH);
-      IOV::lds_to_global(s_vn, LDU, row_ptr<T>(a.vnew, sq.b, tok, h) + v0, a.vnew.st, len);
-      IOV::lds_to_global(s_o, LDU, row_ptr<T>(a.o, sq.b, tok, h) + v0, a.o.st, len);
-    };
 #pragma unroll
-    for (int j = 0; j < LPF; ++j) { issue_b(pb[j], j); issue_a(pa[j], j); }
+    for (int j = 0; j < LPF; ++j) issue_b(pb[j], j);
     stage_b(pb[0], 0);
-    issue_b(pb[0], LPF);
-    // the first loads may be ordered freely by the compiler; were they still pending at the loop
-    // header, its wait-count analysis would carry that order into every iteration
-    wait_all_loads();
+    wait_all_loads();   // see ring A
     ring_loop<LPF>(sq.nchunks, [&](auto slot, const int c) {
       constexpr int j = decltype(slot)::value, jn = (j + 1) % LPF;
       lds_barrier();                                                                     // B1
-      stage_a(pa[j]);
-      // hs[chunk][h][v0 .. v0+BV][K] <- S^T
-      IOHT::lds_to_global(s_hT, LDK, (T*)a.hs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
-      if (c > 0) store_results(c - 1);
-      issue_a(pa[j], c + LPF);
+      issue_b(pb[j], c + LPF);              // chunk c was staged before this barrier: refill its set
       lds_barrier();                                                                     // B2
       if (c + 1 < sq.nchunks) stage_b(pb[jn], (c + 1) & 1);
-      issue_b(pb[jn], c + 1 + LPF);
     });
-    lds_barrier();                                                                       // results of the last chunk
-    store_results(sq.nchunks - 1);
+    lds_barrier();
     return;
   }
 
@@ -271,12 +294,13 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
 
 // ------------------------------------------------------------------------- //
 // backward (reverse order over the chunks; it = 0 is the last chunk)
-//   loaders, chunk c:  B1 | stage q(c), w(c); store dhs(c), dv_new(c+1); prefetch q, w |
-//                      B2 | stage k, P^T, do, decay table of chunk c-1; prefetch them
+//   team 1, chunk c:   B1 | stage q(c), w(c); lift dS'^T(c), dv_new(c+1) out of LDS |
+//                      B2 | store dhs(c), dv_new(c+1); prefetch q, w
+//   team 2, chunk c:   B1 | prefetch k, P^T, do, decay table | B2 | stage those of chunk c-1
 //   consumers, chunk c: dS' -> LDS | B1 | k dS', P^T do, dv_new -> LDS | B2 | dS update
 // ------------------------------------------------------------------------- //
 template <typename T, int K, int V, int BV>
-__global__ __launch_bounds__(2 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
+__global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
   constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDU = BV + LPAD;
   constexpr int MB = K / 64, NB = BV / 16, KS = K / 32;
   constexpr int LPF = GdnStateCfg<T>::LPF;
@@ -315,14 +339,9 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
   typedef TileIO<T, BV, K> IOHT;
 
   if (team == 1) {
-    // --------------------------------- loaders -------------------------------------------
-    // ring A = what phase 2 of the chunk's own step reads (q, w), ring B = what phase 1 reads
-    // (k, P^T, do, gates), staged during phase 2 of the step before
+    // ------------------------- loaders, ring A (q, w) and all stores ----------------------
     struct PreA { typename IOK::Regs rq, rw; int len; };
-    struct PreB { typename IOK::Regs rk; typename IOP::Regs rp; typename IOV::Regs rd; float eb, ed; int len; };
     PreA pa[LPF];
-    PreB pb[LPF];
-    const float scale = a.scale;
     // always issued, chunk index clamped (see k_gdn_state_fwd); `it` counts chunks from the end
     auto issue_a = [&](PreA& P, int it) {
       const int c = max(sq.nchunks - 1 - it, 0);
@@ -331,6 +350,46 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
       IOK::load_nomask(P.rq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, P.len);
       IOK::load_nomask(P.rw, row_ptr<T>(a.w, sq.b, tok, h), a.w.st, P.len);
     };
+    auto stage_a = [&](PreA& P) {
+      IOK::mask(P.rq, P.len);
+      IOK::mask(P.rw, P.len);
+      IOK::store_lds(P.rq, s_q, LDK);
+      IOK::store_lds(P.rw, s_w, LDK);
+    };
+    auto store_results = [&](const typename IOV::Regs& rdv, int c) {
+      const int tok = sq.tok0 + c * CH;
+      const int len = min(CH, sq.len - c * CH);
+      IOV::store_global(rdv, row_ptr<T>(a.dvnew, sq.b, tok, h) + v0, a.dvnew.st, len);
+    };
+#pragma unroll
+    for (int j = 0; j < LPF; ++j) issue_a(pa[j], j);
+    wait_all_loads();   // see k_gdn_state_fwd
+    typename IOHT::Regs rh;
+    typename IOV::Regs rdv;
+    ring_loop<LPF>(sq.nchunks, [&](auto slot, const int it) {
+      constexpr int j = decltype(slot)::value;
+      const int c = sq.nchunks - 1 - it;
+      lds_barrier();                                                                     // B1
+      stage_a(pa[j]);
+      // dS'^T and the previous chunk's dv_new leave LDS now (the consumers rewrite them after B2)
+      IOHT::load_lds(rh, s_dST, LDK);
+      IOV::load_lds(rdv, s_dvn, LDU);
+      lds_barrier();                                                                     // B2
+      IOHT::store_global(rh, (T*)a.dhs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
+      if (it > 0) store_results(rdv, c + 1);
+      issue_a(pa[j], it + LPF);
+    });
+    lds_barrier();                                                                       // dv_new of chunk 0
+    IOV::load_lds(rdv, s_dvn, LDU);
+    store_results(rdv, 0);
+    return;
+  }
+  if (team == 2) {
+    // ------------------------- loaders, ring B (k, P^T, do, decay table) ------------------
+    // staged during phase 2 of the step before the one that reads them in phase 1
+    struct PreB { typename IOK::Regs rk; typename IOP::Regs rp; typename IOV::Regs rd; float eb, ed; int len; };
+    PreB pb[LPF];
+    const float scale = a.scale;
     auto issue_b = [&](PreB& P, int it) {
       const int c = max(sq.nchunks - 1 - it, 0);
       const int tok = sq.tok0 + c * CH;
@@ -342,48 +401,30 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
       P.eb = gc[l];
       P.ed = gc[CH + l];
     };
-    auto stage_a = [&](PreA& P) {
-      IOK::mask(P.rq, P.len);
-      IOK::mask(P.rw, P.len);
-      IOK::store_lds(P.rq, s_q, LDK);
-      IOK::store_lds(P.rw, s_w, LDK);
-    };
     auto stage_b = [&](PreB& P, int buf) {
       IOK::mask(P.rk, P.len);
       IOV::mask(P.rd, P.len);
       IOK::store_lds(P.rk, s_k, LDK);
       IOP::store_lds(P.rp, s_pt, LDC);      // rows and columns past the end are zero as written
       IOV::store_lds(P.rd, s_do, LDU);
-      if (wave_id() == 4) {
+      if (wave_id() == 8) {
         s_qs[buf][l] = scale * P.eb;
         s_ed[buf][l] = P.ed;
         if (l == 63) s_dec[buf] = P.eb;
       }
     };
-    auto store_results = [&](int c) {
-      const int tok = sq.tok0 + c * CH;
-      const int len = min(CH, sq.len - c * CH);
-      IOV::lds_to_global(s_dvn, LDU, row_ptr<T>(a.dvnew, sq.b, tok, h) + v0, a.dvnew.st, len);
-    };
 #pragma unroll
-    for (int j = 0; j < LPF; ++j) { issue_b(pb[j], j); issue_a(pa[j], j); }
+    for (int j = 0; j < LPF; ++j) issue_b(pb[j], j);
     stage_b(pb[0], 0);
-    issue_b(pb[0], LPF);
-    wait_all_loads();   // see k_gdn_state_fwd
+    wait_all_loads();
     ring_loop<LPF>(sq.nchunks, [&](auto slot, const int it) {
       constexpr int j = decltype(slot)::value, jn = (j + 1) % LPF;
-      const int c = sq.nchunks - 1 - it;
       lds_barrier();                                                                     // B1
-      stage_a(pa[j]);
-      IOHT::lds_to_global(s_dST, LDK, (T*)a.dhs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
-      if (it > 0) store_results(c + 1);
-      issue_a(pa[j], it + LPF);
+      issue_b(pb[j], it + LPF);             // this chunk was staged before the barrier: refill its set
       lds_barrier();                                                                     // B2
-      if (c > 0) stage_b(pb[jn], (it + 1) & 1);
-      issue_b(pb[jn], it + 1 + LPF);
+      if (it + 1 < sq.nchunks) stage_b(pb[jn], (it + 1) & 1);
     });
-    lds_barrier();                                                                       // dv_new of chunk 0
-    store_results(0);
+    lds_barrier();
     return;
   }
 
