@@ -75,8 +75,8 @@ typedef struct lmoe_args {
   lmoe_tensor u;       /* [B,T,H,V]   WY factor u (gated delta rule; forward only)     */
   void* tinv;          /* [NT,H,64,64] (I + L)^-1 per chunk (gated delta rule)         */
   void* amat;          /* [NT,H,64,64] intra-chunk attention matrix (chunk_gla)        */
-  void* pmat;          /* [NT,H,2,64,64] P = (q k^T) . Gamma and its transpose per chunk
-                          (gated delta rule; written by the WY preparation)             */
+  void* pmat;          /* [NT,H,64,64] P = (q k^T) . Gamma per chunk (gated delta rule;
+                          written by the WY preparation)                                */
   float* gcum;         /* [NT,H,2,64] fp32 e^{b_j} and e^{b_C - b_j}, b = cumulative log-decay
                           inside the chunk (gated delta rule; written by the WY preparation) */
   /* backward inputs */

@@ -57,7 +57,7 @@ int64_t lmoe_workspace_bytes(int32_t op, int32_t dtype, int32_t part, int32_t B,
   const int64_t rows_k = (int64_t)B * T * H * K, rows_v = (int64_t)B * T * H * V;
   int64_t n = states;                                                    // hs | dhs
   if (op == LMOE_OP_GLA && part == 0) n += tiles;                        // amat
-  if (op == LMOE_OP_GATED_DELTA_RULE) n += part == 0 ? 2 * rows_v + rows_k + 3 * tiles   // vnew, u, w, tinv, pmat
+  if (op == LMOE_OP_GATED_DELTA_RULE) n += part == 0 ? 2 * rows_v + rows_k + 2 * tiles   // vnew, u, w, tinv, pmat
                                                      : rows_v + rows_k;              // dvnew, dw
   int64_t bytes = n * s;
   if (op == LMOE_OP_GATED_DELTA_RULE && part == 0) bytes += (int64_t)NT * H * 2 * LMOE_CHUNK * 4;   // gcum (fp32)

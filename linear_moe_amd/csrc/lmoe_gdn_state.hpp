@@ -3,7 +3,7 @@
 //   forward :  v_new = u - w S,   o = scale [ e^{b_i} q_i S + P v_new ],   S' = e^{b_C} S + k^T (e_d v_new)
 //   backward:  dv_new = scale P^T do + e_d (k dS'),
 //              dS = e^{b_C} dS' + q^T (scale e_b do) - w^T dv_new
-//   with P = (q k^T) . Gamma (written by k_gdn_wy_fwd as P and P^T), e_b = e^{b}, e_d = e^{b_C - b}.
+//   with P = (q k^T) . Gamma (written by k_gdn_wy_fwd), e_b = e^{b}, e_d = e^{b_C - b}.
 //
 // Both kernels keep the per-chunk work of the dependency chain as small as it can be made:
 //   * work-group = 3 teams of 4 waves that meet at two barriers per chunk (B1, B2).
@@ -111,7 +111,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
       const int tok = sq.tok0 + c * CH;
       P.len = min(CH, sq.len - c * CH);
       IOK::load_nomask(P.rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, P.len);
-      IOP::load_nomask(P.rp, (const T*)a.pmat + ((int64_t)(sq.chunk0 + c) * a.H + h) * 2 * CH * CH, CH, CH);
+      IOP::load_nomask(P.rp, (const T*)a.pmat + ((int64_t)(sq.chunk0 + c) * a.H + h) * CH * CH, CH, CH);
     };
     auto stage_a = [&](PreA& P) {
       IOK::mask(P.rk, P.len);
@@ -296,7 +296,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
 // backward (reverse order over the chunks; it = 0 is the last chunk)
 //   team 1, chunk c:   B1 | stage q(c), w(c); lift dS'^T(c), dv_new(c+1) out of LDS |
 //                      B2 | store dhs(c), dv_new(c+1); prefetch q, w
-//   team 2, chunk c:   B1 | prefetch k, P^T, do, decay table | B2 | stage those of chunk c-1
+//   team 2, chunk c:   B1 | prefetch k, P, do, decay table | B2 | stage those of chunk c-1
 //   consumers, chunk c: dS' -> LDS | B1 | k dS', P^T do, dv_new -> LDS | B2 | dS update
 // ------------------------------------------------------------------------- //
 template <typename T, int K, int V, int BV>
@@ -307,7 +307,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
   __shared__ __attribute__((aligned(16))) T s_q[CH * LDK];          // q         [64][K]
   __shared__ __attribute__((aligned(16))) T s_w[CH * LDK];          // w         [64][K]
   __shared__ __attribute__((aligned(16))) T s_k[CH * LDK];          // k         [64][K]
-  __shared__ __attribute__((aligned(16))) T s_pt[CH * LDC];         // P^T       [64][64]
+  __shared__ __attribute__((aligned(16))) T s_p[CH * LDC];          // P         [64][64]
   __shared__ __attribute__((aligned(16))) T s_do[CH * LDU];         // do        [64][BV]
   __shared__ __attribute__((aligned(16))) T s_dST[BV * LDK];        // dS'^T     [BV][K]
   __shared__ __attribute__((aligned(16))) T s_dvT[BV * LDC];        // -dv_new^T [BV][64]
@@ -385,7 +385,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
     return;
   }
   if (team == 2) {
-    // ------------------------- loaders, ring B (k, P^T, do, decay table) ------------------
+    // ------------------------- loaders, ring B (k, P, do, decay table) ------------------
     // staged during phase 2 of the step before the one that reads them in phase 1
     struct PreB { typename IOK::Regs rk; typename IOP::Regs rp; typename IOV::Regs rd; float eb, ed; int len; };
     PreB pb[LPF];
@@ -395,7 +395,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
       const int tok = sq.tok0 + c * CH;
       P.len = min(CH, sq.len - c * CH);
       IOK::load_nomask(P.rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, P.len);
-      IOP::load_nomask(P.rp, (const T*)a.pmat + (((int64_t)(sq.chunk0 + c) * a.H + h) * 2 + 1) * CH * CH, CH, CH);
+      IOP::load_nomask(P.rp, (const T*)a.pmat + ((int64_t)(sq.chunk0 + c) * a.H + h) * CH * CH, CH, CH);
       IOV::load_nomask(P.rd, row_ptr<T>(a.d_o, sq.b, tok, h) + v0, a.d_o.st, P.len);
       const float* gc = a.gcum + ((int64_t)(sq.chunk0 + c) * a.H + h) * 2 * CH;
       P.eb = gc[l];
@@ -405,7 +405,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
       IOK::mask(P.rk, P.len);
       IOV::mask(P.rd, P.len);
       IOK::store_lds(P.rk, s_k, LDK);
-      IOP::store_lds(P.rp, s_pt, LDC);      // rows and columns past the end are zero as written
+      IOP::store_lds(P.rp, s_p, LDC);       // rows and columns past the end are zero as written
       IOV::store_lds(P.rd, s_do, LDU);
       if (wave_id() == 8) {
         s_qs[buf][l] = scale * P.eb;
@@ -466,7 +466,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
     typename ET<T>::frag bdo[CH / 32][NB];
 #pragma unroll
     for (int ks = 0; ks < CH / 32; ++ks) {
-      const typename ET<T>::frag ap = ET<T>::load_frag(s_pt + (16 * wv + fr) * LDC + 32 * ks + fg);
+      // rows 16 wv .. of P^T: P is stored as written, the contraction runs along its rows
+      const typename ET<T>::frag ap = ET<T>::load_frag_t(s_p, LDC, 32 * ks, 16 * wv);
 #pragma unroll
       for (int ni = 0; ni < NB; ++ni) {
         bdo[ks][ni] = ET<T>::load_frag_t(s_do, LDU, 32 * ks, 16 * ni);

@@ -3,8 +3,8 @@
 //   Tinv = (I + L)^-1            (unit lower triangular, fp32)
 //   w = Tinv (k . beta e^{b}),   u = Tinv (v . beta)
 // and the intra-chunk attention matrix the two sequential passes consume,
-//   P = (q k^T) . Gamma  (lower triangle incl. the diagonal), stored as P and as P^T.
-// grid = (NT, H), block = 256.  Writes w, u, Tinv and P, P^T (element type T) and the chunk's
+//   P = (q k^T) . Gamma  (lower triangle incl. the diagonal).
+// grid = (NT, H), block = 256.  Writes w, u, Tinv and P (element type T) and the chunk's
 // decay table e^{b}, e^{b_C - b} (fp32).
 #pragma once
 #include "lmoe_seq.hpp"
@@ -117,9 +117,9 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
     }
   }
   {
-    // P = (q k^T) . Gamma -> global as P and P^T, staged through the (still unused) X tile
+    // P = (q k^T) . Gamma -> global, staged through the (still unused) X tile
     T* s_P = (T*)s_X;
-    T* pg = (T*)a.pmat + ((int64_t)cid * a.H + h) * 2 * CH * CH;
+    T* pg = (T*)a.pmat + ((int64_t)cid * a.H + h) * CH * CH;
     f32x4 pm[1][4];
     acc_zero(pm);
     fq.mask(16 * wv, ci.len);
@@ -136,20 +136,9 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
         pm[0][nj][i] = (r >= cc) ? pm[0][nj][i] * texp<T>(s_b[r] - s_b[cc]) : 0.f;
       }
       acc_to_lds<T>(pm[0][nj], s_P, LDC, 16 * wv, 16 * nj);
-      if constexpr (sizeof(T) == 2) acc_to_lds_t<T>(pm[0][nj], s_P + CH * LDC, LDC, 16 * wv, 16 * nj);
     }
     __syncthreads();
     IO64::lds_to_global(s_P, LDC, pg, CH, CH);
-    if constexpr (sizeof(T) == 2) {
-      IO64::lds_to_global(s_P + CH * LDC, LDC, pg + CH * CH, CH, CH);
-    } else {
-      // an fp32 tile fills the X tile: the transpose takes a second round
-      __syncthreads();
-#pragma unroll
-      for (int nj = 0; nj < 4; ++nj) acc_to_lds_t<T>(pm[0][nj], s_P, LDC, 16 * wv, 16 * nj);
-      __syncthreads();
-      IO64::lds_to_global(s_P, LDC, pg + CH * CH, CH, CH);
-    }
   }
   // k is dead as an operand of k k^T and q k^T: scale it in place to k beta e^{b} (from the registers)
   IOK::store_lds_scaled(rk, s_k, LDK, s_beb);

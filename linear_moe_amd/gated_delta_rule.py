@@ -62,7 +62,7 @@ class GDNCall:
         ht = torch.empty(plan.N, H, K, V, dtype=torch.float32, device=dev) if output_final_state else None
         hs = torch.empty(max(plan.NT, 1), H, K, V, dtype=dt, device=dev)
         tinv = torch.empty(max(plan.NT, 1), H, 64, 64, dtype=dt, device=dev)
-        pmat = torch.empty(max(plan.NT, 1), H, 2, 64, 64, dtype=dt, device=dev)
+        pmat = torch.empty(max(plan.NT, 1), H, 64, 64, dtype=dt, device=dev)
         gcum = torch.empty(max(plan.NT, 1), H, 2, 64, dtype=torch.float32, device=dev)
         w = torch.empty(B, T, H, K, dtype=dt, device=dev)
         u = torch.empty(B, T, H, V, dtype=dt, device=dev)
