@@ -27,15 +27,15 @@ PEAK_MFMA_BF16 = 2.5e15   # dense bf16 MFMA, FLOP/s (MI355X published)
 PEAK_HBM = 8.0e12         # B/s
 CH = 64
 
-STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_state_fwd", 4: "k_state_bwd", 5: "k_bwd_dqk", 6: "k_gdn_wy_bwd"}
+STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_gdn_state_fwd", 4: "k_gdn_state_bwd", 5: "k_bwd_dqk", 6: "k_gdn_wy_bwd"}
 
 # HBM bytes per launch on this workload, from two rocprofv3 --pmc runs of this file (FETCH_SIZE, then
 # WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for the 256 MiB device
 # copy that main() issues first (FETCH_SIZE reads half of the bytes fetched, WRITE_SIZE all of the
 # bytes written).  Summary and commands: profiles/gdn_fwd_bwd_cfg4_hbm_traffic.md.
 CALIB_COPY_BYTES = 256 << 20
-MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 649013210, "k_state_fwd": 1091391848, "k_state_bwd": 956576801,
-                    "k_bwd_dqk": 1646585149, "k_gdn_wy_bwd": 1121118387}
+MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 857625238, "k_gdn_state_fwd": 1145233912, "k_gdn_state_bwd": 1011003237,
+                    "k_bwd_dqk": 1646770043, "k_gdn_wy_bwd": 1118582430}
 
 
 def gdn_inputs(B, T, H, K, V, seed, dtype, device):
@@ -62,12 +62,12 @@ def stage_model(stage, K, V, s=2):
     full 64-token tiles, multiply-add = 2 flops; every input read once, every output written once."""
     c = CH
     kv, ck, cv, cc = K * V, c * K, c * V, c * c
-    if stage == 0:   # k k^T, triangular inverse, w, u | r k,v  w w,u,Tinv
-        return 4 * cc * K + 2 * cc * V + (2 / 3) * c ** 3, 2 * (ck + cv) * s + cc * s + c * (4 + s)
-    if stage == 1:   # w S, k^T v_new, q k^T, q S, P v_new | r q,k,w,u  w v_new,hs,o
-        return 6 * c * kv + 2 * cc * K + 2 * cc * V, (3 * ck + cv) * s + (2 * cv + kv) * s + 4 * c
-    if stage == 4:   # k dS', q^T do, w^T dv_new, q k^T, P^T do | r q,k,w,do  w dv_new,dhs
-        return 6 * c * kv + 2 * cc * K + 2 * cc * V, (3 * ck + cv) * s + (cv + kv) * s + 4 * c
+    if stage == 0:   # k k^T, q k^T, triangular inverse, w, u | r q,k,v  w w,u,Tinv,P,decay table
+        return 6 * cc * K + 2 * cc * V + (2 / 3) * c ** 3, (2 * ck + cv) * s + (ck + cv) * s + 2 * cc * s + c * (8 + 4 + s)
+    if stage == 1:   # w S, q S, k^T v_new, P v_new | r q,k,w,u,P,table  w v_new,hs,o
+        return 6 * c * kv + 2 * cc * V, (3 * ck + cv + cc) * s + (2 * cv + kv) * s + 8 * c
+    if stage == 4:   # k dS', P^T do, q^T do, w^T dv_new | r q,k,w,do,P,table  w dv_new,dhs
+        return 6 * c * kv + 2 * cc * V, (3 * ck + cv + cc) * s + (cv + kv) * s + 8 * c
     if stage == 5:   # do v^T, do S^T, v dS'^T, dv_new S^T, dP k, dP^T q | r do,v_new,dv_new,hs,dhs,q,k  w dq,dk,dw
         return 2 * cc * V + 6 * c * kv + 4 * cc * K, (3 * cv + 2 * kv + 2 * ck) * s + 3 * ck * s + 8 * c
     if stage == 6:   # dT, Tinv^T du, Tinv^T dw, two 64^3 products, dM k, dM^T k_b | r du,dw,k,v,Tinv,dk  w dk,dv
