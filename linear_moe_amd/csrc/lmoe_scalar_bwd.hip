@@ -32,7 +32,7 @@ template <bool GDN> struct BwdDqk {
     static void run(const lmoe_args& a, hipStream_t st) {
       constexpr int BVH = BwdTiles<T, V>::BVH;
       const int grid = persistent_grid(a.NT * a.H, 1);
-      hipLaunchKernelGGL((k_bwd_dqk<T, K, V, BVH, GDN>), dim3(grid), dim3(NTHR), 0, st, a);
+      hipLaunchKernelGGL((k_bwd_dqk<T, K, V, BVH, GDN>), dim3(grid), dim3(2 * NTHR), 0, st, a);
     }
   };
 };

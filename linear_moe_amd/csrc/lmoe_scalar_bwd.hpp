@@ -356,99 +356,177 @@ __global__ __launch_bounds__((GDN ? 3 : 2) * NTHR) void k_state_bwd(const lmoe_a
 }
 
 // ------------------------------------------------------------------------- //
-// dq, dk, gate gradient        persistent: grid = min(NT*H, 2 per CU), one item = (chunk, head)
+// dq, dk, gate gradient        persistent: one work-group per CU, one item = (chunk, head)
 //   phase A: loop over V-slices of width BVH accumulating
 //              dP = do v'^T, dq_i = do S^T, dk_d = v' dS'^T (, dw = dv_new S^T)
 //            (hs, dhs hold S^T, dS'^T: [V][K]; the slice tiles are [BVH][K])
 //   phase B: dq = scale e_b dq_i + (scale dP . Gamma) k ; dk = e_d dk_d + (scale dP . Gamma)^T q
 //            with one LDS copy of (scale dP . Gamma)^T and q, k stored as loaded
-//   The loads of the next slice / of q, k / of the next item's first slice are in flight while
-//   the current step computes (barriers order LDS traffic only).
+//   Work-group = 2 teams of 4 waves on one barrier script.  Team 0 (compute) reads LDS and drives
+//   the matrix cores; wave w owns chunk rows 16 w .. 16 w + 15.  Team 1 (loaders) keeps the next
+//   slice and the next q, k in flight in registers and stages them into two alternating slice
+//   buffers, so a slice is being filled while the previous one is being consumed; the phase B
+//   tiles lie over the second buffer.  It also forms <S, dS'> from the registers it holds and the
+//   gate cumsum of the chunk.
+//   Script per item (NS slices):  R(0) .. R(NS-1) | D | A | b | c | E
+//     loaders : R(s): stage slice s+1 | D: stage q, k, gates | A: stage slice 0 of the next item
+//     compute : R(s): products of slice s | D, A | (dP . Gamma)^T -> LDS | b | products, combine |
+//               c | stores | E
 // ------------------------------------------------------------------------- //
 template <typename T, int K, int V, int BVH, bool GDN>
-__global__ __launch_bounds__(NTHR) void k_bwd_dqk(const lmoe_args a) {
+__global__ __launch_bounds__(2 * NTHR) void k_bwd_dqk(const lmoe_args a) {
   constexpr int LDV = BVH + LPAD, LDC = CH + LPAD, LDK = K + LPAD;
-  constexpr int NBK = K / 16;
-  // phase A tiles
+  constexpr int NBK = K / 16, NS = V / BVH;
+  // tiles of one V-slice
   constexpr int A_DO = 0, A_V = A_DO + CH * LDV, A_H = A_V + CH * LDV, A_DH = A_H + BVH * LDK,
                 A_DVN = A_DH + BVH * LDK, A_END = A_DVN + (GDN ? CH * LDV : 0);
-  // phase B tiles
+  // phase B tiles (relative to the second slice buffer)
   constexpr int B_DPT = 0, B_K = B_DPT + CH * LDC, B_Q = B_K + CH * LDK, B_END = B_Q + CH * LDK;
-  constexpr int NELEM = A_END > B_END ? A_END : B_END;
+  constexpr int BUF1 = A_END;
+  constexpr int NELEM = BUF1 + (A_END > B_END ? A_END : B_END);
+  static_assert(!GDN || 4 * 16 * LDK <= A_END, "the dw store strips fit the first slice buffer");
   __shared__ __attribute__((aligned(16))) T smem[NELEM];
   __shared__ float s_b[64], s_eb[64], s_ed[64], s_db[64], s_red[8];
 
-  const int wv = wave_id(), l = lane_id();
+  const int l = lane_id();
+  const int team = threadIdx.x / NTHR;
   typedef TileIO<T, CH, BVH> IOV;
   typedef TileIO<T, BVH, K> IOH;
   typedef TileIO<T, CH, K> IOK;
   const lmoe_tensor& vs = GDN ? a.vnew : a.v;
   const int nitems = a.NT * a.H;
+  const int stride = gridDim.x;
 
-  typename IOV::Regs rd, rv, rn;
-  typename IOH::Regs rh, rdh;
-  typename IOK::Regs rq, rk;
-  uint32_t graw = 0;
-  auto issueA = [&](int it, int vv) {
-    const int cid = it / a.H, h = it % a.H;
-    const ChunkInfo ci = chunk_info(a, cid);
-    IOV::load_nomask(rd, row_ptr<T>(a.d_o, ci.b, ci.tok, h) + vv, a.d_o.st, ci.len);
-    IOV::load_nomask(rv, row_ptr<T>(vs, ci.b, ci.tok, h) + vv, vs.st, ci.len);
-    IOH::load_nomask(rh, (const T*)a.hs + (((int64_t)cid * a.H + h) * V + vv) * K, K, BVH);
-    IOH::load_nomask(rdh, (const T*)a.dhs + (((int64_t)cid * a.H + h) * V + vv) * K, K, BVH);
-    if constexpr (GDN) IOV::load_nomask(rn, row_ptr<T>(a.dvnew, ci.b, ci.tok, h) + vv, a.dvnew.st, ci.len);
-  };
-  auto issueQK = [&](int it) {
-    const int cid = it / a.H, h = it % a.H;
-    const ChunkInfo ci = chunk_info(a, cid);
-    IOK::load_nomask(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
-    IOK::load_nomask(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
-    graw = gate_prefetch(a, ci.b, ci.tok, ci.len, h);
-  };
+  if (team == 1) {
+    // --------------------------------- loaders -------------------------------------------
+    struct SliceRegs { typename IOV::Regs rd, rv, rn; typename IOH::Regs rh, rdh; int len; };
+    struct QKRegs { typename IOK::Regs rq, rk; uint32_t graw; int len; };
+    SliceRegs S;
+    QKRegs Q;
+    // Every prefetch is issued unconditionally (item index clamped to the last item): a load that
+    // is skipped on some path would make the compiler drain all outstanding loads at every use.
+    auto issue_slice = [&](int it, int vv) {
+      it = min(it, nitems - 1);
+      const int cid = it / a.H, h = it % a.H;
+      const ChunkInfo ci = chunk_info(a, cid);
+      S.len = ci.len;
+      IOV::load_nomask(S.rd, row_ptr<T>(a.d_o, ci.b, ci.tok, h) + vv, a.d_o.st, ci.len);
+      IOV::load_nomask(S.rv, row_ptr<T>(vs, ci.b, ci.tok, h) + vv, vs.st, ci.len);
+      IOH::load_nomask(S.rh, (const T*)a.hs + (((int64_t)cid * a.H + h) * V + vv) * K, K, BVH);
+      IOH::load_nomask(S.rdh, (const T*)a.dhs + (((int64_t)cid * a.H + h) * V + vv) * K, K, BVH);
+      if constexpr (GDN) IOV::load_nomask(S.rn, row_ptr<T>(a.dvnew, ci.b, ci.tok, h) + vv, a.dvnew.st, ci.len);
+    };
+    auto issue_qk = [&](int it) {
+      it = min(it, nitems - 1);
+      const int cid = it / a.H, h = it % a.H;
+      const ChunkInfo ci = chunk_info(a, cid);
+      Q.len = ci.len;
+      IOK::load_nomask(Q.rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
+      IOK::load_nomask(Q.rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
+      Q.graw = gate_prefetch(a, ci.b, ci.tok, ci.len, h);
+    };
+    float hdh = 0.f;   // partial <S, dS'> of the item whose slices are being staged
+    auto stage_slice = [&](int buf) {
+      T* base = smem + buf * BUF1;
+#pragma unroll
+      for (int p = 0; p < IOH::PASSES; ++p)
+#pragma unroll
+        for (int i = 0; i < IOH::VEC; ++i) hdh += ET<T>::to_f(S.rh.v[p][i]) * ET<T>::to_f(S.rdh.v[p][i]);
+      IOV::mask(S.rd, S.len);
+      IOV::mask(S.rv, S.len);
+      IOV::store_lds(S.rd, base + A_DO, LDV);
+      IOV::store_lds(S.rv, base + A_V, LDV);
+      IOH::store_lds(S.rh, base + A_H, LDK);
+      IOH::store_lds(S.rdh, base + A_DH, LDK);
+      if constexpr (GDN) {
+        IOV::mask(S.rn, S.len);
+        IOV::store_lds(S.rn, base + A_DVN, LDV);
+      }
+    };
+    // the slice after slice s of item it
+    auto issue_next = [&](int it, int s) {
+      if (s + 1 < NS) issue_slice(it, (s + 1) * BVH); else issue_slice(it + stride, 0);
+    };
+    const int it0 = blockIdx.x;
+    issue_slice(it0, 0);
+    issue_qk(it0);
+    // the first loads may be ordered freely by the compiler; were they still pending at the loop
+    // header, its wait-count analysis would carry that order into every iteration
+    wait_all_loads();
+    stage_slice(0);
+    issue_next(it0, 0);
+    for (int it = it0; it < nitems; it += stride) {
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        lds_barrier();                                                                   // R(s)
+        if (s + 1 < NS) {
+          stage_slice((s + 1) & 1);        // its buffer was left when the compute team passed R(s)
+          issue_next(it, s + 1);
+        }
+      }
+      lds_barrier();                                                                     // D
+      gate_finish_wave(a, Q.graw, Q.len, l, wave_id() == 4, s_b, s_eb, s_ed);
+      IOK::mask(Q.rq, Q.len);
+      IOK::mask(Q.rk, Q.len);
+      IOK::store_lds(Q.rq, smem + BUF1 + B_Q, LDK);
+      IOK::store_lds(Q.rk, smem + BUF1 + B_K, LDK);
+      hdh = wave_sum(hdh);
+      if (l == 0) s_red[wave_id() - 4] = hdh;
+      hdh = 0.f;
+      lds_barrier();                                                                     // A
+      issue_qk(it + stride);
+      stage_slice(0);                      // slice 0 of the next item (buffer 0 is idle in phase B)
+      issue_next(it + stride, 0);
+      lds_barrier();                                                                     // b
+      lds_barrier();                                                                     // c
+      lds_barrier();                                                                     // E
+    }
+    return;
+  }
 
-  // prefetches are always issued (item index clamped): see k_state_fwd
-  int it = blockIdx.x;
-  if (it < nitems) issueA(it, 0);
-  for (; it < nitems; it += gridDim.x) {
+  // --------------------------------- compute ---------------------------------------------
+  const int wv = wave_id();
+  const int fr = l & 15, fg = 8 * (l >> 4);
+  for (int it = blockIdx.x; it < nitems; it += stride) {
     const int cid = it / a.H, h = it % a.H;
     const ChunkInfo ci = chunk_info(a, cid);
     f32x4 dP[1][4], dqi[1][NBK], dkd[1][NBK], dw[1][GDN ? NBK : 1];
     acc_zero(dP); acc_zero(dqi); acc_zero(dkd); acc_zero(dw);
-    float hdh = 0.f;   // partial <S, dS'>
-    for (int vv = 0; vv < V; vv += BVH) {
 #pragma unroll
-      for (int p = 0; p < IOH::PASSES; ++p)
+    for (int s = 0; s < NS; ++s) {
+      lds_barrier();                                                                     // R(s)
+      const T* base = smem + (s & 1) * BUF1;
+      const T* DO = base + A_DO; const T* VN = base + A_V; const T* DVN = base + A_DVN;
+      const T* HT = base + A_H; const T* DHT = base + A_DH;
 #pragma unroll
-        for (int i = 0; i < IOH::VEC; ++i) hdh += ET<T>::to_f(rh.v[p][i]) * ET<T>::to_f(rdh.v[p][i]);
-      IOV::mask(rd, ci.len);
-      IOV::mask(rv, ci.len);
-      IOV::store_lds(rd, smem + A_DO, LDV);
-      IOV::store_lds(rv, smem + A_V, LDV);
-      IOH::store_lds(rh, smem + A_H, LDK);
-      IOH::store_lds(rdh, smem + A_DH, LDK);
-      if constexpr (GDN) {
-        IOV::mask(rn, ci.len);
-        IOV::store_lds(rn, smem + A_DVN, LDV);
+      for (int kk = 0; kk < BVH; kk += 32) {
+        const typename ET<T>::frag aDO = ET<T>::load_frag(DO + (16 * wv + fr) * LDV + kk + fg);
+        const typename ET<T>::frag aVN = ET<T>::load_frag(VN + (16 * wv + fr) * LDV + kk + fg);
+        typename ET<T>::frag aDVN = aVN;
+        if constexpr (GDN) aDVN = ET<T>::load_frag(DVN + (16 * wv + fr) * LDV + kk + fg);
+#pragma unroll
+        for (int nj = 0; nj < 4; ++nj)
+          ET<T>::mma(dP[0][nj], aDO, ET<T>::load_frag(VN + (16 * nj + fr) * LDV + kk + fg));
+        __builtin_amdgcn_sched_barrier(0);     // bounds the fragments in flight (register budget)
+#pragma unroll
+        for (int ni = 0; ni < NBK; ++ni) {
+          const typename ET<T>::frag bH = ET<T>::load_frag_t(HT, LDK, kk, 16 * ni);
+          ET<T>::mma(dqi[0][ni], aDO, bH);
+          if constexpr (GDN) ET<T>::mma(dw[0][ni], aDVN, bH);
+          ET<T>::mma(dkd[0][ni], aVN, ET<T>::load_frag_t(DHT, LDK, kk, 16 * ni));
+          if (ni % 4 == 3) __builtin_amdgcn_sched_barrier(0);
+        }
       }
-      lds_barrier();
-      if (vv + BVH < V) issueA(it, vv + BVH); else issueQK(it);
-      gemm<T, 1, 4, false, false>(dP, smem + A_DO, LDV, 16 * wv, smem + A_V, LDV, 0, 0, BVH);
-      gemm<T, 1, NBK, false, true>(dqi, smem + A_DO, LDV, 16 * wv, smem + A_H, LDK, 0, 0, BVH);
-      gemm<T, 1, NBK, false, true>(dkd, smem + A_V, LDV, 16 * wv, smem + A_DH, LDK, 0, 0, BVH);
-      if constexpr (GDN) gemm<T, 1, NBK, false, true>(dw, smem + A_DVN, LDV, 16 * wv, smem + A_H, LDK, 0, 0, BVH);
-      lds_barrier();
     }
-    // block reduction of <S, dS'>
-    hdh = wave_sum(hdh);
-    if (l == 0) s_red[wv] = hdh;
-    // phase B operands
-    gate_finish(a, graw, ci.len, s_b, s_eb, s_ed);
-    IOK::mask(rq, ci.len);
-    IOK::mask(rk, ci.len);
-    IOK::store_lds(rq, smem + B_Q, LDK);
-    IOK::store_lds(rk, smem + B_K, LDK);
-    lds_barrier();
-    issueA(min(it + (int)gridDim.x, nitems - 1), 0);
+    lds_barrier();                                                                       // D
+    if constexpr (GDN) {
+      // dw = -dv_new S^T is complete: it leaves its registers now, staged through the first slice
+      // buffer, which is idle until the loaders refill it after A
+      store_strip<T, NBK>(dw, smem + wv * 16 * LDK, row_ptr<T>(a.dw, ci.b, ci.tok + 16 * wv, h), a.dw.st,
+                          ci.len - 16 * wv, -1.0f);
+    }
+    lds_barrier();                                                                       // A
+    T* PB = smem + BUF1;
 #pragma unroll
     for (int nj = 0; nj < 4; ++nj) {
       f32x4 p;
@@ -457,15 +535,17 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dqk(const lmoe_args a) {
         const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * nj + (l & 15);
         p[i] = (r >= cc) ? a.scale * dP[0][nj][i] * texp<T>(s_b[r] - s_b[cc]) : 0.f;
       }
-      acc_to_lds_t<T>(p, smem + B_DPT, LDC, 16 * wv, 16 * nj);      // [j][i]
+      acc_to_lds_t<T>(p, PB + B_DPT, LDC, 16 * wv, 16 * nj);      // [j][i]
     }
-    lds_barrier();
+    lds_barrier();                                                                       // b
     f32x4 dq[1][NBK], dk[1][NBK];
     acc_zero(dq); acc_zero(dk);
     // dq_intra[i][c] = sum_j dPG[i][j] k[j][c] : A = dPG^T stored [j][i] (contraction along rows)
-    gemm<T, 1, NBK, true, true>(dq, smem + B_DPT, LDC, 16 * wv, smem + B_K, LDK, 0, 0, CH);
+    gemm<T, 1, NBK, true, true>(dq, PB + B_DPT, LDC, 16 * wv, PB + B_K, LDK, 0, 0, CH);
+    __builtin_amdgcn_sched_barrier(0);
     // dk_intra[j][c] = sum_i dPG[i][j] q[i][c] : A = dPG^T rows j (contraction along columns)
-    gemm<T, 1, NBK, false, true>(dk, smem + B_DPT, LDC, 16 * wv, smem + B_Q, LDK, 0, 0, CH);
+    gemm<T, 1, NBK, false, true>(dk, PB + B_DPT, LDC, 16 * wv, PB + B_Q, LDK, 0, 0, CH);
+    __builtin_amdgcn_sched_barrier(0);
     // combine and form db_i = q_i.dq_i - k_i.dk_i ; kk = sum_j (dk_d . k_d)_j
     float dbp[4] = {0.f, 0.f, 0.f, 0.f};
     float kk = 0.f;
@@ -474,8 +554,8 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dqk(const lmoe_args a) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
-        const float qv = ET<T>::to_f(smem[B_Q + r * LDK + cc]);
-        const float kv = ET<T>::to_f(smem[B_K + r * LDK + cc]);
+        const float qv = ET<T>::to_f(PB[B_Q + r * LDK + cc]);
+        const float kv = ET<T>::to_f(PB[B_K + r * LDK + cc]);
         const float dqv = a.scale * s_eb[r] * dqi[0][ni][i] + dq[0][ni][i];
         const float dkdv = s_ed[r] * dkd[0][ni][i];
         const float dkv = dkdv + dk[0][ni][i];
@@ -484,7 +564,7 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dqk(const lmoe_args a) {
         dq[0][ni][i] = dqv;
         dk[0][ni][i] = dkv;
       }
-    // reduce db over the 16 lanes that share a row group, kk over the whole block
+    // reduce db over the 16 lanes that share a row group, kk over the whole team
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
 #pragma unroll
@@ -496,16 +576,12 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dqk(const lmoe_args a) {
     }
     kk = wave_sum(kk);
     if (l == 0) s_red[4 + wv] = kk;
-    lds_barrier();     // q, k tiles are dead from here: wave-private slices become store staging
+    lds_barrier();     // c: q, k tiles are dead from here: wave-private slices become store staging
     {
-      T* stg = smem + B_K + wv * 16 * LDK;    // this wave's 16 rows of the k tile, then of the q tile
+      T* stg = PB + B_K + wv * 16 * LDK;    // this wave's 16 rows of the k tile, then of the q tile
       store_strip<T, NBK>(dq, stg, row_ptr<T>(a.dq, ci.b, ci.tok + 16 * wv, h), a.dq.st, ci.len - 16 * wv, 1.0f);
-      T* stg2 = smem + B_Q + wv * 16 * LDK;
+      T* stg2 = PB + B_Q + wv * 16 * LDK;
       store_strip<T, NBK>(dk, stg2, row_ptr<T>(a.dk, ci.b, ci.tok + 16 * wv, h), a.dk.st, ci.len - 16 * wv, 1.0f);
-      if constexpr (GDN) {
-        // dw = -dv_new S^T ; staging reuses the first slice again (same wave, program order)
-        store_strip<T, NBK>(dw, stg, row_ptr<T>(a.dw, ci.b, ci.tok + 16 * wv, h), a.dw.st, ci.len - 16 * wv, -1.0f);
-      }
     }
     if (threadIdx.x < 64) {
       const int j = threadIdx.x;
@@ -518,7 +594,7 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dqk(const lmoe_args a) {
       if constexpr (!GDN) x = wave_rev_scan(x);   // dg; the delta rule finishes db in its WY backward
       if (a.dg.ptr && j < ci.len) ((float*)a.dg.ptr)[row_off(a.dg, ci.b, ci.tok + j, h)] = x;
     }
-    lds_barrier();     // staging and the gate arrays are reused by the next item
+    lds_barrier();     // E: the second buffer and the gate arrays go to the next item
   }
 }
 

@@ -108,6 +108,20 @@ __device__ __forceinline__ void gate_finish(const lmoe_args& a, uint32_t raw, in
   }
 }
 
+// gate_finish for a caller that holds the raw bits in the lanes of one wave of its choice:
+// `active` selects that wave (wave-uniform), `l` is the lane
+__device__ __forceinline__ void gate_finish_wave(const lmoe_args& a, uint32_t raw, int len, int l, bool active,
+                                                 float* sb, float* seb, float* sed) {
+  if (active) {
+    const bool gated = a.gate != LMOE_GATE_NONE && a.g.ptr != nullptr;
+    const float x = wave_incl_scan((gated && l < len) ? scalar_from_raw(raw, a.g_dtype) : 0.f);
+    const float xl = __shfl(x, 63, 64);
+    sb[l] = x;
+    seb[l] = expf(x);
+    sed[l] = expf(xl - x);
+  }
+}
+
 // number of work-groups of a persistent chunk-parallel kernel: `per_cu` per compute unit
 inline int persistent_grid(int nitems, int per_cu) {
   static int ncu = 0;
