@@ -4,18 +4,33 @@
 
 namespace lmoe {
 
+// Width of the V-slice a work-group carries: the narrow slice gives more work-groups (a problem
+// with few (sequence, head) pairs must still reach every CU); with enough pairs the wide slice
+// halves the number of times k, w, q, P are read and stores whole 128-byte lines of o, v_new.
+template <typename T, int V> inline bool wide_slices(const lmoe_args& a) {
+  constexpr int BW = GdnStateCfg<T>::BV_WIDE;
+  return BW <= V && BW != GdnStateCfg<T>::BV && (int64_t)a.N * a.H * (V / BW) >= cu_count();
+}
+template <typename T, int K, int V, int BV> void launch_fwd(const lmoe_args& a, hipStream_t st) {
+  const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BV);
+  hipLaunchKernelGGL((k_gdn_state_fwd<T, K, V, BV>), dim3(grid), dim3(3 * NTHR), 0, st, a);
+}
+template <typename T, int K, int V, int BV> void launch_bwd(const lmoe_args& a, hipStream_t st) {
+  const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BV);
+  hipLaunchKernelGGL((k_gdn_state_bwd<T, K, V, BV>), dim3(grid), dim3(3 * NTHR), 0, st, a);
+}
 template <typename T, int K, int V> struct GdnStateFwd {
   static void run(const lmoe_args& a, hipStream_t st) {
-    constexpr int BV = GdnStateCfg<T>::BV;
-    const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BV);
-    hipLaunchKernelGGL((k_gdn_state_fwd<T, K, V, BV>), dim3(grid), dim3(3 * NTHR), 0, st, a);
+    constexpr int BW = GdnStateCfg<T>::BV_WIDE <= V ? GdnStateCfg<T>::BV_WIDE : GdnStateCfg<T>::BV;
+    if (wide_slices<T, V>(a)) launch_fwd<T, K, V, BW>(a, st);
+    else launch_fwd<T, K, V, GdnStateCfg<T>::BV>(a, st);
   }
 };
 template <typename T, int K, int V> struct GdnStateBwd {
   static void run(const lmoe_args& a, hipStream_t st) {
-    constexpr int BV = GdnStateCfg<T>::BV;
-    const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BV);
-    hipLaunchKernelGGL((k_gdn_state_bwd<T, K, V, BV>), dim3(grid), dim3(3 * NTHR), 0, st, a);
+    constexpr int BW = GdnStateCfg<T>::BV_WIDE <= V ? GdnStateCfg<T>::BV_WIDE : GdnStateCfg<T>::BV;
+    if (wide_slices<T, V>(a)) launch_bwd<T, K, V, BW>(a, st);
+    else launch_bwd<T, K, V, GdnStateCfg<T>::BV>(a, st);
   }
 };
 void launch_gdn_state_fwd(const lmoe_args& a, hipStream_t st) { dispatch<GdnStateFwd>(a, st); }

@@ -32,6 +32,7 @@ namespace lmoe {
 // V-slice / prefetch shape of the sequential passes per element type
 template <typename T> struct GdnStateCfg {
   static constexpr int BV = sizeof(T) == 2 ? 32 : 16;    // V columns per work-group
+  static constexpr int BV_WIDE = sizeof(T) == 2 ? 64 : 16;   // ... when there are enough work-groups anyway
   static constexpr int LPF = sizeof(T) == 2 ? 2 : 1;     // chunks a loader keeps in flight per ring
 };
 

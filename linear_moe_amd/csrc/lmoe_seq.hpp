@@ -123,14 +123,17 @@ __device__ __forceinline__ void gate_finish_wave(const lmoe_args& a, uint32_t ra
 }
 
 // number of work-groups of a persistent chunk-parallel kernel: `per_cu` per compute unit
-inline int persistent_grid(int nitems, int per_cu) {
+inline int cu_count() {
   static int ncu = 0;
   if (ncu == 0) {
     int dev = 0, n = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
     ncu = n;
   }
-  const int g = ncu * per_cu;
+  return ncu;
+}
+inline int persistent_grid(int nitems, int per_cu) {
+  const int g = cu_count() * per_cu;
   return nitems < g ? nitems : g;
 }
 
