@@ -10,8 +10,9 @@
 //   dk_jk = e^{b_Ck - b_jk} (v dS'^T)_jk + sum_{i>=j} dA_ij q_ik e^{b_ik - b_jk}
 //   db_ik = q_ik dq_ik - k_ik dk_ik (+ on the last row: sum_j (dk_d . k_d)_jk + e^{b_Ck} sum_v S_kv dS'_kv)
 //   dg    = reverse cumsum of db over the chunk's tokens
-// The pairwise-exponent sums (A, and the intra-chunk parts of dq, dk) run on the vector ALU in
-// fp32; every other product runs on MFMA through gemm_nt.
+// Pairwise exponents are formed only inside 16-token sub-chunks (vector ALU, fp32); between
+// sub-chunks the decay factors through the cumulative gate at the sub-chunk boundary, which turns
+// those parts into products of scaled tiles on MFMA, like every other product here.
 #pragma once
 #include "lmoe_seq.hpp"
 
@@ -19,9 +20,8 @@ namespace lmoe {
 
 // g tile of the chunk -> fp32 LDS tile s_b[64][K+1] holding the inclusive cumsum over tokens.
 // All threads; ends with a barrier.
-template <typename GT, int K>
+template <typename GT, int K, int LDB = K + 1>
 __device__ __forceinline__ void gla_gate_tile(const lmoe_args& a, int b, int tok, int len, int h, float* s_b) {
-  constexpr int LDB = K + 1;
   typedef TileIO<GT, CH, K> IOG;
   typename IOG::Regs rg;
   IOG::load(rg, row_ptr<GT>(a.g, b, tok, h), a.g.st, len);
@@ -39,35 +39,77 @@ __device__ __forceinline__ void gla_gate_tile(const lmoe_args& a, int b, int tok
 
 // ------------------------------------------------------------------------- //
 // A (intra-chunk attention matrix), grid = (NT, H)
+//   The chunk is cut into four sub-chunks of 16 tokens.  For a block (I, J) with J < I the decay
+//   factors through the cumulative gate at the last token before sub-chunk I, b* = b_{16 I - 1}:
+//     A_ij = sum_k (q_ik e^{b_ik - b*_k}) (k_jk e^{b*_k - b_jk}),   both exponents <= 0,
+//   which is a matrix product of two scaled tiles (MFMA).  Only the four diagonal blocks need the
+//   exponent per pair; they run on the vector ALU in fp32, one block per wave, four pairs per lane.
 // ------------------------------------------------------------------------- //
 template <typename T, typename GT, int K>
 __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
-  constexpr int LDB = K + 1;
-  __shared__ float s_b[CH * LDB], s_q[CH * LDB], s_k[CH * LDB];
+  constexpr int LDB = K + 4, LDK = K + LPAD, LDC = CH + LPAD;
+  __shared__ __attribute__((aligned(16))) float s_b[CH * LDB];
+  __shared__ __attribute__((aligned(16))) T s_q[CH * LDK];        // q, k as loaded
+  __shared__ __attribute__((aligned(16))) T s_k[CH * LDK];
+  __shared__ __attribute__((aligned(16))) T s_qt[16 * LDK];       // scaled operands of one block row
+  __shared__ __attribute__((aligned(16))) T s_kt[48 * LDK];
+  __shared__ __attribute__((aligned(16))) T s_A[CH * LDC];
   const int cid = blockIdx.x, h = blockIdx.y;
   const ChunkInfo ci = chunk_info(a, cid);
+  const int wv = wave_id(), l = lane_id();
   typedef TileIO<T, CH, K> IOK;
+  typedef TileIO<T, CH, CH> IOA;
   {
     typename IOK::Regs rq, rk;
     IOK::load(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
     IOK::load(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
-    IOK::store_lds_f32(rq, s_q, LDB);
-    IOK::store_lds_f32(rk, s_k, LDB);
+    IOK::store_lds(rq, s_q, LDK);
+    IOK::store_lds(rk, s_k, LDK);
   }
-  gla_gate_tile<GT, K>(a, ci.b, ci.tok, ci.len, h, s_b);
-  T* am = (T*)a.amat + ((int64_t)cid * a.H + h) * CH * CH;
-  const int j = threadIdx.x & 63, i0 = threadIdx.x >> 6;
-  for (int r = 0; r < 16; ++r) {
-    const int i = i0 + 4 * r;
-    float s = 0.f;
-    if (i >= j) {
-      const float* qi = s_q + i * LDB; const float* bi = s_b + i * LDB;
-      const float* kj = s_k + j * LDB; const float* bj = s_b + j * LDB;
-#pragma unroll 4
-      for (int kk = 0; kk < K; ++kk) s += qi[kk] * kj[kk] * texp<T>(bi[kk] - bj[kk]);
+  for (int idx = threadIdx.x; idx < CH * LDC; idx += NTHR) s_A[idx] = ET<T>::from_f(0.f);   // blocks above the diagonal
+  gla_gate_tile<GT, K, LDB>(a, ci.b, ci.tok, ci.len, h, s_b);    // barriers inside
+  // ---- diagonal blocks: wave w owns block (w, w); lane -> row i, columns j0 .. j0 + 3 ----
+  {
+    const int i = 16 * wv + (l & 15), j0 = 16 * wv + 4 * (l >> 4);
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int k4 = 0; k4 < K; k4 += 4) {
+      const f32x4 bi = *(const f32x4*)(s_b + i * LDB + k4);
+      float qi[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) qi[e] = ET<T>::to_f(s_q[i * LDK + k4 + e]);
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+        const int j = j0 + jj;
+        const f32x4 bj = *(const f32x4*)(s_b + j * LDB + k4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          acc[jj] += qi[e] * ET<T>::to_f(s_k[j * LDK + k4 + e]) * texp<T>(fminf(bi[e] - bj[e], 0.f));
+      }
     }
-    am[i * CH + j] = ET<T>::from_f(s);
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) s_A[i * LDC + j0 + jj] = ET<T>::from_f(i >= j0 + jj ? acc[jj] : 0.f);
   }
+  // ---- blocks below the diagonal, one block row at a time ----
+  for (int I = 1; I < 4; ++I) {
+    const float* bs = s_b + (16 * I - 1) * LDB;                   // b* of this block row
+    for (int idx = threadIdx.x; idx < 16 * K; idx += NTHR) {
+      const int r = idx / K, c = idx % K, i = 16 * I + r;
+      s_qt[r * LDK + c] = ET<T>::from_f(ET<T>::to_f(s_q[i * LDK + c]) * texp<T>(s_b[i * LDB + c] - bs[c]));
+    }
+    for (int idx = threadIdx.x; idx < 16 * I * K; idx += NTHR) {
+      const int j = idx / K, c = idx % K;
+      s_kt[j * LDK + c] = ET<T>::from_f(ET<T>::to_f(s_k[j * LDK + c]) * texp<T>(bs[c] - s_b[j * LDB + c]));
+    }
+    __syncthreads();
+    if (wv < I) {
+      f32x4 t[1][1];
+      acc_zero(t);
+      gemm<T, 1, 1, false, false>(t, s_qt, LDK, 0, s_kt, LDK, 16 * wv, 0, K);
+      acc_to_lds<T>(t[0][0], s_A, LDC, 16 * I, 16 * wv);
+    }
+    __syncthreads();
+  }
+  IOA::lds_to_global(s_A, LDC, (T*)a.amat + ((int64_t)cid * a.H + h) * CH * CH, CH, CH);
 }
 
 // ------------------------------------------------------------------------- //
