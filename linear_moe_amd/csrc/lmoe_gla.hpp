@@ -349,7 +349,22 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
   // phase A (element type T): do, v, S, dS' slices.  phase B (fp32): dA, q, k, b tiles
   constexpr int A_DO = 0, A_V = A_DO + CH * LDV, A_H = A_V + CH * LDV, A_DH = A_H + K * LDV, A_END = A_DH + K * LDV;
   constexpr int B_DP = 0, B_Q = B_DP + CH * LDP, B_K = B_Q + CH * LDB, B_B = B_K + CH * LDB, B_END = B_B + CH * LDB;
-  constexpr int NBYTES = (A_END * (int)sizeof(T) > B_END * 4) ? A_END * (int)sizeof(T) : B_END * 4;
+  // Sub-chunk form of the intra-chunk sums (see k_gla_intra_fwd): between 16-token sub-chunks the
+  // decay factors through the cumulative gate b* at the sub-chunk boundary,
+  //   dq_i += e^{b_i - b*} [ dA (k e^{b* - b}) ]_i      (j in earlier sub-chunks)
+  //   dk_j += e^{b* - b_j} [ dA^T (q e^{b - b*}) ]_j    (i in later sub-chunks)
+  // two MFMA products per boundary over element-type tiles dA, k~, q~ behind the fp32 tiles; the
+  // pairwise loops below then cover the diagonal blocks only.  Used where the extra tiles fit LDS.
+  constexpr int LDC = CH + LPAD, LDK = K + LPAD;
+  // layout of that form: b (fp32) | q, k as loaded | dA | k~ | q~  (element type T)
+  constexpr int S_B = 0, S_TBASE = CH * LDB * 4;
+  constexpr int T_Q = 0, T_K = T_Q + CH * LDK, T_DA = T_K + CH * LDK, T_KT = T_DA + CH * LDC, T_QT = T_KT + CH * LDK,
+                T_END = T_QT + CH * LDK;
+  constexpr int S_BYTES = S_TBASE + T_END * (int)sizeof(T);
+  constexpr bool SUB = S_BYTES + 4096 <= 160 * 1024;
+  static_assert(!SUB || 2 * CH * LDK * (int)sizeof(T) >= CH * LDB * 4, "the db tile fits over k~, q~");
+  constexpr int B_BYTES = SUB ? S_BYTES : B_END * 4;
+  constexpr int NBYTES = (A_END * (int)sizeof(T) > B_BYTES) ? A_END * (int)sizeof(T) : B_BYTES;
   __shared__ __attribute__((aligned(16))) unsigned char smem_raw[NBYTES];
   __shared__ float s_hdh[K], s_kk[4 * K];
   T* smT = (T*)smem_raw;
@@ -399,23 +414,61 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
     int row, col; IOH::coords(p, row, col);
     if (col == 0 && row < K) s_hdh[row] = x;
   }
-  // phase B tiles (fp32)
+  // phase B tiles
+  T* tQ = (T*)(smem_raw + S_TBASE) + T_Q;
+  T* tK = (T*)(smem_raw + S_TBASE) + T_K;
+  T* tDA = (T*)(smem_raw + S_TBASE) + T_DA;
+  T* tKT = (T*)(smem_raw + S_TBASE) + T_KT;
+  T* tQT = (T*)(smem_raw + S_TBASE) + T_QT;
+  float* sBw = SUB ? smF + S_B / 4 : smF + B_B;
   {
 #pragma unroll
-    for (int nj = 0; nj < 4; ++nj)
+    for (int nj = 0; nj < 4; ++nj) {
+      f32x4 p;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * nj + (l & 15);
-        smF[B_DP + r * LDP + cc] = (r >= cc) ? a.scale * dP[0][nj][i] : 0.f;
+        p[i] = (r >= cc) ? a.scale * dP[0][nj][i] : 0.f;
+        if constexpr (!SUB) smF[B_DP + r * LDP + cc] = p[i];
       }
+      if constexpr (SUB) acc_to_lds<T>(p, tDA, LDC, 16 * wv, 16 * nj);
+    }
     typename IOK::Regs rq, rk;
     IOK::load(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
     IOK::load(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
-    IOK::store_lds_f32(rq, smF + B_Q, LDB);
-    IOK::store_lds_f32(rk, smF + B_K, LDB);
+    if constexpr (SUB) {
+      IOK::store_lds(rq, tQ, LDK);
+      IOK::store_lds(rk, tK, LDK);
+    } else {
+      IOK::store_lds_f32(rq, smF + B_Q, LDB);
+      IOK::store_lds_f32(rk, smF + B_K, LDB);
+    }
   }
-  gla_gate_tile<GT, K>(a, ci.b, ci.tok, ci.len, h, smF + B_B);   // barriers inside
-  const float* sP = smF + B_DP; const float* sQ = smF + B_Q; const float* sK = smF + B_K; const float* sB = smF + B_B;
+  gla_gate_tile<GT, K>(a, ci.b, ci.tok, ci.len, h, sBw);   // barriers inside
+  const float* sB = sBw;
+  // dA, q, k of the pairwise loops and the epilogue, from whichever tiles this layout keeps
+  auto Pm = [&](int r, int j) { if constexpr (SUB) return ET<T>::to_f(tDA[r * LDC + j]); else return smF[B_DP + r * LDP + j]; };
+  auto Qm = [&](int r, int c) { if constexpr (SUB) return ET<T>::to_f(tQ[r * LDK + c]); else return smF[B_Q + r * LDB + c]; };
+  auto Km = [&](int r, int c) { if constexpr (SUB) return ET<T>::to_f(tK[r * LDK + c]); else return smF[B_K + r * LDB + c]; };
+  // off-diagonal parts: wave R takes the dq rows of sub-chunk R, wave R - 1 the dk rows of sub-chunk R - 1
+  f32x4 dqo[1][NBK], dko[1][NBK];
+  acc_zero(dqo); acc_zero(dko);
+  if constexpr (SUB) {
+    for (int R = 1; R < 4; ++R) {
+      const float* bs = sB + (16 * R - 1) * LDB;                  // b* of this boundary
+      for (int idx = threadIdx.x; idx < CH * K; idx += NTHR) {
+        const int r = idx / K, c = idx % K;
+        const float br = sB[r * LDB + c];
+        tKT[r * LDK + c] = ET<T>::from_f(r < 16 * R ? Km(r, c) * texp<T>(bs[c] - br) : 0.f);
+        tQT[r * LDK + c] = ET<T>::from_f(r >= 16 * R ? Qm(r, c) * texp<T>(br - bs[c]) : 0.f);
+      }
+      __syncthreads();
+      if (wv == R) gemm<T, 1, NBK, false, true>(dqo, tDA, LDC, 16 * R, tKT, LDK, 0, 0, CH);
+      if (wv == R - 1) gemm<T, 1, NBK, true, true>(dko, tDA, LDC, 16 * (R - 1), tQT, LDK, 0, 0, CH);
+      __syncthreads();
+    }
+  }
+  const int jlo = SUB ? 16 * wv : 0, ihi = SUB ? 16 * wv + 16 : CH;   // range of the pairwise loops
   T* dqd = row_ptr<T>(a.dq, ci.b, ci.tok, h);
   T* dkd_g = row_ptr<T>(a.dk, ci.b, ci.tok, h);
   float kkp[NBK];                      // per column: sum over this lane's rows of (dk_d . k_d)
@@ -430,9 +483,13 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
       const int r = 16 * wv + 4 * (l >> 4) + i;
       const float br = sB[r * LDB + cc];
       float sq_ = 0.f, sk_ = 0.f;
-      for (int j = 0; j <= r; ++j) sq_ += sP[r * LDP + j] * sK[j * LDB + cc] * texp<T>(br - sB[j * LDB + cc]);
-      for (int ii = r; ii < CH; ++ii) sk_ += sP[ii * LDP + r] * sQ[ii * LDB + cc] * texp<T>(sB[ii * LDB + cc] - br);
-      const float qv = sQ[r * LDB + cc], kv = sK[r * LDB + cc];
+      for (int j = jlo; j <= r; ++j) sq_ += Pm(r, j) * Km(j, cc) * texp<T>(br - sB[j * LDB + cc]);
+      for (int ii = r; ii < ihi; ++ii) sk_ += Pm(ii, r) * Qm(ii, cc) * texp<T>(sB[ii * LDB + cc] - br);
+      if constexpr (SUB) {
+        if (wv >= 1) sq_ += dqo[0][ni][i] * texp<T>(br - sB[(16 * wv - 1) * LDB + cc]);
+        if (wv <= 2) sk_ += dko[0][ni][i] * texp<T>(sB[(16 * wv + 15) * LDB + cc] - br);
+      }
+      const float qv = Qm(r, cc), kv = Km(r, cc);
       const float ed = texp<T>(bC - br);
       const float dqv = a.scale * texp<T>(br) * dqi[0][ni][i] + sq_;
       const float dkdv = dkd[0][ni][i] * ed;
@@ -450,7 +507,7 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
     if (l < 16) s_kk[wv * K + cc] = kkp[ni];
   }
   __syncthreads();   // all reads of the q tile are done: reuse it for db
-  float* sDB = smF + B_Q;
+  float* sDB = SUB ? (float*)tKT : smF + B_Q;
 #pragma unroll
   for (int ni = 0; ni < NBK; ++ni)
 #pragma unroll
