@@ -134,6 +134,16 @@ int lmoe_chunk_gla_bwd(const lmoe_args* a, void* stream);
 int lmoe_chunk_gated_delta_rule_fwd(const lmoe_args* a, void* stream);
 int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream);
 
+/* Row-wise L2 normalisation over the last dimension, y = x / sqrt(sum x^2 + eps), and its
+ * backward dx = dy rstd - (sum dy x) rstd^3 x, for `rows` contiguous rows of D elements
+ * (D in {64, 128, 256}; dtype LMOE_BF16 | LMOE_F32; fp32 arithmetic; pointers 16-byte aligned).
+ * Replaces l2_norm_fn of the reference, which normalises q and k in front of the delta-rule ops:
+ *   linear_moe/model/common_modules/l2norm.py:22-45 (forward kernel), :64-95 (backward kernel),
+ *   :172-201 (autograd wrapper), called at linear_moe/sequence_modeling/gated_deltanet/gated_deltanet.py:105-106. */
+int lmoe_l2norm_fwd(const void* x, void* y, int64_t rows, int32_t D, int32_t dtype, float eps, void* stream);
+int lmoe_l2norm_bwd(const void* x, const void* dy, void* dx, int64_t rows, int32_t D, int32_t dtype, float eps,
+                    void* stream);
+
 /* Launch ONE kernel of an op's pipeline (profiling support: lets a harness time each kernel
  * with events on its own stream).  `a` must be the fully populated argument block of the
  * op's fwd (stages 0-2, 7) or bwd (stages 3-6) entry point, with the intermediates of the

@@ -45,7 +45,7 @@ ENTRY_POINTS = (
     "lmoe_chunk_simple_gla_fwd", "lmoe_chunk_simple_gla_bwd",
     "lmoe_chunk_gla_fwd", "lmoe_chunk_gla_bwd",
     "lmoe_chunk_gated_delta_rule_fwd", "lmoe_chunk_gated_delta_rule_bwd",
-    "lmoe_launch_stage", "lmoe_selftest_gemm", "lmoe_workspace_bytes",
+    "lmoe_launch_stage", "lmoe_selftest_gemm", "lmoe_workspace_bytes", "lmoe_l2norm_fwd", "lmoe_l2norm_bwd",
 )
 
 _lib = None
@@ -72,6 +72,11 @@ def load() -> C.CDLL:
     lib.lmoe_selftest_gemm.argtypes = [C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                        C.c_void_p]
     lib.lmoe_selftest_gemm.restype = C.c_int
+    lib.lmoe_l2norm_fwd.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_float, C.c_void_p]
+    lib.lmoe_l2norm_fwd.restype = C.c_int
+    lib.lmoe_l2norm_bwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_float,
+                                    C.c_void_p]
+    lib.lmoe_l2norm_bwd.restype = C.c_int
     lib.lmoe_workspace_bytes.argtypes = [C.c_int32] * 9
     lib.lmoe_workspace_bytes.restype = C.c_int64
     _lib = lib

@@ -147,6 +147,31 @@ int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream) {
   return launched(op);
 }
 
+static int check_l2norm(const char* nm, const void* x, const void* out, int64_t rows, int32_t D, int32_t dtype) {
+  if (!x || !out) return fail(-1, "%s: null pointer", nm);
+  if (dtype != LMOE_BF16 && dtype != LMOE_F32) return fail(-2, "%s: dtype must be LMOE_BF16 or LMOE_F32", nm);
+  if (D != 64 && D != 128 && D != 256) return fail(-3, "%s: row length %d unsupported (64, 128 or 256)", nm, D);
+  if (rows < 0) return fail(-4, "%s: negative row count", nm);
+  if (((uintptr_t)x | (uintptr_t)out) & 15) return fail(-9, "%s: pointers must be 16-byte aligned", nm);
+  return 0;
+}
+int lmoe_l2norm_fwd(const void* x, void* y, int64_t rows, int32_t D, int32_t dtype, float eps, void* stream) {
+  const char* nm = "lmoe_l2norm_fwd";
+  if (int r = check_l2norm(nm, x, y, rows, D, dtype)) return r;
+  if (rows == 0) return 0;
+  lmoe::launch_l2norm(dtype, D, x, nullptr, y, rows, eps, false, (hipStream_t)stream);
+  return launched(nm);
+}
+int lmoe_l2norm_bwd(const void* x, const void* dy, void* dx, int64_t rows, int32_t D, int32_t dtype, float eps,
+                    void* stream) {
+  const char* nm = "lmoe_l2norm_bwd";
+  if (int r = check_l2norm(nm, x, dx, rows, D, dtype)) return r;
+  if (!dy || ((uintptr_t)dy & 15)) return fail(-1, "%s: dy must be a 16-byte aligned pointer", nm);
+  if (rows == 0) return 0;
+  lmoe::launch_l2norm(dtype, D, x, dy, dx, rows, eps, true, (hipStream_t)stream);
+  return launched(nm);
+}
+
 int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* stream) {
   const char* nm = "lmoe_launch_stage";
   if (int r = check_common(a, nm)) return r;

@@ -42,5 +42,8 @@ void launch_gdn_wy_bwd(const lmoe_args& a, hipStream_t st);
 // chunk_gla: one kernel of the pipeline (stage = ST_GLA_INTRA_FWD, ST_STATE_FWD, ST_OUT_FWD,
 // ST_STATE_BWD, ST_DV, ST_DQK)
 void launch_gla(const lmoe_args& a, int stage, hipStream_t st);
+// row-wise L2 normalisation of `rows` contiguous rows of D in {64, 128, 256} elements (bwd: out = dx)
+void launch_l2norm(int dtype, int D, const void* x, const void* dy, void* out, int64_t rows, float eps, bool bwd,
+                   hipStream_t st);
 void launch_selftest(int dtype, int kd, const void* A, const void* B, float* C, float* G, hipStream_t st);
 }  // namespace lmoe

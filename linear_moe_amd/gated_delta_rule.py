@@ -15,6 +15,7 @@ from typing import Optional, Tuple
 import torch
 
 from . import _lib
+from .l2norm import l2_norm
 from ._host import (SeqPlan, _aligned, _check_inputs, _desc, _state_check, base_args, ptr, stream_ptr)
 
 
@@ -144,14 +145,7 @@ def chunk_gated_delta_rule(
     """q, k: ``[B,T,H,K]``, v: ``[B,T,H,V]``, g (log-space decay) and beta: ``[B,T,H]``
     (``[B,H,T,*]`` with ``head_first=True``).  Returns ``(o, final_state)``."""
     if use_qk_l2norm_in_kernel:
-        q = _l2norm(q)
-        k = _l2norm(k)
+        q = l2_norm(q)
+        k = l2_norm(k)
     return _ChunkGatedDeltaRule.apply(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens,
                                       head_first)
-
-
-def _l2norm(x: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
-    """x * rsqrt(sum x^2 + eps) in fp32 (linear_moe/model/common_modules/l2norm.py:22-45);
-    differentiable torch ops, placed in front of the HIP op."""
-    xf = x.float()
-    return (xf * torch.rsqrt((xf * xf).sum(-1, keepdim=True) + eps)).to(x.dtype)

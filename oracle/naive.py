@@ -241,3 +241,12 @@ def naive_lightning_attn2(q, k, v, s, dtype=torch.float64):
     g = (-s.reshape(1, H, 1).to(dtype)).expand(B, H, T)
     o, _ = naive_recurrent_simple_gla(q, k, v, g, 1.0, None, False, None, True, dtype)
     return o
+
+
+def naive_l2_norm(x: Tensor, eps: float = 1e-6, dtype=torch.float64) -> Tensor:
+    """y = x / sqrt(sum x^2 + eps) over the last dimension
+    (linear_moe/model/common_modules/l2norm.py:22-45: eps sits inside the square root; the backward
+    kernel :64-95 is the derivative of exactly this expression, so autograd through it is the oracle
+    of the gradient too)."""
+    x = x.to(dtype)
+    return x / torch.sqrt((x * x).sum(-1, keepdim=True) + eps)

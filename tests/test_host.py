@@ -148,8 +148,7 @@ def test_fla_shim_resolves_every_name_the_reference_imports():
         "from lightning_attn.ops.triton import lightning_attn2, lightning_attn2_no_decay\n"
         "import linear_moe_amd, torch\n"
         "assert chunk_gated_delta_rule is linear_moe_amd.chunk_gated_delta_rule\n"
-        "x = torch.tensor([[3.0, 4.0]])\n"
-        "assert torch.allclose(l2_norm(x), x / 5.0, atol=1e-6)\n"
+        "assert l2_norm is linear_moe_amd.l2_norm\n"
         "print('ok')\n")
     env = {k: v for k, v in os.environ.items() if k != "PYTHONPATH"}
     env["PYTHONPATH"] = shim

@@ -267,3 +267,24 @@ def test_gate_gradient_identity():
     x = (q * dq).sum(-1) - (k * dk).sum(-1)
     ref = x.flip(2).cumsum(2).flip(2) + (ht * dht).sum((-1, -2))[..., None]
     assert torch.allclose(dg, ref, atol=1e-10)
+
+
+def test_l2_norm_pins():
+    """naive_l2_norm: library routine for eps = 0, hand-computed values that place eps inside the square
+    root, scale invariance, and the backward formula of the reference kernel (l2norm.py:64-95)."""
+    import torch.nn.functional as F
+    x = rnd(7001, 5, 3, 16).double()
+    assert torch.allclose(naive.naive_l2_norm(x, eps=0.0), F.normalize(x, dim=-1, eps=0.0), atol=1e-14)
+    v = torch.tensor([[3.0, 4.0]], dtype=torch.float64)
+    assert torch.allclose(naive.naive_l2_norm(v, eps=0.0), torch.tensor([[0.6, 0.8]], dtype=torch.float64))
+    assert torch.allclose(naive.naive_l2_norm(v, eps=11.0), v / 6.0)                 # sqrt(25 + 11) = 6
+    assert torch.equal(naive.naive_l2_norm(torch.zeros(2, 4)), torch.zeros(2, 4, dtype=torch.float64))
+    big = x * 1e3
+    assert torch.allclose(naive.naive_l2_norm(big), naive.naive_l2_norm(2.5 * big), atol=1e-9)
+    xr = x.clone().requires_grad_(True)
+    dy = rnd(7002, 5, 3, 16).double()
+    (naive.naive_l2_norm(xr, eps=1e-6) * dy).sum().backward()
+    var = (x * x).sum(-1, keepdim=True)
+    rstd = 1.0 / torch.sqrt(var + 1e-6)
+    want = dy * rstd - (dy * x).sum(-1, keepdim=True) * (1.0 / (var + 1e-6)) * rstd * x
+    assert torch.allclose(xr.grad, want, atol=1e-12)
