@@ -27,15 +27,14 @@ PEAK_MFMA_BF16 = 2.5e15   # dense bf16 MFMA, FLOP/s (MI355X published)
 PEAK_HBM = 8.0e12         # B/s
 CH = 64
 
-STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_gdn_state_fwd", 4: "k_gdn_state_bwd", 5: "k_bwd_dqk", 6: "k_gdn_wy_bwd"}
+STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_gdn_state_fwd", 4: "k_gdn_state_bwd", 5: "k_gdn_bwd_chunk"}
 
 # HBM bytes per launch on this workload, from two rocprofv3 --pmc runs of this file (FETCH_SIZE, then
 # WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for the 256 MiB device
 # copy that main() issues first (FETCH_SIZE reads half of the bytes fetched, WRITE_SIZE all of the
 # bytes written).  Summary and commands: profiles/gdn_fwd_bwd_cfg4_hbm_traffic.md.
 CALIB_COPY_BYTES = 256 << 20
-MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 857625238, "k_gdn_state_fwd": 1145233912, "k_gdn_state_bwd": 1011003237,
-                    "k_bwd_dqk": 1646770043, "k_gdn_wy_bwd": 1118582430}
+MEASURED_TRAFFIC = {}
 
 
 def gdn_inputs(B, T, H, K, V, seed, dtype, device):
@@ -68,11 +67,10 @@ def stage_model(stage, K, V, s=2):
         return 6 * c * kv + 2 * cc * V, (3 * ck + cv + cc) * s + (2 * cv + kv) * s + 8 * c
     if stage == 4:   # k dS', P^T do, q^T do, w^T dv_new | r q,k,w,do,P,table  w dv_new,dhs
         return 6 * c * kv + 2 * cc * V, (3 * ck + cv + cc) * s + (cv + kv) * s + 8 * c
-    if stage == 5:   # do v^T, do S^T, v dS'^T, dv_new S^T, dP k, dP^T q | r do,v_new,dv_new,hs,dhs,q,k  w dq,dk,dw
-        return 2 * cc * V + 6 * c * kv + 4 * cc * K, (3 * cv + 2 * kv + 2 * ck) * s + 3 * ck * s + 8 * c
-    if stage == 6:   # dT, Tinv^T du, Tinv^T dw, two 64^3 products, dM k, dM^T k_b | r du,dw,k,v,Tinv,dk  w dk,dv
-        return (2 * cc * (K + V) + 2 * cc * V + 2 * cc * K + 4 * c ** 3 + 4 * cc * K,
-                (2 * cv + 3 * ck + cc) * s + (ck + cv) * s + c * (12 + s))
+    if stage == 5:   # do v'^T, do S^T, v' dS'^T, du S^T, du v^T, Tinv^T du, G k, G^T q, dw k^T, Tinv^T dw,
+        #              two 64^3 products, dM k, dM^T k_b | r do,v',du,v,hs,dhs,q,k,Tinv,g,beta  w dq,dk,dv,dbeta,dg
+        return (4 * cc * V + 6 * c * kv + 2 * cc * V + 4 * cc * K + 4 * cc * K + 4 * c ** 3 + 4 * cc * K,
+                (4 * cv + 2 * kv + 2 * ck + cc) * s + (2 * ck + cv) * s + c * (4 + s + 8))
     raise ValueError(stage)
 
 
@@ -82,7 +80,7 @@ def time_stages(call, lib, reps):
     from linear_moe_amd import _lib
     st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     out = {}
-    for stage in (0, 1, 4, 5, 6):      # stages 2, 3 (separate output / dv kernels) are not part of this op
+    for stage in (0, 1, 4, 5):         # stages 2, 3 (separate output / dv kernels) are not part of this op
         a = call.fwd_args if stage <= 2 else call.bwd_args
         for _ in range(2):
             _lib.check(lib.lmoe_launch_stage(C.byref(a), call.OP, stage, st), "stage")

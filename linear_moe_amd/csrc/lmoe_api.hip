@@ -136,14 +136,13 @@ int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream) {
   if (int r = check_common(a, op)) return r;
   if (a->gate == LMOE_GATE_VECTOR) return fail(-10, "%s: the gate is one scalar per token and head", op);
   if (!a->beta.ptr) return fail(-12, "%s: beta must not be null", op);
-  if (!a->hs || !a->dhs || !a->vnew.ptr || !a->w.ptr || !a->tinv || !a->pmat || !a->gcum || !a->dvnew.ptr || !a->dw.ptr)
-    return fail(-11, "%s: hs, dhs, vnew, w, tinv, pmat, gcum, dvnew and dw must not be null", op);
+  if (!a->hs || !a->dhs || !a->vnew.ptr || !a->w.ptr || !a->tinv || !a->pmat || !a->gcum || !a->dvnew.ptr)
+    return fail(-11, "%s: hs, dhs, vnew, w, tinv, pmat, gcum and dvnew must not be null", op);
   if (!a->d_o.ptr || !a->dq.ptr || !a->dk.ptr || !a->dv.ptr || !a->dg.ptr || !a->dbeta.ptr)
     return fail(-13, "%s: d_o, dq, dk, dv, dg and dbeta must not be null", op);
   if (a->NT == 0 || a->N == 0) return 0;
   lmoe::launch_gdn_state_bwd(*a, (hipStream_t)stream);
-  lmoe::launch_bwd_dqk(*a, true, (hipStream_t)stream);
-  lmoe::launch_gdn_wy_bwd(*a, (hipStream_t)stream);
+  lmoe::launch_gdn_bwd_chunk(*a, (hipStream_t)stream);
   return launched(op);
 }
 
@@ -201,9 +200,14 @@ int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* strea
           lmoe::launch_state_bwd(*a, st);
         }
         break;
-      case lmoe::ST_DQK: lmoe::launch_bwd_dqk(*a, gdn, st); break;
-      case lmoe::ST_GDN_WY_BWD: if (!gdn) return fail(-20, "%s: stage not part of this op", nm);
-        lmoe::launch_gdn_wy_bwd(*a, st); break;
+      case lmoe::ST_DQK:
+        if (gdn) {
+          if (!a->tinv || !a->dvnew.ptr || !a->beta.ptr) return fail(-11, "%s: tinv, dvnew and beta must not be null", nm);
+          lmoe::launch_gdn_bwd_chunk(*a, st);
+        } else {
+          lmoe::launch_bwd_dqk(*a, false, st);
+        }
+        break;
       default: return fail(-20, "%s: stage %d not part of this op", nm, stage);
     }
   } else if (op == LMOE_OP_GLA) {

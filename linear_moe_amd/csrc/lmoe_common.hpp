@@ -12,7 +12,11 @@
 //    8 x v_mfma_f32_16x16x4_f32 for fp32 operands, behind the same fragment
 //    layout (lane l holds row l%16, contraction elements 8*(l/16) .. +7);
 //  * accumulator layout of one 16x16 block: lane l holds rows 4*(l/16)+i
-//    (i = 0..3) of column l%16.
+//    (i = 0..3) of column l%16;
+//  * helpers that index by lane / thread take that index as a last, defaulted argument: a
+//    persistent kernel passes a value it refreshes per item (fresh_index), which keeps the
+//    address arithmetic inside the iteration instead of hoisted into registers for the whole
+//    kernel.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -46,6 +50,12 @@ __device__ __forceinline__ void wait_all_loads() {
   __builtin_amdgcn_sched_barrier(0);
 }
 
+// x, in a form the compiler cannot prove loop-invariant
+__device__ __forceinline__ int fresh_index(int x) {
+  asm volatile("" : "+v"(x));
+  return x;
+}
+
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
 __device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
 
@@ -67,8 +77,8 @@ template <> struct ET<bf16> {
   // ds_read_b64_tr_b16: inside each group of 16 lanes, lane s points at the 4 elements
   // tile[row + s/4][n0 + 4 (s%4) ..] and receives element (s%4) of the lanes 4j + s/4, j = 0..3,
   // i.e. the four rows row..row+3 of its own column.
-  static __device__ __forceinline__ frag load_frag_t(const bf16* tile, int ld, int k0, int n0) {
-    const int l = threadIdx.x & 63, s = l & 15;
+  static __device__ __forceinline__ frag load_frag_t(const bf16* tile, int ld, int k0, int n0, int l = threadIdx.x & 63) {
+    const int s = l & 15;
     const bf16* p = tile + (k0 + 8 * (l >> 4) + (s >> 2)) * ld + n0 + 4 * (s & 3);
     typedef __attribute__((address_space(3))) bf16x4 lds_b4;
     const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_b4*)p);
@@ -93,8 +103,7 @@ template <> struct ET<float> {
     frag f; f.lo = *(const f32x4*)p; f.hi = *(const f32x4*)(p + 4); return f;
   }
   // contraction index along the rows of the tile: plain strided reads (fp32 is the parity path)
-  static __device__ __forceinline__ frag load_frag_t(const float* tile, int ld, int k0, int n0) {
-    const int l = threadIdx.x & 63;
+  static __device__ __forceinline__ frag load_frag_t(const float* tile, int ld, int k0, int n0, int l = threadIdx.x & 63) {
     const float* p = tile + (k0 + 8 * (l >> 4)) * ld + n0 + (l & 15);
     frag f;
 #pragma unroll
@@ -121,8 +130,7 @@ template <typename T> __device__ __forceinline__ float texp(float x) {
 // ------------------------------------------------------------------------- //
 template <typename T, int MB, int NB>
 __device__ __forceinline__ void gemm_nt(f32x4 (&acc)[MB][NB], const T* A, int lda, int arow0,
-                                        const T* B, int ldb, int brow0, int k0, int k1) {
-  const int l = lane_id();
+                                        const T* B, int ldb, int brow0, int k0, int k1, int l = threadIdx.x & 63) {
   const int r = l & 15, kg = (l >> 4) * 8;
   for (int kk = k0; kk < k1; kk += 32) {
     typename ET<T>::frag a[MB], b[NB];
@@ -142,19 +150,18 @@ __device__ __forceinline__ void gemm_nt(f32x4 (&acc)[MB][NB], const T* A, int ld
 //                                     BT = false: B[b0 + n][k]   BT = true: B[k][b0 + n]
 template <typename T, int MB, int NB, bool AT, bool BT>
 __device__ __forceinline__ void gemm(f32x4 (&acc)[MB][NB], const T* A, int lda, int a0,
-                                     const T* B, int ldb, int b0, int k0, int k1) {
-  const int l = lane_id();
+                                     const T* B, int ldb, int b0, int k0, int k1, int l = threadIdx.x & 63) {
   const int r = l & 15, kg = (l >> 4) * 8;
   for (int kk = k0; kk < k1; kk += 32) {
     typename ET<T>::frag a[MB], b[NB];
 #pragma unroll
     for (int mi = 0; mi < MB; ++mi) {
-      if constexpr (AT) a[mi] = ET<T>::load_frag_t(A, lda, kk, a0 + 16 * mi);
+      if constexpr (AT) a[mi] = ET<T>::load_frag_t(A, lda, kk, a0 + 16 * mi, l);
       else a[mi] = ET<T>::load_frag(A + (a0 + 16 * mi + r) * lda + kk + kg);
     }
 #pragma unroll
     for (int ni = 0; ni < NB; ++ni) {
-      if constexpr (BT) b[ni] = ET<T>::load_frag_t(B, ldb, kk, b0 + 16 * ni);
+      if constexpr (BT) b[ni] = ET<T>::load_frag_t(B, ldb, kk, b0 + 16 * ni, l);
       else b[ni] = ET<T>::load_frag(B + (b0 + 16 * ni + r) * ldb + kk + kg);
     }
 #pragma unroll
@@ -178,16 +185,14 @@ __device__ __forceinline__ int acc_col(int ni) { return 16 * ni + (lane_id() & 1
 
 // store one 16x16 accumulator block to an LDS tile as tile[row][col] (row = M index)
 template <typename T>
-__device__ __forceinline__ void acc_to_lds(const f32x4& a, T* tile, int ld, int row0, int col0) {
-  const int l = lane_id();
+__device__ __forceinline__ void acc_to_lds(const f32x4& a, T* tile, int ld, int row0, int col0, int l = threadIdx.x & 63) {
   const int r = row0 + 4 * (l >> 4), c = col0 + (l & 15);
 #pragma unroll
   for (int i = 0; i < 4; ++i) tile[(r + i) * ld + c] = ET<T>::from_f(a[i]);
 }
 // store transposed: tile[col][row] -- the lane's 4 values are contiguous
 template <typename T>
-__device__ __forceinline__ void acc_to_lds_t(const f32x4& a, T* tile, int ld, int row0, int col0) {
-  const int l = lane_id();
+__device__ __forceinline__ void acc_to_lds_t(const f32x4& a, T* tile, int ld, int row0, int col0, int l = threadIdx.x & 63) {
   const int r = row0 + 4 * (l >> 4), c = col0 + (l & 15);
   T* p = tile + c * ld + r;
   if constexpr (sizeof(T) == 2) {
@@ -205,10 +210,9 @@ __device__ __forceinline__ void acc_to_lds_t(const f32x4& a, T* tile, int ld, in
 // to what the destination already holds (read with the same 16-byte vectors).
 template <typename T, int NB, bool ADD = false>
 __device__ __forceinline__ void store_strip(const f32x4 (&acc)[1][NB], T* stg, T* __restrict__ gdst,
-                                            int64_t row_stride, int nvalid, float mul) {
+                                            int64_t row_stride, int nvalid, float mul, int l = threadIdx.x & 63) {
   constexpr int W = NB * 16, LD = W + LPAD, VEC = ET<T>::VEC, VPR = W / VEC;
   typedef typename ET<T>::vec vec;
-  const int l = lane_id();
 #pragma unroll
   for (int ni = 0; ni < NB; ++ni)
 #pragma unroll
@@ -300,29 +304,29 @@ template <typename T, int ROWS, int COLS> struct TileIO {
 
   // thread index inside a team of 256: work-groups of 512 threads use two teams (waves 0-3 and
   // 4-7) that each move whole tiles
-  static __device__ __forceinline__ void coords(int p, int& row, int& col) {
-    const int idx = p * NTHR + (threadIdx.x & (NTHR - 1));
+  static __device__ __forceinline__ void coords(int p, int& row, int& col, int tid = threadIdx.x & (NTHR - 1)) {
+    const int idx = p * NTHR + tid;
     row = idx / VPR; col = (idx % VPR) * VEC;
   }
   // Branch-free loads: rows >= nvalid (nvalid >= 1) re-read the last valid row, so that no load
   // sits behind a branch and the compiler can count outstanding loads exactly (prefetches stay in
   // flight across barriers).  mask() then zeroes the rows >= nvalid; software-pipelined kernels
   // call load_nomask() when they issue a prefetch and mask() when they consume it.
-  static __device__ __forceinline__ void load_nomask(Regs& r, const T* __restrict__ src, int64_t row_stride, int nvalid) {
+  static __device__ __forceinline__ void load_nomask(Regs& r, const T* __restrict__ src, int64_t row_stride, int nvalid, int tid = threadIdx.x & (NTHR - 1)) {
     const int last = (nvalid < ROWS ? nvalid : ROWS) - 1;
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
-      int row, col; coords(p, row, col);
+      int row, col; coords(p, row, col, tid);
       row = row < last ? row : last;
       r.v[p] = *(const vec*)(src + (int64_t)row * row_stride + col);
     }
   }
-  static __device__ __forceinline__ void mask(Regs& r, int nvalid) {
+  static __device__ __forceinline__ void mask(Regs& r, int nvalid, int tid = threadIdx.x & (NTHR - 1)) {
     if (nvalid >= ROWS) return;                 // uniform: full tiles (the common case) skip it
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
-      int row, col; coords(p, row, col);
+      int row, col; coords(p, row, col, tid);
       const bool ok = row < nvalid;
       u32x4 w = __builtin_bit_cast(u32x4, r.v[p]);
 #pragma unroll
@@ -335,10 +339,10 @@ template <typename T, int ROWS, int COLS> struct TileIO {
     mask(r, nvalid);
   }
   // tile[row][col] = x
-  static __device__ __forceinline__ void store_lds(const Regs& r, T* tile, int ld) {
+  static __device__ __forceinline__ void store_lds(const Regs& r, T* tile, int ld, int tid = threadIdx.x & (NTHR - 1)) {
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
-      int row, col; coords(p, row, col);
+      int row, col; coords(p, row, col, tid);
       if (row < ROWS) *(vec*)(tile + row * ld + col) = r.v[p];
     }
   }

@@ -1,14 +1,18 @@
-// Instantiation and launch of the gated-delta-rule WY backward kernel.
+// Instantiation and launch of the chunk-parallel backward kernel of the gated delta rule.
 #include "lmoe_launch.hpp"
-#include "lmoe_gdn_wy_bwd.hpp"
+#include "lmoe_gdn_bwd_chunk.hpp"
 
 namespace lmoe {
 
-template <typename T, int K, int V> struct GdnWyBwd {
+template <typename T, int K, int V> struct GdnBwdChunk {
   static void run(const lmoe_args& a, hipStream_t st) {
-    hipLaunchKernelGGL((k_gdn_wy_bwd<T, K, V>), dim3(a.NT, a.H), dim3(NTHR), 0, st, a);
+    constexpr int BVH = 32;                            // V-slice of stage 1
+    constexpr int NBUF = sizeof(T) == 2 ? 2 : 1;       // slice buffers: two where LDS has the room
+    static_assert(GdnBwdChunkLds<T, K, BVH, NBUF>::BYTES <= 160 * 1024, "LDS budget of k_gdn_bwd_chunk");
+    const int grid = persistent_grid(a.NT * a.H, 1);
+    hipLaunchKernelGGL((k_gdn_bwd_chunk<T, K, V, BVH, NBUF>), dim3(grid), dim3(2 * NTHR), 0, st, a);
   }
 };
-void launch_gdn_wy_bwd(const lmoe_args& a, hipStream_t st) { dispatch<GdnWyBwd>(a, st); }
+void launch_gdn_bwd_chunk(const lmoe_args& a, hipStream_t st) { dispatch<GdnBwdChunk>(a, st); }
 
 }  // namespace lmoe

@@ -38,7 +38,7 @@ void launch_gdn_wy_fwd(const lmoe_args& a, hipStream_t st);
 void launch_bwd_dv(const lmoe_args& a, bool local, hipStream_t st);
 void launch_state_bwd(const lmoe_args& a, hipStream_t st);        // chunk_simple_gla
 void launch_bwd_dqk(const lmoe_args& a, bool gdn, hipStream_t st);
-void launch_gdn_wy_bwd(const lmoe_args& a, hipStream_t st);
+void launch_gdn_bwd_chunk(const lmoe_args& a, hipStream_t st);    // gated delta rule: all chunk-parallel gradients
 // chunk_gla: one kernel of the pipeline (stage = ST_GLA_INTRA_FWD, ST_STATE_FWD, ST_OUT_FWD,
 // ST_STATE_BWD, ST_DV, ST_DQK)
 void launch_gla(const lmoe_args& a, int stage, hipStream_t st);
