@@ -412,18 +412,18 @@ template <typename T, int ROWS, int COLS> struct TileIO {
   }
   // registers <- tile[row][col]  /  global[row][col] <- registers (rows < nvalid): the two halves of
   // lds_to_global for callers that must leave the tile before the stores are issued
-  static __device__ __forceinline__ void load_lds(Regs& r, const T* tile, int ld) {
+  static __device__ __forceinline__ void load_lds(Regs& r, const T* tile, int ld, int tid = threadIdx.x & (NTHR - 1)) {
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
-      int row, col; coords(p, row, col);
+      int row, col; coords(p, row, col, tid);
       row = row < ROWS ? row : ROWS - 1;
       r.v[p] = *(const vec*)(tile + row * ld + col);
     }
   }
-  static __device__ __forceinline__ void store_global(const Regs& r, T* __restrict__ dst, int64_t row_stride, int nvalid) {
+  static __device__ __forceinline__ void store_global(const Regs& r, T* __restrict__ dst, int64_t row_stride, int nvalid, int tid = threadIdx.x & (NTHR - 1)) {
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
-      int row, col; coords(p, row, col);
+      int row, col; coords(p, row, col, tid);
       if (row < ROWS && row < nvalid) *(vec*)(dst + (int64_t)row * row_stride + col) = r.v[p];
     }
   }

@@ -22,28 +22,30 @@
 // Nothing but the final gradients leaves the chip: dw, the two parts of dk and the second read of
 // du stay in registers / LDS.
 //
-// persistent: grid = one work-group per CU, item = (chunk, head).  Work-group = 2 teams of 4 waves on
-// one barrier script.  Team 0 (compute) reads LDS and drives the matrix cores; wave w owns chunk rows
-// 16 w .. 16 w + 15 of every product.  Team 1 (loaders) keeps the next slice, the next q, k and the
-// next item's Tinv, g, beta in flight in registers (whole 128-byte lines per row) and stages them
-// into LDS: slices into NBUF alternating buffers (two where LDS has the room, so that a slice is
-// filled while the previous one is consumed), the stage 2 tiles over the last buffer.  It also forms
-// <S, dS'> from the registers it holds and the gate cumsum of the chunk.
+// persistent: grid = one work-group per CU, item = (chunk, head).  Work-group = 12 waves on one
+// barrier script: 8 compute waves and 4 loader waves.
+//   Compute wave w owns chunk rows 16 (w % 4) .. + 15 and column half w / 4 of every product (half
+//   of K for the K-wide ones, 32 of the 64 columns for the chunk x chunk ones).  The compute waves
+//   touch only LDS and the matrix cores, apart from the 64 floats of dbeta and dg per item.
+//   The loader waves own all other global traffic: they keep the next slice, the next q, k and the
+//   next item's Tinv, g, beta in flight in registers (whole 128-byte lines per row), stage them into
+//   LDS (slices into NBUF alternating buffers, two where LDS has the room, so that a slice is filled
+//   while the previous one is consumed; the stage 2 tiles lie over the last buffer), and lift the
+//   results (dv per slice, dq, dk) out of LDS and store them.  They also form <S, dS'> from the
+//   registers they hold and the gate cumsum of the chunk.
 //   Script per item (NS slices):  R(0) D(0) .. R(NS-1) D(NS-1) | A | b c d e f g h | E
 #pragma once
 #include "lmoe_seq.hpp"
 
 namespace lmoe {
 
-// LDS bytes of k_gdn_bwd_chunk (the launcher falls back to the two-kernel path where it does not fit)
+// LDS bytes of k_gdn_bwd_chunk
 template <typename T, int K, int BVH, int NBUF> struct GdnBwdChunkLds {
   static constexpr int LDV = BVH + LPAD, LDC = CH + LPAD, LDK = K + LPAD;
   static constexpr int A_END = 4 * CH * LDV + 2 * BVH * LDK;
   static constexpr int B_END = 2 * CH * LDK + CH * LDC + CH * LDK;
   static constexpr int NREG = (NBUF - 1) * A_END + (A_END > B_END ? A_END : B_END);
-  static constexpr bool EARLY_DQ = sizeof(T) == 2;
-  static constexpr int STG = 4 * 16 * (EARLY_DQ ? LDK : LDV);
-  static constexpr int BYTES = (NREG + CH * LDC + STG) * (int)sizeof(T) + 8 * 64 * 4;
+  static constexpr int BYTES = (NREG + CH * LDC + CH * LDV) * (int)sizeof(T) + (8 * 64 + 16) * 4;
 };
 
 // gemm with a scheduling fence after every 32-deep step: at most one step's fragments are in flight,
@@ -67,27 +69,25 @@ __device__ __forceinline__ void pin(float (&x)[4]) {
 }
 
 template <typename T, int K, int V, int BVH, int NBUF>
-__global__ __launch_bounds__(2 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
+__global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
   typedef GdnBwdChunkLds<T, K, BVH, NBUF> L;
   constexpr int LDV = L::LDV, LDC = L::LDC, LDK = L::LDK;
-  constexpr int NBK = K / 16, NBH = BVH / 16, NS = V / BVH;
-  constexpr bool EARLY_DQ = L::EARLY_DQ;
-  static_assert(V % BVH == 0 && BVH % 32 == 0, "V-slices");
+  constexpr int NS = V / BVH;
+  constexpr int KH = K / 2, NBK = KH / 16;     // columns / 16-wide tiles of a K-wide product per compute wave
+  static_assert(V % BVH == 0 && BVH == 32, "V-slices: the 8 compute waves split a 64 x 32 slice product 4 x 2");
   static_assert(NBUF == 1 || (NBUF == 2 && NS % 2 == 0), "with two buffers the last slice must sit in the second one");
   // tiles of one V-slice
   constexpr int A_DO = 0, A_VN = A_DO + CH * LDV, A_DVN = A_VN + CH * LDV, A_VV = A_DVN + CH * LDV,
                 A_H = A_VV + CH * LDV, A_DH = A_H + BVH * LDK, A_END = L::A_END;
-  // stage 2 tiles, laid over the last slice buffer: q, k, T0 = G^T then dT^T then (beta dM)^T,
-  // DW = dw (rows), later T1 = X1^T then dM^T in its first 64 x 64
+  // stage 2 tiles, laid over the last slice buffer: q (later dq, then dk, on their way out), k,
+  // T0 = G^T then dT^T then (beta dM)^T, DW = dw (rows), later T1 = X1^T then dM^T in its first 64 x 64
   constexpr int SB = (NBUF - 1) * A_END;
   constexpr int B_Q = SB, B_K = B_Q + CH * LDK, B_T0 = B_K + CH * LDK, B_DW = B_T0 + CH * LDC, B_T1 = B_DW;
   __shared__ __attribute__((aligned(16))) T smem[L::NREG];
   __shared__ __attribute__((aligned(16))) T s_ti[CH * LDC];              // Tinv, whole item
-  __shared__ __attribute__((aligned(16))) T s_stg[L::STG];               // store strips (dv; dq)
-  __shared__ float s_b[64], s_eb[64], s_ed[64], s_beta[64], s_db[64], s_dbeta[64], s_red[8];
+  __shared__ __attribute__((aligned(16))) T s_dv[CH * LDV];              // dv of a slice on its way out
+  __shared__ float s_b[64], s_eb[64], s_ed[64], s_beta[64], s_db[2][64], s_dbeta[2][64], s_red[16];
 
-  const int l = lane_id();
-  const int team = threadIdx.x / NTHR;
   typedef TileIO<T, CH, BVH> IOV;
   typedef TileIO<T, BVH, K> IOH;
   typedef TileIO<T, CH, K> IOK;
@@ -95,14 +95,20 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
   const int nitems = a.NT * a.H;
   const int stride = gridDim.x;
 
-  if (team == 1) {
+  if (threadIdx.x >= 2 * NTHR) {
     // --------------------------------- loaders -------------------------------------------
+    const int l = lane_id();
+    // thread index inside the team, refreshed per item: the per-thread tile offsets are then recomputed
+    // where they are used instead of held (and spilled) for the whole kernel
+    int tid = threadIdx.x & (NTHR - 1);
+    const int lw = wave_id() - 8;            // wave of the loader team
     struct SliceRegs { typename IOV::Regs rd, rvn, rdv, rvv; typename IOH::Regs rh, rdh; int len; };
-    struct ItemRegs { typename IO64::Regs rt; uint32_t graw, braw; int len; };
     struct QKRegs { typename IOK::Regs rq, rk; int len; };
     SliceRegs S;
-    ItemRegs I;
     QKRegs Q;
+    typename IO64::Regs rt;
+    uint32_t graw, braw;
+    int glen;
     // Every prefetch is issued unconditionally (item index clamped to the last item): a load that
     // is skipped on some path would make the compiler drain all outstanding loads at every use.
     auto issue_slice = [&](int it, int vv) {
@@ -110,29 +116,32 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
       const int cid = it / a.H, h = it % a.H;
       const ChunkInfo ci = chunk_info(a, cid);
       S.len = ci.len;
-      IOV::load_nomask(S.rd, row_ptr<T>(a.d_o, ci.b, ci.tok, h) + vv, a.d_o.st, ci.len);
-      IOV::load_nomask(S.rvn, row_ptr<T>(a.vnew, ci.b, ci.tok, h) + vv, a.vnew.st, ci.len);
-      IOV::load_nomask(S.rdv, row_ptr<T>(a.dvnew, ci.b, ci.tok, h) + vv, a.dvnew.st, ci.len);
-      IOV::load_nomask(S.rvv, row_ptr<T>(a.v, ci.b, ci.tok, h) + vv, a.v.st, ci.len);
-      IOH::load_nomask(S.rh, (const T*)a.hs + (((int64_t)cid * a.H + h) * V + vv) * K, K, BVH);
-      IOH::load_nomask(S.rdh, (const T*)a.dhs + (((int64_t)cid * a.H + h) * V + vv) * K, K, BVH);
+      IOV::load_nomask(S.rd, row_ptr<T>(a.d_o, ci.b, ci.tok, h) + vv, a.d_o.st, ci.len, tid);
+      IOV::load_nomask(S.rvn, row_ptr<T>(a.vnew, ci.b, ci.tok, h) + vv, a.vnew.st, ci.len, tid);
+      IOV::load_nomask(S.rdv, row_ptr<T>(a.dvnew, ci.b, ci.tok, h) + vv, a.dvnew.st, ci.len, tid);
+      IOV::load_nomask(S.rvv, row_ptr<T>(a.v, ci.b, ci.tok, h) + vv, a.v.st, ci.len, tid);
+      IOH::load_nomask(S.rh, (const T*)a.hs + (((int64_t)cid * a.H + h) * V + vv) * K, K, BVH, tid);
+      IOH::load_nomask(S.rdh, (const T*)a.dhs + (((int64_t)cid * a.H + h) * V + vv) * K, K, BVH, tid);
     };
-    auto issue_item = [&](int it) {
+    auto issue_tinv = [&](int it) {
+      it = min(it, nitems - 1);
+      IO64::load_nomask(rt, (const T*)a.tinv + (int64_t)it * CH * CH, CH, CH, tid);     // it = cid * H + h
+    };
+    auto issue_gates = [&](int it) {
       it = min(it, nitems - 1);
       const int cid = it / a.H, h = it % a.H;
       const ChunkInfo ci = chunk_info(a, cid);
-      I.len = ci.len;
-      IO64::load_nomask(I.rt, (const T*)a.tinv + ((int64_t)cid * a.H + h) * CH * CH, CH, CH);
-      I.graw = gate_prefetch(a, ci.b, ci.tok, ci.len, h);
-      I.braw = load_scalar_raw(a.beta.ptr, a.beta_dtype, row_off(a.beta, ci.b, ci.tok + min(l, ci.len - 1), h));
+      glen = ci.len;
+      graw = gate_prefetch(a, ci.b, ci.tok, ci.len, h);
+      braw = load_scalar_raw(a.beta.ptr, a.beta_dtype, row_off(a.beta, ci.b, ci.tok + min(l, ci.len - 1), h));
     };
     auto issue_qk = [&](int it) {
       it = min(it, nitems - 1);
       const int cid = it / a.H, h = it % a.H;
       const ChunkInfo ci = chunk_info(a, cid);
       Q.len = ci.len;
-      IOK::load_nomask(Q.rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
-      IOK::load_nomask(Q.rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
+      IOK::load_nomask(Q.rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len, tid);
+      IOK::load_nomask(Q.rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len, tid);
     };
     // the slice after slice s of item it
     auto issue_next = [&](int it, int s) {
@@ -145,35 +154,40 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
       for (int p = 0; p < IOH::PASSES; ++p)
 #pragma unroll
         for (int i = 0; i < IOH::VEC; ++i) hdh += ET<T>::to_f(S.rh.v[p][i]) * ET<T>::to_f(S.rdh.v[p][i]);
-      IOV::mask(S.rd, S.len);
-      IOV::mask(S.rvn, S.len);
-      IOV::mask(S.rdv, S.len);
-      IOV::mask(S.rvv, S.len);
-      IOV::store_lds(S.rd, base + A_DO, LDV);
-      IOV::store_lds(S.rvn, base + A_VN, LDV);
-      IOV::store_lds(S.rdv, base + A_DVN, LDV);
-      IOV::store_lds(S.rvv, base + A_VV, LDV);
-      IOH::store_lds(S.rh, base + A_H, LDK);
-      IOH::store_lds(S.rdh, base + A_DH, LDK);
+      IOV::mask(S.rd, S.len, tid);
+      IOV::mask(S.rvn, S.len, tid);
+      IOV::mask(S.rdv, S.len, tid);
+      IOV::mask(S.rvv, S.len, tid);
+      IOV::store_lds(S.rd, base + A_DO, LDV, tid);
+      IOV::store_lds(S.rvn, base + A_VN, LDV, tid);
+      IOV::store_lds(S.rdv, base + A_DVN, LDV, tid);
+      IOV::store_lds(S.rvv, base + A_VV, LDV, tid);
+      IOH::store_lds(S.rh, base + A_H, LDK, tid);
+      IOH::store_lds(S.rdh, base + A_DH, LDK, tid);
     };
-    // Tinv, gate cumsum and beta of the item (single copies: only between E and R(0))
-    auto stage_item = [&]() {
-      IO64::store_lds(I.rt, s_ti, LDC);
-      gate_finish_wave(a, I.graw, I.len, l, wave_id() == 4, s_b, s_eb, s_ed);
-      if (wave_id() == 5) s_beta[l] = l < I.len ? scalar_from_raw(I.braw, a.beta_dtype) : 0.f;
+    // gate cumsum and beta of the item (single copies: only between E and R(0))
+    auto stage_gates = [&]() {
+      gate_finish_wave(a, graw, glen, l, lw == 0, s_b, s_eb, s_ed);
+      if (lw == 1) s_beta[l] = l < glen ? scalar_from_raw(braw, a.beta_dtype) : 0.f;
     };
     const int it0 = blockIdx.x;
-    issue_item(it0);
+    issue_tinv(it0);
+    issue_gates(it0);
     issue_slice(it0, 0);
     issue_qk(it0);
     // the first loads may be ordered freely by the compiler; were they still pending at the loop
     // header, its wait-count analysis would carry that order into every iteration
     wait_all_loads();
+    IO64::store_lds(rt, s_ti, LDC, tid);
+    issue_tinv(it0 + stride);
     stage_slice(0);
     issue_next(it0, 0);
     for (int it = it0; it < nitems; it += stride) {
-      stage_item();
-      issue_item(it + stride);
+      tid = fresh_index(tid);
+      const int cid = it / a.H, h = it % a.H;
+      const ChunkInfo ci = chunk_info(a, cid);
+      stage_gates();
+      issue_gates(it + stride);
 #pragma unroll
       for (int s = 0; s < NS; ++s) {
         lds_barrier();                                                                   // R(s)
@@ -184,6 +198,11 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
           }
         }
         lds_barrier();                                                                   // D(s)
+        {
+          typename IOV::Regs r;            // dv of the slice
+          IOV::load_lds(r, s_dv, LDV, tid);
+          IOV::store_global(r, row_ptr<T>(a.dv, ci.b, ci.tok, h) + s * BVH, a.dv.st, ci.len, tid);
+        }
         if constexpr (NBUF == 1) {
           if (s + 1 < NS) {
             stage_slice(0);
@@ -191,12 +210,12 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
           }
         }
       }
-      IOK::mask(Q.rq, Q.len);
-      IOK::mask(Q.rk, Q.len);
-      IOK::store_lds(Q.rq, smem + B_Q, LDK);
-      IOK::store_lds(Q.rk, smem + B_K, LDK);
+      IOK::mask(Q.rq, Q.len, tid);
+      IOK::mask(Q.rk, Q.len, tid);
+      IOK::store_lds(Q.rq, smem + B_Q, LDK, tid);
+      IOK::store_lds(Q.rk, smem + B_K, LDK, tid);
       hdh = wave_sum(hdh);
-      if (l == 0) s_red[wave_id() - 4] = hdh;
+      if (l == 0) s_red[lw] = hdh;
       hdh = 0.f;
       lds_barrier();                                                                     // A
       issue_qk(it + stride);
@@ -204,8 +223,26 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
         stage_slice(0);                    // slice 0 of the next item (buffer 0 is idle in stage 2)
         issue_next(it + stride, 0);
       }
-#pragma unroll
-      for (int i = 0; i < 8; ++i) lds_barrier();                                         // b .. h, E
+      lds_barrier();                                                                     // b
+      lds_barrier();                                                                     // c
+      lds_barrier();                                                                     // d: dq lies in the q tile
+      {
+        typename IOK::Regs r;
+        IOK::load_lds(r, smem + B_Q, LDK, tid);
+        IOK::store_global(r, row_ptr<T>(a.dq, ci.b, ci.tok, h), a.dq.st, ci.len, tid);
+      }
+      lds_barrier();                                                                     // e
+      lds_barrier();                                                                     // f: Tinv of this item is dead
+      IO64::store_lds(rt, s_ti, LDC, tid);
+      issue_tinv(it + 2 * stride);
+      lds_barrier();                                                                     // g
+      lds_barrier();                                                                     // h: dk lies in the q tile
+      {
+        typename IOK::Regs r;
+        IOK::load_lds(r, smem + B_Q, LDK, tid);
+        IOK::store_global(r, row_ptr<T>(a.dk, ci.b, ci.tok, h), a.dk.st, ci.len, tid);
+      }
+      lds_barrier();                                                                     // E
       if constexpr (NBUF == 1) {
         stage_slice(0);
         issue_next(it + stride, 0);
@@ -216,18 +253,20 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
 
   // --------------------------------- compute ---------------------------------------------
   const int wv = wave_id();
-  const int r0 = 16 * wv;
+  const int r0 = 16 * (wv & 3);            // rows of this wave
+  const int ch = wv >> 2;                  // column half
+  const int c0 = 32 * ch;                  // first column in a chunk x chunk product
+  const int k0 = KH * ch;                  // first column in a K-wide product
   const float scale = a.scale;
   for (int it = blockIdx.x; it < nitems; it += stride) {
     // the lane index is refreshed per item: address arithmetic derived from it then stays inside
     // the iteration instead of living in registers for the whole kernel
     const int l = fresh_index(lane_id());
     const int fr = l & 15, fg = 8 * (l >> 4);
-    const int cid = it / a.H, h = it % a.H;
-    const ChunkInfo ci = chunk_info(a, cid);
-    f32x4 dP[1][4], dTv[1][4], dqi[1][NBK], dkd[1][NBK], dw[1][NBK];
+    const int rb = r0 + 4 * (l >> 4);      // accumulator element i is row rb + i, column (tile) + fr
+    f32x4 dP[1][2], dTv[1][2], dqi[1][NBK], dkd[1][NBK], dw[1][NBK];
     acc_zero(dP); acc_zero(dTv); acc_zero(dqi); acc_zero(dkd); acc_zero(dw);
-    float dbt[4] = {0.f, 0.f, 0.f, 0.f};      // dbeta of rows r0 + 4 (l/16) + i (partial over lanes)
+    float dbt[4] = {0.f, 0.f, 0.f, 0.f};      // dbeta of rows rb + i (partial over lanes and column halves)
     // ---- stage 1 ----
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
@@ -241,34 +280,28 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
         const typename ET<T>::frag aVN = ET<T>::load_frag(VN + (r0 + fr) * LDV + kk + fg);
         const typename ET<T>::frag aDVN = ET<T>::load_frag(DVN + (r0 + fr) * LDV + kk + fg);
 #pragma unroll
-        for (int nj = 0; nj < 4; ++nj) {
-          ET<T>::mma(dP[0][nj], aDO, ET<T>::load_frag(VN + (16 * nj + fr) * LDV + kk + fg));
-          ET<T>::mma(dTv[0][nj], aDVN, ET<T>::load_frag(VV + (16 * nj + fr) * LDV + kk + fg));
+        for (int nj = 0; nj < 2; ++nj) {
+          ET<T>::mma(dP[0][nj], aDO, ET<T>::load_frag(VN + (c0 + 16 * nj + fr) * LDV + kk + fg));
+          ET<T>::mma(dTv[0][nj], aDVN, ET<T>::load_frag(VV + (c0 + 16 * nj + fr) * LDV + kk + fg));
         }
-        __builtin_amdgcn_sched_barrier(0);      // bounds the fragments in flight (register budget)
 #pragma unroll
         for (int ni = 0; ni < NBK; ++ni) {
-          const typename ET<T>::frag bH = ET<T>::load_frag_t(HT, LDK, kk, 16 * ni, l);
+          const typename ET<T>::frag bH = ET<T>::load_frag_t(HT, LDK, kk, k0 + 16 * ni, l);
           ET<T>::mma(dqi[0][ni], aDO, bH);
           ET<T>::mma(dw[0][ni], aDVN, bH);
-          ET<T>::mma(dkd[0][ni], aVN, ET<T>::load_frag_t(DHT, LDK, kk, 16 * ni, l));
-          if (ni % 4 == 3) __builtin_amdgcn_sched_barrier(0);
+          ET<T>::mma(dkd[0][ni], aVN, ET<T>::load_frag_t(DHT, LDK, kk, k0 + 16 * ni, l));
         }
       }
-      // dv_b = Tinv^T du for this slice
-      f32x4 dvb[1][NBH];
+      // dv_b = Tinv^T du for this slice: rows r0.., columns 16 ch .. + 15 of the slice
+      f32x4 dvb[1][1];
       acc_zero(dvb);
-      gemm_bounded<T, 1, NBH, true, true>(dvb, s_ti, LDC, r0, DVN, LDV, 0, 0, CH, l);
+      gemm<T, 1, 1, true, true>(dvb, s_ti, LDC, r0, DVN, LDV, 16 * ch, 0, CH, l);
 #pragma unroll
-      for (int ni = 0; ni < NBH; ++ni)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int r = r0 + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
-          dbt[i] += dvb[0][ni][i] * ET<T>::to_f(VV[r * LDV + cc]);
-          dvb[0][ni][i] *= s_beta[r];                                                    // final dv
-        }
-      store_strip<T, NBH>(dvb, s_stg + wv * 16 * LDV, row_ptr<T>(a.dv, ci.b, ci.tok + r0, h) + s * BVH, a.dv.st,
-                          ci.len - r0, 1.0f, l);
+      for (int i = 0; i < 4; ++i) {
+        dbt[i] += dvb[0][0][i] * ET<T>::to_f(VV[(rb + i) * LDV + 16 * ch + fr]);
+        dvb[0][0][i] *= s_beta[rb + i];                                                  // final dv
+      }
+      acc_to_lds<T>(dvb[0][0], s_dv, LDV, r0, 16 * ch, l);
       pin(dbt);
       __builtin_amdgcn_sched_barrier(0);
       lds_barrier();                                                                     // D(s)
@@ -277,48 +310,46 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
     // ---- stage 2 ----
     T* Qt = smem + B_Q; T* Kt = smem + B_K; T* T0 = smem + B_T0; T* T1 = smem + B_T1; T* DW = smem + B_DW;
 #pragma unroll
-    for (int nj = 0; nj < 4; ++nj) {
+    for (int nj = 0; nj < 2; ++nj) {
       f32x4 p;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int r = r0 + 4 * (l >> 4) + i, cc = 16 * nj + (l & 15);
+        const int r = rb + i, cc = c0 + 16 * nj + fr;
         p[i] = (r >= cc) ? scale * dP[0][nj][i] * texp<T>(s_b[r] - s_b[cc]) : 0.f;
       }
-      acc_to_lds_t<T>(p, T0, LDC, r0, 16 * nj, l);                                          // G^T [j][i]
+      acc_to_lds_t<T>(p, T0, LDC, r0, c0 + 16 * nj, l);                                  // G^T [j][i]
     }
 #pragma unroll
     for (int ni = 0; ni < NBK; ++ni) {
       f32x4 x;
 #pragma unroll
       for (int i = 0; i < 4; ++i) x[i] = -dw[0][ni][i];                                  // dw = -du S^T
-      acc_to_lds<T>(x, DW, LDK, r0, 16 * ni, l);
+      acc_to_lds<T>(x, DW, LDK, r0, k0 + 16 * ni, l);
     }
     lds_barrier();                                                                       // b
     float dbp[4] = {0.f, 0.f, 0.f, 0.f};
     float kk = 0.f;
-    f32x4 dq[1][NBK], dk[1][NBK], dkbg[1][NBK], dT[1][4];
+    f32x4 dq[1][NBK], dk[1][NBK], dkbg[1][NBK], dT[1][2];
     acc_zero(dq);
-    gemm_bounded<T, 1, NBK, true, true>(dq, T0, LDC, r0, Kt, LDK, 0, 0, CH, l);                     // G k
+    gemm_bounded<T, 1, NBK, true, true>(dq, T0, LDC, r0, Kt, LDK, k0, 0, CH, l);         // G k
 #pragma unroll
     for (int ni = 0; ni < NBK; ++ni)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int r = r0 + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
+        const int r = rb + i, cc = k0 + 16 * ni + fr;
         const float dqv = scale * s_eb[r] * dqi[0][ni][i] + dq[0][ni][i];
         dbp[i] += ET<T>::to_f(Qt[r * LDK + cc]) * dqv;
         dq[0][ni][i] = dqv;                                                              // final dq
       }
     pin(dbp);
-    if constexpr (EARLY_DQ)
-      store_strip<T, NBK>(dq, s_stg + wv * 16 * LDK, row_ptr<T>(a.dq, ci.b, ci.tok + r0, h), a.dq.st, ci.len - r0, 1.0f, l);
     __builtin_amdgcn_sched_barrier(0);
     acc_zero(dk);
-    gemm_bounded<T, 1, NBK, false, true>(dk, T0, LDC, r0, Qt, LDK, 0, 0, CH, l);                    // G^T q
+    gemm_bounded<T, 1, NBK, false, true>(dk, T0, LDC, r0, Qt, LDK, k0, 0, CH, l);        // G^T q
 #pragma unroll
     for (int ni = 0; ni < NBK; ++ni)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int r = r0 + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
+        const int r = rb + i, cc = k0 + 16 * ni + fr;
         const float kv = ET<T>::to_f(Kt[r * LDK + cc]);
         const float dkdv = s_ed[r] * dkd[0][ni][i];
         const float dkv = dkdv + dk[0][ni][i];
@@ -330,12 +361,12 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
     pin(kk);
     __builtin_amdgcn_sched_barrier(0);
     {
-      f32x4 t2[1][4];
+      f32x4 t2[1][2];
       acc_zero(t2);
-      gemm_bounded<T, 1, 4, false, false>(t2, DW, LDK, r0, Kt, LDK, 0, 0, K, l);                    // dw k^T
+      gemm_bounded<T, 1, 2, false, false>(t2, DW, LDK, r0, Kt, LDK, c0, 0, K, l);        // dw k^T
 #pragma unroll
-      for (int nj = 0; nj < 4; ++nj) {
-        const int cc = 16 * nj + (l & 15);
+      for (int nj = 0; nj < 2; ++nj) {
+        const int cc = c0 + 16 * nj + fr;
         const float bj = s_beta[cc], bej = bj * s_eb[cc];
 #pragma unroll
         for (int i = 0; i < 4; ++i) dT[0][nj][i] = dTv[0][nj][i] * bj + t2[0][nj][i] * bej;
@@ -343,53 +374,55 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
     }
     __builtin_amdgcn_sched_barrier(0);
     acc_zero(dkbg);
-    gemm_bounded<T, 1, NBK, true, true>(dkbg, s_ti, LDC, r0, DW, LDK, 0, 0, CH, l);                 // Tinv^T dw
-    lds_barrier();                                                                       // c: G^T, DW read
+    gemm_bounded<T, 1, NBK, true, true>(dkbg, s_ti, LDC, r0, DW, LDK, k0, 0, CH, l);     // Tinv^T dw
+    lds_barrier();                                                                       // c: G^T, DW, q read
 #pragma unroll
-    for (int nj = 0; nj < 4; ++nj) acc_to_lds_t<T>(dT[0][nj], T0, LDC, r0, 16 * nj, l);     // dT^T [n][i]
+    for (int nj = 0; nj < 2; ++nj) acc_to_lds_t<T>(dT[0][nj], T0, LDC, r0, c0 + 16 * nj, l);   // dT^T [n][i]
+#pragma unroll
+    for (int ni = 0; ni < NBK; ++ni) acc_to_lds<T>(dq[0][ni], Qt, LDK, r0, k0 + 16 * ni, l);   // dq on its way out
     lds_barrier();                                                                       // d
     {
       // X1[j][n] = sum_i Tinv[i][j] dT[i][n]
-      f32x4 x1[1][4];
+      f32x4 x1[1][2];
       acc_zero(x1);
-      gemm_bounded<T, 1, 4, true, false>(x1, s_ti, LDC, r0, T0, LDC, 0, 0, CH, l);
+      gemm_bounded<T, 1, 2, true, false>(x1, s_ti, LDC, r0, T0, LDC, c0, 0, CH, l);
 #pragma unroll
-      for (int nj = 0; nj < 4; ++nj) acc_to_lds_t<T>(x1[0][nj], T1, LDC, r0, 16 * nj, l);   // X1^T [n][j]
+      for (int nj = 0; nj < 2; ++nj) acc_to_lds_t<T>(x1[0][nj], T1, LDC, r0, c0 + 16 * nj, l);   // X1^T [n][j]
     }
     lds_barrier();                                                                       // e
     {
-      f32x4 dL[1][4];
+      f32x4 dL[1][2];
       acc_zero(dL);
       // dL[j][m] = - sum_n X1[j][n] Tinv[m][n]
-      gemm_bounded<T, 1, 4, true, false>(dL, T1, LDC, r0, s_ti, LDC, 0, 0, CH, l);
-      lds_barrier();                                                                     // f: X1^T, dT^T read
+      gemm_bounded<T, 1, 2, true, false>(dL, T1, LDC, r0, s_ti, LDC, c0, 0, CH, l);
+      lds_barrier();                                                                     // f: X1^T, dT^T, Tinv read
 #pragma unroll
-      for (int nj = 0; nj < 4; ++nj) {
+      for (int nj = 0; nj < 2; ++nj) {
         f32x4 p, pb;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int r = r0 + 4 * (l >> 4) + i, cc = 16 * nj + (l & 15);
+          const int r = rb + i, cc = c0 + 16 * nj + fr;
           p[i] = (r > cc) ? -dL[0][nj][i] * texp<T>(s_b[r] - s_b[cc]) : 0.f;
           pb[i] = p[i] * s_beta[r];
         }
-        acc_to_lds_t<T>(p, T1, LDC, r0, 16 * nj, l);                                        // dM^T  [j][i]
-        acc_to_lds_t<T>(pb, T0, LDC, r0, 16 * nj, l);                                       // (diag(beta) dM)^T [j][i]
+        acc_to_lds_t<T>(p, T1, LDC, r0, c0 + 16 * nj, l);                                // dM^T  [j][i]
+        acc_to_lds_t<T>(pb, T0, LDC, r0, c0 + 16 * nj, l);                               // (diag(beta) dM)^T [j][i]
       }
     }
     lds_barrier();                                                                       // g
     {
       // dM k first: it closes dk_b (dbeta, the k_b.(dM k) term); then dM^T k_b
       // (k is re-read from LDS through an offset the compiler cannot see through: it would otherwise
-      // keep the 32 values read for the first part of dk in registers across phases c .. g)
+      // keep the values read for the first part of dk in registers across phases c .. g)
       const T* Kr = Kt + fresh_index(0);
       f32x4 m[1][NBK];
       acc_zero(m);
-      gemm_bounded<T, 1, NBK, true, true>(m, T1, LDC, r0, Kt, LDK, 0, 0, CH, l);
+      gemm_bounded<T, 1, NBK, true, true>(m, T1, LDC, r0, Kt, LDK, k0, 0, CH, l);
 #pragma unroll
       for (int ni = 0; ni < NBK; ++ni)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int r = r0 + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
+          const int r = rb + i, cc = k0 + 16 * ni + fr;
           const float kv = ET<T>::to_f(Kr[r * LDK + cc]);
           const float bt = s_beta[r], eb = s_eb[r];
           const float kbv = kv * bt;
@@ -403,15 +436,17 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
       __builtin_amdgcn_sched_barrier(0);
       const T* Kr2 = Kt + fresh_index(0);
       acc_zero(m);
-      gemm_bounded<T, 1, NBK, false, true>(m, T0, LDC, r0, Kt, LDK, 0, 0, CH, l);
+      gemm_bounded<T, 1, NBK, false, true>(m, T0, LDC, r0, Kt, LDK, k0, 0, CH, l);
 #pragma unroll
-      for (int ni = 0; ni < NBK; ++ni)
+      for (int ni = 0; ni < NBK; ++ni) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int r = r0 + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
+          const int r = rb + i, cc = k0 + 16 * ni + fr;
           dbp[i] -= ET<T>::to_f(Kr2[r * LDK + cc]) * m[0][ni][i];
           dk[0][ni][i] += m[0][ni][i];                                                   // final dk
         }
+        acc_to_lds<T>(dk[0][ni], Qt, LDK, r0, k0 + 16 * ni, l);                          // dk on its way out
+      }
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -421,34 +456,39 @@ __global__ __launch_bounds__(2 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
         dbt[i] += __shfl_xor(dbt[i], d, 64);
       }
     }
-    if ((l & 15) == 0) {
+    if (fr == 0) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        s_db[r0 + 4 * (l >> 4) + i] = dbp[i];
-        s_dbeta[r0 + 4 * (l >> 4) + i] = dbt[i];
+        s_db[ch][rb + i] = dbp[i];
+        s_dbeta[ch][rb + i] = dbt[i];
       }
     }
     kk = wave_sum(kk);
     if (l == 0) s_red[4 + wv] = kk;
-    lds_barrier();           // h: q, k tiles are dead: wave-private slices of them stage the stores
-    if constexpr (!EARLY_DQ)
-      store_strip<T, NBK>(dq, Kt + wv * 16 * LDK, row_ptr<T>(a.dq, ci.b, ci.tok + r0, h), a.dq.st, ci.len - r0, 1.0f, l);
-    store_strip<T, NBK>(dk, Qt + wv * 16 * LDK, row_ptr<T>(a.dk, ci.b, ci.tok + r0, h), a.dk.st, ci.len - r0, 1.0f, l);
+    lds_barrier();                                                                       // h
     if (threadIdx.x < 64) {
+      const int cid = it / a.H, h = it % a.H;
+      const ChunkInfo ci = chunk_info(a, cid);
       const int j = threadIdx.x;
       float x = 0.f;
       if (j < ci.len) {
-        ((float*)a.dbeta.ptr)[row_off(a.dbeta, ci.b, ci.tok + j, h)] = s_dbeta[j];
-        x = s_db[j];
+        ((float*)a.dbeta.ptr)[row_off(a.dbeta, ci.b, ci.tok + j, h)] = s_dbeta[0][j] + s_dbeta[1][j];
+        x = s_db[0][j] + s_db[1][j];
         // last-row term; rows past the end of a partial chunk carry zero q, k, so the term may sit
         // on the last valid row without changing the reverse cumulative sum
-        if (j == ci.len - 1)
-          x += s_red[4] + s_red[5] + s_red[6] + s_red[7] + expf(s_b[CH - 1]) * (s_red[0] + s_red[1] + s_red[2] + s_red[3]);
+        if (j == ci.len - 1) {
+          float skk = 0.f, shd = 0.f;
+#pragma unroll
+          for (int w = 0; w < 8; ++w) skk += s_red[4 + w];
+#pragma unroll
+          for (int w = 0; w < 4; ++w) shd += s_red[w];
+          x += skk + expf(s_b[CH - 1]) * shd;
+        }
       }
       x = wave_rev_scan(x);
       if (j < ci.len) ((float*)a.dg.ptr)[row_off(a.dg, ci.b, ci.tok + j, h)] = x;
     }
-    lds_barrier();           // E: the stage 2 region, Tinv and the gate arrays go to the next item
+    lds_barrier();           // E: the stage 2 region and the gate arrays go to the next item
   }
 }
 
