@@ -60,6 +60,16 @@ __device__ __forceinline__ void gemm_bounded(f32x4 (&acc)[MB][NB], const T* A, i
   }
 }
 
+// compile-time loop: f(IC<0>()), .., f(IC<N - 1>())
+template <int I> struct IC { static constexpr int value = I; };
+template <int N, int I = 0, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(IC<I>());
+    static_for<N, I + 1>(f);
+  }
+}
+
 // Forces x to be computed here: without it the compiler moves a running sum's updates down to
 // the sum's first use, and keeps every operand alive (spilled) until then.
 __device__ __forceinline__ void pin(float& x) { asm volatile("" : "+v"(x)); }
@@ -68,7 +78,7 @@ __device__ __forceinline__ void pin(float (&x)[4]) {
   for (int i = 0; i < 4; ++i) pin(x[i]);
 }
 
-template <typename T, int K, int V, int BVH, int NBUF>
+template <typename T, int K, int V, int BVH, int NBUF, int DEPTH>
 __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
   typedef GdnBwdChunkLds<T, K, BVH, NBUF> L;
   constexpr int LDV = L::LDV, LDC = L::LDC, LDK = L::LDK;
@@ -102,68 +112,106 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
     // where they are used instead of held (and spilled) for the whole kernel
     int tid = threadIdx.x & (NTHR - 1);
     const int lw = wave_id() - 8;            // wave of the loader team
-    struct SliceRegs { typename IOV::Regs rd, rvn, rdv, rvv; typename IOH::Regs rh, rdh; int len; };
-    struct QKRegs { typename IOK::Regs rq, rk; int len; };
-    SliceRegs S;
-    QKRegs Q;
+    // The bulk input of an item is a sequence of NU units: the NS slices, then q, then k.  Units go
+    // through DEPTH register sets in rotation (unit u uses set u % DEPTH; NU is a multiple of DEPTH):
+    // staging unit u into LDS frees its set for unit u + DEPTH, so DEPTH - 1 .. DEPTH units are in
+    // flight at any time.  Every load is issued unconditionally (item index clamped to the last item):
+    // a load that is skipped on some path would make the compiler drain all outstanding loads at
+    // every use.
+    constexpr int NU = NS + 2;
+    constexpr int PV = IOV::PASSES, PH = IOH::PASSES, PK = IOK::PASSES;
+    constexpr int NVEC = (4 * PV + 2 * PH) > PK ? (4 * PV + 2 * PH) : PK;
+    static_assert(NU % DEPTH == 0, "units per item and register sets");
+    typedef typename ET<T>::vec vec;
+    struct Unit { vec v[NVEC]; int len; };
+    Unit U[DEPTH];
     typename IO64::Regs rt;
     uint32_t graw, braw;
     int glen;
-    // Every prefetch is issued unconditionally (item index clamped to the last item): a load that
-    // is skipped on some path would make the compiler drain all outstanding loads at every use.
-    auto issue_slice = [&](int it, int vv) {
-      it = min(it, nitems - 1);
+    float hdh = 0.f;   // partial <S, dS'> of the item whose slices are being staged
+    // unit u counted from the first unit of item it (u >= NU: units of the item after it)
+    auto issue = [&](auto uc, int it) {
+      constexpr int u = decltype(uc)::value, unit = u % NU;
+      Unit& R = U[u % DEPTH];
+      it = __builtin_amdgcn_readfirstlane(min(it + (u / NU) * stride, nitems - 1));
       const int cid = it / a.H, h = it % a.H;
       const ChunkInfo ci = chunk_info(a, cid);
-      S.len = ci.len;
-      IOV::load_nomask(S.rd, row_ptr<T>(a.d_o, ci.b, ci.tok, h) + vv, a.d_o.st, ci.len, tid);
-      IOV::load_nomask(S.rvn, row_ptr<T>(a.vnew, ci.b, ci.tok, h) + vv, a.vnew.st, ci.len, tid);
-      IOV::load_nomask(S.rdv, row_ptr<T>(a.dvnew, ci.b, ci.tok, h) + vv, a.dvnew.st, ci.len, tid);
-      IOV::load_nomask(S.rvv, row_ptr<T>(a.v, ci.b, ci.tok, h) + vv, a.v.st, ci.len, tid);
-      IOH::load_nomask(S.rh, (const T*)a.hs + (((int64_t)cid * a.H + h) * V + vv) * K, K, BVH, tid);
-      IOH::load_nomask(S.rdh, (const T*)a.dhs + (((int64_t)cid * a.H + h) * V + vv) * K, K, BVH, tid);
+      R.len = ci.len;
+      if constexpr (unit < NS) {
+        constexpr int vv = unit * BVH;
+        const lmoe_tensor* ts[4] = {&a.d_o, &a.vnew, &a.dvnew, &a.v};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          typename IOV::Regs r;
+          IOV::load_nomask(r, row_ptr<T>(*ts[t], ci.b, ci.tok, h) + vv, ts[t]->st, ci.len, tid);
+#pragma unroll
+          for (int p = 0; p < PV; ++p) R.v[t * PV + p] = r.v[p];
+        }
+        const T* hp[2] = {(const T*)a.hs, (const T*)a.dhs};
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          typename IOH::Regs r;
+          IOH::load_nomask(r, hp[t] + ((int64_t)it * V + vv) * K, K, BVH, tid);         // it = cid * H + h
+#pragma unroll
+          for (int p = 0; p < PH; ++p) R.v[4 * PV + t * PH + p] = r.v[p];
+        }
+      } else {
+        const lmoe_tensor& x = unit == NS ? a.q : a.k;
+        typename IOK::Regs r;
+        IOK::load_nomask(r, row_ptr<T>(x, ci.b, ci.tok, h), x.st, ci.len, tid);
+#pragma unroll
+        for (int p = 0; p < PK; ++p) R.v[p] = r.v[p];
+      }
+    };
+    // unit u (u == NU: slice 0 of the next item) from its registers into LDS; slices go to buffer buf
+    auto stage = [&](auto uc, int buf) {
+      constexpr int u = decltype(uc)::value, unit = u % NU;
+      Unit& R = U[u % DEPTH];
+      if constexpr (unit < NS) {
+        T* base = smem + buf * A_END;
+        constexpr int off[4] = {A_DO, A_VN, A_DVN, A_VV};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          typename IOV::Regs r;
+#pragma unroll
+          for (int p = 0; p < PV; ++p) r.v[p] = R.v[t * PV + p];
+          IOV::mask(r, R.len, tid);
+          IOV::store_lds(r, base + off[t], LDV, tid);
+        }
+        typename IOH::Regs rh, rdh;
+#pragma unroll
+        for (int p = 0; p < PH; ++p) { rh.v[p] = R.v[4 * PV + p]; rdh.v[p] = R.v[4 * PV + PH + p]; }
+#pragma unroll
+        for (int p = 0; p < PH; ++p)
+#pragma unroll
+          for (int i = 0; i < IOH::VEC; ++i) hdh += ET<T>::to_f(rh.v[p][i]) * ET<T>::to_f(rdh.v[p][i]);
+        IOH::store_lds(rh, base + A_H, LDK, tid);
+        IOH::store_lds(rdh, base + A_DH, LDK, tid);
+      } else {
+        typename IOK::Regs r;
+#pragma unroll
+        for (int p = 0; p < PK; ++p) r.v[p] = R.v[p];
+        IOK::mask(r, R.len, tid);
+        IOK::store_lds(r, smem + (unit == NS ? B_Q : B_K), LDK, tid);
+      }
+    };
+    // stage unit u of item it, then request the unit that takes over its registers
+    auto advance = [&](auto uc, int it, int buf) {
+      constexpr int u = decltype(uc)::value;
+      stage(uc, buf);
+      issue(IC<u + DEPTH>(), it);
     };
     auto issue_tinv = [&](int it) {
       it = min(it, nitems - 1);
       IO64::load_nomask(rt, (const T*)a.tinv + (int64_t)it * CH * CH, CH, CH, tid);     // it = cid * H + h
     };
     auto issue_gates = [&](int it) {
-      it = min(it, nitems - 1);
+      it = __builtin_amdgcn_readfirstlane(min(it, nitems - 1));
       const int cid = it / a.H, h = it % a.H;
       const ChunkInfo ci = chunk_info(a, cid);
       glen = ci.len;
       graw = gate_prefetch(a, ci.b, ci.tok, ci.len, h);
       braw = load_scalar_raw(a.beta.ptr, a.beta_dtype, row_off(a.beta, ci.b, ci.tok + min(l, ci.len - 1), h));
-    };
-    auto issue_qk = [&](int it) {
-      it = min(it, nitems - 1);
-      const int cid = it / a.H, h = it % a.H;
-      const ChunkInfo ci = chunk_info(a, cid);
-      Q.len = ci.len;
-      IOK::load_nomask(Q.rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len, tid);
-      IOK::load_nomask(Q.rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len, tid);
-    };
-    // the slice after slice s of item it
-    auto issue_next = [&](int it, int s) {
-      if (s + 1 < NS) issue_slice(it, (s + 1) * BVH); else issue_slice(it + stride, 0);
-    };
-    float hdh = 0.f;   // partial <S, dS'> of the item whose slices are being staged
-    auto stage_slice = [&](int buf) {
-      T* base = smem + buf * A_END;
-#pragma unroll
-      for (int p = 0; p < IOH::PASSES; ++p)
-#pragma unroll
-        for (int i = 0; i < IOH::VEC; ++i) hdh += ET<T>::to_f(S.rh.v[p][i]) * ET<T>::to_f(S.rdh.v[p][i]);
-      IOV::mask(S.rd, S.len, tid);
-      IOV::mask(S.rvn, S.len, tid);
-      IOV::mask(S.rdv, S.len, tid);
-      IOV::mask(S.rvv, S.len, tid);
-      IOV::store_lds(S.rd, base + A_DO, LDV, tid);
-      IOV::store_lds(S.rvn, base + A_VN, LDV, tid);
-      IOV::store_lds(S.rdv, base + A_DVN, LDV, tid);
-      IOV::store_lds(S.rvv, base + A_VV, LDV, tid);
-      IOH::store_lds(S.rh, base + A_H, LDK, tid);
-      IOH::store_lds(S.rdh, base + A_DH, LDK, tid);
     };
     // gate cumsum and beta of the item (single copies: only between E and R(0))
     auto stage_gates = [&]() {
@@ -173,57 +221,41 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
     const int it0 = blockIdx.x;
     issue_tinv(it0);
     issue_gates(it0);
-    issue_slice(it0, 0);
-    issue_qk(it0);
+    issue(IC<0>(), it0);
+    if constexpr (DEPTH == 2) issue(IC<1>(), it0);
     // the first loads may be ordered freely by the compiler; were they still pending at the loop
     // header, its wait-count analysis would carry that order into every iteration
     wait_all_loads();
     IO64::store_lds(rt, s_ti, LDC, tid);
-    issue_tinv(it0 + stride);
-    stage_slice(0);
-    issue_next(it0, 0);
+    advance(IC<0>(), it0, 0);
     for (int it = it0; it < nitems; it += stride) {
       tid = fresh_index(tid);
       const int cid = it / a.H, h = it % a.H;
       const ChunkInfo ci = chunk_info(a, cid);
       stage_gates();
       issue_gates(it + stride);
-#pragma unroll
-      for (int s = 0; s < NS; ++s) {
+      static_for<NS>([&](auto sc) {
+        constexpr int s = decltype(sc)::value;
         lds_barrier();                                                                   // R(s)
-        if constexpr (NBUF == 2) {
-          if (s + 1 < NS) {
-            stage_slice((s + 1) & 1);      // its buffer was left when the compute team passed D(s-1)
-            issue_next(it, s + 1);
-          }
-        }
+        if constexpr (NBUF == 2 && s + 1 < NS)
+          advance(IC<s + 1>(), it, (s + 1) & 1);   // its buffer was left when the compute team passed D(s-1)
         lds_barrier();                                                                   // D(s)
         {
           typename IOV::Regs r;            // dv of the slice
           IOV::load_lds(r, s_dv, LDV, tid);
           IOV::store_global(r, row_ptr<T>(a.dv, ci.b, ci.tok, h) + s * BVH, a.dv.st, ci.len, tid);
         }
-        if constexpr (NBUF == 1) {
-          if (s + 1 < NS) {
-            stage_slice(0);
-            issue_next(it, s + 1);
-          }
-        }
-      }
-      IOK::mask(Q.rq, Q.len, tid);
-      IOK::mask(Q.rk, Q.len, tid);
-      IOK::store_lds(Q.rq, smem + B_Q, LDK, tid);
-      IOK::store_lds(Q.rk, smem + B_K, LDK, tid);
+        if constexpr (NBUF == 1 && s + 1 < NS) advance(IC<s + 1>(), it, 0);
+      });
+      advance(IC<NS>(), it, 0);                                                          // q
+      advance(IC<NS + 1>(), it, 0);                                                      // k
       hdh = wave_sum(hdh);
       if (l == 0) s_red[lw] = hdh;
       hdh = 0.f;
       lds_barrier();                                                                     // A
-      issue_qk(it + stride);
-      if constexpr (NBUF == 2) {
-        stage_slice(0);                    // slice 0 of the next item (buffer 0 is idle in stage 2)
-        issue_next(it + stride, 0);
-      }
+      if constexpr (NBUF == 2) advance(IC<NU>(), it, 0);   // slice 0 of the next item (buffer 0 is idle in stage 2)
       lds_barrier();                                                                     // b
+      issue_tinv(it + stride);
       lds_barrier();                                                                     // c
       lds_barrier();                                                                     // d: dq lies in the q tile
       {
@@ -234,7 +266,6 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
       lds_barrier();                                                                     // e
       lds_barrier();                                                                     // f: Tinv of this item is dead
       IO64::store_lds(rt, s_ti, LDC, tid);
-      issue_tinv(it + 2 * stride);
       lds_barrier();                                                                     // g
       lds_barrier();                                                                     // h: dk lies in the q tile
       {
@@ -243,10 +274,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
         IOK::store_global(r, row_ptr<T>(a.dk, ci.b, ci.tok, h), a.dk.st, ci.len, tid);
       }
       lds_barrier();                                                                     // E
-      if constexpr (NBUF == 1) {
-        stage_slice(0);
-        issue_next(it + stride, 0);
-      }
+      if constexpr (NBUF == 1) advance(IC<NU>(), it, 0);
     }
     return;
   }
