@@ -427,6 +427,28 @@ template <typename T, int ROWS, int COLS> struct TileIO {
       if (row < ROWS && row < nvalid) *(vec*)(dst + (int64_t)row * row_stride + col) = r.v[p];
     }
   }
+  // Branch-free form of load_lds + store_global (nvalid >= 1): a thread whose row is >= nvalid reads
+  // and rewrites row nvalid - 1, i.e. stores the same bytes to the same address as the thread that
+  // owns that row.  No store sits behind a branch, so the compiler can count outstanding memory
+  // operations exactly and the caller's prefetches stay in flight across the stores.
+  static __device__ __forceinline__ void load_lds_clamped(Regs& r, const T* tile, int ld, int nvalid, int tid = threadIdx.x & (NTHR - 1)) {
+    const int last = (nvalid < ROWS ? nvalid : ROWS) - 1;
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      int row, col; coords(p, row, col, tid);
+      row = row < last ? row : last;
+      r.v[p] = *(const vec*)(tile + row * ld + col);
+    }
+  }
+  static __device__ __forceinline__ void store_global_clamped(const Regs& r, T* __restrict__ dst, int64_t row_stride, int nvalid, int tid = threadIdx.x & (NTHR - 1)) {
+    const int last = (nvalid < ROWS ? nvalid : ROWS) - 1;
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      int row, col; coords(p, row, col, tid);
+      row = row < last ? row : last;
+      *(vec*)(dst + (int64_t)row * row_stride + col) = r.v[p];
+    }
+  }
   // global[row][col] = tile[row][col]
   static __device__ __forceinline__ void lds_to_global(const T* tile, int ld, T* __restrict__ dst, int64_t row_stride, int nvalid) {
 #pragma unroll

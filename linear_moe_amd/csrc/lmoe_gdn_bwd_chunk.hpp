@@ -229,7 +229,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
     IO64::store_lds(rt, s_ti, LDC, tid);
     advance(IC<0>(), it0, 0);
     for (int it = it0; it < nitems; it += stride) {
-      tid = fresh_index(tid);
+      tid = fresh_index(tid) & (NTHR - 1);
       const int cid = it / a.H, h = it % a.H;
       const ChunkInfo ci = chunk_info(a, cid);
       stage_gates();
@@ -242,8 +242,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
         lds_barrier();                                                                   // D(s)
         {
           typename IOV::Regs r;            // dv of the slice
-          IOV::load_lds(r, s_dv, LDV, tid);
-          IOV::store_global(r, row_ptr<T>(a.dv, ci.b, ci.tok, h) + s * BVH, a.dv.st, ci.len, tid);
+          IOV::load_lds_clamped(r, s_dv, LDV, ci.len, tid);
+          IOV::store_global_clamped(r, row_ptr<T>(a.dv, ci.b, ci.tok, h) + s * BVH, a.dv.st, ci.len, tid);
         }
         if constexpr (NBUF == 1 && s + 1 < NS) advance(IC<s + 1>(), it, 0);
       });
@@ -260,8 +260,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
       lds_barrier();                                                                     // d: dq lies in the q tile
       {
         typename IOK::Regs r;
-        IOK::load_lds(r, smem + B_Q, LDK, tid);
-        IOK::store_global(r, row_ptr<T>(a.dq, ci.b, ci.tok, h), a.dq.st, ci.len, tid);
+        IOK::load_lds_clamped(r, smem + B_Q, LDK, ci.len, tid);
+        IOK::store_global_clamped(r, row_ptr<T>(a.dq, ci.b, ci.tok, h), a.dq.st, ci.len, tid);
       }
       lds_barrier();                                                                     // e
       lds_barrier();                                                                     // f: Tinv of this item is dead
@@ -270,8 +270,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
       lds_barrier();                                                                     // h: dk lies in the q tile
       {
         typename IOK::Regs r;
-        IOK::load_lds(r, smem + B_Q, LDK, tid);
-        IOK::store_global(r, row_ptr<T>(a.dk, ci.b, ci.tok, h), a.dk.st, ci.len, tid);
+        IOK::load_lds_clamped(r, smem + B_Q, LDK, ci.len, tid);
+        IOK::store_global_clamped(r, row_ptr<T>(a.dk, ci.b, ci.tok, h), a.dk.st, ci.len, tid);
       }
       lds_barrier();                                                                     // E
       if constexpr (NBUF == 1) advance(IC<NU>(), it, 0);

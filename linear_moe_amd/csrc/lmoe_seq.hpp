@@ -8,6 +8,12 @@
 
 namespace lmoe {
 
+// The index arrays of packed input (cu_seqlens, seq_chunk0, chunk_map) are read-only for every
+// kernel: reading them through the constant address space lets a uniform index become a scalar
+// load, which does not wait for (or drain) the vector loads a kernel keeps in flight.
+typedef const __attribute__((address_space(4))) int32_t* const_i32;
+__device__ __forceinline__ const_i32 as_const(const int32_t* p) { return (const_i32)(uintptr_t)p; }
+
 struct SeqInfo {
   int b;        // batch row holding the sequence
   int tok0;     // first token of the sequence inside that batch row
@@ -19,8 +25,9 @@ struct SeqInfo {
 __device__ __forceinline__ SeqInfo seq_info(const lmoe_args& a, int n) {
   SeqInfo s;
   if (a.cu_seqlens) {
-    s.b = 0; s.tok0 = a.cu_seqlens[n]; s.len = a.cu_seqlens[n + 1] - s.tok0;
-    s.chunk0 = a.seq_chunk0[n];
+    const const_i32 cu = as_const(a.cu_seqlens);
+    s.b = 0; s.tok0 = cu[n]; s.len = cu[n + 1] - s.tok0;
+    s.chunk0 = as_const(a.seq_chunk0)[n];
   } else {
     s.b = n; s.tok0 = 0; s.len = a.T;
     s.chunk0 = n * ((a.T + CH - 1) / CH);
@@ -41,10 +48,11 @@ __device__ __forceinline__ ChunkInfo chunk_info(const lmoe_args& a, int cid) {
   ChunkInfo c;
   int lc, slen;
   if (a.cu_seqlens) {
-    c.n = a.chunk_map[2 * cid]; lc = a.chunk_map[2 * cid + 1];
+    const const_i32 cm = as_const(a.chunk_map), cu = as_const(a.cu_seqlens);
+    c.n = cm[2 * cid]; lc = cm[2 * cid + 1];
     c.b = 0;
-    const int t0 = a.cu_seqlens[c.n];
-    slen = a.cu_seqlens[c.n + 1] - t0;
+    const int t0 = cu[c.n];
+    slen = cu[c.n + 1] - t0;
     c.tok = t0 + lc * CH;
   } else {
     const int nts = (a.T + CH - 1) / CH;
