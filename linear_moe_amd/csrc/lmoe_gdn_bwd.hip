@@ -7,7 +7,7 @@ namespace lmoe {
 template <typename T, int K, int V> struct GdnBwdChunk {
   static void run(const lmoe_args& a, hipStream_t st) {
     constexpr int BVH = 32;                            // V-slice of stage 1
-    constexpr int NBUF = sizeof(T) == 2 ? 2 : 1;       // slice buffers: two where LDS has the room
+    constexpr int NBUF = sizeof(T) == 2 ? 3 : 1;       // slice buffers: three where LDS has the room
     constexpr int DEPTH = sizeof(T) == 2 ? 2 : 1;      // register sets of the loaders' prefetch rotation
     static_assert(GdnBwdChunkLds<T, K, BVH, NBUF>::BYTES <= 160 * 1024, "LDS budget of k_gdn_bwd_chunk");
     const int grid = persistent_grid(a.NT * a.H, 1);

@@ -33,7 +33,10 @@
 //   while the previous one is consumed; the stage 2 tiles lie over the last buffer), and lift the
 //   results (dv per slice, dq, dk) out of LDS and store them.  They also form <S, dS'> from the
 //   registers they hold and the gate cumsum of the chunk.
-//   Script per item (NS slices):  R(0) D(0) .. R(NS-1) D(NS-1) | A | b c d e f g h | E
+//   Script per item (NS slices), three slice buffers:  D(0) .. D(NS-1) = A | b c d e f g h | E
+//     (slice s is staged two windows before the compute team reaches it; slices 0, 1 of the next item
+//     during f .. h of this one)
+//   one slice buffer:  [R(0)] D(0) R(1) D(1) .. D(NS-1) | A | b c d e f g h | E | R(0) of the next item
 #pragma once
 #include "lmoe_seq.hpp"
 
@@ -45,7 +48,8 @@ template <typename T, int K, int BVH, int NBUF> struct GdnBwdChunkLds {
   static constexpr int A_END = 4 * CH * LDV + 2 * BVH * LDK;
   static constexpr int B_END = 2 * CH * LDK + CH * LDC + CH * LDK;
   static constexpr int NREG = (NBUF - 1) * A_END + (A_END > B_END ? A_END : B_END);
-  static constexpr int BYTES = (NREG + CH * LDC + CH * LDV) * (int)sizeof(T) + (8 * 64 + 16) * 4;
+  static constexpr int NDV = NBUF == 3 ? 2 : 1;      // copies of the dv strip
+  static constexpr int BYTES = (NREG + CH * LDC + NDV * CH * LDV) * (int)sizeof(T) + (12 * 64 + 16) * 4;
 };
 
 // gemm with a scheduling fence after every 32-deep step: at most one step's fragments are in flight,
@@ -85,7 +89,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
   constexpr int NS = V / BVH;
   constexpr int KH = K / 2, NBK = KH / 16;     // columns / 16-wide tiles of a K-wide product per compute wave
   static_assert(V % BVH == 0 && BVH == 32, "V-slices: the 8 compute waves split a 64 x 32 slice product 4 x 2");
-  static_assert(NBUF == 1 || (NBUF == 2 && NS % 2 == 0), "with two buffers the last slice must sit in the second one");
+  static_assert(NBUF == 1 || NBUF == 3, "one slice buffer, or three in rotation");
   // tiles of one V-slice
   constexpr int A_DO = 0, A_VN = A_DO + CH * LDV, A_DVN = A_VN + CH * LDV, A_VV = A_DVN + CH * LDV,
                 A_H = A_VV + CH * LDV, A_DH = A_H + BVH * LDK, A_END = L::A_END;
@@ -95,8 +99,11 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
   constexpr int B_Q = SB, B_K = B_Q + CH * LDK, B_T0 = B_K + CH * LDK, B_DW = B_T0 + CH * LDC, B_T1 = B_DW;
   __shared__ __attribute__((aligned(16))) T smem[L::NREG];
   __shared__ __attribute__((aligned(16))) T s_ti[CH * LDC];              // Tinv, whole item
-  __shared__ __attribute__((aligned(16))) T s_dv[CH * LDV];              // dv of a slice on its way out
-  __shared__ float s_b[64], s_eb[64], s_ed[64], s_beta[64], s_db[2][64], s_dbeta[2][64], s_red[16];
+  // dv of a slice on its way out; with three slice buffers no barrier separates the loaders' read of
+  // slice s from the compute team's write of slice s + 1: two copies
+  __shared__ __attribute__((aligned(16))) T s_dv[L::NDV][CH * LDV];
+  // gate cumsum, its exponentials and beta: two copies, the loaders fill the next item's during stage 2
+  __shared__ float s_gb[2][64], s_geb[2][64], s_ged[2][64], s_gbeta[2][64], s_db[2][64], s_dbeta[2][64], s_red[16];
 
   typedef TileIO<T, CH, BVH> IOV;
   typedef TileIO<T, BVH, K> IOH;
@@ -213,10 +220,10 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
       graw = gate_prefetch(a, ci.b, ci.tok, ci.len, h);
       braw = load_scalar_raw(a.beta.ptr, a.beta_dtype, row_off(a.beta, ci.b, ci.tok + min(l, ci.len - 1), h));
     };
-    // gate cumsum and beta of the item (single copies: only between E and R(0))
-    auto stage_gates = [&]() {
-      gate_finish_wave(a, graw, glen, l, lw == 0, s_b, s_eb, s_ed);
-      if (lw == 1) s_beta[l] = l < glen ? scalar_from_raw(braw, a.beta_dtype) : 0.f;
+    // gate cumsum and beta of an item into copy par
+    auto stage_gates = [&](int par) {
+      gate_finish_wave(a, graw, glen, l, lw == 0, s_gb[par], s_geb[par], s_ged[par]);
+      if (lw == 1) s_gbeta[par][l] = l < glen ? scalar_from_raw(braw, a.beta_dtype) : 0.f;
     };
     const int it0 = blockIdx.x;
     issue_tinv(it0);
@@ -227,33 +234,54 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
     // header, its wait-count analysis would carry that order into every iteration
     wait_all_loads();
     IO64::store_lds(rt, s_ti, LDC, tid);
+    stage_gates(0);
+    issue_gates(it0 + stride);
     advance(IC<0>(), it0, 0);
+    if constexpr (NBUF == 3) advance(IC<1>(), it0, 1);
+    int par = 0;
+    auto store_dv = [&](const ChunkInfo& ci, int h, int s) {
+      typename IOV::Regs r;
+      IOV::load_lds_clamped(r, s_dv[s % L::NDV], LDV, ci.len, tid);
+      IOV::store_global_clamped(r, row_ptr<T>(a.dv, ci.b, ci.tok, h) + s * BVH, a.dv.st, ci.len, tid);
+    };
+    auto close_hdh = [&]() {
+      hdh = wave_sum(hdh);
+      if (l == 0) s_red[lw] = hdh;
+      hdh = 0.f;
+    };
+    lds_barrier();                                                                       // first slice staged
     for (int it = it0; it < nitems; it += stride) {
       tid = fresh_index(tid) & (NTHR - 1);
       const int cid = it / a.H, h = it % a.H;
       const ChunkInfo ci = chunk_info(a, cid);
-      stage_gates();
-      issue_gates(it + stride);
-      static_for<NS>([&](auto sc) {
-        constexpr int s = decltype(sc)::value;
-        lds_barrier();                                                                   // R(s)
-        if constexpr (NBUF == 2 && s + 1 < NS)
-          advance(IC<s + 1>(), it, (s + 1) & 1);   // its buffer was left when the compute team passed D(s-1)
-        lds_barrier();                                                                   // D(s)
-        {
-          typename IOV::Regs r;            // dv of the slice
-          IOV::load_lds_clamped(r, s_dv, LDV, ci.len, tid);
-          IOV::store_global_clamped(r, row_ptr<T>(a.dv, ci.b, ci.tok, h) + s * BVH, a.dv.st, ci.len, tid);
-        }
-        if constexpr (NBUF == 1 && s + 1 < NS) advance(IC<s + 1>(), it, 0);
-      });
-      advance(IC<NS>(), it, 0);                                                          // q
-      advance(IC<NS + 1>(), it, 0);                                                      // k
-      hdh = wave_sum(hdh);
-      if (l == 0) s_red[lw] = hdh;
-      hdh = 0.f;
-      lds_barrier();                                                                     // A
-      if constexpr (NBUF == 2) advance(IC<NU>(), it, 0);   // slice 0 of the next item (buffer 0 is idle in stage 2)
+      if constexpr (NBUF == 3) {
+        // window w: the compute team works on slice w.  Slice s lives in buffer s % 3 and is staged two
+        // windows ahead; q, k go to the third buffer's region in the last window.
+        static_for<NS>([&](auto wc) {
+          constexpr int w = decltype(wc)::value;
+          if constexpr (w >= 1) store_dv(ci, h, w - 1);
+          if constexpr (w + 2 < NS) advance(IC<w + 2>(), it, (w + 2) % 3);
+          if constexpr (w == NS - 1) {
+            advance(IC<NS>(), it, 0);                                                    // q
+            advance(IC<NS + 1>(), it, 0);                                                // k
+            close_hdh();
+          }
+          lds_barrier();                                                                 // D(w); the last one is A
+        });
+        store_dv(ci, h, NS - 1);
+      } else {
+        static_for<NS>([&](auto sc) {
+          constexpr int s = decltype(sc)::value;
+          if constexpr (s > 0) lds_barrier();                                            // R(s)
+          lds_barrier();                                                                 // D(s)
+          store_dv(ci, h, s);
+          if constexpr (s + 1 < NS) advance(IC<s + 1>(), it, 0);
+        });
+        advance(IC<NS>(), it, 0);                                                        // q
+        advance(IC<NS + 1>(), it, 0);                                                    // k
+        close_hdh();
+        lds_barrier();                                                                   // A
+      }
       lds_barrier();                                                                     // b
       issue_tinv(it + stride);
       lds_barrier();                                                                     // c
@@ -266,7 +294,11 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
       lds_barrier();                                                                     // e
       lds_barrier();                                                                     // f: Tinv of this item is dead
       IO64::store_lds(rt, s_ti, LDC, tid);
+      if constexpr (NBUF == 3) advance(IC<NU>(), it, 0);       // slice 0 of the next item
       lds_barrier();                                                                     // g
+      if constexpr (NBUF == 3) advance(IC<NU + 1>(), it, 1);   // slice 1 of the next item
+      stage_gates(par ^ 1);
+      issue_gates(it + 2 * stride);
       lds_barrier();                                                                     // h: dk lies in the q tile
       {
         typename IOK::Regs r;
@@ -274,7 +306,11 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
         IOK::store_global_clamped(r, row_ptr<T>(a.dk, ci.b, ci.tok, h), a.dk.st, ci.len, tid);
       }
       lds_barrier();                                                                     // E
-      if constexpr (NBUF == 1) advance(IC<NU>(), it, 0);
+      if constexpr (NBUF == 1) {
+        advance(IC<NU>(), it, 0);
+        lds_barrier();                                                                   // R(0) of the next item
+      }
+      par ^= 1;
     }
     return;
   }
@@ -286,7 +322,11 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
   const int c0 = 32 * ch;                  // first column in a chunk x chunk product
   const int k0 = KH * ch;                  // first column in a K-wide product
   const float scale = a.scale;
+  int par = 0;
+  lds_barrier();                                                                         // first slice staged
   for (int it = blockIdx.x; it < nitems; it += stride) {
+    const float* s_b = s_gb[par]; const float* s_eb = s_geb[par]; const float* s_ed = s_ged[par];
+    const float* s_beta = s_gbeta[par];
     // the lane index is refreshed per item: address arithmetic derived from it then stays inside
     // the iteration instead of living in registers for the whole kernel
     const int l = fresh_index(lane_id());
@@ -298,8 +338,10 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
     // ---- stage 1 ----
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
-      lds_barrier();                                                                     // R(s)
-      const T* base = smem + (NBUF == 2 ? (s & 1) * A_END : 0);
+      if constexpr (NBUF == 1) {
+        if (s > 0) lds_barrier();                                                        // R(s)
+      }
+      const T* base = smem + (NBUF == 3 ? (s % 3) * A_END : 0);
       const T* DO = base + A_DO; const T* VN = base + A_VN; const T* DVN = base + A_DVN;
       const T* VV = base + A_VV; const T* HT = base + A_H; const T* DHT = base + A_DH;
 #pragma unroll
@@ -329,12 +371,12 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
         dbt[i] += dvb[0][0][i] * ET<T>::to_f(VV[(rb + i) * LDV + 16 * ch + fr]);
         dvb[0][0][i] *= s_beta[rb + i];                                                  // final dv
       }
-      acc_to_lds<T>(dvb[0][0], s_dv, LDV, r0, 16 * ch, l);
+      acc_to_lds<T>(dvb[0][0], s_dv[s % L::NDV], LDV, r0, 16 * ch, l);
       pin(dbt);
       __builtin_amdgcn_sched_barrier(0);
-      lds_barrier();                                                                     // D(s)
+      lds_barrier();                                                                     // D(s); with three buffers the last one is A
     }
-    lds_barrier();                                                                       // A: q, k staged
+    if constexpr (NBUF == 1) lds_barrier();                                              // A: q, k staged
     // ---- stage 2 ----
     T* Qt = smem + B_Q; T* Kt = smem + B_K; T* T0 = smem + B_T0; T* T1 = smem + B_T1; T* DW = smem + B_DW;
 #pragma unroll
@@ -516,7 +558,9 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
       x = wave_rev_scan(x);
       if (j < ci.len) ((float*)a.dg.ptr)[row_off(a.dg, ci.b, ci.tok + j, h)] = x;
     }
-    lds_barrier();           // E: the stage 2 region and the gate arrays go to the next item
+    lds_barrier();           // E: the stage 2 region goes to the next item
+    if constexpr (NBUF == 1) lds_barrier();                                              // R(0) of the next item
+    par ^= 1;
   }
 }
 
