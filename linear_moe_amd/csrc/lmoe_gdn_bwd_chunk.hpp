@@ -284,6 +284,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
       }
       lds_barrier();                                                                     // b
       issue_tinv(it + stride);
+      stage_gates(par ^ 1);                                    // the next item's; its copy is idle since E of the last item
+      issue_gates(it + 2 * stride);
       lds_barrier();                                                                     // c
       lds_barrier();                                                                     // d: dq lies in the q tile
       {
@@ -297,8 +299,6 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
       if constexpr (NBUF == 3) advance(IC<NU>(), it, 0);       // slice 0 of the next item
       lds_barrier();                                                                     // g
       if constexpr (NBUF == 3) advance(IC<NU + 1>(), it, 1);   // slice 1 of the next item
-      stage_gates(par ^ 1);
-      issue_gates(it + 2 * stride);
       lds_barrier();                                                                     // h: dk lies in the q tile
       {
         typename IOK::Regs r;
