@@ -90,7 +90,6 @@ typedef struct lmoe_args {
   /* backward workspace (caller-allocated, element type = dtype) */
   void* dhs;           /* gradient w.r.t. the state at the END of every chunk, laid out as hs */
   lmoe_tensor dvnew;   /* [B,T,H,V]   gradient of vnew (gated delta rule)              */
-  lmoe_tensor dw;      /* [B,T,H,K]   gradient of w    (gated delta rule)              */
 } lmoe_args;
 
 /* Library version (major*10000 + minor*100 + patch). */
@@ -99,7 +98,7 @@ int lmoe_version(void);
 const char* lmoe_last_error(void);
 
 /* Bytes of caller-allocated intermediates of one call: part 0 = what *_fwd writes for *_bwd
- * (hs, and per op amat / vnew, w, u, tinv, pmat, gcum), part 1 = the backward workspace (dhs, and dvnew, dw
+ * (hs, and per op amat / vnew, w, u, tinv, pmat, gcum), part 1 = the backward workspace (dhs, and dvnew
  * for the gated delta rule).  Each buffer is still passed through its own lmoe_args field; this
  * is the sum a caller that carves them out of one arena must reserve (every buffer's size is a
  * multiple of 256 bytes for the supported K, V).  Negative for an invalid op / dtype / part.
@@ -130,7 +129,7 @@ int lmoe_chunk_gla_bwd(const lmoe_args* a, void* stream);
  * Replaces fla.ops.gated_delta_rule.chunk_gated_delta_rule called at
  *   linear_moe/sequence_modeling/gated_deltanet/gated_deltanet.py:112.
  * fwd uses q,k,v,g,beta,h0 -> o,ht,hs,vnew,w,u,tinv,pmat,gcum.
- * bwd uses q,k,v,g,beta,hs,vnew,w,tinv,pmat,gcum,d_o,dht -> dq,dk,dv,dg,dbeta,dh0 (+ dhs, dvnew, dw). */
+ * bwd uses q,k,v,g,beta,hs,vnew,w,tinv,pmat,gcum,d_o,dht -> dq,dk,dv,dg,dbeta,dh0 (+ dhs, dvnew). */
 int lmoe_chunk_gated_delta_rule_fwd(const lmoe_args* a, void* stream);
 int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream);
 
@@ -146,10 +145,10 @@ int lmoe_l2norm_bwd(const void* x, const void* dy, void* dx, int64_t rows, int32
 
 /* Launch ONE kernel of an op's pipeline (profiling support: lets a harness time each kernel
  * with events on its own stream).  `a` must be the fully populated argument block of the
- * op's fwd (stages 0-2, 7) or bwd (stages 3-6) entry point, with the intermediates of the
+ * op's fwd (stages 0-2, 7) or bwd (stages 3-5) entry point, with the intermediates of the
  * earlier stages already in place.  Stages: 0 gated-delta-rule WY preparation, 1 forward state
- * pass, 2 output, 3 dv / local dv_new, 4 reverse state pass, 5 dq dk and gate gradient,
- * 6 gated-delta-rule WY backward, 7 chunk_gla intra-chunk matrix.
+ * pass, 2 output, 3 dv, 4 reverse state pass, 5 dq dk and gate gradient (gated delta rule: every
+ * gradient that follows the reverse state pass), 7 chunk_gla intra-chunk matrix.
  * No counterpart in the reference (measurement support). */
 #define LMOE_OP_SIMPLE_GLA 0
 #define LMOE_OP_GLA 1

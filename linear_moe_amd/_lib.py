@@ -36,7 +36,7 @@ class Args(C.Structure):
         ("d_o", Tensor4), ("dht", C.c_void_p),
         ("dq", Tensor4), ("dk", Tensor4), ("dv", Tensor4), ("dg", Tensor4), ("dbeta", Tensor4),
         ("dh0", C.c_void_p),
-        ("dhs", C.c_void_p), ("dvnew", Tensor4), ("dw", Tensor4),
+        ("dhs", C.c_void_p), ("dvnew", Tensor4),
     ]
 
 

@@ -58,7 +58,7 @@ int64_t lmoe_workspace_bytes(int32_t op, int32_t dtype, int32_t part, int32_t B,
   int64_t n = states;                                                    // hs | dhs
   if (op == LMOE_OP_GLA && part == 0) n += tiles;                        // amat
   if (op == LMOE_OP_GATED_DELTA_RULE) n += part == 0 ? 2 * rows_v + rows_k + 2 * tiles   // vnew, u, w, tinv, pmat
-                                                     : rows_v + rows_k;              // dvnew, dw
+                                                     : rows_v;                       // dvnew
   int64_t bytes = n * s;
   if (op == LMOE_OP_GATED_DELTA_RULE && part == 0) bytes += (int64_t)NT * H * 2 * LMOE_CHUNK * 4;   // gcum (fp32)
   return bytes;
@@ -84,7 +84,7 @@ int lmoe_chunk_simple_gla_bwd(const lmoe_args* a, void* stream) {
   if (a->NT == 0 || a->N == 0) return 0;
   lmoe::launch_state_bwd(*a, (hipStream_t)stream);
   lmoe::launch_bwd_dv(*a, false, (hipStream_t)stream);
-  lmoe::launch_bwd_dqk(*a, false, (hipStream_t)stream);
+  lmoe::launch_bwd_dqk(*a, (hipStream_t)stream);
   return launched(op);
 }
 static int check_gla(const lmoe_args* a, const char* op) {
@@ -205,7 +205,7 @@ int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* strea
           if (!a->tinv || !a->dvnew.ptr || !a->beta.ptr) return fail(-11, "%s: tinv, dvnew and beta must not be null", nm);
           lmoe::launch_gdn_bwd_chunk(*a, st);
         } else {
-          lmoe::launch_bwd_dqk(*a, false, st);
+          lmoe::launch_bwd_dqk(*a, st);
         }
         break;
       default: return fail(-20, "%s: stage %d not part of this op", nm, stage);

@@ -11,10 +11,10 @@ enum Stage {
   ST_GDN_WY_FWD = 0,   // gated delta rule: w, u, Tinv, P                (chunk-parallel)
   ST_STATE_FWD = 1,    // sequential state pass: hs (, vnew), ht; scalar gates: also the output o
   ST_OUT_FWD = 2,      // chunk_gla: output o                            (chunk-parallel)
-  ST_DV = 3,           // dv (simple_gla / gla) or local part of dv_new  (chunk-parallel)
+  ST_DV = 3,           // dv (simple_gla / gla)                          (chunk-parallel)
   ST_STATE_BWD = 4,    // reverse sequential state pass: dhs (, dv_new), dh0
-  ST_DQK = 5,          // dq, dk, gate gradient (, dw)                   (chunk-parallel)
-  ST_GDN_WY_BWD = 6,   // gated delta rule: backward through w, u        (chunk-parallel)
+  ST_DQK = 5,          // dq, dk, gate gradient; gated delta rule: every gradient that follows the
+                       // reverse state pass (dq, dk, dv, dbeta, dg)     (chunk-parallel)
   ST_GLA_INTRA_FWD = 7 // chunk_gla: intra-chunk attention matrix        (chunk-parallel)
 };
 
@@ -37,7 +37,7 @@ void launch_gdn_state_bwd(const lmoe_args& a, hipStream_t st);
 void launch_gdn_wy_fwd(const lmoe_args& a, hipStream_t st);
 void launch_bwd_dv(const lmoe_args& a, bool local, hipStream_t st);
 void launch_state_bwd(const lmoe_args& a, hipStream_t st);        // chunk_simple_gla
-void launch_bwd_dqk(const lmoe_args& a, bool gdn, hipStream_t st);
+void launch_bwd_dqk(const lmoe_args& a, hipStream_t st);          // chunk_simple_gla
 void launch_gdn_bwd_chunk(const lmoe_args& a, hipStream_t st);    // gated delta rule: all chunk-parallel gradients
 // chunk_gla: one kernel of the pipeline (stage = ST_GLA_INTRA_FWD, ST_STATE_FWD, ST_OUT_FWD,
 // ST_STATE_BWD, ST_DV, ST_DQK)

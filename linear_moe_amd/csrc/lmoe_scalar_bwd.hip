@@ -1,4 +1,4 @@
-// Instantiation and launch of the scalar-gate backward kernels.
+// Instantiation and launch of the backward kernels of chunk_simple_gla.
 #include "lmoe_launch.hpp"
 #include "lmoe_scalar_bwd.hpp"
 
@@ -18,31 +18,25 @@ template <bool LOCAL> struct BwdDv {
     }
   };
 };
-template <bool GDN> struct StateBwd {
-  template <typename T, int K, int V> struct F {
-    static void run(const lmoe_args& a, hipStream_t st) {
-      constexpr int BV = BwdTiles<T, V>::BVS;
-      const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BV);
-      hipLaunchKernelGGL((k_state_bwd<T, K, V, BV, GDN>), dim3(grid), dim3((GDN ? 3 : 2) * NTHR), 0, st, a);
-    }
-  };
+template <typename T, int K, int V> struct StateBwd {
+  static void run(const lmoe_args& a, hipStream_t st) {
+    constexpr int BV = BwdTiles<T, V>::BVS;
+    const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BV);
+    hipLaunchKernelGGL((k_state_bwd<T, K, V, BV>), dim3(grid), dim3(2 * NTHR), 0, st, a);
+  }
 };
-template <bool GDN> struct BwdDqk {
-  template <typename T, int K, int V> struct F {
-    static void run(const lmoe_args& a, hipStream_t st) {
-      constexpr int BVH = BwdTiles<T, V>::BVH;
-      const int grid = persistent_grid(a.NT * a.H, 1);
-      hipLaunchKernelGGL((k_bwd_dqk<T, K, V, BVH, GDN>), dim3(grid), dim3(2 * NTHR), 0, st, a);
-    }
-  };
+template <typename T, int K, int V> struct BwdDqk {
+  static void run(const lmoe_args& a, hipStream_t st) {
+    constexpr int BVH = BwdTiles<T, V>::BVH;
+    const int grid = persistent_grid(a.NT * a.H, 1);
+    hipLaunchKernelGGL((k_bwd_dqk<T, K, V, BVH>), dim3(grid), dim3(2 * NTHR), 0, st, a);
+  }
 };
 
 void launch_bwd_dv(const lmoe_args& a, bool local, hipStream_t st) {
   if (local) dispatch<BwdDv<true>::F>(a, st); else dispatch<BwdDv<false>::F>(a, st);
 }
-void launch_state_bwd(const lmoe_args& a, hipStream_t st) { dispatch<StateBwd<false>::F>(a, st); }
-void launch_bwd_dqk(const lmoe_args& a, bool gdn, hipStream_t st) {
-  if (gdn) dispatch<BwdDqk<true>::F>(a, st); else dispatch<BwdDqk<false>::F>(a, st);
-}
+void launch_state_bwd(const lmoe_args& a, hipStream_t st) { dispatch<StateBwd>(a, st); }
+void launch_bwd_dqk(const lmoe_args& a, hipStream_t st) { dispatch<BwdDqk>(a, st); }
 
 }  // namespace lmoe

@@ -1,17 +1,14 @@
-// Backward kernels for scalar-gated chunks (chunk_simple_gla and chunk_gated_delta_rule).
+// Backward kernels of chunk_simple_gla (one scalar log-decay per token and head).
 // Notation per chunk: b = inclusive cumsum of g, e_b = e^{b}, e_d = e^{b_C - b},
 // Gamma_ij = e^{b_i - b_j} [i >= j], P = (q k^T) . Gamma, S = state at chunk start,
-// dS' = gradient w.r.t. the state at chunk end, v' = v (simple_gla) or v_new (delta rule).
+// dS' = gradient w.r.t. the state at chunk end.
 //
-//   k_bwd_dv    : chunk-parallel   dv = scale P^T do + (k . e_d) dS'     (simple_gla only)
+//   k_bwd_dv    : chunk-parallel   dv = scale P^T do + (k . e_d) dS'
 //   k_state_bwd : reverse sequential pass over the chunks of one (sequence, head, V-slice):
-//                 writes dS' of every chunk (dhs); delta rule: dv_new = dv_loc + (k . e_d) dS'
-//                 with dv_loc = scale P^T do formed in the same kernel;
-//                 dS = e^{b_C} dS' + scale (q . e_b)^T do  (- w^T dv_new)
-//   k_bwd_dqk   : chunk-parallel   dq, dk (delta rule: the part of dk that does not go through
-//                 the WY factors, and dw = -dv_new S^T), gate gradient
-//                 db_i = q_i.dq_i - k_i.dk_i (+ on the last row sum_j (dk_d . k_d)_j + e^{b_C} <S, dS'>)
-//                 and, for simple_gla, dg = reverse cumsum of db.
+//                 writes dS' of every chunk (dhs);  dS = e^{b_C} dS' + scale (q . e_b)^T do
+//   k_bwd_dqk   : chunk-parallel   dq, dk, gate gradient
+//                 db_i = q_i.dq_i - k_i.dk_i (+ on the last row sum_j (dk_d . k_d)_j + e^{b_C} <S, dS'>),
+//                 dg = reverse cumsum of db.
 #pragma once
 #include "lmoe_seq.hpp"
 #include "lmoe_scalar_fwd.hpp"   // scale_frag
@@ -95,29 +92,19 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dv(const lmoe_args a) {
 // reverse state pass: producer / consumer work-group of 512 threads (mirror of k_state_fwd)
 //   grid = ceil(N*H / 8) * 8 * (V / BV) work-groups (1-D); V-slices of one (sequence, head)
 //   share an XCD.  dS slice [K x BV] lives in fp32 MFMA accumulators of waves 0-3 (consumers):
-//        dS' -> LDS | B1 | dv_new = dv_loc + e_d (k dS') -> LDS | B2 |
-//        dS = e^{b_C} dS' + q^T (scale e_b do) - w^T dv_new
-//   Waves 4-7 (loaders) keep the next chunks' q, k, w, do in flight, stage them unscaled and write
-//   dhs (layout [V][K]).  For the delta rule waves 8-11 compute the local part of dv_new of the
-//   next step from the staged tiles:  dv_loc = scale ((q k^T) . Gamma)^T do  (each wave 16 rows of
-//   it, P^T through a wave-private LDS strip), so no separate dv kernel runs for that op.
-//   All teams meet at the same barriers; three waves per SIMD hide each other's latencies.
+//        dS' -> LDS | B1 | B2 | dS = e^{b_C} dS' + q^T (scale e_b do)
+//   Waves 4-7 (loaders) keep the next chunks' q, do in flight, stage them unscaled and write
+//   dhs (layout [V][K]).  Both teams meet at the same barriers.
 // ------------------------------------------------------------------------- //
-template <typename T, int K, int V, int BV, bool GDN>
-__global__ __launch_bounds__((GDN ? 3 : 2) * NTHR) void k_state_bwd(const lmoe_args a) {
+template <typename T, int K, int V, int BV>
+__global__ __launch_bounds__(2 * NTHR) void k_state_bwd(const lmoe_args a) {
   constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDU = BV + LPAD;
   constexpr int MB = K / 64, NB = BV / 16;
   // bf16: two operand buffers; fp32 (the parity path) has LDS for one and pays extra barriers
   constexpr int NBUF = sizeof(T) == 2 ? 2 : 1;
   __shared__ __attribute__((aligned(16))) T s_q[NBUF][CH * LDK];             // q       [64][K]
   __shared__ __attribute__((aligned(16))) T s_do[NBUF][CH * LDU];            // do      [64][BV]
-  __shared__ __attribute__((aligned(16))) T s_k[NBUF][GDN ? CH * LDK : 8];   // k       [64][K]
-  __shared__ __attribute__((aligned(16))) T s_w[NBUF][GDN ? CH * LDK : 8];   // w       [64][K]
-  __shared__ __attribute__((aligned(16))) T s_dvl[NBUF][GDN ? CH * LDU : 8]; // dv_loc  [64][BV]
   __shared__ __attribute__((aligned(16))) T s_dST[BV * LDK];                 // dS'^T   [BV][K]
-  __shared__ __attribute__((aligned(16))) T s_dvT[GDN ? BV * LDC : 8];       // -dv_new^T [BV][64]
-  __shared__ __attribute__((aligned(16))) T s_pt[GDN ? 4 * 16 * LDC : 8];    // producers: P^T strips
-  __shared__ __attribute__((aligned(16))) T s_stg[GDN ? 4 * 16 * LDU : 8];   // consumers: dv_new store
   __shared__ __attribute__((aligned(16))) float s_b[NBUF][64], s_qs[NBUF][64], s_ed[NBUF][64];
   __shared__ float s_dec[NBUF];
 
@@ -128,7 +115,7 @@ __global__ __launch_bounds__((GDN ? 3 : 2) * NTHR) void k_state_bwd(const lmoe_a
   const int v0 = vsl * BV, h = pair % a.H, n = pair / a.H;
   const SeqInfo sq = seq_info(a, n);
   const int l = lane_id();
-  const int team = threadIdx.x / NTHR;      // 0: consumers, 1: loaders, 2: local dv (delta rule)
+  const int team = threadIdx.x / NTHR;      // 0: consumers, 1: loaders
   const bool producer = team == 1;
   if (sq.nchunks == 0) {
     if (a.dh0 && team == 0) {
@@ -147,7 +134,7 @@ __global__ __launch_bounds__((GDN ? 3 : 2) * NTHR) void k_state_bwd(const lmoe_a
   if (producer) {
     // ------------------------------- producers -------------------------------------------
     constexpr int PF = 2;
-    struct Pre { typename IOK::Regs rq, rk, rw; typename IOV::Regs rd; uint32_t graw; int len; };
+    struct Pre { typename IOK::Regs rq; typename IOV::Regs rd; uint32_t graw; int len; };
     Pre pre[PF];
     const int pw = wave_id() - 4;
     const bool gated = a.gate != LMOE_GATE_NONE && a.g.ptr != nullptr;
@@ -160,10 +147,6 @@ __global__ __launch_bounds__((GDN ? 3 : 2) * NTHR) void k_state_bwd(const lmoe_a
       const int len = min(CH, sq.len - c * CH);
       IOK::load_nomask(P.rq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, len);
       IOV::load_nomask(P.rd, row_ptr<T>(a.d_o, sq.b, tok, h) + v0, a.d_o.st, len);
-      if constexpr (GDN) {
-        IOK::load_nomask(P.rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, len);
-        IOK::load_nomask(P.rw, row_ptr<T>(a.w, sq.b, tok, h), a.w.st, len);
-      }
       P.len = len;
       P.graw = load_scalar_raw(gptr, a.g_dtype, gated ? row_off(a.g, sq.b, tok + min(l, len - 1), h) : 0);
     };
@@ -172,12 +155,6 @@ __global__ __launch_bounds__((GDN ? 3 : 2) * NTHR) void k_state_bwd(const lmoe_a
       IOV::mask(P.rd, P.len);
       IOK::store_lds(P.rq, s_q[buf], LDK);
       IOV::store_lds(P.rd, s_do[buf], LDU);
-      if constexpr (GDN) {
-        IOK::mask(P.rk, P.len);
-        IOK::mask(P.rw, P.len);
-        IOK::store_lds(P.rk, s_k[buf], LDK);
-        IOK::store_lds(P.rw, s_w[buf], LDK);
-      }
       if (pw == 0) {
         const float x = wave_incl_scan((gated && l < P.len) ? scalar_from_raw(P.graw, a.g_dtype) : 0.f);
         const float xl = __shfl(x, 63, 64);
@@ -192,7 +169,6 @@ __global__ __launch_bounds__((GDN ? 3 : 2) * NTHR) void k_state_bwd(const lmoe_a
     stage(pre[0], 0);
     issue(pre[0], sq.nchunks - 1 - PF);
     lds_barrier();                                   // P0: the first chunk's tiles are complete
-    if constexpr (GDN) lds_barrier();                // P1: its local dv is complete
     for (int it0 = 0; it0 < sq.nchunks; it0 += PF) {
 #pragma unroll
       for (int j = 0; j < PF; ++j) {
@@ -217,57 +193,6 @@ __global__ __launch_bounds__((GDN ? 3 : 2) * NTHR) void k_state_bwd(const lmoe_a
     return;
   }
 
-  if (team == 2) {
-    // ------------------------------- local dv (delta rule) -------------------------------
-    const int pw = wave_id() - 8;
-    const float scale = a.scale;
-    // local part of dv_new of the chunk staged in `buf`: rows 16 pw .. 16 pw + 15
-    auto dv_local = [&](int buf) {
-      if constexpr (GDN) {
-        T* pt = s_pt + pw * 16 * LDC;
-        f32x4 p[1][4];
-        acc_zero(p);
-        gemm<T, 1, 4, false, false>(p, s_k[buf], LDK, 16 * pw, s_q[buf], LDK, 0, 0, K);   // p[j][i] = k_j . q_i
-#pragma unroll
-        for (int ni = 0; ni < 4; ++ni) {
-          f32x4 x;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int j = 16 * pw + 4 * (l >> 4) + e, i = 16 * ni + (l & 15);
-            x[e] = (i >= j) ? p[0][ni][e] * texp<T>(s_b[buf][i] - s_b[buf][j]) : 0.f;
-          }
-          acc_to_lds<T>(x, pt, LDC, 0, 16 * ni);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        f32x4 d[1][NB];
-        acc_zero(d);
-        gemm<T, 1, NB, false, true>(d, pt, LDC, 0, s_do[buf], LDU, 0, 0, CH);
-#pragma unroll
-        for (int ni = 0; ni < NB; ++ni) {
-          d[0][ni] *= scale;
-          acc_to_lds<T>(d[0][ni], s_dvl[buf], LDU, 16 * pw, 16 * ni);
-        }
-      }
-    };
-    lds_barrier();                                   // P0
-    dv_local(0);
-    lds_barrier();                                   // P1
-    for (int it = 0; it < sq.nchunks; ++it) {
-      const int c = sq.nchunks - 1 - it;
-      const int nb = NBUF == 2 ? ((it + 1) & 1) : 0;
-      lds_barrier();                                                                     // B1
-      lds_barrier();                                                                     // B2
-      if constexpr (NBUF == 1) {
-        lds_barrier();                                                                   // B3
-        lds_barrier();                                                                   // B4
-      }
-      if (c > 0) dv_local(nb);
-    }
-    return;
-  }
-
   // --------------------------------- consumers -------------------------------------------
   const int wv = wave_id();
   const int krow0 = wv * (K / 4);
@@ -284,7 +209,6 @@ __global__ __launch_bounds__((GDN ? 3 : 2) * NTHR) void k_state_bwd(const lmoe_a
           dS[mi][ni][i] = p[(int64_t)(krow0 + acc_row(mi, i)) * V + v0 + acc_col(ni)];
   }
   lds_barrier();                                     // P0
-  if constexpr (GDN) lds_barrier();                  // P1
   for (int it = 0; it < sq.nchunks; ++it) {
     const int c = sq.nchunks - 1 - it;
     const int cur = NBUF == 2 ? (it & 1) : 0;
@@ -298,21 +222,6 @@ __global__ __launch_bounds__((GDN ? 3 : 2) * NTHR) void k_state_bwd(const lmoe_a
     const float dec = s_dec[cur];
     f32x4 t[1][NB];
     acc_zero(t);
-    if constexpr (GDN) {
-      // dv_new = dv_loc + e_d (k dS')   (rows 16 wv .. of the chunk)
-      gemm<T, 1, NB, false, false>(t, s_k[cur], LDK, 16 * wv, s_dST, LDK, 0, 0, K);
-#pragma unroll
-      for (int ni = 0; ni < NB; ++ni) {
-        f32x4 x;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
-          t[0][ni][i] = ET<T>::to_f(ET<T>::from_f(ET<T>::to_f(s_dvl[cur][r * LDU + cc]) + s_ed[cur][r] * t[0][ni][i]));
-          x[i] = -t[0][ni][i];
-        }
-        acc_to_lds_t<T>(x, s_dvT, LDC, 16 * wv, 16 * ni);
-      }
-    }
     lds_barrier();                                                                       // B2
 #pragma unroll
     for (int mi = 0; mi < MB; ++mi)
@@ -332,11 +241,6 @@ __global__ __launch_bounds__((GDN ? 3 : 2) * NTHR) void k_state_bwd(const lmoe_a
       for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
         for (int ni = 0; ni < NB; ++ni) ET<T>::mma(dS[mi][ni], af[mi], bf[ni]);
-    }
-    if constexpr (GDN) {
-      gemm<T, MB, NB, true, false>(dS, s_w[cur], LDK, krow0, s_dvT, LDC, 0, 0, CH);
-      store_strip<T, NB>(t, s_stg + wv * 16 * LDU, row_ptr<T>(a.dvnew, sq.b, tok + 16 * wv, h) + v0, a.dvnew.st,
-                         len - 16 * wv, 1.0f);
     }
     if constexpr (NBUF == 1) {
       lds_barrier();                                                                     // B3
@@ -358,7 +262,7 @@ __global__ __launch_bounds__((GDN ? 3 : 2) * NTHR) void k_state_bwd(const lmoe_a
 // ------------------------------------------------------------------------- //
 // dq, dk, gate gradient        persistent: one work-group per CU, one item = (chunk, head)
 //   phase A: loop over V-slices of width BVH accumulating
-//              dP = do v'^T, dq_i = do S^T, dk_d = v' dS'^T (, dw = dv_new S^T)
+//              dP = do v^T, dq_i = do S^T, dk_d = v dS'^T
 //            (hs, dhs hold S^T, dS'^T: [V][K]; the slice tiles are [BVH][K])
 //   phase B: dq = scale e_b dq_i + (scale dP . Gamma) k ; dk = e_d dk_d + (scale dP . Gamma)^T q
 //            with one LDS copy of (scale dP . Gamma)^T and q, k stored as loaded
@@ -373,18 +277,17 @@ __global__ __launch_bounds__((GDN ? 3 : 2) * NTHR) void k_state_bwd(const lmoe_a
 //     compute : R(s): products of slice s | D, A | (dP . Gamma)^T -> LDS | b | products, combine |
 //               c | stores | E
 // ------------------------------------------------------------------------- //
-template <typename T, int K, int V, int BVH, bool GDN>
+template <typename T, int K, int V, int BVH>
 __global__ __launch_bounds__(2 * NTHR) void k_bwd_dqk(const lmoe_args a) {
   constexpr int LDV = BVH + LPAD, LDC = CH + LPAD, LDK = K + LPAD;
   constexpr int NBK = K / 16, NS = V / BVH;
   // tiles of one V-slice
   constexpr int A_DO = 0, A_V = A_DO + CH * LDV, A_H = A_V + CH * LDV, A_DH = A_H + BVH * LDK,
-                A_DVN = A_DH + BVH * LDK, A_END = A_DVN + (GDN ? CH * LDV : 0);
+                A_END = A_DH + BVH * LDK;
   // phase B tiles (relative to the second slice buffer)
   constexpr int B_DPT = 0, B_K = B_DPT + CH * LDC, B_Q = B_K + CH * LDK, B_END = B_Q + CH * LDK;
   constexpr int BUF1 = A_END;
   constexpr int NELEM = BUF1 + (A_END > B_END ? A_END : B_END);
-  static_assert(!GDN || 4 * 16 * LDK <= A_END, "the dw store strips fit the first slice buffer");
   __shared__ __attribute__((aligned(16))) T smem[NELEM];
   __shared__ float s_b[64], s_eb[64], s_ed[64], s_db[64], s_red[8];
 
@@ -393,13 +296,13 @@ __global__ __launch_bounds__(2 * NTHR) void k_bwd_dqk(const lmoe_args a) {
   typedef TileIO<T, CH, BVH> IOV;
   typedef TileIO<T, BVH, K> IOH;
   typedef TileIO<T, CH, K> IOK;
-  const lmoe_tensor& vs = GDN ? a.vnew : a.v;
+  const lmoe_tensor& vs = a.v;
   const int nitems = a.NT * a.H;
   const int stride = gridDim.x;
 
   if (team == 1) {
     // --------------------------------- loaders -------------------------------------------
-    struct SliceRegs { typename IOV::Regs rd, rv, rn; typename IOH::Regs rh, rdh; int len; };
+    struct SliceRegs { typename IOV::Regs rd, rv; typename IOH::Regs rh, rdh; int len; };
     struct QKRegs { typename IOK::Regs rq, rk; uint32_t graw; int len; };
     SliceRegs S;
     QKRegs Q;
@@ -414,7 +317,6 @@ __global__ __launch_bounds__(2 * NTHR) void k_bwd_dqk(const lmoe_args a) {
       IOV::load_nomask(S.rv, row_ptr<T>(vs, ci.b, ci.tok, h) + vv, vs.st, ci.len);
       IOH::load_nomask(S.rh, (const T*)a.hs + (((int64_t)cid * a.H + h) * V + vv) * K, K, BVH);
       IOH::load_nomask(S.rdh, (const T*)a.dhs + (((int64_t)cid * a.H + h) * V + vv) * K, K, BVH);
-      if constexpr (GDN) IOV::load_nomask(S.rn, row_ptr<T>(a.dvnew, ci.b, ci.tok, h) + vv, a.dvnew.st, ci.len);
     };
     auto issue_qk = [&](int it) {
       it = min(it, nitems - 1);
@@ -438,10 +340,6 @@ __global__ __launch_bounds__(2 * NTHR) void k_bwd_dqk(const lmoe_args a) {
       IOV::store_lds(S.rv, base + A_V, LDV);
       IOH::store_lds(S.rh, base + A_H, LDK);
       IOH::store_lds(S.rdh, base + A_DH, LDK);
-      if constexpr (GDN) {
-        IOV::mask(S.rn, S.len);
-        IOV::store_lds(S.rn, base + A_DVN, LDV);
-      }
     };
     // the slice after slice s of item it
     auto issue_next = [&](int it, int s) {
@@ -490,20 +388,18 @@ __global__ __launch_bounds__(2 * NTHR) void k_bwd_dqk(const lmoe_args a) {
   for (int it = blockIdx.x; it < nitems; it += stride) {
     const int cid = it / a.H, h = it % a.H;
     const ChunkInfo ci = chunk_info(a, cid);
-    f32x4 dP[1][4], dqi[1][NBK], dkd[1][NBK], dw[1][GDN ? NBK : 1];
-    acc_zero(dP); acc_zero(dqi); acc_zero(dkd); acc_zero(dw);
+    f32x4 dP[1][4], dqi[1][NBK], dkd[1][NBK];
+    acc_zero(dP); acc_zero(dqi); acc_zero(dkd);
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
       lds_barrier();                                                                     // R(s)
       const T* base = smem + (s & 1) * BUF1;
-      const T* DO = base + A_DO; const T* VN = base + A_V; const T* DVN = base + A_DVN;
+      const T* DO = base + A_DO; const T* VN = base + A_V;
       const T* HT = base + A_H; const T* DHT = base + A_DH;
 #pragma unroll
       for (int kk = 0; kk < BVH; kk += 32) {
         const typename ET<T>::frag aDO = ET<T>::load_frag(DO + (16 * wv + fr) * LDV + kk + fg);
         const typename ET<T>::frag aVN = ET<T>::load_frag(VN + (16 * wv + fr) * LDV + kk + fg);
-        typename ET<T>::frag aDVN = aVN;
-        if constexpr (GDN) aDVN = ET<T>::load_frag(DVN + (16 * wv + fr) * LDV + kk + fg);
 #pragma unroll
         for (int nj = 0; nj < 4; ++nj)
           ET<T>::mma(dP[0][nj], aDO, ET<T>::load_frag(VN + (16 * nj + fr) * LDV + kk + fg));
@@ -512,19 +408,12 @@ __global__ __launch_bounds__(2 * NTHR) void k_bwd_dqk(const lmoe_args a) {
         for (int ni = 0; ni < NBK; ++ni) {
           const typename ET<T>::frag bH = ET<T>::load_frag_t(HT, LDK, kk, 16 * ni);
           ET<T>::mma(dqi[0][ni], aDO, bH);
-          if constexpr (GDN) ET<T>::mma(dw[0][ni], aDVN, bH);
           ET<T>::mma(dkd[0][ni], aVN, ET<T>::load_frag_t(DHT, LDK, kk, 16 * ni));
           if (ni % 4 == 3) __builtin_amdgcn_sched_barrier(0);
         }
       }
     }
     lds_barrier();                                                                       // D
-    if constexpr (GDN) {
-      // dw = -dv_new S^T is complete: it leaves its registers now, staged through the first slice
-      // buffer, which is idle until the loaders refill it after A
-      store_strip<T, NBK>(dw, smem + wv * 16 * LDK, row_ptr<T>(a.dw, ci.b, ci.tok + 16 * wv, h), a.dw.st,
-                          ci.len - 16 * wv, -1.0f);
-    }
     lds_barrier();                                                                       // A
     T* PB = smem + BUF1;
 #pragma unroll
@@ -591,7 +480,7 @@ __global__ __launch_bounds__(2 * NTHR) void k_bwd_dqk(const lmoe_args a) {
       const float hsum = s_red[0] + s_red[1] + s_red[2] + s_red[3];
       const float ksum = s_red[4] + s_red[5] + s_red[6] + s_red[7];
       if (j == ci.len - 1) x += ksum + expf(s_b[63]) * hsum;
-      if constexpr (!GDN) x = wave_rev_scan(x);   // dg; the delta rule finishes db in its WY backward
+      x = wave_rev_scan(x);   // dg
       if (a.dg.ptr && j < ci.len) ((float*)a.dg.ptr)[row_off(a.dg, ci.b, ci.tok + j, h)] = x;
     }
     lds_barrier();     // E: the second buffer and the gate arrays go to the next item

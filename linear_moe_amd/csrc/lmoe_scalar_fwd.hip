@@ -1,4 +1,4 @@
-// Instantiation and launch of the scalar-gate forward kernels, plus the toolkit self-test.
+// Instantiation and launch of the forward kernel of chunk_simple_gla, plus the toolkit self-test.
 #include "lmoe_launch.hpp"
 #include "lmoe_scalar_fwd.hpp"
 
@@ -9,16 +9,14 @@ template <typename T, int V> struct FwdTiles {
   static constexpr int BVS = sizeof(T) == 4 ? 16 : 32;
 };
 
-template <bool GDN> struct StateFwd {
-  template <typename T, int K, int V> struct F {
-    static void run(const lmoe_args& a, hipStream_t st) {
-      constexpr int BV = FwdTiles<T, V>::BVS;
-      const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BV);
-      hipLaunchKernelGGL((k_state_fwd<T, K, V, BV, GDN>), dim3(grid), dim3(3 * NTHR), 0, st, a);
-    }
-  };
+template <typename T, int K, int V> struct StateFwd {
+  static void run(const lmoe_args& a, hipStream_t st) {
+    constexpr int BV = FwdTiles<T, V>::BVS;
+    const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BV);
+    hipLaunchKernelGGL((k_state_fwd<T, K, V, BV>), dim3(grid), dim3(3 * NTHR), 0, st, a);
+  }
 };
-void launch_state_fwd(const lmoe_args& a, hipStream_t st) { dispatch<StateFwd<false>::F>(a, st); }
+void launch_state_fwd(const lmoe_args& a, hipStream_t st) { dispatch<StateFwd>(a, st); }
 // C = A B^T (64 x 64, contraction along the tile columns) and G = A^T B (KD x KD, contraction
 // along the tile rows, i.e. the transposed-fragment path) over one pair of 64 x KD tiles,
 // through the loaders / fragments / accumulator stores of the toolkit

@@ -1,8 +1,7 @@
-// Forward kernel for scalar-gated chunks (chunk_simple_gla and chunk_gated_delta_rule): one
-// sequential pass over the chunks of one (sequence, head, V-slice) that carries the state,
-// forms v_new = u - w S for the delta rule and the output
-//   o = scale [ e^{b_i} q_i S + ((q k^T) . Gamma) v' ],   S' = e^{b_C} S + (k . e^{b_C - b})^T v',
-//   Gamma_ij = e^{b_i - b_j} [i >= j],  v' = v or v_new.
+// Forward kernel of chunk_simple_gla (one scalar log-decay per token and head): one sequential
+// pass over the chunks of one (sequence, head, V-slice) that carries the state and forms the output
+//   o = scale [ e^{b_i} q_i S + ((q k^T) . Gamma) v ],   S' = e^{b_C} S + (k . e^{b_C - b})^T v,
+//   Gamma_ij = e^{b_i - b_j} [i >= j].
 #pragma once
 #include "lmoe_seq.hpp"
 
@@ -22,19 +21,19 @@ template <typename T> __device__ __forceinline__ void scale_frag(typename ET<T>:
 // state pass + output (forward): work-group of three teams of four waves (768 threads)
 //   grid = ceil(N*H / 8) * 8 * (V / BV) work-groups (1-D).  Work-group -> (sequence, head,
 //   V-slice): the V-slices of one (sequence, head) get ids that are congruent mod 8, i.e. run on
-//   the same XCD and share q, k, w through its L2.
+//   the same XCD and share q, k through its L2.
 //   Team 0 (waves 0-3, consumers) carries the dependency chain of the state and nothing else:
-//        S -> LDS (element type T) | B1 | v_new = u - w S -> LDS | B2 | S = e^{b_C} S + k^T (e_d v_new)
+//        S -> LDS (element type T) | B1 | B2 | S = e^{b_C} S + k^T (e_d v)
 //     wave w owns state rows [w*K/4, (w+1)*K/4) x BV columns in fp32 MFMA accumulators; the row
-//     scaling e_d is applied to the v_new fragments in registers, so k is staged unscaled.
+//     scaling e_d is applied to the v fragments in registers, so k is staged unscaled.
 //   Team 1 (waves 4-7, loaders) keeps the operands of the next PF chunks in flight in registers,
 //     forms the gate cumsum, fills the other LDS buffer and writes hs (layout [V][K]) from the
 //     LDS copy of S.
 //   Team 2 (waves 8-11, output) forms the chunk's output rows 16w..: between B1 and B2
-//     e^{b_i} q S and P = (q k^T) . Gamma (P through a wave-private LDS strip), after B2 P v_new.
+//     e^{b_i} q S and P = (q k^T) . Gamma (P through a wave-private LDS strip), after B2 P v.
 //   All teams meet at the same barriers; three waves per SIMD hide each other's latencies.
 // ------------------------------------------------------------------------- //
-template <typename T, int K, int V, int BV, bool GDN>
+template <typename T, int K, int V, int BV>
 __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
   constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDU = BV + LPAD;
   constexpr int MB = K / 64, NB = BV / 16;
@@ -42,11 +41,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
   constexpr int NBUF = sizeof(T) == 2 ? 2 : 1;
   __shared__ __attribute__((aligned(16))) T s_k[NBUF][CH * LDK];              // k             [64][K]
   __shared__ __attribute__((aligned(16))) T s_q[NBUF][CH * LDK];              // q             [64][K]
-  __shared__ __attribute__((aligned(16))) T s_w[NBUF][GDN ? CH * LDK : 8];    // w             [64][K]
   __shared__ __attribute__((aligned(16))) T s_u[NBUF][CH * LDU];              // u or v        [64][BV]
   __shared__ __attribute__((aligned(16))) T s_hT[BV * LDK];                   // S^T           [BV][K]
-  __shared__ __attribute__((aligned(16))) T s_vT[GDN ? BV * LDC : 8];         // v_new^T       [BV][64]
-  __shared__ __attribute__((aligned(16))) T s_stg[GDN ? 4 * 16 * LDU : 8];    // team 0: v_new store
   __shared__ __attribute__((aligned(16))) T s_pst[4 * 16 * LDC];              // team 2: P strips
   __shared__ __attribute__((aligned(16))) T s_ost[4 * 16 * LDU];              // team 2: o store
   __shared__ __attribute__((aligned(16))) float s_b[NBUF][64], s_eb[NBUF][64], s_ed[NBUF][64];
@@ -78,9 +74,9 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
   if (team == 1) {
     // --------------------------------- loaders -------------------------------------------
     constexpr int PF = 2;
-    struct Pre { typename IOK::Regs rk, rq, rw; typename IOV::Regs ru; uint32_t graw; int len; };
+    struct Pre { typename IOK::Regs rk, rq; typename IOV::Regs ru; uint32_t graw; int len; };
     Pre pre[PF];
-    const lmoe_tensor& us = GDN ? a.u : a.v;
+    const lmoe_tensor& us = a.v;
     const bool gated = a.gate != LMOE_GATE_NONE && a.g.ptr != nullptr;
     const void* gptr = gated ? a.g.ptr : a.k.ptr;
     // Always issued (chunk index clamped to the last chunk; the surplus loads at the end of a
@@ -92,7 +88,6 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
       const int len = min(CH, sq.len - c * CH);
       IOK::load_nomask(P.rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, len);
       IOK::load_nomask(P.rq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, len);
-      if constexpr (GDN) IOK::load_nomask(P.rw, row_ptr<T>(a.w, sq.b, tok, h), a.w.st, len);
       IOV::load_nomask(P.ru, row_ptr<T>(us, sq.b, tok, h) + v0, us.st, len);
       P.len = len;
       P.graw = load_scalar_raw(gptr, a.g_dtype, gated ? row_off(a.g, sq.b, tok + min(l, len - 1), h) : 0);
@@ -105,10 +100,6 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
       IOK::store_lds(P.rk, s_k[buf], LDK);
       IOK::store_lds(P.rq, s_q[buf], LDK);
       IOV::store_lds(P.ru, s_u[buf], LDU);
-      if constexpr (GDN) {
-        IOK::mask(P.rw, P.len);
-        IOK::store_lds(P.rw, s_w[buf], LDK);
-      }
       if (wave_id() == 4) {
         const float x = wave_incl_scan((gated && l < P.len) ? scalar_from_raw(P.graw, a.g_dtype) : 0.f);
         const float xl = __shfl(x, 63, 64);
@@ -174,8 +165,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) o[0][ni][e] *= s_eb[cur][16 * ow + 4 * (l >> 4) + e];
       lds_barrier();                                                                     // B2 (orders pst too)
-      if constexpr (GDN) gemm<T, 1, NB, false, false>(o, pst, LDC, 0, s_vT, LDC, 0, 0, CH);
-      else gemm<T, 1, NB, false, true>(o, pst, LDC, 0, s_u[cur], LDU, 0, 0, CH);
+      gemm<T, 1, NB, false, true>(o, pst, LDC, 0, s_u[cur], LDU, 0, 0, CH);
       store_strip<T, NB>(o, s_ost + ow * 16 * LDU, row_ptr<T>(a.o, sq.b, tok + 16 * ow, h) + v0, a.o.st,
                          len - 16 * ow, a.scale);
       if constexpr (NBUF == 1) lds_barrier();                                            // B3
@@ -209,23 +199,6 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
       for (int ni = 0; ni < NB; ++ni) acc_to_lds_t<T>(S[mi][ni], s_hT, LDK, krow0 + 16 * mi, 16 * ni);
     lds_barrier();                                                                       // B1
     const float dec = s_dec[cur];
-    f32x4 vn[1][NB];
-    acc_zero(vn);
-    if constexpr (GDN) {
-      // v_new = u - w S  (rows 16*wv .. +15 of the chunk)
-      gemm<T, 1, NB, false, false>(vn, s_w[cur], LDK, 16 * wv, s_hT, LDK, 0, 0, K);
-#pragma unroll
-      for (int ni = 0; ni < NB; ++ni) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
-          // round once to the storage type so that the state update, the output and the backward
-          // see the same v_new
-          vn[0][ni][i] = ET<T>::to_f(ET<T>::from_f(ET<T>::to_f(s_u[cur][r * LDU + cc]) - vn[0][ni][i]));
-        }
-        acc_to_lds_t<T>(vn[0][ni], s_vT, LDC, 16 * wv, 16 * ni);
-      }
-    }
     lds_barrier();                                                                       // B2
 #pragma unroll
     for (int mi = 0; mi < MB; ++mi)
@@ -238,8 +211,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
       for (int mi = 0; mi < MB; ++mi) af[mi] = ET<T>::load_frag_t(s_k[cur], LDK, kk, krow0 + 16 * mi);
 #pragma unroll
       for (int ni = 0; ni < NB; ++ni) {
-        if constexpr (GDN) bf[ni] = ET<T>::load_frag(s_vT + (16 * ni + (l & 15)) * LDC + kk + 8 * (l >> 4));
-        else bf[ni] = ET<T>::load_frag_t(s_u[cur], LDU, kk, 16 * ni);
+        bf[ni] = ET<T>::load_frag_t(s_u[cur], LDU, kk, 16 * ni);
         scale_frag<T>(bf[ni], &s_ed[cur][kk + 8 * (l >> 4)]);
       }
 #pragma unroll
@@ -247,9 +219,6 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
 #pragma unroll
         for (int ni = 0; ni < NB; ++ni) ET<T>::mma(S[mi][ni], af[mi], bf[ni]);
     }
-    if constexpr (GDN)
-      store_strip<T, NB>(vn, s_stg + wv * 16 * LDU, row_ptr<T>(a.vnew, sq.b, tok + 16 * wv, h) + v0, a.vnew.st,
-                         len - 16 * wv, 1.0f);
     if constexpr (NBUF == 1) lds_barrier();                                              // B3
   }
   if (a.ht) {

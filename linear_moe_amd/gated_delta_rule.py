@@ -106,11 +106,10 @@ class GDNCall:
         a.dh0 = ptr(dh0)
         dhs = torch.empty_like(hs)
         dvnew = torch.empty(B, T, H, V, dtype=dt, device=dev)
-        dw = torch.empty(B, T, H, K, dtype=dt, device=dev)
-        a.dhs, a.dvnew, a.dw = dhs.data_ptr(), _desc(dvnew, False), _desc(dw, False)
+        a.dhs, a.dvnew = dhs.data_ptr(), _desc(dvnew, False)
         _lib.check(lib.lmoe_chunk_gated_delta_rule_bwd(C.byref(a), stream_ptr()), "chunk_gated_delta_rule backward")
         ctx.bwd_args = a
-        ctx.bwd_keep = (do, dht, dq, dk, dv, dg, dbeta, dh0, dhs, dvnew, dw) if self.keep else None
+        ctx.bwd_keep = (do, dht, dq, dk, dv, dg, dbeta, dh0, dhs, dvnew) if self.keep else None
         dg = None if g is None else dg.to(g.dtype)
         return dq, dk, dv, dg, dbeta.to(beta.dtype), dh0
 
