@@ -1,13 +1,11 @@
 // Device toolkit shared by all chunk kernels (gfx950 / CDNA4, wave64).
 //
 // Conventions used by every kernel in this directory:
-//  * a work-group is 256 threads = 4 wavefronts; a chunk is 64 tokens;
-//  * every LDS tile is stored "contraction-contiguous": element (r, c) at
-//    tile[r * ld + c] where c runs along the index the next MFMA contracts
-//    over.  A product X * Y^T with X:[M x Kd], Y:[N x Kd] therefore needs both
-//    operands as row-major tiles, and one helper (gemm_nt) serves every
-//    product; operands that are needed in both orientations are written to
-//    LDS twice (once transposed) while they are still in registers;
+//  * a team is 256 threads = 4 wavefronts (a work-group is one to three teams); a chunk is 64 tokens;
+//  * an LDS tile lies as it lies in memory: element (r, c) at tile[r * ld + c].  A product that
+//    contracts along the tile columns reads its fragments row-wise (gemm_nt, load_frag); one that
+//    contracts along the tile rows reads them through the transposing LDS read (gemm with AT / BT,
+//    load_frag_t), so no operand is stored twice;
 //  * MFMA shape: v_mfma_f32_16x16x32_bf16 for bf16 operands and
 //    8 x v_mfma_f32_16x16x4_f32 for fp32 operands, behind the same fragment
 //    layout (lane l holds row l%16, contraction elements 8*(l/16) .. +7);
