@@ -143,6 +143,29 @@ int lmoe_l2norm_fwd(const void* x, void* y, int64_t rows, int32_t D, int32_t dty
 int lmoe_l2norm_bwd(const void* x, const void* dy, void* dx, int64_t rows, int32_t D, int32_t dtype, float eps,
                     void* stream);
 
+/* y = l2norm(silu(x)) row-wise, and its backward dx: the two steps the reference applies to q and k of
+ * the gated delta rule in sequence, linear_moe/sequence_modeling/gated_deltanet/gated_deltanet.py:101
+ * (SiLU) and :105-106 (l2_norm_fn), as one pass over the rows.  Arguments as lmoe_l2norm_*. */
+int lmoe_silu_l2norm_fwd(const void* x, void* y, int64_t rows, int32_t D, int32_t dtype, float eps, void* stream);
+int lmoe_silu_l2norm_bwd(const void* x, const void* dy, void* dx, int64_t rows, int32_t D, int32_t dtype, float eps,
+                         void* stream);
+
+/* RMS norm over the last dimension of `rows` contiguous rows of D elements (D in {64, 128, 256}),
+ *   y = x rstd w [* gate sigmoid(gate)],  rstd = 1 / sqrt(mean(x^2) + eps),
+ * w ([D], element type of x) and gate ([rows][D]) may be null; rstd ([rows] fp32) is written when not null.
+ * Replaces rms_norm_fn of the reference (linear_moe/model/common_modules/layernorm.py:515-537 ->
+ * LayerNormFn :383-466 with is_rms_norm; kernels :69-132 forward, :212-300 backward; no bias, no residual),
+ * the output norm of gla.py:95 and retention.py:92; the gate product is the reference's
+ * `o * swish(o_gate)` (linear_moe/sequence_modeling/linear_attention.py:255) folded into the same pass.
+ * Backward: dx, dgate (with gate), and dw ([D] fp32) through dw_part, a caller-allocated fp32
+ * [lmoe_rmsnorm_partials(rows, D, dtype)][D] workspace that is summed in a fixed order
+ * (the reference sums per-SM partial rows the same way, layernorm.py:349-377). dw_part and dw may both be null. */
+int lmoe_rmsnorm_partials(int64_t rows, int32_t D, int32_t dtype);
+int lmoe_rmsnorm_fwd(const void* x, const void* w, const void* gate, void* y, float* rstd, int64_t rows, int32_t D,
+                     int32_t dtype, float eps, void* stream);
+int lmoe_rmsnorm_bwd(const void* x, const void* w, const void* gate, const void* dy, void* dx, void* dgate,
+                     float* dw_part, float* dw, int64_t rows, int32_t D, int32_t dtype, float eps, void* stream);
+
 /* Launch ONE kernel of an op's pipeline (profiling support: lets a harness time each kernel
  * with events on its own stream).  `a` must be the fully populated argument block of the
  * op's fwd (stages 0-2, 7) or bwd (stages 3-5) entry point, with the intermediates of the

@@ -8,7 +8,8 @@ All compute runs in hand-written HIP kernels (``csrc/``) reached through the C A
 from .delta_rule import chunk_delta_rule  # noqa: F401
 from .gated_delta_rule import chunk_gated_delta_rule  # noqa: F401
 from .gla import chunk_gla  # noqa: F401
-from .l2norm import l2_norm, l2_norm_fn  # noqa: F401
+from .l2norm import l2_norm, l2_norm_fn, silu_l2_norm  # noqa: F401
+from .rmsnorm import RMSNorm, rms_norm_fn, rms_norm_swish_gate  # noqa: F401
 from .lightning import lightning_attn2, lightning_attn2_no_decay  # noqa: F401
 from .linear_attn import chunk_linear_attn  # noqa: F401
 from .retention import chunk_retention  # noqa: F401

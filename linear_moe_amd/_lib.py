@@ -46,6 +46,7 @@ ENTRY_POINTS = (
     "lmoe_chunk_gla_fwd", "lmoe_chunk_gla_bwd",
     "lmoe_chunk_gated_delta_rule_fwd", "lmoe_chunk_gated_delta_rule_bwd",
     "lmoe_launch_stage", "lmoe_selftest_gemm", "lmoe_workspace_bytes", "lmoe_l2norm_fwd", "lmoe_l2norm_bwd",
+    "lmoe_silu_l2norm_fwd", "lmoe_silu_l2norm_bwd", "lmoe_rmsnorm_partials", "lmoe_rmsnorm_fwd", "lmoe_rmsnorm_bwd",
 )
 
 _lib = None
@@ -77,6 +78,17 @@ def load() -> C.CDLL:
     lib.lmoe_l2norm_bwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_float,
                                     C.c_void_p]
     lib.lmoe_l2norm_bwd.restype = C.c_int
+    lib.lmoe_silu_l2norm_fwd.argtypes = lib.lmoe_l2norm_fwd.argtypes
+    lib.lmoe_silu_l2norm_fwd.restype = C.c_int
+    lib.lmoe_silu_l2norm_bwd.argtypes = lib.lmoe_l2norm_bwd.argtypes
+    lib.lmoe_silu_l2norm_bwd.restype = C.c_int
+    lib.lmoe_rmsnorm_partials.argtypes = [C.c_int64, C.c_int32, C.c_int32]
+    lib.lmoe_rmsnorm_partials.restype = C.c_int32
+    lib.lmoe_rmsnorm_fwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32,
+                                     C.c_int32, C.c_float, C.c_void_p]
+    lib.lmoe_rmsnorm_fwd.restype = C.c_int
+    lib.lmoe_rmsnorm_bwd.argtypes = [C.c_void_p] * 8 + [C.c_int64, C.c_int32, C.c_int32, C.c_float, C.c_void_p]
+    lib.lmoe_rmsnorm_bwd.restype = C.c_int
     lib.lmoe_workspace_bytes.argtypes = [C.c_int32] * 9
     lib.lmoe_workspace_bytes.restype = C.c_int64
     _lib = lib

@@ -171,6 +171,54 @@ int lmoe_l2norm_bwd(const void* x, const void* dy, void* dx, int64_t rows, int32
   return launched(nm);
 }
 
+int lmoe_silu_l2norm_fwd(const void* x, void* y, int64_t rows, int32_t D, int32_t dtype, float eps, void* stream) {
+  const char* nm = "lmoe_silu_l2norm_fwd";
+  if (int r = check_l2norm(nm, x, y, rows, D, dtype)) return r;
+  if (rows == 0) return 0;
+  lmoe::launch_silu_l2norm(dtype, D, x, nullptr, y, rows, eps, false, (hipStream_t)stream);
+  return launched(nm);
+}
+int lmoe_silu_l2norm_bwd(const void* x, const void* dy, void* dx, int64_t rows, int32_t D, int32_t dtype, float eps,
+                         void* stream) {
+  const char* nm = "lmoe_silu_l2norm_bwd";
+  if (int r = check_l2norm(nm, x, dx, rows, D, dtype)) return r;
+  if (!dy || ((uintptr_t)dy & 15)) return fail(-1, "%s: dy must be a 16-byte aligned pointer", nm);
+  if (rows == 0) return 0;
+  lmoe::launch_silu_l2norm(dtype, D, x, dy, dx, rows, eps, true, (hipStream_t)stream);
+  return launched(nm);
+}
+
+int lmoe_rmsnorm_partials(int64_t rows, int32_t D, int32_t dtype) {
+  const char* nm = "lmoe_rmsnorm_partials";
+  if (dtype != LMOE_BF16 && dtype != LMOE_F32) return fail(-2, "%s: dtype must be LMOE_BF16 or LMOE_F32", nm);
+  if (D != 64 && D != 128 && D != 256) return fail(-3, "%s: row length %d unsupported (64, 128 or 256)", nm, D);
+  if (rows < 0) return fail(-4, "%s: negative row count", nm);
+  return lmoe::rmsnorm_partials(dtype, D, rows);
+}
+int lmoe_rmsnorm_fwd(const void* x, const void* w, const void* gate, void* y, float* rstd, int64_t rows, int32_t D,
+                     int32_t dtype, float eps, void* stream) {
+  const char* nm = "lmoe_rmsnorm_fwd";
+  if (int r = check_l2norm(nm, x, y, rows, D, dtype)) return r;
+  if (((uintptr_t)w | (uintptr_t)gate) & 15) return fail(-9, "%s: pointers must be 16-byte aligned", nm);
+  if (rows == 0) return 0;
+  lmoe::launch_rmsnorm(dtype, D, x, w, gate, nullptr, y, nullptr, rstd, nullptr, nullptr, rows, eps, false,
+                       (hipStream_t)stream);
+  return launched(nm);
+}
+int lmoe_rmsnorm_bwd(const void* x, const void* w, const void* gate, const void* dy, void* dx, void* dgate,
+                     float* dw_part, float* dw, int64_t rows, int32_t D, int32_t dtype, float eps, void* stream) {
+  const char* nm = "lmoe_rmsnorm_bwd";
+  if (int r = check_l2norm(nm, x, dx, rows, D, dtype)) return r;
+  if (!dy) return fail(-1, "%s: dy must not be null", nm);
+  if (((uintptr_t)w | (uintptr_t)gate | (uintptr_t)dy | (uintptr_t)dgate) & 15)
+    return fail(-9, "%s: pointers must be 16-byte aligned", nm);
+  if ((gate != nullptr) != (dgate != nullptr)) return fail(-1, "%s: gate and dgate go together", nm);
+  if ((dw_part != nullptr) != (dw != nullptr)) return fail(-1, "%s: dw_part and dw go together", nm);
+  if (rows == 0) return 0;              // nothing to do (dw is not written)
+  lmoe::launch_rmsnorm(dtype, D, x, w, gate, dy, dx, dgate, nullptr, dw_part, dw, rows, eps, true, (hipStream_t)stream);
+  return launched(nm);
+}
+
 int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* stream) {
   const char* nm = "lmoe_launch_stage";
   if (int r = check_common(a, nm)) return r;

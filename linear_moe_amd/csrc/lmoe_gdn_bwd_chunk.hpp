@@ -316,6 +316,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
   }
 
   // --------------------------------- compute ---------------------------------------------
+  __builtin_amdgcn_s_setprio(3);           // compute waves before the loader wave of their SIMD
   const int wv = wave_id();
   const int r0 = 16 * (wv & 3);            // rows of this wave
   const int ch = wv >> 2;                  // column half

@@ -197,6 +197,9 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
   }
 
   // --------------------------------- consumers -------------------------------------------
+  // the waves that carry the recurrence win every issue slot they ask for over the loader waves of
+  // their SIMD
+  __builtin_amdgcn_s_setprio(3);
   const int wv = wave_id();
   const int krow0 = wv * (K / 4);
   const int fr = l & 15, fg = 8 * (l >> 4);          // fragment row / contraction offset of this lane
@@ -430,6 +433,9 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
   }
 
   // --------------------------------- consumers -------------------------------------------
+  // the waves that carry the recurrence win every issue slot they ask for over the loader waves of
+  // their SIMD
+  __builtin_amdgcn_s_setprio(3);
   const int wv = wave_id();
   const int krow0 = wv * (K / 4);
   const int fr = l & 15, fg = 8 * (l >> 4);

@@ -45,5 +45,12 @@ void launch_gla(const lmoe_args& a, int stage, hipStream_t st);
 // row-wise L2 normalisation of `rows` contiguous rows of D in {64, 128, 256} elements (bwd: out = dx)
 void launch_l2norm(int dtype, int D, const void* x, const void* dy, void* out, int64_t rows, float eps, bool bwd,
                    hipStream_t st);
+// RMS norm of `rows` contiguous rows (w, gate may be null); bwd: out = dx, dw_part = [rmsnorm_partials()][D]
+void launch_rmsnorm(int dtype, int D, const void* x, const void* w, const void* gate, const void* dy, void* out,
+                    void* dgate, float* rstd, float* dw_part, float* dw, int64_t rows, float eps, bool bwd, hipStream_t st);
+int rmsnorm_partials(int dtype, int D, int64_t rows);
+// y = l2norm(silu(x)) (bwd: out = dx)
+void launch_silu_l2norm(int dtype, int D, const void* x, const void* dy, void* out, int64_t rows, float eps, bool bwd,
+                        hipStream_t st);
 void launch_selftest(int dtype, int kd, const void* A, const void* B, float* C, float* G, hipStream_t st);
 }  // namespace lmoe

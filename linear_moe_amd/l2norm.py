@@ -17,7 +17,7 @@ _DIMS = (64, 128, 256)
 
 class _L2Norm(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, eps):
+    def forward(ctx, x, eps, silu=False):
         if not x.is_cuda:
             raise RuntimeError("linear_moe_amd ops are GPU only (no CPU fallback)")
         if x.dtype not in (torch.bfloat16, torch.float32):
@@ -29,9 +29,10 @@ class _L2Norm(torch.autograd.Function):
         xc = x.contiguous()
         y = torch.empty_like(xc)
         dt = _lib.LMOE_F32 if x.dtype == torch.float32 else _lib.LMOE_BF16
-        _lib.check(lib.lmoe_l2norm_fwd(xc.data_ptr(), y.data_ptr(), xc.numel() // D, D, dt, eps, stream_ptr()), "l2_norm")
+        fwd = lib.lmoe_silu_l2norm_fwd if silu else lib.lmoe_l2norm_fwd
+        _lib.check(fwd(xc.data_ptr(), y.data_ptr(), xc.numel() // D, D, dt, eps, stream_ptr()), "l2_norm")
         ctx.save_for_backward(xc)
-        ctx.eps, ctx.dt = eps, dt
+        ctx.eps, ctx.dt, ctx.silu = eps, dt, silu
         return y
 
     @staticmethod
@@ -41,13 +42,20 @@ class _L2Norm(torch.autograd.Function):
         D = xc.shape[-1]
         dyc = dy.contiguous()
         dx = torch.empty_like(xc)
-        _lib.check(lib.lmoe_l2norm_bwd(xc.data_ptr(), dyc.data_ptr(), dx.data_ptr(), xc.numel() // D, D, ctx.dt, ctx.eps,
-                                       stream_ptr()), "l2_norm backward")
-        return dx, None
+        bwd = lib.lmoe_silu_l2norm_bwd if ctx.silu else lib.lmoe_l2norm_bwd
+        _lib.check(bwd(xc.data_ptr(), dyc.data_ptr(), dx.data_ptr(), xc.numel() // D, D, ctx.dt, ctx.eps, stream_ptr()),
+                   "l2_norm backward")
+        return dx, None, None
 
 
 def l2_norm(x: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
     return _L2Norm.apply(x, eps)
+
+
+def silu_l2_norm(x: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
+    """``l2_norm(silu(x))`` in one pass: what the reference does to q and k of the gated delta rule in two
+    (``linear_moe/sequence_modeling/gated_deltanet/gated_deltanet.py:101`` then ``:105-106``)."""
+    return _L2Norm.apply(x, eps, True)
 
 
 l2_norm_fn = l2_norm

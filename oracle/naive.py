@@ -250,3 +250,24 @@ def naive_l2_norm(x: Tensor, eps: float = 1e-6, dtype=torch.float64) -> Tensor:
     of the gradient too)."""
     x = x.to(dtype)
     return x / torch.sqrt((x * x).sum(-1, keepdim=True) + eps)
+
+
+def naive_rms_norm(x: Tensor, weight: Tensor = None, gate: Tensor = None, eps: float = 1e-5, dtype=torch.float64) -> Tensor:
+    """y = x / sqrt(mean(x^2) + eps) * weight [* gate * sigmoid(gate)] over the last dimension
+    (linear_moe/model/common_modules/layernorm.py:113-127 with IS_RMS_NORM: var = sum(x^2) / N,
+    rstd = 1 / sqrt(var + eps), y = x * rstd * w; the gate product is linear_attention.py:255,
+    ``o * swish(o_gate)``).  Autograd through this expression is the oracle of the backward."""
+    x = x.to(dtype)
+    y = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+    if weight is not None:
+        y = y * weight.to(dtype)
+    if gate is not None:
+        g = gate.to(dtype)
+        y = y * g * torch.sigmoid(g)
+    return y
+
+
+def naive_silu_l2_norm(x: Tensor, eps: float = 1e-6, dtype=torch.float64) -> Tensor:
+    """l2_norm(silu(x)) (gated_deltanet.py:101 then :105-106)."""
+    x = x.to(dtype)
+    return naive_l2_norm(x * torch.sigmoid(x), eps, dtype)

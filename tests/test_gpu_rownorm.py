@@ -1,0 +1,82 @@
+"""GPU parity of the row-wise neighbours of the chunk ops (RMS norm with optional swish gate, SiLU + L2
+norm; HIP, through the C ABI) against the fp64 oracle."""
+import pytest
+import torch
+
+from oracle import naive
+from tests.util import TOL, gen, max_abs_rel
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("D", [64, 128, 256])
+@pytest.mark.parametrize("gated", [False, True])
+def test_rms_norm_fwd_bwd(cuda, dtype, D, gated):
+    from linear_moe_amd import rms_norm_fn, rms_norm_swish_gate
+    x = gen(1100 + D, 2, 3, 41, D, dtype=dtype)
+    w = (1.0 + 0.2 * gen(1101 + D, D)).to(dtype)
+    gate = gen(1102 + D, 2, 3, 41, D, dtype=dtype) if gated else None
+    dy = gen(1103 + D, 2, 3, 41, D, dtype=dtype)
+    xr, wr = x.double().requires_grad_(True), w.double().requires_grad_(True)
+    gr = gate.double().requires_grad_(True) if gated else None
+    ref = naive.naive_rms_norm(xr, wr, gr, eps=1e-5)
+    (ref * dy.double()).sum().backward()
+    xd, wd = x.to(cuda).requires_grad_(True), w.to(cuda).requires_grad_(True)
+    gd = gate.to(cuda).requires_grad_(True) if gated else None
+    y = rms_norm_swish_gate(xd, gd, wd, eps=1e-5) if gated else rms_norm_fn(xd, wd, None, eps=1e-5)
+    (y * dy.to(cuda)).sum().backward()
+    torch.cuda.synchronize()
+    assert y.dtype == dtype and y.shape == x.shape
+    assert max_abs_rel(y.detach().cpu(), ref.detach()) < TOL[dtype]
+    assert max_abs_rel(xd.grad.cpu(), xr.grad) < TOL[dtype]
+    assert wd.grad.dtype == dtype
+    assert max_abs_rel(wd.grad.cpu(), wr.grad) < TOL[dtype]
+    if gated:
+        assert max_abs_rel(gd.grad.cpu(), gr.grad) < TOL[dtype]
+
+
+def test_rms_norm_module_and_many_rows(cuda):
+    """The module with the reference's constructor; enough rows that every work-group loops and the
+    weight gradient goes through many partial rows; run twice: bit-identical (fixed summation order)."""
+    from linear_moe_amd import RMSNorm
+    m = RMSNorm(128, eps=1e-5).to(cuda)
+    with torch.no_grad():
+        m.weight.copy_(1.0 + 0.1 * gen(1201, 128))
+    x = gen(1202, 4, 16, 2048, 128)
+    dy = gen(1203, 4, 16, 2048, 128)
+    xr, wr = x.double().requires_grad_(True), m.weight.detach().cpu().double().requires_grad_(True)
+    (naive.naive_rms_norm(xr, wr, None, eps=1e-5) * dy.double()).sum().backward()
+    grads = []
+    for _ in range(2):
+        m.weight.grad = None
+        xd = x.to(cuda).requires_grad_(True)
+        (m(xd) * dy.to(cuda)).sum().backward()
+        torch.cuda.synchronize()
+        grads.append((xd.grad.clone(), m.weight.grad.clone()))
+    assert max_abs_rel(grads[0][0].cpu(), xr.grad) < 1e-5
+    assert max_abs_rel(grads[0][1].cpu(), wr.grad) < 1e-5
+    assert torch.equal(grads[0][0], grads[1][0]) and torch.equal(grads[0][1], grads[1][1])
+    no_affine = RMSNorm(64, elementwise_affine=False).to(cuda)
+    xs = gen(1204, 5, 64)
+    assert max_abs_rel(no_affine(xs.to(cuda)).cpu(), naive.naive_rms_norm(xs, eps=1e-5)) < 1e-5
+    with pytest.raises(ValueError):
+        RMSNorm(48).to(cuda)(torch.zeros(3, 48, device=cuda))
+    assert m(torch.zeros(0, 128, device=cuda)).shape == (0, 128)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("D", [64, 128])
+def test_silu_l2_norm_fwd_bwd(cuda, dtype, D):
+    from linear_moe_amd import silu_l2_norm
+    x = gen(1300 + D, 2, 37, 3, D, dtype=dtype)
+    dy = gen(1301 + D, 2, 37, 3, D, dtype=dtype)
+    xr = x.double().requires_grad_(True)
+    ref = naive.naive_silu_l2_norm(xr, eps=1e-6)
+    (ref * dy.double()).sum().backward()
+    xd = x.to(cuda).requires_grad_(True)
+    y = silu_l2_norm(xd)
+    (y * dy.to(cuda)).sum().backward()
+    torch.cuda.synchronize()
+    assert max_abs_rel(y.detach().cpu(), ref.detach()) < TOL[dtype]
+    assert max_abs_rel(xd.grad.cpu(), xr.grad) < TOL[dtype]

@@ -288,3 +288,34 @@ def test_l2_norm_pins():
     rstd = 1.0 / torch.sqrt(var + 1e-6)
     want = dy * rstd - (dy * x).sum(-1, keepdim=True) * (1.0 / (var + 1e-6)) * rstd * x
     assert torch.allclose(xr.grad, want, atol=1e-12)
+
+
+def test_rms_norm_pins():
+    """naive_rms_norm: torch's own rms_norm and F.silu (independent library routines), hand-computed
+    values that place eps inside the square root and use the mean (not the sum) of squares, and the
+    backward formulas of the reference kernel (layernorm.py:266-286: wdy = w dy, c1 = mean(x^ wdy),
+    dx = (wdy - x^ c1) rstd, dw = sum dy x^) against autograd through the oracle."""
+    import torch.nn.functional as F
+    x = rnd(7101, 4, 3, 16).double()
+    w = rnd(7102, 16).double()
+    gate = rnd(7103, 4, 3, 16).double()
+    assert torch.allclose(naive.naive_rms_norm(x, w, None, eps=1e-5), F.rms_norm(x, (16,), w, 1e-5), atol=1e-13)
+    assert torch.allclose(naive.naive_rms_norm(x, w, gate, eps=1e-5), F.rms_norm(x, (16,), w, 1e-5) * F.silu(gate), atol=1e-13)
+    v = torch.tensor([[3.0, 4.0]], dtype=torch.float64)                      # mean of squares 12.5
+    assert torch.allclose(naive.naive_rms_norm(v, eps=0.0), v / 12.5 ** 0.5)
+    assert torch.allclose(naive.naive_rms_norm(v, eps=3.5), v / 4.0)          # sqrt(12.5 + 3.5) = 4
+    xr, wr = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    dy = rnd(7104, 4, 3, 16).double()
+    (naive.naive_rms_norm(xr, wr, None, eps=1e-5) * dy).sum().backward()
+    rstd = 1.0 / torch.sqrt((x * x).mean(-1, keepdim=True) + 1e-5)
+    xhat, wdy = x * rstd, w * dy
+    c1 = (xhat * wdy).mean(-1, keepdim=True)
+    assert torch.allclose(xr.grad, (wdy - xhat * c1) * rstd, atol=1e-12)
+    assert torch.allclose(wr.grad, (dy * xhat).sum((0, 1)), atol=1e-12)
+
+
+def test_silu_l2_norm_pins():
+    import torch.nn.functional as F
+    x = rnd(7201, 3, 5, 16).double()
+    assert torch.allclose(naive.naive_silu_l2_norm(x, eps=0.0), F.normalize(F.silu(x), dim=-1, eps=0.0), atol=1e-14)
+    assert torch.allclose(naive.naive_silu_l2_norm(x, eps=1e-6), naive.naive_l2_norm(F.silu(x), eps=1e-6), atol=1e-15)
