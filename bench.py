@@ -118,6 +118,50 @@ def cpu_baseline(B, T, H, K, V, seed, min_seconds=10.0):
                       f"torch port, {dt:.1f} s"}
 
 
+def neighbours(lib, rows, D, dev, reps):
+    """Row-wise kernels around the op on `rows` x D bf16 (the q / k / o rows of the headline workload):
+    seconds per launch from events on the launch stream, and algorithmic GB/s (every operand read
+    once, every result written once) against the HBM peak."""
+    import torch
+    from linear_moe_amd import _lib
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    mk = lambda: torch.randn(rows, D, device=dev, dtype=torch.bfloat16)
+    x, dy, gate, out, out2 = mk(), mk(), mk(), mk(), mk()
+    w = torch.ones(D, device=dev, dtype=torch.bfloat16)
+    part = torch.empty(lib.lmoe_rmsnorm_partials(rows, D, _lib.LMOE_BF16), D, device=dev, dtype=torch.float32)
+    dw = torch.empty(D, device=dev, dtype=torch.float32)
+    p = lambda t: C.c_void_p(t.data_ptr())
+    bf = _lib.LMOE_BF16
+    cases = {   # name: (launch, tensors of rows x D moved)
+        "l2norm_fwd": (lambda: lib.lmoe_l2norm_fwd(p(x), p(out), rows, D, bf, 1e-6, st), 2),
+        "l2norm_bwd": (lambda: lib.lmoe_l2norm_bwd(p(x), p(dy), p(out), rows, D, bf, 1e-6, st), 3),
+        "silu_l2norm_fwd": (lambda: lib.lmoe_silu_l2norm_fwd(p(x), p(out), rows, D, bf, 1e-6, st), 2),
+        "silu_l2norm_bwd": (lambda: lib.lmoe_silu_l2norm_bwd(p(x), p(dy), p(out), rows, D, bf, 1e-6, st), 3),
+        "rmsnorm_fwd": (lambda: lib.lmoe_rmsnorm_fwd(p(x), p(w), None, p(out), None, rows, D, bf, 1e-5, st), 2),
+        "rmsnorm_bwd": (lambda: lib.lmoe_rmsnorm_bwd(p(x), p(w), None, p(dy), p(out), None, p(part), p(dw), rows, D, bf,
+                                                     1e-5, st), 3),
+        "rmsnorm_gate_fwd": (lambda: lib.lmoe_rmsnorm_fwd(p(x), p(w), p(gate), p(out), None, rows, D, bf, 1e-5, st), 3),
+        "rmsnorm_gate_bwd": (lambda: lib.lmoe_rmsnorm_bwd(p(x), p(w), p(gate), p(dy), p(out), p(out2), p(part), p(dw),
+                                                          rows, D, bf, 1e-5, st), 5),
+    }
+    res = {}
+    for name, (launch, ntens) in cases.items():
+        for _ in range(3):
+            _lib.check(launch(), name)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            launch()
+        e1.record()
+        e1.synchronize()
+        sec = e0.elapsed_time(e1) * 1e-3 / reps
+        nbytes = ntens * rows * D * 2
+        res[name] = {"us": round(sec * 1e6, 1), "bytes": nbytes, "GB/s": round(nbytes / sec / 1e9, 1),
+                     "frac_hbm_peak": round(nbytes / sec / PEAK_HBM, 3)}
+    return {"metric": "row-wise neighbour kernels, algorithmic GB/s", "unit": "GB/s", "dtype": "bf16",
+            "config": {"workload": f"{rows} rows x {D} bf16 (q / k / o rows of B=4 H=16 T=8192)"}, "kernels": res}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -125,6 +169,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--stage-reps", type=int, default=20)
+    ap.add_argument("--neighbours", action="store_true",
+                    help="instead of the headline step: the row-wise kernels around the op (L2 norm, SiLU + L2 norm, "
+                         "RMS norm with and without the swish gate) on the rows of the same workload, one JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the op shards over batch and heads without "
@@ -140,6 +187,9 @@ def main():
     lib = _lib.load()
     dev = torch.device("cuda:0")
     B, T, H, K, V, seed = 4, 8192, 16, 128, 128, 1004
+    if args.neighbours:
+        print(json.dumps(neighbours(lib, B * T * H, K, dev, args.stage_reps)))
+        return
     x = gdn_inputs(B, T, H, K, V, seed, torch.bfloat16, dev)
 
     # known-size device copy: the yardstick for the FETCH_SIZE / WRITE_SIZE counters under rocprofv3

@@ -166,6 +166,26 @@ int lmoe_rmsnorm_fwd(const void* x, const void* w, const void* gate, void* y, fl
 int lmoe_rmsnorm_bwd(const void* x, const void* w, const void* gate, const void* dy, void* dx, void* dgate,
                      float* dw_part, float* dw, int64_t rows, int32_t D, int32_t dtype, float eps, void* stream);
 
+/* Gate construction of the gated delta rule for a, b of shape [rows][H] (element type by dtype):
+ *   beta = sigmoid(b)  (element type of b),   g = -exp(A_log[h]) softplus(a + dt_bias[h])  (fp32)
+ * as linear_moe/sequence_modeling/linear_attention.py:153-154 forms them in front of the op (parameters
+ * :92-113).  Backward: da, db in the element type, dparams = [dA_log | ddt_bias] ([2][H] fp32) through
+ * `part`, a caller-allocated fp32 [lmoe_gdn_gates_partials(rows, H)][2][H] workspace summed in a fixed order. */
+int lmoe_gdn_gates_partials(int64_t rows, int32_t H);
+int lmoe_gdn_gates_fwd(const void* a, const void* b, const float* A_log, const float* dt_bias, float* g, void* beta,
+                       int64_t rows, int32_t H, int32_t dtype, void* stream);
+int lmoe_gdn_gates_bwd(const void* a, const void* b, const float* A_log, const float* dt_bias, const float* dg,
+                       const void* dbeta, void* da, void* db, float* part, float* dparams, int64_t rows, int32_t H,
+                       int32_t dtype, void* stream);
+
+/* Gate of chunk_gla over n contiguous elements (n a multiple of 8, 16-byte aligned):
+ *   gk = max(logsigmoid(x) / normalizer, clamp_min)      (clamp_min = -INFINITY: no clamp)
+ * as linear_moe/sequence_modeling/gla/gla.py:85 (normalizer) and :90-91 (clamp_min); backward
+ *   dx = dy (1 - sigmoid(x)) / normalizer where gk > clamp_min, else 0. */
+int lmoe_gla_gate_fwd(const void* x, void* y, int64_t n, int32_t dtype, float normalizer, float clamp_min, void* stream);
+int lmoe_gla_gate_bwd(const void* x, const void* dy, void* dx, int64_t n, int32_t dtype, float normalizer,
+                      float clamp_min, void* stream);
+
 /* Launch ONE kernel of an op's pipeline (profiling support: lets a harness time each kernel
  * with events on its own stream).  `a` must be the fully populated argument block of the
  * op's fwd (stages 0-2, 7) or bwd (stages 3-5) entry point, with the intermediates of the

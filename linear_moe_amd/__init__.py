@@ -7,6 +7,7 @@ All compute runs in hand-written HIP kernels (``csrc/``) reached through the C A
 """
 from .delta_rule import chunk_delta_rule  # noqa: F401
 from .gated_delta_rule import chunk_gated_delta_rule  # noqa: F401
+from .gates import gdn_gates, gla_gate  # noqa: F401
 from .gla import chunk_gla  # noqa: F401
 from .l2norm import l2_norm, l2_norm_fn, silu_l2_norm  # noqa: F401
 from .rmsnorm import RMSNorm, rms_norm_fn, rms_norm_swish_gate  # noqa: F401
@@ -16,4 +17,5 @@ from .retention import chunk_retention  # noqa: F401
 from .simple_gla import chunk_simple_gla  # noqa: F401
 
 __all__ = ["chunk_simple_gla", "chunk_gla", "chunk_gated_delta_rule", "chunk_delta_rule", "chunk_retention", "chunk_linear_attn",
-           "lightning_attn2", "lightning_attn2_no_decay", "l2_norm", "l2_norm_fn"]
+           "lightning_attn2", "lightning_attn2_no_decay", "l2_norm", "l2_norm_fn", "silu_l2_norm", "rms_norm_fn",
+           "rms_norm_swish_gate", "RMSNorm", "gdn_gates", "gla_gate"]

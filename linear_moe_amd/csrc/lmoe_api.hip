@@ -219,6 +219,63 @@ int lmoe_rmsnorm_bwd(const void* x, const void* w, const void* gate, const void*
   return launched(nm);
 }
 
+static int check_gates(const char* nm, int64_t rows, int32_t H, int32_t dtype) {
+  if (dtype != LMOE_BF16 && dtype != LMOE_F32) return fail(-2, "%s: dtype must be LMOE_BF16 or LMOE_F32", nm);
+  if (H <= 0 || H > 256) return fail(-3, "%s: H = %d outside 1..256", nm, H);
+  if (rows < 0) return fail(-4, "%s: negative row count", nm);
+  return 0;
+}
+int lmoe_gdn_gates_partials(int64_t rows, int32_t H) {
+  if (int r = check_gates("lmoe_gdn_gates_partials", rows, H, LMOE_F32)) return r;
+  return lmoe::gdn_gates_partials(rows, H);
+}
+int lmoe_gdn_gates_fwd(const void* a, const void* b, const float* A_log, const float* dt_bias, float* g, void* beta,
+                       int64_t rows, int32_t H, int32_t dtype, void* stream) {
+  const char* nm = "lmoe_gdn_gates_fwd";
+  if (int r = check_gates(nm, rows, H, dtype)) return r;
+  if (!a || !b || !A_log || !dt_bias || !g || !beta) return fail(-1, "%s: null pointer", nm);
+  if (rows == 0) return 0;
+  lmoe::launch_gdn_gates(dtype, a, b, A_log, dt_bias, g, beta, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, rows,
+                         H, false, (hipStream_t)stream);
+  return launched(nm);
+}
+int lmoe_gdn_gates_bwd(const void* a, const void* b, const float* A_log, const float* dt_bias, const float* dg,
+                       const void* dbeta, void* da, void* db, float* part, float* dparams, int64_t rows, int32_t H,
+                       int32_t dtype, void* stream) {
+  const char* nm = "lmoe_gdn_gates_bwd";
+  if (int r = check_gates(nm, rows, H, dtype)) return r;
+  if (!a || !b || !A_log || !dt_bias || !dg || !dbeta || !da || !db || !dparams) return fail(-1, "%s: null pointer", nm);
+  if (rows == 0) return 0;
+  if (!part) return fail(-1, "%s: part must not be null", nm);
+  lmoe::launch_gdn_gates(dtype, a, b, A_log, dt_bias, nullptr, nullptr, dg, dbeta, da, db, part, dparams, rows, H, true,
+                         (hipStream_t)stream);
+  return launched(nm);
+}
+static int check_gla_gate(const char* nm, const void* x, const void* out, int64_t n, int32_t dtype, float normalizer) {
+  if (!x || !out) return fail(-1, "%s: null pointer", nm);
+  if (dtype != LMOE_BF16 && dtype != LMOE_F32) return fail(-2, "%s: dtype must be LMOE_BF16 or LMOE_F32", nm);
+  if (n < 0 || n % 8) return fail(-4, "%s: element count must be a non-negative multiple of 8", nm);
+  if (!(normalizer > 0.f)) return fail(-5, "%s: normalizer must be positive", nm);
+  if (((uintptr_t)x | (uintptr_t)out) & 15) return fail(-9, "%s: pointers must be 16-byte aligned", nm);
+  return 0;
+}
+int lmoe_gla_gate_fwd(const void* x, void* y, int64_t n, int32_t dtype, float normalizer, float clamp_min, void* stream) {
+  const char* nm = "lmoe_gla_gate_fwd";
+  if (int r = check_gla_gate(nm, x, y, n, dtype, normalizer)) return r;
+  if (n == 0) return 0;
+  lmoe::launch_gla_gate(dtype, x, nullptr, y, n, normalizer, clamp_min, false, (hipStream_t)stream);
+  return launched(nm);
+}
+int lmoe_gla_gate_bwd(const void* x, const void* dy, void* dx, int64_t n, int32_t dtype, float normalizer,
+                      float clamp_min, void* stream) {
+  const char* nm = "lmoe_gla_gate_bwd";
+  if (int r = check_gla_gate(nm, x, dx, n, dtype, normalizer)) return r;
+  if (!dy || ((uintptr_t)dy & 15)) return fail(-1, "%s: dy must be a 16-byte aligned pointer", nm);
+  if (n == 0) return 0;
+  lmoe::launch_gla_gate(dtype, x, dy, dx, n, normalizer, clamp_min, true, (hipStream_t)stream);
+  return launched(nm);
+}
+
 int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* stream) {
   const char* nm = "lmoe_launch_stage";
   if (int r = check_common(a, nm)) return r;

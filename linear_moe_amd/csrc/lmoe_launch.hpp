@@ -52,5 +52,13 @@ int rmsnorm_partials(int dtype, int D, int64_t rows);
 // y = l2norm(silu(x)) (bwd: out = dx)
 void launch_silu_l2norm(int dtype, int D, const void* x, const void* dy, void* out, int64_t rows, float eps, bool bwd,
                         hipStream_t st);
+// gate construction of the gated delta rule (rows x H elements; bwd also fills dparams = [dA_log | ddt_bias])
+void launch_gdn_gates(int dtype, const void* a, const void* b, const float* A_log, const float* dt_bias, float* g,
+                      void* beta, const float* dg, const void* dbeta, void* da, void* db, float* part, float* dparams,
+                      int64_t rows, int H, bool bwd, hipStream_t st);
+int gdn_gates_partials(int64_t rows, int H);
+// chunk_gla gate: logsigmoid(x) / normalizer, clamped from below (n elements, a multiple of 8)
+void launch_gla_gate(int dtype, const void* x, const void* dy, void* out, int64_t n, float normalizer, float clamp_min,
+                     bool bwd, hipStream_t st);
 void launch_selftest(int dtype, int kd, const void* A, const void* B, float* C, float* G, hipStream_t st);
 }  // namespace lmoe

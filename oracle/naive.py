@@ -271,3 +271,18 @@ def naive_silu_l2_norm(x: Tensor, eps: float = 1e-6, dtype=torch.float64) -> Ten
     """l2_norm(silu(x)) (gated_deltanet.py:101 then :105-106)."""
     x = x.to(dtype)
     return naive_l2_norm(x * torch.sigmoid(x), eps, dtype)
+
+
+def naive_gdn_gates(a: Tensor, b: Tensor, A_log: Tensor, dt_bias: Tensor, dtype=torch.float64):
+    """(g, beta) of the gated delta rule (linear_moe/sequence_modeling/linear_attention.py:153-154):
+    beta = sigmoid(b), g = -exp(A_log) * softplus(a + dt_bias)."""
+    import torch.nn.functional as F
+    g = -torch.exp(A_log.to(dtype)) * F.softplus(a.to(dtype) + dt_bias.to(dtype))
+    return g, torch.sigmoid(b.to(dtype))
+
+
+def naive_gla_gate(x: Tensor, normalizer: float = 16.0, clamp_min=None, dtype=torch.float64) -> Tensor:
+    """gk of chunk_gla (linear_moe/sequence_modeling/gla/gla.py:85, :90-91)."""
+    import torch.nn.functional as F
+    y = F.logsigmoid(x.to(dtype)) / normalizer
+    return y if clamp_min is None else torch.clamp_min(y, clamp_min)

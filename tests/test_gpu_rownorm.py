@@ -80,3 +80,57 @@ def test_silu_l2_norm_fwd_bwd(cuda, dtype, D):
     torch.cuda.synchronize()
     assert max_abs_rel(y.detach().cpu(), ref.detach()) < TOL[dtype]
     assert max_abs_rel(xd.grad.cpu(), xr.grad) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H", [16, 12, 32])
+def test_gdn_gates_fwd_bwd(cuda, dtype, H):
+    """Gate construction of the gated delta rule with the reference's parameter laws (A ~ U(0, 16),
+    dt log-uniform in [1e-3, 0.1] -> dt_bias = softplus^-1(dt)); enough rows for several partial rows."""
+    import math
+    from linear_moe_amd import gdn_gates
+    B, T = 3, 1031
+    a = 2.0 * gen(1400 + H, B, T, H, dtype=dtype)
+    b = 2.0 * gen(1401 + H, B, T, H, dtype=dtype)
+    gg = torch.Generator().manual_seed(1402 + H)
+    A_log = torch.log(torch.rand(H, generator=gg) * 16 + 1e-3)
+    dtv = torch.exp(torch.rand(H, generator=gg) * (math.log(0.1) - math.log(1e-3)) + math.log(1e-3)).clamp(min=1e-4)
+    dt_bias = dtv + torch.log(-torch.expm1(-dtv))
+    dg, dbeta = gen(1403 + H, B, T, H), gen(1404 + H, B, T, H, dtype=dtype)
+    ar, br = a.double().requires_grad_(True), b.double().requires_grad_(True)
+    Ar, Dr = A_log.double().requires_grad_(True), dt_bias.double().requires_grad_(True)
+    g_ref, beta_ref = naive.naive_gdn_gates(ar, br, Ar, Dr)
+    ((g_ref * dg.double()).sum() + (beta_ref * dbeta.double()).sum()).backward()
+    ad, bd = a.to(cuda).requires_grad_(True), b.to(cuda).requires_grad_(True)
+    Ad, Dd = A_log.to(cuda).requires_grad_(True), dt_bias.to(cuda).requires_grad_(True)
+    g, beta = gdn_gates(ad, bd, Ad, Dd)
+    ((g * dg.to(cuda)).sum() + (beta.float() * dbeta.to(cuda).float()).sum()).backward()
+    torch.cuda.synchronize()
+    assert g.dtype == torch.float32 and beta.dtype == dtype
+    tol = TOL[dtype]
+    assert max_abs_rel(g.detach().cpu(), g_ref.detach()) < (1e-5 if dtype == torch.float32 else tol)
+    assert max_abs_rel(beta.detach().cpu(), beta_ref.detach()) < tol
+    assert max_abs_rel(ad.grad.cpu(), ar.grad) < tol
+    assert max_abs_rel(bd.grad.cpu(), br.grad) < tol
+    assert max_abs_rel(Ad.grad.cpu(), Ar.grad) < tol
+    assert max_abs_rel(Dd.grad.cpu(), Dr.grad) < tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("clamp", [None, -0.05])
+def test_gla_gate_fwd_bwd(cuda, dtype, clamp):
+    from linear_moe_amd import gla_gate
+    x = 3.0 * gen(1500, 2, 4, 133, 64, dtype=dtype)
+    dy = gen(1501, 2, 4, 133, 64, dtype=dtype)
+    xr = x.double().requires_grad_(True)
+    ref = naive.naive_gla_gate(xr, 16.0, clamp)
+    (ref * dy.double()).sum().backward()
+    xd = x.to(cuda).requires_grad_(True)
+    y = gla_gate(xd, 16.0, clamp)
+    (y * dy.to(cuda)).sum().backward()
+    torch.cuda.synchronize()
+    assert y.dtype == dtype and (y <= 0).all()
+    assert max_abs_rel(y.detach().cpu(), ref.detach()) < TOL[dtype]
+    # elements that sit on the clamp within rounding may go either way: compare away from it
+    far = (ref.detach() - (clamp if clamp is not None else -1e30)).abs() > 1e-3
+    assert max_abs_rel((xd.grad.cpu() * far), (xr.grad * far)) < TOL[dtype]

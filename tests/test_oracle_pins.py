@@ -319,3 +319,23 @@ def test_silu_l2_norm_pins():
     x = rnd(7201, 3, 5, 16).double()
     assert torch.allclose(naive.naive_silu_l2_norm(x, eps=0.0), F.normalize(F.silu(x), dim=-1, eps=0.0), atol=1e-14)
     assert torch.allclose(naive.naive_silu_l2_norm(x, eps=1e-6), naive.naive_l2_norm(F.silu(x), eps=1e-6), atol=1e-15)
+
+
+def test_gate_construction_pins():
+    """Hand-computed values: softplus(0) = log 2, sigmoid(0) = 1/2, logsigmoid(0) = -log 2; the limits
+    softplus(z) -> z and logsigmoid(z) -> z; the clamp; g <= 0 always."""
+    import math
+    z = torch.zeros(1, 2, dtype=torch.float64)
+    A_log = torch.tensor([0.0, math.log(3.0)], dtype=torch.float64)
+    g, beta = naive.naive_gdn_gates(z, z, A_log, torch.zeros(2, dtype=torch.float64))
+    assert torch.allclose(g, torch.tensor([[-math.log(2.0), -3.0 * math.log(2.0)]], dtype=torch.float64))
+    assert torch.allclose(beta, torch.full((1, 2), 0.5, dtype=torch.float64))
+    big = torch.full((1, 2), 40.0, dtype=torch.float64)
+    g2, _ = naive.naive_gdn_gates(big, z, A_log, torch.ones(2, dtype=torch.float64))
+    assert torch.allclose(g2, torch.tensor([[-41.0, -123.0]], dtype=torch.float64))
+    assert (naive.naive_gdn_gates(rnd(7301, 5, 2).double(), z, A_log, torch.zeros(2, dtype=torch.float64))[0] <= 0).all()
+    x = torch.tensor([0.0, -50.0, 50.0, -1.0], dtype=torch.float64)
+    y = naive.naive_gla_gate(x, 16.0)
+    assert torch.allclose(y[:3], torch.tensor([-math.log(2.0) / 16, -50.0 / 16, 0.0], dtype=torch.float64), atol=1e-15)
+    assert torch.allclose(y[3], torch.tensor(-math.log1p(math.e) / 16, dtype=torch.float64))
+    assert torch.equal(naive.naive_gla_gate(x, 16.0, clamp_min=-1.0)[1], torch.tensor(-1.0, dtype=torch.float64))
