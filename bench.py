@@ -144,8 +144,30 @@ def neighbours(lib, rows, D, dev, reps):
         "rmsnorm_gate_bwd": (lambda: lib.lmoe_rmsnorm_bwd(p(x), p(w), p(gate), p(dy), p(out), p(out2), p(part), p(dw),
                                                           rows, D, bf, 1e-5, st), 5),
     }
+    # gate construction: gated delta rule on [B*T][H] (a, b bf16 -> g fp32, beta bf16), chunk_gla on the
+    # gate tensor of contract config 3 ([8,16,2048,64] bf16)
+    Hh = 16
+    grows = rows // Hh
+    ga, gb = (torch.randn(grows, Hh, device=dev, dtype=torch.bfloat16) for _ in range(2))
+    gA, gD = torch.zeros(Hh, device=dev), torch.zeros(Hh, device=dev)
+    gg, gdg = torch.empty(grows, Hh, device=dev), torch.randn(grows, Hh, device=dev)
+    gbeta, gda, gdb = (torch.empty(grows, Hh, device=dev, dtype=torch.bfloat16) for _ in range(3))
+    gpart = torch.empty(lib.lmoe_gdn_gates_partials(grows, Hh), 2, Hh, device=dev)
+    gdpar = torch.empty(2, Hh, device=dev)
+    ngla = 8 * 16 * 2048 * 64
+    extra = {   # name: (launch, bytes moved)
+        "gdn_gates_fwd": (lambda: lib.lmoe_gdn_gates_fwd(p(ga), p(gb), p(gA), p(gD), p(gg), p(gbeta), grows, Hh, bf, st),
+                          grows * Hh * (2 + 2 + 4 + 2)),
+        "gdn_gates_bwd": (lambda: lib.lmoe_gdn_gates_bwd(p(ga), p(gb), p(gA), p(gD), p(gdg), p(gbeta), p(gda), p(gdb),
+                                                         p(gpart), p(gdpar), grows, Hh, bf, st),
+                          grows * Hh * (2 + 2 + 4 + 2 + 2 + 2)),
+        "gla_gate_fwd": (lambda: lib.lmoe_gla_gate_fwd(p(x), p(out), ngla, bf, 16.0, float("-inf"), st), ngla * 4),
+        "gla_gate_bwd": (lambda: lib.lmoe_gla_gate_bwd(p(x), p(dy), p(out), ngla, bf, 16.0, float("-inf"), st), ngla * 6),
+    }
     res = {}
-    for name, (launch, ntens) in cases.items():
+    cases = {n: (f, k * rows * D * 2) for n, (f, k) in cases.items()}
+    cases.update(extra)
+    for name, (launch, nbytes) in cases.items():
         for _ in range(3):
             _lib.check(launch(), name)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -155,7 +177,6 @@ def neighbours(lib, rows, D, dev, reps):
         e1.record()
         e1.synchronize()
         sec = e0.elapsed_time(e1) * 1e-3 / reps
-        nbytes = ntens * rows * D * 2
         res[name] = {"us": round(sec * 1e6, 1), "bytes": nbytes, "GB/s": round(nbytes / sec / 1e9, 1),
                      "frac_hbm_peak": round(nbytes / sec / PEAK_HBM, 3)}
     return {"metric": "row-wise neighbour kernels, algorithmic GB/s", "unit": "GB/s", "dtype": "bf16",
