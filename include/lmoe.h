@@ -198,6 +198,14 @@ int lmoe_gla_gate_bwd(const void* x, const void* dy, void* dx, int64_t n, int32_
 #define LMOE_OP_GATED_DELTA_RULE 2
 int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* stream);
 
+/* Token-by-token forward of an op (op = LMOE_OP_*; the delta rule without a gate: gate = LMOE_GATE_NONE):
+ * the state stays in registers, nothing is saved for a backward.  For decoding (T = 1 with h0 / ht) and
+ * short sequences.  Uses q, k, v, g, beta, h0, scale, cu_seqlens (+ seq_chunk0, chunk_map as for the chunk
+ * entry points) -> o, ht.  Stands where the reference selects fla's fused_recurrent_* callables
+ * (la_mode = 'fused_recurrent': linear_moe/sequence_modeling/gated_deltanet/gated_deltanet.py:72-73,
+ * gla/gla.py:58-59, deltanet/deltanet.py:81-82, basic_linear_attention/basic_linear_attention.py:99-100). */
+int lmoe_fused_recurrent_fwd(const lmoe_args* a, int32_t op, void* stream);
+
 /* Toolkit self-test over one pair of 64 x kd tiles A, B (element type by dtype, kd in {64,128}),
  * through the same tile loaders, MFMA fragments and accumulator stores the kernels use:
  * C[64][64] (fp32) = A B^T (contraction along tile columns), G[kd][kd] (fp32) = A^T B

@@ -48,6 +48,7 @@ ENTRY_POINTS = (
     "lmoe_launch_stage", "lmoe_selftest_gemm", "lmoe_workspace_bytes", "lmoe_l2norm_fwd", "lmoe_l2norm_bwd",
     "lmoe_silu_l2norm_fwd", "lmoe_silu_l2norm_bwd", "lmoe_rmsnorm_partials", "lmoe_rmsnorm_fwd", "lmoe_rmsnorm_bwd",
     "lmoe_gdn_gates_partials", "lmoe_gdn_gates_fwd", "lmoe_gdn_gates_bwd", "lmoe_gla_gate_fwd", "lmoe_gla_gate_bwd",
+    "lmoe_fused_recurrent_fwd",
 )
 
 _lib = None
@@ -101,6 +102,8 @@ def load() -> C.CDLL:
     lib.lmoe_gla_gate_bwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_float, C.c_float,
                                       C.c_void_p]
     lib.lmoe_gla_gate_bwd.restype = C.c_int
+    lib.lmoe_fused_recurrent_fwd.argtypes = [C.POINTER(Args), C.c_int32, C.c_void_p]
+    lib.lmoe_fused_recurrent_fwd.restype = C.c_int
     lib.lmoe_workspace_bytes.argtypes = [C.c_int32] * 9
     lib.lmoe_workspace_bytes.restype = C.c_int64
     _lib = lib

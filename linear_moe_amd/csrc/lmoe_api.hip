@@ -219,6 +219,20 @@ int lmoe_rmsnorm_bwd(const void* x, const void* w, const void* gate, const void*
   return launched(nm);
 }
 
+int lmoe_fused_recurrent_fwd(const lmoe_args* a, int32_t op, void* stream) {
+  const char* nm = "lmoe_fused_recurrent_fwd";
+  if (int r = check_common(a, nm)) return r;
+  if (op != LMOE_OP_SIMPLE_GLA && op != LMOE_OP_GLA && op != LMOE_OP_GATED_DELTA_RULE)
+    return fail(-21, "%s: unknown op %d", nm, op);
+  if (!a->o.ptr) return fail(-11, "%s: o must not be null", nm);
+  if (op == LMOE_OP_GLA && (a->gate != LMOE_GATE_VECTOR || !a->g.ptr)) return fail(-10, "%s: chunk_gla needs a vector gate", nm);
+  if (op != LMOE_OP_GLA && a->gate == LMOE_GATE_VECTOR) return fail(-10, "%s: vector gates belong to LMOE_OP_GLA", nm);
+  if (op == LMOE_OP_GATED_DELTA_RULE && !a->beta.ptr) return fail(-12, "%s: beta must not be null", nm);
+  if (a->N == 0 || a->T == 0) return 0;
+  lmoe::launch_recurrent(*a, op == LMOE_OP_GATED_DELTA_RULE, (hipStream_t)stream);
+  return launched(nm);
+}
+
 static int check_gates(const char* nm, int64_t rows, int32_t H, int32_t dtype) {
   if (dtype != LMOE_BF16 && dtype != LMOE_F32) return fail(-2, "%s: dtype must be LMOE_BF16 or LMOE_F32", nm);
   if (H <= 0 || H > 256) return fail(-3, "%s: H = %d outside 1..256", nm, H);

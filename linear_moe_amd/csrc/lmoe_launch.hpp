@@ -60,5 +60,7 @@ int gdn_gates_partials(int64_t rows, int H);
 // chunk_gla gate: logsigmoid(x) / normalizer, clamped from below (n elements, a multiple of 8)
 void launch_gla_gate(int dtype, const void* x, const void* dy, void* out, int64_t n, float normalizer, float clamp_min,
                      bool bwd, hipStream_t st);
+// token-by-token forward (decoding); delta = the (gated) delta rule
+void launch_recurrent(const lmoe_args& a, bool delta, hipStream_t st);
 void launch_selftest(int dtype, int kd, const void* A, const void* B, float* C, float* G, hipStream_t st);
 }  // namespace lmoe
