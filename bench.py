@@ -164,6 +164,21 @@ def neighbours(lib, rows, D, dev, reps):
         "gla_gate_fwd": (lambda: lib.lmoe_gla_gate_fwd(p(x), p(out), ngla, bf, 16.0, float("-inf"), st), ngla * 4),
         "gla_gate_bwd": (lambda: lib.lmoe_gla_gate_bwd(p(x), p(dy), p(out), ngla, bf, 16.0, float("-inf"), st), ngla * 6),
     }
+    # one decoding step of the gated delta rule (token-by-token kernel): 256 sequences, H = 16, K = V = 128,
+    # fp32 state read and written once
+    from linear_moe_amd._host import SeqPlan, _desc, base_args
+    Nd, Hd = 256, 16
+    dq, dk, dv, do_ = (torch.randn(Nd, 1, Hd, D, device=dev, dtype=torch.bfloat16) for _ in range(4))
+    dgt = -torch.rand(Nd, 1, Hd, device=dev)
+    dbt = torch.rand(Nd, 1, Hd, device=dev, dtype=torch.bfloat16)
+    dh0 = torch.randn(Nd, Hd, D, D, device=dev) * 0.1
+    dht = torch.empty_like(dh0)
+    da = base_args(dq, dk, dv, False, None, SeqPlan(Nd, 1, None, dev), (Nd, 1, Hd, D, D))
+    da.gate, da.g, da.g_dtype = _lib.GATE_SCALAR, _desc(dgt, False), _lib.LMOE_F32
+    da.beta, da.beta_dtype = _desc(dbt, False), bf
+    da.h0, da.ht, da.o = dh0.data_ptr(), dht.data_ptr(), _desc(do_, False)
+    extra["gdn_decode_step_256seq"] = (lambda: lib.lmoe_fused_recurrent_fwd(C.byref(da), 2, st),
+                                       2 * dh0.numel() * 4 + 4 * Nd * Hd * D * 2)
     res = {}
     cases = {n: (f, k * rows * D * 2) for n, (f, k) in cases.items()}
     cases.update(extra)
