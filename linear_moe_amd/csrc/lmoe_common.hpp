@@ -271,8 +271,7 @@ __device__ __forceinline__ void frag_keep_if(f32frag& f, bool ok) {
 template <typename T, int D> struct RowFrags {
   static constexpr int KS = D / 32;
   typename ET<T>::frag f[KS];
-  __device__ __forceinline__ void load(const T* __restrict__ base, int64_t row_stride, int row0, int last) {
-    const int l = threadIdx.x & 63;
+  __device__ __forceinline__ void load(const T* __restrict__ base, int64_t row_stride, int row0, int last, int l = threadIdx.x & 63) {
     int r = row0 + (l & 15);
     r = r < last ? r : last;
     const T* p = base + (int64_t)r * row_stride + 8 * (l >> 4);
@@ -345,10 +344,10 @@ template <typename T, int ROWS, int COLS> struct TileIO {
     }
   }
   // tile[row][col] = x * rs[row]
-  static __device__ __forceinline__ void store_lds_scaled(const Regs& r, T* tile, int ld, const float* rs) {
+  static __device__ __forceinline__ void store_lds_scaled(const Regs& r, T* tile, int ld, const float* rs, int tid = threadIdx.x & (NTHR - 1)) {
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
-      int row, col; coords(p, row, col);
+      int row, col; coords(p, row, col, tid);
       if (row < ROWS) {
         const float s = rs[row];
         vec o;
@@ -448,10 +447,10 @@ template <typename T, int ROWS, int COLS> struct TileIO {
     }
   }
   // global[row][col] = tile[row][col]
-  static __device__ __forceinline__ void lds_to_global(const T* tile, int ld, T* __restrict__ dst, int64_t row_stride, int nvalid) {
+  static __device__ __forceinline__ void lds_to_global(const T* tile, int ld, T* __restrict__ dst, int64_t row_stride, int nvalid, int tid = threadIdx.x & (NTHR - 1)) {
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
-      int row, col; coords(p, row, col);
+      int row, col; coords(p, row, col, tid);
       if (row < ROWS && row < nvalid) *(vec*)(dst + (int64_t)row * row_stride + col) = *(const vec*)(tile + row * ld + col);
     }
   }

@@ -4,8 +4,10 @@
 //   w = Tinv (k . beta e^{b}),   u = Tinv (v . beta)
 // and the intra-chunk attention matrix the two sequential passes consume,
 //   P = (q k^T) . Gamma  (lower triangle incl. the diagonal).
-// grid = (NT, H), block = 256.  Writes w, u, Tinv and P (element type T) and the chunk's
-// decay table e^{b}, e^{b_C - b} (fp32).
+// persistent: grid = a few work-groups of 256 threads per CU, item = (chunk, head).  The inputs of
+// the next item (q rows as fragments, k, v tiles, gate, beta) are requested at the top of an item and
+// stay in flight behind its LDS-only barriers.  Writes w, u, Tinv and P (element type T) and the
+// chunk's decay table e^{b}, e^{b_C - b} (fp32).
 #pragma once
 #include "lmoe_seq.hpp"
 
@@ -14,16 +16,19 @@ namespace lmoe {
 // In-LDS inverse of the unit lower triangular matrix I + L (64 x 64, fp32).
 //   sL : strictly lower part L (upper part and diagonal must be 0), leading dimension ldl
 //   sX : receives (I + L)^-1, leading dimension ldx
-//   sY : scratch for one 16 x 16 block per wave... (4 * 256 floats)
-// Block forward substitution with 16 x 16 blocks: the four diagonal blocks are inverted by
-// the four waves (one column per lane), the off-diagonal blocks follow by block distance:
-//   X_IJ = - X_II * sum_{M = J}^{I-1} L_IM X_MJ.
-// Must be called by all 256 threads; sL must be complete (barrier before the call).
-__device__ __forceinline__ void tri_inverse_64(const float* sL, int ldl, float* sX, int ldx, float* sY) {
-  const int wv = wave_id(), l = lane_id(), tid = threadIdx.x;
+//   sY : scratch, one 16 x 17 fp32 block per wave (4 * 272 floats)
+// Block forward substitution with 16 x 16 blocks.  The four diagonal blocks are inverted by the
+// four waves on the vector ALU (one column per lane).  The off-diagonal blocks follow by block
+// distance d = I - J, one block per wave, on the matrix cores in fp32 (v_mfma_f32_16x16x4_f32):
+//   Y = sum_{M = J}^{I-1} L_IM X_MJ   (4 d instructions),   X_IJ = - X_II Y   (4 instructions),
+// with Y passed through the wave's own scratch block, so a round needs one work-group barrier.
+// Must be called by all 256 threads (l, tid: lane and thread index); sL must be complete (barrier
+// before the call).
+__device__ __forceinline__ void tri_inverse_64(const float* sL, int ldl, float* sX, int ldx, float* sY, int l, int tid) {
+  const int wv = wave_id();
   // clear X (upper blocks stay zero)
   for (int idx = tid; idx < CH * CH; idx += NTHR) sX[(idx >> 6) * ldx + (idx & 63)] = 0.f;
-  __syncthreads();
+  lds_barrier();
   if (l < 16) {
     const int o = 16 * wv;
     float x[16];
@@ -37,25 +42,30 @@ __device__ __forceinline__ void tri_inverse_64(const float* sL, int ldl, float* 
 #pragma unroll
     for (int i = 0; i < 16; ++i) sX[(o + i) * ldx + o + l] = x[i];
   }
-  __syncthreads();
-  const int r = tid >> 4, c = tid & 15;   // one entry of a 16 x 16 block per thread
+  lds_barrier();
+  // operand layout of the 16 x 16 x 4 instruction: A[m = l % 16][k = l / 16], B[k = l / 16][n = l % 16],
+  // result rows 4 (l / 16) + i of column l % 16
+  const int r16 = l & 15, k4 = l >> 4;
+  float* yb = sY + wv * 272;
   for (int d = 1; d < 4; ++d) {
-    // Y_IJ = sum_{M=J}^{I-1} L_IM X_MJ for all blocks with I - J = d
-    for (int J = 0; J + d < 4; ++J) {
-      const int I = J + d;
-      float y = 0.f;
-      for (int m = 16 * J; m < 16 * I; ++m) y += sL[(16 * I + r) * ldl + m] * sX[m * ldx + 16 * J + c];
-      sY[J * 256 + tid] = y;
-    }
-    __syncthreads();
-    for (int J = 0; J + d < 4; ++J) {
-      const int I = J + d;
-      float x = 0.f;
+    if (wv + d < 4) {                      // wave-uniform: block (I, J) = (wv + d, wv)
+      const int J = wv, I = wv + d;
+      f32x4 y = {0.f, 0.f, 0.f, 0.f};
+      for (int m = 16 * J; m < 16 * I; m += 4)
+        y = __builtin_amdgcn_mfma_f32_16x16x4f32(sL[(16 * I + r16) * ldl + m + k4], sX[(m + k4) * ldx + 16 * J + r16], y, 0, 0, 0);
 #pragma unroll
-      for (int m = 0; m < 16; ++m) x -= sX[(16 * I + r) * ldx + 16 * I + m] * sY[J * 256 + m * 16 + c];
-      sX[(16 * I + r) * ldx + 16 * J + c] = x;
+      for (int i = 0; i < 4; ++i) yb[(4 * k4 + i) * 17 + r16] = y[i];
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      f32x4 x = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int m = 0; m < 16; m += 4)
+        x = __builtin_amdgcn_mfma_f32_16x16x4f32(sX[(16 * I + r16) * ldx + 16 * I + m + k4], yb[(m + k4) * 17 + r16], x, 0, 0, 0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sX[(16 * I + 4 * k4 + i) * ldx + 16 * J + r16] = -x[i];
     }
-    __syncthreads();
+    lds_barrier();
   }
 }
 
@@ -68,43 +78,65 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
   __shared__ __attribute__((aligned(16))) T s_vb[CH * LDV];
   __shared__ __attribute__((aligned(16))) float s_L[CH * LDC];   // L, later Tinv in element type T
   __shared__ __attribute__((aligned(16))) float s_X[CH * LDC];
-  __shared__ float s_Y[3 * 256];
+  __shared__ float s_Y[4 * 272];
   __shared__ float s_b[64], s_eb[64], s_beta[64], s_beb[64];
   // Tinv as an MFMA operand: fp32 uses s_X in place, bf16 a copy in the (dead) L tile
   T* s_Tm = sizeof(T) == 4 ? (T*)s_X : (T*)s_L;
 
-  const int cid = blockIdx.x, h = blockIdx.y;
-  const ChunkInfo ci = chunk_info(a, cid);
   const int wv = wave_id(), l = lane_id();
   typedef TileIO<T, CH, K> IOK;
   typedef TileIO<T, CH, V> IOV;
   typedef TileIO<T, CH, CH> IO64;
-  typename IOK::Regs rk;
-  typename IOV::Regs rv;
-  // q enters only as the A operand of q k^T: each wave takes its 16 rows straight into fragments
-  RowFrags<T, K> fq;
-  fq.load(row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, 16 * wv, ci.len - 1);
-  IOK::load(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
-  IOV::load(rv, row_ptr<T>(a.v, ci.b, ci.tok, h), a.v.st, ci.len);
-  if (threadIdx.x >= 64 && threadIdx.x < 128) {
-    const int j = threadIdx.x - 64;
-    s_beta[j] = j < ci.len ? load_scalar(a.beta.ptr, a.beta_dtype, row_off(a.beta, ci.b, ci.tok + j, h)) : 0.f;
-  }
-  chunk_gate_cumsum(a, ci.b, ci.tok, ci.len, h, s_b, s_eb, nullptr);    // barrier inside
-  if (threadIdx.x < 64) {
-    s_beb[threadIdx.x] = s_beta[threadIdx.x] * s_eb[threadIdx.x];
+  const int nitems = a.NT * a.H;
+  // inputs of one item on their way in (always requested, item index clamped: a load that is skipped on
+  // some path would make the compiler drain all outstanding loads at every use)
+  struct Pre { typename IOK::Regs rk; typename IOV::Regs rv; RowFrags<T, K> fq; uint32_t graw, braw; };
+  Pre pre;
+  auto issue = [&](int it) {
+    it = min(it, nitems - 1);
+    const int cid = it / a.H, h = it % a.H;
+    const ChunkInfo ci = chunk_info(a, cid);
+    // q enters only as the A operand of q k^T: each wave takes its 16 rows straight into fragments
+    pre.fq.load(row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, 16 * wv, ci.len - 1);
+    IOK::load_nomask(pre.rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
+    IOV::load_nomask(pre.rv, row_ptr<T>(a.v, ci.b, ci.tok, h), a.v.st, ci.len);
+    pre.graw = gate_prefetch(a, ci.b, ci.tok, ci.len, h);
+    pre.braw = load_scalar_raw(a.beta.ptr, a.beta_dtype, row_off(a.beta, ci.b, ci.tok + min(l, ci.len - 1), h));
+  };
+  issue(blockIdx.x);
+  wait_all_loads();   // the first loads may be ordered freely; the loop's waits must not inherit that order
+  for (int it = blockIdx.x; it < nitems; it += gridDim.x) {
+  // lane / thread index refreshed per item: the address arithmetic derived from them stays inside the
+  // iteration instead of living in registers for the whole kernel
+  const int l = fresh_index(lane_id());
+  const int tid = fresh_index((int)threadIdx.x) & (NTHR - 1);
+  const int cid = it / a.H, h = it % a.H;
+  const ChunkInfo ci = chunk_info(a, cid);
+  typename IOK::Regs rk = pre.rk;
+  typename IOV::Regs rv = pre.rv;
+  RowFrags<T, K> fq = pre.fq;
+  const uint32_t graw = pre.graw, braw = pre.braw;
+  issue(it + gridDim.x);
+  IOK::mask(rk, ci.len, tid);
+  IOV::mask(rv, ci.len, tid);
+  lds_barrier();      // the previous item has left every tile
+  if (wv == 1) s_beta[l] = l < ci.len ? scalar_from_raw(braw, a.beta_dtype) : 0.f;
+  gate_finish(a, graw, ci.len, s_b, s_eb, nullptr);
+  lds_barrier();
+  if (tid < 64) {
+    s_beb[tid] = s_beta[tid] * s_eb[tid];
     // decay table of the chunk for the sequential passes: e^{b_j}, e^{b_C - b_j}
     float* gc = a.gcum + ((int64_t)cid * a.H + h) * 2 * CH;
-    gc[threadIdx.x] = s_eb[threadIdx.x];
-    gc[CH + threadIdx.x] = expf(s_b[CH - 1] - s_b[threadIdx.x]);
+    gc[tid] = s_eb[tid];
+    gc[CH + tid] = expf(s_b[CH - 1] - s_b[tid]);
   }
-  IOK::store_lds(rk, s_k, LDK);
-  IOV::store_lds_scaled(rv, s_vb, LDV, s_beta);
-  __syncthreads();
+  IOK::store_lds(rk, s_k, LDK, tid);
+  IOV::store_lds_scaled(rv, s_vb, LDV, s_beta, tid);
+  lds_barrier();
   {
     f32x4 m[1][4];
     acc_zero(m);
-    gemm<T, 1, 4, false, false>(m, s_k, LDK, 16 * wv, s_k, LDK, 0, 0, K);
+    gemm<T, 1, 4, false, false>(m, s_k, LDK, 16 * wv, s_k, LDK, 0, 0, K, l);
 #pragma unroll
     for (int nj = 0; nj < 4; ++nj) {
       f32x4 p;
@@ -113,7 +145,7 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
         const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * nj + (l & 15);
         p[i] = (r > cc) ? s_beta[r] * m[0][nj][i] * texp<T>(s_b[r] - s_b[cc]) : 0.f;
       }
-      acc_to_lds<float>(p, s_L, LDC, 16 * wv, 16 * nj);
+      acc_to_lds<float>(p, s_L, LDC, 16 * wv, 16 * nj, l);
     }
   }
   {
@@ -135,18 +167,18 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
         const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * nj + (l & 15);
         pm[0][nj][i] = (r >= cc) ? pm[0][nj][i] * texp<T>(s_b[r] - s_b[cc]) : 0.f;
       }
-      acc_to_lds<T>(pm[0][nj], s_P, LDC, 16 * wv, 16 * nj);
+      acc_to_lds<T>(pm[0][nj], s_P, LDC, 16 * wv, 16 * nj, l);
     }
-    __syncthreads();
-    IO64::lds_to_global(s_P, LDC, pg, CH, CH);
+    lds_barrier();
+    IO64::lds_to_global(s_P, LDC, pg, CH, CH, tid);
   }
   // k is dead as an operand of k k^T and q k^T: scale it in place to k beta e^{b} (from the registers)
-  IOK::store_lds_scaled(rk, s_k, LDK, s_beb);
-  __syncthreads();   // L is complete, the P staging has been read: the inverse may overwrite X
-  tri_inverse_64(s_L, LDC, s_X, LDC, s_Y);       // barriers inside; s_L is dead afterwards
+  IOK::store_lds_scaled(rk, s_k, LDK, s_beb, tid);
+  lds_barrier();   // L is complete, the P staging has been read: the inverse may overwrite X
+  tri_inverse_64(s_L, LDC, s_X, LDC, s_Y, l, tid);       // barriers inside; s_L is dead afterwards
   {
     T* tg = (T*)a.tinv + ((int64_t)cid * a.H + h) * CH * CH;
-    for (int idx = threadIdx.x; idx < CH * CH / 4; idx += NTHR) {
+    for (int idx = tid; idx < CH * CH / 4; idx += NTHR) {
       const int r = idx >> 4, c = (idx & 15) * 4;
       const f32x4 x = *(const f32x4*)(s_X + r * LDC + c);
       if constexpr (sizeof(T) == 2) {
@@ -158,17 +190,18 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
       }
     }
   }
-  __syncthreads();
+  lds_barrier();
   // w = Tinv (k beta e^{b}),  u = Tinv (v beta): contraction over the rows of the [64][D] tiles
   f32x4 w[1][NBK];
   acc_zero(w);
-  gemm<T, 1, NBK, false, true>(w, s_Tm, LDC, 16 * wv, s_k, LDK, 0, 0, CH);
+  gemm<T, 1, NBK, false, true>(w, s_Tm, LDC, 16 * wv, s_k, LDK, 0, 0, CH, l);
   f32x4 u[1][NBV];
   acc_zero(u);
-  gemm<T, 1, NBV, false, true>(u, s_Tm, LDC, 16 * wv, s_vb, LDV, 0, 0, CH);
-  __syncthreads();   // k, v tiles are dead: wave-private slices of them stage the stores
-  store_strip<T, NBK>(w, s_k + wv * 16 * LDK, row_ptr<T>(a.w, ci.b, ci.tok + 16 * wv, h), a.w.st, ci.len - 16 * wv, 1.0f);
-  store_strip<T, NBV>(u, s_vb + wv * 16 * LDV, row_ptr<T>(a.u, ci.b, ci.tok + 16 * wv, h), a.u.st, ci.len - 16 * wv, 1.0f);
+  gemm<T, 1, NBV, false, true>(u, s_Tm, LDC, 16 * wv, s_vb, LDV, 0, 0, CH, l);
+  lds_barrier();   // k, v tiles are dead: wave-private slices of them stage the stores
+  store_strip<T, NBK>(w, s_k + wv * 16 * LDK, row_ptr<T>(a.w, ci.b, ci.tok + 16 * wv, h), a.w.st, ci.len - 16 * wv, 1.0f, l);
+  store_strip<T, NBV>(u, s_vb + wv * 16 * LDV, row_ptr<T>(a.u, ci.b, ci.tok + 16 * wv, h), a.u.st, ci.len - 16 * wv, 1.0f, l);
+  }   // items
 }
 
 }  // namespace lmoe
