@@ -179,6 +179,19 @@ def neighbours(lib, rows, D, dev, reps):
     da.h0, da.ht, da.o = dh0.data_ptr(), dht.data_ptr(), _desc(do_, False)
     extra["gdn_decode_step_256seq"] = (lambda: lib.lmoe_fused_recurrent_fwd(C.byref(da), 2, st),
                                        2 * dh0.numel() * 4 + 4 * Nd * Hd * D * 2)
+    # mixture-of-memories routing: B = 4, S = 8192, hidden 2048, 4 memories, top-2 -> 65536 packed rows
+    from linear_moe_amd import mom_plan
+    mB, mS, mE, mk, mD = 4, 8192, 4, 2, 2048
+    msel = torch.topk(torch.rand(mB, mS, mE, device=dev), mk, dim=-1)[1]
+    plan = mom_plan(msel, mE)
+    mx = torch.randn(mB * mS, mD, device=dev, dtype=torch.bfloat16)
+    mxp = torch.empty(plan.T_total, mD, device=dev, dtype=torch.bfloat16)
+    mw = torch.rand(mB * mS, mk, device=dev, dtype=torch.bfloat16)
+    mo = torch.empty_like(mx)
+    extra["mom_pack"] = (lambda: lib.lmoe_mom_gather(p(mx), p(plan.src_token), None, p(mxp), plan.T_total, mD, bf, st),
+                         (mx.numel() + mxp.numel()) * 2)
+    extra["mom_combine"] = (lambda: lib.lmoe_mom_combine(p(mxp), p(plan.row_of), p(mw), p(mo), mB * mS, mk, mD, bf, st),
+                            (mxp.numel() + mo.numel()) * 2)
     res = {}
     cases = {n: (f, k * rows * D * 2) for n, (f, k) in cases.items()}
     cases.update(extra)

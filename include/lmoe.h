@@ -186,6 +186,23 @@ int lmoe_gla_gate_fwd(const void* x, void* y, int64_t n, int32_t dtype, float no
 int lmoe_gla_gate_bwd(const void* x, const void* dy, void* dx, int64_t n, int32_t dtype, float normalizer,
                       float clamp_min, void* stream);
 
+/* Row routing for mixture-of-memories layers.  The reference pads the tokens routed to each (memory, batch
+ * row) to a common capacity (`transform`, linear_moe/sequence_modeling/mom_linear_attention.py:15-77), calls
+ * the op once per memory (:369-409) and scatters the results back (`reconstruct`, :79-120).  Here the routed
+ * tokens are packed into one variable-length batch (one cu_seqlens call of the op for all memories):
+ *   lmoe_mom_gather : out[i] = scale[i] * src[idx[i]]            rows of D elements; idx[i] < 0 -> zeros;
+ *                                                                scale ([nout], element type) may be null
+ *   lmoe_mom_combine: out[t] = sum_k w[t][k] * src[idx[t][k]]    idx < 0 skipped; w ([ntok][topk]) null -> 1
+ *   lmoe_mom_rowdot : dw[t][k] = <g[t], src[idx[t][k]]>          the gradient of combine w.r.t. w
+ * (pack = gather, its backward = combine with w = null; unpack = combine, its backward = gather with scale
+ * and rowdot).  D a multiple of 8; idx int32 on the device; no atomics. */
+int lmoe_mom_gather(const void* src, const int32_t* idx, const void* scale, void* out, int64_t nout, int32_t D,
+                    int32_t dtype, void* stream);
+int lmoe_mom_combine(const void* src, const int32_t* idx, const void* w, void* out, int64_t ntok, int32_t topk, int32_t D,
+                     int32_t dtype, void* stream);
+int lmoe_mom_rowdot(const void* src, const int32_t* idx, const void* g, void* dw, int64_t ntok, int32_t topk, int32_t D,
+                    int32_t dtype, void* stream);
+
 /* Launch ONE kernel of an op's pipeline (profiling support: lets a harness time each kernel
  * with events on its own stream).  `a` must be the fully populated argument block of the
  * op's fwd (stages 0-2, 7) or bwd (stages 3-5) entry point, with the intermediates of the

@@ -13,6 +13,7 @@ from .l2norm import l2_norm, l2_norm_fn, silu_l2_norm  # noqa: F401
 from .rmsnorm import RMSNorm, rms_norm_fn, rms_norm_swish_gate  # noqa: F401
 from .lightning import lightning_attn2, lightning_attn2_no_decay  # noqa: F401
 from .linear_attn import chunk_linear_attn  # noqa: F401
+from .mom import MomPlan, mom_combine, mom_pack, mom_plan  # noqa: F401
 from .recurrent import (fused_recurrent_delta_rule, fused_recurrent_gated_delta_rule, fused_recurrent_gla,  # noqa: F401
                         fused_recurrent_simple_gla)
 from .retention import chunk_retention  # noqa: F401
@@ -21,4 +22,4 @@ from .simple_gla import chunk_simple_gla  # noqa: F401
 __all__ = ["chunk_simple_gla", "chunk_gla", "chunk_gated_delta_rule", "chunk_delta_rule", "chunk_retention", "chunk_linear_attn",
            "lightning_attn2", "lightning_attn2_no_decay", "l2_norm", "l2_norm_fn", "silu_l2_norm", "rms_norm_fn",
            "rms_norm_swish_gate", "RMSNorm", "gdn_gates", "gla_gate", "fused_recurrent_simple_gla", "fused_recurrent_gla",
-           "fused_recurrent_gated_delta_rule", "fused_recurrent_delta_rule"]
+           "fused_recurrent_gated_delta_rule", "fused_recurrent_delta_rule", "mom_plan", "mom_pack", "mom_combine", "MomPlan"]

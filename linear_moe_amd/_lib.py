@@ -48,7 +48,7 @@ ENTRY_POINTS = (
     "lmoe_launch_stage", "lmoe_selftest_gemm", "lmoe_workspace_bytes", "lmoe_l2norm_fwd", "lmoe_l2norm_bwd",
     "lmoe_silu_l2norm_fwd", "lmoe_silu_l2norm_bwd", "lmoe_rmsnorm_partials", "lmoe_rmsnorm_fwd", "lmoe_rmsnorm_bwd",
     "lmoe_gdn_gates_partials", "lmoe_gdn_gates_fwd", "lmoe_gdn_gates_bwd", "lmoe_gla_gate_fwd", "lmoe_gla_gate_bwd",
-    "lmoe_fused_recurrent_fwd",
+    "lmoe_fused_recurrent_fwd", "lmoe_mom_gather", "lmoe_mom_combine", "lmoe_mom_rowdot",
 )
 
 _lib = None
@@ -104,6 +104,11 @@ def load() -> C.CDLL:
     lib.lmoe_gla_gate_bwd.restype = C.c_int
     lib.lmoe_fused_recurrent_fwd.argtypes = [C.POINTER(Args), C.c_int32, C.c_void_p]
     lib.lmoe_fused_recurrent_fwd.restype = C.c_int
+    lib.lmoe_mom_gather.argtypes = [C.c_void_p] * 4 + [C.c_int64, C.c_int32, C.c_int32, C.c_void_p]
+    lib.lmoe_mom_gather.restype = C.c_int
+    for fn in (lib.lmoe_mom_combine, lib.lmoe_mom_rowdot):
+        fn.argtypes = [C.c_void_p] * 4 + [C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]
+        fn.restype = C.c_int
     lib.lmoe_workspace_bytes.argtypes = [C.c_int32] * 9
     lib.lmoe_workspace_bytes.restype = C.c_int64
     _lib = lib

@@ -233,6 +233,42 @@ int lmoe_fused_recurrent_fwd(const lmoe_args* a, int32_t op, void* stream) {
   return launched(nm);
 }
 
+static int check_mom(const char* nm, const void* src, const void* idx, const void* out, int64_t n, int32_t D, int32_t dtype) {
+  if (!src || !idx || !out) return fail(-1, "%s: null pointer", nm);
+  if (dtype != LMOE_BF16 && dtype != LMOE_F32) return fail(-2, "%s: dtype must be LMOE_BF16 or LMOE_F32", nm);
+  if (D <= 0 || D % 8) return fail(-3, "%s: row length %d must be a positive multiple of 8", nm, D);
+  if (n < 0) return fail(-4, "%s: negative row count", nm);
+  if (((uintptr_t)src | (uintptr_t)out) & 15) return fail(-9, "%s: row pointers must be 16-byte aligned", nm);
+  return 0;
+}
+int lmoe_mom_gather(const void* src, const int32_t* idx, const void* scale, void* out, int64_t nout, int32_t D,
+                    int32_t dtype, void* stream) {
+  const char* nm = "lmoe_mom_gather";
+  if (int r = check_mom(nm, src, idx, out, nout, D, dtype)) return r;
+  if (nout == 0) return 0;
+  lmoe::launch_mom_gather(dtype, src, idx, scale, out, nout, D, (hipStream_t)stream);
+  return launched(nm);
+}
+int lmoe_mom_combine(const void* src, const int32_t* idx, const void* w, void* out, int64_t ntok, int32_t topk, int32_t D,
+                     int32_t dtype, void* stream) {
+  const char* nm = "lmoe_mom_combine";
+  if (int r = check_mom(nm, src, idx, out, ntok, D, dtype)) return r;
+  if (topk <= 0) return fail(-4, "%s: topk must be positive", nm);
+  if (ntok == 0) return 0;
+  lmoe::launch_mom_combine(dtype, src, idx, w, out, ntok, topk, D, (hipStream_t)stream);
+  return launched(nm);
+}
+int lmoe_mom_rowdot(const void* src, const int32_t* idx, const void* g, void* dw, int64_t ntok, int32_t topk, int32_t D,
+                    int32_t dtype, void* stream) {
+  const char* nm = "lmoe_mom_rowdot";
+  if (int r = check_mom(nm, src, idx, dw, ntok, D, dtype)) return r;
+  if (!g || ((uintptr_t)g & 15)) return fail(-1, "%s: g must be a 16-byte aligned pointer", nm);
+  if (topk <= 0) return fail(-4, "%s: topk must be positive", nm);
+  if (ntok == 0) return 0;
+  lmoe::launch_mom_rowdot(dtype, src, idx, g, dw, ntok, topk, D, (hipStream_t)stream);
+  return launched(nm);
+}
+
 static int check_gates(const char* nm, int64_t rows, int32_t H, int32_t dtype) {
   if (dtype != LMOE_BF16 && dtype != LMOE_F32) return fail(-2, "%s: dtype must be LMOE_BF16 or LMOE_F32", nm);
   if (H <= 0 || H > 256) return fail(-3, "%s: H = %d outside 1..256", nm, H);

@@ -330,7 +330,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
     const float* s_beta = s_gbeta[par];
     // the lane index is refreshed per item: address arithmetic derived from it then stays inside
     // the iteration instead of living in registers for the whole kernel
-    const int l = fresh_index(lane_id());
+    const int l = fresh_index(lane_id()) & 63;
     const int fr = l & 15, fg = 8 * (l >> 4);
     const int rb = r0 + 4 * (l >> 4);      // accumulator element i is row rb + i, column (tile) + fr
     f32x4 dP[1][2], dTv[1][2], dqi[1][NBK], dkd[1][NBK], dw[1][NBK];

@@ -108,7 +108,7 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
   for (int it = blockIdx.x; it < nitems; it += gridDim.x) {
   // lane / thread index refreshed per item: the address arithmetic derived from them stays inside the
   // iteration instead of living in registers for the whole kernel
-  const int l = fresh_index(lane_id());
+  const int l = fresh_index(lane_id()) & 63;
   const int tid = fresh_index((int)threadIdx.x) & (NTHR - 1);
   const int cid = it / a.H, h = it % a.H;
   const ChunkInfo ci = chunk_info(a, cid);

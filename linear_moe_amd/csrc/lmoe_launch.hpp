@@ -60,6 +60,13 @@ int gdn_gates_partials(int64_t rows, int H);
 // chunk_gla gate: logsigmoid(x) / normalizer, clamped from below (n elements, a multiple of 8)
 void launch_gla_gate(int dtype, const void* x, const void* dy, void* out, int64_t n, float normalizer, float clamp_min,
                      bool bwd, hipStream_t st);
+// row routing of mixture-of-memories layers (rows of D elements, D a multiple of 8)
+void launch_mom_gather(int dtype, const void* src, const int32_t* idx, const void* scale, void* out, int64_t nout, int D,
+                       hipStream_t st);
+void launch_mom_combine(int dtype, const void* src, const int32_t* idx, const void* w, void* out, int64_t ntok, int topk,
+                        int D, hipStream_t st);
+void launch_mom_rowdot(int dtype, const void* src, const int32_t* idx, const void* g, void* dw, int64_t ntok, int topk,
+                       int D, hipStream_t st);
 // token-by-token forward (decoding); delta = the (gated) delta rule
 void launch_recurrent(const lmoe_args& a, bool delta, hipStream_t st);
 void launch_selftest(int dtype, int kd, const void* A, const void* B, float* C, float* G, hipStream_t st);

@@ -339,3 +339,37 @@ def test_gate_construction_pins():
     assert torch.allclose(y[:3], torch.tensor([-math.log(2.0) / 16, -50.0 / 16, 0.0], dtype=torch.float64), atol=1e-15)
     assert torch.allclose(y[3], torch.tensor(-math.log1p(math.e) / 16, dtype=torch.float64))
     assert torch.equal(naive.naive_gla_gate(x, 16.0, clamp_min=-1.0)[1], torch.tensor(-1.0, dtype=torch.float64))
+
+
+def test_mom_routing_pins():
+    """oracle/mom.py (transform / reconstruct of mom_linear_attention.py:15-120): hand-written expectations
+    for a tiny routing (time order, truncation keeps the LAST tokens, zeros on the LEFT), and the properties
+    that a wrong side / index would break: every kept (token, choice) appears exactly once; with weights that
+    sum to one, no truncation and the identity in place of the op, reconstruct(transform(x)) = x."""
+    from oracle import mom
+    x = torch.arange(1.0, 5.0).view(1, 4, 1) * torch.ones(1, 4, 8)             # token t carries the value t + 1
+    sel = torch.tensor([[[0], [1], [0], [0]]])
+    pad, max_len, kept = mom.transform(x, sel, 2, capacity=1.0)
+    assert max_len == 3 and pad.shape == (2, 1, 4, 8)
+    assert pad[0, 0, :, 0].tolist() == [0.0, 1.0, 3.0, 4.0]                    # memory 0: tokens 0, 2, 3, right-aligned
+    assert pad[1, 0, :, 0].tolist() == [0.0, 0.0, 0.0, 2.0]                    # memory 1: token 1
+    pad, max_len, kept = mom.transform(x, sel, 2, capacity=0.5)                # capacity_len 2: token 0 is dropped
+    assert max_len == 2 and pad[0, 0, :, 0].tolist() == [3.0, 4.0] and pad[1, 0, :, 0].tolist() == [0.0, 2.0]
+    assert kept[0][0] == [(2, 0), (3, 0)] and kept[0][1] == [(1, 0)]
+    w = torch.ones(1, 4, 1)
+    rec = mom.reconstruct(pad, kept, w)
+    assert rec[0, :, 0].tolist() == [0.0, 2.0, 3.0, 4.0]                       # the dropped token gets nothing
+    # random routing, topk = 2
+    g = torch.Generator().manual_seed(7401)
+    B, S, E, topk, D = 2, 23, 4, 2, 8
+    scores = torch.rand(B, S, E, generator=g)
+    wts, sel = torch.topk(scores, topk, dim=-1)
+    wts = wts / wts.sum(-1, keepdim=True)
+    xr = torch.randn(B, S, D, generator=g, dtype=torch.float64)
+    pad, max_len, kept = mom.transform(xr, sel, E, capacity=1.0)
+    seen = sorted((b, t, k) for b in range(B) for e in range(E) for (t, k) in kept[b][e])
+    assert seen == sorted((b, t, k) for b in range(B) for t in range(S) for k in range(topk))
+    for b in range(B):
+        for e in range(E):
+            assert kept[b][e] == sorted(kept[b][e]) and all(int(sel[b, t, k]) == e for t, k in kept[b][e])
+    assert torch.allclose(mom.reconstruct(pad, kept, wts.double()), xr, atol=1e-12)
