@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Headline benchmark: chunk_gated_delta_rule forward + backward on one MI355X.
 
-Workload (BASELINE.json configs[3], the one the metric is quoted on): B=4, H=16, T=8192,
+Workload (the configuration the metric is quoted on): B=4, H=16, T=8192,
 K=V=128, bf16; q,k ~ N(0,1) L2-normalised, v ~ N(0,1), beta = sigmoid(N(0,1)),
 g = -exp(A_h) softplus(x + dt_bias_h), dO ~ N(0,1).  A "step" is one forward + one backward of
 the op over that batch with all inputs resident in HBM.
@@ -264,7 +264,8 @@ def main():
     dt = (time.perf_counter() - t0) / args.steps
 
     tokens = B * T
-    # whole-op algorithmic work per token and head (SURVEY 8d model): fwd 6CK+4CV+6KV+(2/3)C^2, x3
+    # whole-op algorithmic work per token and head: fwd 6CK+4CV+6KV+(2/3)C^2 flops, x3 for fwd+bwd;
+    # bytes: every input read once, every output written once
     f_tok = 3 * (6 * CH * K + 4 * CH * V + 6 * K * V + (2 / 3) * CH * CH)
     b_tok = (6 * K + 5 * V) * 2 + 3 * 2 + 12
     flops, bytes_ = f_tok * tokens * H, b_tok * tokens * H
@@ -291,7 +292,7 @@ def main():
         "value": tokens / dt, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "chunk_gated_delta_rule fwd+bwd B=4 H=16 T=8192 K=V=128 (BASELINE configs[3])",
+        "config": {"workload": "chunk_gated_delta_rule fwd+bwd B=4 H=16 T=8192 K=V=128 (contract config 4 of 5)",
                    "B": B, "T": T, "H": H, "K": K, "V": V, "chunk": CH},
         "mfma_frac": flops / dt / PEAK_MFMA_BF16, "hbm_frac_algorithmic": bytes_ / dt / PEAK_HBM,
         "tflops": flops / dt / 1e12,

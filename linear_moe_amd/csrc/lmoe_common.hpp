@@ -65,6 +65,7 @@ template <typename T> struct ET;
 template <> struct ET<bf16> {
   static constexpr int VEC = 8;                       // elements per 16-byte vector
   typedef bf16x8 vec;
+  typedef bf16x4 vec4;      // four consecutive elements (one accumulator column group)
   typedef bf16x8 frag;
   static __device__ __forceinline__ vec zero() { vec z; for (int i = 0; i < 8; ++i) z[i] = (bf16)0.0f; return z; }
   static __device__ __forceinline__ float to_f(bf16 x) { return (float)x; }
@@ -93,6 +94,7 @@ struct f32frag { f32x4 lo, hi; };
 template <> struct ET<float> {
   static constexpr int VEC = 4;
   typedef f32x4 vec;
+  typedef f32x4 vec4;
   typedef f32frag frag;
   static __device__ __forceinline__ vec zero() { vec z = {0.f, 0.f, 0.f, 0.f}; return z; }
   static __device__ __forceinline__ float to_f(float x) { return x; }

@@ -54,10 +54,11 @@ template <int L, typename F> __device__ __forceinline__ void ring_loop(int n, F&
 
 // ------------------------------------------------------------------------- //
 // forward
-//   team 1, chunk c:   B1 | stage k(c), P(c); lift S^T(c), o(c-1), v_new(c-1) out of LDS |
-//                      B2 | store hs(c), o(c-1), v_new(c-1); prefetch k, P
+//   team 1, chunk c:   B1 | stage k(c), P(c); lift S^T(c), o(c-1) out of LDS |
+//                      B2 | lift v_new(c); store hs(c), o(c-1), v_new(c); prefetch k, P
 //   team 2, chunk c:   B1 | prefetch w, q, u, decay table | B2 | stage those of chunk c+1
 //   consumers, chunk c: S -> LDS | B1 | w S, q S, v_new -> LDS | B2 | S update, P v_new, o -> LDS
+//   (team 1 lifts v_new(c) right after B2 and stores it in the same half-step)
 // ------------------------------------------------------------------------- //
 template <typename T, int K, int V, int BV>
 __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
@@ -70,8 +71,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
   __shared__ __attribute__((aligned(16))) T s_p[CH * LDC];          // P             [64][64]
   __shared__ __attribute__((aligned(16))) T s_u[CH * LDU];          // u             [64][BV]
   __shared__ __attribute__((aligned(16))) T s_hT[BV * LDK];         // S^T           [BV][K]
-  __shared__ __attribute__((aligned(16))) T s_vT[BV * LDC];         // v_new^T       [BV][64]
-  __shared__ __attribute__((aligned(16))) T s_vn[CH * LDU];         // v_new         [64][BV] (to be stored)
+  __shared__ __attribute__((aligned(16))) T s_vn[CH * LDU];         // v_new         [64][BV] (MFMA operand through transposing reads, and stored)
   __shared__ __attribute__((aligned(16))) T s_o[CH * LDU];          // o             [64][BV] (to be stored)
   __shared__ __attribute__((aligned(16))) float s_eb[2][64], s_ed[2][64];
   __shared__ float s_dec[2];                                        // e^{b_C}; gate arrays: buffer c & 1
@@ -119,12 +119,11 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
       IOK::store_lds(P.rk, s_k, LDK);
       IOP::store_lds(P.rp, s_p, LDC);       // rows and columns past the end are zero as written
     };
-    // o and v_new of chunk c: registers -> global
-    auto store_results = [&](const typename IOV::Regs& rvn, const typename IOV::Regs& ro, int c) {
+    // a result tile of chunk c: registers -> global
+    auto store_result = [&](const typename IOV::Regs& r, const lmoe_tensor& dst, int c) {
       const int tok = sq.tok0 + c * CH;
       const int len = min(CH, sq.len - c * CH);
-      IOV::store_global(rvn, row_ptr<T>(a.vnew, sq.b, tok, h) + v0, a.vnew.st, len);
-      IOV::store_global(ro, row_ptr<T>(a.o, sq.b, tok, h) + v0, a.o.st, len);
+      IOV::store_global(r, row_ptr<T>(dst, sq.b, tok, h) + v0, dst.st, len);
     };
 #pragma unroll
     for (int j = 0; j < LPF; ++j) issue_a(pa[j], j);
@@ -137,20 +136,21 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
       constexpr int j = decltype(slot)::value;
       lds_barrier();                                                                     // B1
       stage_a(pa[j]);
-      // S^T and the previous chunk's results leave LDS now (the consumers rewrite them after B2)
+      // S^T and the previous chunk's o leave LDS now (the consumers rewrite them after B2)
       IOHT::load_lds(rh, s_hT, LDK);
-      IOV::load_lds(rvn, s_vn, LDU);
       IOV::load_lds(ro, s_o, LDU);
       lds_barrier();                                                                     // B2
+      // v_new of this chunk is complete (the consumers rewrite it after the next B1)
+      IOV::load_lds(rvn, s_vn, LDU);
       // hs[chunk][h][v0 .. v0+BV][K] <- S^T
       IOHT::store_global(rh, (T*)a.hs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
-      if (c > 0) store_results(rvn, ro, c - 1);
+      if (c > 0) store_result(ro, a.o, c - 1);
+      store_result(rvn, a.vnew, c);
       issue_a(pa[j], c + LPF);
     });
-    lds_barrier();                                                                       // results of the last chunk
-    IOV::load_lds(rvn, s_vn, LDU);
+    lds_barrier();                                                                       // o of the last chunk
     IOV::load_lds(ro, s_o, LDU);
-    store_results(rvn, ro, sq.nchunks - 1);
+    store_result(ro, a.o, sq.nchunks - 1);
     return;
   }
   if (team == 2) {
@@ -224,7 +224,10 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
 #pragma unroll
       for (int ni = 0; ni < NB; ++ni) acc_to_lds_t<T>(S[mi][ni], s_hT, LDK, krow0 + 16 * mi, 16 * ni);
     lds_barrier();                                                                       // B1
-    // w S and q S over the same S^T fragments (rows 16 wv .. of the chunk)
+    // (w S)^T and (q S)^T over the same S^T fragments, for the tokens 16 wv .. of the chunk.  The
+    // products are formed transposed (S^T as the A operand): a lane then holds four consecutive V
+    // columns of one token, so u is read and v_new, o are written with 8-byte LDS accesses in token-major
+    // layout (2-byte LDS accesses cost as many cycles as 8-byte ones).
     f32x4 vn[1][NB], o[1][NB];
     acc_zero(vn);
     acc_zero(o);
@@ -235,21 +238,23 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
 #pragma unroll
       for (int ni = 0; ni < NB; ++ni) {
         const typename ET<T>::frag bS = ET<T>::load_frag(s_hT + (16 * ni + fr) * LDK + 32 * ks + fg);
-        ET<T>::mma(vn[0][ni], aw, bS);
-        ET<T>::mma(o[0][ni], aq, bS);
+        ET<T>::mma(vn[0][ni], bS, aw);
+        ET<T>::mma(o[0][ni], bS, aq);
       }
     }
+    const int tk = 16 * wv + (l & 15);       // token of this lane in the transposed accumulators
+    const float ebt = s_eb[cur][tk];
 #pragma unroll
     for (int ni = 0; ni < NB; ++ni) {
+      const typename ET<T>::vec4 u4 = *(const typename ET<T>::vec4*)(s_u + tk * LDU + 16 * ni + 4 * (l >> 4));
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
         // v_new = u - w S, rounded once to the storage type so that the state update, the
         // output and the backward see the same values
-        vn[0][ni][i] = ET<T>::to_f(ET<T>::from_f(ET<T>::to_f(s_u[r * LDU + cc]) - vn[0][ni][i]));
-        o[0][ni][i] *= s_eb[cur][r];
+        vn[0][ni][i] = ET<T>::to_f(ET<T>::from_f(ET<T>::to_f(u4[i]) - vn[0][ni][i]));
+        o[0][ni][i] *= ebt;
       }
-      acc_to_lds_t<T>(vn[0][ni], s_vT, LDC, 16 * wv, 16 * ni);
+      acc_to_lds_t<T>(vn[0][ni], s_vn, LDU, 16 * ni, 16 * wv);      // s_vn[token][v]
     }
     const float dec = s_dec[cur];
     lds_barrier();                                                                       // B2
@@ -266,8 +271,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
       for (int mi = 0; mi < MB; ++mi) af[mi] = ET<T>::load_frag_t(s_k, LDK, 32 * ks, krow0 + 16 * mi);
 #pragma unroll
       for (int ni = 0; ni < NB; ++ni) {
-        bv[ni] = ET<T>::load_frag(s_vT + (16 * ni + fr) * LDC + 32 * ks + fg);
-        ET<T>::mma(o[0][ni], ap, bv[ni]);
+        bv[ni] = ET<T>::load_frag_t(s_vn, LDU, 32 * ks, 16 * ni);       // rows: V columns, contraction: tokens
+        ET<T>::mma(o[0][ni], bv[ni], ap);
         scale_frag8<T>(bv[ni], &s_ed[cur][32 * ks + fg]);
       }
 #pragma unroll
@@ -277,10 +282,9 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
     }
 #pragma unroll
     for (int ni = 0; ni < NB; ++ni) {
-      // results for the loaders (they store the previous chunk's during phase 1, hence not earlier)
+      // o for the loaders (they lift the previous chunk's during phase 1, hence not earlier)
       o[0][ni] *= scale;
-      acc_to_lds<T>(o[0][ni], s_o, LDU, 16 * wv, 16 * ni);
-      acc_to_lds<T>(vn[0][ni], s_vn, LDU, 16 * wv, 16 * ni);
+      acc_to_lds_t<T>(o[0][ni], s_o, LDU, 16 * ni, 16 * wv);         // s_o[token][v]
     }
   }
   lds_barrier();                                                                         // results of the last chunk

@@ -1,4 +1,4 @@
-"""The five configurations of the contract (BASELINE.json configs[0..4]) at full size on the GPU.
+"""The five configurations of the contract at full size on the GPU.
 
 Parity: the HIP result is compared with the CPU oracle on a slice the oracle finishes in
 seconds (batch rows and heads are independent, so a slice of them is an exact sub-problem);
