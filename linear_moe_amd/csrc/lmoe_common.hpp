@@ -254,6 +254,15 @@ template <typename T> __device__ __forceinline__ void scale_frag8(typename ET<T>
   }
 }
 
+// f = -f
+__device__ __forceinline__ void frag_negate(bf16x8& f) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  u32x4 w = __builtin_bit_cast(u32x4, f);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] ^= 0x80008000u;
+  f = __builtin_bit_cast(bf16x8, w);
+}
+__device__ __forceinline__ void frag_negate(f32frag& f) { f.lo = -f.lo; f.hi = -f.hi; }
 __device__ __forceinline__ void frag_keep_if(bf16x8& f, bool ok) {
   typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
   u32x4 w = __builtin_bit_cast(u32x4, f);

@@ -318,8 +318,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
   __shared__ __attribute__((aligned(16))) T s_p[CH * LDC];          // P         [64][64]
   __shared__ __attribute__((aligned(16))) T s_do[CH * LDU];         // do        [64][BV]
   __shared__ __attribute__((aligned(16))) T s_dST[BV * LDK];        // dS'^T     [BV][K]
-  __shared__ __attribute__((aligned(16))) T s_dvT[BV * LDC];        // -dv_new^T [BV][64]
-  __shared__ __attribute__((aligned(16))) T s_dvn[CH * LDU];        // dv_new    [64][BV] (to be stored)
+  __shared__ __attribute__((aligned(16))) T s_dvn[CH * LDU];        // dv_new    [64][BV] (MFMA operand through transposing reads, and stored)
   __shared__ __attribute__((aligned(16))) float s_qs[2][64], s_ed[2][64];
   __shared__ float s_dec[2];                                        // gate arrays: buffer it & 1
 
@@ -379,17 +378,16 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
       const int c = sq.nchunks - 1 - it;
       lds_barrier();                                                                     // B1
       stage_a(pa[j]);
-      // dS'^T and the previous chunk's dv_new leave LDS now (the consumers rewrite them after B2)
+      // dS'^T leaves LDS now (the consumers rewrite it after B2)
       IOHT::load_lds(rh, s_dST, LDK);
-      IOV::load_lds(rdv, s_dvn, LDU);
       lds_barrier();                                                                     // B2
+      // dv_new of this chunk is complete (the consumers rewrite it after the next B1)
+      IOV::load_lds(rdv, s_dvn, LDU);
       IOHT::store_global(rh, (T*)a.dhs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
-      if (it > 0) store_results(rdv, c + 1);
+      store_results(rdv, c);
       issue_a(pa[j], it + LPF);
     });
-    lds_barrier();                                                                       // dv_new of chunk 0
-    IOV::load_lds(rdv, s_dvn, LDU);
-    store_results(rdv, 0);
+    lds_barrier();
     return;
   }
   if (team == 2) {
@@ -463,7 +461,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
 #pragma unroll
       for (int ni = 0; ni < NB; ++ni) acc_to_lds_t<T>(dS[mi][ni], s_dST, LDK, krow0 + 16 * mi, 16 * ni);
     lds_barrier();                                                                       // B1
-    // t = k dS'  and  dv_loc = P^T do   (rows 16 wv .. of the chunk)
+    // t = (k dS')^T  and  dv_loc = (P^T do)^T for the tokens 16 wv .. of the chunk: formed transposed,
+    // so that a lane holds four consecutive V columns of one token (see k_gdn_state_fwd)
     f32x4 t[1][NB], dvl[1][NB];
     acc_zero(t);
     acc_zero(dvl);
@@ -472,7 +471,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
       const typename ET<T>::frag ak = ET<T>::load_frag(s_k + (16 * wv + fr) * LDK + 32 * ks + fg);
 #pragma unroll
       for (int ni = 0; ni < NB; ++ni)
-        ET<T>::mma(t[0][ni], ak, ET<T>::load_frag(s_dST + (16 * ni + fr) * LDK + 32 * ks + fg));
+        ET<T>::mma(t[0][ni], ET<T>::load_frag(s_dST + (16 * ni + fr) * LDK + 32 * ks + fg), ak);
     }
     typename ET<T>::frag bdo[CH / 32][NB];
 #pragma unroll
@@ -482,24 +481,21 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
 #pragma unroll
       for (int ni = 0; ni < NB; ++ni) {
         bdo[ks][ni] = ET<T>::load_frag_t(s_do, LDU, 32 * ks, 16 * ni);
-        ET<T>::mma(dvl[0][ni], ap, bdo[ks][ni]);
+        ET<T>::mma(dvl[0][ni], bdo[ks][ni], ap);
       }
     }
 #pragma unroll
     for (int ks = 0; ks < CH / 32; ++ks)
 #pragma unroll
       for (int ni = 0; ni < NB; ++ni) scale_frag8<T>(bdo[ks][ni], &s_qs[cur][32 * ks + fg]);
+    const float edt = s_ed[cur][16 * wv + (l & 15)];       // the token of this lane
 #pragma unroll
     for (int ni = 0; ni < NB; ++ni) {
-      f32x4 x;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int r = 16 * wv + 4 * (l >> 4) + i;
-        // dv_new, rounded once to the storage type (the WY backward reads the stored values)
-        t[0][ni][i] = ET<T>::to_f(ET<T>::from_f(scale * dvl[0][ni][i] + s_ed[cur][r] * t[0][ni][i]));
-        x[i] = -t[0][ni][i];
-      }
-      acc_to_lds_t<T>(x, s_dvT, LDC, 16 * wv, 16 * ni);
+      for (int i = 0; i < 4; ++i)
+        // dv_new, rounded once to the storage type (the chunk-parallel backward reads the stored values)
+        t[0][ni][i] = ET<T>::to_f(ET<T>::from_f(scale * dvl[0][ni][i] + edt * t[0][ni][i]));
+      acc_to_lds_t<T>(t[0][ni], s_dvn, LDU, 16 * ni, 16 * wv);      // s_dvn[token][v]
     }
     const float dec = s_dec[cur];
     lds_barrier();                                                                       // B2
@@ -517,7 +513,10 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
         aw[mi] = ET<T>::load_frag_t(s_w, LDK, 32 * ks, krow0 + 16 * mi);
       }
 #pragma unroll
-      for (int ni = 0; ni < NB; ++ni) bn[ni] = ET<T>::load_frag(s_dvT + (16 * ni + fr) * LDC + 32 * ks + fg);
+      for (int ni = 0; ni < NB; ++ni) {
+        bn[ni] = ET<T>::load_frag_t(s_dvn, LDU, 32 * ks, 16 * ni);    // rows: V columns, contraction: tokens
+        frag_negate(bn[ni]);
+      }
 #pragma unroll
       for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
@@ -526,11 +525,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
           ET<T>::mma(dS[mi][ni], aw[mi], bn[ni]);
         }
     }
-    // dv_new for the loaders (they store the previous chunk's during phase 1, hence not earlier)
-#pragma unroll
-    for (int ni = 0; ni < NB; ++ni) acc_to_lds<T>(t[0][ni], s_dvn, LDU, 16 * wv, 16 * ni);
   }
-  lds_barrier();                                                                         // dv_new of chunk 0
+  lds_barrier();
   if (a.dh0) {
     float* p = a.dh0 + ((int64_t)n * a.H + h) * K * V;
 #pragma unroll
