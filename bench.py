@@ -192,6 +192,20 @@ def neighbours(lib, rows, D, dev, reps):
                          (mx.numel() + mxp.numel()) * 2)
     extra["mom_combine"] = (lambda: lib.lmoe_mom_combine(p(mxp), p(plan.row_of), p(mw), p(mo), mB * mS, mk, mD, bf, st),
                             (mxp.numel() + mo.numel()) * 2)
+    # HGRN2 gates on the forget projection of contract config 3's shape (bf16 in, k bf16 + g fp32 out), and the
+    # Taylor feature map of Based on [8,16,2048] rows of D = 16 -> 153 features in 192 padded columns
+    hk, hg, hdg = torch.empty(ngla, device=dev, dtype=torch.bfloat16), torch.empty(ngla, device=dev), torch.randn(ngla, device=dev)
+    extra["hgrn2_gates_fwd"] = (lambda: lib.lmoe_hgrn2_gate_fwd(p(x), None, p(hk), p(hg), ngla, 64, bf, st), ngla * (2 + 2 + 4))
+    extra["hgrn2_gates_bwd"] = (lambda: lib.lmoe_hgrn2_gate_bwd(p(x), None, p(dy), p(hdg), p(out), ngla, 64, bf, st),
+                                ngla * (2 + 2 + 4 + 2))
+    frows, fD, fKp = 8 * 16 * 2048, 16, 192
+    fx, fdx = (torch.randn(frows, fD, device=dev, dtype=torch.bfloat16) for _ in range(2))
+    fy = torch.randn(frows * fKp, device=dev, dtype=torch.bfloat16)
+    fc = (1.0, fD ** -0.25, (2.0 * fD) ** -0.5, fD ** -0.5)
+    extra["taylor_featmap_fwd"] = (lambda: lib.lmoe_quad_featmap_fwd(p(fx), p(fy), frows, fD, fKp, *fc, bf, st),
+                                   frows * (fD + fKp) * 2)
+    extra["taylor_featmap_bwd"] = (lambda: lib.lmoe_quad_featmap_bwd(p(fx), p(fy), p(fdx), frows, fD, fKp, *fc, bf, st),
+                                   frows * (2 * fD + fKp) * 2)
     res = {}
     cases = {n: (f, k * rows * D * 2) for n, (f, k) in cases.items()}
     cases.update(extra)

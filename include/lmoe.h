@@ -186,6 +186,30 @@ int lmoe_gla_gate_fwd(const void* x, void* y, int64_t n, int32_t dtype, float no
 int lmoe_gla_gate_bwd(const void* x, const void* dy, void* dx, int64_t n, int32_t dtype, float normalizer,
                       float clamp_min, void* stream);
 
+/* Gates of HGRN2 over n contiguous elements whose last dimension is D (n a multiple of D, D a multiple of 8):
+ *   k = 1 - G (element type),  g = log G (fp32),  G = lb + (1 - lb) sigmoid(f),
+ * lower_bound ([D] fp32) null: lb = 0, i.e. k = 1 - sigmoid(f), g = logsigmoid(f)
+ * (linear_moe/sequence_modeling/linear_rnn.py:327-335; the op is then called as chunk_gla(q, k, i, g),
+ * linear_moe/sequence_modeling/hgrn2/hgrn2.py:76).  Backward: df from dk (element type) and dg (fp32). */
+int lmoe_hgrn2_gate_fwd(const void* f, const float* lower_bound, void* k, float* g, int64_t n, int32_t D, int32_t dtype,
+                        void* stream);
+int lmoe_hgrn2_gate_bwd(const void* f, const float* lower_bound, const void* dk, const float* dg, void* df, int64_t n,
+                        int32_t D, int32_t dtype, void* stream);
+
+/* Quadratic feature maps in front of chunk_linear_attn, rows of D in {8, 16, 32} numbers:
+ *   phi(x) = [ c0 (if c0 != 0) | c1 x_i (if c1 != 0) | cd x_i^2 | co x_i x_j (i < j, row-major) ]
+ * TaylorFeatureMap of Based (linear_moe/model/common_modules/feature_map.py:190-203; call
+ * linear_moe/sequence_modeling/based/based.py:68): c0 = 1, c1 = D^-1/4, cd = (2D)^-1/2, co = D^-1/2;
+ * RebasedFeatureMap flattened (feature_map.py:243-246; call .../rebased/rebased.py:72): c0 = c1 = 0,
+ * cd = D^-1/2, co = (2/D)^1/2.  lmoe_quad_featmap_features gives the feature count F; the output is zero-padded to
+ * Kp >= F (a multiple of 64) and laid out as key blocks of 128 columns (the last may have 64): block b is a
+ * contiguous [rows][width_b] matrix at element offset rows * 128 * b.  Backward: dx from dy in that layout. */
+int lmoe_quad_featmap_features(int32_t D, float c0, float c1);
+int lmoe_quad_featmap_fwd(const void* x, void* y, int64_t rows, int32_t D, int32_t Kp, float c0, float c1, float cd,
+                          float co, int32_t dtype, void* stream);
+int lmoe_quad_featmap_bwd(const void* x, const void* dy, void* dx, int64_t rows, int32_t D, int32_t Kp, float c0,
+                          float c1, float cd, float co, int32_t dtype, void* stream);
+
 /* Row routing for mixture-of-memories layers.  The reference pads the tokens routed to each (memory, batch
  * row) to a common capacity (`transform`, linear_moe/sequence_modeling/mom_linear_attention.py:15-77), calls
  * the op once per memory (:369-409) and scatters the results back (`reconstruct`, :79-120).  Here the routed

@@ -48,6 +48,8 @@ ENTRY_POINTS = (
     "lmoe_launch_stage", "lmoe_selftest_gemm", "lmoe_workspace_bytes", "lmoe_l2norm_fwd", "lmoe_l2norm_bwd",
     "lmoe_silu_l2norm_fwd", "lmoe_silu_l2norm_bwd", "lmoe_rmsnorm_partials", "lmoe_rmsnorm_fwd", "lmoe_rmsnorm_bwd",
     "lmoe_gdn_gates_partials", "lmoe_gdn_gates_fwd", "lmoe_gdn_gates_bwd", "lmoe_gla_gate_fwd", "lmoe_gla_gate_bwd",
+    "lmoe_hgrn2_gate_fwd", "lmoe_hgrn2_gate_bwd", "lmoe_quad_featmap_features", "lmoe_quad_featmap_fwd",
+    "lmoe_quad_featmap_bwd",
     "lmoe_fused_recurrent_fwd", "lmoe_mom_gather", "lmoe_mom_combine", "lmoe_mom_rowdot",
 )
 
@@ -102,6 +104,18 @@ def load() -> C.CDLL:
     lib.lmoe_gla_gate_bwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_float, C.c_float,
                                       C.c_void_p]
     lib.lmoe_gla_gate_bwd.restype = C.c_int
+    lib.lmoe_hgrn2_gate_fwd.argtypes = [C.c_void_p] * 4 + [C.c_int64, C.c_int32, C.c_int32, C.c_void_p]
+    lib.lmoe_hgrn2_gate_fwd.restype = C.c_int
+    lib.lmoe_hgrn2_gate_bwd.argtypes = [C.c_void_p] * 5 + [C.c_int64, C.c_int32, C.c_int32, C.c_void_p]
+    lib.lmoe_hgrn2_gate_bwd.restype = C.c_int
+    lib.lmoe_quad_featmap_features.argtypes = [C.c_int32, C.c_float, C.c_float]
+    lib.lmoe_quad_featmap_features.restype = C.c_int
+    lib.lmoe_quad_featmap_fwd.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32] + [C.c_float] * 4 + [
+        C.c_int32, C.c_void_p]
+    lib.lmoe_quad_featmap_fwd.restype = C.c_int
+    lib.lmoe_quad_featmap_bwd.argtypes = [C.c_void_p] * 3 + [C.c_int64, C.c_int32, C.c_int32] + [C.c_float] * 4 + [
+        C.c_int32, C.c_void_p]
+    lib.lmoe_quad_featmap_bwd.restype = C.c_int
     lib.lmoe_fused_recurrent_fwd.argtypes = [C.POINTER(Args), C.c_int32, C.c_void_p]
     lib.lmoe_fused_recurrent_fwd.restype = C.c_int
     lib.lmoe_mom_gather.argtypes = [C.c_void_p] * 4 + [C.c_int64, C.c_int32, C.c_int32, C.c_void_p]

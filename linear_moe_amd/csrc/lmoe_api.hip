@@ -326,6 +326,64 @@ int lmoe_gla_gate_bwd(const void* x, const void* dy, void* dx, int64_t n, int32_
   return launched(nm);
 }
 
+static int check_hgrn2(const char* nm, const void* f, const void* lb, int64_t n, int32_t D, int32_t dtype) {
+  if (!f) return fail(-1, "%s: null pointer", nm);
+  if (dtype != LMOE_BF16 && dtype != LMOE_F32) return fail(-2, "%s: dtype must be LMOE_BF16 or LMOE_F32", nm);
+  if (D <= 0 || D % 8) return fail(-4, "%s: D must be a positive multiple of 8", nm);
+  if (n < 0 || n % D) return fail(-4, "%s: element count must be a non-negative multiple of D", nm);
+  if (((uintptr_t)f & 15) || ((uintptr_t)lb & 3)) return fail(-9, "%s: pointers must be 16-byte aligned", nm);
+  return 0;
+}
+int lmoe_hgrn2_gate_fwd(const void* f, const float* lower_bound, void* k, float* g, int64_t n, int32_t D, int32_t dtype,
+                        void* stream) {
+  const char* nm = "lmoe_hgrn2_gate_fwd";
+  if (int r = check_hgrn2(nm, f, lower_bound, n, D, dtype)) return r;
+  if (!k || !g || (((uintptr_t)k | (uintptr_t)g) & 15)) return fail(-1, "%s: k and g must be 16-byte aligned pointers", nm);
+  if (n == 0) return 0;
+  lmoe::launch_hgrn2_gate(dtype, f, lower_bound, k, g, nullptr, nullptr, nullptr, n, D, false, (hipStream_t)stream);
+  return launched(nm);
+}
+int lmoe_hgrn2_gate_bwd(const void* f, const float* lower_bound, const void* dk, const float* dg, void* df, int64_t n,
+                        int32_t D, int32_t dtype, void* stream) {
+  const char* nm = "lmoe_hgrn2_gate_bwd";
+  if (int r = check_hgrn2(nm, f, lower_bound, n, D, dtype)) return r;
+  if (!dk || !dg || !df || (((uintptr_t)dk | (uintptr_t)dg | (uintptr_t)df) & 15))
+    return fail(-1, "%s: dk, dg and df must be 16-byte aligned pointers", nm);
+  if (n == 0) return 0;
+  lmoe::launch_hgrn2_gate(dtype, f, lower_bound, nullptr, nullptr, dk, dg, df, n, D, true, (hipStream_t)stream);
+  return launched(nm);
+}
+
+int lmoe_quad_featmap_features(int32_t D, float c0, float c1) { return lmoe::quad_featmap_features(D, c0, c1); }
+static int check_featmap(const char* nm, const void* x, const void* y, int64_t rows, int32_t D, int32_t Kp, float c0,
+                         float c1, int32_t dtype) {
+  if (!x || !y) return fail(-1, "%s: null pointer", nm);
+  if (dtype != LMOE_BF16 && dtype != LMOE_F32) return fail(-2, "%s: dtype must be LMOE_BF16 or LMOE_F32", nm);
+  if (D != 8 && D != 16 && D != 32) return fail(-4, "%s: D must be 8, 16 or 32", nm);
+  if (rows < 0) return fail(-4, "%s: negative row count", nm);
+  if (Kp <= 0 || Kp % 64 || Kp < lmoe::quad_featmap_features(D, c0, c1))
+    return fail(-4, "%s: Kp must be a multiple of 64 not below the feature count %d", nm, lmoe::quad_featmap_features(D, c0, c1));
+  if (((uintptr_t)x | (uintptr_t)y) & 15) return fail(-9, "%s: pointers must be 16-byte aligned", nm);
+  return 0;
+}
+int lmoe_quad_featmap_fwd(const void* x, void* y, int64_t rows, int32_t D, int32_t Kp, float c0, float c1, float cd,
+                          float co, int32_t dtype, void* stream) {
+  const char* nm = "lmoe_quad_featmap_fwd";
+  if (int r = check_featmap(nm, x, y, rows, D, Kp, c0, c1, dtype)) return r;
+  if (rows == 0) return 0;
+  lmoe::launch_quad_featmap(dtype, x, y, nullptr, nullptr, rows, D, Kp, c0, c1, cd, co, false, (hipStream_t)stream);
+  return launched(nm);
+}
+int lmoe_quad_featmap_bwd(const void* x, const void* dy, void* dx, int64_t rows, int32_t D, int32_t Kp, float c0,
+                          float c1, float cd, float co, int32_t dtype, void* stream) {
+  const char* nm = "lmoe_quad_featmap_bwd";
+  if (int r = check_featmap(nm, x, dx, rows, D, Kp, c0, c1, dtype)) return r;
+  if (!dy || ((uintptr_t)dy & 15)) return fail(-1, "%s: dy must be a 16-byte aligned pointer", nm);
+  if (rows == 0) return 0;
+  lmoe::launch_quad_featmap(dtype, x, nullptr, dy, dx, rows, D, Kp, c0, c1, cd, co, true, (hipStream_t)stream);
+  return launched(nm);
+}
+
 int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* stream) {
   const char* nm = "lmoe_launch_stage";
   if (int r = check_common(a, nm)) return r;

@@ -10,6 +10,11 @@
 //    adds the partial rows in a fixed order.
 //  * chunk_gla (linear_moe/sequence_modeling/gla/gla.py:85, :90-91):
 //        gk = max(logsigmoid(x) / normalizer, clamp_min),   dx = dy (1 - sigmoid(x)) / normalizer [gk > clamp_min]
+//  * HGRN2 (linear_moe/sequence_modeling/linear_rnn.py:327-335): from the forget projection f, in fp32,
+//        k = 1 - sigmoid(f),  g = logsigmoid(f)                                   (no lower bound)
+//        G = lb + (1 - lb) sigmoid(f),  k = 1 - G,  g = log G                     (lower bound lb[col])
+//    k in the dtype of f, g in fp32.  Backward, with s = sigmoid(f) (lb = 0, G = s without a bound):
+//        df = (dg / G - dk) (1 - lb) s (1 - s)
 #include "lmoe_launch.hpp"
 #include "lmoe_seq.hpp"
 
@@ -119,6 +124,72 @@ __global__ __launch_bounds__(NTHR) void k_gla_gate(const T* __restrict__ x, cons
     }
     *(vec*)(out + i * VEC) = o;
   }
+}
+
+template <typename T, bool BWD>
+__global__ __launch_bounds__(NTHR) void k_hgrn2_gate(const T* __restrict__ f, const float* __restrict__ lb,
+                                                     T* __restrict__ k, float* __restrict__ g, const T* __restrict__ dk,
+                                                     const float* __restrict__ dg, T* __restrict__ df, int64_t nvec, int D) {
+  constexpr int VEC = ET<T>::VEC;
+  typedef typename ET<T>::vec vec;
+  for (int64_t i = (int64_t)blockIdx.x * NTHR + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * NTHR) {
+    const vec fv = *(const vec*)(f + i * VEC);
+    const int col = (int)((i * VEC) % D);
+    float lo[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) lo[j] = lb ? lb[col + j] : 0.0f;
+    if constexpr (BWD) {
+      const vec dkv = *(const vec*)(dk + i * VEC);
+      float dgv[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; j += 4) {
+        const f32x4 t = *(const f32x4*)(dg + i * VEC + j);
+        dgv[j] = t[0], dgv[j + 1] = t[1], dgv[j + 2] = t[2], dgv[j + 3] = t[3];
+      }
+      vec o;
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float z = ET<T>::to_f(fv[j]), s = sigm(z), G = lo[j] + (1.0f - lo[j]) * s;
+        // dg / G: for lb = 0 this is dg / s, and (1 / s) s (1 - s) = 1 - s stays finite as s -> 0
+        const float dgG = lb ? dgv[j] / G * s : dgv[j];
+        o[j] = ET<T>::from_f((dgG - ET<T>::to_f(dkv[j]) * s) * (1.0f - lo[j]) * (1.0f - s));
+      }
+      *(vec*)(df + i * VEC) = o;
+    } else {
+      vec kv;
+      float lgv[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float z = ET<T>::to_f(fv[j]);
+        float G, lg;
+        if (lb) {
+          G = lo[j] + (1.0f - lo[j]) * sigm(z);
+          lg = __logf(G);
+        } else {
+          G = sigm(z);
+          lg = logsigmoidf_(z);
+        }
+        kv[j] = ET<T>::from_f(1.0f - G);
+        lgv[j] = lg;
+      }
+      *(vec*)(k + i * VEC) = kv;
+#pragma unroll
+      for (int j = 0; j < VEC; j += 4) *(f32x4*)(g + i * VEC + j) = f32x4{lgv[j], lgv[j + 1], lgv[j + 2], lgv[j + 3]};
+    }
+  }
+}
+
+void launch_hgrn2_gate(int dtype, const void* f, const float* lb, void* k, float* g, const void* dk, const float* dg,
+                       void* df, int64_t n, int D, bool bwd, hipStream_t st) {
+#define LMOE_G(T)                                                                                                     \
+  {                                                                                                                   \
+    const int64_t nvec = n / ET<T>::VEC, blocks = (nvec + NTHR - 1) / NTHR, cap = (int64_t)cu_count() * 8;            \
+    const int grid = (int)(blocks < cap ? blocks : cap);                                                              \
+    if (bwd) hipLaunchKernelGGL((k_hgrn2_gate<T, true>), dim3(grid), dim3(NTHR), 0, st, (const T*)f, lb, (T*)nullptr, (float*)nullptr, (const T*)dk, dg, (T*)df, nvec, D); \
+    else hipLaunchKernelGGL((k_hgrn2_gate<T, false>), dim3(grid), dim3(NTHR), 0, st, (const T*)f, lb, (T*)k, g, (const T*)nullptr, (const float*)nullptr, (T*)nullptr, nvec, D); \
+  }
+  if (dtype == LMOE_BF16) LMOE_G(bf16) else LMOE_G(float)
+#undef LMOE_G
 }
 
 void launch_gla_gate(int dtype, const void* x, const void* dy, void* out, int64_t n, float normalizer, float clamp_min,

@@ -60,6 +60,13 @@ int gdn_gates_partials(int64_t rows, int H);
 // chunk_gla gate: logsigmoid(x) / normalizer, clamped from below (n elements, a multiple of 8)
 void launch_gla_gate(int dtype, const void* x, const void* dy, void* out, int64_t n, float normalizer, float clamp_min,
                      bool bwd, hipStream_t st);
+// HGRN2 gates: k = 1 - G, g = log G, G = lb + (1 - lb) sigmoid(f) (n elements, last dimension D, lb [D] or null)
+void launch_hgrn2_gate(int dtype, const void* f, const float* lb, void* k, float* g, const void* dk, const float* dg,
+                       void* df, int64_t n, int D, bool bwd, hipStream_t st);
+// quadratic feature maps (Taylor / ReBased) into key blocks of 128 columns
+int quad_featmap_features(int D, float c0, float c1);
+void launch_quad_featmap(int dtype, const void* x, void* y, const void* dy, void* dx, int64_t rows, int D, int Kp,
+                         float c0, float c1, float cd, float co, bool bwd, hipStream_t st);
 // row routing of mixture-of-memories layers (rows of D elements, D a multiple of 8)
 void launch_mom_gather(int dtype, const void* src, const int32_t* idx, const void* scale, void* out, int64_t nout, int D,
                        hipStream_t st);

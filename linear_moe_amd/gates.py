@@ -5,6 +5,8 @@
 (``linear_moe/sequence_modeling/linear_attention.py:153-154``; parameters ``:92-113``).
 ``gla_gate``: ``logsigmoid(x) / normalizer`` with the optional lower clamp of
 ``linear_moe/sequence_modeling/gla/gla.py:85, :90-91``.
+``hgrn2_gates``: ``k = 1 - sigmoid(f)``, ``g = logsigmoid(f)`` (fp32), optionally with a lower bound
+(``linear_moe/sequence_modeling/linear_rnn.py:327-335``), in front of ``chunk_gla(q, k, i, g)``.
 """
 from __future__ import annotations
 
@@ -98,3 +100,46 @@ class _GlaGate(torch.autograd.Function):
 def gla_gate(x: torch.Tensor, normalizer: float = 16.0, clamp_min=None) -> torch.Tensor:
     """``max(logsigmoid(x) / normalizer, clamp_min)`` in the dtype of x."""
     return _GlaGate.apply(x, normalizer, clamp_min)
+
+
+class _Hgrn2Gates(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, f, lower_bound):
+        if not f.is_cuda:
+            raise RuntimeError("linear_moe_amd ops are GPU only (no CPU fallback)")
+        D = f.shape[-1]
+        if D % 8:
+            raise ValueError("hgrn2_gates: the last dimension must be a multiple of 8")
+        lb = None
+        if lower_bound is not None:
+            if lower_bound.shape != (D,):
+                raise ValueError(f"hgrn2_gates: lower_bound must have shape ({D},)")
+            lb = lower_bound.detach().float().contiguous()
+        lib = _lib.load()
+        fc = f.contiguous()
+        k = torch.empty_like(fc)
+        g = torch.empty(fc.shape, dtype=torch.float32, device=f.device)
+        _lib.check(lib.lmoe_hgrn2_gate_fwd(fc.data_ptr(), None if lb is None else lb.data_ptr(), k.data_ptr(), g.data_ptr(),
+                                           fc.numel(), D, _dt(f), stream_ptr()), "hgrn2_gates")
+        ctx.save_for_backward(fc, lb)
+        return k, g
+
+    @staticmethod
+    def backward(ctx, dk, dg):
+        fc, lb = ctx.saved_tensors
+        lib = _lib.load()
+        dkc = torch.zeros_like(fc) if dk is None else dk.to(fc.dtype).contiguous()
+        dgc = torch.zeros_like(fc, dtype=torch.float32) if dg is None else dg.float().contiguous()
+        df = torch.empty_like(fc)
+        _lib.check(lib.lmoe_hgrn2_gate_bwd(fc.data_ptr(), None if lb is None else lb.data_ptr(), dkc.data_ptr(),
+                                           dgc.data_ptr(), df.data_ptr(), fc.numel(), fc.shape[-1], _dt(fc), stream_ptr()),
+                   "hgrn2_gates backward")
+        return df, None
+
+
+def hgrn2_gates(f: torch.Tensor, lower_bound: torch.Tensor = None):
+    """(k, g) for the forget projection f of shape [..., D]: k in the dtype of f, g fp32.  ``lower_bound`` ([D]) is
+    taken as a constant (no gradient flows to it)."""
+    if lower_bound is not None and lower_bound.requires_grad:
+        raise NotImplementedError("hgrn2_gates: no gradient for lower_bound; pass lower_bound.detach()")
+    return _Hgrn2Gates.apply(f, lower_bound)

@@ -1,7 +1,11 @@
 """``chunk_linear_attn``: chunk_simple_gla without decay, optionally normalised by
 q . cumsum(k).  Called by the reference at
 ``linear_moe/sequence_modeling/basic_linear_attention/basic_linear_attention.py:133`` and, with
-``normalize=True, scale=1``, by ``.../based/based.py:69`` and ``.../rebased/rebased.py:76``."""
+``normalize=True, scale=1``, by ``.../based/based.py:69`` and ``.../rebased/rebased.py:76``.
+
+The key dimension may be any size: without decay the op is a sum over key blocks, so q and k are taken either as
+tensors (split here into blocks of 128 / 64 columns, zero-padded) or as the key blocks the feature maps of
+``feature_map.py`` write directly."""
 from __future__ import annotations
 
 from typing import Optional, Tuple
@@ -21,9 +25,52 @@ def chunk_linear_attn(
     normalize: bool = True,
     head_first: bool = True,
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
-    o, ht = chunk_simple_gla(q, k, v, None, scale, initial_state, output_final_state, None, head_first)
+    qb, kb = _key_blocks(q), _key_blocks(k)
+    if [b.shape for b in qb] != [b.shape for b in kb]:
+        raise ValueError("chunk_linear_attn: q and k must agree in shape")
+    K = sum(b.shape[-1] for b in qb)          # padded key dimension
+    if scale is None:
+        scale = (q.features if hasattr(q, "features") else q.shape[-1]) ** -0.5
+    if initial_state is not None and initial_state.shape[-2] != K:
+        if initial_state.shape[-2] > K:
+            raise ValueError(f"chunk_linear_attn: initial_state has {initial_state.shape[-2]} key rows, q has {K}")
+        initial_state = torch.nn.functional.pad(initial_state, (0, 0, 0, K - initial_state.shape[-2]))
+    tdim = 2 if head_first else 1
+    o, hts, z, k0 = None, [], None, 0
+    for qi, ki in zip(qb, kb):
+        w = qi.shape[-1]
+        h0 = None if initial_state is None else initial_state[..., k0:k0 + w, :].contiguous()
+        oi, hi = chunk_simple_gla(qi, ki, v, None, scale, h0, output_final_state, None, head_first)
+        o = oi if o is None else o + oi
+        hts.append(hi)
+        if normalize:
+            zi = (qi * ki.cumsum(tdim)).sum(-1, keepdim=True)
+            z = zi if z is None else z + zi
+        k0 += w
     if normalize:
-        tdim = 2 if head_first else 1
-        z = (q * k.cumsum(tdim)).sum(-1, keepdim=True) + 1e-10
-        o = o / z
+        o = o / (z + 1e-10)
+    ht = None
+    if output_final_state:
+        ht = hts[0] if len(hts) == 1 else torch.cat(hts, dim=-2)
+        feats = q.features if hasattr(q, "features") else q.shape[-1]
+        if feats != K:
+            ht = ht[..., :feats, :]
     return o, ht
+
+
+def _key_blocks(x):
+    """x as a list of contiguous key blocks of 128 / 64 columns (zero-padded)."""
+    if isinstance(x, (tuple, list)):
+        return list(x)
+    K = x.shape[-1]
+    if K in (64, 128):
+        return [x]
+    Kp = -(-K // 64) * 64
+    if Kp != K:
+        x = torch.nn.functional.pad(x, (0, Kp - K))
+    out, k0 = [], 0
+    while k0 < Kp:
+        w = 128 if Kp - k0 >= 128 else 64
+        out.append(x[..., k0:k0 + w].contiguous())
+        k0 += w
+    return out

@@ -286,3 +286,50 @@ def naive_gla_gate(x: Tensor, normalizer: float = 16.0, clamp_min=None, dtype=to
     import torch.nn.functional as F
     y = F.logsigmoid(x.to(dtype)) / normalizer
     return y if clamp_min is None else torch.clamp_min(y, clamp_min)
+
+
+def naive_hgrn2_gates(f: Tensor, lower_bound: Tensor = None, dtype=torch.float64):
+    """(k, g) of HGRN2 (linear_moe/sequence_modeling/linear_rnn.py:327-335): without a lower bound
+    k = 1 - sigmoid(f), g = logsigmoid(f); with one G = lb + (1 - lb) sigmoid(f), k = 1 - G, g = log G."""
+    import torch.nn.functional as F
+    f = f.to(dtype)
+    if lower_bound is None:
+        return 1 - torch.sigmoid(f), F.logsigmoid(f)
+    G = lower_bound.to(dtype) + (1 - lower_bound.to(dtype)) * torch.sigmoid(f)
+    return 1 - G, torch.log(G)
+
+
+def _pair_products(x: Tensor):
+    """(off-diagonal x_i x_j for i < j in row-major order of the strict upper triangle, diagonal x_i^2):
+    ``flatten_diag_outer_product_off1(x, x)`` of linear_moe/model/common_modules/feature_map.py:24-30, as loops."""
+    D = x.shape[-1]
+    off = [x[..., i] * x[..., j] for i in range(D) for j in range(i + 1, D)]
+    diag = [x[..., i] * x[..., i] for i in range(D)]
+    return torch.stack(off, dim=-1), torch.stack(diag, dim=-1)
+
+
+def naive_taylor_feature_map(x: Tensor, dtype=torch.float64) -> Tensor:
+    """TaylorFeatureMap of Based (feature_map.py:190-203): [1 | x / D^(1/4) | x_i^2 / sqrt(2 D) | x_i x_j / sqrt(D)]."""
+    x = x.to(dtype)
+    D = x.shape[-1]
+    off, diag = _pair_products(x)
+    rd = math.sqrt(D)
+    return torch.cat([torch.ones_like(x[..., :1]), x / math.sqrt(rd), diag / (rd * math.sqrt(2.0)), off / rd], dim=-1)
+
+
+def naive_rebased_feature_map(x: Tensor, gamma: Tensor = None, beta: Tensor = None, normalize: bool = True,
+                              eps: float = 1e-6, dtype=torch.float64) -> Tensor:
+    """RebasedFeatureMap with flatten=True (feature_map.py:206-246; its layer norm has eps 1e-6, layernorm.py:474):
+    x' = gamma * norm(x) + beta, then [x'_i^2 / sqrt(D) | x'_i x'_j sqrt(2 / D)]."""
+    x = x.to(dtype)
+    D = x.shape[-1]
+    if normalize:
+        mu = x.mean(-1, keepdim=True)
+        var = ((x - mu) ** 2).mean(-1, keepdim=True)
+        x = (x - mu) / torch.sqrt(var + eps)
+    if gamma is not None:
+        x = x * gamma.to(dtype)
+    if beta is not None:
+        x = x + beta.to(dtype)
+    off, diag = _pair_products(x)
+    return torch.cat([diag * D ** -0.5, off * (2.0 / D) ** 0.5], dim=-1)

@@ -1,0 +1,190 @@
+"""GPU parity of the callers that ride on the chunk ops: HGRN2 gates in front of chunk_gla, the quadratic
+feature maps of Based / ReBased in front of chunk_linear_attn over key blocks, and sequence-parallel slice
+transitions (HIP, through the C ABI) against the fp64 oracle."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import naive
+from tests.util import TOL, gen, max_abs_rel
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("bound", [False, True])
+def test_hgrn2_gates_fwd_bwd(cuda, dtype, bound):
+    from linear_moe_amd.gates import hgrn2_gates
+    D = 64
+    f = (2 * gen(2101, 3, 37, D)).to(dtype)
+    lb = torch.sigmoid(gen(2102, D)) * 0.9 if bound else None
+    dk, dg = gen(2103, 3, 37, D, dtype=dtype), gen(2104, 3, 37, D)
+    fr = f.double().requires_grad_(True)
+    kr, gr = naive.naive_hgrn2_gates(fr, lb)
+    ((kr * dk.double()).sum() + (gr * dg.double()).sum()).backward()
+    fd = f.to(cuda).requires_grad_(True)
+    k, g = hgrn2_gates(fd, None if lb is None else lb.to(cuda))
+    ((k * dk.to(cuda)).sum() + (g * dg.to(cuda)).sum()).backward()
+    torch.cuda.synchronize()
+    assert k.dtype == dtype and g.dtype == torch.float32
+    assert max_abs_rel(k.detach().cpu(), kr.detach()) < TOL[dtype]
+    # g is fp32 whatever the dtype of f
+    assert max_abs_rel(g.detach().cpu(), gr.detach()) < TOL[torch.float32] * 10
+    assert max_abs_rel(fd.grad.cpu(), fr.grad) < TOL[dtype]
+
+
+def test_hgrn2_path_matches_oracle(cuda):
+    """q, f, i -> gates -> chunk_gla(q, k, i, g) as HGRN2 calls it (g in fp32, the rest bf16), forward and
+    the gradient that reaches f through both k and g."""
+    from linear_moe_amd import chunk_gla
+    from linear_moe_amd.gates import hgrn2_gates
+    B, H, T, D = 2, 2, 150, 64
+    dt = torch.bfloat16
+    q, f, i = gen(2111, B, H, T, D, dtype=dt), gen(2112, B, H, T, D, dtype=dt), gen(2113, B, H, T, D, dtype=dt)
+    do = gen(2114, B, H, T, D, dtype=dt)
+    fr, qr, ir = (x.double().requires_grad_(True) for x in (f, q, i))
+    kr, gr = naive.naive_hgrn2_gates(fr)
+    ref, _ = naive.naive_recurrent_gla(qr, kr.detach().to(dt).double() + (kr - kr.detach()), ir, gr)
+    (ref * do.double()).sum().backward()
+    fd, qd, idd = (x.to(cuda).requires_grad_(True) for x in (f, q, i))
+    k, g = hgrn2_gates(fd)
+    o, _ = chunk_gla(qd, k, idd, g)
+    (o * do.to(cuda)).sum().backward()
+    torch.cuda.synchronize()
+    assert max_abs_rel(o.detach().cpu(), ref.detach()) < TOL[dt]
+    for a, b in ((fd, fr), (qd, qr), (idd, ir)):
+        assert max_abs_rel(a.grad.cpu(), b.grad) < TOL[dt]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("D", [8, 16, 32])
+@pytest.mark.parametrize("kind", ["taylor", "rebased"])
+def test_feature_maps_fwd_bwd(cuda, dtype, D, kind):
+    from linear_moe_amd.feature_map import rebased_feature_map, taylor_feature_map
+    x = gen(2200 + D, 2, 3, 75, D, dtype=dtype)
+    ga, be = (1 + 0.1 * gen(2201, D)).to(dtype), (0.1 * gen(2202, D)).to(dtype)
+    xr = x.double().requires_grad_(True)
+    if kind == "taylor":
+        ref = naive.naive_taylor_feature_map(xr)
+    else:
+        ref = naive.naive_rebased_feature_map(xr, ga.double(), be.double())
+    dy = gen(2203 + D, *ref.shape, dtype=dtype)
+    (ref * dy.double()).sum().backward()
+    xd = x.to(cuda).requires_grad_(True)
+    blocks = taylor_feature_map(xd) if kind == "taylor" else rebased_feature_map(xd, ga.to(cuda), be.to(cuda))
+    assert blocks.features == ref.shape[-1]
+    widths = [b.shape[-1] for b in blocks]
+    assert all(w == 128 for w in widths[:-1]) and widths[-1] in (64, 128) and sum(widths) >= blocks.features
+    assert all(b.is_contiguous() for b in blocks)
+    full = torch.cat(tuple(blocks), dim=-1)
+    assert torch.count_nonzero(full[..., blocks.features:]) == 0            # the padding is zero
+    y = blocks.dense()
+    (y * dy.to(cuda)).sum().backward()
+    torch.cuda.synchronize()
+    assert max_abs_rel(y.detach().cpu(), ref.detach()) < TOL[dtype]
+    assert max_abs_rel(xd.grad.cpu(), xr.grad) < TOL[dtype]
+
+
+@pytest.mark.parametrize("kind", ["taylor", "rebased"])
+def test_based_path_matches_oracle(cuda, kind):
+    """feature map -> chunk_linear_attn(normalize=True, scale=1) over key blocks, as Based / ReBased call it,
+    forward and gradients; and the same features handed over as one dense tensor (fla's layout) give the same."""
+    from linear_moe_amd import chunk_linear_attn
+    from linear_moe_amd.feature_map import rebased_feature_map, taylor_feature_map
+    B, H, T, D, V = 2, 2, 200, 16, 64
+    dt = torch.bfloat16
+    q, k = (0.5 * gen(2301, B, H, T, D)).to(dt), (0.5 * gen(2302, B, H, T, D)).to(dt)
+    v, do = gen(2303, B, H, T, V, dtype=dt), gen(2304, B, H, T, V, dtype=dt)
+    fm_ref = naive.naive_taylor_feature_map if kind == "taylor" else (lambda x: naive.naive_rebased_feature_map(x, None, None))
+    fm = taylor_feature_map if kind == "taylor" else (lambda x: rebased_feature_map(x))
+    qr, kr, vr = (x.double().requires_grad_(True) for x in (q, k, v))
+    ref, _ = naive.naive_linear_attn(fm_ref(qr), fm_ref(kr), vr, scale=1.0, normalize=True)
+    (ref * do.double()).sum().backward()
+    qd, kd, vd = (x.to(cuda).requires_grad_(True) for x in (q, k, v))
+    o, ht = chunk_linear_attn(fm(qd), fm(kd), vd, scale=1.0, normalize=True, output_final_state=True)
+    (o * do.to(cuda)).sum().backward()
+    torch.cuda.synchronize()
+    assert ht.shape == (B, H, fm_ref(qr).shape[-1], V)
+    # the normaliser q . cumsum(k) is formed in bf16 by torch, as fla does; its rounding dominates the error
+    tol = 3 * TOL[dt]
+    assert max_abs_rel(o.detach().cpu(), ref.detach()) < tol
+    for a, b in ((qd, qr), (kd, kr), (vd, vr)):
+        assert max_abs_rel(a.grad.cpu(), b.grad) < tol
+    with torch.no_grad():
+        o2, _ = chunk_linear_attn(fm(qd).dense(), fm(kd).dense(), vd, scale=1.0, normalize=True)
+    assert max_abs_rel(o2.cpu(), o.detach().cpu()) < 1e-2
+
+
+def test_parallel_based_and_rebased_weights(cuda):
+    """parallel_based / parallel_rebased against masked attention with the polynomial weights written out:
+    o_t = sum_{s<=t} w(q_t.k_s) v_s / (sum_{s<=t} w(q_t.k_s) + eps), w = 1 + x + x^2/2 resp. x^2, x = q.k/sqrt(D)."""
+    from linear_moe_amd.based import parallel_based, parallel_rebased
+    B, H, T, D, V = 1, 2, 130, 16, 64
+    dt = torch.float32
+    q, k, v = 0.7 * gen(2501, B, H, T, D), 0.7 * gen(2502, B, H, T, D), gen(2503, B, H, T, V)
+    x = torch.einsum("bhtd,bhsd->bhts", q.double(), k.double()) / D ** 0.5
+    mask = torch.tril(torch.ones(T, T, dtype=torch.float64))
+    for fn, w, eps in ((parallel_based, 1 + x + x * x / 2, 1e-6), (parallel_rebased, x * x, 1e-5)):
+        w = w * mask
+        ref = (w @ v.double()) / (w.sum(-1, keepdim=True) + eps)
+        if fn is parallel_based:
+            o = fn(q.to(cuda), k.to(cuda), v.to(cuda), True, True)
+        else:
+            o = fn(q.to(cuda), k.to(cuda), v.to(cuda), eps, True, True)
+        torch.cuda.synchronize()
+        # ReBased: the first tokens divide by a weight sum that can be tiny; fp32 throughout keeps them accurate
+        assert max_abs_rel(o.cpu(), ref) < 1e-4, fn.__name__
+
+
+@pytest.mark.parametrize("op", ["linear", "simple_gla", "gla", "gdn"])
+def test_slice_transitions_compose_on_gpu(cuda, op):
+    """Four T-slices, each run from the state that the transitions of the lower slices give, equal the whole
+    sequence in one call: outputs, and gradients that cross slice boundaries through initial_state."""
+    from linear_moe_amd import chunk_gated_delta_rule, chunk_gla, chunk_simple_gla, lasp
+    B, H, T, K, V = 2, 2, 512, 64, 64
+    dt = torch.bfloat16
+    cuts = [0, 128, 200, 391, 512]
+    q, k = gen(2401, B, T, H, K), F.normalize(gen(2402, B, T, H, K), dim=-1)
+    v, do = gen(2403, B, T, H, V), gen(2404, B, T, H, V)
+    g = F.logsigmoid(gen(2405, B, T, H) + 3.0)
+    gk = F.logsigmoid(gen(2406, B, T, H, K) + 3.0)
+    beta = torch.sigmoid(gen(2407, B, T, H))
+    scale = K ** -0.5
+
+    def run(qq, kk, vv, gg, gkk, bb, h0):
+        if op == "linear":
+            return chunk_simple_gla(qq, kk, vv, None, scale, h0, False, None, False)[0]
+        if op == "simple_gla":
+            return chunk_simple_gla(qq, kk, vv, gg, scale, h0, False, None, False)[0]
+        if op == "gla":
+            return chunk_gla(qq, kk, vv, gkk, scale, h0, False, None, False)[0]
+        return chunk_gated_delta_rule(qq, kk, vv, gg, bb, scale, h0, False, None, False)[0]
+
+    def transition(kk, vv, gg, gkk, bb):
+        if op == "linear":
+            return lasp.simple_gla_transition(kk, vv, None, head_first=False)
+        if op == "simple_gla":
+            return lasp.simple_gla_transition(kk, vv, gg, head_first=False)
+        if op == "gla":
+            return lasp.gla_transition(kk, vv, gkk, head_first=False)
+        return lasp.gated_delta_rule_transition(kk, vv, gg, bb, head_first=False)
+
+    def leaves():
+        return [x.to(dt).to(cuda).requires_grad_(True) for x in (q, k, v)] + [g.to(cuda), gk.to(cuda), beta.to(dt).to(cuda)]
+
+    full = leaves()
+    o_full = run(*full, None)
+    (o_full * do.to(dt).to(cuda)).sum().backward()
+    part = leaves()
+    outs, trans = [], []
+    for a, b in zip(cuts[:-1], cuts[1:]):
+        sl = [x[:, a:b].contiguous() for x in part]
+        outs.append(run(*sl, lasp.combine_transitions(trans)))
+        trans.append(transition(*sl[1:]))
+    o_part = torch.cat(outs, dim=1)
+    (o_part * do.to(dt).to(cuda)).sum().backward()
+    torch.cuda.synchronize()
+    ref = o_full.detach().float().cpu()
+    assert max_abs_rel(o_part.detach().float().cpu(), ref) < TOL[dt]
+    for a, b in zip(part[:3], full[:3]):
+        assert max_abs_rel(a.grad.float().cpu(), b.grad.float().cpu()) < TOL[dt]

@@ -144,6 +144,8 @@ def test_fla_shim_resolves_every_name_the_reference_imports():
         "from fla.ops.retention import (chunk_retention, fused_chunk_retention, fused_recurrent_retention,\n"
         "                               parallel_retention)\n"
         "from fla.ops.simple_gla import chunk_simple_gla\n"
+        "from fla.ops.based import parallel_based\n"
+        "from fla.ops.rebased import parallel_rebased\n"
         "from fla.modules.l2norm import l2_norm\n"
         "from lightning_attn.ops.triton import lightning_attn2, lightning_attn2_no_decay\n"
         "import linear_moe_amd, torch\n"

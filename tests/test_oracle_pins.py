@@ -341,6 +341,91 @@ def test_gate_construction_pins():
     assert torch.equal(naive.naive_gla_gate(x, 16.0, clamp_min=-1.0)[1], torch.tensor(-1.0, dtype=torch.float64))
 
 
+def test_hgrn2_gate_pins():
+    """k + exp(g) = 1 always (k = 1 - G, g = log G); f = 0 gives k = 1/2, g = -log 2; a lower bound of 1 closes
+    the gate (k = 0, g = 0) and of 0 changes nothing; G >= lb."""
+    import math
+    f = rnd(7401, 3, 5, 8).double() * 3
+    k, g = naive.naive_hgrn2_gates(f)
+    assert torch.allclose(k + g.exp(), torch.ones_like(k), atol=1e-15)
+    k0, g0 = naive.naive_hgrn2_gates(torch.zeros(1, 8, dtype=torch.float64))
+    assert torch.allclose(k0, torch.full((1, 8), 0.5, dtype=torch.float64)) and torch.allclose(g0, torch.full((1, 8), -math.log(2.0), dtype=torch.float64))
+    lb = torch.tensor([0.0, 1.0, 0.25, 0.5, 0.0, 1.0, 0.75, 0.1], dtype=torch.float64)
+    kl, gl = naive.naive_hgrn2_gates(f, lb)
+    assert torch.allclose(kl + gl.exp(), torch.ones_like(kl), atol=1e-15)
+    assert torch.equal(kl[..., 1], torch.zeros_like(kl[..., 1])) and torch.equal(gl[..., 5], torch.zeros_like(gl[..., 5]))
+    assert torch.allclose(kl[..., 0], k[..., 0]) and torch.allclose(gl[..., 4], g[..., 4])
+    assert (gl.exp() >= lb - 1e-15).all()
+    # f -> -inf with lb = 0.25: G -> 0.25
+    kk, gg = naive.naive_hgrn2_gates(torch.full((1, 8), -60.0, dtype=torch.float64), lb)
+    assert torch.allclose(gg[0, 2], torch.tensor(math.log(0.25), dtype=torch.float64))
+
+
+def test_feature_map_pins():
+    """Kernel identities the maps are built for: Taylor phi(q).phi(k) = 1 + s + s^2/2, s = q.k/sqrt(D); ReBased
+    (no norm, gamma = 1) phi(q).phi(k) = (q.k)^2/D.  Feature order against torch.triu_indices, the indexing the
+    reference uses (feature_map.py:24-30), and feature counts 1 + D + D(D+1)/2 and D(D+1)/2."""
+    D = 16
+    q, k = rnd(7501, 2, 3, 7, D).double(), rnd(7502, 2, 3, 7, D).double()
+    s = (q * k).sum(-1) / D ** 0.5
+    pq, pk = naive.naive_taylor_feature_map(q), naive.naive_taylor_feature_map(k)
+    assert pq.shape[-1] == 1 + D + D * (D + 1) // 2 == 153
+    assert torch.allclose((pq * pk).sum(-1), 1 + s + s * s / 2, atol=1e-12)
+    one = torch.ones(D, dtype=torch.float64)
+    rq = naive.naive_rebased_feature_map(q, one, None, normalize=False)
+    rk = naive.naive_rebased_feature_map(k, one, None, normalize=False)
+    assert rq.shape[-1] == D * (D + 1) // 2 == 136
+    assert torch.allclose((rq * rk).sum(-1), (q * k).sum(-1) ** 2 / D, atol=1e-12)
+    # order: [diag | off] for ReBased, [1 | x | diag | off] for Taylor, off in triu_indices(D, D, 1) order
+    z = torch.einsum("...i,...j->...ij", q, q)
+    iu = torch.triu_indices(D, D, 1)
+    ar = torch.arange(D)
+    assert torch.allclose(rq[..., :D], z[..., ar, ar] * D ** -0.5) and torch.allclose(rq[..., D:], z[..., iu[0], iu[1]] * (2.0 / D) ** 0.5)
+    assert torch.allclose(pq[..., 1 + D:1 + 2 * D], z[..., ar, ar] / (2.0 * D) ** 0.5)
+    assert torch.allclose(pq[..., 1 + 2 * D:], z[..., iu[0], iu[1]] / D ** 0.5)
+    assert torch.allclose(pq[..., 1:1 + D], q / D ** 0.25) and torch.equal(pq[..., 0], torch.ones_like(pq[..., 0]))
+    # the norm in front of the ReBased map is torch's layer norm with eps 1e-6
+    ga, be = 1 + 0.1 * rnd(7503, D).double(), 0.1 * rnd(7504, D).double()
+    ln = F.layer_norm(q, (D,), ga, be, 1e-6)
+    assert torch.allclose(naive.naive_rebased_feature_map(q, ga, be), naive.naive_rebased_feature_map(ln, None, None, normalize=False), atol=1e-13)
+
+
+def test_slice_transitions_compose():
+    """Sequence-parallel composition: running slices from the state the transitions of lower slices give equals
+    the whole sequence (ungated, scalar and per-channel gates: S_out = decay S_in + M; delta rule: S_out = P S_in
+    + M with P the final state of the v = 0 recurrence started from the identity)."""
+    B, H, T, K, V = 1, 2, 24, 4, 3
+    q, k, v = rnd(7601, B, H, T, K).double(), F.normalize(rnd(7602, B, H, T, K).double(), dim=-1), rnd(7603, B, H, T, V).double()
+    g = F.logsigmoid(rnd(7604, B, H, T).double())
+    gk = F.logsigmoid(rnd(7605, B, H, T, K).double())
+    beta = torch.sigmoid(rnd(7606, B, H, T).double())
+    cuts = [0, 5, 16, 24]
+    zero = torch.zeros(B, H, K, V, dtype=torch.float64)
+    eye = torch.eye(K, dtype=torch.float64).expand(B, H, K, K)
+    sl = lambda x, a, b: x[:, :, a:b]
+    cases = {
+        "scalar": (lambda a, b, h0: naive.naive_recurrent_simple_gla(sl(q, a, b), sl(k, a, b), sl(v, a, b), sl(g, a, b), 1.0, h0, True),
+                   lambda a, b: sl(g, a, b).sum(2).exp()[..., None, None]),
+        "channel": (lambda a, b, h0: naive.naive_recurrent_gla(sl(q, a, b), sl(k, a, b), sl(v, a, b), sl(gk, a, b), 1.0, h0, True),
+                    lambda a, b: sl(gk, a, b).sum(2).exp()[..., None]),
+    }
+    for name, (run, decay) in cases.items():
+        full, _ = run(0, T, zero)
+        state, outs = zero, []
+        for a, b in zip(cuts[:-1], cuts[1:]):
+            outs.append(run(a, b, state)[0])
+            state = decay(a, b) * state + run(a, b, zero)[1]
+        assert torch.allclose(torch.cat(outs, 2), full, atol=1e-12), name
+    rung = lambda a, b, h0, vv: naive.naive_recurrent_gated_delta_rule(sl(q, a, b), sl(k, a, b), vv, sl(g, a, b), sl(beta, a, b), 1.0, h0, True, head_first=True)
+    full, _ = rung(0, T, zero, v)
+    state, outs = zero, []
+    for a, b in zip(cuts[:-1], cuts[1:]):
+        outs.append(rung(a, b, state, sl(v, a, b))[0])
+        P = rung(a, b, eye, torch.zeros(B, H, b - a, K, dtype=torch.float64))[1]
+        state = P @ state + rung(a, b, zero, sl(v, a, b))[1]
+    assert torch.allclose(torch.cat(outs, 2), full, atol=1e-12)
+
+
 def test_mom_routing_pins():
     """oracle/mom.py (transform / reconstruct of mom_linear_attention.py:15-120): hand-written expectations
     for a tiny routing (time order, truncation keeps the LAST tokens, zeros on the LEFT), and the properties
