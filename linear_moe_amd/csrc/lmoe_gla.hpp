@@ -18,23 +18,46 @@
 
 namespace lmoe {
 
-// g tile of the chunk -> fp32 LDS tile s_b[64][K+1] holding the inclusive cumsum over tokens.
-// All threads; ends with a barrier.
+// g tile of the chunk -> fp32 LDS tile s_b[64][LDB] holding the inclusive cumsum over tokens.
+// The scan: a thread takes one channel over a segment of 64 K / 256 tokens (its values in registers, so the
+// LDS reads are independent of each other), the segment totals go through a small LDS array, and every thread
+// adds the totals of the segments before its own.  All 256 threads; ends with a barrier.
+template <typename GT, int K>
+struct GlaGate {
+  typedef TileIO<GT, CH, K> IOG;
+  typedef typename IOG::Regs Regs;
+  static __device__ __forceinline__ void issue(Regs& rg, const lmoe_args& a, int b, int tok, int len, int h) {
+    IOG::load_nomask(rg, row_ptr<GT>(a.g, b, tok, h), a.g.st, len);
+  }
+  template <int LDB>
+  static __device__ __forceinline__ void finish(Regs& rg, int len, float* s_b) {
+    constexpr int NSEG = NTHR / K, SEG = CH / NSEG;
+    static_assert(NTHR % K == 0 && CH % NSEG == 0, "one channel and one token segment per thread");
+    __shared__ float s_tot[NSEG * K];
+    IOG::mask(rg, len);
+    IOG::store_lds_f32(rg, s_b, LDB);
+    __syncthreads();
+    const int c = threadIdx.x % K, sg = threadIdx.x / K;
+    float v[SEG];
+#pragma unroll
+    for (int r = 0; r < SEG; ++r) v[r] = s_b[(sg * SEG + r) * LDB + c];
+#pragma unroll
+    for (int r = 1; r < SEG; ++r) v[r] += v[r - 1];
+    s_tot[sg * K + c] = v[SEG - 1];
+    __syncthreads();
+    float off = 0.f;
+#pragma unroll
+    for (int q = 0; q < NSEG - 1; ++q) off += q < sg ? s_tot[q * K + c] : 0.f;
+#pragma unroll
+    for (int r = 0; r < SEG; ++r) s_b[(sg * SEG + r) * LDB + c] = v[r] + off;
+    __syncthreads();
+  }
+};
 template <typename GT, int K, int LDB = K + 1>
 __device__ __forceinline__ void gla_gate_tile(const lmoe_args& a, int b, int tok, int len, int h, float* s_b) {
-  typedef TileIO<GT, CH, K> IOG;
-  typename IOG::Regs rg;
-  IOG::load(rg, row_ptr<GT>(a.g, b, tok, h), a.g.st, len);
-  IOG::store_lds_f32(rg, s_b, LDB);
-  __syncthreads();
-  if (threadIdx.x < K) {
-    float acc = 0.f;
-    for (int r = 0; r < CH; ++r) {
-      acc += s_b[r * LDB + threadIdx.x];
-      s_b[r * LDB + threadIdx.x] = acc;
-    }
-  }
-  __syncthreads();
+  typename GlaGate<GT, K>::Regs rg;
+  GlaGate<GT, K>::issue(rg, a, b, tok, len, h);
+  GlaGate<GT, K>::template finish<LDB>(rg, len, s_b);
 }
 
 // ------------------------------------------------------------------------- //
@@ -139,15 +162,29 @@ __global__ __launch_bounds__(NTHR) void k_gla_state_fwd(const lmoe_args a) {
   }
   typedef TileIO<T, CH, K> IOK;
   typedef TileIO<T, CH, BV> IOV;
+  typedef GlaGate<GT, K> GG;
+  // the next chunk's g, k, v are requested before this chunk's work (chunk index clamped: every load is issued)
+  typename GG::Regs pg;
+  typename IOK::Regs pk;
+  typename IOV::Regs pv;
+  auto issue = [&](int c) {
+    c = min(c, sq.nchunks - 1);
+    const int tok = sq.tok0 + c * CH, len = min(CH, sq.len - c * CH);
+    GG::issue(pg, a, sq.b, tok, len, h);
+    IOK::load_nomask(pk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, len);
+    IOV::load_nomask(pv, row_ptr<T>(a.v, sq.b, tok, h) + v0, a.v.st, len);
+  };
+  if (sq.nchunks > 0) issue(0);
   for (int c = 0; c < sq.nchunks; ++c) {
-    const int tok = sq.tok0 + c * CH;
     const int len = min(CH, sq.len - c * CH);
-    gla_gate_tile<GT, K>(a, sq.b, tok, len, h, s_b);
-    typename IOK::Regs rk;
-    IOK::load(rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, len);
+    typename GG::Regs rg = pg;
+    typename IOK::Regs rk = pk;
+    typename IOV::Regs rv = pv;
+    issue(c + 1);
+    GG::template finish<LDB>(rg, len, s_b);
+    IOK::mask(rk, len);
     IOK::store_lds_t_elem(rk, s_kT, LDC, [&](int r, int cc) { return texp<T>(s_b[63 * LDB + cc] - s_b[r * LDB + cc]); });
-    typename IOV::Regs rv;
-    IOV::load(rv, row_ptr<T>(a.v, sq.b, tok, h) + v0, a.v.st, len);
+    IOV::mask(rv, len);
     IOV::store_lds_t(rv, s_vT, LDC, nullptr);
     T* hs = (T*)a.hs + ((int64_t)(sq.chunk0 + c) * a.H + h) * K * V;
 #pragma unroll
@@ -251,16 +288,30 @@ __global__ __launch_bounds__(NTHR) void k_gla_state_bwd(const lmoe_args a) {
   }
   typedef TileIO<T, CH, K> IOK;
   typedef TileIO<T, CH, BV> IOV;
+  typedef GlaGate<GT, K> GG;
   const float scale = a.scale;
+  // the next chunk's g, q, do are requested before this chunk's work (chunk index clamped: every load is issued)
+  typename GG::Regs pg;
+  typename IOK::Regs pq;
+  typename IOV::Regs pd;
+  auto issue = [&](int c) {
+    c = max(c, 0);
+    const int tok = sq.tok0 + c * CH, len = min(CH, sq.len - c * CH);
+    GG::issue(pg, a, sq.b, tok, len, h);
+    IOK::load_nomask(pq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, len);
+    IOV::load_nomask(pd, row_ptr<T>(a.d_o, sq.b, tok, h) + v0, a.d_o.st, len);
+  };
+  if (sq.nchunks > 0) issue(sq.nchunks - 1);
   for (int c = sq.nchunks - 1; c >= 0; --c) {
-    const int tok = sq.tok0 + c * CH;
     const int len = min(CH, sq.len - c * CH);
-    gla_gate_tile<GT, K>(a, sq.b, tok, len, h, s_b);
-    typename IOK::Regs rq;
-    IOK::load(rq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, len);
+    typename GG::Regs rg = pg;
+    typename IOK::Regs rq = pq;
+    typename IOV::Regs rd = pd;
+    issue(c - 1);
+    GG::template finish<LDB>(rg, len, s_b);
+    IOK::mask(rq, len);
     IOK::store_lds_t_elem(rq, s_qT, LDC, [&](int r, int cc) { return scale * texp<T>(s_b[r * LDB + cc]); });
-    typename IOV::Regs rd;
-    IOV::load(rd, row_ptr<T>(a.d_o, sq.b, tok, h) + v0, a.d_o.st, len);
+    IOV::mask(rd, len);
     IOV::store_lds_t(rd, s_doT, LDC, nullptr);
     T* dhs = (T*)a.dhs + ((int64_t)(sq.chunk0 + c) * a.H + h) * K * V;
 #pragma unroll
@@ -473,38 +524,83 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
   T* dkd_g = row_ptr<T>(a.dk, ci.b, ci.tok, h);
   float kkp[NBK];                      // per column: sum over this lane's rows of (dk_d . k_d)
   float dbv[NBK][4];
+  static_assert(NBK % 4 == 0, "column tiles are taken four at a time");
 #pragma unroll
-  for (int ni = 0; ni < NBK; ++ni) {
-    const int cc = 16 * ni + (l & 15);
-    const float bC = sB[63 * LDB + cc];
-    kkp[ni] = 0.f;
+  for (int nh = 0; nh < NBK; nh += 4) {
+    // Diagonal block of this wave's sub-chunk, for four column tiles at a time.  One pass over the 16 tokens
+    // j of the sub-chunk serves both sums: dA is lower triangular (zero above the diagonal), so
+    //   sq[r] += dA(r, j) k_j e,   sk[r] += dA(j, r) q_j e,   e = e^{-|b_r - b_j|}
+    // (b decreases along the chunk: the exponent wanted is b_r - b_j for j <= r and b_j - b_r for j >= r;
+    // where it is not, the dA factor is zero).  k_j, q_j, b_j are read once per token and column and serve
+    // the lane's four rows; the dA values are read once per token and serve the four column tiles.
+    float sqv[4][4], skv[4][4], brv[4][4];
+    if constexpr (SUB) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int r = 16 * wv + 4 * (l >> 4) + i;
-      const float br = sB[r * LDB + cc];
-      float sq_ = 0.f, sk_ = 0.f;
-      for (int j = jlo; j <= r; ++j) sq_ += Pm(r, j) * Km(j, cc) * texp<T>(br - sB[j * LDB + cc]);
-      for (int ii = r; ii < ihi; ++ii) sk_ += Pm(ii, r) * Qm(ii, cc) * texp<T>(sB[ii * LDB + cc] - br);
-      if constexpr (SUB) {
-        if (wv >= 1) sq_ += dqo[0][ni][i] * texp<T>(br - sB[(16 * wv - 1) * LDB + cc]);
-        if (wv <= 2) sk_ += dko[0][ni][i] * texp<T>(sB[(16 * wv + 15) * LDB + cc] - br);
-      }
-      const float qv = Qm(r, cc), kv = Km(r, cc);
-      const float ed = texp<T>(bC - br);
-      const float dqv = a.scale * texp<T>(br) * dqi[0][ni][i] + sq_;
-      const float dkdv = dkd[0][ni][i] * ed;
-      const float dkv = dkdv + sk_;
-      kkp[ni] += kv * dkdv;
-      dbv[ni][i] = qv * dqv - kv * dkv;
-      if (r < ci.len) {
-        dqd[(int64_t)r * a.dq.st + cc] = ET<T>::from_f(dqv);
-        dkd_g[(int64_t)r * a.dk.st + cc] = ET<T>::from_f(dkv);
+      for (int n4 = 0; n4 < 4; ++n4)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          sqv[n4][i] = skv[n4][i] = 0.f;
+          brv[n4][i] = sB[(16 * wv + 4 * (l >> 4) + i) * LDB + 16 * (nh + n4) + (l & 15)];
+        }
+      for (int jj = 0; jj < 16; ++jj) {
+        const int j = 16 * wv + jj;
+        float pq[4], pk[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int r = 16 * wv + 4 * (l >> 4) + i;
+          pq[i] = Pm(r, j);
+          pk[i] = Pm(j, r);
+        }
+#pragma unroll
+        for (int n4 = 0; n4 < 4; ++n4) {
+          const int cc = 16 * (nh + n4) + (l & 15);
+          const float kj = Km(j, cc), qj = Qm(j, cc), bj = sB[j * LDB + cc];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float e = texp<T>(-fabsf(brv[n4][i] - bj));
+            sqv[n4][i] += pq[i] * kj * e;
+            skv[n4][i] += pk[i] * qj * e;
+          }
+        }
       }
     }
-    // sum over the 4 row groups of the wave
-    kkp[ni] += __shfl_xor(kkp[ni], 16, 64);
-    kkp[ni] += __shfl_xor(kkp[ni], 32, 64);
-    if (l < 16) s_kk[wv * K + cc] = kkp[ni];
+#pragma unroll
+    for (int n4 = 0; n4 < 4; ++n4) {
+      const int ni = nh + n4;
+      const int cc = 16 * ni + (l & 15);
+      const float bC = sB[63 * LDB + cc];
+      kkp[ni] = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = 16 * wv + 4 * (l >> 4) + i;
+        const float br = sB[r * LDB + cc];
+        float sq_ = 0.f, sk_ = 0.f;
+        if constexpr (SUB) {
+          sq_ = sqv[n4][i];
+          sk_ = skv[n4][i];
+          if (wv >= 1) sq_ += dqo[0][ni][i] * texp<T>(br - sB[(16 * wv - 1) * LDB + cc]);
+          if (wv <= 2) sk_ += dko[0][ni][i] * texp<T>(sB[(16 * wv + 15) * LDB + cc] - br);
+        } else {
+          for (int j = jlo; j <= r; ++j) sq_ += Pm(r, j) * Km(j, cc) * texp<T>(br - sB[j * LDB + cc]);
+          for (int ii = r; ii < ihi; ++ii) sk_ += Pm(ii, r) * Qm(ii, cc) * texp<T>(sB[ii * LDB + cc] - br);
+        }
+        const float qv = Qm(r, cc), kv = Km(r, cc);
+        const float ed = texp<T>(bC - br);
+        const float dqv = a.scale * texp<T>(br) * dqi[0][ni][i] + sq_;
+        const float dkdv = dkd[0][ni][i] * ed;
+        const float dkv = dkdv + sk_;
+        kkp[ni] += kv * dkdv;
+        dbv[ni][i] = qv * dqv - kv * dkv;
+        if (r < ci.len) {
+          dqd[(int64_t)r * a.dq.st + cc] = ET<T>::from_f(dqv);
+          dkd_g[(int64_t)r * a.dk.st + cc] = ET<T>::from_f(dkv);
+        }
+      }
+      // sum over the 4 row groups of the wave
+      kkp[ni] += __shfl_xor(kkp[ni], 16, 64);
+      kkp[ni] += __shfl_xor(kkp[ni], 32, 64);
+      if (l < 16) s_kk[wv * K + cc] = kkp[ni];
+    }
   }
   __syncthreads();   // all reads of the q tile are done: reuse it for db
   float* sDB = SUB ? (float*)tKT : smF + B_Q;
