@@ -433,23 +433,40 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
   float hdh[IOH::PASSES];
 #pragma unroll
   for (int p = 0; p < IOH::PASSES; ++p) hdh[p] = 0.f;
-  for (int vv = 0; vv < V; vv += BVH) {
-    {
-      typename IOV::Regs rd, rv;
-      IOV::load(rd, row_ptr<T>(a.d_o, ci.b, ci.tok, h) + vv, a.d_o.st, ci.len);
-      IOV::load(rv, row_ptr<T>(a.v, ci.b, ci.tok, h) + vv, a.v.st, ci.len);
-      typename IOH::Regs rh, rdh;
-      IOH::load(rh, (const T*)a.hs + ((int64_t)cid * a.H + h) * K * V + vv, V, K);
-      IOH::load(rdh, (const T*)a.dhs + ((int64_t)cid * a.H + h) * K * V + vv, V, K);
+  // Loads run one stage ahead of their use: slice s + 1 is requested before slice s is staged, and q, k, g
+  // before the last slice is.
+  constexpr int NSL = V / BVH;
+  struct Slice { typename IOV::Regs rd, rv; typename IOH::Regs rh, rdh; };
+  Slice sl[2];
+  typename IOK::Regs rq, rk;
+  typename GlaGate<GT, K>::Regs rg;
+  auto issue_slice = [&](Slice& x, int vv) {
+    IOV::load_nomask(x.rd, row_ptr<T>(a.d_o, ci.b, ci.tok, h) + vv, a.d_o.st, ci.len);
+    IOV::load_nomask(x.rv, row_ptr<T>(a.v, ci.b, ci.tok, h) + vv, a.v.st, ci.len);
+    IOH::load_nomask(x.rh, (const T*)a.hs + ((int64_t)cid * a.H + h) * K * V + vv, V, K);
+    IOH::load_nomask(x.rdh, (const T*)a.dhs + ((int64_t)cid * a.H + h) * K * V + vv, V, K);
+  };
+  issue_slice(sl[0], 0);
 #pragma unroll
-      for (int p = 0; p < IOH::PASSES; ++p)
-#pragma unroll
-        for (int i = 0; i < IOH::VEC; ++i) hdh[p] += ET<T>::to_f(rh.v[p][i]) * ET<T>::to_f(rdh.v[p][i]);
-      IOV::store_lds(rd, smT + A_DO, LDV);
-      IOV::store_lds(rv, smT + A_V, LDV);
-      IOH::store_lds(rh, smT + A_H, LDV);
-      IOH::store_lds(rdh, smT + A_DH, LDV);
+  for (int si = 0; si < NSL; ++si) {
+    Slice& x = sl[si & 1];
+    if (si + 1 < NSL) {
+      issue_slice(sl[(si + 1) & 1], (si + 1) * BVH);
+    } else {
+      IOK::load_nomask(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
+      IOK::load_nomask(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
+      GlaGate<GT, K>::issue(rg, a, ci.b, ci.tok, ci.len, h);
     }
+    IOV::mask(x.rd, ci.len);
+    IOV::mask(x.rv, ci.len);
+#pragma unroll
+    for (int p = 0; p < IOH::PASSES; ++p)
+#pragma unroll
+      for (int i = 0; i < IOH::VEC; ++i) hdh[p] += ET<T>::to_f(x.rh.v[p][i]) * ET<T>::to_f(x.rdh.v[p][i]);
+    IOV::store_lds(x.rd, smT + A_DO, LDV);
+    IOV::store_lds(x.rv, smT + A_V, LDV);
+    IOH::store_lds(x.rh, smT + A_H, LDV);
+    IOH::store_lds(x.rdh, smT + A_DH, LDV);
     __syncthreads();
     gemm_nt<T, 1, 4>(dP, smT + A_DO, LDV, 16 * wv, smT + A_V, LDV, 0, 0, BVH);
     gemm_nt<T, 1, NBK>(dqi, smT + A_DO, LDV, 16 * wv, smT + A_H, LDV, 0, 0, BVH);
@@ -484,9 +501,8 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
       }
       if constexpr (SUB) acc_to_lds<T>(p, tDA, LDC, 16 * wv, 16 * nj);
     }
-    typename IOK::Regs rq, rk;
-    IOK::load(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
-    IOK::load(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
+    IOK::mask(rq, ci.len);
+    IOK::mask(rk, ci.len);
     if constexpr (SUB) {
       IOK::store_lds(rq, tQ, LDK);
       IOK::store_lds(rk, tK, LDK);
@@ -495,7 +511,7 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
       IOK::store_lds_f32(rk, smF + B_K, LDB);
     }
   }
-  gla_gate_tile<GT, K>(a, ci.b, ci.tok, ci.len, h, sBw);   // barriers inside
+  GlaGate<GT, K>::template finish<LDB>(rg, ci.len, sBw);   // barriers inside
   const float* sB = sBw;
   // dA, q, k of the pairwise loops and the epilogue, from whichever tiles this layout keeps
   auto Pm = [&](int r, int j) { if constexpr (SUB) return ET<T>::to_f(tDA[r * LDC + j]); else return smF[B_DP + r * LDP + j]; };
@@ -612,15 +628,27 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
       sDB[r * LDB + cc] = dbv[ni][i];
     }
   __syncthreads();
-  if (threadIdx.x < K) {
-    const int cc = threadIdx.x;
-    const float last = s_kk[cc] + s_kk[K + cc] + s_kk[2 * K + cc] + s_kk[3 * K + cc] +
-                       texp<T>(sB[63 * LDB + cc]) * s_hdh[cc];
+  // dg = reverse cumsum of db over the tokens (+ the last-row term): a thread takes one channel over a segment
+  // of tokens, the segment totals go through LDS (rows past the end of a partial chunk have zero db)
+  {
+    constexpr int NSEG = NTHR / K, SEG = CH / NSEG;
+    __shared__ float s_seg[NTHR];
+    const int cc = threadIdx.x % K, sg = threadIdx.x / K;
+    float v[SEG];
+#pragma unroll
+    for (int r = 0; r < SEG; ++r) v[r] = sDB[(sg * SEG + r) * LDB + cc];
+#pragma unroll
+    for (int r = SEG - 2; r >= 0; --r) v[r] += v[r + 1];
+    s_seg[sg * K + cc] = v[0];
+    __syncthreads();
+    float off = s_kk[cc] + s_kk[K + cc] + s_kk[2 * K + cc] + s_kk[3 * K + cc] + texp<T>(sB[63 * LDB + cc]) * s_hdh[cc];
+#pragma unroll
+    for (int q = 1; q < NSEG; ++q) off += q > sg ? s_seg[q * K + cc] : 0.f;
     float* dg = (float*)a.dg.ptr + row_off(a.dg, ci.b, ci.tok, h);
-    float acc = last;   // rows past the end of a partial chunk have zero db
-    for (int r = ci.len - 1; r >= 0; --r) {
-      acc += sDB[r * LDB + cc];
-      dg[(int64_t)r * a.dg.st + cc] = acc;
+#pragma unroll
+    for (int r = 0; r < SEG; ++r) {
+      const int row = sg * SEG + r;
+      if (row < ci.len) dg[(int64_t)row * a.dg.st + cc] = v[r] + off;
     }
   }
 }
