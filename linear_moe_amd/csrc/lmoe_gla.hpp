@@ -18,6 +18,8 @@
 
 namespace lmoe {
 
+constexpr int cmax(int a, int b) { return a > b ? a : b; }
+
 // g tile of the chunk -> fp32 LDS tile s_b[64][LDB] holding the inclusive cumsum over tokens.
 // The scan: a thread takes one channel over a segment of 64 K / 256 tokens (its values in registers, so the
 // LDS reads are independent of each other), the segment totals go through a small LDS array, and every thread
@@ -29,11 +31,11 @@ struct GlaGate {
   static __device__ __forceinline__ void issue(Regs& rg, const lmoe_args& a, int b, int tok, int len, int h) {
     IOG::load_nomask(rg, row_ptr<GT>(a.g, b, tok, h), a.g.st, len);
   }
+  // tot: NTHR floats of LDS for the segment totals
   template <int LDB>
-  static __device__ __forceinline__ void finish(Regs& rg, int len, float* s_b) {
+  static __device__ __forceinline__ void finish(Regs& rg, int len, float* s_b, float* s_tot) {
     constexpr int NSEG = NTHR / K, SEG = CH / NSEG;
     static_assert(NTHR % K == 0 && CH % NSEG == 0, "one channel and one token segment per thread");
-    __shared__ float s_tot[NSEG * K];
     IOG::mask(rg, len);
     IOG::store_lds_f32(rg, s_b, LDB);
     __syncthreads();
@@ -51,6 +53,11 @@ struct GlaGate {
 #pragma unroll
     for (int r = 0; r < SEG; ++r) s_b[(sg * SEG + r) * LDB + c] = v[r] + off;
     __syncthreads();
+  }
+  template <int LDB>
+  static __device__ __forceinline__ void finish(Regs& rg, int len, float* s_b) {
+    __shared__ float s_tot[NTHR];
+    finish<LDB>(rg, len, s_b, s_tot);
   }
 };
 template <typename GT, int K, int LDB = K + 1>
@@ -90,7 +97,12 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
     IOK::store_lds(rk, s_k, LDK);
   }
   for (int idx = threadIdx.x; idx < CH * LDC; idx += NTHR) s_A[idx] = ET<T>::from_f(0.f);   // blocks above the diagonal
-  gla_gate_tile<GT, K, LDB>(a, ci.b, ci.tok, ci.len, h, s_b);    // barriers inside
+  {
+    typename GlaGate<GT, K>::Regs rg;
+    GlaGate<GT, K>::issue(rg, a, ci.b, ci.tok, ci.len, h);
+    static_assert(16 * LDK * sizeof(T) >= NTHR * 4, "the scan's scratch fits the q~ tile");
+    GlaGate<GT, K>::template finish<LDB>(rg, ci.len, s_b, (float*)s_qt);    // barriers inside
+  }
   // ---- diagonal blocks: wave w owns block (w, w); lane -> row i, columns j0 .. j0 + 3 ----
   {
     const int i = 16 * wv + (l & 15), j0 = 16 * wv + 4 * (l >> 4);
@@ -219,37 +231,48 @@ template <typename T, typename GT, int K, int V, int BV>
 __global__ __launch_bounds__(NTHR) void k_gla_out_fwd(const lmoe_args a) {
   constexpr int LDB = K + 1, LDK = K + LPAD, LDC = CH + LPAD;
   constexpr int NB = BV / 16;
-  __shared__ float s_b[CH * LDB];
-  __shared__ __attribute__((aligned(16))) T s_q[CH * LDK];
-  __shared__ __attribute__((aligned(16))) T s_hT[BV * LDK];
-  __shared__ __attribute__((aligned(16))) T s_P[CH * LDC];
-  __shared__ __attribute__((aligned(16))) T s_vT[BV * LDC];
+  // Two LDS regions, each used twice (small LDS -> more work-groups per CU, which is what hides the load
+  // latency of these one-shot work-groups):  R0: gate cumsum b (fp32) + scan scratch, then S^T, then v^T;
+  // R1: q e^{b}, then A.  Every load is requested up front and waits in registers for its region.
+  constexpr int R0_BYTES = cmax(cmax(CH * LDB * 4 + NTHR * 4, BV * LDK * (int)sizeof(T)), BV * LDC * (int)sizeof(T));
+  constexpr int R1_ELEMS = cmax(CH * LDK, CH * LDC);
+  __shared__ __attribute__((aligned(16))) unsigned char r0[R0_BYTES];
+  __shared__ __attribute__((aligned(16))) T r1[R1_ELEMS];
+  float* s_b = (float*)r0;
+  T* s_hT = (T*)r0; T* s_vT = (T*)r0;
+  T* s_q = r1; T* s_P = r1;
   const int cid = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * BV;
   const ChunkInfo ci = chunk_info(a, cid);
   const int wv = wave_id(), l = lane_id();
-  gla_gate_tile<GT, K>(a, ci.b, ci.tok, ci.len, h, s_b);
   typedef TileIO<T, CH, K> IOK;
   typedef TileIO<T, CH, BV> IOV;
   typedef TileIO<T, K, BV> IOH;
   typedef TileIO<T, CH, CH> IOA;
-  {
-    typename IOK::Regs rq;
-    IOK::load(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
-    IOK::store_lds_elem(rq, s_q, LDK, [&](int r, int cc) { return texp<T>(s_b[r * LDB + cc]); });
-    typename IOV::Regs rv;
-    IOV::load(rv, row_ptr<T>(a.v, ci.b, ci.tok, h) + v0, a.v.st, ci.len);
-    IOV::store_lds_t(rv, s_vT, LDC, nullptr);
-    typename IOH::Regs rh;
-    IOH::load(rh, (const T*)a.hs + ((int64_t)cid * a.H + h) * K * V + v0, V, K);
-    IOH::store_lds_t(rh, s_hT, LDK, nullptr);
-    typename IOA::Regs ra;
-    IOA::load(ra, (const T*)a.amat + ((int64_t)cid * a.H + h) * CH * CH, CH, CH);
-    IOA::store_lds(ra, s_P, LDC);
-  }
+  typedef GlaGate<GT, K> GG;
+  typename GG::Regs rg;
+  typename IOK::Regs rq;
+  typename IOV::Regs rv;
+  typename IOH::Regs rh;
+  typename IOA::Regs ra;
+  GG::issue(rg, a, ci.b, ci.tok, ci.len, h);
+  IOK::load_nomask(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
+  IOH::load_nomask(rh, (const T*)a.hs + ((int64_t)cid * a.H + h) * K * V + v0, V, K);
+  IOA::load_nomask(ra, (const T*)a.amat + ((int64_t)cid * a.H + h) * CH * CH, CH, CH);
+  IOV::load_nomask(rv, row_ptr<T>(a.v, ci.b, ci.tok, h) + v0, a.v.st, ci.len);
+  GG::template finish<LDB>(rg, ci.len, s_b, s_b + CH * LDB);                             // barriers inside
+  IOK::mask(rq, ci.len);
+  IOK::store_lds_elem(rq, s_q, LDK, [&](int r, int cc) { return texp<T>(s_b[r * LDB + cc]); });
+  __syncthreads();                                                                       // b is dead
+  IOH::store_lds_t(rh, s_hT, LDK, nullptr);
   __syncthreads();
   f32x4 o[1][NB];
   acc_zero(o);
   gemm_nt<T, 1, NB>(o, s_q, LDK, 16 * wv, s_hT, LDK, 0, 0, K);
+  __syncthreads();                                                                       // q e^{b}, S^T are dead
+  IOA::store_lds(ra, s_P, LDC);
+  IOV::mask(rv, ci.len);
+  IOV::store_lds_t(rv, s_vT, LDC, nullptr);
+  __syncthreads();
   gemm_nt<T, 1, NB>(o, s_P, LDC, 16 * wv, s_vT, LDC, 0, 0, CH);
   T* od = row_ptr<T>(a.o, ci.b, ci.tok, h) + v0;
 #pragma unroll
@@ -346,47 +369,55 @@ template <typename T, typename GT, int K, int V, int BV>
 __global__ __launch_bounds__(NTHR) void k_gla_bwd_dv(const lmoe_args a) {
   constexpr int LDB = K + 1, LDK = K + LPAD, LDC = CH + LPAD;
   constexpr int NB = BV / 16;
-  __shared__ float s_b[CH * LDB];
-  __shared__ __attribute__((aligned(16))) T s_kd[CH * LDK];
-  __shared__ __attribute__((aligned(16))) T s_dhT[BV * LDK];
-  __shared__ __attribute__((aligned(16))) T s_PT[CH * LDC];
-  __shared__ __attribute__((aligned(16))) T s_doT[BV * LDC];
+  // two LDS regions, each used twice (see k_gla_out_fwd):  R0: b + scan scratch, then dS'^T, then do^T;
+  // R1: k e^{b_C - b}, then A^T
+  constexpr int R0_BYTES = cmax(cmax(CH * LDB * 4 + NTHR * 4, BV * LDK * (int)sizeof(T)), BV * LDC * (int)sizeof(T));
+  constexpr int R1_ELEMS = cmax(CH * LDK, CH * LDC);
+  __shared__ __attribute__((aligned(16))) unsigned char r0[R0_BYTES];
+  __shared__ __attribute__((aligned(16))) T r1[R1_ELEMS];
+  float* s_b = (float*)r0;
+  T* s_dhT = (T*)r0; T* s_doT = (T*)r0;
+  T* s_kd = r1; T* s_PT = r1;
   const int cid = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * BV;
   const ChunkInfo ci = chunk_info(a, cid);
   const int wv = wave_id(), l = lane_id();
-  gla_gate_tile<GT, K>(a, ci.b, ci.tok, ci.len, h, s_b);
   typedef TileIO<T, CH, K> IOK;
   typedef TileIO<T, CH, BV> IOV;
   typedef TileIO<T, K, BV> IOH;
   typedef TileIO<T, CH, CH> IOA;
-  {
-    typename IOK::Regs rk;
-    IOK::load(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
-    IOK::store_lds_elem(rk, s_kd, LDK, [&](int r, int cc) { return texp<T>(s_b[63 * LDB + cc] - s_b[r * LDB + cc]); });
-    typename IOV::Regs rd;
-    IOV::load(rd, row_ptr<T>(a.d_o, ci.b, ci.tok, h) + v0, a.d_o.st, ci.len);
-    IOV::store_lds_t(rd, s_doT, LDC, nullptr);
-    typename IOH::Regs rh;
-    IOH::load(rh, (const T*)a.dhs + ((int64_t)cid * a.H + h) * K * V + v0, V, K);
-    IOH::store_lds_t(rh, s_dhT, LDK, nullptr);
-    typename IOA::Regs ra;
-    IOA::load(ra, (const T*)a.amat + ((int64_t)cid * a.H + h) * CH * CH, CH, CH);
-    IOA::store_lds_t(ra, s_PT, LDC, nullptr);
-  }
+  typedef GlaGate<GT, K> GG;
+  typename GG::Regs rg;
+  typename IOK::Regs rk;
+  typename IOV::Regs rd;
+  typename IOH::Regs rh;
+  typename IOA::Regs ra;
+  GG::issue(rg, a, ci.b, ci.tok, ci.len, h);
+  IOK::load_nomask(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
+  IOH::load_nomask(rh, (const T*)a.dhs + ((int64_t)cid * a.H + h) * K * V + v0, V, K);
+  IOA::load_nomask(ra, (const T*)a.amat + ((int64_t)cid * a.H + h) * CH * CH, CH, CH);
+  IOV::load_nomask(rd, row_ptr<T>(a.d_o, ci.b, ci.tok, h) + v0, a.d_o.st, ci.len);
+  GG::template finish<LDB>(rg, ci.len, s_b, s_b + CH * LDB);                             // barriers inside
+  IOK::mask(rk, ci.len);
+  IOK::store_lds_elem(rk, s_kd, LDK, [&](int r, int cc) { return texp<T>(s_b[63 * LDB + cc] - s_b[r * LDB + cc]); });
+  __syncthreads();                                                                       // b is dead
+  IOH::store_lds_t(rh, s_dhT, LDK, nullptr);
   __syncthreads();
-  f32x4 dv[1][NB];
-  acc_zero(dv);
+  f32x4 dv[1][NB], dv2[1][NB];
+  acc_zero(dv); acc_zero(dv2);
+  gemm_nt<T, 1, NB>(dv2, s_kd, LDK, 16 * wv, s_dhT, LDK, 0, 0, K);
+  __syncthreads();                                                                       // k e^{..}, dS'^T are dead
+  IOA::store_lds_t(ra, s_PT, LDC, nullptr);
+  IOV::mask(rd, ci.len);
+  IOV::store_lds_t(rd, s_doT, LDC, nullptr);
+  __syncthreads();
   gemm_nt<T, 1, NB>(dv, s_PT, LDC, 16 * wv, s_doT, LDC, 0, 0, CH);
-#pragma unroll
-  for (int ni = 0; ni < NB; ++ni) dv[0][ni] *= a.scale;
-  gemm_nt<T, 1, NB>(dv, s_kd, LDK, 16 * wv, s_dhT, LDK, 0, 0, K);
   T* dd = row_ptr<T>(a.dv, ci.b, ci.tok, h) + v0;
 #pragma unroll
   for (int ni = 0; ni < NB; ++ni)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
-      if (r < ci.len) dd[(int64_t)r * a.dv.st + cc] = ET<T>::from_f(dv[0][ni][i]);
+      if (r < ci.len) dd[(int64_t)r * a.dv.st + cc] = ET<T>::from_f(a.scale * dv[0][ni][i] + dv2[0][ni][i]);
     }
 }
 
