@@ -34,8 +34,8 @@ STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_gdn_state_fwd", 4: "k_gdn_state_bwd", 5:
 # copy that main() issues first (FETCH_SIZE reads half of the bytes fetched, WRITE_SIZE all of the
 # bytes written).  Summary and commands: profiles/gdn_fwd_bwd_cfg4_hbm_traffic.md.
 CALIB_COPY_BYTES = 256 << 20
-MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 835757110, "k_gdn_state_fwd": 1145226210, "k_gdn_state_bwd": 1011013644,
-                    "k_gdn_bwd_chunk": 1883778163}
+MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 835791600, "k_gdn_state_fwd": 1145229793, "k_gdn_state_bwd": 1010960861,
+                    "k_gdn_bwd_chunk": 1885054894}
 
 
 def gdn_inputs(B, T, H, K, V, seed, dtype, device):
@@ -225,6 +225,79 @@ def neighbours(lib, rows, D, dev, reps):
             "config": {"workload": f"{rows} rows x {D} bf16 (q / k / o rows of B=4 H=16 T=8192)"}, "kernels": res}
 
 
+def other_configs(dev, steps, warmup):
+    """The four contract configurations beside the headline one, through the Python entry points (inputs of
+    the contract's laws, drawn on the GPU: this leg times, the parity tests check): ms per call, tokens/s and
+    the algorithmic bytes (every input read once, every output written once) against the HBM peak."""
+    import torch
+    import torch.nn.functional as F
+    import linear_moe_amd as L
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps
+
+    rn = lambda *s, dt=torch.bfloat16: torch.randn(*s, device=dev, dtype=dt)
+    res = {}
+    # 1: basic linear attention forward, fp32
+    B, H, T, K = 1, 4, 512, 64
+    q, k, v = (rn(B, H, T, K, dt=torch.float32) for _ in range(3))
+    with torch.no_grad():
+        sec = timed(lambda: L.chunk_linear_attn(q, k, v, normalize=False))
+    res["1 linear_attn fwd fp32 B=1 H=4 T=512 K=V=64"] = (sec, B * T, B * T * H * (2 * K + 2 * K) * 4)
+    # 2: retention forward, bf16
+    B, H, T, K = 4, 16, 4096, 128
+    q, k, v = (rn(B, H, T, K) for _ in range(3))
+    with torch.no_grad():
+        sec = timed(lambda: L.chunk_retention(q, k, v, output_final_state=True))
+    res["2 retention fwd bf16 B=4 H=16 T=4096 K=V=128"] = (sec, B * T, B * T * H * ((2 * K + 2 * K) * 2 + 4))
+    # 3: chunk_gla forward + backward, bf16
+    B, H, T, K, V = 8, 16, 2048, 64, 128
+    q, k = (rn(B, H, T, K).requires_grad_(True) for _ in range(2))
+    v = rn(B, H, T, V).requires_grad_(True)
+    g = (F.logsigmoid(rn(B, H, T, K, dt=torch.float32)) / 16).bfloat16().requires_grad_(True)
+    do = rn(B, H, T, V)
+
+    def f3():    # autograd.grad: no accumulation into .grad, which would be timed with the op
+        o, _ = L.chunk_gla(q, k, v, g)
+        torch.autograd.grad([o], [q, k, v, g], [do])
+    sec = timed(f3)
+    res["3 chunk_gla fwd+bwd bf16 B=8 H=16 T=2048 K=64 V=128"] = (sec, B * T, B * T * H * (9 * K + 5 * V) * 2)
+    # 5: packed gated delta rule forward + backward, 16 sequences of log-normal lengths, 65536 tokens
+    N, Tt, H, K, V = 16, 65536, 32, 128, 128
+    gen = torch.Generator().manual_seed(1005)
+    raw = torch.exp(8 + torch.randn(N, generator=gen))
+    lens = torch.clamp((raw / raw.sum() * Tt).floor().long(), min=1)
+    lens[lens.argmax()] += Tt - lens.sum()
+    cu = torch.zeros(N + 1, dtype=torch.int32)
+    cu[1:] = lens.cumsum(0)
+    cu = cu.to(dev)
+    q = F.normalize(rn(1, Tt, H, K, dt=torch.float32), dim=-1).bfloat16().requires_grad_(True)
+    k = F.normalize(rn(1, Tt, H, K, dt=torch.float32), dim=-1).bfloat16().requires_grad_(True)
+    v = rn(1, Tt, H, V).requires_grad_(True)
+    beta = torch.rand(1, Tt, H, device=dev).bfloat16().requires_grad_(True)
+    g = (-torch.rand(1, Tt, H, device=dev)).requires_grad_(True)
+    h0 = (rn(N, H, K, V, dt=torch.float32) * 0.1).requires_grad_(True)
+    do, dht = rn(1, Tt, H, V), rn(N, H, K, V, dt=torch.float32)
+
+    def f5():
+        o, ht = L.chunk_gated_delta_rule(q, k, v, g, beta, None, h0, True, cu, False)
+        torch.autograd.grad([o, ht], [q, k, v, g, beta, h0], [do, dht])
+    sec = timed(f5)
+    res["5 packed gated_delta_rule fwd+bwd bf16 16 seqs 65536 tokens H=32 K=V=128"] = (
+        sec, Tt, Tt * H * ((6 * K + 5 * V) * 2 + 3 * 2 + 12) + 4 * N * H * K * V * 4)
+    return {"metric": "contract configurations 1, 2, 3, 5: ms per call, tokens/s", "unit": "ms", "steps": steps,
+            "warmup": warmup, "data": "synthetic",
+            "configs": {n: {"ms": round(sec * 1e3, 4), "tokens_per_s": round(tok / sec), "algorithmic_bytes": nb,
+                            "frac_hbm_peak": round(nb / sec / PEAK_HBM, 4)} for n, (sec, tok, nb) in res.items()}}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -235,6 +308,8 @@ def main():
     ap.add_argument("--neighbours", action="store_true",
                     help="instead of the headline step: the row-wise kernels around the op (L2 norm, SiLU + L2 norm, "
                          "RMS norm with and without the swish gate) on the rows of the same workload, one JSON line")
+    ap.add_argument("--other-configs", action="store_true",
+                    help="instead of the headline step: contract configurations 1, 2, 3 and 5, one JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the op shards over batch and heads without "
@@ -252,6 +327,9 @@ def main():
     B, T, H, K, V, seed = 4, 8192, 16, 128, 128, 1004
     if args.neighbours:
         print(json.dumps(neighbours(lib, B * T * H, K, dev, args.stage_reps)))
+        return
+    if args.other_configs:
+        print(json.dumps(other_configs(dev, args.steps, args.warmup)))
         return
     x = gdn_inputs(B, T, H, K, V, seed, torch.bfloat16, dev)
 
