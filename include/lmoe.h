@@ -78,7 +78,10 @@ typedef struct lmoe_args {
   void* pmat;          /* [NT,H,64,64] P = (q k^T) . Gamma per chunk (gated delta rule;
                           written by the WY preparation)                                */
   float* gcum;         /* [NT,H,2,64] fp32 e^{b_j} and e^{b_C - b_j}, b = cumulative log-decay
-                          inside the chunk (gated delta rule; written by the WY preparation) */
+                          inside the chunk (gated delta rule; written by the WY preparation);
+                          chunk_gla: [NT,H,K] fp32 e^{b_C} per channel, the decay of a whole chunk */
+  void* qe;            /* [NT,H,64,K] q e^{b}       per chunk, rows past its end zero (chunk_gla) */
+  void* ke;            /* [NT,H,64,K] k e^{b_C - b} per chunk, rows past its end zero (chunk_gla) */
   /* backward inputs */
   lmoe_tensor d_o;     /* [B,T,H,V] gradient of o                                      */
   const float* dht;    /* [N,H,K,V] fp32 gradient of the final state or NULL           */
@@ -98,7 +101,7 @@ int lmoe_version(void);
 const char* lmoe_last_error(void);
 
 /* Bytes of caller-allocated intermediates of one call: part 0 = what *_fwd writes for *_bwd
- * (hs, and per op amat / vnew, w, u, tinv, pmat, gcum), part 1 = the backward workspace (dhs, and dvnew
+ * (hs, and per op amat, qe, ke, gcum / vnew, w, u, tinv, pmat, gcum), part 1 = the backward workspace (dhs, and dvnew
  * for the gated delta rule).  Each buffer is still passed through its own lmoe_args field; this
  * is the sum a caller that carves them out of one arena must reserve (every buffer's size is a
  * multiple of 256 bytes for the supported K, V).  Negative for an invalid op / dtype / part.
@@ -120,7 +123,8 @@ int lmoe_chunk_simple_gla_bwd(const lmoe_args* a, void* stream);
 /* chunk_gla: S_t = diag(e^{g_t}) S_{t-1} + k_t^T v_t, g_t in R^K (gate = VECTOR).
  * Replaces fla.ops.gla.chunk_gla called at
  *   linear_moe/sequence_modeling/gla/gla.py:94 and linear_moe/sequence_modeling/hgrn2/hgrn2.py:76.
- * fwd uses q,k,v,g,h0 -> o,ht,hs,amat.  bwd uses those + d_o,dht -> dq,dk,dv,dg,dh0 (+ dhs). */
+ * fwd uses q,k,v,g,h0 -> o,ht,hs,amat,qe,ke,gcum (the gated operands of the state passes, formed once by
+ * the chunk-parallel kernel).  bwd uses those + d_o,dht -> dq,dk,dv,dg,dh0 (+ dhs). */
 int lmoe_chunk_gla_fwd(const lmoe_args* a, void* stream);
 int lmoe_chunk_gla_bwd(const lmoe_args* a, void* stream);
 

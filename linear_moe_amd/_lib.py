@@ -33,6 +33,7 @@ class Args(C.Structure):
         ("o", Tensor4), ("ht", C.c_void_p),
         ("hs", C.c_void_p), ("vnew", Tensor4), ("w", Tensor4), ("u", Tensor4),
         ("tinv", C.c_void_p), ("amat", C.c_void_p), ("pmat", C.c_void_p), ("gcum", C.c_void_p),
+        ("qe", C.c_void_p), ("ke", C.c_void_p),
         ("d_o", Tensor4), ("dht", C.c_void_p),
         ("dq", Tensor4), ("dk", Tensor4), ("dv", Tensor4), ("dg", Tensor4), ("dbeta", Tensor4),
         ("dh0", C.c_void_p),

@@ -56,11 +56,12 @@ int64_t lmoe_workspace_bytes(int32_t op, int32_t dtype, int32_t part, int32_t B,
   const int64_t states = (int64_t)NT * H * K * V, tiles = (int64_t)NT * H * LMOE_CHUNK * LMOE_CHUNK;
   const int64_t rows_k = (int64_t)B * T * H * K, rows_v = (int64_t)B * T * H * V;
   int64_t n = states;                                                    // hs | dhs
-  if (op == LMOE_OP_GLA && part == 0) n += tiles;                        // amat
+  if (op == LMOE_OP_GLA && part == 0) n += tiles + 2 * (int64_t)NT * H * LMOE_CHUNK * K;   // amat, qe, ke
   if (op == LMOE_OP_GATED_DELTA_RULE) n += part == 0 ? 2 * rows_v + rows_k + 2 * tiles   // vnew, u, w, tinv, pmat
                                                      : rows_v;                       // dvnew
   int64_t bytes = n * s;
   if (op == LMOE_OP_GATED_DELTA_RULE && part == 0) bytes += (int64_t)NT * H * 2 * LMOE_CHUNK * 4;   // gcum (fp32)
+  if (op == LMOE_OP_GLA && part == 0) bytes += (int64_t)NT * H * K * 4;                              // gcum (fp32)
   return bytes;
 }
 
@@ -91,7 +92,8 @@ static int check_gla(const lmoe_args* a, const char* op) {
   if (int r = check_common(a, op)) return r;
   if (a->gate != LMOE_GATE_VECTOR || !a->g.ptr) return fail(-10, "%s: needs a vector gate g [B,T,H,K]", op);
   if (a->dtype == LMOE_F32 && a->g_dtype != LMOE_F32) return fail(-14, "%s: fp32 q/k/v need an fp32 gate", op);
-  if (!a->hs || !a->amat) return fail(-11, "%s: hs and amat must not be null", op);
+  if (!a->hs || !a->amat || !a->qe || !a->ke || !a->gcum)
+    return fail(-11, "%s: hs, amat, qe, ke and gcum must not be null", op);
   return 0;
 }
 

@@ -10,6 +10,10 @@
 //   dk_jk = e^{b_Ck - b_jk} (v dS'^T)_jk + sum_{i>=j} dA_ij q_ik e^{b_ik - b_jk}
 //   db_ik = q_ik dq_ik - k_ik dk_ik (+ on the last row: sum_j (dk_d . k_d)_jk + e^{b_Ck} sum_v S_kv dS'_kv)
 //   dg    = reverse cumsum of db over the chunk's tokens
+// The gated operands q e^{b} and k e^{b_C - b} and the chunk decay e^{b_C} are formed once, by the
+// chunk-parallel kernel that computes A (it holds q, k and b in LDS anyway), and stored per chunk
+// ([NT,H,64,K], rows past the end of a partial chunk zero): the two sequential state passes and the
+// output / dv kernels then need neither the gate nor a scan nor an exponential.
 // Pairwise exponents are formed only inside 16-token sub-chunks (vector ALU, fp32); between
 // sub-chunks the decay factors through the cumulative gate at the sub-chunk boundary, which turns
 // those parts into products of scaled tiles on MFMA, like every other product here.
@@ -103,6 +107,27 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
     static_assert(16 * LDK * sizeof(T) >= NTHR * 4, "the scan's scratch fits the q~ tile");
     GlaGate<GT, K>::template finish<LDB>(rg, ci.len, s_b, (float*)s_qt);    // barriers inside
   }
+  // ---- gated operands for the other kernels: q e^{b}, k e^{b_C - b}, e^{b_C} ----
+  {
+    constexpr int VEC = ET<T>::VEC;
+    typedef typename ET<T>::vec vec;
+    T* qe = (T*)a.qe + ((int64_t)cid * a.H + h) * CH * K;
+    T* ke = (T*)a.ke + ((int64_t)cid * a.H + h) * CH * K;
+    for (int e = threadIdx.x; e < CH * K / VEC; e += NTHR) {
+      const int r = e / (K / VEC), c0 = (e % (K / VEC)) * VEC;
+      const vec qv = *(const vec*)(s_q + r * LDK + c0), kv = *(const vec*)(s_k + r * LDK + c0);
+      vec qo, ko;
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float b = s_b[r * LDB + c0 + j], bC = s_b[63 * LDB + c0 + j];
+        qo[j] = ET<T>::from_f(ET<T>::to_f(qv[j]) * texp<T>(b));
+        ko[j] = ET<T>::from_f(ET<T>::to_f(kv[j]) * texp<T>(bC - b));
+      }
+      *(vec*)(qe + r * K + c0) = qo;
+      *(vec*)(ke + r * K + c0) = ko;
+    }
+    if (threadIdx.x < K) a.gcum[((int64_t)cid * a.H + h) * K + threadIdx.x] = texp<T>(s_b[63 * LDB + threadIdx.x]);
+  }
   // ---- diagonal blocks: wave w owns block (w, w); lane -> row i, columns j0 .. j0 + 3 ----
   {
     const int i = 16 * wv + (l & 15), j0 = 16 * wv + 4 * (l >> 4);
@@ -152,11 +177,11 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
 // ------------------------------------------------------------------------- //
 template <typename T, typename GT, int K, int V, int BV>
 __global__ __launch_bounds__(NTHR) void k_gla_state_fwd(const lmoe_args a) {
-  constexpr int LDB = K + 1, LDC = CH + LPAD;
+  constexpr int LDK = K + LPAD, LDU = BV + LPAD;
   constexpr int MB = K / 64, NB = BV / 16;
-  __shared__ float s_b[CH * LDB];
-  __shared__ __attribute__((aligned(16))) T s_kT[K * LDC];
-  __shared__ __attribute__((aligned(16))) T s_vT[BV * LDC];
+  __shared__ __attribute__((aligned(16))) T s_k[CH * LDK];     // k e^{b_C - b}     [64][K]
+  __shared__ __attribute__((aligned(16))) T s_v[CH * LDU];     // v                 [64][BV]
+  __shared__ __attribute__((aligned(16))) T s_h[K * LDU];      // S on its way out  [K][BV]
   const int v0 = blockIdx.x * BV, h = blockIdx.y, n = blockIdx.z;
   const SeqInfo sq = seq_info(a, n);
   const int wv = wave_id();
@@ -174,43 +199,58 @@ __global__ __launch_bounds__(NTHR) void k_gla_state_fwd(const lmoe_args a) {
   }
   typedef TileIO<T, CH, K> IOK;
   typedef TileIO<T, CH, BV> IOV;
-  typedef GlaGate<GT, K> GG;
-  // the next chunk's g, k, v are requested before this chunk's work (chunk index clamped: every load is issued)
-  typename GG::Regs pg;
+  typedef TileIO<T, K, BV> IOH;
+  // the next chunk's operands are requested before this chunk's work (chunk index clamped: every load is issued)
   typename IOK::Regs pk;
   typename IOV::Regs pv;
+  float pdec[MB][4];
   auto issue = [&](int c) {
     c = min(c, sq.nchunks - 1);
-    const int tok = sq.tok0 + c * CH, len = min(CH, sq.len - c * CH);
-    GG::issue(pg, a, sq.b, tok, len, h);
-    IOK::load_nomask(pk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, len);
-    IOV::load_nomask(pv, row_ptr<T>(a.v, sq.b, tok, h) + v0, a.v.st, len);
+    const int64_t item = (int64_t)(sq.chunk0 + c) * a.H + h;
+    IOK::load_nomask(pk, (const T*)a.ke + item * CH * K, K, CH);
+    IOV::load_nomask(pv, row_ptr<T>(a.v, sq.b, sq.tok0 + c * CH, h) + v0, a.v.st, min(CH, sq.len - c * CH));
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) pdec[mi][i] = a.gcum[item * K + krow0 + acc_row(mi, i)];
   };
   if (sq.nchunks > 0) issue(0);
   for (int c = 0; c < sq.nchunks; ++c) {
     const int len = min(CH, sq.len - c * CH);
-    typename GG::Regs rg = pg;
     typename IOK::Regs rk = pk;
     typename IOV::Regs rv = pv;
-    issue(c + 1);
-    GG::template finish<LDB>(rg, len, s_b);
-    IOK::mask(rk, len);
-    IOK::store_lds_t_elem(rk, s_kT, LDC, [&](int r, int cc) { return texp<T>(s_b[63 * LDB + cc] - s_b[r * LDB + cc]); });
-    IOV::mask(rv, len);
-    IOV::store_lds_t(rv, s_vT, LDC, nullptr);
-    T* hs = (T*)a.hs + ((int64_t)(sq.chunk0 + c) * a.H + h) * K * V;
+    float dec[MB][4];
 #pragma unroll
     for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
-      for (int ni = 0; ni < NB; ++ni)
+      for (int i = 0; i < 4; ++i) dec[mi][i] = pdec[mi][i];
+    issue(c + 1);
+    IOK::store_lds(rk, s_k, LDK);
+    IOV::mask(rv, len);
+    IOV::store_lds(rv, s_v, LDU);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int kr = krow0 + acc_row(mi, i);
-          hs[(int64_t)kr * V + v0 + acc_col(ni)] = ET<T>::from_f(S[mi][ni][i]);
-          S[mi][ni][i] *= texp<T>(s_b[63 * LDB + kr]);
-        }
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) {
+        acc_to_lds<T>(S[mi][ni], s_h, LDU, krow0 + 16 * mi, 16 * ni);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) S[mi][ni][i] *= dec[mi][i];
+      }
     __syncthreads();
-    gemm_nt<T, MB, NB>(S, s_kT, LDC, krow0, s_vT, LDC, 0, 0, CH);
+    IOH::lds_to_global(s_h, LDU, (T*)a.hs + ((int64_t)(sq.chunk0 + c) * a.H + h) * K * V + v0, V, K);
+    // S += (k e^{b_C - b})^T v
+#pragma unroll
+    for (int kk = 0; kk < CH; kk += 32) {
+      typename ET<T>::frag af[MB], bf[NB];
+#pragma unroll
+      for (int mi = 0; mi < MB; ++mi) af[mi] = ET<T>::load_frag_t(s_k, LDK, kk, krow0 + 16 * mi);
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) bf[ni] = ET<T>::load_frag_t(s_v, LDU, kk, 16 * ni);
+#pragma unroll
+      for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) ET<T>::mma(S[mi][ni], af[mi], bf[ni]);
+    }
     __syncthreads();
   }
   if (a.ht) {
@@ -229,17 +269,16 @@ __global__ __launch_bounds__(NTHR) void k_gla_state_fwd(const lmoe_args a) {
 // ------------------------------------------------------------------------- //
 template <typename T, typename GT, int K, int V, int BV>
 __global__ __launch_bounds__(NTHR) void k_gla_out_fwd(const lmoe_args a) {
-  constexpr int LDB = K + 1, LDK = K + LPAD, LDC = CH + LPAD;
+  constexpr int LDK = K + LPAD, LDC = CH + LPAD;
   constexpr int NB = BV / 16;
   // Two LDS regions, each used twice (small LDS -> more work-groups per CU, which is what hides the load
-  // latency of these one-shot work-groups):  R0: gate cumsum b (fp32) + scan scratch, then S^T, then v^T;
-  // R1: q e^{b}, then A.  Every load is requested up front and waits in registers for its region.
-  constexpr int R0_BYTES = cmax(cmax(CH * LDB * 4 + NTHR * 4, BV * LDK * (int)sizeof(T)), BV * LDC * (int)sizeof(T));
+  // latency of these one-shot work-groups):  R0: S^T, then v^T;  R1: q e^{b} (as stored by k_gla_intra_fwd),
+  // then A.  Every load is requested up front and waits in registers for its region.
+  constexpr int R0_ELEMS = cmax(BV * LDK, BV * LDC);
   constexpr int R1_ELEMS = cmax(CH * LDK, CH * LDC);
-  __shared__ __attribute__((aligned(16))) unsigned char r0[R0_BYTES];
+  __shared__ __attribute__((aligned(16))) T r0[R0_ELEMS];
   __shared__ __attribute__((aligned(16))) T r1[R1_ELEMS];
-  float* s_b = (float*)r0;
-  T* s_hT = (T*)r0; T* s_vT = (T*)r0;
+  T* s_hT = r0; T* s_vT = r0;
   T* s_q = r1; T* s_P = r1;
   const int cid = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * BV;
   const ChunkInfo ci = chunk_info(a, cid);
@@ -248,21 +287,15 @@ __global__ __launch_bounds__(NTHR) void k_gla_out_fwd(const lmoe_args a) {
   typedef TileIO<T, CH, BV> IOV;
   typedef TileIO<T, K, BV> IOH;
   typedef TileIO<T, CH, CH> IOA;
-  typedef GlaGate<GT, K> GG;
-  typename GG::Regs rg;
   typename IOK::Regs rq;
   typename IOV::Regs rv;
   typename IOH::Regs rh;
   typename IOA::Regs ra;
-  GG::issue(rg, a, ci.b, ci.tok, ci.len, h);
-  IOK::load_nomask(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
+  IOK::load_nomask(rq, (const T*)a.qe + ((int64_t)cid * a.H + h) * CH * K, K, CH);
   IOH::load_nomask(rh, (const T*)a.hs + ((int64_t)cid * a.H + h) * K * V + v0, V, K);
   IOA::load_nomask(ra, (const T*)a.amat + ((int64_t)cid * a.H + h) * CH * CH, CH, CH);
   IOV::load_nomask(rv, row_ptr<T>(a.v, ci.b, ci.tok, h) + v0, a.v.st, ci.len);
-  GG::template finish<LDB>(rg, ci.len, s_b, s_b + CH * LDB);                             // barriers inside
-  IOK::mask(rq, ci.len);
-  IOK::store_lds_elem(rq, s_q, LDK, [&](int r, int cc) { return texp<T>(s_b[r * LDB + cc]); });
-  __syncthreads();                                                                       // b is dead
+  IOK::store_lds(rq, s_q, LDK);
   IOH::store_lds_t(rh, s_hT, LDK, nullptr);
   __syncthreads();
   f32x4 o[1][NB];
@@ -289,11 +322,11 @@ __global__ __launch_bounds__(NTHR) void k_gla_out_fwd(const lmoe_args a) {
 // ------------------------------------------------------------------------- //
 template <typename T, typename GT, int K, int V, int BV>
 __global__ __launch_bounds__(NTHR) void k_gla_state_bwd(const lmoe_args a) {
-  constexpr int LDB = K + 1, LDC = CH + LPAD;
+  constexpr int LDK = K + LPAD, LDU = BV + LPAD;
   constexpr int MB = K / 64, NB = BV / 16;
-  __shared__ float s_b[CH * LDB];
-  __shared__ __attribute__((aligned(16))) T s_qT[K * LDC];
-  __shared__ __attribute__((aligned(16))) T s_doT[BV * LDC];
+  __shared__ __attribute__((aligned(16))) T s_q[CH * LDK];     // q e^{b}             [64][K]
+  __shared__ __attribute__((aligned(16))) T s_do[CH * LDU];    // do                  [64][BV]
+  __shared__ __attribute__((aligned(16))) T s_h[K * LDU];      // dS' on its way out  [K][BV]
   const int v0 = blockIdx.x * BV, h = blockIdx.y, n = blockIdx.z;
   const SeqInfo sq = seq_info(a, n);
   const int wv = wave_id();
@@ -311,44 +344,65 @@ __global__ __launch_bounds__(NTHR) void k_gla_state_bwd(const lmoe_args a) {
   }
   typedef TileIO<T, CH, K> IOK;
   typedef TileIO<T, CH, BV> IOV;
-  typedef GlaGate<GT, K> GG;
+  typedef TileIO<T, K, BV> IOH;
   const float scale = a.scale;
-  // the next chunk's g, q, do are requested before this chunk's work (chunk index clamped: every load is issued)
-  typename GG::Regs pg;
+  // the next chunk's operands are requested before this chunk's work (chunk index clamped: every load is issued)
   typename IOK::Regs pq;
   typename IOV::Regs pd;
+  float pdec[MB][4];
   auto issue = [&](int c) {
     c = max(c, 0);
-    const int tok = sq.tok0 + c * CH, len = min(CH, sq.len - c * CH);
-    GG::issue(pg, a, sq.b, tok, len, h);
-    IOK::load_nomask(pq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, len);
-    IOV::load_nomask(pd, row_ptr<T>(a.d_o, sq.b, tok, h) + v0, a.d_o.st, len);
+    const int64_t item = (int64_t)(sq.chunk0 + c) * a.H + h;
+    IOK::load_nomask(pq, (const T*)a.qe + item * CH * K, K, CH);
+    IOV::load_nomask(pd, row_ptr<T>(a.d_o, sq.b, sq.tok0 + c * CH, h) + v0, a.d_o.st, min(CH, sq.len - c * CH));
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) pdec[mi][i] = a.gcum[item * K + krow0 + acc_row(mi, i)];
   };
   if (sq.nchunks > 0) issue(sq.nchunks - 1);
   for (int c = sq.nchunks - 1; c >= 0; --c) {
     const int len = min(CH, sq.len - c * CH);
-    typename GG::Regs rg = pg;
     typename IOK::Regs rq = pq;
     typename IOV::Regs rd = pd;
-    issue(c - 1);
-    GG::template finish<LDB>(rg, len, s_b);
-    IOK::mask(rq, len);
-    IOK::store_lds_t_elem(rq, s_qT, LDC, [&](int r, int cc) { return scale * texp<T>(s_b[r * LDB + cc]); });
-    IOV::mask(rd, len);
-    IOV::store_lds_t(rd, s_doT, LDC, nullptr);
-    T* dhs = (T*)a.dhs + ((int64_t)(sq.chunk0 + c) * a.H + h) * K * V;
+    float dec[MB][4];
 #pragma unroll
     for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
-      for (int ni = 0; ni < NB; ++ni)
+      for (int i = 0; i < 4; ++i) dec[mi][i] = pdec[mi][i];
+    issue(c - 1);
+    IOK::store_lds(rq, s_q, LDK);
+    IOV::mask(rd, len);
+    IOV::store_lds(rd, s_do, LDU);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int kr = krow0 + acc_row(mi, i);
-          dhs[(int64_t)kr * V + v0 + acc_col(ni)] = ET<T>::from_f(dS[mi][ni][i]);
-          dS[mi][ni][i] *= texp<T>(s_b[63 * LDB + kr]);
-        }
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) {
+        acc_to_lds<T>(dS[mi][ni], s_h, LDU, krow0 + 16 * mi, 16 * ni);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dS[mi][ni][i] *= dec[mi][i];
+      }
     __syncthreads();
-    gemm_nt<T, MB, NB>(dS, s_qT, LDC, krow0, s_doT, LDC, 0, 0, CH);
+    IOH::lds_to_global(s_h, LDU, (T*)a.dhs + ((int64_t)(sq.chunk0 + c) * a.H + h) * K * V + v0, V, K);
+    // dS += scale (q e^{b})^T do
+    f32x4 t[MB][NB];
+    acc_zero(t);
+#pragma unroll
+    for (int kk = 0; kk < CH; kk += 32) {
+      typename ET<T>::frag af[MB], bf[NB];
+#pragma unroll
+      for (int mi = 0; mi < MB; ++mi) af[mi] = ET<T>::load_frag_t(s_q, LDK, kk, krow0 + 16 * mi);
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) bf[ni] = ET<T>::load_frag_t(s_do, LDU, kk, 16 * ni);
+#pragma unroll
+      for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) ET<T>::mma(t[mi][ni], af[mi], bf[ni]);
+    }
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) dS[mi][ni] += scale * t[mi][ni];
     __syncthreads();
   }
   if (a.dh0) {
@@ -367,16 +421,15 @@ __global__ __launch_bounds__(NTHR) void k_gla_state_bwd(const lmoe_args a) {
 // ------------------------------------------------------------------------- //
 template <typename T, typename GT, int K, int V, int BV>
 __global__ __launch_bounds__(NTHR) void k_gla_bwd_dv(const lmoe_args a) {
-  constexpr int LDB = K + 1, LDK = K + LPAD, LDC = CH + LPAD;
+  constexpr int LDK = K + LPAD, LDC = CH + LPAD;
   constexpr int NB = BV / 16;
-  // two LDS regions, each used twice (see k_gla_out_fwd):  R0: b + scan scratch, then dS'^T, then do^T;
-  // R1: k e^{b_C - b}, then A^T
-  constexpr int R0_BYTES = cmax(cmax(CH * LDB * 4 + NTHR * 4, BV * LDK * (int)sizeof(T)), BV * LDC * (int)sizeof(T));
+  // two LDS regions, each used twice (see k_gla_out_fwd):  R0: dS'^T, then do^T;  R1: k e^{b_C - b} (as stored
+  // by k_gla_intra_fwd), then A^T
+  constexpr int R0_ELEMS = cmax(BV * LDK, BV * LDC);
   constexpr int R1_ELEMS = cmax(CH * LDK, CH * LDC);
-  __shared__ __attribute__((aligned(16))) unsigned char r0[R0_BYTES];
+  __shared__ __attribute__((aligned(16))) T r0[R0_ELEMS];
   __shared__ __attribute__((aligned(16))) T r1[R1_ELEMS];
-  float* s_b = (float*)r0;
-  T* s_dhT = (T*)r0; T* s_doT = (T*)r0;
+  T* s_dhT = r0; T* s_doT = r0;
   T* s_kd = r1; T* s_PT = r1;
   const int cid = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * BV;
   const ChunkInfo ci = chunk_info(a, cid);
@@ -385,21 +438,15 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dv(const lmoe_args a) {
   typedef TileIO<T, CH, BV> IOV;
   typedef TileIO<T, K, BV> IOH;
   typedef TileIO<T, CH, CH> IOA;
-  typedef GlaGate<GT, K> GG;
-  typename GG::Regs rg;
   typename IOK::Regs rk;
   typename IOV::Regs rd;
   typename IOH::Regs rh;
   typename IOA::Regs ra;
-  GG::issue(rg, a, ci.b, ci.tok, ci.len, h);
-  IOK::load_nomask(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
+  IOK::load_nomask(rk, (const T*)a.ke + ((int64_t)cid * a.H + h) * CH * K, K, CH);
   IOH::load_nomask(rh, (const T*)a.dhs + ((int64_t)cid * a.H + h) * K * V + v0, V, K);
   IOA::load_nomask(ra, (const T*)a.amat + ((int64_t)cid * a.H + h) * CH * CH, CH, CH);
   IOV::load_nomask(rd, row_ptr<T>(a.d_o, ci.b, ci.tok, h) + v0, a.d_o.st, ci.len);
-  GG::template finish<LDB>(rg, ci.len, s_b, s_b + CH * LDB);                             // barriers inside
-  IOK::mask(rk, ci.len);
-  IOK::store_lds_elem(rk, s_kd, LDK, [&](int r, int cc) { return texp<T>(s_b[63 * LDB + cc] - s_b[r * LDB + cc]); });
-  __syncthreads();                                                                       // b is dead
+  IOK::store_lds(rk, s_kd, LDK);
   IOH::store_lds_t(rh, s_dhT, LDK, nullptr);
   __syncthreads();
   f32x4 dv[1][NB], dv2[1][NB];

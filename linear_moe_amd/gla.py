@@ -50,9 +50,14 @@ class GLACall:
         ht = torch.empty(plan.N, H, K, V, dtype=torch.float32, device=dev) if output_final_state else None
         hs = torch.empty(max(plan.NT, 1), H, K, V, dtype=dt, device=dev)
         amat = torch.empty(max(plan.NT, 1), H, 64, 64, dtype=dt, device=dev)
+        # gated operands of the state passes (q e^b, k e^{b_C - b}, e^{b_C}), formed once per chunk
+        qe = torch.empty(max(plan.NT, 1), H, 64, K, dtype=dt, device=dev)
+        ke = torch.empty_like(qe)
+        gdec = torch.empty(max(plan.NT, 1), H, K, dtype=torch.float32, device=dev)
         a.o, a.ht, a.hs, a.amat = _desc(o, head_first), ptr(ht), hs.data_ptr(), amat.data_ptr()
+        a.qe, a.ke, a.gcum = qe.data_ptr(), ke.data_ptr(), gdec.data_ptr()
         _lib.check(lib.lmoe_chunk_gla_fwd(C.byref(a), stream_ptr()), "chunk_gla forward")
-        self.saved = (q, k, v, g, h0, hs, amat)
+        self.saved = (q, k, v, g, h0, hs, amat, qe, ke, gdec)
         self.fwd_args, self.fwd_keep = a, ((o, ht) if self.keep else None)
         self.plan, self.dims, self.head_first, self.scale = plan, dims, head_first, scale
         self.has_h0 = initial_state is not None
@@ -60,12 +65,13 @@ class GLACall:
 
     def backward(self, do, dht):
         lib = _lib.load()
-        q, k, v, g, h0, hs, amat = self.saved
+        q, k, v, g, h0, hs, amat, qe, ke, gdec = self.saved
         plan, dims, head_first = self.plan, self.dims, self.head_first
         do = _aligned(do)
         a = base_args(q, k, v, head_first, self.scale, plan, dims)
         self._gate(a, g, head_first)
         a.h0, a.hs, a.amat = ptr(h0), hs.data_ptr(), amat.data_ptr()
+        a.qe, a.ke, a.gcum = qe.data_ptr(), ke.data_ptr(), gdec.data_ptr()
         a.d_o = _desc(do, head_first)
         dht = None if dht is None else dht.float().contiguous()
         a.dht = ptr(dht)
