@@ -123,6 +123,13 @@ template <> struct ET<float> {
 template <typename T> __device__ __forceinline__ float texp(float x) {
   if constexpr (sizeof(T) == 4) return expf(x); else return __expf(x);
 }
+// The same with the argument scaled once up front: e^x = texp_scaled(x * TEXP_PRESCALE<T>); on the bf16 path the
+// scale is log2(e) and the call is the bare hardware exp2, which saves a multiply per exponential in loops that
+// form many exponentials of differences of the same few values.
+template <typename T> constexpr float TEXP_PRESCALE = sizeof(T) == 4 ? 1.0f : 1.4426950408889634f;
+template <typename T> __device__ __forceinline__ float texp_scaled(float x) {
+  if constexpr (sizeof(T) == 4) return expf(x); else return __builtin_amdgcn_exp2f(x);
+}
 
 // ------------------------------------------------------------------------- //
 // gemm_nt: acc[mi][ni] += A[arow0 + 16 mi + r][k] * B[brow0 + 16 ni + c][k], k in [k0, k1)

@@ -37,7 +37,8 @@ struct GlaGate {
   }
   // tot: NTHR floats of LDS for the segment totals
   template <int LDB>
-  static __device__ __forceinline__ void finish(Regs& rg, int len, float* s_b, float* s_tot) {
+  // mult: factor applied to the stored cumsum (1, or TEXP_PRESCALE<T> for kernels that only form exponentials of it)
+  static __device__ __forceinline__ void finish(Regs& rg, int len, float* s_b, float* s_tot, float mult = 1.0f) {
     constexpr int NSEG = NTHR / K, SEG = CH / NSEG;
     static_assert(NTHR % K == 0 && CH % NSEG == 0, "one channel and one token segment per thread");
     IOG::mask(rg, len);
@@ -55,7 +56,7 @@ struct GlaGate {
 #pragma unroll
     for (int q = 0; q < NSEG - 1; ++q) off += q < sg ? s_tot[q * K + c] : 0.f;
 #pragma unroll
-    for (int r = 0; r < SEG; ++r) s_b[(sg * SEG + r) * LDB + c] = v[r] + off;
+    for (int r = 0; r < SEG; ++r) s_b[(sg * SEG + r) * LDB + c] = (v[r] + off) * mult;
     __syncthreads();
   }
   template <int LDB>
@@ -105,7 +106,7 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
     typename GlaGate<GT, K>::Regs rg;
     GlaGate<GT, K>::issue(rg, a, ci.b, ci.tok, ci.len, h);
     static_assert(16 * LDK * sizeof(T) >= NTHR * 4, "the scan's scratch fits the q~ tile");
-    GlaGate<GT, K>::template finish<LDB>(rg, ci.len, s_b, (float*)s_qt);    // barriers inside
+    GlaGate<GT, K>::template finish<LDB>(rg, ci.len, s_b, (float*)s_qt, TEXP_PRESCALE<T>);    // barriers inside; b in exp2 units
   }
   // ---- gated operands for the other kernels: q e^{b}, k e^{b_C - b}, e^{b_C} ----
   {
@@ -120,13 +121,13 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
         const float b = s_b[r * LDB + c0 + j], bC = s_b[63 * LDB + c0 + j];
-        qo[j] = ET<T>::from_f(ET<T>::to_f(qv[j]) * texp<T>(b));
-        ko[j] = ET<T>::from_f(ET<T>::to_f(kv[j]) * texp<T>(bC - b));
+        qo[j] = ET<T>::from_f(ET<T>::to_f(qv[j]) * texp_scaled<T>(b));
+        ko[j] = ET<T>::from_f(ET<T>::to_f(kv[j]) * texp_scaled<T>(bC - b));
       }
       *(vec*)(qe + r * K + c0) = qo;
       *(vec*)(ke + r * K + c0) = ko;
     }
-    if (threadIdx.x < K) a.gcum[((int64_t)cid * a.H + h) * K + threadIdx.x] = texp<T>(s_b[63 * LDB + threadIdx.x]);
+    if (threadIdx.x < K) a.gcum[((int64_t)cid * a.H + h) * K + threadIdx.x] = texp_scaled<T>(s_b[63 * LDB + threadIdx.x]);
   }
   // ---- diagonal blocks: wave w owns block (w, w); lane -> row i, columns j0 .. j0 + 3 ----
   {
@@ -143,7 +144,7 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
         const f32x4 bj = *(const f32x4*)(s_b + j * LDB + k4);
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          acc[jj] += qi[e] * ET<T>::to_f(s_k[j * LDK + k4 + e]) * texp<T>(fminf(bi[e] - bj[e], 0.f));
+          acc[jj] += qi[e] * ET<T>::to_f(s_k[j * LDK + k4 + e]) * texp_scaled<T>(fminf(bi[e] - bj[e], 0.f));
       }
     }
 #pragma unroll
@@ -154,11 +155,11 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
     const float* bs = s_b + (16 * I - 1) * LDB;                   // b* of this block row
     for (int idx = threadIdx.x; idx < 16 * K; idx += NTHR) {
       const int r = idx / K, c = idx % K, i = 16 * I + r;
-      s_qt[r * LDK + c] = ET<T>::from_f(ET<T>::to_f(s_q[i * LDK + c]) * texp<T>(s_b[i * LDB + c] - bs[c]));
+      s_qt[r * LDK + c] = ET<T>::from_f(ET<T>::to_f(s_q[i * LDK + c]) * texp_scaled<T>(s_b[i * LDB + c] - bs[c]));
     }
     for (int idx = threadIdx.x; idx < 16 * I * K; idx += NTHR) {
       const int j = idx / K, c = idx % K;
-      s_kt[j * LDK + c] = ET<T>::from_f(ET<T>::to_f(s_k[j * LDK + c]) * texp<T>(bs[c] - s_b[j * LDB + c]));
+      s_kt[j * LDK + c] = ET<T>::from_f(ET<T>::to_f(s_k[j * LDK + c]) * texp_scaled<T>(bs[c] - s_b[j * LDB + c]));
     }
     __syncthreads();
     if (wv < I) {
@@ -634,7 +635,7 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           sqv[n4][i] = skv[n4][i] = 0.f;
-          brv[n4][i] = sB[(16 * wv + 4 * (l >> 4) + i) * LDB + 16 * (nh + n4) + (l & 15)];
+          brv[n4][i] = sB[(16 * wv + 4 * (l >> 4) + i) * LDB + 16 * (nh + n4) + (l & 15)] * TEXP_PRESCALE<T>;
         }
       for (int jj = 0; jj < 16; ++jj) {
         const int j = 16 * wv + jj;
@@ -648,10 +649,10 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
 #pragma unroll
         for (int n4 = 0; n4 < 4; ++n4) {
           const int cc = 16 * (nh + n4) + (l & 15);
-          const float kj = Km(j, cc), qj = Qm(j, cc), bj = sB[j * LDB + cc];
+          const float kj = Km(j, cc), qj = Qm(j, cc), bj = sB[j * LDB + cc] * TEXP_PRESCALE<T>;
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const float e = texp<T>(-fabsf(brv[n4][i] - bj));
+            const float e = texp_scaled<T>(-fabsf(brv[n4][i] - bj));
             sqv[n4][i] += pq[i] * kj * e;
             skv[n4][i] += pk[i] * qj * e;
           }
