@@ -18,11 +18,11 @@ static void launch_gla_t(const lmoe_args& a, int stage, hipStream_t st) {
     case ST_GLA_INTRA_FWD:
       hipLaunchKernelGGL((k_gla_intra_fwd<T, GT, K>), dim3(a.NT, a.H), block, 0, st, a); break;
     case ST_STATE_FWD:
-      hipLaunchKernelGGL((k_gla_state_fwd<T, GT, K, V, Tl::BVS>), dim3(V / Tl::BVS, a.H, a.N), block, 0, st, a); break;
+      hipLaunchKernelGGL((k_gla_state_fwd<T, GT, K, V, Tl::BVS>), dim3((a.N * a.H + 7) / 8 * 8 * (V / Tl::BVS)), block, 0, st, a); break;
     case ST_OUT_FWD:
       hipLaunchKernelGGL((k_gla_out_fwd<T, GT, K, V, Tl::BVO>), dim3(a.NT, a.H, V / Tl::BVO), block, 0, st, a); break;
     case ST_STATE_BWD:
-      hipLaunchKernelGGL((k_gla_state_bwd<T, GT, K, V, Tl::BVS>), dim3(V / Tl::BVS, a.H, a.N), block, 0, st, a); break;
+      hipLaunchKernelGGL((k_gla_state_bwd<T, GT, K, V, Tl::BVS>), dim3((a.N * a.H + 7) / 8 * 8 * (V / Tl::BVS)), block, 0, st, a); break;
     case ST_DV:
       hipLaunchKernelGGL((k_gla_bwd_dv<T, GT, K, V, Tl::BVO>), dim3(a.NT, a.H, V / Tl::BVO), block, 0, st, a); break;
     case ST_DQK:

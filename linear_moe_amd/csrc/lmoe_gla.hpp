@@ -174,7 +174,7 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
 }
 
 // ------------------------------------------------------------------------- //
-// forward state pass, grid = (V / BV, H, N)
+// forward state pass, 1-D grid (XCD-aware, see the kernel)
 // ------------------------------------------------------------------------- //
 template <typename T, typename GT, int K, int V, int BV>
 __global__ __launch_bounds__(NTHR) void k_gla_state_fwd(const lmoe_args a) {
@@ -183,7 +183,13 @@ __global__ __launch_bounds__(NTHR) void k_gla_state_fwd(const lmoe_args a) {
   __shared__ __attribute__((aligned(16))) T s_k[CH * LDK];     // k e^{b_C - b}     [64][K]
   __shared__ __attribute__((aligned(16))) T s_v[CH * LDU];     // v                 [64][BV]
   __shared__ __attribute__((aligned(16))) T s_h[K * LDU];      // S on its way out  [K][BV]
-  const int v0 = blockIdx.x * BV, h = blockIdx.y, n = blockIdx.z;
+  // 1-D grid of ceil(N H / 8) * 8 * (V / BV) work-groups; the V-slices of one (sequence, head) get ids that are
+  // congruent mod 8, i.e. run on the same XCD and share its gated k (q) rows through that XCD's L2
+  constexpr int NVS = V / BV;
+  const int xcd = blockIdx.x & 7, jj = blockIdx.x >> 3;
+  const int pair = (jj / NVS) * 8 + xcd;
+  if (pair >= a.N * a.H) return;
+  const int v0 = (jj % NVS) * BV, h = pair % a.H, n = pair / a.H;
   const SeqInfo sq = seq_info(a, n);
   const int wv = wave_id();
   const int krow0 = wv * (K / 4);
@@ -201,58 +207,61 @@ __global__ __launch_bounds__(NTHR) void k_gla_state_fwd(const lmoe_args a) {
   typedef TileIO<T, CH, K> IOK;
   typedef TileIO<T, CH, BV> IOV;
   typedef TileIO<T, K, BV> IOH;
-  // the next chunk's operands are requested before this chunk's work (chunk index clamped: every load is issued)
-  typename IOK::Regs pk;
-  typename IOV::Regs pv;
-  float pdec[MB][4];
-  auto issue = [&](int c) {
+  // The operands of the next PF chunks are kept in flight in PF register sets (chunk index clamped: every load
+  // is issued; the surplus ones at the end are never used): one chunk of this pass is shorter than a trip to HBM.
+  constexpr int PF = 3;
+  struct Pre { typename IOK::Regs rk; typename IOV::Regs rv; float dec[MB][4]; };
+  Pre pre[PF];
+  auto issue = [&](Pre& P, int c) {
     c = min(c, sq.nchunks - 1);
     const int64_t item = (int64_t)(sq.chunk0 + c) * a.H + h;
-    IOK::load_nomask(pk, (const T*)a.ke + item * CH * K, K, CH);
-    IOV::load_nomask(pv, row_ptr<T>(a.v, sq.b, sq.tok0 + c * CH, h) + v0, a.v.st, min(CH, sq.len - c * CH));
+    IOK::load_nomask(P.rk, (const T*)a.ke + item * CH * K, K, CH);
+    IOV::load_nomask(P.rv, row_ptr<T>(a.v, sq.b, sq.tok0 + c * CH, h) + v0, a.v.st, min(CH, sq.len - c * CH));
 #pragma unroll
     for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) pdec[mi][i] = a.gcum[item * K + krow0 + acc_row(mi, i)];
+      for (int i = 0; i < 4; ++i) P.dec[mi][i] = a.gcum[item * K + krow0 + acc_row(mi, i)];
   };
-  if (sq.nchunks > 0) issue(0);
-  for (int c = 0; c < sq.nchunks; ++c) {
-    const int len = min(CH, sq.len - c * CH);
-    typename IOK::Regs rk = pk;
-    typename IOV::Regs rv = pv;
-    float dec[MB][4];
+  if (sq.nchunks > 0) {
 #pragma unroll
-    for (int mi = 0; mi < MB; ++mi)
+    for (int j = 0; j < PF; ++j) issue(pre[j], j);
+  }
+  for (int c0 = 0; c0 < sq.nchunks; c0 += PF) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) dec[mi][i] = pdec[mi][i];
-    issue(c + 1);
-    IOK::store_lds(rk, s_k, LDK);
-    IOV::mask(rv, len);
-    IOV::store_lds(rv, s_v, LDU);
-#pragma unroll
-    for (int mi = 0; mi < MB; ++mi)
-#pragma unroll
-      for (int ni = 0; ni < NB; ++ni) {
-        acc_to_lds<T>(S[mi][ni], s_h, LDU, krow0 + 16 * mi, 16 * ni);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) S[mi][ni][i] *= dec[mi][i];
-      }
-    __syncthreads();
-    IOH::lds_to_global(s_h, LDU, (T*)a.hs + ((int64_t)(sq.chunk0 + c) * a.H + h) * K * V + v0, V, K);
-    // S += (k e^{b_C - b})^T v
-#pragma unroll
-    for (int kk = 0; kk < CH; kk += 32) {
-      typename ET<T>::frag af[MB], bf[NB];
-#pragma unroll
-      for (int mi = 0; mi < MB; ++mi) af[mi] = ET<T>::load_frag_t(s_k, LDK, kk, krow0 + 16 * mi);
-#pragma unroll
-      for (int ni = 0; ni < NB; ++ni) bf[ni] = ET<T>::load_frag_t(s_v, LDU, kk, 16 * ni);
+    for (int j = 0; j < PF; ++j) {
+      const int c = c0 + j;
+      if (c >= sq.nchunks) break;
+      const int len = min(CH, sq.len - c * CH);
+      Pre& P = pre[j];
+      IOK::store_lds(P.rk, s_k, LDK);
+      IOV::mask(P.rv, len);
+      IOV::store_lds(P.rv, s_v, LDU);
 #pragma unroll
       for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < NB; ++ni) ET<T>::mma(S[mi][ni], af[mi], bf[ni]);
+        for (int ni = 0; ni < NB; ++ni) {
+          acc_to_lds<T>(S[mi][ni], s_h, LDU, krow0 + 16 * mi, 16 * ni);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) S[mi][ni][i] *= P.dec[mi][i];
+        }
+      issue(P, c + PF);
+      lds_barrier();      // LDS-only: the loads stay in flight
+      IOH::lds_to_global(s_h, LDU, (T*)a.hs + ((int64_t)(sq.chunk0 + c) * a.H + h) * K * V + v0, V, K);
+      // S += (k e^{b_C - b})^T v
+#pragma unroll
+      for (int kk = 0; kk < CH; kk += 32) {
+        typename ET<T>::frag af[MB], bf[NB];
+#pragma unroll
+        for (int mi = 0; mi < MB; ++mi) af[mi] = ET<T>::load_frag_t(s_k, LDK, kk, krow0 + 16 * mi);
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) bf[ni] = ET<T>::load_frag_t(s_v, LDU, kk, 16 * ni);
+#pragma unroll
+        for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+          for (int ni = 0; ni < NB; ++ni) ET<T>::mma(S[mi][ni], af[mi], bf[ni]);
+      }
+      lds_barrier();
     }
-    __syncthreads();
   }
   if (a.ht) {
     float* ht = a.ht + ((int64_t)n * a.H + h) * K * V;
@@ -298,15 +307,15 @@ __global__ __launch_bounds__(NTHR) void k_gla_out_fwd(const lmoe_args a) {
   IOV::load_nomask(rv, row_ptr<T>(a.v, ci.b, ci.tok, h) + v0, a.v.st, ci.len);
   IOK::store_lds(rq, s_q, LDK);
   IOH::store_lds_t(rh, s_hT, LDK, nullptr);
-  __syncthreads();
+  lds_barrier();
   f32x4 o[1][NB];
   acc_zero(o);
   gemm_nt<T, 1, NB>(o, s_q, LDK, 16 * wv, s_hT, LDK, 0, 0, K);
-  __syncthreads();                                                                       // q e^{b}, S^T are dead
+  lds_barrier();                                                                       // q e^{b}, S^T are dead
   IOA::store_lds(ra, s_P, LDC);
   IOV::mask(rv, ci.len);
   IOV::store_lds_t(rv, s_vT, LDC, nullptr);
-  __syncthreads();
+  lds_barrier();
   gemm_nt<T, 1, NB>(o, s_P, LDC, 16 * wv, s_vT, LDC, 0, 0, CH);
   T* od = row_ptr<T>(a.o, ci.b, ci.tok, h) + v0;
 #pragma unroll
@@ -319,7 +328,7 @@ __global__ __launch_bounds__(NTHR) void k_gla_out_fwd(const lmoe_args a) {
 }
 
 // ------------------------------------------------------------------------- //
-// reverse state pass, grid = (V / BV, H, N)
+// reverse state pass, 1-D grid (XCD-aware, see k_gla_state_fwd)
 // ------------------------------------------------------------------------- //
 template <typename T, typename GT, int K, int V, int BV>
 __global__ __launch_bounds__(NTHR) void k_gla_state_bwd(const lmoe_args a) {
@@ -328,7 +337,13 @@ __global__ __launch_bounds__(NTHR) void k_gla_state_bwd(const lmoe_args a) {
   __shared__ __attribute__((aligned(16))) T s_q[CH * LDK];     // q e^{b}             [64][K]
   __shared__ __attribute__((aligned(16))) T s_do[CH * LDU];    // do                  [64][BV]
   __shared__ __attribute__((aligned(16))) T s_h[K * LDU];      // dS' on its way out  [K][BV]
-  const int v0 = blockIdx.x * BV, h = blockIdx.y, n = blockIdx.z;
+  // 1-D grid of ceil(N H / 8) * 8 * (V / BV) work-groups; the V-slices of one (sequence, head) get ids that are
+  // congruent mod 8, i.e. run on the same XCD and share its gated k (q) rows through that XCD's L2
+  constexpr int NVS = V / BV;
+  const int xcd = blockIdx.x & 7, jj = blockIdx.x >> 3;
+  const int pair = (jj / NVS) * 8 + xcd;
+  if (pair >= a.N * a.H) return;
+  const int v0 = (jj % NVS) * BV, h = pair % a.H, n = pair / a.H;
   const SeqInfo sq = seq_info(a, n);
   const int wv = wave_id();
   const int krow0 = wv * (K / 4);
@@ -347,64 +362,66 @@ __global__ __launch_bounds__(NTHR) void k_gla_state_bwd(const lmoe_args a) {
   typedef TileIO<T, CH, BV> IOV;
   typedef TileIO<T, K, BV> IOH;
   const float scale = a.scale;
-  // the next chunk's operands are requested before this chunk's work (chunk index clamped: every load is issued)
-  typename IOK::Regs pq;
-  typename IOV::Regs pd;
-  float pdec[MB][4];
-  auto issue = [&](int c) {
+  // the operands of the next PF chunks are kept in flight in PF register sets (see k_gla_state_fwd)
+  constexpr int PF = 3;
+  struct Pre { typename IOK::Regs rq; typename IOV::Regs rd; float dec[MB][4]; };
+  Pre pre[PF];
+  auto issue = [&](Pre& P, int c) {
     c = max(c, 0);
     const int64_t item = (int64_t)(sq.chunk0 + c) * a.H + h;
-    IOK::load_nomask(pq, (const T*)a.qe + item * CH * K, K, CH);
-    IOV::load_nomask(pd, row_ptr<T>(a.d_o, sq.b, sq.tok0 + c * CH, h) + v0, a.d_o.st, min(CH, sq.len - c * CH));
+    IOK::load_nomask(P.rq, (const T*)a.qe + item * CH * K, K, CH);
+    IOV::load_nomask(P.rd, row_ptr<T>(a.d_o, sq.b, sq.tok0 + c * CH, h) + v0, a.d_o.st, min(CH, sq.len - c * CH));
 #pragma unroll
     for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) pdec[mi][i] = a.gcum[item * K + krow0 + acc_row(mi, i)];
+      for (int i = 0; i < 4; ++i) P.dec[mi][i] = a.gcum[item * K + krow0 + acc_row(mi, i)];
   };
-  if (sq.nchunks > 0) issue(sq.nchunks - 1);
-  for (int c = sq.nchunks - 1; c >= 0; --c) {
-    const int len = min(CH, sq.len - c * CH);
-    typename IOK::Regs rq = pq;
-    typename IOV::Regs rd = pd;
-    float dec[MB][4];
+  if (sq.nchunks > 0) {
 #pragma unroll
-    for (int mi = 0; mi < MB; ++mi)
+    for (int j = 0; j < PF; ++j) issue(pre[j], sq.nchunks - 1 - j);
+  }
+  for (int c0 = sq.nchunks - 1; c0 >= 0; c0 -= PF) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) dec[mi][i] = pdec[mi][i];
-    issue(c - 1);
-    IOK::store_lds(rq, s_q, LDK);
-    IOV::mask(rd, len);
-    IOV::store_lds(rd, s_do, LDU);
-#pragma unroll
-    for (int mi = 0; mi < MB; ++mi)
-#pragma unroll
-      for (int ni = 0; ni < NB; ++ni) {
-        acc_to_lds<T>(dS[mi][ni], s_h, LDU, krow0 + 16 * mi, 16 * ni);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) dS[mi][ni][i] *= dec[mi][i];
-      }
-    __syncthreads();
-    IOH::lds_to_global(s_h, LDU, (T*)a.dhs + ((int64_t)(sq.chunk0 + c) * a.H + h) * K * V + v0, V, K);
-    // dS += scale (q e^{b})^T do
-    f32x4 t[MB][NB];
-    acc_zero(t);
-#pragma unroll
-    for (int kk = 0; kk < CH; kk += 32) {
-      typename ET<T>::frag af[MB], bf[NB];
-#pragma unroll
-      for (int mi = 0; mi < MB; ++mi) af[mi] = ET<T>::load_frag_t(s_q, LDK, kk, krow0 + 16 * mi);
-#pragma unroll
-      for (int ni = 0; ni < NB; ++ni) bf[ni] = ET<T>::load_frag_t(s_do, LDU, kk, 16 * ni);
+    for (int j = 0; j < PF; ++j) {
+      const int c = c0 - j;
+      if (c < 0) break;
+      const int len = min(CH, sq.len - c * CH);
+      Pre& P = pre[j];
+      IOK::store_lds(P.rq, s_q, LDK);
+      IOV::mask(P.rd, len);
+      IOV::store_lds(P.rd, s_do, LDU);
 #pragma unroll
       for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < NB; ++ni) ET<T>::mma(t[mi][ni], af[mi], bf[ni]);
+        for (int ni = 0; ni < NB; ++ni) {
+          acc_to_lds<T>(dS[mi][ni], s_h, LDU, krow0 + 16 * mi, 16 * ni);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) dS[mi][ni][i] *= P.dec[mi][i];
+        }
+      issue(P, c - PF);
+      lds_barrier();      // LDS-only: the loads stay in flight
+      IOH::lds_to_global(s_h, LDU, (T*)a.dhs + ((int64_t)(sq.chunk0 + c) * a.H + h) * K * V + v0, V, K);
+      // dS += scale (q e^{b})^T do
+      f32x4 t[MB][NB];
+      acc_zero(t);
+#pragma unroll
+      for (int kk = 0; kk < CH; kk += 32) {
+        typename ET<T>::frag af[MB], bf[NB];
+#pragma unroll
+        for (int mi = 0; mi < MB; ++mi) af[mi] = ET<T>::load_frag_t(s_q, LDK, kk, krow0 + 16 * mi);
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) bf[ni] = ET<T>::load_frag_t(s_do, LDU, kk, 16 * ni);
+#pragma unroll
+        for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+          for (int ni = 0; ni < NB; ++ni) ET<T>::mma(t[mi][ni], af[mi], bf[ni]);
+      }
+#pragma unroll
+      for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) dS[mi][ni] += scale * t[mi][ni];
+      lds_barrier();
     }
-#pragma unroll
-    for (int mi = 0; mi < MB; ++mi)
-#pragma unroll
-      for (int ni = 0; ni < NB; ++ni) dS[mi][ni] += scale * t[mi][ni];
-    __syncthreads();
   }
   if (a.dh0) {
     float* p = a.dh0 + ((int64_t)n * a.H + h) * K * V;
@@ -449,15 +466,15 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dv(const lmoe_args a) {
   IOV::load_nomask(rd, row_ptr<T>(a.d_o, ci.b, ci.tok, h) + v0, a.d_o.st, ci.len);
   IOK::store_lds(rk, s_kd, LDK);
   IOH::store_lds_t(rh, s_dhT, LDK, nullptr);
-  __syncthreads();
+  lds_barrier();
   f32x4 dv[1][NB], dv2[1][NB];
   acc_zero(dv); acc_zero(dv2);
   gemm_nt<T, 1, NB>(dv2, s_kd, LDK, 16 * wv, s_dhT, LDK, 0, 0, K);
-  __syncthreads();                                                                       // k e^{..}, dS'^T are dead
+  lds_barrier();                                                                       // k e^{..}, dS'^T are dead
   IOA::store_lds_t(ra, s_PT, LDC, nullptr);
   IOV::mask(rd, ci.len);
   IOV::store_lds_t(rd, s_doT, LDC, nullptr);
-  __syncthreads();
+  lds_barrier();
   gemm_nt<T, 1, NB>(dv, s_PT, LDC, 16 * wv, s_doT, LDC, 0, 0, CH);
   T* dd = row_ptr<T>(a.dv, ci.b, ci.tok, h) + v0;
 #pragma unroll
@@ -546,11 +563,11 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
     IOV::store_lds(x.rv, smT + A_V, LDV);
     IOH::store_lds(x.rh, smT + A_H, LDV);
     IOH::store_lds(x.rdh, smT + A_DH, LDV);
-    __syncthreads();
+    lds_barrier();      // LDS-only barriers: the loads requested above stay in flight
     gemm_nt<T, 1, 4>(dP, smT + A_DO, LDV, 16 * wv, smT + A_V, LDV, 0, 0, BVH);
     gemm_nt<T, 1, NBK>(dqi, smT + A_DO, LDV, 16 * wv, smT + A_H, LDV, 0, 0, BVH);
     gemm_nt<T, 1, NBK>(dkd, smT + A_V, LDV, 16 * wv, smT + A_DH, LDV, 0, 0, BVH);
-    __syncthreads();
+    lds_barrier();
   }
   // per state row k: sum_v S_kv dS'_kv  (the IOH::VPR adjacent threads of a pass share a row)
 #pragma unroll
