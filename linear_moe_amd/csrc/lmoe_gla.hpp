@@ -23,6 +23,11 @@
 namespace lmoe {
 
 constexpr int cmax(int a, int b) { return a > b ? a : b; }
+// largest decay exponent over one 16-token sub-chunk up to which chunk_gla factors its diagonal blocks through a
+// reference gate (e^60 ~ 1e26 leaves fp32 / bf16 range to spare for the operand it multiplies)
+constexpr float GLA_SAFE_EXP = 60.0f;
+// first row of the k~ copy of block row I inside the stacked tile: 0, 16, 48, 96
+constexpr int KT_ROW0(int I) { return 8 * I * (I + 1); }
 
 // g tile of the chunk -> fp32 LDS tile s_b[64][LDB] holding the inclusive cumsum over tokens.
 // The scan: a thread takes one channel over a segment of 64 K / 256 tokens (its values in registers, so the
@@ -86,8 +91,11 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
   __shared__ __attribute__((aligned(16))) float s_b[CH * LDB];
   __shared__ __attribute__((aligned(16))) T s_q[CH * LDK];        // q, k as loaded
   __shared__ __attribute__((aligned(16))) T s_k[CH * LDK];
-  __shared__ __attribute__((aligned(16))) T s_qt[16 * LDK];       // scaled operands of one block row
-  __shared__ __attribute__((aligned(16))) T s_kt[48 * LDK];
+  // all block rows at once where LDS has room for the stacked k~ tile (everything but fp32 with K = 128), else
+  // one block row at a time with the diagonal blocks always on the vector ALU
+  constexpr bool ONE_PASS = (CH * LDB * 4 + (3 * CH * LDK + 160 * LDK + CH * LDC) * (int)sizeof(T)) <= 150 * 1024;
+  __shared__ __attribute__((aligned(16))) T s_qt[(ONE_PASS ? CH : 16) * LDK];   // q~: rows scaled to the reference of their block row
+  __shared__ __attribute__((aligned(16))) T s_kt[(ONE_PASS ? 160 : 48) * LDK];  // k~ of block rows 0..3: 16 + 32 + 48 + 64 rows
   __shared__ __attribute__((aligned(16))) T s_A[CH * LDC];
   const int cid = blockIdx.x, h = blockIdx.y;
   const ChunkInfo ci = chunk_info(a, cid);
@@ -105,7 +113,6 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
   {
     typename GlaGate<GT, K>::Regs rg;
     GlaGate<GT, K>::issue(rg, a, ci.b, ci.tok, ci.len, h);
-    static_assert(16 * LDK * sizeof(T) >= NTHR * 4, "the scan's scratch fits the q~ tile");
     GlaGate<GT, K>::template finish<LDB>(rg, ci.len, s_b, (float*)s_qt, TEXP_PRESCALE<T>);    // barriers inside; b in exp2 units
   }
   // ---- gated operands for the other kernels: q e^{b}, k e^{b_C - b}, e^{b_C} ----
@@ -129,8 +136,33 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
     }
     if (threadIdx.x < K) a.gcum[((int64_t)cid * a.H + h) * K + threadIdx.x] = texp_scaled<T>(s_b[63 * LDB + threadIdx.x]);
   }
-  // ---- diagonal blocks: wave w owns block (w, w); lane -> row i, columns j0 .. j0 + 3 ----
-  {
+  // ---- is the decay inside every 16-token sub-chunk small enough to factor the diagonal blocks too? ----
+  // Block row I (tokens 16 I ..) takes the cumulative gate just before it as its reference, b* = b_{16 I - 1}
+  // (0 for I = 0):  A_ij = sum_k (q_ik e^{b_ik - b*_k}) (k_jk e^{b*_k - b_jk}).  For j before the block row both
+  // exponents are <= 0.  For j inside it the second one is the decay over at most 16 tokens, >= 0: taken only
+  // if it stays below GLA_SAFE_EXP for every channel, otherwise that diagonal block forms its exponent per pair
+  // on the vector ALU (always safe; what fla's diagonal sub-blocks do).
+  int unsafe = 0;
+  if (threadIdx.x < K) {
+#pragma unroll
+    for (int I = 0; I < 4; ++I) {
+      const float ref = I == 0 ? 0.f : s_b[(16 * I - 1) * LDB + threadIdx.x];
+      if (!(ref - s_b[(16 * I + 15) * LDB + threadIdx.x] <= GLA_SAFE_EXP * TEXP_PRESCALE<T>)) unsafe |= 1 << I;
+    }
+  }
+  if constexpr (ONE_PASS) {
+    // bitwise OR over the work-group (the barrier-with-predicate intrinsics only tell zero from non-zero)
+    __shared__ int s_unsafe;
+    if (threadIdx.x == 0) s_unsafe = 0;
+    __syncthreads();
+    if (unsafe) atomicOr(&s_unsafe, unsafe);
+    __syncthreads();
+    unsafe = s_unsafe;
+  } else {
+    unsafe = 15;
+  }
+  // ---- diagonal blocks that cannot be factored: wave w owns block (w, w); lane -> row i, columns j0 .. j0 + 3 ----
+  if ((unsafe >> wv) & 1) {
     const int i = 16 * wv + (l & 15), j0 = 16 * wv + 4 * (l >> 4);
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     for (int k4 = 0; k4 < K; k4 += 4) {
@@ -150,25 +182,59 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) s_A[i * LDC + j0 + jj] = ET<T>::from_f(i >= j0 + jj ? acc[jj] : 0.f);
   }
-  // ---- blocks below the diagonal, one block row at a time ----
-  for (int I = 1; I < 4; ++I) {
-    const float* bs = s_b + (16 * I - 1) * LDB;                   // b* of this block row
-    for (int idx = threadIdx.x; idx < 16 * K; idx += NTHR) {
-      const int r = idx / K, c = idx % K, i = 16 * I + r;
-      s_qt[r * LDK + c] = ET<T>::from_f(ET<T>::to_f(s_q[i * LDK + c]) * texp_scaled<T>(s_b[i * LDB + c] - bs[c]));
-    }
-    for (int idx = threadIdx.x; idx < 16 * I * K; idx += NTHR) {
+  if constexpr (ONE_PASS) {
+  // ---- scaled operands of all block rows at once: q~ (64 rows), k~ of block row I = rows 0 .. 16 I + 15 ----
+  for (int idx = threadIdx.x; idx < CH * K; idx += NTHR) {
+    const int i = idx / K, c = idx % K, I = i >> 4;
+    const float ref = I == 0 ? 0.f : s_b[(16 * I - 1) * LDB + c];
+    s_qt[i * LDK + c] = ET<T>::from_f(ET<T>::to_f(s_q[i * LDK + c]) * texp_scaled<T>(s_b[i * LDB + c] - ref));
+  }
+#pragma unroll
+  for (int I = 0; I < 4; ++I) {
+    T* kt = s_kt + KT_ROW0(I) * LDK;
+    for (int idx = threadIdx.x; idx < 16 * (I + 1) * K; idx += NTHR) {
       const int j = idx / K, c = idx % K;
-      s_kt[j * LDK + c] = ET<T>::from_f(ET<T>::to_f(s_k[j * LDK + c]) * texp_scaled<T>(bs[c] - s_b[j * LDB + c]));
+      const float ref = I == 0 ? 0.f : s_b[(16 * I - 1) * LDB + c];
+      kt[j * LDK + c] = ET<T>::from_f(ET<T>::to_f(s_k[j * LDK + c]) * texp_scaled<T>(ref - s_b[j * LDB + c]));
     }
-    __syncthreads();
-    if (wv < I) {
-      f32x4 t[1][1];
-      acc_zero(t);
-      gemm<T, 1, 1, false, false>(t, s_qt, LDK, 0, s_kt, LDK, 16 * wv, 0, K);
-      acc_to_lds<T>(t[0][0], s_A, LDC, 16 * I, 16 * wv);
+  }
+  __syncthreads();
+  // wave w: the blocks (I, w), I = w .. 3; the diagonal one masked to i >= j
+#pragma unroll
+  for (int I = 0; I < 4; ++I) {
+    if (wv > I || (wv == I && ((unsafe >> I) & 1))) continue;
+    f32x4 t[1][1];
+    acc_zero(t);
+    gemm<T, 1, 1, false, false>(t, s_qt, LDK, 16 * I, s_kt + KT_ROW0(I) * LDK, LDK, 16 * wv, 0, K);
+    if (wv == I) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (4 * (l >> 4) + e < (l & 15)) t[0][0][e] = 0.f;
     }
-    __syncthreads();
+    acc_to_lds<T>(t[0][0], s_A, LDC, 16 * I, 16 * wv);
+  }
+  __syncthreads();
+  } else {
+    // ---- blocks below the diagonal, one block row at a time ----
+    for (int I = 1; I < 4; ++I) {
+      const float* bs = s_b + (16 * I - 1) * LDB;                   // b* of this block row
+      for (int idx = threadIdx.x; idx < 16 * K; idx += NTHR) {
+        const int r = idx / K, c = idx % K, i = 16 * I + r;
+        s_qt[r * LDK + c] = ET<T>::from_f(ET<T>::to_f(s_q[i * LDK + c]) * texp_scaled<T>(s_b[i * LDB + c] - bs[c]));
+      }
+      for (int idx = threadIdx.x; idx < 16 * I * K; idx += NTHR) {
+        const int j = idx / K, c = idx % K;
+        s_kt[j * LDK + c] = ET<T>::from_f(ET<T>::to_f(s_k[j * LDK + c]) * texp_scaled<T>(bs[c] - s_b[j * LDB + c]));
+      }
+      __syncthreads();
+      if (wv < I) {
+        f32x4 t[1][1];
+        acc_zero(t);
+        gemm<T, 1, 1, false, false>(t, s_qt, LDK, 0, s_kt, LDK, 16 * wv, 0, K);
+        acc_to_lds<T>(t[0][0], s_A, LDC, 16 * I, 16 * wv);
+      }
+      __syncthreads();
+    }
   }
   IOA::lds_to_global(s_A, LDC, (T*)a.amat + ((int64_t)cid * a.H + h) * CH * CH, CH, CH);
 }

@@ -14,6 +14,9 @@ CASES = [
     (1, 2, 130, 128, 128, True, False, True, 1.0),     # HGRN2-style gate: logsigmoid in fp32
     (1, 2, 64, 128, 64, False, True, True, 0.25),      # strong decay (4 * logsigmoid)
     (1, 1, 3, 64, 64, True, True, False, 16.0),
+    # decay over 16 tokens far beyond what the diagonal blocks may factor through a reference gate: every
+    # diagonal block takes the per-pair path (the case above mixes both, the first two factor all of them)
+    (1, 2, 130, 64, 128, True, True, True, 0.1),
 ]
 
 
