@@ -571,11 +571,10 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
   constexpr int LDC = CH + LPAD, LDK = K + LPAD;
   // layout of that form: b (fp32) | q, k as loaded | dA | k~ | q~  (element type T)
   constexpr int S_B = 0, S_TBASE = CH * LDB * 4;
-  constexpr int T_Q = 0, T_K = T_Q + CH * LDK, T_DA = T_K + CH * LDK, T_KT = T_DA + CH * LDC, T_QT = T_KT + CH * LDK,
-                T_END = T_QT + CH * LDK;
+  constexpr int T_Q = 0, T_K = T_Q + CH * LDK, T_DA = T_K + CH * LDK, T_KT = T_DA + CH * LDC, T_END = T_KT + 192 * LDK;
   constexpr int S_BYTES = S_TBASE + T_END * (int)sizeof(T);
   constexpr bool SUB = S_BYTES + 4096 <= 160 * 1024;
-  static_assert(!SUB || 2 * CH * LDK * (int)sizeof(T) >= CH * LDB * 4, "the db tile fits over k~, q~");
+  static_assert(!SUB || 192 * LDK * (int)sizeof(T) >= CH * LDB * 4, "the db tile fits over the stacked k~, q~ tile");
   constexpr int B_BYTES = SUB ? S_BYTES : B_END * 4;
   constexpr int NBYTES = (A_END * (int)sizeof(T) > B_BYTES) ? A_END * (int)sizeof(T) : B_BYTES;
   __shared__ __attribute__((aligned(16))) unsigned char smem_raw[NBYTES];
@@ -649,7 +648,6 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
   T* tK = (T*)(smem_raw + S_TBASE) + T_K;
   T* tDA = (T*)(smem_raw + S_TBASE) + T_DA;
   T* tKT = (T*)(smem_raw + S_TBASE) + T_KT;
-  T* tQT = (T*)(smem_raw + S_TBASE) + T_QT;
   float* sBw = SUB ? smF + S_B / 4 : smF + B_B;
   {
 #pragma unroll
@@ -679,21 +677,74 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
   auto Pm = [&](int r, int j) { if constexpr (SUB) return ET<T>::to_f(tDA[r * LDC + j]); else return smF[B_DP + r * LDP + j]; };
   auto Qm = [&](int r, int c) { if constexpr (SUB) return ET<T>::to_f(tQ[r * LDK + c]); else return smF[B_Q + r * LDB + c]; };
   auto Km = [&](int r, int c) { if constexpr (SUB) return ET<T>::to_f(tK[r * LDK + c]); else return smF[B_K + r * LDB + c]; };
-  // off-diagonal parts: wave R takes the dq rows of sub-chunk R, wave R - 1 the dk rows of sub-chunk R - 1
+  // Intra-chunk sums through reference gates (see k_gla_intra_fwd).  Wave w owns sub-chunk w:
+  //   dq rows:  e^{b_i - ref_w}  [ dA(rows of w, j < 16 w + 16) (k_j e^{ref_w - b_j}) ],   ref_w  = b_{16 w - 1} (0 for w = 0)
+  //   dk rows:  e^{ref'_w - b_j} [ dA^T(rows of w, i >= 16 w)   (q_i e^{b_i - ref'_w}) ],  ref'_w = b_{16 w + 15}
+  // Tokens outside the wave's own sub-chunk have exponents <= 0; inside it the exponent is a decay over at
+  // most 16 tokens, taken only if it stays below GLA_SAFE_EXP for every channel of the sub-chunk: otherwise
+  // those rows of the scaled operand are zero and the diagonal block takes the per-pair loops below.
+  // Two rounds over one stacked LDS tile: sub-chunks {0, 3}, then {1, 2} (contraction ranges in multiples of 32
+  // tokens: k~ of sub-chunk 0 / 1 / 2 / 3 holds 32 / 32 / 64 / 64 rows, q~ 64 / 64 / 32 / 32).
+  int unsafe = 0;
   f32x4 dqo[1][NBK], dko[1][NBK];
   acc_zero(dqo); acc_zero(dko);
   if constexpr (SUB) {
-    for (int R = 1; R < 4; ++R) {
-      const float* bs = sB + (16 * R - 1) * LDB;                  // b* of this boundary
-      for (int idx = threadIdx.x; idx < CH * K; idx += NTHR) {
-        const int r = idx / K, c = idx % K;
-        const float br = sB[r * LDB + c];
-        tKT[r * LDK + c] = ET<T>::from_f(r < 16 * R ? Km(r, c) * texp<T>(bs[c] - br) : 0.f);
-        tQT[r * LDK + c] = ET<T>::from_f(r >= 16 * R ? Qm(r, c) * texp<T>(br - bs[c]) : 0.f);
+    __shared__ int s_unsafe;
+    if (threadIdx.x == 0) s_unsafe = 0;
+    if (threadIdx.x < K) {
+#pragma unroll
+      for (int I = 0; I < 4; ++I) {
+        const float ref = I == 0 ? 0.f : sB[(16 * I - 1) * LDB + threadIdx.x];
+        if (!(ref - sB[(16 * I + 15) * LDB + threadIdx.x] <= GLA_SAFE_EXP)) unsafe |= 1 << I;
+      }
+    }
+    __syncthreads();
+    if (unsafe) atomicOr(&s_unsafe, unsafe);
+    __syncthreads();
+    unsafe = s_unsafe;
+#pragma unroll
+    for (int rd = 0; rd < 2; ++rd) {
+      // segment s of the stacked tile: s = 0, 1: k~ of sub-chunks wa, wb; s = 2, 3: q~ of sub-chunks wa, wb
+      const int wa = rd == 0 ? 0 : 1, wb = rd == 0 ? 3 : 2;
+      constexpr int SEGROW[4] = {0, 32, 96, 160};                       // k~(wa) 32 | k~(wb) 64 | q~(wa) 64 | q~(wb) 32
+      constexpr int VEC = ET<T>::VEC;
+      typedef typename ET<T>::vec vec;
+      for (int idx = threadIdx.x; idx < 192 * (K / VEC); idx += NTHR) {
+        const int sr = idx / (K / VEC), c0 = (idx % (K / VEC)) * VEC;   // one 16-byte piece of one stacked row
+        const int sg = sr < 32 ? 0 : sr < 96 ? 1 : sr < 160 ? 2 : 3;
+        const int w = (sg & 1) ? wb : wa;
+        const bool own_ok = !((unsafe >> w) & 1);
+        // token of this row, whether the row is in use, and the two gate rows whose difference is the exponent
+        int tok, hi_row, lo_row;                                        // exponent = b[hi_row] - b[lo_row] (hi_row < 0: 0)
+        bool use;
+        if (sg < 2) {
+          tok = sr - SEGROW[sg];
+          use = tok < 16 * w + 16 && (tok < 16 * w || own_ok);
+          hi_row = 16 * w - 1, lo_row = tok;                            // k_j e^{ref_w - b_j}
+        } else {
+          tok = (w < 2 ? 0 : 32) + sr - SEGROW[sg];
+          use = tok >= 16 * w && (tok >= 16 * w + 16 || own_ok);
+          hi_row = tok, lo_row = 16 * w + 15;                           // q_i e^{b_i - ref'_w}
+        }
+        vec o = ET<T>::zero();
+        if (use) {
+          const vec x = *(const vec*)((sg < 2 ? tK : tQ) + tok * LDK + c0);
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            const float hi = hi_row < 0 ? 0.f : sB[hi_row * LDB + c0 + e];
+            o[e] = ET<T>::from_f(ET<T>::to_f(x[e]) * texp<T>(hi - sB[lo_row * LDB + c0 + e]));
+          }
+        }
+        *(vec*)(tKT + sr * LDK + c0) = o;
       }
       __syncthreads();
-      if (wv == R) gemm<T, 1, NBK, false, true>(dqo, tDA, LDC, 16 * R, tKT, LDK, 0, 0, CH);
-      if (wv == R - 1) gemm<T, 1, NBK, true, true>(dko, tDA, LDC, 16 * (R - 1), tQT, LDK, 0, 0, CH);
+      if (wv == wa || wv == wb) {
+        const int sg = wv == wa ? 0 : 1;
+        const int nk = wv < 2 ? 32 : 64;                                // tokens j < nk
+        gemm<T, 1, NBK, false, true>(dqo, tDA, LDC, 16 * wv, tKT + SEGROW[sg] * LDK, LDK, 0, 0, nk);
+        const int i0 = wv < 2 ? 0 : 32;                                 // tokens i >= i0
+        gemm<T, 1, NBK, true, true>(dko, tDA, LDC, 16 * wv, tKT + (SEGROW[2 + sg] - i0) * LDK, LDK, 0, i0, CH);
+      }
       __syncthreads();
     }
   }
@@ -712,7 +763,11 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
     // where it is not, the dA factor is zero).  k_j, q_j, b_j are read once per token and column and serve
     // the lane's four rows; the dA values are read once per token and serve the four column tiles.
     float sqv[4][4], skv[4][4], brv[4][4];
-    if constexpr (SUB) {
+#pragma unroll
+    for (int n4 = 0; n4 < 4; ++n4)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sqv[n4][i] = skv[n4][i] = 0.f;
+    if (SUB && ((unsafe >> wv) & 1)) {
 #pragma unroll
       for (int n4 = 0; n4 < 4; ++n4)
 #pragma unroll
@@ -756,8 +811,8 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
         if constexpr (SUB) {
           sq_ = sqv[n4][i];
           sk_ = skv[n4][i];
-          if (wv >= 1) sq_ += dqo[0][ni][i] * texp<T>(br - sB[(16 * wv - 1) * LDB + cc]);
-          if (wv <= 2) sk_ += dko[0][ni][i] * texp<T>(sB[(16 * wv + 15) * LDB + cc] - br);
+          sq_ += dqo[0][ni][i] * texp<T>(br - (wv == 0 ? 0.f : sB[(16 * wv - 1) * LDB + cc]));
+          sk_ += dko[0][ni][i] * texp<T>(sB[(16 * wv + 15) * LDB + cc] - br);
         } else {
           for (int j = jlo; j <= r; ++j) sq_ += Pm(r, j) * Km(j, cc) * texp<T>(br - sB[j * LDB + cc]);
           for (int ii = r; ii < ihi; ++ii) sk_ += Pm(ii, r) * Qm(ii, cc) * texp<T>(sB[ii * LDB + cc] - br);
