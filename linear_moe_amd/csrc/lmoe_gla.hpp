@@ -184,18 +184,24 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
   }
   if constexpr (ONE_PASS) {
   // ---- scaled operands of all block rows at once: q~ (64 rows), k~ of block row I = rows 0 .. 16 I + 15 ----
-  for (int idx = threadIdx.x; idx < CH * K; idx += NTHR) {
-    const int i = idx / K, c = idx % K, I = i >> 4;
-    const float ref = I == 0 ? 0.f : s_b[(16 * I - 1) * LDB + c];
-    s_qt[i * LDK + c] = ET<T>::from_f(ET<T>::to_f(s_q[i * LDK + c]) * texp_scaled<T>(s_b[i * LDB + c] - ref));
-  }
+  {
+    constexpr int VEC = ET<T>::VEC;
+    typedef typename ET<T>::vec vec;
+    // stacked rows 0 .. 63: q~; 64 .. 223: k~ of block rows 0 .. 3 (16-byte pieces)
+    for (int idx = threadIdx.x; idx < (CH + 160) * (K / VEC); idx += NTHR) {
+      const int sr = idx / (K / VEC), c0 = (idx % (K / VEC)) * VEC;
+      const bool isq = sr < CH;
+      const int kr = sr - CH;                                           // row of the stacked k~ tile
+      const int I = isq ? (sr >> 4) : (kr < 16 ? 0 : kr < 48 ? 1 : kr < 96 ? 2 : 3);
+      const int tok = isq ? sr : kr - KT_ROW0(I);
+      const vec x = *(const vec*)((isq ? s_q : s_k) + tok * LDK + c0);
+      vec o;
 #pragma unroll
-  for (int I = 0; I < 4; ++I) {
-    T* kt = s_kt + KT_ROW0(I) * LDK;
-    for (int idx = threadIdx.x; idx < 16 * (I + 1) * K; idx += NTHR) {
-      const int j = idx / K, c = idx % K;
-      const float ref = I == 0 ? 0.f : s_b[(16 * I - 1) * LDB + c];
-      kt[j * LDK + c] = ET<T>::from_f(ET<T>::to_f(s_k[j * LDK + c]) * texp_scaled<T>(ref - s_b[j * LDB + c]));
+      for (int e = 0; e < VEC; ++e) {
+        const float ref = I == 0 ? 0.f : s_b[(16 * I - 1) * LDB + c0 + e], bt = s_b[tok * LDB + c0 + e];
+        o[e] = ET<T>::from_f(ET<T>::to_f(x[e]) * texp_scaled<T>(isq ? bt - ref : ref - bt));
+      }
+      *(vec*)((isq ? s_qt + sr * LDK : s_kt + kr * LDK) + c0) = o;
     }
   }
   __syncthreads();
