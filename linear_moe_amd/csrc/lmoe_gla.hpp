@@ -830,7 +830,12 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
         const float dkv = dkdv + sk_;
         kkp[ni] += kv * dkdv;
         dbv[ni][i] = qv * dqv - kv * dkv;
-        if (r < ci.len) {
+        if constexpr (SUB) {
+          // on their way out through the q, k tiles: this element of them is read by this lane only from here on
+          // (the per-pair loops above read other rows' elements of the columns of this group before this point)
+          tQ[r * LDK + cc] = ET<T>::from_f(dqv);
+          tK[r * LDK + cc] = ET<T>::from_f(dkv);
+        } else if (r < ci.len) {
           dqd[(int64_t)r * a.dq.st + cc] = ET<T>::from_f(dqv);
           dkd_g[(int64_t)r * a.dk.st + cc] = ET<T>::from_f(dkv);
         }
@@ -842,6 +847,10 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
     }
   }
   __syncthreads();   // all reads of the q tile are done: reuse it for db
+  if constexpr (SUB) {
+    IOK::lds_to_global(tQ, LDK, dqd, a.dq.st, ci.len);
+    IOK::lds_to_global(tK, LDK, dkd_g, a.dk.st, ci.len);
+  }
   float* sDB = SUB ? (float*)tKT : smF + B_Q;
 #pragma unroll
   for (int ni = 0; ni < NBK; ++ni)
