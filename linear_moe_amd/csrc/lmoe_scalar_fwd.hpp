@@ -22,15 +22,16 @@ template <typename T> __device__ __forceinline__ void scale_frag(typename ET<T>:
 //   grid = ceil(N*H / 8) * 8 * (V / BV) work-groups (1-D).  Work-group -> (sequence, head,
 //   V-slice): the V-slices of one (sequence, head) get ids that are congruent mod 8, i.e. run on
 //   the same XCD and share q, k through its L2.
-//   Team 0 (waves 0-3, consumers) carries the dependency chain of the state and nothing else:
-//        S -> LDS (element type T) | B1 | B2 | S = e^{b_C} S + k^T (e_d v)
+//   Team 0 (waves 0-3, consumers) carries the dependency chain of the state; between B1 and B2, where
+//     that chain waits for nobody, it forms P = (q k^T) . Gamma for the output team (wave-private LDS strips):
+//        S -> LDS (element type T) | B1 | P -> LDS | B2 | S = e^{b_C} S + k^T (e_d v)
 //     wave w owns state rows [w*K/4, (w+1)*K/4) x BV columns in fp32 MFMA accumulators; the row
 //     scaling e_d is applied to the v fragments in registers, so k is staged unscaled.
 //   Team 1 (waves 4-7, loaders) keeps the operands of the next PF chunks in flight in registers,
 //     forms the gate cumsum, fills the other LDS buffer and writes hs (layout [V][K]) from the
 //     LDS copy of S.
 //   Team 2 (waves 8-11, output) forms the chunk's output rows 16w..: between B1 and B2
-//     e^{b_i} q S and P = (q k^T) . Gamma (P through a wave-private LDS strip), after B2 P v.
+//     e^{b_i} q S, after B2 P v (P from the strip consumer wave w wrote).
 //   All teams meet at the same barriers; three waves per SIMD hide each other's latencies.
 // ------------------------------------------------------------------------- //
 template <typename T, int K, int V, int BV>
@@ -119,11 +120,11 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
         const int c = c0 + j;
         if (c >= sq.nchunks) break;
         lds_barrier();                                                                   // B1
+        // the next chunk's operands first (always: past the end it is the last chunk again, never consumed),
+        // so that the wait for their loads does not sit behind the store below
+        if constexpr (NBUF == 2) stage(pre[(j + 1) % PF], (c + 1) & 1);
         // hs[chunk][h][v0 .. v0+BV][K] <- S^T
         IOHT::lds_to_global(s_hT, LDK, (T*)a.hs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
-        if constexpr (NBUF == 2) {
-          if (c + 1 < sq.nchunks) stage(pre[(j + 1) % PF], (c + 1) & 1);
-        }
         lds_barrier();                                                                   // B2
         if constexpr (NBUF == 1) {
           lds_barrier();                                                                 // B3: buffer read
@@ -147,19 +148,6 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
       f32x4 o[1][NB];
       acc_zero(o);
       gemm<T, 1, NB, false, false>(o, s_q[cur], LDK, 16 * ow, s_hT, LDK, 0, 0, K);
-      f32x4 p[1][4];
-      acc_zero(p);
-      gemm<T, 1, 4, false, false>(p, s_q[cur], LDK, 16 * ow, s_k[cur], LDK, 0, 0, K);
-#pragma unroll
-      for (int nj = 0; nj < 4; ++nj) {
-        f32x4 x;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int i = 16 * ow + 4 * (l >> 4) + e, j = 16 * nj + (l & 15);
-          x[e] = (i >= j) ? p[0][nj][e] * texp<T>(s_b[cur][i] - s_b[cur][j]) : 0.f;
-        }
-        acc_to_lds<T>(x, pst, LDC, 0, 16 * nj);
-      }
 #pragma unroll
       for (int ni = 0; ni < NB; ++ni)
 #pragma unroll
@@ -199,6 +187,23 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
       for (int ni = 0; ni < NB; ++ni) acc_to_lds_t<T>(S[mi][ni], s_hT, LDK, krow0 + 16 * mi, 16 * ni);
     lds_barrier();                                                                       // B1
     const float dec = s_dec[cur];
+    // rows 16 wv .. of P = (q k^T) . Gamma for the output team (it reads them after B2): the consumers are idle
+    // between B1 and B2, the output team is not
+    {
+      f32x4 p[1][4];
+      acc_zero(p);
+      gemm<T, 1, 4, false, false>(p, s_q[cur], LDK, 16 * wv, s_k[cur], LDK, 0, 0, K);
+#pragma unroll
+      for (int nj = 0; nj < 4; ++nj) {
+        f32x4 x;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int i = 16 * wv + 4 * (l >> 4) + e, j = 16 * nj + (l & 15);
+          x[e] = (i >= j) ? p[0][nj][e] * texp<T>(s_b[cur][i] - s_b[cur][j]) : 0.f;
+        }
+        acc_to_lds<T>(x, s_pst + wv * 16 * LDC, LDC, 0, 16 * nj);
+      }
+    }
     lds_barrier();                                                                       // B2
 #pragma unroll
     for (int mi = 0; mi < MB; ++mi)
