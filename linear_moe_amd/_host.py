@@ -43,6 +43,23 @@ def _check_inputs(q, k, v, head_first: bool, cu_seqlens) -> Tuple[int, int, int,
     return B, T, H, K, V
 
 
+def no_tokens(q, k, v, head_first: bool, cu_seqlens, initial_state, output_final_state: bool):
+    """The call without any token (T = 0, or a batch of zero rows): nothing to launch.  Returns None when there
+    are tokens, else ``(o, final_state)``: an empty o and the initial state handed through (so that its gradient
+    is the gradient of the final state), zeros without one."""
+    B, T, H, K, V = _check_inputs(q, k, v, head_first, cu_seqlens)
+    if B * T > 0:
+        return None
+    N = B if cu_seqlens is None else cu_seqlens.numel() - 1
+    _state_check(initial_state, N, H, K, V, "initial_state")
+    o = torch.empty_like(v)
+    if not output_final_state:
+        return o, None
+    if initial_state is None:
+        return o, torch.zeros(N, H, K, V, dtype=torch.float32, device=q.device)
+    return o, initial_state.float() + 0
+
+
 def _desc(x: Optional[torch.Tensor], head_first: bool) -> Tensor4:
     """Stride descriptor of a [B,H,T,(D)] or [B,T,H,(D)] tensor."""
     if x is None:

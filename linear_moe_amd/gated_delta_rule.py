@@ -16,7 +16,7 @@ import torch
 
 from . import _lib
 from .l2norm import l2_norm
-from ._host import (SeqPlan, _aligned, _check_inputs, _desc, _state_check, base_args, ptr, stream_ptr)
+from ._host import (SeqPlan, _aligned, _check_inputs, _desc, _state_check, base_args, no_tokens, ptr, stream_ptr)
 
 
 def _scalar_dt(x: torch.Tensor) -> int:
@@ -146,5 +146,8 @@ def chunk_gated_delta_rule(
     if use_qk_l2norm_in_kernel:
         q = l2_norm(q)
         k = l2_norm(k)
+    r = no_tokens(q, k, v, head_first, cu_seqlens, initial_state, output_final_state)
+    if r is not None:
+        return r
     return _ChunkGatedDeltaRule.apply(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens,
                                       head_first)

@@ -13,7 +13,7 @@ from typing import Optional, Tuple
 import torch
 
 from . import _lib
-from ._host import (SeqPlan, _aligned, _check_inputs, _desc, _state_check, base_args, ptr, stream_ptr)
+from ._host import (SeqPlan, _aligned, _check_inputs, _desc, _state_check, base_args, no_tokens, ptr, stream_ptr)
 
 
 class GLACall:
@@ -116,4 +116,7 @@ def chunk_gla(
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """q, k, g: ``[B,H,T,K]``, v: ``[B,H,T,V]`` (``[B,T,H,*]`` with ``head_first=False``); g is the
     per-channel log-space decay.  Returns ``(o, final_state)``."""
+    r = no_tokens(q, k, v, head_first, cu_seqlens, initial_state, output_final_state)
+    if r is not None:
+        return r
     return _ChunkGLA.apply(q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first)

@@ -13,7 +13,7 @@ from typing import Optional, Tuple
 import torch
 
 from . import _lib
-from ._host import (SeqPlan, _aligned, _check_inputs, _desc, _state_check, base_args, ptr, stream_ptr)
+from ._host import (SeqPlan, _aligned, _check_inputs, _desc, _state_check, base_args, no_tokens, ptr, stream_ptr)
 
 
 class SimpleGLACall:
@@ -123,4 +123,7 @@ def chunk_simple_gla(
     """q, k: ``[B,H,T,K]``, v: ``[B,H,T,V]`` (``[B,T,H,*]`` with ``head_first=False``);
     g: ``[B,H,T]`` log-space decay or None.  Returns ``(o, final_state)`` with ``o`` shaped like
     ``v`` and ``final_state`` fp32 ``[N,H,K,V]`` or None."""
+    r = no_tokens(q, k, v, head_first, cu_seqlens, initial_state, output_final_state)
+    if r is not None:
+        return r
     return _ChunkSimpleGLA.apply(q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first)
