@@ -9,9 +9,17 @@ import torch
 from .simple_gla import chunk_simple_gla
 
 
+_DECAY = {}
+
+
 def retention_log_decay(H: int, device=None) -> torch.Tensor:
-    h = torch.arange(H, dtype=torch.float32, device=device)
-    return torch.log1p(-torch.pow(2.0, -5.0 - h))
+    """log(1 - 2^(-5-h)) for h < H, fp32 (formed once per head count and device, then reused: the call itself
+    then launches nothing but the op)."""
+    key = (H, str(device))
+    if key not in _DECAY:
+        h = torch.arange(H, dtype=torch.float64)
+        _DECAY[key] = torch.log1p(-torch.pow(2.0, -5.0 - h)).float().to(device)
+    return _DECAY[key]
 
 
 def chunk_retention(
