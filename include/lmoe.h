@@ -87,7 +87,7 @@ typedef struct lmoe_args {
   const float* dht;    /* [N,H,K,V] fp32 gradient of the final state or NULL           */
   /* backward outputs */
   lmoe_tensor dq, dk, dv; /* same shapes as q,k,v, element type = dtype                */
-  lmoe_tensor dg;      /* fp32, shape of g                                             */
+  lmoe_tensor dg;      /* shape of g; fp32, except chunk_gla: element type of g (g_dtype) */
   lmoe_tensor dbeta;   /* fp32, shape of beta                                          */
   float* dh0;          /* [N,H,K,V] fp32 or NULL                                       */
   /* backward workspace (caller-allocated, element type = dtype) */

@@ -876,11 +876,11 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
     float off = s_kk[cc] + s_kk[K + cc] + s_kk[2 * K + cc] + s_kk[3 * K + cc] + texp<T>(sB[63 * LDB + cc]) * s_hdh[cc];
 #pragma unroll
     for (int q = 1; q < NSEG; ++q) off += q > sg ? s_seg[q * K + cc] : 0.f;
-    float* dg = (float*)a.dg.ptr + row_off(a.dg, ci.b, ci.tok, h);
+    GT* dg = (GT*)a.dg.ptr + row_off(a.dg, ci.b, ci.tok, h);      // dg in the element type of g
 #pragma unroll
     for (int r = 0; r < SEG; ++r) {
       const int row = sg * SEG + r;
-      if (row < ci.len) dg[(int64_t)row * a.dg.st + cc] = v[r] + off;
+      if (row < ci.len) dg[(int64_t)row * a.dg.st + cc] = ET<GT>::from_f(v[r] + off);
     }
   }
 }

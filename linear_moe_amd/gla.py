@@ -77,7 +77,7 @@ class GLACall:
         a.dht = ptr(dht)
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
         a.dq, a.dk, a.dv = _desc(dq, head_first), _desc(dk, head_first), _desc(dv, head_first)
-        dg = torch.empty(g.shape, dtype=torch.float32, device=q.device)
+        dg = torch.empty(g.shape, dtype=g.dtype, device=q.device)      # written in the dtype of g by the kernel
         a.dg = _desc(dg, head_first)
         dh0 = torch.empty_like(h0) if self.has_h0 else None
         a.dh0 = ptr(dh0)
