@@ -16,7 +16,7 @@ static void launch_gla_t(const lmoe_args& a, int stage, hipStream_t st) {
   const dim3 block(NTHR);
   switch (stage) {
     case ST_GLA_INTRA_FWD:
-      hipLaunchKernelGGL((k_gla_intra_fwd<T, GT, K>), dim3(a.NT, a.H), block, 0, st, a); break;
+      hipLaunchKernelGGL((k_gla_intra_fwd<T, GT, K>), dim3(persistent_grid(a.NT * a.H, 2)), block, 0, st, a); break;
     case ST_STATE_FWD:
       hipLaunchKernelGGL((k_gla_state_fwd<T, GT, K, V, Tl::BVS>), dim3((a.N * a.H + 7) / 8 * 8 * (V / Tl::BVS)), block, 0, st, a); break;
     case ST_OUT_FWD:

@@ -32,7 +32,8 @@ constexpr int KT_ROW0(int I) { return 8 * I * (I + 1); }
 // g tile of the chunk -> fp32 LDS tile s_b[64][LDB] holding the inclusive cumsum over tokens.
 // The scan: a thread takes one channel over a segment of 64 K / 256 tokens (its values in registers, so the
 // LDS reads are independent of each other), the segment totals go through a small LDS array, and every thread
-// adds the totals of the segments before its own.  All 256 threads; ends with a barrier.
+// adds the totals of the segments before its own.  All 256 threads; ends with a barrier (the barriers order
+// LDS traffic only: loads a caller keeps in flight stay in flight).
 template <typename GT, int K>
 struct GlaGate {
   typedef TileIO<GT, CH, K> IOG;
@@ -48,7 +49,7 @@ struct GlaGate {
     static_assert(NTHR % K == 0 && CH % NSEG == 0, "one channel and one token segment per thread");
     IOG::mask(rg, len);
     IOG::store_lds_f32(rg, s_b, LDB);
-    __syncthreads();
+    lds_barrier();
     const int c = threadIdx.x % K, sg = threadIdx.x / K;
     float v[SEG];
 #pragma unroll
@@ -56,13 +57,13 @@ struct GlaGate {
 #pragma unroll
     for (int r = 1; r < SEG; ++r) v[r] += v[r - 1];
     s_tot[sg * K + c] = v[SEG - 1];
-    __syncthreads();
+    lds_barrier();
     float off = 0.f;
 #pragma unroll
     for (int q = 0; q < NSEG - 1; ++q) off += q < sg ? s_tot[q * K + c] : 0.f;
 #pragma unroll
     for (int r = 0; r < SEG; ++r) s_b[(sg * SEG + r) * LDB + c] = (v[r] + off) * mult;
-    __syncthreads();
+    lds_barrier();
   }
   template <int LDB>
   static __device__ __forceinline__ void finish(Regs& rg, int len, float* s_b) {
@@ -78,7 +79,7 @@ __device__ __forceinline__ void gla_gate_tile(const lmoe_args& a, int b, int tok
 }
 
 // ------------------------------------------------------------------------- //
-// A (intra-chunk attention matrix), grid = (NT, H)
+// A (intra-chunk attention matrix), persistent grid over the (chunk, head) items
 //   The chunk is cut into four sub-chunks of 16 tokens.  For a block (I, J) with J < I the decay
 //   factors through the cumulative gate at the last token before sub-chunk I, b* = b_{16 I - 1}:
 //     A_ij = sum_k (q_ik e^{b_ik - b*_k}) (k_jk e^{b*_k - b_jk}),   both exponents <= 0,
@@ -97,24 +98,38 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
   __shared__ __attribute__((aligned(16))) T s_qt[(ONE_PASS ? CH : 16) * LDK];   // q~: rows scaled to the reference of their block row
   __shared__ __attribute__((aligned(16))) T s_kt[(ONE_PASS ? 160 : 48) * LDK];  // k~ of block rows 0..3: 16 + 32 + 48 + 64 rows
   __shared__ __attribute__((aligned(16))) T s_A[CH * LDC];
-  const int cid = blockIdx.x, h = blockIdx.y;
-  const ChunkInfo ci = chunk_info(a, cid);
   const int wv = wave_id(), l = lane_id();
   typedef TileIO<T, CH, K> IOK;
   typedef TileIO<T, CH, CH> IOA;
+  typedef GlaGate<GT, K> GG;
+  // persistent: item = (chunk, head); the next item's q, k, g are requested at the top of an item and stay in
+  // flight behind its LDS-only barriers (item index clamped: every load is issued)
+  const int nitems = a.NT * a.H;
+  struct Pre { typename IOK::Regs rq, rk; typename GG::Regs rg; };
+  Pre pre;
+  auto issue = [&](int it) {
+    it = min(it, nitems - 1);
+    const int cid = it / a.H, h = it % a.H;
+    const ChunkInfo ci = chunk_info(a, cid);
+    IOK::load_nomask(pre.rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
+    IOK::load_nomask(pre.rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
+    GG::issue(pre.rg, a, ci.b, ci.tok, ci.len, h);
+  };
+  issue(blockIdx.x);
+  for (int it = blockIdx.x; it < nitems; it += gridDim.x) {
+  const int cid = it / a.H, h = it % a.H;
+  const ChunkInfo ci = chunk_info(a, cid);
   {
-    typename IOK::Regs rq, rk;
-    IOK::load(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
-    IOK::load(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
+    typename IOK::Regs rq = pre.rq, rk = pre.rk;
+    IOK::mask(rq, ci.len);
+    IOK::mask(rk, ci.len);
     IOK::store_lds(rq, s_q, LDK);
     IOK::store_lds(rk, s_k, LDK);
   }
+  typename GG::Regs rg = pre.rg;
+  issue(it + gridDim.x);
   for (int idx = threadIdx.x; idx < CH * LDC; idx += NTHR) s_A[idx] = ET<T>::from_f(0.f);   // blocks above the diagonal
-  {
-    typename GlaGate<GT, K>::Regs rg;
-    GlaGate<GT, K>::issue(rg, a, ci.b, ci.tok, ci.len, h);
-    GlaGate<GT, K>::template finish<LDB>(rg, ci.len, s_b, (float*)s_qt, TEXP_PRESCALE<T>);    // barriers inside; b in exp2 units
-  }
+  GG::template finish<LDB>(rg, ci.len, s_b, (float*)s_qt, TEXP_PRESCALE<T>);    // barriers inside; b in exp2 units
   // ---- gated operands for the other kernels: q e^{b}, k e^{b_C - b}, e^{b_C} ----
   {
     constexpr int VEC = ET<T>::VEC;
@@ -154,9 +169,9 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
     // bitwise OR over the work-group (the barrier-with-predicate intrinsics only tell zero from non-zero)
     __shared__ int s_unsafe;
     if (threadIdx.x == 0) s_unsafe = 0;
-    __syncthreads();
+    lds_barrier();
     if (unsafe) atomicOr(&s_unsafe, unsafe);
-    __syncthreads();
+    lds_barrier();
     unsafe = s_unsafe;
   } else {
     unsafe = 15;
@@ -204,7 +219,7 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
       *(vec*)((isq ? s_qt + sr * LDK : s_kt + kr * LDK) + c0) = o;
     }
   }
-  __syncthreads();
+  lds_barrier();
   // wave w: the blocks (I, w), I = w .. 3; the diagonal one masked to i >= j
 #pragma unroll
   for (int I = 0; I < 4; ++I) {
@@ -219,7 +234,7 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
     }
     acc_to_lds<T>(t[0][0], s_A, LDC, 16 * I, 16 * wv);
   }
-  __syncthreads();
+  lds_barrier();
   } else {
     // ---- blocks below the diagonal, one block row at a time ----
     for (int I = 1; I < 4; ++I) {
@@ -232,17 +247,19 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
         const int j = idx / K, c = idx % K;
         s_kt[j * LDK + c] = ET<T>::from_f(ET<T>::to_f(s_k[j * LDK + c]) * texp_scaled<T>(bs[c] - s_b[j * LDB + c]));
       }
-      __syncthreads();
+      lds_barrier();
       if (wv < I) {
         f32x4 t[1][1];
         acc_zero(t);
         gemm<T, 1, 1, false, false>(t, s_qt, LDK, 0, s_kt, LDK, 16 * wv, 0, K);
         acc_to_lds<T>(t[0][0], s_A, LDC, 16 * I, 16 * wv);
       }
-      __syncthreads();
+      lds_barrier();
     }
   }
   IOA::lds_to_global(s_A, LDC, (T*)a.amat + ((int64_t)cid * a.H + h) * CH * CH, CH, CH);
+  lds_barrier();      // the tiles are rewritten by the next item
+  }
 }
 
 // ------------------------------------------------------------------------- //
