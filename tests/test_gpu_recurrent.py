@@ -10,7 +10,9 @@ from tests.util import TOL, gen, max_abs_rel
 
 pytestmark = pytest.mark.gpu
 
-SHAPES = [(2, 1, 3, 64, 128), (1, 7, 2, 128, 64), (2, 70, 2, 128, 128), (1, 130, 2, 64, 64)]
+# T <= 4 tokens per sequence take the decoding-step kernel, longer ones the token-block kernel
+SHAPES = [(2, 1, 3, 64, 128), (2, 3, 2, 128, 128), (1, 4, 3, 64, 64), (1, 7, 2, 128, 64), (2, 70, 2, 128, 128),
+          (1, 130, 2, 64, 64)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
