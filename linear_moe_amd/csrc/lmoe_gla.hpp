@@ -397,23 +397,28 @@ __global__ __launch_bounds__(NTHR) void k_gla_out_fwd(const lmoe_args a) {
   IOK::store_lds(rq, s_q, LDK);
   IOH::store_lds_t(rh, s_hT, LDK, nullptr);
   lds_barrier();
-  f32x4 o[1][NB];
+  // the products are formed transposed (o^T = S^T (q e^b)^T, then += v^T A^T): a lane then holds four consecutive V
+  // columns of one token and stores them as one 8-byte piece
+  f32x4 o[NB][1];
   acc_zero(o);
-  gemm_nt<T, 1, NB>(o, s_q, LDK, 16 * wv, s_hT, LDK, 0, 0, K);
+  gemm_nt<T, NB, 1>(o, s_hT, LDK, 0, s_q, LDK, 16 * wv, 0, K);
   lds_barrier();                                                                       // q e^{b}, S^T are dead
   IOA::store_lds(ra, s_P, LDC);
   IOV::mask(rv, ci.len);
   IOV::store_lds_t(rv, s_vT, LDC, nullptr);
   lds_barrier();
-  gemm_nt<T, 1, NB>(o, s_P, LDC, 16 * wv, s_vT, LDC, 0, 0, CH);
-  T* od = row_ptr<T>(a.o, ci.b, ci.tok, h) + v0;
+  gemm_nt<T, NB, 1>(o, s_vT, LDC, 0, s_P, LDC, 16 * wv, 0, CH);
+  const int r = 16 * wv + (l & 15);
+  if (r < ci.len) {
+    T* od = row_ptr<T>(a.o, ci.b, ci.tok + r, h) + v0 + 4 * (l >> 4);
 #pragma unroll
-  for (int ni = 0; ni < NB; ++ni)
+    for (int ni = 0; ni < NB; ++ni) {
+      typename ET<T>::vec4 x;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
-      if (r < ci.len) od[(int64_t)r * a.o.st + cc] = ET<T>::from_f(o[0][ni][i] * a.scale);
+      for (int i = 0; i < 4; ++i) x[i] = ET<T>::from_f(o[ni][0][i] * a.scale);
+      *(typename ET<T>::vec4*)(od + 16 * ni) = x;
     }
+  }
 }
 
 // ------------------------------------------------------------------------- //
@@ -556,23 +561,27 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dv(const lmoe_args a) {
   IOK::store_lds(rk, s_kd, LDK);
   IOH::store_lds_t(rh, s_dhT, LDK, nullptr);
   lds_barrier();
-  f32x4 dv[1][NB], dv2[1][NB];
+  // products formed transposed (see k_gla_out_fwd): 8-byte stores of four consecutive V columns per token
+  f32x4 dv[NB][1], dv2[NB][1];
   acc_zero(dv); acc_zero(dv2);
-  gemm_nt<T, 1, NB>(dv2, s_kd, LDK, 16 * wv, s_dhT, LDK, 0, 0, K);
+  gemm_nt<T, NB, 1>(dv2, s_dhT, LDK, 0, s_kd, LDK, 16 * wv, 0, K);
   lds_barrier();                                                                       // k e^{..}, dS'^T are dead
   IOA::store_lds_t(ra, s_PT, LDC, nullptr);
   IOV::mask(rd, ci.len);
   IOV::store_lds_t(rd, s_doT, LDC, nullptr);
   lds_barrier();
-  gemm_nt<T, 1, NB>(dv, s_PT, LDC, 16 * wv, s_doT, LDC, 0, 0, CH);
-  T* dd = row_ptr<T>(a.dv, ci.b, ci.tok, h) + v0;
+  gemm_nt<T, NB, 1>(dv, s_doT, LDC, 0, s_PT, LDC, 16 * wv, 0, CH);
+  const int r = 16 * wv + (l & 15);
+  if (r < ci.len) {
+    T* dd = row_ptr<T>(a.dv, ci.b, ci.tok + r, h) + v0 + 4 * (l >> 4);
 #pragma unroll
-  for (int ni = 0; ni < NB; ++ni)
+    for (int ni = 0; ni < NB; ++ni) {
+      typename ET<T>::vec4 x;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * ni + (l & 15);
-      if (r < ci.len) dd[(int64_t)r * a.dv.st + cc] = ET<T>::from_f(a.scale * dv[0][ni][i] + dv2[0][ni][i]);
+      for (int i = 0; i < 4; ++i) x[i] = ET<T>::from_f(a.scale * dv[ni][0][i] + dv2[ni][0][i]);
+      *(typename ET<T>::vec4*)(dd + 16 * ni) = x;
     }
+  }
 }
 
 // ------------------------------------------------------------------------- //
