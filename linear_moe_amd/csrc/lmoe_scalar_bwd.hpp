@@ -98,7 +98,7 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dv(const lmoe_args a) {
 // ------------------------------------------------------------------------- //
 template <typename T, int K, int V, int BV>
 __global__ __launch_bounds__(2 * NTHR) void k_state_bwd(const lmoe_args a) {
-  constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDU = BV + LPAD;
+  constexpr int LDK = K + LPAD, LDU = BV + LPAD;
   constexpr int MB = K / 64, NB = BV / 16;
   // bf16: two operand buffers; fp32 (the parity path) has LDS for one and pays extra barriers
   constexpr int NBUF = sizeof(T) == 2 ? 2 : 1;
@@ -212,8 +212,6 @@ __global__ __launch_bounds__(2 * NTHR) void k_state_bwd(const lmoe_args a) {
   for (int it = 0; it < sq.nchunks; ++it) {
     const int c = sq.nchunks - 1 - it;
     const int cur = NBUF == 2 ? (it & 1) : 0;
-    const int tok = sq.tok0 + c * CH;
-    const int len = min(CH, sq.len - c * CH);
 #pragma unroll
     for (int mi = 0; mi < MB; ++mi)
 #pragma unroll

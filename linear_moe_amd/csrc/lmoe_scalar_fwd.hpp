@@ -178,8 +178,6 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
   }
   for (int c = 0; c < sq.nchunks; ++c) {
     const int cur = NBUF == 2 ? (c & 1) : 0;
-    const int tok = sq.tok0 + c * CH;
-    const int len = min(CH, sq.len - c * CH);
     // S (state at chunk start) -> LDS as S^T
 #pragma unroll
     for (int mi = 0; mi < MB; ++mi)
