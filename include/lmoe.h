@@ -116,7 +116,8 @@ int64_t lmoe_workspace_bytes(int32_t op, int32_t dtype, int32_t part, int32_t B,
  *   linear_moe/sequence_modeling/retention/retention.py:91                (chunk_retention)
  *   linear_moe/sequence_modeling/basic_linear_attention/basic_linear_attention.py:133 (chunk_linear_attn)
  *   linear_moe/sequence_modeling/lightning_attention/lightning_attention.py:121-123 (lightning_attn2)
- * fwd uses q,k,v,g,h0 -> o,ht,hs.  bwd uses q,k,v,g,hs,d_o,dht -> dq,dk,dv,dg,dh0 (+ dhs). */
+ * fwd uses q,k,v,g,h0 -> o,ht,hs (hs may be NULL: a forward-only call, which then saves nothing for a backward).
+ * bwd uses q,k,v,g,hs,d_o,dht -> dq,dk,dv,dg,dh0 (+ dhs). */
 int lmoe_chunk_simple_gla_fwd(const lmoe_args* a, void* stream);
 int lmoe_chunk_simple_gla_bwd(const lmoe_args* a, void* stream);
 

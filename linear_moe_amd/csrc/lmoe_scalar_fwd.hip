@@ -13,7 +13,8 @@ template <typename T, int K, int V> struct StateFwd {
   static void run(const lmoe_args& a, hipStream_t st) {
     constexpr int BV = FwdTiles<T, V>::BVS;
     const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BV);
-    hipLaunchKernelGGL((k_state_fwd<T, K, V, BV>), dim3(grid), dim3(3 * NTHR), 0, st, a);
+    if (a.hs) hipLaunchKernelGGL((k_state_fwd<T, K, V, BV, true>), dim3(grid), dim3(3 * NTHR), 0, st, a);
+    else hipLaunchKernelGGL((k_state_fwd<T, K, V, BV, false>), dim3(grid), dim3(3 * NTHR), 0, st, a);
   }
 };
 void launch_state_fwd(const lmoe_args& a, hipStream_t st) { dispatch<StateFwd>(a, st); }

@@ -29,12 +29,12 @@ template <typename T> __device__ __forceinline__ void scale_frag(typename ET<T>:
 //     scaling e_d is applied to the v fragments in registers, so k is staged unscaled.
 //   Team 1 (waves 4-7, loaders) keeps the operands of the next PF chunks in flight in registers,
 //     forms the gate cumsum, fills the other LDS buffer and writes hs (layout [V][K]) from the
-//     LDS copy of S.
+//     LDS copy of S (SAVE; a forward-only call passes hs = NULL and nothing is written).
 //   Team 2 (waves 8-11, output) forms the chunk's output rows 16w..: between B1 and B2
 //     e^{b_i} q S, after B2 P v (P from the strip consumer wave w wrote).
 //   All teams meet at the same barriers; three waves per SIMD hide each other's latencies.
 // ------------------------------------------------------------------------- //
-template <typename T, int K, int V, int BV>
+template <typename T, int K, int V, int BV, bool SAVE>
 __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
   constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDU = BV + LPAD;
   constexpr int MB = K / 64, NB = BV / 16;
@@ -123,8 +123,9 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
         // the next chunk's operands first (always: past the end it is the last chunk again, never consumed),
         // so that the wait for their loads does not sit behind the store below
         if constexpr (NBUF == 2) stage(pre[(j + 1) % PF], (c + 1) & 1);
-        // hs[chunk][h][v0 .. v0+BV][K] <- S^T
-        IOHT::lds_to_global(s_hT, LDK, (T*)a.hs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
+        // hs[chunk][h][v0 .. v0+BV][K] <- S^T (only the backward reads it: SAVE = false for forward-only calls)
+        if constexpr (SAVE)
+          IOHT::lds_to_global(s_hT, LDK, (T*)a.hs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
         lds_barrier();                                                                   // B2
         if constexpr (NBUF == 1) {
           lds_barrier();                                                                 // B3: buffer read

@@ -27,7 +27,8 @@ class SimpleGLACall:
         # blocks stay valid for lmoe_launch_stage; the autograd path must not (reference cycle)
         self.keep = keep
 
-    def forward(self, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first):
+    def forward(self, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first, save=True):
+        """save=False: a forward-only call (nothing requires a gradient): the per-chunk states are not written."""
         ctx = self
         lib = _lib.load()
         dims = _check_inputs(q, k, v, head_first, cu_seqlens)
@@ -49,10 +50,10 @@ class SimpleGLACall:
         a.h0 = ptr(h0)
         o = torch.empty_like(v)
         ht = torch.empty(plan.N, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
-        hs = torch.empty(max(plan.NT, 1), H, K, V, dtype=q.dtype, device=q.device)
+        hs = torch.empty(max(plan.NT, 1), H, K, V, dtype=q.dtype, device=q.device) if save else None
         a.o = _desc(o, head_first)
         a.ht = ptr(ht)
-        a.hs = hs.data_ptr()
+        a.hs = ptr(hs)
         _lib.check(lib.lmoe_chunk_simple_gla_fwd(C.byref(a), stream_ptr()), "chunk_simple_gla forward")
         ctx.saved = (q, k, v, g, h0, hs)
         ctx.fwd_args, ctx.fwd_keep = a, ((o, ht) if self.keep else None)
@@ -99,7 +100,8 @@ class _ChunkSimpleGLA(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first):
         call = SimpleGLACall()
-        o, ht = call.forward(q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first)
+        o, ht = call.forward(q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first,
+                             save=any(ctx.needs_input_grad))
         ctx.call = call
         return o, ht
 

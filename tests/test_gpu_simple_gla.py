@@ -3,6 +3,7 @@ import ctypes as C
 
 import pytest
 import torch
+import torch.nn.functional as F
 
 from oracle import naive
 from tests.util import TOL, gen, max_abs_rel
@@ -125,3 +126,18 @@ def test_simple_gla_bwd_varlen(cuda, dtype):
     torch.cuda.synchronize()
     for n, r in ref.items():
         assert max_abs_rel(dev[n].grad.cpu(), r) < TOL[dtype], n
+
+
+def test_forward_only_call_equals_the_saving_call(cuda):
+    """Without anything that requires a gradient the per-chunk states are not written (hs = NULL through the C ABI):
+    outputs and final state are bit-identical to those of the call that saves them for a backward."""
+    from linear_moe_amd import chunk_simple_gla
+    B, H, T, K, V = 2, 3, 300, 128, 64
+    q, k, v = (gen(4000 + i, B, H, T, D, dtype=torch.bfloat16).to(cuda) for i, D in enumerate((K, K, V)))
+    g = F.logsigmoid(gen(4003, B, H, T)).to(cuda)
+    h0 = (gen(4004, B, H, K, V) * 0.5).to(cuda)
+    with torch.no_grad():
+        o1, ht1 = chunk_simple_gla(q, k, v, g, None, h0, True)
+    o2, ht2 = chunk_simple_gla(q.clone().requires_grad_(True), k, v, g, None, h0, True)
+    torch.cuda.synchronize()
+    assert torch.equal(o1, o2.detach()) and torch.equal(ht1, ht2.detach())
