@@ -133,7 +133,8 @@ int lmoe_chunk_gla_bwd(const lmoe_args* a, void* stream);
  * o_t = scale q_t S_t.
  * Replaces fla.ops.gated_delta_rule.chunk_gated_delta_rule called at
  *   linear_moe/sequence_modeling/gated_deltanet/gated_deltanet.py:112.
- * fwd uses q,k,v,g,beta,h0 -> o,ht,hs,vnew,w,u,tinv,pmat,gcum.
+ * fwd uses q,k,v,g,beta,h0 -> o,ht,hs,vnew,w,u,tinv,pmat,gcum (hs, vnew and tinv, which only the backward reads,
+ * may all be NULL: a forward-only call).
  * bwd uses q,k,v,g,beta,hs,vnew,w,tinv,pmat,gcum,d_o,dht -> dq,dk,dv,dg,dbeta,dh0 (+ dhs, dvnew). */
 int lmoe_chunk_gated_delta_rule_fwd(const lmoe_args* a, void* stream);
 int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream);

@@ -13,7 +13,8 @@ template <typename T, int V> inline bool wide_slices(const lmoe_args& a) {
 }
 template <typename T, int K, int V, int BV> void launch_fwd(const lmoe_args& a, hipStream_t st) {
   const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BV);
-  hipLaunchKernelGGL((k_gdn_state_fwd<T, K, V, BV>), dim3(grid), dim3(3 * NTHR), 0, st, a);
+  if (a.hs) hipLaunchKernelGGL((k_gdn_state_fwd<T, K, V, BV, true>), dim3(grid), dim3(3 * NTHR), 0, st, a);
+  else hipLaunchKernelGGL((k_gdn_state_fwd<T, K, V, BV, false>), dim3(grid), dim3(3 * NTHR), 0, st, a);
 }
 template <typename T, int K, int V, int BV> void launch_bwd(const lmoe_args& a, hipStream_t st) {
   const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BV);

@@ -60,7 +60,8 @@ template <int L, typename F> __device__ __forceinline__ void ring_loop(int n, F&
 //   consumers, chunk c: S -> LDS | B1 | w S, q S, v_new -> LDS | B2 | S update, P v_new, o -> LDS
 //   (team 1 lifts v_new(c) right after B2 and stores it in the same half-step)
 // ------------------------------------------------------------------------- //
-template <typename T, int K, int V, int BV>
+// SAVE = false (forward-only call): hs and v_new, which only the backward reads, are not written
+template <typename T, int K, int V, int BV, bool SAVE>
 __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
   constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDU = BV + LPAD;
   constexpr int MB = K / 64, NB = BV / 16, KS = K / 32;
@@ -137,15 +138,17 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
       lds_barrier();                                                                     // B1
       stage_a(pa[j]);
       // S^T and the previous chunk's o leave LDS now (the consumers rewrite them after B2)
-      IOHT::load_lds(rh, s_hT, LDK);
+      if constexpr (SAVE) IOHT::load_lds(rh, s_hT, LDK);
       IOV::load_lds(ro, s_o, LDU);
       lds_barrier();                                                                     // B2
       // v_new of this chunk is complete (the consumers rewrite it after the next B1)
-      IOV::load_lds(rvn, s_vn, LDU);
-      // hs[chunk][h][v0 .. v0+BV][K] <- S^T
-      IOHT::store_global(rh, (T*)a.hs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
+      if constexpr (SAVE) {
+        IOV::load_lds(rvn, s_vn, LDU);
+        // hs[chunk][h][v0 .. v0+BV][K] <- S^T
+        IOHT::store_global(rh, (T*)a.hs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
+      }
       if (c > 0) store_result(ro, a.o, c - 1);
-      store_result(rvn, a.vnew, c);
+      if constexpr (SAVE) store_result(rvn, a.vnew, c);
       issue_a(pa[j], c + LPF);
     });
     lds_barrier();                                                                       // o of the last chunk

@@ -69,7 +69,8 @@ __device__ __forceinline__ void tri_inverse_64(const float* sL, int ldl, float* 
   }
 }
 
-template <typename T, int K, int V>
+// SAVE = false (forward-only call): Tinv, which only the backward reads, is not written
+template <typename T, int K, int V, bool SAVE>
 __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(const lmoe_args a) {
   constexpr int LDK = K + LPAD, LDV = V + LPAD, LDC = CH + LPAD;
   constexpr int NBK = K / 16, NBV = V / 16;
@@ -184,9 +185,9 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
       if constexpr (sizeof(T) == 2) {
         bf16x4 y; y[0] = (bf16)x[0]; y[1] = (bf16)x[1]; y[2] = (bf16)x[2]; y[3] = (bf16)x[3];
         *(bf16x4*)(s_Tm + r * LDC + c) = y;
-        *(bf16x4*)(tg + r * CH + c) = y;
+        if constexpr (SAVE) *(bf16x4*)(tg + r * CH + c) = y;
       } else {
-        *(f32x4*)(tg + r * CH + c) = x;
+        if constexpr (SAVE) *(f32x4*)(tg + r * CH + c) = x;
       }
     }
   }

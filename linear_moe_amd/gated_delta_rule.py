@@ -35,7 +35,9 @@ class GDNCall:
         # blocks stay valid for lmoe_launch_stage; the autograd path must not (reference cycle)
         self.keep = keep
 
-    def forward(self, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, head_first):
+    def forward(self, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, head_first, save=True):
+        """save=False: a forward-only call (nothing requires a gradient): what only the backward reads (the
+        per-chunk states, v_new, Tinv) is neither allocated nor written."""
         ctx = self
         lib = _lib.load()
         dims = _check_inputs(q, k, v, head_first, cu_seqlens)
@@ -61,14 +63,14 @@ class GDNCall:
         dev, dt = q.device, q.dtype
         o = torch.empty_like(v)
         ht = torch.empty(plan.N, H, K, V, dtype=torch.float32, device=dev) if output_final_state else None
-        hs = torch.empty(max(plan.NT, 1), H, K, V, dtype=dt, device=dev)
-        tinv = torch.empty(max(plan.NT, 1), H, 64, 64, dtype=dt, device=dev)
+        hs = torch.empty(max(plan.NT, 1), H, K, V, dtype=dt, device=dev) if save else None
+        tinv = torch.empty(max(plan.NT, 1), H, 64, 64, dtype=dt, device=dev) if save else None
         pmat = torch.empty(max(plan.NT, 1), H, 64, 64, dtype=dt, device=dev)
         gcum = torch.empty(max(plan.NT, 1), H, 2, 64, dtype=torch.float32, device=dev)
         w = torch.empty(B, T, H, K, dtype=dt, device=dev)
         u = torch.empty(B, T, H, V, dtype=dt, device=dev)
-        vnew = torch.empty(B, T, H, V, dtype=dt, device=dev)
-        a.o, a.ht, a.hs, a.tinv = _desc(o, head_first), ptr(ht), hs.data_ptr(), tinv.data_ptr()
+        vnew = torch.empty(B, T, H, V, dtype=dt, device=dev) if save else None
+        a.o, a.ht, a.hs, a.tinv = _desc(o, head_first), ptr(ht), ptr(hs), ptr(tinv)
         a.pmat, a.gcum = pmat.data_ptr(), gcum.data_ptr()
         a.w, a.u, a.vnew = _desc(w, False), _desc(u, False), _desc(vnew, False)
         _lib.check(lib.lmoe_chunk_gated_delta_rule_fwd(C.byref(a), stream_ptr()), "chunk_gated_delta_rule forward")
@@ -118,7 +120,8 @@ class _ChunkGatedDeltaRule(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, head_first):
         call = GDNCall()
-        o, ht = call.forward(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, head_first)
+        o, ht = call.forward(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, head_first,
+                             save=any(ctx.needs_input_grad))
         ctx.call = call
         return o, ht
 

@@ -141,3 +141,17 @@ def test_delta_rule_fwd_bwd(cuda, dtype, case):
     for n, r in ref.items():
         err = max_abs_rel(dev[n].grad.cpu(), r)
         assert err < tol, (n, err)
+
+
+def test_forward_only_call_equals_the_saving_call(cuda):
+    """Without anything that requires a gradient, what only the backward reads (per-chunk states, v_new, Tinv) is
+    neither allocated nor written (NULL through the C ABI): outputs and final state are bit-identical."""
+    from linear_moe_amd import chunk_gated_delta_rule
+    B, T, H, K, V = 2, 300, 3, 128, 128
+    q, k, v, g, beta = (x.to(cuda) for x in gdn_inputs(4100, B, T, H, K, V, torch.bfloat16, False))
+    h0 = (gen(4110, B, H, K, V) * 0.5).to(cuda)
+    with torch.no_grad():
+        o1, ht1 = chunk_gated_delta_rule(q, k, v, g, beta, None, h0, True, None, False)
+    o2, ht2 = chunk_gated_delta_rule(q.clone().requires_grad_(True), k, v, g, beta, None, h0, True, None, False)
+    torch.cuda.synchronize()
+    assert torch.equal(o1, o2.detach()) and torch.equal(ht1, ht2.detach())
