@@ -6,7 +6,7 @@ namespace lmoe {
 
 template <typename T, int V> struct BwdTiles {
   static constexpr int BVS = sizeof(T) == 4 ? 16 : 32;                // V-slice of the sequential pass
-  static constexpr int BVD = (sizeof(T) == 4 && V == 128) ? 64 : V;   // V-slice of k_bwd_dv
+  static constexpr int BVD = V == 128 ? 64 : V;                       // V-slice of k_bwd_dv (LDS for 2-3 work-groups per CU)
   static constexpr int BVH = sizeof(T) == 4 ? 32 : 64;                // V-slice loop of k_bwd_dqk
 };
 

@@ -23,13 +23,18 @@ template <typename T, int K, int V, int BV, bool LOCAL>
 __global__ __launch_bounds__(NTHR) void k_bwd_dv(const lmoe_args a) {
   constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDV = BV + LPAD;
   constexpr int NB = BV / 16;
-  __shared__ __attribute__((aligned(16))) T s_q[CH * LDK];
+  // One-shot work-groups: what hides their load latency is the number of them a CU holds, so LDS is used twice.
+  //   region A: q (for P), then dS'^T;   region B: do, then the staging strips of the result;   k and P^T apart.
+  // Every load is requested up front and waits in registers for its region.
+  constexpr int RA = (CH * LDK > (LOCAL ? 8 : BV * LDK)) ? CH * LDK : BV * LDK;
+  constexpr int RB = (CH * LDV > 4 * 16 * LDV) ? CH * LDV : 4 * 16 * LDV;
+  __shared__ __attribute__((aligned(16))) T s_ra[RA];
   __shared__ __attribute__((aligned(16))) T s_k[CH * LDK];
-  __shared__ __attribute__((aligned(16))) T s_do[CH * LDV];
-  __shared__ __attribute__((aligned(16))) T s_dhT[LOCAL ? 8 : BV * LDK];
+  __shared__ __attribute__((aligned(16))) T s_rb[RB];
   __shared__ __attribute__((aligned(16))) T s_PT[CH * LDC];
-  __shared__ __attribute__((aligned(16))) T s_stg[4 * 16 * LDV];
   __shared__ float s_b[64], s_ed[64];
+  T* s_q = s_ra; T* s_dhT = s_ra;
+  T* s_do = s_rb; T* s_stg = s_rb;
 
   const int cid = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * BV;
   const ChunkInfo ci = chunk_info(a, cid);
@@ -37,21 +42,20 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dv(const lmoe_args a) {
   typedef TileIO<T, CH, K> IOK;
   typedef TileIO<T, CH, BV> IOV;
   typedef TileIO<T, BV, K> IOH;
+  typename IOH::Regs rh;
   {
     typename IOK::Regs rq, rk;
     IOK::load(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
     IOK::load(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
     typename IOV::Regs rd;
     IOV::load(rd, row_ptr<T>(a.d_o, ci.b, ci.tok, h) + v0, a.d_o.st, ci.len);
-    typename IOH::Regs rh;
     if constexpr (!LOCAL) IOH::load(rh, (const T*)a.dhs + (((int64_t)cid * a.H + h) * V + v0) * K, K, BV);
     chunk_gate_cumsum(a, ci.b, ci.tok, ci.len, h, s_b, nullptr, s_ed);
     IOK::store_lds(rq, s_q, LDK);
     IOK::store_lds(rk, s_k, LDK);
     IOV::store_lds(rd, s_do, LDV);
-    if constexpr (!LOCAL) IOH::store_lds(rh, s_dhT, LDK);
   }
-  __syncthreads();
+  lds_barrier();
   {
     // P^T stored as s_PT[j][i]; wave w computes rows i = 16w.. of P and writes them transposed
     f32x4 s[1][4];
@@ -68,12 +72,14 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dv(const lmoe_args a) {
       acc_to_lds_t<T>(p, s_PT, LDC, 16 * wv, 16 * nj);
     }
   }
-  __syncthreads();
+  lds_barrier();                                                                         // q is dead
+  if constexpr (!LOCAL) IOH::store_lds(rh, s_dhT, LDK);
   f32x4 dv[1][NB];
   acc_zero(dv);
   gemm<T, 1, NB, false, true>(dv, s_PT, LDC, 16 * wv, s_do, LDV, 0, 0, CH);
 #pragma unroll
   for (int ni = 0; ni < NB; ++ni) dv[0][ni] *= a.scale;
+  lds_barrier();                                                                         // dS'^T staged; do is dead
   if constexpr (!LOCAL) {
     f32x4 t[1][NB];
     acc_zero(t);
