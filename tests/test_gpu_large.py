@@ -52,3 +52,32 @@ def test_offsets_beyond_32_bits(cuda, op):
         assert torch.equal(a, b), i
     del big, small
     torch.cuda.empty_cache()
+
+
+def test_row_kernels_beyond_32_bits(cuda):
+    """Row-wise neighbours on 2^24 + 1000 rows of 128 (2.15 G elements): the last rows equal a small call."""
+    from linear_moe_amd import gla_gate, l2_norm, rms_norm_fn, silu_l2_norm
+    if torch.cuda.get_device_properties(0).total_memory < 150 * 2**30:
+        pytest.skip("needs about 40 GB of GPU memory")
+    rows, D, tail = 2**24 + 1000, 128, 777
+    assert rows * D > 2**31
+    g_ = torch.Generator(device=cuda).manual_seed(6)
+    x = torch.randn(rows, D, device=cuda, generator=g_, dtype=torch.float32).bfloat16()
+    dy = torch.randn(tail, D, device=cuda, generator=g_, dtype=torch.float32).bfloat16()
+    w = (1 + 0.1 * torch.randn(D, device=cuda, generator=g_)).bfloat16()
+    fns = {"l2_norm": lambda t: l2_norm(t), "silu_l2_norm": lambda t: silu_l2_norm(t),
+           "rms_norm": lambda t: rms_norm_fn(t, w, None, eps=1e-5), "gla_gate": lambda t: gla_gate(t, 16.0)}
+    for name, fn in fns.items():
+        xb = x.clone().requires_grad_(True)
+        yb = fn(xb)
+        dyb = torch.zeros_like(yb)
+        dyb[-tail:] = dy
+        (gb,) = torch.autograd.grad(yb, xb, dyb)
+        xs = x[-tail:].clone().requires_grad_(True)
+        ys = fn(xs)
+        (gs,) = torch.autograd.grad(ys, xs, dy)
+        torch.cuda.synchronize()
+        assert torch.equal(yb[-tail:].detach(), ys.detach()), name
+        assert torch.equal(gb[-tail:], gs), name
+        del xb, yb, dyb, gb
+        torch.cuda.empty_cache()
