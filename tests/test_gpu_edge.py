@@ -118,3 +118,49 @@ def test_forward_and_backward_can_be_captured_in_a_graph(cuda):
         graph.replay()
         torch.cuda.synchronize()
         assert all(torch.equal(a, b) for a, b in zip(outs, ref))
+
+
+@pytest.mark.parametrize("op", OPS)
+def test_strided_views_need_no_copy_and_give_the_same(cuda, op):
+    """q, k, v as slices of one fused projection output [B, T, H, K + K + V] (row stride larger than the row), the
+    head-first call on transposed views of the same memory, and do as a strided view: bit for bit what contiguous
+    tensors give (the C ABI takes element strides; nothing is copied for 16-byte aligned rows)."""
+    dtype = torch.bfloat16
+    B, T, H, K, V = 2, 150, 2, 64, 128
+    ins = _inputs(op, T, H, K, V, dtype, 3300)
+    ins = {n: (x.expand(B, *x.shape[1:]).clone() if x.shape[0] == 1 else x) for n, x in ins.items()}
+    ins = {n: x + 0.01 * torch.arange(B, dtype=x.dtype).view(B, *([1] * (x.dim() - 1))) for n, x in ins.items()}
+    fused = torch.cat([ins["q"], ins["k"], ins["v"]], dim=-1).to(cuda)          # [B, T, H, 2K + V]
+    views = dict(q=fused[..., :K], k=fused[..., K:2 * K], v=fused[..., 2 * K:])
+    assert not views["q"].is_contiguous()
+    do_wide = gen(3310, B, T, H, 2 * V, dtype=dtype).to(cuda)
+    do = do_wide[..., V:]
+
+    def run(q, k, v, do, head_first):
+        t = dict(ins)
+        leaves = dict(q=q.detach().requires_grad_(True), k=k.detach().requires_grad_(True), v=v.detach().requires_grad_(True))
+        for n in ("g", "beta"):
+            if n in t:
+                x = t[n].to(cuda)
+                leaves[n] = (x.transpose(1, 2) if head_first else x).detach().requires_grad_(True)
+        from linear_moe_amd import chunk_gated_delta_rule, chunk_gla, chunk_simple_gla
+        if op == "simple_gla":
+            o, _ = chunk_simple_gla(leaves["q"], leaves["k"], leaves["v"], leaves["g"], None, None, False, None, head_first)
+        elif op == "gla":
+            o, _ = chunk_gla(leaves["q"], leaves["k"], leaves["v"], leaves["g"], None, None, False, None, head_first)
+        else:
+            o, _ = chunk_gated_delta_rule(leaves["q"], leaves["k"], leaves["v"], leaves["g"], leaves["beta"], None, None,
+                                          False, None, head_first)
+        grads = torch.autograd.grad(o, [leaves["q"], leaves["k"], leaves["v"]], do)
+        return [o.detach()] + list(grads)
+
+    ref = run(views["q"].contiguous(), views["k"].contiguous(), views["v"].contiguous(), do.contiguous(), False)
+    got = run(views["q"], views["k"], views["v"], do, False)
+    torch.cuda.synchronize()
+    for a, b in zip(got, ref):
+        assert torch.equal(a, b)
+    tr = lambda x: x.transpose(1, 2)                                             # [B, H, T, D] views, not contiguous
+    got_hf = run(tr(views["q"]), tr(views["k"]), tr(views["v"]), tr(do), True)
+    torch.cuda.synchronize()
+    for a, b in zip(got_hf, ref):
+        assert torch.equal(tr(a), b)
