@@ -333,7 +333,11 @@ template <typename T, int ROWS, int COLS> struct TileIO {
     for (int p = 0; p < PASSES; ++p) {
       int row, col; coords(p, row, col, tid);
       row = row < last ? row : last;
+#ifdef LMOE_NT_LD
+      r.v[p] = __builtin_nontemporal_load((const vec*)(src + (int64_t)row * row_stride + col));
+#else
       r.v[p] = *(const vec*)(src + (int64_t)row * row_stride + col);
+#endif
     }
   }
   static __device__ __forceinline__ void mask(Regs& r, int nvalid, int tid = threadIdx.x & (NTHR - 1)) {
@@ -439,7 +443,11 @@ template <typename T, int ROWS, int COLS> struct TileIO {
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
       int row, col; coords(p, row, col, tid);
+#ifdef LMOE_NT_ST
+      if (row < ROWS && row < nvalid) __builtin_nontemporal_store(r.v[p], (vec*)(dst + (int64_t)row * row_stride + col));
+#else
       if (row < ROWS && row < nvalid) *(vec*)(dst + (int64_t)row * row_stride + col) = r.v[p];
+#endif
     }
   }
   // Branch-free form of load_lds + store_global (nvalid >= 1): a thread whose row is >= nvalid reads
@@ -461,7 +469,11 @@ template <typename T, int ROWS, int COLS> struct TileIO {
     for (int p = 0; p < PASSES; ++p) {
       int row, col; coords(p, row, col, tid);
       row = row < last ? row : last;
+#ifdef LMOE_NT_ST
+      __builtin_nontemporal_store(r.v[p], (vec*)(dst + (int64_t)row * row_stride + col));
+#else
       *(vec*)(dst + (int64_t)row * row_stride + col) = r.v[p];
+#endif
     }
   }
   // global[row][col] = tile[row][col]

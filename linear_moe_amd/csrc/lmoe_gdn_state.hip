@@ -1,4 +1,7 @@
 // Instantiation and launch of the sequential passes of the gated delta rule.
+#ifdef LMOE_NT_STATE
+#define LMOE_NT_LD
+#endif
 #include "lmoe_launch.hpp"
 #include "lmoe_gdn_state.hpp"
 

@@ -27,7 +27,11 @@ namespace lmoe {
 __device__ __forceinline__ void tri_inverse_64(const float* sL, int ldl, float* sX, int ldx, float* sY, int l, int tid) {
   const int wv = wave_id();
   // clear X (upper blocks stay zero)
-  for (int idx = tid; idx < CH * CH; idx += NTHR) sX[(idx >> 6) * ldx + (idx & 63)] = 0.f;
+#pragma unroll
+  for (int p = 0; p < CH * CH / NTHR; ++p) {
+    const int idx = p * NTHR + tid;
+    sX[(idx >> 6) * ldx + (idx & 63)] = 0.f;
+  }
   lds_barrier();
   if (l < 16) {
     const int o = 16 * wv;
@@ -89,22 +93,34 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
   typedef TileIO<T, CH, V> IOV;
   typedef TileIO<T, CH, CH> IO64;
   const int nitems = a.NT * a.H;
-  // inputs of one item on their way in (always requested, item index clamped: a load that is skipped on
-  // some path would make the compiler drain all outstanding loads at every use)
-  struct Pre { typename IOK::Regs rk; typename IOV::Regs rv; RowFrags<T, K> fq; uint32_t graw, braw; };
-  Pre pre;
-  auto issue = [&](int it) {
+  // Inputs of an item: one register set, refilled for the next item of this work-group as soon as the
+  // current item has consumed a part (v after it is staged, q after q k^T, k after its second staging, gate
+  // and beta after the gate phase), so the requests are spread over the item instead of arriving as one
+  // burst: a burst of 48 KB per work-group fills the CU's queue of outstanding requests and the waves
+  // stall at the issue (measured: 1.4 us of an 11 us item).  Always requested, item index clamped: a load
+  // that is skipped on some path would make the compiler drain all outstanding loads at every use.
+  typename IOK::Regs rk;
+  typename IOV::Regs rv;
+  RowFrags<T, K> fq;
+  uint32_t graw, braw;
+  auto item_of = [&](int it, int& h) {
     it = min(it, nitems - 1);
-    const int cid = it / a.H, h = it % a.H;
-    const ChunkInfo ci = chunk_info(a, cid);
-    // q enters only as the A operand of q k^T: each wave takes its 16 rows straight into fragments
-    pre.fq.load(row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, 16 * wv, ci.len - 1);
-    IOK::load_nomask(pre.rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
-    IOV::load_nomask(pre.rv, row_ptr<T>(a.v, ci.b, ci.tok, h), a.v.st, ci.len);
-    pre.graw = gate_prefetch(a, ci.b, ci.tok, ci.len, h);
-    pre.braw = load_scalar_raw(a.beta.ptr, a.beta_dtype, row_off(a.beta, ci.b, ci.tok + min(l, ci.len - 1), h));
+    h = it % a.H;
+    return chunk_info(a, it / a.H);
   };
-  issue(blockIdx.x);
+  // q enters only as the A operand of q k^T: each wave takes its 16 rows straight into fragments
+  auto issue_q = [&](int it) { int h; const ChunkInfo ci = item_of(it, h); fq.load(row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, 16 * wv, ci.len - 1); };
+  auto issue_k = [&](int it) { int h; const ChunkInfo ci = item_of(it, h); IOK::load_nomask(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len); };
+  auto issue_v = [&](int it) { int h; const ChunkInfo ci = item_of(it, h); IOV::load_nomask(rv, row_ptr<T>(a.v, ci.b, ci.tok, h), a.v.st, ci.len); };
+  auto issue_gb = [&](int it) {
+    int h; const ChunkInfo ci = item_of(it, h);
+    graw = gate_prefetch(a, ci.b, ci.tok, ci.len, h);
+    braw = load_scalar_raw(a.beta.ptr, a.beta_dtype, row_off(a.beta, ci.b, ci.tok + min(l, ci.len - 1), h));
+  };
+  issue_q(blockIdx.x);
+  issue_k(blockIdx.x);
+  issue_v(blockIdx.x);
+  issue_gb(blockIdx.x);
   wait_all_loads();   // the first loads may be ordered freely; the loop's waits must not inherit that order
   for (int it = blockIdx.x; it < nitems; it += gridDim.x) {
   // lane / thread index refreshed per item: the address arithmetic derived from them stays inside the
@@ -113,26 +129,27 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
   const int tid = fresh_index((int)threadIdx.x) & (NTHR - 1);
   const int cid = it / a.H, h = it % a.H;
   const ChunkInfo ci = chunk_info(a, cid);
-  typename IOK::Regs rk = pre.rk;
-  typename IOV::Regs rv = pre.rv;
-  RowFrags<T, K> fq = pre.fq;
-  const uint32_t graw = pre.graw, braw = pre.braw;
-  issue(it + gridDim.x);
+  const int nxt = it + gridDim.x;
   IOK::mask(rk, ci.len, tid);
   IOV::mask(rv, ci.len, tid);
   lds_barrier();      // the previous item has left every tile
   if (wv == 1) s_beta[l] = l < ci.len ? scalar_from_raw(braw, a.beta_dtype) : 0.f;
   gate_finish(a, graw, ci.len, s_b, s_eb, nullptr);
+  issue_gb(nxt);
   lds_barrier();
-  if (tid < 64) {
-    s_beb[tid] = s_beta[tid] * s_eb[tid];
-    // decay table of the chunk for the sequential passes: e^{b_j}, e^{b_C - b_j}
+  if (tid < 64) s_beb[tid] = s_beta[tid] * s_eb[tid];
+  {
+    // decay table of the chunk for the sequential passes: e^{b_j}, e^{b_C - b_j}.  Every global store of
+    // this loop is issued by all threads on every path (here two threads write each entry), so that the
+    // compiler can count the operations behind the prefetch above exactly: a store under a condition made
+    // the wait for the next item's inputs a wait for this item's last stores as well
+    const int j = tid & 63;
     float* gc = a.gcum + ((int64_t)cid * a.H + h) * 2 * CH;
-    gc[tid] = s_eb[tid];
-    gc[CH + tid] = expf(s_b[CH - 1] - s_b[tid]);
+    gc[tid & 127] = (tid & 64) ? expf(s_b[CH - 1] - s_b[j]) : s_eb[j];
   }
   IOK::store_lds(rk, s_k, LDK, tid);
   IOV::store_lds_scaled(rv, s_vb, LDV, s_beta, tid);
+  issue_v(nxt);
   lds_barrier();
   {
     f32x4 m[1][4];
@@ -170,16 +187,20 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
       }
       acc_to_lds<T>(pm[0][nj], s_P, LDC, 16 * wv, 16 * nj, l);
     }
+    issue_q(nxt);
     lds_barrier();
     IO64::lds_to_global(s_P, LDC, pg, CH, CH, tid);
   }
   // k is dead as an operand of k k^T and q k^T: scale it in place to k beta e^{b} (from the registers)
   IOK::store_lds_scaled(rk, s_k, LDK, s_beb, tid);
+  issue_k(nxt);
   lds_barrier();   // L is complete, the P staging has been read: the inverse may overwrite X
   tri_inverse_64(s_L, LDC, s_X, LDC, s_Y, l, tid);       // barriers inside; s_L is dead afterwards
   {
     T* tg = (T*)a.tinv + ((int64_t)cid * a.H + h) * CH * CH;
-    for (int idx = tid; idx < CH * CH / 4; idx += NTHR) {
+#pragma unroll
+    for (int p = 0; p < CH * CH / 4 / NTHR; ++p) {      // fixed trip count: see the decay table above
+      const int idx = p * NTHR + tid;
       const int r = idx >> 4, c = (idx & 15) * 4;
       const f32x4 x = *(const f32x4*)(s_X + r * LDC + c);
       if constexpr (sizeof(T) == 2) {
@@ -199,9 +220,21 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
   f32x4 u[1][NBV];
   acc_zero(u);
   gemm<T, 1, NBV, false, true>(u, s_Tm, LDC, 16 * wv, s_vb, LDV, 0, 0, CH, l);
-  lds_barrier();   // k, v tiles are dead: wave-private slices of them stage the stores
-  store_strip<T, NBK>(w, s_k + wv * 16 * LDK, row_ptr<T>(a.w, ci.b, ci.tok + 16 * wv, h), a.w.st, ci.len - 16 * wv, 1.0f, l);
-  store_strip<T, NBV>(u, s_vb + wv * 16 * LDV, row_ptr<T>(a.u, ci.b, ci.tok + 16 * wv, h), a.u.st, ci.len - 16 * wv, 1.0f, l);
+  lds_barrier();   // k, v tiles are dead: they stage the stores
+#pragma unroll
+  for (int ni = 0; ni < NBK; ++ni) acc_to_lds<T>(w[0][ni], s_k, LDK, 16 * wv, 16 * ni, l);
+#pragma unroll
+  for (int ni = 0; ni < NBV; ++ni) acc_to_lds<T>(u[0][ni], s_vb, LDV, 16 * wv, 16 * ni, l);
+  lds_barrier();
+  {
+    // branch-free (rows past the end of a partial chunk rewrite its last row with the same bytes)
+    typename IOK::Regs ow;
+    typename IOV::Regs ou;
+    IOK::load_lds_clamped(ow, s_k, LDK, ci.len, tid);
+    IOV::load_lds_clamped(ou, s_vb, LDV, ci.len, tid);
+    IOK::store_global_clamped(ow, row_ptr<T>(a.w, ci.b, ci.tok, h), a.w.st, ci.len, tid);
+    IOV::store_global_clamped(ou, row_ptr<T>(a.u, ci.b, ci.tok, h), a.u.st, ci.len, tid);
+  }
   }   // items
 }
 
