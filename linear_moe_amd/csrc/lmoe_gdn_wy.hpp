@@ -152,42 +152,52 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
   issue_v(nxt);
   lds_barrier();
   {
-    f32x4 m[1][4];
-    acc_zero(m);
-    gemm<T, 1, 4, false, false>(m, s_k, LDK, 16 * wv, s_k, LDK, 0, 0, K, l);
-#pragma unroll
-    for (int nj = 0; nj < 4; ++nj) {
-      f32x4 p;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * nj + (l & 15);
-        p[i] = (r > cc) ? s_beta[r] * m[0][nj][i] * texp<T>(s_b[r] - s_b[cc]) : 0.f;
-      }
-      acc_to_lds<float>(p, s_L, LDC, 16 * wv, 16 * nj, l);
-    }
-  }
-  {
-    // P = (q k^T) . Gamma -> global, staged through the (still unused) X tile
+    // L (from k k^T) and P = (q k^T) . Gamma over the same k fragments; the blocks above the diagonal are
+    // zero and skipped (wave-uniform), and one exponential per element serves both.  P goes to global
+    // memory, staged through the (still unused) X tile
     T* s_P = (T*)s_X;
     T* pg = (T*)a.pmat + ((int64_t)cid * a.H + h) * CH * CH;
-    f32x4 pm[1][4];
-    acc_zero(pm);
+    f32x4 m[4], pm[4];
+#pragma unroll
+    for (int nj = 0; nj < 4; ++nj) { m[nj] = f32x4{0.f, 0.f, 0.f, 0.f}; pm[nj] = m[nj]; }
     fq.mask(16 * wv, ci.len);
+    const int fr = l & 15, fg = 8 * (l >> 4);
 #pragma unroll
-    for (int ks = 0; ks < K / 32; ++ks)
+    for (int ks = 0; ks < K / 32; ++ks) {
+      const typename ET<T>::frag ak = ET<T>::load_frag(s_k + (16 * wv + fr) * LDK + 32 * ks + fg);
 #pragma unroll
-      for (int nj = 0; nj < 4; ++nj)
-        ET<T>::mma(pm[0][nj], fq.f[ks], ET<T>::load_frag(s_k + (16 * nj + (l & 15)) * LDK + 32 * ks + 8 * (l >> 4)));
-#pragma unroll
-    for (int nj = 0; nj < 4; ++nj) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int r = 16 * wv + 4 * (l >> 4) + i, cc = 16 * nj + (l & 15);
-        pm[0][nj][i] = (r >= cc) ? pm[0][nj][i] * texp<T>(s_b[r] - s_b[cc]) : 0.f;
+      for (int nj = 0; nj < 4; ++nj) {
+        if (nj <= wv) {
+          const typename ET<T>::frag bk = ET<T>::load_frag(s_k + (16 * nj + fr) * LDK + 32 * ks + fg);
+          ET<T>::mma(m[nj], ak, bk);
+          ET<T>::mma(pm[nj], fq.f[ks], bk);
+        }
       }
-      acc_to_lds<T>(pm[0][nj], s_P, LDC, 16 * wv, 16 * nj, l);
     }
     issue_q(nxt);
+    float br[4], betar[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      br[i] = s_b[16 * wv + 4 * (l >> 4) + i];
+      betar[i] = s_beta[16 * wv + 4 * (l >> 4) + i];
+    }
+#pragma unroll
+    for (int nj = 0; nj < 4; ++nj) {
+      f32x4 pl = {0.f, 0.f, 0.f, 0.f}, pp = {0.f, 0.f, 0.f, 0.f};
+      if (nj <= wv) {
+        const int cc = 16 * nj + fr;
+        const float bc = s_b[cc];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int r = 16 * wv + 4 * (l >> 4) + i;
+          const float e = texp<T>(br[i] - bc);
+          pl[i] = (r > cc) ? betar[i] * m[nj][i] * e : 0.f;
+          pp[i] = (r >= cc) ? pm[nj][i] * e : 0.f;
+        }
+      }
+      acc_to_lds<float>(pl, s_L, LDC, 16 * wv, 16 * nj, l);
+      acc_to_lds<T>(pp, s_P, LDC, 16 * wv, 16 * nj, l);
+    }
     lds_barrier();
     IO64::lds_to_global(s_P, LDC, pg, CH, CH, tid);
   }
