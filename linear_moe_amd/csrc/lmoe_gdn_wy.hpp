@@ -223,18 +223,30 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
     }
   }
   lds_barrier();
-  // w = Tinv (k beta e^{b}),  u = Tinv (v beta): contraction over the rows of the [64][D] tiles
-  f32x4 w[1][NBK];
-  acc_zero(w);
-  gemm<T, 1, NBK, false, true>(w, s_Tm, LDC, 16 * wv, s_k, LDK, 0, 0, CH, l);
-  f32x4 u[1][NBV];
-  acc_zero(u);
-  gemm<T, 1, NBV, false, true>(u, s_Tm, LDC, 16 * wv, s_vb, LDV, 0, 0, CH, l);
+  // w = Tinv (k beta e^{b}),  u = Tinv (v beta): contraction over the rows of the [64][D] tiles.  Formed
+  // transposed (the tile as the A operand through transposing LDS reads, Tinv rows as B), so that a lane
+  // holds four consecutive columns of one token and the results go back to LDS as 8-byte writes.  Tinv is
+  // lower triangular: the second half of the contraction is zero for the first 32 tokens
+  f32x4 w[NBK], u[NBV];
+#pragma unroll
+  for (int ni = 0; ni < NBK; ++ni) w[ni] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int ni = 0; ni < NBV; ++ni) u[ni] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int ks = 0; ks < CH / 32; ++ks) {
+    if (ks == 0 || wv >= 2) {
+      const typename ET<T>::frag bt = ET<T>::load_frag(s_Tm + (16 * wv + (l & 15)) * LDC + 32 * ks + 8 * (l >> 4));
+#pragma unroll
+      for (int ni = 0; ni < NBK; ++ni) ET<T>::mma(w[ni], ET<T>::load_frag_t(s_k, LDK, 32 * ks, 16 * ni), bt);
+#pragma unroll
+      for (int ni = 0; ni < NBV; ++ni) ET<T>::mma(u[ni], ET<T>::load_frag_t(s_vb, LDV, 32 * ks, 16 * ni), bt);
+    }
+  }
   lds_barrier();   // k, v tiles are dead: they stage the stores
 #pragma unroll
-  for (int ni = 0; ni < NBK; ++ni) acc_to_lds<T>(w[0][ni], s_k, LDK, 16 * wv, 16 * ni, l);
+  for (int ni = 0; ni < NBK; ++ni) acc_to_lds_t<T>(w[ni], s_k, LDK, 16 * ni, 16 * wv, l);
 #pragma unroll
-  for (int ni = 0; ni < NBV; ++ni) acc_to_lds<T>(u[0][ni], s_vb, LDV, 16 * wv, 16 * ni, l);
+  for (int ni = 0; ni < NBV; ++ni) acc_to_lds_t<T>(u[ni], s_vb, LDV, 16 * ni, 16 * wv, l);
   lds_barrier();
   {
     // branch-free (rows past the end of a partial chunk rewrite its last row with the same bytes)
