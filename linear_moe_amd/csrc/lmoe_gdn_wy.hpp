@@ -84,7 +84,7 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
   __shared__ __attribute__((aligned(16))) float s_L[CH * LDC];   // L, later Tinv in element type T
   __shared__ __attribute__((aligned(16))) float s_X[CH * LDC];
   __shared__ float s_Y[4 * 272];
-  __shared__ float s_b[64], s_eb[64], s_beta[64], s_beb[64];
+  __shared__ float s_b[64], s_beta[64], s_beb[64];
   // Tinv as an MFMA operand: fp32 uses s_X in place, bf16 a copy in the (dead) L tile
   T* s_Tm = sizeof(T) == 4 ? (T*)s_X : (T*)s_L;
 
@@ -133,22 +133,37 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
   IOK::mask(rk, ci.len, tid);
   IOV::mask(rv, ci.len, tid);
   lds_barrier();      // the previous item has left every tile
-  if (wv == 1) s_beta[l] = l < ci.len ? scalar_from_raw(braw, a.beta_dtype) : 0.f;
-  gate_finish(a, graw, ci.len, s_b, s_eb, nullptr);
+  // Every wave holds the gates and beta of all 64 tokens (lane = token) and forms the cumulative gate for
+  // itself: the staging below needs no value from another wave, so one barrier covers gate and staging
+  const bool gated = a.gate != LMOE_GATE_NONE && a.g.ptr != nullptr;
+  const float bl = l < ci.len ? scalar_from_raw(braw, a.beta_dtype) : 0.f;
+  const float xb = wave_incl_scan((gated && l < ci.len) ? scalar_from_raw(graw, a.g_dtype) : 0.f);
+  const float eb = expf(xb), ed = expf(__shfl(xb, 63, 64) - xb);
   issue_gb(nxt);
-  lds_barrier();
-  if (tid < 64) s_beb[tid] = s_beta[tid] * s_eb[tid];
+  if (wv == 0) {
+    s_b[l] = xb;
+    s_beta[l] = bl;
+    s_beb[l] = bl * eb;
+  }
   {
     // decay table of the chunk for the sequential passes: e^{b_j}, e^{b_C - b_j}.  Every global store of
-    // this loop is issued by all threads on every path (here two threads write each entry), so that the
-    // compiler can count the operations behind the prefetch above exactly: a store under a condition made
+    // this loop is issued by all threads on every path (here two waves write each entry), so that the
+    // compiler can count the operations behind the prefetches exactly: a store under a condition made
     // the wait for the next item's inputs a wait for this item's last stores as well
-    const int j = tid & 63;
     float* gc = a.gcum + ((int64_t)cid * a.H + h) * 2 * CH;
-    gc[tid & 127] = (tid & 64) ? expf(s_b[CH - 1] - s_b[j]) : s_eb[j];
+    gc[tid & 127] = (tid & 64) ? ed : eb;
   }
   IOK::store_lds(rk, s_k, LDK, tid);
-  IOV::store_lds_scaled(rv, s_vb, LDV, s_beta, tid);
+#pragma unroll
+  for (int p = 0; p < IOV::PASSES; ++p) {       // v beta, beta of the row from the lane that holds it
+    int row, col;
+    IOV::coords(p, row, col, tid);
+    const float sc = __shfl(bl, row & 63, 64);
+    typename IOV::vec o;
+#pragma unroll
+    for (int i = 0; i < IOV::VEC; ++i) o[i] = ET<T>::from_f(ET<T>::to_f(rv.v[p][i]) * sc);
+    *(typename IOV::vec*)(s_vb + row * LDV + col) = o;
+  }
   issue_v(nxt);
   lds_barrier();
   {
