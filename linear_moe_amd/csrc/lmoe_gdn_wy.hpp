@@ -9,6 +9,7 @@
 // stay in flight behind its LDS-only barriers.  Writes w, u, Tinv and P (element type T) and the
 // chunk's decay table e^{b}, e^{b_C - b} (fp32).
 #pragma once
+#include <type_traits>
 #include "lmoe_seq.hpp"
 
 namespace lmoe {
@@ -34,17 +35,44 @@ __device__ __forceinline__ void tri_inverse_64(const float* sL, int ldl, float* 
   }
   lds_barrier();
   if (l < 16) {
-    const int o = 16 * wv;
+    // lane c solves column c by forward substitution; every lane reads the same coefficients (broadcast
+    // reads of whole rows).  The rows are requested in three batches ahead of their use: reading each
+    // coefficient where it is used cost one LDS round trip per row (1.3 us of an 11 us item)
+    const float* lb = sL + 16 * wv * ldl + 16 * wv;
+    f32x4 c[16][4];
+    auto rows = [&](auto i0, auto i1) {
+#pragma unroll
+      for (int i = decltype(i0)::value; i < decltype(i1)::value; ++i)
+#pragma unroll
+        for (int j = 0; j < (i + 3) / 4; ++j) c[i][j] = *(const f32x4*)(lb + i * ldl + 4 * j);
+    };
     float x[16];
+    auto solve = [&](auto i0, auto i1) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      float s = (i == l) ? 1.f : 0.f;
+      for (int i = decltype(i0)::value; i < decltype(i1)::value; ++i) {
+        float s = (i == l) ? 1.f : 0.f;
 #pragma unroll
-      for (int m = 0; m < i; ++m) s -= sL[(o + i) * ldl + o + m] * x[m];
-      x[i] = s;
-    }
+        for (int m = 0; m < i; ++m) s -= c[i][m >> 2][m & 3] * x[m];
+        x[i] = s;
+      }
+    };
+    typedef std::integral_constant<int, 0> I0;
+    typedef std::integral_constant<int, 8> I8;
+    typedef std::integral_constant<int, 12> I12;
+    typedef std::integral_constant<int, 16> I16;
+    rows(I0(), I8());
+    __builtin_amdgcn_sched_barrier(0);
+    rows(I8(), I12());
+    __builtin_amdgcn_sched_barrier(0);
+    solve(I0(), I8());
+    __builtin_amdgcn_sched_barrier(0);
+    rows(I12(), I16());
+    __builtin_amdgcn_sched_barrier(0);
+    solve(I8(), I12());
+    __builtin_amdgcn_sched_barrier(0);
+    solve(I12(), I16());
 #pragma unroll
-    for (int i = 0; i < 16; ++i) sX[(o + i) * ldx + o + l] = x[i];
+    for (int i = 0; i < 16; ++i) sX[(16 * wv + i) * ldx + 16 * wv + l] = x[i];
   }
   lds_barrier();
   // operand layout of the 16 x 16 x 4 instruction: A[m = l % 16][k = l / 16], B[k = l / 16][n = l % 16],
