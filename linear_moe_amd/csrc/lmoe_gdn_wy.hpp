@@ -79,21 +79,36 @@ __device__ __forceinline__ void tri_inverse_64(const float* sL, int ldl, float* 
   // result rows 4 (l / 16) + i of column l % 16
   const int r16 = l & 15, k4 = l >> 4;
   float* yb = sY + wv * 272;
+#pragma unroll
   for (int d = 1; d < 4; ++d) {
     if (wv + d < 4) {                      // wave-uniform: block (I, J) = (wv + d, wv)
       const int J = wv, I = wv + d;
+      // every operand of the round is requested before the first product (one LDS round trip instead of
+      // one per instruction)
+      float la[12], xb[12], xd[4];
+#pragma unroll
+      for (int t = 0; t < 4 * d; ++t) {
+        la[t] = sL[(16 * I + r16) * ldl + 16 * J + 4 * t + k4];
+        xb[t] = sX[(16 * J + 4 * t + k4) * ldx + 16 * J + r16];
+      }
+#pragma unroll
+      for (int t = 0; t < 4; ++t) xd[t] = sX[(16 * I + r16) * ldx + 16 * I + 4 * t + k4];
+      __builtin_amdgcn_sched_barrier(0);
       f32x4 y = {0.f, 0.f, 0.f, 0.f};
-      for (int m = 16 * J; m < 16 * I; m += 4)
-        y = __builtin_amdgcn_mfma_f32_16x16x4f32(sL[(16 * I + r16) * ldl + m + k4], sX[(m + k4) * ldx + 16 * J + r16], y, 0, 0, 0);
+#pragma unroll
+      for (int t = 0; t < 4 * d; ++t) y = __builtin_amdgcn_mfma_f32_16x16x4f32(la[t], xb[t], y, 0, 0, 0);
 #pragma unroll
       for (int i = 0; i < 4; ++i) yb[(4 * k4 + i) * 17 + r16] = y[i];
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      float yv[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) yv[t] = yb[(4 * t + k4) * 17 + r16];
+      __builtin_amdgcn_sched_barrier(0);
       f32x4 x = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int m = 0; m < 16; m += 4)
-        x = __builtin_amdgcn_mfma_f32_16x16x4f32(sX[(16 * I + r16) * ldx + 16 * I + m + k4], yb[(m + k4) * 17 + r16], x, 0, 0, 0);
+      for (int t = 0; t < 4; ++t) x = __builtin_amdgcn_mfma_f32_16x16x4f32(xd[t], yv[t], x, 0, 0, 0);
 #pragma unroll
       for (int i = 0; i < 4; ++i) sX[(16 * I + 4 * k4 + i) * ldx + 16 * J + r16] = -x[i];
     }
