@@ -505,13 +505,19 @@ __device__ __forceinline__ float scalar_from_raw(uint32_t raw, int dtype) {
 }
 
 // inclusive prefix sum across the 64 lanes of a wavefront
+// (data-parallel-primitive moves on the vector ALU: shifts by 1, 2, 4, 8 inside each row of 16 lanes, then
+// the last lane of rows 0 and 2 into rows 1 and 3, then lane 31 into rows 2 and 3; six exchanges through the
+// LDS crossbar cost about 0.2 us on a chain that has nothing else to do)
+template <int CTRL, int ROWS> __device__ __forceinline__ float dpp_or_zero(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, ROWS, 0xf, false));
+}
 __device__ __forceinline__ float wave_incl_scan(float x) {
-  const int l = lane_id();
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    float y = __shfl_up(x, d, 64);
-    if (l >= d) x += y;
-  }
+  x += dpp_or_zero<0x111, 0xf>(x);      // row_shr:1
+  x += dpp_or_zero<0x112, 0xf>(x);      // row_shr:2
+  x += dpp_or_zero<0x114, 0xf>(x);      // row_shr:4
+  x += dpp_or_zero<0x118, 0xf>(x);      // row_shr:8
+  x += dpp_or_zero<0x142, 0xa>(x);      // row_bcast:15 into rows 1 and 3
+  x += dpp_or_zero<0x143, 0xc>(x);      // row_bcast:31 into rows 2 and 3
   return x;
 }
 // inclusive suffix sum (reverse cumulative sum) across the 64 lanes
