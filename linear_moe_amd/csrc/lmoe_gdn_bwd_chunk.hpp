@@ -242,7 +242,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
     auto store_dv = [&](const ChunkInfo& ci, int h, int s) {
       typename IOV::Regs r;
       IOV::load_lds_clamped(r, s_dv[s % L::NDV], LDV, ci.len, tid);
-      IOV::store_global_clamped(r, row_ptr<T>(a.dv, ci.b, ci.tok, h) + s * BVH, a.dv.st, ci.len, tid);
+      IOV::template store_global_clamped<true>(r, row_ptr<T>(a.dv, ci.b, ci.tok, h) + s * BVH, a.dv.st, ci.len, tid);
     };
     auto close_hdh = [&]() {
       hdh = wave_sum(hdh);
@@ -291,7 +291,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
       {
         typename IOK::Regs r;
         IOK::load_lds_clamped(r, smem + B_Q, LDK, ci.len, tid);
-        IOK::store_global_clamped(r, row_ptr<T>(a.dq, ci.b, ci.tok, h), a.dq.st, ci.len, tid);
+        IOK::template store_global_clamped<true>(r, row_ptr<T>(a.dq, ci.b, ci.tok, h), a.dq.st, ci.len, tid);
       }
       lds_barrier();                                                                     // e
       lds_barrier();                                                                     // f: Tinv of this item is dead
@@ -303,7 +303,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
       {
         typename IOK::Regs r;
         IOK::load_lds_clamped(r, smem + B_Q, LDK, ci.len, tid);
-        IOK::store_global_clamped(r, row_ptr<T>(a.dk, ci.b, ci.tok, h), a.dk.st, ci.len, tid);
+        IOK::template store_global_clamped<true>(r, row_ptr<T>(a.dk, ci.b, ci.tok, h), a.dk.st, ci.len, tid);
       }
       lds_barrier();                                                                     // E
       if constexpr (NBUF == 1) {

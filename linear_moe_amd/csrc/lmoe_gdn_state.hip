@@ -1,7 +1,4 @@
 // Instantiation and launch of the sequential passes of the gated delta rule.
-#ifdef LMOE_NT_STATE
-#define LMOE_NT_LD
-#endif
 #include "lmoe_launch.hpp"
 #include "lmoe_gdn_state.hpp"
 

@@ -124,7 +124,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
     auto store_result = [&](const typename IOV::Regs& r, const lmoe_tensor& dst, int c) {
       const int tok = sq.tok0 + c * CH;
       const int len = min(CH, sq.len - c * CH);
-      IOV::store_global(r, row_ptr<T>(dst, sq.b, tok, h) + v0, dst.st, len);
+      IOV::template store_global<true>(r, row_ptr<T>(dst, sq.b, tok, h) + v0, dst.st, len);
     };
 #pragma unroll
     for (int j = 0; j < LPF; ++j) issue_a(pa[j], j);
@@ -145,7 +145,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
       if constexpr (SAVE) {
         IOV::load_lds(rvn, s_vn, LDU);
         // hs[chunk][h][v0 .. v0+BV][K] <- S^T
-        IOHT::store_global(rh, (T*)a.hs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
+        IOHT::template store_global<true>(rh, (T*)a.hs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
       }
       if (c > 0) store_result(ro, a.o, c - 1);
       if constexpr (SAVE) store_result(rvn, a.vnew, c);
@@ -369,7 +369,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
     auto store_results = [&](const typename IOV::Regs& rdv, int c) {
       const int tok = sq.tok0 + c * CH;
       const int len = min(CH, sq.len - c * CH);
-      IOV::store_global(rdv, row_ptr<T>(a.dvnew, sq.b, tok, h) + v0, a.dvnew.st, len);
+      IOV::template store_global<true>(rdv, row_ptr<T>(a.dvnew, sq.b, tok, h) + v0, a.dvnew.st, len);
     };
 #pragma unroll
     for (int j = 0; j < LPF; ++j) issue_a(pa[j], j);
@@ -386,7 +386,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
       lds_barrier();                                                                     // B2
       // dv_new of this chunk is complete (the consumers rewrite it after the next B1)
       IOV::load_lds(rdv, s_dvn, LDU);
-      IOHT::store_global(rh, (T*)a.dhs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
+      IOHT::template store_global<true>(rh, (T*)a.dhs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
       store_results(rdv, c);
       issue_a(pa[j], it + LPF);
     });

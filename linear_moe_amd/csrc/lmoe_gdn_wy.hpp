@@ -312,8 +312,8 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
     typename IOV::Regs ou;
     IOK::load_lds_clamped(ow, s_k, LDK, ci.len, tid);
     IOV::load_lds_clamped(ou, s_vb, LDV, ci.len, tid);
-    IOK::store_global_clamped(ow, row_ptr<T>(a.w, ci.b, ci.tok, h), a.w.st, ci.len, tid);
-    IOV::store_global_clamped(ou, row_ptr<T>(a.u, ci.b, ci.tok, h), a.u.st, ci.len, tid);
+    IOK::template store_global_clamped<true>(ow, row_ptr<T>(a.w, ci.b, ci.tok, h), a.w.st, ci.len, tid);
+    IOV::template store_global_clamped<true>(ou, row_ptr<T>(a.u, ci.b, ci.tok, h), a.u.st, ci.len, tid);
   }
   }   // items
 }
