@@ -23,17 +23,19 @@ namespace lmoe {
 // distance d = I - J, one block per wave, on the matrix cores in fp32 (v_mfma_f32_16x16x4_f32):
 //   Y = sum_{M = J}^{I-1} L_IM X_MJ   (4 d instructions),   X_IJ = - X_II Y   (4 instructions),
 // with Y passed through the wave's own scratch block, so a round needs one work-group barrier.
-// Must be called by all 256 threads (l, tid: lane and thread index); sL must be complete (barrier
-// before the call).
+// Must be called by all 256 threads (l, tid: lane and thread index); sL must be complete and sX free
+// (barrier before the call).
 __device__ __forceinline__ void tri_inverse_64(const float* sL, int ldl, float* sX, int ldx, float* sY, int l, int tid) {
   const int wv = wave_id();
   // clear X (upper blocks stay zero)
+  // the six blocks above the diagonal are zero; nothing else writes them, so no barrier before the rest
+  {
+    const int r = tid >> 4, c = tid & 15;
 #pragma unroll
-  for (int p = 0; p < CH * CH / NTHR; ++p) {
-    const int idx = p * NTHR + tid;
-    sX[(idx >> 6) * ldx + (idx & 63)] = 0.f;
+    for (int I = 0; I < 3; ++I)
+#pragma unroll
+      for (int J = I + 1; J < 4; ++J) sX[(16 * I + r) * ldx + 16 * J + c] = 0.f;
   }
-  lds_barrier();
   if (l < 16) {
     // lane c solves column c by forward substitution; every lane reads the same coefficients (broadcast
     // reads of whole rows).  The rows are requested in three batches ahead of their use: reading each
@@ -127,7 +129,8 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
   __shared__ __attribute__((aligned(16))) float s_L[CH * LDC];   // L, later Tinv in element type T
   __shared__ __attribute__((aligned(16))) float s_X[CH * LDC];
   __shared__ float s_Y[4 * 272];
-  __shared__ float s_b[64], s_beta[64], s_beb[64];
+  __shared__ __attribute__((aligned(16))) float s_b[64];
+  __shared__ float s_beta[64], s_beb[64];
   // Tinv as an MFMA operand: fp32 uses s_X in place, bf16 a copy in the (dead) L tile
   T* s_Tm = sizeof(T) == 4 ? (T*)s_X : (T*)s_L;
 
@@ -227,34 +230,29 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
       for (int nj = 0; nj < 4; ++nj) {
         if (nj <= wv) {
           const typename ET<T>::frag bk = ET<T>::load_frag(s_k + (16 * nj + fr) * LDK + 32 * ks + fg);
-          ET<T>::mma(m[nj], ak, bk);
-          ET<T>::mma(pm[nj], fq.f[ks], bk);
+          ET<T>::mma(m[nj], bk, ak);          // transposed: a lane holds four consecutive columns of one row
+          ET<T>::mma(pm[nj], bk, fq.f[ks]);
         }
       }
     }
     issue_q(nxt);
-    float br[4], betar[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      br[i] = s_b[16 * wv + 4 * (l >> 4) + i];
-      betar[i] = s_beta[16 * wv + 4 * (l >> 4) + i];
-    }
+    const int r = 16 * wv + fr;
+    const float br = s_b[r], betar = s_beta[r];
 #pragma unroll
     for (int nj = 0; nj < 4; ++nj) {
       f32x4 pl = {0.f, 0.f, 0.f, 0.f}, pp = {0.f, 0.f, 0.f, 0.f};
       if (nj <= wv) {
-        const int cc = 16 * nj + fr;
-        const float bc = s_b[cc];
+        const int cc0 = 16 * nj + 4 * (l >> 4);
+        const f32x4 bc = *(const f32x4*)(s_b + cc0);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int r = 16 * wv + 4 * (l >> 4) + i;
-          const float e = texp<T>(br[i] - bc);
-          pl[i] = (r > cc) ? betar[i] * m[nj][i] * e : 0.f;
-          pp[i] = (r >= cc) ? pm[nj][i] * e : 0.f;
+          const float e = texp<T>(br - bc[i]);
+          pl[i] = (r > cc0 + i) ? betar * m[nj][i] * e : 0.f;
+          pp[i] = (r >= cc0 + i) ? pm[nj][i] * e : 0.f;
         }
       }
-      acc_to_lds<float>(pl, s_L, LDC, 16 * wv, 16 * nj, l);
-      acc_to_lds<T>(pp, s_P, LDC, 16 * wv, 16 * nj, l);
+      acc_to_lds_t<float>(pl, s_L, LDC, 16 * nj, 16 * wv, l);      // s_L[r][cc0 ..]: one 16-byte write
+      acc_to_lds_t<T>(pp, s_P, LDC, 16 * nj, 16 * wv, l);
     }
     lds_barrier();
     IO64::lds_to_global(s_P, LDC, pg, CH, CH, tid);
