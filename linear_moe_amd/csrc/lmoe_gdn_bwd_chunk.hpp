@@ -257,16 +257,22 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
       if constexpr (NBUF == 3) {
         // window w: the compute team works on slice w.  Slice s lives in buffer s % 3 and is staged two
         // windows ahead; q, k go to the third buffer's region in the last window.
+        // In every window the loaders fill LDS first and meet the compute team at the barrier; the requests
+        // that refill the freed registers follow the barrier.  Requests stall at the issue while the CU's
+        // queue is full (32 KB take about a microsecond): issued before the barrier, that stall held up
+        // the compute team in five windows of twelve (a quarter of the item, traced per barrier).
         static_for<NS>([&](auto wc) {
           constexpr int w = decltype(wc)::value;
           if constexpr (w >= 1) store_dv(ci, h, w - 1);
-          if constexpr (w + 2 < NS) advance(IC<w + 2>(), it, (w + 2) % 3);
+          if constexpr (w + 2 < NS) stage(IC<w + 2>(), (w + 2) % 3);
           if constexpr (w == NS - 1) {
-            advance(IC<NS>(), it, 0);                                                    // q
-            advance(IC<NS + 1>(), it, 0);                                                // k
+            stage(IC<NS>(), 0);                                                          // q
+            stage(IC<NS + 1>(), 0);                                                      // k
             close_hdh();
           }
           lds_barrier();                                                                 // D(w); the last one is A
+          if constexpr (w + 2 < NS) issue(IC<w + 2 + DEPTH>(), it);
+          if constexpr (w == NS - 1) issue(IC<NS + DEPTH>(), it);                        // slice 0 of the next item
         });
         store_dv(ci, h, NS - 1);
       } else {
@@ -283,6 +289,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
         lds_barrier();                                                                   // A
       }
       lds_barrier();                                                                     // b
+      if constexpr (NBUF == 3) issue(IC<NS + 1 + DEPTH>(), it);                          // slice 1 of the next item
       issue_tinv(it + stride);
       stage_gates(par ^ 1);                                    // the next item's; its copy is idle since E of the last item
       issue_gates(it + 2 * stride);
@@ -296,10 +303,14 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
       lds_barrier();                                                                     // e
       lds_barrier();                                                                     // f: Tinv of this item is dead
       IO64::store_lds(rt, s_ti, LDC, tid);
-      if constexpr (NBUF == 3) advance(IC<NU>(), it, 0);       // slice 0 of the next item
+      if constexpr (NBUF == 3) stage(IC<NU>(), 0);             // slice 0 of the next item
       lds_barrier();                                                                     // g
-      if constexpr (NBUF == 3) advance(IC<NU + 1>(), it, 1);   // slice 1 of the next item
+      if constexpr (NBUF == 3) {
+        issue(IC<NU + DEPTH>(), it);                           // slice 2 of the next item
+        stage(IC<NU + 1>(), 1);                                // slice 1 of the next item
+      }
       lds_barrier();                                                                     // h: dk lies in the q tile
+      if constexpr (NBUF == 3) issue(IC<NU + 1 + DEPTH>(), it);                          // slice 3 of the next item
       {
         typename IOK::Regs r;
         IOK::load_lds_clamped(r, smem + B_Q, LDK, ci.len, tid);
