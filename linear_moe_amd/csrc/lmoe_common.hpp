@@ -475,11 +475,12 @@ template <typename T, int ROWS, int COLS> struct TileIO {
     }
   }
   // global[row][col] = tile[row][col]
+  template <bool STREAM = false>
   static __device__ __forceinline__ void lds_to_global(const T* tile, int ld, T* __restrict__ dst, int64_t row_stride, int nvalid, int tid = threadIdx.x & (NTHR - 1)) {
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
       int row, col; coords(p, row, col, tid);
-      if (row < ROWS && row < nvalid) *(vec*)(dst + (int64_t)row * row_stride + col) = *(const vec*)(tile + row * ld + col);
+      if (row < ROWS && row < nvalid) put<STREAM>(*(const vec*)(tile + row * ld + col), (vec*)(dst + (int64_t)row * row_stride + col));
     }
   }
 };

@@ -255,7 +255,7 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
       acc_to_lds_t<T>(pp, s_P, LDC, 16 * nj, 16 * wv, l);
     }
     lds_barrier();
-    IO64::lds_to_global(s_P, LDC, pg, CH, CH, tid);
+    IO64::template lds_to_global<true>(s_P, LDC, pg, CH, CH, tid);
   }
   // k is dead as an operand of k k^T and q k^T: scale it in place to k beta e^{b} (from the registers)
   IOK::store_lds_scaled(rk, s_k, LDK, s_beb, tid);
@@ -272,9 +272,9 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
       if constexpr (sizeof(T) == 2) {
         bf16x4 y; y[0] = (bf16)x[0]; y[1] = (bf16)x[1]; y[2] = (bf16)x[2]; y[3] = (bf16)x[3];
         *(bf16x4*)(s_Tm + r * LDC + c) = y;
-        if constexpr (SAVE) *(bf16x4*)(tg + r * CH + c) = y;
+        if constexpr (SAVE) __builtin_nontemporal_store(y, (bf16x4*)(tg + r * CH + c));
       } else {
-        if constexpr (SAVE) *(f32x4*)(tg + r * CH + c) = x;
+        if constexpr (SAVE) __builtin_nontemporal_store(x, (f32x4*)(tg + r * CH + c));
       }
     }
   }
