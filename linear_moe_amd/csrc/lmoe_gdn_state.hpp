@@ -316,13 +316,14 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
   constexpr int MB = K / 64, NB = BV / 16, KS = K / 32;
   constexpr int LPF = GdnStateCfg<T>::LPF;
   __shared__ __attribute__((aligned(16))) T s_q[CH * LDK];          // q         [64][K]
-  __shared__ __attribute__((aligned(16))) T s_w[CH * LDK];          // w         [64][K]
+  __shared__ __attribute__((aligned(16))) T s_w[CH * LDK];          // w         [64][K]: formed here, Tinv (k beta e^b)
+  __shared__ __attribute__((aligned(16))) T s_ti[CH * LDC];         // Tinv      [64][64]
   __shared__ __attribute__((aligned(16))) T s_k[CH * LDK];          // k         [64][K]
   __shared__ __attribute__((aligned(16))) T s_p[CH * LDC];          // P         [64][64]
   __shared__ __attribute__((aligned(16))) T s_do[CH * LDU];         // do        [64][BV]
   __shared__ __attribute__((aligned(16))) T s_dST[BV * LDK];        // dS'^T     [BV][K]
   __shared__ __attribute__((aligned(16))) T s_dvn[CH * LDU];        // dv_new    [64][BV] (MFMA operand through transposing reads, and stored)
-  __shared__ __attribute__((aligned(16))) float s_qs[2][64], s_ed[2][64];
+  __shared__ __attribute__((aligned(16))) float s_qs[2][64], s_ed[2][64], s_f[64];   // s_f = beta e^{b} (read in phase 1 only: one copy)
   __shared__ float s_dec[2];                                        // gate arrays: buffer it & 1
 
   constexpr int NVS = V / BV;
@@ -349,8 +350,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
   typedef TileIO<T, BV, K> IOHT;
 
   if (team == 1) {
-    // ------------------------- loaders, ring A (q, w) and all stores ----------------------
-    struct PreA { typename IOK::Regs rq, rw; int len; };
+    // ------------------------- loaders, ring A (q) and all stores -------------------------
+    struct PreA { typename IOK::Regs rq; int len; };
     PreA pa[LPF];
     // always issued, chunk index clamped (see k_gdn_state_fwd); `it` counts chunks from the end
     auto issue_a = [&](PreA& P, int it) {
@@ -358,13 +359,10 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
       const int tok = sq.tok0 + c * CH;
       P.len = min(CH, sq.len - c * CH);
       IOK::load_nomask(P.rq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, P.len);
-      IOK::load_nomask(P.rw, row_ptr<T>(a.w, sq.b, tok, h), a.w.st, P.len);
     };
     auto stage_a = [&](PreA& P) {
       IOK::mask(P.rq, P.len);
-      IOK::mask(P.rw, P.len);
       IOK::store_lds(P.rq, s_q, LDK);
-      IOK::store_lds(P.rw, s_w, LDK);
     };
     auto store_results = [&](const typename IOV::Regs& rdv, int c) {
       const int tok = sq.tok0 + c * CH;
@@ -394,9 +392,9 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
     return;
   }
   if (team == 2) {
-    // ------------------------- loaders, ring B (k, P, do, decay table) ------------------
+    // ------------------------- loaders, ring B (k, P, Tinv, do, decay table, beta) ------
     // staged during phase 2 of the step before the one that reads them in phase 1
-    struct PreB { typename IOK::Regs rk; typename IOP::Regs rp; typename IOV::Regs rd; float eb, ed; int len; };
+    struct PreB { typename IOK::Regs rk; typename IOP::Regs rp, rt; typename IOV::Regs rd; float eb, ed; uint32_t braw; int len; };
     PreB pb[LPF];
     const float scale = a.scale;
     auto issue_b = [&](PreB& P, int it) {
@@ -405,7 +403,9 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
       P.len = min(CH, sq.len - c * CH);
       IOK::load_nomask(P.rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, P.len);
       IOP::load_nomask(P.rp, (const T*)a.pmat + ((int64_t)(sq.chunk0 + c) * a.H + h) * CH * CH, CH, CH);
+      IOP::load_nomask(P.rt, (const T*)a.tinv + ((int64_t)(sq.chunk0 + c) * a.H + h) * CH * CH, CH, CH);
       IOV::load_nomask(P.rd, row_ptr<T>(a.d_o, sq.b, tok, h) + v0, a.d_o.st, P.len);
+      P.braw = load_scalar_raw(a.beta.ptr, a.beta_dtype, row_off(a.beta, sq.b, tok + min(l, P.len - 1), h));
       const float* gc = a.gcum + ((int64_t)(sq.chunk0 + c) * a.H + h) * 2 * CH;
       P.eb = gc[l];
       P.ed = gc[CH + l];
@@ -415,8 +415,10 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
       IOV::mask(P.rd, P.len);
       IOK::store_lds(P.rk, s_k, LDK);
       IOP::store_lds(P.rp, s_p, LDC);       // rows and columns past the end are zero as written
+      IOP::store_lds(P.rt, s_ti, LDC);
       IOV::store_lds(P.rd, s_do, LDU);
       if (wave_id() == 8) {
+        s_f[l] = l < P.len ? scalar_from_raw(P.braw, a.beta_dtype) * P.eb : 0.f;
         s_qs[buf][l] = scale * P.eb;
         s_ed[buf][l] = P.ed;
         if (l == 63) s_dec[buf] = P.eb;
@@ -466,6 +468,25 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
     lds_barrier();                                                                       // B1
     // t = (k dS')^T  and  dv_loc = (P^T do)^T for the tokens 16 wv .. of the chunk: formed transposed,
     // so that a lane holds four consecutive V columns of one token (see k_gdn_state_fwd)
+    // w = Tinv (k beta e^{b}) is not read from memory (16 KB per chunk and work-group through a request queue
+    // that bounds this kernel) but formed here: wave w forms rows 16 w .. from Tinv (8 KB, its columns scaled
+    // by beta e^{b}) and the k tile, transposed (8-byte LDS writes); phase 2 reads the whole tile after B2.
+    {
+      f32x4 wacc[K / 16];
+#pragma unroll
+      for (int ni = 0; ni < K / 16; ++ni) wacc[ni] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < CH / 32; ++ks) {
+        if (ks == 0 || wv >= 2) {            // Tinv is lower triangular
+          typename ET<T>::frag bt = ET<T>::load_frag(s_ti + (16 * wv + fr) * LDC + 32 * ks + fg);
+          scale_frag8<T>(bt, &s_f[32 * ks + fg]);
+#pragma unroll
+          for (int ni = 0; ni < K / 16; ++ni) ET<T>::mma(wacc[ni], ET<T>::load_frag_t(s_k, LDK, 32 * ks, 16 * ni), bt);
+        }
+      }
+#pragma unroll
+      for (int ni = 0; ni < K / 16; ++ni) acc_to_lds_t<T>(wacc[ni], s_w, LDK, 16 * ni, 16 * wv);
+    }
     f32x4 t[1][NB], dvl[1][NB];
     acc_zero(t);
     acc_zero(dvl);
