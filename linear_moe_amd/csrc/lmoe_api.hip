@@ -128,9 +128,10 @@ int lmoe_chunk_gated_delta_rule_fwd(const lmoe_args* a, void* stream) {
   if (!a->beta.ptr) return fail(-12, "%s: beta must not be null", op);
   if (!a->o.ptr || !a->w.ptr || !a->u.ptr || !a->pmat || !a->gcum)
     return fail(-11, "%s: o, w, u, pmat and gcum must not be null", op);
-  // what only the backward reads: all three, or none (a forward-only call)
-  if ((a->hs != nullptr) != (a->vnew.ptr != nullptr) || (a->hs != nullptr) != (a->tinv != nullptr))
-    return fail(-11, "%s: hs, vnew and tinv must be given together (or all be null: forward only)", op);
+  // what only the backward reads: hs and vnew together or not at all (a forward-only call); tinv goes with
+  // them, and may also be given alone (the state pass then forms w from it instead of reading w)
+  if ((a->hs != nullptr) != (a->vnew.ptr != nullptr) || (a->hs != nullptr && a->tinv == nullptr))
+    return fail(-11, "%s: hs and vnew must be given together, and tinv with them (all null: forward only)", op);
   if (a->NT == 0 || a->N == 0) return 0;
   lmoe::launch_gdn_wy_fwd(*a, (hipStream_t)stream);
   lmoe::launch_gdn_state_fwd(*a, (hipStream_t)stream);

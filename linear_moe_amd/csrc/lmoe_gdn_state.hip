@@ -13,8 +13,16 @@ template <typename T, int V> inline bool wide_slices(const lmoe_args& a) {
 }
 template <typename T, int K, int V, int BV> void launch_fwd(const lmoe_args& a, hipStream_t st) {
   const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BV);
-  if (a.hs) hipLaunchKernelGGL((k_gdn_state_fwd<T, K, V, BV, true>), dim3(grid), dim3(3 * NTHR), 0, st, a);
-  else hipLaunchKernelGGL((k_gdn_state_fwd<T, K, V, BV, false>), dim3(grid), dim3(3 * NTHR), 0, st, a);
+  // w formed on the chip from Tinv where Tinv is there and LDS has room for a second k tile
+  constexpr bool CAN_WT = sizeof(T) == 2;
+  const bool wt = CAN_WT && a.tinv != nullptr;
+  if (a.hs) {
+    if (wt) hipLaunchKernelGGL((k_gdn_state_fwd<T, K, V, BV, true, CAN_WT>), dim3(grid), dim3(3 * NTHR), 0, st, a);
+    else hipLaunchKernelGGL((k_gdn_state_fwd<T, K, V, BV, true, false>), dim3(grid), dim3(3 * NTHR), 0, st, a);
+  } else {
+    if (wt) hipLaunchKernelGGL((k_gdn_state_fwd<T, K, V, BV, false, CAN_WT>), dim3(grid), dim3(3 * NTHR), 0, st, a);
+    else hipLaunchKernelGGL((k_gdn_state_fwd<T, K, V, BV, false, false>), dim3(grid), dim3(3 * NTHR), 0, st, a);
+  }
 }
 template <typename T, int K, int V, int BV> void launch_bwd(const lmoe_args& a, hipStream_t st) {
   const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BV);

@@ -61,13 +61,21 @@ template <int L, typename F> __device__ __forceinline__ void ring_loop(int n, F&
 //   (team 1 lifts v_new(c) right after B2 and stores it in the same half-step)
 // ------------------------------------------------------------------------- //
 // SAVE = false (forward-only call): hs and v_new, which only the backward reads, are not written
-template <typename T, int K, int V, int BV, bool SAVE>
+template <typename T, int K, int V, int BV, bool SAVE, bool WT>
 __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
   constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDU = BV + LPAD;
   constexpr int MB = K / 64, NB = BV / 16, KS = K / 32;
   constexpr int LPF = GdnStateCfg<T>::LPF;
-  __shared__ __attribute__((aligned(16))) T s_k[CH * LDK];          // k             [64][K]
+  // WT: w = Tinv (k beta e^{b}) is not read from memory (16 KB per chunk and work-group through a request
+  // queue that bounds this kernel) but formed on the chip: during phase 2 of chunk c consumer wave w forms
+  // rows 16 w .. of w(c+1) from Tinv(c+1) (8 KB, columns scaled by beta e^{b}) and k(c+1), which the loaders
+  // then stage one chunk early into the second of two k tiles.  WT = false (fp32: LDS has no room for that;
+  // or no Tinv given): w is read as written by the WY preparation.
+  static_assert(!WT || sizeof(T) == 2, "the second k tile fits for 2-byte elements only");
+  __shared__ __attribute__((aligned(16))) T s_k[(WT ? 2 : 1) * CH * LDK];   // k          [64][K] (WT: of chunks c, c + 1)
   __shared__ __attribute__((aligned(16))) T s_w[CH * LDK];          // w             [64][K]
+  __shared__ __attribute__((aligned(16))) T s_ti[WT ? CH * LDC : 8];   // Tinv       [64][64]
+  __shared__ __attribute__((aligned(16))) float s_f[64];            // beta e^{b} of the chunk whose w is formed
   __shared__ __attribute__((aligned(16))) T s_q[CH * LDK];          // q             [64][K]
   __shared__ __attribute__((aligned(16))) T s_p[CH * LDC];          // P             [64][64]
   __shared__ __attribute__((aligned(16))) T s_u[CH * LDU];          // u             [64][BV]
@@ -103,7 +111,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
 
   if (team == 1) {
     // ------------------------- loaders, ring A (k, P) and all stores ----------------------
-    struct PreA { typename IOK::Regs rk; typename IOP::Regs rp; int len; };
+    struct PreA { typename IOK::Regs rk; typename IOP::Regs rp, rt; uint32_t braw; float eb; int len; };
     PreA pa[LPF];
     // Always issued (chunk index clamped to the last chunk; the surplus loads at the end of a
     // sequence are never consumed): a prefetch that is skipped on some path would make the
@@ -114,11 +122,24 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
       P.len = min(CH, sq.len - c * CH);
       IOK::load_nomask(P.rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, P.len);
       IOP::load_nomask(P.rp, (const T*)a.pmat + ((int64_t)(sq.chunk0 + c) * a.H + h) * CH * CH, CH, CH);
+      if constexpr (WT) {
+        IOP::load_nomask(P.rt, (const T*)a.tinv + ((int64_t)(sq.chunk0 + c) * a.H + h) * CH * CH, CH, CH);
+        P.braw = load_scalar_raw(a.beta.ptr, a.beta_dtype, row_off(a.beta, sq.b, tok + min(l, P.len - 1), h));
+        P.eb = a.gcum[((int64_t)(sq.chunk0 + c) * a.H + h) * 2 * CH + l];
+      }
     };
     auto stage_a = [&](PreA& P) {
       IOK::mask(P.rk, P.len);
       IOK::store_lds(P.rk, s_k, LDK);
       IOP::store_lds(P.rp, s_p, LDC);       // rows and columns past the end are zero as written
+    };
+    // WT: P of chunk c for its phase 2; k, Tinv, beta e^{b} of chunk c + 1 for the w the consumers form then
+    auto stage_p = [&](PreA& P) { IOP::store_lds(P.rp, s_p, LDC); };
+    auto stage_k = [&](PreA& P, int c) {
+      IOK::mask(P.rk, P.len);
+      IOK::store_lds(P.rk, s_k + (c & 1) * CH * LDK, LDK);
+      IOP::store_lds(P.rt, s_ti, LDC);
+      if (wave_id() == 4) s_f[l] = l < P.len ? scalar_from_raw(P.braw, a.beta_dtype) * P.eb : 0.f;
     };
     // a result tile of chunk c: registers -> global
     auto store_result = [&](const typename IOV::Regs& r, const lmoe_tensor& dst, int c) {
@@ -131,12 +152,21 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
     // the first loads may be ordered freely by the compiler; were they still pending at the loop
     // header, its wait-count analysis would carry that order into every iteration
     wait_all_loads();
+    if constexpr (WT) {
+      stage_k(pa[0], 0);
+      lds_barrier();                                                                     // B0: the consumers form w(0)
+    }
     typename IOHT::Regs rh;
     typename IOV::Regs rvn, ro;
     ring_loop<LPF>(sq.nchunks, [&](auto slot, const int c) {
-      constexpr int j = decltype(slot)::value;
+      constexpr int j = decltype(slot)::value, jn = (j + 1) % LPF;
       lds_barrier();                                                                     // B1
-      stage_a(pa[j]);
+      if constexpr (WT) {
+        stage_p(pa[j]);
+        stage_k(pa[jn], c + 1);             // (past the last chunk: a clamped copy of it, never used)
+      } else {
+        stage_a(pa[j]);
+      }
       // S^T and the previous chunk's o leave LDS now (the consumers rewrite them after B2)
       if constexpr (SAVE) IOHT::load_lds(rh, s_hT, LDK);
       IOV::load_lds(ro, s_o, LDU);
@@ -159,13 +189,13 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
   if (team == 2) {
     // ------------------------- loaders, ring B (w, q, u, decay table) ---------------------
     // staged during phase 2 of the step before the one that reads them in phase 1
-    struct PreB { typename IOK::Regs rw, rq; typename IOV::Regs ru; float eb, ed; int len; };
+    struct PreB { typename IOK::Regs rw, rq; typename IOV::Regs ru; float eb, ed; int len; };   // rw unused with WT
     PreB pb[LPF];
     auto issue_b = [&](PreB& P, int c) {
       c = min(c, sq.nchunks - 1);
       const int tok = sq.tok0 + c * CH;
       P.len = min(CH, sq.len - c * CH);
-      IOK::load_nomask(P.rw, row_ptr<T>(a.w, sq.b, tok, h), a.w.st, P.len);
+      if constexpr (!WT) IOK::load_nomask(P.rw, row_ptr<T>(a.w, sq.b, tok, h), a.w.st, P.len);
       IOK::load_nomask(P.rq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, P.len);
       IOV::load_nomask(P.ru, row_ptr<T>(a.u, sq.b, tok, h) + v0, a.u.st, P.len);
       const float* gc = a.gcum + ((int64_t)(sq.chunk0 + c) * a.H + h) * 2 * CH;
@@ -173,9 +203,11 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
       P.ed = gc[CH + l];
     };
     auto stage_b = [&](PreB& P, int buf) {
-      IOK::mask(P.rw, P.len);
+      if constexpr (!WT) {
+        IOK::mask(P.rw, P.len);
+        IOK::store_lds(P.rw, s_w, LDK);
+      }
       IOV::mask(P.ru, P.len);
-      IOK::store_lds(P.rw, s_w, LDK);
       IOK::store_lds(P.rq, s_q, LDK);       // rows past the end only reach output rows that are not stored
       IOV::store_lds(P.ru, s_u, LDU);
       if (wave_id() == 8) {
@@ -188,6 +220,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
     for (int j = 0; j < LPF; ++j) issue_b(pb[j], j);
     stage_b(pb[0], 0);
     wait_all_loads();   // see ring A
+    if constexpr (WT) lds_barrier();                                                     // B0
     ring_loop<LPF>(sq.nchunks, [&](auto slot, const int c) {
       constexpr int j = decltype(slot)::value, jn = (j + 1) % LPF;
       lds_barrier();                                                                     // B1
@@ -219,8 +252,31 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
         for (int i = 0; i < 4; ++i)
           S[mi][ni][i] = h0[(int64_t)(krow0 + acc_row(mi, i)) * V + v0 + acc_col(ni)];
   }
+  // rows 16 wv .. of w(c) into the w tile (read back by this wave only, after the next barrier)
+  auto form_w = [&](int c) {
+    const T* kt = s_k + (c & 1) * CH * LDK;
+    f32x4 wacc[K / 16];
+#pragma unroll
+    for (int ni = 0; ni < K / 16; ++ni) wacc[ni] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < CH / 32; ++ks) {
+      if (ks == 0 || wv >= 2) {            // Tinv is lower triangular
+        typename ET<T>::frag bt = ET<T>::load_frag(s_ti + (16 * wv + fr) * LDC + 32 * ks + fg);
+        scale_frag8<T>(bt, &s_f[32 * ks + fg]);
+#pragma unroll
+        for (int ni = 0; ni < K / 16; ++ni) ET<T>::mma(wacc[ni], ET<T>::load_frag_t(kt, LDK, 32 * ks, 16 * ni), bt);
+      }
+    }
+#pragma unroll
+    for (int ni = 0; ni < K / 16; ++ni) acc_to_lds_t<T>(wacc[ni], s_w, LDK, 16 * ni, 16 * wv);
+  };
+  if constexpr (WT) {
+    lds_barrier();                                                                       // B0: k, Tinv of chunk 0 staged
+    form_w(0);
+  }
   for (int c = 0; c < sq.nchunks; ++c) {
     const int cur = c & 1;
+    const T* s_kc = s_k + (WT ? cur * CH * LDK : 0);
     // S (state at chunk start) -> LDS as S^T
 #pragma unroll
     for (int mi = 0; mi < MB; ++mi)
@@ -271,7 +327,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
       typename ET<T>::frag af[MB], bv[NB];
       const typename ET<T>::frag ap = ET<T>::load_frag(s_p + (16 * wv + fr) * LDC + 32 * ks + fg);
 #pragma unroll
-      for (int mi = 0; mi < MB; ++mi) af[mi] = ET<T>::load_frag_t(s_k, LDK, 32 * ks, krow0 + 16 * mi);
+      for (int mi = 0; mi < MB; ++mi) af[mi] = ET<T>::load_frag_t(s_kc, LDK, 32 * ks, krow0 + 16 * mi);
 #pragma unroll
       for (int ni = 0; ni < NB; ++ni) {
         bv[ni] = ET<T>::load_frag_t(s_vn, LDU, 32 * ks, 16 * ni);       // rows: V columns, contraction: tokens
@@ -289,6 +345,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
       o[0][ni] *= scale;
       acc_to_lds_t<T>(o[0][ni], s_o, LDU, 16 * ni, 16 * wv);         // s_o[token][v]
     }
+    if constexpr (WT) form_w(c + 1);         // off the chain: the loaders' requests bound this window
   }
   lds_barrier();                                                                         // results of the last chunk
   if (a.ht) {

@@ -64,7 +64,8 @@ class GDNCall:
         o = torch.empty_like(v)
         ht = torch.empty(plan.N, H, K, V, dtype=torch.float32, device=dev) if output_final_state else None
         hs = torch.empty(max(plan.NT, 1), H, K, V, dtype=dt, device=dev) if save else None
-        tinv = torch.empty(max(plan.NT, 1), H, 64, 64, dtype=dt, device=dev) if save else None
+        # always: the backward reads it, and the forward state pass forms w from it (8 KB per chunk and head)
+        tinv = torch.empty(max(plan.NT, 1), H, 64, 64, dtype=dt, device=dev)
         pmat = torch.empty(max(plan.NT, 1), H, 64, 64, dtype=dt, device=dev)
         gcum = torch.empty(max(plan.NT, 1), H, 2, 64, dtype=torch.float32, device=dev)
         w = torch.empty(B, T, H, K, dtype=dt, device=dev)
