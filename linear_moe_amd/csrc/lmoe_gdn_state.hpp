@@ -66,8 +66,9 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
   constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDU = BV + LPAD;
   constexpr int MB = K / 64, NB = BV / 16, KS = K / 32;
   constexpr int LPF = GdnStateCfg<T>::LPF;
-  // WT: w = Tinv (k beta e^{b}) is not read from memory (16 KB per chunk and work-group through a request
-  // queue that bounds this kernel) but formed on the chip: during phase 2 of chunk c consumer wave w forms
+  // WT: w = Tinv (k beta e^{b}) and u = Tinv (v beta) are not read from memory (w: 16 KB per chunk and work-group
+  // through a request queue that bounds this kernel; neither is then written by the WY preparation) but formed on
+  // the chip: during phase 2 of chunk c consumer wave w forms
   // rows 16 w .. of w(c+1) from Tinv(c+1) (8 KB, columns scaled by beta e^{b}) and k(c+1), which the loaders
   // then stage one chunk early into the second of two k tiles.  WT = false (fp32: LDS has no room for that;
   // or no Tinv given): w is read as written by the WY preparation.
@@ -75,7 +76,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
   __shared__ __attribute__((aligned(16))) T s_k[(WT ? 2 : 1) * CH * LDK];   // k          [64][K] (WT: of chunks c, c + 1)
   __shared__ __attribute__((aligned(16))) T s_w[CH * LDK];          // w             [64][K]
   __shared__ __attribute__((aligned(16))) T s_ti[WT ? CH * LDC : 8];   // Tinv       [64][64]
-  __shared__ __attribute__((aligned(16))) float s_f[64];            // beta e^{b} of the chunk whose w is formed
+  __shared__ __attribute__((aligned(16))) T s_v[WT ? CH * LDU : 8];    // v          [64][BV] of the chunk whose u is formed
+  __shared__ __attribute__((aligned(16))) float s_f[64], s_be[64];  // beta e^{b}, beta of the chunk whose w, u are formed
   __shared__ __attribute__((aligned(16))) T s_q[CH * LDK];          // q             [64][K]
   __shared__ __attribute__((aligned(16))) T s_p[CH * LDC];          // P             [64][64]
   __shared__ __attribute__((aligned(16))) T s_u[CH * LDU];          // u             [64][BV]
@@ -111,7 +113,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
 
   if (team == 1) {
     // ------------------------- loaders, ring A (k, P) and all stores ----------------------
-    struct PreA { typename IOK::Regs rk; typename IOP::Regs rp, rt; uint32_t braw; float eb; int len; };
+    struct PreA { typename IOK::Regs rk; typename IOP::Regs rp, rt; typename IOV::Regs rv; uint32_t braw; float eb; int len; };
     PreA pa[LPF];
     // Always issued (chunk index clamped to the last chunk; the surplus loads at the end of a
     // sequence are never consumed): a prefetch that is skipped on some path would make the
@@ -124,6 +126,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
       IOP::load_nomask(P.rp, (const T*)a.pmat + ((int64_t)(sq.chunk0 + c) * a.H + h) * CH * CH, CH, CH);
       if constexpr (WT) {
         IOP::load_nomask(P.rt, (const T*)a.tinv + ((int64_t)(sq.chunk0 + c) * a.H + h) * CH * CH, CH, CH);
+        IOV::load_nomask(P.rv, row_ptr<T>(a.v, sq.b, tok, h) + v0, a.v.st, P.len);
         P.braw = load_scalar_raw(a.beta.ptr, a.beta_dtype, row_off(a.beta, sq.b, tok + min(l, P.len - 1), h));
         P.eb = a.gcum[((int64_t)(sq.chunk0 + c) * a.H + h) * 2 * CH + l];
       }
@@ -133,13 +136,19 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
       IOK::store_lds(P.rk, s_k, LDK);
       IOP::store_lds(P.rp, s_p, LDC);       // rows and columns past the end are zero as written
     };
-    // WT: P of chunk c for its phase 2; k, Tinv, beta e^{b} of chunk c + 1 for the w the consumers form then
+    // WT: P of chunk c for its phase 2; k, Tinv, v, beta, beta e^{b} of chunk c + 1 for the w, u the consumers form then
     auto stage_p = [&](PreA& P) { IOP::store_lds(P.rp, s_p, LDC); };
     auto stage_k = [&](PreA& P, int c) {
       IOK::mask(P.rk, P.len);
       IOK::store_lds(P.rk, s_k + (c & 1) * CH * LDK, LDK);
       IOP::store_lds(P.rt, s_ti, LDC);
-      if (wave_id() == 4) s_f[l] = l < P.len ? scalar_from_raw(P.braw, a.beta_dtype) * P.eb : 0.f;
+      IOV::mask(P.rv, P.len);
+      IOV::store_lds(P.rv, s_v, LDU);
+      if (wave_id() == 4) {
+        const float be = l < P.len ? scalar_from_raw(P.braw, a.beta_dtype) : 0.f;
+        s_be[l] = be;
+        s_f[l] = be * P.eb;
+      }
     };
     // a result tile of chunk c: registers -> global
     auto store_result = [&](const typename IOV::Regs& r, const lmoe_tensor& dst, int c) {
@@ -197,7 +206,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
       P.len = min(CH, sq.len - c * CH);
       if constexpr (!WT) IOK::load_nomask(P.rw, row_ptr<T>(a.w, sq.b, tok, h), a.w.st, P.len);
       IOK::load_nomask(P.rq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, P.len);
-      IOV::load_nomask(P.ru, row_ptr<T>(a.u, sq.b, tok, h) + v0, a.u.st, P.len);
+      if constexpr (!WT) IOV::load_nomask(P.ru, row_ptr<T>(a.u, sq.b, tok, h) + v0, a.u.st, P.len);
       const float* gc = a.gcum + ((int64_t)(sq.chunk0 + c) * a.H + h) * 2 * CH;
       P.eb = gc[l];
       P.ed = gc[CH + l];
@@ -207,9 +216,11 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
         IOK::mask(P.rw, P.len);
         IOK::store_lds(P.rw, s_w, LDK);
       }
-      IOV::mask(P.ru, P.len);
       IOK::store_lds(P.rq, s_q, LDK);       // rows past the end only reach output rows that are not stored
-      IOV::store_lds(P.ru, s_u, LDU);
+      if constexpr (!WT) {
+        IOV::mask(P.ru, P.len);
+        IOV::store_lds(P.ru, s_u, LDU);
+      }
       if (wave_id() == 8) {
         s_eb[buf][l] = P.eb;
         s_ed[buf][l] = P.ed;
@@ -252,23 +263,31 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
         for (int i = 0; i < 4; ++i)
           S[mi][ni][i] = h0[(int64_t)(krow0 + acc_row(mi, i)) * V + v0 + acc_col(ni)];
   }
-  // rows 16 wv .. of w(c) into the w tile (read back by this wave only, after the next barrier)
+  // rows 16 wv .. of w(c) and u(c) into the w and u tiles (read back by this wave only, after the next barrier)
   auto form_w = [&](int c) {
     const T* kt = s_k + (c & 1) * CH * LDK;
-    f32x4 wacc[K / 16];
+    f32x4 wacc[K / 16], uacc[NB];
 #pragma unroll
     for (int ni = 0; ni < K / 16; ++ni) wacc[ni] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ni = 0; ni < NB; ++ni) uacc[ni] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ks = 0; ks < CH / 32; ++ks) {
       if (ks == 0 || wv >= 2) {            // Tinv is lower triangular
         typename ET<T>::frag bt = ET<T>::load_frag(s_ti + (16 * wv + fr) * LDC + 32 * ks + fg);
+        typename ET<T>::frag bu = bt;
         scale_frag8<T>(bt, &s_f[32 * ks + fg]);
+        scale_frag8<T>(bu, &s_be[32 * ks + fg]);
 #pragma unroll
         for (int ni = 0; ni < K / 16; ++ni) ET<T>::mma(wacc[ni], ET<T>::load_frag_t(kt, LDK, 32 * ks, 16 * ni), bt);
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) ET<T>::mma(uacc[ni], ET<T>::load_frag_t(s_v, LDU, 32 * ks, 16 * ni), bu);
       }
     }
 #pragma unroll
     for (int ni = 0; ni < K / 16; ++ni) acc_to_lds_t<T>(wacc[ni], s_w, LDK, 16 * ni, 16 * wv);
+#pragma unroll
+    for (int ni = 0; ni < NB; ++ni) acc_to_lds_t<T>(uacc[ni], s_u, LDU, 16 * ni, 16 * wv);     // u = Tinv (v beta)
   };
   if constexpr (WT) {
     lds_barrier();                                                                       // B0: k, Tinv of chunk 0 staged

@@ -118,7 +118,9 @@ __device__ __forceinline__ void tri_inverse_64(const float* sL, int ldl, float* 
   }
 }
 
-// SAVE = false (forward-only call): Tinv, which only the backward reads, is not written
+// SAVE = false (no Tinv buffer given): Tinv is not written.  With Tinv written and 2-byte elements the
+// sequential passes form w and u on the chip from Tinv, k, v (LEAN below): neither is formed or written here and v
+// is not read.
 template <typename T, int K, int V, bool SAVE>
 __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(const lmoe_args a) {
   constexpr int LDK = K + LPAD, LDV = V + LPAD, LDC = CH + LPAD;
@@ -133,6 +135,7 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
   __shared__ float s_beta[64], s_beb[64];
   // Tinv as an MFMA operand: fp32 uses s_X in place, bf16 a copy in the (dead) L tile
   T* s_Tm = sizeof(T) == 4 ? (T*)s_X : (T*)s_L;
+  constexpr bool LEAN = SAVE && sizeof(T) == 2;
 
   const int wv = wave_id(), l = lane_id();
   typedef TileIO<T, CH, K> IOK;
@@ -157,7 +160,9 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
   // q enters only as the A operand of q k^T: each wave takes its 16 rows straight into fragments
   auto issue_q = [&](int it) { int h; const ChunkInfo ci = item_of(it, h); fq.load(row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, 16 * wv, ci.len - 1); };
   auto issue_k = [&](int it) { int h; const ChunkInfo ci = item_of(it, h); IOK::load_nomask(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len); };
-  auto issue_v = [&](int it) { int h; const ChunkInfo ci = item_of(it, h); IOV::load_nomask(rv, row_ptr<T>(a.v, ci.b, ci.tok, h), a.v.st, ci.len); };
+  auto issue_v = [&](int it) {
+    if constexpr (!LEAN) { int h; const ChunkInfo ci = item_of(it, h); IOV::load_nomask(rv, row_ptr<T>(a.v, ci.b, ci.tok, h), a.v.st, ci.len); }
+  };
   auto issue_gb = [&](int it) {
     int h; const ChunkInfo ci = item_of(it, h);
     graw = gate_prefetch(a, ci.b, ci.tok, ci.len, h);
@@ -177,7 +182,7 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
   const ChunkInfo ci = chunk_info(a, cid);
   const int nxt = it + gridDim.x;
   IOK::mask(rk, ci.len, tid);
-  IOV::mask(rv, ci.len, tid);
+  if constexpr (!LEAN) IOV::mask(rv, ci.len, tid);
   lds_barrier();      // the previous item has left every tile
   // Every wave holds the gates and beta of all 64 tokens (lane = token) and forms the cumulative gate for
   // itself: the staging below needs no value from another wave, so one barrier covers gate and staging
@@ -200,15 +205,17 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
     gc[tid & 127] = (tid & 64) ? ed : eb;
   }
   IOK::store_lds(rk, s_k, LDK, tid);
+  if constexpr (!LEAN) {
 #pragma unroll
-  for (int p = 0; p < IOV::PASSES; ++p) {       // v beta, beta of the row from the lane that holds it
-    int row, col;
-    IOV::coords(p, row, col, tid);
-    const float sc = __shfl(bl, row & 63, 64);
-    typename IOV::vec o;
+    for (int p = 0; p < IOV::PASSES; ++p) {       // v beta, beta of the row from the lane that holds it
+      int row, col;
+      IOV::coords(p, row, col, tid);
+      const float sc = __shfl(bl, row & 63, 64);
+      typename IOV::vec o;
 #pragma unroll
-    for (int i = 0; i < IOV::VEC; ++i) o[i] = ET<T>::from_f(ET<T>::to_f(rv.v[p][i]) * sc);
-    *(typename IOV::vec*)(s_vb + row * LDV + col) = o;
+      for (int i = 0; i < IOV::VEC; ++i) o[i] = ET<T>::from_f(ET<T>::to_f(rv.v[p][i]) * sc);
+      *(typename IOV::vec*)(s_vb + row * LDV + col) = o;
+    }
   }
   issue_v(nxt);
   lds_barrier();
@@ -258,7 +265,7 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
     IO64::template lds_to_global<true>(s_P, LDC, pg, CH, CH, tid);
   }
   // k is dead as an operand of k k^T and q k^T: scale it in place to k beta e^{b} (from the registers)
-  IOK::store_lds_scaled(rk, s_k, LDK, s_beb, tid);
+  if constexpr (!LEAN) IOK::store_lds_scaled(rk, s_k, LDK, s_beb, tid);
   issue_k(nxt);
   lds_barrier();   // L is complete, the P staging has been read: the inverse may overwrite X
   tri_inverse_64(s_L, LDC, s_X, LDC, s_Y, l, tid);       // barriers inside; s_L is dead afterwards
@@ -271,13 +278,14 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
       const f32x4 x = *(const f32x4*)(s_X + r * LDC + c);
       if constexpr (sizeof(T) == 2) {
         bf16x4 y; y[0] = (bf16)x[0]; y[1] = (bf16)x[1]; y[2] = (bf16)x[2]; y[3] = (bf16)x[3];
-        *(bf16x4*)(s_Tm + r * LDC + c) = y;
+        if constexpr (!LEAN) *(bf16x4*)(s_Tm + r * LDC + c) = y;
         if constexpr (SAVE) __builtin_nontemporal_store(y, (bf16x4*)(tg + r * CH + c));
       } else {
         if constexpr (SAVE) __builtin_nontemporal_store(x, (f32x4*)(tg + r * CH + c));
       }
     }
   }
+  if constexpr (!LEAN) {
   lds_barrier();
   // w = Tinv (k beta e^{b}),  u = Tinv (v beta): contraction over the rows of the [64][D] tiles.  Formed
   // transposed (the tile as the A operand through transposing LDS reads, Tinv rows as B), so that a lane
@@ -312,6 +320,7 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
     IOV::load_lds_clamped(ou, s_vb, LDV, ci.len, tid);
     IOK::template store_global_clamped<true>(ow, row_ptr<T>(a.w, ci.b, ci.tok, h), a.w.st, ci.len, tid);
     IOV::template store_global_clamped<true>(ou, row_ptr<T>(a.u, ci.b, ci.tok, h), a.u.st, ci.len, tid);
+  }
   }
   }   // items
 }
