@@ -6,7 +6,7 @@ namespace lmoe {
 
 template <typename T, int K, int V> struct GdnWyFwd {
   static void run(const lmoe_args& a, hipStream_t st) {
-        const int grid = persistent_grid(a.NT * a.H, sizeof(T) == 2 ? 2 : 1);
+        const int grid = persistent_grid(a.NT * a.H, sizeof(T) == 2 ? (a.tinv ? 3 : 2) : 1);
     if (a.tinv) hipLaunchKernelGGL((k_gdn_wy_fwd<T, K, V, true>), dim3(grid), dim3(NTHR), 0, st, a);
     else hipLaunchKernelGGL((k_gdn_wy_fwd<T, K, V, false>), dim3(grid), dim3(NTHR), 0, st, a);
   }

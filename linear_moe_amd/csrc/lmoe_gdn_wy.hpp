@@ -122,20 +122,23 @@ __device__ __forceinline__ void tri_inverse_64(const float* sL, int ldl, float* 
 // sequential passes form w and u on the chip from Tinv, k, v (LEAN below): neither is formed or written here and v
 // is not read.
 template <typename T, int K, int V, bool SAVE>
-__global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(const lmoe_args a) {
-  constexpr int LDK = K + LPAD, LDV = V + LPAD, LDC = CH + LPAD;
+__global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? (SAVE ? 3 : 2) : 1)) void k_gdn_wy_fwd(const lmoe_args a) {
+  constexpr bool LEAN = SAVE && sizeof(T) == 2;
+  // lean: three work-groups per CU (53 KB of LDS each: fp32 tiles padded by 4 instead of 8, the inverse's
+  // scratch in the k tile, which is dead by then)
+  constexpr int LDK = K + LPAD, LDV = V + LPAD, LDC = CH + (LEAN ? 4 : LPAD), LDP = CH + LPAD;
   constexpr int NBK = K / 16, NBV = V / 16;
   // k (raw, for k k^T), then overwritten in place by k beta e^{b}; v beta; both stored [64][D]
   __shared__ __attribute__((aligned(16))) T s_k[CH * LDK];
   __shared__ __attribute__((aligned(16))) T s_vb[CH * LDV];
   __shared__ __attribute__((aligned(16))) float s_L[CH * LDC];   // L, later Tinv in element type T
   __shared__ __attribute__((aligned(16))) float s_X[CH * LDC];
-  __shared__ float s_Y[4 * 272];
+  __shared__ float s_Yown[LEAN ? 4 : 4 * 272];
+  float* s_Y = LEAN ? (float*)s_k : s_Yown;
   __shared__ __attribute__((aligned(16))) float s_b[64];
   __shared__ float s_beta[64], s_beb[64];
   // Tinv as an MFMA operand: fp32 uses s_X in place, bf16 a copy in the (dead) L tile
   T* s_Tm = sizeof(T) == 4 ? (T*)s_X : (T*)s_L;
-  constexpr bool LEAN = SAVE && sizeof(T) == 2;
 
   const int wv = wave_id(), l = lane_id();
   typedef TileIO<T, CH, K> IOK;
@@ -259,10 +262,10 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? 2 : 1)) void k_gdn_wy_fwd(c
         }
       }
       acc_to_lds_t<float>(pl, s_L, LDC, 16 * nj, 16 * wv, l);      // s_L[r][cc0 ..]: one 16-byte write
-      acc_to_lds_t<T>(pp, s_P, LDC, 16 * nj, 16 * wv, l);
+      acc_to_lds_t<T>(pp, s_P, LDP, 16 * nj, 16 * wv, l);
     }
     lds_barrier();
-    IO64::template lds_to_global<true>(s_P, LDC, pg, CH, CH, tid);
+    IO64::template lds_to_global<true>(s_P, LDP, pg, CH, CH, tid);
   }
   // k is dead as an operand of k k^T and q k^T: scale it in place to k beta e^{b} (from the registers)
   if constexpr (!LEAN) IOK::store_lds_scaled(rk, s_k, LDK, s_beb, tid);
