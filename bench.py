@@ -62,12 +62,17 @@ def stage_model(stage, K, V, s=2):
     full 64-token tiles, multiply-add = 2 flops; every input read once, every output written once."""
     c = CH
     kv, ck, cv, cc = K * V, c * K, c * V, c * c
-    if stage == 0:   # k k^T, q k^T, triangular inverse, w, u | r q,k,v  w w,u,Tinv,P,decay table
+    lean = s == 2     # 2-byte elements: w = Tinv (k beta e^b), u = Tinv (v beta) are formed inside the state passes
+    if stage == 0:   # k k^T, q k^T, triangular inverse (, w, u) | r q,k,g,beta(,v)  w Tinv,P,decay table(,w,u)
+        if lean:
+            return 4 * cc * K + (2 / 3) * c ** 3, 2 * ck * s + 2 * cc * s + c * (8 + 4 + s)
         return 6 * cc * K + 2 * cc * V + (2 / 3) * c ** 3, (2 * ck + cv) * s + (ck + cv) * s + 2 * cc * s + c * (8 + 4 + s)
-    if stage == 1:   # w S, q S, k^T v_new, P v_new | r q,k,w,u,P,table  w v_new,hs,o
+    if stage == 1:   # (w, u,) w S, q S, k^T v_new, P v_new | r q,k,Tinv,v,P,table,beta (q,k,w,u,P,table)  w v_new,hs,o
+        if lean:
+            return 6 * c * kv + 2 * cc * V + 2 * cc * K + 2 * cc * V, (2 * ck + cv + 2 * cc) * s + (2 * cv + kv) * s + c * (8 + s)
         return 6 * c * kv + 2 * cc * V, (3 * ck + cv + cc) * s + (2 * cv + kv) * s + 8 * c
-    if stage == 4:   # k dS', P^T do, q^T do, w^T dv_new | r q,k,w,do,P,table  w dv_new,dhs
-        return 6 * c * kv + 2 * cc * V, (3 * ck + cv + cc) * s + (cv + kv) * s + 8 * c
+    if stage == 4:   # w, k dS', P^T do, q^T do, w^T dv_new | r q,k,Tinv,do,P,table,beta  w dv_new,dhs
+        return 6 * c * kv + 2 * cc * V + 2 * cc * K, (2 * ck + cv + 2 * cc) * s + (cv + kv) * s + c * (8 + s)
     if stage == 5:   # do v'^T, do S^T, v' dS'^T, du S^T, du v^T, Tinv^T du, G k, G^T q, dw k^T, Tinv^T dw,
         #              two 64^3 products, dM k, dM^T k_b | r do,v',du,v,hs,dhs,q,k,Tinv,g,beta  w dq,dk,dv,dbeta,dg
         return (4 * cc * V + 6 * c * kv + 2 * cc * V + 4 * cc * K + 4 * cc * K + 4 * c ** 3 + 4 * cc * K,

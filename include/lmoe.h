@@ -133,12 +133,12 @@ int lmoe_chunk_gla_bwd(const lmoe_args* a, void* stream);
  * o_t = scale q_t S_t.
  * Replaces fla.ops.gated_delta_rule.chunk_gated_delta_rule called at
  *   linear_moe/sequence_modeling/gated_deltanet/gated_deltanet.py:112.
- * fwd uses q,k,v,g,beta,h0 -> o,ht,hs,vnew,w,u,tinv,pmat,gcum.  hs and vnew, which only the backward reads, may
- * both be NULL (a forward-only call); tinv may then be NULL too, but should be given: with it the 2-byte state
- * pass forms w on the chip from tinv and k instead of reading it (less memory traffic; the results of a call
- * with and without tinv differ in the last bit of w).
- * bwd uses q,k,v,g,beta,hs,vnew,tinv,pmat,gcum,d_o,dht -> dq,dk,dv,dg,dbeta,dh0 (+ dhs, dvnew); w is read by the
- * fp32 kernels only. */
+ * fwd uses q,k,v,g,beta,h0 -> o,ht,hs,vnew,tinv,pmat,gcum (+ w,u).  hs and vnew, which only the backward reads,
+ * may both be NULL (a forward-only call); tinv may then be NULL too, but should be given: with it the 2-byte
+ * state pass forms w and u on the chip from tinv, k, v, beta instead of reading them, and w, u are neither
+ * written nor needed (they may be NULL; less memory traffic; the results of a call with and without tinv differ
+ * in the last bit of w, u).  4-byte elements, or no tinv: w and u are required.
+ * bwd uses q,k,v,g,beta,hs,vnew,tinv,pmat,gcum,d_o,dht -> dq,dk,dv,dg,dbeta,dh0 (+ dhs, dvnew). */
 int lmoe_chunk_gated_delta_rule_fwd(const lmoe_args* a, void* stream);
 int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream);
 

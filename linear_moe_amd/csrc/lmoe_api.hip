@@ -57,8 +57,8 @@ int64_t lmoe_workspace_bytes(int32_t op, int32_t dtype, int32_t part, int32_t B,
   const int64_t rows_k = (int64_t)B * T * H * K, rows_v = (int64_t)B * T * H * V;
   int64_t n = states;                                                    // hs | dhs
   if (op == LMOE_OP_GLA && part == 0) n += tiles + 2 * (int64_t)NT * H * LMOE_CHUNK * K;   // amat, qe, ke
-  if (op == LMOE_OP_GATED_DELTA_RULE) n += part == 0 ? 2 * rows_v + rows_k + 2 * tiles   // vnew, u, w, tinv, pmat
-                                                     : rows_v;                       // dvnew
+  // vnew, tinv, pmat, and for 4-byte elements u, w (the 2-byte state passes form them on the chip) | dvnew
+  if (op == LMOE_OP_GATED_DELTA_RULE) n += part == 0 ? rows_v + 2 * tiles + (s == 4 ? rows_v + rows_k : 0) : rows_v;
   int64_t bytes = n * s;
   if (op == LMOE_OP_GATED_DELTA_RULE && part == 0) bytes += (int64_t)NT * H * 2 * LMOE_CHUNK * 4;   // gcum (fp32)
   if (op == LMOE_OP_GLA && part == 0) bytes += (int64_t)NT * H * K * 4;                              // gcum (fp32)
@@ -126,8 +126,10 @@ int lmoe_chunk_gated_delta_rule_fwd(const lmoe_args* a, void* stream) {
   if (int r = check_common(a, op)) return r;
   if (a->gate == LMOE_GATE_VECTOR) return fail(-10, "%s: the gate is one scalar per token and head", op);
   if (!a->beta.ptr) return fail(-12, "%s: beta must not be null", op);
-  if (!a->o.ptr || !a->w.ptr || !a->u.ptr || !a->pmat || !a->gcum)
-    return fail(-11, "%s: o, w, u, pmat and gcum must not be null", op);
+  if (!a->o.ptr || !a->pmat || !a->gcum) return fail(-11, "%s: o, pmat and gcum must not be null", op);
+  // w, u are written and read only where the state pass does not form them itself from tinv
+  if ((a->dtype != LMOE_BF16 || !a->tinv) && (!a->w.ptr || !a->u.ptr))
+    return fail(-11, "%s: w and u must not be null (4-byte elements, or no tinv given)", op);
   // what only the backward reads: hs and vnew together or not at all (a forward-only call); tinv goes with
   // them, and may also be given alone (the state pass then forms w from it instead of reading w)
   if ((a->hs != nullptr) != (a->vnew.ptr != nullptr) || (a->hs != nullptr && a->tinv == nullptr))
@@ -142,8 +144,8 @@ int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream) {
   if (int r = check_common(a, op)) return r;
   if (a->gate == LMOE_GATE_VECTOR) return fail(-10, "%s: the gate is one scalar per token and head", op);
   if (!a->beta.ptr) return fail(-12, "%s: beta must not be null", op);
-  if (!a->hs || !a->dhs || !a->vnew.ptr || !a->w.ptr || !a->tinv || !a->pmat || !a->gcum || !a->dvnew.ptr)
-    return fail(-11, "%s: hs, dhs, vnew, w, tinv, pmat, gcum and dvnew must not be null", op);
+  if (!a->hs || !a->dhs || !a->vnew.ptr || !a->tinv || !a->pmat || !a->gcum || !a->dvnew.ptr)
+    return fail(-11, "%s: hs, dhs, vnew, tinv, pmat, gcum and dvnew must not be null", op);
   if (!a->d_o.ptr || !a->dq.ptr || !a->dk.ptr || !a->dv.ptr || !a->dg.ptr || !a->dbeta.ptr)
     return fail(-13, "%s: d_o, dq, dk, dv, dg and dbeta must not be null", op);
   if (a->NT == 0 || a->N == 0) return 0;
@@ -413,7 +415,8 @@ int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* strea
         lmoe::launch_bwd_dv(*a, false, st); break;
       case lmoe::ST_STATE_BWD:
         if (gdn) {
-          if (!a->pmat || !a->gcum) return fail(-11, "%s: pmat and gcum must not be null", nm);
+          if (!a->pmat || !a->gcum || !a->tinv || !a->beta.ptr)
+            return fail(-11, "%s: pmat, gcum, tinv and beta must not be null", nm);
           lmoe::launch_gdn_state_bwd(*a, st);
         } else {
           lmoe::launch_state_bwd(*a, st);

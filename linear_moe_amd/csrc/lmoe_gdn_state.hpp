@@ -593,8 +593,10 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
     for (int ni = 0; ni < NB; ++ni) {
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        // dv_new, rounded once to the storage type (the chunk-parallel backward reads the stored values)
-        t[0][ni][i] = ET<T>::to_f(ET<T>::from_f(scale * dvl[0][ni][i] + edt * t[0][ni][i]));
+        // dv_new, rounded once to the storage type (the chunk-parallel backward reads the stored values).
+        // The fused multiply-add is spelled out: left to the compiler, a sum of two products is contracted
+        // one way or the other per instantiation, and the wide and narrow slices then differ in the last bit.
+        t[0][ni][i] = ET<T>::to_f(ET<T>::from_f(__builtin_fmaf(scale, dvl[0][ni][i], edt * t[0][ni][i])));
       acc_to_lds_t<T>(t[0][ni], s_dvn, LDU, 16 * ni, 16 * wv);      // s_dvn[token][v]
     }
     const float dec = s_dec[cur];

@@ -68,15 +68,16 @@ class GDNCall:
         tinv = torch.empty(max(plan.NT, 1), H, 64, 64, dtype=dt, device=dev)
         pmat = torch.empty(max(plan.NT, 1), H, 64, 64, dtype=dt, device=dev)
         gcum = torch.empty(max(plan.NT, 1), H, 2, 64, dtype=torch.float32, device=dev)
-        w = torch.empty(B, T, H, K, dtype=dt, device=dev)
-        u = torch.empty(B, T, H, V, dtype=dt, device=dev)
+        # w, u: the bf16 state passes form them on the chip from tinv; only the fp32 forward pass reads them
+        w = torch.empty(B, T, H, K, dtype=dt, device=dev) if dt == torch.float32 else None
+        u = torch.empty(B, T, H, V, dtype=dt, device=dev) if dt == torch.float32 else None
         vnew = torch.empty(B, T, H, V, dtype=dt, device=dev) if save else None
         a.o, a.ht, a.hs, a.tinv = _desc(o, head_first), ptr(ht), ptr(hs), ptr(tinv)
         a.pmat, a.gcum = pmat.data_ptr(), gcum.data_ptr()
         a.w, a.u, a.vnew = _desc(w, False), _desc(u, False), _desc(vnew, False)
         _lib.check(lib.lmoe_chunk_gated_delta_rule_fwd(C.byref(a), stream_ptr()), "chunk_gated_delta_rule forward")
-        ctx.saved = (q, k, v, g, beta, h0, hs, tinv, pmat, gcum, w, vnew)
-        ctx.fwd_args, ctx.fwd_keep = a, ((o, ht, u) if self.keep else None)
+        ctx.saved = (q, k, v, g, beta, h0, hs, tinv, pmat, gcum, vnew)
+        ctx.fwd_args, ctx.fwd_keep = a, ((o, ht, w, u) if self.keep else None)
         ctx.plan, ctx.dims, ctx.head_first, ctx.scale = plan, dims, head_first, scale
         ctx.has_h0 = initial_state is not None
         return o, ht
@@ -84,7 +85,7 @@ class GDNCall:
     def backward(self, do, dht):
         ctx = self
         lib = _lib.load()
-        q, k, v, g, beta, h0, hs, tinv, pmat, gcum, w, vnew = ctx.saved
+        q, k, v, g, beta, h0, hs, tinv, pmat, gcum, vnew = ctx.saved
         plan, dims, head_first = ctx.plan, ctx.dims, ctx.head_first
         B, T, H, K, V = dims
         do = _aligned(do)
@@ -95,7 +96,7 @@ class GDNCall:
         a.beta, a.beta_dtype = _desc(beta, head_first), _scalar_dt(beta)
         a.h0, a.hs, a.tinv, a.pmat = ptr(h0), hs.data_ptr(), tinv.data_ptr(), pmat.data_ptr()
         a.gcum = gcum.data_ptr()
-        a.w, a.vnew = _desc(w, False), _desc(vnew, False)
+        a.vnew = _desc(vnew, False)
         a.d_o = _desc(do, head_first)
         dht = None if dht is None else dht.float().contiguous()
         a.dht = ptr(dht)
