@@ -34,8 +34,8 @@ STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_gdn_state_fwd", 4: "k_gdn_state_bwd", 5:
 # copy that main() issues first (FETCH_SIZE reads half of the bytes fetched, WRITE_SIZE all of the
 # bytes written).  Summary and commands: profiles/gdn_fwd_bwd_cfg4_hbm_traffic.md.
 CALIB_COPY_BYTES = 256 << 20
-MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 835417594, "k_gdn_state_fwd": 1197427009, "k_gdn_state_bwd": 1024167366,
-                    "k_gdn_bwd_chunk": 1896521392}
+MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 432417222, "k_gdn_state_fwd": 1128774601, "k_gdn_state_bwd": 980265694,
+                    "k_gdn_bwd_chunk": 1897687630}
 
 
 def gdn_inputs(B, T, H, K, V, seed, dtype, device):

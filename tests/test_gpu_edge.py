@@ -164,3 +164,35 @@ def test_strided_views_need_no_copy_and_give_the_same(cuda, op):
     torch.cuda.synchronize()
     for a, b in zip(got_hf, ref):
         assert torch.equal(tr(a), b)
+
+
+@pytest.mark.parametrize("op", OPS)
+def test_a_sequence_gives_the_same_bits_alone_and_inside_a_large_packed_batch(cuda, op):
+    """The sequential passes carry 64 V columns per work-group when sequences x heads alone fill the GPU and 32
+    otherwise: a choice of the launch that must not show in the results.  One sequence out of 17 x 16 heads
+    (wide slices) against the same sequence as a call of its own (narrow slices), outputs and all gradients."""
+    N, Ls, H, K, V = 17, 200, 16, 128, 128
+    T = N * Ls
+    ins = {n: x.to(cuda) for n, x in _inputs(op, T, H, K, V, torch.bfloat16, 3300).items()}
+    h0 = (gen(3310, N, H, K, V) * 0.1).to(cuda)
+    do, dht = gen(3311, 1, T, H, V, dtype=torch.bfloat16).to(cuda), gen(3312, N, H, K, V).to(cuda)
+    cu = (torch.arange(N + 1, dtype=torch.int32) * Ls).to(cuda)
+    names = list(ins)
+
+    def run(ins, h0, cu, do, dht):
+        leaves = {n: x.clone().requires_grad_(True) for n, x in dict(ins, h0=h0).items()}
+        o, ht = _call(op, leaves, leaves["h0"], cu, True)
+        grads = torch.autograd.grad([o, ht], [leaves[n] for n in names + ["h0"]], [do, dht])
+        return (o.detach(), ht.detach()) + tuple(grads)
+
+    s = N - 1
+    sl = slice(s * Ls, (s + 1) * Ls)
+    cut = lambda x: x[:, sl].contiguous()
+    alone = run({n: cut(x) for n, x in ins.items()}, h0[s:s + 1].contiguous(), None, cut(do), dht[s:s + 1].contiguous())
+    packed = run(ins, h0, cu, do, dht)
+    torch.cuda.synchronize()
+    per_seq = (1, len(packed) - 1)                     # ht and dh0 are per sequence, the rest per token
+    labels = ["o", "ht"] + ["d" + n for n in names] + ["dh0"]
+    for i, (a, b) in enumerate(zip(packed, alone)):
+        a = a[s:s + 1] if i in per_seq else a[:, sl]
+        assert torch.equal(a, b), labels[i]
