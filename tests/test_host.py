@@ -69,6 +69,36 @@ def test_invalid_arguments_are_rejected_without_a_launch():
     assert lib.lmoe_selftest_gemm(0, 64, None, None, None, None, None) == -1
 
 
+def test_gated_delta_rule_needs_w_and_u_only_where_the_state_pass_reads_them():
+    """2-byte elements with a Tinv buffer: the state pass forms w, u itself, they may be NULL.  4-byte elements, or no
+    Tinv: they are required.  A call without chunks validates and returns before any launch (no GPU needed)."""
+    from linear_moe_amd import _lib
+    lib = _lib.load()
+    fake = 0x1000                                  # never dereferenced: NT == 0
+
+    def args(dtype, tinv, wu):
+        a = _lib.Args()
+        a.dtype, a.B, a.T, a.H, a.K, a.V, a.N, a.NT = dtype, 1, 0, 1, 64, 64, 1, 0
+        a.scale, a.gate, a.g_dtype, a.beta_dtype = 1.0, 1, _lib.LMOE_F32, dtype
+        for n in ("q", "k", "v", "g", "beta", "o"):
+            setattr(a, n, _lib.Tensor4(fake, 0, 64, 64))
+        a.pmat = a.gcum = fake
+        a.tinv = fake if tinv else None
+        if wu:
+            a.w = a.u = _lib.Tensor4(fake, 0, 64, 64)
+        return a
+
+    for dtype in (_lib.LMOE_BF16, _lib.LMOE_F32):
+        for tinv in (False, True):
+            for wu in (False, True):
+                a = args(dtype, tinv, wu)
+                rc = lib.lmoe_chunk_gated_delta_rule_fwd(C.byref(a), None)
+                needed = dtype == _lib.LMOE_F32 or not tinv
+                assert rc == (-11 if needed and not wu else 0), (dtype, tinv, wu)
+                if rc:
+                    assert b"w and u must not be null" in lib.lmoe_last_error()
+
+
 def test_workspace_bytes_matches_the_buffers_the_host_layer_allocates():
     from linear_moe_amd import _lib
     lib = _lib.load()
