@@ -13,6 +13,7 @@ from typing import Optional, Tuple
 
 import torch
 
+from ._host import no_tokens
 from .gated_delta_rule import _ChunkGatedDeltaRule
 
 
@@ -30,5 +31,8 @@ def chunk_delta_rule(
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     if BT not in (16, 32, 64):
         raise ValueError(f"chunk size must be 16, 32 or 64, got {BT}")
+    r = no_tokens(q, k, v, head_first, cu_seqlens, initial_state, output_final_state)
+    if r is not None:
+        return r
     return _ChunkGatedDeltaRule.apply(q, k, v, None, beta, scale, initial_state, output_final_state, cu_seqlens,
                                       head_first)

@@ -44,7 +44,9 @@ def chunk_linear_attn(
         o = oi if o is None else o + oi
         hts.append(hi)
         if normalize:
-            zi = (qi * ki.cumsum(tdim)).sum(-1, keepdim=True)
+            # the normaliser carries the scale of the numerator (fla normalises with q * scale), so that
+            # the scale cancels in o up to the epsilon
+            zi = ((qi * scale) * ki.cumsum(tdim)).sum(-1, keepdim=True)
             z = zi if z is None else z + zi
         k0 += w
     if normalize:

@@ -205,17 +205,19 @@ def naive_retention(q, k, v, scale=None, initial_state=None, output_final_state=
 
 def naive_linear_attn(q, k, v, scale=None, initial_state=None, output_final_state=False,
                       normalize=True, head_first=True, dtype=torch.float64, eps=1e-10):
-    """chunk_linear_attn: simple_gla with g=None; normalize divides o by q . cumsum(k) + eps.
+    """chunk_linear_attn: simple_gla with g=None; normalize divides o by (scale q) . cumsum(k) + eps, i.e.
+    o_t = sum_{s<=t} a_ts v_s / (sum_{s<=t} a_ts + eps) with a_ts = scale q_t . k_s: the scale cancels up to eps
+    (call sites: basic_linear_attention.py:133 with the default scale, based.py:69 / rebased.py:76 with scale 1).
 
-    The eps value is recalled from fla (not checkable offline): parity unpinned for
-    normalize=True; the reference's default path is normalize=False
-    (linear_moe/arguments.py:533-536).
+    The value of eps is recalled from fla (not checkable offline): parity unpinned for that constant only; the
+    formula is pinned by its closed form and a hand-worked case in tests/test_oracle_pins.py.
     """
     o, ht = naive_recurrent_simple_gla(q, k, v, None, scale, initial_state, output_final_state,
                                        None, head_first, dtype)
     if normalize:
         qh, kh = (_to_head_first(x, head_first).to(dtype) for x in (q, k))
-        z = (qh * kh.cumsum(2)).sum(-1, keepdim=True) + eps
+        sc = q.shape[-1] ** -0.5 if scale is None else scale
+        z = sc * (qh * kh.cumsum(2)).sum(-1, keepdim=True) + eps
         o = _to_head_first(_to_head_first(o, head_first) / z, head_first)
     return o, ht
 

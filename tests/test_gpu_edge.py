@@ -67,6 +67,22 @@ def test_packed_batch_with_empty_sequences(cuda, op, dtype):
         assert max_abs_rel(dev[n].grad.cpu(), r) < tol, n
 
 
+def test_delta_rule_without_tokens_hands_the_state_through(cuda):
+    """chunk_delta_rule with T = 0: the final state is the initial state (zeros without one), never uninitialised."""
+    from linear_moe_amd import chunk_delta_rule
+    B, H, K, V = 2, 2, 64, 128
+    q, k, v = (torch.zeros(B, H, 0, D, dtype=torch.bfloat16, device=cuda) for D in (K, K, V))
+    beta = torch.zeros(B, H, 0, dtype=torch.bfloat16, device=cuda)
+    h0 = (gen(3110, B, H, K, V) * 0.5).to(cuda).requires_grad_(True)
+    dht = gen(3111, B, H, K, V).to(cuda)
+    o, ht = chunk_delta_rule(q, k, v, beta, 64, None, h0, True)
+    assert o.shape == (B, H, 0, V)
+    (ht * dht).sum().backward()
+    assert torch.equal(ht.detach(), h0.detach()) and torch.equal(h0.grad, dht)
+    _, ht = chunk_delta_rule(q, k, v, beta, 64, None, None, True)
+    assert torch.equal(ht, torch.zeros(B, H, K, V, device=cuda))
+
+
 @pytest.mark.parametrize("op", OPS)
 def test_no_tokens_at_all(cuda, op):
     dtype = torch.bfloat16

@@ -163,25 +163,79 @@ def test_python_layer_validates_before_launch():
         _check_inputs(g, g, g, True, None)
 
 
+REFERENCE_PKG = "/root/reference/linear_moe"
+
+# the import lines of the reference as of this writing; used where the reference is not mounted
+_KNOWN_IMPORTS = {
+    "fla.ops.gla": ["chunk_gla", "fused_chunk_gla", "fused_recurrent_gla"],
+    "fla.ops.gated_delta_rule": ["chunk_gated_delta_rule", "fused_recurrent_gated_delta_rule"],
+    "fla.ops.delta_rule": ["chunk_delta_rule", "fused_chunk_delta_rule", "fused_recurrent_delta_rule"],
+    "fla.ops.linear_attn": ["chunk_linear_attn", "fused_chunk_linear_attn", "fused_recurrent_linear_attn"],
+    "fla.ops.retention": ["chunk_retention", "fused_chunk_retention", "fused_recurrent_retention",
+                          "parallel_retention"],
+    "fla.ops.based": ["parallel_based"], "fla.ops.rebased": ["parallel_rebased"],
+    "fla.ops.rwkv6": ["chunk_rwkv6", "fused_recurrent_rwkv6"],
+    "fla.ops.rwkv7": ["chunk_rwkv7", "fused_recurrent_rwkv7"],
+    "fla.ops.rotary": ["apply_rotary"], "fla.modules.rotary": ["RotaryEmbedding"],
+    "fla.modules.l2norm": ["l2_norm"],
+    "lightning_attn.ops.triton": ["lightning_attn2", "lightning_attn2_no_decay"],
+}
+
+
+def _reference_imports():
+    """{module: sorted names} of every ``from fla... import`` / ``from lightning_attn... import`` statement in the
+    reference's package, read from the source text with ``ast`` (nothing of the reference is imported or run)."""
+    import ast
+    found = {}
+    for dirpath, _, files in os.walk(REFERENCE_PKG):
+        for f in files:
+            if not f.endswith(".py"):
+                continue
+            try:
+                tree = ast.parse(open(os.path.join(dirpath, f), encoding="utf-8", errors="replace").read())
+            except SyntaxError:
+                continue
+            for node in ast.walk(tree):
+                if isinstance(node, ast.ImportFrom) and node.module and node.level == 0 and \
+                        node.module.split(".")[0] in ("fla", "lightning_attn"):
+                    found.setdefault(node.module, set()).update(a.name for a in node.names)
+                elif isinstance(node, ast.Import):
+                    for a in node.names:
+                        if a.name.split(".")[0] in ("fla", "lightning_attn"):
+                            found.setdefault(a.name, set())
+    return {m: sorted(n) for m, n in found.items()}
+
+
 def test_fla_shim_resolves_every_name_the_reference_imports():
     """A fresh interpreter with only the shim directory on its path (as the reference's launcher sets
-    PYTHONPATH=$FLA_PATH) finds every operator name of the reference's import lines."""
+    PYTHONPATH=$FLA_PATH) resolves every ``fla`` / ``lightning_attn`` import statement found in the reference's
+    sources (collected at test time where the reference is mounted; the recorded list otherwise, and the two
+    must agree), plus ``fla.ops.simple_gla``."""
     shim = os.path.join(ROOT, "linear_moe_amd", "fla_shim")
-    code = (
-        "from fla.ops.gla import chunk_gla, fused_chunk_gla, fused_recurrent_gla\n"
-        "from fla.ops.gated_delta_rule import chunk_gated_delta_rule, fused_recurrent_gated_delta_rule\n"
-        "from fla.ops.delta_rule import chunk_delta_rule, fused_chunk_delta_rule, fused_recurrent_delta_rule\n"
-        "from fla.ops.linear_attn import chunk_linear_attn, fused_chunk_linear_attn, fused_recurrent_linear_attn\n"
-        "from fla.ops.retention import (chunk_retention, fused_chunk_retention, fused_recurrent_retention,\n"
-        "                               parallel_retention)\n"
-        "from fla.ops.simple_gla import chunk_simple_gla\n"
-        "from fla.ops.based import parallel_based\n"
-        "from fla.ops.rebased import parallel_rebased\n"
+    imports = dict(_KNOWN_IMPORTS)
+    if os.path.isdir(REFERENCE_PKG):
+        scanned = _reference_imports()
+        assert scanned, "no fla import found in the reference: the scan is broken"
+        assert scanned == {m: sorted(n) for m, n in _KNOWN_IMPORTS.items()}, \
+            "the reference imports names the recorded list does not hold (or the reverse)"
+        imports = scanned
+    lines = [f"from {m} import {', '.join(n)}" if n else f"import {m}" for m, n in sorted(imports.items())]
+    code = "\n".join(lines) + (
+        "\nfrom fla.ops.simple_gla import chunk_simple_gla\n"
         "from fla.modules.l2norm import l2_norm\n"
-        "from lightning_attn.ops.triton import lightning_attn2, lightning_attn2_no_decay\n"
+        "from fla.ops.gated_delta_rule import chunk_gated_delta_rule\n"
+        "from fla.ops.rotary import apply_rotary\n"
+        "from fla.ops.rwkv6 import chunk_rwkv6\n"
         "import linear_moe_amd, torch\n"
         "assert chunk_gated_delta_rule is linear_moe_amd.chunk_gated_delta_rule\n"
         "assert l2_norm is linear_moe_amd.l2_norm\n"
+        "for fn in (apply_rotary, chunk_rwkv6):\n"
+        "    try:\n"
+        "        fn()\n"
+        "    except NotImplementedError:\n"
+        "        pass\n"
+        "    else:\n"
+        "        raise SystemExit('a name off the path must raise when called')\n"
         "print('ok')\n")
     env = {k: v for k, v in os.environ.items() if k != "PYTHONPATH"}
     env["PYTHONPATH"] = shim

@@ -37,6 +37,34 @@ def test_default_scale_is_rsqrt_k():
     assert torch.allclose(o, 0.25 * torch.tril(q @ k.transpose(-1, -2)) @ v, atol=1e-12)
 
 
+def test_linear_attn_normalised_closed_form_and_by_hand():
+    """normalize=True: o_t = sum_{s<=t} a_ts v_s / (sum_{s<=t} a_ts + eps), a_ts = scale q_t.k_s -- the scale sits in
+    the numerator AND in the normaliser (a normaliser built from the unscaled q is off by 1/scale)."""
+    q, k, v = rnd(11, 2, 3, 41, 8).abs(), rnd(12, 2, 3, 41, 8).abs(), rnd(13, 2, 3, 41, 5)
+    for scale, eps in ((None, 1e-10), (1.0, 1e-10), (0.37, 1e-10), (0.37, 0.5)):
+        o, ht = naive.naive_linear_attn(q, k, v, scale=scale, output_final_state=True, normalize=True, eps=eps)
+        sc = 8 ** -0.5 if scale is None else scale
+        A = torch.tril(sc * q @ k.transpose(-1, -2))
+        assert torch.allclose(o, (A @ v) / (A.sum(-1, keepdim=True) + eps), atol=1e-12)
+        assert torch.allclose(ht, k.transpose(-1, -2) @ v, atol=1e-12)          # the state is not normalised
+        o_tf, _ = naive.naive_linear_attn(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), scale=scale,
+                                          normalize=True, head_first=False, eps=eps)
+        assert torch.allclose(o_tf.transpose(1, 2), o, atol=1e-12)
+    # by hand, T = 2, K = V = 1, scale 1/2, eps = 1 (large on purpose: it shows where the scale sits):
+    # a00 = .5*2*5 = 5, a10 = .5*3*5 = 7.5, a11 = .5*3*7 = 10.5;  o0 = 5*11/(5+1),  o1 = (7.5*11 + 10.5*13)/(18+1)
+    t = lambda *x: torch.tensor(x, dtype=D).reshape(1, 1, 2, 1)
+    o, _ = naive.naive_linear_attn(t(2, 3), t(5, 7), t(11, 13), scale=0.5, normalize=True, eps=1.0)
+    assert torch.allclose(o.flatten(), torch.tensor([55 / 6, 219 / 19], dtype=D), atol=1e-13)
+    # Based end to end: Taylor features, scale 1 -> weights 1 + s + s^2/2 with s = q.k / sqrt(D)
+    Dh = 4
+    q, k, v = 0.5 * rnd(14, 1, 2, 23, Dh), 0.5 * rnd(15, 1, 2, 23, Dh), rnd(16, 1, 2, 23, 3)
+    o, _ = naive.naive_linear_attn(naive.naive_taylor_feature_map(q), naive.naive_taylor_feature_map(k), v, scale=1.0,
+                                   normalize=True)
+    x = q @ k.transpose(-1, -2) / Dh ** 0.5
+    W = torch.tril(1 + x + x * x / 2)
+    assert torch.allclose(o, (W @ v) / (W.sum(-1, keepdim=True) + 1e-10), atol=1e-12)
+
+
 def test_retention_closed_form():
     B, H, T = 1, 4, 50
     q, k, v = rnd(4, B, H, T, 8), rnd(5, B, H, T, 8), rnd(6, B, H, T, 6)
