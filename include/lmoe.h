@@ -175,6 +175,18 @@ int lmoe_rmsnorm_fwd(const void* x, const void* w, const void* gate, void* y, fl
 int lmoe_rmsnorm_bwd(const void* x, const void* w, const void* gate, const void* dy, void* dx, void* dgate,
                      float* dw_part, float* dw, int64_t rows, int32_t D, int32_t dtype, float eps, void* stream);
 
+/* lmoe_rmsnorm_bwd for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc): the same kernels, the same results bit for bit, with the partial rows of dw in a scratch
+ * array the library holds itself (static device memory, 2 MiB per GPU until the process ends) instead of a
+ * caller-allocated dw_part.  No counterpart in the reference.  Calls no hipMalloc / hipFree.  dw ([D] fp32) is
+ * required (a caller that wants no dw needs no workspace either: lmoe_rmsnorm_bwd with dw_part = dw = NULL).
+ * Returns -23 when rows x D needs more partial rows than the scratch holds (2048 rows of 256 floats: never on a GPU
+ * of up to 256 compute units).  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU
+ * (two streams, two threads) race; every call overwrites the rows it later reads, so nothing has to be cleared
+ * between calls. */
+int lmoe_rmsnorm_bwd_noalloc(const void* x, const void* w, const void* gate, const void* dy, void* dx, void* dgate,
+                             float* dw, int64_t rows, int32_t D, int32_t dtype, float eps, void* stream);
+
 /* Gate construction of the gated delta rule for a, b of shape [rows][H] (element type by dtype):
  *   beta = sigmoid(b)  (element type of b),   g = -exp(A_log[h]) softplus(a + dt_bias[h])  (fp32)
  * as linear_moe/sequence_modeling/linear_attention.py:153-154 forms them in front of the op (parameters

@@ -47,7 +47,7 @@ ENTRY_POINTS = (
     "lmoe_chunk_gla_fwd", "lmoe_chunk_gla_bwd",
     "lmoe_chunk_gated_delta_rule_fwd", "lmoe_chunk_gated_delta_rule_bwd",
     "lmoe_launch_stage", "lmoe_selftest_gemm", "lmoe_workspace_bytes", "lmoe_l2norm_fwd", "lmoe_l2norm_bwd",
-    "lmoe_silu_l2norm_fwd", "lmoe_silu_l2norm_bwd", "lmoe_rmsnorm_partials", "lmoe_rmsnorm_fwd", "lmoe_rmsnorm_bwd",
+    "lmoe_silu_l2norm_fwd", "lmoe_silu_l2norm_bwd", "lmoe_rmsnorm_partials", "lmoe_rmsnorm_fwd", "lmoe_rmsnorm_bwd", "lmoe_rmsnorm_bwd_noalloc",
     "lmoe_gdn_gates_partials", "lmoe_gdn_gates_fwd", "lmoe_gdn_gates_bwd", "lmoe_gla_gate_fwd", "lmoe_gla_gate_bwd",
     "lmoe_hgrn2_gate_fwd", "lmoe_hgrn2_gate_bwd", "lmoe_quad_featmap_features", "lmoe_quad_featmap_fwd",
     "lmoe_quad_featmap_bwd",
@@ -94,6 +94,8 @@ def load() -> C.CDLL:
     lib.lmoe_rmsnorm_fwd.restype = C.c_int
     lib.lmoe_rmsnorm_bwd.argtypes = [C.c_void_p] * 8 + [C.c_int64, C.c_int32, C.c_int32, C.c_float, C.c_void_p]
     lib.lmoe_rmsnorm_bwd.restype = C.c_int
+    lib.lmoe_rmsnorm_bwd_noalloc.argtypes = [C.c_void_p] * 7 + [C.c_int64, C.c_int32, C.c_int32, C.c_float, C.c_void_p]
+    lib.lmoe_rmsnorm_bwd_noalloc.restype = C.c_int
     lib.lmoe_gdn_gates_partials.argtypes = [C.c_int64, C.c_int32]
     lib.lmoe_gdn_gates_partials.restype = C.c_int
     lib.lmoe_gdn_gates_fwd.argtypes = [C.c_void_p] * 6 + [C.c_int64, C.c_int32, C.c_int32, C.c_void_p]

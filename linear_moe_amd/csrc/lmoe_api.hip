@@ -227,6 +227,26 @@ int lmoe_rmsnorm_bwd(const void* x, const void* w, const void* gate, const void*
   return launched(nm);
 }
 
+int lmoe_rmsnorm_bwd_noalloc(const void* x, const void* w, const void* gate, const void* dy, void* dx, void* dgate,
+                             float* dw, int64_t rows, int32_t D, int32_t dtype, float eps, void* stream) {
+  const char* nm = "lmoe_rmsnorm_bwd_noalloc";
+  if (int r = check_l2norm(nm, x, dx, rows, D, dtype)) return r;
+  if (!dy || !dw) return fail(-1, "%s: dy and dw must not be null", nm);
+  if (((uintptr_t)w | (uintptr_t)gate | (uintptr_t)dy | (uintptr_t)dgate) & 15)
+    return fail(-9, "%s: pointers must be 16-byte aligned", nm);
+  if ((gate != nullptr) != (dgate != nullptr)) return fail(-1, "%s: gate and dgate go together", nm);
+  if (rows == 0) return 0;              // nothing to do (dw is not written)
+  float* part = nullptr;
+  int64_t cap = 0;
+  if (int e = lmoe::rmsnorm_scratch(&part, &cap)) return fail(e, "%s: no address for the library's scratch array: %s", nm, hipGetErrorString((hipError_t)e));
+  const int64_t need = (int64_t)lmoe::rmsnorm_partials(dtype, D, rows) * D;
+  if (need > cap)
+    return fail(-23, "%s: %lld partial rows of %d floats exceed the library's scratch (%lld floats); use lmoe_rmsnorm_bwd "
+                     "with a caller-allocated dw_part", nm, (long long)(need / D), D, (long long)cap);
+  lmoe::launch_rmsnorm(dtype, D, x, w, gate, dy, dx, dgate, nullptr, part, dw, rows, eps, true, (hipStream_t)stream);
+  return launched(nm);
+}
+
 int lmoe_fused_recurrent_fwd(const lmoe_args* a, int32_t op, void* stream) {
   const char* nm = "lmoe_fused_recurrent_fwd";
   if (int r = check_common(a, nm)) return r;

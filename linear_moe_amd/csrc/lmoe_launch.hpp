@@ -49,6 +49,8 @@ void launch_l2norm(int dtype, int D, const void* x, const void* dy, void* out, i
 void launch_rmsnorm(int dtype, int D, const void* x, const void* w, const void* gate, const void* dy, void* out,
                     void* dgate, float* rstd, float* dw_part, float* dw, int64_t rows, float eps, bool bwd, hipStream_t st);
 int rmsnorm_partials(int dtype, int D, int64_t rows);
+// the library-owned partial-row scratch of the current device (set up on its first use there); 0 or a hipError_t
+int rmsnorm_scratch(float** ptr, int64_t* capacity_floats);
 // y = l2norm(silu(x)) (bwd: out = dx)
 void launch_silu_l2norm(int dtype, int D, const void* x, const void* dy, void* out, int64_t rows, float eps, bool bwd,
                         hipStream_t st);

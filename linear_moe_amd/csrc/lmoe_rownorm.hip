@@ -11,6 +11,8 @@
 //    one fp32 partial row; k_colsum adds the partial rows in a fixed order (bit-reproducible).
 //  * SiLU followed by the L2 norm of q and k rows:  y = silu(x) / sqrt(sum silu(x)^2 + eps)
 //    (linear_moe/sequence_modeling/gated_deltanet/gated_deltanet.py:101-106) and its backward.
+#include <mutex>
+
 #include "lmoe_launch.hpp"
 #include "lmoe_seq.hpp"
 
@@ -148,6 +150,34 @@ static void rmsnorm_t(const void* x, const void* w, const void* gate, const void
     else hipLaunchKernelGGL((k_rmsnorm_bwd<T, D, false>), dim3(grid), dim3(NTHR), 0, st, (const T*)x, (const T*)w, (const T*)nullptr, (const T*)dy, (T*)out, (T*)nullptr, dw_part, rows, eps);
     if (dw_part) hipLaunchKernelGGL(k_colsum, dim3(D), dim3(NTHR), 0, st, (const float*)dw_part, dw, grid, D);
   }
+}
+
+// Library-owned scratch of the allocation-free backward entry point: the fp32 partial rows of dw for the largest grid
+// this file launches on a 256-CU GPU (8 work-groups per CU) at the widest row, 2 MiB per GPU, held until the process
+// ends.  The array's name is a host-side handle, not a device address: host code only ever uses the address that
+// hipGetSymbolAddress returns for the current device (each GPU holds its own copy).
+constexpr int64_t RMS_SCRATCH_FLOATS = 2048 * 256;
+static __device__ __align__(256) float scratch[RMS_SCRATCH_FLOATS];
+
+int rmsnorm_scratch(float** out, int64_t* capacity_floats) {
+  constexpr int MAXDEV = 64;
+  static float* ptrs[MAXDEV] = {};
+  static std::mutex mu;
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= MAXDEV) return (int)hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptrs[dev]) {
+    float* p = nullptr;
+    e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!p) return (int)hipErrorInvalidSymbol;
+    ptrs[dev] = p;
+  }
+  *out = ptrs[dev];
+  *capacity_floats = RMS_SCRATCH_FLOATS;
+  return 0;
 }
 
 // number of fp32 partial rows k_rmsnorm_bwd writes (the caller sizes dw_part with it)
