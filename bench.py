@@ -33,9 +33,25 @@ STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_gdn_state_fwd", 4: "k_gdn_state_bwd", 5:
 # WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for the 256 MiB device
 # copy that main() issues first (FETCH_SIZE reads half of the bytes fetched, WRITE_SIZE all of the
 # bytes written).  Summary and commands: profiles/gdn_fwd_bwd_cfg4_hbm_traffic.md.
+# The figures belong to the kernel sources they were measured on: TRAFFIC_SOURCES_SHA16 is the digest of those
+# sources (kernel_sources_sha16()) at that time, and a build whose sources differ reports traffic = null
+# rather than a stale number.
 CALIB_COPY_BYTES = 256 << 20
 MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 432417222, "k_gdn_state_fwd": 1128774601, "k_gdn_state_bwd": 980265694,
                     "k_gdn_bwd_chunk": 1897687630}
+TRAFFIC_SOURCES_SHA16 = "50306358452a3c02"
+TRAFFIC_SOURCES = ("lmoe_common.hpp", "lmoe_seq.hpp", "lmoe_gdn_wy.hpp", "lmoe_gdn_state.hpp", "lmoe_gdn_bwd_chunk.hpp",
+                   "lmoe_gdn_fwd.hip", "lmoe_gdn_state.hip", "lmoe_gdn_bwd.hip")
+
+
+def kernel_sources_sha16():
+    """Digest of the sources of the four gated-delta-rule kernels (what MEASURED_TRAFFIC was counted on)."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in TRAFFIC_SOURCES:
+        with open(os.path.join(ROOT, "linear_moe_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
 
 
 def gdn_inputs(B, T, H, K, V, seed, dtype, device):
@@ -345,20 +361,37 @@ def main():
     torch.cuda.synchronize()
     del src, dst
 
+    from linear_moe_amd import chunk_gated_delta_rule
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / args.steps
+
+    # the step as a user of the library runs it: the public entry point under autograd (its allocations, the
+    # autograd bookkeeping and the casts of the gradients to the input dtypes are inside the timed region)
+    leaves = [x[n].requires_grad_(True) for n in ("q", "k", "v", "g", "beta")]
+
+    def step_public():
+        o, _ = chunk_gated_delta_rule(*leaves, None, None, False, None, False)
+        torch.autograd.grad([o], leaves, [x["do"]])
+
+    dt = timed(step_public)
+
+    # the same kernels driven through the call object (no autograd): what the per-kernel timing below uses
     call = GDNCall(keep=True)
+    xd = {n: t.detach() for n, t in x.items()}
 
-    def step():
-        call.forward(x["q"], x["k"], x["v"], x["g"], x["beta"], None, None, False, None, False)
-        call.backward(x["do"], None)
+    def step_direct():
+        call.forward(xd["q"], xd["k"], xd["v"], xd["g"], xd["beta"], None, None, False, None, False)
+        call.backward(xd["do"], None)
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    dt = (time.perf_counter() - t0) / args.steps
+    dt_direct = timed(step_direct)
 
     tokens = B * T
     # whole-op algorithmic work per token and head: fwd 6CK+4CV+6KV+(2/3)C^2 flops, x3 for fwd+bwd;
@@ -378,7 +411,14 @@ def main():
     else:
         roof = {"bound": "hbm", "achieved": b_c * units / stages[dom] / 1e9, "peak": PEAK_HBM / 1e9, "unit": "GB/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = MEASURED_TRAFFIC.get(STAGE_NAMES[dom])
+    # the same roofline for the whole op on its minimal traffic (every input read once, every output written once):
+    # `frac` above is the dominant kernel on ITS bytes, which include intermediates the pipeline writes and re-reads
+    roof["frac_whole_op"] = bytes_ / dt / PEAK_HBM
+    roof["mfma_frac_whole_op"] = flops / dt / PEAK_MFMA_BF16
+    fresh = kernel_sources_sha16() == TRAFFIC_SOURCES_SHA16
+    roof["traffic"] = MEASURED_TRAFFIC.get(STAGE_NAMES[dom]) if fresh else None
+    if not fresh:
+        roof["traffic_note"] = "kernel sources changed since the counters were read: not re-measured"
     roof["kernel"] = STAGE_NAMES[dom]
     roof["kernel_us"] = stages[dom] * 1e6
     roof["flops_per_launch"] = f_c * units
@@ -387,7 +427,7 @@ def main():
     rec = {
         "metric": "chunk GDN fwd+bwd tokens/s @T=8k,H=16,D=128 bf16; % bf16 MFMA peak",
         "value": tokens / dt, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": dt * 1e3, "ms_per_step_call_object": dt_direct * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "chunk_gated_delta_rule fwd+bwd B=4 H=16 T=8192 K=V=128 (contract config 4 of 5)",
                    "B": B, "T": T, "H": H, "K": K, "V": V, "chunk": CH},

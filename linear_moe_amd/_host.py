@@ -82,7 +82,7 @@ def _aligned(x: torch.Tensor) -> torch.Tensor:
 
 class SeqPlan:
     """Chunk bookkeeping of one call: number of sequences / chunks and, for packed input,
-    the device tables the kernels index with."""
+    the device tables the kernels index with.  Build through ``seq_plan`` (cached)."""
 
     def __init__(self, B: int, T: int, cu_seqlens: Optional[torch.Tensor], device):
         self.cu = None
@@ -92,6 +92,10 @@ class SeqPlan:
             self.N = B
             self.NT = B * ((T + CHUNK - 1) // CHUNK)
             return
+        if cu_seqlens.is_cuda and torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("cu_seqlens has no chunk plan yet and one cannot be built while a HIP graph is being "
+                               "captured (it reads the offsets on the host): call the op once with this cu_seqlens "
+                               "tensor, or linear_moe_amd.prepare_cu_seqlens(cu_seqlens, T), before the capture")
         cu_host = cu_seqlens.detach().to("cpu", torch.int64)
         if cu_host.dim() != 1 or cu_host.numel() < 2:
             raise ValueError("cu_seqlens must be a 1-D tensor of N+1 offsets")
@@ -109,6 +113,36 @@ class SeqPlan:
         self.cu = cu_host.to(torch.int32).to(device)
         self.chunk_map = cmap.to(device)
         self.seq_chunk0 = c0.to(torch.int32).to(device)
+
+
+# Plans of the cu_seqlens tensors seen last, newest first.  An entry holds the tensor itself (so its address cannot be
+# reused by another tensor while the entry lives) and its version counter (an in-place change makes a new plan).
+# One packed batch is used by the forward and the backward of every layer: only the first of those calls reads the
+# offsets on the host; the others -- and everything replayed from a HIP graph -- involve no host synchronisation.
+_PLAN_CACHE: list = []
+_PLAN_CACHE_SIZE = 8
+
+
+def seq_plan(B: int, T: int, cu_seqlens: Optional[torch.Tensor], device) -> SeqPlan:
+    if cu_seqlens is None:
+        return SeqPlan(B, T, None, device)
+    for i, (cu, version, t, dev, plan) in enumerate(_PLAN_CACHE):
+        if cu is cu_seqlens and version == cu_seqlens._version and t == T and dev == device:
+            if i:
+                _PLAN_CACHE.insert(0, _PLAN_CACHE.pop(i))
+            return plan
+    plan = SeqPlan(B, T, cu_seqlens, device)
+    _PLAN_CACHE.insert(0, (cu_seqlens, cu_seqlens._version, T, device, plan))
+    del _PLAN_CACHE[_PLAN_CACHE_SIZE:]
+    return plan
+
+
+def prepare_cu_seqlens(cu_seqlens: torch.Tensor, T: int, device=None) -> SeqPlan:
+    """Build (and cache) the chunk tables of a packed batch ahead of its first use, e.g. before a HIP graph capture or
+    off the critical path of a step.  ``T`` is the total number of tokens (``cu_seqlens[-1]``)."""
+    if device is None:
+        device = cu_seqlens.device if cu_seqlens.is_cuda else torch.device("cuda", torch.cuda.current_device())
+    return seq_plan(1, T, cu_seqlens, device)
 
 
 def _state_check(x: Optional[torch.Tensor], N, H, K, V, name: str) -> Optional[torch.Tensor]:

@@ -551,7 +551,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
     if (threadIdx.x < 64) {
       const int cid = it / a.H, h = it % a.H;
       const ChunkInfo ci = chunk_info(a, cid);
-      const int j = threadIdx.x;
+      // refreshed: the LDS addresses derived from it are otherwise hoisted out of the item loop and spilled
+      const int j = fresh_index(threadIdx.x) & 63;
       float x = 0.f;
       if (j < ci.len) {
         ((float*)a.dbeta.ptr)[row_off(a.dbeta, ci.b, ci.tok + j, h)] = s_dbeta[0][j] + s_dbeta[1][j];

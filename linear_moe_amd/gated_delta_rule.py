@@ -16,7 +16,7 @@ import torch
 
 from . import _lib
 from .l2norm import l2_norm
-from ._host import (SeqPlan, _aligned, _check_inputs, _desc, _state_check, base_args, no_tokens, ptr, stream_ptr)
+from ._host import (seq_plan, _aligned, _check_inputs, _desc, _state_check, base_args, no_tokens, ptr, stream_ptr)
 
 
 def _scalar_dt(x: torch.Tensor) -> int:
@@ -43,7 +43,7 @@ class GDNCall:
         dims = _check_inputs(q, k, v, head_first, cu_seqlens)
         B, T, H, K, V = dims
         q, k, v = _aligned(q), _aligned(k), _aligned(v)
-        plan = SeqPlan(B, T, cu_seqlens, q.device)
+        plan = seq_plan(B, T, cu_seqlens, q.device)
         want = (B, H, T) if head_first else (B, T, H)
         if beta is None or tuple(beta.shape) != want:
             raise ValueError(f"beta must have shape {want}")

@@ -13,7 +13,7 @@ from typing import Optional, Tuple
 import torch
 
 from . import _lib
-from ._host import (SeqPlan, _aligned, _check_inputs, _desc, _state_check, base_args, no_tokens, ptr, stream_ptr)
+from ._host import (seq_plan, _aligned, _check_inputs, _desc, _state_check, base_args, no_tokens, ptr, stream_ptr)
 
 
 class GLACall:
@@ -40,7 +40,7 @@ class GLACall:
         if q.dtype == torch.float32 or g.dtype not in (torch.float32, torch.bfloat16):
             g = g.float()
         q, k, v, g = _aligned(q), _aligned(k), _aligned(v), _aligned(g)
-        plan = SeqPlan(B, T, cu_seqlens, q.device)
+        plan = seq_plan(B, T, cu_seqlens, q.device)
         h0 = _state_check(initial_state, plan.N, H, K, V, "initial_state")
         a = base_args(q, k, v, head_first, scale, plan, dims)
         self._gate(a, g, head_first)

@@ -15,7 +15,7 @@ from typing import Optional, Tuple
 import torch
 
 from . import _lib
-from ._host import SeqPlan, _aligned, _check_inputs, _desc, _state_check, base_args, ptr, stream_ptr
+from ._host import seq_plan, _aligned, _check_inputs, _desc, _state_check, base_args, ptr, stream_ptr
 from .delta_rule import chunk_delta_rule
 from .gated_delta_rule import chunk_gated_delta_rule
 from .gla import chunk_gla
@@ -38,7 +38,7 @@ def _recurrent(op, q, k, v, g, beta, scale, initial_state, output_final_state, c
     dims = _check_inputs(q, k, v, head_first, cu_seqlens)
     B, T, H, K, V = dims
     q, k, v = _aligned(q.detach()), _aligned(k.detach()), _aligned(v.detach())
-    plan = SeqPlan(B, T, cu_seqlens, q.device)
+    plan = seq_plan(B, T, cu_seqlens, q.device)
     a = base_args(q, k, v, head_first, scale, plan, dims)
     tok = (B, H, T) if head_first else (B, T, H)
     a.gate = _lib.GATE_NONE

@@ -13,7 +13,7 @@ from typing import Optional, Tuple
 import torch
 
 from . import _lib
-from ._host import (SeqPlan, _aligned, _check_inputs, _desc, _state_check, base_args, no_tokens, ptr, stream_ptr)
+from ._host import (seq_plan, _aligned, _check_inputs, _desc, _state_check, base_args, no_tokens, ptr, stream_ptr)
 
 
 class SimpleGLACall:
@@ -34,7 +34,7 @@ class SimpleGLACall:
         dims = _check_inputs(q, k, v, head_first, cu_seqlens)
         B, T, H, K, V = dims
         q, k, v = _aligned(q), _aligned(k), _aligned(v)
-        plan = SeqPlan(B, T, cu_seqlens, q.device)
+        plan = seq_plan(B, T, cu_seqlens, q.device)
         if g is not None:
             want = (B, H, T) if head_first else (B, T, H)
             if tuple(g.shape) != want:

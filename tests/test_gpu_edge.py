@@ -102,23 +102,33 @@ def test_no_tokens_at_all(cuda, op):
     assert torch.equal(h0.grad, dht)
 
 
-def test_forward_and_backward_can_be_captured_in_a_graph(cuda):
+@pytest.mark.parametrize("packed", [False, True])
+def test_forward_and_backward_can_be_captured_in_a_graph(cuda, packed):
     """The library allocates nothing and launches only on the stream it is given, so a forward + backward of the
     gated delta rule can be captured into a HIP graph; every replay (with eager work between the replays)
-    reproduces the eager results bit for bit."""
+    reproduces the eager results bit for bit.  Packed input too: the chunk tables of a cu_seqlens tensor are built
+    by the first (eager) call that sees it, and no later call reads the offsets on the host."""
+    from linear_moe_amd import _host
     from linear_moe_amd.gated_delta_rule import GDNCall
-    B, T, H, K, V = 2, 300, 2, 128, 128
+    B, T, H, K, V = (1, 600, 2, 128, 128) if packed else (2, 300, 2, 128, 128)
     dt = torch.bfloat16
     q, k = gen(3200, B, T, H, K, dtype=dt).to(cuda), F.normalize(gen(3201, B, T, H, K), dim=-1).to(dt).to(cuda)
     v, do = gen(3202, B, T, H, V, dtype=dt).to(cuda), gen(3203, B, T, H, V, dtype=dt).to(cuda)
     g, beta = F.logsigmoid(gen(3204, B, T, H)).to(cuda), torch.sigmoid(gen(3205, B, T, H)).to(dt).to(cuda)
+    cu = torch.tensor([0, 70, 70, 333, 600], dtype=torch.int32, device=cuda) if packed else None
+    N = 4 if packed else B
+    h0 = (0.1 * gen(3206, N, H, K, V)).to(cuda) if packed else None
+    dht = gen(3207, N, H, K, V).to(cuda) if packed else None
     call = GDNCall(keep=True)
 
     def step():
-        o, _ = call.forward(q, k, v, g, beta, None, None, False, None, False)
-        return (o,) + tuple(x for x in call.backward(do, None) if x is not None)
+        o, ht = call.forward(q, k, v, g, beta, None, h0, packed, cu, False)
+        return (o,) + ((ht,) if packed else ()) + tuple(x for x in call.backward(do, dht) if x is not None)
 
     ref = [x.clone() for x in step()]
+    if packed:                                          # the plan is cached now: no call below builds one
+        n_plans = len(_host._PLAN_CACHE)
+        assert any(e[0] is cu for e in _host._PLAN_CACHE)
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
@@ -134,6 +144,13 @@ def test_forward_and_backward_can_be_captured_in_a_graph(cuda):
         graph.replay()
         torch.cuda.synchronize()
         assert all(torch.equal(a, b) for a, b in zip(outs, ref))
+    if packed:
+        assert len(_host._PLAN_CACHE) == n_plans
+        # a cu_seqlens tensor without a plan cannot get one during a capture: a clear error, not a sync inside it
+        g2 = torch.cuda.CUDAGraph()
+        with pytest.raises(RuntimeError, match="before the capture"):
+            with torch.cuda.graph(g2):
+                call.forward(q, k, v, g, beta, None, h0, True, cu.clone(), False)
 
 
 @pytest.mark.parametrize("op", OPS)

@@ -81,6 +81,11 @@ BWD_CASES = [
     (1, 256, 2, 128, 128, False, False, True),
     (1, 130, 2, 64, 128, True, True, True),
     (1, 3, 1, 64, 64, True, False, False),
+    # K = 64, V = 128 time-first over several chunks with a partial one: the shape on which a build of the
+    # chunk-parallel backward that refreshed the lane index once per helper call (instead of once per item) gave
+    # wrong dq, dk in fp32 -- kept as a fixed case (the random trials reach this shape only by chance of the seed)
+    (2, 330, 3, 64, 128, True, False, False),
+    (1, 200, 2, 128, 64, False, False, True),
 ]
 
 

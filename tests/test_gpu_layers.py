@@ -1,0 +1,42 @@
+"""The token-mixer layer composed end to end on the GPU kernels, in the reference's order of operations
+(tests/layers.py: LinearAttention.forward around GatedDeltaNet.forward / GLA.forward), forward and every gradient
+(hidden states and all parameters) against the same chain of fp64 oracle functions."""
+import pytest
+import torch
+
+from tests.layers import GatedDeltaNetLayer, GLALayer
+from tests.util import gen, max_abs_rel
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("kind", ["gated_deltanet", "gla"])
+def test_layer_matches_the_oracle_chain(cuda, kind, dtype):
+    hidden, H, D, T, B = 256, 2, 128, 200, 2
+    layer = (GatedDeltaNetLayer if kind == "gated_deltanet" else GLALayer)(hidden, H, D, seed=5)
+    x = gen(5100, T, B, hidden)
+    dy = gen(5101, T, B, hidden)
+    # oracle: fp64 on the CPU, on the parameters and inputs as the device sees them (rounded to dtype once)
+    ref_layer = (GatedDeltaNetLayer if kind == "gated_deltanet" else GLALayer)(hidden, H, D, seed=5)
+    if dtype == torch.bfloat16:
+        with torch.no_grad():
+            for p in ref_layer.parameters():
+                if p.dim() == 2 or p is getattr(ref_layer, "gk_bias", None) or p is getattr(ref_layer, "norm_weight", None):
+                    p.copy_(p.to(dtype).float())            # the projections run in dtype; A_log, dt_bias stay fp32
+    xr = x.to(dtype).double().requires_grad_(True)
+    yr = ref_layer.oracle_forward(xr)
+    ref_params = dict(ref_layer.named_parameters())
+    ref_grads = torch.autograd.grad((yr * dy.double()).sum(), [xr] + list(ref_params.values()))
+    layer = layer.to(cuda)
+    xd = x.to(dtype).to(cuda).requires_grad_(True)
+    y = layer(xd)
+    assert y.shape == (T, B, hidden) and y.dtype == dtype
+    grads = torch.autograd.grad((y * dy.to(dtype).to(cuda)).sum(), [xd] + list(layer.parameters()))
+    torch.cuda.synchronize()
+    # the chain has six roundings to dtype between the projections and the output; the bars are those of the ops
+    tol = 1e-4 if dtype == torch.float32 else 4e-2
+    assert max_abs_rel(y.detach().cpu(), yr.detach()) < tol
+    names = ["x"] + list(ref_params)
+    for n, gd, gr in zip(names, grads, ref_grads):
+        assert max_abs_rel(gd.cpu(), gr) < tol, n

@@ -133,6 +133,31 @@ def test_seq_plan_tables():
             SeqPlan(1, 270, torch.tensor(bad), "cpu")
 
 
+def test_seq_plan_is_built_once_per_cu_seqlens_tensor():
+    """The chunk tables of a packed batch are built on the first call that sees its cu_seqlens tensor; later calls with
+    the same tensor (the other layers, the backward, every step that reuses the batch) take them from the cache without
+    touching the offsets -- no host read, hence no synchronisation.  An in-place change or another tensor with equal
+    contents makes a new plan."""
+    from linear_moe_amd import _host
+    _host._PLAN_CACHE.clear()
+    cu = torch.tensor([0, 1, 65, 200], dtype=torch.int32)
+    p1 = _host.seq_plan(1, 200, cu, "cpu")
+    assert _host.seq_plan(1, 200, cu, "cpu") is p1
+    other = cu.clone()
+    p2 = _host.seq_plan(1, 200, other, "cpu")
+    assert p2 is not p1 and p2.chunk_map.tolist() == p1.chunk_map.tolist()
+    assert _host.seq_plan(1, 200, cu, "cpu") is p1                 # still cached behind the newer entry
+    cu[1] = 2                                                      # in-place change: the version counter moves
+    p3 = _host.seq_plan(1, 200, cu, "cpu")
+    assert p3 is not p1 and p3.cu.tolist() == [0, 2, 65, 200]
+    for i in range(_host._PLAN_CACHE_SIZE + 3):                    # bounded
+        _host.seq_plan(1, 200, torch.tensor([0, 100 + i, 200]), "cpu")
+    assert len(_host._PLAN_CACHE) == _host._PLAN_CACHE_SIZE
+    assert _host.prepare_cu_seqlens(other, 200, "cpu").NT == 1 + 1 + 3
+    with pytest.raises(ValueError):
+        _host.seq_plan(1, 201, other, "cpu")                       # another T: validated afresh
+
+
 def test_python_layer_validates_before_launch():
     import linear_moe_amd as L
     q = torch.zeros(1, 2, 8, 64)
