@@ -104,15 +104,17 @@ def time_stages(call, lib, reps):
     out = {}
     for stage in (0, 1, 4, 5):         # stages 2, 3 (separate output / dv kernels) are not part of this op
         a = call.fwd_args if stage <= 2 else call.bwd_args
-        for _ in range(2):
+        n_warm = max(2, reps // 2)
+        n_timed = max(1, reps - n_warm)
+        for _ in range(n_warm):
             _lib.check(lib.lmoe_launch_stage(C.byref(a), call.OP, stage, st), "stage")
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        for _ in range(reps):
+        for _ in range(n_timed):
             lib.lmoe_launch_stage(C.byref(a), call.OP, stage, st)
         e1.record()
         e1.synchronize()
-        out[stage] = e0.elapsed_time(e1) * 1e-3 / reps
+        out[stage] = e0.elapsed_time(e1) * 1e-3 / n_timed
     return out
 
 
@@ -325,7 +327,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--stage-reps", type=int, default=20)
+    ap.add_argument("--stage-reps", type=int, default=40)
     ap.add_argument("--neighbours", action="store_true",
                     help="instead of the headline step: the row-wise kernels around the op (L2 norm, SiLU + L2 norm, "
                          "RMS norm with and without the swish gate) on the rows of the same workload, one JSON line")
@@ -381,9 +383,7 @@ def main():
         o, _ = chunk_gated_delta_rule(*leaves, None, None, False, None, False)
         torch.autograd.grad([o], leaves, [x["do"]])
 
-    dt = timed(step_public)
-
-    # the same kernels driven through the call object (no autograd): what the per-kernel timing below uses
+    # the same kernels driven through the call object (no autograd): what the per-kernel timing uses
     call = GDNCall(keep=True)
     xd = {n: t.detach() for n, t in x.items()}
 
@@ -391,7 +391,17 @@ def main():
         call.forward(xd["q"], xd["k"], xd["v"], xd["g"], xd["beta"], None, None, False, None, False)
         call.backward(xd["do"], None)
 
+    # What runs first after start-up is slow: the first 25 or so steps on a GPU that has been idle (even for 0.2 s),
+    # on memory the allocator has just obtained, take up to 8 % longer than every later one (measured: step by
+    # step the time falls from 1.3x to 1.0x over about 30 steps, and rises again after a pause or after
+    # torch.cuda.empty_cache(); single kernels and whole steps alike).  The op lives inside long training runs, so
+    # `value` is the steady-state figure: the timed region (`warmup` untimed steps, then exactly `steps` timed ones)
+    # is run twice back to back, the second pass is reported, and the first is kept in the record as
+    # ms_per_step_first_pass.
+    dt_first = timed(step_public)
+    dt = timed(step_public)
     dt_direct = timed(step_direct)
+    stages = time_stages(call, lib, args.stage_reps)
 
     tokens = B * T
     # whole-op algorithmic work per token and head: fwd 6CK+4CV+6KV+(2/3)C^2 flops, x3 for fwd+bwd;
@@ -400,7 +410,6 @@ def main():
     b_tok = (6 * K + 5 * V) * 2 + 3 * 2 + 12
     flops, bytes_ = f_tok * tokens * H, b_tok * tokens * H
 
-    stages = time_stages(call, lib, args.stage_reps)
     dom = max(stages, key=stages.get)
     f_c, b_c = stage_model(dom, K, V)
     units = (B * T // CH) * H
@@ -429,6 +438,9 @@ def main():
         "value": tokens / dt, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": dt * 1e3, "ms_per_step_call_object": dt_direct * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
+        "ms_per_step_first_pass": dt_first * 1e3,
+        "order": "the timed region (warmup + steps) runs twice back to back; value is the second pass (steady state), "
+                 "ms_per_step_first_pass the first (GPU just woken up, memory just allocated)",
         "config": {"workload": "chunk_gated_delta_rule fwd+bwd B=4 H=16 T=8192 K=V=128 (contract config 4 of 5)",
                    "B": B, "T": T, "H": H, "K": K, "V": V, "chunk": CH},
         "mfma_frac": flops / dt / PEAK_MFMA_BF16, "hbm_frac_algorithmic": bytes_ / dt / PEAK_HBM,
