@@ -248,6 +248,56 @@ def neighbours(lib, rows, D, dev, reps):
             "config": {"workload": f"{rows} rows x {D} bf16 (q / k / o rows of B=4 H=16 T=8192)"}, "kernels": res}
 
 
+def trace_state_fwd(lib, x, dims, work_group=16):
+    """Per-phase breakdown of one chunk period of the forward sequential pass (k_gdn_state_fwd_reg) on the headline
+    workload: the traced instance of the kernel records the shader clock where each team of the traced work-group
+    arrives at and leaves the two barriers of a chunk and at a few points in between
+    (lmoe_trace_gdn_state_fwd, include/lmoe.h).  Returns averages over the middle chunks of the sequence, in cycles
+    after the release of barrier 1 of the same chunk (negative: before it, i.e. in the previous chunk's phase 2)."""
+    import torch
+    from linear_moe_amd import _lib
+    from linear_moe_amd.gated_delta_rule import GDNCall
+    B, T, H, K, V = dims
+    call = GDNCall(keep=True)
+    call.forward(x["q"], x["k"], x["v"], x["g"], x["beta"], None, None, False, None, False)
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    slots, chunks, marks = 4, 128, 8
+    tr = torch.zeros(slots * chunks * marks, dtype=torch.int64, device=x["q"].device)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for _ in range(3):
+        _lib.check(lib.lmoe_trace_gdn_state_fwd(C.byref(call.fwd_args), tr.data_ptr(), work_group, st), "trace")
+    e0.record()
+    _lib.check(lib.lmoe_trace_gdn_state_fwd(C.byref(call.fwd_args), tr.data_ptr(), work_group, st), "trace")
+    e1.record()
+    e1.synchronize()
+    traced_us = e0.elapsed_time(e1) * 1e3
+    t = tr.cpu().view(slots, chunks, marks).double()
+    nch = min(chunks, (T + CH - 1) // CH)
+    c0, c1 = nch // 4, nch - nch // 4
+    ref = t[0, c0:c1, 1]                                          # the consumer leaves barrier 1
+    period = float((t[0, c0 + 1:c1 + 1, 1] - t[0, c0:c1, 1]).mean())
+    names = {0: {0: "arrives_b1", 1: "leaves_b1", 5: "kS_formed", 2: "arrives_b2_vnew_written", 3: "leaves_b2",
+                 6: "state_updated", 4: "state_written"},
+             1: {0: "arrives_b1", 1: "leaves_b1", 2: "arrives_b2_qS_formed", 3: "leaves_b2", 4: "o_written"},
+             2: {0: "arrives_b1", 1: "leaves_b1", 2: "arrives_b2_tiles_staged", 3: "leaves_b2", 4: "stores_issued",
+                 5: "loads_issued"},
+             3: {0: "arrives_b1", 1: "leaves_b1", 2: "arrives_b2_loads_issued", 3: "leaves_b2", 4: "tiles_staged"}}
+    teams = {0: "consumer_wave", 1: "helper_wave", 2: "loader_team_1", 3: "loader_team_2"}
+    out = {}
+    for s_, nm in teams.items():
+        out[nm] = {}
+        for m, label in names[s_].items():
+            d = float((t[s_, c0:c1, m] - ref).mean())
+            if m == 0:
+                d += period                                      # arrival at barrier 1 of the NEXT chunk
+                label = "arrives_next_b1"
+            out[nm][label] = round(d)
+    return {"metric": "k_gdn_state_fwd_reg: shader-clock cycles after barrier 1 of a chunk, per team (traced build)",
+            "unit": "cycles", "work_group": work_group, "chunks_averaged": [c0, c1], "period_cycles": round(period),
+            "traced_kernel_us": round(traced_us, 1), "cycles_per_us": round(period * nch / traced_us, 1),
+            "teams": out}
+
+
 def other_configs(dev, steps, warmup):
     """The four contract configurations beside the headline one, through the Python entry points (inputs of
     the contract's laws, drawn on the GPU: this leg times, the parity tests check): ms per call, tokens/s and
@@ -331,6 +381,9 @@ def main():
     ap.add_argument("--neighbours", action="store_true",
                     help="instead of the headline step: the row-wise kernels around the op (L2 norm, SiLU + L2 norm, "
                          "RMS norm with and without the swish gate) on the rows of the same workload, one JSON line")
+    ap.add_argument("--trace-state-fwd", action="store_true",
+                    help="instead of the headline step: the per-phase breakdown of one chunk period of the forward "
+                         "sequential pass on the headline workload, one JSON line")
     ap.add_argument("--other-configs", action="store_true",
                     help="instead of the headline step: contract configurations 1, 2, 3 and 5, one JSON line")
     args = ap.parse_args()
@@ -355,6 +408,9 @@ def main():
         print(json.dumps(other_configs(dev, args.steps, args.warmup)))
         return
     x = gdn_inputs(B, T, H, K, V, seed, torch.bfloat16, dev)
+    if args.trace_state_fwd:
+        print(json.dumps(trace_state_fwd(lib, x, (B, T, H, K, V))))
+        return
 
     # known-size device copy: the yardstick for the FETCH_SIZE / WRITE_SIZE counters under rocprofv3
     src = torch.empty(CALIB_COPY_BYTES, dtype=torch.uint8, device=dev).fill_(1)

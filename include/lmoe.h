@@ -70,7 +70,9 @@ typedef struct lmoe_args {
   /* intermediates written by *_fwd and read by *_bwd (caller-allocated, element type = dtype) */
   void* hs;            /* state at the start of every chunk: [NT,H,V,K] (transposed) for
                           simple_gla and the gated delta rule, [NT,H,K,V] for chunk_gla    */
-  lmoe_tensor vnew;    /* [B,T,H,V]   delta-rule pseudo values (gated delta rule)      */
+  lmoe_tensor vnew;    /* delta-rule pseudo values (gated delta rule): only .ptr is used, the layout is the
+                          library's: [NT,H,V/32,64,32] (chunk, head, 32-column slice, token in chunk, column),
+                          NT*H*64*V elements                                                          */
   lmoe_tensor w;       /* [B,T,H,K]   WY factor w (gated delta rule)                   */
   lmoe_tensor u;       /* [B,T,H,V]   WY factor u (gated delta rule; forward only)     */
   void* tinv;          /* [NT,H,64,64] (I + L)^-1 per chunk (gated delta rule)         */
@@ -92,7 +94,7 @@ typedef struct lmoe_args {
   float* dh0;          /* [N,H,K,V] fp32 or NULL                                       */
   /* backward workspace (caller-allocated, element type = dtype) */
   void* dhs;           /* gradient w.r.t. the state at the END of every chunk, laid out as hs */
-  lmoe_tensor dvnew;   /* [B,T,H,V]   gradient of vnew (gated delta rule)              */
+  lmoe_tensor dvnew;   /* gradient of vnew (gated delta rule): .ptr only, laid out as vnew */
 } lmoe_args;
 
 /* Library version (major*10000 + minor*100 + patch). */
@@ -259,6 +261,21 @@ int lmoe_mom_rowdot(const void* src, const int32_t* idx, const void* g, void* dw
 #define LMOE_OP_GLA 1
 #define LMOE_OP_GATED_DELTA_RULE 2
 int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* stream);
+
+/* Per-phase timing of the forward sequential pass of the gated delta rule (profiling support; no counterpart in the
+ * reference).  Runs the pass once for the problem `a` (the fully populated argument block of
+ * lmoe_chunk_gated_delta_rule_fwd, after its WY preparation has run: lmoe_launch_stage stage 0) with the instance
+ * that records the shader clock in work-group `work_group`, and leaves in `trace` (device memory,
+ * int64 [4 slots][128 chunks][8 marks], zero where nothing was recorded; sequences longer than 128 chunks are traced
+ * for their first 128) the cycle counter at these points of every chunk:
+ *   slot 0, the consumer wave (carries the state):  0 arrives at barrier 1, 1 leaves it, 5 k S formed, 2 arrives at
+ *           barrier 2 (v_new written), 3 leaves it, 6 state updated, 4 state written for the next chunk
+ *   slot 1, the helper wave (forms the output):     0, 1, 2 (q S formed), 3 as above, 4 o written
+ *   slot 2, loader team 1 (k, P; all stores):       0, 1, 2 (tiles staged, results lifted), 3, 4 stores issued,
+ *           5 loads issued
+ *   slot 3, loader team 2 (q, Tinv, v, gates):      0, 1, 2 loads issued, 3, 4 tiles staged
+ * Instance available for LMOE_BF16, K = V = 128, with tinv and hs given (-24 otherwise). */
+int lmoe_trace_gdn_state_fwd(const lmoe_args* a, int64_t* trace, int32_t work_group, void* stream);
 
 /* Token-by-token forward of an op (op = LMOE_OP_*; the delta rule without a gate: gate = LMOE_GATE_NONE):
  * the state stays in registers, nothing is saved for a backward.  For decoding (T = 1 with h0 / ht) and

@@ -19,6 +19,7 @@ import sys
 # preparation two or three work-groups of 4 waves)
 GUARDED = {
     "k_gdn_state_fwd": 3,
+    "k_gdn_state_fwd_reg": 3,
     "k_gdn_state_bwd": 3,
     "k_gdn_bwd_chunk": 3,
     "k_gdn_wy_fwd": 2,
@@ -55,7 +56,7 @@ def main(paths):
                 # Itanium mangling: <len><name>I<template args>; DF16b = __bf16
                 if f"{len(kern)}{kern}I" not in name:
                     continue
-                two_byte = f"{kern}IDF16b" in name
+                two_byte = f"{kern}IDF16b" in name or kern.endswith("_reg")     # the _reg kernels exist for bf16 only
                 line = (f"{kern:<18} {'bf16' if two_byte else 'fp32'} vgpr {r.get('vgpr', -1):3d} agpr {r.get('agpr', -1):3d} "
                         f"scratch {r.get('scratch', -1):4d} B  vgpr-spill {r.get('vspill', -1):3d}  waves/SIMD {r.get('occ', -1)}  "
                         f"lds {r.get('lds', -1)}  {name}")

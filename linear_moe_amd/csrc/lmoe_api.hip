@@ -58,7 +58,8 @@ int64_t lmoe_workspace_bytes(int32_t op, int32_t dtype, int32_t part, int32_t B,
   int64_t n = states;                                                    // hs | dhs
   if (op == LMOE_OP_GLA && part == 0) n += tiles + 2 * (int64_t)NT * H * LMOE_CHUNK * K;   // amat, qe, ke
   // vnew, tinv, pmat, and for 4-byte elements u, w (the 2-byte state passes form them on the chip) | dvnew
-  if (op == LMOE_OP_GATED_DELTA_RULE) n += part == 0 ? rows_v + 2 * tiles + (s == 4 ? rows_v + rows_k : 0) : rows_v;
+  const int64_t blocks_v = (int64_t)NT * H * LMOE_CHUNK * V;             // vnew | dvnew: whole chunks, [NT,H,V/32,64,32]
+  if (op == LMOE_OP_GATED_DELTA_RULE) n += part == 0 ? blocks_v + 2 * tiles + (s == 4 ? rows_v + rows_k : 0) : blocks_v;
   int64_t bytes = n * s;
   if (op == LMOE_OP_GATED_DELTA_RULE && part == 0) bytes += (int64_t)NT * H * 2 * LMOE_CHUNK * 4;   // gcum (fp32)
   if (op == LMOE_OP_GLA && part == 0) bytes += (int64_t)NT * H * K * 4;                              // gcum (fp32)
@@ -244,6 +245,18 @@ int lmoe_rmsnorm_bwd_noalloc(const void* x, const void* w, const void* gate, con
     return fail(-23, "%s: %lld partial rows of %d floats exceed the library's scratch (%lld floats); use lmoe_rmsnorm_bwd "
                      "with a caller-allocated dw_part", nm, (long long)(need / D), D, (long long)cap);
   lmoe::launch_rmsnorm(dtype, D, x, w, gate, dy, dx, dgate, nullptr, part, dw, rows, eps, true, (hipStream_t)stream);
+  return launched(nm);
+}
+
+int lmoe_trace_gdn_state_fwd(const lmoe_args* a, int64_t* trace, int32_t work_group, void* stream) {
+  const char* nm = "lmoe_trace_gdn_state_fwd";
+  if (int r = check_common(a, nm)) return r;
+  if (!trace) return fail(-1, "%s: trace must not be null", nm);
+  if (a->gate == LMOE_GATE_VECTOR || !a->beta.ptr || !a->o.ptr || !a->pmat || !a->gcum || !a->vnew.ptr)
+    return fail(-11, "%s: needs the populated argument block of lmoe_chunk_gated_delta_rule_fwd", nm);
+  if (a->NT == 0 || a->N == 0) return fail(-4, "%s: nothing to trace in an empty problem", nm);
+  if (!lmoe::launch_gdn_state_fwd_trace(*a, (long long*)trace, work_group, (hipStream_t)stream))
+    return fail(-24, "%s: traced instance exists for bf16, K = V = 128 with tinv and hs given, work_group inside the grid", nm);
   return launched(nm);
 }
 

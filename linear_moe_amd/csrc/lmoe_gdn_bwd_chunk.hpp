@@ -146,11 +146,14 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
       R.len = ci.len;
       if constexpr (unit < NS) {
         constexpr int vv = unit * BVH;
+        static_assert(BVH == SLICE_COLS, "a slice of this kernel is one block of vnew / dvnew");
         const lmoe_tensor* ts[4] = {&a.d_o, &a.vnew, &a.dvnew, &a.v};
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
           typename IOV::Regs r;
-          IOV::load_nomask(r, row_ptr<T>(*ts[t], ci.b, ci.tok, h) + vv, ts[t]->st, ci.len, tid);
+          // do, v: the caller's rows; vnew, dvnew: one contiguous block per (chunk, head, slice)
+          if (t == 1 || t == 2) IOV::load_nomask(r, slice_ptr<T>(*ts[t], cid, h, a.H, V, vv), SLICE_COLS, ci.len, tid);
+          else IOV::load_nomask(r, row_ptr<T>(*ts[t], ci.b, ci.tok, h) + vv, ts[t]->st, ci.len, tid);
 #pragma unroll
           for (int p = 0; p < PV; ++p) R.v[t * PV + p] = r.v[p];
         }

@@ -1,6 +1,7 @@
 // Instantiation and launch of the sequential passes of the gated delta rule.
 #include "lmoe_launch.hpp"
 #include "lmoe_gdn_state.hpp"
+#include "lmoe_gdn_state_reg.hpp"
 
 namespace lmoe {
 
@@ -16,6 +17,13 @@ template <typename T, int K, int V, int BV> void launch_fwd(const lmoe_args& a, 
   // w formed on the chip from Tinv where Tinv is there and LDS has room for a second k tile
   constexpr bool CAN_WT = sizeof(T) == 2;
   const bool wt = CAN_WT && a.tinv != nullptr;
+  if constexpr (CAN_WT && BV == 32) {
+    if (wt) {       // 2-byte elements with Tinv: the state stays in registers (lmoe_gdn_state_reg.hpp)
+      if (a.hs) hipLaunchKernelGGL((k_gdn_state_fwd_reg<K, V, true>), dim3(grid), dim3(3 * NTHR), 0, st, a, (long long*)nullptr, -1);
+      else hipLaunchKernelGGL((k_gdn_state_fwd_reg<K, V, false>), dim3(grid), dim3(3 * NTHR), 0, st, a, (long long*)nullptr, -1);
+      return;
+    }
+  }
   if (a.hs) {
     if (wt) hipLaunchKernelGGL((k_gdn_state_fwd<T, K, V, BV, true, CAN_WT>), dim3(grid), dim3(3 * NTHR), 0, st, a);
     else hipLaunchKernelGGL((k_gdn_state_fwd<T, K, V, BV, true, false>), dim3(grid), dim3(3 * NTHR), 0, st, a);
@@ -31,7 +39,10 @@ template <typename T, int K, int V, int BV> void launch_bwd(const lmoe_args& a, 
 template <typename T, int K, int V> struct GdnStateFwd {
   static void run(const lmoe_args& a, hipStream_t st) {
     constexpr int BW = GdnStateCfg<T>::BV_WIDE <= V ? GdnStateCfg<T>::BV_WIDE : GdnStateCfg<T>::BV;
-    if (wide_slices<T, V>(a)) launch_fwd<T, K, V, BW>(a, st);
+    // the register-resident pass is bound by its products, not by latency: twice the columns take twice as long,
+    // so it keeps the narrow slice (more work-groups) whatever the problem size
+    const bool reg = sizeof(T) == 2 && a.tinv != nullptr;
+    if (!reg && wide_slices<T, V>(a)) launch_fwd<T, K, V, BW>(a, st);
     else launch_fwd<T, K, V, GdnStateCfg<T>::BV>(a, st);
   }
 };
@@ -43,6 +54,14 @@ template <typename T, int K, int V> struct GdnStateBwd {
   }
 };
 void launch_gdn_state_fwd(const lmoe_args& a, hipStream_t st) { dispatch<GdnStateFwd>(a, st); }
+// the traced instance of the register-resident forward pass (2-byte elements, K = V = 128, saving call)
+bool launch_gdn_state_fwd_trace(const lmoe_args& a, long long* tr, int work_group, hipStream_t st) {
+  if (a.dtype != LMOE_BF16 || a.K != 128 || a.V != 128 || !a.tinv || !a.hs) return false;
+  const int grid = ((a.N * a.H + 7) / 8) * 8 * (128 / 32);
+  if (work_group < 0 || work_group >= grid) return false;
+  hipLaunchKernelGGL((k_gdn_state_fwd_reg<128, 128, true, true>), dim3(grid), dim3(3 * NTHR), 0, st, a, tr, work_group);
+  return true;
+}
 void launch_gdn_state_bwd(const lmoe_args& a, hipStream_t st) { dispatch<GdnStateBwd>(a, st); }
 
 }  // namespace lmoe

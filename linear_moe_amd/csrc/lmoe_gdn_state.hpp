@@ -36,20 +36,28 @@ template <typename T> struct GdnStateCfg {
   static constexpr int LPF = sizeof(T) == 2 ? 2 : 1;     // chunks a loader keeps in flight per ring
 };
 
-// Runs step(slot, i) for i = 0 .. n-1 with slot = i % L as a compile-time constant (L = 1 or 2).
+// Runs step(slot, i) for i = 0 .. n-1 with slot = i % L as a compile-time constant.
 // Whole groups of L steps run without an exit in between: an early exit inside a group would be
 // one more path to the loop header, on which the compiler could count only the loads of the
 // first step as issued and would drain the prefetch ring on every trip.
+template <int L, int J = 0, typename F> __device__ __forceinline__ void ring_group(int i, F& step) {
+  if constexpr (J < L) {
+    step(std::integral_constant<int, J>(), i + J);
+    ring_group<L, J + 1>(i, step);
+  }
+}
+template <int L, int J = 0, typename F> __device__ __forceinline__ void ring_tail(int i, int n, F& step) {
+  if constexpr (J < L - 1) {
+    if (i + J < n) {
+      step(std::integral_constant<int, J>(), i + J);
+      ring_tail<L, J + 1>(i, n, step);
+    }
+  }
+}
 template <int L, typename F> __device__ __forceinline__ void ring_loop(int n, F&& step) {
-  static_assert(L == 1 || L == 2, "rings of one or two register sets");
   int i = 0;
-  for (; i + L <= n; i += L) {
-    step(std::integral_constant<int, 0>(), i);
-    if constexpr (L == 2) step(std::integral_constant<int, 1>(), i + 1);
-  }
-  if constexpr (L == 2) {
-    if (i < n) step(std::integral_constant<int, 0>(), i);
-  }
+  for (; i + L <= n; i += L) ring_group<L>(i, step);
+  ring_tail<L>(i, n, step);
 }
 
 // ------------------------------------------------------------------------- //
@@ -166,7 +174,11 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
       lds_barrier();                                                                     // B0: the consumers form w(0)
     }
     typename IOHT::Regs rh;
-    typename IOV::Regs rvn, ro;
+    typename IOV::Regs ro;
+    // v_new leaves in blocks of at most 32 columns (the layout of vnew: see slice_ptr)
+    constexpr int SBW = BV < SLICE_COLS ? BV : SLICE_COLS, NSB = BV / SBW;
+    typedef TileIO<T, CH, SBW> IOS;
+    typename IOS::Regs rvn[NSB];
     ring_loop<LPF>(sq.nchunks, [&](auto slot, const int c) {
       constexpr int j = decltype(slot)::value, jn = (j + 1) % LPF;
       lds_barrier();                                                                     // B1
@@ -182,12 +194,17 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
       lds_barrier();                                                                     // B2
       // v_new of this chunk is complete (the consumers rewrite it after the next B1)
       if constexpr (SAVE) {
-        IOV::load_lds(rvn, s_vn, LDU);
+#pragma unroll
+        for (int sb = 0; sb < NSB; ++sb) IOS::load_lds(rvn[sb], s_vn + SBW * sb, LDU);
         // hs[chunk][h][v0 .. v0+BV][K] <- S^T
         IOHT::template store_global<true>(rh, (T*)a.hs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
       }
       if (c > 0) store_result(ro, a.o, c - 1);
-      if constexpr (SAVE) store_result(rvn, a.vnew, c);
+      if constexpr (SAVE) {
+#pragma unroll
+        for (int sb = 0; sb < NSB; ++sb)
+          IOS::template store_global<true>(rvn[sb], slice_ptr<T>(a.vnew, sq.chunk0 + c, h, a.H, V, v0 + SBW * sb), SLICE_COLS, min(CH, sq.len - c * CH));
+      }
       issue_a(pa[j], c + LPF);
     });
     lds_barrier();                                                                       // o of the last chunk
@@ -440,16 +457,20 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
       IOK::mask(P.rq, P.len);
       IOK::store_lds(P.rq, s_q, LDK);
     };
-    auto store_results = [&](const typename IOV::Regs& rdv, int c) {
-      const int tok = sq.tok0 + c * CH;
+    // dv_new leaves in blocks of at most 32 columns (the layout of dvnew: see slice_ptr)
+    constexpr int SBW = BV < SLICE_COLS ? BV : SLICE_COLS, NSB = BV / SBW;
+    typedef TileIO<T, CH, SBW> IOS;
+    auto store_results = [&](const typename IOS::Regs (&rdv)[NSB], int c) {
       const int len = min(CH, sq.len - c * CH);
-      IOV::template store_global<true>(rdv, row_ptr<T>(a.dvnew, sq.b, tok, h) + v0, a.dvnew.st, len);
+#pragma unroll
+      for (int sb = 0; sb < NSB; ++sb)
+        IOS::template store_global<true>(rdv[sb], slice_ptr<T>(a.dvnew, sq.chunk0 + c, h, a.H, V, v0 + SBW * sb), SLICE_COLS, len);
     };
 #pragma unroll
     for (int j = 0; j < LPF; ++j) issue_a(pa[j], j);
     wait_all_loads();   // see k_gdn_state_fwd
     typename IOHT::Regs rh;
-    typename IOV::Regs rdv;
+    typename IOS::Regs rdv[NSB];
     ring_loop<LPF>(sq.nchunks, [&](auto slot, const int it) {
       constexpr int j = decltype(slot)::value;
       const int c = sq.nchunks - 1 - it;
@@ -459,7 +480,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
       IOHT::load_lds(rh, s_dST, LDK);
       lds_barrier();                                                                     // B2
       // dv_new of this chunk is complete (the consumers rewrite it after the next B1)
-      IOV::load_lds(rdv, s_dvn, LDU);
+#pragma unroll
+      for (int sb = 0; sb < NSB; ++sb) IOS::load_lds(rdv[sb], s_dvn + SBW * sb, LDU);
       IOHT::template store_global<true>(rh, (T*)a.dhs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
       store_results(rdv, c);
       issue_a(pa[j], it + LPF);

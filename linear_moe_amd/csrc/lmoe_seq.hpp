@@ -71,6 +71,16 @@ template <typename T>
 __device__ __forceinline__ T* row_ptr(const lmoe_tensor& x, int b, int tok, int h) {
   return (T*)x.ptr + (int64_t)b * x.sb + (int64_t)tok * x.st + (int64_t)h * x.sh;
 }
+// The pseudo values of the gated delta rule and their gradient (vnew, dvnew) are library-side buffers laid out for the
+// kernels that pass them on, not token-major: [chunk][head][V / 32][64 tokens][32 columns].  A 32-column slice of a
+// chunk is one contiguous 4 KB (2-byte elements) block: the sequential passes write it as whole 128-byte lines
+// (token-major, a slice's rows are 64-byte pieces 4 KB apart) and the chunk-parallel backward reads it in one piece.
+// Pointer to (chunk cid, head h, column v0, token 0); the token stride is SLICE_COLS elements.
+constexpr int SLICE_COLS = 32;
+template <typename T>
+__device__ __forceinline__ T* slice_ptr(const lmoe_tensor& x, int cid, int h, int H, int V, int v0) {
+  return (T*)x.ptr + (((int64_t)cid * H + h) * (V / SLICE_COLS) + v0 / SLICE_COLS) * (CH * SLICE_COLS) + v0 % SLICE_COLS;
+}
 __device__ __forceinline__ int64_t row_off(const lmoe_tensor& x, int b, int tok, int h) {
   return (int64_t)b * x.sb + (int64_t)tok * x.st + (int64_t)h * x.sh;
 }

@@ -71,10 +71,12 @@ class GDNCall:
         # w, u: the bf16 state passes form them on the chip from tinv; only the fp32 forward pass reads them
         w = torch.empty(B, T, H, K, dtype=dt, device=dev) if dt == torch.float32 else None
         u = torch.empty(B, T, H, V, dtype=dt, device=dev) if dt == torch.float32 else None
-        vnew = torch.empty(B, T, H, V, dtype=dt, device=dev) if save else None
+        # library-side layout [chunk, head, 32-column slice, token in chunk, column] (see include/lmoe.h)
+        vnew = torch.empty(max(plan.NT, 1), H, V // 32, 64, 32, dtype=dt, device=dev) if save else None
         a.o, a.ht, a.hs, a.tinv = _desc(o, head_first), ptr(ht), ptr(hs), ptr(tinv)
         a.pmat, a.gcum = pmat.data_ptr(), gcum.data_ptr()
-        a.w, a.u, a.vnew = _desc(w, False), _desc(u, False), _desc(vnew, False)
+        a.w, a.u = _desc(w, False), _desc(u, False)
+        a.vnew.ptr = ptr(vnew)
         _lib.check(lib.lmoe_chunk_gated_delta_rule_fwd(C.byref(a), stream_ptr()), "chunk_gated_delta_rule forward")
         ctx.saved = (q, k, v, g, beta, h0, hs, tinv, pmat, gcum, vnew)
         ctx.fwd_args, ctx.fwd_keep = a, ((o, ht, w, u) if self.keep else None)
@@ -96,7 +98,7 @@ class GDNCall:
         a.beta, a.beta_dtype = _desc(beta, head_first), _scalar_dt(beta)
         a.h0, a.hs, a.tinv, a.pmat = ptr(h0), hs.data_ptr(), tinv.data_ptr(), pmat.data_ptr()
         a.gcum = gcum.data_ptr()
-        a.vnew = _desc(vnew, False)
+        a.vnew.ptr = vnew.data_ptr()
         a.d_o = _desc(do, head_first)
         dht = None if dht is None else dht.float().contiguous()
         a.dht = ptr(dht)
@@ -109,8 +111,9 @@ class GDNCall:
         dh0 = torch.empty_like(h0) if ctx.has_h0 else None
         a.dh0 = ptr(dh0)
         dhs = torch.empty_like(hs)
-        dvnew = torch.empty(B, T, H, V, dtype=dt, device=dev)
-        a.dhs, a.dvnew = dhs.data_ptr(), _desc(dvnew, False)
+        dvnew = torch.empty_like(vnew)
+        a.dhs = dhs.data_ptr()
+        a.dvnew.ptr = dvnew.data_ptr()
         _lib.check(lib.lmoe_chunk_gated_delta_rule_bwd(C.byref(a), stream_ptr()), "chunk_gated_delta_rule backward")
         ctx.bwd_args = a
         ctx.bwd_keep = (do, dht, dq, dk, dv, dg, dbeta, dh0, dhs, dvnew) if self.keep else None

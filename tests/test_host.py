@@ -106,8 +106,9 @@ def test_workspace_bytes_matches_the_buffers_the_host_layer_allocates():
     NT = B * ((T + 63) // 64)
     for dtype, s in ((_lib.LMOE_BF16, 2), (_lib.LMOE_F32, 4)):
         states, tiles, rk, rv = NT * H * K * V, NT * H * 64 * 64, B * T * H * K, B * T * H * V
+        bv = NT * H * 64 * V          # vnew / dvnew: whole chunks in the library's blocked layout [NT,H,V/32,64,32]
         want = {(0, 0): states, (0, 1): states, (1, 0): states + tiles + 2 * NT * H * 64 * K, (1, 1): states,
-                (2, 0): states + 2 * tiles + rv + (rk + rv if s == 4 else 0), (2, 1): states + rv}
+                (2, 0): states + 2 * tiles + bv + (rk + rv if s == 4 else 0), (2, 1): states + bv}
         for (op, part), n in want.items():
             extra = NT * H * 2 * 64 * 4 if (op, part) == (2, 0) else 0      # fp32 gate table of the delta rule
             extra = NT * H * K * 4 if (op, part) == (1, 0) else extra       # fp32 chunk decays of chunk_gla
