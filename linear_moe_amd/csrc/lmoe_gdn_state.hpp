@@ -121,7 +121,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
 
   if (team == 1) {
     // ------------------------- loaders, ring A (k, P) and all stores ----------------------
-    struct PreA { typename IOK::Regs rk; typename IOP::Regs rp, rt; typename IOV::Regs rv; uint32_t braw; float eb; int len; };
+    struct PreA { typename IOK::Regs rk; typename IOP::Regs rp, rt; typename IOV::Regs rv; float be, f; int len; };
     PreA pa[LPF];
     // Always issued (chunk index clamped to the last chunk; the surplus loads at the end of a
     // sequence are never consumed): a prefetch that is skipped on some path would make the
@@ -135,8 +135,9 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
       if constexpr (WT) {
         IOP::load_nomask(P.rt, (const T*)a.tinv + ((int64_t)(sq.chunk0 + c) * a.H + h) * CH * CH, CH, CH);
         IOV::load_nomask(P.rv, row_ptr<T>(a.v, sq.b, tok, h) + v0, a.v.st, P.len);
-        P.braw = load_scalar_raw(a.beta.ptr, a.beta_dtype, row_off(a.beta, sq.b, tok + min(l, P.len - 1), h));
-        P.eb = a.gcum[((int64_t)(sq.chunk0 + c) * a.H + h) * 2 * CH + l];
+        const float* gc = a.gcum + ((int64_t)(sq.chunk0 + c) * a.H + h) * 4 * CH;
+        P.be = gc[2 * CH + l];
+        P.f = gc[3 * CH + l];
       }
     };
     auto stage_a = [&](PreA& P) {
@@ -153,9 +154,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
       IOV::mask(P.rv, P.len);
       IOV::store_lds(P.rv, s_v, LDU);
       if (wave_id() == 4) {
-        const float be = l < P.len ? scalar_from_raw(P.braw, a.beta_dtype) : 0.f;
-        s_be[l] = be;
-        s_f[l] = be * P.eb;
+        s_be[l] = P.be;
+        s_f[l] = P.f;
       }
     };
     // a result tile of chunk c: registers -> global
@@ -224,7 +224,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
       if constexpr (!WT) IOK::load_nomask(P.rw, row_ptr<T>(a.w, sq.b, tok, h), a.w.st, P.len);
       IOK::load_nomask(P.rq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, P.len);
       if constexpr (!WT) IOV::load_nomask(P.ru, row_ptr<T>(a.u, sq.b, tok, h) + v0, a.u.st, P.len);
-      const float* gc = a.gcum + ((int64_t)(sq.chunk0 + c) * a.H + h) * 2 * CH;
+      const float* gc = a.gcum + ((int64_t)(sq.chunk0 + c) * a.H + h) * 4 * CH;
       P.eb = gc[l];
       P.ed = gc[CH + l];
     };
@@ -492,7 +492,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
   if (team == 2) {
     // ------------------------- loaders, ring B (k, P, Tinv, do, decay table, beta) ------
     // staged during phase 2 of the step before the one that reads them in phase 1
-    struct PreB { typename IOK::Regs rk; typename IOP::Regs rp, rt; typename IOV::Regs rd; float eb, ed; uint32_t braw; int len; };
+    struct PreB { typename IOK::Regs rk; typename IOP::Regs rp, rt; typename IOV::Regs rd; float eb, ed, f; int len; };
     PreB pb[LPF];
     const float scale = a.scale;
     auto issue_b = [&](PreB& P, int it) {
@@ -503,10 +503,10 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
       IOP::load_nomask(P.rp, (const T*)a.pmat + ((int64_t)(sq.chunk0 + c) * a.H + h) * CH * CH, CH, CH);
       IOP::load_nomask(P.rt, (const T*)a.tinv + ((int64_t)(sq.chunk0 + c) * a.H + h) * CH * CH, CH, CH);
       IOV::load_nomask(P.rd, row_ptr<T>(a.d_o, sq.b, tok, h) + v0, a.d_o.st, P.len);
-      P.braw = load_scalar_raw(a.beta.ptr, a.beta_dtype, row_off(a.beta, sq.b, tok + min(l, P.len - 1), h));
-      const float* gc = a.gcum + ((int64_t)(sq.chunk0 + c) * a.H + h) * 2 * CH;
+      const float* gc = a.gcum + ((int64_t)(sq.chunk0 + c) * a.H + h) * 4 * CH;
       P.eb = gc[l];
       P.ed = gc[CH + l];
+      P.f = gc[3 * CH + l];
     };
     auto stage_b = [&](PreB& P, int buf) {
       IOK::mask(P.rk, P.len);
@@ -516,7 +516,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
       IOP::store_lds(P.rt, s_ti, LDC);
       IOV::store_lds(P.rd, s_do, LDU);
       if (wave_id() == 8) {
-        s_f[l] = l < P.len ? scalar_from_raw(P.braw, a.beta_dtype) * P.eb : 0.f;
+        s_f[l] = P.f;
         s_qs[buf][l] = scale * P.eb;
         s_ed[buf][l] = P.ed;
         if (l == 63) s_dec[buf] = P.eb;

@@ -57,7 +57,9 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd_reg(const lmoe_args 
   constexpr int BV = 32;
   constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDU = BV + LPAD;
   constexpr int KT = K / 16, KS = K / 32;
-  constexpr int LPF = GdnStateCfg<T>::LPF;
+  // register sets per prefetch ring (deeper rings were measured: 3 and 4 sets for either team change nothing, the pass
+  // is bound by what the memory system delivers for its traffic, not by the lead of its requests)
+  constexpr int LPA = GdnStateCfg<T>::LPF, LPB = GdnStateCfg<T>::LPF;
   __shared__ __attribute__((aligned(16))) T s_k[2 * CH * LDK];      // k [64][K] of chunks c, c + 1
   __shared__ __attribute__((aligned(16))) T s_q[CH * LDK];          // q [64][K]
   __shared__ __attribute__((aligned(16))) T s_ti[CH * LDC];         // Tinv [64][64]
@@ -107,7 +109,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd_reg(const lmoe_args 
   if (team == 1) {
     // ------------------------- loaders, ring A (k, P) and all stores ----------------------
     struct PreA { typename IOK::Regs rk; typename IOP::Regs rp; int len; };
-    PreA pa[LPF];
+    PreA pa[LPA];
     auto issue_a = [&](PreA& P, int c) {      // always issued, chunk index clamped (see k_gdn_state_fwd)
       c = min(c, sq.nchunks - 1);
       const int tok = sq.tok0 + c * CH;
@@ -126,14 +128,14 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd_reg(const lmoe_args 
       IOV::template store_global<true>(r, row_ptr<T>(dst, sq.b, tok, h) + v0, dst.st, len);
     };
 #pragma unroll
-    for (int j = 0; j < LPF; ++j) issue_a(pa[j], j);
+    for (int j = 0; j < LPA; ++j) issue_a(pa[j], j);
     wait_all_loads();
     stage_k(pa[0], 0);
     lds_barrier();                                                                       // B0
     typename IOHT::Regs rh;
     typename IOV::Regs rvn, ro;
-    ring_loop<LPF>(sq.nchunks, [&](auto slot, const int c) {
-      constexpr int j = decltype(slot)::value, jn = (j + 1) % LPF;
+    ring_loop<LPA>(sq.nchunks, [&](auto slot, const int c) {
+      constexpr int j = decltype(slot)::value, jn = (j + 1) % LPA;
       if (wave_id() == 4) TR(2, c, 0);
       lds_barrier();                                                                     // B1
       if (wave_id() == 4) TR(2, c, 1);
@@ -151,7 +153,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd_reg(const lmoe_args 
       if (c > 0) store_result(ro, a.o, c - 1);
       if constexpr (SAVE) IOV::template store_global<true>(rvn, slice_ptr<T>(a.vnew, sq.chunk0 + c, h, a.H, V, v0), SLICE_COLS, min(CH, sq.len - c * CH));
       if (wave_id() == 4) TR(2, c, 4);
-      issue_a(pa[j], c + LPF);
+      issue_a(pa[j], c + LPA);
       if (wave_id() == 4) TR(2, c, 5);
     });
     lds_barrier();                                                                       // o of the last chunk
@@ -165,8 +167,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd_reg(const lmoe_args 
   }
   if (team == 2) {
     // ------------------------- loaders, ring B (q, Tinv, v, gates) ------------------------
-    struct PreB { typename IOK::Regs rq; typename IOP::Regs rt; typename IOV::Regs rv; float eb, ed; uint32_t braw; int len; };
-    PreB pb[LPF];
+    struct PreB { typename IOK::Regs rq; typename IOP::Regs rt; typename IOV::Regs rv; float eb, ed, be, f; int len; };
+    PreB pb[LPB];
     auto issue_b = [&](PreB& P, int c) {
       c = min(c, sq.nchunks - 1);
       const int tok = sq.tok0 + c * CH;
@@ -174,10 +176,11 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd_reg(const lmoe_args 
       IOK::load_nomask(P.rq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, P.len);
       IOP::load_nomask(P.rt, (const T*)a.tinv + ((int64_t)(sq.chunk0 + c) * a.H + h) * CH * CH, CH, CH);
       IOV::load_nomask(P.rv, row_ptr<T>(a.v, sq.b, tok, h) + v0, a.v.st, P.len);
-      P.braw = load_scalar_raw(a.beta.ptr, a.beta_dtype, row_off(a.beta, sq.b, tok + min(l, P.len - 1), h));
-      const float* gc = a.gcum + ((int64_t)(sq.chunk0 + c) * a.H + h) * 2 * CH;
+      const float* gc = a.gcum + ((int64_t)(sq.chunk0 + c) * a.H + h) * 4 * CH;
       P.eb = gc[l];
       P.ed = gc[CH + l];
+      P.be = gc[2 * CH + l];
+      P.f = gc[3 * CH + l];
     };
     auto stage_b = [&](PreB& P, int buf) {
       IOK::store_lds(P.rq, s_q, LDK);       // rows past the end only reach output rows that are not stored
@@ -185,25 +188,24 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd_reg(const lmoe_args 
       IOV::mask(P.rv, P.len);
       IOV::store_lds(P.rv, s_v, LDU);
       if (wave_id() == 8) {
-        const float be = l < P.len ? scalar_from_raw(P.braw, a.beta_dtype) : 0.f;
-        s_be[l] = be;
-        s_f[l] = be * P.eb;
+        s_be[l] = P.be;
+        s_f[l] = P.f;
         s_eb[buf][l] = P.eb;
         s_ed[buf][l] = P.ed;
         if (l == 63) s_dec[buf] = P.eb;
       }
     };
 #pragma unroll
-    for (int j = 0; j < LPF; ++j) issue_b(pb[j], j);
+    for (int j = 0; j < LPB; ++j) issue_b(pb[j], j);
     wait_all_loads();
     stage_b(pb[0], 0);
     lds_barrier();                                                                       // B0
-    ring_loop<LPF>(sq.nchunks, [&](auto slot, const int c) {
-      constexpr int j = decltype(slot)::value, jn = (j + 1) % LPF;
+    ring_loop<LPB>(sq.nchunks, [&](auto slot, const int c) {
+      constexpr int j = decltype(slot)::value, jn = (j + 1) % LPB;
       if (wave_id() == 8) TR(3, c, 0);
       lds_barrier();                                                                     // B1
       if (wave_id() == 8) TR(3, c, 1);
-      issue_b(pb[j], c + LPF);              // chunk c was staged before this barrier: refill its set
+      issue_b(pb[j], c + LPB);              // chunk c was staged before this barrier: refill its set
       if (wave_id() == 8) TR(3, c, 2);
       lds_barrier();                                                                     // B2
       if (wave_id() == 8) TR(3, c, 3);

@@ -200,12 +200,15 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? (SAVE ? 3 : 2) : 1)) void k
     s_beb[l] = bl * eb;
   }
   {
-    // decay table of the chunk for the sequential passes: e^{b_j}, e^{b_C - b_j}.  Every global store of
+    // gate table of the chunk for the sequential passes: e^{b_j}, e^{b_C - b_j}, beta_j, beta_j e^{b_j}.  Every global store of
     // this loop is issued by all threads on every path (here two waves write each entry), so that the
     // compiler can count the operations behind the prefetches exactly: a store under a condition made
     // the wait for the next item's inputs a wait for this item's last stores as well
-    float* gc = a.gcum + ((int64_t)cid * a.H + h) * 2 * CH;
-    gc[tid & 127] = (tid & 64) ? ed : eb;
+    // (rows 2, 3: beta and beta e^{b}, zero past the end of the chunk -- the sequential passes then read no beta,
+    // whose run-time element type would put a load behind a branch in their prefetch loops)
+    float* gc = a.gcum + ((int64_t)cid * a.H + h) * 4 * CH;
+    const int row = tid >> 6;
+    gc[tid] = row == 0 ? eb : row == 1 ? ed : row == 2 ? bl : bl * eb;
   }
   IOK::store_lds(rk, s_k, LDK, tid);
   if constexpr (!LEAN) {
