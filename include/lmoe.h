@@ -77,11 +77,12 @@ typedef struct lmoe_args {
   lmoe_tensor u;       /* [B,T,H,V]   WY factor u (gated delta rule; forward only)     */
   void* tinv;          /* [NT,H,64,64] (I + L)^-1 per chunk (gated delta rule)         */
   void* amat;          /* [NT,H,64,64] intra-chunk attention matrix (chunk_gla)        */
-  void* pmat;          /* [NT,H,64,64] P = (q k^T) . Gamma per chunk (gated delta rule;
-                          written by the WY preparation)                                */
-  float* gcum;         /* gated delta rule: [NT,H,4,64] fp32 gate table per chunk, written by the WY preparation:
-                          e^{b_j}, e^{b_C - b_j}, beta_j, beta_j e^{b_j} (b = cumulative log-decay inside the chunk;
-                          beta rows zero past the end of a partial chunk);
+  void* pmat;          /* [NT,H,64,64] P = (q k^T) . Gamma per chunk (gated delta rule; written by the
+                          WY preparation, or, for bf16 calls with tinv, by the forward state pass and
+                          only when hs is given: a forward-only bf16 call leaves it untouched)      */
+  float* gcum;         /* gated delta rule: [NT,H,5,64] fp32 gate table per chunk, written by the WY preparation:
+                          e^{b_j}, e^{b_C - b_j}, beta_j, beta_j e^{b_j}, b_j (b = cumulative log-decay inside the
+                          chunk; beta rows zero past the end of a partial chunk);
                           chunk_gla: [NT,H,K] fp32 e^{b_C} per channel, the decay of a whole chunk */
   void* qe;            /* [NT,H,64,K] q e^{b}       per chunk, rows past its end zero (chunk_gla) */
   void* ke;            /* [NT,H,64,K] k e^{b_C - b} per chunk, rows past its end zero (chunk_gla) */

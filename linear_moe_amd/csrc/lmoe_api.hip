@@ -61,7 +61,7 @@ int64_t lmoe_workspace_bytes(int32_t op, int32_t dtype, int32_t part, int32_t B,
   const int64_t blocks_v = (int64_t)NT * H * LMOE_CHUNK * V;             // vnew | dvnew: whole chunks, [NT,H,V/32,64,32]
   if (op == LMOE_OP_GATED_DELTA_RULE) n += part == 0 ? blocks_v + 2 * tiles + (s == 4 ? rows_v + rows_k : 0) : blocks_v;
   int64_t bytes = n * s;
-  if (op == LMOE_OP_GATED_DELTA_RULE && part == 0) bytes += (int64_t)NT * H * 4 * LMOE_CHUNK * 4;   // gcum (fp32)
+  if (op == LMOE_OP_GATED_DELTA_RULE && part == 0) bytes += (int64_t)NT * H * 5 * LMOE_CHUNK * 4;   // gcum (fp32)
   if (op == LMOE_OP_GLA && part == 0) bytes += (int64_t)NT * H * K * 4;                              // gcum (fp32)
   return bytes;
 }

@@ -28,6 +28,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int CH = 64;        // chunk length (tokens)
+constexpr int GATE_ROWS = 5;  // rows of the gated delta rule's per-chunk gate table (e^b, e^{b_C - b}, beta, beta e^b, b)
 constexpr int NTHR = 256;     // threads per work-group
 constexpr int LPAD = 8;       // LDS row padding in elements (16 B for bf16, 32 B for fp32)
 

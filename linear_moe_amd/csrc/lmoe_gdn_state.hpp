@@ -135,7 +135,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
       if constexpr (WT) {
         IOP::load_nomask(P.rt, (const T*)a.tinv + ((int64_t)(sq.chunk0 + c) * a.H + h) * CH * CH, CH, CH);
         IOV::load_nomask(P.rv, row_ptr<T>(a.v, sq.b, tok, h) + v0, a.v.st, P.len);
-        const float* gc = a.gcum + ((int64_t)(sq.chunk0 + c) * a.H + h) * 4 * CH;
+        const float* gc = a.gcum + ((int64_t)(sq.chunk0 + c) * a.H + h) * GATE_ROWS * CH;
         P.be = gc[2 * CH + l];
         P.f = gc[3 * CH + l];
       }
@@ -224,7 +224,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
       if constexpr (!WT) IOK::load_nomask(P.rw, row_ptr<T>(a.w, sq.b, tok, h), a.w.st, P.len);
       IOK::load_nomask(P.rq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, P.len);
       if constexpr (!WT) IOV::load_nomask(P.ru, row_ptr<T>(a.u, sq.b, tok, h) + v0, a.u.st, P.len);
-      const float* gc = a.gcum + ((int64_t)(sq.chunk0 + c) * a.H + h) * 4 * CH;
+      const float* gc = a.gcum + ((int64_t)(sq.chunk0 + c) * a.H + h) * GATE_ROWS * CH;
       P.eb = gc[l];
       P.ed = gc[CH + l];
     };
@@ -503,7 +503,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
       IOP::load_nomask(P.rp, (const T*)a.pmat + ((int64_t)(sq.chunk0 + c) * a.H + h) * CH * CH, CH, CH);
       IOP::load_nomask(P.rt, (const T*)a.tinv + ((int64_t)(sq.chunk0 + c) * a.H + h) * CH * CH, CH, CH);
       IOV::load_nomask(P.rd, row_ptr<T>(a.d_o, sq.b, tok, h) + v0, a.d_o.st, P.len);
-      const float* gc = a.gcum + ((int64_t)(sq.chunk0 + c) * a.H + h) * 4 * CH;
+      const float* gc = a.gcum + ((int64_t)(sq.chunk0 + c) * a.H + h) * GATE_ROWS * CH;
       P.eb = gc[l];
       P.ed = gc[CH + l];
       P.f = gc[3 * CH + l];

@@ -17,9 +17,17 @@
 //   * w and u are never formed: v_new = Tinv Z costs 6 products (Tinv is lower triangular) on top of X = k S.
 //   * Helper wave j (waves 2, 3) forms the output of the same 16 columns from what the consumers leave in LDS anyway
 //     (S^T at chunk start, which is the checkpoint the loaders store, and v_new): q S in phase 1, P v_new in phase 2,
-//     transposed so that a lane holds four consecutive columns of one token (8-byte writes of o).
-//   * Loader teams as in k_gdn_state_fwd: team 1 stages P(c), k(c+1) in phase 1 and carries all stores; team 2
+//     transposed so that a lane holds four consecutive columns of one token (8-byte writes of o).  
+//   * Loader teams as in k_gdn_state_fwd: team 1 stages k(c+1) in phase 1 and carries all stores; team 2
 //     stages q, Tinv, v, gates of chunk c+1 in phase 2.
+//   * The intra-chunk matrix P = (q k^T) . Gamma is formed here, by the four waves of team 2 in phase 1 (their loads
+//     for a later chunk are in flight by then and they have nothing else to do): the ten 16 x 16 blocks of the lower
+//     triangle, three or two per wave, from the q and k tiles and the gate table's b row into the P tile that the
+//     helpers read in phase 2.  The WY preparation then reads no q and writes no P, this pass reads none (8 KB per
+//     chunk and work-group less through the CU's memory pipe, which bounds it), and a forward-only call never has P
+//     in memory.  A call that saves for the backward writes P once: every V-slice work-group stores its share of
+//     the rows.  (Formed on the helper waves instead, as registers that feed (P v_new)^T directly, the pass was 45 us
+//     slower at T = 8192: 48 more products per chunk on a wave that shares a phase with the consumers.)
 #pragma once
 #include <type_traits>
 #include "lmoe_gdn_state.hpp"
@@ -69,6 +77,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd_reg(const lmoe_args 
   __shared__ __attribute__((aligned(16))) T s_vn[CH * LDU];         // v_new [64][BV]
   __shared__ __attribute__((aligned(16))) T s_o[CH * LDU];          // o [64][BV]
   __shared__ __attribute__((aligned(16))) float s_f[64], s_be[64];  // beta e^{b}, beta
+  __shared__ __attribute__((aligned(16))) float s_b[64];            // cumulative log-decay b
   __shared__ __attribute__((aligned(16))) float s_eb[2][64], s_ed[2][64];
   __shared__ float s_dec[2];                                        // e^{b_C}; buffer c & 1
   __shared__ long long s_tr[TRACE ? TRACE_SLOTS * TRACE_CHUNKS * TRACE_MARKS : 1];
@@ -108,20 +117,23 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd_reg(const lmoe_args 
 
   if (team == 1) {
     // ------------------------- loaders, ring A (k, P) and all stores ----------------------
-    struct PreA { typename IOK::Regs rk; typename IOP::Regs rp; int len; };
+    struct PreA { typename IOK::Regs rk; int len; };
     PreA pa[LPA];
     auto issue_a = [&](PreA& P, int c) {      // always issued, chunk index clamped (see k_gdn_state_fwd)
       c = min(c, sq.nchunks - 1);
       const int tok = sq.tok0 + c * CH;
       P.len = min(CH, sq.len - c * CH);
       IOK::load_nomask(P.rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, P.len);
-      IOP::load_nomask(P.rp, (const T*)a.pmat + ((int64_t)(sq.chunk0 + c) * a.H + h) * CH * CH, CH, CH);
     };
-    auto stage_p = [&](PreA& P) { IOP::store_lds(P.rp, s_p, LDC); };
     auto stage_k = [&](PreA& P, int c) {
       IOK::mask(P.rk, P.len);
       IOK::store_lds(P.rk, s_k + (c & 1) * CH * LDK, LDK);
     };
+    // this work-group's share of the rows of P (team 2 leaves the whole matrix in s_p): 64 / NVS rows, every
+    // thread stores (threads beyond the share repeat a row with the same bytes: no store sits behind a branch)
+    constexpr int PROWS = CH / NVS;
+    const int pidx = (threadIdx.x & (NTHR - 1)) % (PROWS * 8);
+    const int prow = vsl * PROWS + pidx / 8, pcol = (pidx % 8) * 8;
     auto store_result = [&](const typename IOV::Regs& r, const lmoe_tensor& dst, int c) {
       const int tok = sq.tok0 + c * CH;
       const int len = min(CH, sq.len - c * CH);
@@ -139,7 +151,6 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd_reg(const lmoe_args 
       if (wave_id() == 4) TR(2, c, 0);
       lds_barrier();                                                                     // B1
       if (wave_id() == 4) TR(2, c, 1);
-      stage_p(pa[j]);
       stage_k(pa[jn], c + 1);               // (past the last chunk: a clamped copy of it, never used)
       if constexpr (SAVE) IOHT::load_lds(rh, s_hT, LDK);
       IOV::load_lds(ro, s_o, LDU);
@@ -148,7 +159,9 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd_reg(const lmoe_args 
       if (wave_id() == 4) TR(2, c, 3);
       if constexpr (SAVE) {
         IOV::load_lds(rvn, s_vn, LDU);
+        const typename ET<T>::vec pv = *(const typename ET<T>::vec*)(s_p + prow * LDC + pcol);
         IOHT::template store_global<true>(rh, (T*)a.hs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
+        __builtin_nontemporal_store(pv, (typename ET<T>::vec*)((T*)a.pmat + (((int64_t)(sq.chunk0 + c) * a.H + h) * CH + prow) * CH + pcol));
       }
       if (c > 0) store_result(ro, a.o, c - 1);
       if constexpr (SAVE) IOV::template store_global<true>(rvn, slice_ptr<T>(a.vnew, sq.chunk0 + c, h, a.H, V, v0), SLICE_COLS, min(CH, sq.len - c * CH));
@@ -167,7 +180,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd_reg(const lmoe_args 
   }
   if (team == 2) {
     // ------------------------- loaders, ring B (q, Tinv, v, gates) ------------------------
-    struct PreB { typename IOK::Regs rq; typename IOP::Regs rt; typename IOV::Regs rv; float eb, ed, be, f; int len; };
+    struct PreB { typename IOK::Regs rq; typename IOP::Regs rt; typename IOV::Regs rv; float eb, ed, be, f, bb; int len; };
     PreB pb[LPB];
     auto issue_b = [&](PreB& P, int c) {
       c = min(c, sq.nchunks - 1);
@@ -176,11 +189,12 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd_reg(const lmoe_args 
       IOK::load_nomask(P.rq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, P.len);
       IOP::load_nomask(P.rt, (const T*)a.tinv + ((int64_t)(sq.chunk0 + c) * a.H + h) * CH * CH, CH, CH);
       IOV::load_nomask(P.rv, row_ptr<T>(a.v, sq.b, tok, h) + v0, a.v.st, P.len);
-      const float* gc = a.gcum + ((int64_t)(sq.chunk0 + c) * a.H + h) * 4 * CH;
+      const float* gc = a.gcum + ((int64_t)(sq.chunk0 + c) * a.H + h) * GATE_ROWS * CH;
       P.eb = gc[l];
       P.ed = gc[CH + l];
       P.be = gc[2 * CH + l];
       P.f = gc[3 * CH + l];
+      P.bb = gc[4 * CH + l];
     };
     auto stage_b = [&](PreB& P, int buf) {
       IOK::store_lds(P.rq, s_q, LDK);       // rows past the end only reach output rows that are not stored
@@ -190,11 +204,68 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd_reg(const lmoe_args 
       if (wave_id() == 8) {
         s_be[l] = P.be;
         s_f[l] = P.f;
+        s_b[l] = P.bb;
         s_eb[buf][l] = P.eb;
         s_ed[buf][l] = P.ed;
         if (l == 63) s_dec[buf] = P.eb;
       }
     };
+    // P = (q k^T) . Gamma of the chunk in the tiles, Gamma_ij = e^{b_i - b_j} for i >= j (rows past the end of a
+    // partial chunk: 0; its columns are zero through k): block number x = wave, wave + 4, wave + 8 of the ten blocks
+    // (ti, tj <= ti) of the lower triangle, formed transposed (k rows as the A operand) so that a lane holds four
+    // consecutive columns of one row (8-byte writes).  The six blocks above the diagonal are cleared once.
+    const int wt = wave_id() - 8;
+    auto form_p = [&](int c) {
+      const int fr = l & 15, g = l >> 4;
+      const T* s_kc = s_k + (c & 1) * CH * LDK;
+      const int len = min(CH, sq.len - c * CH);
+      int ti[3], tj[3];
+#pragma unroll
+      for (int x = 0; x < 3; ++x) {
+        const int idx = min(wt + 4 * x, 9);
+        ti[x] = idx >= 6 ? 3 : idx >= 3 ? 2 : idx >= 1 ? 1 : 0;
+        tj[x] = idx - ti[x] * (ti[x] + 1) / 2;
+      }
+      const int nx = wt < 2 ? 3 : 2;        // wave-uniform
+      f32x4 pc[3];
+#pragma unroll
+      for (int x = 0; x < 3; ++x) pc[x] = f32x4{0.f, 0.f, 0.f, 0.f};
+      // (one set of fragments, no read-ahead: the team's prefetch rings leave the registers for no more, and nobody
+      //  waits for these waves)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        typename ET<T>::frag fq[3], fk[3];
+#pragma unroll
+        for (int x = 0; x < 3; ++x) {
+          fq[x] = ET<T>::load_frag(s_q + (16 * ti[x] + fr) * LDK + 32 * ks + 8 * g);
+          fk[x] = ET<T>::load_frag(s_kc + (16 * tj[x] + fr) * LDK + 32 * ks + 8 * g);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int x = 0; x < 3; ++x)
+          if (x < nx) ET<T>::mma(pc[x], fk[x], fq[x]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int x = 0; x < 3; ++x) {
+        if (x < nx) {
+          const int i = 16 * ti[x] + fr, j0 = 16 * tj[x] + 4 * g;
+          const float bi = s_b[i];
+          const f32x4 bj = *(const f32x4*)&s_b[j0];
+          bf16x4 y;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) y[e] = (bf16)((i >= j0 + e && i < len) ? pc[x][e] * texp<T>(bi - bj[e]) : 0.f);
+          *(bf16x4*)(s_p + i * LDC + j0) = y;
+        }
+      }
+    };
+    {
+      const int t = threadIdx.x & (NTHR - 1), r = t >> 4, cc = t & 15;
+#pragma unroll
+      for (int I = 0; I < 3; ++I)
+#pragma unroll
+        for (int J = I + 1; J < 4; ++J) s_p[(16 * I + r) * LDC + 16 * J + cc] = (T)0.f;
+    }
 #pragma unroll
     for (int j = 0; j < LPB; ++j) issue_b(pb[j], j);
     wait_all_loads();
@@ -206,6 +277,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd_reg(const lmoe_args 
       lds_barrier();                                                                     // B1
       if (wave_id() == 8) TR(3, c, 1);
       issue_b(pb[j], c + LPB);              // chunk c was staged before this barrier: refill its set
+      form_p(c);
       if (wave_id() == 8) TR(3, c, 2);
       lds_barrier();                                                                     // B2
       if (wave_id() == 8) TR(3, c, 3);

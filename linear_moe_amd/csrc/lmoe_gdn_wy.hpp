@@ -3,7 +3,8 @@
 //   Tinv = (I + L)^-1            (unit lower triangular, fp32)
 //   w = Tinv (k . beta e^{b}),   u = Tinv (v . beta)
 // and the intra-chunk attention matrix the two sequential passes consume,
-//   P = (q k^T) . Gamma  (lower triangle incl. the diagonal).
+//   P = (q k^T) . Gamma  (lower triangle incl. the diagonal)
+// (not in the lean form below: the register-resident forward pass forms P itself and q is not read here).
 // persistent: grid = a few work-groups of 256 threads per CU, item = (chunk, head).  The inputs of
 // the next item (q rows as fragments, k, v tiles, gate, beta) are requested at the top of an item and
 // stay in flight behind its LDS-only barriers.  Writes w, u, Tinv and P (element type T) and the
@@ -120,7 +121,8 @@ __device__ __forceinline__ void tri_inverse_64(const float* sL, int ldl, float* 
 
 // SAVE = false (no Tinv buffer given): Tinv is not written.  With Tinv written and 2-byte elements the
 // sequential passes form w and u on the chip from Tinv, k, v (LEAN below): neither is formed or written here and v
-// is not read.
+// is not read; the forward pass (k_gdn_state_fwd_reg) also forms P from q, k and the gate table, so P is not formed
+// and q is not read here either: a lean item reads k, g, beta and writes Tinv and the gate table.
 template <typename T, int K, int V, bool SAVE>
 __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? (SAVE ? 3 : 2) : 1)) void k_gdn_wy_fwd(const lmoe_args a) {
   constexpr bool LEAN = SAVE && sizeof(T) == 2;
@@ -161,7 +163,7 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? (SAVE ? 3 : 2) : 1)) void k
     return chunk_info(a, it / a.H);
   };
   // q enters only as the A operand of q k^T: each wave takes its 16 rows straight into fragments
-  auto issue_q = [&](int it) { int h; const ChunkInfo ci = item_of(it, h); fq.load(row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, 16 * wv, ci.len - 1); };
+  auto issue_q = [&](int it) { if constexpr (LEAN) return; int h; const ChunkInfo ci = item_of(it, h); fq.load(row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, 16 * wv, ci.len - 1); };
   auto issue_k = [&](int it) { int h; const ChunkInfo ci = item_of(it, h); IOK::load_nomask(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len); };
   auto issue_v = [&](int it) {
     if constexpr (!LEAN) { int h; const ChunkInfo ci = item_of(it, h); IOV::load_nomask(rv, row_ptr<T>(a.v, ci.b, ci.tok, h), a.v.st, ci.len); }
@@ -200,15 +202,16 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? (SAVE ? 3 : 2) : 1)) void k
     s_beb[l] = bl * eb;
   }
   {
-    // gate table of the chunk for the sequential passes: e^{b_j}, e^{b_C - b_j}, beta_j, beta_j e^{b_j}.  Every global store of
+    // gate table of the chunk for the sequential passes: e^{b_j}, e^{b_C - b_j}, beta_j, beta_j e^{b_j}, b_j.  Every global store of
     // this loop is issued by all threads on every path (here two waves write each entry), so that the
     // compiler can count the operations behind the prefetches exactly: a store under a condition made
     // the wait for the next item's inputs a wait for this item's last stores as well
     // (rows 2, 3: beta and beta e^{b}, zero past the end of the chunk -- the sequential passes then read no beta,
     // whose run-time element type would put a load behind a branch in their prefetch loops)
-    float* gc = a.gcum + ((int64_t)cid * a.H + h) * 4 * CH;
+    float* gc = a.gcum + ((int64_t)cid * a.H + h) * GATE_ROWS * CH;
     const int row = tid >> 6;
     gc[tid] = row == 0 ? eb : row == 1 ? ed : row == 2 ? bl : bl * eb;
+    gc[4 * CH + l] = xb;       // (all four waves, the same bytes)
   }
   IOK::store_lds(rk, s_k, LDK, tid);
   if constexpr (!LEAN) {
@@ -234,7 +237,7 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? (SAVE ? 3 : 2) : 1)) void k
     f32x4 m[4], pm[4];
 #pragma unroll
     for (int nj = 0; nj < 4; ++nj) { m[nj] = f32x4{0.f, 0.f, 0.f, 0.f}; pm[nj] = m[nj]; }
-    fq.mask(16 * wv, ci.len);
+    if constexpr (!LEAN) fq.mask(16 * wv, ci.len);
     const int fr = l & 15, fg = 8 * (l >> 4);
 #pragma unroll
     for (int ks = 0; ks < K / 32; ++ks) {
@@ -244,7 +247,7 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? (SAVE ? 3 : 2) : 1)) void k
         if (nj <= wv) {
           const typename ET<T>::frag bk = ET<T>::load_frag(s_k + (16 * nj + fr) * LDK + 32 * ks + fg);
           ET<T>::mma(m[nj], bk, ak);          // transposed: a lane holds four consecutive columns of one row
-          ET<T>::mma(pm[nj], bk, fq.f[ks]);
+          if constexpr (!LEAN) ET<T>::mma(pm[nj], bk, fq.f[ks]);
         }
       }
     }
@@ -265,10 +268,12 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? (SAVE ? 3 : 2) : 1)) void k
         }
       }
       acc_to_lds_t<float>(pl, s_L, LDC, 16 * nj, 16 * wv, l);      // s_L[r][cc0 ..]: one 16-byte write
-      acc_to_lds_t<T>(pp, s_P, LDP, 16 * nj, 16 * wv, l);
+      if constexpr (!LEAN) acc_to_lds_t<T>(pp, s_P, LDP, 16 * nj, 16 * wv, l);
     }
-    lds_barrier();
-    IO64::template lds_to_global<true>(s_P, LDP, pg, CH, CH, tid);
+    if constexpr (!LEAN) {
+      lds_barrier();
+      IO64::template lds_to_global<true>(s_P, LDP, pg, CH, CH, tid);
+    }
   }
   // k is dead as an operand of k k^T and q k^T: scale it in place to k beta e^{b} (from the registers)
   if constexpr (!LEAN) IOK::store_lds_scaled(rk, s_k, LDK, s_beb, tid);

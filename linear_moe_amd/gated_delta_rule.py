@@ -67,7 +67,7 @@ class GDNCall:
         # always: the backward reads it, and the forward state pass forms w from it (8 KB per chunk and head)
         tinv = torch.empty(max(plan.NT, 1), H, 64, 64, dtype=dt, device=dev)
         pmat = torch.empty(max(plan.NT, 1), H, 64, 64, dtype=dt, device=dev)
-        gcum = torch.empty(max(plan.NT, 1), H, 4, 64, dtype=torch.float32, device=dev)
+        gcum = torch.empty(max(plan.NT, 1), H, 5, 64, dtype=torch.float32, device=dev)
         # w, u: the bf16 state passes form them on the chip from tinv; only the fp32 forward pass reads them
         w = torch.empty(B, T, H, K, dtype=dt, device=dev) if dt == torch.float32 else None
         u = torch.empty(B, T, H, V, dtype=dt, device=dev) if dt == torch.float32 else None

@@ -110,7 +110,7 @@ def test_workspace_bytes_matches_the_buffers_the_host_layer_allocates():
         want = {(0, 0): states, (0, 1): states, (1, 0): states + tiles + 2 * NT * H * 64 * K, (1, 1): states,
                 (2, 0): states + 2 * tiles + bv + (rk + rv if s == 4 else 0), (2, 1): states + bv}
         for (op, part), n in want.items():
-            extra = NT * H * 4 * 64 * 4 if (op, part) == (2, 0) else 0      # fp32 gate table of the delta rule
+            extra = NT * H * 5 * 64 * 4 if (op, part) == (2, 0) else 0      # fp32 gate table of the delta rule
             extra = NT * H * K * 4 if (op, part) == (1, 0) else extra       # fp32 chunk decays of chunk_gla
             assert lib.lmoe_workspace_bytes(op, dtype, part, B, T, H, K, V, NT) == n * s + extra
     assert lib.lmoe_workspace_bytes(5, 0, 0, B, T, H, K, V, NT) == -21
