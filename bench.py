@@ -279,8 +279,8 @@ def trace_state_fwd(lib, x, dims, work_group=16):
     names = {0: {0: "arrives_b1", 1: "leaves_b1", 5: "kS_formed", 2: "arrives_b2_vnew_written", 3: "leaves_b2",
                  6: "state_updated", 4: "state_written"},
              1: {0: "arrives_b1", 1: "leaves_b1", 2: "arrives_b2_qS_formed", 3: "leaves_b2", 4: "o_written"},
-             2: {0: "arrives_b1", 1: "leaves_b1", 2: "arrives_b2_tiles_staged", 3: "leaves_b2", 4: "stores_issued",
-                 5: "loads_issued"},
+             2: {0: "arrives_b1", 1: "leaves_b1", 6: "k_staged", 2: "arrives_b2_P_formed", 3: "leaves_b2",
+                 4: "stores_issued", 5: "loads_issued"},
              3: {0: "arrives_b1", 1: "leaves_b1", 2: "arrives_b2_loads_issued", 3: "leaves_b2", 4: "tiles_staged"}}
     teams = {0: "consumer_wave", 1: "helper_wave", 2: "loader_team_1", 3: "loader_team_2"}
     out = {}

@@ -20,8 +20,8 @@
 //     transposed so that a lane holds four consecutive columns of one token (8-byte writes of o).  
 //   * Loader teams as in k_gdn_state_fwd: team 1 stages k(c+1) in phase 1 and carries all stores; team 2
 //     stages q, Tinv, v, gates of chunk c+1 in phase 2.
-//   * The intra-chunk matrix P = (q k^T) . Gamma is formed here, by the four waves of team 2 in phase 1 (their loads
-//     for a later chunk are in flight by then and they have nothing else to do): the ten 16 x 16 blocks of the lower
+//   * The intra-chunk matrix P = (q k^T) . Gamma is formed here, by the four waves of team 1 in phase 1 (behind their
+//     staging of k, where they would otherwise wait for the consumers): the ten 16 x 16 blocks of the lower
 //     triangle, three or two per wave, from the q and k tiles and the gate table's b row into the P tile that the
 //     helpers read in phase 2.  The WY preparation then reads no q and writes no P, this pass reads none (8 KB per
 //     chunk and work-group less through the CU's memory pipe, which bounds it), and a forward-only call never has P
@@ -129,7 +129,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd_reg(const lmoe_args 
       IOK::mask(P.rk, P.len);
       IOK::store_lds(P.rk, s_k + (c & 1) * CH * LDK, LDK);
     };
-    // this work-group's share of the rows of P (team 2 leaves the whole matrix in s_p): 64 / NVS rows, every
+    // this work-group's share of the rows of P (formed below, the whole matrix in s_p): 64 / NVS rows, every
     // thread stores (threads beyond the share repeat a row with the same bytes: no store sits behind a branch)
     constexpr int PROWS = CH / NVS;
     const int pidx = (threadIdx.x & (NTHR - 1)) % (PROWS * 8);
@@ -139,6 +139,64 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd_reg(const lmoe_args 
       const int len = min(CH, sq.len - c * CH);
       IOV::template store_global<true>(r, row_ptr<T>(dst, sq.b, tok, h) + v0, dst.st, len);
     };
+    // P = (q k^T) . Gamma of the chunk in the tiles, Gamma_ij = e^{b_i - b_j} for i >= j (rows past the end of a
+    // partial chunk: 0; its columns are zero through k): block number x = wave, wave + 4, wave + 8 of the ten blocks
+    // (ti, tj <= ti) of the lower triangle, formed transposed (k rows as the A operand) so that a lane holds four
+    // consecutive columns of one row (8-byte writes).  The six blocks above the diagonal are cleared once.
+    const int wt = wave_id() - 4;
+    auto form_p = [&](int c) {
+      const int fr = l & 15, g = l >> 4;
+      const T* s_kc = s_k + (c & 1) * CH * LDK;
+      const int len = min(CH, sq.len - c * CH);
+      int ti[3], tj[3];
+#pragma unroll
+      for (int x = 0; x < 3; ++x) {
+        const int idx = min(wt + 4 * x, 9);
+        ti[x] = idx >= 6 ? 3 : idx >= 3 ? 2 : idx >= 1 ? 1 : 0;
+        tj[x] = idx - ti[x] * (ti[x] + 1) / 2;
+      }
+      const int nx = wt < 2 ? 3 : 2;        // wave-uniform
+      f32x4 pc[3];
+#pragma unroll
+      for (int x = 0; x < 3; ++x) pc[x] = f32x4{0.f, 0.f, 0.f, 0.f};
+      typename ET<T>::frag fq[2][3], fk[2][3];
+      auto fetch = [&](int ks, int buf) {
+#pragma unroll
+        for (int x = 0; x < 3; ++x) {
+          fq[buf][x] = ET<T>::load_frag(s_q + (16 * ti[x] + fr) * LDK + 32 * ks + 8 * g);
+          fk[buf][x] = ET<T>::load_frag(s_kc + (16 * tj[x] + fr) * LDK + 32 * ks + 8 * g);
+        }
+      };
+      fetch(0, 0);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        if (ks + 1 < KS) fetch(ks + 1, (ks + 1) & 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int x = 0; x < 3; ++x)
+          if (x < nx) ET<T>::mma(pc[x], fk[ks & 1][x], fq[ks & 1][x]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int x = 0; x < 3; ++x) {
+        if (x < nx) {
+          const int i = 16 * ti[x] + fr, j0 = 16 * tj[x] + 4 * g;
+          const float bi = s_b[i];
+          const f32x4 bj = *(const f32x4*)&s_b[j0];
+          bf16x4 y;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) y[e] = (bf16)((i >= j0 + e && i < len) ? pc[x][e] * texp<T>(bi - bj[e]) : 0.f);
+          *(bf16x4*)(s_p + i * LDC + j0) = y;
+        }
+      }
+    };
+    {
+      const int t = threadIdx.x & (NTHR - 1), r = t >> 4, cc = t & 15;
+#pragma unroll
+      for (int I = 0; I < 3; ++I)
+#pragma unroll
+        for (int J = I + 1; J < 4; ++J) s_p[(16 * I + r) * LDC + 16 * J + cc] = (T)0.f;
+    }
 #pragma unroll
     for (int j = 0; j < LPA; ++j) issue_a(pa[j], j);
     wait_all_loads();
@@ -154,6 +212,11 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd_reg(const lmoe_args 
       stage_k(pa[jn], c + 1);               // (past the last chunk: a clamped copy of it, never used)
       if constexpr (SAVE) IOHT::load_lds(rh, s_hT, LDK);
       IOV::load_lds(ro, s_o, LDU);
+      if (wave_id() == 4) TR(2, c, 6);
+      // behind the staging: the first thousand cycles after the barrier every wave of the work-group reads LDS and
+      // a read of this team's takes that long to come back (measured: formed first, P was ready 250 cycles later
+      // and k staged 600 cycles later than in this order)
+      form_p(c);
       if (wave_id() == 4) TR(2, c, 2);
       lds_barrier();                                                                     // B2
       if (wave_id() == 4) TR(2, c, 3);
@@ -210,62 +273,6 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd_reg(const lmoe_args 
         if (l == 63) s_dec[buf] = P.eb;
       }
     };
-    // P = (q k^T) . Gamma of the chunk in the tiles, Gamma_ij = e^{b_i - b_j} for i >= j (rows past the end of a
-    // partial chunk: 0; its columns are zero through k): block number x = wave, wave + 4, wave + 8 of the ten blocks
-    // (ti, tj <= ti) of the lower triangle, formed transposed (k rows as the A operand) so that a lane holds four
-    // consecutive columns of one row (8-byte writes).  The six blocks above the diagonal are cleared once.
-    const int wt = wave_id() - 8;
-    auto form_p = [&](int c) {
-      const int fr = l & 15, g = l >> 4;
-      const T* s_kc = s_k + (c & 1) * CH * LDK;
-      const int len = min(CH, sq.len - c * CH);
-      int ti[3], tj[3];
-#pragma unroll
-      for (int x = 0; x < 3; ++x) {
-        const int idx = min(wt + 4 * x, 9);
-        ti[x] = idx >= 6 ? 3 : idx >= 3 ? 2 : idx >= 1 ? 1 : 0;
-        tj[x] = idx - ti[x] * (ti[x] + 1) / 2;
-      }
-      const int nx = wt < 2 ? 3 : 2;        // wave-uniform
-      f32x4 pc[3];
-#pragma unroll
-      for (int x = 0; x < 3; ++x) pc[x] = f32x4{0.f, 0.f, 0.f, 0.f};
-      // (one set of fragments, no read-ahead: the team's prefetch rings leave the registers for no more, and nobody
-      //  waits for these waves)
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        typename ET<T>::frag fq[3], fk[3];
-#pragma unroll
-        for (int x = 0; x < 3; ++x) {
-          fq[x] = ET<T>::load_frag(s_q + (16 * ti[x] + fr) * LDK + 32 * ks + 8 * g);
-          fk[x] = ET<T>::load_frag(s_kc + (16 * tj[x] + fr) * LDK + 32 * ks + 8 * g);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int x = 0; x < 3; ++x)
-          if (x < nx) ET<T>::mma(pc[x], fk[x], fq[x]);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-#pragma unroll
-      for (int x = 0; x < 3; ++x) {
-        if (x < nx) {
-          const int i = 16 * ti[x] + fr, j0 = 16 * tj[x] + 4 * g;
-          const float bi = s_b[i];
-          const f32x4 bj = *(const f32x4*)&s_b[j0];
-          bf16x4 y;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) y[e] = (bf16)((i >= j0 + e && i < len) ? pc[x][e] * texp<T>(bi - bj[e]) : 0.f);
-          *(bf16x4*)(s_p + i * LDC + j0) = y;
-        }
-      }
-    };
-    {
-      const int t = threadIdx.x & (NTHR - 1), r = t >> 4, cc = t & 15;
-#pragma unroll
-      for (int I = 0; I < 3; ++I)
-#pragma unroll
-        for (int J = I + 1; J < 4; ++J) s_p[(16 * I + r) * LDC + 16 * J + cc] = (T)0.f;
-    }
 #pragma unroll
     for (int j = 0; j < LPB; ++j) issue_b(pb[j], j);
     wait_all_loads();
@@ -277,7 +284,6 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd_reg(const lmoe_args 
       lds_barrier();                                                                     // B1
       if (wave_id() == 8) TR(3, c, 1);
       issue_b(pb[j], c + LPB);              // chunk c was staged before this barrier: refill its set
-      form_p(c);
       if (wave_id() == 8) TR(3, c, 2);
       lds_barrier();                                                                     // B2
       if (wave_id() == 8) TR(3, c, 3);
