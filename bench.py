@@ -24,10 +24,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_MFMA_BF16 = 2.5e15   # dense bf16 MFMA, FLOP/s (MI355X published)
+PEAK_MFMA_F32 = 157.3e12  # dense fp32 MFMA, FLOP/s (MI355X published)
 PEAK_HBM = 8.0e12         # B/s
 CH = 64
 
-STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_gdn_state_fwd", 4: "k_gdn_state_bwd", 5: "k_gdn_bwd_chunk"}
+STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_gdn_state_fwd_reg", 4: "k_gdn_state_bwd", 5: "k_gdn_bwd_chunk"}
 
 # HBM bytes per launch on this workload, from two rocprofv3 --pmc runs of this file (FETCH_SIZE, then
 # WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for the 256 MiB device
@@ -37,11 +38,29 @@ STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_gdn_state_fwd", 4: "k_gdn_state_bwd", 5:
 # sources (kernel_sources_sha16()) at that time, and a build whose sources differ reports traffic = null
 # rather than a stale number.
 CALIB_COPY_BYTES = 256 << 20
-MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 432417222, "k_gdn_state_fwd": 1128774601, "k_gdn_state_bwd": 980265694,
-                    "k_gdn_bwd_chunk": 1897687630}
-TRAFFIC_SOURCES_SHA16 = "50306358452a3c02"
-TRAFFIC_SOURCES = ("lmoe_common.hpp", "lmoe_seq.hpp", "lmoe_gdn_wy.hpp", "lmoe_gdn_state.hpp", "lmoe_gdn_bwd_chunk.hpp",
+MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237241639, "k_gdn_state_fwd_reg": 1118538293, "k_gdn_state_bwd": 945962362,
+                    "k_gdn_bwd_chunk": 1899113770}
+TRAFFIC_SOURCES_SHA16 = "523b1b53ec10092f"
+TRAFFIC_SOURCES = ("lmoe_common.hpp", "lmoe_seq.hpp", "lmoe_gdn_wy.hpp", "lmoe_gdn_state.hpp", "lmoe_gdn_state_reg.hpp", "lmoe_gdn_bwd_chunk.hpp",
                    "lmoe_gdn_fwd.hip", "lmoe_gdn_state.hip", "lmoe_gdn_bwd.hip")
+
+
+# HBM bytes per call of the other contract configurations (bench.py --other-configs), same counters and scaling,
+# summed over the kernels of the call; key = configuration number
+OTHER_TRAFFIC = {"1": 2235899, "2": 272837190, "3": 1548253856, "5": 16928727197}
+OTHER_TRAFFIC_SHA16 = "b61c52b4cb26e96a"
+
+
+def all_sources_sha16():
+    """Digest of every kernel source of the library (what OTHER_TRAFFIC was counted on)."""
+    import glob
+    import hashlib
+    h = hashlib.sha256()
+    d = os.path.join(ROOT, "linear_moe_amd", "csrc")
+    for path in sorted(glob.glob(os.path.join(d, "*.hpp")) + glob.glob(os.path.join(d, "*.hip"))):
+        with open(path, "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
 
 
 def kernel_sources_sha16():
@@ -79,16 +98,16 @@ def stage_model(stage, K, V, s=2):
     c = CH
     kv, ck, cv, cc = K * V, c * K, c * V, c * c
     lean = s == 2     # 2-byte elements: w = Tinv (k beta e^b), u = Tinv (v beta) are formed inside the state passes
-    if stage == 0:   # k k^T, q k^T, triangular inverse (, w, u) | r q,k,g,beta(,v)  w Tinv,P,decay table(,w,u)
+    if stage == 0:   # k k^T(, q k^T), triangular inverse(, w, u) | r k,g,beta(,q,v)  w Tinv,gate table(,P,w,u)
+        if lean:     # (the table has five fp32 rows; g is read as fp32)
+            return 2 * cc * K + (2 / 3) * c ** 3, ck * s + cc * s + c * (20 + 4 + s)
+        return 6 * cc * K + 2 * cc * V + (2 / 3) * c ** 3, (2 * ck + cv) * s + (ck + cv) * s + 2 * cc * s + c * (20 + 4 + s)
+    if stage == 1:   # k S, Tinv Z, q S, q k^T, P v_new, k^T v_new | r q,k,Tinv,v,table (q,k,w,u,P,table)  w v_new,hs,o,P
         if lean:
-            return 4 * cc * K + (2 / 3) * c ** 3, 2 * ck * s + 2 * cc * s + c * (8 + 4 + s)
-        return 6 * cc * K + 2 * cc * V + (2 / 3) * c ** 3, (2 * ck + cv) * s + (ck + cv) * s + 2 * cc * s + c * (8 + 4 + s)
-    if stage == 1:   # (w, u,) w S, q S, k^T v_new, P v_new | r q,k,Tinv,v,P,table,beta (q,k,w,u,P,table)  w v_new,hs,o
-        if lean:
-            return 6 * c * kv + 2 * cc * V + 2 * cc * K + 2 * cc * V, (2 * ck + cv + 2 * cc) * s + (2 * cv + kv) * s + c * (8 + s)
+            return 6 * c * kv + 4 * cc * V + 2 * cc * K, (2 * ck + cv + cc) * s + (2 * cv + kv + cc) * s + 20 * c
         return 6 * c * kv + 2 * cc * V, (3 * ck + cv + cc) * s + (2 * cv + kv) * s + 8 * c
-    if stage == 4:   # w, k dS', P^T do, q^T do, w^T dv_new | r q,k,Tinv,do,P,table,beta  w dv_new,dhs
-        return 6 * c * kv + 2 * cc * V + 2 * cc * K, (2 * ck + cv + 2 * cc) * s + (cv + kv) * s + c * (8 + s)
+    if stage == 4:   # w, k dS', P^T do, q^T do, w^T dv_new | r q,k,Tinv,do,P,table  w dv_new,dhs
+        return 6 * c * kv + 2 * cc * V + 2 * cc * K, (2 * ck + cv + 2 * cc) * s + (cv + kv) * s + 12 * c
     if stage == 5:   # do v'^T, do S^T, v' dS'^T, du S^T, du v^T, Tinv^T du, G k, G^T q, dw k^T, Tinv^T dw,
         #              two 64^3 products, dM k, dM^T k_b | r do,v',du,v,hs,dhs,q,k,Tinv,g,beta  w dq,dk,dv,dbeta,dg
         return (4 * cc * V + 6 * c * kv + 2 * cc * V + 4 * cc * K + 4 * cc * K + 4 * c ** 3 + 4 * cc * K,
@@ -323,13 +342,16 @@ def other_configs(dev, steps, warmup):
     q, k, v = (rn(B, H, T, K, dt=torch.float32) for _ in range(3))
     with torch.no_grad():
         sec = timed(lambda: L.chunk_linear_attn(q, k, v, normalize=False))
-    res["1 linear_attn fwd fp32 B=1 H=4 T=512 K=V=64"] = (sec, B * T, B * T * H * (2 * K + 2 * K) * 4)
+    sg_flops = lambda K, V: 2 * CH * K + 2 * CH * V + 4 * K * V       # per token and head, forward: q k^T, P v, q S, k^T v
+    res["1 linear_attn fwd fp32 B=1 H=4 T=512 K=V=64"] = (sec, B * T, B * T * H * (2 * K + 2 * K) * 4,
+                                                          B * T * H * sg_flops(K, K), PEAK_MFMA_F32)
     # 2: retention forward, bf16
     B, H, T, K = 4, 16, 4096, 128
     q, k, v = (rn(B, H, T, K) for _ in range(3))
     with torch.no_grad():
         sec = timed(lambda: L.chunk_retention(q, k, v, output_final_state=True))
-    res["2 retention fwd bf16 B=4 H=16 T=4096 K=V=128"] = (sec, B * T, B * T * H * ((2 * K + 2 * K) * 2 + 4))
+    res["2 retention fwd bf16 B=4 H=16 T=4096 K=V=128"] = (sec, B * T, B * T * H * ((2 * K + 2 * K) * 2 + 4),
+                                                           B * T * H * sg_flops(K, K), PEAK_MFMA_BF16)
     # 3: chunk_gla forward + backward, bf16
     B, H, T, K, V = 8, 16, 2048, 64, 128
     q, k = (rn(B, H, T, K).requires_grad_(True) for _ in range(2))
@@ -341,7 +363,8 @@ def other_configs(dev, steps, warmup):
         o, _ = L.chunk_gla(q, k, v, g)
         torch.autograd.grad([o], [q, k, v, g], [do])
     sec = timed(f3)
-    res["3 chunk_gla fwd+bwd bf16 B=8 H=16 T=2048 K=64 V=128"] = (sec, B * T, B * T * H * (9 * K + 5 * V) * 2)
+    res["3 chunk_gla fwd+bwd bf16 B=8 H=16 T=2048 K=64 V=128"] = (sec, B * T, B * T * H * (9 * K + 5 * V) * 2,
+                                                                  3 * B * T * H * sg_flops(K, V), PEAK_MFMA_BF16)
     # 5: packed gated delta rule forward + backward, 16 sequences of log-normal lengths, 65536 tokens
     N, Tt, H, K, V = 16, 65536, 32, 128, 128
     gen = torch.Generator().manual_seed(1005)
@@ -364,11 +387,23 @@ def other_configs(dev, steps, warmup):
         torch.autograd.grad([o, ht], [q, k, v, g, beta, h0], [do, dht])
     sec = timed(f5)
     res["5 packed gated_delta_rule fwd+bwd bf16 16 seqs 65536 tokens H=32 K=V=128"] = (
-        sec, Tt, Tt * H * ((6 * K + 5 * V) * 2 + 3 * 2 + 12) + 4 * N * H * K * V * 4)
+        sec, Tt, Tt * H * ((6 * K + 5 * V) * 2 + 3 * 2 + 12) + 4 * N * H * K * V * 4,
+        3 * Tt * H * (6 * CH * K + 4 * CH * V + 6 * K * V + (2 / 3) * CH * CH), PEAK_MFMA_BF16)
+    # one roofline record per configuration, for the whole call on its minimal traffic (every input read once, every
+    # output written once): all five are bound by HBM on that count (arithmetic intensity below peak flops / peak
+    # bytes).  `traffic` = HBM bytes per call summed over its kernels, from the FETCH_SIZE / WRITE_SIZE counters
+    # (OTHER_TRAFFIC, measured on the sources OTHER_TRAFFIC_SHA16 names; null when the sources have changed since)
+    fresh = all_sources_sha16() == OTHER_TRAFFIC_SHA16
+    out = {}
+    for n, (sec, tok, nb, fl, peak_f) in res.items():
+        out[n] = {"ms": round(sec * 1e3, 4), "tokens_per_s": round(tok / sec), "algorithmic_bytes": nb,
+                  "algorithmic_flops": round(fl), "frac_hbm_peak": round(nb / sec / PEAK_HBM, 4),
+                  "roofline": {"bound": "hbm", "achieved": round(nb / sec / 1e9, 1), "peak": PEAK_HBM / 1e9,
+                               "unit": "GB/s", "frac": round(nb / sec / PEAK_HBM, 4),
+                               "mfma_frac": round(fl / sec / peak_f, 4),
+                               "traffic": OTHER_TRAFFIC.get(n[0]) if fresh else None}}
     return {"metric": "contract configurations 1, 2, 3, 5: ms per call, tokens/s", "unit": "ms", "steps": steps,
-            "warmup": warmup, "data": "synthetic",
-            "configs": {n: {"ms": round(sec * 1e3, 4), "tokens_per_s": round(tok / sec), "algorithmic_bytes": nb,
-                            "frac_hbm_peak": round(nb / sec / PEAK_HBM, 4)} for n, (sec, tok, nb) in res.items()}}
+            "warmup": warmup, "data": "synthetic", "configs": out}
 
 
 def main():
@@ -401,6 +436,13 @@ def main():
     lib = _lib.load()
     dev = torch.device("cuda:0")
     B, T, H, K, V, seed = 4, 8192, 16, 128, 128, 1004
+    # known-size device copy: the yardstick for the FETCH_SIZE / WRITE_SIZE counters under rocprofv3
+    src = torch.empty(CALIB_COPY_BYTES, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
+
     if args.neighbours:
         print(json.dumps(neighbours(lib, B * T * H, K, dev, args.stage_reps)))
         return
@@ -411,13 +453,6 @@ def main():
     if args.trace_state_fwd:
         print(json.dumps(trace_state_fwd(lib, x, (B, T, H, K, V))))
         return
-
-    # known-size device copy: the yardstick for the FETCH_SIZE / WRITE_SIZE counters under rocprofv3
-    src = torch.empty(CALIB_COPY_BYTES, dtype=torch.uint8, device=dev).fill_(1)
-    dst = torch.empty_like(src)
-    dst.copy_(src)
-    torch.cuda.synchronize()
-    del src, dst
 
     from linear_moe_amd import chunk_gated_delta_rule
 
