@@ -168,6 +168,17 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd_reg(const lmoe_args 
         }
       };
       fetch(0, 0);
+      // the decay factors (masked) while the first fragments are on their way: behind the products only a multiply,
+      // a conversion and the write are left
+      f32x4 gm[3];
+#pragma unroll
+      for (int x = 0; x < 3; ++x) {
+        const int i = 16 * ti[x] + fr, j0 = 16 * tj[x] + 4 * g;
+        const float bi = s_b[i];
+        const f32x4 bj = *(const f32x4*)&s_b[j0];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) gm[x][e] = (i >= j0 + e && i < len) ? texp<T>(bi - bj[e]) : 0.f;
+      }
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         if (ks + 1 < KS) fetch(ks + 1, (ks + 1) & 1);
@@ -181,11 +192,9 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd_reg(const lmoe_args 
       for (int x = 0; x < 3; ++x) {
         if (x < nx) {
           const int i = 16 * ti[x] + fr, j0 = 16 * tj[x] + 4 * g;
-          const float bi = s_b[i];
-          const f32x4 bj = *(const f32x4*)&s_b[j0];
           bf16x4 y;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) y[e] = (bf16)((i >= j0 + e && i < len) ? pc[x][e] * texp<T>(bi - bj[e]) : 0.f);
+          for (int e = 0; e < 4; ++e) y[e] = (bf16)(pc[x][e] * gm[x][e]);
           *(bf16x4*)(s_p + i * LDC + j0) = y;
         }
       }
