@@ -368,16 +368,19 @@ __global__ __launch_bounds__(NTHR) void k_gla_state_fwd(const lmoe_args a) {
 // ------------------------------------------------------------------------- //
 template <typename T, typename GT, int K, int V, int BV>
 __global__ __launch_bounds__(NTHR) void k_gla_out_fwd(const lmoe_args a) {
-  constexpr int LDK = K + LPAD, LDC = CH + LPAD;
+  constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDV = BV + LPAD;
   constexpr int NB = BV / 16;
   // Two LDS regions, each used twice (small LDS -> more work-groups per CU, which is what hides the load
-  // latency of these one-shot work-groups):  R0: S^T, then v^T;  R1: q e^{b} (as stored by k_gla_intra_fwd),
-  // then A.  Every load is requested up front and waits in registers for its region.
-  constexpr int R0_ELEMS = cmax(BV * LDK, BV * LDC);
+  // latency of these one-shot work-groups):  R0: S, then v;  R1: q e^{b} (as stored by k_gla_intra_fwd),
+  // then A.  Every load is requested up front and waits in registers for its region.  S and v are staged as
+  // they lie in memory (16-byte writes) and enter the products, which contract over their rows, through
+  // transposing reads (staged transposed, element by element, these two kernels spent 70 % of their cycles
+  // in LDS bank conflicts).
+  constexpr int R0_ELEMS = cmax(K * LDV, CH * LDV);
   constexpr int R1_ELEMS = cmax(CH * LDK, CH * LDC);
   __shared__ __attribute__((aligned(16))) T r0[R0_ELEMS];
   __shared__ __attribute__((aligned(16))) T r1[R1_ELEMS];
-  T* s_hT = r0; T* s_vT = r0;
+  T* s_h = r0; T* s_v = r0;
   T* s_q = r1; T* s_P = r1;
   const int cid = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * BV;
   const ChunkInfo ci = chunk_info(a, cid);
@@ -395,19 +398,19 @@ __global__ __launch_bounds__(NTHR) void k_gla_out_fwd(const lmoe_args a) {
   IOA::load_nomask(ra, (const T*)a.amat + ((int64_t)cid * a.H + h) * CH * CH, CH, CH);
   IOV::load_nomask(rv, row_ptr<T>(a.v, ci.b, ci.tok, h) + v0, a.v.st, ci.len);
   IOK::store_lds(rq, s_q, LDK);
-  IOH::store_lds_t(rh, s_hT, LDK, nullptr);
+  IOH::store_lds(rh, s_h, LDV);
   lds_barrier();
   // the products are formed transposed (o^T = S^T (q e^b)^T, then += v^T A^T): a lane then holds four consecutive V
   // columns of one token and stores them as one 8-byte piece
   f32x4 o[NB][1];
   acc_zero(o);
-  gemm_nt<T, NB, 1>(o, s_hT, LDK, 0, s_q, LDK, 16 * wv, 0, K);
-  lds_barrier();                                                                       // q e^{b}, S^T are dead
+  gemm<T, NB, 1, true, false>(o, s_h, LDV, 0, s_q, LDK, 16 * wv, 0, K);
+  lds_barrier();                                                                       // q e^{b}, S are dead
   IOA::store_lds(ra, s_P, LDC);
   IOV::mask(rv, ci.len);
-  IOV::store_lds_t(rv, s_vT, LDC, nullptr);
+  IOV::store_lds(rv, s_v, LDV);
   lds_barrier();
-  gemm_nt<T, NB, 1>(o, s_vT, LDC, 0, s_P, LDC, 16 * wv, 0, CH);
+  gemm<T, NB, 1, true, false>(o, s_v, LDV, 0, s_P, LDC, 16 * wv, 0, CH);
   const int r = 16 * wv + (l & 15);
   if (r < ci.len) {
     T* od = row_ptr<T>(a.o, ci.b, ci.tok + r, h) + v0 + 4 * (l >> 4);
@@ -533,16 +536,17 @@ __global__ __launch_bounds__(NTHR) void k_gla_state_bwd(const lmoe_args a) {
 // ------------------------------------------------------------------------- //
 template <typename T, typename GT, int K, int V, int BV>
 __global__ __launch_bounds__(NTHR) void k_gla_bwd_dv(const lmoe_args a) {
-  constexpr int LDK = K + LPAD, LDC = CH + LPAD;
+  constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDV = BV + LPAD;
   constexpr int NB = BV / 16;
-  // two LDS regions, each used twice (see k_gla_out_fwd):  R0: dS'^T, then do^T;  R1: k e^{b_C - b} (as stored
-  // by k_gla_intra_fwd), then A^T
-  constexpr int R0_ELEMS = cmax(BV * LDK, BV * LDC);
+  // two LDS regions, each used twice (see k_gla_out_fwd):  R0: dS', then do;  R1: k e^{b_C - b} (as stored
+  // by k_gla_intra_fwd), then A; all staged as they lie in memory, transposing reads where a product contracts
+  // over the rows of a tile
+  constexpr int R0_ELEMS = cmax(K * LDV, CH * LDV);
   constexpr int R1_ELEMS = cmax(CH * LDK, CH * LDC);
   __shared__ __attribute__((aligned(16))) T r0[R0_ELEMS];
   __shared__ __attribute__((aligned(16))) T r1[R1_ELEMS];
-  T* s_dhT = r0; T* s_doT = r0;
-  T* s_kd = r1; T* s_PT = r1;
+  T* s_dh = r0; T* s_do = r0;
+  T* s_kd = r1; T* s_P = r1;
   const int cid = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * BV;
   const ChunkInfo ci = chunk_info(a, cid);
   const int wv = wave_id(), l = lane_id();
@@ -559,18 +563,18 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dv(const lmoe_args a) {
   IOA::load_nomask(ra, (const T*)a.amat + ((int64_t)cid * a.H + h) * CH * CH, CH, CH);
   IOV::load_nomask(rd, row_ptr<T>(a.d_o, ci.b, ci.tok, h) + v0, a.d_o.st, ci.len);
   IOK::store_lds(rk, s_kd, LDK);
-  IOH::store_lds_t(rh, s_dhT, LDK, nullptr);
+  IOH::store_lds(rh, s_dh, LDV);
   lds_barrier();
   // products formed transposed (see k_gla_out_fwd): 8-byte stores of four consecutive V columns per token
   f32x4 dv[NB][1], dv2[NB][1];
   acc_zero(dv); acc_zero(dv2);
-  gemm_nt<T, NB, 1>(dv2, s_dhT, LDK, 0, s_kd, LDK, 16 * wv, 0, K);
-  lds_barrier();                                                                       // k e^{..}, dS'^T are dead
-  IOA::store_lds_t(ra, s_PT, LDC, nullptr);
+  gemm<T, NB, 1, true, false>(dv2, s_dh, LDV, 0, s_kd, LDK, 16 * wv, 0, K);
+  lds_barrier();                                                                       // k e^{..}, dS' are dead
+  IOA::store_lds(ra, s_P, LDC);
   IOV::mask(rd, ci.len);
-  IOV::store_lds_t(rd, s_doT, LDC, nullptr);
+  IOV::store_lds(rd, s_do, LDV);
   lds_barrier();
-  gemm_nt<T, NB, 1>(dv, s_doT, LDC, 0, s_PT, LDC, 16 * wv, 0, CH);
+  gemm<T, NB, 1, true, true>(dv, s_do, LDV, 0, s_P, LDC, 16 * wv, 0, CH);
   const int r = 16 * wv + (l & 15);
   if (r < ci.len) {
     T* dd = row_ptr<T>(a.dv, ci.b, ci.tok + r, h) + v0 + 4 * (l >> 4);
