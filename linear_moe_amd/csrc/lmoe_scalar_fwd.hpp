@@ -22,9 +22,9 @@ template <typename T> __device__ __forceinline__ void scale_frag(typename ET<T>:
 //   grid = ceil(N*H / 8) * 8 * (V / BV) work-groups (1-D).  Work-group -> (sequence, head,
 //   V-slice): the V-slices of one (sequence, head) get ids that are congruent mod 8, i.e. run on
 //   the same XCD and share q, k through its L2.
-//   Team 0 (waves 0-3, consumers) carries the dependency chain of the state; between B1 and B2, where
-//     that chain waits for nobody, it forms P = (q k^T) . Gamma for the output team (wave-private LDS strips):
-//        S -> LDS (element type T) | B1 | P -> LDS | B2 | S = e^{b_C} S + k^T (e_d v)
+//   Team 0 (waves 0-3, consumers) carries the dependency chain of the state and, in the same window, forms
+//     P = (q k^T) . Gamma for the output team (wave-private LDS strips):
+//        S -> LDS (element type T) | B1 | S = e^{b_C} S + k^T (e_d v), P -> LDS | B2
 //     wave w owns state rows [w*K/4, (w+1)*K/4) x BV columns in fp32 MFMA accumulators; the row
 //     scaling e_d is applied to the v fragments in registers, so k is staged unscaled.
 //   Team 1 (waves 4-7, loaders) keeps the operands of the next PF chunks in flight in registers,
@@ -148,7 +148,25 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
       lds_barrier();                                                                     // B1
       f32x4 o[1][NB];
       acc_zero(o);
-      gemm<T, 1, NB, false, false>(o, s_q[cur], LDK, 16 * ow, s_hT, LDK, 0, 0, K);
+      if constexpr (sizeof(T) == 4) {
+        gemm<T, 1, NB, false, false>(o, s_q[cur], LDK, 16 * ow, s_hT, LDK, 0, 0, K);
+      } else {
+        // all fragments requested before the first product (see the consumers' P window)
+        constexpr int KS = K / 32;
+        const int fr = l & 15, fg = 8 * (l >> 4);
+        typename ET<T>::frag fq[KS], fh[KS][NB];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          fq[ks] = ET<T>::load_frag(s_q[cur] + (16 * ow + fr) * LDK + 32 * ks + fg);
+#pragma unroll
+          for (int ni = 0; ni < NB; ++ni) fh[ks][ni] = ET<T>::load_frag(s_hT + (16 * ni + fr) * LDK + 32 * ks + fg);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+          for (int ni = 0; ni < NB; ++ni) ET<T>::mma(o[0][ni], fq[ks], fh[ks][ni]);
+      }
 #pragma unroll
       for (int ni = 0; ni < NB; ++ni)
 #pragma unroll
@@ -186,43 +204,84 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
       for (int ni = 0; ni < NB; ++ni) acc_to_lds_t<T>(S[mi][ni], s_hT, LDK, krow0 + 16 * mi, 16 * ni);
     lds_barrier();                                                                       // B1
     const float dec = s_dec[cur];
-    // rows 16 wv .. of P = (q k^T) . Gamma for the output team (it reads them after B2): the consumers are idle
-    // between B1 and B2, the output team is not
+    // S = e^{b_C} S + k^T (e_d v'): the row scaling e_d is applied to the v' fragments in registers.  In this
+    // window, not behind B2: the copy of S for the output team was written before B1, nothing here waits for
+    // the P rows below, and behind B2 the consumers then go straight to the next chunk's copy
     {
-      f32x4 p[1][4];
-      acc_zero(p);
-      gemm<T, 1, 4, false, false>(p, s_q[cur], LDK, 16 * wv, s_k[cur], LDK, 0, 0, K);
+      typename ET<T>::frag af[CH / 32][MB], bf[CH / 32][NB];
+#pragma unroll
+      for (int kq = 0; kq < CH / 32; ++kq) {
+#pragma unroll
+        for (int mi = 0; mi < MB; ++mi) af[kq][mi] = ET<T>::load_frag_t(s_k[cur], LDK, 32 * kq, krow0 + 16 * mi);
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) bf[kq][ni] = ET<T>::load_frag_t(s_u[cur], LDU, 32 * kq, 16 * ni);
+      }
+#pragma unroll
+      for (int kq = 0; kq < CH / 32; ++kq)
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) scale_frag<T>(bf[kq][ni], &s_ed[cur][32 * kq + 8 * (l >> 4)]);
+#pragma unroll
+      for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) S[mi][ni] *= dec;
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int kq = 0; kq < CH / 32; ++kq)
+#pragma unroll
+        for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+          for (int ni = 0; ni < NB; ++ni) ET<T>::mma(S[mi][ni], af[kq][mi], bf[kq][ni]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // rows 16 wv .. of P = (q k^T) . Gamma for the output team (it reads them after B2)
+    {
+      // every fragment and gate value is requested before the first product (left to the compiler, each read is
+      // waited for where it is used and the window is a chain of LDS round trips); blocks above the diagonal
+      // (nj > wv) are zero and skipped
+      // (2-byte elements; the fp32 fragments of a whole K = 128 window do not fit the registers: looped product)
+      constexpr int KS = K / 32;
+      const int fr = l & 15, fg = 8 * (l >> 4);
+      const f32x4 bi = *(const f32x4*)&s_b[cur][16 * wv + 4 * (l >> 4)];
+      float bj[4];
+#pragma unroll
+      for (int nj = 0; nj < 4; ++nj) bj[nj] = s_b[cur][16 * nj + fr];
+      f32x4 p[4];
+#pragma unroll
+      for (int nj = 0; nj < 4; ++nj) p[nj] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if constexpr (sizeof(T) == 2) {
+        typename ET<T>::frag fq[KS], fk[KS][4];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          fq[ks] = ET<T>::load_frag(s_q[cur] + (16 * wv + fr) * LDK + 32 * ks + fg);
+#pragma unroll
+          for (int nj = 0; nj < 4; ++nj)
+            if (nj <= wv) fk[ks][nj] = ET<T>::load_frag(s_k[cur] + (16 * nj + fr) * LDK + 32 * ks + fg);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+          for (int nj = 0; nj < 4; ++nj)
+            if (nj <= wv) ET<T>::mma(p[nj], fq[ks], fk[ks][nj]);
+      } else {
+        f32x4 pp[1][4];
+        acc_zero(pp);
+        gemm<T, 1, 4, false, false>(pp, s_q[cur], LDK, 16 * wv, s_k[cur], LDK, 0, 0, K);
+#pragma unroll
+        for (int nj = 0; nj < 4; ++nj) p[nj] = pp[0][nj];
+      }
 #pragma unroll
       for (int nj = 0; nj < 4; ++nj) {
         f32x4 x;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const int i = 16 * wv + 4 * (l >> 4) + e, j = 16 * nj + (l & 15);
-          x[e] = (i >= j) ? p[0][nj][e] * texp<T>(s_b[cur][i] - s_b[cur][j]) : 0.f;
+          const int i = 16 * wv + 4 * (l >> 4) + e, j = 16 * nj + fr;
+          x[e] = (i >= j) ? p[nj][e] * texp<T>(bi[e] - bj[nj]) : 0.f;
         }
         acc_to_lds<T>(x, s_pst + wv * 16 * LDC, LDC, 0, 16 * nj);
       }
     }
     lds_barrier();                                                                       // B2
-#pragma unroll
-    for (int mi = 0; mi < MB; ++mi)
-#pragma unroll
-      for (int ni = 0; ni < NB; ++ni) S[mi][ni] *= dec;
-    // S += k^T (e_d v'): the row scaling e_d is applied to the v' fragments in registers
-    for (int kk = 0; kk < CH; kk += 32) {
-      typename ET<T>::frag af[MB], bf[NB];
-#pragma unroll
-      for (int mi = 0; mi < MB; ++mi) af[mi] = ET<T>::load_frag_t(s_k[cur], LDK, kk, krow0 + 16 * mi);
-#pragma unroll
-      for (int ni = 0; ni < NB; ++ni) {
-        bf[ni] = ET<T>::load_frag_t(s_u[cur], LDU, kk, 16 * ni);
-        scale_frag<T>(bf[ni], &s_ed[cur][kk + 8 * (l >> 4)]);
-      }
-#pragma unroll
-      for (int mi = 0; mi < MB; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < NB; ++ni) ET<T>::mma(S[mi][ni], af[mi], bf[ni]);
-    }
     if constexpr (NBUF == 1) lds_barrier();                                              // B3
   }
   if (a.ht) {
