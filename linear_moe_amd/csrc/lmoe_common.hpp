@@ -136,46 +136,100 @@ template <typename T> __device__ __forceinline__ float texp_scaled(float x) {
 // gemm_nt: acc[mi][ni] += A[arow0 + 16 mi + r][k] * B[brow0 + 16 ni + c][k], k in [k0, k1)
 // (k0, k1 multiples of 32).  A, B: LDS tiles with leading dimensions lda, ldb.
 // ------------------------------------------------------------------------- //
-template <typename T, int MB, int NB>
+// PIPE (2-byte elements only): the fragments of step kk + 32 are requested before the products of step kk are
+// issued (left to the compiler, every read is waited for right where it is used: a chain of LDS round trips).
+// It costs a second set of fragment registers: for kernels whose latency is on a dependency chain, not for the
+// one-shot kernels that live on occupancy.  The callers pass constant bounds, so the loop unrolls and the two
+// fragment sets stay in registers.
+template <typename T, int MB, int NB, bool PIPE = false>
 __device__ __forceinline__ void gemm_nt(f32x4 (&acc)[MB][NB], const T* A, int lda, int arow0,
                                         const T* B, int ldb, int brow0, int k0, int k1, int l = threadIdx.x & 63) {
   const int r = l & 15, kg = (l >> 4) * 8;
-  for (int kk = k0; kk < k1; kk += 32) {
-    typename ET<T>::frag a[MB], b[NB];
+  if constexpr (sizeof(T) == 2 && PIPE) {
+    typename ET<T>::frag a[2][MB], b[2][NB];
+    auto fetch = [&](int kk, int buf) {
 #pragma unroll
-    for (int mi = 0; mi < MB; ++mi) a[mi] = ET<T>::load_frag(A + (arow0 + 16 * mi + r) * lda + kk + kg);
+      for (int mi = 0; mi < MB; ++mi) a[buf][mi] = ET<T>::load_frag(A + (arow0 + 16 * mi + r) * lda + kk + kg);
 #pragma unroll
-    for (int ni = 0; ni < NB; ++ni) b[ni] = ET<T>::load_frag(B + (brow0 + 16 * ni + r) * ldb + kk + kg);
+      for (int ni = 0; ni < NB; ++ni) b[buf][ni] = ET<T>::load_frag(B + (brow0 + 16 * ni + r) * ldb + kk + kg);
+    };
+    fetch(k0, 0);
 #pragma unroll
-    for (int mi = 0; mi < MB; ++mi)
+    for (int kk = k0, it = 0; kk < k1; kk += 32, ++it) {
+      if (kk + 32 < k1) fetch(kk + 32, (it + 1) & 1);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int ni = 0; ni < NB; ++ni) ET<T>::mma(acc[mi][ni], a[mi], b[ni]);
+      for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) ET<T>::mma(acc[mi][ni], a[it & 1][mi], b[it & 1][ni]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  } else {
+    for (int kk = k0; kk < k1; kk += 32) {
+      typename ET<T>::frag a[MB], b[NB];
+#pragma unroll
+      for (int mi = 0; mi < MB; ++mi) a[mi] = ET<T>::load_frag(A + (arow0 + 16 * mi + r) * lda + kk + kg);
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) b[ni] = ET<T>::load_frag(B + (brow0 + 16 * ni + r) * ldb + kk + kg);
+#pragma unroll
+      for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) ET<T>::mma(acc[mi][ni], a[mi], b[ni]);
+    }
   }
 }
 
 // gemm: like gemm_nt, but either operand may be stored with the contraction index along the
 // rows of its tile (AT / BT = true):  AT = false: A[a0 + m][k]   AT = true: A[k][a0 + m]
 //                                     BT = false: B[b0 + n][k]   BT = true: B[k][b0 + n]
-template <typename T, int MB, int NB, bool AT, bool BT>
+template <typename T, int MB, int NB, bool AT, bool BT, bool PIPE = false>
 __device__ __forceinline__ void gemm(f32x4 (&acc)[MB][NB], const T* A, int lda, int a0,
                                      const T* B, int ldb, int b0, int k0, int k1, int l = threadIdx.x & 63) {
   const int r = l & 15, kg = (l >> 4) * 8;
-  for (int kk = k0; kk < k1; kk += 32) {
-    typename ET<T>::frag a[MB], b[NB];
+  if constexpr (sizeof(T) == 2 && PIPE) {
+    // fragments one step ahead of the products, as in gemm_nt
+    typename ET<T>::frag a[2][MB], b[2][NB];
+    auto fetch = [&](int kk, int buf) {
 #pragma unroll
-    for (int mi = 0; mi < MB; ++mi) {
-      if constexpr (AT) a[mi] = ET<T>::load_frag_t(A, lda, kk, a0 + 16 * mi, l);
-      else a[mi] = ET<T>::load_frag(A + (a0 + 16 * mi + r) * lda + kk + kg);
+      for (int mi = 0; mi < MB; ++mi) {
+        if constexpr (AT) a[buf][mi] = ET<T>::load_frag_t(A, lda, kk, a0 + 16 * mi, l);
+        else a[buf][mi] = ET<T>::load_frag(A + (a0 + 16 * mi + r) * lda + kk + kg);
+      }
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) {
+        if constexpr (BT) b[buf][ni] = ET<T>::load_frag_t(B, ldb, kk, b0 + 16 * ni, l);
+        else b[buf][ni] = ET<T>::load_frag(B + (b0 + 16 * ni + r) * ldb + kk + kg);
+      }
+    };
+    fetch(k0, 0);
+#pragma unroll
+    for (int kk = k0, it = 0; kk < k1; kk += 32, ++it) {
+      if (kk + 32 < k1) fetch(kk + 32, (it + 1) & 1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) ET<T>::mma(acc[mi][ni], a[it & 1][mi], b[it & 1][ni]);
+      __builtin_amdgcn_sched_barrier(0);
     }
+  } else {
+    for (int kk = k0; kk < k1; kk += 32) {
+      typename ET<T>::frag a[MB], b[NB];
 #pragma unroll
-    for (int ni = 0; ni < NB; ++ni) {
-      if constexpr (BT) b[ni] = ET<T>::load_frag_t(B, ldb, kk, b0 + 16 * ni, l);
-      else b[ni] = ET<T>::load_frag(B + (b0 + 16 * ni + r) * ldb + kk + kg);
+      for (int mi = 0; mi < MB; ++mi) {
+        if constexpr (AT) a[mi] = ET<T>::load_frag_t(A, lda, kk, a0 + 16 * mi, l);
+        else a[mi] = ET<T>::load_frag(A + (a0 + 16 * mi + r) * lda + kk + kg);
+      }
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) {
+        if constexpr (BT) b[ni] = ET<T>::load_frag_t(B, ldb, kk, b0 + 16 * ni, l);
+        else b[ni] = ET<T>::load_frag(B + (b0 + 16 * ni + r) * ldb + kk + kg);
+      }
+#pragma unroll
+      for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) ET<T>::mma(acc[mi][ni], a[mi], b[ni]);
     }
-#pragma unroll
-    for (int mi = 0; mi < MB; ++mi)
-#pragma unroll
-      for (int ni = 0; ni < NB; ++ni) ET<T>::mma(acc[mi][ni], a[mi], b[ni]);
   }
 }
 

@@ -226,7 +226,7 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
     if (wv > I || (wv == I && ((unsafe >> I) & 1))) continue;
     f32x4 t[1][1];
     acc_zero(t);
-    gemm<T, 1, 1, false, false>(t, s_qt, LDK, 16 * I, s_kt + KT_ROW0(I) * LDK, LDK, 16 * wv, 0, K);
+    gemm<T, 1, 1, false, false, true>(t, s_qt, LDK, 16 * I, s_kt + KT_ROW0(I) * LDK, LDK, 16 * wv, 0, K);
     if (wv == I) {
 #pragma unroll
       for (int e = 0; e < 4; ++e)
@@ -251,7 +251,7 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
       if (wv < I) {
         f32x4 t[1][1];
         acc_zero(t);
-        gemm<T, 1, 1, false, false>(t, s_qt, LDK, 0, s_kt, LDK, 16 * wv, 0, K);
+        gemm<T, 1, 1, false, false, true>(t, s_qt, LDK, 0, s_kt, LDK, 16 * wv, 0, K);
         acc_to_lds<T>(t[0][0], s_A, LDC, 16 * I, 16 * wv);
       }
       lds_barrier();
@@ -665,9 +665,9 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
     IOH::store_lds(x.rh, smT + A_H, LDV);
     IOH::store_lds(x.rdh, smT + A_DH, LDV);
     lds_barrier();      // LDS-only barriers: the loads requested above stay in flight
-    gemm_nt<T, 1, 4>(dP, smT + A_DO, LDV, 16 * wv, smT + A_V, LDV, 0, 0, BVH);
-    gemm_nt<T, 1, NBK>(dqi, smT + A_DO, LDV, 16 * wv, smT + A_H, LDV, 0, 0, BVH);
-    gemm_nt<T, 1, NBK>(dkd, smT + A_V, LDV, 16 * wv, smT + A_DH, LDV, 0, 0, BVH);
+    gemm_nt<T, 1, 4, true>(dP, smT + A_DO, LDV, 16 * wv, smT + A_V, LDV, 0, 0, BVH);
+    gemm_nt<T, 1, NBK, true>(dqi, smT + A_DO, LDV, 16 * wv, smT + A_H, LDV, 0, 0, BVH);
+    gemm_nt<T, 1, NBK, true>(dkd, smT + A_V, LDV, 16 * wv, smT + A_DH, LDV, 0, 0, BVH);
     lds_barrier();
   }
   // per state row k: sum_v S_kv dS'_kv  (the IOH::VPR adjacent threads of a pass share a row)
