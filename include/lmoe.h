@@ -141,7 +141,8 @@ int lmoe_chunk_gla_bwd(const lmoe_args* a, void* stream);
  * may both be NULL (a forward-only call); tinv may then be NULL too, but should be given: with it the 2-byte
  * state pass forms w and u on the chip from tinv, k, v, beta instead of reading them, and w, u are neither
  * written nor needed (they may be NULL; less memory traffic; the results of a call with and without tinv differ
- * in the last bit of w, u).  4-byte elements, or no tinv: w and u are required.
+ * in the last bit of w, u).  4-byte elements, or no tinv: w and u are required.  pmat: required for 4-byte elements,
+ * without tinv, or when hs is given; a forward-only 2-byte call with tinv forms P on the chip and may pass NULL.
  * bwd uses q,k,v,g,beta,hs,vnew,tinv,pmat,gcum,d_o,dht -> dq,dk,dv,dg,dbeta,dh0 (+ dhs, dvnew). */
 int lmoe_chunk_gated_delta_rule_fwd(const lmoe_args* a, void* stream);
 int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream);

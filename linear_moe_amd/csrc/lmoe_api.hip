@@ -127,7 +127,11 @@ int lmoe_chunk_gated_delta_rule_fwd(const lmoe_args* a, void* stream) {
   if (int r = check_common(a, op)) return r;
   if (a->gate == LMOE_GATE_VECTOR) return fail(-10, "%s: the gate is one scalar per token and head", op);
   if (!a->beta.ptr) return fail(-12, "%s: beta must not be null", op);
-  if (!a->o.ptr || !a->pmat || !a->gcum) return fail(-11, "%s: o, pmat and gcum must not be null", op);
+  if (!a->o.ptr || !a->gcum) return fail(-11, "%s: o and gcum must not be null", op);
+  // P reaches memory where the WY preparation forms it (4-byte elements, or no tinv) or where the backward will
+  // read it (hs given); a forward-only 2-byte call with tinv forms it inside the state pass and never stores it
+  if ((a->dtype != LMOE_BF16 || !a->tinv || a->hs) && !a->pmat)
+    return fail(-11, "%s: pmat must not be null (4-byte elements, no tinv given, or hs given)", op);
   // w, u are written and read only where the state pass does not form them itself from tinv
   if ((a->dtype != LMOE_BF16 || !a->tinv) && (!a->w.ptr || !a->u.ptr))
     return fail(-11, "%s: w and u must not be null (4-byte elements, or no tinv given)", op);
@@ -434,11 +438,13 @@ int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* strea
   if (op == LMOE_OP_SIMPLE_GLA || gdn) {
     switch (stage) {
       case lmoe::ST_GDN_WY_FWD: if (!gdn) return fail(-20, "%s: stage not part of this op", nm);
-        if (!a->pmat || !a->gcum) return fail(-11, "%s: pmat and gcum must not be null", nm);
+        if (!a->gcum || ((a->dtype != LMOE_BF16 || !a->tinv) && !a->pmat))
+          return fail(-11, "%s: gcum (and pmat: 4-byte elements or no tinv) must not be null", nm);
         lmoe::launch_gdn_wy_fwd(*a, st); break;
       case lmoe::ST_STATE_FWD:
         if (gdn) {
-          if (!a->pmat || !a->gcum) return fail(-11, "%s: pmat and gcum must not be null", nm);
+          if (!a->gcum || ((a->dtype != LMOE_BF16 || !a->tinv || a->hs) && !a->pmat))
+            return fail(-11, "%s: gcum (and pmat: 4-byte elements, no tinv, or hs given) must not be null", nm);
           lmoe::launch_gdn_state_fwd(*a, st);
         } else {
           lmoe::launch_state_fwd(*a, st);

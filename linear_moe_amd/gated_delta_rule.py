@@ -66,7 +66,8 @@ class GDNCall:
         hs = torch.empty(max(plan.NT, 1), H, K, V, dtype=dt, device=dev) if save else None
         # always: the backward reads it, and the forward state pass forms w from it (8 KB per chunk and head)
         tinv = torch.empty(max(plan.NT, 1), H, 64, 64, dtype=dt, device=dev)
-        pmat = torch.empty(max(plan.NT, 1), H, 64, 64, dtype=dt, device=dev)
+        # P: the bf16 forward pass forms it on the chip and stores it only for the backward
+        pmat = torch.empty(max(plan.NT, 1), H, 64, 64, dtype=dt, device=dev) if (save or dt == torch.float32) else None
         gcum = torch.empty(max(plan.NT, 1), H, 5, 64, dtype=torch.float32, device=dev)
         # w, u: the bf16 state passes form them on the chip from tinv; only the fp32 forward pass reads them
         w = torch.empty(B, T, H, K, dtype=dt, device=dev) if dt == torch.float32 else None
@@ -74,7 +75,7 @@ class GDNCall:
         # library-side layout [chunk, head, 32-column slice, token in chunk, column] (see include/lmoe.h)
         vnew = torch.empty(max(plan.NT, 1), H, V // 32, 64, 32, dtype=dt, device=dev) if save else None
         a.o, a.ht, a.hs, a.tinv = _desc(o, head_first), ptr(ht), ptr(hs), ptr(tinv)
-        a.pmat, a.gcum = pmat.data_ptr(), gcum.data_ptr()
+        a.pmat, a.gcum = ptr(pmat), gcum.data_ptr()
         a.w, a.u = _desc(w, False), _desc(u, False)
         a.vnew.ptr = ptr(vnew)
         _lib.check(lib.lmoe_chunk_gated_delta_rule_fwd(C.byref(a), stream_ptr()), "chunk_gated_delta_rule forward")
