@@ -33,14 +33,74 @@ def _check_inputs(q, k, v, head_first: bool, cu_seqlens) -> Tuple[int, int, int,
     else:
         B, T, H, K = q.shape
     V = v.shape[-1]
-    if K not in (64, 128) or V not in (64, 128):
-        raise ValueError(f"head dims K={K}, V={V} unsupported: K and V must be 64 or 128")
+    if K not in HEAD_DIMS or V not in HEAD_DIMS:
+        raise ValueError(f"head dims K={K}, V={V} unsupported: the kernels take K and V of 64 or 128 "
+                         "(the public ops pad and split other sizes before they get here)")
     if cu_seqlens is not None:
         if head_first:
             raise ValueError("cu_seqlens requires head_first=False ([1, T, H, D] packed input)")
         if B != 1:
             raise ValueError(f"cu_seqlens requires batch size 1 (packed input), got B={B}")
     return B, T, H, K, V
+
+
+HEAD_DIMS = (64, 128)      # what the kernels are instantiated for
+
+
+def dim_blocks(D: int):
+    """D columns as the blocks the kernels take: ``[(start, stop, width)]`` with width 128 or 64 (the last block
+    zero-padded up to its width)."""
+    if D < 1:
+        raise ValueError(f"head dimension must be positive, got {D}")
+    out, d0 = [], 0
+    while D - d0 > 128:
+        out.append((d0, d0 + 128, 128))
+        d0 += 128
+    out.append((d0, D, 64 if D - d0 <= 64 else 128))
+    return out
+
+
+def by_head_dim_blocks(core, q, k, v, gk, initial_state, output_final_state: bool, sum_over_k: bool, name: str):
+    """An op on head dimensions the kernels are not instantiated for, as calls on blocks of 128 / 64 columns.
+
+    The columns of v (and of the state) are independent in all three ops, so V is cut into blocks and the outputs
+    are concatenated; a short block is zero-padded (zero columns of v give zero columns of o and of the state).
+    K: zero columns of q and k change nothing, so a short K is padded; ``sum_over_k`` ops (no delta rule: the op is
+    a sum over key blocks) also take K > 128 as several blocks whose outputs are added in fp32.  ``core(q, k, v, gk,
+    h0) -> (o, ht)`` runs the op on supported dimensions (``gk``: the per-channel gate of chunk_gla or None).
+    Everything around ``core`` is differentiable torch code.  Each V block repeats the work that depends on q, k
+    only (for the delta rule the WY preparation): the supported dimensions are the fast path."""
+    pad = torch.nn.functional.pad
+    K, V = q.shape[-1], v.shape[-1]
+    kb, vb = dim_blocks(K), dim_blocks(V)
+    if len(kb) > 1 and not sum_over_k:
+        raise ValueError(f"{name}: K={K} unsupported: the delta rule needs the whole key in one block (K <= 128)")
+    if initial_state is not None and tuple(initial_state.shape[-2:]) != (K, V):
+        raise ValueError(f"{name}: initial_state must end in [{K}, {V}], got {tuple(initial_state.shape)}")
+    cut = lambda x, d0, d1, w: pad(x[..., d0:d1], (0, w - (d1 - d0))).contiguous()
+    qs = [(cut(q, k0, k1, w), cut(k, k0, k1, w), None if gk is None else cut(gk, k0, k1, w)) for k0, k1, w in kb]
+    o_cols, ht_cols = [], []
+    for v0, v1, vw in vb:
+        v_ = cut(v, v0, v1, vw)
+        o_v, ht_rows = None, []
+        for (k0, k1, kw), (q_, k_, g_) in zip(kb, qs):
+            h0 = None
+            if initial_state is not None:
+                h0 = pad(initial_state[..., k0:k1, v0:v1], (0, vw - (v1 - v0), 0, kw - (k1 - k0))).contiguous()
+            o_, ht_ = core(q_, k_, v_, g_, h0)
+            if len(kb) > 1:
+                o_ = o_.to(torch.promote_types(o_.dtype, torch.float32))
+            o_v = o_ if o_v is None else o_v + o_
+            if output_final_state:
+                ht_rows.append(ht_[..., :k1 - k0, :v1 - v0])
+        o_cols.append(o_v[..., :v1 - v0].to(v.dtype))
+        if output_final_state:
+            ht_cols.append(ht_rows[0] if len(ht_rows) == 1 else torch.cat(ht_rows, dim=-2))
+    o = o_cols[0] if len(o_cols) == 1 else torch.cat(o_cols, dim=-1)
+    ht = None
+    if output_final_state:
+        ht = ht_cols[0] if len(ht_cols) == 1 else torch.cat(ht_cols, dim=-1)
+    return o, ht
 
 
 def no_tokens(q, k, v, head_first: bool, cu_seqlens, initial_state, output_final_state: bool):

@@ -16,7 +16,8 @@ import torch
 
 from . import _lib
 from .l2norm import l2_norm
-from ._host import (seq_plan, _aligned, _check_inputs, _desc, _state_check, base_args, no_tokens, ptr, stream_ptr)
+from ._host import (HEAD_DIMS, seq_plan, _aligned, _check_inputs, _desc, _state_check, base_args, by_head_dim_blocks,
+                    no_tokens, ptr, stream_ptr)
 
 
 def _scalar_dt(x: torch.Tensor) -> int:
@@ -151,10 +152,18 @@ def chunk_gated_delta_rule(
     use_qk_l2norm_in_kernel: bool = False,
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """q, k: ``[B,T,H,K]``, v: ``[B,T,H,V]``, g (log-space decay) and beta: ``[B,T,H]``
-    (``[B,H,T,*]`` with ``head_first=True``).  Returns ``(o, final_state)``."""
+    (``[B,H,T,*]`` with ``head_first=True``).  Returns ``(o, final_state)``.  K, V of 64 or 128 run as they are;
+    a smaller K is zero-padded, any other V is cut into blocks of 128 / 64 columns (``_host.by_head_dim_blocks``)."""
     if use_qk_l2norm_in_kernel:
         q = l2_norm(q)
         k = l2_norm(k)
+    if q.dim() == 4 and v.dim() == 4 and (q.shape[-1] not in HEAD_DIMS or v.shape[-1] not in HEAD_DIMS):
+        # e.g. expand_v = 2 with a head dimension of 128: V = 256 as two blocks of 128 columns
+        sc = q.shape[-1] ** -0.5 if scale is None else scale          # of the whole key, not of the padded one
+        return by_head_dim_blocks(
+            lambda q_, k_, v_, _g, h0: chunk_gated_delta_rule(q_, k_, v_, g, beta, sc, h0, output_final_state,
+                                                              cu_seqlens, head_first),
+            q, k, v, None, initial_state, output_final_state, False, "chunk_gated_delta_rule")
     r = no_tokens(q, k, v, head_first, cu_seqlens, initial_state, output_final_state)
     if r is not None:
         return r

@@ -13,7 +13,8 @@ from typing import Optional, Tuple
 import torch
 
 from . import _lib
-from ._host import (seq_plan, _aligned, _check_inputs, _desc, _state_check, base_args, no_tokens, ptr, stream_ptr)
+from ._host import (HEAD_DIMS, seq_plan, _aligned, _check_inputs, _desc, _state_check, base_args, by_head_dim_blocks,
+                    no_tokens, ptr, stream_ptr)
 
 
 class GLACall:
@@ -116,6 +117,13 @@ def chunk_gla(
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """q, k, g: ``[B,H,T,K]``, v: ``[B,H,T,V]`` (``[B,T,H,*]`` with ``head_first=False``); g is the
     per-channel log-space decay.  Returns ``(o, final_state)``."""
+    if q.dim() == 4 and v.dim() == 4 and (q.shape[-1] not in HEAD_DIMS or v.shape[-1] not in HEAD_DIMS):
+        if g is None or g.shape != q.shape:
+            raise ValueError("chunk_gla: g must have the shape of q")
+        sc = q.shape[-1] ** -0.5 if scale is None else scale          # of the whole key, not of a block
+        return by_head_dim_blocks(
+            lambda q_, k_, v_, g_, h0: chunk_gla(q_, k_, v_, g_, sc, h0, output_final_state, cu_seqlens, head_first),
+            q, k, v, g, initial_state, output_final_state, True, "chunk_gla")
     r = no_tokens(q, k, v, head_first, cu_seqlens, initial_state, output_final_state)
     if r is not None:
         return r

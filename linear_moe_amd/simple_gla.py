@@ -13,7 +13,8 @@ from typing import Optional, Tuple
 import torch
 
 from . import _lib
-from ._host import (seq_plan, _aligned, _check_inputs, _desc, _state_check, base_args, no_tokens, ptr, stream_ptr)
+from ._host import (HEAD_DIMS, seq_plan, _aligned, _check_inputs, _desc, _state_check, base_args, by_head_dim_blocks,
+                    no_tokens, ptr, stream_ptr)
 
 
 class SimpleGLACall:
@@ -124,7 +125,13 @@ def chunk_simple_gla(
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """q, k: ``[B,H,T,K]``, v: ``[B,H,T,V]`` (``[B,T,H,*]`` with ``head_first=False``);
     g: ``[B,H,T]`` log-space decay or None.  Returns ``(o, final_state)`` with ``o`` shaped like
-    ``v`` and ``final_state`` fp32 ``[N,H,K,V]`` or None."""
+    ``v`` and ``final_state`` fp32 ``[N,H,K,V]`` or None.  K, V of 64 or 128 run as they are; any other size is
+    padded / cut into such blocks (``_host.by_head_dim_blocks``)."""
+    if q.dim() == 4 and v.dim() == 4 and (q.shape[-1] not in HEAD_DIMS or v.shape[-1] not in HEAD_DIMS):
+        sc = q.shape[-1] ** -0.5 if scale is None else scale          # of the whole key, not of a block
+        return by_head_dim_blocks(
+            lambda q_, k_, v_, _g, h0: chunk_simple_gla(q_, k_, v_, g, sc, h0, output_final_state, cu_seqlens, head_first),
+            q, k, v, None, initial_state, output_final_state, True, "chunk_simple_gla")
     r = no_tokens(q, k, v, head_first, cu_seqlens, initial_state, output_final_state)
     if r is not None:
         return r

@@ -267,3 +267,64 @@ def test_fla_shim_resolves_every_name_the_reference_imports():
     env["PYTHONPATH"] = shim
     out = subprocess.check_output([sys.executable, "-c", code], env=env, cwd=tempfile.gettempdir())
     assert out.strip() == b"ok"
+
+
+def test_head_dim_blocks_plan():
+    from linear_moe_amd._host import dim_blocks
+    assert dim_blocks(64) == [(0, 64, 64)] and dim_blocks(128) == [(0, 128, 128)]
+    assert dim_blocks(16) == [(0, 16, 64)] and dim_blocks(96) == [(0, 96, 128)]
+    assert dim_blocks(256) == [(0, 128, 128), (128, 256, 128)]
+    assert dim_blocks(192) == [(0, 128, 128), (128, 192, 64)]
+    for d in range(1, 400):
+        b = dim_blocks(d)
+        assert b[0][0] == 0 and b[-1][1] == d and all(x[1] == y[0] for x, y in zip(b, b[1:]))
+        assert all(w in (64, 128) and 0 < d1 - d0 <= w for d0, d1, w in b)
+    with pytest.raises(ValueError):
+        dim_blocks(0)
+
+
+@pytest.mark.parametrize("op,K,V", [("gla", 160, 80), ("gla", 48, 256), ("gdn", 96, 256), ("gdn", 32, 48)])
+def test_ops_on_other_head_dims_are_the_op_on_padded_blocks(op, K, V):
+    """The pad / cut / add logic around the kernels, with the fp64 token recurrence standing in for the kernels (on
+    the block sizes the kernels take, asserted): outputs, final state and every gradient equal the recurrence on
+    the whole head dimensions."""
+    from oracle import naive
+    from linear_moe_amd._host import by_head_dim_blocks
+    from tests.util import gen
+    B, T, H = 2, 9, 2
+    dd = torch.float64
+    q, k = gen(1, B, T, H, K, dtype=dd), gen(2, B, T, H, K, dtype=dd)
+    v, h0 = gen(3, B, T, H, V, dtype=dd), gen(4, B, H, K, V, dtype=dd) * 0.3
+    if op == "gdn":
+        k = torch.nn.functional.normalize(k, dim=-1)
+    gk = torch.nn.functional.logsigmoid(gen(5, B, T, H, K, dtype=dd)) if op == "gla" else None
+    g = -torch.rand(B, T, H, generator=torch.Generator().manual_seed(6), dtype=dd)
+    beta = torch.rand(B, T, H, generator=torch.Generator().manual_seed(7), dtype=dd)
+    scale = K ** -0.5
+    seen = []
+
+    def core(q_, k_, v_, g_, h_):
+        seen.append((q_.shape[-1], v_.shape[-1]))
+        if op == "gla":
+            return naive.naive_recurrent_gla(q_, k_, v_, g_, scale, h_, True, None, False)
+        return naive.naive_recurrent_gated_delta_rule(q_, k_, v_, g, beta, scale, h_, True, None, False)
+
+    leaves = [x.clone().requires_grad_(True) for x in (q, k, v, h0)] + ([gk.clone().requires_grad_(True)] if op == "gla" else [])
+    o, ht = by_head_dim_blocks(core, leaves[0], leaves[1], leaves[2], leaves[4] if op == "gla" else None, leaves[3], True,
+                               op == "gla", op)
+    assert all(kk in (64, 128) and vv in (64, 128) for kk, vv in seen)
+    ref_leaves = [x.clone().requires_grad_(True) for x in (q, k, v, h0)] + ([gk.clone().requires_grad_(True)] if op == "gla" else [])
+    if op == "gla":
+        ro, rht = naive.naive_recurrent_gla(ref_leaves[0], ref_leaves[1], ref_leaves[2], ref_leaves[4], scale, ref_leaves[3], True, None, False)
+    else:
+        ro, rht = naive.naive_recurrent_gated_delta_rule(ref_leaves[0], ref_leaves[1], ref_leaves[2], g, beta, scale, ref_leaves[3], True, None, False)
+    assert o.shape == ro.shape and ht.shape == rht.shape
+    assert torch.allclose(o, ro, atol=1e-10) and torch.allclose(ht, rht, atol=1e-10)
+    do, dht = gen(8, *o.shape, dtype=dd), gen(9, *ht.shape, dtype=dd)
+    gr = torch.autograd.grad((o * do).sum() + (ht * dht).sum(), leaves)
+    rr = torch.autograd.grad((ro * do).sum() + (rht * dht).sum(), ref_leaves)
+    for a, b in zip(gr, rr):
+        assert torch.allclose(a, b, atol=1e-9)
+    if op == "gdn":
+        with pytest.raises(ValueError, match="one block"):
+            by_head_dim_blocks(core, torch.zeros(1, 2, 1, 160), torch.zeros(1, 2, 1, 160), v[:1, :2, :1], None, None, False, False, op)
