@@ -79,8 +79,12 @@ def _trial(seed, trial, cuda):
     loss = (o * do.to(dtype).to(cuda)).sum() + ((ht * dht.to(cuda)).sum() if want_ht else 0)
     gg = torch.autograd.grad(loss, list(dl.values()))
     torch.cuda.synchronize()
-    # fp32: the cumulative gate of a chunk is itself an fp32 sum; at |b| ~ 100 its rounding alone is 1e-5 of e^b
-    tol = 2e-2 if dtype == torch.bfloat16 else (1e-5 if strength <= 1.0 else 1e-4)
+    # fp32 with the strongest gates (3 x logsigmoid: |b| up to ~180 inside a chunk): 2.5e-5 instead of 1e-5.  The
+    # cumulative gate of a chunk is an fp32 sum here as in fla; its rounding alone, with everything else exact, costs
+    # up to 3e-6 of the outputs and 6e-6 of dg at this strength (tests/test_oracle_pins.py::
+    # test_fp32_gate_scan_alone_costs_a_third_of_the_fp32_bar_at_strength_3), and the kernels measure 8e-6 on the
+    # outputs and 1.2e-5 on dg over the three ops
+    tol = 2e-2 if dtype == torch.bfloat16 else (1e-5 if strength <= 1.0 else 2.5e-5)
     what = f"seed {seed} trial {trial}: op={op} {dtype} K={K} V={V} H={H} T={T} B={B} lens={lens} head_first={hf} " \
            f"h0={use_h0} ht={want_ht} g={gdt} x{strength}"
     assert _rel(o.detach().cpu(), ro.detach()) < tol, what
