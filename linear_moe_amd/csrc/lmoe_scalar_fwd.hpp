@@ -22,16 +22,15 @@ template <typename T> __device__ __forceinline__ void scale_frag(typename ET<T>:
 //   grid = ceil(N*H / 8) * 8 * (V / BV) work-groups (1-D).  Work-group -> (sequence, head,
 //   V-slice): the V-slices of one (sequence, head) get ids that are congruent mod 8, i.e. run on
 //   the same XCD and share q, k through its L2.
-//   Team 0 (waves 0-3, consumers) carries the dependency chain of the state and, in the same window, forms
-//     P = (q k^T) . Gamma for the output team (wave-private LDS strips):
-//        S -> LDS (element type T) | B1 | S = e^{b_C} S + k^T (e_d v), P -> LDS | B2
+//   Team 0 (waves 0-3, consumers) carries the dependency chain of the state and nothing else:
+//        S -> LDS (element type T) | B1 | S = e^{b_C} S + k^T (e_d v) | B2
 //     wave w owns state rows [w*K/4, (w+1)*K/4) x BV columns in fp32 MFMA accumulators; the row
 //     scaling e_d is applied to the v fragments in registers, so k is staged unscaled.
 //   Team 1 (waves 4-7, loaders) keeps the operands of the next PF chunks in flight in registers,
 //     forms the gate cumsum, fills the other LDS buffer and writes hs (layout [V][K]) from the
 //     LDS copy of S (SAVE; a forward-only call passes hs = NULL and nothing is written).
-//   Team 2 (waves 8-11, output) forms the chunk's output rows 16w..: between B1 and B2
-//     e^{b_i} q S, after B2 P v (P from the strip consumer wave w wrote).
+//   Team 2 (waves 8-11, output) forms the chunk's output rows 16w.. between B1 and B2: e^{b_i} q S, its rows of
+//     P = (q k^T) . Gamma (through a wave-private LDS strip) and P v; the rows are stored after B2.
 //   All teams meet at the same barriers; three waves per SIMD hide each other's latencies.
 // ------------------------------------------------------------------------- //
 template <typename T, int K, int V, int BV, bool SAVE>
@@ -146,33 +145,69 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
       const int tok = sq.tok0 + c * CH;
       const int len = min(CH, sq.len - c * CH);
       lds_barrier();                                                                     // B1
-      f32x4 o[1][NB];
+      // Everything of output rows 16 ow .. happens in this window, where the consumers only update the state:
+      // e^{b} q S, the rows of P = (q k^T) . Gamma (blocks above the diagonal are zero and skipped), and P v with P
+      // through this wave's own LDS strip (no work-group barrier between them).  Every fragment and gate value is
+      // requested before the first product (left to the compiler, each read is waited for where it is used and
+      // the window is a chain of LDS round trips).  fp32: looped products (its fragments do not fit the registers).
+      f32x4 o[1][NB], p[4];
       acc_zero(o);
+#pragma unroll
+      for (int nj = 0; nj < 4; ++nj) p[nj] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const int fr = l & 15, fg = 8 * (l >> 4);
+      const f32x4 bi = *(const f32x4*)&s_b[cur][16 * ow + 4 * (l >> 4)];
+      float bj[4];
+#pragma unroll
+      for (int nj = 0; nj < 4; ++nj) bj[nj] = s_b[cur][16 * nj + fr];
       if constexpr (sizeof(T) == 4) {
         gemm<T, 1, NB, false, false>(o, s_q[cur], LDK, 16 * ow, s_hT, LDK, 0, 0, K);
+        f32x4 pp[1][4];
+        acc_zero(pp);
+        gemm<T, 1, 4, false, false>(pp, s_q[cur], LDK, 16 * ow, s_k[cur], LDK, 0, 0, K);
+#pragma unroll
+        for (int nj = 0; nj < 4; ++nj) p[nj] = pp[0][nj];
       } else {
-        // all fragments requested before the first product (see the consumers' P window)
         constexpr int KS = K / 32;
-        const int fr = l & 15, fg = 8 * (l >> 4);
-        typename ET<T>::frag fq[KS], fh[KS][NB];
+        typename ET<T>::frag fq[KS], fh[KS][NB], fk[KS][4];
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
           fq[ks] = ET<T>::load_frag(s_q[cur] + (16 * ow + fr) * LDK + 32 * ks + fg);
 #pragma unroll
           for (int ni = 0; ni < NB; ++ni) fh[ks][ni] = ET<T>::load_frag(s_hT + (16 * ni + fr) * LDK + 32 * ks + fg);
+#pragma unroll
+          for (int nj = 0; nj < 4; ++nj)
+            if (nj <= ow) fk[ks][nj] = ET<T>::load_frag(s_k[cur] + (16 * nj + fr) * LDK + 32 * ks + fg);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
+        for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
           for (int ni = 0; ni < NB; ++ni) ET<T>::mma(o[0][ni], fq[ks], fh[ks][ni]);
+#pragma unroll
+          for (int nj = 0; nj < 4; ++nj)
+            if (nj <= ow) ET<T>::mma(p[nj], fq[ks], fk[ks][nj]);
+        }
       }
 #pragma unroll
       for (int ni = 0; ni < NB; ++ni)
 #pragma unroll
         for (int e = 0; e < 4; ++e) o[0][ni][e] *= s_eb[cur][16 * ow + 4 * (l >> 4) + e];
-      lds_barrier();                                                                     // B2 (orders pst too)
-      gemm<T, 1, NB, false, true>(o, pst, LDC, 0, s_u[cur], LDU, 0, 0, CH);
+#pragma unroll
+      for (int nj = 0; nj < 4; ++nj) {
+        f32x4 x;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int i = 16 * ow + 4 * (l >> 4) + e, j = 16 * nj + fr;
+          x[e] = (i >= j) ? p[nj][e] * texp<T>(bi[e] - bj[nj]) : 0.f;
+        }
+        acc_to_lds<T>(x, pst, LDC, 0, 16 * nj);
+      }
+      // the strip is this wave's own: ordering inside the wave is enough
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      gemm<T, 1, NB, false, true, true>(o, pst, LDC, 0, s_u[cur], LDU, 0, 0, CH);
+      lds_barrier();                                                                     // B2
       store_strip<T, NB>(o, s_ost + ow * 16 * LDU, row_ptr<T>(a.o, sq.b, tok + 16 * ow, h) + v0, a.o.st,
                          len - 16 * ow, a.scale);
       if constexpr (NBUF == 1) lds_barrier();                                            // B3
@@ -232,54 +267,6 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
 #pragma unroll
           for (int ni = 0; ni < NB; ++ni) ET<T>::mma(S[mi][ni], af[kq][mi], bf[kq][ni]);
       __builtin_amdgcn_sched_barrier(0);
-    }
-    // rows 16 wv .. of P = (q k^T) . Gamma for the output team (it reads them after B2)
-    {
-      // every fragment and gate value is requested before the first product (left to the compiler, each read is
-      // waited for where it is used and the window is a chain of LDS round trips); blocks above the diagonal
-      // (nj > wv) are zero and skipped
-      // (2-byte elements; the fp32 fragments of a whole K = 128 window do not fit the registers: looped product)
-      constexpr int KS = K / 32;
-      const int fr = l & 15, fg = 8 * (l >> 4);
-      const f32x4 bi = *(const f32x4*)&s_b[cur][16 * wv + 4 * (l >> 4)];
-      float bj[4];
-#pragma unroll
-      for (int nj = 0; nj < 4; ++nj) bj[nj] = s_b[cur][16 * nj + fr];
-      f32x4 p[4];
-#pragma unroll
-      for (int nj = 0; nj < 4; ++nj) p[nj] = f32x4{0.f, 0.f, 0.f, 0.f};
-      if constexpr (sizeof(T) == 2) {
-        typename ET<T>::frag fq[KS], fk[KS][4];
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          fq[ks] = ET<T>::load_frag(s_q[cur] + (16 * wv + fr) * LDK + 32 * ks + fg);
-#pragma unroll
-          for (int nj = 0; nj < 4; ++nj)
-            if (nj <= wv) fk[ks][nj] = ET<T>::load_frag(s_k[cur] + (16 * nj + fr) * LDK + 32 * ks + fg);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-          for (int nj = 0; nj < 4; ++nj)
-            if (nj <= wv) ET<T>::mma(p[nj], fq[ks], fk[ks][nj]);
-      } else {
-        f32x4 pp[1][4];
-        acc_zero(pp);
-        gemm<T, 1, 4, false, false>(pp, s_q[cur], LDK, 16 * wv, s_k[cur], LDK, 0, 0, K);
-#pragma unroll
-        for (int nj = 0; nj < 4; ++nj) p[nj] = pp[0][nj];
-      }
-#pragma unroll
-      for (int nj = 0; nj < 4; ++nj) {
-        f32x4 x;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int i = 16 * wv + 4 * (l >> 4) + e, j = 16 * nj + fr;
-          x[e] = (i >= j) ? p[nj][e] * texp<T>(bi[e] - bj[nj]) : 0.f;
-        }
-        acc_to_lds<T>(x, s_pst + wv * 16 * LDC, LDC, 0, 16 * nj);
-      }
     }
     lds_barrier();                                                                       // B2
     if constexpr (NBUF == 1) lds_barrier();                                              // B3
