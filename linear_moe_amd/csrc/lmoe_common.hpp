@@ -302,6 +302,49 @@ __device__ __forceinline__ void store_strip(const f32x4 (&acc)[1][NB], T* stg, T
   }
 }
 
+// The same for a strip held transposed (acc[ni]: rows = columns 16 ni + 4 (l / 16) + e of the strip, column = row l % 16
+// of the strip, i.e. a lane holds four consecutive columns of one row): 8-byte writes into the staging area.
+template <typename T, int NB>
+__device__ __forceinline__ void store_strip_t(const f32x4 (&acc)[NB], T* stg, T* __restrict__ gdst,
+                                              int64_t row_stride, int nvalid, float mul, int l = threadIdx.x & 63) {
+  constexpr int W = NB * 16, LD = W + LPAD, VEC = ET<T>::VEC, VPR = W / VEC;
+  typedef typename ET<T>::vec vec;
+#pragma unroll
+  for (int ni = 0; ni < NB; ++ni) {
+    const f32x4 x = acc[ni] * mul;
+    acc_to_lds_t<T>(x, stg, LD, 16 * ni, 0, l);
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+  for (int idx = l; idx < 16 * VPR; idx += 64) {
+    const int r = idx / VPR, c = (idx % VPR) * VEC;
+    if (r < nvalid) *(vec*)(gdst + (int64_t)r * row_stride + c) = *(const vec*)(stg + r * LD + c);
+  }
+}
+
+// Operands that never leave the registers.  A pair of 16-wide accumulator blocks of a transposed product lies in a
+// lane as elements e = 0..3 of block 2s (contraction index 32 s + 4 g + e, g = l / 16) and of block 2s + 1
+// (32 s + 16 + 4 g + e); frag_of_blocks packs them into an MFMA operand in that numbering, and
+// load_frag_t_blocks reads the other operand (a tile with the contraction index along its rows) in the same
+// numbering through the transposing LDS read: lane (c = l % 16, g) receives tile[k0 + 4 g + e][n0 + c] and
+// tile[k0 + 16 + 4 g + e][n0 + c].  The contraction index may be numbered freely as long as both operands agree.
+__device__ __forceinline__ bf16x8 frag_of_blocks(const f32x4& a, const f32x4& b) {
+  bf16x8 f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { f[i] = (bf16)a[i]; f[4 + i] = (bf16)b[i]; }
+  return f;
+}
+__device__ __forceinline__ bf16x8 load_frag_t_blocks(const bf16* tile, int ld, int k0, int n0, int l = threadIdx.x & 63) {
+  const int s = l & 15;
+  const bf16* p = tile + (k0 + 4 * (l >> 4) + (s >> 2)) * ld + n0 + 4 * (s & 3);
+  typedef __attribute__((address_space(3))) bf16x4 lds_b4;
+  const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_b4*)p);
+  const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_b4*)(p + 16 * ld));
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
 // ------------------------------------------------------------------------- //
 // fragments held in registers
 // ------------------------------------------------------------------------- //

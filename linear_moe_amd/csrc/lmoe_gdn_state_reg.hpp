@@ -51,13 +51,7 @@ __device__ __forceinline__ bf16x8 load_frag_t_state(const bf16* tile, int ld, in
   const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_b4*)(p + 4 * ld));
   return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
-// two accumulator blocks -> the 8 contraction elements of a B (or A) operand
-__device__ __forceinline__ bf16x8 frag_of_blocks(const f32x4& a, const f32x4& b) {
-  bf16x8 f;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) { f[i] = (bf16)a[i]; f[4 + i] = (bf16)b[i]; }
-  return f;
-}
+// (frag_of_blocks, lmoe_common.hpp: two accumulator blocks -> the 8 contraction elements of an operand)
 
 template <int K, int V, bool SAVE, bool TRACE = false>
 __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd_reg(const lmoe_args a, long long* tr, int traced_wg) {

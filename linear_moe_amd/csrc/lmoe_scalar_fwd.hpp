@@ -30,7 +30,7 @@ template <typename T> __device__ __forceinline__ void scale_frag(typename ET<T>:
 //     forms the gate cumsum, fills the other LDS buffer and writes hs (layout [V][K]) from the
 //     LDS copy of S (SAVE; a forward-only call passes hs = NULL and nothing is written).
 //   Team 2 (waves 8-11, output) forms the chunk's output rows 16w.. between B1 and B2: e^{b_i} q S, its rows of
-//     P = (q k^T) . Gamma (through a wave-private LDS strip) and P v; the rows are stored after B2.
+//     P = (q k^T) . Gamma (kept in registers as an MFMA operand) and P v; the rows are stored after B2.
 //   All teams meet at the same barriers; three waves per SIMD hide each other's latencies.
 // ------------------------------------------------------------------------- //
 template <typename T, int K, int V, int BV, bool SAVE>
@@ -146,29 +146,51 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
       const int len = min(CH, sq.len - c * CH);
       lds_barrier();                                                                     // B1
       // Everything of output rows 16 ow .. happens in this window, where the consumers only update the state:
-      // e^{b} q S, the rows of P = (q k^T) . Gamma (blocks above the diagonal are zero and skipped), and P v with P
-      // through this wave's own LDS strip (no work-group barrier between them).  Every fragment and gate value is
-      // requested before the first product (left to the compiler, each read is waited for where it is used and
-      // the window is a chain of LDS round trips).  fp32: looped products (its fragments do not fit the registers).
-      f32x4 o[1][NB], p[4];
-      acc_zero(o);
-#pragma unroll
-      for (int nj = 0; nj < 4; ++nj) p[nj] = f32x4{0.f, 0.f, 0.f, 0.f};
+      // e^{b} q S, the rows of P = (q k^T) . Gamma (blocks above the diagonal are zero and skipped), and P v.
       const int fr = l & 15, fg = 8 * (l >> 4);
-      const f32x4 bi = *(const f32x4*)&s_b[cur][16 * ow + 4 * (l >> 4)];
-      float bj[4];
-#pragma unroll
-      for (int nj = 0; nj < 4; ++nj) bj[nj] = s_b[cur][16 * nj + fr];
       if constexpr (sizeof(T) == 4) {
-        gemm<T, 1, NB, false, false>(o, s_q[cur], LDK, 16 * ow, s_hT, LDK, 0, 0, K);
-        f32x4 pp[1][4];
+        // fp32 (the parity path): looped products, P through this wave's own LDS strip
+        f32x4 o[1][NB], pp[1][4];
+        acc_zero(o);
         acc_zero(pp);
+        const f32x4 bi = *(const f32x4*)&s_b[cur][16 * ow + 4 * (l >> 4)];
+        float bj[4];
+#pragma unroll
+        for (int nj = 0; nj < 4; ++nj) bj[nj] = s_b[cur][16 * nj + fr];
+        gemm<T, 1, NB, false, false>(o, s_q[cur], LDK, 16 * ow, s_hT, LDK, 0, 0, K);
         gemm<T, 1, 4, false, false>(pp, s_q[cur], LDK, 16 * ow, s_k[cur], LDK, 0, 0, K);
 #pragma unroll
-        for (int nj = 0; nj < 4; ++nj) p[nj] = pp[0][nj];
+        for (int ni = 0; ni < NB; ++ni)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o[0][ni][e] *= s_eb[cur][16 * ow + 4 * (l >> 4) + e];
+#pragma unroll
+        for (int nj = 0; nj < 4; ++nj) {
+          f32x4 x;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int i = 16 * ow + 4 * (l >> 4) + e, j = 16 * nj + fr;
+            x[e] = (i >= j) ? pp[0][nj][e] * texp<T>(bi[e] - bj[nj]) : 0.f;
+          }
+          acc_to_lds<T>(x, pst, LDC, 0, 16 * nj);
+        }
+        // the strip is this wave's own: ordering inside the wave is enough
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        gemm<T, 1, NB, false, true>(o, pst, LDC, 0, s_u[cur], LDU, 0, 0, CH);
+        lds_barrier();                                                                   // B2
+        store_strip<T, NB>(o, s_ost + ow * 16 * LDU, row_ptr<T>(a.o, sq.b, tok + 16 * ow, h) + v0, a.o.st,
+                           len - 16 * ow, a.scale);
       } else {
-        constexpr int KS = K / 32;
-        typename ET<T>::frag fq[KS], fh[KS][NB], fk[KS][4];
+        // 2-byte elements.  All three products are formed transposed (the MFMA operands swapped), so that a lane
+        // holds four consecutive columns of ONE token: P^T = k q^T then lies in the lanes as the operand of
+        // (P v)^T = v^T P^T needs it (frag_of_blocks; v^T read in the matching numbering, load_frag_t_blocks) and
+        // never goes through LDS, the gate factors of a lane are one b_i and four consecutive b_j, and the result
+        // leaves as 8-byte writes.  Every fragment and gate value is requested before the first product (left to the
+        // compiler, each read is waited for where it is used and the window is a chain of LDS round trips).
+        constexpr int KS = K / 32, CS = CH / 32;
+        const int g4 = 4 * (l >> 4);
+        typename ET<T>::frag fq[KS], fh[KS][NB], fk[KS][4], fv[CS][NB];
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
           fq[ks] = ET<T>::load_frag(s_q[cur] + (16 * ow + fr) * LDK + 32 * ks + fg);
@@ -179,37 +201,52 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
             if (nj <= ow) fk[ks][nj] = ET<T>::load_frag(s_k[cur] + (16 * nj + fr) * LDK + 32 * ks + fg);
         }
         __builtin_amdgcn_sched_barrier(0);
+        f32x4 ot[NB], pt[4];
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) ot[ni] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int nj = 0; nj < 4; ++nj) pt[nj] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
-          for (int ni = 0; ni < NB; ++ni) ET<T>::mma(o[0][ni], fq[ks], fh[ks][ni]);
+          for (int ni = 0; ni < NB; ++ni) ET<T>::mma(ot[ni], fh[ks][ni], fq[ks]);      // (q S)^T: column x token
 #pragma unroll
           for (int nj = 0; nj < 4; ++nj)
-            if (nj <= ow) ET<T>::mma(p[nj], fq[ks], fk[ks][nj]);
+            if (nj <= ow) ET<T>::mma(pt[nj], fk[ks][nj], fq[ks]);                       // P^T: token j x token i
         }
-      }
+        // second batch (the fragments above are dead by now: all of them at once do not fit the registers)
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int ni = 0; ni < NB; ++ni)
+        for (int kq = 0; kq < CS; ++kq)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) o[0][ni][e] *= s_eb[cur][16 * ow + 4 * (l >> 4) + e];
+          for (int ni = 0; ni < NB; ++ni)
+            if (2 * kq <= ow) fv[kq][ni] = load_frag_t_blocks(s_u[cur], LDU, 32 * kq, 16 * ni, l);
+        const float bi = s_b[cur][16 * ow + fr], ebi = s_eb[cur][16 * ow + fr];
+        f32x4 bj[4];
 #pragma unroll
-      for (int nj = 0; nj < 4; ++nj) {
-        f32x4 x;
+        for (int nj = 0; nj < 4; ++nj) bj[nj] = *(const f32x4*)&s_b[cur][16 * nj + g4];
+        __builtin_amdgcn_sched_barrier(0);
+        const int i = 16 * ow + fr;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int i = 16 * ow + 4 * (l >> 4) + e, j = 16 * nj + fr;
-          x[e] = (i >= j) ? p[nj][e] * texp<T>(bi[e] - bj[nj]) : 0.f;
+        for (int ni = 0; ni < NB; ++ni) ot[ni] *= ebi;
+#pragma unroll
+        for (int nj = 0; nj < 4; ++nj)
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            pt[nj][e] = (i >= 16 * nj + g4 + e) ? pt[nj][e] * texp<T>(bi - bj[nj][e]) : 0.f;
+#pragma unroll
+        for (int kq = 0; kq < CS; ++kq) {
+          if (2 * kq <= ow) {        // tokens j >= 32 only reach the rows of waves 2, 3
+            const typename ET<T>::frag fp = frag_of_blocks(pt[2 * kq], pt[2 * kq + 1]);
+#pragma unroll
+            for (int ni = 0; ni < NB; ++ni) ET<T>::mma(ot[ni], fv[kq][ni], fp);         // (P v)^T
+          }
         }
-        acc_to_lds<T>(x, pst, LDC, 0, 16 * nj);
+        __builtin_amdgcn_sched_barrier(0);
+        lds_barrier();                                                                   // B2
+        store_strip_t<T, NB>(ot, s_ost + ow * 16 * LDU, row_ptr<T>(a.o, sq.b, tok + 16 * ow, h) + v0, a.o.st,
+                             len - 16 * ow, a.scale);
       }
-      // the strip is this wave's own: ordering inside the wave is enough
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      gemm<T, 1, NB, false, true, true>(o, pst, LDC, 0, s_u[cur], LDU, 0, 0, CH);
-      lds_barrier();                                                                     // B2
-      store_strip<T, NB>(o, s_ost + ow * 16 * LDU, row_ptr<T>(a.o, sq.b, tok + 16 * ow, h) + v0, a.o.st,
-                         len - 16 * ow, a.scale);
       if constexpr (NBUF == 1) lds_barrier();                                            // B3
     }
     return;
