@@ -38,17 +38,17 @@ STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_gdn_state_fwd_reg", 4: "k_gdn_state_bwd"
 # sources (kernel_sources_sha16()) at that time, and a build whose sources differ reports traffic = null
 # rather than a stale number.
 CALIB_COPY_BYTES = 256 << 20
-MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237243536, "k_gdn_state_fwd_reg": 1117137601, "k_gdn_state_bwd": 945961314,
-                    "k_gdn_bwd_chunk": 1899242186}
-TRAFFIC_SOURCES_SHA16 = "48644f82270f92d3"
+MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237241774, "k_gdn_state_fwd_reg": 1116410418, "k_gdn_state_bwd": 945961993,
+                    "k_gdn_bwd_chunk": 1899497310}
+TRAFFIC_SOURCES_SHA16 = "508fc52e88a73456"
 TRAFFIC_SOURCES = ("lmoe_common.hpp", "lmoe_seq.hpp", "lmoe_gdn_wy.hpp", "lmoe_gdn_state.hpp", "lmoe_gdn_state_reg.hpp", "lmoe_gdn_bwd_chunk.hpp",
                    "lmoe_gdn_fwd.hip", "lmoe_gdn_state.hip", "lmoe_gdn_bwd.hip")
 
 
 # HBM bytes per call of the other contract configurations (bench.py --other-configs), same counters and scaling,
 # summed over the kernels of the call; key = configuration number
-OTHER_TRAFFIC = {"1": 2219521, "2": 272839110, "3": 1548094122, "5": 16916894035}
-OTHER_TRAFFIC_SHA16 = "2804adff68c0593f"
+OTHER_TRAFFIC = {"1": 2225660, "2": 272839866, "3": 1547999228, "5": 16913294511}
+OTHER_TRAFFIC_SHA16 = "e5f9ce7c4566025a"
 
 
 def all_sources_sha16():
