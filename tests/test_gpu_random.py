@@ -92,13 +92,13 @@ def _trial(seed, trial, cuda):
         assert _rel(ht.detach().cpu(), rht.detach()) < tol, what
     grads = dict(zip(rl, zip(gg, rg)))
     for n, (a, b) in grads.items():
-        # dg is a difference of terms of the size of q.dq: where it vanishes identically (no state ahead of a one-token
-        # sequence) the error is measured against those terms
-        floor = 0.1 * float(grads['q'][1].abs().max() * rl['q'].detach().abs().max()) if n == 'g' else 0.0
+        # dg is a difference of terms of the size of q.dq (a sum over the K channels of a token): where it vanishes
+        # identically (no state ahead of a one-token sequence) the error is measured against those terms
+        floor = float((grads['q'][1] * rl['q'].detach()).sum(-1).abs().max()) if n == 'g' else 0.0
         assert _rel(a.cpu(), b, floor) < tol, (what, n)
 
 
-@pytest.mark.parametrize("seed", [1, 2, 3])
+@pytest.mark.parametrize("seed", [1, 2, 3, 4, 5, 6])
 def test_random_problems(cuda, seed):
     for trial in range(60):
         _trial(seed, trial, cuda)
