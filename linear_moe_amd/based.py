@@ -21,13 +21,8 @@ def _poly_attn(q, k, v, c0, c1, c2, scale, use_normalize, eps):
     # sqrt(2 c2) scale x_i x_j]
     fm = lambda x: quad_feature_map(x, c0 ** 0.5, (c1 * scale) ** 0.5, c2 ** 0.5 * scale, (2.0 * c2) ** 0.5 * scale)
     qb, kb = fm(q), fm(k)
-    o, _ = chunk_linear_attn(qb, kb, v, scale=1.0, normalize=False)
-    if use_normalize:
-        z = None
-        for qi, ki in zip(qb, kb):
-            zi = (qi * ki.cumsum(2)).sum(-1, keepdim=True)
-            z = zi if z is None else z + zi
-        o = o / (z + eps)
+    # (the normaliser is one more value column inside the kernels: chunk_linear_attn)
+    o, _ = chunk_linear_attn(qb, kb, v, scale=1.0, normalize=use_normalize, _eps=eps)
     return o.to(v.dtype)
 
 

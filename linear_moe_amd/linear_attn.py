@@ -24,7 +24,10 @@ def chunk_linear_attn(
     output_final_state: bool = False,
     normalize: bool = True,
     head_first: bool = True,
+    _eps: float = 1e-10,
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """``_eps`` (not part of fla's signature): the epsilon of the normaliser, for the callers in this package whose
+    reference functions carry their own (``based.py``)."""
     qb, kb = _key_blocks(q), _key_blocks(k)
     if [b.shape for b in qb] != [b.shape for b in kb]:
         raise ValueError("chunk_linear_attn: q and k must agree in shape")
@@ -35,28 +38,37 @@ def chunk_linear_attn(
         if initial_state.shape[-2] > K:
             raise ValueError(f"chunk_linear_attn: initial_state has {initial_state.shape[-2]} key rows, q has {K}")
         initial_state = torch.nn.functional.pad(initial_state, (0, 0, 0, K - initial_state.shape[-2]))
-    tdim = 2 if head_first else 1
-    o, hts, z, k0 = None, [], None, 0
+    # The normaliser z_i = scale sum_{j<=i} q_i . k_j is the op itself with one more value column of ones (fla
+    # normalises with q * scale, so the scale cancels in o up to the epsilon): it is formed inside the kernels, in
+    # the fp32 state, instead of by a cumulative sum over k in HBM.  chunk_simple_gla cuts the V + 1 columns into
+    # the blocks the kernels take; the carried state has no normaliser column (the sum starts inside the call).
+    V = v.shape[-1]
+    if normalize:
+        v = torch.cat([v, v.new_ones(*v.shape[:-1], 1)], dim=-1)
+        if initial_state is not None:
+            initial_state = torch.nn.functional.pad(initial_state, (0, 1))
+    o, hts, k0 = None, [], 0
     for qi, ki in zip(qb, kb):
         w = qi.shape[-1]
         h0 = None if initial_state is None else initial_state[..., k0:k0 + w, :].contiguous()
         oi, hi = chunk_simple_gla(qi, ki, v, None, scale, h0, output_final_state, None, head_first)
+        if len(qb) > 1:
+            oi = oi.float()
         o = oi if o is None else o + oi
         hts.append(hi)
-        if normalize:
-            # the normaliser carries the scale of the numerator (fla normalises with q * scale), so that
-            # the scale cancels in o up to the epsilon
-            zi = ((qi * scale) * ki.cumsum(tdim)).sum(-1, keepdim=True)
-            z = zi if z is None else z + zi
         k0 += w
     if normalize:
-        o = o / (z + 1e-10)
+        o = o.float()
+        o = o[..., :V] / (o[..., V:] + _eps)
+    o = o.to(v.dtype)
     ht = None
     if output_final_state:
         ht = hts[0] if len(hts) == 1 else torch.cat(hts, dim=-2)
         feats = q.features if hasattr(q, "features") else q.shape[-1]
         if feats != K:
             ht = ht[..., :feats, :]
+        if normalize:
+            ht = ht[..., :V]
     return o, ht
 
 
