@@ -38,8 +38,8 @@ STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_gdn_state_fwd_reg", 4: "k_gdn_state_bwd"
 # sources (kernel_sources_sha16()) at that time, and a build whose sources differ reports traffic = null
 # rather than a stale number.
 CALIB_COPY_BYTES = 256 << 20
-MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237241774, "k_gdn_state_fwd_reg": 1116410418, "k_gdn_state_bwd": 945961993,
-                    "k_gdn_bwd_chunk": 1899497310}
+MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237244044, "k_gdn_state_fwd_reg": 1117018555, "k_gdn_state_bwd": 945962556,
+                    "k_gdn_bwd_chunk": 1899370989}
 TRAFFIC_SOURCES_SHA16 = "508fc52e88a73456"
 TRAFFIC_SOURCES = ("lmoe_common.hpp", "lmoe_seq.hpp", "lmoe_gdn_wy.hpp", "lmoe_gdn_state.hpp", "lmoe_gdn_state_reg.hpp", "lmoe_gdn_bwd_chunk.hpp",
                    "lmoe_gdn_fwd.hip", "lmoe_gdn_state.hip", "lmoe_gdn_bwd.hip")
@@ -47,8 +47,8 @@ TRAFFIC_SOURCES = ("lmoe_common.hpp", "lmoe_seq.hpp", "lmoe_gdn_wy.hpp", "lmoe_g
 
 # HBM bytes per call of the other contract configurations (bench.py --other-configs), same counters and scaling,
 # summed over the kernels of the call; key = configuration number
-OTHER_TRAFFIC = {"1": 2225660, "2": 272839866, "3": 1547999228, "5": 16913294511}
-OTHER_TRAFFIC_SHA16 = "e5f9ce7c4566025a"
+OTHER_TRAFFIC = {"1": 2228727, "2": 272917723, "3": 1548112021, "5": 16909265279}
+OTHER_TRAFFIC_SHA16 = "7a5d17dfbe6920cd"
 
 
 def all_sources_sha16():
@@ -317,6 +317,56 @@ def trace_state_fwd(lib, x, dims, work_group=16):
             "teams": out}
 
 
+def trace_simple_gla_fwd(lib, dev, work_group=16):
+    """The same breakdown for the forward pass of chunk_simple_gla (k_state_fwd_b) on contract configuration 2
+    (retention, forward-only, B=4 H=16 T=4096 K=V=128 bf16): lmoe_trace_simple_gla_fwd, include/lmoe.h."""
+    import torch
+    from linear_moe_amd import _lib
+    from linear_moe_amd.retention import retention_log_decay
+    from linear_moe_amd.simple_gla import SimpleGLACall
+    B, H, T, K = 4, 16, 4096, 128
+    q, k, v = (torch.randn(B, H, T, K, device=dev, dtype=torch.bfloat16) for _ in range(3))
+    g = retention_log_decay(H, dev)[None, :, None].expand(B, H, T)
+    call = SimpleGLACall(keep=True)
+    call.forward(q, k, v, g, None, None, True, None, True, save=False)
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    slots, chunks, marks = 3, 24, 8
+    tr = torch.zeros(slots * chunks * marks, dtype=torch.int64, device=dev)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for _ in range(3):
+        _lib.check(lib.lmoe_trace_simple_gla_fwd(C.byref(call.fwd_args), tr.data_ptr(), work_group, st), "trace")
+    e0.record()
+    _lib.check(lib.lmoe_trace_simple_gla_fwd(C.byref(call.fwd_args), tr.data_ptr(), work_group, st), "trace")
+    e1.record()
+    e1.synchronize()
+    traced_us = e0.elapsed_time(e1) * 1e3
+    t = tr.cpu().view(slots, chunks, marks).double()
+    nall = (T + CH - 1) // CH
+    nch = min(chunks, nall)
+    c0, c1 = nch // 4, nch - nch // 4
+    ref = t[0, c0:c1, 1]
+    period = float((t[0, c0 + 1:c1 + 1, 1] - t[0, c0:c1, 1]).mean())
+    names = {0: {0: "arrives_barrier", 1: "leaves_barrier", 5: "state_updated", 6: "state_copied", 2: "next_P_below_diagonal_formed"},
+             1: {0: "arrives_barrier", 1: "leaves_barrier", 5: "loads_issued", 2: "staged", 4: "hs_stored"},
+             2: {0: "arrives_barrier", 1: "leaves_barrier", 5: "qS_issued", 2: "Pv_done", 4: "rows_stored",
+                 6: "next_P_diagonal_formed"}}
+    teams = {0: "consumer_wave", 1: "loader_wave", 2: "output_wave"}
+    out = {}
+    for s_, nm in teams.items():
+        out[nm] = {}
+        for m, label in names[s_].items():
+            d = float((t[s_, c0:c1, m] - ref).mean())
+            if m == 0:
+                d += period
+                label = "arrives_next_barrier"
+            out[nm][label] = round(d)
+    return {"metric": "k_state_fwd_b: shader-clock cycles after the barrier of a chunk, per team (traced build)",
+            "unit": "cycles", "config": {"workload": "retention fwd bf16 B=4 H=16 T=4096 K=V=128"},
+            "work_group": work_group, "chunks_averaged": [c0, c1], "period_cycles": round(period),
+            "traced_kernel_us": round(traced_us, 1), "cycles_per_us": round(period * nall / traced_us, 1),
+            "teams": out}
+
+
 def other_configs(dev, steps, warmup):
     """The four contract configurations beside the headline one, through the Python entry points (inputs of
     the contract's laws, drawn on the GPU: this leg times, the parity tests check): ms per call, tokens/s and
@@ -419,6 +469,9 @@ def main():
     ap.add_argument("--trace-state-fwd", action="store_true",
                     help="instead of the headline step: the per-phase breakdown of one chunk period of the forward "
                          "sequential pass on the headline workload, one JSON line")
+    ap.add_argument("--trace-simple-gla-fwd", action="store_true",
+                    help="instead of the headline step: the same breakdown for the forward pass of chunk_simple_gla "
+                         "on contract configuration 2, one JSON line")
     ap.add_argument("--other-configs", action="store_true",
                     help="instead of the headline step: contract configurations 1, 2, 3 and 5, one JSON line")
     args = ap.parse_args()
@@ -448,6 +501,9 @@ def main():
         return
     if args.other_configs:
         print(json.dumps(other_configs(dev, args.steps, args.warmup)))
+        return
+    if args.trace_simple_gla_fwd:
+        print(json.dumps(trace_simple_gla_fwd(lib, dev)))
         return
     x = gdn_inputs(B, T, H, K, V, seed, torch.bfloat16, dev)
     if args.trace_state_fwd:

@@ -51,7 +51,7 @@ ENTRY_POINTS = (
     "lmoe_gdn_gates_partials", "lmoe_gdn_gates_fwd", "lmoe_gdn_gates_bwd", "lmoe_gla_gate_fwd", "lmoe_gla_gate_bwd",
     "lmoe_hgrn2_gate_fwd", "lmoe_hgrn2_gate_bwd", "lmoe_quad_featmap_features", "lmoe_quad_featmap_fwd",
     "lmoe_quad_featmap_bwd",
-    "lmoe_fused_recurrent_fwd", "lmoe_trace_gdn_state_fwd", "lmoe_mom_gather", "lmoe_mom_combine", "lmoe_mom_rowdot",
+    "lmoe_fused_recurrent_fwd", "lmoe_trace_gdn_state_fwd", "lmoe_trace_simple_gla_fwd", "lmoe_mom_gather", "lmoe_mom_combine", "lmoe_mom_rowdot",
 )
 
 _lib = None
@@ -123,6 +123,8 @@ def load() -> C.CDLL:
     lib.lmoe_fused_recurrent_fwd.restype = C.c_int
     lib.lmoe_trace_gdn_state_fwd.argtypes = [C.POINTER(Args), C.c_void_p, C.c_int32, C.c_void_p]
     lib.lmoe_trace_gdn_state_fwd.restype = C.c_int
+    lib.lmoe_trace_simple_gla_fwd.argtypes = [C.POINTER(Args), C.c_void_p, C.c_int32, C.c_void_p]
+    lib.lmoe_trace_simple_gla_fwd.restype = C.c_int
     lib.lmoe_mom_gather.argtypes = [C.c_void_p] * 4 + [C.c_int64, C.c_int32, C.c_int32, C.c_void_p]
     lib.lmoe_mom_gather.restype = C.c_int
     for fn in (lib.lmoe_mom_combine, lib.lmoe_mom_rowdot):

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Build-time guard of the register-steered kernels.
 
-The hot kernels of the gated delta rule rely on the compiler keeping their working set in registers (explicit
+The hot kernels of the gated delta rule and the forward pass of chunk_simple_gla rely on the compiler keeping their working set in registers (explicit
 steering: refreshed lane indices, pinned sums, fenced products).  A compiler or source change that makes one of them
 spill, or lowers the number of waves it runs with, costs a large factor in speed without failing any test.  This
 script reads the per-kernel resource reports that ``-Rpass-analysis=kernel-resource-usage`` wrote at compile time
@@ -18,6 +18,7 @@ import sys
 # passes and the chunk-parallel backward run one work-group of 12 waves per CU = 3 waves per SIMD; the WY
 # preparation two or three work-groups of 4 waves)
 GUARDED = {
+    "k_state_fwd_b": 3,
     "k_gdn_state_fwd": 3,
     "k_gdn_state_fwd_reg": 3,
     "k_gdn_state_bwd": 3,

@@ -252,6 +252,18 @@ int lmoe_rmsnorm_bwd_noalloc(const void* x, const void* w, const void* gate, con
   return launched(nm);
 }
 
+int lmoe_trace_simple_gla_fwd(const lmoe_args* a, int64_t* trace, int32_t work_group, void* stream) {
+  const char* nm = "lmoe_trace_simple_gla_fwd";
+  if (int r = check_common(a, nm)) return r;
+  if (!trace) return fail(-1, "%s: trace must not be null", nm);
+  if (a->gate == LMOE_GATE_VECTOR || !a->o.ptr)
+    return fail(-11, "%s: needs the populated argument block of lmoe_chunk_simple_gla_fwd", nm);
+  if (a->NT == 0 || a->N == 0) return fail(-4, "%s: nothing to trace in an empty problem", nm);
+  if (!lmoe::launch_state_fwd_trace(*a, (long long*)trace, work_group, (hipStream_t)stream))
+    return fail(-24, "%s: traced instance exists for bf16, K = V = 128, forward-only (hs NULL), work_group inside the grid", nm);
+  return launched(nm);
+}
+
 int lmoe_trace_gdn_state_fwd(const lmoe_args* a, int64_t* trace, int32_t work_group, void* stream) {
   const char* nm = "lmoe_trace_gdn_state_fwd";
   if (int r = check_common(a, nm)) return r;

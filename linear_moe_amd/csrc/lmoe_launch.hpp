@@ -32,6 +32,8 @@ inline void dispatch(const lmoe_args& a, hipStream_t st) {
 }
 
 void launch_state_fwd(const lmoe_args& a, hipStream_t st);        // chunk_simple_gla
+// traced forward pass of chunk_simple_gla (bf16, K = V = 128, forward-only): false when the problem is not of that shape
+bool launch_state_fwd_trace(const lmoe_args& a, long long* tr, int work_group, hipStream_t st);
 void launch_gdn_state_fwd(const lmoe_args& a, hipStream_t st);    // gated delta rule
 void launch_gdn_state_bwd(const lmoe_args& a, hipStream_t st);
 // traced forward pass (bf16, K = V = 128, Tinv and hs given): false when the problem is not of that shape

@@ -13,11 +13,25 @@ template <typename T, int K, int V> struct StateFwd {
   static void run(const lmoe_args& a, hipStream_t st) {
     constexpr int BV = FwdTiles<T, V>::BVS;
     const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BV);
-    if (a.hs) hipLaunchKernelGGL((k_state_fwd<T, K, V, BV, true>), dim3(grid), dim3(3 * NTHR), 0, st, a);
-    else hipLaunchKernelGGL((k_state_fwd<T, K, V, BV, false>), dim3(grid), dim3(3 * NTHR), 0, st, a);
+    if constexpr (sizeof(T) == 2) {
+      if (a.hs) hipLaunchKernelGGL((k_state_fwd_b<T, K, V, BV, true>), dim3(grid), dim3(3 * NTHR), 0, st, a, (long long*)nullptr, -1);
+      else hipLaunchKernelGGL((k_state_fwd_b<T, K, V, BV, false>), dim3(grid), dim3(3 * NTHR), 0, st, a, (long long*)nullptr, -1);
+    } else {
+      if (a.hs) hipLaunchKernelGGL((k_state_fwd<T, K, V, BV, true>), dim3(grid), dim3(3 * NTHR), 0, st, a);
+      else hipLaunchKernelGGL((k_state_fwd<T, K, V, BV, false>), dim3(grid), dim3(3 * NTHR), 0, st, a);
+    }
   }
 };
 void launch_state_fwd(const lmoe_args& a, hipStream_t st) { dispatch<StateFwd>(a, st); }
+// the traced instance of the pass (2-byte elements, K = V = 128, forward-only call)
+bool launch_state_fwd_trace(const lmoe_args& a, long long* tr, int work_group, hipStream_t st) {
+  if (a.dtype != LMOE_BF16 || a.K != 128 || a.V != 128 || a.hs) return false;
+  constexpr int BV = FwdTiles<bf16, 128>::BVS;
+  const int grid = ((a.N * a.H + 7) / 8) * 8 * (128 / BV);
+  if (work_group < 0 || work_group >= grid) return false;
+  hipLaunchKernelGGL((k_state_fwd_b<bf16, 128, 128, BV, false, true>), dim3(grid), dim3(3 * NTHR), 0, st, a, tr, work_group);
+  return true;
+}
 // C = A B^T (64 x 64, contraction along the tile columns) and G = A^T B (KD x KD, contraction
 // along the tile rows, i.e. the transposed-fragment path) over one pair of 64 x KD tiles,
 // through the loaders / fragments / accumulator stores of the toolkit

@@ -18,7 +18,9 @@ template <typename T> __device__ __forceinline__ void scale_frag(typename ET<T>:
 }
 
 // ------------------------------------------------------------------------- //
-// state pass + output (forward): work-group of three teams of four waves (768 threads)
+// state pass + output (forward), fp32 elements (the parity path): work-group of three teams of four waves
+// (768 threads); the LDS holds one operand buffer, so a chunk costs three barriers.  k_state_fwd_b below is the pass
+// for 2-byte elements.
 //   grid = ceil(N*H / 8) * 8 * (V / BV) work-groups (1-D).  Work-group -> (sequence, head,
 //   V-slice): the V-slices of one (sequence, head) get ids that are congruent mod 8, i.e. run on
 //   the same XCD and share q, k through its L2.
@@ -27,26 +29,25 @@ template <typename T> __device__ __forceinline__ void scale_frag(typename ET<T>:
 //     wave w owns state rows [w*K/4, (w+1)*K/4) x BV columns in fp32 MFMA accumulators; the row
 //     scaling e_d is applied to the v fragments in registers, so k is staged unscaled.
 //   Team 1 (waves 4-7, loaders) keeps the operands of the next PF chunks in flight in registers,
-//     forms the gate cumsum, fills the other LDS buffer and writes hs (layout [V][K]) from the
+//     forms the gate cumsum, fills the LDS buffer and writes hs (layout [V][K]) from the
 //     LDS copy of S (SAVE; a forward-only call passes hs = NULL and nothing is written).
 //   Team 2 (waves 8-11, output) forms the chunk's output rows 16w.. between B1 and B2: e^{b_i} q S, its rows of
-//     P = (q k^T) . Gamma (kept in registers as an MFMA operand) and P v; the rows are stored after B2.
+//     P = (q k^T) . Gamma (through a wave-private LDS strip) and P v; the rows are stored after B2.
 //   All teams meet at the same barriers; three waves per SIMD hide each other's latencies.
 // ------------------------------------------------------------------------- //
 template <typename T, int K, int V, int BV, bool SAVE>
 __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
+  static_assert(sizeof(T) == 4, "fp32 elements; 2-byte elements: k_state_fwd_b");
   constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDU = BV + LPAD;
   constexpr int MB = K / 64, NB = BV / 16;
-  // bf16: two operand buffers; fp32 (the parity path) has LDS for one and pays a third barrier
-  constexpr int NBUF = sizeof(T) == 2 ? 2 : 1;
-  __shared__ __attribute__((aligned(16))) T s_k[NBUF][CH * LDK];              // k             [64][K]
-  __shared__ __attribute__((aligned(16))) T s_q[NBUF][CH * LDK];              // q             [64][K]
-  __shared__ __attribute__((aligned(16))) T s_u[NBUF][CH * LDU];              // u or v        [64][BV]
+  __shared__ __attribute__((aligned(16))) T s_k[1][CH * LDK];              // k             [64][K]
+  __shared__ __attribute__((aligned(16))) T s_q[1][CH * LDK];              // q             [64][K]
+  __shared__ __attribute__((aligned(16))) T s_u[1][CH * LDU];              // u or v        [64][BV]
   __shared__ __attribute__((aligned(16))) T s_hT[BV * LDK];                   // S^T           [BV][K]
   __shared__ __attribute__((aligned(16))) T s_pst[4 * 16 * LDC];              // team 2: P strips
   __shared__ __attribute__((aligned(16))) T s_ost[4 * 16 * LDU];              // team 2: o store
-  __shared__ __attribute__((aligned(16))) float s_b[NBUF][64], s_eb[NBUF][64], s_ed[NBUF][64];
-  __shared__ float s_dec[NBUF];                                               // e^{b_C} per buffer
+  __shared__ __attribute__((aligned(16))) float s_b[1][64], s_eb[1][64], s_ed[1][64];
+  __shared__ float s_dec[1];                                               // e^{b_C} per buffer
 
   constexpr int NVS = V / BV;
   const int xcd = blockIdx.x & 7, jj = blockIdx.x >> 3;
@@ -119,17 +120,12 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
         const int c = c0 + j;
         if (c >= sq.nchunks) break;
         lds_barrier();                                                                   // B1
-        // the next chunk's operands first (always: past the end it is the last chunk again, never consumed),
-        // so that the wait for their loads does not sit behind the store below
-        if constexpr (NBUF == 2) stage(pre[(j + 1) % PF], (c + 1) & 1);
         // hs[chunk][h][v0 .. v0+BV][K] <- S^T (only the backward reads it: SAVE = false for forward-only calls)
         if constexpr (SAVE)
           IOHT::lds_to_global(s_hT, LDK, (T*)a.hs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
         lds_barrier();                                                                   // B2
-        if constexpr (NBUF == 1) {
-          lds_barrier();                                                                 // B3: buffer read
-          if (c + 1 < sq.nchunks) stage(pre[(j + 1) % PF], 0);
-        }
+        lds_barrier();                                                                   // B3: buffer read
+        if (c + 1 < sq.nchunks) stage(pre[(j + 1) % PF], 0);
         issue(pre[(j + 1) % PF], c + 1 + PF);
       }
     }
@@ -141,113 +137,46 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
     const int ow = wave_id() - 8;
     T* pst = s_pst + ow * 16 * LDC;
     for (int c = 0; c < sq.nchunks; ++c) {
-      const int cur = NBUF == 2 ? (c & 1) : 0;
+      constexpr int cur = 0;
       const int tok = sq.tok0 + c * CH;
       const int len = min(CH, sq.len - c * CH);
       lds_barrier();                                                                     // B1
       // Everything of output rows 16 ow .. happens in this window, where the consumers only update the state:
       // e^{b} q S, the rows of P = (q k^T) . Gamma (blocks above the diagonal are zero and skipped), and P v.
-      const int fr = l & 15, fg = 8 * (l >> 4);
-      if constexpr (sizeof(T) == 4) {
-        // fp32 (the parity path): looped products, P through this wave's own LDS strip
-        f32x4 o[1][NB], pp[1][4];
-        acc_zero(o);
-        acc_zero(pp);
-        const f32x4 bi = *(const f32x4*)&s_b[cur][16 * ow + 4 * (l >> 4)];
-        float bj[4];
+      const int fr = l & 15;
+      // looped products, P through this wave's own LDS strip
+      f32x4 o[1][NB], pp[1][4];
+      acc_zero(o);
+      acc_zero(pp);
+      const f32x4 bi = *(const f32x4*)&s_b[cur][16 * ow + 4 * (l >> 4)];
+      float bj[4];
 #pragma unroll
-        for (int nj = 0; nj < 4; ++nj) bj[nj] = s_b[cur][16 * nj + fr];
-        gemm<T, 1, NB, false, false>(o, s_q[cur], LDK, 16 * ow, s_hT, LDK, 0, 0, K);
-        gemm<T, 1, 4, false, false>(pp, s_q[cur], LDK, 16 * ow, s_k[cur], LDK, 0, 0, K);
+      for (int nj = 0; nj < 4; ++nj) bj[nj] = s_b[cur][16 * nj + fr];
+      gemm<T, 1, NB, false, false>(o, s_q[cur], LDK, 16 * ow, s_hT, LDK, 0, 0, K);
+      gemm<T, 1, 4, false, false>(pp, s_q[cur], LDK, 16 * ow, s_k[cur], LDK, 0, 0, K);
 #pragma unroll
-        for (int ni = 0; ni < NB; ++ni)
+      for (int ni = 0; ni < NB; ++ni)
 #pragma unroll
-          for (int e = 0; e < 4; ++e) o[0][ni][e] *= s_eb[cur][16 * ow + 4 * (l >> 4) + e];
+        for (int e = 0; e < 4; ++e) o[0][ni][e] *= s_eb[cur][16 * ow + 4 * (l >> 4) + e];
 #pragma unroll
-        for (int nj = 0; nj < 4; ++nj) {
-          f32x4 x;
+      for (int nj = 0; nj < 4; ++nj) {
+        f32x4 x;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int i = 16 * ow + 4 * (l >> 4) + e, j = 16 * nj + fr;
-            x[e] = (i >= j) ? pp[0][nj][e] * texp<T>(bi[e] - bj[nj]) : 0.f;
-          }
-          acc_to_lds<T>(x, pst, LDC, 0, 16 * nj);
+        for (int e = 0; e < 4; ++e) {
+          const int i = 16 * ow + 4 * (l >> 4) + e, j = 16 * nj + fr;
+          x[e] = (i >= j) ? pp[0][nj][e] * texp<T>(bi[e] - bj[nj]) : 0.f;
         }
-        // the strip is this wave's own: ordering inside the wave is enough
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        gemm<T, 1, NB, false, true>(o, pst, LDC, 0, s_u[cur], LDU, 0, 0, CH);
-        lds_barrier();                                                                   // B2
-        store_strip<T, NB>(o, s_ost + ow * 16 * LDU, row_ptr<T>(a.o, sq.b, tok + 16 * ow, h) + v0, a.o.st,
-                           len - 16 * ow, a.scale);
-      } else {
-        // 2-byte elements.  All three products are formed transposed (the MFMA operands swapped), so that a lane
-        // holds four consecutive columns of ONE token: P^T = k q^T then lies in the lanes as the operand of
-        // (P v)^T = v^T P^T needs it (frag_of_blocks; v^T read in the matching numbering, load_frag_t_blocks) and
-        // never goes through LDS, the gate factors of a lane are one b_i and four consecutive b_j, and the result
-        // leaves as 8-byte writes.  Every fragment and gate value is requested before the first product (left to the
-        // compiler, each read is waited for where it is used and the window is a chain of LDS round trips).
-        constexpr int KS = K / 32, CS = CH / 32;
-        const int g4 = 4 * (l >> 4);
-        typename ET<T>::frag fq[KS], fh[KS][NB], fk[KS][4], fv[CS][NB];
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          fq[ks] = ET<T>::load_frag(s_q[cur] + (16 * ow + fr) * LDK + 32 * ks + fg);
-#pragma unroll
-          for (int ni = 0; ni < NB; ++ni) fh[ks][ni] = ET<T>::load_frag(s_hT + (16 * ni + fr) * LDK + 32 * ks + fg);
-#pragma unroll
-          for (int nj = 0; nj < 4; ++nj)
-            if (nj <= ow) fk[ks][nj] = ET<T>::load_frag(s_k[cur] + (16 * nj + fr) * LDK + 32 * ks + fg);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        f32x4 ot[NB], pt[4];
-#pragma unroll
-        for (int ni = 0; ni < NB; ++ni) ot[ni] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int nj = 0; nj < 4; ++nj) pt[nj] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-#pragma unroll
-          for (int ni = 0; ni < NB; ++ni) ET<T>::mma(ot[ni], fh[ks][ni], fq[ks]);      // (q S)^T: column x token
-#pragma unroll
-          for (int nj = 0; nj < 4; ++nj)
-            if (nj <= ow) ET<T>::mma(pt[nj], fk[ks][nj], fq[ks]);                       // P^T: token j x token i
-        }
-        // second batch (the fragments above are dead by now: all of them at once do not fit the registers)
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int kq = 0; kq < CS; ++kq)
-#pragma unroll
-          for (int ni = 0; ni < NB; ++ni)
-            if (2 * kq <= ow) fv[kq][ni] = load_frag_t_blocks(s_u[cur], LDU, 32 * kq, 16 * ni, l);
-        const float bi = s_b[cur][16 * ow + fr], ebi = s_eb[cur][16 * ow + fr];
-        f32x4 bj[4];
-#pragma unroll
-        for (int nj = 0; nj < 4; ++nj) bj[nj] = *(const f32x4*)&s_b[cur][16 * nj + g4];
-        __builtin_amdgcn_sched_barrier(0);
-        const int i = 16 * ow + fr;
-#pragma unroll
-        for (int ni = 0; ni < NB; ++ni) ot[ni] *= ebi;
-#pragma unroll
-        for (int nj = 0; nj < 4; ++nj)
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            pt[nj][e] = (i >= 16 * nj + g4 + e) ? pt[nj][e] * texp<T>(bi - bj[nj][e]) : 0.f;
-#pragma unroll
-        for (int kq = 0; kq < CS; ++kq) {
-          if (2 * kq <= ow) {        // tokens j >= 32 only reach the rows of waves 2, 3
-            const typename ET<T>::frag fp = frag_of_blocks(pt[2 * kq], pt[2 * kq + 1]);
-#pragma unroll
-            for (int ni = 0; ni < NB; ++ni) ET<T>::mma(ot[ni], fv[kq][ni], fp);         // (P v)^T
-          }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        lds_barrier();                                                                   // B2
-        store_strip_t<T, NB>(ot, s_ost + ow * 16 * LDU, row_ptr<T>(a.o, sq.b, tok + 16 * ow, h) + v0, a.o.st,
-                             len - 16 * ow, a.scale);
+        acc_to_lds<T>(x, pst, LDC, 0, 16 * nj);
       }
-      if constexpr (NBUF == 1) lds_barrier();                                            // B3
+      // the strip is this wave's own: ordering inside the wave is enough
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      gemm<T, 1, NB, false, true>(o, pst, LDC, 0, s_u[cur], LDU, 0, 0, CH);
+      lds_barrier();                                                                     // B2
+      store_strip<T, NB>(o, s_ost + ow * 16 * LDU, row_ptr<T>(a.o, sq.b, tok + 16 * ow, h) + v0, a.o.st,
+                         len - 16 * ow, a.scale);
+      lds_barrier();                                                                     // B3
     }
     return;
   }
@@ -268,7 +197,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
           S[mi][ni][i] = h0[(int64_t)(krow0 + acc_row(mi, i)) * V + v0 + acc_col(ni)];
   }
   for (int c = 0; c < sq.nchunks; ++c) {
-    const int cur = NBUF == 2 ? (c & 1) : 0;
+    constexpr int cur = 0;
     // S (state at chunk start) -> LDS as S^T
 #pragma unroll
     for (int mi = 0; mi < MB; ++mi)
@@ -306,8 +235,362 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
       __builtin_amdgcn_sched_barrier(0);
     }
     lds_barrier();                                                                       // B2
-    if constexpr (NBUF == 1) lds_barrier();                                              // B3
+    lds_barrier();                                                                       // B3
   }
+  if (a.ht) {
+    float* ht = a.ht + ((int64_t)n * a.H + h) * K * V;
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          ht[(int64_t)(krow0 + acc_row(mi, i)) * V + v0 + acc_col(ni)] = S[mi][ni][i];
+  }
+}
+
+// ------------------------------------------------------------------------- //
+// The same pass for 2-byte elements, one barrier per chunk: whatever a window reads was completed in the window
+// before.  Three operand buffers (chunk c is worked on, chunk c + 1 is complete, chunk c + 2 is being staged), two
+// copies of S^T and two of P = (q k^T) . Gamma.  Window c, between barrier c and barrier c + 1:
+//   consumers: S = e^{b_C} S + k^T (e_d v) on buffer c % 3, S -> s_hT[(c + 1) & 1], then the blocks of P of chunk
+//              c + 1 below the diagonal -> s_P[(c + 1) & 1] (the state update alone takes a third of a window; the
+//              output team, which formed its rows of P itself in an earlier version, was the longest chain of it)
+//   loaders:   loads of chunk c + 4 issued into the register set that the last window's staging freed, chunk c + 2
+//              staged into buffer (c + 2) % 3, hs <- s_hT[c & 1] (SAVE)
+//   output:    rows 16 w .. of o = e^b q S (s_hT[c & 1]) + P (s_P[c & 1]) v, stored from registers, then the
+//              diagonal blocks of P of chunk c + 1
+// Time stamps of the traced instance (TRACE = true): one wave of each team notes the shader clock where it arrives
+// at and leaves the barrier of a chunk and at a few points in between; the stamps sit in LDS (a global store
+// per stamp would perturb the wave that is measured) and each of those waves copies its own out at the end:
+// tr[slot][chunk][mark], slots 0 consumers, 1 loaders, 2 output team; marks: include/lmoe.h.
+// ------------------------------------------------------------------------- //
+constexpr int SFWD_TRACE_CHUNKS = 24, SFWD_TRACE_MARKS = 8, SFWD_TRACE_SLOTS = 3;
+
+template <typename T, int K, int V, int BV, bool SAVE, bool TRACE = false>
+__global__ __launch_bounds__(3 * NTHR) void k_state_fwd_b(const lmoe_args a, long long* tr, int traced_wg) {
+  static_assert(sizeof(T) == 2, "2-byte elements");
+  constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDU = BV + LPAD;
+  constexpr int MB = K / 64, NB = BV / 16, KS = K / 32, CS = CH / 32;
+  __shared__ __attribute__((aligned(16))) T s_k[3][CH * LDK];                 // k             [64][K]
+  __shared__ __attribute__((aligned(16))) T s_q[3][CH * LDK];                 // q             [64][K]
+  __shared__ __attribute__((aligned(16))) T s_u[3][CH * LDU];                 // v             [64][BV]
+  __shared__ __attribute__((aligned(16))) T s_hT[2][BV * LDK];                // S^T           [BV][K]
+  __shared__ __attribute__((aligned(16))) T s_P[2][CH * LDC];                 // P             [64][64]
+  __shared__ __attribute__((aligned(16))) float s_b[3][64], s_eb[3][64], s_ed[3][64];
+  __shared__ float s_dec[3];                                                  // e^{b_C} per buffer
+  // (the low 32 bits of the clock: the LDS has no room for more beside the buffers of the pass)
+  __shared__ uint32_t s_tr[TRACE ? SFWD_TRACE_SLOTS * SFWD_TRACE_CHUNKS * SFWD_TRACE_MARKS : 1];
+  auto TR = [&](int slot, int c, int mark) {
+    if constexpr (TRACE) {
+      if ((int)blockIdx.x == traced_wg && (threadIdx.x & 63) == 0 && c < SFWD_TRACE_CHUNKS)
+        s_tr[(slot * SFWD_TRACE_CHUNKS + c) * SFWD_TRACE_MARKS + mark] = (uint32_t)__builtin_readcyclecounter();
+    }
+  };
+  auto trace_out = [&](int slot) {       // by the wave that wrote the slot: ordering inside the wave is enough
+    if constexpr (TRACE) {
+      if ((int)blockIdx.x == traced_wg) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        constexpr int N = SFWD_TRACE_CHUNKS * SFWD_TRACE_MARKS;
+        for (int i = threadIdx.x & 63; i < N; i += 64) tr[slot * N + i] = s_tr[slot * N + i];
+      }
+    }
+  };
+  if constexpr (TRACE) {
+    for (int i = threadIdx.x; i < SFWD_TRACE_SLOTS * SFWD_TRACE_CHUNKS * SFWD_TRACE_MARKS; i += 3 * NTHR) s_tr[i] = 0;
+    __syncthreads();
+  }
+
+  constexpr int NVS = V / BV;
+  const int xcd = blockIdx.x & 7, jj = blockIdx.x >> 3;
+  const int vsl = jj % NVS, pair = (jj / NVS) * 8 + xcd;
+  if (pair >= a.N * a.H) return;
+  const int v0 = vsl * BV, h = pair % a.H, n = pair / a.H;
+  const SeqInfo sq = seq_info(a, n);
+  const int l = lane_id();
+  // (wave-uniform by construction; said to the compiler, so that the branches on it are scalar branches: a matrix
+  // instruction runs whatever the lane mask, and a short masked region is not jumped over)
+  const int wave = __builtin_amdgcn_readfirstlane(wave_id());
+  const int team = wave >> 2;
+  if (sq.nchunks == 0) {
+    // empty sequence: the final state is the initial state
+    if (a.ht && team == 0) {
+      for (int idx = threadIdx.x; idx < K * BV; idx += NTHR) {
+        const int r = idx / BV, c = v0 + idx % BV;
+        const int64_t o = ((int64_t)n * a.H + h) * K * V + (int64_t)r * V + c;
+        a.ht[o] = a.h0 ? a.h0[o] : 0.f;
+      }
+    }
+    return;
+  }
+  typedef TileIO<T, CH, K> IOK;
+  typedef TileIO<T, CH, BV> IOV;
+  typedef TileIO<T, BV, K> IOHT;
+
+  // Blocks (ti, tj[0 .. n)) of P of chunk c (16 x 16 each, one q strip against n <= 2 k strips), formed transposed so
+  // that a lane holds four consecutive columns of one row (8-byte writes).  The ten blocks on and below the diagonal
+  // are dealt to eight waves: the output team takes the diagonal (wave w: block (w, w)) once its rows are stored,
+  // the consumers the six blocks below it (waves 0, 1: rows 3, 2 against k strips 0, 1; wave 2: (3, 2); wave 3: (1, 0)).
+  // Every fragment is requested before the first product: the LDS is busiest right behind the barrier, a read comes
+  // back after several hundred cycles, and a product loop that requests one step ahead pays that once per step.
+  auto p_blocks = [&](int c, int ti, int tja, int tjb, int n) {
+    const int cb = c % 3, fr = l & 15, g = l >> 4;
+    const T *qc = s_q[cb], *kc = s_k[cb];
+    T* Pn = s_P[c & 1];
+    typename ET<T>::frag fq[KS], fka[KS], fkb[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      fq[ks] = ET<T>::load_frag(qc + (16 * ti + fr) * LDK + 32 * ks + 8 * g);
+      fka[ks] = ET<T>::load_frag(kc + (16 * tja + fr) * LDK + 32 * ks + 8 * g);
+      if (n == 2) fkb[ks] = ET<T>::load_frag(kc + (16 * tjb + fr) * LDK + 32 * ks + 8 * g);
+    }
+    // the decay factors (masked: only the diagonal block has entries above the diagonal) while the fragments are on
+    // their way
+    const int i = 16 * ti + fr;
+    const float bi = s_b[cb][i];
+    const f32x4 bja = *(const f32x4*)&s_b[cb][16 * tja + 4 * g], bjb = *(const f32x4*)&s_b[cb][16 * tjb + 4 * g];
+    f32x4 ga, gb;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      ga[e] = (i >= 16 * tja + 4 * g + e) ? texp<T>(bi - bja[e]) : 0.f;
+      gb[e] = texp<T>(bi - bjb[e]);
+    }
+    f32x4 pa = {0.f, 0.f, 0.f, 0.f}, pb = {0.f, 0.f, 0.f, 0.f};
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      ET<T>::mma(pa, fka[ks], fq[ks]);
+      if (n == 2) ET<T>::mma(pb, fkb[ks], fq[ks]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    bf16x4 y;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) y[e] = (bf16)(pa[e] * ga[e]);
+    *(bf16x4*)(Pn + i * LDC + 16 * tja + 4 * g) = y;
+    if (n == 2) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) y[e] = (bf16)(pb[e] * gb[e]);
+      *(bf16x4*)(Pn + i * LDC + 16 * tjb + 4 * g) = y;
+    }
+  };
+
+  if (team == 1) {
+    // --------------------------------- loaders -------------------------------------------
+    struct Pre { typename IOK::Regs rk, rq; typename IOV::Regs ru; uint32_t graw; int len; };
+    Pre pre[3];                                              // register set = chunk % 3
+    const bool gated = a.gate != LMOE_GATE_NONE && a.g.ptr != nullptr;
+    const void* gptr = gated ? a.g.ptr : a.k.ptr;
+    // Always issued (chunk index clamped to the last chunk; the surplus loads at the end of a
+    // sequence are never consumed): a prefetch that is skipped on some path would make the
+    // compiler drain all outstanding loads at every consumer of a register set.
+    auto issue = [&](Pre& P, int c) {
+      c = min(c, sq.nchunks - 1);
+      const int tok = sq.tok0 + c * CH;
+      const int len = min(CH, sq.len - c * CH);
+      IOK::load_nomask(P.rk, row_ptr<T>(a.k, sq.b, tok, h), a.k.st, len);
+      IOK::load_nomask(P.rq, row_ptr<T>(a.q, sq.b, tok, h), a.q.st, len);
+      IOV::load_nomask(P.ru, row_ptr<T>(a.v, sq.b, tok, h) + v0, a.v.st, len);
+      P.len = len;
+      P.graw = load_scalar_raw(gptr, a.g_dtype, gated ? row_off(a.g, sq.b, tok + min(l, len - 1), h) : 0);
+    };
+    // registers -> LDS buffer `buf`
+    auto stage = [&](Pre& P, int buf) {
+      IOK::mask(P.rk, P.len);
+      IOK::mask(P.rq, P.len);
+      IOV::mask(P.ru, P.len);
+      IOK::store_lds(P.rk, s_k[buf], LDK);
+      IOK::store_lds(P.rq, s_q[buf], LDK);
+      IOV::store_lds(P.ru, s_u[buf], LDU);
+      if (wave == 4) {
+        const float x = wave_incl_scan((gated && l < P.len) ? scalar_from_raw(P.graw, a.g_dtype) : 0.f);
+        const float xl = __shfl(x, 63, 64);
+        s_b[buf][l] = x;
+        s_eb[buf][l] = expf(x);
+        s_ed[buf][l] = expf(xl - x);
+        if (l == 0) s_dec[buf] = expf(xl);
+      }
+    };
+#pragma unroll
+    for (int j = 0; j < 3; ++j) issue(pre[j], j);
+    stage(pre[0], 0);
+    issue(pre[0], 3);
+    stage(pre[1], 1);
+    {
+      // blocks of P above the diagonal: zero, and never written again
+      const int t = threadIdx.x & (NTHR - 1), r = t >> 4, cc = t & 15;
+#pragma unroll
+      for (int I = 0; I < 3; ++I)
+#pragma unroll
+        for (int J = I + 1; J < 4; ++J) {
+          s_P[0][(16 * I + r) * LDC + 16 * J + cc] = (T)0.f;
+          s_P[1][(16 * I + r) * LDC + 16 * J + cc] = (T)0.f;
+        }
+    }
+    lds_barrier();                                                                       // chunks 0, 1 staged
+    for (int c0 = 0; c0 < sq.nchunks; c0 += 3) {
+#pragma unroll
+      for (int j = 0; j < 3; ++j) {
+        const int c = c0 + j;
+        if (c >= sq.nchunks) break;
+        if (wave == 4) TR(1, c, 0);
+        lds_barrier();
+        if (wave == 4) TR(1, c, 1);
+        // (both always: past the end it is the last chunk again, never consumed)
+        issue(pre[(j + 1) % 3], c + 4);
+        if (wave == 4) TR(1, c, 5);
+        stage(pre[(j + 2) % 3], (j + 2) % 3);
+        if (wave == 4) TR(1, c, 2);
+        // hs[chunk][h][v0 .. v0+BV][K] <- S^T (only the backward reads it: SAVE = false for forward-only calls)
+        if constexpr (SAVE)
+          IOHT::lds_to_global(s_hT[c & 1], LDK, (T*)a.hs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
+        if (wave == 4) TR(1, c, 4);
+      }
+    }
+    if (wave == 4) trace_out(1);
+    return;
+  }
+
+  if (team == 2) {
+    // --------------------------------- output --------------------------------------------
+    const int ow = wave - 8;
+    const int fr = l & 15, fg = 8 * (l >> 4), g4 = 4 * (l >> 4);
+    lds_barrier();                                                                       // chunks 0, 1 staged
+    p_blocks(0, ow, ow, ow, 1);
+    for (int c = 0; c < sq.nchunks; ++c) {
+      const int cur = c % 3;
+      const int tok = sq.tok0 + c * CH;
+      const int len = min(CH, sq.len - c * CH);
+      if (ow == 0) TR(2, c, 0);
+      lds_barrier();
+      if (ow == 0) TR(2, c, 1);
+      // Both products are formed transposed (the MFMA operands swapped), so that a lane holds four consecutive
+      // columns of ONE token and the result leaves as 8-byte stores.  Every fragment is requested before the first
+      // product (left to the compiler, each read is waited for where it is used and the window is a chain of LDS
+      // round trips).
+      typename ET<T>::frag fq[KS], fh[KS][NB], fp[CS], fv[CS][NB];
+      const T *Pc = s_P[c & 1], *hT = s_hT[c & 1];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        fq[ks] = ET<T>::load_frag(s_q[cur] + (16 * ow + fr) * LDK + 32 * ks + fg);
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) fh[ks][ni] = ET<T>::load_frag(hT + (16 * ni + fr) * LDK + 32 * ks + fg);
+      }
+#pragma unroll
+      for (int kq = 0; kq < CS; ++kq) {
+        if (2 * kq <= ow) {          // tokens j >= 32 only reach the rows of waves 2, 3
+          fp[kq] = ET<T>::load_frag(Pc + (16 * ow + fr) * LDC + 32 * kq + fg);
+#pragma unroll
+          for (int ni = 0; ni < NB; ++ni) fv[kq][ni] = ET<T>::load_frag_t(s_u[cur], LDU, 32 * kq, 16 * ni, l);
+        }
+      }
+      const float ebi = s_eb[cur][16 * ow + fr];
+      __builtin_amdgcn_sched_barrier(0);
+      f32x4 ot[NB], pv[NB];
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) ot[ni] = pv[ni] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) ET<T>::mma(ot[ni], fh[ks][ni], fq[ks]);          // (q S)^T: column x token
+      if (ow == 0) TR(2, c, 5);
+#pragma unroll
+      for (int kq = 0; kq < CS; ++kq) {
+        if (2 * kq <= ow) {
+#pragma unroll
+          for (int ni = 0; ni < NB; ++ni) ET<T>::mma(pv[ni], fv[kq][ni], fp[kq]);         // (P v)^T
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (ow == 0) TR(2, c, 2);
+      // lane: token 16 ow + fr, columns 16 ni + g4 .. + 3
+      T* orow = row_ptr<T>(a.o, sq.b, tok + 16 * ow + fr, h) + v0 + g4;
+      if (16 * ow + fr < len) {
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) {
+          const f32x4 x = (ot[ni] * ebi + pv[ni]) * a.scale;
+          bf16x4 y;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) y[e] = (bf16)x[e];
+          *(bf16x4*)(orow + 16 * ni) = y;
+        }
+      }
+      if (ow == 0) TR(2, c, 4);
+      if (c + 1 < sq.nchunks) p_blocks(c + 1, ow, ow, ow, 1);
+      if (ow == 0) TR(2, c, 6);
+    }
+    if (ow == 0) trace_out(2);
+    return;
+  }
+
+  // --------------------------------- consumers -------------------------------------------
+  const int wv = wave;
+  const int krow0 = wv * (K / 4);
+  f32x4 S[MB][NB];
+  acc_zero(S);
+  if (a.h0) {
+    const float* h0 = a.h0 + ((int64_t)n * a.H + h) * K * V;
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          S[mi][ni][i] = h0[(int64_t)(krow0 + acc_row(mi, i)) * V + v0 + acc_col(ni)];
+  }
+  auto copy_state = [&](int buf) {          // S -> LDS as S^T
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) acc_to_lds_t<T>(S[mi][ni], s_hT[buf], LDK, krow0 + 16 * mi, 16 * ni);
+  };
+  const int pti = wv == 0 ? 3 : wv == 1 ? 2 : wv == 2 ? 3 : 1, ptja = wv == 2 ? 2 : 0, pn = wv < 2 ? 2 : 1;
+  copy_state(0);
+  lds_barrier();                                                                         // chunks 0, 1 staged
+  p_blocks(0, pti, ptja, 1, pn);
+  for (int c = 0; c < sq.nchunks; ++c) {
+    const int cur = c % 3;
+    if (wv == 0) TR(0, c, 0);
+    lds_barrier();
+    if (wv == 0) TR(0, c, 1);
+    const float dec = s_dec[cur];
+    // S = e^{b_C} S + k^T (e_d v'): the row scaling e_d is applied to the v' fragments in registers
+    {
+      typename ET<T>::frag af[CS][MB], bf[CS][NB];
+#pragma unroll
+      for (int kq = 0; kq < CS; ++kq) {
+#pragma unroll
+        for (int mi = 0; mi < MB; ++mi) af[kq][mi] = ET<T>::load_frag_t(s_k[cur], LDK, 32 * kq, krow0 + 16 * mi);
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) bf[kq][ni] = ET<T>::load_frag_t(s_u[cur], LDU, 32 * kq, 16 * ni);
+      }
+#pragma unroll
+      for (int kq = 0; kq < CS; ++kq)
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) scale_frag<T>(bf[kq][ni], &s_ed[cur][32 * kq + 8 * (l >> 4)]);
+#pragma unroll
+      for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) S[mi][ni] *= dec;
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int kq = 0; kq < CS; ++kq)
+#pragma unroll
+        for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+          for (int ni = 0; ni < NB; ++ni) ET<T>::mma(S[mi][ni], af[kq][mi], bf[kq][ni]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (wv == 0) TR(0, c, 5);
+    if (c + 1 < sq.nchunks) {
+      copy_state((c + 1) & 1);
+      if (wv == 0) TR(0, c, 6);
+      p_blocks(c + 1, pti, ptja, 1, pn);
+    }
+    if (wv == 0) TR(0, c, 2);
+  }
+  if (wv == 0) trace_out(0);
   if (a.ht) {
     float* ht = a.ht + ((int64_t)n * a.H + h) * K * V;
 #pragma unroll
