@@ -38,17 +38,17 @@ STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_gdn_state_fwd_reg", 4: "k_gdn_state_bwd"
 # sources (kernel_sources_sha16()) at that time, and a build whose sources differ reports traffic = null
 # rather than a stale number.
 CALIB_COPY_BYTES = 256 << 20
-MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237244044, "k_gdn_state_fwd_reg": 1117018555, "k_gdn_state_bwd": 945962556,
-                    "k_gdn_bwd_chunk": 1899370989}
-TRAFFIC_SOURCES_SHA16 = "508fc52e88a73456"
+MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237242191, "k_gdn_state_fwd_reg": 1117396758, "k_gdn_state_bwd": 945964919,
+                    "k_gdn_bwd_chunk": 1898543552}
+TRAFFIC_SOURCES_SHA16 = "b16ebe487baf9d02"
 TRAFFIC_SOURCES = ("lmoe_common.hpp", "lmoe_seq.hpp", "lmoe_gdn_wy.hpp", "lmoe_gdn_state.hpp", "lmoe_gdn_state_reg.hpp", "lmoe_gdn_bwd_chunk.hpp",
                    "lmoe_gdn_fwd.hip", "lmoe_gdn_state.hip", "lmoe_gdn_bwd.hip")
 
 
 # HBM bytes per call of the other contract configurations (bench.py --other-configs), same counters and scaling,
 # summed over the kernels of the call; key = configuration number
-OTHER_TRAFFIC = {"1": 2228727, "2": 272917723, "3": 1548112021, "5": 16909265279}
-OTHER_TRAFFIC_SHA16 = "7a5d17dfbe6920cd"
+OTHER_TRAFFIC = {"1": 2227714, "2": 272922994, "3": 1548124726, "5": 16902934168}
+OTHER_TRAFFIC_SHA16 = "c194ab1a37a49579"
 
 
 def all_sources_sha16():

@@ -56,7 +56,9 @@ __device__ __forceinline__ int fresh_index(int x) {
 }
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
-__device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
+// (uniform over the wave by construction; said to the compiler, so that what derives from it lives in scalar
+// registers and the branches on it are scalar branches)
+__device__ __forceinline__ int wave_id() { return __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); }
 
 // ------------------------------------------------------------------------- //
 // element traits

@@ -593,7 +593,9 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dv(const lmoe_args a) {
 // ------------------------------------------------------------------------- //
 template <typename T, typename GT, int K, int V, int BVH>
 __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
-  constexpr int LDV = BVH + LPAD, LDB = K + 1, LDP = CH + 1;
+  // (LDB: rows of the fp32 gate tile start on 16-byte boundaries, and the rows 4 apart that the lanes of an accumulator
+  // column read fall into different banks)
+  constexpr int LDV = BVH + LPAD, LDB = K + 4, LDP = CH + 1;
   constexpr int NBK = K / 16;
   // phase A (element type T): do, v, S, dS' slices.  phase B (fp32): dA, q, k, b tiles
   constexpr int A_DO = 0, A_V = A_DO + CH * LDV, A_H = A_V + CH * LDV, A_DH = A_H + K * LDV, A_END = A_DH + K * LDV;
@@ -644,16 +646,19 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
     IOH::load_nomask(x.rdh, (const T*)a.dhs + ((int64_t)cid * a.H + h) * K * V + vv, V, K);
   };
   issue_slice(sl[0], 0);
+  auto issue_qkg = [&]() {
+    IOK::load_nomask(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
+    IOK::load_nomask(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
+    GlaGate<GT, K>::issue(rg, a, ci.b, ci.tok, ci.len, h);
+  };
+  // with two slices everything is requested at the start (a load of this kernel takes 5 to 9 thousand cycles to
+  // arrive, the work on a slice 1500); with more, q, k, g go out with the last slice
+  constexpr bool QKG_EARLY = NSL <= 2;
 #pragma unroll
   for (int si = 0; si < NSL; ++si) {
     Slice& x = sl[si & 1];
-    if (si + 1 < NSL) {
-      issue_slice(sl[(si + 1) & 1], (si + 1) * BVH);
-    } else {
-      IOK::load_nomask(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
-      IOK::load_nomask(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
-      GlaGate<GT, K>::issue(rg, a, ci.b, ci.tok, ci.len, h);
-    }
+    if (si + 1 < NSL) issue_slice(sl[(si + 1) & 1], (si + 1) * BVH);
+    if (QKG_EARLY ? si == 0 : si + 1 == NSL) issue_qkg();
     IOV::mask(x.rd, ci.len);
     IOV::mask(x.rv, ci.len);
 #pragma unroll
@@ -745,31 +750,55 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
       constexpr int SEGROW[4] = {0, 32, 96, 160};                       // k~(wa) 32 | k~(wb) 64 | q~(wa) 64 | q~(wb) 32
       constexpr int VEC = ET<T>::VEC;
       typedef typename ET<T>::vec vec;
-      for (int idx = threadIdx.x; idx < 192 * (K / VEC); idx += NTHR) {
-        const int sr = idx / (K / VEC), c0 = (idx % (K / VEC)) * VEC;   // one 16-byte piece of one stacked row
-        const int sg = sr < 32 ? 0 : sr < 96 ? 1 : sr < 160 ? 2 : 3;
+      // A thread keeps its 16-byte column group c0 and takes one stacked row out of every RPI: the segment of a row
+      // is then known at compile time, the gate row that a whole segment shares (its reference) is read once, and
+      // every gate value arrives in 16-byte reads
+      constexpr int PPR = K / VEC, RPI = NTHR / PPR, NIT = 192 / RPI;
+      static_assert(32 % RPI == 0 && NTHR % PPR == 0, "segment boundaries fall between the passes");
+      const int c0 = (threadIdx.x % PPR) * VEC, rin = threadIdx.x / PPR;
+      auto gate_row = [&](int row, float (&b)[VEC]) {
+#pragma unroll
+        for (int e4 = 0; e4 < VEC; e4 += 4) {
+          const f32x4 t = *(const f32x4*)(sB + row * LDB + c0 + e4);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) b[e4 + e] = t[e];
+        }
+      };
+      float ref[4][VEC];                                                // k~: b_{16 w - 1} (0 for w = 0); q~: b_{16 w + 15}
+#pragma unroll
+      for (int sg = 0; sg < 4; ++sg) {
+        const int w = (sg & 1) ? wb : wa;
+        if (sg < 2 && w == 0) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) ref[sg][e] = 0.f;
+        } else {
+          gate_row(sg < 2 ? 16 * w - 1 : 16 * w + 15, ref[sg]);
+        }
+      }
+#pragma unroll
+      for (int it = 0; it < NIT; ++it) {
+        const int sr0 = it * RPI, sg = sr0 < 32 ? 0 : sr0 < 96 ? 1 : sr0 < 160 ? 2 : 3;   // known after unrolling
+        const int sr = sr0 + rin;
         const int w = (sg & 1) ? wb : wa;
         const bool own_ok = !((unsafe >> w) & 1);
-        // token of this row, whether the row is in use, and the two gate rows whose difference is the exponent
-        int tok, hi_row, lo_row;                                        // exponent = b[hi_row] - b[lo_row] (hi_row < 0: 0)
+        // token of this row and whether the row is in use
+        int tok;
         bool use;
         if (sg < 2) {
           tok = sr - SEGROW[sg];
-          use = tok < 16 * w + 16 && (tok < 16 * w || own_ok);
-          hi_row = 16 * w - 1, lo_row = tok;                            // k_j e^{ref_w - b_j}
+          use = tok < 16 * w + 16 && (tok < 16 * w || own_ok);          // k_j e^{ref_w - b_j}
         } else {
           tok = (w < 2 ? 0 : 32) + sr - SEGROW[sg];
-          use = tok >= 16 * w && (tok >= 16 * w + 16 || own_ok);
-          hi_row = tok, lo_row = 16 * w + 15;                           // q_i e^{b_i - ref'_w}
+          use = tok >= 16 * w && (tok >= 16 * w + 16 || own_ok);        // q_i e^{b_i - ref'_w}
         }
         vec o = ET<T>::zero();
         if (use) {
           const vec x = *(const vec*)((sg < 2 ? tK : tQ) + tok * LDK + c0);
+          float bt[VEC];
+          gate_row(tok, bt);
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) {
-            const float hi = hi_row < 0 ? 0.f : sB[hi_row * LDB + c0 + e];
-            o[e] = ET<T>::from_f(ET<T>::to_f(x[e]) * texp<T>(hi - sB[lo_row * LDB + c0 + e]));
-          }
+          for (int e = 0; e < VEC; ++e)
+            o[e] = ET<T>::from_f(ET<T>::to_f(x[e]) * texp<T>(sg < 2 ? ref[sg][e] - bt[e] : bt[e] - ref[sg][e]));
         }
         *(vec*)(tKT + sr * LDK + c0) = o;
       }
@@ -838,24 +867,30 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
       const int ni = nh + n4;
       const int cc = 16 * ni + (l & 15);
       const float bC = sB[63 * LDB + cc];
+      // Two exponentials per element, e^{b_r - ref_w} and e^{ref'_w - b_r} (both exponents <= 0); the other two
+      // factors of a row follow from them through one factor per column: e^{b_r} = e^{ref_w} e^{b_r - ref_w},
+      // e^{b_C - b_r} = e^{b_C - ref'_w} e^{ref'_w - b_r}
+      const float refq = wv == 0 ? 0.f : sB[(16 * wv - 1) * LDB + cc], refk = sB[(16 * wv + 15) * LDB + cc];
+      const float eref = texp<T>(refq), eC = texp<T>(bC - refk);
       kkp[ni] = 0.f;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int r = 16 * wv + 4 * (l >> 4) + i;
         const float br = sB[r * LDB + cc];
+        const float e1 = texp<T>(br - refq), e2 = texp<T>(refk - br);
         float sq_ = 0.f, sk_ = 0.f;
         if constexpr (SUB) {
           sq_ = sqv[n4][i];
           sk_ = skv[n4][i];
-          sq_ += dqo[0][ni][i] * texp<T>(br - (wv == 0 ? 0.f : sB[(16 * wv - 1) * LDB + cc]));
-          sk_ += dko[0][ni][i] * texp<T>(sB[(16 * wv + 15) * LDB + cc] - br);
+          sq_ += dqo[0][ni][i] * e1;
+          sk_ += dko[0][ni][i] * e2;
         } else {
           for (int j = jlo; j <= r; ++j) sq_ += Pm(r, j) * Km(j, cc) * texp<T>(br - sB[j * LDB + cc]);
           for (int ii = r; ii < ihi; ++ii) sk_ += Pm(ii, r) * Qm(ii, cc) * texp<T>(sB[ii * LDB + cc] - br);
         }
         const float qv = Qm(r, cc), kv = Km(r, cc);
-        const float ed = texp<T>(bC - br);
-        const float dqv = a.scale * texp<T>(br) * dqi[0][ni][i] + sq_;
+        const float ed = eC * e2;
+        const float dqv = a.scale * (eref * e1) * dqi[0][ni][i] + sq_;
         const float dkdv = dkd[0][ni][i] * ed;
         const float dkv = dkdv + sk_;
         kkp[ni] += kv * dkdv;
