@@ -38,8 +38,8 @@ STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_gdn_state_fwd_reg", 4: "k_gdn_state_bwd"
 # sources (kernel_sources_sha16()) at that time, and a build whose sources differ reports traffic = null
 # rather than a stale number.
 CALIB_COPY_BYTES = 256 << 20
-MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237242191, "k_gdn_state_fwd_reg": 1117396758, "k_gdn_state_bwd": 945964919,
-                    "k_gdn_bwd_chunk": 1898543552}
+MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237241818, "k_gdn_state_fwd_reg": 1118587559, "k_gdn_state_bwd": 945963116,
+                    "k_gdn_bwd_chunk": 1892917955}
 TRAFFIC_SOURCES_SHA16 = "b16ebe487baf9d02"
 TRAFFIC_SOURCES = ("lmoe_common.hpp", "lmoe_seq.hpp", "lmoe_gdn_wy.hpp", "lmoe_gdn_state.hpp", "lmoe_gdn_state_reg.hpp", "lmoe_gdn_bwd_chunk.hpp",
                    "lmoe_gdn_fwd.hip", "lmoe_gdn_state.hip", "lmoe_gdn_bwd.hip")
@@ -47,8 +47,8 @@ TRAFFIC_SOURCES = ("lmoe_common.hpp", "lmoe_seq.hpp", "lmoe_gdn_wy.hpp", "lmoe_g
 
 # HBM bytes per call of the other contract configurations (bench.py --other-configs), same counters and scaling,
 # summed over the kernels of the call; key = configuration number
-OTHER_TRAFFIC = {"1": 2227714, "2": 272922994, "3": 1548124726, "5": 16902934168}
-OTHER_TRAFFIC_SHA16 = "c194ab1a37a49579"
+OTHER_TRAFFIC = {"1": 2231802, "2": 272911910, "3": 1547963516, "5": 16920815387}
+OTHER_TRAFFIC_SHA16 = "da7c467f33b038a2"
 
 
 def all_sources_sha16():
@@ -346,10 +346,11 @@ def trace_simple_gla_fwd(lib, dev, work_group=16):
     c0, c1 = nch // 4, nch - nch // 4
     ref = t[0, c0:c1, 1]
     period = float((t[0, c0 + 1:c1 + 1, 1] - t[0, c0:c1, 1]).mean())
-    names = {0: {0: "arrives_barrier", 1: "leaves_barrier", 5: "state_updated", 6: "state_copied", 2: "next_P_below_diagonal_formed"},
+    names = {0: {0: "arrives_barrier", 1: "leaves_barrier", 5: "state_updated", 6: "state_copied", 2: "next_P_below_diagonal_formed",
+                 3: "next_operands_read"},
              1: {0: "arrives_barrier", 1: "leaves_barrier", 5: "loads_issued", 2: "staged", 4: "hs_stored"},
              2: {0: "arrives_barrier", 1: "leaves_barrier", 5: "qS_issued", 2: "Pv_done", 4: "rows_stored",
-                 6: "next_P_diagonal_formed"}}
+                 6: "next_P_diagonal_formed_next_operands_read"}}
     teams = {0: "consumer_wave", 1: "loader_wave", 2: "output_wave"}
     out = {}
     for s_, nm in teams.items():

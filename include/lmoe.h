@@ -283,9 +283,11 @@ int lmoe_trace_gdn_state_fwd(const lmoe_args* a, int64_t* trace, int32_t work_gr
 /* The same for the forward pass of chunk_simple_gla on 2-byte elements (k_state_fwd_b, one barrier per chunk):
  * trace = 3 x 24 x 8 int64 device words, trace[slot][chunk][mark] (chunks beyond 24 are not recorded), stamps of one
  * wave per team of work-group `work_group`.  Marks: 0 arrives at the barrier of the chunk, 1 leaves it, and
- *   slot 0, consumers: 5 state updated, 6 state copied to LDS, 2 their blocks of P of the next chunk formed
+ *   slot 0, consumers: 5 state updated, 6 state copied to LDS, 2 their blocks of P of the next chunk formed, 3 the
+ *     operands of the next state update read
  *   slot 1, loaders: 5 loads of chunk c + 4 issued, 2 chunk c + 2 staged, 4 per-chunk state stored (saving calls)
  *   slot 2, output team: 5 products of q S issued, 2 (P v)^T done, 4 rows stored, 6 its block of P of the next chunk
+ *     formed and the next chunk's q rows and v^T fragments read
  * Instance available for LMOE_BF16, K = V = 128, forward-only calls (hs NULL; -24 otherwise).  No counterpart in
  * the reference (profiling support). */
 int lmoe_trace_simple_gla_fwd(const lmoe_args* a, int64_t* trace, int32_t work_group, void* stream);

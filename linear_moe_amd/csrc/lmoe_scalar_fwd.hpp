@@ -331,8 +331,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd_b(const lmoe_args a, lon
 
   // Blocks (ti, tj[0 .. n)) of P of chunk c (16 x 16 each, one q strip against n <= 2 k strips), formed transposed so
   // that a lane holds four consecutive columns of one row (8-byte writes).  The ten blocks on and below the diagonal
-  // are dealt to eight waves: the output team takes the diagonal (wave w: block (w, w)) once its rows are stored,
-  // the consumers the six blocks below it (waves 0, 1: rows 3, 2 against k strips 0, 1; wave 2: (3, 2); wave 3: (1, 0)).
+  // are dealt to eight waves: the output team takes the diagonal (wave w: block (w, w), p_diag) once its rows are
+  // stored, the consumers the six blocks below it (waves 0, 1: rows 3, 2 against k strips 0, 1; wave 2: (3, 2); wave 3: (1, 0)).
   // Every fragment is requested before the first product: the LDS is busiest right behind the barrier, a read comes
   // back after several hundred cycles, and a product loop that requests one step ahead pays that once per step.
   auto p_blocks = [&](int c, int ti, int tja, int tjb, int n) {
@@ -457,9 +457,48 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd_b(const lmoe_args a, lon
     const int ow = wave - 8;
     const int fr = l & 15, fg = 8 * (l >> 4), g4 = 4 * (l >> 4);
     lds_barrier();                                                                       // chunks 0, 1 staged
-    p_blocks(0, ow, ow, ow, 1);
+    // What the window of a chunk reads of its own operand buffer - the q rows, the v^T fragments, the gate factor -
+    // was staged two windows earlier: it is read at the end of the window before, when the LDS is quiet, and not in
+    // the rush behind the barrier, where only S^T and P (written in the window before) are left to read.
+    typename ET<T>::frag fq[KS], fv[CS][NB];
+    float ebi;
+    auto preread = [&](int c) {
+      const int cb = c % 3;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) fq[ks] = ET<T>::load_frag(s_q[cb] + (16 * ow + fr) * LDK + 32 * ks + fg);
+#pragma unroll
+      for (int kq = 0; kq < CS; ++kq) {
+        if (2 * kq <= ow) {          // tokens j >= 32 only reach the rows of waves 2, 3
+#pragma unroll
+          for (int ni = 0; ni < NB; ++ni) fv[kq][ni] = ET<T>::load_frag_t(s_u[cb], LDU, 32 * kq, 16 * ni, l);
+        }
+      }
+      ebi = s_eb[cb][16 * ow + fr];
+    };
+    // the diagonal block (ow, ow) of P of chunk c from the q rows that preread(c) has just fetched
+    auto p_diag = [&](int c) {
+      const int cb = c % 3, g = l >> 4;
+      typename ET<T>::frag fk[KS];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) fk[ks] = ET<T>::load_frag(s_k[cb] + (16 * ow + fr) * LDK + 32 * ks + fg);
+      const int i = 16 * ow + fr;
+      const float bi = s_b[cb][i];
+      const f32x4 bj = *(const f32x4*)&s_b[cb][16 * ow + 4 * g];
+      f32x4 gm, pa = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) gm[e] = (fr >= 4 * g + e) ? texp<T>(bi - bj[e]) : 0.f;
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) ET<T>::mma(pa, fk[ks], fq[ks]);
+      __builtin_amdgcn_sched_barrier(0);
+      bf16x4 y;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) y[e] = (bf16)(pa[e] * gm[e]);
+      *(bf16x4*)(s_P[c & 1] + i * LDC + 16 * ow + 4 * g) = y;
+    };
+    preread(0);
+    p_diag(0);
     for (int c = 0; c < sq.nchunks; ++c) {
-      const int cur = c % 3;
       const int tok = sq.tok0 + c * CH;
       const int len = min(CH, sq.len - c * CH);
       if (ow == 0) TR(2, c, 0);
@@ -469,23 +508,15 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd_b(const lmoe_args a, lon
       // columns of ONE token and the result leaves as 8-byte stores.  Every fragment is requested before the first
       // product (left to the compiler, each read is waited for where it is used and the window is a chain of LDS
       // round trips).
-      typename ET<T>::frag fq[KS], fh[KS][NB], fp[CS], fv[CS][NB];
+      typename ET<T>::frag fh[KS][NB], fp[CS];
       const T *Pc = s_P[c & 1], *hT = s_hT[c & 1];
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        fq[ks] = ET<T>::load_frag(s_q[cur] + (16 * ow + fr) * LDK + 32 * ks + fg);
+      for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
         for (int ni = 0; ni < NB; ++ni) fh[ks][ni] = ET<T>::load_frag(hT + (16 * ni + fr) * LDK + 32 * ks + fg);
-      }
 #pragma unroll
-      for (int kq = 0; kq < CS; ++kq) {
-        if (2 * kq <= ow) {          // tokens j >= 32 only reach the rows of waves 2, 3
-          fp[kq] = ET<T>::load_frag(Pc + (16 * ow + fr) * LDC + 32 * kq + fg);
-#pragma unroll
-          for (int ni = 0; ni < NB; ++ni) fv[kq][ni] = ET<T>::load_frag_t(s_u[cur], LDU, 32 * kq, 16 * ni, l);
-        }
-      }
-      const float ebi = s_eb[cur][16 * ow + fr];
+      for (int kq = 0; kq < CS; ++kq)
+        if (2 * kq <= ow) fp[kq] = ET<T>::load_frag(Pc + (16 * ow + fr) * LDC + 32 * kq + fg);
       __builtin_amdgcn_sched_barrier(0);
       f32x4 ot[NB], pv[NB];
 #pragma unroll
@@ -517,7 +548,10 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd_b(const lmoe_args a, lon
         }
       }
       if (ow == 0) TR(2, c, 4);
-      if (c + 1 < sq.nchunks) p_blocks(c + 1, ow, ow, ow, 1);
+      if (c + 1 < sq.nchunks) {
+        preread(c + 1);
+        p_diag(c + 1);
+      }
       if (ow == 0) TR(2, c, 6);
     }
     if (ow == 0) trace_out(2);
@@ -549,46 +583,52 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd_b(const lmoe_args a, lon
   copy_state(0);
   lds_barrier();                                                                         // chunks 0, 1 staged
   p_blocks(0, pti, ptja, 1, pn);
+  // The operands of the state update of a chunk were staged two windows earlier: they are read (and the row scaling
+  // e_d applied to the v' fragments) at the end of the window before, when the LDS is quiet; behind the barrier the
+  // update is eight products on registers.
+  typename ET<T>::frag af[CS][MB], bf[CS][NB];
+  float dec;
+  auto preread = [&](int c) {
+    const int cb = c % 3;
+#pragma unroll
+    for (int kq = 0; kq < CS; ++kq) {
+#pragma unroll
+      for (int mi = 0; mi < MB; ++mi) af[kq][mi] = ET<T>::load_frag_t(s_k[cb], LDK, 32 * kq, krow0 + 16 * mi);
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) bf[kq][ni] = ET<T>::load_frag_t(s_u[cb], LDU, 32 * kq, 16 * ni);
+    }
+    dec = s_dec[cb];
+#pragma unroll
+    for (int kq = 0; kq < CS; ++kq)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) scale_frag<T>(bf[kq][ni], &s_ed[cb][32 * kq + 8 * (l >> 4)]);
+  };
+  preread(0);
   for (int c = 0; c < sq.nchunks; ++c) {
-    const int cur = c % 3;
     if (wv == 0) TR(0, c, 0);
     lds_barrier();
     if (wv == 0) TR(0, c, 1);
-    const float dec = s_dec[cur];
-    // S = e^{b_C} S + k^T (e_d v'): the row scaling e_d is applied to the v' fragments in registers
-    {
-      typename ET<T>::frag af[CS][MB], bf[CS][NB];
+    // S = e^{b_C} S + k^T (e_d v')
 #pragma unroll
-      for (int kq = 0; kq < CS; ++kq) {
+    for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
-        for (int mi = 0; mi < MB; ++mi) af[kq][mi] = ET<T>::load_frag_t(s_k[cur], LDK, 32 * kq, krow0 + 16 * mi);
+      for (int ni = 0; ni < NB; ++ni) S[mi][ni] *= dec;
 #pragma unroll
-        for (int ni = 0; ni < NB; ++ni) bf[kq][ni] = ET<T>::load_frag_t(s_u[cur], LDU, 32 * kq, 16 * ni);
-      }
-#pragma unroll
-      for (int kq = 0; kq < CS; ++kq)
-#pragma unroll
-        for (int ni = 0; ni < NB; ++ni) scale_frag<T>(bf[kq][ni], &s_ed[cur][32 * kq + 8 * (l >> 4)]);
+    for (int kq = 0; kq < CS; ++kq)
 #pragma unroll
       for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < NB; ++ni) S[mi][ni] *= dec;
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int kq = 0; kq < CS; ++kq)
-#pragma unroll
-        for (int mi = 0; mi < MB; ++mi)
-#pragma unroll
-          for (int ni = 0; ni < NB; ++ni) ET<T>::mma(S[mi][ni], af[kq][mi], bf[kq][ni]);
-      __builtin_amdgcn_sched_barrier(0);
-    }
+        for (int ni = 0; ni < NB; ++ni) ET<T>::mma(S[mi][ni], af[kq][mi], bf[kq][ni]);
+    __builtin_amdgcn_sched_barrier(0);
     if (wv == 0) TR(0, c, 5);
     if (c + 1 < sq.nchunks) {
       copy_state((c + 1) & 1);
       if (wv == 0) TR(0, c, 6);
       p_blocks(c + 1, pti, ptja, 1, pn);
+      if (wv == 0) TR(0, c, 2);
+      preread(c + 1);
     }
-    if (wv == 0) TR(0, c, 2);
+    if (wv == 0) TR(0, c, 3);
   }
   if (wv == 0) trace_out(0);
   if (a.ht) {
