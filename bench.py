@@ -38,8 +38,8 @@ STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_gdn_state_fwd_reg", 4: "k_gdn_state_bwd"
 # sources (kernel_sources_sha16()) at that time, and a build whose sources differ reports traffic = null
 # rather than a stale number.
 CALIB_COPY_BYTES = 256 << 20
-MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237241818, "k_gdn_state_fwd_reg": 1118587559, "k_gdn_state_bwd": 945963116,
-                    "k_gdn_bwd_chunk": 1892917955}
+MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237243234, "k_gdn_state_fwd_reg": 1118149997, "k_gdn_state_bwd": 945961393,
+                    "k_gdn_bwd_chunk": 1899325051}
 TRAFFIC_SOURCES_SHA16 = "b16ebe487baf9d02"
 TRAFFIC_SOURCES = ("lmoe_common.hpp", "lmoe_seq.hpp", "lmoe_gdn_wy.hpp", "lmoe_gdn_state.hpp", "lmoe_gdn_state_reg.hpp", "lmoe_gdn_bwd_chunk.hpp",
                    "lmoe_gdn_fwd.hip", "lmoe_gdn_state.hip", "lmoe_gdn_bwd.hip")
@@ -47,8 +47,8 @@ TRAFFIC_SOURCES = ("lmoe_common.hpp", "lmoe_seq.hpp", "lmoe_gdn_wy.hpp", "lmoe_g
 
 # HBM bytes per call of the other contract configurations (bench.py --other-configs), same counters and scaling,
 # summed over the kernels of the call; key = configuration number
-OTHER_TRAFFIC = {"1": 2231802, "2": 272911910, "3": 1547963516, "5": 16920815387}
-OTHER_TRAFFIC_SHA16 = "da7c467f33b038a2"
+OTHER_TRAFFIC = {"1": 2231806, "2": 272912295, "3": 1548446998, "5": 16910958251}
+OTHER_TRAFFIC_SHA16 = "8e33b58c4c3110db"
 
 
 def all_sources_sha16():

@@ -29,6 +29,18 @@ constexpr float GLA_SAFE_EXP = 60.0f;
 // first row of the k~ copy of block row I inside the stacked tile: 0, 16, 48, 96
 constexpr int KT_ROW0(int I) { return 8 * I * (I + 1); }
 
+// N consecutive fp32 values of an LDS tile whose rows start on 16-byte boundaries, as 16-byte reads (left to the
+// compiler, a column group of the gate tile arrives as N scalar reads)
+template <int N> __device__ __forceinline__ void load_f32_group(const float* p, float (&b)[N]) {
+  static_assert(N % 4 == 0, "whole 16-byte pieces");
+#pragma unroll
+  for (int e4 = 0; e4 < N; e4 += 4) {
+    const f32x4 t = *(const f32x4*)(p + e4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) b[e4 + e] = t[e];
+  }
+}
+
 // g tile of the chunk -> fp32 LDS tile s_b[64][LDB] holding the inclusive cumsum over tokens.
 // The scan: a thread takes one channel over a segment of 64 K / 256 tokens (its values in registers, so the
 // LDS reads are independent of each other), the segment totals go through a small LDS array, and every thread
@@ -128,7 +140,11 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
   }
   typename GG::Regs rg = pre.rg;
   issue(it + gridDim.x);
-  for (int idx = threadIdx.x; idx < CH * LDC; idx += NTHR) s_A[idx] = ET<T>::from_f(0.f);   // blocks above the diagonal
+  {                                                                                        // blocks above the diagonal
+    constexpr int VEC = ET<T>::VEC;
+    static_assert((CH * LDC) % VEC == 0, "whole 16-byte pieces");
+    for (int idx = threadIdx.x; idx < CH * LDC / VEC; idx += NTHR) *(typename ET<T>::vec*)(s_A + idx * VEC) = ET<T>::zero();
+  }
   GG::template finish<LDB>(rg, ci.len, s_b, (float*)s_qt, TEXP_PRESCALE<T>);    // barriers inside; b in exp2 units
   // ---- gated operands for the other kernels: q e^{b}, k e^{b_C - b}, e^{b_C} ----
   {
@@ -136,15 +152,20 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
     typedef typename ET<T>::vec vec;
     T* qe = (T*)a.qe + ((int64_t)cid * a.H + h) * CH * K;
     T* ke = (T*)a.ke + ((int64_t)cid * a.H + h) * CH * K;
-    for (int e = threadIdx.x; e < CH * K / VEC; e += NTHR) {
+    static_assert(CH * K / VEC % NTHR == 0, "whole passes");
+#pragma unroll
+    for (int ps = 0; ps < CH * K / VEC / NTHR; ++ps) {
+      const int e = ps * NTHR + threadIdx.x;
       const int r = e / (K / VEC), c0 = (e % (K / VEC)) * VEC;
       const vec qv = *(const vec*)(s_q + r * LDK + c0), kv = *(const vec*)(s_k + r * LDK + c0);
       vec qo, ko;
+      float b[VEC], bC[VEC];
+      load_f32_group(s_b + r * LDB + c0, b);
+      load_f32_group(s_b + 63 * LDB + c0, bC);
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
-        const float b = s_b[r * LDB + c0 + j], bC = s_b[63 * LDB + c0 + j];
-        qo[j] = ET<T>::from_f(ET<T>::to_f(qv[j]) * texp_scaled<T>(b));
-        ko[j] = ET<T>::from_f(ET<T>::to_f(kv[j]) * texp_scaled<T>(bC - b));
+        qo[j] = ET<T>::from_f(ET<T>::to_f(qv[j]) * texp_scaled<T>(b[j]));
+        ko[j] = ET<T>::from_f(ET<T>::to_f(kv[j]) * texp_scaled<T>(bC[j] - b[j]));
       }
       *(vec*)(qe + r * K + c0) = qo;
       *(vec*)(ke + r * K + c0) = ko;
@@ -202,8 +223,13 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
   {
     constexpr int VEC = ET<T>::VEC;
     typedef typename ET<T>::vec vec;
-    // stacked rows 0 .. 63: q~; 64 .. 223: k~ of block rows 0 .. 3 (16-byte pieces)
-    for (int idx = threadIdx.x; idx < (CH + 160) * (K / VEC); idx += NTHR) {
+    // stacked rows 0 .. 63: q~; 64 .. 223: k~ of block rows 0 .. 3 (16-byte pieces).  Unrolled: a pass is a chain of
+    // LDS reads, exponentials and a write, and seven (fourteen) of them one after the other cost a third of an item
+    constexpr int NPASS = (CH + 160) * (K / VEC) / NTHR;
+    static_assert((CH + 160) * (K / VEC) % NTHR == 0, "whole passes");
+#pragma unroll
+    for (int ps = 0; ps < NPASS; ++ps) {
+      const int idx = ps * NTHR + threadIdx.x;
       const int sr = idx / (K / VEC), c0 = (idx % (K / VEC)) * VEC;
       const bool isq = sr < CH;
       const int kr = sr - CH;                                           // row of the stacked k~ tile
@@ -211,10 +237,13 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
       const int tok = isq ? sr : kr - KT_ROW0(I);
       const vec x = *(const vec*)((isq ? s_q : s_k) + tok * LDK + c0);
       vec o;
+      float ref[VEC], bt[VEC];
+      load_f32_group(s_b + tok * LDB + c0, bt);
+      load_f32_group(s_b + (I == 0 ? 0 : 16 * I - 1) * LDB + c0, ref);      // (row 0 for I = 0: read, not used)
 #pragma unroll
       for (int e = 0; e < VEC; ++e) {
-        const float ref = I == 0 ? 0.f : s_b[(16 * I - 1) * LDB + c0 + e], bt = s_b[tok * LDB + c0 + e];
-        o[e] = ET<T>::from_f(ET<T>::to_f(x[e]) * texp_scaled<T>(isq ? bt - ref : ref - bt));
+        const float d = I == 0 ? bt[e] : bt[e] - ref[e];
+        o[e] = ET<T>::from_f(ET<T>::to_f(x[e]) * texp_scaled<T>(isq ? d : -d));
       }
       *(vec*)((isq ? s_qt + sr * LDK : s_kt + kr * LDK) + c0) = o;
     }
@@ -756,14 +785,7 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
       constexpr int PPR = K / VEC, RPI = NTHR / PPR, NIT = 192 / RPI;
       static_assert(32 % RPI == 0 && NTHR % PPR == 0, "segment boundaries fall between the passes");
       const int c0 = (threadIdx.x % PPR) * VEC, rin = threadIdx.x / PPR;
-      auto gate_row = [&](int row, float (&b)[VEC]) {
-#pragma unroll
-        for (int e4 = 0; e4 < VEC; e4 += 4) {
-          const f32x4 t = *(const f32x4*)(sB + row * LDB + c0 + e4);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) b[e4 + e] = t[e];
-        }
-      };
+      auto gate_row = [&](int row, float (&b)[VEC]) { load_f32_group(sB + row * LDB + c0, b); };
       float ref[4][VEC];                                                // k~: b_{16 w - 1} (0 for w = 0); q~: b_{16 w + 15}
 #pragma unroll
       for (int sg = 0; sg < 4; ++sg) {
