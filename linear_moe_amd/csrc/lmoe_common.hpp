@@ -619,20 +619,32 @@ __device__ __forceinline__ float wave_incl_scan(float x) {
   x += dpp_or_zero<0x143, 0xc>(x);      // row_bcast:31 into rows 2 and 3
   return x;
 }
-// inclusive suffix sum (reverse cumulative sum) across the 64 lanes
-__device__ __forceinline__ float wave_rev_scan(float x) {
-  const int l = lane_id();
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    float y = __shfl_down(x, d, 64);
-    if (l + d < 64) x += y;
-  }
+// sum over aligned groups of N consecutive lanes (N = 2, 4, 8, 16: inside a row of 16 lanes), every lane of a group
+// receives the total: lane exchanges on the vector ALU (pairs, quads, the mirrored half-row, the mirrored row)
+// instead of trips through the LDS crossbar
+template <int N> __device__ __forceinline__ float group_sum(float x) {
+  static_assert(N == 1 || N == 2 || N == 4 || N == 8 || N == 16, "a power of two inside a row of 16 lanes");
+  if constexpr (N >= 2) x += dpp_or_zero<0xB1, 0xf>(x);     // quad_perm [1, 0, 3, 2]
+  if constexpr (N >= 4) x += dpp_or_zero<0x4E, 0xf>(x);     // quad_perm [2, 3, 0, 1]
+  if constexpr (N >= 8) x += dpp_or_zero<0x141, 0xf>(x);    // row_half_mirror
+  if constexpr (N >= 16) x += dpp_or_zero<0x140, 0xf>(x);   // row_mirror
   return x;
 }
+// inclusive suffix sum (reverse cumulative sum) across the 64 lanes: total - (prefix sum before the lane), with the
+// prefix sums from the exchanges on the vector ALU above (six dependent exchanges through the LDS crossbar sat on the
+// path of the one wave every other wave of the work-group waits for).  The difference is exact to an ulp of the
+// largest prefix sum, which is at most twice the largest suffix sum.
+__device__ __forceinline__ float wave_rev_scan(float x) {
+  const float incl = wave_incl_scan(x);
+  const float total = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, incl), 63));
+  return total - (incl - x);
+}
+// sum over the 64 lanes, in every lane: the row totals, then the four of them through scalar registers
 __device__ __forceinline__ float wave_sum(float x) {
-#pragma unroll
-  for (int d = 32; d >= 1; d >>= 1) x += __shfl_xor(x, d, 64);
-  return x;
+  x = group_sum<16>(x);
+  const int xi = __builtin_bit_cast(int, x);
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 0)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 16)) +
+         (__builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 32)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 48)));
 }
 
 }  // namespace lmoe

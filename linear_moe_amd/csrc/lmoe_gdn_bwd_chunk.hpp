@@ -535,11 +535,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-#pragma unroll
-      for (int d = 1; d < 16; d <<= 1) {
-        dbp[i] += __shfl_xor(dbp[i], d, 64);
-        dbt[i] += __shfl_xor(dbt[i], d, 64);
-      }
+      dbp[i] = group_sum<16>(dbp[i]);
+      dbt[i] = group_sum<16>(dbt[i]);
     }
     if (fr == 0) {
 #pragma unroll

@@ -707,9 +707,7 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
   // per state row k: sum_v S_kv dS'_kv  (the IOH::VPR adjacent threads of a pass share a row)
 #pragma unroll
   for (int p = 0; p < IOH::PASSES; ++p) {
-    float x = hdh[p];
-#pragma unroll
-    for (int d = 1; d < IOH::VPR; d <<= 1) x += __shfl_xor(x, d, 64);
+    const float x = group_sum<IOH::VPR>(hdh[p]);
     int row, col; IOH::coords(p, row, col);
     if (col == 0 && row < K) s_hdh[row] = x;
   }

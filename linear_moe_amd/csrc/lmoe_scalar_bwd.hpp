@@ -459,10 +459,7 @@ __global__ __launch_bounds__(2 * NTHR) void k_bwd_dqk(const lmoe_args a) {
       }
     // reduce db over the 16 lanes that share a row group, kk over the whole team
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-#pragma unroll
-      for (int d = 1; d < 16; d <<= 1) dbp[i] += __shfl_xor(dbp[i], d, 64);
-    }
+    for (int i = 0; i < 4; ++i) dbp[i] = group_sum<16>(dbp[i]);
     if ((l & 15) == 0) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) s_db[16 * wv + 4 * (l >> 4) + i] = dbp[i];
