@@ -48,7 +48,7 @@ TRAFFIC_SOURCES = ("lmoe_common.hpp", "lmoe_seq.hpp", "lmoe_gdn_wy.hpp", "lmoe_g
 # HBM bytes per call of the other contract configurations (bench.py --other-configs), same counters and scaling,
 # summed over the kernels of the call; key = configuration number
 OTHER_TRAFFIC = {"1": 2231801, "2": 272911932, "3": 1548409952, "5": 16902360948}
-OTHER_TRAFFIC_SHA16 = "3cee0cbac2315421"
+OTHER_TRAFFIC_SHA16 = "bbf08de5f608707b"
 
 
 def all_sources_sha16():

@@ -253,13 +253,18 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
 // The same pass for 2-byte elements, one barrier per chunk: whatever a window reads was completed in the window
 // before.  Three operand buffers (chunk c is worked on, chunk c + 1 is complete, chunk c + 2 is being staged), two
 // copies of S^T and two of P = (q k^T) . Gamma.  Window c, between barrier c and barrier c + 1:
-//   consumers: S = e^{b_C} S + k^T (e_d v) on buffer c % 3, S -> s_hT[(c + 1) & 1], then the blocks of P of chunk
-//              c + 1 below the diagonal -> s_P[(c + 1) & 1] (the state update alone takes a third of a window; the
-//              output team, which formed its rows of P itself in an earlier version, was the longest chain of it)
+//   consumers: S = e^{b_C} S + k^T (e_d v) on fragments of chunk c read before the barrier, S -> s_hT[(c + 1) & 1],
+//              then the blocks of P of chunk c + 1 below the diagonal -> s_P[(c + 1) & 1] (the output team, which
+//              formed its rows of P itself in an earlier version, was the longest chain of the window), then the
+//              fragments of chunk c + 1 for the next update
 //   loaders:   loads of chunk c + 4 issued into the register set that the last window's staging freed, chunk c + 2
 //              staged into buffer (c + 2) % 3, hs <- s_hT[c & 1] (SAVE)
-//   output:    rows 16 w .. of o = e^b q S (s_hT[c & 1]) + P (s_P[c & 1]) v, stored from registers, then the
-//              diagonal blocks of P of chunk c + 1
+//   output:    rows 16 w .. of o = e^b q S (s_hT[c & 1]) + P (s_P[c & 1]) v on q rows and v fragments read before
+//              the barrier, stored from registers, then the q rows and v fragments of chunk c + 1 and, from those q
+//              rows, the diagonal blocks of P of chunk c + 1
+// A chunk's own operands are staged two windows before its window: what is read of them is read at the end of the
+// window before, when the LDS is quiet.  Behind the barrier, where all twelve waves ask for data at once and a read
+// takes about a thousand cycles to return, only S^T and P (written in the window before) are left to read.
 // Time stamps of the traced instance (TRACE = true): one wave of each team notes the shader clock where it arrives
 // at and leaves the barrier of a chunk and at a few points in between; the stamps sit in LDS (a global store
 // per stamp would perturb the wave that is measured) and each of those waves copies its own out at the end:
