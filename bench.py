@@ -344,8 +344,9 @@ def trace_simple_gla_fwd(lib, dev, work_group=16):
     nall = (T + CH - 1) // CH
     nch = min(chunks, nall)
     c0, c1 = nch // 4, nch - nch // 4
+    wrap = lambda d: ((d + 2.0 ** 31) % 2.0 ** 32) - 2.0 ** 31     # the stamps are the low 32 bits of the clock
     ref = t[0, c0:c1, 1]
-    period = float((t[0, c0 + 1:c1 + 1, 1] - t[0, c0:c1, 1]).mean())
+    period = float(wrap(t[0, c0 + 1:c1 + 1, 1] - t[0, c0:c1, 1]).mean())
     names = {0: {0: "arrives_barrier", 1: "leaves_barrier", 5: "state_updated", 6: "state_copied", 2: "next_P_below_diagonal_formed",
                  3: "next_operands_read"},
              1: {0: "arrives_barrier", 1: "leaves_barrier", 5: "loads_issued", 2: "staged", 4: "hs_stored"},
@@ -356,7 +357,7 @@ def trace_simple_gla_fwd(lib, dev, work_group=16):
     for s_, nm in teams.items():
         out[nm] = {}
         for m, label in names[s_].items():
-            d = float((t[s_, c0:c1, m] - ref).mean())
+            d = float(wrap(t[s_, c0:c1, m] - ref).mean())
             if m == 0:
                 d += period
                 label = "arrives_next_barrier"

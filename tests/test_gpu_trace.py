@@ -9,13 +9,21 @@ import torch
 pytestmark = pytest.mark.gpu
 
 
-def _ordered(t, nch, marks):
-    """stamps of one slot: marks in the given order rise within a chunk, and from chunk to chunk"""
+def _ordered(t, nch, marks, bits=64):
+    """stamps of one slot: marks in the given order rise within a chunk, and from chunk to chunk (bits = 32: the
+    stamps are the low 32 bits of the clock, differences are taken modulo 2^32)"""
     t = t[:nch]
     assert (t[:, marks] > 0).all()
+
+    def later(b, a):
+        d = b - a
+        if bits == 32:
+            d = ((d + 2 ** 31) % 2 ** 32) - 2 ** 31
+        return (d >= 0).all()
+
     for a, b in zip(marks, marks[1:]):
-        assert (t[:, b] >= t[:, a]).all(), (a, b)
-    assert (t[1:, marks[0]] >= t[:-1, marks[-1]]).all()
+        assert later(t[:, b], t[:, a]), (a, b)
+    assert later(t[1:, marks[0]], t[:-1, marks[-1]])
 
 
 def test_traced_simple_gla_forward_is_the_forward_and_its_stamps_are_ordered():
@@ -38,12 +46,13 @@ def test_traced_simple_gla_forward_is_the_forward_and_its_stamps_are_ordered():
     assert torch.equal(o, o_ref) and torch.equal(ht, ht_ref)
     t = tr.cpu().view(3, 24, 8)
     nch = (T + 63) // 64
-    _ordered(t[0], nch - 1, [0, 1, 5, 6, 2, 3])      # (the last chunk has no next one to prepare)
-    _ordered(t[1], nch, [0, 1, 5, 2, 4])
-    _ordered(t[2], nch, [0, 1, 5, 2, 4, 6])
+    _ordered(t[0], nch - 1, [0, 1, 5, 6, 2, 3], bits=32)      # (the last chunk has no next one to prepare)
+    _ordered(t[1], nch, [0, 1, 5, 2, 4], bits=32)
+    _ordered(t[2], nch, [0, 1, 5, 2, 4, 6], bits=32)
     assert (t[:, nch:] == 0).all()
     # the teams meet at the barrier: nobody leaves the barrier of a chunk before everybody has arrived at it
-    assert (t[:, :nch, 1].min(0).values >= t[:, :nch, 0].max(0).values).all()
+    d = t[:, None, :nch, 1] - t[None, :, :nch, 0]              # leave of team i minus arrival of team j, modulo 2^32
+    assert ((((d + 2 ** 31) % 2 ** 32) - 2 ** 31) >= 0).all()
     # instances that do not exist are refused, not run
     call2 = SimpleGLACall(keep=True)
     call2.forward(q, k, v, g, None, None, False, None, False, save=True)
