@@ -6,6 +6,10 @@ namespace lmoe {
 
 template <typename T, int V> struct GlaTiles {
   static constexpr int BVS = 32;                                      // sequential passes
+  // ... 64 where that still fills the chip (2-byte elements): the V slices of a (sequence, head) each fetch all of the
+  // gated k (q) rows, so two wide slices ask the memory system for a quarter less per output column than four narrow
+  // ones.  A state element is the same sum over the tokens in either split: the results do not depend on the choice.
+  static constexpr int BVS_WIDE = (sizeof(T) == 2 && V >= 64) ? 64 : BVS;
   static constexpr int BVO = (sizeof(T) == 4 && V == 128) ? 64 : V;   // output / dv kernels
   static constexpr int BVH = sizeof(T) == 4 ? 32 : 64;                // V-slice loop of dq/dk/dg
 };
@@ -14,15 +18,20 @@ template <typename T, typename GT, int K, int V>
 static void launch_gla_t(const lmoe_args& a, int stage, hipStream_t st) {
   typedef GlaTiles<T, V> Tl;
   const dim3 block(NTHR);
+  const bool wide = Tl::BVS_WIDE != Tl::BVS && (int64_t)a.N * a.H * (V / Tl::BVS_WIDE) >= cu_count();
   switch (stage) {
     case ST_GLA_INTRA_FWD:
       hipLaunchKernelGGL((k_gla_intra_fwd<T, GT, K>), dim3(persistent_grid(a.NT * a.H, 2)), block, 0, st, a); break;
     case ST_STATE_FWD:
-      hipLaunchKernelGGL((k_gla_state_fwd<T, GT, K, V, Tl::BVS>), dim3((a.N * a.H + 7) / 8 * 8 * (V / Tl::BVS)), block, 0, st, a); break;
+      if (wide) hipLaunchKernelGGL((k_gla_state_fwd<T, GT, K, V, Tl::BVS_WIDE>), dim3((a.N * a.H + 7) / 8 * 8 * (V / Tl::BVS_WIDE)), block, 0, st, a);
+      else hipLaunchKernelGGL((k_gla_state_fwd<T, GT, K, V, Tl::BVS>), dim3((a.N * a.H + 7) / 8 * 8 * (V / Tl::BVS)), block, 0, st, a);
+      break;
     case ST_OUT_FWD:
       hipLaunchKernelGGL((k_gla_out_fwd<T, GT, K, V, Tl::BVO>), dim3(a.NT, a.H, V / Tl::BVO), block, 0, st, a); break;
     case ST_STATE_BWD:
-      hipLaunchKernelGGL((k_gla_state_bwd<T, GT, K, V, Tl::BVS>), dim3((a.N * a.H + 7) / 8 * 8 * (V / Tl::BVS)), block, 0, st, a); break;
+      if (wide) hipLaunchKernelGGL((k_gla_state_bwd<T, GT, K, V, Tl::BVS_WIDE>), dim3((a.N * a.H + 7) / 8 * 8 * (V / Tl::BVS_WIDE)), block, 0, st, a);
+      else hipLaunchKernelGGL((k_gla_state_bwd<T, GT, K, V, Tl::BVS>), dim3((a.N * a.H + 7) / 8 * 8 * (V / Tl::BVS)), block, 0, st, a);
+      break;
     case ST_DV:
       hipLaunchKernelGGL((k_gla_bwd_dv<T, GT, K, V, Tl::BVO>), dim3(a.NT, a.H, V / Tl::BVO), block, 0, st, a); break;
     case ST_DQK:
