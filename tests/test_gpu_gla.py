@@ -72,3 +72,25 @@ def test_gla_varlen(cuda, dtype):
     for n, r in ref.items():
         err = max_abs_rel(dev[n].grad.cpu(), r)
         assert err < tol, (n, err)
+
+
+def test_gla_results_do_not_depend_on_the_width_of_the_v_slices(cuda):
+    """The state passes take 64-wide V slices when there are enough (sequence, head) pairs to fill the chip with them
+    and 32-wide ones otherwise: a batch of 64 copies of a problem (wide) gives, row for row, the bits of the problem
+    alone (narrow)."""
+    from linear_moe_amd import chunk_gla
+    B, H, T, K, V = 1, 4, 200, 64, 128
+    q, k, v = gen(40, B, T, H, K).bfloat16(), gen(41, B, T, H, K).bfloat16(), gen(42, B, T, H, V).bfloat16()
+    g = (F.logsigmoid(gen(43, B, T, H, K)) / 4).bfloat16()
+    h0, do, dht = gen(44, B, H, K, V) * 0.5, gen(45, B, T, H, V).bfloat16(), gen(46, B, H, K, V)
+
+    def run(rep):
+        ins = [x.to(cuda).repeat(rep, *([1] * (x.dim() - 1))).requires_grad_(True) for x in (q, k, v, g, h0)]
+        o, ht = chunk_gla(ins[0], ins[1], ins[2], ins[3], None, ins[4], True, None, False)
+        grads = torch.autograd.grad([o, ht], ins, [do.to(cuda).repeat(rep, 1, 1, 1), dht.to(cuda).repeat(rep, 1, 1, 1)])
+        return [o, ht] + list(grads)
+
+    one, many = run(1), run(64)
+    torch.cuda.synchronize()
+    for a, b in zip(one, many):
+        assert torch.equal(a[0], b[0]) and torch.equal(a[0], b[63])
