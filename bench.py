@@ -38,8 +38,8 @@ STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_gdn_state_fwd_reg", 4: "k_gdn_state_bwd"
 # sources (kernel_sources_sha16()) at that time, and a build whose sources differ reports traffic = null
 # rather than a stale number.
 CALIB_COPY_BYTES = 256 << 20
-MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237243858, "k_gdn_state_fwd_reg": 1117613984, "k_gdn_state_bwd": 945963954,
-                    "k_gdn_bwd_chunk": 1898523039}
+MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237240853, "k_gdn_state_fwd_reg": 1118201928, "k_gdn_state_bwd": 945959318,
+                    "k_gdn_bwd_chunk": 1898516268}
 TRAFFIC_SOURCES_SHA16 = "51354044d042ec1d"
 TRAFFIC_SOURCES = ("lmoe_common.hpp", "lmoe_seq.hpp", "lmoe_gdn_wy.hpp", "lmoe_gdn_state.hpp", "lmoe_gdn_state_reg.hpp", "lmoe_gdn_bwd_chunk.hpp",
                    "lmoe_gdn_fwd.hip", "lmoe_gdn_state.hip", "lmoe_gdn_bwd.hip")
@@ -47,8 +47,8 @@ TRAFFIC_SOURCES = ("lmoe_common.hpp", "lmoe_seq.hpp", "lmoe_gdn_wy.hpp", "lmoe_g
 
 # HBM bytes per call of the other contract configurations (bench.py --other-configs), same counters and scaling,
 # summed over the kernels of the call; key = configuration number
-OTHER_TRAFFIC = {"1": 2231808, "2": 272912541, "3": 1547659052, "5": 16900897264}
-OTHER_TRAFFIC_SHA16 = "1ab39e90960c6dd3"
+OTHER_TRAFFIC = {"1": 2231801, "2": 272912028, "3": 1547651818, "5": 16893342544}
+OTHER_TRAFFIC_SHA16 = "ddeaf4cd78bb31f7"
 
 
 def all_sources_sha16():

@@ -21,6 +21,15 @@ template <bool LOCAL> struct BwdDv {
 template <typename T, int K, int V> struct StateBwd {
   static void run(const lmoe_args& a, hipStream_t st) {
     constexpr int BV = BwdTiles<T, V>::BVS;
+    // 64-wide slices where they still fill the chip (2-byte elements): every V slice of a (sequence, head) fetches all
+    // of q and k, so two wide slices ask the memory system for less per output column than four narrow ones; a state
+    // element is the same sum over the tokens in either split
+    constexpr int BW = (sizeof(T) == 2 && V >= 64) ? 64 : BV;
+    if (BW != BV && (int64_t)a.N * a.H * (V / BW) >= cu_count()) {
+      const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BW);
+      hipLaunchKernelGGL((k_state_bwd<T, K, V, BW>), dim3(grid), dim3(2 * NTHR), 0, st, a);
+      return;
+    }
     const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BV);
     hipLaunchKernelGGL((k_state_bwd<T, K, V, BV>), dim3(grid), dim3(2 * NTHR), 0, st, a);
   }

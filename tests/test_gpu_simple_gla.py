@@ -141,3 +141,25 @@ def test_forward_only_call_equals_the_saving_call(cuda):
     o2, ht2 = chunk_simple_gla(q.clone().requires_grad_(True), k, v, g, None, h0, True)
     torch.cuda.synchronize()
     assert torch.equal(o1, o2.detach()) and torch.equal(ht1, ht2.detach())
+
+
+def test_simple_gla_backward_does_not_depend_on_the_width_of_the_v_slices(cuda):
+    """The reverse state pass takes 64-wide V slices when there are enough (sequence, head) pairs to fill the chip
+    with them and 32-wide ones otherwise: a batch of 64 copies of a problem (wide) gives, row for row, the bits of the
+    problem alone (narrow)."""
+    from linear_moe_amd import chunk_simple_gla
+    B, H, T, K, V = 1, 4, 200, 128, 128
+    q, k, v = gen(50, B, T, H, K).bfloat16(), gen(51, B, T, H, K).bfloat16(), gen(52, B, T, H, V).bfloat16()
+    g = torch.nn.functional.logsigmoid(gen(53, B, T, H))
+    h0, do, dht = gen(54, B, H, K, V) * 0.5, gen(55, B, T, H, V).bfloat16(), gen(56, B, H, K, V)
+
+    def run(rep):
+        ins = [x.to(cuda).repeat(rep, *([1] * (x.dim() - 1))).requires_grad_(True) for x in (q, k, v, g, h0)]
+        o, ht = chunk_simple_gla(ins[0], ins[1], ins[2], ins[3], None, ins[4], True, None, False)
+        grads = torch.autograd.grad([o, ht], ins, [do.to(cuda).repeat(rep, 1, 1, 1), dht.to(cuda).repeat(rep, 1, 1, 1)])
+        return [o, ht] + list(grads)
+
+    one, many = run(1), run(64)
+    torch.cuda.synchronize()
+    for a, b in zip(one, many):
+        assert torch.equal(a[0], b[0]) and torch.equal(a[0], b[63])
