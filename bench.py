@@ -38,8 +38,7 @@ STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_gdn_state_fwd_reg", 4: "k_gdn_state_bwd"
 # sources (kernel_sources_sha16()) at that time, and a build whose sources differ reports traffic = null
 # rather than a stale number.
 CALIB_COPY_BYTES = 256 << 20
-MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237240853, "k_gdn_state_fwd_reg": 1118201928, "k_gdn_state_bwd": 945959318,
-                    "k_gdn_bwd_chunk": 1898516268}
+MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237242457, "k_gdn_state_fwd_reg": 1119621582, "k_gdn_state_bwd": 945960489, "k_gdn_bwd_chunk": 1898587576}
 TRAFFIC_SOURCES_SHA16 = "51354044d042ec1d"
 TRAFFIC_SOURCES = ("lmoe_common.hpp", "lmoe_seq.hpp", "lmoe_gdn_wy.hpp", "lmoe_gdn_state.hpp", "lmoe_gdn_state_reg.hpp", "lmoe_gdn_bwd_chunk.hpp",
                    "lmoe_gdn_fwd.hip", "lmoe_gdn_state.hip", "lmoe_gdn_bwd.hip")
@@ -47,8 +46,8 @@ TRAFFIC_SOURCES = ("lmoe_common.hpp", "lmoe_seq.hpp", "lmoe_gdn_wy.hpp", "lmoe_g
 
 # HBM bytes per call of the other contract configurations (bench.py --other-configs), same counters and scaling,
 # summed over the kernels of the call; key = configuration number
-OTHER_TRAFFIC = {"1": 2231801, "2": 272912028, "3": 1547651818, "5": 16893342544}
-OTHER_TRAFFIC_SHA16 = "ddeaf4cd78bb31f7"
+OTHER_TRAFFIC = {"1": 2223610, "2": 272924219, "3": 1547649854, "5": 16925504064}
+OTHER_TRAFFIC_SHA16 = "71cd874c1e6d14fc"
 
 
 def all_sources_sha16():

@@ -14,6 +14,17 @@ template <typename T, int K, int V> struct StateFwd {
     constexpr int BV = FwdTiles<T, V>::BVS;
     const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BV);
     if constexpr (sizeof(T) == 2) {
+      // 64-wide slices where they still fill the chip: every V slice of a (sequence, head) fetches all of q and k and
+      // forms all of P, so two wide slices cost less per output column than four narrow ones; the results do not
+      // depend on the width (a state element and an output element are the same sums in either split)
+      if constexpr (V >= 64) {
+        if ((int64_t)a.N * a.H * (V / 64) >= cu_count()) {
+          const int gw = ((a.N * a.H + 7) / 8) * 8 * (V / 64);
+          if (a.hs) hipLaunchKernelGGL((k_state_fwd_b<T, K, V, 64, true>), dim3(gw), dim3(3 * NTHR), 0, st, a, (long long*)nullptr, -1);
+          else hipLaunchKernelGGL((k_state_fwd_b<T, K, V, 64, false>), dim3(gw), dim3(3 * NTHR), 0, st, a, (long long*)nullptr, -1);
+          return;
+        }
+      }
       if (a.hs) hipLaunchKernelGGL((k_state_fwd_b<T, K, V, BV, true>), dim3(grid), dim3(3 * NTHR), 0, st, a, (long long*)nullptr, -1);
       else hipLaunchKernelGGL((k_state_fwd_b<T, K, V, BV, false>), dim3(grid), dim3(3 * NTHR), 0, st, a, (long long*)nullptr, -1);
     } else {

@@ -251,19 +251,20 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
 
 // ------------------------------------------------------------------------- //
 // The same pass for 2-byte elements, one barrier per chunk: whatever a window reads was completed in the window
-// before.  Three operand buffers (chunk c is worked on, chunk c + 1 is complete, chunk c + 2 is being staged), two
-// copies of S^T and two of P = (q k^T) . Gamma.  Window c, between barrier c and barrier c + 1:
+// before.  Two operand buffers (chunk c + 1 is complete, chunk c + 2 is being staged over chunk c, whose operands the
+// waves already hold in registers), two copies of S^T and two of P = (q k^T) . Gamma.  Window c, between barrier c and
+// barrier c + 1:
 //   consumers: S = e^{b_C} S + k^T (e_d v) on fragments of chunk c read before the barrier, S -> s_hT[(c + 1) & 1],
 //              then the blocks of P of chunk c + 1 below the diagonal -> s_P[(c + 1) & 1] (the output team, which
 //              formed its rows of P itself in an earlier version, was the longest chain of the window), then the
 //              fragments of chunk c + 1 for the next update
 //   loaders:   loads of chunk c + 4 issued into the register set that the last window's staging freed, chunk c + 2
-//              staged into buffer (c + 2) % 3, hs <- s_hT[c & 1] (SAVE)
+//              staged into buffer c & 1, hs <- s_hT[c & 1] (SAVE)
 //   output:    rows 16 w .. of o = e^b q S (s_hT[c & 1]) + P (s_P[c & 1]) v on q rows and v fragments read before
 //              the barrier, stored from registers, then the q rows and v fragments of chunk c + 1 and, from those q
 //              rows, the diagonal blocks of P of chunk c + 1
 // A chunk's own operands are staged two windows before its window: what is read of them is read at the end of the
-// window before, when the LDS is quiet.  Behind the barrier, where all twelve waves ask for data at once and a read
+// window before, when the LDS is quiet, and their buffer is free for the chunk after the next one as the window opens.  Behind the barrier, where all twelve waves ask for data at once and a read
 // takes about a thousand cycles to return, only S^T and P (written in the window before) are left to read.
 // Time stamps of the traced instance (TRACE = true): one wave of each team notes the shader clock where it arrives
 // at and leaves the barrier of a chunk and at a few points in between; the stamps sit in LDS (a global store
@@ -277,13 +278,13 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd_b(const lmoe_args a, lon
   static_assert(sizeof(T) == 2, "2-byte elements");
   constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDU = BV + LPAD;
   constexpr int MB = K / 64, NB = BV / 16, KS = K / 32, CS = CH / 32;
-  __shared__ __attribute__((aligned(16))) T s_k[3][CH * LDK];                 // k             [64][K]
-  __shared__ __attribute__((aligned(16))) T s_q[3][CH * LDK];                 // q             [64][K]
-  __shared__ __attribute__((aligned(16))) T s_u[3][CH * LDU];                 // v             [64][BV]
+  __shared__ __attribute__((aligned(16))) T s_k[2][CH * LDK];                 // k             [64][K]
+  __shared__ __attribute__((aligned(16))) T s_q[2][CH * LDK];                 // q             [64][K]
+  __shared__ __attribute__((aligned(16))) T s_u[2][CH * LDU];                 // v             [64][BV]
   __shared__ __attribute__((aligned(16))) T s_hT[2][BV * LDK];                // S^T           [BV][K]
   __shared__ __attribute__((aligned(16))) T s_P[2][CH * LDC];                 // P             [64][64]
-  __shared__ __attribute__((aligned(16))) float s_b[3][64], s_eb[3][64], s_ed[3][64];
-  __shared__ float s_dec[3];                                                  // e^{b_C} per buffer
+  __shared__ __attribute__((aligned(16))) float s_b[2][64], s_eb[2][64], s_ed[2][64];
+  __shared__ float s_dec[2];                                                  // e^{b_C} per buffer
   // (the low 32 bits of the clock: the LDS has no room for more beside the buffers of the pass)
   __shared__ uint32_t s_tr[TRACE ? SFWD_TRACE_SLOTS * SFWD_TRACE_CHUNKS * SFWD_TRACE_MARKS : 1];
   auto TR = [&](int slot, int c, int mark) {
@@ -332,7 +333,6 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd_b(const lmoe_args a, lon
   }
   typedef TileIO<T, CH, K> IOK;
   typedef TileIO<T, CH, BV> IOV;
-  typedef TileIO<T, BV, K> IOHT;
 
   // Blocks (ti, tj[0 .. n)) of P of chunk c (16 x 16 each, one q strip against n <= 2 k strips), formed transposed so
   // that a lane holds four consecutive columns of one row (8-byte writes).  The ten blocks on and below the diagonal
@@ -341,7 +341,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd_b(const lmoe_args a, lon
   // Every fragment is requested before the first product: the LDS is busiest right behind the barrier, a read comes
   // back after several hundred cycles, and a product loop that requests one step ahead pays that once per step.
   auto p_blocks = [&](int c, int ti, int tja, int tjb, int n) {
-    const int cb = c % 3, fr = l & 15, g = l >> 4;
+    const int cb = c & 1, fr = l & 15, g = l >> 4;
     const T *qc = s_q[cb], *kc = s_k[cb];
     T* Pn = s_P[c & 1];
     typename ET<T>::frag fq[KS], fka[KS], fkb[KS];
@@ -417,6 +417,20 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd_b(const lmoe_args a, lon
         if (l == 0) s_dec[buf] = expf(xl);
       }
     };
+    // hs[chunk][h][v0 .. v0+BV][K] <- S^T (only the backward reads it: SAVE = false for forward-only calls)
+    auto save_state = [&](int c) {
+      if constexpr (SAVE) {
+        T* hs = (T*)a.hs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K;
+        // a wide slice of a 128-wide key has few registers left beside three register sets in flight: a quarter of
+        // the rows at a time there
+        constexpr int RS = (BV >= 64 && K >= 128) ? BV / 4 : BV;
+#pragma unroll
+        for (int r0 = 0; r0 < BV; r0 += RS) {
+          if constexpr (RS < BV) __builtin_amdgcn_sched_barrier(0);
+          TileIO<T, RS, K>::lds_to_global(s_hT[c & 1] + r0 * LDK, LDK, hs + r0 * K, K, RS);
+        }
+      }
+    };
 #pragma unroll
     for (int j = 0; j < 3; ++j) issue(pre[j], j);
     stage(pre[0], 0);
@@ -445,11 +459,9 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd_b(const lmoe_args a, lon
         // (both always: past the end it is the last chunk again, never consumed)
         issue(pre[(j + 1) % 3], c + 4);
         if (wave == 4) TR(1, c, 5);
-        stage(pre[(j + 2) % 3], (j + 2) % 3);
+        stage(pre[(j + 2) % 3], c & 1);          // chunk c + 2 takes the buffer of chunk c
         if (wave == 4) TR(1, c, 2);
-        // hs[chunk][h][v0 .. v0+BV][K] <- S^T (only the backward reads it: SAVE = false for forward-only calls)
-        if constexpr (SAVE)
-          IOHT::lds_to_global(s_hT[c & 1], LDK, (T*)a.hs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
+        save_state(c);
         if (wave == 4) TR(1, c, 4);
       }
     }
@@ -468,7 +480,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd_b(const lmoe_args a, lon
     typename ET<T>::frag fq[KS], fv[CS][NB];
     float ebi;
     auto preread = [&](int c) {
-      const int cb = c % 3;
+      const int cb = c & 1;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) fq[ks] = ET<T>::load_frag(s_q[cb] + (16 * ow + fr) * LDK + 32 * ks + fg);
 #pragma unroll
@@ -482,7 +494,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd_b(const lmoe_args a, lon
     };
     // the diagonal block (ow, ow) of P of chunk c from the q rows that preread(c) has just fetched
     auto p_diag = [&](int c) {
-      const int cb = c % 3, g = l >> 4;
+      const int cb = c & 1, g = l >> 4;
       typename ET<T>::frag fk[KS];
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) fk[ks] = ET<T>::load_frag(s_k[cb] + (16 * ow + fr) * LDK + 32 * ks + fg);
@@ -594,7 +606,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd_b(const lmoe_args a, lon
   typename ET<T>::frag af[CS][MB], bf[CS][NB];
   float dec;
   auto preread = [&](int c) {
-    const int cb = c % 3;
+    const int cb = c & 1;
 #pragma unroll
     for (int kq = 0; kq < CS; ++kq) {
 #pragma unroll

@@ -143,12 +143,13 @@ def test_forward_only_call_equals_the_saving_call(cuda):
     assert torch.equal(o1, o2.detach()) and torch.equal(ht1, ht2.detach())
 
 
-def test_simple_gla_backward_does_not_depend_on_the_width_of_the_v_slices(cuda):
-    """The reverse state pass takes 64-wide V slices when there are enough (sequence, head) pairs to fill the chip
-    with them and 32-wide ones otherwise: a batch of 64 copies of a problem (wide) gives, row for row, the bits of the
-    problem alone (narrow)."""
+@pytest.mark.parametrize("K", [64, 128])
+def test_simple_gla_does_not_depend_on_the_width_of_the_v_slices(cuda, K):
+    """Both state passes take 64-wide V slices when there are enough (sequence, head) pairs to fill the chip with them
+    and 32-wide ones otherwise: a batch of 64 copies of a problem (wide) gives, row for row, the bits of the problem
+    alone (narrow) - outputs, final state and every gradient."""
     from linear_moe_amd import chunk_simple_gla
-    B, H, T, K, V = 1, 4, 200, 128, 128
+    B, H, T, V = 1, 4, 200, 128
     q, k, v = gen(50, B, T, H, K).bfloat16(), gen(51, B, T, H, K).bfloat16(), gen(52, B, T, H, V).bfloat16()
     g = torch.nn.functional.logsigmoid(gen(53, B, T, H))
     h0, do, dht = gen(54, B, H, K, V) * 0.5, gen(55, B, T, H, V).bfloat16(), gen(56, B, H, K, V)
@@ -163,3 +164,7 @@ def test_simple_gla_backward_does_not_depend_on_the_width_of_the_v_slices(cuda):
     torch.cuda.synchronize()
     for a, b in zip(one, many):
         assert torch.equal(a[0], b[0]) and torch.equal(a[0], b[63])
+    with torch.no_grad():          # the forward-only instance (no per-chunk states written) of the wide pass
+        o, ht = chunk_simple_gla(*[x.to(cuda).repeat(64, *([1] * (x.dim() - 1))) for x in (q, k, v, g)], None,
+                                 h0.to(cuda).repeat(64, 1, 1, 1), True, None, False)
+    assert torch.equal(o[63], one[0][0]) and torch.equal(ht[63], one[1][0])
