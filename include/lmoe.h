@@ -258,7 +258,9 @@ int lmoe_mom_rowdot(const void* src, const int32_t* idx, const void* g, void* dw
  * op's fwd (stages 0-2, 7) or bwd (stages 3-5) entry point, with the intermediates of the
  * earlier stages already in place.  Stages: 0 gated-delta-rule WY preparation, 1 forward state
  * pass, 2 output, 3 dv, 4 reverse state pass, 5 dq dk and gate gradient (gated delta rule: every
- * gradient that follows the reverse state pass), 7 chunk_gla intra-chunk matrix.
+ * gradient that follows the reverse state pass; chunk_simple_gla with 2-byte elements: dv as well, so that its
+ * backward entry point does not run stage 3, which stays available and gives the same dv), 7 chunk_gla intra-chunk
+ * matrix.
  * No counterpart in the reference (measurement support). */
 #define LMOE_OP_SIMPLE_GLA 0
 #define LMOE_OP_GLA 1

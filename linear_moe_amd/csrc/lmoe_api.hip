@@ -85,7 +85,8 @@ int lmoe_chunk_simple_gla_bwd(const lmoe_args* a, void* stream) {
   if (a->gate == LMOE_GATE_SCALAR && !a->dg.ptr) return fail(-13, "%s: dg must not be null for a gated call", op);
   if (a->NT == 0 || a->N == 0) return 0;
   lmoe::launch_state_bwd(*a, (hipStream_t)stream);
-  lmoe::launch_bwd_dv(*a, false, (hipStream_t)stream);
+  // 2-byte elements: dv is formed by the kernel that forms dq and dk, from the tiles it holds anyway
+  if (a->dtype == LMOE_F32) lmoe::launch_bwd_dv(*a, false, (hipStream_t)stream);
   lmoe::launch_bwd_dqk(*a, (hipStream_t)stream);
   return launched(op);
 }
@@ -478,6 +479,8 @@ int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* strea
           if (!a->tinv || !a->dvnew.ptr || !a->beta.ptr) return fail(-11, "%s: tinv, dvnew and beta must not be null", nm);
           lmoe::launch_gdn_bwd_chunk(*a, st);
         } else {
+          if (!a->hs || !a->dhs || !a->d_o.ptr || !a->dq.ptr || !a->dk.ptr || (a->dtype != LMOE_F32 && !a->dv.ptr))
+            return fail(-11, "%s: hs, dhs, d_o, dq, dk (and dv: 2-byte elements) must not be null", nm);
           lmoe::launch_bwd_dqk(*a, st);
         }
         break;

@@ -38,7 +38,8 @@ template <typename T, int K, int V> struct BwdDqk {
   static void run(const lmoe_args& a, hipStream_t st) {
     constexpr int BVH = BwdTiles<T, V>::BVH;
     const int grid = persistent_grid(a.NT * a.H, 1);
-    hipLaunchKernelGGL((k_bwd_dqk<T, K, V, BVH>), dim3(grid), dim3(2 * NTHR), 0, st, a);
+    if constexpr (sizeof(T) == 2) hipLaunchKernelGGL((k_bwd_dqkv<T, K, V, BVH>), dim3(grid), dim3(2 * NTHR), 0, st, a);
+    else hipLaunchKernelGGL((k_bwd_dqk<T, K, V, BVH>), dim3(grid), dim3(2 * NTHR), 0, st, a);
   }
 };
 

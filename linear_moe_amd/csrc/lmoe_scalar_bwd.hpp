@@ -9,6 +9,7 @@
 //   k_bwd_dqk   : chunk-parallel   dq, dk, gate gradient
 //                 db_i = q_i.dq_i - k_i.dk_i (+ on the last row sum_j (dk_d . k_d)_j + e^{b_C} <S, dS'>),
 //                 dg = reverse cumsum of db.
+//   k_bwd_dqkv  : k_bwd_dqk and k_bwd_dv in one kernel (2-byte elements; the fp32 path runs the two)
 #pragma once
 #include "lmoe_seq.hpp"
 #include "lmoe_scalar_fwd.hpp"   // scale_frag
@@ -87,7 +88,7 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dv(const lmoe_args a) {
 #pragma unroll
     for (int ni = 0; ni < NB; ++ni)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) dv[0][ni][i] += t[0][ni][i] * s_ed[16 * wv + 4 * (l >> 4) + i];
+      for (int i = 0; i < 4; ++i) dv[0][ni][i] = __builtin_fmaf(t[0][ni][i], s_ed[16 * wv + 4 * (l >> 4) + i], dv[0][ni][i]);
   }
   const lmoe_tensor& dst = LOCAL ? a.dvnew : a.dv;
   store_strip<T, NB>(dv, s_stg + wv * 16 * LDV, row_ptr<T>(dst, ci.b, ci.tok + 16 * wv, h) + v0, dst.st,
@@ -485,6 +486,306 @@ __global__ __launch_bounds__(2 * NTHR) void k_bwd_dqk(const lmoe_args a) {
       if (a.dg.ptr && j < ci.len) ((float*)a.dg.ptr)[row_off(a.dg, ci.b, ci.tok + j, h)] = x;
     }
     lds_barrier();     // E: the second buffer and the gate arrays go to the next item
+  }
+}
+
+// ------------------------------------------------------------------------- //
+// dq, dk, dv, gate gradient in one kernel (2-byte elements)     persistent: one work-group per CU,
+// one item = (chunk, head).  k_bwd_dqk with the work of k_bwd_dv folded in: the do, dS'^T, q and k tiles that dv
+// needs lie in LDS for dq and dk anyway, so dv costs this kernel no load, and q, k, do and dhs are not fetched a
+// second time by a kernel of their own.
+//   start of an item : wave w forms columns 16 w .. of P = (q k^T) . Gamma transposed (lane: four consecutive rows i
+//                      of one column j, 8-byte writes into its own rows of the P^T tile) and keeps those rows and
+//                      its k rows as matrix operands in registers
+//   slice s          : dP, dq_i, dk_d as in k_bwd_dqk, and  dv^T = scale do^T P + dS'^T (k . e_d)^T  formed
+//                      transposed, so that a lane holds four consecutive columns of one token: 8-byte stores
+//                      straight from the accumulators
+//   phase B          : as in k_bwd_dqk; (scale dP . Gamma)^T takes the place of P^T
+//   q, k and the gate arrays of an item are staged while the item before stores its results (its own staging strips
+//   lie in the slice buffer that is idle then); the gate arrays alternate between two sets.
+//   Script per item (NS slices):  [slice 0] R(1) .. R(NS-1) | D | A | b | c | E
+//     loaders : R(s): stage slice s+1 | D: <S, dS'> | A: stage slice 0 of the next item | c: stage q, k, gates of
+//               the next item, request those of the one after
+//     compute : P^T strip | products of slice s, dv stores | D, A | (dP . Gamma)^T -> LDS | b | products, combine |
+//               c | stores | E
+// Every sum is formed in the order of k_bwd_dv and k_bwd_dqk: the results are theirs bit for bit.
+// ------------------------------------------------------------------------- //
+template <typename T, int K, int V, int BVH>
+__global__ __launch_bounds__(2 * NTHR) void k_bwd_dqkv(const lmoe_args a) {
+  static_assert(sizeof(T) == 2, "2-byte elements");
+  constexpr int LDV = BVH + LPAD, LDC = CH + LPAD, LDK = K + LPAD;
+  constexpr int NBK = K / 16, NS = V / BVH, NBV = BVH / 16, KS = K / 32, CS = CH / 32;
+  // tiles of one V-slice (two buffers)
+  constexpr int A_DO = 0, A_V = A_DO + CH * LDV, A_H = A_V + CH * LDV, A_DH = A_H + BVH * LDK,
+                A_END = A_DH + BVH * LDK;
+  constexpr int BUF1 = A_END;
+  // tiles of the item
+  constexpr int B_PT = 2 * A_END, B_K = B_PT + CH * LDC, B_Q = B_K + CH * LDK, NELEM = B_Q + CH * LDK;
+  static_assert(2 * 4 * 16 * LDK <= A_END, "the store staging strips fit the idle slice buffer");
+  __shared__ __attribute__((aligned(16))) T smem[NELEM];
+  __shared__ __attribute__((aligned(16))) float s_b[2][64], s_eb[2][64], s_ed[2][64];
+  __shared__ float s_db[64], s_red[8];
+
+  const int l = lane_id();
+  const int team = threadIdx.x / NTHR;
+  typedef TileIO<T, CH, BVH> IOV;
+  typedef TileIO<T, BVH, K> IOH;
+  typedef TileIO<T, CH, K> IOK;
+  const int nitems = a.NT * a.H;
+  const int stride = gridDim.x;
+
+  if (team == 1) {
+    // --------------------------------- loaders -------------------------------------------
+    struct SliceRegs { typename IOV::Regs rd, rv; typename IOH::Regs rh, rdh; int len; };
+    struct QKRegs { typename IOK::Regs rq, rk; uint32_t graw; int len; };
+    SliceRegs S;
+    QKRegs Q;
+    // Every prefetch is issued unconditionally (item index clamped to the last item): a load that
+    // is skipped on some path would make the compiler drain all outstanding loads at every use.
+    auto issue_slice = [&](int it, int vv) {
+      it = min(it, nitems - 1);
+      const int cid = it / a.H, h = it % a.H;
+      const ChunkInfo ci = chunk_info(a, cid);
+      S.len = ci.len;
+      IOV::load_nomask(S.rd, row_ptr<T>(a.d_o, ci.b, ci.tok, h) + vv, a.d_o.st, ci.len);
+      IOV::load_nomask(S.rv, row_ptr<T>(a.v, ci.b, ci.tok, h) + vv, a.v.st, ci.len);
+      IOH::load_nomask(S.rh, (const T*)a.hs + (((int64_t)cid * a.H + h) * V + vv) * K, K, BVH);
+      IOH::load_nomask(S.rdh, (const T*)a.dhs + (((int64_t)cid * a.H + h) * V + vv) * K, K, BVH);
+    };
+    auto issue_qk = [&](int it) {
+      it = min(it, nitems - 1);
+      const int cid = it / a.H, h = it % a.H;
+      const ChunkInfo ci = chunk_info(a, cid);
+      Q.len = ci.len;
+      IOK::load_nomask(Q.rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
+      IOK::load_nomask(Q.rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
+      Q.graw = gate_prefetch(a, ci.b, ci.tok, ci.len, h);
+    };
+    float hdh = 0.f;   // partial <S, dS'> of the item whose slices are being staged
+    auto stage_slice = [&](int buf) {
+      T* base = smem + buf * BUF1;
+#pragma unroll
+      for (int p = 0; p < IOH::PASSES; ++p)
+#pragma unroll
+        for (int i = 0; i < IOH::VEC; ++i) hdh += ET<T>::to_f(S.rh.v[p][i]) * ET<T>::to_f(S.rdh.v[p][i]);
+      IOV::mask(S.rd, S.len);
+      IOV::mask(S.rv, S.len);
+      IOV::store_lds(S.rd, base + A_DO, LDV);
+      IOV::store_lds(S.rv, base + A_V, LDV);
+      IOH::store_lds(S.rh, base + A_H, LDK);
+      IOH::store_lds(S.rdh, base + A_DH, LDK);
+    };
+    auto stage_qk = [&](int par) {
+      gate_finish_wave(a, Q.graw, Q.len, l, wave_id() == 4, s_b[par], s_eb[par], s_ed[par]);
+      IOK::mask(Q.rq, Q.len);
+      IOK::mask(Q.rk, Q.len);
+      IOK::store_lds(Q.rq, smem + B_Q, LDK);
+      IOK::store_lds(Q.rk, smem + B_K, LDK);
+    };
+    // the slice after slice s of item it
+    auto issue_next = [&](int it, int s) {
+      if (s + 1 < NS) issue_slice(it, (s + 1) * BVH); else issue_slice(it + stride, 0);
+    };
+    const int it0 = blockIdx.x;
+    issue_slice(it0, 0);
+    issue_qk(it0);
+    // the first loads may be ordered freely by the compiler; were they still pending at the loop
+    // header, its wait-count analysis would carry that order into every iteration
+    wait_all_loads();
+    stage_slice(0);
+    stage_qk(0);
+    issue_qk(it0 + stride);
+    issue_next(it0, 0);
+    lds_barrier();                                                                       // first item staged
+    int par = 0;
+    for (int it = it0; it < nitems; it += stride, par ^= 1) {
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        if (s > 0) lds_barrier();                                                        // R(s)
+        if (s + 1 < NS) {
+          stage_slice((s + 1) & 1);        // its buffer was left when the compute team passed R(s) (s = 0: E)
+          issue_next(it, s + 1);
+        }
+      }
+      lds_barrier();                                                                     // D
+      hdh = wave_sum(hdh);
+      if (l == 0) s_red[wave_id() - 4] = hdh;
+      hdh = 0.f;
+      lds_barrier();                                                                     // A
+      stage_slice(0);                      // slice 0 of the next item (buffer 0 is idle in phase B)
+      issue_next(it + stride, 0);
+      lds_barrier();                                                                     // b
+      lds_barrier();                                                                     // c
+      stage_qk(par ^ 1);                   // q, k of this item were read for the last time before c
+      issue_qk(it + 2 * stride);
+      lds_barrier();                                                                     // E
+    }
+    return;
+  }
+
+  // --------------------------------- compute ---------------------------------------------
+  const int wv = wave_id();
+  const T* QT = smem + B_Q;
+  const T* KT = smem + B_K;
+  T* PT = smem + B_PT;
+  lds_barrier();                                                                         // first item staged
+  int par = 0;
+  for (int it = blockIdx.x; it < nitems; it += stride, par ^= 1) {
+    const int cid = it / a.H, h = it % a.H;
+    const ChunkInfo ci = chunk_info(a, cid);
+    // (the lane index refreshed per item: what derives from it is recomputed where it is used instead of being kept,
+    // and spilled, for the whole kernel)
+    const int lf = fresh_index(l);
+    const int fr = lf & 15, g = lf >> 4, fg = 8 * g;
+    const int j = 16 * wv + fr;            // the token of this lane in transposed products
+    // rows j = 16 wv .. of P^T (zero where i < j), written by and for this wave only
+    typename ET<T>::frag fk[KS], fpt[CS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) fk[ks] = ET<T>::load_frag(KT + j * LDK + 32 * ks + fg);
+    const float bj = s_b[par][j], edj = s_ed[par][j];
+#pragma unroll
+    for (int ib = 0; ib < 4; ++ib) {
+      bf16x4 y = {(bf16)0.f, (bf16)0.f, (bf16)0.f, (bf16)0.f};
+      if (ib >= wv) {
+        typename ET<T>::frag fq[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) fq[ks] = ET<T>::load_frag(QT + (16 * ib + fr) * LDK + 32 * ks + fg);
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) ET<T>::mma(acc, fq[ks], fk[ks]);
+        const f32x4 bi = *(const f32x4*)&s_b[par][16 * ib + 4 * g];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) y[e] = (bf16)((16 * ib + 4 * g + e >= j) ? acc[e] * texp<T>(bi[e] - bj) : 0.f);
+      }
+      *(bf16x4*)(PT + j * LDC + 16 * ib + 4 * g) = y;
+    }
+#pragma unroll
+    for (int kq = 0; kq < CS; ++kq) fpt[kq] = ET<T>::load_frag(PT + j * LDC + 32 * kq + fg);
+
+    f32x4 dP[1][4], dqi[1][NBK], dkd[1][NBK];
+    acc_zero(dP); acc_zero(dqi); acc_zero(dkd);
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      if (s > 0) lds_barrier();                                                          // R(s)
+      const T* base = smem + (s & 1) * BUF1;
+      const T* DO = base + A_DO; const T* VN = base + A_V;
+      const T* HT = base + A_H; const T* DHT = base + A_DH;
+#pragma unroll
+      for (int kk = 0; kk < BVH; kk += 32) {
+        const typename ET<T>::frag aDO = ET<T>::load_frag(DO + (16 * wv + fr) * LDV + kk + fg);
+        const typename ET<T>::frag aVN = ET<T>::load_frag(VN + (16 * wv + fr) * LDV + kk + fg);
+#pragma unroll
+        for (int nj = 0; nj < 4; ++nj)
+          ET<T>::mma(dP[0][nj], aDO, ET<T>::load_frag(VN + (16 * nj + fr) * LDV + kk + fg));
+        __builtin_amdgcn_sched_barrier(0);     // bounds the fragments in flight (register budget)
+#pragma unroll
+        for (int ni = 0; ni < NBK; ++ni) {
+          const typename ET<T>::frag bH = ET<T>::load_frag_t(HT, LDK, kk, 16 * ni, lf);
+          ET<T>::mma(dqi[0][ni], aDO, bH);
+          ET<T>::mma(dkd[0][ni], aVN, ET<T>::load_frag_t(DHT, LDK, kk, 16 * ni, lf));
+          if (ni % 4 == 3) __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      // dv^T of the slice: lane = token j, columns 16 ni + 4 g .. + 3
+      f32x4 t1[NBV], t2[NBV];
+#pragma unroll
+      for (int ni = 0; ni < NBV; ++ni) t1[ni] = t2[ni] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kq = 0; kq < CS; ++kq) {
+        if (2 * kq + 1 >= wv) {            // rows i < 32 of P^T are zero for the waves 2, 3
+#pragma unroll
+          for (int ni = 0; ni < NBV; ++ni) ET<T>::mma(t1[ni], ET<T>::load_frag_t(DO, LDV, 32 * kq, 16 * ni, lf), fpt[kq]);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+        for (int ni = 0; ni < NBV; ++ni)
+          ET<T>::mma(t2[ni], ET<T>::load_frag(DHT + (16 * ni + fr) * LDK + 32 * ks + fg), fk[ks]);
+        if (ks % 2 == 1) __builtin_amdgcn_sched_barrier(0);     // bounds the fragments in flight (register budget)
+      }
+      if (j < ci.len) {
+        T* drow = row_ptr<T>(a.dv, ci.b, ci.tok + j, h) + s * BVH + 4 * g;
+#pragma unroll
+        for (int ni = 0; ni < NBV; ++ni) {
+          bf16x4 y;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            // (the rounding steps of k_bwd_dv: the product with the scale rounded, then one fused multiply-add)
+            y[e] = (bf16)__builtin_fmaf(t2[ni][e], edj, __fmul_rn(t1[ni][e], a.scale));
+          }
+          *(bf16x4*)(drow + 16 * ni) = y;
+        }
+      }
+    }
+    lds_barrier();                                                                       // D
+    lds_barrier();                                                                       // A
+#pragma unroll
+    for (int nj = 0; nj < 4; ++nj) {
+      f32x4 p;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = 16 * wv + 4 * g + i, cc = 16 * nj + fr;
+        p[i] = (r >= cc) ? a.scale * dP[0][nj][i] * texp<T>(s_b[par][r] - s_b[par][cc]) : 0.f;
+      }
+      acc_to_lds_t<T>(p, PT, LDC, 16 * wv, 16 * nj, lf);      // [j][i]
+    }
+    lds_barrier();                                                                       // b
+    f32x4 dq[1][NBK], dk[1][NBK];
+    acc_zero(dq); acc_zero(dk);
+    // dq_intra[i][c] = sum_j dPG[i][j] k[j][c] : A = dPG^T stored [j][i] (contraction along rows)
+    gemm<T, 1, NBK, true, true>(dq, PT, LDC, 16 * wv, KT, LDK, 0, 0, CH, lf);
+    __builtin_amdgcn_sched_barrier(0);
+    // dk_intra[j][c] = sum_i dPG[i][j] q[i][c] : A = dPG^T rows j (contraction along columns)
+    gemm<T, 1, NBK, false, true>(dk, PT, LDC, 16 * wv, QT, LDK, 0, 0, CH, lf);
+    __builtin_amdgcn_sched_barrier(0);
+    // combine and form db_i = q_i.dq_i - k_i.dk_i ; kk = sum_j (dk_d . k_d)_j
+    float dbp[4] = {0.f, 0.f, 0.f, 0.f};
+    float kk = 0.f;
+#pragma unroll
+    for (int ni = 0; ni < NBK; ++ni)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = 16 * wv + 4 * g + i, cc = 16 * ni + fr;
+        const float qv = ET<T>::to_f(QT[r * LDK + cc]);
+        const float kv = ET<T>::to_f(KT[r * LDK + cc]);
+        const float dqv = a.scale * s_eb[par][r] * dqi[0][ni][i] + dq[0][ni][i];
+        const float dkdv = s_ed[par][r] * dkd[0][ni][i];
+        const float dkv = dkdv + dk[0][ni][i];
+        dbp[i] += qv * dqv - kv * dkv;
+        kk += kv * dkdv;
+        dq[0][ni][i] = dqv;
+        dk[0][ni][i] = dkv;
+      }
+    // reduce db over the 16 lanes that share a row group, kk over the whole team
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dbp[i] = group_sum<16>(dbp[i]);
+    if (fr == 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) s_db[16 * wv + 4 * g + i] = dbp[i];
+    }
+    kk = wave_sum(kk);
+    if (lf == 0) s_red[4 + wv] = kk;
+    lds_barrier();     // c: the q, k tiles go to the next item; the idle slice buffer is the store staging
+    {
+      T* stg = smem + BUF1 + wv * 16 * LDK;
+      store_strip<T, NBK>(dq, stg, row_ptr<T>(a.dq, ci.b, ci.tok + 16 * wv, h), a.dq.st, ci.len - 16 * wv, 1.0f, lf);
+      T* stg2 = smem + BUF1 + (4 + wv) * 16 * LDK;
+      store_strip<T, NBK>(dk, stg2, row_ptr<T>(a.dk, ci.b, ci.tok + 16 * wv, h), a.dk.st, ci.len - 16 * wv, 1.0f, lf);
+    }
+    if (threadIdx.x < 64) {
+      const int t = threadIdx.x;
+      float x = s_db[t];
+      // last-row term; rows past the end of a partial chunk carry zero q, k, so the term may sit
+      // on the last valid row without changing the reverse cumulative sum
+      const float hsum = s_red[0] + s_red[1] + s_red[2] + s_red[3];
+      const float ksum = s_red[4] + s_red[5] + s_red[6] + s_red[7];
+      if (t == ci.len - 1) x += ksum + expf(s_b[par][63]) * hsum;
+      x = wave_rev_scan(x);   // dg
+      if (a.dg.ptr && t < ci.len) ((float*)a.dg.ptr)[row_off(a.dg, ci.b, ci.tok + t, h)] = x;
+    }
+    lds_barrier();     // E: the staging strips and the P^T tile go to the next item
   }
 }
 

@@ -168,3 +168,32 @@ def test_simple_gla_does_not_depend_on_the_width_of_the_v_slices(cuda, K):
         o, ht = chunk_simple_gla(*[x.to(cuda).repeat(64, *([1] * (x.dim() - 1))) for x in (q, k, v, g)], None,
                                  h0.to(cuda).repeat(64, 1, 1, 1), True, None, False)
     assert torch.equal(o[63], one[0][0]) and torch.equal(ht[63], one[1][0])
+
+
+@pytest.mark.parametrize("B,H,T,K,V,varlen", [(2, 3, 200, 128, 128, False), (1, 4, 64, 64, 64, False),
+                                              (2, 2, 130, 64, 128, False), (1, 2, 333, 128, 64, False),
+                                              (1, 4, 700, 128, 128, True)])
+def test_dv_of_the_fused_backward_kernel_equals_the_kernel_of_its_own(cuda, B, H, T, K, V, varlen):
+    """With 2-byte elements dv is formed by the kernel that forms dq and dk, from the tiles that kernel holds anyway,
+    as transposed products; the chunk-parallel dv kernel (what the fp32 path runs, still reachable as a stage) forms
+    the same sums in the same order: bit for bit the same dv, partial chunks and packed sequences included."""
+    from linear_moe_amd import _lib
+    from linear_moe_amd.simple_gla import SimpleGLACall
+    lib = _lib.load()
+    q, k = gen(70, B, T, H, K).bfloat16().to(cuda), gen(71, B, T, H, K).bfloat16().to(cuda)
+    v, do = gen(72, B, T, H, V).bfloat16().to(cuda), gen(73, B, T, H, V).bfloat16().to(cuda)
+    g = F.logsigmoid(gen(74, B, T, H)).to(cuda)
+    cu = torch.tensor([0, 100, 101, 450, 700], device=cuda, dtype=torch.int32) if varlen else None
+    N = 4 if varlen else B
+    h0, dht = (gen(75, N, H, K, V) * 0.3).to(cuda), gen(76, N, H, K, V).to(cuda)
+    call = SimpleGLACall(keep=True)
+    call.forward(q, k, v, g, None, h0, True, cu, False)
+    dq, dk, dv, dg, dh0 = call.backward(do, dht)
+    torch.cuda.synchronize()
+    fused = dv.clone()
+    assert fused.abs().max() > 0
+    dv.zero_()
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _lib.check(lib.lmoe_launch_stage(C.byref(call.bwd_args), call.OP, 3, st), "dv stage")      # 3: the dv kernel
+    torch.cuda.synchronize()
+    assert torch.equal(fused, dv)
