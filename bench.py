@@ -38,7 +38,7 @@ STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_gdn_state_fwd_reg", 4: "k_gdn_state_bwd"
 # sources (kernel_sources_sha16()) at that time, and a build whose sources differ reports traffic = null
 # rather than a stale number.
 CALIB_COPY_BYTES = 256 << 20
-MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237242457, "k_gdn_state_fwd_reg": 1119621582, "k_gdn_state_bwd": 945960489, "k_gdn_bwd_chunk": 1898587576}
+MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237242501, "k_gdn_state_fwd_reg": 1119125993, "k_gdn_state_bwd": 945960119, "k_gdn_bwd_chunk": 1898515894}
 TRAFFIC_SOURCES_SHA16 = "51354044d042ec1d"
 TRAFFIC_SOURCES = ("lmoe_common.hpp", "lmoe_seq.hpp", "lmoe_gdn_wy.hpp", "lmoe_gdn_state.hpp", "lmoe_gdn_state_reg.hpp", "lmoe_gdn_bwd_chunk.hpp",
                    "lmoe_gdn_fwd.hip", "lmoe_gdn_state.hip", "lmoe_gdn_bwd.hip")
@@ -46,8 +46,8 @@ TRAFFIC_SOURCES = ("lmoe_common.hpp", "lmoe_seq.hpp", "lmoe_gdn_wy.hpp", "lmoe_g
 
 # HBM bytes per call of the other contract configurations (bench.py --other-configs), same counters and scaling,
 # summed over the kernels of the call; key = configuration number
-OTHER_TRAFFIC = {"1": 2223610, "2": 272924219, "3": 1547649854, "5": 16925504064}
-OTHER_TRAFFIC_SHA16 = "71cd874c1e6d14fc"
+OTHER_TRAFFIC = {"1": 2223612, "2": 272920454, "3": 1547656280, "5": 16903689853, "6": 1444726072}
+OTHER_TRAFFIC_SHA16 = "76755e72d356cd98"
 
 
 def all_sources_sha16():
@@ -369,9 +369,10 @@ def trace_simple_gla_fwd(lib, dev, work_group=16):
 
 
 def other_configs(dev, steps, warmup):
-    """The four contract configurations beside the headline one, through the Python entry points (inputs of
-    the contract's laws, drawn on the GPU: this leg times, the parity tests check): ms per call, tokens/s and
-    the algorithmic bytes (every input read once, every output written once) against the HBM peak."""
+    """The four contract configurations beside the headline one, and the forward + backward of chunk_simple_gla on
+    the shape of configuration 2, through the Python entry points (inputs of the contract's laws, drawn on the GPU:
+    this leg times, the parity tests check): ms per call, tokens/s and the algorithmic bytes (every input read once,
+    every output written once) against the HBM peak."""
     import torch
     import torch.nn.functional as F
     import linear_moe_amd as L
@@ -440,6 +441,19 @@ def other_configs(dev, steps, warmup):
     res["5 packed gated_delta_rule fwd+bwd bf16 16 seqs 65536 tokens H=32 K=V=128"] = (
         sec, Tt, Tt * H * ((6 * K + 5 * V) * 2 + 3 * 2 + 12) + 4 * N * H * K * V * 4,
         3 * Tt * H * (6 * CH * K + 4 * CH * V + 6 * K * V + (2 / 3) * CH * CH), PEAK_MFMA_BF16)
+    # 6 (not a contract configuration): the shape of configuration 2 with its backward, the training step of the
+    # chunk_simple_gla family (retention, lightning attention, basic linear attention); per-token log-decays
+    B, H, T, K = 4, 16, 4096, 128
+    q, k, v = (rn(B, T, H, K).requires_grad_(True) for _ in range(3))
+    g = (-torch.rand(B, T, H, device=dev) * 0.1).requires_grad_(True)
+    do = rn(B, T, H, K)
+
+    def f6():
+        o, _ = L.chunk_simple_gla(q, k, v, g, head_first=False)
+        torch.autograd.grad([o], [q, k, v, g], [do])
+    sec = timed(f6)
+    res["6 simple_gla fwd+bwd bf16 B=4 H=16 T=4096 K=V=128"] = (sec, B * T, B * T * H * ((6 * K + 5 * K) * 2 + 12),
+                                                                3 * B * T * H * sg_flops(K, K), PEAK_MFMA_BF16)
     # one roofline record per configuration, for the whole call on its minimal traffic (every input read once, every
     # output written once): all five are bound by HBM on that count (arithmetic intensity below peak flops / peak
     # bytes).  `traffic` = HBM bytes per call summed over its kernels, from the FETCH_SIZE / WRITE_SIZE counters
@@ -453,7 +467,8 @@ def other_configs(dev, steps, warmup):
                                "unit": "GB/s", "frac": round(nb / sec / PEAK_HBM, 4),
                                "mfma_frac": round(fl / sec / peak_f, 4),
                                "traffic": OTHER_TRAFFIC.get(n[0]) if fresh else None}}
-    return {"metric": "contract configurations 1, 2, 3, 5: ms per call, tokens/s", "unit": "ms", "steps": steps,
+    return {"metric": "contract configurations 1, 2, 3, 5 and the training step on the shape of 2 (6): ms per call, "
+                      "tokens/s", "unit": "ms", "steps": steps,
             "warmup": warmup, "data": "synthetic", "configs": out}
 
 
