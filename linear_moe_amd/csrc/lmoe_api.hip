@@ -119,7 +119,8 @@ int lmoe_chunk_gla_bwd(const lmoe_args* a, void* stream) {
   if (a->NT == 0 || a->N == 0) return 0;
   hipStream_t st = (hipStream_t)stream;
   lmoe::launch_gla(*a, lmoe::ST_STATE_BWD, st);
-  lmoe::launch_gla(*a, lmoe::ST_DV, st);
+  // 2-byte elements: dv is formed by the kernel that forms dq, dk and dg, from the slices it stages anyway
+  if (a->dtype == LMOE_F32) lmoe::launch_gla(*a, lmoe::ST_DV, st);
   lmoe::launch_gla(*a, lmoe::ST_DQK, st);
   return launched(op);
 }

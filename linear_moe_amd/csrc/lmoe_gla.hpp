@@ -611,7 +611,7 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dv(const lmoe_args a) {
     for (int ni = 0; ni < NB; ++ni) {
       typename ET<T>::vec4 x;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) x[i] = ET<T>::from_f(a.scale * dv[ni][0][i] + dv2[ni][0][i]);
+      for (int i = 0; i < 4; ++i) x[i] = ET<T>::from_f(__builtin_fmaf(a.scale, dv[ni][0][i], dv2[ni][0][i]));
       *(typename ET<T>::vec4*)(dd + 16 * ni) = x;
     }
   }
@@ -621,13 +621,18 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dv(const lmoe_args a) {
 // dq, dk, dg, grid = (NT, H)
 // ------------------------------------------------------------------------- //
 template <typename T, typename GT, int K, int V, int BVH>
-__global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
+__global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu((K <= 64 && sizeof(T) == 2) ? 2 : 1))) void k_gla_bwd_dqkg(const lmoe_args a) {
   // (LDB: rows of the fp32 gate tile start on 16-byte boundaries, and the rows 4 apart that the lanes of an accumulator
   // column read fall into different banks)
   constexpr int LDV = BVH + LPAD, LDB = K + 4, LDP = CH + 1;
   constexpr int NBK = K / 16;
   // phase A (element type T): do, v, S, dS' slices.  phase B (fp32): dA, q, k, b tiles
-  constexpr int A_DO = 0, A_V = A_DO + CH * LDV, A_H = A_V + CH * LDV, A_DH = A_H + K * LDV, A_END = A_DH + K * LDV;
+  constexpr int A_DO = 0, A_V = A_DO + CH * LDV, A_H = A_V + CH * LDV, A_DH = A_H + K * LDV, A_END0 = A_DH + K * LDV;
+  // 2-byte elements: dv is formed here as well, from the do and dS' slices that phase A stages anyway and two more
+  // tiles, k e^{b_C - b} and A as k_gla_intra_fwd stored them (the chunk-parallel dv kernel, which fetched do and
+  // dS' a second time, is not run)
+  constexpr bool DV = sizeof(T) == 2;
+  constexpr int A_KE = A_END0, A_AM = A_KE + (DV ? CH * (K + LPAD) : 0), A_END = A_AM + (DV ? CH * (CH + LPAD) : 0);
   constexpr int B_DP = 0, B_Q = B_DP + CH * LDP, B_K = B_Q + CH * LDB, B_B = B_K + CH * LDB, B_END = B_B + CH * LDB;
   // Sub-chunk form of the intra-chunk sums (see k_gla_intra_fwd): between 16-token sub-chunks the
   // decay factors through the cumulative gate b* at the sub-chunk boundary,
@@ -675,6 +680,13 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
     IOH::load_nomask(x.rdh, (const T*)a.dhs + ((int64_t)cid * a.H + h) * K * V + vv, V, K);
   };
   issue_slice(sl[0], 0);
+  typedef TileIO<T, CH, CH> IOA;
+  typename IOK::Regs rke;
+  typename IOA::Regs ram;
+  if constexpr (DV) {
+    IOK::load_nomask(rke, (const T*)a.ke + ((int64_t)cid * a.H + h) * CH * K, K, CH);
+    IOA::load_nomask(ram, (const T*)a.amat + ((int64_t)cid * a.H + h) * CH * CH, CH, CH);
+  }
   auto issue_qkg = [&]() {
     IOK::load_nomask(rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
     IOK::load_nomask(rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
@@ -698,10 +710,36 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dqkg(const lmoe_args a) {
     IOV::store_lds(x.rv, smT + A_V, LDV);
     IOH::store_lds(x.rh, smT + A_H, LDV);
     IOH::store_lds(x.rdh, smT + A_DH, LDV);
+    if constexpr (DV) {
+      if (si == 0) {
+        IOK::store_lds(rke, smT + A_KE, LDK);
+        IOA::store_lds(ram, smT + A_AM, LDC);
+      }
+    }
     lds_barrier();      // LDS-only barriers: the loads requested above stay in flight
     gemm_nt<T, 1, 4, true>(dP, smT + A_DO, LDV, 16 * wv, smT + A_V, LDV, 0, 0, BVH);
     gemm_nt<T, 1, NBK, true>(dqi, smT + A_DO, LDV, 16 * wv, smT + A_H, LDV, 0, 0, BVH);
     gemm_nt<T, 1, NBK, true>(dkd, smT + A_V, LDV, 16 * wv, smT + A_DH, LDV, 0, 0, BVH);
+    if constexpr (DV) {
+      // dv^T of the slice = scale do^T A + dS'^T (k e^{b_C - b})^T, the products and the rounding of k_gla_bwd_dv
+      // (same operands, same order): a lane holds four consecutive V columns of one token, 8-byte stores
+      constexpr int NBV = BVH / 16;
+      f32x4 dv[NBV][1], dv2[NBV][1];
+      acc_zero(dv); acc_zero(dv2);
+      gemm<T, NBV, 1, true, false>(dv2, smT + A_DH, LDV, 0, smT + A_KE, LDK, 16 * wv, 0, K);
+      gemm<T, NBV, 1, true, true>(dv, smT + A_DO, LDV, 0, smT + A_AM, LDC, 16 * wv, 0, CH);
+      const int r = 16 * wv + (l & 15);
+      if (r < ci.len) {
+        T* dd = row_ptr<T>(a.dv, ci.b, ci.tok + r, h) + si * BVH + 4 * (l >> 4);
+#pragma unroll
+        for (int ni = 0; ni < NBV; ++ni) {
+          typename ET<T>::vec4 y;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) y[i] = ET<T>::from_f(__builtin_fmaf(a.scale, dv[ni][0][i], dv2[ni][0][i]));
+          *(typename ET<T>::vec4*)(dd + 16 * ni) = y;
+        }
+      }
+    }
     lds_barrier();
   }
   // per state row k: sum_v S_kv dS'_kv  (the IOH::VPR adjacent threads of a pass share a row)

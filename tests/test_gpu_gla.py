@@ -94,3 +94,35 @@ def test_gla_results_do_not_depend_on_the_width_of_the_v_slices(cuda):
     torch.cuda.synchronize()
     for a, b in zip(one, many):
         assert torch.equal(a[0], b[0]) and torch.equal(a[0], b[63])
+
+
+@pytest.mark.parametrize("B,H,T,K,V,varlen,gdt", [(2, 3, 200, 128, 128, False, torch.float32),
+                                                  (1, 4, 64, 64, 64, False, torch.bfloat16),
+                                                  (2, 2, 130, 64, 128, False, torch.bfloat16),
+                                                  (1, 2, 333, 128, 64, False, torch.float32),
+                                                  (1, 4, 700, 64, 128, True, torch.bfloat16)])
+def test_gla_dv_of_the_fused_backward_kernel_equals_the_kernel_of_its_own(cuda, B, H, T, K, V, varlen, gdt):
+    """With 2-byte elements dv is formed by the kernel that forms dq, dk and dg, from the do and dS' slices it stages
+    anyway; the chunk-parallel dv kernel (what the fp32 path runs, still reachable as a stage) forms the same products
+    in the same order: bit for bit the same dv, partial chunks and packed sequences included."""
+    import ctypes as C
+    from linear_moe_amd import _lib
+    from linear_moe_amd.gla import GLACall
+    lib = _lib.load()
+    q, k = gen(80, B, T, H, K).bfloat16().to(cuda), gen(81, B, T, H, K).bfloat16().to(cuda)
+    v, do = gen(82, B, T, H, V).bfloat16().to(cuda), gen(83, B, T, H, V).bfloat16().to(cuda)
+    g = (F.logsigmoid(gen(84, B, T, H, K)) / 16).to(gdt).to(cuda)
+    cu = torch.tensor([0, 100, 101, 450, 700], device=cuda, dtype=torch.int32) if varlen else None
+    N = 4 if varlen else B
+    h0, dht = (gen(85, N, H, K, V) * 0.3).to(cuda), gen(86, N, H, K, V).to(cuda)
+    call = GLACall(keep=True)
+    call.forward(q, k, v, g, None, h0, True, cu, False)
+    dq, dk, dv, dg, dh0 = call.backward(do, dht)
+    torch.cuda.synchronize()
+    fused = dv.clone()
+    assert fused.abs().max() > 0
+    dv.zero_()
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _lib.check(lib.lmoe_launch_stage(C.byref(call.bwd_args), call.OP, 3, st), "dv stage")      # 3: the dv kernel
+    torch.cuda.synchronize()
+    assert torch.equal(fused, dv)
