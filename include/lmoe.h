@@ -97,6 +97,11 @@ typedef struct lmoe_args {
   /* backward workspace (caller-allocated, element type = dtype) */
   void* dhs;           /* gradient w.r.t. the state at the END of every chunk, laid out as hs */
   lmoe_tensor dvnew;   /* gradient of vnew (gated delta rule): .ptr only, laid out as vnew */
+  /* packed input, optional: device int32 [N], a permutation of 0..N-1 = the order in which the sequential state passes
+   * take the sequences (their work-groups are dispatched in that order).  Longest first keeps a batch of unequal
+   * lengths from ending on one long sequence that started late; NULL = as given.  Results do not depend on it.
+   * No counterpart in fla, whose state kernels take the sequences in the order of cu_seqlens. */
+  const int32_t* seq_order;
 } lmoe_args;
 
 /* Library version (major*10000 + minor*100 + patch). */
@@ -258,9 +263,9 @@ int lmoe_mom_rowdot(const void* src, const int32_t* idx, const void* g, void* dw
  * op's fwd (stages 0-2, 7) or bwd (stages 3-5) entry point, with the intermediates of the
  * earlier stages already in place.  Stages: 0 gated-delta-rule WY preparation, 1 forward state
  * pass, 2 output, 3 dv, 4 reverse state pass, 5 dq dk and gate gradient (gated delta rule: every
- * gradient that follows the reverse state pass; chunk_simple_gla with 2-byte elements: dv as well, so that its
- * backward entry point does not run stage 3, which stays available and gives the same dv), 7 chunk_gla intra-chunk
- * matrix.
+ * gradient that follows the reverse state pass; chunk_simple_gla and chunk_gla with 2-byte elements: dv as well, so
+ * that their backward entry points do not run stage 3, which stays available and gives the same dv), 7 chunk_gla
+ * intra-chunk matrix.
  * No counterpart in the reference (measurement support). */
 #define LMOE_OP_SIMPLE_GLA 0
 #define LMOE_OP_GLA 1

@@ -148,6 +148,7 @@ class SeqPlan:
         self.cu = None
         self.chunk_map = None
         self.seq_chunk0 = None
+        self.seq_order = None
         if cu_seqlens is None:
             self.N = B
             self.NT = B * ((T + CHUNK - 1) // CHUNK)
@@ -173,6 +174,10 @@ class SeqPlan:
         self.cu = cu_host.to(torch.int32).to(device)
         self.chunk_map = cmap.to(device)
         self.seq_chunk0 = c0.to(torch.int32).to(device)
+        # the sequential passes take the longest sequences first (their work-groups are dispatched in index order): a
+        # batch of unequal lengths then does not end on a long sequence that started late
+        if self.N > 1 and int(nch.max()) != int(nch.min()):
+            self.seq_order = torch.argsort(nch, descending=True, stable=True).to(torch.int32).to(device)
 
 
 # Plans of the cu_seqlens tensors seen last, newest first.  An entry holds the tensor itself (so its address cannot be
@@ -224,6 +229,7 @@ def base_args(q, k, v, head_first: bool, scale: Optional[float], plan: SeqPlan, 
         a.cu_seqlens = plan.cu.data_ptr()
         a.chunk_map = plan.chunk_map.data_ptr()
         a.seq_chunk0 = plan.seq_chunk0.data_ptr()
+        a.seq_order = ptr(plan.seq_order)
     a.q, a.k, a.v = _desc(q, head_first), _desc(k, head_first), _desc(v, head_first)
     return a
 

@@ -38,6 +38,7 @@ class Args(C.Structure):
         ("dq", Tensor4), ("dk", Tensor4), ("dv", Tensor4), ("dg", Tensor4), ("dbeta", Tensor4),
         ("dh0", C.c_void_p),
         ("dhs", C.c_void_p), ("dvnew", Tensor4),
+        ("seq_order", C.c_void_p),
     ]
 
 

@@ -307,7 +307,7 @@ __global__ __launch_bounds__(NTHR) void k_gla_state_fwd(const lmoe_args a) {
   const int xcd = blockIdx.x & 7, jj = blockIdx.x >> 3;
   const int pair = (jj / NVS) * 8 + xcd;
   if (pair >= a.N * a.H) return;
-  const int v0 = (jj % NVS) * BV, h = pair % a.H, n = pair / a.H;
+  const int v0 = (jj % NVS) * BV, h = pair % a.H, n = seq_at(a, pair / a.H);
   const SeqInfo sq = seq_info(a, n);
   const int wv = wave_id();
   const int krow0 = wv * (K / 4);
@@ -469,7 +469,7 @@ __global__ __launch_bounds__(NTHR) void k_gla_state_bwd(const lmoe_args a) {
   const int xcd = blockIdx.x & 7, jj = blockIdx.x >> 3;
   const int pair = (jj / NVS) * 8 + xcd;
   if (pair >= a.N * a.H) return;
-  const int v0 = (jj % NVS) * BV, h = pair % a.H, n = pair / a.H;
+  const int v0 = (jj % NVS) * BV, h = pair % a.H, n = seq_at(a, pair / a.H);
   const SeqInfo sq = seq_info(a, n);
   const int wv = wave_id();
   const int krow0 = wv * (K / 4);
@@ -618,7 +618,7 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dv(const lmoe_args a) {
 }
 
 // ------------------------------------------------------------------------- //
-// dq, dk, dg, grid = (NT, H)
+// dq, dk, dg (2-byte elements: dv as well), grid = (NT, H)
 // ------------------------------------------------------------------------- //
 template <typename T, typename GT, int K, int V, int BVH>
 __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu((K <= 64 && sizeof(T) == 2) ? 2 : 1))) void k_gla_bwd_dqkg(const lmoe_args a) {

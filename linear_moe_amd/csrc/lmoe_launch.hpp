@@ -11,7 +11,7 @@ enum Stage {
   ST_GDN_WY_FWD = 0,   // gated delta rule: w, u, Tinv, P                (chunk-parallel)
   ST_STATE_FWD = 1,    // sequential state pass: hs (, vnew), ht; scalar gates: also the output o
   ST_OUT_FWD = 2,      // chunk_gla: output o                            (chunk-parallel)
-  ST_DV = 3,           // dv (gla; simple_gla: fp32 only, ST_DQK forms it for 2-byte elements) (chunk-parallel)
+  ST_DV = 3,           // dv (simple_gla / gla; the backward entry points run it for fp32 only: ST_DQK forms dv for 2-byte elements)
   ST_STATE_BWD = 4,    // reverse sequential state pass: dhs (, dv_new), dh0
   ST_DQK = 5,          // dq, dk, gate gradient; gated delta rule: every gradient that follows the
                        // reverse state pass (dq, dk, dv, dbeta, dg)     (chunk-parallel)

@@ -53,7 +53,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
   const int xcd = blockIdx.x & 7, jj = blockIdx.x >> 3;
   const int vsl = jj % NVS, pair = (jj / NVS) * 8 + xcd;
   if (pair >= a.N * a.H) return;
-  const int v0 = vsl * BV, h = pair % a.H, n = pair / a.H;
+  const int v0 = vsl * BV, h = pair % a.H, n = seq_at(a, pair / a.H);
   const SeqInfo sq = seq_info(a, n);
   const int l = lane_id();
   const int team = threadIdx.x / NTHR;
@@ -313,7 +313,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd_b(const lmoe_args a, lon
   const int xcd = blockIdx.x & 7, jj = blockIdx.x >> 3;
   const int vsl = jj % NVS, pair = (jj / NVS) * 8 + xcd;
   if (pair >= a.N * a.H) return;
-  const int v0 = vsl * BV, h = pair % a.H, n = pair / a.H;
+  const int v0 = vsl * BV, h = pair % a.H, n = seq_at(a, pair / a.H);
   const SeqInfo sq = seq_info(a, n);
   const int l = lane_id();
   // (wave-uniform by construction; said to the compiler, so that the branches on it are scalar branches: a matrix

@@ -36,6 +36,13 @@ __device__ __forceinline__ SeqInfo seq_info(const lmoe_args& a, int n) {
   return s;
 }
 
+// The i-th sequence a sequential pass takes: work-groups are dispatched in the order of their index, so a packed
+// batch of unequal lengths runs its longest sequences first when the caller passes such an order (seq_order; NULL =
+// as given).  Which work-group computes a (sequence, head, slice) does not change what it computes.
+__device__ __forceinline__ int seq_at(const lmoe_args& a, int i) {
+  return a.seq_order ? as_const(a.seq_order)[i] : i;
+}
+
 struct ChunkInfo {
   int n;       // sequence
   int b;       // batch row

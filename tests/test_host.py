@@ -129,6 +129,9 @@ def test_seq_plan_tables():
     assert p.seq_chunk0.tolist() == [0, 1, 2, 5, 7, 7]
     assert p.chunk_map.tolist() == [[0, 0], [1, 0], [2, 0], [2, 1], [2, 2], [3, 0], [3, 1]]
     assert p.cu.dtype == torch.int32
+    # the order in which the sequential passes take the sequences: by number of chunks, longest first, ties as given
+    assert p.seq_order.dtype == torch.int32 and p.seq_order.tolist() == [2, 3, 0, 1, 4]
+    assert SeqPlan(1, 256, torch.tensor([0, 64, 128, 256 - 64, 256]), "cpu").seq_order is None      # equal lengths
     for bad in ([1, 5, 270], [0, 50, 40, 270], [0, 100]):
         with pytest.raises(ValueError):
             SeqPlan(1, 270, torch.tensor(bad), "cpu")
