@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Build-time guard of the register-steered kernels.
 
-The hot kernels of the gated delta rule and the forward pass of chunk_simple_gla rely on the compiler keeping their working set in registers (explicit
+The hot kernels of the gated delta rule and the forward pass and the fused backward kernel of chunk_simple_gla rely on the compiler keeping their working set in registers (explicit
 steering: refreshed lane indices, pinned sums, fenced products).  A compiler or source change that makes one of them
 spill, or lowers the number of waves it runs with, costs a large factor in speed without failing any test.  This
 script reads the per-kernel resource reports that ``-Rpass-analysis=kernel-resource-usage`` wrote at compile time
@@ -24,6 +24,7 @@ GUARDED = {
     "k_gdn_state_bwd": 3,
     "k_gdn_bwd_chunk": 3,
     "k_gdn_wy_fwd": 2,
+    "k_bwd_dqkv": 2,          # one work-group of 8 waves per CU; its first version spilled loop-invariant lane arithmetic
 }
 FIELDS = {"ScratchSize [bytes/lane]": "scratch", "VGPRs Spill": "vspill", "Occupancy [waves/SIMD]": "occ",
           "VGPRs": "vgpr", "AGPRs": "agpr", "LDS Size [bytes/block]": "lds"}
