@@ -229,3 +229,37 @@ def test_a_sequence_gives_the_same_bits_alone_and_inside_a_large_packed_batch(cu
     for i, (a, b) in enumerate(zip(packed, alone)):
         a = a[s:s + 1] if i in per_seq else a[:, sl]
         assert torch.equal(a, b), labels[i]
+
+
+@pytest.mark.parametrize("op", OPS)
+def test_the_order_in_which_the_passes_take_the_sequences_does_not_show(cuda, op):
+    """The plan of a packed batch of unequal lengths lists the sequences longest first and the sequential passes take
+    them in that order (their work-groups are dispatched by index): which work-group computes a sequence must not
+    change what it computes.  Same call with the order as planned and with the order taken away: the same bits."""
+    from linear_moe_amd import _host
+    lens = [70, 300, 1, 64, 129, 500, 33]
+    T, N, H, K, V = sum(lens), len(lens), 5, 64, 128
+    ins = {n: x.to(cuda) for n, x in _inputs(op, T, H, K, V, torch.bfloat16, 3400).items()}
+    h0 = (gen(3410, N, H, K, V) * 0.1).to(cuda)
+    do, dht = gen(3411, 1, T, H, V, dtype=torch.bfloat16).to(cuda), gen(3412, N, H, K, V).to(cuda)
+    cu = torch.tensor([0] + lens, dtype=torch.int32).cumsum(0).to(torch.int32).to(cuda)
+    names = list(ins)
+
+    def run():
+        leaves = {n: x.clone().requires_grad_(True) for n, x in dict(ins, h0=h0).items()}
+        o, ht = _call(op, leaves, leaves["h0"], cu, True)
+        grads = torch.autograd.grad([o, ht], [leaves[n] for n in names + ["h0"]], [do, dht])
+        return (o.detach(), ht.detach()) + tuple(grads)
+
+    plan = _host.prepare_cu_seqlens(cu, T)
+    order = plan.seq_order
+    assert order is not None and order.tolist()[:2] == [5, 1]
+    try:
+        planned = run()
+        plan.seq_order = None
+        as_given = run()
+    finally:
+        plan.seq_order = order
+    torch.cuda.synchronize()
+    for a, b in zip(planned, as_given):
+        assert torch.equal(a, b)
