@@ -264,8 +264,9 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
 //              the barrier, stored from registers, then the q rows and v fragments of chunk c + 1 and, from those q
 //              rows, the diagonal blocks of P of chunk c + 1
 // A chunk's own operands are staged two windows before its window: what is read of them is read at the end of the
-// window before, when the LDS is quiet, and their buffer is free for the chunk after the next one as the window opens.  Behind the barrier, where all twelve waves ask for data at once and a read
-// takes about a thousand cycles to return, only S^T and P (written in the window before) are left to read.
+// window before, when the LDS is quiet, and their buffer is free for the chunk after the next one as the window
+// opens.  Behind the barrier, where all twelve waves ask for data at once and a read takes about a thousand cycles
+// to return, only S^T and P (written in the window before) are left to read.
 // Time stamps of the traced instance (TRACE = true): one wave of each team notes the shader clock where it arrives
 // at and leaves the barrier of a chunk and at a few points in between; the stamps sit in LDS (a global store
 // per stamp would perturb the wave that is measured) and each of those waves copies its own out at the end:
@@ -285,7 +286,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd_b(const lmoe_args a, lon
   __shared__ __attribute__((aligned(16))) T s_P[2][CH * LDC];                 // P             [64][64]
   __shared__ __attribute__((aligned(16))) float s_b[2][64], s_eb[2][64], s_ed[2][64];
   __shared__ float s_dec[2];                                                  // e^{b_C} per buffer
-  // (the low 32 bits of the clock: the LDS has no room for more beside the buffers of the pass)
+  // (the low 32 bits of the clock: whoever reads the stamps takes their differences modulo 2^32)
   __shared__ uint32_t s_tr[TRACE ? SFWD_TRACE_SLOTS * SFWD_TRACE_CHUNKS * SFWD_TRACE_MARKS : 1];
   auto TR = [&](int slot, int c, int mark) {
     if constexpr (TRACE) {
