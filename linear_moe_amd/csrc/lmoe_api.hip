@@ -90,24 +90,27 @@ int lmoe_chunk_simple_gla_bwd(const lmoe_args* a, void* stream) {
   lmoe::launch_bwd_dqk(*a, (hipStream_t)stream);
   return launched(op);
 }
-static int check_gla(const lmoe_args* a, const char* op) {
+static int check_gla(const lmoe_args* a, const char* op, bool need_hs = true) {
   if (int r = check_common(a, op)) return r;
   if (a->gate != LMOE_GATE_VECTOR || !a->g.ptr) return fail(-10, "%s: needs a vector gate g [B,T,H,K]", op);
   if (a->dtype == LMOE_F32 && a->g_dtype != LMOE_F32) return fail(-14, "%s: fp32 q/k/v need an fp32 gate", op);
-  if (!a->hs || !a->amat || !a->qe || !a->ke || !a->gcum)
+  if ((need_hs && !a->hs) || !a->amat || !a->qe || !a->ke || !a->gcum)
     return fail(-11, "%s: hs, amat, qe, ke and gcum must not be null", op);
   return 0;
 }
 
 int lmoe_chunk_gla_fwd(const lmoe_args* a, void* stream) {
   const char* op = "lmoe_chunk_gla_fwd";
-  if (int r = check_gla(a, op)) return r;
+  // hs == NULL: a forward-only call, nothing saved -- where the state pass forms the output itself (2-byte
+  // elements, K = 64); the other instances hand the states to their output kernel through hs
+  if (int r = check_gla(a, op, false)) return r;
+  if (!a->hs && !lmoe::gla_fwd_fused(*a)) return fail(-11, "%s: hs must not be null for this dtype / K", op);
   if (!a->o.ptr) return fail(-11, "%s: o must not be null", op);
   if (a->NT == 0 || a->N == 0) return 0;
   hipStream_t st = (hipStream_t)stream;
   lmoe::launch_gla(*a, lmoe::ST_GLA_INTRA_FWD, st);
   lmoe::launch_gla(*a, lmoe::ST_STATE_FWD, st);
-  lmoe::launch_gla(*a, lmoe::ST_OUT_FWD, st);
+  if (!lmoe::gla_fwd_fused(*a)) lmoe::launch_gla(*a, lmoe::ST_OUT_FWD, st);      // else the state pass formed o
   return launched(op);
 }
 

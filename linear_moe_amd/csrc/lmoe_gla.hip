@@ -23,6 +23,21 @@ static void launch_gla_t(const lmoe_args& a, int stage, hipStream_t st) {
     case ST_GLA_INTRA_FWD:
       hipLaunchKernelGGL((k_gla_intra_fwd<T, GT, K>), dim3(persistent_grid(a.NT * a.H, 2)), block, 0, st, a); break;
     case ST_STATE_FWD:
+      if constexpr (sizeof(T) == 2 && K == 64) {
+        // 2-byte elements, K = 64: the pass that holds the state also forms the output (k_gla_fwd_fused; at K = 128
+        // its loaders' three register sets do not fit beside the other teams' registers); hs == NULL: nothing saved
+        const int pairs8 = (a.N * a.H + 7) / 8 * 8;
+        if constexpr (Tl::BVS_WIDE != Tl::BVS) {
+          if (wide) {
+            if (a.hs) hipLaunchKernelGGL((k_gla_fwd_fused<T, K, V, Tl::BVS_WIDE, true>), dim3(pairs8 * (V / Tl::BVS_WIDE)), dim3(3 * NTHR), 0, st, a);
+            else hipLaunchKernelGGL((k_gla_fwd_fused<T, K, V, Tl::BVS_WIDE, false>), dim3(pairs8 * (V / Tl::BVS_WIDE)), dim3(3 * NTHR), 0, st, a);
+            break;
+          }
+        }
+        if (a.hs) hipLaunchKernelGGL((k_gla_fwd_fused<T, K, V, Tl::BVS, true>), dim3(pairs8 * (V / Tl::BVS)), dim3(3 * NTHR), 0, st, a);
+        else hipLaunchKernelGGL((k_gla_fwd_fused<T, K, V, Tl::BVS, false>), dim3(pairs8 * (V / Tl::BVS)), dim3(3 * NTHR), 0, st, a);
+        break;
+      }
       if (wide) hipLaunchKernelGGL((k_gla_state_fwd<T, GT, K, V, Tl::BVS_WIDE>), dim3((a.N * a.H + 7) / 8 * 8 * (V / Tl::BVS_WIDE)), block, 0, st, a);
       else hipLaunchKernelGGL((k_gla_state_fwd<T, GT, K, V, Tl::BVS>), dim3((a.N * a.H + 7) / 8 * 8 * (V / Tl::BVS)), block, 0, st, a);
       break;
@@ -47,6 +62,9 @@ static void launch_gla_kv(const lmoe_args& a, int stage, hipStream_t st) {
   else if (a.K == 128 && a.V == 64) launch_gla_t<T, GT, 128, 64>(a, stage, st);
   else launch_gla_t<T, GT, 128, 128>(a, stage, st);
 }
+
+// whether the forward state pass of this problem also forms the output (then ST_OUT_FWD is not part of the forward)
+bool gla_fwd_fused(const lmoe_args& a) { return a.dtype == LMOE_BF16 && a.K == 64; }
 
 // (dtype, g_dtype) must be (bf16, bf16), (bf16, f32) or (f32, f32): checked by the caller
 void launch_gla(const lmoe_args& a, int stage, hipStream_t st) {

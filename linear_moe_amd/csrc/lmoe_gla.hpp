@@ -393,6 +393,253 @@ __global__ __launch_bounds__(NTHR) void k_gla_state_fwd(const lmoe_args a) {
 }
 
 // ------------------------------------------------------------------------- //
+// forward state pass AND output in one kernel (2-byte elements), 1-D grid as k_gla_state_fwd, 768 threads.
+// The three-team, one-barrier-per-chunk design of the scalar-gate forward pass (k_state_fwd_b, lmoe_scalar_fwd.hpp)
+// on the operands k_gla_intra_fwd stored: q e^{b}, k e^{b_C - b}, the intra-chunk matrix A and the chunk decay
+// e^{b_C}, so that the pass needs no gate, no exponential and forms no P.  The output leaves the kernel that holds the
+// state: S is not read back from memory by a kernel of its own (k_gla_out_fwd fetched hs, q e^{b}, A and v again).
+//   consumers (waves 0-3):  S = diag(e^{b_C}) S + (k e^{b_C - b})^T v in fp32 accumulators (wave w: K rows K/4 w ..),
+//                           S^T of the next chunk -> s_hT, then the fragments of the next update
+//   loaders   (waves 4-7):  three register sets of (k~, q~, v, A, decay), chunk c + 2 staged into the buffer of
+//                           chunk c as window c opens; with SAVE hs[chunk] <- S (layout [K][V]) through transposing
+//                           reads of s_hT: a lane holds eight consecutive V columns of one K row, 16-byte stores
+//   output    (waves 8-11): rows 16 w .. of o^T = S^T q~^T + v^T A^T in one accumulator (the products, their order
+//                           and the rounding of k_gla_out_fwd: the same bits), stored from registers
+// Two buffers of every tile: what a window reads of a chunk's own operands was read into registers at the end of the
+// window before (see k_state_fwd_b).
+// ------------------------------------------------------------------------- //
+template <typename T, int K, int V, int BV, bool SAVE>
+__global__ __launch_bounds__(3 * NTHR) void k_gla_fwd_fused(const lmoe_args a) {
+  static_assert(sizeof(T) == 2, "2-byte elements");
+  constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDU = BV + LPAD;
+  constexpr int MB = K / 64, NB = BV / 16, KS = K / 32, CS = CH / 32;
+  __shared__ __attribute__((aligned(16))) T s_k[2][CH * LDK];                 // k e^{b_C - b}  [64][K]
+  __shared__ __attribute__((aligned(16))) T s_q[2][CH * LDK];                 // q e^{b}        [64][K]
+  __shared__ __attribute__((aligned(16))) T s_u[2][CH * LDU];                 // v              [64][BV]
+  __shared__ __attribute__((aligned(16))) T s_hT[2][BV * LDK];                // S^T            [BV][K]
+  __shared__ __attribute__((aligned(16))) T s_P[2][CH * LDC];                 // A              [64][64]
+  __shared__ __attribute__((aligned(16))) float s_dec[2][K];                  // e^{b_C}        [K]
+
+  constexpr int NVS = V / BV;
+  const int xcd = blockIdx.x & 7, jj = blockIdx.x >> 3;
+  const int pair = (jj / NVS) * 8 + xcd;
+  if (pair >= a.N * a.H) return;
+  const int v0 = (jj % NVS) * BV, h = pair % a.H, n = seq_at(a, pair / a.H);
+  const SeqInfo sq = seq_info(a, n);
+  const int l = lane_id();
+  // (wave-uniform by construction; said to the compiler, so that the branches on it are scalar branches: a matrix
+  // instruction runs whatever the lane mask, and a short masked region is not jumped over)
+  const int wave = __builtin_amdgcn_readfirstlane(wave_id());
+  const int team = wave >> 2;
+  if (sq.nchunks == 0) {
+    // empty sequence: the final state is the initial state
+    if (a.ht && team == 0) {
+      for (int idx = threadIdx.x; idx < K * BV; idx += NTHR) {
+        const int r = idx / BV, c = v0 + idx % BV;
+        const int64_t o = ((int64_t)n * a.H + h) * K * V + (int64_t)r * V + c;
+        a.ht[o] = a.h0 ? a.h0[o] : 0.f;
+      }
+    }
+    return;
+  }
+  typedef TileIO<T, CH, K> IOK;
+  typedef TileIO<T, CH, BV> IOV;
+  typedef TileIO<T, CH, CH> IOA;
+
+  if (team == 1) {
+    // --------------------------------- loaders -------------------------------------------
+    const int tid = threadIdx.x & (NTHR - 1);
+    struct Pre { typename IOK::Regs rk, rq; typename IOV::Regs ru; typename IOA::Regs ra; float dec; int len; };
+    Pre pre[3];                                              // register set = chunk % 3
+    // Always issued (chunk index clamped to the last chunk; the surplus loads at the end of a sequence are never
+    // consumed): a prefetch that is skipped on some path would make the compiler drain all outstanding loads at
+    // every consumer of a register set.
+    auto issue = [&](Pre& P, int c) {
+      c = min(c, sq.nchunks - 1);
+      const int64_t item = (int64_t)(sq.chunk0 + c) * a.H + h;
+      const int len = min(CH, sq.len - c * CH);
+      IOK::load_nomask(P.rk, (const T*)a.ke + item * CH * K, K, CH);
+      IOK::load_nomask(P.rq, (const T*)a.qe + item * CH * K, K, CH);
+      IOV::load_nomask(P.ru, row_ptr<T>(a.v, sq.b, sq.tok0 + c * CH, h) + v0, a.v.st, len);
+      IOA::load_nomask(P.ra, (const T*)a.amat + item * CH * CH, CH, CH);
+      P.dec = a.gcum[item * K + min(tid, K - 1)];
+      P.len = len;
+    };
+    // registers -> LDS buffer `buf`
+    auto stage = [&](Pre& P, int buf) {
+      IOV::mask(P.ru, P.len);
+      IOK::store_lds(P.rk, s_k[buf], LDK);
+      IOK::store_lds(P.rq, s_q[buf], LDK);
+      IOV::store_lds(P.ru, s_u[buf], LDU);
+      IOA::store_lds(P.ra, s_P[buf], LDC);
+      if (tid < K) s_dec[buf][tid] = P.dec;
+    };
+    // hs[chunk][h][K][v0 .. v0+BV] <- S (only the backward reads it: SAVE = false for forward-only calls): S^T read
+    // through the transposing LDS read, lane (c, g): K row 16 kb + c, V columns 32 vb + 8 g .. + 7
+    auto save_state = [&](int c) {
+      if constexpr (SAVE) {
+        T* hs = (T*)a.hs + ((int64_t)(sq.chunk0 + c) * a.H + h) * K * V + v0;
+#pragma unroll
+        for (int kb = 0; kb < K / 64; ++kb)
+#pragma unroll
+          for (int vb = 0; vb < BV / 32; ++vb) {
+            const int k0 = 16 * (4 * kb + (wave - 4));
+            const typename ET<T>::frag x = ET<T>::load_frag_t(s_hT[c & 1], LDK, 32 * vb, k0, l);
+            *(typename ET<T>::vec*)(hs + (int64_t)(k0 + (l & 15)) * V + 32 * vb + 8 * (l >> 4)) = x;
+          }
+      }
+    };
+#pragma unroll
+    for (int j = 0; j < 3; ++j) issue(pre[j], j);
+    stage(pre[0], 0);
+    issue(pre[0], 3);
+    stage(pre[1], 1);
+    lds_barrier();                                                                       // chunks 0, 1 staged
+    for (int c0 = 0; c0 < sq.nchunks; c0 += 3) {
+#pragma unroll
+      for (int j = 0; j < 3; ++j) {
+        const int c = c0 + j;
+        if (c >= sq.nchunks) break;
+        lds_barrier();
+        // (both always: past the end it is the last chunk again, never consumed)
+        issue(pre[(j + 1) % 3], c + 4);
+        stage(pre[(j + 2) % 3], c & 1);          // chunk c + 2 takes the buffers of chunk c
+        save_state(c);
+      }
+    }
+    return;
+  }
+
+  if (team == 2) {
+    // --------------------------------- output --------------------------------------------
+    const int ow = wave - 8;
+    const int fr = l & 15, fg = 8 * (l >> 4), g4 = 4 * (l >> 4);
+    lds_barrier();                                                                       // chunks 0, 1 staged
+    typename ET<T>::frag fq[KS], fv[CS][NB], fp[CS];
+    auto preread = [&](int c) {
+      const int cb = c & 1;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) fq[ks] = ET<T>::load_frag(s_q[cb] + (16 * ow + fr) * LDK + 32 * ks + fg);
+#pragma unroll
+      for (int kq = 0; kq < CS; ++kq) {
+        if (2 * kq <= ow) {          // tokens j >= 32 only reach the rows of waves 2, 3 (A is lower triangular)
+#pragma unroll
+          for (int ni = 0; ni < NB; ++ni) fv[kq][ni] = ET<T>::load_frag_t(s_u[cb], LDU, 32 * kq, 16 * ni, l);
+          fp[kq] = ET<T>::load_frag(s_P[cb] + (16 * ow + fr) * LDC + 32 * kq + fg);
+        }
+      }
+    };
+    preread(0);
+    for (int c = 0; c < sq.nchunks; ++c) {
+      const int tok = sq.tok0 + c * CH;
+      const int len = min(CH, sq.len - c * CH);
+      lds_barrier();
+      typename ET<T>::frag fh[KS][NB];
+      const T* hT = s_hT[c & 1];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) fh[ks][ni] = ET<T>::load_frag(hT + (16 * ni + fr) * LDK + 32 * ks + fg);
+      __builtin_amdgcn_sched_barrier(0);
+      f32x4 o[NB];
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) o[ni] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) ET<T>::mma(o[ni], fh[ks][ni], fq[ks]);            // (q~ S)^T: column x token
+#pragma unroll
+      for (int kq = 0; kq < CS; ++kq) {
+        if (2 * kq <= ow) {
+#pragma unroll
+          for (int ni = 0; ni < NB; ++ni) ET<T>::mma(o[ni], fv[kq][ni], fp[kq]);           // + (A v)^T
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      // lane: token 16 ow + fr, columns 16 ni + g4 .. + 3
+      if (16 * ow + fr < len) {
+        T* orow = row_ptr<T>(a.o, sq.b, tok + 16 * ow + fr, h) + v0 + g4;
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) {
+          typename ET<T>::vec4 y;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) y[e] = ET<T>::from_f(o[ni][e] * a.scale);
+          *(typename ET<T>::vec4*)(orow + 16 * ni) = y;
+        }
+      }
+      if (c + 1 < sq.nchunks) preread(c + 1);
+    }
+    return;
+  }
+
+  // --------------------------------- consumers -------------------------------------------
+  const int wv = wave;
+  const int krow0 = wv * (K / 4);
+  f32x4 S[MB][NB];
+  acc_zero(S);
+  if (a.h0) {
+    const float* h0 = a.h0 + ((int64_t)n * a.H + h) * K * V;
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) S[mi][ni][i] = h0[(int64_t)(krow0 + acc_row(mi, i)) * V + v0 + acc_col(ni)];
+  }
+  auto copy_state = [&](int buf) {          // S -> LDS as S^T
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) acc_to_lds_t<T>(S[mi][ni], s_hT[buf], LDK, krow0 + 16 * mi, 16 * ni);
+  };
+  copy_state(0);
+  lds_barrier();                                                                         // chunks 0, 1 staged
+  typename ET<T>::frag af[CS][MB], bf[CS][NB];
+  f32x4 dec[MB];
+  auto preread = [&](int c) {
+    const int cb = c & 1;
+#pragma unroll
+    for (int kq = 0; kq < CS; ++kq) {
+#pragma unroll
+      for (int mi = 0; mi < MB; ++mi) af[kq][mi] = ET<T>::load_frag_t(s_k[cb], LDK, 32 * kq, krow0 + 16 * mi);
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) bf[kq][ni] = ET<T>::load_frag_t(s_u[cb], LDU, 32 * kq, 16 * ni);
+    }
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi) dec[mi] = *(const f32x4*)&s_dec[cb][krow0 + 16 * mi + 4 * (l >> 4)];
+  };
+  preread(0);
+  for (int c = 0; c < sq.nchunks; ++c) {
+    lds_barrier();
+    // S = diag(e^{b_C}) S + (k e^{b_C - b})^T v
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) S[mi][ni] *= dec[mi];
+#pragma unroll
+    for (int kq = 0; kq < CS; ++kq)
+#pragma unroll
+      for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) ET<T>::mma(S[mi][ni], af[kq][mi], bf[kq][ni]);
+    __builtin_amdgcn_sched_barrier(0);
+    if (c + 1 < sq.nchunks) {
+      copy_state((c + 1) & 1);
+      preread(c + 1);
+    }
+  }
+  if (a.ht) {
+    float* ht = a.ht + ((int64_t)n * a.H + h) * K * V;
+#pragma unroll
+    for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ht[(int64_t)(krow0 + acc_row(mi, i)) * V + v0 + acc_col(ni)] = S[mi][ni][i];
+  }
+}
+
+// ------------------------------------------------------------------------- //
 // output, grid = (NT, H, V / BV)
 // ------------------------------------------------------------------------- //
 template <typename T, typename GT, int K, int V, int BV>

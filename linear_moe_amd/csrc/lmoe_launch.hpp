@@ -46,6 +46,8 @@ void launch_gdn_bwd_chunk(const lmoe_args& a, hipStream_t st);    // gated delta
 // chunk_gla: one kernel of the pipeline (stage = ST_GLA_INTRA_FWD, ST_STATE_FWD, ST_OUT_FWD,
 // ST_STATE_BWD, ST_DV, ST_DQK)
 void launch_gla(const lmoe_args& a, int stage, hipStream_t st);
+// whether ST_STATE_FWD of this problem also forms the output o (then the forward does not run ST_OUT_FWD)
+bool gla_fwd_fused(const lmoe_args& a);
 // row-wise L2 normalisation of `rows` contiguous rows of D in {64, 128, 256} elements (bwd: out = dx)
 void launch_l2norm(int dtype, int D, const void* x, const void* dy, void* out, int64_t rows, float eps, bool bwd,
                    hipStream_t st);

@@ -31,7 +31,9 @@ class GLACall:
         a.g = _desc(g, head_first)
         a.g_dtype = _lib.LMOE_F32 if g.dtype == torch.float32 else _lib.LMOE_BF16
 
-    def forward(self, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first):
+    def forward(self, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first, save=True):
+        """save=False: a forward-only call (nothing requires a gradient): the per-chunk states are not written where
+        the state pass forms the output itself (bf16, K = 64); elsewhere the output kernel reads them."""
         lib = _lib.load()
         dims = _check_inputs(q, k, v, head_first, cu_seqlens)
         B, T, H, K, V = dims
@@ -49,13 +51,14 @@ class GLACall:
         dev, dt = q.device, q.dtype
         o = torch.empty_like(v)
         ht = torch.empty(plan.N, H, K, V, dtype=torch.float32, device=dev) if output_final_state else None
-        hs = torch.empty(max(plan.NT, 1), H, K, V, dtype=dt, device=dev)
+        fused = dt == torch.bfloat16 and K == 64
+        hs = torch.empty(max(plan.NT, 1), H, K, V, dtype=dt, device=dev) if (save or not fused) else None
         amat = torch.empty(max(plan.NT, 1), H, 64, 64, dtype=dt, device=dev)
         # gated operands of the state passes (q e^b, k e^{b_C - b}, e^{b_C}), formed once per chunk
         qe = torch.empty(max(plan.NT, 1), H, 64, K, dtype=dt, device=dev)
         ke = torch.empty_like(qe)
         gdec = torch.empty(max(plan.NT, 1), H, K, dtype=torch.float32, device=dev)
-        a.o, a.ht, a.hs, a.amat = _desc(o, head_first), ptr(ht), hs.data_ptr(), amat.data_ptr()
+        a.o, a.ht, a.hs, a.amat = _desc(o, head_first), ptr(ht), ptr(hs), amat.data_ptr()
         a.qe, a.ke, a.gcum = qe.data_ptr(), ke.data_ptr(), gdec.data_ptr()
         _lib.check(lib.lmoe_chunk_gla_fwd(C.byref(a), stream_ptr()), "chunk_gla forward")
         self.saved = (q, k, v, g, h0, hs, amat, qe, ke, gdec)
@@ -94,7 +97,8 @@ class _ChunkGLA(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first):
         call = GLACall()
-        o, ht = call.forward(q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first)
+        o, ht = call.forward(q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first,
+                             save=any(ctx.needs_input_grad))
         ctx.call, ctx.g_dtype = call, g.dtype
         return o, ht
 

@@ -126,3 +126,48 @@ def test_gla_dv_of_the_fused_backward_kernel_equals_the_kernel_of_its_own(cuda, 
     _lib.check(lib.lmoe_launch_stage(C.byref(call.bwd_args), call.OP, 3, st), "dv stage")      # 3: the dv kernel
     torch.cuda.synchronize()
     assert torch.equal(fused, dv)
+
+
+@pytest.mark.parametrize("B,H,T,K,V,varlen", [(2, 3, 200, 64, 128, False), (1, 4, 64, 64, 64, False),
+                                              (64, 4, 130, 64, 128, False), (1, 4, 700, 64, 128, True)])
+def test_gla_output_of_the_fused_forward_pass_equals_the_output_kernel(cuda, B, H, T, K, V, varlen):
+    """With 2-byte elements and K = 64 the forward state pass forms the output as well (three teams, one barrier per
+    chunk, the state never read back); the chunk-parallel output kernel (what the other instances run, still
+    reachable as a stage) forms the same products in the same order from the per-chunk states the pass has saved:
+    bit for bit the same o — narrow and wide V slices (the batch of 64), partial chunks, packed sequences."""
+    import ctypes as C
+    from linear_moe_amd import _lib
+    from linear_moe_amd.gla import GLACall
+    lib = _lib.load()
+    q, k = gen(90, B, T, H, K).bfloat16().to(cuda), gen(91, B, T, H, K).bfloat16().to(cuda)
+    v = gen(92, B, T, H, V).bfloat16().to(cuda)
+    g = (F.logsigmoid(gen(93, B, T, H, K)) / 16).bfloat16().to(cuda)
+    cu = torch.tensor([0, 100, 101, 450, 700], device=cuda, dtype=torch.int32) if varlen else None
+    N = 4 if varlen else B
+    h0 = (gen(94, N, H, K, V) * 0.3).to(cuda)
+    call = GLACall(keep=True)
+    o, ht = call.forward(q, k, v, g, None, h0, True, cu, False)
+    torch.cuda.synchronize()
+    fused = o.clone()
+    assert fused.abs().max() > 0
+    o.zero_()
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _lib.check(lib.lmoe_launch_stage(C.byref(call.fwd_args), call.OP, 2, st), "output stage")   # 2: the output kernel
+    torch.cuda.synchronize()
+    assert torch.equal(fused, o)
+
+
+def test_gla_forward_only_call_equals_the_saving_call(cuda):
+    """Nothing requires a gradient: the per-chunk states are neither allocated nor written (bf16, K = 64: the state
+    pass forms the output itself); the output and the final state are those of the call that saves them."""
+    from linear_moe_amd import chunk_gla
+    B, H, T, K, V = 2, 4, 300, 64, 128
+    q, k = gen(95, B, T, H, K).bfloat16().to(cuda), gen(96, B, T, H, K).bfloat16().to(cuda)
+    v = gen(97, B, T, H, V).bfloat16().to(cuda)
+    g = (F.logsigmoid(gen(98, B, T, H, K)) / 16).bfloat16().to(cuda)
+    h0 = (gen(99, B, H, K, V) * 0.3).to(cuda)
+    with torch.no_grad():
+        o1, ht1 = chunk_gla(q, k, v, g, None, h0, True, None, False)
+    o2, ht2 = chunk_gla(q.clone().requires_grad_(True), k, v, g, None, h0, True, None, False)
+    torch.cuda.synchronize()
+    assert torch.equal(o1, o2.detach()) and torch.equal(ht1, ht2.detach())
