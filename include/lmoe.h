@@ -135,8 +135,8 @@ int lmoe_chunk_simple_gla_bwd(const lmoe_args* a, void* stream);
  *   linear_moe/sequence_modeling/gla/gla.py:94 and linear_moe/sequence_modeling/hgrn2/hgrn2.py:76.
  * fwd uses q,k,v,g,h0 -> o,ht,hs,amat,qe,ke,gcum (the gated operands of the state passes, formed once by
  * the chunk-parallel kernel).  bwd uses those + d_o,dht -> dq,dk,dv,dg,dh0 (+ dhs).  hs, which only the backward
- * reads where the forward state pass forms the output itself (2-byte elements with K = 64), may be NULL there (a
- * forward-only call: nothing saved); the other instances hand the states to their output kernel through it. */
+ * reads where the forward state pass forms the output itself (2-byte elements), may be NULL there (a forward-only
+ * call: nothing saved); the 4-byte instances hand the states to their output kernel through it. */
 int lmoe_chunk_gla_fwd(const lmoe_args* a, void* stream);
 int lmoe_chunk_gla_bwd(const lmoe_args* a, void* stream);
 

@@ -102,9 +102,9 @@ static int check_gla(const lmoe_args* a, const char* op, bool need_hs = true) {
 int lmoe_chunk_gla_fwd(const lmoe_args* a, void* stream) {
   const char* op = "lmoe_chunk_gla_fwd";
   // hs == NULL: a forward-only call, nothing saved -- where the state pass forms the output itself (2-byte
-  // elements, K = 64); the other instances hand the states to their output kernel through hs
+  // elements); the 4-byte instances hand the states to their output kernel through hs
   if (int r = check_gla(a, op, false)) return r;
-  if (!a->hs && !lmoe::gla_fwd_fused(*a)) return fail(-11, "%s: hs must not be null for this dtype / K", op);
+  if (!a->hs && !lmoe::gla_fwd_fused(*a)) return fail(-11, "%s: hs must not be null for 4-byte elements", op);
   if (!a->o.ptr) return fail(-11, "%s: o must not be null", op);
   if (a->NT == 0 || a->N == 0) return 0;
   hipStream_t st = (hipStream_t)stream;

@@ -23,14 +23,21 @@ static void launch_gla_t(const lmoe_args& a, int stage, hipStream_t st) {
     case ST_GLA_INTRA_FWD:
       hipLaunchKernelGGL((k_gla_intra_fwd<T, GT, K>), dim3(persistent_grid(a.NT * a.H, 2)), block, 0, st, a); break;
     case ST_STATE_FWD:
-      if constexpr (sizeof(T) == 2 && K == 64) {
-        // 2-byte elements, K = 64: the pass that holds the state also forms the output (k_gla_fwd_fused; at K = 128
-        // its loaders' three register sets do not fit beside the other teams' registers); hs == NULL: nothing saved
+      if constexpr (sizeof(T) == 2) {
+        // 2-byte elements: the pass that holds the state also forms the output (k_gla_fwd_fused); hs == NULL: nothing
+        // saved
         const int pairs8 = (a.N * a.H + 7) / 8 * 8;
         if constexpr (Tl::BVS_WIDE != Tl::BVS) {
-          if (wide) {
-            if (a.hs) hipLaunchKernelGGL((k_gla_fwd_fused<T, K, V, Tl::BVS_WIDE, true>), dim3(pairs8 * (V / Tl::BVS_WIDE)), dim3(3 * NTHR), 0, st, a);
-            else hipLaunchKernelGGL((k_gla_fwd_fused<T, K, V, Tl::BVS_WIDE, false>), dim3(pairs8 * (V / Tl::BVS_WIDE)), dim3(3 * NTHR), 0, st, a);
+          // (the saving instance of a wide slice at K = 128 has no registers left for the copy of the state beside the
+          // loaders' three register sets: saving calls keep the narrow slice there)
+          if (wide && (K == 64 || !a.hs)) {
+            if constexpr (K == 64) {
+              if (a.hs) {
+                hipLaunchKernelGGL((k_gla_fwd_fused<T, K, V, Tl::BVS_WIDE, true>), dim3(pairs8 * (V / Tl::BVS_WIDE)), dim3(3 * NTHR), 0, st, a);
+                break;
+              }
+            }
+            hipLaunchKernelGGL((k_gla_fwd_fused<T, K, V, Tl::BVS_WIDE, false>), dim3(pairs8 * (V / Tl::BVS_WIDE)), dim3(3 * NTHR), 0, st, a);
             break;
           }
         }
@@ -64,7 +71,7 @@ static void launch_gla_kv(const lmoe_args& a, int stage, hipStream_t st) {
 }
 
 // whether the forward state pass of this problem also forms the output (then ST_OUT_FWD is not part of the forward)
-bool gla_fwd_fused(const lmoe_args& a) { return a.dtype == LMOE_BF16 && a.K == 64; }
+bool gla_fwd_fused(const lmoe_args& a) { return a.dtype == LMOE_BF16; }
 
 // (dtype, g_dtype) must be (bf16, bf16), (bf16, f32) or (f32, f32): checked by the caller
 void launch_gla(const lmoe_args& a, int stage, hipStream_t st) {

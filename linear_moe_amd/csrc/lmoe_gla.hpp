@@ -400,11 +400,12 @@ __global__ __launch_bounds__(NTHR) void k_gla_state_fwd(const lmoe_args a) {
 // state: S is not read back from memory by a kernel of its own (k_gla_out_fwd fetched hs, q e^{b}, A and v again).
 //   consumers (waves 0-3):  S = diag(e^{b_C}) S + (k e^{b_C - b})^T v in fp32 accumulators (wave w: K rows K/4 w ..),
 //                           S^T of the next chunk -> s_hT, then the fragments of the next update
-//   loaders   (waves 4-7):  three register sets of (k~, q~, v, A, decay), chunk c + 2 staged into the buffer of
+//   loaders   (waves 4-7):  three register sets of (k~, q~, v, decay), chunk c + 2 staged into the buffer of
 //                           chunk c as window c opens; with SAVE hs[chunk] <- S (layout [K][V]) through transposing
 //                           reads of s_hT: a lane holds eight consecutive V columns of one K row, 16-byte stores
 //   output    (waves 8-11): rows 16 w .. of o^T = S^T q~^T + v^T A^T in one accumulator (the products, their order
-//                           and the rounding of k_gla_out_fwd: the same bits), stored from registers
+//                           and the rounding of k_gla_out_fwd: the same bits), stored from registers; its rows of A
+//                           come straight from memory into the lanes that use them, two chunks ahead
 // Two buffers of every tile: what a window reads of a chunk's own operands was read into registers at the end of the
 // window before (see k_state_fwd_b).
 // ------------------------------------------------------------------------- //
@@ -417,7 +418,6 @@ __global__ __launch_bounds__(3 * NTHR) void k_gla_fwd_fused(const lmoe_args a) {
   __shared__ __attribute__((aligned(16))) T s_q[2][CH * LDK];                 // q e^{b}        [64][K]
   __shared__ __attribute__((aligned(16))) T s_u[2][CH * LDU];                 // v              [64][BV]
   __shared__ __attribute__((aligned(16))) T s_hT[2][BV * LDK];                // S^T            [BV][K]
-  __shared__ __attribute__((aligned(16))) T s_P[2][CH * LDC];                 // A              [64][64]
   __shared__ __attribute__((aligned(16))) float s_dec[2][K];                  // e^{b_C}        [K]
 
   constexpr int NVS = V / BV;
@@ -444,12 +444,11 @@ __global__ __launch_bounds__(3 * NTHR) void k_gla_fwd_fused(const lmoe_args a) {
   }
   typedef TileIO<T, CH, K> IOK;
   typedef TileIO<T, CH, BV> IOV;
-  typedef TileIO<T, CH, CH> IOA;
 
   if (team == 1) {
     // --------------------------------- loaders -------------------------------------------
     const int tid = threadIdx.x & (NTHR - 1);
-    struct Pre { typename IOK::Regs rk, rq; typename IOV::Regs ru; typename IOA::Regs ra; float dec; int len; };
+    struct Pre { typename IOK::Regs rk, rq; typename IOV::Regs ru; float dec; int len; };
     Pre pre[3];                                              // register set = chunk % 3
     // Always issued (chunk index clamped to the last chunk; the surplus loads at the end of a sequence are never
     // consumed): a prefetch that is skipped on some path would make the compiler drain all outstanding loads at
@@ -461,7 +460,6 @@ __global__ __launch_bounds__(3 * NTHR) void k_gla_fwd_fused(const lmoe_args a) {
       IOK::load_nomask(P.rk, (const T*)a.ke + item * CH * K, K, CH);
       IOK::load_nomask(P.rq, (const T*)a.qe + item * CH * K, K, CH);
       IOV::load_nomask(P.ru, row_ptr<T>(a.v, sq.b, sq.tok0 + c * CH, h) + v0, a.v.st, len);
-      IOA::load_nomask(P.ra, (const T*)a.amat + item * CH * CH, CH, CH);
       P.dec = a.gcum[item * K + min(tid, K - 1)];
       P.len = len;
     };
@@ -471,7 +469,6 @@ __global__ __launch_bounds__(3 * NTHR) void k_gla_fwd_fused(const lmoe_args a) {
       IOK::store_lds(P.rk, s_k[buf], LDK);
       IOK::store_lds(P.rq, s_q[buf], LDK);
       IOV::store_lds(P.ru, s_u[buf], LDU);
-      IOA::store_lds(P.ra, s_P[buf], LDC);
       if (tid < K) s_dec[buf][tid] = P.dec;
     };
     // hs[chunk][h][K][v0 .. v0+BV] <- S (only the backward reads it: SAVE = false for forward-only calls): S^T read
@@ -515,7 +512,20 @@ __global__ __launch_bounds__(3 * NTHR) void k_gla_fwd_fused(const lmoe_args a) {
     const int ow = wave - 8;
     const int fr = l & 15, fg = 8 * (l >> 4), g4 = 4 * (l >> 4);
     lds_barrier();                                                                       // chunks 0, 1 staged
-    typename ET<T>::frag fq[KS], fv[CS][NB], fp[CS];
+    typename ET<T>::frag fq[KS], fv[CS][NB];
+    // The rows of A of this wave enter only as its own matrix operand: they come straight from memory into the
+    // registers of the lane that uses them (row 16 ow + fr, 8 tokens per 32), two chunks ahead, in two register
+    // sets (chunk parity) - no LDS tile, nothing for the loaders to stage.  Always requested (chunk index clamped),
+    // blocks above the diagonal included (zeros as stored): no load sits behind a branch.
+    typename ET<T>::frag fp[2][CS];
+    auto issue_A = [&](typename ET<T>::frag (&f)[CS], int c) {
+      c = min(c, sq.nchunks - 1);
+      const T* A = (const T*)a.amat + ((int64_t)(sq.chunk0 + c) * a.H + h) * CH * CH + (16 * ow + fr) * CH + fg;
+#pragma unroll
+      for (int kq = 0; kq < CS; ++kq) f[kq] = *(const typename ET<T>::vec*)(A + 32 * kq);
+    };
+    issue_A(fp[0], 0);
+    issue_A(fp[1], 1);
     auto preread = [&](int c) {
       const int cb = c & 1;
 #pragma unroll
@@ -525,12 +535,15 @@ __global__ __launch_bounds__(3 * NTHR) void k_gla_fwd_fused(const lmoe_args a) {
         if (2 * kq <= ow) {          // tokens j >= 32 only reach the rows of waves 2, 3 (A is lower triangular)
 #pragma unroll
           for (int ni = 0; ni < NB; ++ni) fv[kq][ni] = ET<T>::load_frag_t(s_u[cb], LDU, 32 * kq, 16 * ni, l);
-          fp[kq] = ET<T>::load_frag(s_P[cb] + (16 * ow + fr) * LDC + 32 * kq + fg);
         }
       }
     };
     preread(0);
-    for (int c = 0; c < sq.nchunks; ++c) {
+    for (int c0 = 0; c0 < sq.nchunks; c0 += 2) {
+#pragma unroll
+     for (int j = 0; j < 2; ++j) {
+      const int c = c0 + j;
+      if (c >= sq.nchunks) break;
       const int tok = sq.tok0 + c * CH;
       const int len = min(CH, sq.len - c * CH);
       lds_barrier();
@@ -552,10 +565,11 @@ __global__ __launch_bounds__(3 * NTHR) void k_gla_fwd_fused(const lmoe_args a) {
       for (int kq = 0; kq < CS; ++kq) {
         if (2 * kq <= ow) {
 #pragma unroll
-          for (int ni = 0; ni < NB; ++ni) ET<T>::mma(o[ni], fv[kq][ni], fp[kq]);           // + (A v)^T
+          for (int ni = 0; ni < NB; ++ni) ET<T>::mma(o[ni], fv[kq][ni], fp[j][kq]);        // + (A v)^T
         }
       }
       __builtin_amdgcn_sched_barrier(0);
+      issue_A(fp[j], c + 2);
       // lane: token 16 ow + fr, columns 16 ni + g4 .. + 3
       if (16 * ow + fr < len) {
         T* orow = row_ptr<T>(a.o, sq.b, tok + 16 * ow + fr, h) + v0 + g4;
@@ -568,6 +582,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gla_fwd_fused(const lmoe_args a) {
         }
       }
       if (c + 1 < sq.nchunks) preread(c + 1);
+     }
     }
     return;
   }

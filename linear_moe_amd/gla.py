@@ -33,7 +33,7 @@ class GLACall:
 
     def forward(self, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first, save=True):
         """save=False: a forward-only call (nothing requires a gradient): the per-chunk states are not written where
-        the state pass forms the output itself (bf16, K = 64); elsewhere the output kernel reads them."""
+        the state pass forms the output itself (bf16); the fp32 path's output kernel reads them."""
         lib = _lib.load()
         dims = _check_inputs(q, k, v, head_first, cu_seqlens)
         B, T, H, K, V = dims
@@ -51,7 +51,7 @@ class GLACall:
         dev, dt = q.device, q.dtype
         o = torch.empty_like(v)
         ht = torch.empty(plan.N, H, K, V, dtype=torch.float32, device=dev) if output_final_state else None
-        fused = dt == torch.bfloat16 and K == 64
+        fused = dt == torch.bfloat16
         hs = torch.empty(max(plan.NT, 1), H, K, V, dtype=dt, device=dev) if (save or not fused) else None
         amat = torch.empty(max(plan.NT, 1), H, 64, 64, dtype=dt, device=dev)
         # gated operands of the state passes (q e^b, k e^{b_C - b}, e^{b_C}), formed once per chunk

@@ -129,12 +129,14 @@ def test_gla_dv_of_the_fused_backward_kernel_equals_the_kernel_of_its_own(cuda, 
 
 
 @pytest.mark.parametrize("B,H,T,K,V,varlen", [(2, 3, 200, 64, 128, False), (1, 4, 64, 64, 64, False),
-                                              (64, 4, 130, 64, 128, False), (1, 4, 700, 64, 128, True)])
+                                              (64, 4, 130, 64, 128, False), (1, 4, 700, 64, 128, True),
+                                              (2, 3, 200, 128, 128, False), (1, 2, 333, 128, 64, False),
+                                              (1, 4, 700, 128, 128, True)])
 def test_gla_output_of_the_fused_forward_pass_equals_the_output_kernel(cuda, B, H, T, K, V, varlen):
-    """With 2-byte elements and K = 64 the forward state pass forms the output as well (three teams, one barrier per
-    chunk, the state never read back); the chunk-parallel output kernel (what the other instances run, still
-    reachable as a stage) forms the same products in the same order from the per-chunk states the pass has saved:
-    bit for bit the same o — narrow and wide V slices (the batch of 64), partial chunks, packed sequences."""
+    """With 2-byte elements the forward state pass forms the output as well (three teams, one barrier per chunk, the
+    state never read back); the chunk-parallel output kernel (what the fp32 path runs, still reachable as a stage)
+    forms the same products in the same order from the per-chunk states the pass has saved: bit for bit the same o —
+    narrow and wide V slices (the batch of 64), partial chunks, packed sequences."""
     import ctypes as C
     from linear_moe_amd import _lib
     from linear_moe_amd.gla import GLACall
@@ -158,8 +160,8 @@ def test_gla_output_of_the_fused_forward_pass_equals_the_output_kernel(cuda, B, 
 
 
 def test_gla_forward_only_call_equals_the_saving_call(cuda):
-    """Nothing requires a gradient: the per-chunk states are neither allocated nor written (bf16, K = 64: the state
-    pass forms the output itself); the output and the final state are those of the call that saves them."""
+    """Nothing requires a gradient: the per-chunk states are neither allocated nor written (bf16: the state pass forms
+    the output itself); the output and the final state are those of the call that saves them."""
     from linear_moe_amd import chunk_gla
     B, H, T, K, V = 2, 4, 300, 64, 128
     q, k = gen(95, B, T, H, K).bfloat16().to(cuda), gen(96, B, T, H, K).bfloat16().to(cuda)
