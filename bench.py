@@ -38,7 +38,7 @@ STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_gdn_state_fwd_reg", 4: "k_gdn_state_bwd"
 # sources (kernel_sources_sha16()) at that time, and a build whose sources differ reports traffic = null
 # rather than a stale number.
 CALIB_COPY_BYTES = 256 << 20
-MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237241154, "k_gdn_state_fwd_reg": 1119273843, "k_gdn_state_bwd": 946202866, "k_gdn_bwd_chunk": 1898809038}
+MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237241817, "k_gdn_state_fwd_reg": 1119611928, "k_gdn_state_bwd": 946250372, "k_gdn_bwd_chunk": 1898358547}
 TRAFFIC_SOURCES_SHA16 = "a0ad676c6194a4cd"
 TRAFFIC_SOURCES = ("lmoe_common.hpp", "lmoe_seq.hpp", "lmoe_gdn_wy.hpp", "lmoe_gdn_state.hpp", "lmoe_gdn_state_reg.hpp", "lmoe_gdn_bwd_chunk.hpp",
                    "lmoe_gdn_fwd.hip", "lmoe_gdn_state.hip", "lmoe_gdn_bwd.hip")
@@ -46,8 +46,8 @@ TRAFFIC_SOURCES = ("lmoe_common.hpp", "lmoe_seq.hpp", "lmoe_gdn_wy.hpp", "lmoe_g
 
 # HBM bytes per call of the other contract configurations (bench.py --other-configs), same counters and scaling,
 # summed over the kernels of the call; key = configuration number
-OTHER_TRAFFIC = {"1": 2230782, "2": 272920209, "3": 1413455001, "5": 16899973980, "6": 1444818074}
-OTHER_TRAFFIC_SHA16 = "9efc328a07e02a87"
+OTHER_TRAFFIC = {"1": 2230780, "2": 272922640, "3": 1281288183, "5": 16909907572, "6": 1444912378}
+OTHER_TRAFFIC_SHA16 = "4216e5427f3bcb71"
 
 
 def all_sources_sha16():

@@ -24,6 +24,7 @@ GUARDED = {
     "k_gdn_state_bwd": 3,
     "k_gdn_bwd_chunk": 3,
     "k_gdn_wy_fwd": 2,
+    "k_gla_fwd_fused": 3,
     "k_bwd_dqkv": 2,          # one work-group of 8 waves per CU; its first version spilled loop-invariant lane arithmetic
 }
 FIELDS = {"ScratchSize [bytes/lane]": "scratch", "VGPRs Spill": "vspill", "Occupancy [waves/SIMD]": "occ",
