@@ -264,7 +264,9 @@ int lmoe_mom_rowdot(const void* src, const int32_t* idx, const void* g, void* dw
  * with events on its own stream).  `a` must be the fully populated argument block of the
  * op's fwd (stages 0-2, 7) or bwd (stages 3-5) entry point, with the intermediates of the
  * earlier stages already in place.  Stages: 0 gated-delta-rule WY preparation, 1 forward state
- * pass, 2 output, 3 dv, 4 reverse state pass, 5 dq dk and gate gradient (gated delta rule: every
+ * pass (scalar gates, and chunk_gla with 2-byte elements: the output o as well, so that the forward entry point
+ * does not run stage 2, which stays available and gives the same o from the saved states), 2 output (chunk_gla),
+ * 3 dv, 4 reverse state pass, 5 dq dk and gate gradient (gated delta rule: every
  * gradient that follows the reverse state pass; chunk_simple_gla and chunk_gla with 2-byte elements: dv as well, so
  * that their backward entry points do not run stage 3, which stays available and gives the same dv), 7 chunk_gla
  * intra-chunk matrix.

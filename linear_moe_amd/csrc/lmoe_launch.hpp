@@ -9,8 +9,8 @@ namespace lmoe {
 // Stages of the three ops (argument of lmoe_launch_stage; declared in include/lmoe.h)
 enum Stage {
   ST_GDN_WY_FWD = 0,   // gated delta rule: w, u, Tinv, P                (chunk-parallel)
-  ST_STATE_FWD = 1,    // sequential state pass: hs (, vnew), ht; scalar gates: also the output o
-  ST_OUT_FWD = 2,      // chunk_gla: output o                            (chunk-parallel)
+  ST_STATE_FWD = 1,    // sequential state pass: hs (, vnew), ht; scalar gates and 2-byte chunk_gla: also the output o
+  ST_OUT_FWD = 2,      // chunk_gla: output o (the forward runs it for fp32 only)   (chunk-parallel)
   ST_DV = 3,           // dv (simple_gla / gla; the backward entry points run it for fp32 only: ST_DQK forms dv for 2-byte elements)
   ST_STATE_BWD = 4,    // reverse sequential state pass: dhs (, dv_new), dh0
   ST_DQK = 5,          // dq, dk, gate gradient; gated delta rule: every gradient that follows the
