@@ -99,6 +99,32 @@ def test_gated_delta_rule_needs_w_and_u_only_where_the_state_pass_reads_them():
                     assert b"w and u must not be null" in lib.lmoe_last_error()
 
 
+def test_chunk_gla_forward_needs_hs_only_where_an_output_kernel_reads_it():
+    """2-byte elements: the forward state pass forms the output itself and hs, which only the backward reads, may be
+    NULL (a forward-only call).  4-byte elements hand the states to their output kernel through hs: required.  A
+    call without chunks validates and returns before any launch (no GPU needed)."""
+    from linear_moe_amd import _lib
+    lib = _lib.load()
+    fake = 0x1000                                  # never dereferenced: NT == 0
+    for dtype in (_lib.LMOE_BF16, _lib.LMOE_F32):
+        for with_hs in (False, True):
+            a = _lib.Args()
+            a.dtype, a.B, a.T, a.H, a.K, a.V, a.N, a.NT = dtype, 1, 0, 1, 64, 64, 1, 0
+            a.scale, a.gate, a.g_dtype = 1.0, _lib.GATE_VECTOR, _lib.LMOE_F32
+            for n in ("q", "k", "v", "g", "o"):
+                setattr(a, n, _lib.Tensor4(fake, 0, 64, 64))
+            a.amat = a.qe = a.ke = a.gcum = fake
+            a.hs = fake if with_hs else None
+            rc = lib.lmoe_chunk_gla_fwd(C.byref(a), None)
+            assert rc == (-11 if dtype == _lib.LMOE_F32 and not with_hs else 0), (dtype, with_hs)
+            if rc:
+                assert b"hs must not be null" in lib.lmoe_last_error()
+            if not with_hs:                        # the backward always needs it
+                a.dhs = fake
+                a.d_o = a.dq = a.dk = a.dv = a.dg = _lib.Tensor4(fake, 0, 64, 64)
+                assert lib.lmoe_chunk_gla_bwd(C.byref(a), None) == -11
+
+
 def test_workspace_bytes_matches_the_buffers_the_host_layer_allocates():
     from linear_moe_amd import _lib
     lib = _lib.load()
