@@ -480,7 +480,7 @@ int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* strea
         break;
       case lmoe::ST_DQK:
         if (gdn) {
-          if (!a->tinv || !a->dvnew.ptr || !a->beta.ptr) return fail(-11, "%s: tinv, dvnew and beta must not be null", nm);
+          if (!a->dvnew.ptr || !a->beta.ptr) return fail(-11, "%s: dvnew and beta must not be null", nm);
           lmoe::launch_gdn_bwd_chunk(*a, st);
         } else {
           if (!a->hs || !a->dhs || !a->d_o.ptr || !a->dq.ptr || !a->dk.ptr || (a->dtype != LMOE_F32 && !a->dv.ptr))

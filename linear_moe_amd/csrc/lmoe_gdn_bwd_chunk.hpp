@@ -1,42 +1,42 @@
 // Gated delta rule, chunk-parallel part of the backward: everything that follows the reverse
 // state pass, for one (chunk, head) at a time, in one kernel.
 //
-// Inputs per chunk: do, v' = v_new, du = dv_new, S^T and dS'^T (hs, dhs: [V][K]), q, k, v, Tinv, g,
-// beta.  With b = cumulative gate inside the chunk, Gamma_ij = e^{b_i - b_j}, k_b = beta k,
-// k_bg = k_b e^{b}:
+// The WY form of a chunk is v_new = Tinv Z with Z = beta (v - e^{b} k S) and Tinv = (I + L)^{-1},
+// L = strictlower((beta k k^T) . Gamma): v_new solves (I + L) v_new = Z.  Its backward needs no product
+// with Tinv once dZ = Tinv^T dv_new is known (the reverse state pass writes dZ, not dv_new):
+//     dv = beta dZ,   d(k beta e^{b}) = -dZ S^T,   dL = -strictlower(dZ v_new^T),   dS -= (k beta e^{b})^T dZ.
+//
+// Inputs per chunk: do, v' = v_new, dZ, S^T and dS'^T (hs, dhs: [V][K]), q, k, v, g, beta.  With
+// b = cumulative gate inside the chunk, Gamma_ij = e^{b_i - b_j}, k_b = beta k, k_bg = k_b e^{b}:
 //   stage 1 (loop over V-slices of width BVH, contraction over the slice's columns)
 //     dP   += do v'^T            dq_i += do S^T         dk_d += v' dS'^T
-//     dw   -= du S^T             dT_v += du v^T
-//     dv_b  = Tinv^T du  (slice) -> dv = dv_b beta (stored),  dbeta += <dv_b, v>
+//     dk_bg -= dZ S^T            dLf  += dZ v'^T
+//     (loader waves, from the registers they stage:  dv = beta dZ, stored;  dbeta += <dZ, v>)
 //   stage 2
-//     G    = scale (dP . Gamma) [i >= j]
+//     G    = scale (dP . Gamma) [i >= j],     dM = -(dLf . Gamma) [i > j]       (L = M . Gamma_s, M = k_b k^T)
 //     dq   = scale e_b dq_i + G k                       (stored)
-//     dk   = e_d dk_d + G^T q                           (the part that does not pass through w, u)
-//     dT   = dT_v . beta_j + (dw k^T) . (beta_j e^{b_j})
-//     dk_bg = Tinv^T dw
-//     dL   = - strictlower(Tinv^T dT Tinv^T),   dM = dL . Gamma_s        (L = M . Gamma_s, M = k_b k^T)
+//     dk   = e_d dk_d + G^T q                           (the part that does not pass through the WY form)
 //     dk_b = dM k + dk_bg e^{b}
 //     dk  += dM^T k_b + dk_b beta                       (stored);   dbeta += <dk_b, k>
 //     db_i = q_i.dq_i - k_i.dk_i(first part) + k_b.(dM k) - k.(dM^T k_b) + dk_bg.k_bg
 //            (+ on the last row  sum_j (e_d dk_d . k)_j + e^{b_C} <S, dS'>),   dg = reverse cumsum of db
-// Nothing but the final gradients leaves the chip: dw, the two parts of dk and the second read of
-// du stay in registers / LDS.
+// Nothing but the final gradients leaves the chip.
 //
 // persistent: grid = one work-group per CU, item = (chunk, head).  Work-group = 12 waves on one
 // barrier script: 8 compute waves and 4 loader waves.
 //   Compute wave w owns chunk rows 16 (w % 4) .. + 15 and column half w / 4 of every product (half
 //   of K for the K-wide ones, 32 of the 64 columns for the chunk x chunk ones).  The compute waves
 //   touch only LDS and the matrix cores, apart from the 64 floats of dbeta and dg per item.
-//   The loader waves own all other global traffic: they keep the next slice, the next q, k and the
-//   next item's Tinv, g, beta in flight in registers (whole 128-byte lines per row), stage them into
-//   LDS (slices into NBUF alternating buffers, two where LDS has the room, so that a slice is filled
-//   while the previous one is consumed; the stage 2 tiles lie over the last buffer), and lift the
-//   results (dv per slice, dq, dk) out of LDS and store them.  They also form <S, dS'> from the
-//   registers they hold and the gate cumsum of the chunk.
-//   Script per item (NS slices), three slice buffers:  D(0) .. D(NS-1) = A | b c d e f g h | E
-//     (slice s is staged two windows before the compute team reaches it; slices 0, 1 of the next item
-//     during f .. h of this one)
-//   one slice buffer:  [R(0)] D(0) R(1) D(1) .. D(NS-1) | A | b c d e f g h | E | R(0) of the next item
+//   The loader waves own all other global traffic: they keep the next slices, the next q and k and the
+//   next item's g, beta in flight in registers (whole 128-byte lines per row), stage them into
+//   LDS (slices into NBUF alternating buffers, q and k into tiles of their own; the three chunk x chunk
+//   tiles of stage 2 lie over the last slice buffer), form dv and the value part of dbeta from the
+//   registers on the way, and lift dq, dk out of LDS and store them.  They also form <S, dS'> from
+//   the registers they hold and the gate cumsum of the chunk.
+//   Script per item (NS = 4 slices), three slice buffers:   D0 D1 D2 A | b c d
+//     window w: the compute team works on slice w (buffer w % 3); the loaders stage slice w + 2, then q
+//     (window 2) and k (window 3), and slices 0, 1 of the next item during b .. d
+//   one slice buffer:  [R(0)] D(0) R(1) D(1) .. D(NS-1) | A | b c d | R(0) of the next item
 #pragma once
 #include "lmoe_seq.hpp"
 
@@ -45,11 +45,11 @@ namespace lmoe {
 // LDS bytes of k_gdn_bwd_chunk
 template <typename T, int K, int BVH, int NBUF> struct GdnBwdChunkLds {
   static constexpr int LDV = BVH + LPAD, LDC = CH + LPAD, LDK = K + LPAD;
-  static constexpr int A_END = 4 * CH * LDV + 2 * BVH * LDK;
-  static constexpr int B_END = 2 * CH * LDK + CH * LDC + CH * LDK;
-  static constexpr int NREG = (NBUF - 1) * A_END + (A_END > B_END ? A_END : B_END);
-  static constexpr int NDV = NBUF == 3 ? 2 : 1;      // copies of the dv strip
-  static constexpr int BYTES = (NREG + CH * LDC + NDV * CH * LDV) * (int)sizeof(T) + (12 * 64 + 16) * 4;
+  static constexpr int A_END = 3 * CH * LDV + 2 * BVH * LDK;      // do, v_new, dZ; S^T, dS'^T of one slice
+  static constexpr int T_END = 3 * CH * LDC;                      // G^T, dM^T, (beta dM)^T: over the last slice buffer
+  static constexpr int S_END = (NBUF - 1) * A_END + (A_END > T_END ? A_END : T_END);   // slice buffers, the last one widened to hold the tiles
+  static constexpr int NREG = S_END + 2 * CH * LDK;               // ..; q, k
+  static constexpr int BYTES = NREG * (int)sizeof(T) + (13 * 64 + 16) * 4;
 };
 
 // gemm with a scheduling fence after every 32-deep step: at most one step's fragments are in flight,
@@ -91,24 +91,19 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
   static_assert(V % BVH == 0 && BVH == 32, "V-slices: the 8 compute waves split a 64 x 32 slice product 4 x 2");
   static_assert(NBUF == 1 || NBUF == 3, "one slice buffer, or three in rotation");
   // tiles of one V-slice
-  constexpr int A_DO = 0, A_VN = A_DO + CH * LDV, A_DVN = A_VN + CH * LDV, A_VV = A_DVN + CH * LDV,
-                A_H = A_VV + CH * LDV, A_DH = A_H + BVH * LDK, A_END = L::A_END;
-  // stage 2 tiles, laid over the last slice buffer: q (later dq, then dk, on their way out), k,
-  // T0 = G^T then dT^T then (beta dM)^T, DW = dw (rows), later T1 = X1^T then dM^T in its first 64 x 64
-  constexpr int SB = (NBUF - 1) * A_END;
-  constexpr int B_Q = SB, B_K = B_Q + CH * LDK, B_T0 = B_K + CH * LDK, B_DW = B_T0 + CH * LDC, B_T1 = B_DW;
+  constexpr int A_DO = 0, A_VN = A_DO + CH * LDV, A_DZ = A_VN + CH * LDV,
+                A_H = A_DZ + CH * LDV, A_DH = A_H + BVH * LDK, A_END = L::A_END;
+  // stage 2: q (later dq on its way out) and k (later dk) in tiles of their own; T0 = G^T, T1 = dM^T,
+  // T2 = (diag(beta) dM)^T over the last slice buffer
+  constexpr int B_T0 = (NBUF - 1) * A_END, B_T1 = B_T0 + CH * LDC, B_T2 = B_T1 + CH * LDC;
+  constexpr int B_Q = L::S_END, B_K = B_Q + CH * LDK;
   __shared__ __attribute__((aligned(16))) T smem[L::NREG];
-  __shared__ __attribute__((aligned(16))) T s_ti[CH * LDC];              // Tinv, whole item
-  // dv of a slice on its way out; with three slice buffers no barrier separates the loaders' read of
-  // slice s from the compute team's write of slice s + 1: two copies
-  __shared__ __attribute__((aligned(16))) T s_dv[L::NDV][CH * LDV];
   // gate cumsum, its exponentials and beta: two copies, the loaders fill the next item's during stage 2
-  __shared__ float s_gb[2][64], s_geb[2][64], s_ged[2][64], s_gbeta[2][64], s_db[2][64], s_dbeta[2][64], s_red[16];
+  __shared__ float s_gb[2][64], s_geb[2][64], s_ged[2][64], s_gbeta[2][64], s_db[2][64], s_dbeta[2][64], s_dbv[64], s_red[16];
 
   typedef TileIO<T, CH, BVH> IOV;
   typedef TileIO<T, BVH, K> IOH;
   typedef TileIO<T, CH, K> IOK;
-  typedef TileIO<T, CH, CH> IO64;
   const int nitems = a.NT * a.H;
   const int stride = gridDim.x;
 
@@ -132,10 +127,12 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
     typedef typename ET<T>::vec vec;
     struct Unit { vec v[NVEC]; int len; };
     Unit U[DEPTH];
-    typename IO64::Regs rt;
     uint32_t graw, braw;
     int glen;
     float hdh = 0.f;   // partial <S, dS'> of the item whose slices are being staged
+    float dbv[PV];     // partial <dZ, v> of this thread's rows of that item
+#pragma unroll
+    for (int p = 0; p < PV; ++p) dbv[p] = 0.f;
     // unit u counted from the first unit of item it (u >= NU: units of the item after it)
     auto issue = [&](auto uc, int it) {
       constexpr int u = decltype(uc)::value, unit = u % NU;
@@ -151,7 +148,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
           typename IOV::Regs r;
-          // do, v: the caller's rows; vnew, dvnew: one contiguous block per (chunk, head, slice)
+          // do, v: the caller's rows; vnew, dvnew (= dZ): one contiguous block per (chunk, head, slice)
           if (t == 1 || t == 2) IOV::load_nomask(r, slice_ptr<T>(*ts[t], cid, h, a.H, V, vv), SLICE_COLS, ci.len, tid);
           else IOV::load_nomask(r, row_ptr<T>(*ts[t], ci.b, ci.tok, h) + vv, ts[t]->st, ci.len, tid);
 #pragma unroll
@@ -173,15 +170,37 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
         for (int p = 0; p < PK; ++p) R.v[p] = r.v[p];
       }
     };
-    // unit u (u == NU: slice 0 of the next item) from its registers into LDS; slices go to buffer buf
-    auto stage = [&](auto uc, int buf) {
+    // dv of a slice on its way from the registers to memory
+    struct DV { typename IOV::Regs r; };
+    // unit u (u >= NU: of the next item) from its registers into LDS; slices go to buffer buf, and their dv = beta dZ
+    // into d (gp = the copy of the gate arrays that holds the beta of the unit's item)
+    auto stage = [&](auto uc, int buf, int gp, DV& d) {
       constexpr int u = decltype(uc)::value, unit = u % NU;
       Unit& R = U[u % DEPTH];
       if constexpr (unit < NS) {
         T* base = smem + buf * A_END;
-        constexpr int off[4] = {A_DO, A_VN, A_DVN, A_VV};
+        // dv and <dZ, v> first, from the registers as loaded: rows past the end of a partial chunk repeat its last row
+        // there, which is what the branch-free store of dv rewrites
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
+        for (int p = 0; p < PV; ++p) {
+          int row, col; IOV::coords(p, row, col, tid);
+          const float bt = s_gbeta[gp][min(row, R.len - 1)];
+          const vec z = R.v[2 * PV + p], vv = R.v[3 * PV + p];
+          vec o;
+          float s = 0.f;
+#pragma unroll
+          for (int i = 0; i < IOV::VEC; ++i) {
+            const float zf = ET<T>::to_f(z[i]);
+            o[i] = ET<T>::from_f(zf * bt);
+            s += zf * ET<T>::to_f(vv[i]);
+          }
+          d.r.v[p] = o;
+          s = group_sum<IOV::VPR>(s);                   // the VPR lanes that hold one row are neighbours
+          dbv[p] += row < R.len ? s : 0.f;
+        }
+        constexpr int off[3] = {A_DO, A_VN, A_DZ};
+#pragma unroll
+        for (int t = 0; t < 3; ++t) {
           typename IOV::Regs r;
 #pragma unroll
           for (int p = 0; p < PV; ++p) r.v[p] = R.v[t * PV + p];
@@ -205,15 +224,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
         IOK::store_lds(r, smem + (unit == NS ? B_Q : B_K), LDK, tid);
       }
     };
-    // stage unit u of item it, then request the unit that takes over its registers
-    auto advance = [&](auto uc, int it, int buf) {
-      constexpr int u = decltype(uc)::value;
-      stage(uc, buf);
-      issue(IC<u + DEPTH>(), it);
-    };
-    auto issue_tinv = [&](int it) {
-      it = min(it, nitems - 1);
-      IO64::load_nomask(rt, (const T*)a.tinv + (int64_t)it * CH * CH, CH, CH, tid);     // it = cid * H + h
+    auto store_dv = [&](const DV& d, const ChunkInfo& ci, int h, int s) {
+      IOV::template store_global_clamped<true>(d.r, row_ptr<T>(a.dv, ci.b, ci.tok, h) + s * BVH, a.dv.st, ci.len, tid);
     };
     auto issue_gates = [&](int it) {
       it = __builtin_amdgcn_readfirstlane(min(it, nitems - 1));
@@ -228,100 +240,110 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
       gate_finish_wave(a, graw, glen, l, lw == 0, s_gb[par], s_geb[par], s_ged[par]);
       if (lw == 1) s_gbeta[par][l] = l < glen ? scalar_from_raw(braw, a.beta_dtype) : 0.f;
     };
-    const int it0 = blockIdx.x;
-    issue_tinv(it0);
-    issue_gates(it0);
-    issue(IC<0>(), it0);
-    if constexpr (DEPTH == 2) issue(IC<1>(), it0);
-    // the first loads may be ordered freely by the compiler; were they still pending at the loop
-    // header, its wait-count analysis would carry that order into every iteration
-    wait_all_loads();
-    IO64::store_lds(rt, s_ti, LDC, tid);
-    stage_gates(0);
-    issue_gates(it0 + stride);
-    advance(IC<0>(), it0, 0);
-    if constexpr (NBUF == 3) advance(IC<1>(), it0, 1);
-    int par = 0;
-    auto store_dv = [&](const ChunkInfo& ci, int h, int s) {
-      typename IOV::Regs r;
-      IOV::load_lds_clamped(r, s_dv[s % L::NDV], LDV, ci.len, tid);
-      IOV::template store_global_clamped<true>(r, row_ptr<T>(a.dv, ci.b, ci.tok, h) + s * BVH, a.dv.st, ci.len, tid);
-    };
-    auto close_hdh = [&]() {
+    // the sums of an item whose slices have all been staged
+    auto close_item = [&]() {
       hdh = wave_sum(hdh);
       if (l == 0) s_red[lw] = hdh;
       hdh = 0.f;
+#pragma unroll
+      for (int p = 0; p < PV; ++p) {
+        int row, col; IOV::coords(p, row, col, tid);
+        if (col == 0) s_dbv[row] = dbv[p];
+        dbv[p] = 0.f;
+      }
     };
+    const int it0 = blockIdx.x;
+    DV d0, d1;
+    issue_gates(it0);
+    static_for<DEPTH>([&](auto jc) { issue(jc, it0); });
+    // the first loads may be ordered freely by the compiler; were they still pending at the loop
+    // header, its wait-count analysis would carry that order into every iteration
+    wait_all_loads();
+    stage_gates(0);
+    issue_gates(it0 + stride);
+    lds_barrier();                                                                       // beta of the first item staged
+    {
+      const ChunkInfo ci = chunk_info(a, it0 / a.H);
+      stage(IC<0>(), 0, 0, d0);
+      issue(IC<DEPTH>(), it0);
+      store_dv(d0, ci, it0 % a.H, 0);
+      if constexpr (NBUF == 3) {
+        stage(IC<1>(), 1, 0, d1);
+        issue(IC<1 + DEPTH>(), it0);
+        store_dv(d1, ci, it0 % a.H, 1);
+      }
+    }
+    int par = 0;
     lds_barrier();                                                                       // first slice staged
     for (int it = it0; it < nitems; it += stride) {
       tid = fresh_index(tid) & (NTHR - 1);
       const int cid = it / a.H, h = it % a.H;
       const ChunkInfo ci = chunk_info(a, cid);
+      // the item after this one (past the end: the last item once more, see issue)
+      const int itn = __builtin_amdgcn_readfirstlane(min(it + stride, nitems - 1));
+      const int hn = itn % a.H;
+      const ChunkInfo cin = chunk_info(a, itn / a.H);
       if constexpr (NBUF == 3) {
         // window w: the compute team works on slice w.  Slice s lives in buffer s % 3 and is staged two
-        // windows ahead; q, k go to the third buffer's region in the last window.
-        // In every window the loaders fill LDS first and meet the compute team at the barrier; the requests
-        // that refill the freed registers follow the barrier.  Requests stall at the issue while the CU's
-        // queue is full (32 KB take about a microsecond): issued before the barrier, that stall held up
-        // the compute team in five windows of twelve (a quarter of the item, traced per barrier).
+        // windows ahead; q and k follow in windows 2 and 3.
+        // In every window the loaders fill LDS first and meet the compute team at the barrier; the stores and the
+        // requests that refill the freed registers follow the barrier.  Requests stall at the issue while the CU's
+        // queue is full (32 KB take about a microsecond): issued before the barrier, that stall holds up the
+        // compute team.
         static_for<NS>([&](auto wc) {
-          constexpr int w = decltype(wc)::value;
-          if constexpr (w >= 1) store_dv(ci, h, w - 1);
-          if constexpr (w + 2 < NS) stage(IC<w + 2>(), (w + 2) % 3);
-          if constexpr (w == NS - 1) {
-            stage(IC<NS>(), 0);                                                          // q
-            stage(IC<NS + 1>(), 0);                                                      // k
-            close_hdh();
-          }
+          constexpr int w = decltype(wc)::value, u = w + 2;    // u < NS: a slice (buffer u % 3), then q, then k
+          stage(IC<u>(), u % 3, par, d0);
+          if constexpr (w == NS - 1) close_item();
           lds_barrier();                                                                 // D(w); the last one is A
-          if constexpr (w + 2 < NS) issue(IC<w + 2 + DEPTH>(), it);
-          if constexpr (w == NS - 1) issue(IC<NS + DEPTH>(), it);                        // slice 0 of the next item
+          if constexpr (u < NS) store_dv(d0, ci, h, u);
+          if constexpr (w < NS - 1) issue(IC<u + DEPTH>(), it);                          // q, k, slice 0 of the next item
         });
-        store_dv(ci, h, NS - 1);
+        issue(IC<NS + 1 + DEPTH>(), it);                                                 // slice 1 of the next item
+        stage_gates(par ^ 1);                                  // the next item's; its copy is idle since d of the last item
+        issue_gates(it + 2 * stride);
+        lds_barrier();                                                                   // b
+        stage(IC<NU>(), 0, par ^ 1, d0);                       // slice 0 of the next item (buffer 0: slice 3 is done)
+        lds_barrier();                                                                   // c
+        store_dv(d0, cin, hn, 0);
+        issue(IC<NU + DEPTH>(), it);                                                     // slice 2 of the next item
+        stage(IC<NU + 1>(), 1, par ^ 1, d1);                   // slice 1 of the next item
+        lds_barrier();                                                                   // d: dq, dk lie in the q, k tiles
+        store_dv(d1, cin, hn, 1);
+        issue(IC<NU + 1 + DEPTH>(), it);                                                 // slice 3 of the next item
       } else {
         static_for<NS>([&](auto sc) {
           constexpr int s = decltype(sc)::value;
           if constexpr (s > 0) lds_barrier();                                            // R(s)
           lds_barrier();                                                                 // D(s)
-          store_dv(ci, h, s);
-          if constexpr (s + 1 < NS) advance(IC<s + 1>(), it, 0);
+          if constexpr (s + 1 < NS) {
+            stage(IC<s + 1>(), 0, par, d0);
+            issue(IC<s + 1 + DEPTH>(), it);
+            store_dv(d0, ci, h, s + 1);
+          }
         });
-        advance(IC<NS>(), it, 0);                                                        // q
-        advance(IC<NS + 1>(), it, 0);                                                    // k
-        close_hdh();
+        stage(IC<NS>(), 0, par, d0);                                                     // q
+        issue(IC<NS + DEPTH>(), it);
+        stage(IC<NS + 1>(), 0, par, d0);                                                 // k
+        issue(IC<NS + 1 + DEPTH>(), it);
+        close_item();
         lds_barrier();                                                                   // A
+        stage_gates(par ^ 1);
+        issue_gates(it + 2 * stride);
+        lds_barrier();                                                                   // b
+        lds_barrier();                                                                   // c
+        lds_barrier();                                                                   // d
       }
-      lds_barrier();                                                                     // b
-      if constexpr (NBUF == 3) issue(IC<NS + 1 + DEPTH>(), it);                          // slice 1 of the next item
-      issue_tinv(it + stride);
-      stage_gates(par ^ 1);                                    // the next item's; its copy is idle since E of the last item
-      issue_gates(it + 2 * stride);
-      lds_barrier();                                                                     // c
-      lds_barrier();                                                                     // d: dq lies in the q tile
       {
         typename IOK::Regs r;
         IOK::load_lds_clamped(r, smem + B_Q, LDK, ci.len, tid);
         IOK::template store_global_clamped<true>(r, row_ptr<T>(a.dq, ci.b, ci.tok, h), a.dq.st, ci.len, tid);
-      }
-      lds_barrier();                                                                     // e
-      lds_barrier();                                                                     // f: Tinv of this item is dead
-      IO64::store_lds(rt, s_ti, LDC, tid);
-      if constexpr (NBUF == 3) stage(IC<NU>(), 0);             // slice 0 of the next item
-      lds_barrier();                                                                     // g
-      if constexpr (NBUF == 3) {
-        issue(IC<NU + DEPTH>(), it);                           // slice 2 of the next item
-        stage(IC<NU + 1>(), 1);                                // slice 1 of the next item
-      }
-      lds_barrier();                                                                     // h: dk lies in the q tile
-      if constexpr (NBUF == 3) issue(IC<NU + 1 + DEPTH>(), it);                          // slice 3 of the next item
-      {
-        typename IOK::Regs r;
-        IOK::load_lds_clamped(r, smem + B_Q, LDK, ci.len, tid);
+        IOK::load_lds_clamped(r, smem + B_K, LDK, ci.len, tid);
         IOK::template store_global_clamped<true>(r, row_ptr<T>(a.dk, ci.b, ci.tok, h), a.dk.st, ci.len, tid);
       }
-      lds_barrier();                                                                     // E
       if constexpr (NBUF == 1) {
-        advance(IC<NU>(), it, 0);
+        stage(IC<NU>(), 0, par ^ 1, d0);                       // slice 0 of the next item
+        issue(IC<NU + DEPTH>(), it);
+        store_dv(d0, cin, hn, 0);
         lds_barrier();                                                                   // R(0) of the next item
       }
       par ^= 1;
@@ -338,6 +360,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
   const int k0 = KH * ch;                  // first column in a K-wide product
   const float scale = a.scale;
   int par = 0;
+  lds_barrier();                                                                         // beta of the first item staged
   lds_barrier();                                                                         // first slice staged
   for (int it = blockIdx.x; it < nitems; it += stride) {
     const float* s_b = s_gb[par]; const float* s_eb = s_geb[par]; const float* s_ed = s_ged[par];
@@ -347,9 +370,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
     const int l = fresh_index(lane_id()) & 63;
     const int fr = l & 15, fg = 8 * (l >> 4);
     const int rb = r0 + 4 * (l >> 4);      // accumulator element i is row rb + i, column (tile) + fr
-    f32x4 dP[1][2], dTv[1][2], dqi[1][NBK], dkd[1][NBK], dw[1][NBK];
-    acc_zero(dP); acc_zero(dTv); acc_zero(dqi); acc_zero(dkd); acc_zero(dw);
-    float dbt[4] = {0.f, 0.f, 0.f, 0.f};      // dbeta of rows rb + i (partial over lanes and column halves)
+    f32x4 dP[1][2], dLf[1][2], dqi[1][NBK], dkd[1][NBK], dkbg[1][NBK];
+    acc_zero(dP); acc_zero(dLf); acc_zero(dqi); acc_zero(dkd); acc_zero(dkbg);
     // ---- stage 1 ----
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
@@ -357,64 +379,53 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
         if (s > 0) lds_barrier();                                                        // R(s)
       }
       const T* base = smem + (NBUF == 3 ? (s % 3) * A_END : 0);
-      const T* DO = base + A_DO; const T* VN = base + A_VN; const T* DVN = base + A_DVN;
-      const T* VV = base + A_VV; const T* HT = base + A_H; const T* DHT = base + A_DH;
+      const T* DO = base + A_DO; const T* VN = base + A_VN; const T* DZ = base + A_DZ;
+      const T* HT = base + A_H; const T* DHT = base + A_DH;
 #pragma unroll
       for (int kk = 0; kk < BVH; kk += 32) {
         const typename ET<T>::frag aDO = ET<T>::load_frag(DO + (r0 + fr) * LDV + kk + fg);
         const typename ET<T>::frag aVN = ET<T>::load_frag(VN + (r0 + fr) * LDV + kk + fg);
-        const typename ET<T>::frag aDVN = ET<T>::load_frag(DVN + (r0 + fr) * LDV + kk + fg);
+        const typename ET<T>::frag aDZ = ET<T>::load_frag(DZ + (r0 + fr) * LDV + kk + fg);
 #pragma unroll
         for (int nj = 0; nj < 2; ++nj) {
-          ET<T>::mma(dP[0][nj], aDO, ET<T>::load_frag(VN + (c0 + 16 * nj + fr) * LDV + kk + fg));
-          ET<T>::mma(dTv[0][nj], aDVN, ET<T>::load_frag(VV + (c0 + 16 * nj + fr) * LDV + kk + fg));
+          const typename ET<T>::frag bVN = ET<T>::load_frag(VN + (c0 + 16 * nj + fr) * LDV + kk + fg);
+          ET<T>::mma(dP[0][nj], aDO, bVN);
+          ET<T>::mma(dLf[0][nj], aDZ, bVN);
         }
 #pragma unroll
         for (int ni = 0; ni < NBK; ++ni) {
           const typename ET<T>::frag bH = ET<T>::load_frag_t(HT, LDK, kk, k0 + 16 * ni, l);
           ET<T>::mma(dqi[0][ni], aDO, bH);
-          ET<T>::mma(dw[0][ni], aDVN, bH);
+          ET<T>::mma(dkbg[0][ni], aDZ, bH);                                              // + dZ S^T: dk_bg is its negative
           ET<T>::mma(dkd[0][ni], aVN, ET<T>::load_frag_t(DHT, LDK, kk, k0 + 16 * ni, l));
         }
       }
-      // dv_b = Tinv^T du for this slice: rows r0.., columns 16 ch .. + 15 of the slice
-      f32x4 dvb[1][1];
-      acc_zero(dvb);
-      gemm<T, 1, 1, true, true>(dvb, s_ti, LDC, r0, DVN, LDV, 16 * ch, 0, CH, l);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        dbt[i] += dvb[0][0][i] * ET<T>::to_f(VV[(rb + i) * LDV + 16 * ch + fr]);
-        dvb[0][0][i] *= s_beta[rb + i];                                                  // final dv
-      }
-      acc_to_lds<T>(dvb[0][0], s_dv[s % L::NDV], LDV, r0, 16 * ch, l);
-      pin(dbt);
       __builtin_amdgcn_sched_barrier(0);
       lds_barrier();                                                                     // D(s); with three buffers the last one is A
     }
     if constexpr (NBUF == 1) lds_barrier();                                              // A: q, k staged
     // ---- stage 2 ----
-    T* Qt = smem + B_Q; T* Kt = smem + B_K; T* T0 = smem + B_T0; T* T1 = smem + B_T1; T* DW = smem + B_DW;
+    T* Qt = smem + B_Q; T* Kt = smem + B_K; T* T0 = smem + B_T0; T* T1 = smem + B_T1; T* T2 = smem + B_T2;
 #pragma unroll
     for (int nj = 0; nj < 2; ++nj) {
-      f32x4 p;
+      f32x4 g, m, mb;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int r = rb + i, cc = c0 + 16 * nj + fr;
-        p[i] = (r >= cc) ? scale * dP[0][nj][i] * texp<T>(s_b[r] - s_b[cc]) : 0.f;
+        const float e = (r >= cc) ? texp<T>(s_b[r] - s_b[cc]) : 0.f;
+        g[i] = scale * dP[0][nj][i] * e;
+        m[i] = (r > cc) ? -dLf[0][nj][i] * e : 0.f;
+        mb[i] = m[i] * s_beta[r];
       }
-      acc_to_lds_t<T>(p, T0, LDC, r0, c0 + 16 * nj, l);                                  // G^T [j][i]
-    }
-#pragma unroll
-    for (int ni = 0; ni < NBK; ++ni) {
-      f32x4 x;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) x[i] = -dw[0][ni][i];                                  // dw = -du S^T
-      acc_to_lds<T>(x, DW, LDK, r0, k0 + 16 * ni, l);
+      acc_to_lds_t<T>(g, T0, LDC, r0, c0 + 16 * nj, l);                                  // G^T [j][i]
+      acc_to_lds_t<T>(m, T1, LDC, r0, c0 + 16 * nj, l);                                  // dM^T [j][i]
+      acc_to_lds_t<T>(mb, T2, LDC, r0, c0 + 16 * nj, l);                                 // (diag(beta) dM)^T [j][i]
     }
     lds_barrier();                                                                       // b
-    float dbp[4] = {0.f, 0.f, 0.f, 0.f};
+    float dbp[4] = {0.f, 0.f, 0.f, 0.f};      // db of rows rb + i (partial over lanes and column halves)
+    float dbt[4] = {0.f, 0.f, 0.f, 0.f};      // dbeta of rows rb + i, the part through k_b
     float kk = 0.f;
-    f32x4 dq[1][NBK], dk[1][NBK], dkbg[1][NBK], dT[1][2];
+    f32x4 dq[1][NBK], dk[1][NBK];
     acc_zero(dq);
     gemm_bounded<T, 1, NBK, true, true>(dq, T0, LDC, r0, Kt, LDK, k0, 0, CH, l);         // G k
 #pragma unroll
@@ -446,59 +457,9 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
     pin(kk);
     __builtin_amdgcn_sched_barrier(0);
     {
-      f32x4 t2[1][2];
-      acc_zero(t2);
-      gemm_bounded<T, 1, 2, false, false>(t2, DW, LDK, r0, Kt, LDK, c0, 0, K, l);        // dw k^T
-#pragma unroll
-      for (int nj = 0; nj < 2; ++nj) {
-        const int cc = c0 + 16 * nj + fr;
-        const float bj = s_beta[cc], bej = bj * s_eb[cc];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) dT[0][nj][i] = dTv[0][nj][i] * bj + t2[0][nj][i] * bej;
-      }
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    acc_zero(dkbg);
-    gemm_bounded<T, 1, NBK, true, true>(dkbg, s_ti, LDC, r0, DW, LDK, k0, 0, CH, l);     // Tinv^T dw
-    lds_barrier();                                                                       // c: G^T, DW, q read
-#pragma unroll
-    for (int nj = 0; nj < 2; ++nj) acc_to_lds_t<T>(dT[0][nj], T0, LDC, r0, c0 + 16 * nj, l);   // dT^T [n][i]
-#pragma unroll
-    for (int ni = 0; ni < NBK; ++ni) acc_to_lds<T>(dq[0][ni], Qt, LDK, r0, k0 + 16 * ni, l);   // dq on its way out
-    lds_barrier();                                                                       // d
-    {
-      // X1[j][n] = sum_i Tinv[i][j] dT[i][n]
-      f32x4 x1[1][2];
-      acc_zero(x1);
-      gemm_bounded<T, 1, 2, true, false>(x1, s_ti, LDC, r0, T0, LDC, c0, 0, CH, l);
-#pragma unroll
-      for (int nj = 0; nj < 2; ++nj) acc_to_lds_t<T>(x1[0][nj], T1, LDC, r0, c0 + 16 * nj, l);   // X1^T [n][j]
-    }
-    lds_barrier();                                                                       // e
-    {
-      f32x4 dL[1][2];
-      acc_zero(dL);
-      // dL[j][m] = - sum_n X1[j][n] Tinv[m][n]
-      gemm_bounded<T, 1, 2, true, false>(dL, T1, LDC, r0, s_ti, LDC, c0, 0, CH, l);
-      lds_barrier();                                                                     // f: X1^T, dT^T, Tinv read
-#pragma unroll
-      for (int nj = 0; nj < 2; ++nj) {
-        f32x4 p, pb;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int r = rb + i, cc = c0 + 16 * nj + fr;
-          p[i] = (r > cc) ? -dL[0][nj][i] * texp<T>(s_b[r] - s_b[cc]) : 0.f;
-          pb[i] = p[i] * s_beta[r];
-        }
-        acc_to_lds_t<T>(p, T1, LDC, r0, c0 + 16 * nj, l);                                // dM^T  [j][i]
-        acc_to_lds_t<T>(pb, T0, LDC, r0, c0 + 16 * nj, l);                               // (diag(beta) dM)^T [j][i]
-      }
-    }
-    lds_barrier();                                                                       // g
-    {
       // dM k first: it closes dk_b (dbeta, the k_b.(dM k) term); then dM^T k_b
       // (k is re-read from LDS through an offset the compiler cannot see through: it would otherwise
-      // keep the values read for the first part of dk in registers across phases c .. g)
+      // keep the values read for the first part of dk in registers)
       const T* Kr = Kt + fresh_index(0);
       f32x4 m[1][NBK];
       acc_zero(m);
@@ -511,9 +472,10 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
           const float kv = ET<T>::to_f(Kr[r * LDK + cc]);
           const float bt = s_beta[r], eb = s_eb[r];
           const float kbv = kv * bt;
-          const float dkb = m[0][ni][i] + dkbg[0][ni][i] * eb;
+          const float dkbgv = -dkbg[0][ni][i];
+          const float dkb = m[0][ni][i] + dkbgv * eb;
           dbt[i] += dkb * kv;
-          dbp[i] += kbv * m[0][ni][i] + dkbg[0][ni][i] * kbv * eb;
+          dbp[i] += kbv * m[0][ni][i] + dkbgv * kbv * eb;
           dk[0][ni][i] += dkb * bt;
         }
       pin(dbp);
@@ -521,22 +483,27 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
       __builtin_amdgcn_sched_barrier(0);
       const T* Kr2 = Kt + fresh_index(0);
       acc_zero(m);
-      gemm_bounded<T, 1, NBK, false, true>(m, T0, LDC, r0, Kt, LDK, k0, 0, CH, l);
+      gemm_bounded<T, 1, NBK, false, true>(m, T2, LDC, r0, Kt, LDK, k0, 0, CH, l);
 #pragma unroll
-      for (int ni = 0; ni < NBK; ++ni) {
+      for (int ni = 0; ni < NBK; ++ni)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int r = rb + i, cc = k0 + 16 * ni + fr;
           dbp[i] -= ET<T>::to_f(Kr2[r * LDK + cc]) * m[0][ni][i];
           dk[0][ni][i] += m[0][ni][i];                                                   // final dk
         }
-        acc_to_lds<T>(dk[0][ni], Qt, LDK, r0, k0 + 16 * ni, l);                          // dk on its way out
-      }
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       dbp[i] = group_sum<16>(dbp[i]);
       dbt[i] = group_sum<16>(dbt[i]);
+    }
+    kk = wave_sum(kk);
+    lds_barrier();                                                                       // c: q, k, the chunk x chunk tiles read
+#pragma unroll
+    for (int ni = 0; ni < NBK; ++ni) {
+      acc_to_lds<T>(dq[0][ni], Qt, LDK, r0, k0 + 16 * ni, l);                            // dq, dk on their way out
+      acc_to_lds<T>(dk[0][ni], Kt, LDK, r0, k0 + 16 * ni, l);
     }
     if (fr == 0) {
 #pragma unroll
@@ -545,9 +512,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
         s_dbeta[ch][rb + i] = dbt[i];
       }
     }
-    kk = wave_sum(kk);
     if (l == 0) s_red[4 + wv] = kk;
-    lds_barrier();                                                                       // h
+    lds_barrier();                                                                       // d
     if (threadIdx.x < 64) {
       const int cid = it / a.H, h = it % a.H;
       const ChunkInfo ci = chunk_info(a, cid);
@@ -555,7 +521,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
       const int j = fresh_index(threadIdx.x) & 63;
       float x = 0.f;
       if (j < ci.len) {
-        ((float*)a.dbeta.ptr)[row_off(a.dbeta, ci.b, ci.tok + j, h)] = s_dbeta[0][j] + s_dbeta[1][j];
+        ((float*)a.dbeta.ptr)[row_off(a.dbeta, ci.b, ci.tok + j, h)] = s_dbeta[0][j] + s_dbeta[1][j] + s_dbv[j];
         x = s_db[0][j] + s_db[1][j];
         // last-row term; rows past the end of a partial chunk carry zero q, k, so the term may sit
         // on the last valid row without changing the reverse cumulative sum
@@ -571,7 +537,6 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
       x = wave_rev_scan(x);
       if (j < ci.len) ((float*)a.dg.ptr)[row_off(a.dg, ci.b, ci.tok + j, h)] = x;
     }
-    lds_barrier();           // E: the stage 2 region goes to the next item
     if constexpr (NBUF == 1) lds_barrier();                                              // R(0) of the next item
     par ^= 1;
   }

@@ -398,10 +398,16 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
 
 // ------------------------------------------------------------------------- //
 // backward (reverse order over the chunks; it = 0 is the last chunk)
-//   team 1, chunk c:   B1 | stage q(c), w(c); lift dS'^T(c), dv_new(c+1) out of LDS |
-//                      B2 | store dhs(c), dv_new(c+1); prefetch q, w
-//   team 2, chunk c:   B1 | prefetch k, P, do, decay table | B2 | stage those of chunk c-1
+//   team 1, chunk c:   B1 | stage q(c); lift dS'^T(c) out of LDS; read its rows of Tinv^T |
+//                      B2 | dZ(c) = Tinv^T dv_new(c) for its 16 tokens per wave; store dhs(c), dZ(c); prefetch q
+//   team 2, chunk c:   B1 | prefetch k, P, Tinv, do, decay table | B2 | stage those of chunk c-1
 //   consumers, chunk c: dS' -> LDS | B1 | k dS', P^T do, dv_new -> LDS | B2 | dS update
+// What leaves for the chunk-parallel backward is not dv_new but dZ = Tinv^T dv_new, the gradient with
+// respect to Z = beta (v - e^{b} k S) (v_new = Tinv Z, i.e. (I + L) v_new = Z): with it every gradient of
+// the WY form is a product with dZ -- dv = beta dZ, d(k beta e^{b}) = -dZ S^T, dL = -strictlower(dZ v_new^T)
+// -- and the chunk-parallel kernel needs neither Tinv nor a product of three 64 x 64 matrices.  The
+// recurrence itself keeps w^T dv_new ( = (k beta e^{b})^T dZ): dZ is formed off the chain, by the team
+// that stores it.
 // ------------------------------------------------------------------------- //
 template <typename T, int K, int V, int BV>
 __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
@@ -415,7 +421,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
   __shared__ __attribute__((aligned(16))) T s_p[CH * LDC];          // P         [64][64]
   __shared__ __attribute__((aligned(16))) T s_do[CH * LDU];         // do        [64][BV]
   __shared__ __attribute__((aligned(16))) T s_dST[BV * LDK];        // dS'^T     [BV][K]
-  __shared__ __attribute__((aligned(16))) T s_dvn[CH * LDU];        // dv_new    [64][BV] (MFMA operand through transposing reads, and stored)
+  __shared__ __attribute__((aligned(16))) T s_dvn[CH * LDU];        // dv_new    [64][BV] (MFMA operand through transposing reads)
+  __shared__ __attribute__((aligned(16))) T s_dz[sizeof(T) == 2 ? CH * LDU : 8];   // dZ [64][BV] on its way out (2-byte elements; each loader wave its own 16 rows)
   __shared__ __attribute__((aligned(16))) float s_qs[2][64], s_ed[2][64], s_f[64];   // s_f = beta e^{b} (read in phase 1 only: one copy)
   __shared__ float s_dec[2];                                        // gate arrays: buffer it & 1
 
@@ -457,20 +464,16 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
       IOK::mask(P.rq, P.len);
       IOK::store_lds(P.rq, s_q, LDK);
     };
-    // dv_new leaves in blocks of at most 32 columns (the layout of dvnew: see slice_ptr)
-    constexpr int SBW = BV < SLICE_COLS ? BV : SLICE_COLS, NSB = BV / SBW;
-    typedef TileIO<T, CH, SBW> IOS;
-    auto store_results = [&](const typename IOS::Regs (&rdv)[NSB], int c) {
-      const int len = min(CH, sq.len - c * CH);
-#pragma unroll
-      for (int sb = 0; sb < NSB; ++sb)
-        IOS::template store_global<true>(rdv[sb], slice_ptr<T>(a.dvnew, sq.chunk0 + c, h, a.H, V, v0 + SBW * sb), SLICE_COLS, len);
-    };
+    // dZ = Tinv^T dv_new: wave wt of this team forms the 16 tokens 16 wt .. (transposed, so that a lane holds four
+    // consecutive columns of one token), parks them in its own rows of s_dz and stores those rows: no barrier of the
+    // work-group is involved.  dZ lies in memory like v_new (blocks of 32 columns, see slice_ptr).
+    const int wt = wave_id() - 4;
+    constexpr int VEC = ET<T>::VEC, VPRW = BV / VEC, NDZ = (16 * VPRW + 63) / 64;
+    typedef typename ET<T>::vec vec;
 #pragma unroll
     for (int j = 0; j < LPF; ++j) issue_a(pa[j], j);
     wait_all_loads();   // see k_gdn_state_fwd
     typename IOHT::Regs rh;
-    typename IOS::Regs rdv[NSB];
     ring_loop<LPF>(sq.nchunks, [&](auto slot, const int it) {
       constexpr int j = decltype(slot)::value;
       const int c = sq.nchunks - 1 - it;
@@ -478,12 +481,52 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
       stage_a(pa[j]);
       // dS'^T leaves LDS now (the consumers rewrite it after B2)
       IOHT::load_lds(rh, s_dST, LDK);
+      // rows 16 wt .. of Tinv^T (team 2 restages the tile after B2); Tinv is lower triangular
+      typename ET<T>::frag tf[CH / 32];
+#pragma unroll
+      for (int ks = 0; ks < CH / 32; ++ks) tf[ks] = ET<T>::load_frag_t(s_ti, LDC, 32 * ks, 16 * wt, l);
       lds_barrier();                                                                     // B2
       // dv_new of this chunk is complete (the consumers rewrite it after the next B1)
+      f32x4 dz[NB];
 #pragma unroll
-      for (int sb = 0; sb < NSB; ++sb) IOS::load_lds(rdv[sb], s_dvn + SBW * sb, LDU);
+      for (int ni = 0; ni < NB; ++ni) dz[ni] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < CH / 32; ++ks) {
+        if (ks == CH / 32 - 1 || wt < 2) {
+#pragma unroll
+          for (int ni = 0; ni < NB; ++ni) ET<T>::mma(dz[ni], ET<T>::load_frag_t(s_dvn, LDU, 32 * ks, 16 * ni, l), tf[ks]);
+        }
+      }
+      const int len = min(CH, sq.len - c * CH);
+      vec zv[NDZ];
+      if constexpr (sizeof(T) == 2) {
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) acc_to_lds_t<T>(dz[ni], s_dz, LDU, 16 * ni, 16 * wt, l);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int x = 0; x < NDZ; ++x) {
+          const int idx = min(l + 64 * x, 16 * VPRW - 1);
+          zv[x] = *(const vec*)(s_dz + (16 * wt + idx / VPRW) * LDU + (idx % VPRW) * VEC);
+        }
+      }
       IOHT::template store_global<true>(rh, (T*)a.dhs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
-      store_results(rdv, c);
+      if constexpr (sizeof(T) == 2) {
+#pragma unroll
+        for (int x = 0; x < NDZ; ++x) {
+          const int idx = l + 64 * x, tokr = 16 * wt + idx / VPRW, col = (idx % VPRW) * VEC;
+          if (idx < 16 * VPRW && tokr < len)
+            __builtin_nontemporal_store(zv[x], (vec*)(slice_ptr<T>(a.dvnew, sq.chunk0 + c, h, a.H, V, v0 + col) + tokr * SLICE_COLS));
+        }
+      } else {
+        // 4-byte elements: the four consecutive columns a lane holds are one 16-byte vector
+        const int tokr = 16 * wt + (l & 15);
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni)
+          if (tokr < len)
+            *(f32x4*)(slice_ptr<T>(a.dvnew, sq.chunk0 + c, h, a.H, V, v0 + 16 * ni + 4 * (l >> 4)) + tokr * SLICE_COLS) = dz[ni];
+      }
       issue_a(pa[j], it + LPF);
     });
     lds_barrier();
