@@ -3,7 +3,7 @@
 #include "lmoe_gdn_bwd_chunk.hpp"
 
 #ifndef LMOE_BWD_DEPTH
-#define LMOE_BWD_DEPTH 2
+#define LMOE_BWD_DEPTH 3
 #endif
 namespace lmoe {
 

@@ -398,32 +398,40 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd(const lmoe_args a) {
 
 // ------------------------------------------------------------------------- //
 // backward (reverse order over the chunks; it = 0 is the last chunk)
+//     dv_new = scale P^T do + e_d (k dS'),   dZ = Tinv^T dv_new,
+//     dS = e^{b_C} dS' + q^T (scale e_b do) - (k beta e^{b})^T dZ
+//   dZ is the gradient with respect to Z = beta (v - e^{b} k S)  (v_new = Tinv Z, i.e. (I + L) v_new = Z).  It is
+//   what leaves for the chunk-parallel backward instead of dv_new: with it every gradient of the WY form is one
+//   product with dZ -- dv = beta dZ, d(k beta e^{b}) = -dZ S^T, dL = -strictlower(dZ v_new^T) -- and that kernel
+//   needs neither Tinv nor a product of three 64 x 64 matrices.  It also carries the recurrence: w^T dv_new with
+//   w = Tinv (k beta e^{b}) is (k beta e^{b})^T dZ, so w (a 64 x 64 x K product per chunk on the waves of the
+//   chain) is never formed; the 64 x 64 x BV product for dZ runs on the team that stores it while the consumers
+//   add q^T (scale e_b do), at the price of a third barrier per chunk.
 //   team 1, chunk c:   B1 | stage q(c); lift dS'^T(c) out of LDS; read its rows of Tinv^T |
-//                      B2 | dZ(c) = Tinv^T dv_new(c) for its 16 tokens per wave; store dhs(c), dZ(c); prefetch q
-//   team 2, chunk c:   B1 | prefetch k, P, Tinv, do, decay table | B2 | stage those of chunk c-1
-//   consumers, chunk c: dS' -> LDS | B1 | k dS', P^T do, dv_new -> LDS | B2 | dS update
-// What leaves for the chunk-parallel backward is not dv_new but dZ = Tinv^T dv_new, the gradient with
-// respect to Z = beta (v - e^{b} k S) (v_new = Tinv Z, i.e. (I + L) v_new = Z): with it every gradient of
-// the WY form is a product with dZ -- dv = beta dZ, d(k beta e^{b}) = -dZ S^T, dL = -strictlower(dZ v_new^T)
-// -- and the chunk-parallel kernel needs neither Tinv nor a product of three 64 x 64 matrices.  The
-// recurrence itself keeps w^T dv_new ( = (k beta e^{b})^T dZ): dZ is formed off the chain, by the team
-// that stores it.
+//                      B2 | dZ(c) for its 16 tokens per wave -> LDS | B3 | store dhs(c), dZ(c); prefetch q
+//   team 2, chunk c:   B1 | prefetch k, P, Tinv, do, decay table | B2 | stage those of chunk c-1 | B3 |
+//                      (4-byte elements: one k tile, staged behind B3, when the consumers hold its fragments)
+//   consumers, chunk c: dS' -> LDS | B1 | k dS', P^T do, dv_new -> LDS | B2 | dS = e^{b_C} dS + q^T (..);
+//                      fragments of (k beta e^{b})^T | B3 | dS -= (k beta e^{b})^T dZ
 // ------------------------------------------------------------------------- //
 template <typename T, int K, int V, int BV>
 __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
   constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDU = BV + LPAD;
   constexpr int MB = K / 64, NB = BV / 16, KS = K / 32;
   constexpr int LPF = GdnStateCfg<T>::LPF;
+  // 2-byte elements: two k tiles (chunk c is read until B3, chunk c - 1 is staged behind B2); 4-byte elements have
+  // the room for one, which team 2 refills behind B3
+  constexpr bool LATE = sizeof(T) == 4;
+  constexpr int NKB = LATE ? 1 : 2;
   __shared__ __attribute__((aligned(16))) T s_q[CH * LDK];          // q         [64][K]
-  __shared__ __attribute__((aligned(16))) T s_w[CH * LDK];          // w         [64][K]: formed here, Tinv (k beta e^b)
   __shared__ __attribute__((aligned(16))) T s_ti[CH * LDC];         // Tinv      [64][64]
-  __shared__ __attribute__((aligned(16))) T s_k[CH * LDK];          // k         [64][K]
+  __shared__ __attribute__((aligned(16))) T s_k[NKB * CH * LDK];    // k         [64][K]
   __shared__ __attribute__((aligned(16))) T s_p[CH * LDC];          // P         [64][64]
   __shared__ __attribute__((aligned(16))) T s_do[CH * LDU];         // do        [64][BV]
   __shared__ __attribute__((aligned(16))) T s_dST[BV * LDK];        // dS'^T     [BV][K]
   __shared__ __attribute__((aligned(16))) T s_dvn[CH * LDU];        // dv_new    [64][BV] (MFMA operand through transposing reads)
-  __shared__ __attribute__((aligned(16))) T s_dz[sizeof(T) == 2 ? CH * LDU : 8];   // dZ [64][BV] on its way out (2-byte elements; each loader wave its own 16 rows)
-  __shared__ __attribute__((aligned(16))) float s_qs[2][64], s_ed[2][64], s_f[64];   // s_f = beta e^{b} (read in phase 1 only: one copy)
+  __shared__ __attribute__((aligned(16))) T s_dz[CH * LDU];         // dZ        [64][BV] (likewise, and stored)
+  __shared__ __attribute__((aligned(16))) float s_qs[2][64], s_ed[2][64], s_f[NKB][64];   // s_f = beta e^{b}: goes with the k tile
   __shared__ float s_dec[2];                                        // gate arrays: buffer it & 1
 
   constexpr int NVS = V / BV;
@@ -450,7 +458,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
   typedef TileIO<T, BV, K> IOHT;
 
   if (team == 1) {
-    // ------------------------- loaders, ring A (q) and all stores -------------------------
+    // ------------------------- loaders, ring A (q), dZ and all stores ---------------------
     struct PreA { typename IOK::Regs rq; int len; };
     PreA pa[LPF];
     // always issued, chunk index clamped (see k_gdn_state_fwd); `it` counts chunks from the end
@@ -465,8 +473,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
       IOK::store_lds(P.rq, s_q, LDK);
     };
     // dZ = Tinv^T dv_new: wave wt of this team forms the 16 tokens 16 wt .. (transposed, so that a lane holds four
-    // consecutive columns of one token), parks them in its own rows of s_dz and stores those rows: no barrier of the
-    // work-group is involved.  dZ lies in memory like v_new (blocks of 32 columns, see slice_ptr).
+    // consecutive columns of one token) into its rows of s_dz, which the consumers read behind B3 and which it
+    // stores itself.  dZ lies in memory like v_new (blocks of 32 columns, see slice_ptr).
     const int wt = wave_id() - 4;
     constexpr int VEC = ET<T>::VEC, VPRW = BV / VEC, NDZ = (16 * VPRW + 63) / 64;
     typedef typename ET<T>::vec vec;
@@ -479,14 +487,13 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
       const int c = sq.nchunks - 1 - it;
       lds_barrier();                                                                     // B1
       stage_a(pa[j]);
-      // dS'^T leaves LDS now (the consumers rewrite it after B2)
+      // dS'^T leaves LDS now (the consumers rewrite it at the end of the chunk)
       IOHT::load_lds(rh, s_dST, LDK);
-      // rows 16 wt .. of Tinv^T (team 2 restages the tile after B2); Tinv is lower triangular
+      // rows 16 wt .. of Tinv^T (team 2 restages the tile behind B2); Tinv is lower triangular
       typename ET<T>::frag tf[CH / 32];
 #pragma unroll
       for (int ks = 0; ks < CH / 32; ++ks) tf[ks] = ET<T>::load_frag_t(s_ti, LDC, 32 * ks, 16 * wt, l);
-      lds_barrier();                                                                     // B2
-      // dv_new of this chunk is complete (the consumers rewrite it after the next B1)
+      lds_barrier();                                                                     // B2: dv_new of this chunk is complete
       f32x4 dz[NB];
 #pragma unroll
       for (int ni = 0; ni < NB; ++ni) dz[ni] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -497,35 +504,23 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
           for (int ni = 0; ni < NB; ++ni) ET<T>::mma(dz[ni], ET<T>::load_frag_t(s_dvn, LDU, 32 * ks, 16 * ni, l), tf[ks]);
         }
       }
+      // rounded once to the storage type: the recurrence and the chunk-parallel backward see the same values
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) acc_to_lds_t<T>(dz[ni], s_dz, LDU, 16 * ni, 16 * wt, l);
+      lds_barrier();                                                                     // B3
       const int len = min(CH, sq.len - c * CH);
       vec zv[NDZ];
-      if constexpr (sizeof(T) == 2) {
 #pragma unroll
-        for (int ni = 0; ni < NB; ++ni) acc_to_lds_t<T>(dz[ni], s_dz, LDU, 16 * ni, 16 * wt, l);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-        for (int x = 0; x < NDZ; ++x) {
-          const int idx = min(l + 64 * x, 16 * VPRW - 1);
-          zv[x] = *(const vec*)(s_dz + (16 * wt + idx / VPRW) * LDU + (idx % VPRW) * VEC);
-        }
+      for (int x = 0; x < NDZ; ++x) {
+        const int idx = min(l + 64 * x, 16 * VPRW - 1);
+        zv[x] = *(const vec*)(s_dz + (16 * wt + idx / VPRW) * LDU + (idx % VPRW) * VEC);
       }
       IOHT::template store_global<true>(rh, (T*)a.dhs + (((int64_t)(sq.chunk0 + c) * a.H + h) * V + v0) * K, K, BV);
-      if constexpr (sizeof(T) == 2) {
 #pragma unroll
-        for (int x = 0; x < NDZ; ++x) {
-          const int idx = l + 64 * x, tokr = 16 * wt + idx / VPRW, col = (idx % VPRW) * VEC;
-          if (idx < 16 * VPRW && tokr < len)
-            __builtin_nontemporal_store(zv[x], (vec*)(slice_ptr<T>(a.dvnew, sq.chunk0 + c, h, a.H, V, v0 + col) + tokr * SLICE_COLS));
-        }
-      } else {
-        // 4-byte elements: the four consecutive columns a lane holds are one 16-byte vector
-        const int tokr = 16 * wt + (l & 15);
-#pragma unroll
-        for (int ni = 0; ni < NB; ++ni)
-          if (tokr < len)
-            *(f32x4*)(slice_ptr<T>(a.dvnew, sq.chunk0 + c, h, a.H, V, v0 + 16 * ni + 4 * (l >> 4)) + tokr * SLICE_COLS) = dz[ni];
+      for (int x = 0; x < NDZ; ++x) {
+        const int idx = l + 64 * x, tokr = 16 * wt + idx / VPRW, col = (idx % VPRW) * VEC;
+        if (idx < 16 * VPRW && tokr < len)
+          __builtin_nontemporal_store(zv[x], (vec*)(slice_ptr<T>(a.dvnew, sq.chunk0 + c, h, a.H, V, v0 + col) + tokr * SLICE_COLS));
       }
       issue_a(pa[j], it + LPF);
     });
@@ -552,14 +547,15 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
       P.f = gc[3 * CH + l];
     };
     auto stage_b = [&](PreB& P, int buf) {
+      const int kb = LATE ? 0 : buf;
       IOK::mask(P.rk, P.len);
       IOV::mask(P.rd, P.len);
-      IOK::store_lds(P.rk, s_k, LDK);
+      IOK::store_lds(P.rk, s_k + kb * CH * LDK, LDK);
       IOP::store_lds(P.rp, s_p, LDC);       // rows and columns past the end are zero as written
       IOP::store_lds(P.rt, s_ti, LDC);
       IOV::store_lds(P.rd, s_do, LDU);
       if (wave_id() == 8) {
-        s_f[l] = P.f;
+        s_f[kb][l] = P.f;
         s_qs[buf][l] = scale * P.eb;
         s_ed[buf][l] = P.ed;
         if (l == 63) s_dec[buf] = P.eb;
@@ -574,7 +570,13 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
       lds_barrier();                                                                     // B1
       issue_b(pb[j], it + LPF);             // this chunk was staged before the barrier: refill its set
       lds_barrier();                                                                     // B2
-      if (it + 1 < sq.nchunks) stage_b(pb[jn], (it + 1) & 1);
+      if constexpr (!LATE) {
+        if (it + 1 < sq.nchunks) stage_b(pb[jn], (it + 1) & 1);
+      }
+      lds_barrier();                                                                     // B3
+      if constexpr (LATE) {
+        if (it + 1 < sq.nchunks) stage_b(pb[jn], (it + 1) & 1);
+      }
     });
     lds_barrier();
     return;
@@ -602,6 +604,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
   }
   for (int it = 0; it < sq.nchunks; ++it) {
     const int cur = it & 1;
+    const T* s_kc = s_k + (LATE ? 0 : cur) * CH * LDK;
+    const float* s_fc = s_f[LATE ? 0 : cur];
 #pragma unroll
     for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
@@ -609,31 +613,12 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
     lds_barrier();                                                                       // B1
     // t = (k dS')^T  and  dv_loc = (P^T do)^T for the tokens 16 wv .. of the chunk: formed transposed,
     // so that a lane holds four consecutive V columns of one token (see k_gdn_state_fwd)
-    // w = Tinv (k beta e^{b}) is not read from memory (16 KB per chunk and work-group through a request queue
-    // that bounds this kernel) but formed here: wave w forms rows 16 w .. from Tinv (8 KB, its columns scaled
-    // by beta e^{b}) and the k tile, transposed (8-byte LDS writes); phase 2 reads the whole tile after B2.
-    {
-      f32x4 wacc[K / 16];
-#pragma unroll
-      for (int ni = 0; ni < K / 16; ++ni) wacc[ni] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int ks = 0; ks < CH / 32; ++ks) {
-        if (ks == 0 || wv >= 2) {            // Tinv is lower triangular
-          typename ET<T>::frag bt = ET<T>::load_frag(s_ti + (16 * wv + fr) * LDC + 32 * ks + fg);
-          scale_frag8<T>(bt, &s_f[32 * ks + fg]);
-#pragma unroll
-          for (int ni = 0; ni < K / 16; ++ni) ET<T>::mma(wacc[ni], ET<T>::load_frag_t(s_k, LDK, 32 * ks, 16 * ni), bt);
-        }
-      }
-#pragma unroll
-      for (int ni = 0; ni < K / 16; ++ni) acc_to_lds_t<T>(wacc[ni], s_w, LDK, 16 * ni, 16 * wv);
-    }
     f32x4 t[1][NB], dvl[1][NB];
     acc_zero(t);
     acc_zero(dvl);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const typename ET<T>::frag ak = ET<T>::load_frag(s_k + (16 * wv + fr) * LDK + 32 * ks + fg);
+      const typename ET<T>::frag ak = ET<T>::load_frag(s_kc + (16 * wv + fr) * LDK + 32 * ks + fg);
 #pragma unroll
       for (int ni = 0; ni < NB; ++ni)
         ET<T>::mma(t[0][ni], ET<T>::load_frag(s_dST + (16 * ni + fr) * LDK + 32 * ks + fg), ak);
@@ -658,7 +643,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
     for (int ni = 0; ni < NB; ++ni) {
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        // dv_new, rounded once to the storage type (the chunk-parallel backward reads the stored values).
+        // dv_new, rounded once to the storage type.
         // The fused multiply-add is spelled out: left to the compiler, a sum of two products is contracted
         // one way or the other per instantiation, and the wide and narrow slices then differ in the last bit.
         t[0][ni][i] = ET<T>::to_f(ET<T>::from_f(__builtin_fmaf(scale, dvl[0][ni][i], edt * t[0][ni][i])));
@@ -670,27 +655,38 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_bwd(const lmoe_args a) {
     for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
       for (int ni = 0; ni < NB; ++ni) dS[mi][ni] *= dec;
-    // dS += q^T (scale e_b do) - w^T dv_new
+    // dS += q^T (scale e_b do), while team 1 forms dZ; the fragments of (k beta e^{b})^T for what follows B3 are
+    // requested here too
+    typename ET<T>::frag aw[CH / 32][MB];
 #pragma unroll
     for (int ks = 0; ks < CH / 32; ++ks) {
-      typename ET<T>::frag aq[MB], aw[MB], bn[NB];
+      typename ET<T>::frag aq[MB];
 #pragma unroll
       for (int mi = 0; mi < MB; ++mi) {
         aq[mi] = ET<T>::load_frag_t(s_q, LDK, 32 * ks, krow0 + 16 * mi);
-        aw[mi] = ET<T>::load_frag_t(s_w, LDK, 32 * ks, krow0 + 16 * mi);
-      }
-#pragma unroll
-      for (int ni = 0; ni < NB; ++ni) {
-        bn[ni] = ET<T>::load_frag_t(s_dvn, LDU, 32 * ks, 16 * ni);    // rows: V columns, contraction: tokens
-        frag_negate(bn[ni]);
+        aw[ks][mi] = ET<T>::load_frag_t(s_kc, LDK, 32 * ks, krow0 + 16 * mi);
       }
 #pragma unroll
       for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < NB; ++ni) {
-          ET<T>::mma(dS[mi][ni], aq[mi], bdo[ks][ni]);
-          ET<T>::mma(dS[mi][ni], aw[mi], bn[ni]);
-        }
+        for (int ni = 0; ni < NB; ++ni) ET<T>::mma(dS[mi][ni], aq[mi], bdo[ks][ni]);
+#pragma unroll
+      for (int mi = 0; mi < MB; ++mi) {
+        scale_frag8<T>(aw[ks][mi], &s_fc[32 * ks + fg]);
+        frag_negate(aw[ks][mi]);
+      }
+    }
+    lds_barrier();                                                                       // B3: dZ of this chunk is complete
+    // dS -= (k beta e^{b})^T dZ
+#pragma unroll
+    for (int ks = 0; ks < CH / 32; ++ks) {
+      typename ET<T>::frag bn[NB];
+#pragma unroll
+      for (int ni = 0; ni < NB; ++ni) bn[ni] = ET<T>::load_frag_t(s_dz, LDU, 32 * ks, 16 * ni);    // rows: V columns, contraction: tokens
+#pragma unroll
+      for (int mi = 0; mi < MB; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NB; ++ni) ET<T>::mma(dS[mi][ni], aw[ks][mi], bn[ni]);
     }
   }
   lds_barrier();
