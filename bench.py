@@ -247,6 +247,19 @@ def neighbours(lib, rows, D, dev, reps):
                                    frows * (fD + fKp) * 2)
     extra["taylor_featmap_bwd"] = (lambda: lib.lmoe_quad_featmap_bwd(p(fx), p(fy), p(fdx), frows, fD, fKp, *fc, bf, st),
                                    frows * (2 * fD + fKp) * 2)
+    # prologue / epilogue of the gated-delta-rule mixer on the headline shape (rows = B T H): the fused projection
+    # [T, B, H, 3 D] in, q^, k^, silu(v) out; o x swish(gate) with the change of layout
+    pB, pH = 4, 16
+    pT = rows // (pB * pH)
+    pqkv, pdqkv = (torch.randn(pT, pB, pH * 3 * D, device=dev, dtype=torch.bfloat16) for _ in range(2))
+    extra["gdn_qkv_prologue_fwd"] = (lambda: lib.lmoe_gdn_qkv_prologue_fwd(p(pqkv), p(x), p(dy), p(gate), pT, pB, pH, D, bf, 1e-6, st),
+                                     6 * rows * D * 2)
+    extra["gdn_qkv_prologue_bwd"] = (lambda: lib.lmoe_gdn_qkv_prologue_bwd(p(pqkv), p(x), p(dy), p(gate), p(pdqkv), pT, pB, pH, D, bf,
+                                                                           1e-6, st), 9 * rows * D * 2)
+    extra["swish_gate_relayout_fwd"] = (lambda: lib.lmoe_swish_gate_relayout_fwd(p(x), p(gate), p(out), pT, pB, pH * D, bf, st),
+                                        3 * rows * D * 2)
+    extra["swish_gate_relayout_bwd"] = (lambda: lib.lmoe_swish_gate_relayout_bwd(p(x), p(gate), p(dy), p(out), p(out2), pT, pB,
+                                                                                 pH * D, bf, st), 5 * rows * D * 2)
     res = {}
     cases = {n: (f, k * rows * D * 2) for n, (f, k) in cases.items()}
     cases.update(extra)
@@ -366,6 +379,77 @@ def trace_simple_gla_fwd(lib, dev, work_group=16):
             "work_group": work_group, "chunks_averaged": [c0, c1], "period_cycles": round(period),
             "traced_kernel_us": round(traced_us, 1), "cycles_per_us": round(period * nall / traced_us, 1),
             "teams": out}
+
+
+def layer_bench(dev, steps, warmup):
+    """The token-mixer path of the reference's gated-delta-rule layer between its projections (GEMMs left out):
+    q / k / v split, layout change, SiLU, L2 norm, gate construction, the chunk op, layout change back and
+    o * swish(o_gate) (linear_moe/sequence_modeling/linear_attention.py:153-163, 255 around
+    gated_deltanet/gated_deltanet.py:99-114), forward + backward on the headline shape.  `unfused` is the chain of
+    strided copies, row kernels and eager elementwise ops; `fused` the one-pass prologue / epilogue kernels."""
+    import torch
+    import torch.nn.functional as F
+    import linear_moe_amd as L
+    B, T, H, D = 4, 8192, 16, 128
+    g_ = torch.Generator().manual_seed(1004)
+    rn = lambda *s: torch.randn(*s, generator=g_, dtype=torch.float32)
+    bf = lambda x: x.to(torch.bfloat16).to(dev).requires_grad_(True)
+    qkv, o_gate = bf(rn(T, B, H * 3 * D)), bf(rn(T, B, H * D))
+    a, b = bf(rn(B, T, H)), bf(rn(B, T, H))
+    A_log = torch.log(torch.rand(H, generator=g_) * 15 + 1).to(dev).requires_grad_(True)
+    dt_bias = (rn(H) * 0.1).to(dev).requires_grad_(True)
+    dy = rn(T, B, H * D).to(torch.bfloat16).to(dev)
+    leaves = [qkv, o_gate, a, b, A_log, dt_bias]
+
+    def mixer(fused):
+        gk, beta = L.gdn_gates(a, b, A_log, dt_bias)
+        if fused:
+            q, k, v = L.gdn_qkv_prologue(qkv, H, D)
+        else:
+            q, k, v = torch.split(qkv.view(T, B, H, 3 * D), [D, D, D], dim=3)
+            q, k, v = (t.transpose(0, 1).contiguous() for t in (q, k, v))
+            q, k, v = L.silu_l2_norm(q), L.silu_l2_norm(k), F.silu(v)
+        o, _ = L.chunk_gated_delta_rule(q, k, v, gk, beta, head_first=False)
+        if fused:
+            return L.swish_gate_relayout(o, o_gate)
+        return o.transpose(0, 1).reshape(T, B, H * D) * F.silu(o_gate)
+
+    def step(fused):
+        torch.autograd.grad([mixer(fused)], leaves, [dy])
+
+    # the op alone on inputs of the same laws as the headline (what the layer's neighbours are compared with)
+    x = gdn_inputs(B, T, H, D, D, 1004, torch.bfloat16, dev)
+    ol = [x[n].requires_grad_(True) for n in ("q", "k", "v", "g", "beta")]
+
+    def step_op():
+        o, _ = L.chunk_gated_delta_rule(*ol, None, None, False, None, False)
+        torch.autograd.grad([o], ol, [x["do"]])
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps
+
+    for fn in (step_op, lambda: step(False), lambda: step(True)):      # everything warm before anything is timed
+        timed(fn)
+    t_op = timed(step_op)
+    t_un = timed(lambda: step(False))
+    t_fu = timed(lambda: step(True))
+    t_un2 = timed(lambda: step(False))
+    t_fu2 = timed(lambda: step(True))
+    t_un, t_fu = min(t_un, t_un2), min(t_fu, t_fu2)
+    return {"metric": "gated-delta-rule token mixer between its projections, fwd+bwd, ms", "unit": "ms",
+            "config": {"workload": "B=4 T=8192 H=16 D=128 bf16: split, layout, SiLU, L2 norm, gates, chunk op, layout, swish gate"},
+            "steps": steps, "warmup": warmup, "op_alone_ms": t_op * 1e3,
+            "unfused_ms": t_un * 1e3, "fused_ms": t_fu * 1e3,
+            "neighbours_unfused_ms": (t_un - t_op) * 1e3, "neighbours_fused_ms": (t_fu - t_op) * 1e3,
+            "neighbours_share_unfused": (t_un - t_op) / t_un, "neighbours_share_fused": (t_fu - t_op) / t_fu,
+            "tokens_per_s_fused": B * T / t_fu}
 
 
 def other_configs(dev, steps, warmup):
@@ -492,6 +576,9 @@ def main():
     ap.add_argument("--trace-simple-gla-fwd", action="store_true",
                     help="instead of the headline step: the same breakdown for the forward pass of chunk_simple_gla "
                          "on contract configuration 2, one JSON line")
+    ap.add_argument("--layer", action="store_true",
+                    help="instead of the headline step: the token-mixer path of the gated-delta-rule layer between its "
+                         "projections (no GEMMs), with and without the one-pass prologue / epilogue kernels, one JSON line")
     ap.add_argument("--other-configs", action="store_true",
                     help="instead of the headline step: contract configurations 1, 2, 3 and 5, one JSON line")
     args = ap.parse_args()
@@ -521,6 +608,9 @@ def main():
         return
     if args.other_configs:
         print(json.dumps(other_configs(dev, args.steps, args.warmup)))
+        return
+    if args.layer:
+        print(json.dumps(layer_bench(dev, args.steps, args.warmup)))
         return
     if args.trace_simple_gla_fwd:
         print(json.dumps(trace_simple_gla_fwd(lib, dev)))

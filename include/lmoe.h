@@ -171,6 +171,26 @@ int lmoe_silu_l2norm_fwd(const void* x, void* y, int64_t rows, int32_t D, int32_
 int lmoe_silu_l2norm_bwd(const void* x, const void* dy, void* dx, int64_t rows, int32_t D, int32_t dtype, float eps,
                          void* stream);
 
+/* The gated-delta-rule mixer's prologue on its fused projection, in one pass: qkv is [T][B][H][3 D] (q | k | v per
+ * head, contiguous, as linear_moe/sequence_modeling/linear_attention.py:146 produces and :159-163 splits it);
+ *   q = l2norm(silu(q_in)),  k = l2norm(silu(k_in)),  v = silu(v_in)      each [B][T][H][D] contiguous,
+ * i.e. 'n b h d -> b n h d', SiLU and l2_norm_fn of gated_deltanet/gated_deltanet.py:99, :101, :105-106 (eps inside
+ * the root, as lmoe_silu_l2norm_*).  bwd: dqkv [T][B][H][3 D] from dq, dk, dv [B][T][H][D] and qkv.
+ * D in {64, 128}; pointers 16-byte aligned; fp32 arithmetic. */
+int lmoe_gdn_qkv_prologue_fwd(const void* qkv, void* q, void* k, void* v, int32_t T, int32_t B, int32_t H, int32_t D,
+                              int32_t dtype, float eps, void* stream);
+int lmoe_gdn_qkv_prologue_bwd(const void* qkv, const void* dq, const void* dk, const void* dv, void* dqkv, int32_t T,
+                              int32_t B, int32_t H, int32_t D, int32_t dtype, float eps, void* stream);
+
+/* The same mixer's epilogue in one pass: y[t][b][:] = o[b][t][:] * swish(gate[t][b][:]) for rows of W = H D
+ * elements, i.e. 'b n h d -> n b (h d)' of gated_deltanet.py:114 and `o * self.la_gate_fn(o_gate)` of
+ * linear_moe/sequence_modeling/linear_attention.py:255 (la_gate_fn = swish).  bwd: d_o [B][T][W] and
+ * dgate [T][B][W] from dy [T][B][W], o and gate.  W a multiple of 8; pointers 16-byte aligned. */
+int lmoe_swish_gate_relayout_fwd(const void* o, const void* gate, void* y, int32_t T, int32_t B, int32_t W, int32_t dtype,
+                                 void* stream);
+int lmoe_swish_gate_relayout_bwd(const void* o, const void* gate, const void* dy, void* d_o, void* dgate, int32_t T,
+                                 int32_t B, int32_t W, int32_t dtype, void* stream);
+
 /* RMS norm over the last dimension of `rows` contiguous rows of D elements (D in {64, 128, 256}),
  *   y = x rstd w [* gate sigmoid(gate)],  rstd = 1 / sqrt(mean(x^2) + eps),
  * w ([D], element type of x) and gate ([rows][D]) may be null; rstd ([rows] fp32) is written when not null.

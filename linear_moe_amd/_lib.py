@@ -48,7 +48,8 @@ ENTRY_POINTS = (
     "lmoe_chunk_gla_fwd", "lmoe_chunk_gla_bwd",
     "lmoe_chunk_gated_delta_rule_fwd", "lmoe_chunk_gated_delta_rule_bwd",
     "lmoe_launch_stage", "lmoe_selftest_gemm", "lmoe_workspace_bytes", "lmoe_l2norm_fwd", "lmoe_l2norm_bwd",
-    "lmoe_silu_l2norm_fwd", "lmoe_silu_l2norm_bwd", "lmoe_rmsnorm_partials", "lmoe_rmsnorm_fwd", "lmoe_rmsnorm_bwd", "lmoe_rmsnorm_bwd_noalloc",
+    "lmoe_silu_l2norm_fwd", "lmoe_silu_l2norm_bwd", "lmoe_gdn_qkv_prologue_fwd", "lmoe_gdn_qkv_prologue_bwd",
+    "lmoe_swish_gate_relayout_fwd", "lmoe_swish_gate_relayout_bwd", "lmoe_rmsnorm_partials", "lmoe_rmsnorm_fwd", "lmoe_rmsnorm_bwd", "lmoe_rmsnorm_bwd_noalloc",
     "lmoe_gdn_gates_partials", "lmoe_gdn_gates_fwd", "lmoe_gdn_gates_bwd", "lmoe_gla_gate_fwd", "lmoe_gla_gate_bwd",
     "lmoe_hgrn2_gate_fwd", "lmoe_hgrn2_gate_bwd", "lmoe_quad_featmap_features", "lmoe_quad_featmap_fwd",
     "lmoe_quad_featmap_bwd",
@@ -88,6 +89,14 @@ def load() -> C.CDLL:
     lib.lmoe_silu_l2norm_fwd.restype = C.c_int
     lib.lmoe_silu_l2norm_bwd.argtypes = lib.lmoe_l2norm_bwd.argtypes
     lib.lmoe_silu_l2norm_bwd.restype = C.c_int
+    lib.lmoe_gdn_qkv_prologue_fwd.argtypes = [C.c_void_p] * 4 + [C.c_int32] * 5 + [C.c_float, C.c_void_p]
+    lib.lmoe_gdn_qkv_prologue_fwd.restype = C.c_int
+    lib.lmoe_gdn_qkv_prologue_bwd.argtypes = [C.c_void_p] * 5 + [C.c_int32] * 5 + [C.c_float, C.c_void_p]
+    lib.lmoe_gdn_qkv_prologue_bwd.restype = C.c_int
+    lib.lmoe_swish_gate_relayout_fwd.argtypes = [C.c_void_p] * 3 + [C.c_int32] * 4 + [C.c_void_p]
+    lib.lmoe_swish_gate_relayout_fwd.restype = C.c_int
+    lib.lmoe_swish_gate_relayout_bwd.argtypes = [C.c_void_p] * 5 + [C.c_int32] * 4 + [C.c_void_p]
+    lib.lmoe_swish_gate_relayout_bwd.restype = C.c_int
     lib.lmoe_rmsnorm_partials.argtypes = [C.c_int64, C.c_int32, C.c_int32]
     lib.lmoe_rmsnorm_partials.restype = C.c_int32
     lib.lmoe_rmsnorm_fwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32,

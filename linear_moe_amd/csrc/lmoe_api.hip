@@ -206,6 +206,60 @@ int lmoe_silu_l2norm_bwd(const void* x, const void* dy, void* dx, int64_t rows, 
   return launched(nm);
 }
 
+static int check_layerio(const char* nm, int32_t T, int32_t B, int32_t dtype) {
+  if (dtype != LMOE_BF16 && dtype != LMOE_F32) return fail(-2, "%s: dtype must be LMOE_BF16 or LMOE_F32", nm);
+  if (T < 0 || B < 0) return fail(-4, "%s: negative dimension", nm);
+  return 0;
+}
+int lmoe_gdn_qkv_prologue_fwd(const void* qkv, void* q, void* k, void* v, int32_t T, int32_t B, int32_t H, int32_t D,
+                              int32_t dtype, float eps, void* stream) {
+  const char* nm = "lmoe_gdn_qkv_prologue_fwd";
+  if (int r = check_layerio(nm, T, B, dtype)) return r;
+  if (!qkv || !q || !k || !v) return fail(-1, "%s: null pointer", nm);
+  if (D != 64 && D != 128) return fail(-3, "%s: head dimension %d unsupported (64 or 128)", nm, D);
+  if (H <= 0) return fail(-4, "%s: H must be positive", nm);
+  if (((uintptr_t)qkv | (uintptr_t)q | (uintptr_t)k | (uintptr_t)v) & 15) return fail(-9, "%s: pointers must be 16-byte aligned", nm);
+  if ((int64_t)T * B == 0) return 0;
+  lmoe::launch_gdn_qkv_prologue(dtype, D, qkv, nullptr, nullptr, nullptr, q, k, v, T, B, H, eps, false, (hipStream_t)stream);
+  return launched(nm);
+}
+int lmoe_gdn_qkv_prologue_bwd(const void* qkv, const void* dq, const void* dk, const void* dv, void* dqkv, int32_t T,
+                              int32_t B, int32_t H, int32_t D, int32_t dtype, float eps, void* stream) {
+  const char* nm = "lmoe_gdn_qkv_prologue_bwd";
+  if (int r = check_layerio(nm, T, B, dtype)) return r;
+  if (!qkv || !dq || !dk || !dv || !dqkv) return fail(-1, "%s: null pointer", nm);
+  if (D != 64 && D != 128) return fail(-3, "%s: head dimension %d unsupported (64 or 128)", nm, D);
+  if (H <= 0) return fail(-4, "%s: H must be positive", nm);
+  if (((uintptr_t)qkv | (uintptr_t)dq | (uintptr_t)dk | (uintptr_t)dv | (uintptr_t)dqkv) & 15)
+    return fail(-9, "%s: pointers must be 16-byte aligned", nm);
+  if ((int64_t)T * B == 0) return 0;
+  lmoe::launch_gdn_qkv_prologue(dtype, D, qkv, dq, dk, dv, dqkv, nullptr, nullptr, T, B, H, eps, true, (hipStream_t)stream);
+  return launched(nm);
+}
+int lmoe_swish_gate_relayout_fwd(const void* o, const void* gate, void* y, int32_t T, int32_t B, int32_t W, int32_t dtype,
+                                 void* stream) {
+  const char* nm = "lmoe_swish_gate_relayout_fwd";
+  if (int r = check_layerio(nm, T, B, dtype)) return r;
+  if (!o || !gate || !y) return fail(-1, "%s: null pointer", nm);
+  if (W <= 0 || W % 8) return fail(-3, "%s: row length %d must be a positive multiple of 8", nm, W);
+  if (((uintptr_t)o | (uintptr_t)gate | (uintptr_t)y) & 15) return fail(-9, "%s: pointers must be 16-byte aligned", nm);
+  if ((int64_t)T * B == 0) return 0;
+  lmoe::launch_swish_gate_relayout(dtype, o, gate, nullptr, y, nullptr, T, B, W, false, (hipStream_t)stream);
+  return launched(nm);
+}
+int lmoe_swish_gate_relayout_bwd(const void* o, const void* gate, const void* dy, void* d_o, void* dgate, int32_t T,
+                                 int32_t B, int32_t W, int32_t dtype, void* stream) {
+  const char* nm = "lmoe_swish_gate_relayout_bwd";
+  if (int r = check_layerio(nm, T, B, dtype)) return r;
+  if (!o || !gate || !dy || !d_o || !dgate) return fail(-1, "%s: null pointer", nm);
+  if (W <= 0 || W % 8) return fail(-3, "%s: row length %d must be a positive multiple of 8", nm, W);
+  if (((uintptr_t)o | (uintptr_t)gate | (uintptr_t)dy | (uintptr_t)d_o | (uintptr_t)dgate) & 15)
+    return fail(-9, "%s: pointers must be 16-byte aligned", nm);
+  if ((int64_t)T * B == 0) return 0;
+  lmoe::launch_swish_gate_relayout(dtype, o, gate, dy, d_o, dgate, T, B, W, true, (hipStream_t)stream);
+  return launched(nm);
+}
+
 int lmoe_rmsnorm_partials(int64_t rows, int32_t D, int32_t dtype) {
   const char* nm = "lmoe_rmsnorm_partials";
   if (dtype != LMOE_BF16 && dtype != LMOE_F32) return fail(-2, "%s: dtype must be LMOE_BF16 or LMOE_F32", nm);

@@ -60,6 +60,12 @@ int rmsnorm_scratch(float** ptr, int64_t* capacity_floats);
 // y = l2norm(silu(x)) (bwd: out = dx)
 void launch_silu_l2norm(int dtype, int D, const void* x, const void* dy, void* out, int64_t rows, float eps, bool bwd,
                         hipStream_t st);
+// the gated-delta-rule mixer's prologue on the fused projection [T, B, H, 3 D] (fwd: o0, o1, o2 = q^, k^, silu(v) in
+// [B, T, H, D]; bwd: o0 = d(projection)) and its epilogue o * swish(o_gate) with the change of layout (W = H D)
+void launch_gdn_qkv_prologue(int dtype, int D, const void* qkv, const void* dq, const void* dk, const void* dv, void* o0,
+                             void* o1, void* o2, int Tn, int Bn, int H, float eps, bool bwd, hipStream_t st);
+void launch_swish_gate_relayout(int dtype, const void* o, const void* gate, const void* dy, void* out, void* dgate, int Tn,
+                                int Bn, int W, bool bwd, hipStream_t st);
 // gate construction of the gated delta rule (rows x H elements; bwd also fills dparams = [dA_log | ddt_bias])
 void launch_gdn_gates(int dtype, const void* a, const void* b, const float* A_log, const float* dt_bias, float* g,
                       void* beta, const float* dg, const void* dbeta, void* da, void* db, float* part, float* dparams,

@@ -275,6 +275,24 @@ def naive_silu_l2_norm(x: Tensor, eps: float = 1e-6, dtype=torch.float64) -> Ten
     return naive_l2_norm(x * torch.sigmoid(x), eps, dtype)
 
 
+def naive_gdn_qkv_prologue(qkv: Tensor, H: int, D: int, eps: float = 1e-6, dtype=torch.float64):
+    """The gated-delta-rule mixer between its fused projection and the op, step by step as the reference does it:
+    view [T, B, H, 3 D] and split into q, k, v (linear_moe/sequence_modeling/linear_attention.py:159-163),
+    'n b h d -> b n h d' (gated_deltanet/gated_deltanet.py:99), SiLU on all three (:101), l2 norm of q and k
+    (:105-106).  Returns q, k, v, each [B, T, H, D]."""
+    T, B = qkv.shape[0], qkv.shape[1]
+    q, k, v = torch.split(qkv.to(dtype).reshape(T, B, H, 3 * D), [D, D, D], dim=3)
+    q, k, v = (x.transpose(0, 1) for x in (q, k, v))
+    return naive_silu_l2_norm(q, eps, dtype), naive_silu_l2_norm(k, eps, dtype), v * torch.sigmoid(v)
+
+
+def naive_swish_gate_relayout(o: Tensor, o_gate: Tensor, dtype=torch.float64) -> Tensor:
+    """'b n h d -> n b (h d)' (gated_deltanet.py:114), then o * swish(o_gate) (linear_attention.py:255)."""
+    B, T, H, D = o.shape
+    g = o_gate.to(dtype).reshape(T, B, H * D)
+    return o.to(dtype).transpose(0, 1).reshape(T, B, H * D) * (g * torch.sigmoid(g))
+
+
 def naive_gdn_gates(a: Tensor, b: Tensor, A_log: Tensor, dt_bias: Tensor, dtype=torch.float64):
     """(g, beta) of the gated delta rule (linear_moe/sequence_modeling/linear_attention.py:153-154):
     beta = sigmoid(b), g = -exp(A_log) * softplus(a + dt_bias)."""

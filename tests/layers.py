@@ -31,19 +31,27 @@ class GatedDeltaNetLayer(nn.Module):
         qkv = F.linear(x, self.qkv_proj.to(x.dtype)).view(T, B, self.H, 3 * self.D)
         return torch.split(qkv, [self.D, self.D, self.D], dim=3)          # each [T, B, H, D] (a strided view)
 
-    def forward(self, x):
+    def forward(self, x, fused: bool = True):
+        """fused: the one-pass prologue / epilogue kernels; otherwise the chain of copies, row kernels and eager
+        elementwise ops they replace (same numbers to the rounding of the element type)."""
         import linear_moe_amd as L
         T, B, _ = x.shape
-        q, k, v = self._split(x)
         o_gate = F.linear(x, self.o_gate_proj.to(x.dtype))
         xt = x.transpose(0, 1)                                             # [B, T, hidden]
         gk, beta = L.gdn_gates(F.linear(xt, self.a_proj.to(x.dtype)), F.linear(xt, self.beta_proj.to(x.dtype)),
                                self.A_log, self.dt_bias)                   # [B, T, H]: fp32 log-decay, beta
-        q, k, v = (t.transpose(0, 1).contiguous() for t in (q, k, v))      # [B, T, H, D]
-        q, k, v = L.silu_l2_norm(q), L.silu_l2_norm(k), F.silu(v)
+        if fused:
+            q, k, v = L.gdn_qkv_prologue(F.linear(x, self.qkv_proj.to(x.dtype)), self.H, self.D)
+        else:
+            q, k, v = self._split(x)
+            q, k, v = (t.transpose(0, 1).contiguous() for t in (q, k, v))  # [B, T, H, D]
+            q, k, v = L.silu_l2_norm(q), L.silu_l2_norm(k), F.silu(v)
         o, _ = L.chunk_gated_delta_rule(q, k, v, gk, beta, head_first=False)
-        o = o.transpose(0, 1).reshape(T, B, self.H * self.D)               # 'b n h d -> n b (h d)'
-        o = o * F.silu(o_gate)
+        if fused:
+            o = L.swish_gate_relayout(o, o_gate)
+        else:
+            o = o.transpose(0, 1).reshape(T, B, self.H * self.D)           # 'b n h d -> n b (h d)'
+            o = o * F.silu(o_gate)
         return F.linear(o, self.o_proj.to(x.dtype))
 
     def oracle_forward(self, x):

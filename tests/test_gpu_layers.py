@@ -43,3 +43,23 @@ def test_layer_matches_the_oracle_chain(cuda, kind, dtype):
         # absolute sum; in bf16 the rounding of every term (dg comes through bf16 q, k, v) does not cancel with it
         t = 2 * tol if (dtype == torch.bfloat16 and n in ("A_log", "dt_bias")) else tol
         assert max_abs_rel(gd.cpu(), gr) < t, n
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gdn_layer_fused_prologue_epilogue_equals_the_unfused_chain(cuda, dtype):
+    """The one-pass prologue / epilogue kernels against the chain of copies, row kernels and eager ops they replace:
+    the same layer output and hidden-state gradient to the rounding of the element type."""
+    hidden, H, D, T, B = 256, 2, 128, 130, 2
+    layer = GatedDeltaNetLayer(hidden, H, D, seed=6).to(cuda)
+    x = gen(5200, T, B, hidden).to(dtype).to(cuda)
+    dy = gen(5201, T, B, hidden).to(dtype).to(cuda)
+    outs = []
+    for fused in (True, False):
+        xd = x.clone().requires_grad_(True)
+        y = layer(xd, fused=fused)
+        (gx,) = torch.autograd.grad((y * dy).sum(), [xd])
+        outs.append((y.detach(), gx))
+    torch.cuda.synchronize()
+    tol = 2e-5 if dtype == torch.float32 else 3e-2
+    assert max_abs_rel(outs[0][0].cpu(), outs[1][0].cpu()) < tol
+    assert max_abs_rel(outs[0][1].cpu(), outs[1][1].cpu()) < tol

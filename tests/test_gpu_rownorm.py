@@ -134,3 +134,49 @@ def test_gla_gate_fwd_bwd(cuda, dtype, clamp):
     # elements that sit on the clamp within rounding may go either way: compare away from it
     far = (ref.detach() - (clamp if clamp is not None else -1e30)).abs() > 1e-3
     assert max_abs_rel((xd.grad.cpu() * far), (xr.grad * far)) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("D", [64, 128])
+def test_gdn_qkv_prologue_fwd_bwd(cuda, dtype, D):
+    """One pass over the fused projection [T, B, H 3 D] against split -> transpose -> SiLU -> L2 norm."""
+    from linear_moe_amd import gdn_qkv_prologue
+    T, B, H = 37, 3, 5
+    qkv = gen(1300 + D, T, B, H * 3 * D, dtype=dtype)
+    dq, dk, dv = (gen(1301 + D + i, B, T, H, D, dtype=dtype) for i in range(3))
+    xr = qkv.double().requires_grad_(True)
+    rq, rk, rv = naive.naive_gdn_qkv_prologue(xr, H, D)
+    ((rq * dq.double()).sum() + (rk * dk.double()).sum() + (rv * dv.double()).sum()).backward()
+    xd = qkv.to(cuda).requires_grad_(True)
+    q, k, v = gdn_qkv_prologue(xd, H, D)
+    ((q * dq.to(cuda)).sum() + (k * dk.to(cuda)).sum() + (v * dv.to(cuda)).sum()).backward()
+    torch.cuda.synchronize()
+    for got, ref in ((q, rq), (k, rk), (v, rv)):
+        assert got.shape == (B, T, H, D) and got.dtype == dtype and got.is_contiguous()
+        assert max_abs_rel(got.detach().cpu(), ref.detach()) < TOL[dtype]
+    assert xd.grad.shape == qkv.shape
+    assert max_abs_rel(xd.grad.cpu(), xr.grad) < TOL[dtype]
+    # the same numbers as the three-kernel chain it replaces, to the rounding of the element type
+    from linear_moe_amd import silu_l2_norm
+    q3 = silu_l2_norm(xd.detach().view(T, B, H, 3 * D)[..., :D].transpose(0, 1).contiguous())
+    assert max_abs_rel(q.detach().cpu(), q3.cpu()) < (1e-6 if dtype == torch.float32 else 8e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swish_gate_relayout_fwd_bwd(cuda, dtype):
+    from linear_moe_amd import swish_gate_relayout
+    T, B, H, D = 29, 3, 3, 64
+    o = gen(1400, B, T, H, D, dtype=dtype)
+    gate = gen(1401, T, B, H * D, dtype=dtype)
+    dy = gen(1402, T, B, H * D, dtype=dtype)
+    orf, grf = o.double().requires_grad_(True), gate.double().requires_grad_(True)
+    ref = naive.naive_swish_gate_relayout(orf, grf)
+    (ref * dy.double()).sum().backward()
+    od, gd = o.to(cuda).requires_grad_(True), gate.to(cuda).requires_grad_(True)
+    y = swish_gate_relayout(od, gd)
+    (y * dy.to(cuda)).sum().backward()
+    torch.cuda.synchronize()
+    assert y.shape == (T, B, H * D) and y.dtype == dtype
+    assert max_abs_rel(y.detach().cpu(), ref.detach()) < TOL[dtype]
+    assert max_abs_rel(od.grad.cpu(), orf.grad) < TOL[dtype]
+    assert max_abs_rel(gd.grad.cpu(), grf.grad) < TOL[dtype]

@@ -349,6 +349,28 @@ def test_silu_l2_norm_pins():
     assert torch.allclose(naive.naive_silu_l2_norm(x, eps=1e-6), naive.naive_l2_norm(F.silu(x), eps=1e-6), atol=1e-15)
 
 
+def test_mixer_prologue_and_epilogue_layouts_by_hand():
+    """Which element goes where: qkv [T, B, H, 3 D] holds q | k | v per head; outputs are [B, T, H, D]; the
+    epilogue multiplies o[b, t] with the gate row [t, b].  Checked element by element against the formulas."""
+    T, B, H, D = 3, 2, 2, 4
+    qkv = torch.arange(T * B * H * 3 * D, dtype=torch.float64).reshape(T, B, H * 3 * D) / 50 - 1.0
+    q, k, v = naive.naive_gdn_qkv_prologue(qkv, H, D, eps=1e-6)
+    assert q.shape == k.shape == v.shape == (B, T, H, D)
+    silu = lambda x: x / (1 + torch.exp(-x))
+    for (t, b, h) in [(0, 0, 0), (2, 1, 1), (1, 0, 1)]:
+        row = qkv[t, b, h * 3 * D:(h + 1) * 3 * D]
+        sq, sk = silu(row[:D]), silu(row[D:2 * D])
+        assert torch.allclose(q[b, t, h], sq / torch.sqrt((sq * sq).sum() + 1e-6), atol=1e-14)
+        assert torch.allclose(k[b, t, h], sk / torch.sqrt((sk * sk).sum() + 1e-6), atol=1e-14)
+        assert torch.allclose(v[b, t, h], silu(row[2 * D:]), atol=1e-14)
+    o = torch.randn(B, T, H, D, dtype=torch.float64)
+    gate = torch.randn(T, B, H * D, dtype=torch.float64)
+    y = naive.naive_swish_gate_relayout(o, gate)
+    assert y.shape == (T, B, H * D)
+    assert torch.allclose(y[2, 1, D + 1], o[1, 2, 1, 1] * silu(gate[2, 1, D + 1]), atol=1e-14)
+    assert torch.allclose(y[0, 1, 3], o[1, 0, 0, 3] * silu(gate[0, 1, 3]), atol=1e-14)
+
+
 def test_gate_construction_pins():
     """Hand-computed values: softplus(0) = log 2, sigmoid(0) = 1/2, logsigmoid(0) = -log 2; the limits
     softplus(z) -> z and logsigmoid(z) -> z; the clamp; g <= 0 always."""
