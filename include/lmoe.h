@@ -102,6 +102,10 @@ typedef struct lmoe_args {
    * lengths from ending on one long sequence that started late; NULL = as given.  Results do not depend on it.
    * No counterpart in fla, whose state kernels take the sequences in the order of cu_seqlens. */
   const int32_t* seq_order;
+  /* packed input, optional: device int32 [1], the number of chunks of the call when NT above is only an upper bound of
+   * it (tables built on the device from offsets that were never read on the host: chunk_map has NT rows, the first
+   * *nt_dev of them valid; every per-chunk buffer is sized for NT).  NULL = NT is exact.  No counterpart in fla. */
+  const int32_t* nt_dev;
 } lmoe_args;
 
 /* Library version (major*10000 + minor*100 + patch). */

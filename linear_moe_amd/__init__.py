@@ -5,7 +5,7 @@ Drop-in for the ``fla.ops`` callables the reference's token mixers import
 All compute runs in hand-written HIP kernels (``csrc/``) reached through the C ABI of
 ``liblmoe_hip.so`` (``include/lmoe.h``); there is no fallback path.
 """
-from ._host import prepare_cu_seqlens  # noqa: F401
+from ._host import forget_cu_seqlens, prepare_cu_seqlens  # noqa: F401
 from .delta_rule import chunk_delta_rule  # noqa: F401
 from .gated_delta_rule import chunk_gated_delta_rule  # noqa: F401
 from . import lasp  # noqa: F401
@@ -27,4 +27,4 @@ __all__ = ["chunk_simple_gla", "chunk_gla", "chunk_gated_delta_rule", "chunk_del
            "lightning_attn2", "lightning_attn2_no_decay", "l2_norm", "l2_norm_fn", "silu_l2_norm", "gdn_qkv_prologue", "swish_gate_relayout", "rms_norm_fn",
            "rms_norm_swish_gate", "RMSNorm", "gdn_gates", "gla_gate", "fused_recurrent_simple_gla", "fused_recurrent_gla",
            "fused_recurrent_gated_delta_rule", "fused_recurrent_delta_rule", "mom_plan", "mom_pack", "mom_combine", "MomPlan",
-           "prepare_cu_seqlens", "hgrn2_gates", "taylor_feature_map", "rebased_feature_map", "quad_feature_map", "KeyBlocks", "lasp"]
+           "prepare_cu_seqlens", "forget_cu_seqlens", "hgrn2_gates", "taylor_feature_map", "rebased_feature_map", "quad_feature_map", "KeyBlocks", "lasp"]

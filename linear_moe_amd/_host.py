@@ -142,24 +142,31 @@ def _aligned(x: torch.Tensor) -> torch.Tensor:
 
 class SeqPlan:
     """Chunk bookkeeping of one call: number of sequences / chunks and, for packed input,
-    the device tables the kernels index with.  Build through ``seq_plan`` (cached)."""
+    the device tables the kernels index with.  Build through ``seq_plan`` (cached).
+
+    Offsets on the host (a CPU ``cu_seqlens``) are validated and give exact tables.  Offsets on the device are never
+    read back: the tables are built there by a handful of small device operations, sized for the upper bound
+    ``NT <= ceil(T / 64) + N`` of the chunk count (every sequence ends in at most one partial chunk), with the true
+    count in ``nt_dev`` for the kernels; nothing synchronises with the host, so the build can run inside a HIP
+    graph capture and a replay follows the offsets the buffer holds at that time.  Device offsets are trusted
+    (start at 0, non-decreasing, last <= T), as fla trusts them."""
 
     def __init__(self, B: int, T: int, cu_seqlens: Optional[torch.Tensor], device):
         self.cu = None
         self.chunk_map = None
         self.seq_chunk0 = None
         self.seq_order = None
+        self.nt_dev = None
         if cu_seqlens is None:
             self.N = B
             self.NT = B * ((T + CHUNK - 1) // CHUNK)
             return
-        if cu_seqlens.is_cuda and torch.cuda.is_current_stream_capturing():
-            raise RuntimeError("cu_seqlens has no chunk plan yet and one cannot be built while a HIP graph is being "
-                               "captured (it reads the offsets on the host): call the op once with this cu_seqlens "
-                               "tensor, or linear_moe_amd.prepare_cu_seqlens(cu_seqlens, T), before the capture")
-        cu_host = cu_seqlens.detach().to("cpu", torch.int64)
-        if cu_host.dim() != 1 or cu_host.numel() < 2:
+        if cu_seqlens.dim() != 1 or cu_seqlens.numel() < 2:
             raise ValueError("cu_seqlens must be a 1-D tensor of N+1 offsets")
+        if cu_seqlens.is_cuda:
+            self._build_on_device(T, cu_seqlens)
+            return
+        cu_host = cu_seqlens.detach().to("cpu", torch.int64)
         lens = cu_host[1:] - cu_host[:-1]
         if int(cu_host[0]) != 0 or int(cu_host[-1]) != T or bool((lens < 0).any()):
             raise ValueError("cu_seqlens must start at 0, be non-decreasing and end at T")
@@ -179,11 +186,33 @@ class SeqPlan:
         if self.N > 1 and int(nch.max()) != int(nch.min()):
             self.seq_order = torch.argsort(nch, descending=True, stable=True).to(torch.int32).to(device)
 
+    def _build_on_device(self, T: int, cu_seqlens: torch.Tensor):
+        dev = cu_seqlens.device
+        N = cu_seqlens.numel() - 1
+        nt_max = (T + CHUNK - 1) // CHUNK + N
+        cu = cu_seqlens.detach().to(torch.int64)
+        nch = (cu[1:] - cu[:-1] + (CHUNK - 1)) // CHUNK                        # chunks per sequence
+        c0 = torch.cat([cu.new_zeros(1), torch.cumsum(nch, 0)])                 # [N + 1] first chunk of every sequence
+        # rows past the true count belong to a sequence "N" that no kernel ever visits
+        counts = torch.cat([nch, nt_max - c0[-1:]])
+        seq_of = torch.repeat_interleave(torch.arange(N + 1, device=dev), counts, output_size=nt_max)
+        local = torch.arange(nt_max, device=dev) - torch.cat([c0, c0[-1:]])[seq_of]
+        self.N, self.NT = N, nt_max
+        self.cu = cu.to(torch.int32).contiguous()
+        self.chunk_map = torch.stack([seq_of, local], 1).to(torch.int32).contiguous()
+        self.seq_chunk0 = c0.to(torch.int32).contiguous()
+        self.nt_dev = c0[-1:].to(torch.int32).contiguous()
+        if N > 1:
+            self.seq_order = torch.argsort(nch, descending=True, stable=True).to(torch.int32).contiguous()
+
 
 # Plans of the cu_seqlens tensors seen last, newest first.  An entry holds the tensor itself (so its address cannot be
-# reused by another tensor while the entry lives) and its version counter (an in-place change makes a new plan).
-# One packed batch is used by the forward and the backward of every layer: only the first of those calls reads the
-# offsets on the host; the others -- and everything replayed from a HIP graph -- involve no host synchronisation.
+# reused by another tensor while the entry lives) and its version counter (an in-place change through torch makes a new
+# plan).  One packed batch is used by the forward and the backward of every layer: only the first of those calls
+# builds the tables.  A write that torch does not see (another library writing into the buffer, ``.data`` tricks) leaves
+# a stale entry behind: ``forget_cu_seqlens`` drops it.  While a HIP graph is being captured nothing is taken from or
+# put into the cache: the tables of device offsets are built inside the capture, so that a replay follows the offsets
+# the buffer holds when it runs.
 _PLAN_CACHE: list = []
 _PLAN_CACHE_SIZE = 8
 
@@ -191,6 +220,8 @@ _PLAN_CACHE_SIZE = 8
 def seq_plan(B: int, T: int, cu_seqlens: Optional[torch.Tensor], device) -> SeqPlan:
     if cu_seqlens is None:
         return SeqPlan(B, T, None, device)
+    if cu_seqlens.is_cuda and torch.cuda.is_current_stream_capturing():
+        return SeqPlan(B, T, cu_seqlens, device)
     for i, (cu, version, t, dev, plan) in enumerate(_PLAN_CACHE):
         if cu is cu_seqlens and version == cu_seqlens._version and t == T and dev == device:
             if i:
@@ -203,11 +234,21 @@ def seq_plan(B: int, T: int, cu_seqlens: Optional[torch.Tensor], device) -> SeqP
 
 
 def prepare_cu_seqlens(cu_seqlens: torch.Tensor, T: int, device=None) -> SeqPlan:
-    """Build (and cache) the chunk tables of a packed batch ahead of its first use, e.g. before a HIP graph capture or
-    off the critical path of a step.  ``T`` is the total number of tokens (``cu_seqlens[-1]``)."""
+    """Build (and cache) the chunk tables of a packed batch ahead of its first use, off the critical path of a step.
+    ``T`` is the total number of tokens (``cu_seqlens[-1]``; for offsets on the device: the number of rows of the
+    packed tensors, which may exceed it)."""
     if device is None:
         device = cu_seqlens.device if cu_seqlens.is_cuda else torch.device("cuda", torch.cuda.current_device())
     return seq_plan(1, T, cu_seqlens, device)
+
+
+def forget_cu_seqlens(cu_seqlens: Optional[torch.Tensor] = None) -> None:
+    """Drop the cached chunk tables of ``cu_seqlens`` (of every tensor when None): to be called after the offsets were
+    changed by a write that torch's version counter does not see."""
+    if cu_seqlens is None:
+        _PLAN_CACHE.clear()
+    else:
+        _PLAN_CACHE[:] = [e for e in _PLAN_CACHE if e[0] is not cu_seqlens]
 
 
 def _state_check(x: Optional[torch.Tensor], N, H, K, V, name: str) -> Optional[torch.Tensor]:
@@ -230,6 +271,7 @@ def base_args(q, k, v, head_first: bool, scale: Optional[float], plan: SeqPlan, 
         a.chunk_map = plan.chunk_map.data_ptr()
         a.seq_chunk0 = plan.seq_chunk0.data_ptr()
         a.seq_order = ptr(plan.seq_order)
+        a.nt_dev = ptr(plan.nt_dev)
     a.q, a.k, a.v = _desc(q, head_first), _desc(k, head_first), _desc(v, head_first)
     return a
 

@@ -39,6 +39,7 @@ class Args(C.Structure):
         ("dh0", C.c_void_p),
         ("dhs", C.c_void_p), ("dvnew", Tensor4),
         ("seq_order", C.c_void_p),
+        ("nt_dev", C.c_void_p),
     ]
 
 

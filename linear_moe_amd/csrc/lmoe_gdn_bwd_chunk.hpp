@@ -104,7 +104,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
   typedef TileIO<T, CH, BVH> IOV;
   typedef TileIO<T, BVH, K> IOH;
   typedef TileIO<T, CH, K> IOK;
-  const int nitems = a.NT * a.H;
+  const int nitems = num_chunks(a) * a.H;
+  if (nitems <= 0) return;                   // (a chunk count read on the device may be zero)
   const int stride = gridDim.x;
 
   if (threadIdx.x >= 2 * NTHR) {
@@ -252,7 +253,9 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
         dbv[p] = 0.f;
       }
     };
-    const int it0 = blockIdx.x;
+    // (a launch sized by an upper bound of the chunk count may hold work-groups without an item: they stage the last
+    // item like every load past the end and skip the loop)
+    const int it0 = min((int)blockIdx.x, nitems - 1);
     DV d0, d1;
     issue_gates(it0);
     static_for<DEPTH>([&](auto jc) { issue(jc, it0); });
@@ -275,7 +278,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
     }
     int par = 0;
     lds_barrier();                                                                       // first slice staged
-    for (int it = it0; it < nitems; it += stride) {
+    for (int it = blockIdx.x; it < nitems; it += stride) {
       tid = fresh_index(tid) & (NTHR - 1);
       const int cid = it / a.H, h = it % a.H;
       const ChunkInfo ci = chunk_info(a, cid);

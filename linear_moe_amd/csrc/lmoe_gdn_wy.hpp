@@ -146,7 +146,8 @@ __global__ __launch_bounds__(NTHR, (sizeof(T) == 2 ? (SAVE ? 3 : 2) : 1)) void k
   typedef TileIO<T, CH, K> IOK;
   typedef TileIO<T, CH, V> IOV;
   typedef TileIO<T, CH, CH> IO64;
-  const int nitems = a.NT * a.H;
+  const int nitems = num_chunks(a) * a.H;
+  if (nitems <= 0) return;                   // (a chunk count read on the device may be zero)
   // Inputs of an item: one register set, refilled for the next item of this work-group as soon as the
   // current item has consumed a part (v after it is staged, q after q k^T, k after its second staging, gate
   // and beta after the gate phase), so the requests are spread over the item instead of arriving as one

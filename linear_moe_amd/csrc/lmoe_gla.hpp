@@ -116,7 +116,8 @@ __global__ __launch_bounds__(NTHR) void k_gla_intra_fwd(const lmoe_args a) {
   typedef GlaGate<GT, K> GG;
   // persistent: item = (chunk, head); the next item's q, k, g are requested at the top of an item and stay in
   // flight behind its LDS-only barriers (item index clamped: every load is issued)
-  const int nitems = a.NT * a.H;
+  const int nitems = num_chunks(a) * a.H;
+  if (nitems <= 0) return;                   // (a chunk count read on the device may be zero)
   struct Pre { typename IOK::Regs rq, rk; typename GG::Regs rg; };
   Pre pre;
   auto issue = [&](int it) {
@@ -674,6 +675,7 @@ __global__ __launch_bounds__(NTHR) void k_gla_out_fwd(const lmoe_args a) {
   T* s_h = r0; T* s_v = r0;
   T* s_q = r1; T* s_P = r1;
   const int cid = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * BV;
+  if (cid >= num_chunks(a)) return;          // launch sized by an upper bound of the chunk count
   const ChunkInfo ci = chunk_info(a, cid);
   const int wv = wave_id(), l = lane_id();
   typedef TileIO<T, CH, K> IOK;
@@ -839,6 +841,7 @@ __global__ __launch_bounds__(NTHR) void k_gla_bwd_dv(const lmoe_args a) {
   T* s_dh = r0; T* s_do = r0;
   T* s_kd = r1; T* s_P = r1;
   const int cid = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * BV;
+  if (cid >= num_chunks(a)) return;          // launch sized by an upper bound of the chunk count
   const ChunkInfo ci = chunk_info(a, cid);
   const int wv = wave_id(), l = lane_id();
   typedef TileIO<T, CH, K> IOK;
@@ -917,6 +920,7 @@ __global__ __launch_bounds__(NTHR) __attribute__((amdgpu_waves_per_eu((K <= 64 &
   float* smF = (float*)smem_raw;
 
   const int cid = blockIdx.x, h = blockIdx.y;
+  if (cid >= num_chunks(a)) return;          // launch sized by an upper bound of the chunk count
   const ChunkInfo ci = chunk_info(a, cid);
   const int wv = wave_id(), l = lane_id();
   typedef TileIO<T, CH, BVH> IOV;

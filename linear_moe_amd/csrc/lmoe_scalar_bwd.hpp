@@ -38,6 +38,7 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dv(const lmoe_args a) {
   T* s_do = s_rb; T* s_stg = s_rb;
 
   const int cid = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * BV;
+  if (cid >= num_chunks(a)) return;          // launch sized by an upper bound of the chunk count
   const ChunkInfo ci = chunk_info(a, cid);
   const int wv = wave_id(), l = lane_id();
   typedef TileIO<T, CH, K> IOK;
@@ -302,7 +303,8 @@ __global__ __launch_bounds__(2 * NTHR) void k_bwd_dqk(const lmoe_args a) {
   typedef TileIO<T, BVH, K> IOH;
   typedef TileIO<T, CH, K> IOK;
   const lmoe_tensor& vs = a.v;
-  const int nitems = a.NT * a.H;
+  const int nitems = num_chunks(a) * a.H;
+  if (nitems <= 0) return;                   // (a chunk count read on the device may be zero)
   const int stride = gridDim.x;
 
   if (team == 1) {
@@ -531,7 +533,8 @@ __global__ __launch_bounds__(2 * NTHR) void k_bwd_dqkv(const lmoe_args a) {
   typedef TileIO<T, CH, BVH> IOV;
   typedef TileIO<T, BVH, K> IOH;
   typedef TileIO<T, CH, K> IOK;
-  const int nitems = a.NT * a.H;
+  const int nitems = num_chunks(a) * a.H;
+  if (nitems <= 0) return;                   // (a chunk count read on the device may be zero)
   const int stride = gridDim.x;
 
   if (team == 1) {

@@ -43,6 +43,13 @@ __device__ __forceinline__ int seq_at(const lmoe_args& a, int i) {
   return a.seq_order ? as_const(a.seq_order)[i] : i;
 }
 
+// Number of chunks of the call.  Packed input whose offsets never left the device comes with tables sized for an upper
+// bound (a.NT >= the true count, which a.nt_dev holds): launches are sized by the bound, and no kernel touches a
+// chunk index at or beyond the true count.
+__device__ __forceinline__ int num_chunks(const lmoe_args& a) {
+  return a.nt_dev ? as_const(a.nt_dev)[0] : a.NT;
+}
+
 struct ChunkInfo {
   int n;       // sequence
   int b;       // batch row

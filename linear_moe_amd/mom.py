@@ -35,46 +35,66 @@ class MomPlan:
     topk: int
     num_memories: int
     T_total: int
-    max_len: int
     src_token: torch.Tensor     # [T_total] int32: flat token index b * S + t of every packed row
     src_choice: torch.Tensor    # [T_total] int32: flat (token, k) index of every packed row
     row_of: torch.Tensor        # [B * S, topk] int32: packed row of every (token, k), -1 if dropped
-    cu_seqlens: torch.Tensor    # [num_memories * B + 1] int32
-    mem_offsets: torch.Tensor   # [num_memories + 1] int64 (host): row range of every memory
+    cu_seqlens: torch.Tensor    # [num_memories * B + 1] int32 (device)
+    max_len_dev: torch.Tensor   # 0-dim int64 (device): tokens kept per sequence at most
+    mem_offsets_dev: torch.Tensor   # [num_memories + 1] int64 (device): row range of every memory
+
+    # the two figures a caller may want on the host are read back only when asked for
+    @property
+    def max_len(self) -> int:
+        return int(self.max_len_dev)
+
+    @property
+    def mem_offsets(self) -> torch.Tensor:
+        return self.mem_offsets_dev.to("cpu")
 
 
-def mom_plan(selected_memories: torch.Tensor, num_memories: int, capacity: Optional[float] = None) -> MomPlan:
+def mom_plan(selected_memories: torch.Tensor, num_memories: int, capacity: Optional[float] = None,
+             check: bool = False) -> MomPlan:
     """Index tables for ``selected_memories`` [B, S, topk] (as ``torch.topk`` returns them,
-    mom_linear_attention.py:288).  ``capacity``: the reference's capacity factor; ``None`` keeps every token."""
+    mom_linear_attention.py:288).  ``capacity``: the reference's capacity factor; ``None`` keeps every token.
+
+    Built by device operations only (stable sort by (memory, batch row), counts, prefix sums, scatters), as the
+    reference builds its tables on the device (mom_linear_attention.py:28-66).  Without a capacity nothing is read
+    back to the host: every routed token is kept, ``T_total = B * S * topk`` is known up front, and pack -> op ->
+    combine can run inside a HIP graph capture with the plan in it.  With a capacity the number of surviving rows is
+    the one device-to-host read of the call.  ``check`` validates the memory indices (two more reads)."""
     if selected_memories.dim() != 3:
         raise ValueError("selected_memories must be [B, S, topk]")
     B, S, topk = selected_memories.shape
     dev = selected_memories.device
     sel = selected_memories.reshape(-1).to(torch.int64)                        # flat (b, t, k)
-    if sel.numel() and (int(sel.min()) < 0 or int(sel.max()) >= num_memories):
+    if check and sel.numel() and (int(sel.min()) < 0 or int(sel.max()) >= num_memories):
         raise ValueError("selected_memories out of range")
-    flat = torch.arange(sel.numel(), device=dev)
+    n = sel.numel()
+    flat = torch.arange(n, device=dev)
     b_of = flat // (S * topk)
     key = sel * B + b_of                                                       # memory-major sequences
     order = torch.argsort(key, stable=True)                                    # time order inside a sequence
-    lens = torch.bincount(key, minlength=num_memories * B)
-    longest = int(lens.max()) if lens.numel() else 0
-    max_len = longest if capacity is None else min(longest, math.ceil(S * capacity))
-    starts = torch.cumsum(lens, 0) - lens
-    skey = key[order]
-    pos = torch.arange(order.numel(), device=dev) - starts[skey]               # position inside its sequence
-    keep = pos >= (lens[skey] - max_len)                                       # the last max_len survive
-    kept_lens = torch.clamp(lens, max=max_len)
+    lens = torch.zeros(num_memories * B, dtype=torch.int64, device=dev).scatter_add_(0, key, torch.ones_like(key))
+    longest = lens.max() if lens.numel() else torch.zeros((), dtype=torch.int64, device=dev)
+    row_of = torch.full((n,), -1, dtype=torch.int32, device=dev)
     cu = torch.zeros(num_memories * B + 1, dtype=torch.int64, device=dev)
-    cu[1:] = torch.cumsum(kept_lens, 0)
-    rows = order[keep]                                                         # flat (token, k) of packed rows
-    T_total = int(rows.numel())
-    row_of = torch.full((B * S * topk,), -1, dtype=torch.int32, device=dev)
+    if capacity is None:
+        max_len_dev = longest
+        cu[1:] = torch.cumsum(lens, 0)
+        rows, T_total = order, n                                               # every (token, k), sorted
+    else:
+        max_len_dev = torch.clamp(longest, max=math.ceil(S * capacity))
+        starts = torch.cumsum(lens, 0) - lens
+        skey = key[order]
+        pos = flat - starts[skey]                                              # position inside its sequence
+        keep = pos >= (lens[skey] - max_len_dev)                               # the last max_len survive
+        cu[1:] = torch.cumsum(torch.minimum(lens, max_len_dev), 0)
+        rows = order[keep]                                                     # (the one read: how many survive)
+        T_total = int(rows.numel())
     row_of[rows] = torch.arange(T_total, dtype=torch.int32, device=dev)
-    mem_off = cu[::B].to("cpu")
-    return MomPlan(B, S, topk, num_memories, T_total, max_len, (rows // topk).to(torch.int32).contiguous(),
+    return MomPlan(B, S, topk, num_memories, T_total, (rows // topk).to(torch.int32).contiguous(),
                    rows.to(torch.int32).contiguous(), row_of.view(B * S, topk).contiguous(),
-                   cu.to(torch.int32).contiguous(), mem_off)
+                   cu.to(torch.int32).contiguous(), max_len_dev, cu[::B].contiguous())
 
 
 def _dt(t):

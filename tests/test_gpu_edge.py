@@ -106,8 +106,8 @@ def test_no_tokens_at_all(cuda, op):
 def test_forward_and_backward_can_be_captured_in_a_graph(cuda, packed):
     """The library allocates nothing and launches only on the stream it is given, so a forward + backward of the
     gated delta rule can be captured into a HIP graph; every replay (with eager work between the replays)
-    reproduces the eager results bit for bit.  Packed input too: the chunk tables of a cu_seqlens tensor are built
-    by the first (eager) call that sees it, and no later call reads the offsets on the host."""
+    reproduces the eager results bit for bit.  Packed input too: the chunk tables of offsets on the device are built
+    on the device, inside the capture."""
     from linear_moe_amd import _host
     from linear_moe_amd.gated_delta_rule import GDNCall
     B, T, H, K, V = (1, 600, 2, 128, 128) if packed else (2, 300, 2, 128, 128)
@@ -145,12 +145,74 @@ def test_forward_and_backward_can_be_captured_in_a_graph(cuda, packed):
         torch.cuda.synchronize()
         assert all(torch.equal(a, b) for a, b in zip(outs, ref))
     if packed:
-        assert len(_host._PLAN_CACHE) == n_plans
-        # a cu_seqlens tensor without a plan cannot get one during a capture: a clear error, not a sync inside it
-        g2 = torch.cuda.CUDAGraph()
-        with pytest.raises(RuntimeError, match="before the capture"):
-            with torch.cuda.graph(g2):
-                call.forward(q, k, v, g, beta, None, h0, True, cu.clone(), False)
+        assert len(_host._PLAN_CACHE) == n_plans        # a capture neither reads nor fills the cache
+
+
+@pytest.mark.parametrize("op", OPS)
+def test_offsets_on_the_device_give_the_bits_of_offsets_on_the_host(cuda, op):
+    """Offsets handed over on the device are never read back: the chunk tables are built there, sized for an upper
+    bound of the chunk count, with the true count on the device for the kernels.  Same call with the offsets as a host
+    tensor (validated, exact tables): the same bits, outputs, states and every gradient."""
+    lens = [70, 0, 300, 1, 64, 129]
+    T, N, H, K, V = sum(lens), len(lens), 3, 64, 128
+    ins = {n: x.to(cuda) for n, x in _inputs(op, T, H, K, V, torch.bfloat16, 3500).items()}
+    h0 = (gen(3510, N, H, K, V) * 0.1).to(cuda)
+    do, dht = gen(3511, 1, T, H, V, dtype=torch.bfloat16).to(cuda), gen(3512, N, H, K, V).to(cuda)
+    cu_host = torch.tensor([0] + lens, dtype=torch.int32).cumsum(0).to(torch.int32)
+    names = list(ins)
+
+    def run(cu):
+        leaves = {n: x.clone().requires_grad_(True) for n, x in dict(ins, h0=h0).items()}
+        o, ht = _call(op, leaves, leaves["h0"], cu, True)
+        grads = torch.autograd.grad([o, ht], [leaves[n] for n in names + ["h0"]], [do, dht])
+        return (o.detach(), ht.detach()) + tuple(grads)
+
+    from linear_moe_amd import _host
+    on_dev = run(cu_host.to(cuda))
+    on_host = run(cu_host)
+    torch.cuda.synchronize()
+    plan = _host.prepare_cu_seqlens(cu_host.to(cuda), T)
+    assert plan.nt_dev is not None and int(plan.nt_dev) == sum((x + 63) // 64 for x in lens) < plan.NT
+    for a, b in zip(on_dev, on_host):
+        assert torch.equal(a, b)
+
+
+def test_a_captured_packed_step_follows_the_offsets_it_finds_at_replay(cuda):
+    """A forward + backward on packed input captured with its offsets in a static device buffer: the chunk tables are
+    part of the graph, so after new offsets (other lengths, another number of chunks) were copied into the buffer a
+    replay gives what an eager call on those offsets gives, bit for bit."""
+    from linear_moe_amd.gated_delta_rule import GDNCall
+    T, H, K, V, dt = 640, 2, 128, 128, torch.bfloat16
+    q, k = gen(3600, 1, T, H, K, dtype=dt).to(cuda), F.normalize(gen(3601, 1, T, H, K), dim=-1).to(dt).to(cuda)
+    v, do = gen(3602, 1, T, H, V, dtype=dt).to(cuda), gen(3603, 1, T, H, V, dtype=dt).to(cuda)
+    g, beta = F.logsigmoid(gen(3604, 1, T, H)).to(cuda), torch.sigmoid(gen(3605, 1, T, H)).to(dt).to(cuda)
+    offsets = [[0, 70, 70, 333, 640], [0, 1, 200, 639, 640], [0, 128, 256, 384, 640]]      # 11, 12 and 10 chunks
+    h0, dht = (0.1 * gen(3606, 4, H, K, V)).to(cuda), gen(3607, 4, H, K, V).to(cuda)
+
+    def step(call, cu):
+        o, ht = call.forward(q, k, v, g, beta, None, h0, True, cu, False)
+        return (o, ht) + tuple(x for x in call.backward(do, dht) if x is not None)
+
+    refs = [[x.clone() for x in step(GDNCall(keep=True), torch.tensor(o_, dtype=torch.int32, device=cuda))] for o_ in offsets]
+    cu = torch.tensor(offsets[0], dtype=torch.int32, device=cuda)
+    call = GDNCall(keep=True)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step(call, cu)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = step(call, cu)
+    for i in (0, 1, 2, 1, 0):
+        cu.copy_(torch.tensor(offsets[i], dtype=torch.int32))
+        for x in outs:
+            x.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(outs, refs[i]):
+            assert torch.equal(a, b), i
 
 
 @pytest.mark.parametrize("op", OPS)

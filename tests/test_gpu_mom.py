@@ -134,3 +134,46 @@ def test_packed_flow_equals_the_padded_flow_around_the_gated_delta_rule(cuda, ca
     torch.cuda.synchronize()
     assert out.shape == (B, S, H * V)
     assert max_abs_rel(out.cpu(), ref) < 1e-5
+
+
+def test_routing_to_result_captures_into_a_graph_and_follows_new_routing_at_replay(cuda):
+    """Without a capacity nothing of the routing is read on the host: plan, pack, the packed op and combine are
+    device work only, so the whole path from the selected memories to the mixed result captures into a HIP graph, and
+    a replay after other routing was copied into the captured buffers gives what an eager run on that routing gives."""
+    from linear_moe_amd import chunk_gated_delta_rule, mom_combine, mom_pack, mom_plan
+    B, S, E, topk, H, K, V = 2, 150, 3, 2, 2, 64, 64
+    d = lambda t: t.to(cuda)
+    q = d(F.normalize(gen(3302, B, S, H * K).view(B, S, H, K), dim=-1).reshape(B, S, H * K))
+    k = d(F.normalize(gen(3303, B, S, H * K).view(B, S, H, K), dim=-1).reshape(B, S, H * K))
+    v = d(gen(3304, B, S, H * V))
+    gb = d(torch.cat([-F.softplus(gen(3305, B, S, H)) * 0.3, torch.sigmoid(gen(3306, B, S, H)), torch.zeros(B, S, 8 - 2 * H)], -1))
+    routings = [routing(3310 + i, B, S, E, topk) for i in range(3)]
+    sel, wts = d(routings[0][1]).clone(), d(routings[0][0]).clone()
+
+    def run(sel, wts):
+        plan = mom_plan(sel, E)
+        T = plan.T_total
+        assert T == B * S * topk
+        qp, kp, vp, gbp = (mom_pack(t, plan) for t in (q, k, v, gb))
+        o, _ = chunk_gated_delta_rule(qp.view(1, T, H, K), kp.view(1, T, H, K), vp.view(1, T, H, V),
+                                      gbp[:, :H].contiguous().view(1, T, H), gbp[:, H:2 * H].contiguous().view(1, T, H),
+                                      cu_seqlens=plan.cu_seqlens)
+        return mom_combine(o.reshape(T, H * V), plan, wts)
+
+    refs = [run(d(s_), d(w_)).clone() for (w_, s_) in routings]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run(sel, wts)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = run(sel, wts)
+    for i in (0, 1, 2, 0):
+        sel.copy_(d(routings[i][1]))
+        wts.copy_(d(routings[i][0]))
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, refs[i]), i

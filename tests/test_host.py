@@ -163,6 +163,27 @@ def test_seq_plan_tables():
             SeqPlan(1, 270, torch.tensor(bad), "cpu")
 
 
+def test_tables_built_without_reading_the_offsets_equal_the_validated_ones():
+    """The table builder for offsets that stay on the device (run here on CPU tensors: it is made of torch operations
+    only, none of which needs a value on the host) against the host path: the first NT rows of chunk_map, the first
+    chunks, the count and the order agree; the rows past the count belong to no sequence."""
+    from linear_moe_amd._host import SeqPlan
+    for lens in ([5, 64, 0, 200, 1, 65], [64, 64], [1], [0, 0, 130]):
+        T = sum(lens)
+        cu = torch.tensor([0] + lens).cumsum(0).to(torch.int32)
+        exact = SeqPlan(1, T, cu, "cpu")
+        dev = SeqPlan.__new__(SeqPlan)
+        dev.seq_order = None
+        dev._build_on_device(T, cu)
+        nt = int(dev.nt_dev)
+        assert nt == exact.NT <= dev.NT == (T + 63) // 64 + len(lens)
+        assert torch.equal(dev.chunk_map[:nt], exact.chunk_map) and torch.equal(dev.seq_chunk0, exact.seq_chunk0)
+        assert (dev.chunk_map[nt:, 0] == len(lens)).all()
+        assert dev.chunk_map.dtype == dev.seq_chunk0.dtype == dev.nt_dev.dtype == torch.int32
+        if exact.seq_order is not None:
+            assert torch.equal(dev.seq_order, exact.seq_order)
+
+
 def test_seq_plan_is_built_once_per_cu_seqlens_tensor():
     """The chunk tables of a packed batch are built on the first call that sees its cu_seqlens tensor; later calls with
     the same tensor (the other layers, the backward, every step that reuses the batch) take them from the cache without
