@@ -115,3 +115,91 @@ class GLALayer(nn.Module):
         o = o.permute(2, 0, 1, 3).reshape(T, B, self.H * self.D)
         o = o * F.silu(o_gate)
         return o @ P(self.o_proj).T
+
+
+class _CoreBase(nn.Module):
+    """Shared by the three core modules below: q, k, v arrive as [T, B, H, D] (what LinearAttention.forward hands
+    to ``core_linear_attention``, linear_attention.py:248-252), go to 'b h n d', and the result returns as
+    'n b (h d)' behind an RMS norm over head_v_dim."""
+
+    def __init__(self, heads: int, head_dim: int, seed: int, eps: float = 1e-5):
+        super().__init__()
+        g = torch.Generator().manual_seed(seed)
+        self.H, self.D, self.eps = heads, head_dim, eps
+        self.norm_weight = nn.Parameter(1 + 0.1 * torch.randn(head_dim, generator=g))
+
+    @staticmethod
+    def _in(x):
+        return x.permute(1, 2, 0, 3)                                                  # 'n b h d -> b h n d'
+
+    def _out(self, o, norm):
+        o = norm(o)
+        T = o.shape[2]
+        return o.permute(2, 0, 1, 3).reshape(T, o.shape[0], self.H * self.D)          # 'b h n d -> n b (h d)'
+
+
+class RetentionCore(_CoreBase):
+    """Retention.forward (retention/retention.py:78-96): feature map (swish) on q, k, chunk_retention, RMSNorm."""
+
+    def forward(self, q, k, v):
+        import linear_moe_amd as L
+        q, k, v = (self._in(x).contiguous() for x in (q, k, v))
+        q, k = F.silu(q), F.silu(k)
+        o, _ = L.chunk_retention(q, k, v)
+        return self._out(o, lambda x: L.rms_norm_fn(x, self.norm_weight.to(x.dtype), None, eps=self.eps))
+
+    def oracle_forward(self, q, k, v):
+        q, k, v = (self._in(x) for x in (q, k, v))
+        o, _ = naive.naive_retention(F.silu(q), F.silu(k), v)
+        return self._out(o, lambda x: naive.naive_rms_norm(x, self.norm_weight.double(), None, self.eps))
+
+
+class BasicLinearAttentionCore(_CoreBase):
+    """BasicLinearAttention.forward (basic_linear_attention/basic_linear_attention.py:114-138) with the 'elu' feature
+    map (:75-79), la_norm_q / la_norm_k (:127-130) and chunk_linear_attn(normalize=la_do_feature_map_norm) at its
+    default scale (:133)."""
+
+    def __init__(self, heads, head_dim, seed, normalize=True, norm_qk=True):
+        super().__init__(heads, head_dim, seed)
+        self.normalize, self.norm_qk = normalize, norm_qk
+
+    def _maps(self, q, k):
+        q, k = F.elu(q) + 1, F.elu(k) + 1
+        if self.norm_qk:
+            q, k = q / (q.sum(-1, True) + 1e-4), k / (k.sum(-1, True) + 1e-4)
+        return q, k
+
+    def forward(self, q, k, v):
+        import linear_moe_amd as L
+        q, k, v = (self._in(x).contiguous() for x in (q, k, v))
+        q, k = self._maps(q, k)
+        o, _ = L.chunk_linear_attn(q, k, v, normalize=self.normalize)
+        return self._out(o, lambda x: L.rms_norm_fn(x, self.norm_weight.to(x.dtype), None, eps=self.eps))
+
+    def oracle_forward(self, q, k, v):
+        q, k, v = (self._in(x) for x in (q, k, v))
+        q, k = self._maps(q, k)
+        o, _ = naive.naive_linear_attn(q, k, v, normalize=self.normalize)
+        return self._out(o, lambda x: naive.naive_rms_norm(x, self.norm_weight.double(), None, self.eps))
+
+
+class LightningCore(_CoreBase):
+    """LightningAttention.forward (lightning_attention/lightning_attention.py:108-126) on tensor-parallel rank `rank` of
+    `tp`: the slopes of all `heads * tp` heads (:79-105), chunked per rank as :54-61 does, feature map (swish) on q, k,
+    lightning_attn2(q, k, v, slope_rate), RMSNorm."""
+
+    def __init__(self, heads, head_dim, seed, tp=1, rank=0):
+        super().__init__(heads, head_dim, seed)
+        slopes = naive.lightning_slopes(heads * tp).reshape(heads * tp, 1, 1)
+        self.register_buffer("slope_rate", torch.chunk(slopes, tp, 0)[rank].float())
+
+    def forward(self, q, k, v):
+        import linear_moe_amd as L
+        q, k, v = (self._in(x).contiguous() for x in (q, k, v))
+        o = L.lightning_attn2(F.silu(q), F.silu(k), v, self.slope_rate)
+        return self._out(o, lambda x: L.rms_norm_fn(x, self.norm_weight.to(x.dtype), None, eps=self.eps))
+
+    def oracle_forward(self, q, k, v):
+        q, k, v = (self._in(x) for x in (q, k, v))
+        o = naive.naive_lightning_attn2(F.silu(q), F.silu(k), v, self.slope_rate.double())
+        return self._out(o, lambda x: naive.naive_rms_norm(x, self.norm_weight.double(), None, self.eps))

@@ -63,3 +63,43 @@ def test_gdn_layer_fused_prologue_epilogue_equals_the_unfused_chain(cuda, dtype)
     tol = 2e-5 if dtype == torch.float32 else 3e-2
     assert max_abs_rel(outs[0][0].cpu(), outs[1][0].cpu()) < tol
     assert max_abs_rel(outs[0][1].cpu(), outs[1][1].cpu()) < tol
+
+
+CORES = {
+    "retention": lambda: __import__("tests.layers", fromlist=["x"]).RetentionCore(4, 64, seed=7),
+    "basic_normalized": lambda: __import__("tests.layers", fromlist=["x"]).BasicLinearAttentionCore(3, 64, seed=8),
+    "basic_plain": lambda: __import__("tests.layers", fromlist=["x"]).BasicLinearAttentionCore(3, 64, seed=8, normalize=False, norm_qk=False),
+    "lightning_tp2_rank1": lambda: __import__("tests.layers", fromlist=["x"]).LightningCore(6, 128, seed=9, tp=2, rank=1),
+}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("kind", list(CORES))
+def test_core_modules_of_the_other_dispatch_branches(cuda, kind, dtype):
+    """The core modules LinearAttention.forward dispatches to besides the gated delta rule and GLA
+    (linear_attention.py:218-252): Retention, BasicLinearAttention (with and without the feature-map normalisation and
+    the normaliser of chunk_linear_attn at its default scale), LightningAttention with the slopes of one tensor-parallel
+    rank -- each in the reference's order of operations on the GPU kernels, output and dq, dk, dv and the norm weight
+    against the same chain of fp64 oracle functions."""
+    core = CORES[kind]()
+    T, B, H, D = 150, 2, core.H, core.D
+    q, k, v = (gen(5300 + i, T, B, H, D).to(dtype) for i in range(3))
+    dy = gen(5303, T, B, H * D).to(dtype)
+    ref_core = CORES[kind]()
+    if dtype == torch.bfloat16:
+        with torch.no_grad():
+            ref_core.norm_weight.copy_(ref_core.norm_weight.to(dtype).float())
+    lr = [x.double().requires_grad_(True) for x in (q, k, v)]
+    yr = ref_core.oracle_forward(*lr)
+    gr = torch.autograd.grad((yr * dy.double()).sum(), lr + [ref_core.norm_weight])
+    core = core.to(cuda)
+    ld = [x.to(cuda).requires_grad_(True) for x in (q, k, v)]
+    y = core(*ld)
+    assert y.shape == (T, B, H * D) and y.dtype == dtype
+    gd = torch.autograd.grad((y * dy.to(cuda)).sum(), ld + [core.norm_weight])
+    torch.cuda.synchronize()
+    # three chained roundings (feature map, op, norm); the normalised basic module divides two rounded sums
+    tol = 5e-5 if dtype == torch.float32 else 4e-2
+    assert max_abs_rel(y.detach().cpu(), yr.detach()) < tol
+    for n, a, b in zip(("dq", "dk", "dv", "dw"), gd, gr):
+        assert max_abs_rel(a.cpu(), b) < tol, n
