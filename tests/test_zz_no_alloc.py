@@ -74,3 +74,40 @@ def test_rmsnorm_bwd_noalloc_rejects_bad_arguments(cuda):
     rc = lib.lmoe_rmsnorm_bwd_noalloc(x.data_ptr(), None, None, x.data_ptr(), x.data_ptr(), None, dw.data_ptr(), 4, 96,
                                       _lib.LMOE_BF16, 1e-5, st)
     assert rc < 0
+
+
+def test_rmsnorm_bwd_noalloc_inside_a_graph_capture(cuda):
+    """What the entry point is for: a caller under HIP graph capture.  The address of the scratch array is looked up on
+    the first call on a device, which is host work that does not belong into a capture: one eager call (any size)
+    resolves it, the captured call then only launches.  Replays, with eager work and another eager call of the entry
+    point on a smaller input between them, reproduce the workspace entry point bit for bit."""
+    from linear_moe_amd import _lib
+    lib = _lib.load()
+    rows, D, dt = 3000, 128, _lib.LMOE_BF16
+    x, dy, gate = (gen(4200 + i, rows, D, dtype=torch.bfloat16).to(cuda) for i in range(3))
+    w = (1 + 0.1 * gen(4203, D)).to(torch.bfloat16).to(cuda)
+    p = lambda t: t.data_ptr()
+    part = torch.empty(lib.lmoe_rmsnorm_partials(rows, D, dt), D, dtype=torch.float32, device=cuda)
+    ref = [torch.empty_like(x), torch.empty_like(x), torch.empty(D, dtype=torch.float32, device=cuda)]
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _lib.check(lib.lmoe_rmsnorm_bwd(p(x), p(w), p(gate), p(dy), p(ref[0]), p(ref[1]), p(part), p(ref[2]), rows, D, dt, 1e-5, st), "ref")
+    out = [torch.empty_like(x), torch.empty_like(x), torch.empty(D, dtype=torch.float32, device=cuda)]
+    small = [torch.empty(7, D, dtype=torch.bfloat16, device=cuda), torch.empty(D, dtype=torch.float32, device=cuda)]
+
+    def call(stream, n, dx, dgate, dw):
+        _lib.check(lib.lmoe_rmsnorm_bwd_noalloc(p(x), p(w), p(gate), p(dy), p(dx), p(dgate), p(dw), n, D, dt, 1e-5,
+                                                C.c_void_p(stream.cuda_stream)), "noalloc")
+
+    call(torch.cuda.current_stream(), 7, small[0], small[0], small[1])       # resolves the scratch address, eagerly
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(torch.cuda.current_stream(), rows, *out)
+    for _ in range(3):
+        for t in out:
+            t.zero_()
+        call(torch.cuda.current_stream(), 7, small[0], small[0], small[1])   # shares the array: overwrites a prefix of it
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert all(torch.equal(a, b) for a, b in zip(out, ref))
