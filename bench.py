@@ -38,16 +38,16 @@ STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_gdn_state_fwd_reg", 4: "k_gdn_state_bwd"
 # sources (kernel_sources_sha16()) at that time, and a build whose sources differ reports traffic = null
 # rather than a stale number.
 CALIB_COPY_BYTES = 256 << 20
-MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237243472, "k_gdn_state_fwd_reg": 1119040061, "k_gdn_state_bwd": 946326302, "k_gdn_bwd_chunk": 1898773639}
-TRAFFIC_SOURCES_SHA16 = "a0ad676c6194a4cd"
+MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237243453, "k_gdn_state_fwd_reg": 1119409063, "k_gdn_state_bwd": 945960392, "k_gdn_bwd_chunk": 1834053754}
+TRAFFIC_SOURCES_SHA16 = "990483523988793a"
 TRAFFIC_SOURCES = ("lmoe_common.hpp", "lmoe_seq.hpp", "lmoe_gdn_wy.hpp", "lmoe_gdn_state.hpp", "lmoe_gdn_state_reg.hpp", "lmoe_gdn_bwd_chunk.hpp",
                    "lmoe_gdn_fwd.hip", "lmoe_gdn_state.hip", "lmoe_gdn_bwd.hip")
 
 
 # HBM bytes per call of the other contract configurations (bench.py --other-configs), same counters and scaling,
 # summed over the kernels of the call; key = configuration number
-OTHER_TRAFFIC = {"1": 2230713, "2": 272912955, "3": 1281633960, "5": 16910222101, "6": 1444950284}
-OTHER_TRAFFIC_SHA16 = "b72963f72fb40331"
+OTHER_TRAFFIC = {"1": 2230718, "2": 272913415, "3": 1281283146, "5": 16675972468, "6": 1444848249}
+OTHER_TRAFFIC_SHA16 = "e93cf3e3fb42e6d6"
 
 
 def all_sources_sha16():

@@ -138,8 +138,15 @@ def chunk_forward(op: str, q, k, v, g=None, beta=None, scale=None, h0=None, C: i
 # backward (manual, per chunk)
 # --------------------------------------------------------------------------- #
 def chunk_backward(op: str, q, k, v, g, beta, scale, h0, do, dht, saved, C: int = CHUNK,
-                   dtype=torch.float32):
-    """Manual backward.  Returns dq, dk, dv, dg, dbeta, dh0 (entries None where not applicable)."""
+                   dtype=torch.float32, solve_form: bool = False):
+    """Manual backward.  Returns dq, dk, dv, dg, dbeta, dh0 (entries None where not applicable).
+
+    ``solve_form`` (gated delta rule): the backward of the WY form written through dZ = T^T dv_new, the gradient
+    with respect to Z = beta (v - e^b k S) (v_new = T Z solves (I + L) v_new = Z): dv = beta dZ,
+    d(k beta e^b) = -dZ S^T, dL = -strictlower(dZ v_new^T), and the state recurrence subtracts (k beta e^b)^T dZ.
+    It is what the HIP kernels compute; the default is the w / u form (dT = du v_b^T + dw k_bg^T,
+    dL = -T^T dT T^T), which fla's kernels follow.  Both are pinned against autograd and against each other in
+    tests/test_oracle_pins.py."""
     B, H, T, K = q.shape
     V = v.shape[-1]
     scale = K ** -0.5 if scale is None else scale
@@ -180,7 +187,11 @@ def chunk_backward(op: str, q, k, v, g, beta, scale, h0, do, dht, saved, C: int 
         dec = decay[:, :, c]
         dec = dec[..., None] if vector else dec[..., None, None]
         dS_new = scale * (q_g[:, :, c].transpose(-1, -2) @ doc[:, :, c]) + dec * dS
-        if op == 'gdn':
+        if op == 'gdn' and solve_form:
+            dz_c = saved['Tm'][:, :, c].transpose(-1, -2) @ dvn[c]
+            kbg_c = kc[:, :, c] * _chunks(beta, C)[:, :, c][..., None] * e_b[:, :, c]
+            dS_new = dS_new - kbg_c.transpose(-1, -2) @ dz_c
+        elif op == 'gdn':
             dS_new = dS_new - w[:, :, c].transpose(-1, -2) @ dvn[c]
         dS = dS_new
     dh0 = dS
@@ -225,12 +236,18 @@ def chunk_backward(op: str, q, k, v, g, beta, scale, h0, do, dht, saved, C: int 
         dPG = dP * Gam
         dq = dq_inter + dPG @ kc
         dk = dk_d * e_d + dPG.transpose(-1, -2) @ qc
-        dw = -(dvn @ hs.transpose(-1, -2))
-        du = dvn
-        dT = du @ v_b.transpose(-1, -2) + dw @ k_bg.transpose(-1, -2)
-        dv_b = Tm.transpose(-1, -2) @ du
-        dk_bg = Tm.transpose(-1, -2) @ dw
-        dL = -(Tm.transpose(-1, -2) @ dT @ Tm.transpose(-1, -2)) * mask_s
+        if solve_form:
+            dZ = Tm.transpose(-1, -2) @ dvn
+            dv_b = dZ
+            dk_bg = -(dZ @ hs.transpose(-1, -2))
+            dL = -(dZ @ vnew.transpose(-1, -2)) * mask_s
+        else:
+            dw = -(dvn @ hs.transpose(-1, -2))
+            du = dvn
+            dT = du @ v_b.transpose(-1, -2) + dw @ k_bg.transpose(-1, -2)
+            dv_b = Tm.transpose(-1, -2) @ du
+            dk_bg = Tm.transpose(-1, -2) @ dw
+            dL = -(Tm.transpose(-1, -2) @ dT @ Tm.transpose(-1, -2)) * mask_s
         dM = dL * Gam_s
         dk_b = dM @ kc + dk_bg * e_b
         dk = dk + dM.transpose(-1, -2) @ k_b + dk_b * bc

@@ -284,6 +284,27 @@ def test_chunked_matches_naive_and_autograd(op, C):
         assert torch.allclose(a, b, atol=1e-9 * max(1.0, a.abs().max().item()))
 
 
+def test_wy_backward_through_dZ_equals_the_w_u_form_and_autograd():
+    """The form of the gated delta rule's backward that the HIP kernels compute (everything through
+    dZ = T^T dv_new: no product with T in the chunk-parallel part, no w in the state recurrence) against the
+    w / u form and against autograd through the token recurrence, in fp64 on a case with a partial last chunk, an
+    initial state and a gradient of the final state."""
+    B, H, T, K, V = 1, 2, 200, 16, 24
+    q, k = rnd(81, B, H, T, K), F.normalize(rnd(82, B, H, T, K), dim=-1)
+    v, do = rnd(83, B, H, T, V), rnd(86, B, H, T, V)
+    g, beta = -torch.rand(B, H, T, dtype=torch.float64, generator=torch.Generator().manual_seed(84)) * 0.5, torch.sigmoid(rnd(85, B, H, T))
+    h0, dht = rnd(87, B, H, K, V) * 0.1, rnd(88, B, H, K, V)
+    _, _, saved = chunked.chunk_forward('gdn', q, k, v, g, beta, None, h0, 64, torch.float64)
+    a = chunked.chunk_backward('gdn', q, k, v, g, beta, None, h0, do, dht, saved, 64, torch.float64)
+    b = chunked.chunk_backward('gdn', q, k, v, g, beta, None, h0, do, dht, saved, 64, torch.float64, solve_form=True)
+    leaves = [x.clone().requires_grad_(True) for x in (q, k, v, g, beta, h0)]
+    o, ht = naive.naive_recurrent_gated_delta_rule(*leaves[:5], None, leaves[5], True, None, True)
+    ref = torch.autograd.grad((o * do).sum() + (ht * dht).sum(), leaves)
+    for x, y, r in zip(a, b, ref):
+        assert (x - y).abs().max() < 1e-12 * max(1.0, r.abs().max().item())
+        assert (y - r).abs().max() < 1e-11 * max(1.0, r.abs().max().item())
+
+
 def test_gate_gradient_identity():
     # dg_t = sum_{s>=t} (q_s.dq_s - k_s.dk_s) + <S_T, dht>   (simple_gla)
     B, H, T, K, V = 1, 2, 40, 4, 3
