@@ -153,7 +153,12 @@ def chunk_gated_delta_rule(
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """q, k: ``[B,T,H,K]``, v: ``[B,T,H,V]``, g (log-space decay) and beta: ``[B,T,H]``
     (``[B,H,T,*]`` with ``head_first=True``).  Returns ``(o, final_state)``.  K, V of 64 or 128 run as they are;
-    a smaller K is zero-padded, any other V is cut into blocks of 128 / 64 columns (``_host.by_head_dim_blocks``)."""
+    a smaller K is zero-padded, any other V is cut into blocks of 128 / 64 columns (``_host.by_head_dim_blocks``).
+
+    ``use_qk_l2norm_in_kernel=True`` gives the results of fla's flag, not its fusion: q and k go through the ``l2_norm``
+    kernel (one read and one write of each, forward and backward) in front of the op, the op's kernels do not
+    normalise.  A caller that holds the fused projection of the mixer gets q^, k^ and silu(v) in one pass from
+    ``layer_io.gdn_qkv_prologue`` instead."""
     if use_qk_l2norm_in_kernel:
         q = l2_norm(q)
         k = l2_norm(k)
