@@ -640,8 +640,6 @@ __device__ __forceinline__ float wave_rev_scan(float x) {
   return total - (incl - x);
 }
 // sum over the 64 lanes, in every lane: the row totals, then the four of them through scalar registers
-// (call it with all 64 lanes active: a lane that is switched off contributes what its register held before, and
-// readlane of a lane that is off reads that stale value)
 __device__ __forceinline__ float wave_sum(float x) {
   x = group_sum<16>(x);
   const int xi = __builtin_bit_cast(int, x);
