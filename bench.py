@@ -538,6 +538,29 @@ def other_configs(dev, steps, warmup):
     sec = timed(f6)
     res["6 simple_gla fwd+bwd bf16 B=4 H=16 T=4096 K=V=128"] = (sec, B * T, B * T * H * ((6 * K + 5 * K) * 2 + 12),
                                                                 3 * B * T * H * sg_flops(K, K), PEAK_MFMA_BF16)
+    # 7 (not a contract configuration): the headline shape with a value head of 256 columns (expand_v = 2), in one
+    # call (kernel instances for K = 128, V = 256) and as the two calls on 128 columns each that it would otherwise
+    # be cut into (each repeats the WY preparation and the reads of q, k; dq, dk, dg, dbeta are added afterwards)
+    B, T, H, K, V = 4, 8192, 16, 128, 256
+    q = F.normalize(rn(B, T, H, K, dt=torch.float32), dim=-1).bfloat16().requires_grad_(True)
+    k = F.normalize(rn(B, T, H, K, dt=torch.float32), dim=-1).bfloat16().requires_grad_(True)
+    v = rn(B, T, H, V).requires_grad_(True)
+    beta = torch.rand(B, T, H, device=dev).bfloat16().requires_grad_(True)
+    g = (-torch.rand(B, T, H, device=dev) * 0.1).requires_grad_(True)
+    do = rn(B, T, H, V)
+
+    def f7():
+        o, _ = L.chunk_gated_delta_rule(q, k, v, g, beta)
+        torch.autograd.grad([o], [q, k, v, g, beta], [do])
+
+    def f7_halves():
+        o = torch.cat([L.chunk_gated_delta_rule(q, k, v[..., c:c + 128], g, beta, K ** -0.5)[0] for c in (0, 128)], -1)
+        torch.autograd.grad([o], [q, k, v, g, beta], [do])
+    sec = timed(f7)
+    extras = {"7": {"as_two_calls_on_128_columns_ms": round(timed(f7_halves) * 1e3, 4)}}
+    res["7 gated_delta_rule fwd+bwd bf16 B=4 T=8192 H=16 K=128 V=256"] = (
+        sec, B * T, B * T * H * ((6 * K + 5 * V) * 2 + 3 * 2 + 12),
+        3 * B * T * H * (6 * CH * K + 4 * CH * V + 6 * K * V + (2 / 3) * CH * CH), PEAK_MFMA_BF16)
     # one roofline record per configuration, for the whole call on its minimal traffic (every input read once, every
     # output written once): all five are bound by HBM on that count (arithmetic intensity below peak flops / peak
     # bytes).  `traffic` = HBM bytes per call summed over its kernels, from the FETCH_SIZE / WRITE_SIZE counters
@@ -551,8 +574,9 @@ def other_configs(dev, steps, warmup):
                                "unit": "GB/s", "frac": round(nb / sec / PEAK_HBM, 4),
                                "mfma_frac": round(fl / sec / peak_f, 4),
                                "traffic": OTHER_TRAFFIC.get(n[0]) if fresh else None}}
-    return {"metric": "contract configurations 1, 2, 3, 5 and the training step on the shape of 2 (6): ms per call, "
-                      "tokens/s", "unit": "ms", "steps": steps,
+        out[n].update(extras.get(n[0], {}))
+    return {"metric": "contract configurations 1, 2, 3, 5, the training step on the shape of 2 (6) and the headline "
+                      "shape with V = 256 (7): ms per call, tokens/s", "unit": "ms", "steps": steps,
             "warmup": warmup, "data": "synthetic", "configs": out}
 
 

@@ -154,7 +154,9 @@ int lmoe_chunk_gla_bwd(const lmoe_args* a, void* stream);
  * written nor needed (they may be NULL; less memory traffic; the results of a call with and without tinv differ
  * in the last bit of w, u).  4-byte elements, or no tinv: w and u are required.  pmat: required for 4-byte elements,
  * without tinv, or when hs is given; a forward-only 2-byte call with tinv forms P on the chip and may pass NULL.
- * bwd uses q,k,v,g,beta,hs,vnew,tinv,pmat,gcum,d_o,dht -> dq,dk,dv,dg,dbeta,dh0 (+ dhs, dvnew). */
+ * bwd uses q,k,v,g,beta,hs,vnew,tinv,pmat,gcum,d_o,dht -> dq,dk,dv,dg,dbeta,dh0 (+ dhs, dvnew).
+ * Head dimensions: K, V in {64, 128}, and K = 128 with V = 256 (the value head of expand_v = 2 at a head dimension
+ * of 128, linear_moe/arguments.py:595-598): one pass over q and k and one WY preparation serve all 256 columns. */
 int lmoe_chunk_gated_delta_rule_fwd(const lmoe_args* a, void* stream);
 int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream);
 

@@ -19,7 +19,8 @@ from ._lib import Args, Tensor4, CHUNK
 _DT = {torch.bfloat16: _lib.LMOE_BF16, torch.float32: _lib.LMOE_F32}
 
 
-def _check_inputs(q, k, v, head_first: bool, cu_seqlens) -> Tuple[int, int, int, int, int]:
+def _check_inputs(q, k, v, head_first: bool, cu_seqlens, wide_v: bool = False) -> Tuple[int, int, int, int, int]:
+    """wide_v: the op also has kernels for K = 128 with V = 256 (the gated delta rule)."""
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
         raise ValueError("q, k, v must be 4-dimensional")
     if not (q.is_cuda and k.is_cuda and v.is_cuda):
@@ -33,7 +34,7 @@ def _check_inputs(q, k, v, head_first: bool, cu_seqlens) -> Tuple[int, int, int,
     else:
         B, T, H, K = q.shape
     V = v.shape[-1]
-    if K not in HEAD_DIMS or V not in HEAD_DIMS:
+    if (K not in HEAD_DIMS or V not in HEAD_DIMS) and not (wide_v and (K, V) == WIDE_V):
         raise ValueError(f"head dims K={K}, V={V} unsupported: the kernels take K and V of 64 or 128 "
                          "(the public ops pad and split other sizes before they get here)")
     if cu_seqlens is not None:
@@ -45,22 +46,24 @@ def _check_inputs(q, k, v, head_first: bool, cu_seqlens) -> Tuple[int, int, int,
 
 
 HEAD_DIMS = (64, 128)      # what the kernels are instantiated for
+WIDE_V = (128, 256)        # and, for the gated delta rule, this (K, V) as well
 
 
-def dim_blocks(D: int):
-    """D columns as the blocks the kernels take: ``[(start, stop, width)]`` with width 128 or 64 (the last block
-    zero-padded up to its width)."""
+def dim_blocks(D: int, widest: int = 128):
+    """D columns as the blocks the kernels take: ``[(start, stop, width)]`` with width 64, 128 or (``widest=256``)
+    256 (the last block zero-padded up to its width)."""
     if D < 1:
         raise ValueError(f"head dimension must be positive, got {D}")
     out, d0 = [], 0
-    while D - d0 > 128:
-        out.append((d0, d0 + 128, 128))
-        d0 += 128
-    out.append((d0, D, 64 if D - d0 <= 64 else 128))
+    while D - d0 > widest:
+        out.append((d0, d0 + widest, widest))
+        d0 += widest
+    out.append((d0, D, 64 if D - d0 <= 64 else 128 if D - d0 <= 128 else 256))
     return out
 
 
-def by_head_dim_blocks(core, q, k, v, gk, initial_state, output_final_state: bool, sum_over_k: bool, name: str):
+def by_head_dim_blocks(core, q, k, v, gk, initial_state, output_final_state: bool, sum_over_k: bool, name: str,
+                       wide_v: bool = False):
     """An op on head dimensions the kernels are not instantiated for, as calls on blocks of 128 / 64 columns.
 
     The columns of v (and of the state) are independent in all three ops, so V is cut into blocks and the outputs
@@ -69,10 +72,12 @@ def by_head_dim_blocks(core, q, k, v, gk, initial_state, output_final_state: boo
     a sum over key blocks) also take K > 128 as several blocks whose outputs are added in fp32.  ``core(q, k, v, gk,
     h0) -> (o, ht)`` runs the op on supported dimensions (``gk``: the per-channel gate of chunk_gla or None).
     Everything around ``core`` is differentiable torch code.  Each V block repeats the work that depends on q, k
-    only (for the delta rule the WY preparation): the supported dimensions are the fast path."""
+    only (for the delta rule the WY preparation): the supported dimensions are the fast path.  ``wide_v``: with a key
+    of more than 64 columns (one block of 128) the op takes value blocks of 256 columns."""
     pad = torch.nn.functional.pad
     K, V = q.shape[-1], v.shape[-1]
-    kb, vb = dim_blocks(K), dim_blocks(V)
+    kb = dim_blocks(K)
+    vb = dim_blocks(V, 256 if wide_v and len(kb) == 1 and kb[0][2] == 128 else 128)
     if len(kb) > 1 and not sum_over_k:
         raise ValueError(f"{name}: K={K} unsupported: the delta rule needs the whole key in one block (K <= 128)")
     if initial_state is not None and tuple(initial_state.shape[-2:]) != (K, V):
@@ -103,11 +108,11 @@ def by_head_dim_blocks(core, q, k, v, gk, initial_state, output_final_state: boo
     return o, ht
 
 
-def no_tokens(q, k, v, head_first: bool, cu_seqlens, initial_state, output_final_state: bool):
+def no_tokens(q, k, v, head_first: bool, cu_seqlens, initial_state, output_final_state: bool, wide_v: bool = False):
     """The call without any token (T = 0, or a batch of zero rows): nothing to launch.  Returns None when there
     are tokens, else ``(o, final_state)``: an empty o and the initial state handed through (so that its gradient
     is the gradient of the final state), zeros without one."""
-    B, T, H, K, V = _check_inputs(q, k, v, head_first, cu_seqlens)
+    B, T, H, K, V = _check_inputs(q, k, v, head_first, cu_seqlens, wide_v)
     if B * T > 0:
         return None
     N = B if cu_seqlens is None else cu_seqlens.numel() - 1

@@ -18,11 +18,13 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
-int check_common(const lmoe_args* a, const char* op) {
+// wide_v: the op has instances for K = 128, V = 256 (the gated delta rule)
+int check_common(const lmoe_args* a, const char* op, bool wide_v = false) {
   if (!a) return fail(-1, "%s: null argument block", op);
   if (a->dtype != LMOE_BF16 && a->dtype != LMOE_F32) return fail(-2, "%s: dtype must be LMOE_BF16 or LMOE_F32", op);
-  if (!((a->K == 64 || a->K == 128) && (a->V == 64 || a->V == 128)))
-    return fail(-3, "%s: head dims K=%d V=%d unsupported (K, V must be 64 or 128)", op, a->K, a->V);
+  if (!((a->K == 64 || a->K == 128) && (a->V == 64 || a->V == 128)) && !(wide_v && a->K == 128 && a->V == 256))
+    return fail(-3, "%s: head dims K=%d V=%d unsupported (K, V must be 64 or 128%s)", op, a->K, a->V,
+                wide_v ? "; or K = 128 with V = 256" : "");
   if (a->B < 0 || a->T < 0 || a->H <= 0 || a->N < 0 || a->NT < 0) return fail(-4, "%s: negative dimension", op);
   if (a->cu_seqlens && (a->B != 1 || !a->chunk_map || !a->seq_chunk0))
     return fail(-5, "%s: packed input needs B == 1, chunk_map and seq_chunk0", op);
@@ -129,10 +131,11 @@ int lmoe_chunk_gla_bwd(const lmoe_args* a, void* stream) {
 }
 int lmoe_chunk_gated_delta_rule_fwd(const lmoe_args* a, void* stream) {
   const char* op = "lmoe_chunk_gated_delta_rule_fwd";
-  if (int r = check_common(a, op)) return r;
+  if (int r = check_common(a, op, true)) return r;
   if (a->gate == LMOE_GATE_VECTOR) return fail(-10, "%s: the gate is one scalar per token and head", op);
   if (!a->beta.ptr) return fail(-12, "%s: beta must not be null", op);
   if (!a->o.ptr || !a->gcum) return fail(-11, "%s: o and gcum must not be null", op);
+  if (a->V == 256 && a->dtype == LMOE_BF16 && !a->tinv) return fail(-11, "%s: V = 256 with 2-byte elements needs tinv", op);
   // P reaches memory where the WY preparation forms it (4-byte elements, or no tinv) or where the backward will
   // read it (hs given); a forward-only 2-byte call with tinv forms it inside the state pass and never stores it
   if ((a->dtype != LMOE_BF16 || !a->tinv || a->hs) && !a->pmat)
@@ -151,7 +154,7 @@ int lmoe_chunk_gated_delta_rule_fwd(const lmoe_args* a, void* stream) {
 }
 int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream) {
   const char* op = "lmoe_chunk_gated_delta_rule_bwd";
-  if (int r = check_common(a, op)) return r;
+  if (int r = check_common(a, op, true)) return r;
   if (a->gate == LMOE_GATE_VECTOR) return fail(-10, "%s: the gate is one scalar per token and head", op);
   if (!a->beta.ptr) return fail(-12, "%s: beta must not be null", op);
   if (!a->hs || !a->dhs || !a->vnew.ptr || !a->tinv || !a->pmat || !a->gcum || !a->dvnew.ptr)
@@ -502,7 +505,7 @@ int lmoe_quad_featmap_bwd(const void* x, const void* dy, void* dx, int64_t rows,
 
 int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* stream) {
   const char* nm = "lmoe_launch_stage";
-  if (int r = check_common(a, nm)) return r;
+  if (int r = check_common(a, nm, op == LMOE_OP_GATED_DELTA_RULE)) return r;
   if (a->NT == 0 || a->N == 0) return 0;
   hipStream_t st = (hipStream_t)stream;
   const bool gdn = op == LMOE_OP_GATED_DELTA_RULE;
@@ -511,11 +514,13 @@ int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* strea
       case lmoe::ST_GDN_WY_FWD: if (!gdn) return fail(-20, "%s: stage not part of this op", nm);
         if (!a->gcum || ((a->dtype != LMOE_BF16 || !a->tinv) && !a->pmat))
           return fail(-11, "%s: gcum (and pmat: 4-byte elements or no tinv) must not be null", nm);
+        if (a->V == 256 && a->dtype == LMOE_BF16 && !a->tinv) return fail(-11, "%s: V = 256 with 2-byte elements needs tinv", nm);
         lmoe::launch_gdn_wy_fwd(*a, st); break;
       case lmoe::ST_STATE_FWD:
         if (gdn) {
           if (!a->gcum || ((a->dtype != LMOE_BF16 || !a->tinv || a->hs) && !a->pmat))
             return fail(-11, "%s: gcum (and pmat: 4-byte elements, no tinv, or hs given) must not be null", nm);
+          if (a->V == 256 && a->dtype == LMOE_BF16 && !a->tinv) return fail(-11, "%s: V = 256 with 2-byte elements needs tinv", nm);
           lmoe::launch_gdn_state_fwd(*a, st);
         } else {
           lmoe::launch_state_fwd(*a, st);

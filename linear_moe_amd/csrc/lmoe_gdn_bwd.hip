@@ -16,6 +16,6 @@ template <typename T, int K, int V> struct GdnBwdChunk {
     hipLaunchKernelGGL((k_gdn_bwd_chunk<T, K, V, BVH, NBUF, DEPTH>), dim3(grid), dim3(3 * NTHR), 0, st, a);
   }
 };
-void launch_gdn_bwd_chunk(const lmoe_args& a, hipStream_t st) { dispatch<GdnBwdChunk>(a, st); }
+void launch_gdn_bwd_chunk(const lmoe_args& a, hipStream_t st) { dispatch_gdn<GdnBwdChunk>(a, st); }
 
 }  // namespace lmoe

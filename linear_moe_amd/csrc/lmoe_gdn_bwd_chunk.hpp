@@ -139,6 +139,10 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
       constexpr int u = decltype(uc)::value, unit = u % NU;
       Unit& R = U[u % DEPTH];
       it = __builtin_amdgcn_readfirstlane(min(it + (u / NU) * stride, nitems - 1));
+      // with many slices per item the scalar addresses of all of them, formed at the top of the item, do not fit the
+      // scalar registers: the item index is made opaque per unit, so that each unit's addresses are formed where it
+      // is requested
+      if constexpr (NS > 4) asm volatile("" : "+s"(it));
       const int cid = it / a.H, h = it % a.H;
       const ChunkInfo ci = chunk_info(a, cid);
       R.len = ci.len;
@@ -198,6 +202,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
           d.r.v[p] = o;
           s = group_sum<IOV::VPR>(s);                   // the VPR lanes that hold one row are neighbours
           dbv[p] += row < R.len ? s : 0.f;
+          pin(dbv[p]);
         }
         constexpr int off[3] = {A_DO, A_VN, A_DZ};
 #pragma unroll
@@ -215,6 +220,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
         for (int p = 0; p < PH; ++p)
 #pragma unroll
           for (int i = 0; i < IOH::VEC; ++i) hdh += ET<T>::to_f(rh.v[p][i]) * ET<T>::to_f(rdh.v[p][i]);
+        pin(hdh);                                         // here, not where the item is closed (the tiles would stay live)
         IOH::store_lds(rh, base + A_H, LDK, tid);
         IOH::store_lds(rdh, base + A_DH, LDK, tid);
       } else {

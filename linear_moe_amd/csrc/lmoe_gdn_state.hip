@@ -24,12 +24,15 @@ template <typename T, int K, int V, int BV> void launch_fwd(const lmoe_args& a, 
       return;
     }
   }
-  if (a.hs) {
-    if (wt) hipLaunchKernelGGL((k_gdn_state_fwd<T, K, V, BV, true, CAN_WT>), dim3(grid), dim3(3 * NTHR), 0, st, a);
-    else hipLaunchKernelGGL((k_gdn_state_fwd<T, K, V, BV, true, false>), dim3(grid), dim3(3 * NTHR), 0, st, a);
-  } else {
-    if (wt) hipLaunchKernelGGL((k_gdn_state_fwd<T, K, V, BV, false, CAN_WT>), dim3(grid), dim3(3 * NTHR), 0, st, a);
-    else hipLaunchKernelGGL((k_gdn_state_fwd<T, K, V, BV, false, false>), dim3(grid), dim3(3 * NTHR), 0, st, a);
+  // (2-byte elements at V = 256 run with Tinv only, i.e. above: the entry points reject a call without it)
+  if constexpr (!(CAN_WT && V > 128)) {
+    if (a.hs) {
+      if (wt) hipLaunchKernelGGL((k_gdn_state_fwd<T, K, V, BV, true, CAN_WT>), dim3(grid), dim3(3 * NTHR), 0, st, a);
+      else hipLaunchKernelGGL((k_gdn_state_fwd<T, K, V, BV, true, false>), dim3(grid), dim3(3 * NTHR), 0, st, a);
+    } else {
+      if (wt) hipLaunchKernelGGL((k_gdn_state_fwd<T, K, V, BV, false, CAN_WT>), dim3(grid), dim3(3 * NTHR), 0, st, a);
+      else hipLaunchKernelGGL((k_gdn_state_fwd<T, K, V, BV, false, false>), dim3(grid), dim3(3 * NTHR), 0, st, a);
+    }
   }
 }
 template <typename T, int K, int V, int BV> void launch_bwd(const lmoe_args& a, hipStream_t st) {
@@ -53,7 +56,7 @@ template <typename T, int K, int V> struct GdnStateBwd {
     else launch_bwd<T, K, V, GdnStateCfg<T>::BV>(a, st);
   }
 };
-void launch_gdn_state_fwd(const lmoe_args& a, hipStream_t st) { dispatch<GdnStateFwd>(a, st); }
+void launch_gdn_state_fwd(const lmoe_args& a, hipStream_t st) { dispatch_gdn<GdnStateFwd>(a, st); }
 // the traced instance of the register-resident forward pass (2-byte elements, K = V = 128, saving call)
 bool launch_gdn_state_fwd_trace(const lmoe_args& a, long long* tr, int work_group, hipStream_t st) {
   if (a.dtype != LMOE_BF16 || a.K != 128 || a.V != 128 || !a.tinv || !a.hs) return false;
@@ -62,6 +65,6 @@ bool launch_gdn_state_fwd_trace(const lmoe_args& a, long long* tr, int work_grou
   hipLaunchKernelGGL((k_gdn_state_fwd_reg<128, 128, true, true>), dim3(grid), dim3(3 * NTHR), 0, st, a, tr, work_group);
   return true;
 }
-void launch_gdn_state_bwd(const lmoe_args& a, hipStream_t st) { dispatch<GdnStateBwd>(a, st); }
+void launch_gdn_state_bwd(const lmoe_args& a, hipStream_t st) { dispatch_gdn<GdnStateBwd>(a, st); }
 
 }  // namespace lmoe

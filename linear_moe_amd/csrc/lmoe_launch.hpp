@@ -31,6 +31,20 @@ inline void dispatch(const lmoe_args& a, hipStream_t st) {
 #undef LMOE_KV
 }
 
+// the kernels of the gated delta rule also exist for K = 128, V = 256 (a value head twice as wide as the key head:
+// expand_v = 2 at a head dimension of 128); the state passes cut V into slices anyway and the chunk-parallel
+// backward loops over them, so one WY preparation and one read of q, k per kernel serve all 256 columns
+template <template <typename, int, int> class F>
+inline void dispatch_gdn(const lmoe_args& a, hipStream_t st) {
+  typedef __bf16 bf16_t;
+  if (a.K == 128 && a.V == 256) {
+    if (a.dtype == LMOE_BF16) F<bf16_t, 128, 256>::run(a, st);
+    else F<float, 128, 256>::run(a, st);
+    return;
+  }
+  dispatch<F>(a, st);
+}
+
 void launch_state_fwd(const lmoe_args& a, hipStream_t st);        // chunk_simple_gla
 // traced forward pass of chunk_simple_gla (bf16, K = V = 128, forward-only): false when the problem is not of that shape
 bool launch_state_fwd_trace(const lmoe_args& a, long long* tr, int work_group, hipStream_t st);

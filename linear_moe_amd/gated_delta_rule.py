@@ -16,7 +16,7 @@ import torch
 
 from . import _lib
 from .l2norm import l2_norm
-from ._host import (HEAD_DIMS, seq_plan, _aligned, _check_inputs, _desc, _state_check, base_args, by_head_dim_blocks,
+from ._host import (HEAD_DIMS, WIDE_V, seq_plan, _aligned, _check_inputs, _desc, _state_check, base_args, by_head_dim_blocks,
                     no_tokens, ptr, stream_ptr)
 
 
@@ -41,7 +41,7 @@ class GDNCall:
         per-chunk states, v_new, Tinv) is neither allocated nor written."""
         ctx = self
         lib = _lib.load()
-        dims = _check_inputs(q, k, v, head_first, cu_seqlens)
+        dims = _check_inputs(q, k, v, head_first, cu_seqlens, wide_v=True)
         B, T, H, K, V = dims
         q, k, v = _aligned(q), _aligned(k), _aligned(v)
         plan = seq_plan(B, T, cu_seqlens, q.device)
@@ -152,8 +152,9 @@ def chunk_gated_delta_rule(
     use_qk_l2norm_in_kernel: bool = False,
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """q, k: ``[B,T,H,K]``, v: ``[B,T,H,V]``, g (log-space decay) and beta: ``[B,T,H]``
-    (``[B,H,T,*]`` with ``head_first=True``).  Returns ``(o, final_state)``.  K, V of 64 or 128 run as they are;
-    a smaller K is zero-padded, any other V is cut into blocks of 128 / 64 columns (``_host.by_head_dim_blocks``).
+    (``[B,H,T,*]`` with ``head_first=True``).  Returns ``(o, final_state)``.  K, V of 64 or 128 and K = 128 with
+    V = 256 (``expand_v = 2``) run as they are; a smaller K is zero-padded, any other V is cut into blocks of
+    256 (K > 64) / 128 / 64 columns (``_host.by_head_dim_blocks``).
 
     ``use_qk_l2norm_in_kernel=True`` gives the results of fla's flag, not its fusion: q and k go through the ``l2_norm``
     kernel (one read and one write of each, forward and backward) in front of the op, the op's kernels do not
@@ -162,14 +163,15 @@ def chunk_gated_delta_rule(
     if use_qk_l2norm_in_kernel:
         q = l2_norm(q)
         k = l2_norm(k)
-    if q.dim() == 4 and v.dim() == 4 and (q.shape[-1] not in HEAD_DIMS or v.shape[-1] not in HEAD_DIMS):
-        # e.g. expand_v = 2 with a head dimension of 128: V = 256 as two blocks of 128 columns
+    if q.dim() == 4 and v.dim() == 4 and (q.shape[-1] not in HEAD_DIMS or v.shape[-1] not in HEAD_DIMS) \
+            and (q.shape[-1], v.shape[-1]) != WIDE_V:
+        # e.g. K = 96 (padded to 128), V = 320 (a block of 256 and one of 64 columns)
         sc = q.shape[-1] ** -0.5 if scale is None else scale          # of the whole key, not of the padded one
         return by_head_dim_blocks(
             lambda q_, k_, v_, _g, h0: chunk_gated_delta_rule(q_, k_, v_, g, beta, sc, h0, output_final_state,
                                                               cu_seqlens, head_first),
-            q, k, v, None, initial_state, output_final_state, False, "chunk_gated_delta_rule")
-    r = no_tokens(q, k, v, head_first, cu_seqlens, initial_state, output_final_state)
+            q, k, v, None, initial_state, output_final_state, False, "chunk_gated_delta_rule", wide_v=True)
+    r = no_tokens(q, k, v, head_first, cu_seqlens, initial_state, output_final_state, wide_v=True)
     if r is not None:
         return r
     return _ChunkGatedDeltaRule.apply(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens,

@@ -38,6 +38,9 @@ CASES = [
     (2, 130, 2, 64, 128, True, True, True),
     (1, 64, 2, 128, 64, True, False, False),
     (1, 5, 1, 64, 64, False, False, True),
+    # the value head of expand_v = 2 (kernel instances of their own: one pass over q, k for all 256 columns)
+    (2, 200, 2, 128, 256, True, False, False),
+    (1, 130, 3, 128, 256, False, True, True),
 ]
 
 
@@ -86,6 +89,9 @@ BWD_CASES = [
     # wrong dq, dk in fp32 -- kept as a fixed case (the random trials reach this shape only by chance of the seed)
     (2, 330, 3, 64, 128, True, False, False),
     (1, 200, 2, 128, 64, False, False, True),
+    (2, 200, 2, 128, 256, True, False, False),
+    (1, 330, 3, 128, 256, False, True, True),
+    (1, 7, 1, 128, 256, True, False, False),
 ]
 
 
@@ -125,7 +131,44 @@ def test_gdn_bwd_varlen(cuda, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("case", [(2, 200, 2, 128, 128, True), (1, 70, 2, 64, 128, False)])
+def test_gdn_bwd_varlen_wide_value_head(cuda, dtype):
+    cu = torch.tensor([0, 64, 65, 200, 333], dtype=torch.int32)
+    T, H, K, V, N = 333, 2, 128, 256, 4
+    q, k, v, g, beta = gdn_inputs(420, 1, T, H, K, V, dtype, False, True)
+    ins = dict(q=q, k=k, v=v, g=g, beta=beta, h0=gen(434, N, H, K, V) * 0.1)
+    _gdn_bwd_check(cuda, dtype, ins, gen(435, 1, T, H, V, dtype=dtype), gen(436, N, H, K, V), cu, False)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gdn_wide_value_head_equals_its_two_halves(cuda, dtype):
+    """V = 256 in one call against the two calls on 128 columns each that the op used to be cut into: the columns of v
+    are independent, so o, the final state and dv agree bit for bit (the same slice kernels on the same operands);
+    dq, dk, dg, dbeta are sums over all columns and agree to rounding (one sum over 256 columns against two rounded
+    sums of 128)."""
+    from linear_moe_amd import chunk_gated_delta_rule
+    B, T, H, K, V = 2, 300, 3, 128, 256
+    q, k, v, g, beta = gdn_inputs(440, B, T, H, K, V, dtype, False, True)
+    h0, do, dht = gen(454, B, H, K, V) * 0.1, gen(455, B, T, H, V, dtype=dtype), gen(456, B, H, K, V)
+    res = []
+    for halves in (False, True):
+        d = {n: x.to(cuda).requires_grad_(True) for n, x in dict(q=q, k=k, v=v, g=g, beta=beta, h0=h0).items()}
+        if halves:
+            parts = [chunk_gated_delta_rule(d['q'], d['k'], d['v'][..., c:c + 128], d['g'], d['beta'], K ** -0.5,
+                                            d['h0'][..., c:c + 128], True) for c in (0, 128)]
+            o, ht = torch.cat([p[0] for p in parts], -1), torch.cat([p[1] for p in parts], -1)
+        else:
+            o, ht = chunk_gated_delta_rule(d['q'], d['k'], d['v'], d['g'], d['beta'], None, d['h0'], True)
+        ((o * do.to(cuda)).sum() + (ht * dht.to(cuda)).sum()).backward()
+        res.append((o.detach(), ht.detach(), {n: x.grad for n, x in d.items()}))
+    (o1, ht1, g1), (o2, ht2, g2) = res
+    assert torch.equal(o1, o2) and torch.equal(ht1, ht2)
+    assert torch.equal(g1['v'], g2['v']) and torch.equal(g1['h0'], g2['h0'])
+    for n in ('q', 'k', 'g', 'beta'):
+        assert max_abs_rel(g1[n].cpu(), g2[n].cpu()) < TOL[dtype], n
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", [(2, 200, 2, 128, 128, True), (1, 70, 2, 64, 128, False), (1, 130, 2, 128, 256, True)])
 def test_delta_rule_fwd_bwd(cuda, dtype, case):
     """chunk_delta_rule as the reference calls it (deltanet.py:127-130): head-first, positional chunk size."""
     from linear_moe_amd import chunk_delta_rule

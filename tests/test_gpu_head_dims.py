@@ -1,5 +1,6 @@
-"""Head dimensions the kernels are not instantiated for (anything but 64 and 128): the public ops pad and cut them
-into blocks of 128 / 64 columns (``linear_moe_amd/_host.py::by_head_dim_blocks``).  HIP through the C ABI against the
+"""Head dimensions the kernels are not instantiated for (anything but 64 and 128, and K = 128 with V = 256 for the
+delta rule): the public ops pad and cut them into blocks of 128 / 64 columns, the delta rule with a key block of 128
+also into value blocks of 256 (``linear_moe_amd/_host.py::by_head_dim_blocks``).  HIP through the C ABI against the
 token-recurrence oracle on the whole head dimensions; e.g. ``expand_v = 2`` with a head dimension of 128 (V = 256,
 ``linear_moe/model/common_modules/linear_attention.py`` of the reference scales ``head_v_dim`` that way)."""
 import pytest
@@ -28,7 +29,7 @@ def _check(cuda, dtype, ins, do, dht, ref_fn, run):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("K,V", [(128, 256), (96, 192), (32, 48), (64, 80)])
+@pytest.mark.parametrize("K,V", [(128, 256), (96, 192), (32, 48), (64, 80), (128, 320), (64, 256)])
 def test_gated_delta_rule_other_head_dims(cuda, dtype, K, V):
     from linear_moe_amd import chunk_gated_delta_rule
     B, T, H = 2, 130, 2
