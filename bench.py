@@ -561,6 +561,20 @@ def other_configs(dev, steps, warmup):
     res["7 gated_delta_rule fwd+bwd bf16 B=4 T=8192 H=16 K=128 V=256"] = (
         sec, B * T, B * T * H * ((6 * K + 5 * V) * 2 + 3 * 2 + 12),
         3 * B * T * H * (6 * CH * K + 4 * CH * V + 6 * K * V + (2 / 3) * CH * CH), PEAK_MFMA_BF16)
+    # 8 (not a contract configuration): chunk_linear_attn with its normaliser (the default of the reference's
+    # BasicLinearAttention), forward + backward on the shape of configuration 2, beside the same call without it
+    B, H, T, K = 4, 16, 4096, 128
+    q, k = (torch.rand(B, H, T, K, device=dev).bfloat16().requires_grad_(True) for _ in range(2))
+    v = rn(B, H, T, K).requires_grad_(True)
+    do = rn(B, H, T, K)
+
+    def f8(normalize):
+        o, _ = L.chunk_linear_attn(q, k, v, normalize=normalize)
+        torch.autograd.grad([o], [q, k, v], [do])
+    sec = timed(lambda: f8(True))
+    extras["8"] = {"without_normaliser_ms": round(timed(lambda: f8(False)) * 1e3, 4)}
+    res["8 linear_attn normalize=True fwd+bwd bf16 B=4 H=16 T=4096 K=V=128"] = (
+        sec, B * T, B * T * H * ((6 * K + 5 * K) * 2), 3 * B * T * H * sg_flops(K, K), PEAK_MFMA_BF16)
     # one roofline record per configuration, for the whole call on its minimal traffic (every input read once, every
     # output written once): all five are bound by HBM on that count (arithmetic intensity below peak flops / peak
     # bytes).  `traffic` = HBM bytes per call summed over its kernels, from the FETCH_SIZE / WRITE_SIZE counters
@@ -576,7 +590,7 @@ def other_configs(dev, steps, warmup):
                                "traffic": OTHER_TRAFFIC.get(n[0]) if fresh else None}}
         out[n].update(extras.get(n[0], {}))
     return {"metric": "contract configurations 1, 2, 3, 5, the training step on the shape of 2 (6) and the headline "
-                      "shape with V = 256 (7): ms per call, tokens/s", "unit": "ms", "steps": steps,
+                      "shape with V = 256 (7), chunk_linear_attn with its normaliser (8): ms per call, tokens/s", "unit": "ms", "steps": steps,
             "warmup": warmup, "data": "synthetic", "configs": out}
 
 

@@ -106,6 +106,19 @@ typedef struct lmoe_args {
    * it (tables built on the device from offsets that were never read on the host: chunk_map has NT rows, the first
    * *nt_dev of them valid; every per-chunk buffer is sized for NT).  NULL = NT is exact.  No counterpart in fla. */
   const int32_t* nt_dev;
+  /* chunk_simple_gla with the output normalised inside the kernels (2-byte elements, gate = NONE):
+   *   o_t = scale q_t S_t / (den_t + norm_eps),   den_t = scale q_t . sum_{s <= t} k_s   (the sum starts inside the call)
+   * what fla.ops.linear_attn.chunk_linear_attn(normalize=True) forms behind its kernel with a cumulative sum over k in
+   * memory (linear_moe/sequence_modeling/basic_linear_attention/basic_linear_attention.py:133).  normalize = 0: the
+   * fields below are ignored.
+   * fwd writes den (the divisor den_t + norm_eps, fp32, laid out like g) and, when hs is given, zs (fp32 [NT,H,K]:
+   * the sum of the keys before each chunk).  bwd reads them and o (the normalised output the forward wrote) beside
+   * d_o (the gradient of that output), and uses norm_ws, fp32 [NT,H,V/32,64+K], as workspace. */
+  int32_t normalize;
+  float norm_eps;
+  lmoe_tensor den;
+  float* zs;
+  float* norm_ws;
 } lmoe_args;
 
 /* Library version (major*10000 + minor*100 + patch). */
@@ -130,7 +143,8 @@ int64_t lmoe_workspace_bytes(int32_t op, int32_t dtype, int32_t part, int32_t B,
  *   linear_moe/sequence_modeling/basic_linear_attention/basic_linear_attention.py:133 (chunk_linear_attn)
  *   linear_moe/sequence_modeling/lightning_attention/lightning_attention.py:121-123 (lightning_attn2)
  * fwd uses q,k,v,g,h0 -> o,ht,hs (hs may be NULL: a forward-only call, which then saves nothing for a backward).
- * bwd uses q,k,v,g,hs,d_o,dht -> dq,dk,dv,dg,dh0 (+ dhs). */
+ * bwd uses q,k,v,g,hs,d_o,dht -> dq,dk,dv,dg,dh0 (+ dhs).
+ * With normalize = 1 (see lmoe_args): fwd also -> den (, zs); bwd also uses o, den, zs (+ norm_ws). */
 int lmoe_chunk_simple_gla_fwd(const lmoe_args* a, void* stream);
 int lmoe_chunk_simple_gla_bwd(const lmoe_args* a, void* stream);
 

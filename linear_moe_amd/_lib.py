@@ -40,6 +40,8 @@ class Args(C.Structure):
         ("dhs", C.c_void_p), ("dvnew", Tensor4),
         ("seq_order", C.c_void_p),
         ("nt_dev", C.c_void_p),
+        ("normalize", C.c_int32), ("norm_eps", C.c_float), ("den", Tensor4), ("zs", C.c_void_p),
+        ("norm_ws", C.c_void_p),
     ]
 
 

@@ -34,6 +34,17 @@ int check_common(const lmoe_args* a, const char* op, bool wide_v = false) {
   return 0;
 }
 
+// chunk_simple_gla with the output normalised inside the kernels (lmoe_args.normalize)
+int check_normalize(const lmoe_args* a, const char* op, bool bwd) {
+  if (!a->normalize) return 0;
+  if (a->dtype != LMOE_BF16) return fail(-15, "%s: normalize needs 2-byte elements", op);
+  if (a->gate != LMOE_GATE_NONE) return fail(-15, "%s: normalize needs gate = LMOE_GATE_NONE", op);
+  if (!a->den.ptr) return fail(-11, "%s: normalize needs den", op);
+  if (!bwd && a->hs && !a->zs) return fail(-11, "%s: normalize with hs given needs zs", op);
+  if (bwd && (!a->zs || !a->norm_ws || !a->o.ptr)) return fail(-11, "%s: normalize needs o, zs and norm_ws", op);
+  return 0;
+}
+
 int launched(const char* op) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail((int)e, "%s: launch failed: %s", op, hipGetErrorString(e));
@@ -73,6 +84,7 @@ int lmoe_chunk_simple_gla_fwd(const lmoe_args* a, void* stream) {
   if (int r = check_common(a, op)) return r;
   if (a->gate == LMOE_GATE_VECTOR) return fail(-10, "%s: vector gates belong to lmoe_chunk_gla_fwd", op);
   if (!a->o.ptr) return fail(-11, "%s: o must not be null", op);      // hs == NULL: forward only, nothing saved
+  if (int r = check_normalize(a, op, false)) return r;
   if (a->NT == 0 || a->N == 0) return 0;
   lmoe::launch_state_fwd(*a, (hipStream_t)stream);
   return launched(op);
@@ -85,6 +97,7 @@ int lmoe_chunk_simple_gla_bwd(const lmoe_args* a, void* stream) {
   if (!a->hs || !a->dhs || !a->d_o.ptr || !a->dq.ptr || !a->dk.ptr || !a->dv.ptr)
     return fail(-11, "%s: hs, dhs, d_o, dq, dk and dv must not be null", op);
   if (a->gate == LMOE_GATE_SCALAR && !a->dg.ptr) return fail(-13, "%s: dg must not be null for a gated call", op);
+  if (int r = check_normalize(a, op, true)) return r;
   if (a->NT == 0 || a->N == 0) return 0;
   lmoe::launch_state_bwd(*a, (hipStream_t)stream);
   // 2-byte elements: dv is formed by the kernel that forms dq and dk, from the tiles it holds anyway
@@ -506,6 +519,8 @@ int lmoe_quad_featmap_bwd(const void* x, const void* dy, void* dx, int64_t rows,
 int lmoe_launch_stage(const lmoe_args* a, int32_t op, int32_t stage, void* stream) {
   const char* nm = "lmoe_launch_stage";
   if (int r = check_common(a, nm, op == LMOE_OP_GATED_DELTA_RULE)) return r;
+  if (op == LMOE_OP_SIMPLE_GLA)
+    if (int r = check_normalize(a, nm, stage != lmoe::ST_STATE_FWD)) return r;
   if (a->NT == 0 || a->N == 0) return 0;
   hipStream_t st = (hipStream_t)stream;
   const bool gdn = op == LMOE_OP_GATED_DELTA_RULE;

@@ -26,20 +26,32 @@ template <typename T, int K, int V> struct StateBwd {
     // element is the same sum over the tokens in either split
     constexpr int BW = (sizeof(T) == 2 && V >= 64) ? 64 : BV;
     if (BW != BV && (int64_t)a.N * a.H * (V / BW) >= cu_count()) {
-      const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BW);
-      hipLaunchKernelGGL((k_state_bwd<T, K, V, BW>), dim3(grid), dim3(2 * NTHR), 0, st, a);
+      launch<BW>(a, st);
       return;
     }
-    const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BV);
-    hipLaunchKernelGGL((k_state_bwd<T, K, V, BV>), dim3(grid), dim3(2 * NTHR), 0, st, a);
+    launch<BV>(a, st);
+  }
+  template <int BVX> static void launch(const lmoe_args& a, hipStream_t st) {
+    const dim3 grid(((a.N * a.H + 7) / 8) * 8 * (V / BVX)), block(2 * NTHR);
+    if constexpr (sizeof(T) == 2) {        // the pass behind the normalised output exists for 2-byte elements
+      if (a.normalize) {
+        hipLaunchKernelGGL((k_state_bwd<T, K, V, BVX, true>), grid, block, 0, st, a);
+        return;
+      }
+    }
+    hipLaunchKernelGGL((k_state_bwd<T, K, V, BVX>), grid, block, 0, st, a);
   }
 };
 template <typename T, int K, int V> struct BwdDqk {
   static void run(const lmoe_args& a, hipStream_t st) {
     constexpr int BVH = BwdTiles<T, V>::BVH;
     const int grid = persistent_grid(a.NT * a.H, 1);
-    if constexpr (sizeof(T) == 2) hipLaunchKernelGGL((k_bwd_dqkv<T, K, V, BVH>), dim3(grid), dim3(2 * NTHR), 0, st, a);
-    else hipLaunchKernelGGL((k_bwd_dqk<T, K, V, BVH>), dim3(grid), dim3(2 * NTHR), 0, st, a);
+    if constexpr (sizeof(T) == 2) {
+      if (a.normalize) hipLaunchKernelGGL((k_bwd_dqkv<T, K, V, BVH, true>), dim3(grid), dim3(2 * NTHR), 0, st, a);
+      else hipLaunchKernelGGL((k_bwd_dqkv<T, K, V, BVH>), dim3(grid), dim3(2 * NTHR), 0, st, a);
+    } else {
+      hipLaunchKernelGGL((k_bwd_dqk<T, K, V, BVH>), dim3(grid), dim3(2 * NTHR), 0, st, a);
+    }
   }
 };
 

@@ -104,10 +104,20 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dv(const lmoe_args a) {
 //   Waves 4-7 (loaders) keep the next chunks' q, do in flight, stage them unscaled and write
 //   dhs (layout [V][K]).  Both teams meet at the same barriers.
 // ------------------------------------------------------------------------- //
-template <typename T, int K, int V, int BV>
+// NORM (ungated calls with the output normalised in the forward pass): d_o is the gradient of the normalised output
+// o' = o / D, D = den + eps.  The pass then runs on do = d_o / D (folded into the row factor of the do fragments) and
+// carries, beside dS, the gradient dz of the column of ones that forms den, whose "do" is dden_i = -(d_o_i . o'_i) / D_i.
+// A V slice sees only its columns of d_o and o': it forms the partial row dots over those, and since everything
+// downstream is linear in dden it carries the partial dz that belongs to them; the chunk-parallel kernel adds the
+// partial sums of all slices.  Per chunk, head and 32 columns of V one row of norm_ws: [64] scale dden (partial),
+// [K] dz at the end of the chunk (partial); a slice of 64 columns fills the first of its two rows and zeroes the other.
+constexpr int NORM_SLOT_COLS = 32;
+template <typename T, int K, int V, int BV, bool NORM = false>
 __global__ __launch_bounds__(2 * NTHR) void k_state_bwd(const lmoe_args a) {
   constexpr int LDK = K + LPAD, LDU = BV + LPAD;
   constexpr int MB = K / 64, NB = BV / 16;
+  static_assert(!NORM || sizeof(T) == 2, "the normalised pass exists for 2-byte elements");
+  constexpr int WS_ROW = CH + K, WS_SLOTS = V / NORM_SLOT_COLS, SLOTS_PER_SLICE = BV / NORM_SLOT_COLS;
   // bf16: two operand buffers; fp32 (the parity path) has LDS for one and pays extra barriers
   constexpr int NBUF = sizeof(T) == 2 ? 2 : 1;
   __shared__ __attribute__((aligned(16))) T s_q[NBUF][CH * LDK];             // q       [64][K]
@@ -115,6 +125,7 @@ __global__ __launch_bounds__(2 * NTHR) void k_state_bwd(const lmoe_args a) {
   __shared__ __attribute__((aligned(16))) T s_dST[BV * LDK];                 // dS'^T   [BV][K]
   __shared__ __attribute__((aligned(16))) float s_b[NBUF][64], s_qs[NBUF][64], s_ed[NBUF][64];
   __shared__ float s_dec[NBUF];
+  __shared__ __attribute__((aligned(16))) float s_dd[NORM ? NBUF : 1][NORM ? 64 : 4];    // NORM: scale dden (partial)
 
   constexpr int NVS = V / BV;
   const int xcd = blockIdx.x & 7, jj = blockIdx.x >> 3;
@@ -125,6 +136,10 @@ __global__ __launch_bounds__(2 * NTHR) void k_state_bwd(const lmoe_args a) {
   const int l = lane_id();
   const int team = threadIdx.x / NTHR;      // 0: consumers, 1: loaders
   const bool producer = team == 1;
+  // NORM: the rows of norm_ws of this slice in chunk c
+  auto ws_row = [&](int c) {
+    return a.norm_ws + (((int64_t)(sq.chunk0 + c) * a.H + h) * WS_SLOTS + vsl * SLOTS_PER_SLICE) * WS_ROW;
+  };
   if (sq.nchunks == 0) {
     if (a.dh0 && team == 0) {
       for (int idx = threadIdx.x; idx < K * BV; idx += NTHR) {
@@ -142,7 +157,8 @@ __global__ __launch_bounds__(2 * NTHR) void k_state_bwd(const lmoe_args a) {
   if (producer) {
     // ------------------------------- producers -------------------------------------------
     constexpr int PF = 2;
-    struct Pre { typename IOK::Regs rq; typename IOV::Regs rd; uint32_t graw; int len; };
+    // (NORM: the slice of the normalised output, D of the rows this thread holds of it and of row = lane; c = chunk)
+    struct Pre { typename IOK::Regs rq; typename IOV::Regs rd, ro; float rD[IOV::PASSES], dl; uint32_t graw; int len, c; };
     Pre pre[PF];
     const int pw = wave_id() - 4;
     const bool gated = a.gate != LMOE_GATE_NONE && a.g.ptr != nullptr;
@@ -157,13 +173,50 @@ __global__ __launch_bounds__(2 * NTHR) void k_state_bwd(const lmoe_args a) {
       IOV::load_nomask(P.rd, row_ptr<T>(a.d_o, sq.b, tok, h) + v0, a.d_o.st, len);
       P.len = len;
       P.graw = load_scalar_raw(gptr, a.g_dtype, gated ? row_off(a.g, sq.b, tok + min(l, len - 1), h) : 0);
+      if constexpr (NORM) {
+        P.c = c;
+        IOV::load_nomask(P.ro, row_ptr<T>(a.o, sq.b, tok, h) + v0, a.o.st, len);
+        const float* den = (const float*)a.den.ptr;
+#pragma unroll
+        for (int p = 0; p < IOV::PASSES; ++p) {
+          int row, col; IOV::coords(p, row, col);
+          P.rD[p] = den[row_off(a.den, sq.b, tok + min(row, len - 1), h)];
+        }
+        P.dl = den[row_off(a.den, sq.b, tok + min(l, len - 1), h)];
+      }
     };
     auto stage = [&](Pre& P, int buf) {
+      if constexpr (NORM) {
+        // partial row dots of d_o and o' over the columns of this slice -> scale dden (partial), for the consumers and
+        // for the chunk-parallel kernel; from the registers as loaded (rows past the end of a partial chunk: zero)
+        float* ws = ws_row(P.c);
+#pragma unroll
+        for (int p = 0; p < IOV::PASSES; ++p) {
+          int row, col; IOV::coords(p, row, col);
+          float sum = 0.f;
+#pragma unroll
+          for (int i = 0; i < IOV::VEC; ++i) sum += ET<T>::to_f(P.rd.v[p][i]) * ET<T>::to_f(P.ro.v[p][i]);
+          sum = group_sum<IOV::VPR>(sum);               // the VPR lanes that hold one row are neighbours
+          const float dd = row < P.len ? -scale * sum / P.rD[p] : 0.f;
+          if (col == 0) {
+            s_dd[buf][row] = dd;
+            ws[row] = dd;
+            if constexpr (SLOTS_PER_SLICE == 2) ws[WS_ROW + row] = 0.f;
+          }
+        }
+      }
       IOK::mask(P.rq, P.len);
       IOV::mask(P.rd, P.len);
       IOK::store_lds(P.rq, s_q[buf], LDK);
       IOV::store_lds(P.rd, s_do[buf], LDU);
-      if (pw == 0) {
+      if constexpr (NORM) {
+        if (pw == 0) {                     // ungated: the row factor of the do fragments is scale / D
+          s_b[buf][l] = 0.f;
+          s_qs[buf][l] = scale / P.dl;
+          s_ed[buf][l] = 1.f;
+          if (l == 0) s_dec[buf] = 1.f;
+        }
+      } else if (pw == 0) {
         const float x = wave_incl_scan((gated && l < P.len) ? scalar_from_raw(P.graw, a.g_dtype) : 0.f);
         const float xl = __shfl(x, 63, 64);
         s_b[buf][l] = x;
@@ -216,6 +269,9 @@ __global__ __launch_bounds__(2 * NTHR) void k_state_bwd(const lmoe_args a) {
         for (int i = 0; i < 4; ++i)
           dS[mi][ni][i] = p[(int64_t)(krow0 + acc_row(mi, i)) * V + v0 + acc_col(ni)];
   }
+  f32x4 dz[NORM ? MB : 1];                  // NORM: gradient of the column of ones (the same sum in every column)
+#pragma unroll
+  for (int mi = 0; mi < (NORM ? MB : 1); ++mi) dz[mi] = f32x4{0.f, 0.f, 0.f, 0.f};
   lds_barrier();                                     // P0
   for (int it = 0; it < sq.nchunks; ++it) {
     const int c = sq.nchunks - 1 - it;
@@ -224,6 +280,18 @@ __global__ __launch_bounds__(2 * NTHR) void k_state_bwd(const lmoe_args a) {
     for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
       for (int ni = 0; ni < NB; ++ni) acc_to_lds_t<T>(dS[mi][ni], s_dST, LDK, krow0 + 16 * mi, 16 * ni);
+    if constexpr (NORM) {
+      // dz at the end of chunk c (partial): from this team, which has no loads in flight that a store could wait for
+      if ((l & 15) == 0) {
+        float* ws = ws_row(c) + CH;
+#pragma unroll
+        for (int mi = 0; mi < MB; ++mi) {
+          const int row = krow0 + 16 * mi + 4 * (l >> 4);
+          *(f32x4*)&ws[row] = dz[mi];
+          if constexpr (SLOTS_PER_SLICE == 2) *(f32x4*)&ws[WS_ROW + row] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+      }
+    }
     lds_barrier();                                                                       // B1
     const float dec = s_dec[cur];
     f32x4 t[1][NB];
@@ -247,6 +315,14 @@ __global__ __launch_bounds__(2 * NTHR) void k_state_bwd(const lmoe_args a) {
       for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
         for (int ni = 0; ni < NB; ++ni) ET<T>::mma(dS[mi][ni], af[mi], bf[ni]);
+      if constexpr (NORM) {                 // dz += q^T (scale dden): sixteen equal columns
+        const f32x4 d0 = *(const f32x4*)&s_dd[cur][kk + 8 * (l >> 4)], d1 = *(const f32x4*)&s_dd[cur][kk + 8 * (l >> 4) + 4];
+        typename ET<T>::frag fd;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { fd[e] = (bf16)d0[e]; fd[e + 4] = (bf16)d1[e]; }
+#pragma unroll
+        for (int mi = 0; mi < MB; ++mi) ET<T>::mma(dz[mi], af[mi], fd);
+      }
     }
     if constexpr (NBUF == 1) {
       lds_barrier();                                                                     // B3
@@ -512,9 +588,17 @@ __global__ __launch_bounds__(2 * NTHR) void k_bwd_dqk(const lmoe_args a) {
 //               c | stores | E
 // Every sum is formed in the order of k_bwd_dv and k_bwd_dqk: the results are theirs bit for bit.
 // ------------------------------------------------------------------------- //
-template <typename T, int K, int V, int BVH>
+// NORM (see k_state_bwd): d_o is the gradient of the normalised output.  With rD = 1 / D, dd = scale dden (the sum of
+// the partial rows of norm_ws), z = the sum of the keys before the chunk (zs) and dz = the gradient of the column of
+// ones at the end of the chunk (the sum of the partial rows of norm_ws), ungated:
+//   dv: P^T formed with its rows i scaled by rD_i;   dP_ij -> scale dP_ij rD_i + dd_i;
+//   dq_i = scale rD_i dq_i,inter + dd_i z + (dP k)_i;   dk_j = dk_d,j + dz + (dP^T q)_j
+// i.e. row and column factors on sums the kernel forms anyway; d_o itself is staged as it is.
+template <typename T, int K, int V, int BVH, bool NORM = false>
 __global__ __launch_bounds__(2 * NTHR) void k_bwd_dqkv(const lmoe_args a) {
   static_assert(sizeof(T) == 2, "2-byte elements");
+  constexpr int WS_ROW = CH + K, WS_SLOTS = V / NORM_SLOT_COLS;
+  static_assert(CH + K <= NTHR, "one loader thread per entry of a row of norm_ws");
   constexpr int LDV = BVH + LPAD, LDC = CH + LPAD, LDK = K + LPAD;
   constexpr int NBK = K / 16, NS = V / BVH, NBV = BVH / 16, KS = K / 32, CS = CH / 32;
   // tiles of one V-slice (two buffers)
@@ -527,6 +611,9 @@ __global__ __launch_bounds__(2 * NTHR) void k_bwd_dqkv(const lmoe_args a) {
   __shared__ __attribute__((aligned(16))) T smem[NELEM];
   __shared__ __attribute__((aligned(16))) float s_b[2][64], s_eb[2][64], s_ed[2][64];
   __shared__ float s_db[64], s_red[8];
+  // NORM: rD and dd per row, z and dz per key column (two sets, like the gate arrays)
+  __shared__ __attribute__((aligned(16))) float s_rD[NORM ? 2 : 1][NORM ? 64 : 4], s_dd[NORM ? 2 : 1][NORM ? 64 : 4];
+  __shared__ __attribute__((aligned(16))) float s_z[NORM ? 2 : 1][NORM ? K : 4], s_dz[NORM ? 2 : 1][NORM ? K : 4];
 
   const int l = lane_id();
   const int team = threadIdx.x / NTHR;
@@ -540,9 +627,11 @@ __global__ __launch_bounds__(2 * NTHR) void k_bwd_dqkv(const lmoe_args a) {
   if (team == 1) {
     // --------------------------------- loaders -------------------------------------------
     struct SliceRegs { typename IOV::Regs rd, rv; typename IOH::Regs rh, rdh; int len; };
-    struct QKRegs { typename IOK::Regs rq, rk; uint32_t graw; int len; };
+    // (NORM: thread e < 64 + K holds entry e of the rows of norm_ws and D of row e or z of column e - 64)
+    struct QKRegs { typename IOK::Regs rq, rk; uint32_t graw; int len; float ws[NORM ? WS_SLOTS : 1], x; };
     SliceRegs S;
     QKRegs Q;
+    const int e_norm = min((int)(threadIdx.x & (NTHR - 1)), WS_ROW - 1);
     // Every prefetch is issued unconditionally (item index clamped to the last item): a load that
     // is skipped on some path would make the compiler drain all outstanding loads at every use.
     auto issue_slice = [&](int it, int vv) {
@@ -563,6 +652,14 @@ __global__ __launch_bounds__(2 * NTHR) void k_bwd_dqkv(const lmoe_args a) {
       IOK::load_nomask(Q.rq, row_ptr<T>(a.q, ci.b, ci.tok, h), a.q.st, ci.len);
       IOK::load_nomask(Q.rk, row_ptr<T>(a.k, ci.b, ci.tok, h), a.k.st, ci.len);
       Q.graw = gate_prefetch(a, ci.b, ci.tok, ci.len, h);
+      if constexpr (NORM) {
+        const float* ws = a.norm_ws + (int64_t)it * WS_SLOTS * WS_ROW + e_norm;          // it = cid * H + h
+#pragma unroll
+        for (int sl = 0; sl < WS_SLOTS; ++sl) Q.ws[sl] = ws[sl * WS_ROW];
+        const float* den = (const float*)a.den.ptr + row_off(a.den, ci.b, ci.tok + min(e_norm, ci.len - 1), h);
+        const float* zc = a.zs + (int64_t)it * K + max(e_norm - CH, 0);
+        Q.x = *(e_norm < CH ? den : zc);
+      }
     };
     float hdh = 0.f;   // partial <S, dS'> of the item whose slices are being staged
     auto stage_slice = [&](int buf) {
@@ -579,6 +676,19 @@ __global__ __launch_bounds__(2 * NTHR) void k_bwd_dqkv(const lmoe_args a) {
       IOH::store_lds(S.rdh, base + A_DH, LDK);
     };
     auto stage_qk = [&](int par) {
+      if constexpr (NORM) {
+        float sum = 0.f;
+#pragma unroll
+        for (int sl = 0; sl < WS_SLOTS; ++sl) sum += Q.ws[sl];
+        const int e = threadIdx.x & (NTHR - 1);
+        if (e < CH) {
+          s_dd[par][e] = sum;                                // (zero past the end of a partial chunk)
+          s_rD[par][e] = e < Q.len ? 1.f / Q.x : 0.f;
+        } else if (e < WS_ROW) {
+          s_dz[par][e - CH] = sum;
+          s_z[par][e - CH] = Q.x;
+        }
+      }
       gate_finish_wave(a, Q.graw, Q.len, l, wave_id() == 4, s_b[par], s_eb[par], s_ed[par]);
       IOK::mask(Q.rq, Q.len);
       IOK::mask(Q.rk, Q.len);
@@ -657,6 +767,11 @@ __global__ __launch_bounds__(2 * NTHR) void k_bwd_dqkv(const lmoe_args a) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) ET<T>::mma(acc, fq[ks], fk[ks]);
         const f32x4 bi = *(const f32x4*)&s_b[par][16 * ib + 4 * g];
+        if constexpr (NORM) {
+          const f32x4 rdi = *(const f32x4*)&s_rD[par][16 * ib + 4 * g];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[e] *= rdi[e];
+        }
 #pragma unroll
         for (int e = 0; e < 4; ++e) y[e] = (bf16)((16 * ib + 4 * g + e >= j) ? acc[e] * texp<T>(bi[e] - bj) : 0.f);
       }
@@ -730,7 +845,8 @@ __global__ __launch_bounds__(2 * NTHR) void k_bwd_dqkv(const lmoe_args a) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int r = 16 * wv + 4 * g + i, cc = 16 * nj + fr;
-        p[i] = (r >= cc) ? a.scale * dP[0][nj][i] * texp<T>(s_b[par][r] - s_b[par][cc]) : 0.f;
+        if constexpr (NORM) p[i] = (r >= cc) ? a.scale * dP[0][nj][i] * s_rD[par][r] + s_dd[par][r] : 0.f;
+        else p[i] = (r >= cc) ? a.scale * dP[0][nj][i] * texp<T>(s_b[par][r] - s_b[par][cc]) : 0.f;
       }
       acc_to_lds_t<T>(p, PT, LDC, 16 * wv, 16 * nj, lf);      // [j][i]
     }
@@ -753,8 +869,14 @@ __global__ __launch_bounds__(2 * NTHR) void k_bwd_dqkv(const lmoe_args a) {
         const int r = 16 * wv + 4 * g + i, cc = 16 * ni + fr;
         const float qv = ET<T>::to_f(QT[r * LDK + cc]);
         const float kv = ET<T>::to_f(KT[r * LDK + cc]);
-        const float dqv = a.scale * s_eb[par][r] * dqi[0][ni][i] + dq[0][ni][i];
-        const float dkdv = s_ed[par][r] * dkd[0][ni][i];
+        float dqv, dkdv;
+        if constexpr (NORM) {
+          dqv = a.scale * s_rD[par][r] * dqi[0][ni][i] + s_dd[par][r] * s_z[par][cc] + dq[0][ni][i];
+          dkdv = dkd[0][ni][i] + s_dz[par][cc];
+        } else {
+          dqv = a.scale * s_eb[par][r] * dqi[0][ni][i] + dq[0][ni][i];
+          dkdv = s_ed[par][r] * dkd[0][ni][i];
+        }
         const float dkv = dkdv + dk[0][ni][i];
         dbp[i] += qv * dqv - kv * dkv;
         kk += kv * dkdv;

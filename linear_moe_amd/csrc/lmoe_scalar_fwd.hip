@@ -9,25 +9,34 @@ template <typename T, int V> struct FwdTiles {
   static constexpr int BVS = sizeof(T) == 4 ? 16 : 32;
 };
 
+// the pass for 2-byte elements on V slices of BV columns: saving or forward-only, plain or with the normalised output
+template <typename T, int K, int V, int BV> void launch_fwd_b(const lmoe_args& a, hipStream_t st) {
+  const dim3 grid(((a.N * a.H + 7) / 8) * 8 * (V / BV)), block(3 * NTHR);
+  long long* const no_trace = nullptr;
+  if (a.normalize) {
+    if (a.hs) hipLaunchKernelGGL((k_state_fwd_b<T, K, V, BV, true, false, true>), grid, block, 0, st, a, no_trace, -1);
+    else hipLaunchKernelGGL((k_state_fwd_b<T, K, V, BV, false, false, true>), grid, block, 0, st, a, no_trace, -1);
+  } else {
+    if (a.hs) hipLaunchKernelGGL((k_state_fwd_b<T, K, V, BV, true>), grid, block, 0, st, a, no_trace, -1);
+    else hipLaunchKernelGGL((k_state_fwd_b<T, K, V, BV, false>), grid, block, 0, st, a, no_trace, -1);
+  }
+}
 template <typename T, int K, int V> struct StateFwd {
   static void run(const lmoe_args& a, hipStream_t st) {
     constexpr int BV = FwdTiles<T, V>::BVS;
-    const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BV);
     if constexpr (sizeof(T) == 2) {
       // 64-wide slices where they still fill the chip: every V slice of a (sequence, head) fetches all of q and k and
       // forms all of P, so two wide slices cost less per output column than four narrow ones; the results do not
       // depend on the width (a state element and an output element are the same sums in either split)
       if constexpr (V >= 64) {
         if ((int64_t)a.N * a.H * (V / 64) >= cu_count()) {
-          const int gw = ((a.N * a.H + 7) / 8) * 8 * (V / 64);
-          if (a.hs) hipLaunchKernelGGL((k_state_fwd_b<T, K, V, 64, true>), dim3(gw), dim3(3 * NTHR), 0, st, a, (long long*)nullptr, -1);
-          else hipLaunchKernelGGL((k_state_fwd_b<T, K, V, 64, false>), dim3(gw), dim3(3 * NTHR), 0, st, a, (long long*)nullptr, -1);
+          launch_fwd_b<T, K, V, 64>(a, st);
           return;
         }
       }
-      if (a.hs) hipLaunchKernelGGL((k_state_fwd_b<T, K, V, BV, true>), dim3(grid), dim3(3 * NTHR), 0, st, a, (long long*)nullptr, -1);
-      else hipLaunchKernelGGL((k_state_fwd_b<T, K, V, BV, false>), dim3(grid), dim3(3 * NTHR), 0, st, a, (long long*)nullptr, -1);
+      launch_fwd_b<T, K, V, BV>(a, st);
     } else {
+      const int grid = ((a.N * a.H + 7) / 8) * 8 * (V / BV);
       if (a.hs) hipLaunchKernelGGL((k_state_fwd<T, K, V, BV, true>), dim3(grid), dim3(3 * NTHR), 0, st, a);
       else hipLaunchKernelGGL((k_state_fwd<T, K, V, BV, false>), dim3(grid), dim3(3 * NTHR), 0, st, a);
     }

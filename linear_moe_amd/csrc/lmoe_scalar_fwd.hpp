@@ -274,9 +274,14 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
 // ------------------------------------------------------------------------- //
 constexpr int SFWD_TRACE_CHUNKS = 24, SFWD_TRACE_MARKS = 8, SFWD_TRACE_SLOTS = 3;
 
-template <typename T, int K, int V, int BV, bool SAVE, bool TRACE = false>
+// NORM (ungated calls): the output leaves divided by den + eps, den_i = scale q_i . (sum of the keys up to i) - the
+// op with one more value column of ones, carried beside the state as one more accumulator column (z = the sum of the
+// keys of the chunks before, fp32 in LDS and, for the backward, in zs) and formed by every V slice for itself:
+// consumers z += k^T 1, output team q z and the row sums of P as two more products against a fragment of ones.
+template <typename T, int K, int V, int BV, bool SAVE, bool TRACE = false, bool NORM = false>
 __global__ __launch_bounds__(3 * NTHR) void k_state_fwd_b(const lmoe_args a, long long* tr, int traced_wg) {
   static_assert(sizeof(T) == 2, "2-byte elements");
+  static_assert(!(NORM && TRACE), "the traced instance is the plain pass");
   constexpr int LDK = K + LPAD, LDC = CH + LPAD, LDU = BV + LPAD;
   constexpr int MB = K / 64, NB = BV / 16, KS = K / 32, CS = CH / 32;
   __shared__ __attribute__((aligned(16))) T s_k[2][CH * LDK];                 // k             [64][K]
@@ -286,6 +291,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd_b(const lmoe_args a, lon
   __shared__ __attribute__((aligned(16))) T s_P[2][CH * LDC];                 // P             [64][64]
   __shared__ __attribute__((aligned(16))) float s_b[2][64], s_eb[2][64], s_ed[2][64];
   __shared__ float s_dec[2];                                                  // e^{b_C} per buffer
+  __shared__ __attribute__((aligned(16))) float s_z[NORM ? 2 : 1][NORM ? K : 4];   // NORM: the sum of the keys before a chunk
   // (the low 32 bits of the clock: whoever reads the stamps takes their differences modulo 2^32)
   __shared__ uint32_t s_tr[TRACE ? SFWD_TRACE_SLOTS * SFWD_TRACE_CHUNKS * SFWD_TRACE_MARKS : 1];
   auto TR = [&](int slot, int c, int mark) {
@@ -535,6 +541,19 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd_b(const lmoe_args a, lon
 #pragma unroll
       for (int kq = 0; kq < CS; ++kq)
         if (2 * kq <= ow) fp[kq] = ET<T>::load_frag(Pc + (16 * ow + fr) * LDC + 32 * kq + fg);
+      f32x4 oz = {0.f, 0.f, 0.f, 0.f};
+      if constexpr (NORM) {
+        // q z, with z as a matrix operand of sixteen equal rows (every lane group reads the same eight columns):
+        // every row of the accumulator holds the same sum
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const f32x4 z0 = *(const f32x4*)&s_z[c & 1][32 * ks + fg], z1 = *(const f32x4*)&s_z[c & 1][32 * ks + fg + 4];
+          typename ET<T>::frag fz;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) { fz[e] = (bf16)z0[e]; fz[e + 4] = (bf16)z1[e]; }
+          ET<T>::mma(oz, fz, fq[ks]);
+        }
+      }
       __builtin_amdgcn_sched_barrier(0);
       f32x4 ot[NB], pv[NB];
 #pragma unroll
@@ -551,6 +570,21 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd_b(const lmoe_args a, lon
           for (int ni = 0; ni < NB; ++ni) ET<T>::mma(pv[ni], fv[kq][ni], fp[kq]);         // (P v)^T
         }
       }
+      float rden = 1.f;
+      if constexpr (NORM) {
+        // the row sums of P (as rounded for P v), again the same sum in every row of the accumulator
+        typename ET<T>::frag one8;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) one8[e] = (bf16)1.f;
+        f32x4 pz = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kq = 0; kq < CS; ++kq)
+          if (2 * kq <= ow) ET<T>::mma(pz, one8, fp[kq]);
+        const float dsum = (oz[0] * ebi + pz[0]) * a.scale + a.norm_eps;
+        rden = 1.f / dsum;
+        if (vsl == 0 && l < 16 && 16 * ow + fr < len)
+          ((float*)a.den.ptr)[row_off(a.den, sq.b, tok + 16 * ow + fr, h)] = dsum;
+      }
       __builtin_amdgcn_sched_barrier(0);
       if (ow == 0) TR(2, c, 2);
       // lane: token 16 ow + fr, columns 16 ni + g4 .. + 3
@@ -558,7 +592,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd_b(const lmoe_args a, lon
       if (16 * ow + fr < len) {
 #pragma unroll
         for (int ni = 0; ni < NB; ++ni) {
-          const f32x4 x = (ot[ni] * ebi + pv[ni]) * a.scale;
+          const f32x4 x = (ot[ni] * ebi + pv[ni]) * (NORM ? a.scale * rden : a.scale);
           bf16x4 y;
 #pragma unroll
           for (int e = 0; e < 4; ++e) y[e] = (bf16)x[e];
@@ -591,11 +625,27 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd_b(const lmoe_args a, lon
         for (int i = 0; i < 4; ++i)
           S[mi][ni][i] = h0[(int64_t)(krow0 + acc_row(mi, i)) * V + v0 + acc_col(ni)];
   }
-  auto copy_state = [&](int buf) {          // S -> LDS as S^T
+  f32x4 Sz[NORM ? MB : 1];                  // NORM: the column of ones (every column of the tile holds the same sum)
+#pragma unroll
+  for (int mi = 0; mi < (NORM ? MB : 1); ++mi) Sz[mi] = f32x4{0.f, 0.f, 0.f, 0.f};
+  auto copy_state = [&](int c) {            // S at the start of chunk c -> LDS as S^T
+    const int buf = c & 1;
 #pragma unroll
     for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
       for (int ni = 0; ni < NB; ++ni) acc_to_lds_t<T>(S[mi][ni], s_hT[buf], LDK, krow0 + 16 * mi, 16 * ni);
+    if constexpr (NORM) {
+      // z beside it, and (SAVE) to zs for the backward: from this team, which has no loads in flight that a store
+      // could be made to wait for, and by every V slice (they hold the same sums bit for bit)
+      if ((l & 15) == 0) {
+#pragma unroll
+        for (int mi = 0; mi < MB; ++mi) {
+          const int row = krow0 + 16 * mi + 4 * (l >> 4);
+          *(f32x4*)&s_z[buf][row] = Sz[mi];
+          if constexpr (SAVE) *(f32x4*)&a.zs[((int64_t)(sq.chunk0 + c) * a.H + h) * K + row] = Sz[mi];
+        }
+      }
+    }
   };
   const int pti = wv == 0 ? 3 : wv == 1 ? 2 : wv == 2 ? 3 : 1, ptja = wv == 2 ? 2 : 0, pn = wv < 2 ? 2 : 1;
   copy_state(0);
@@ -637,10 +687,19 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd_b(const lmoe_args a, lon
       for (int mi = 0; mi < MB; ++mi)
 #pragma unroll
         for (int ni = 0; ni < NB; ++ni) ET<T>::mma(S[mi][ni], af[kq][mi], bf[kq][ni]);
+    if constexpr (NORM) {                   // z += k^T 1 (ungated: no decay; rows past the end of a chunk are zero)
+      typename ET<T>::frag one8;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) one8[e] = (bf16)1.f;
+#pragma unroll
+      for (int kq = 0; kq < CS; ++kq)
+#pragma unroll
+        for (int mi = 0; mi < MB; ++mi) ET<T>::mma(Sz[mi], af[kq][mi], one8);
+    }
     __builtin_amdgcn_sched_barrier(0);
     if (wv == 0) TR(0, c, 5);
     if (c + 1 < sq.nchunks) {
-      copy_state((c + 1) & 1);
+      copy_state(c + 1);
       if (wv == 0) TR(0, c, 6);
       p_blocks(c + 1, pti, ptja, 1, pn);
       if (wv == 0) TR(0, c, 2);

@@ -12,7 +12,7 @@ from typing import Optional, Tuple
 
 import torch
 
-from .simple_gla import chunk_simple_gla
+from .simple_gla import can_normalize, chunk_simple_gla, chunk_simple_gla_normalized
 
 
 def chunk_linear_attn(
@@ -40,9 +40,18 @@ def chunk_linear_attn(
         initial_state = torch.nn.functional.pad(initial_state, (0, 0, 0, K - initial_state.shape[-2]))
     # The normaliser z_i = scale sum_{j<=i} q_i . k_j is the op itself with one more value column of ones (fla
     # normalises with q * scale, so the scale cancels in o up to the epsilon): it is formed inside the kernels, in
-    # the fp32 state, instead of by a cumulative sum over k in HBM.  chunk_simple_gla cuts the V + 1 columns into
-    # the blocks the kernels take; the carried state has no normaliser column (the sum starts inside the call).
+    # the fp32 state, instead of by a cumulative sum over k in HBM.
     V = v.shape[-1]
+    if normalize and len(qb) == 1 and can_normalize(qb[0], v):
+        # one key block of bfloat16: the kernels carry the column themselves and divide before they store
+        o, ht = chunk_simple_gla_normalized(qb[0], kb[0], v, scale, initial_state, output_final_state, None,
+                                            head_first, _eps)
+        if ht is not None and ht.shape[-2] != (q.features if hasattr(q, "features") else q.shape[-1]):
+            ht = ht[..., :(q.features if hasattr(q, "features") else q.shape[-1]), :]
+        return o, ht
+    # otherwise (fp32, several key blocks, other head dimensions) the column is appended here: chunk_simple_gla cuts
+    # the V + 1 columns into the blocks the kernels take; the carried state has no normaliser column (the sum starts
+    # inside the call).
     if normalize:
         v = torch.cat([v, v.new_ones(*v.shape[:-1], 1)], dim=-1)
         if initial_state is not None:

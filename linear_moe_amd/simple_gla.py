@@ -28,8 +28,11 @@ class SimpleGLACall:
         # blocks stay valid for lmoe_launch_stage; the autograd path must not (reference cycle)
         self.keep = keep
 
-    def forward(self, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first, save=True):
-        """save=False: a forward-only call (nothing requires a gradient): the per-chunk states are not written."""
+    def forward(self, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first, save=True,
+                norm_eps=None):
+        """save=False: a forward-only call (nothing requires a gradient): the per-chunk states are not written.
+        norm_eps: the output leaves the kernels divided by ``scale q_t . sum_{s<=t} k_s + norm_eps`` (ungated calls
+        on 2-byte elements: ``can_normalize``)."""
         ctx = self
         lib = _lib.load()
         dims = _check_inputs(q, k, v, head_first, cu_seqlens)
@@ -55,14 +58,24 @@ class SimpleGLACall:
         a.o = _desc(o, head_first)
         a.ht = ptr(ht)
         a.hs = ptr(hs)
+        den = zs = None
+        if norm_eps is not None:
+            if g is not None or q.dtype != torch.bfloat16:
+                raise ValueError("the normalised output exists for ungated calls on bfloat16")
+            den = torch.empty((B, H, T) if head_first else (B, T, H), dtype=torch.float32, device=q.device)
+            zs = torch.empty(max(plan.NT, 1), H, K, dtype=torch.float32, device=q.device) if save else None
+            a.normalize, a.norm_eps, a.den, a.zs = 1, norm_eps, _desc(den, head_first), ptr(zs)
         _lib.check(lib.lmoe_chunk_simple_gla_fwd(C.byref(a), stream_ptr()), "chunk_simple_gla forward")
         ctx.saved = (q, k, v, g, h0, hs)
+        ctx.norm = None if norm_eps is None else (norm_eps, den, zs)
         ctx.fwd_args, ctx.fwd_keep = a, ((o, ht) if self.keep else None)
         ctx.plan, ctx.dims, ctx.head_first, ctx.scale = plan, dims, head_first, scale
         ctx.has_h0 = initial_state is not None
         return o, ht
 
-    def backward(self, do, dht):
+    def backward(self, do, dht, o=None):
+        """o: the output of the forward call, for a call with norm_eps (handed in by the caller, who holds it: this
+        object must not, it would close a reference cycle through the autograd graph)."""
         ctx = self
         lib = _lib.load()
         q, k, v, g, h0, hs = ctx.saved
@@ -89,9 +102,16 @@ class SimpleGLACall:
         a.dh0 = ptr(dh0)
         dhs = torch.empty_like(hs)
         a.dhs = dhs.data_ptr()
+        norm_ws = None
+        if ctx.norm is not None:
+            norm_eps, den, zs = ctx.norm
+            o = _aligned(o)
+            norm_ws = torch.empty(max(plan.NT, 1), H, V // 32, 64 + K, dtype=torch.float32, device=q.device)
+            a.normalize, a.norm_eps, a.den, a.zs = 1, norm_eps, _desc(den, head_first), zs.data_ptr()
+            a.o, a.norm_ws = _desc(o, head_first), norm_ws.data_ptr()
         _lib.check(lib.lmoe_chunk_simple_gla_bwd(C.byref(a), stream_ptr()), "chunk_simple_gla backward")
         ctx.bwd_args = a
-        ctx.bwd_keep = (do, dht, dq, dk, dv, dg, dh0, dhs) if self.keep else None
+        ctx.bwd_keep = (do, dht, dq, dk, dv, dg, dh0, dhs, norm_ws, o) if self.keep else None
         if dg is not None and dg.dtype != g.dtype:
             dg = dg.to(g.dtype)
         return dq, dk, dv, dg, dh0
@@ -99,17 +119,42 @@ class SimpleGLACall:
 
 class _ChunkSimpleGLA(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first):
+    def forward(ctx, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first, norm_eps=None):
         call = SimpleGLACall()
         o, ht = call.forward(q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first,
-                             save=any(ctx.needs_input_grad))
+                             save=any(ctx.needs_input_grad), norm_eps=norm_eps)
         ctx.call = call
+        if norm_eps is not None:
+            ctx.save_for_backward(o)          # the backward of the normalisation reads the output
         return o, ht
 
     @staticmethod
     def backward(ctx, do, dht):
-        dq, dk, dv, dg, dh0 = ctx.call.backward(do, dht)
-        return dq, dk, dv, dg, None, dh0, None, None, None
+        o = ctx.saved_tensors[0] if ctx.saved_tensors else None
+        dq, dk, dv, dg, dh0 = ctx.call.backward(do, dht, o)
+        return dq, dk, dv, dg, None, dh0, None, None, None, None
+
+
+def can_normalize(q, v, g=None) -> bool:
+    """Whether ``chunk_simple_gla_normalized`` takes this call: ungated, bfloat16, head dimensions of 64 or 128."""
+    return (g is None and q.dim() == 4 and v.dim() == 4 and q.dtype == torch.bfloat16
+            and q.shape[-1] in HEAD_DIMS and v.shape[-1] in HEAD_DIMS)
+
+
+def chunk_simple_gla_normalized(q, k, v, scale=None, initial_state=None, output_final_state=False, cu_seqlens=None,
+                                head_first=True, eps: float = 1e-10):
+    """The ungated op with the normaliser of ``fla.ops.linear_attn.chunk_linear_attn(normalize=True)`` inside the
+    kernels: ``o_t = scale q_t S_t / (scale q_t . sum_{s<=t} k_s + eps)`` -- the sum of the keys is carried beside the
+    state as one more column, nothing passes through memory between the op and the division, and the backward folds
+    the gradient of the divisor into the sums it forms anyway.  ``initial_state`` seeds S only: the sum of the keys
+    starts inside the call.  Returns ``(o, final_state)``."""
+    if not can_normalize(q, v):
+        raise ValueError("chunk_simple_gla_normalized: bfloat16 q, k, v with head dimensions of 64 or 128")
+    r = no_tokens(q, k, v, head_first, cu_seqlens, initial_state, output_final_state)
+    if r is not None:
+        return r
+    return _ChunkSimpleGLA.apply(q, k, v, None, scale, initial_state, output_final_state, cu_seqlens, head_first,
+                                 float(eps))
 
 
 def chunk_simple_gla(

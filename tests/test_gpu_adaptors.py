@@ -72,3 +72,78 @@ def test_linear_attn_normalised_default_scale(cuda, scale, head_first):
     assert max_abs_rel(tf(o.detach().cpu()), ref.detach()) < 1e-5
     for gd, gr, n in zip(grads, ref_g, "qkv"):
         assert max_abs_rel(tf(gd.cpu()), gr) < 1e-5, n
+
+
+def _normalised_closed_form(q, k, v, h0, do, dht, sc, lens=None, eps=1e-10):
+    """fp64: o_t = (sum_s a_ts v_s + sc q_t h0) / (sum_s a_ts + eps), a_ts = sc q_t.k_s [s <= t]; [B,H,T,*] inputs
+    (lens: the sequences packed along T of a batch of one).  Returns o, final state and their gradients."""
+    ins = [x.double().requires_grad_(True) for x in (q, k, v, h0)]
+    qd, kd, vd, hd = ins
+    T = q.shape[2]
+    bounds = [0, T] if lens is None else [0] + list(torch.tensor(lens).cumsum(0))
+    os_, hts = [], []
+    for n in range(len(bounds) - 1):
+        a0, a1 = int(bounds[n]), int(bounds[n + 1])
+        hn = hd if lens is None else hd[n:n + 1]
+        A = torch.tril(sc * qd[:, :, a0:a1] @ kd[:, :, a0:a1].transpose(-1, -2))
+        os_.append((A @ vd[:, :, a0:a1] + sc * qd[:, :, a0:a1] @ hn) / (A.sum(-1, keepdim=True) + eps))
+        hts.append(hn + kd[:, :, a0:a1].transpose(-1, -2) @ vd[:, :, a0:a1])
+    o, ht = torch.cat(os_, 2), torch.cat(hts, 0)
+    grads = torch.autograd.grad((o * do.double()).sum() + (ht * dht.double()).sum(), ins)
+    return o.detach(), ht.detach(), grads
+
+
+@pytest.mark.parametrize("head_first", [True, False])
+@pytest.mark.parametrize("shape", [(2, 3, 333, 64, 64), (2, 2, 200, 128, 128), (1, 3, 130, 64, 128), (1, 2, 70, 128, 64),
+                                   (4, 32, 130, 128, 128), (8, 32, 65, 64, 64)])
+def test_linear_attn_normalised_inside_the_kernels(cuda, shape, head_first):
+    """bfloat16 with one key block: the kernels carry the sum of the keys beside the state and divide before they
+    store; the backward folds the gradient of the divisor into its own sums.  Against the closed form in fp64 on the
+    same bf16 inputs, output, final state and every gradient (the last two shapes run the 64-column slices of the
+    state passes, the others the 32-column ones)."""
+    from linear_moe_amd import chunk_linear_attn
+    B, H, T, K, V = shape
+    bf = torch.bfloat16
+    q, k = (gen(3301, B, H, T, K).abs() + 0.1).to(bf), (gen(3302, B, H, T, K).abs() + 0.1).to(bf)
+    v, do = gen(3303, B, H, T, V, dtype=bf), gen(3304, B, H, T, V, dtype=bf)
+    h0, dht = gen(3305, B, H, K, V) * 0.5, gen(3306, B, H, K, V)
+    sc = K ** -0.5
+    ref_o, ref_ht, ref_g = _normalised_closed_form(q, k, v, h0, do, dht, sc)
+    tf = (lambda x: x) if head_first else (lambda x: x.transpose(1, 2).contiguous())
+    dev_in = [tf(x).to(cuda).requires_grad_(True) for x in (q, k, v)] + [h0.to(cuda).requires_grad_(True)]
+    o, ht = chunk_linear_attn(*dev_in[:3], initial_state=dev_in[3], output_final_state=True, normalize=True,
+                              head_first=head_first)
+    grads = torch.autograd.grad((o * tf(do).to(cuda)).sum() + (ht * dht.to(cuda)).sum(), dev_in)
+    torch.cuda.synchronize()
+    assert o.dtype == bf
+    assert max_abs_rel(tf(o.detach().cpu()), ref_o) < TOL[bf]
+    assert max_abs_rel(ht.detach().cpu(), ref_ht) < TOL[bf]
+    for gd, gr, n in zip(grads, ref_g, ("q", "k", "v", "h0")):
+        gd = gd.cpu() if n == "h0" else tf(gd.cpu())
+        assert max_abs_rel(gd, gr) < TOL[bf], n
+
+
+def test_normalised_op_on_packed_sequences_and_forward_only(cuda):
+    """The normalised op on sequences packed along T (the sum of the keys starts anew in every sequence), and a
+    forward-only call (nothing saved) giving the bits of the saving one."""
+    from linear_moe_amd.simple_gla import chunk_simple_gla_normalized
+    lens, H, K, V = [70, 1, 129, 64], 2, 128, 128
+    T, N, bf = sum(lens), len(lens), torch.bfloat16
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    q, k = (gen(3401, 1, H, T, K).abs() + 0.1).to(bf), (gen(3402, 1, H, T, K).abs() + 0.1).to(bf)
+    v, do = gen(3403, 1, H, T, V, dtype=bf), gen(3404, 1, H, T, V, dtype=bf)
+    h0, dht = gen(3405, N, H, K, V) * 0.5, gen(3406, N, H, K, V)
+    ref_o, ref_ht, ref_g = _normalised_closed_form(q, k, v, h0, do, dht, K ** -0.5, lens)
+    tf = lambda x: x.transpose(1, 2).contiguous()
+    dev_in = [tf(x).to(cuda).requires_grad_(True) for x in (q, k, v)] + [h0.to(cuda).requires_grad_(True)]
+    o, ht = chunk_simple_gla_normalized(*dev_in[:3], None, dev_in[3], True, cu.to(cuda), False)
+    grads = torch.autograd.grad((o * tf(do).to(cuda)).sum() + (ht * dht.to(cuda)).sum(), dev_in)
+    with torch.no_grad():
+        o2, ht2 = chunk_simple_gla_normalized(*dev_in[:3], None, dev_in[3], True, cu.to(cuda), False)
+    torch.cuda.synchronize()
+    assert torch.equal(o2, o.detach()) and torch.equal(ht2, ht.detach())
+    assert max_abs_rel(tf(o.detach().cpu()), ref_o) < TOL[bf]
+    assert max_abs_rel(ht.detach().cpu(), ref_ht) < TOL[bf]
+    for gd, gr, n in zip(grads, ref_g, ("q", "k", "v", "h0")):
+        gd = gd.cpu() if n == "h0" else tf(gd.cpu())
+        assert max_abs_rel(gd, gr) < TOL[bf], n
