@@ -386,7 +386,8 @@ def layer_bench(dev, steps, warmup):
     q / k / v split, layout change, SiLU, L2 norm, gate construction, the chunk op, layout change back and
     o * swish(o_gate) (linear_moe/sequence_modeling/linear_attention.py:153-163, 255 around
     gated_deltanet/gated_deltanet.py:99-114), forward + backward on the headline shape.  `unfused` is the chain of
-    strided copies, row kernels and eager elementwise ops; `fused` the one-pass prologue / epilogue kernels."""
+    strided copies, row kernels and eager elementwise ops; `fused` the one-pass prologue / epilogue kernels;
+    `mixer_core` prologue and op as one call (the op applies SiLU to v where it reads the projection)."""
     import torch
     import torch.nn.functional as F
     import linear_moe_amd as L
@@ -401,8 +402,10 @@ def layer_bench(dev, steps, warmup):
     dy = rn(T, B, H * D).to(torch.bfloat16).to(dev)
     leaves = [qkv, o_gate, a, b, A_log, dt_bias]
 
-    def mixer(fused):
+    def mixer(fused, core=False):
         gk, beta = L.gdn_gates(a, b, A_log, dt_bias)
+        if core:       # prologue and op in one call: silu(v) never written, dv written into the projection's gradient
+            return L.swish_gate_relayout(L.gdn_mixer_core(qkv, gk, beta, H, D), o_gate)
         if fused:
             q, k, v = L.gdn_qkv_prologue(qkv, H, D)
         else:
@@ -414,8 +417,8 @@ def layer_bench(dev, steps, warmup):
             return L.swish_gate_relayout(o, o_gate)
         return o.transpose(0, 1).reshape(T, B, H * D) * F.silu(o_gate)
 
-    def step(fused):
-        torch.autograd.grad([mixer(fused)], leaves, [dy])
+    def step(fused, core=False):
+        torch.autograd.grad([mixer(fused, core)], leaves, [dy])
 
     # the op alone on inputs of the same laws as the headline (what the layer's neighbours are compared with)
     x = gdn_inputs(B, T, H, D, D, 1004, torch.bfloat16, dev)
@@ -435,21 +438,25 @@ def layer_bench(dev, steps, warmup):
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / steps
 
-    for fn in (step_op, lambda: step(False), lambda: step(True)):      # everything warm before anything is timed
+    for fn in (step_op, lambda: step(False), lambda: step(True), lambda: step(True, True)):   # everything warm first
         timed(fn)
     t_op = timed(step_op)
     t_un = timed(lambda: step(False))
     t_fu = timed(lambda: step(True))
+    t_co = timed(lambda: step(True, True))
     t_un2 = timed(lambda: step(False))
     t_fu2 = timed(lambda: step(True))
-    t_un, t_fu = min(t_un, t_un2), min(t_fu, t_fu2)
+    t_co2 = timed(lambda: step(True, True))
+    t_un, t_fu, t_co = min(t_un, t_un2), min(t_fu, t_fu2), min(t_co, t_co2)
     return {"metric": "gated-delta-rule token mixer between its projections, fwd+bwd, ms", "unit": "ms",
             "config": {"workload": "B=4 T=8192 H=16 D=128 bf16: split, layout, SiLU, L2 norm, gates, chunk op, layout, swish gate"},
             "steps": steps, "warmup": warmup, "op_alone_ms": t_op * 1e3,
-            "unfused_ms": t_un * 1e3, "fused_ms": t_fu * 1e3,
+            "unfused_ms": t_un * 1e3, "fused_ms": t_fu * 1e3, "mixer_core_ms": t_co * 1e3,
             "neighbours_unfused_ms": (t_un - t_op) * 1e3, "neighbours_fused_ms": (t_fu - t_op) * 1e3,
+            "neighbours_mixer_core_ms": (t_co - t_op) * 1e3,
             "neighbours_share_unfused": (t_un - t_op) / t_un, "neighbours_share_fused": (t_fu - t_op) / t_fu,
-            "tokens_per_s_fused": B * T / t_fu}
+            "neighbours_share_mixer_core": (t_co - t_op) / t_co,
+            "tokens_per_s_fused": B * T / t_fu, "tokens_per_s_mixer_core": B * T / t_co}
 
 
 def other_configs(dev, steps, warmup):

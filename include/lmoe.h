@@ -113,12 +113,19 @@ typedef struct lmoe_args {
    * fields below are ignored.
    * fwd writes den (the divisor den_t + norm_eps, fp32, laid out like g) and, when hs is given, zs (fp32 [NT,H,K]:
    * the sum of the keys before each chunk).  bwd reads them and o (the normalised output the forward wrote) beside
-   * d_o (the gradient of that output), and uses norm_ws, fp32 [NT,H,V/32,64+K], as workspace. */
+   * d_o (the gradient of that output), and uses norm_ws, fp32 [NT,H,V/32,64+K], as workspace.  (These three
+   * buffers are not part of what lmoe_workspace_bytes counts, which has no argument for the flag.) */
   int32_t normalize;
   float norm_eps;
   lmoe_tensor den;
   float* zs;
   float* norm_ws;
+  /* gated delta rule, 2-byte elements with tinv: v_act = 1 makes the kernels take silu(v) where they read v (the
+   * activation the reference applies in front of the op, gated_deltanet/gated_deltanet.py:101) and return in dv the
+   * gradient with respect to v as given (dv = silu'(v) times the gradient of silu(v)).  0 = v as given.  No
+   * counterpart in fla's signature: a caller that holds the fused projection saves the pass that would write silu(v)
+   * and the one that would apply silu' (see lmoe_gdn_qkv_prologue_*). */
+  int32_t v_act;
 } lmoe_args;
 
 /* Library version (major*10000 + minor*100 + patch). */
@@ -196,6 +203,9 @@ int lmoe_silu_l2norm_bwd(const void* x, const void* dy, void* dx, int64_t rows, 
  *   q = l2norm(silu(q_in)),  k = l2norm(silu(k_in)),  v = silu(v_in)      each [B][T][H][D] contiguous,
  * i.e. 'n b h d -> b n h d', SiLU and l2_norm_fn of gated_deltanet/gated_deltanet.py:99, :101, :105-106 (eps inside
  * the root, as lmoe_silu_l2norm_*).  bwd: dqkv [T][B][H][3 D] from dq, dk, dv [B][T][H][D] and qkv.
+ * v == NULL (fwd) / dv == NULL (bwd): v is left to the op, which is then called with lmoe_args.v_act = 1 on the v
+ * block of qkv itself (a strided view) and writes its gradient into the v block of dqkv; bwd then fills only the q
+ * and k blocks of dqkv.
  * D in {64, 128}; pointers 16-byte aligned; fp32 arithmetic. */
 int lmoe_gdn_qkv_prologue_fwd(const void* qkv, void* q, void* k, void* v, int32_t T, int32_t B, int32_t H, int32_t D,
                               int32_t dtype, float eps, void* stream);

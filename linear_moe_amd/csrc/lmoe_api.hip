@@ -149,6 +149,7 @@ int lmoe_chunk_gated_delta_rule_fwd(const lmoe_args* a, void* stream) {
   if (!a->beta.ptr) return fail(-12, "%s: beta must not be null", op);
   if (!a->o.ptr || !a->gcum) return fail(-11, "%s: o and gcum must not be null", op);
   if (a->V == 256 && a->dtype == LMOE_BF16 && !a->tinv) return fail(-11, "%s: V = 256 with 2-byte elements needs tinv", op);
+  if (a->v_act && (a->dtype != LMOE_BF16 || !a->tinv)) return fail(-15, "%s: v_act needs 2-byte elements and tinv", op);
   // P reaches memory where the WY preparation forms it (4-byte elements, or no tinv) or where the backward will
   // read it (hs given); a forward-only 2-byte call with tinv forms it inside the state pass and never stores it
   if ((a->dtype != LMOE_BF16 || !a->tinv || a->hs) && !a->pmat)
@@ -174,6 +175,7 @@ int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream) {
     return fail(-11, "%s: hs, dhs, vnew, tinv, pmat, gcum and dvnew must not be null", op);
   if (!a->d_o.ptr || !a->dq.ptr || !a->dk.ptr || !a->dv.ptr || !a->dg.ptr || !a->dbeta.ptr)
     return fail(-13, "%s: d_o, dq, dk, dv, dg and dbeta must not be null", op);
+  if (a->v_act && a->dtype != LMOE_BF16) return fail(-15, "%s: v_act needs 2-byte elements", op);
   if (a->NT == 0 || a->N == 0) return 0;
   lmoe::launch_gdn_state_bwd(*a, (hipStream_t)stream);
   lmoe::launch_gdn_bwd_chunk(*a, (hipStream_t)stream);
@@ -231,7 +233,7 @@ int lmoe_gdn_qkv_prologue_fwd(const void* qkv, void* q, void* k, void* v, int32_
                               int32_t dtype, float eps, void* stream) {
   const char* nm = "lmoe_gdn_qkv_prologue_fwd";
   if (int r = check_layerio(nm, T, B, dtype)) return r;
-  if (!qkv || !q || !k || !v) return fail(-1, "%s: null pointer", nm);
+  if (!qkv || !q || !k) return fail(-1, "%s: null pointer", nm);           // v == NULL: v is left to the op
   if (D != 64 && D != 128) return fail(-3, "%s: head dimension %d unsupported (64 or 128)", nm, D);
   if (H <= 0) return fail(-4, "%s: H must be positive", nm);
   if (((uintptr_t)qkv | (uintptr_t)q | (uintptr_t)k | (uintptr_t)v) & 15) return fail(-9, "%s: pointers must be 16-byte aligned", nm);
@@ -243,7 +245,7 @@ int lmoe_gdn_qkv_prologue_bwd(const void* qkv, const void* dq, const void* dk, c
                               int32_t B, int32_t H, int32_t D, int32_t dtype, float eps, void* stream) {
   const char* nm = "lmoe_gdn_qkv_prologue_bwd";
   if (int r = check_layerio(nm, T, B, dtype)) return r;
-  if (!qkv || !dq || !dk || !dv || !dqkv) return fail(-1, "%s: null pointer", nm);
+  if (!qkv || !dq || !dk || !dqkv) return fail(-1, "%s: null pointer", nm);  // dv == NULL: the op wrote that block
   if (D != 64 && D != 128) return fail(-3, "%s: head dimension %d unsupported (64 or 128)", nm, D);
   if (H <= 0) return fail(-4, "%s: H must be positive", nm);
   if (((uintptr_t)qkv | (uintptr_t)dq | (uintptr_t)dk | (uintptr_t)dv | (uintptr_t)dqkv) & 15)

@@ -121,6 +121,12 @@ template <> struct ET<float> {
   }
 };
 
+// SiLU and its derivative in the form every kernel that applies them shares (the results agree bit for bit between
+// the row kernels in front of the op and the op's own staging)
+__device__ __forceinline__ float sigmoid_fast(float z) { return 1.0f / (1.0f + __expf(-z)); }
+__device__ __forceinline__ float silu_of(float z) { return z * sigmoid_fast(z); }
+__device__ __forceinline__ float silu_grad(float z) { const float a = sigmoid_fast(z); return a * (1.0f + z * (1.0f - a)); }
+
 // e^x for the pairwise decay factors: library expf on the fp32 path (keeps 1e-5 parity),
 // the hardware exp2 path for bf16 operands
 template <typename T> __device__ __forceinline__ float texp(float x) {
@@ -640,6 +646,8 @@ __device__ __forceinline__ float wave_rev_scan(float x) {
   return total - (incl - x);
 }
 // sum over the 64 lanes, in every lane: the row totals, then the four of them through scalar registers
+// (to be called with all 64 lanes active, like group_sum: a lane that is switched off contributes whatever its
+// register held, and reading lane 0, 16, 32 or 48 while it is off returns that stale value)
 __device__ __forceinline__ float wave_sum(float x) {
   x = group_sum<16>(x);
   const int xi = __builtin_bit_cast(int, x);

@@ -196,8 +196,16 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
 #pragma unroll
           for (int i = 0; i < IOV::VEC; ++i) {
             const float zf = ET<T>::to_f(z[i]);
-            o[i] = ET<T>::from_f(zf * bt);
-            s += zf * ET<T>::to_f(vv[i]);
+            if (a.v_act) {
+              // v as given is the argument of a SiLU: the op runs on silu(v) (rounded to the element type, as the
+              // forward pass staged it) and dv is the gradient with respect to the argument
+              const float vr = ET<T>::to_f(vv[i]);
+              o[i] = ET<T>::from_f(zf * bt * silu_grad(vr));
+              s += zf * ET<T>::to_f(ET<T>::from_f(silu_of(vr)));
+            } else {
+              o[i] = ET<T>::from_f(zf * bt);
+              s += zf * ET<T>::to_f(vv[i]);
+            }
           }
           d.r.v[p] = o;
           s = group_sum<IOV::VPR>(s);                   // the VPR lanes that hold one row are neighbours

@@ -265,6 +265,12 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_state_fwd_reg(const lmoe_args 
     auto stage_b = [&](PreB& P, int buf) {
       IOK::store_lds(P.rq, s_q, LDK);       // rows past the end only reach output rows that are not stored
       IOP::store_lds(P.rt, s_ti, LDC);
+      if (a.v_act) {                         // v = silu(v as given): the activation in front of the op, applied here
+#pragma unroll
+        for (int p = 0; p < IOV::PASSES; ++p)
+#pragma unroll
+          for (int i = 0; i < IOV::VEC; ++i) P.rv.v[p][i] = ET<T>::from_f(silu_of(ET<T>::to_f(P.rv.v[p][i])));
+      }
       IOV::mask(P.rv, P.len);
       IOV::store_lds(P.rv, s_v, LDU);
       if (wave_id() == 8) {

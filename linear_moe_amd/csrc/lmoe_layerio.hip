@@ -17,7 +17,7 @@
 namespace lmoe {
 
 namespace {
-__device__ __forceinline__ float sigm(float z) { return 1.0f / (1.0f + __expf(-z)); }
+__device__ __forceinline__ float sigm(float z) { return sigmoid_fast(z); }
 // sum over the LPR neighbouring lanes that hold one row
 template <int LPR> __device__ __forceinline__ float row_sum(float x) {
   if constexpr (LPR <= 16) {
@@ -30,7 +30,9 @@ template <int LPR> __device__ __forceinline__ float row_sum(float x) {
 }
 
 // rows are (t, b, h) in the projection and (b, t, h) in the op's tensors
-template <typename T, int D, bool BWD>
+// WITH_V = false: v is left to the op (which then applies SiLU to the column block of the projection itself and writes
+// its gradient into that block of d(projection)): q^ and k^ only; the backward leaves the v block of d(projection) alone
+template <typename T, int D, bool BWD, bool WITH_V>
 __global__ __launch_bounds__(NTHR) void k_gdn_qkv_prologue(const T* __restrict__ qkv, const T* __restrict__ dq,
                                                            const T* __restrict__ dk, const T* __restrict__ dv,
                                                            T* __restrict__ o0, T* __restrict__ o1, T* __restrict__ o2,
@@ -45,21 +47,28 @@ __global__ __launch_bounds__(NTHR) void k_gdn_qkv_prologue(const T* __restrict__
     const int64_t bt = r / H;
     const int t = (int)(bt % Tn), b = (int)(bt / Tn);
     const T* src = qkv + (((int64_t)t * Bn + b) * H + h) * (3 * D) + lr * VEC;
-    const vec xq = *(const vec*)src, xk = *(const vec*)(src + D), xv = *(const vec*)(src + 2 * D);
+    const vec xq = *(const vec*)src, xk = *(const vec*)(src + D);
     float sq[VEC], sk[VEC], gq[VEC], gk[VEC], ssq = 0.f, ssk = 0.f;
     vec ov;
-    vec dvv;
-    if constexpr (BWD) dvv = *(const vec*)(dv + r * D + lr * VEC);
+    if constexpr (WITH_V) {
+      const vec xv = *(const vec*)(src + 2 * D);
+      vec dvv;
+      if constexpr (BWD) dvv = *(const vec*)(dv + r * D + lr * VEC);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        const float zv = ET<T>::to_f(xv[i]), av = sigm(zv);
+        if constexpr (BWD) ov[i] = ET<T>::from_f(ET<T>::to_f(dvv[i]) * av * (1.0f + zv * (1.0f - av)));
+        else ov[i] = ET<T>::from_f(zv * av);
+      }
+    }
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
-      const float zq = ET<T>::to_f(xq[i]), zk = ET<T>::to_f(xk[i]), zv = ET<T>::to_f(xv[i]);
-      const float aq = sigm(zq), ak = sigm(zk), av = sigm(zv);
+      const float zq = ET<T>::to_f(xq[i]), zk = ET<T>::to_f(xk[i]);
+      const float aq = sigm(zq), ak = sigm(zk);
       sq[i] = zq * aq; sk[i] = zk * ak;
       gq[i] = aq * (1.0f + zq * (1.0f - aq));       // silu'(z)
       gk[i] = ak * (1.0f + zk * (1.0f - ak));
       ssq += sq[i] * sq[i]; ssk += sk[i] * sk[i];
-      if constexpr (BWD) ov[i] = ET<T>::from_f(ET<T>::to_f(dvv[i]) * av * (1.0f + zv * (1.0f - av)));
-      else ov[i] = ET<T>::from_f(zv * av);
     }
     ssq = row_sum<LPR>(ssq); ssk = row_sum<LPR>(ssk);
     const float rq = 1.0f / sqrtf(ssq + eps), rk = 1.0f / sqrtf(ssk + eps);
@@ -79,13 +88,14 @@ __global__ __launch_bounds__(NTHR) void k_gdn_qkv_prologue(const T* __restrict__
         ok[i] = ET<T>::from_f((fk[i] * rk - ck * sk[i]) * gk[i]);
       }
       T* dst = o0 + (((int64_t)t * Bn + b) * H + h) * (3 * D) + lr * VEC;       // d(projection)
-      *(vec*)dst = oq; *(vec*)(dst + D) = ok; *(vec*)(dst + 2 * D) = ov;
+      *(vec*)dst = oq; *(vec*)(dst + D) = ok;
+      if constexpr (WITH_V) *(vec*)(dst + 2 * D) = ov;
     } else {
 #pragma unroll
       for (int i = 0; i < VEC; ++i) { oq[i] = ET<T>::from_f(sq[i] * rq); ok[i] = ET<T>::from_f(sk[i] * rk); }
       *(vec*)(o0 + r * D + lr * VEC) = oq;
       *(vec*)(o1 + r * D + lr * VEC) = ok;
-      *(vec*)(o2 + r * D + lr * VEC) = ov;
+      if constexpr (WITH_V) *(vec*)(o2 + r * D + lr * VEC) = ov;
     }
   }
 }
@@ -131,8 +141,14 @@ void prologue_t(const void* qkv, const void* dq, const void* dk, const void* dv,
   constexpr int RPB = NTHR / (D / ET<T>::VEC);
   const int64_t rows = (int64_t)Tn * Bn * H, blocks = (rows + RPB - 1) / RPB, cap = (int64_t)cu_count() * 8;
   const int grid = (int)(blocks < cap ? blocks : cap);
-  if (bwd) hipLaunchKernelGGL((k_gdn_qkv_prologue<T, D, true>), dim3(grid), dim3(NTHR), 0, st, (const T*)qkv, (const T*)dq, (const T*)dk, (const T*)dv, (T*)o0, (T*)nullptr, (T*)nullptr, Tn, Bn, H, eps);
-  else hipLaunchKernelGGL((k_gdn_qkv_prologue<T, D, false>), dim3(grid), dim3(NTHR), 0, st, (const T*)qkv, (const T*)nullptr, (const T*)nullptr, (const T*)nullptr, (T*)o0, (T*)o1, (T*)o2, Tn, Bn, H, eps);
+  // v handed in (forward: o2, backward: dv) or left to the op
+  const bool with_v = bwd ? dv != nullptr : o2 != nullptr;
+#define LMOE_P(BWD, WV)                                                                                                  \
+  hipLaunchKernelGGL((k_gdn_qkv_prologue<T, D, BWD, WV>), dim3(grid), dim3(NTHR), 0, st, (const T*)qkv, (const T*)dq,    \
+                     (const T*)dk, (const T*)dv, (T*)o0, (T*)o1, (T*)o2, Tn, Bn, H, eps)
+  if (bwd) { if (with_v) LMOE_P(true, true); else LMOE_P(true, false); }
+  else { if (with_v) LMOE_P(false, true); else LMOE_P(false, false); }
+#undef LMOE_P
 }
 }  // namespace
 

@@ -36,9 +36,12 @@ class GDNCall:
         # blocks stay valid for lmoe_launch_stage; the autograd path must not (reference cycle)
         self.keep = keep
 
-    def forward(self, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, head_first, save=True):
+    def forward(self, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, head_first, save=True,
+                v_act=False):
         """save=False: a forward-only call (nothing requires a gradient): what only the backward reads (the
-        per-chunk states, v_new, Tinv) is neither allocated nor written."""
+        per-chunk states, v_new, Tinv) is neither allocated nor written.
+        v_act: v is the argument of the SiLU in front of the op (bfloat16 only): the kernels apply it where they
+        read v, and ``backward`` returns the gradient with respect to that argument."""
         ctx = self
         lib = _lib.load()
         dims = _check_inputs(q, k, v, head_first, cu_seqlens, wide_v=True)
@@ -62,7 +65,8 @@ class GDNCall:
         a.beta, a.beta_dtype = _desc(beta, head_first), _scalar_dt(beta)
         a.h0 = ptr(h0)
         dev, dt = q.device, q.dtype
-        o = torch.empty_like(v)
+        # (v_act: v is a block of a wider tensor; o is a tensor of its own)
+        o = torch.empty(v.shape, dtype=dt, device=dev) if v_act else torch.empty_like(v)
         ht = torch.empty(plan.N, H, K, V, dtype=torch.float32, device=dev) if output_final_state else None
         hs = torch.empty(max(plan.NT, 1), H, K, V, dtype=dt, device=dev) if save else None
         # always: the backward reads it, and the forward state pass forms w from it (8 KB per chunk and head)
@@ -79,6 +83,10 @@ class GDNCall:
         a.pmat, a.gcum = ptr(pmat), gcum.data_ptr()
         a.w, a.u = _desc(w, False), _desc(u, False)
         a.vnew.ptr = ptr(vnew)
+        if v_act and dt != torch.bfloat16:
+            raise ValueError("v_act exists for bfloat16")
+        a.v_act = int(bool(v_act))
+        ctx.v_act = bool(v_act)
         _lib.check(lib.lmoe_chunk_gated_delta_rule_fwd(C.byref(a), stream_ptr()), "chunk_gated_delta_rule forward")
         ctx.saved = (q, k, v, g, beta, h0, hs, tinv, pmat, gcum, vnew)
         ctx.fwd_args, ctx.fwd_keep = a, ((o, ht, w, u) if self.keep else None)
@@ -86,7 +94,9 @@ class GDNCall:
         ctx.has_h0 = initial_state is not None
         return o, ht
 
-    def backward(self, do, dht):
+    def backward(self, do, dht, dv_out=None):
+        """dv_out: where dv goes (a tensor of v's shape, any strides the kernels take: e.g. the v block of the gradient
+        of a fused projection); default: a new tensor like v."""
         ctx = self
         lib = _lib.load()
         q, k, v, g, beta, h0, hs, tinv, pmat, gcum, vnew = ctx.saved
@@ -105,8 +115,12 @@ class GDNCall:
         dht = None if dht is None else dht.float().contiguous()
         a.dht = ptr(dht)
         dev, dt = q.device, q.dtype
-        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        dq, dk = torch.empty_like(q), torch.empty_like(k)
+        dv = torch.empty_like(v) if dv_out is None else dv_out
+        if dv.shape != v.shape or dv.dtype != dt or _aligned(dv) is not dv:
+            raise ValueError("dv_out must have the shape and dtype of v, 16-byte aligned rows, a contiguous last dimension")
         a.dq, a.dk, a.dv = _desc(dq, head_first), _desc(dk, head_first), _desc(dv, head_first)
+        a.v_act = int(ctx.v_act)
         dg = torch.empty(beta.shape, dtype=torch.float32, device=dev)
         dbeta = torch.empty(beta.shape, dtype=torch.float32, device=dev)
         a.dg, a.dbeta = _desc(dg, head_first), _desc(dbeta, head_first)

@@ -56,6 +56,58 @@ class _QKVPrologue(torch.autograd.Function):
         return dx.view(ctx.shape), None, None, None
 
 
+class _GDNMixerCore(torch.autograd.Function):
+    """Prologue and op as one node of the graph, so that the gradient of the projection is one buffer that the op's
+    backward (v block) and the prologue's backward (q and k blocks) fill in place."""
+
+    @staticmethod
+    def forward(ctx, qkv, g, beta, H, D, eps, scale):
+        from .gated_delta_rule import GDNCall
+        dt = _dt(qkv)
+        if dt != _lib.LMOE_BF16:
+            raise ValueError("gdn_mixer_core: bfloat16 only (the op applies SiLU to v in its 2-byte kernels)")
+        T, B = qkv.shape[0], qkv.shape[1]
+        if qkv.dim() not in (3, 4) or qkv.numel() != T * B * H * 3 * D:
+            raise ValueError(f"gdn_mixer_core: {tuple(qkv.shape)} is not [T, B, {H} heads x 3 x {D}]")
+        if D not in (64, 128):
+            raise ValueError(f"gdn_mixer_core: head dimension {D} unsupported (64 or 128)")
+        lib = _lib.load()
+        x = qkv.contiguous()
+        q, k = (torch.empty(B, T, H, D, dtype=qkv.dtype, device=qkv.device) for _ in range(2))
+        _lib.check(lib.lmoe_gdn_qkv_prologue_fwd(x.data_ptr(), q.data_ptr(), k.data_ptr(), None, T, B, H, D, dt, eps,
+                                                 stream_ptr()), "gdn_mixer_core prologue")
+        v = x.view(T, B, H, 3 * D)[..., 2 * D:].transpose(0, 1)            # [B, T, H, D], strided: the op reads it in place
+        call = GDNCall()
+        o, _ = call.forward(q, k, v, g, beta, scale, None, False, None, False,
+                            save=any(ctx.needs_input_grad[:3]), v_act=True)
+        ctx.call = call
+        ctx.save_for_backward(x)
+        ctx.dims, ctx.eps, ctx.dt, ctx.shape = (T, B, H, D), eps, dt, qkv.shape
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        T, B, H, D = ctx.dims
+        lib = _lib.load()
+        (x,) = ctx.saved_tensors
+        dx = torch.empty_like(x)
+        dv = dx.view(T, B, H, 3 * D)[..., 2 * D:].transpose(0, 1)          # the op writes the v block itself
+        dq, dk, _, dg, dbeta, _ = ctx.call.backward(do, None, dv_out=dv)
+        _lib.check(lib.lmoe_gdn_qkv_prologue_bwd(x.data_ptr(), dq.data_ptr(), dk.data_ptr(), None, dx.data_ptr(),
+                                                 T, B, H, D, ctx.dt, ctx.eps, stream_ptr()), "gdn_mixer_core backward")
+        return dx.view(ctx.shape), dg, dbeta, None, None, None, None
+
+
+def gdn_mixer_core(qkv: torch.Tensor, g: torch.Tensor, beta: torch.Tensor, num_heads: int, head_dim: int,
+                   eps: float = 1e-6, scale=None) -> torch.Tensor:
+    """``gdn_qkv_prologue`` and ``chunk_gated_delta_rule(..., head_first=False)`` in one call (bfloat16): q^ and k^ are
+    written as by the prologue, v is never written -- the op reads the v block of ``qkv`` in place and applies SiLU
+    where it stages it, and in the backward writes ``silu'(v)`` times its dv straight into the v block of the
+    projection's gradient, whose q and k blocks the prologue's backward fills.  ``g``, ``beta``: ``[B, T, H]``.
+    Returns o ``[B, T, H, D]``, the bits of the two-call path."""
+    return _GDNMixerCore.apply(qkv, g, beta, num_heads, head_dim, eps, scale)
+
+
 def gdn_qkv_prologue(qkv: torch.Tensor, num_heads: int, head_dim: int, eps: float = 1e-6):
     """``qkv`` ``[T, B, H * 3 D]`` (per head q | k | v) -> ``l2norm(silu(q))``, ``l2norm(silu(k))``, ``silu(v)``,
     each ``[B, T, H, D]`` contiguous: the inputs of ``chunk_gated_delta_rule(..., head_first=False)``."""

@@ -31,15 +31,19 @@ class GatedDeltaNetLayer(nn.Module):
         qkv = F.linear(x, self.qkv_proj.to(x.dtype)).view(T, B, self.H, 3 * self.D)
         return torch.split(qkv, [self.D, self.D, self.D], dim=3)          # each [T, B, H, D] (a strided view)
 
-    def forward(self, x, fused: bool = True):
+    def forward(self, x, fused: bool = True, core: bool = False):
         """fused: the one-pass prologue / epilogue kernels; otherwise the chain of copies, row kernels and eager
-        elementwise ops they replace (same numbers to the rounding of the element type)."""
+        elementwise ops they replace (same numbers to the rounding of the element type).  core (with fused, bfloat16):
+        prologue and op as one call that never writes silu(v) (``gdn_mixer_core``)."""
         import linear_moe_amd as L
         T, B, _ = x.shape
         o_gate = F.linear(x, self.o_gate_proj.to(x.dtype))
         xt = x.transpose(0, 1)                                             # [B, T, hidden]
         gk, beta = L.gdn_gates(F.linear(xt, self.a_proj.to(x.dtype)), F.linear(xt, self.beta_proj.to(x.dtype)),
                                self.A_log, self.dt_bias)                   # [B, T, H]: fp32 log-decay, beta
+        if fused and core:
+            o = L.gdn_mixer_core(F.linear(x, self.qkv_proj.to(x.dtype)), gk, beta, self.H, self.D)
+            return F.linear(L.swish_gate_relayout(o, o_gate), self.o_proj.to(x.dtype))
         if fused:
             q, k, v = L.gdn_qkv_prologue(F.linear(x, self.qkv_proj.to(x.dtype)), self.H, self.D)
         else:

@@ -3,9 +3,11 @@
 (hidden states and all parameters) against the same chain of fp64 oracle functions."""
 import pytest
 import torch
+import torch.nn.functional as F
 
+from oracle import naive
 from tests.layers import GatedDeltaNetLayer, GLALayer
-from tests.util import gen, max_abs_rel
+from tests.util import TOL, gen, max_abs_rel
 
 pytestmark = pytest.mark.gpu
 
@@ -63,6 +65,63 @@ def test_gdn_layer_fused_prologue_epilogue_equals_the_unfused_chain(cuda, dtype)
     tol = 2e-5 if dtype == torch.float32 else 3e-2
     assert max_abs_rel(outs[0][0].cpu(), outs[1][0].cpu()) < tol
     assert max_abs_rel(outs[0][1].cpu(), outs[1][1].cpu()) < tol
+
+
+@pytest.mark.parametrize("D", [128, 64])
+def test_gdn_mixer_core_equals_prologue_then_op(cuda, D):
+    """gdn_mixer_core (q^, k^ written, silu(v) applied where the op stages v, dv written straight into the v block of
+    the projection's gradient) against gdn_qkv_prologue followed by chunk_gated_delta_rule: the same output bit for
+    bit (the same q^, k^ and the same rounded silu(v) reach the same kernels), the same dg, dbeta and q / k blocks of
+    the projection's gradient bit for bit, its v block to the rounding of the element type (one rounding of
+    beta dZ silu'(v) instead of two)."""
+    import linear_moe_amd as L
+    T, B, H = 200, 2, 3
+    bf = torch.bfloat16
+    qkv = gen(5250, T, B, H * 3 * D).to(bf).to(cuda)
+    g = (-torch.rand(B, T, H, generator=torch.Generator().manual_seed(5251)) * 0.2).to(cuda)
+    beta = torch.rand(B, T, H, generator=torch.Generator().manual_seed(5252)).to(bf).to(cuda)
+    do = gen(5253, B, T, H, D).to(bf).to(cuda)
+    res = []
+    for core in (True, False):
+        leaves = [t.clone().requires_grad_(True) for t in (qkv, g, beta)]
+        if core:
+            o = L.gdn_mixer_core(*leaves, H, D)
+        else:
+            q, k, v = L.gdn_qkv_prologue(leaves[0], H, D)
+            o, _ = L.chunk_gated_delta_rule(q, k, v, leaves[1], leaves[2], head_first=False)
+        res.append((o.detach(), torch.autograd.grad((o * do).sum(), leaves)))
+    torch.cuda.synchronize()
+    (o1, g1), (o2, g2) = res
+    assert o1.is_contiguous() and torch.equal(o1, o2)
+    assert torch.equal(g1[1], g2[1]) and torch.equal(g1[2], g2[2])
+    d1, d2 = (x.view(T, B, H, 3 * D) for x in (g1[0], g2[0]))
+    assert torch.equal(d1[..., :2 * D], d2[..., :2 * D])
+    assert max_abs_rel(d1[..., 2 * D:].float().cpu(), d2[..., 2 * D:].float().cpu()) < 1e-2
+    # and against the oracle chain in fp64: silu'(v) times the gradient of the op with respect to silu(v)
+    x64 = qkv.double().cpu().view(T, B, H, 3 * D).requires_grad_(True)
+    q, k, v = (t.transpose(0, 1) for t in torch.split(x64, [D, D, D], dim=3))
+    oo, _ = naive.naive_recurrent_gated_delta_rule(naive.naive_silu_l2_norm(q), naive.naive_silu_l2_norm(k), F.silu(v),
+                                                   g.double().cpu(), beta.double().cpu(), None, None, False, None, False)
+    (gx,) = torch.autograd.grad((oo * do.double().cpu()).sum(), [x64])
+    assert max_abs_rel(o1.cpu(), oo.detach()) < TOL[bf]
+    assert max_abs_rel(d1.cpu(), gx) < 4e-2
+
+
+def test_gdn_layer_with_the_mixer_core(cuda):
+    """The composed layer through gdn_mixer_core against the layer through prologue + op (bfloat16)."""
+    hidden, H, D, T, B = 256, 2, 128, 130, 2
+    layer = GatedDeltaNetLayer(hidden, H, D, seed=6).to(cuda)
+    x = gen(5200, T, B, hidden).to(torch.bfloat16).to(cuda)
+    dy = gen(5201, T, B, hidden).to(torch.bfloat16).to(cuda)
+    outs = []
+    for core in (True, False):
+        xd = x.clone().requires_grad_(True)
+        y = layer(xd, fused=True, core=core)
+        outs.append((y.detach(), torch.autograd.grad((y * dy).sum(), [xd] + list(layer.parameters()))))
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0][0], outs[1][0])
+    for a, b in zip(outs[0][1], outs[1][1]):
+        assert max_abs_rel(a.float().cpu(), b.float().cpu()) < 1e-2
 
 
 CORES = {
