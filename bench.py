@@ -38,16 +38,18 @@ STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_gdn_state_fwd_reg", 4: "k_gdn_state_bwd"
 # sources (kernel_sources_sha16()) at that time, and a build whose sources differ reports traffic = null
 # rather than a stale number.
 CALIB_COPY_BYTES = 256 << 20
-MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237243453, "k_gdn_state_fwd_reg": 1119409063, "k_gdn_state_bwd": 945960392, "k_gdn_bwd_chunk": 1834053754}
-TRAFFIC_SOURCES_SHA16 = "990483523988793a"
+MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237242262, "k_gdn_state_fwd_reg": 1119492165, "k_gdn_state_bwd": 945960857,
+                    "k_gdn_bwd_chunk": 1826536716}
+TRAFFIC_SOURCES_SHA16 = "ccaf947085530fdb"
 TRAFFIC_SOURCES = ("lmoe_common.hpp", "lmoe_seq.hpp", "lmoe_gdn_wy.hpp", "lmoe_gdn_state.hpp", "lmoe_gdn_state_reg.hpp", "lmoe_gdn_bwd_chunk.hpp",
                    "lmoe_gdn_fwd.hip", "lmoe_gdn_state.hip", "lmoe_gdn_bwd.hip")
 
 
 # HBM bytes per call of the other contract configurations (bench.py --other-configs), same counters and scaling,
 # summed over the kernels of the call; key = configuration number
-OTHER_TRAFFIC = {"1": 2230718, "2": 272913415, "3": 1281283146, "5": 16675972468, "6": 1444848249}
-OTHER_TRAFFIC_SHA16 = "e93cf3e3fb42e6d6"
+OTHER_TRAFFIC = {"1": 2230780, "2": 272919654, "3": 1281245622, "5": 16656576830, "6": 1444809804, "7": 6577677394,
+                 "8": 1510754015}
+OTHER_TRAFFIC_SHA16 = "b720200d83053913"
 
 
 def all_sources_sha16():
@@ -459,7 +461,7 @@ def layer_bench(dev, steps, warmup):
             "tokens_per_s_fused": B * T / t_fu, "tokens_per_s_mixer_core": B * T / t_co}
 
 
-def other_configs(dev, steps, warmup):
+def other_configs(dev, steps, warmup, comparisons=True):
     """The four contract configurations beside the headline one, and the forward + backward of chunk_simple_gla on
     the shape of configuration 2, through the Python entry points (inputs of the contract's laws, drawn on the GPU:
     this leg times, the parity tests check): ms per call, tokens/s and the algorithmic bytes (every input read once,
@@ -564,7 +566,8 @@ def other_configs(dev, steps, warmup):
         o = torch.cat([L.chunk_gated_delta_rule(q, k, v[..., c:c + 128], g, beta, K ** -0.5)[0] for c in (0, 128)], -1)
         torch.autograd.grad([o], [q, k, v, g, beta], [do])
     sec = timed(f7)
-    extras = {"7": {"as_two_calls_on_128_columns_ms": round(timed(f7_halves) * 1e3, 4)}}
+    # (comparisons=False: a profile of the command then holds one problem per kernel instance)
+    extras = {"7": {"as_two_calls_on_128_columns_ms": round(timed(f7_halves) * 1e3, 4)}} if comparisons else {}
     res["7 gated_delta_rule fwd+bwd bf16 B=4 T=8192 H=16 K=128 V=256"] = (
         sec, B * T, B * T * H * ((6 * K + 5 * V) * 2 + 3 * 2 + 12),
         3 * B * T * H * (6 * CH * K + 4 * CH * V + 6 * K * V + (2 / 3) * CH * CH), PEAK_MFMA_BF16)
@@ -579,7 +582,8 @@ def other_configs(dev, steps, warmup):
         o, _ = L.chunk_linear_attn(q, k, v, normalize=normalize)
         torch.autograd.grad([o], [q, k, v], [do])
     sec = timed(lambda: f8(True))
-    extras["8"] = {"without_normaliser_ms": round(timed(lambda: f8(False)) * 1e3, 4)}
+    if comparisons:
+        extras["8"] = {"without_normaliser_ms": round(timed(lambda: f8(False)) * 1e3, 4)}
     res["8 linear_attn normalize=True fwd+bwd bf16 B=4 H=16 T=4096 K=V=128"] = (
         sec, B * T, B * T * H * ((6 * K + 5 * K) * 2), 3 * B * T * H * sg_flops(K, K), PEAK_MFMA_BF16)
     # one roofline record per configuration, for the whole call on its minimal traffic (every input read once, every
@@ -625,7 +629,12 @@ def main():
                     help="instead of the headline step: the token-mixer path of the gated-delta-rule layer between its "
                          "projections (no GEMMs), with and without the one-pass prologue / epilogue kernels, one JSON line")
     ap.add_argument("--other-configs", action="store_true",
-                    help="instead of the headline step: contract configurations 1, 2, 3 and 5, one JSON line")
+                    help="instead of the headline step: contract configurations 1, 2, 3 and 5, the training step on the "
+                         "shape of 2, V = 256 and the normalised linear attention, one JSON line")
+    ap.add_argument("--skip-comparisons", action="store_true",
+                    help="with --other-configs: leave out the legs that run the same problems through the slower paths "
+                         "(V = 256 as two calls, linear attention without its normaliser), so that a profile of the "
+                         "command holds one problem per kernel instance")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the op shards over batch and heads without "
@@ -652,7 +661,7 @@ def main():
         print(json.dumps(neighbours(lib, B * T * H, K, dev, args.stage_reps)))
         return
     if args.other_configs:
-        print(json.dumps(other_configs(dev, args.steps, args.warmup)))
+        print(json.dumps(other_configs(dev, args.steps, args.warmup, not args.skip_comparisons)))
         return
     if args.layer:
         print(json.dumps(layer_bench(dev, args.steps, args.warmup)))
