@@ -99,6 +99,58 @@ def test_gated_delta_rule_needs_w_and_u_only_where_the_state_pass_reads_them():
                     assert b"w and u must not be null" in lib.lmoe_last_error()
 
 
+def test_options_outside_flas_signature_are_validated_before_any_launch():
+    """V = 256 belongs to the gated delta rule alone (2-byte calls then need tinv); normalize belongs to ungated 2-byte
+    calls of chunk_simple_gla and names the buffers it needs; v_act needs 2-byte elements and tinv.  Calls without
+    chunks validate and return before any launch (no GPU needed)."""
+    from linear_moe_amd import _lib
+    lib = _lib.load()
+    fake = 0x1000                                  # never dereferenced: NT == 0
+
+    def args(dtype, K=128, V=128):
+        a = _lib.Args()
+        a.dtype, a.B, a.T, a.H, a.K, a.V, a.N, a.NT = dtype, 1, 0, 1, K, V, 1, 0
+        a.scale, a.gate, a.g_dtype, a.beta_dtype = 1.0, _lib.GATE_SCALAR, _lib.LMOE_F32, dtype
+        for n in ("q", "k", "v", "g", "beta", "o", "w", "u"):
+            setattr(a, n, _lib.Tensor4(fake, 0, 64, 64))
+        a.pmat = a.gcum = a.tinv = fake
+        return a
+
+    a = args(_lib.LMOE_BF16, V=256)
+    assert lib.lmoe_chunk_gated_delta_rule_fwd(C.byref(a), None) == 0
+    assert lib.lmoe_chunk_simple_gla_fwd(C.byref(a), None) == -3 and b"V=256" in lib.lmoe_last_error()
+    a.tinv = None
+    assert lib.lmoe_chunk_gated_delta_rule_fwd(C.byref(a), None) == -11 and b"needs tinv" in lib.lmoe_last_error()
+    assert lib.lmoe_chunk_gated_delta_rule_fwd(C.byref(args(_lib.LMOE_F32, V=256)), None) == 0
+    assert lib.lmoe_chunk_gated_delta_rule_fwd(C.byref(args(_lib.LMOE_BF16, K=64, V=256)), None) == -3
+    # v_act
+    a = args(_lib.LMOE_BF16)
+    a.v_act = 1
+    assert lib.lmoe_chunk_gated_delta_rule_fwd(C.byref(a), None) == 0
+    a.dtype = a.beta_dtype = _lib.LMOE_F32
+    assert lib.lmoe_chunk_gated_delta_rule_fwd(C.byref(a), None) == -15 and b"v_act" in lib.lmoe_last_error()
+    # normalize
+    a = args(_lib.LMOE_BF16)
+    a.gate, a.normalize, a.norm_eps = _lib.GATE_NONE, 1, 1e-10
+    assert lib.lmoe_chunk_simple_gla_fwd(C.byref(a), None) == -11 and b"den" in lib.lmoe_last_error()
+    a.den = _lib.Tensor4(fake, 0, 1, 1)
+    assert lib.lmoe_chunk_simple_gla_fwd(C.byref(a), None) == 0          # forward only: hs NULL, zs not needed
+    a.hs = fake
+    assert lib.lmoe_chunk_simple_gla_fwd(C.byref(a), None) == -11 and b"zs" in lib.lmoe_last_error()
+    a.zs = fake
+    assert lib.lmoe_chunk_simple_gla_fwd(C.byref(a), None) == 0
+    a.gate = _lib.GATE_SCALAR
+    assert lib.lmoe_chunk_simple_gla_fwd(C.byref(a), None) == -15 and b"LMOE_GATE_NONE" in lib.lmoe_last_error()
+    a.gate, a.dtype = _lib.GATE_NONE, _lib.LMOE_F32
+    assert lib.lmoe_chunk_simple_gla_fwd(C.byref(a), None) == -15 and b"2-byte" in lib.lmoe_last_error()
+    a.dtype = _lib.LMOE_BF16
+    a.dhs = fake
+    a.d_o = a.dq = a.dk = a.dv = _lib.Tensor4(fake, 0, 64, 64)
+    assert lib.lmoe_chunk_simple_gla_bwd(C.byref(a), None) == -11 and b"norm_ws" in lib.lmoe_last_error()
+    a.norm_ws = fake
+    assert lib.lmoe_chunk_simple_gla_bwd(C.byref(a), None) == 0
+
+
 def test_chunk_gla_forward_needs_hs_only_where_an_output_kernel_reads_it():
     """2-byte elements: the forward state pass forms the output itself and hs, which only the backward reads, may be
     NULL (a forward-only call).  4-byte elements hand the states to their output kernel through hs: required.  A
