@@ -718,6 +718,31 @@ def main():
     dt = timed(step_public)
     warmup_effective = 2 * args.warmup + args.steps + settle_extra
     dt_direct = timed(step_direct)
+    # beside the headline: per-step statistics (an event pair per step), forward and backward on their own, and the
+    # step with the caches flushed in front of it (512 MiB written between steps: twice the memory-side cache), all
+    # through the call object, after everything above has run
+    def per_step(fn, flush=None):
+        ms = []
+        for _ in range(args.steps):
+            if flush is not None:
+                flush.add_(1)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            e1.synchronize()
+            ms.append(e0.elapsed_time(e1))
+        ms.sort()
+        return {"median": ms[len(ms) // 2], "min": ms[0], "max": ms[-1]}
+
+    def fwd_only():
+        call.forward(xd["q"], xd["k"], xd["v"], xd["g"], xd["beta"], None, None, False, None, False)
+
+    def bwd_only():
+        call.backward(xd["do"], None)
+    fwd_only()
+    stats = {"step": per_step(step_direct), "fwd": per_step(fwd_only), "bwd": per_step(bwd_only),
+             "step_caches_flushed": per_step(step_direct, torch.zeros(512 << 20, dtype=torch.uint8, device=dev))}
     stages = time_stages(call, lib, args.stage_reps)
 
     tokens = B * T
@@ -768,6 +793,7 @@ def main():
         "tflops": flops / dt / 1e12,
         "kernels_us": {STAGE_NAMES[s]: round(t * 1e6, 1) for s, t in stages.items()},
         "kernels_sum_ms": sum(stages.values()) * 1e3,
+        "ms_per_step_stats": {k: {n: round(v, 4) for n, v in d.items()} for k, d in stats.items()},
         "roofline": roof,
     }
     if not args.no_cpu:
