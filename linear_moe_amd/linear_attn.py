@@ -42,13 +42,19 @@ def chunk_linear_attn(
     # normalises with q * scale, so the scale cancels in o up to the epsilon): it is formed inside the kernels, in
     # the fp32 state, instead of by a cumulative sum over k in HBM.
     V = v.shape[-1]
-    if normalize and len(qb) == 1 and can_normalize(qb[0], v):
-        # one key block of bfloat16: the kernels carry the column themselves and divide before they store
-        o, ht = chunk_simple_gla_normalized(qb[0], kb[0], v, scale, initial_state, output_final_state, None,
-                                            head_first, _eps)
-        if ht is not None and ht.shape[-2] != (q.features if hasattr(q, "features") else q.shape[-1]):
-            ht = ht[..., :(q.features if hasattr(q, "features") else q.shape[-1]), :]
-        return o, ht
+    if normalize and len(qb) == 1 and V <= 128 and v.dim() == 4 and v.dtype == torch.bfloat16:
+        # one key block of bfloat16: the kernels carry the column themselves and divide before they store (a value
+        # head that is not 64 or 128 wide is zero-padded to the next of the two: zero columns stay zero)
+        Vp = 64 if V <= 64 else 128
+        pad = torch.nn.functional.pad
+        vp = v if Vp == V else pad(v, (0, Vp - V))
+        h0 = initial_state if (initial_state is None or Vp == V) else pad(initial_state, (0, Vp - V))
+        if can_normalize(qb[0], vp):
+            o, ht = chunk_simple_gla_normalized(qb[0], kb[0], vp, scale, h0, output_final_state, None, head_first, _eps)
+            feats = q.features if hasattr(q, "features") else q.shape[-1]
+            if ht is not None and (ht.shape[-2] != feats or Vp != V):
+                ht = ht[..., :feats, :V]
+            return (o if Vp == V else o[..., :V]), ht
     # otherwise (fp32, several key blocks, other head dimensions) the column is appended here: chunk_simple_gla cuts
     # the V + 1 columns into the blocks the kernels take; the carried state has no normaliser column (the sum starts
     # inside the call).

@@ -95,12 +95,12 @@ def _normalised_closed_form(q, k, v, h0, do, dht, sc, lens=None, eps=1e-10):
 
 @pytest.mark.parametrize("head_first", [True, False])
 @pytest.mark.parametrize("shape", [(2, 3, 333, 64, 64), (2, 2, 200, 128, 128), (1, 3, 130, 64, 128), (1, 2, 70, 128, 64),
-                                   (4, 32, 130, 128, 128), (8, 32, 65, 64, 64)])
+                                   (4, 32, 130, 128, 128), (8, 32, 65, 64, 64), (1, 2, 100, 96, 80), (1, 2, 66, 32, 16)])
 def test_linear_attn_normalised_inside_the_kernels(cuda, shape, head_first):
     """bfloat16 with one key block: the kernels carry the sum of the keys beside the state and divide before they
     store; the backward folds the gradient of the divisor into its own sums.  Against the closed form in fp64 on the
-    same bf16 inputs, output, final state and every gradient (the last two shapes run the 64-column slices of the
-    state passes, the others the 32-column ones)."""
+    same bf16 inputs, output, final state and every gradient (shapes five and six run the 64-column slices of the
+    state passes, the others the 32-column ones; the last two have head dimensions the host pads)."""
     from linear_moe_amd import chunk_linear_attn
     B, H, T, K, V = shape
     bf = torch.bfloat16
