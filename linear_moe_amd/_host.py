@@ -162,6 +162,7 @@ class SeqPlan:
         self.seq_chunk0 = None
         self.seq_order = None
         self.nt_dev = None
+        self.host_offsets = None
         if cu_seqlens is None:
             self.N = B
             self.NT = B * ((T + CHUNK - 1) // CHUNK)
@@ -172,6 +173,7 @@ class SeqPlan:
             self._build_on_device(T, cu_seqlens)
             return
         cu_host = cu_seqlens.detach().to("cpu", torch.int64)
+        self.host_offsets = cu_host.clone()      # what the tables were built from (compared on a cache hit)
         lens = cu_host[1:] - cu_host[:-1]
         if int(cu_host[0]) != 0 or int(cu_host[-1]) != T or bool((lens < 0).any()):
             raise ValueError("cu_seqlens must start at 0, be non-decreasing and end at T")
@@ -229,6 +231,10 @@ def seq_plan(B: int, T: int, cu_seqlens: Optional[torch.Tensor], device) -> SeqP
         return SeqPlan(B, T, cu_seqlens, device)
     for i, (cu, version, t, dev, plan) in enumerate(_PLAN_CACHE):
         if cu is cu_seqlens and version == cu_seqlens._version and t == T and dev == device:
+            # offsets on the host cost nothing to compare: a write the version counter did not see is caught here
+            if not cu_seqlens.is_cuda and not torch.equal(plan.host_offsets, cu_seqlens.detach().to(torch.int64)):
+                del _PLAN_CACHE[i]
+                break
             if i:
                 _PLAN_CACHE.insert(0, _PLAN_CACHE.pop(i))
             return plan

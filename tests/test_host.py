@@ -259,6 +259,12 @@ def test_seq_plan_is_built_once_per_cu_seqlens_tensor():
     assert _host.prepare_cu_seqlens(other, 200, "cpu").NT == 1 + 1 + 3
     with pytest.raises(ValueError):
         _host.seq_plan(1, 201, other, "cpu")                       # another T: validated afresh
+    # a write that the version counter does not see: offsets on the host are compared on a hit, the stale entry goes
+    p4 = _host.seq_plan(1, 200, other, "cpu")
+    other.data[1] = 3
+    p5 = _host.seq_plan(1, 200, other, "cpu")
+    assert p5 is not p4 and p5.cu.tolist() == [0, 3, 65, 200]
+    assert _host.seq_plan(1, 200, other, "cpu") is p5
 
 
 def test_python_layer_validates_before_launch():
