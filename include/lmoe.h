@@ -114,7 +114,11 @@ typedef struct lmoe_args {
    * fwd writes den (the divisor den_t + norm_eps, fp32, laid out like g) and, when hs is given, zs (fp32 [NT,H,K]:
    * the sum of the keys before each chunk).  bwd reads them and o (the normalised output the forward wrote) beside
    * d_o (the gradient of that output), and uses norm_ws, fp32 [NT,H,V/32,64+K], as workspace.  (These three
-   * buffers are not part of what lmoe_workspace_bytes counts, which has no argument for the flag.) */
+   * buffers are not part of what lmoe_workspace_bytes counts, which has no argument for the flag.)
+   * normalize = 2: for a caller that adds the den of several key blocks before it divides (the op is a sum over key
+   * blocks).  fwd writes o undivided and den (norm_eps is added as given: pass 0) beside it, and zs; bwd takes d_o,
+   * the gradient of that o, and dden (fp32, laid out like den), the gradient of den, and uses zs and norm_ws; o and
+   * den are not read. */
   int32_t normalize;
   float norm_eps;
   lmoe_tensor den;
@@ -126,6 +130,7 @@ typedef struct lmoe_args {
    * counterpart in fla's signature: a caller that holds the fused projection saves the pass that would write silu(v)
    * and the one that would apply silu' (see lmoe_gdn_qkv_prologue_*). */
   int32_t v_act;
+  lmoe_tensor dden;    /* normalize = 2, bwd: gradient of den (fp32, laid out like den) */
 } lmoe_args;
 
 /* Library version (major*10000 + minor*100 + patch). */

@@ -41,7 +41,7 @@ class Args(C.Structure):
         ("seq_order", C.c_void_p),
         ("nt_dev", C.c_void_p),
         ("normalize", C.c_int32), ("norm_eps", C.c_float), ("den", Tensor4), ("zs", C.c_void_p),
-        ("norm_ws", C.c_void_p), ("v_act", C.c_int32),
+        ("norm_ws", C.c_void_p), ("v_act", C.c_int32), ("dden", Tensor4),
     ]
 
 

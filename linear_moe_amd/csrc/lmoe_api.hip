@@ -37,11 +37,15 @@ int check_common(const lmoe_args* a, const char* op, bool wide_v = false) {
 // chunk_simple_gla with the output normalised inside the kernels (lmoe_args.normalize)
 int check_normalize(const lmoe_args* a, const char* op, bool bwd) {
   if (!a->normalize) return 0;
+  if (a->normalize != 1 && a->normalize != 2) return fail(-15, "%s: normalize must be 0, 1 or 2", op);
   if (a->dtype != LMOE_BF16) return fail(-15, "%s: normalize needs 2-byte elements", op);
   if (a->gate != LMOE_GATE_NONE) return fail(-15, "%s: normalize needs gate = LMOE_GATE_NONE", op);
-  if (!a->den.ptr) return fail(-11, "%s: normalize needs den", op);
+  if (!bwd && !a->den.ptr) return fail(-11, "%s: normalize needs den", op);
   if (!bwd && a->hs && !a->zs) return fail(-11, "%s: normalize with hs given needs zs", op);
-  if (bwd && (!a->zs || !a->norm_ws || !a->o.ptr)) return fail(-11, "%s: normalize needs o, zs and norm_ws", op);
+  if (bwd && a->normalize == 1 && (!a->den.ptr || !a->zs || !a->norm_ws || !a->o.ptr))
+    return fail(-11, "%s: normalize = 1 needs o, den, zs and norm_ws", op);
+  if (bwd && a->normalize == 2 && (!a->dden.ptr || !a->zs || !a->norm_ws))
+    return fail(-11, "%s: normalize = 2 needs dden, zs and norm_ws", op);
   return 0;
 }
 

@@ -34,8 +34,12 @@ template <typename T, int K, int V> struct StateBwd {
   template <int BVX> static void launch(const lmoe_args& a, hipStream_t st) {
     const dim3 grid(((a.N * a.H + 7) / 8) * 8 * (V / BVX)), block(2 * NTHR);
     if constexpr (sizeof(T) == 2) {        // the pass behind the normalised output exists for 2-byte elements
-      if (a.normalize) {
-        hipLaunchKernelGGL((k_state_bwd<T, K, V, BVX, true>), grid, block, 0, st, a);
+      if (a.normalize == 1) {
+        hipLaunchKernelGGL((k_state_bwd<T, K, V, BVX, 1>), grid, block, 0, st, a);
+        return;
+      }
+      if (a.normalize == 2) {
+        hipLaunchKernelGGL((k_state_bwd<T, K, V, BVX, 2>), grid, block, 0, st, a);
         return;
       }
     }
@@ -47,7 +51,8 @@ template <typename T, int K, int V> struct BwdDqk {
     constexpr int BVH = BwdTiles<T, V>::BVH;
     const int grid = persistent_grid(a.NT * a.H, 1);
     if constexpr (sizeof(T) == 2) {
-      if (a.normalize) hipLaunchKernelGGL((k_bwd_dqkv<T, K, V, BVH, true>), dim3(grid), dim3(2 * NTHR), 0, st, a);
+      if (a.normalize == 1) hipLaunchKernelGGL((k_bwd_dqkv<T, K, V, BVH, 1>), dim3(grid), dim3(2 * NTHR), 0, st, a);
+      else if (a.normalize == 2) hipLaunchKernelGGL((k_bwd_dqkv<T, K, V, BVH, 2>), dim3(grid), dim3(2 * NTHR), 0, st, a);
       else hipLaunchKernelGGL((k_bwd_dqkv<T, K, V, BVH>), dim3(grid), dim3(2 * NTHR), 0, st, a);
     } else {
       hipLaunchKernelGGL((k_bwd_dqk<T, K, V, BVH>), dim3(grid), dim3(2 * NTHR), 0, st, a);

@@ -111,8 +111,11 @@ __global__ __launch_bounds__(NTHR) void k_bwd_dv(const lmoe_args a) {
 // downstream is linear in dden it carries the partial dz that belongs to them; the chunk-parallel kernel adds the
 // partial sums of all slices.  Per chunk, head and 32 columns of V one row of norm_ws: [64] scale dden (partial),
 // [K] dz at the end of the chunk (partial); a slice of 64 columns fills the first of its two rows and zeroes the other.
+// NORM = 2: the forward handed out o undivided and den beside it (a caller that adds the den of several key blocks
+// before it divides): d_o is the gradient of o as it stands and dden comes in as a tensor; it enters once, in the first
+// V slice (the other slices carry zeros).
 constexpr int NORM_SLOT_COLS = 32;
-template <typename T, int K, int V, int BV, bool NORM = false>
+template <typename T, int K, int V, int BV, int NORM = 0>
 __global__ __launch_bounds__(2 * NTHR) void k_state_bwd(const lmoe_args a) {
   constexpr int LDK = K + LPAD, LDU = BV + LPAD;
   constexpr int MB = K / 64, NB = BV / 16;
@@ -173,7 +176,7 @@ __global__ __launch_bounds__(2 * NTHR) void k_state_bwd(const lmoe_args a) {
       IOV::load_nomask(P.rd, row_ptr<T>(a.d_o, sq.b, tok, h) + v0, a.d_o.st, len);
       P.len = len;
       P.graw = load_scalar_raw(gptr, a.g_dtype, gated ? row_off(a.g, sq.b, tok + min(l, len - 1), h) : 0);
-      if constexpr (NORM) {
+      if constexpr (NORM == 1) {
         P.c = c;
         IOV::load_nomask(P.ro, row_ptr<T>(a.o, sq.b, tok, h) + v0, a.o.st, len);
         const float* den = (const float*)a.den.ptr;
@@ -184,9 +187,22 @@ __global__ __launch_bounds__(2 * NTHR) void k_state_bwd(const lmoe_args a) {
         }
         P.dl = den[row_off(a.den, sq.b, tok + min(l, len - 1), h)];
       }
+      if constexpr (NORM == 2) {
+        P.c = c;
+        P.dl = ((const float*)a.dden.ptr)[row_off(a.dden, sq.b, tok + min(l, len - 1), h)];
+      }
     };
     auto stage = [&](Pre& P, int buf) {
-      if constexpr (NORM) {
+      if constexpr (NORM == 2) {
+        if (pw == 0) {                     // scale dden as given, once: in the first V slice
+          float* ws = ws_row(P.c);
+          const float dd = (vsl == 0 && l < P.len) ? scale * P.dl : 0.f;
+          s_dd[buf][l] = dd;
+          ws[l] = dd;
+          if constexpr (SLOTS_PER_SLICE == 2) ws[WS_ROW + l] = 0.f;
+        }
+      }
+      if constexpr (NORM == 1) {
         // partial row dots of d_o and o' over the columns of this slice -> scale dden (partial), for the consumers and
         // for the chunk-parallel kernel; from the registers as loaded (rows past the end of a partial chunk: zero)
         float* ws = ws_row(P.c);
@@ -209,7 +225,7 @@ __global__ __launch_bounds__(2 * NTHR) void k_state_bwd(const lmoe_args a) {
       IOV::mask(P.rd, P.len);
       IOK::store_lds(P.rq, s_q[buf], LDK);
       IOV::store_lds(P.rd, s_do[buf], LDU);
-      if constexpr (NORM) {
+      if constexpr (NORM == 1) {
         if (pw == 0) {                     // ungated: the row factor of the do fragments is scale / D
           s_b[buf][l] = 0.f;
           s_qs[buf][l] = scale / P.dl;
@@ -594,7 +610,8 @@ __global__ __launch_bounds__(2 * NTHR) void k_bwd_dqk(const lmoe_args a) {
 //   dv: P^T formed with its rows i scaled by rD_i;   dP_ij -> scale dP_ij rD_i + dd_i;
 //   dq_i = scale rD_i dq_i,inter + dd_i z + (dP k)_i;   dk_j = dk_d,j + dz + (dP^T q)_j
 // i.e. row and column factors on sums the kernel forms anyway; d_o itself is staged as it is.
-template <typename T, int K, int V, int BVH, bool NORM = false>
+// NORM = 2 (o undivided, den beside it, see k_state_bwd): rD = 1 and dd, dz come from the rows of norm_ws alone.
+template <typename T, int K, int V, int BVH, int NORM = 0>
 __global__ __launch_bounds__(2 * NTHR) void k_bwd_dqkv(const lmoe_args a) {
   static_assert(sizeof(T) == 2, "2-byte elements");
   constexpr int WS_ROW = CH + K, WS_SLOTS = V / NORM_SLOT_COLS;
@@ -656,7 +673,8 @@ __global__ __launch_bounds__(2 * NTHR) void k_bwd_dqkv(const lmoe_args a) {
         const float* ws = a.norm_ws + (int64_t)it * WS_SLOTS * WS_ROW + e_norm;          // it = cid * H + h
 #pragma unroll
         for (int sl = 0; sl < WS_SLOTS; ++sl) Q.ws[sl] = ws[sl * WS_ROW];
-        const float* den = (const float*)a.den.ptr + row_off(a.den, ci.b, ci.tok + min(e_norm, ci.len - 1), h);
+        const lmoe_tensor& dt = NORM == 1 ? a.den : a.dden;               // (NORM = 2: read, not used, for rows)
+        const float* den = (const float*)dt.ptr + row_off(dt, ci.b, ci.tok + min(e_norm, ci.len - 1), h);
         const float* zc = a.zs + (int64_t)it * K + max(e_norm - CH, 0);
         Q.x = *(e_norm < CH ? den : zc);
       }
@@ -683,7 +701,7 @@ __global__ __launch_bounds__(2 * NTHR) void k_bwd_dqkv(const lmoe_args a) {
         const int e = threadIdx.x & (NTHR - 1);
         if (e < CH) {
           s_dd[par][e] = sum;                                // (zero past the end of a partial chunk)
-          s_rD[par][e] = e < Q.len ? 1.f / Q.x : 0.f;
+          s_rD[par][e] = e < Q.len ? (NORM == 1 ? 1.f / Q.x : 1.f) : 0.f;
         } else if (e < WS_ROW) {
           s_dz[par][e - CH] = sum;
           s_z[par][e - CH] = Q.x;

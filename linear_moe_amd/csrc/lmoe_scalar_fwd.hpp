@@ -274,7 +274,8 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd(const lmoe_args a) {
 // ------------------------------------------------------------------------- //
 constexpr int SFWD_TRACE_CHUNKS = 24, SFWD_TRACE_MARKS = 8, SFWD_TRACE_SLOTS = 3;
 
-// NORM (ungated calls): the output leaves divided by den + eps, den_i = scale q_i . (sum of the keys up to i) - the
+// NORM (ungated calls): the output leaves divided by den + eps (lmoe_args.normalize = 1; 2: undivided, with den handed
+// out beside it for a caller that adds the den of several key blocks first), den_i = scale q_i . (sum of the keys up to i) - the
 // op with one more value column of ones, carried beside the state as one more accumulator column (z = the sum of the
 // keys of the chunks before, fp32 in LDS and, for the backward, in zs) and formed by every V slice for itself:
 // consumers z += k^T 1, output team q z and the row sums of P as two more products against a fragment of ones.
@@ -581,7 +582,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_state_fwd_b(const lmoe_args a, lon
         for (int kq = 0; kq < CS; ++kq)
           if (2 * kq <= ow) ET<T>::mma(pz, one8, fp[kq]);
         const float dsum = (oz[0] * ebi + pz[0]) * a.scale + a.norm_eps;
-        rden = 1.f / dsum;
+        rden = a.normalize == 2 ? 1.f : 1.f / dsum;      // 2: den is handed out beside o, the caller divides
         if (vsl == 0 && l < 16 && 16 * ow + fr < len)
           ((float*)a.den.ptr)[row_off(a.den, sq.b, tok + 16 * ow + fr, h)] = dsum;
       }

@@ -12,7 +12,7 @@ from typing import Optional, Tuple
 
 import torch
 
-from .simple_gla import can_normalize, chunk_simple_gla, chunk_simple_gla_normalized
+from .simple_gla import can_normalize, chunk_simple_gla, chunk_simple_gla_normalized, chunk_simple_gla_with_den
 
 
 def chunk_linear_attn(
@@ -42,16 +42,31 @@ def chunk_linear_attn(
     # normalises with q * scale, so the scale cancels in o up to the epsilon): it is formed inside the kernels, in
     # the fp32 state, instead of by a cumulative sum over k in HBM.
     V = v.shape[-1]
-    if normalize and len(qb) == 1 and V <= 128 and v.dim() == 4 and v.dtype == torch.bfloat16:
-        # one key block of bfloat16: the kernels carry the column themselves and divide before they store (a value
-        # head that is not 64 or 128 wide is zero-padded to the next of the two: zero columns stay zero)
+    if normalize and V <= 128 and v.dim() == 4 and v.dtype == torch.bfloat16:
+        # bfloat16: the kernels carry the column themselves (a value head that is not 64 or 128 wide is zero-padded to
+        # the next of the two: zero columns stay zero).  One key block: they also divide before they store.  Several
+        # (the feature maps of Based / ReBased): the divisor is the sum over the blocks, so every block hands out its
+        # den beside its undivided output and the division follows the two sums.
         Vp = 64 if V <= 64 else 128
         pad = torch.nn.functional.pad
         vp = v if Vp == V else pad(v, (0, Vp - V))
         h0 = initial_state if (initial_state is None or Vp == V) else pad(initial_state, (0, Vp - V))
-        if can_normalize(qb[0], vp):
-            o, ht = chunk_simple_gla_normalized(qb[0], kb[0], vp, scale, h0, output_final_state, None, head_first, _eps)
-            feats = q.features if hasattr(q, "features") else q.shape[-1]
+        feats = q.features if hasattr(q, "features") else q.shape[-1]
+        if all(can_normalize(qi, vp) for qi in qb):
+            if len(qb) == 1:
+                o, ht = chunk_simple_gla_normalized(qb[0], kb[0], vp, scale, h0, output_final_state, None, head_first, _eps)
+            else:
+                o, den, hts, k0 = None, None, [], 0
+                for qi, ki in zip(qb, kb):
+                    w = qi.shape[-1]
+                    h0i = None if h0 is None else h0[..., k0:k0 + w, :].contiguous()
+                    oi, di, hi = chunk_simple_gla_with_den(qi, ki, vp, scale, h0i, output_final_state, None, head_first)
+                    o = oi.float() if o is None else o + oi.float()
+                    den = di if den is None else den + di
+                    hts.append(hi)
+                    k0 += w
+                o = (o / (den.unsqueeze(-1) + _eps)).to(v.dtype)
+                ht = torch.cat(hts, dim=-2) if output_final_state else None
             if ht is not None and (ht.shape[-2] != feats or Vp != V):
                 ht = ht[..., :feats, :V]
             return (o if Vp == V else o[..., :V]), ht

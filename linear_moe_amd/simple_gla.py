@@ -29,10 +29,12 @@ class SimpleGLACall:
         self.keep = keep
 
     def forward(self, q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first, save=True,
-                norm_eps=None):
+                norm_eps=None, emit_den=False):
         """save=False: a forward-only call (nothing requires a gradient): the per-chunk states are not written.
         norm_eps: the output leaves the kernels divided by ``scale q_t . sum_{s<=t} k_s + norm_eps`` (ungated calls
-        on 2-byte elements: ``can_normalize``)."""
+        on 2-byte elements: ``can_normalize``).  emit_den (instead of norm_eps): the output stays undivided and
+        ``scale q_t . sum_{s<=t} k_s`` is kept in ``self.den`` for the caller (who adds those of several key blocks
+        before dividing); ``backward`` then takes the gradient of den beside that of o."""
         ctx = self
         lib = _lib.load()
         dims = _check_inputs(q, k, v, head_first, cu_seqlens)
@@ -59,23 +61,28 @@ class SimpleGLACall:
         a.ht = ptr(ht)
         a.hs = ptr(hs)
         den = zs = None
+        if emit_den:
+            norm_eps = 0.0
         if norm_eps is not None:
             if g is not None or q.dtype != torch.bfloat16:
                 raise ValueError("the normalised output exists for ungated calls on bfloat16")
             den = torch.empty((B, H, T) if head_first else (B, T, H), dtype=torch.float32, device=q.device)
             zs = torch.empty(max(plan.NT, 1), H, K, dtype=torch.float32, device=q.device) if save else None
-            a.normalize, a.norm_eps, a.den, a.zs = 1, norm_eps, _desc(den, head_first), ptr(zs)
+            a.normalize, a.norm_eps, a.den, a.zs = (2 if emit_den else 1), norm_eps, _desc(den, head_first), ptr(zs)
         _lib.check(lib.lmoe_chunk_simple_gla_fwd(C.byref(a), stream_ptr()), "chunk_simple_gla forward")
         ctx.saved = (q, k, v, g, h0, hs)
-        ctx.norm = None if norm_eps is None else (norm_eps, den, zs)
+        # (emit_den: den belongs to the caller, the backward does not read it)
+        ctx.norm = None if norm_eps is None else (norm_eps, None if emit_den else den, zs)
+        ctx.emit_den, self.den = emit_den, (den if emit_den else None)
         ctx.fwd_args, ctx.fwd_keep = a, ((o, ht) if self.keep else None)
         ctx.plan, ctx.dims, ctx.head_first, ctx.scale = plan, dims, head_first, scale
         ctx.has_h0 = initial_state is not None
         return o, ht
 
-    def backward(self, do, dht, o=None):
+    def backward(self, do, dht, o=None, dden=None):
         """o: the output of the forward call, for a call with norm_eps (handed in by the caller, who holds it: this
-        object must not, it would close a reference cycle through the autograd graph)."""
+        object must not, it would close a reference cycle through the autograd graph).  dden: the gradient of den,
+        for a call with emit_den (None: zero)."""
         ctx = self
         lib = _lib.load()
         q, k, v, g, h0, hs = ctx.saved
@@ -105,13 +112,18 @@ class SimpleGLACall:
         norm_ws = None
         if ctx.norm is not None:
             norm_eps, den, zs = ctx.norm
-            o = _aligned(o)
             norm_ws = torch.empty(max(plan.NT, 1), H, V // 32, 64 + K, dtype=torch.float32, device=q.device)
-            a.normalize, a.norm_eps, a.den, a.zs = 1, norm_eps, _desc(den, head_first), zs.data_ptr()
-            a.o, a.norm_ws = _desc(o, head_first), norm_ws.data_ptr()
+            a.norm_eps, a.zs, a.norm_ws = norm_eps, zs.data_ptr(), norm_ws.data_ptr()
+            if ctx.emit_den:
+                shape = (B, H, T) if head_first else (B, T, H)
+                dden = torch.zeros(shape, dtype=torch.float32, device=q.device) if dden is None else dden.float().contiguous()
+                a.normalize, a.dden = 2, _desc(dden, head_first)
+            else:
+                o = _aligned(o)
+                a.normalize, a.den, a.o = 1, _desc(den, head_first), _desc(o, head_first)
         _lib.check(lib.lmoe_chunk_simple_gla_bwd(C.byref(a), stream_ptr()), "chunk_simple_gla backward")
         ctx.bwd_args = a
-        ctx.bwd_keep = (do, dht, dq, dk, dv, dg, dh0, dhs, norm_ws, o) if self.keep else None
+        ctx.bwd_keep = (do, dht, dq, dk, dv, dg, dh0, dhs, norm_ws, o, dden) if self.keep else None
         if dg is not None and dg.dtype != g.dtype:
             dg = dg.to(g.dtype)
         return dq, dk, dv, dg, dh0
@@ -133,6 +145,36 @@ class _ChunkSimpleGLA(torch.autograd.Function):
         o = ctx.saved_tensors[0] if ctx.saved_tensors else None
         dq, dk, dv, dg, dh0 = ctx.call.backward(do, dht, o)
         return dq, dk, dv, dg, None, dh0, None, None, None, None
+
+
+class _ChunkSimpleGLAWithDen(torch.autograd.Function):
+    """The ungated op with den = scale q_t . sum_{s<=t} k_s as a second output (nothing divided)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, scale, initial_state, output_final_state, cu_seqlens, head_first):
+        call = SimpleGLACall()
+        o, ht = call.forward(q, k, v, None, scale, initial_state, output_final_state, cu_seqlens, head_first,
+                             save=any(ctx.needs_input_grad), emit_den=True)
+        ctx.call = call
+        den, call.den = call.den, None
+        return o, den, ht
+
+    @staticmethod
+    def backward(ctx, do, dden, dht):
+        if do is None:
+            do = torch.zeros(ctx.call.saved[2].shape, dtype=ctx.call.saved[2].dtype, device=ctx.call.saved[2].device)
+        dq, dk, dv, _, dh0 = ctx.call.backward(do, dht, None, dden)
+        return dq, dk, dv, None, dh0, None, None, None
+
+
+def chunk_simple_gla_with_den(q, k, v, scale=None, initial_state=None, output_final_state=False, cu_seqlens=None,
+                              head_first=True):
+    """The ungated op and, beside its (undivided) output, ``den_t = scale q_t . sum_{s<=t} k_s`` (fp32, ``[B,H,T]`` /
+    ``[B,T,H]``): for ``chunk_linear_attn(normalize=True)`` over several key blocks, where the divisor is the sum of
+    the blocks' den.  Differentiable in both outputs.  Returns ``(o, den, final_state)``."""
+    if not can_normalize(q, v):
+        raise ValueError("chunk_simple_gla_with_den: bfloat16 q, k, v with head dimensions of 64 or 128")
+    return _ChunkSimpleGLAWithDen.apply(q, k, v, scale, initial_state, output_final_state, cu_seqlens, head_first)
 
 
 def can_normalize(q, v, g=None) -> bool:

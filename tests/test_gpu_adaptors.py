@@ -147,3 +147,35 @@ def test_normalised_op_on_packed_sequences_and_forward_only(cuda):
     for gd, gr, n in zip(grads, ref_g, ("q", "k", "v", "h0")):
         gd = gd.cpu() if n == "h0" else tf(gd.cpu())
         assert max_abs_rel(gd, gr) < TOL[bf], n
+
+
+@pytest.mark.parametrize("shape", [(2, 2, 200, 128, 128), (8, 32, 70, 64, 64)])
+def test_op_with_den_as_a_second_output(cuda, shape):
+    """chunk_simple_gla_with_den: o undivided and den = scale q . cumsum(k) beside it, each with a gradient of its own
+    (what chunk_linear_attn(normalize=True) over several key blocks is built from), against the closed form in fp64."""
+    from linear_moe_amd.simple_gla import chunk_simple_gla_with_den
+    B, H, T, K, V = shape
+    bf = torch.bfloat16
+    q, k = (gen(3501, B, H, T, K).abs() + 0.1).to(bf), (gen(3502, B, H, T, K).abs() + 0.1).to(bf)
+    v, do = gen(3503, B, H, T, V, dtype=bf), gen(3504, B, H, T, V, dtype=bf)
+    dd = gen(3505, B, H, T)
+    sc = K ** -0.5
+    ins = [x.double().requires_grad_(True) for x in (q, k, v)]
+    A = torch.tril(sc * ins[0] @ ins[1].transpose(-1, -2))
+    ref_o, ref_den = A @ ins[2], A.sum(-1)
+    ref_g = torch.autograd.grad((ref_o * do.double()).sum() + (ref_den * dd.double()).sum(), ins)
+    dev_in = [x.to(cuda).requires_grad_(True) for x in (q, k, v)]
+    o, den, ht = chunk_simple_gla_with_den(*dev_in)
+    grads = torch.autograd.grad((o * do.to(cuda)).sum() + (den * dd.to(cuda)).sum(), dev_in)
+    torch.cuda.synchronize()
+    assert ht is None and den.dtype == torch.float32 and den.shape == (B, H, T)
+    assert max_abs_rel(o.detach().cpu(), ref_o.detach()) < TOL[bf]
+    assert max_abs_rel(den.detach().cpu(), ref_den.detach()) < TOL[bf]
+    for gd, gr, n in zip(grads, ref_g, "qkv"):
+        assert max_abs_rel(gd.cpu(), gr) < TOL[bf], n
+    # den alone (o unused): the gradient of o is zero
+    dev_in = [x.to(cuda).requires_grad_(True) for x in (q, k, v)]
+    _, den, _ = chunk_simple_gla_with_den(*dev_in)
+    gq, gk = torch.autograd.grad((den * dd.to(cuda)).sum(), dev_in[:2])
+    rq, rk = torch.autograd.grad((torch.tril(sc * ins[0] @ ins[1].transpose(-1, -2)).sum(-1) * dd.double()).sum(), ins[:2])
+    assert max_abs_rel(gq.cpu(), rq) < TOL[bf] and max_abs_rel(gk.cpu(), rk) < TOL[bf]

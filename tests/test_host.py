@@ -149,6 +149,13 @@ def test_options_outside_flas_signature_are_validated_before_any_launch():
     assert lib.lmoe_chunk_simple_gla_bwd(C.byref(a), None) == -11 and b"norm_ws" in lib.lmoe_last_error()
     a.norm_ws = fake
     assert lib.lmoe_chunk_simple_gla_bwd(C.byref(a), None) == 0
+    a.normalize = 2                                # den as a second output: the backward wants its gradient
+    assert lib.lmoe_chunk_simple_gla_fwd(C.byref(a), None) == 0
+    assert lib.lmoe_chunk_simple_gla_bwd(C.byref(a), None) == -11 and b"dden" in lib.lmoe_last_error()
+    a.dden = _lib.Tensor4(fake, 0, 1, 1)
+    assert lib.lmoe_chunk_simple_gla_bwd(C.byref(a), None) == 0
+    a.normalize = 3
+    assert lib.lmoe_chunk_simple_gla_fwd(C.byref(a), None) == -15
 
 
 def test_chunk_gla_forward_needs_hs_only_where_an_output_kernel_reads_it():
