@@ -49,16 +49,19 @@ TRAFFIC_SOURCES = ("lmoe_common.hpp", "lmoe_seq.hpp", "lmoe_gdn_wy.hpp", "lmoe_g
 # summed over the kernels of the call; key = configuration number
 OTHER_TRAFFIC = {"1": 2232825, "2": 272914747, "3": 1280815689, "5": 16649364530, "6": 1445168033, "7": 6572069208,
                  "8": 1510779865}
-OTHER_TRAFFIC_SHA16 = "a33db7548f1a8dfd"
+OTHER_TRAFFIC_SHA16 = "d77541745afd733e"
 
 
 def all_sources_sha16():
-    """Digest of every kernel source of the library (what OTHER_TRAFFIC was counted on)."""
+    """Digest of every kernel source of the library (what OTHER_TRAFFIC was counted on; lmoe_api.hip, which holds
+    validation and dispatch but no kernel, is left out)."""
     import glob
     import hashlib
     h = hashlib.sha256()
     d = os.path.join(ROOT, "linear_moe_amd", "csrc")
     for path in sorted(glob.glob(os.path.join(d, "*.hpp")) + glob.glob(os.path.join(d, "*.hip"))):
+        if os.path.basename(path) == "lmoe_api.hip":
+            continue
         with open(path, "rb") as f:
             h.update(f.read())
     return h.hexdigest()[:16]

@@ -58,7 +58,7 @@ int launched(const char* op) {
 
 extern "C" {
 
-int lmoe_version(void) { return 101; }
+int lmoe_version(void) { return 102; }
 const char* lmoe_last_error(void) { return g_err; }
 
 int64_t lmoe_workspace_bytes(int32_t op, int32_t dtype, int32_t part, int32_t B, int32_t T, int32_t H, int32_t K,
