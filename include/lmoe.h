@@ -131,6 +131,14 @@ typedef struct lmoe_args {
    * and the one that would apply silu' (see lmoe_gdn_qkv_prologue_*). */
   int32_t v_act;
   lmoe_tensor dden;    /* normalize = 2, bwd: gradient of den (fp32, laid out like den) */
+  /* gated delta rule, bwd, 2-byte elements: q_raw, k_raw given (both or neither; shaped and typed like q, k, any
+   * strides the kernels take) say that q = l2norm(silu(q_raw)) and k = l2norm(silu(k_raw)) row by row, with qk_eps
+   * inside the root (what gated_deltanet/gated_deltanet.py:101, :105-106 apply in front of the op and
+   * lmoe_gdn_qkv_prologue_fwd forms): dq and dk then leave as the gradients with respect to q_raw and k_raw, so that
+   * a caller who holds the fused projection needs no pass of its own for the backward of the two activations.  No
+   * counterpart in fla's signature. */
+  lmoe_tensor q_raw, k_raw;
+  float qk_eps;
 } lmoe_args;
 
 /* Library version (major*10000 + minor*100 + patch). */

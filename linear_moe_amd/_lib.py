@@ -42,6 +42,7 @@ class Args(C.Structure):
         ("nt_dev", C.c_void_p),
         ("normalize", C.c_int32), ("norm_eps", C.c_float), ("den", Tensor4), ("zs", C.c_void_p),
         ("norm_ws", C.c_void_p), ("v_act", C.c_int32), ("dden", Tensor4),
+        ("q_raw", Tensor4), ("k_raw", Tensor4), ("qk_eps", C.c_float),
     ]
 
 

@@ -180,6 +180,9 @@ int lmoe_chunk_gated_delta_rule_bwd(const lmoe_args* a, void* stream) {
   if (!a->d_o.ptr || !a->dq.ptr || !a->dk.ptr || !a->dv.ptr || !a->dg.ptr || !a->dbeta.ptr)
     return fail(-13, "%s: d_o, dq, dk, dv, dg and dbeta must not be null", op);
   if (a->v_act && a->dtype != LMOE_BF16) return fail(-15, "%s: v_act needs 2-byte elements", op);
+  if ((a->q_raw.ptr != nullptr) != (a->k_raw.ptr != nullptr)) return fail(-11, "%s: q_raw and k_raw go together", op);
+  if (a->q_raw.ptr && (a->dtype != LMOE_BF16 || a->V > 128))
+    return fail(-15, "%s: q_raw, k_raw need 2-byte elements and V <= 128", op);
   if (a->NT == 0 || a->N == 0) return 0;
   lmoe::launch_gdn_state_bwd(*a, (hipStream_t)stream);
   lmoe::launch_gdn_bwd_chunk(*a, (hipStream_t)stream);

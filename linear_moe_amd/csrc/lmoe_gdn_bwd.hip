@@ -13,6 +13,13 @@ template <typename T, int K, int V> struct GdnBwdChunk {
     constexpr int DEPTH = sizeof(T) == 2 ? ((V / BVH + 2) % 3 == 0 ? 3 : 2) : 1;
     static_assert(GdnBwdChunkLds<T, K, BVH, NBUF>::BYTES <= 160 * 1024, "LDS budget of k_gdn_bwd_chunk");
     const int grid = persistent_grid(a.NT * a.H, 1);
+    if constexpr (sizeof(T) == 2 && V <= 128) {      // (the entry point rejects q_raw with V = 256)
+      if (a.q_raw.ptr) {       // dq, dk with respect to the rows behind q = l2norm(silu(.)), k likewise
+        // (two register sets: the raw rows of the item take the room of the third)
+        hipLaunchKernelGGL((k_gdn_bwd_chunk<T, K, V, BVH, NBUF, 2, true>), dim3(grid), dim3(3 * NTHR), 0, st, a);
+        return;
+      }
+    }
     hipLaunchKernelGGL((k_gdn_bwd_chunk<T, K, V, BVH, NBUF, DEPTH>), dim3(grid), dim3(3 * NTHR), 0, st, a);
   }
 };

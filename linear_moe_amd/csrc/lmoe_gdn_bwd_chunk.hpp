@@ -82,8 +82,14 @@ __device__ __forceinline__ void pin(float (&x)[4]) {
   for (int i = 0; i < 4; ++i) pin(x[i]);
 }
 
-template <typename T, int K, int V, int BVH, int NBUF, int DEPTH>
+// QKACT: q and k as given are l2norm(silu(.)) of rows of a projection that the caller holds (lmoe_args.q_raw, k_raw):
+// dq and dk leave as the gradients with respect to those rows - the backward of the L2 norm and of SiLU is applied to
+// the dq, dk tiles on their way from LDS to memory, by the loader threads that store them, from the raw rows, which
+// are requested when stage 2 begins.  (What it costs is those rows: 32 KB more per item through a request path that is
+// full; the arithmetic, spread over the first windows of the next item or not, is a tenth of it.)
+template <typename T, int K, int V, int BVH, int NBUF, int DEPTH, bool QKACT = false>
 __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
+  static_assert(!QKACT || (sizeof(T) == 2 && NBUF == 3), "the activation backward exists for 2-byte elements");
   typedef GdnBwdChunkLds<T, K, BVH, NBUF> L;
   constexpr int LDV = L::LDV, LDC = L::LDC, LDK = L::LDK;
   constexpr int NS = V / BVH;
@@ -267,6 +273,42 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
         dbv[p] = 0.f;
       }
     };
+    // QKACT: the raw rows behind q and k of an item, and the backward of y = l2norm(silu(x)) on a tile of dy:
+    //   s = silu(x), r = (|s|^2 + eps)^-1/2, dx = silu'(x) (dy r - (dy . s) r^3 s)
+    // with the sums of a row over the VPR neighbouring lanes that hold it (the arithmetic, step for step, of the row
+    // kernel that does the same in front of the op: the results agree bit for bit)
+    typename IOK::Regs XQ, XK;
+    auto issue_raw = [&](int it) __attribute__((always_inline)) {
+      if constexpr (QKACT) {
+        const int cid = it / a.H, h = it % a.H;
+        const ChunkInfo ci = chunk_info(a, cid);
+        IOK::load_nomask(XQ, row_ptr<T>(a.q_raw, ci.b, ci.tok, h), a.q_raw.st, ci.len, tid);
+        IOK::load_nomask(XK, row_ptr<T>(a.k_raw, ci.b, ci.tok, h), a.k_raw.st, ci.len, tid);
+      }
+    };
+    auto act_backward = [&](typename IOK::Regs& r, const typename IOK::Regs& X) __attribute__((always_inline)) {
+      if constexpr (QKACT) {
+#pragma unroll
+        for (int p = 0; p < PK; ++p) {
+          float sv[IOK::VEC], gv[IOK::VEC], fv[IOK::VEC], ss = 0.f, c = 0.f;
+#pragma unroll
+          for (int i = 0; i < IOK::VEC; ++i) {
+            const float x = ET<T>::to_f(X.v[p][i]), sg = sigmoid_fast(x);
+            sv[i] = x * sg;
+            gv[i] = sg * (1.0f + x * (1.0f - sg));
+            ss += sv[i] * sv[i];
+          }
+#pragma unroll
+          for (int i = 0; i < IOK::VEC; ++i) { fv[i] = ET<T>::to_f(r.v[p][i]); c += fv[i] * sv[i]; }
+          ss = group_sum<IOK::VPR>(ss);
+          c = group_sum<IOK::VPR>(c);
+          const float rn = 1.0f / sqrtf(ss + a.qk_eps);
+          c = c * rn * rn * rn;
+#pragma unroll
+          for (int i = 0; i < IOK::VEC; ++i) r.v[p][i] = ET<T>::from_f((fv[i] * rn - c * sv[i]) * gv[i]);
+        }
+      }
+    };
     // (a launch sized by an upper bound of the chunk count may hold work-groups without an item: they stage the last
     // item like every load past the end and skip the loop)
     const int it0 = min((int)blockIdx.x, nitems - 1);
@@ -315,6 +357,7 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
           if constexpr (u < NS) store_dv(d0, ci, h, u);
           if constexpr (w < NS - 1) issue(IC<u + DEPTH>(), it);                          // q, k, slice 0 of the next item
         });
+        issue_raw(it);                                                                   // (QKACT) used behind d
         issue(IC<NS + 1 + DEPTH>(), it);                                                 // slice 1 of the next item
         stage_gates(par ^ 1);                                  // the next item's; its copy is idle since d of the last item
         issue_gates(it + 2 * stride);
@@ -353,8 +396,10 @@ __global__ __launch_bounds__(3 * NTHR) void k_gdn_bwd_chunk(const lmoe_args a) {
       {
         typename IOK::Regs r;
         IOK::load_lds_clamped(r, smem + B_Q, LDK, ci.len, tid);
+        act_backward(r, XQ);
         IOK::template store_global_clamped<true>(r, row_ptr<T>(a.dq, ci.b, ci.tok, h), a.dq.st, ci.len, tid);
         IOK::load_lds_clamped(r, smem + B_K, LDK, ci.len, tid);
+        act_backward(r, XK);
         IOK::template store_global_clamped<true>(r, row_ptr<T>(a.dk, ci.b, ci.tok, h), a.dk.st, ci.len, tid);
       }
       if constexpr (NBUF == 1) {

@@ -94,9 +94,11 @@ class GDNCall:
         ctx.has_h0 = initial_state is not None
         return o, ht
 
-    def backward(self, do, dht, dv_out=None):
-        """dv_out: where dv goes (a tensor of v's shape, any strides the kernels take: e.g. the v block of the gradient
-        of a fused projection); default: a new tensor like v."""
+    def backward(self, do, dht, dv_out=None, dq_out=None, dk_out=None, qk_raw=None, qk_eps=1e-6):
+        """dv_out, dq_out, dk_out: where the gradients go (tensors of the shapes of v, q, k, any strides the kernels
+        take: e.g. the blocks of the gradient of a fused projection); default: new tensors.  qk_raw = (q_raw, k_raw)
+        (bfloat16): q and k of the forward were l2norm(silu(.)) of these rows (eps qk_eps inside the root), and dq,
+        dk are returned with respect to them."""
         ctx = self
         lib = _lib.load()
         q, k, v, g, beta, h0, hs, tinv, pmat, gcum, vnew = ctx.saved
@@ -115,12 +117,23 @@ class GDNCall:
         dht = None if dht is None else dht.float().contiguous()
         a.dht = ptr(dht)
         dev, dt = q.device, q.dtype
-        dq, dk = torch.empty_like(q), torch.empty_like(k)
+        dq = torch.empty_like(q) if dq_out is None else dq_out
+        dk = torch.empty_like(k) if dk_out is None else dk_out
         dv = torch.empty_like(v) if dv_out is None else dv_out
-        if dv.shape != v.shape or dv.dtype != dt or _aligned(dv) is not dv:
-            raise ValueError("dv_out must have the shape and dtype of v, 16-byte aligned rows, a contiguous last dimension")
+        for n, t, like in (("dq_out", dq, q), ("dk_out", dk, k), ("dv_out", dv, v)):
+            if t.shape != like.shape or t.dtype != dt or _aligned(t) is not t:
+                raise ValueError(f"{n} must have the shape and dtype of its input, 16-byte aligned rows, a contiguous "
+                                 "last dimension")
         a.dq, a.dk, a.dv = _desc(dq, head_first), _desc(dk, head_first), _desc(dv, head_first)
         a.v_act = int(ctx.v_act)
+        if qk_raw is not None:
+            q_raw, k_raw = qk_raw
+            if dt != torch.bfloat16:
+                raise ValueError("qk_raw exists for bfloat16")
+            for t, like in ((q_raw, q), (k_raw, k)):
+                if t.shape != like.shape or t.dtype != dt or _aligned(t) is not t:
+                    raise ValueError("qk_raw: the shapes and dtype of q, k, 16-byte aligned rows, a contiguous last dimension")
+            a.q_raw, a.k_raw, a.qk_eps = _desc(q_raw, head_first), _desc(k_raw, head_first), float(qk_eps)
         dg = torch.empty(beta.shape, dtype=torch.float32, device=dev)
         dbeta = torch.empty(beta.shape, dtype=torch.float32, device=dev)
         a.dg, a.dbeta = _desc(dg, head_first), _desc(dbeta, head_first)
@@ -132,7 +145,7 @@ class GDNCall:
         a.dvnew.ptr = dvnew.data_ptr()
         _lib.check(lib.lmoe_chunk_gated_delta_rule_bwd(C.byref(a), stream_ptr()), "chunk_gated_delta_rule backward")
         ctx.bwd_args = a
-        ctx.bwd_keep = (do, dht, dq, dk, dv, dg, dbeta, dh0, dhs, dvnew) if self.keep else None
+        ctx.bwd_keep = (do, dht, dq, dk, dv, dg, dbeta, dh0, dhs, dvnew, qk_raw) if self.keep else None
         dg = None if g is None else dg.to(g.dtype)
         return dq, dk, dv, dg, dbeta.to(beta.dtype), dh0
 

@@ -88,13 +88,16 @@ class _GDNMixerCore(torch.autograd.Function):
     @staticmethod
     def backward(ctx, do):
         T, B, H, D = ctx.dims
-        lib = _lib.load()
         (x,) = ctx.saved_tensors
+        # the op writes all three blocks of the projection's gradient itself: dv as silu'(v) times its dv, dq and dk
+        # through the backward of the L2 norm and of SiLU, applied to its dq, dk tiles on their way out, from the raw
+        # rows of the projection
         dx = torch.empty_like(x)
-        dv = dx.view(T, B, H, 3 * D)[..., 2 * D:].transpose(0, 1)          # the op writes the v block itself
-        dq, dk, _, dg, dbeta, _ = ctx.call.backward(do, None, dv_out=dv)
-        _lib.check(lib.lmoe_gdn_qkv_prologue_bwd(x.data_ptr(), dq.data_ptr(), dk.data_ptr(), None, dx.data_ptr(),
-                                                 T, B, H, D, ctx.dt, ctx.eps, stream_ptr()), "gdn_mixer_core backward")
+        blocks = lambda t: [t.view(T, B, H, 3 * D)[..., i * D:(i + 1) * D].transpose(0, 1) for i in range(3)]
+        dxq, dxk, dxv = blocks(dx)
+        xq, xk, _ = blocks(x)
+        _, _, _, dg, dbeta, _ = ctx.call.backward(do, None, dv_out=dxv, dq_out=dxq, dk_out=dxk, qk_raw=(xq, xk),
+                                                  qk_eps=ctx.eps)
         return dx.view(ctx.shape), dg, dbeta, None, None, None, None
 
 
@@ -102,8 +105,9 @@ def gdn_mixer_core(qkv: torch.Tensor, g: torch.Tensor, beta: torch.Tensor, num_h
                    eps: float = 1e-6, scale=None) -> torch.Tensor:
     """``gdn_qkv_prologue`` and ``chunk_gated_delta_rule(..., head_first=False)`` in one call (bfloat16): q^ and k^ are
     written as by the prologue, v is never written -- the op reads the v block of ``qkv`` in place and applies SiLU
-    where it stages it, and in the backward writes ``silu'(v)`` times its dv straight into the v block of the
-    projection's gradient, whose q and k blocks the prologue's backward fills.  ``g``, ``beta``: ``[B, T, H]``.
+    where it stages it.  The backward is the op's alone: it writes ``silu'(v)`` times its dv straight into the v block
+    of the projection's gradient and sends its dq, dk through the backward of the L2 norm and of SiLU on their way
+    into the q and k blocks (no pass of the prologue's own).  ``g``, ``beta``: ``[B, T, H]``.
     Returns o ``[B, T, H, D]``, the bits of the two-call path."""
     return _GDNMixerCore.apply(qkv, g, beta, num_heads, head_dim, eps, scale)
 

@@ -129,6 +129,22 @@ def test_options_outside_flas_signature_are_validated_before_any_launch():
     assert lib.lmoe_chunk_gated_delta_rule_fwd(C.byref(a), None) == 0
     a.dtype = a.beta_dtype = _lib.LMOE_F32
     assert lib.lmoe_chunk_gated_delta_rule_fwd(C.byref(a), None) == -15 and b"v_act" in lib.lmoe_last_error()
+    # q_raw / k_raw (backward): both or neither, 2-byte elements, V <= 128
+    def bwd_args(dtype, V=128):
+        b = args(dtype, V=V)
+        b.hs = b.dhs = fake
+        b.vnew.ptr = b.dvnew.ptr = fake
+        b.d_o = b.dq = b.dk = b.dv = b.dg = b.dbeta = _lib.Tensor4(fake, 0, 64, 64)
+        return b
+    b = bwd_args(_lib.LMOE_BF16)
+    assert lib.lmoe_chunk_gated_delta_rule_bwd(C.byref(b), None) == 0
+    b.q_raw = _lib.Tensor4(fake, 0, 64, 64)
+    assert lib.lmoe_chunk_gated_delta_rule_bwd(C.byref(b), None) == -11 and b"go together" in lib.lmoe_last_error()
+    b.k_raw = _lib.Tensor4(fake, 0, 64, 64)
+    assert lib.lmoe_chunk_gated_delta_rule_bwd(C.byref(b), None) == 0
+    for bad in (bwd_args(_lib.LMOE_F32), bwd_args(_lib.LMOE_BF16, V=256)):
+        bad.q_raw = bad.k_raw = _lib.Tensor4(fake, 0, 64, 64)
+        assert lib.lmoe_chunk_gated_delta_rule_bwd(C.byref(bad), None) == -15
     # normalize
     a = args(_lib.LMOE_BF16)
     a.gate, a.normalize, a.norm_eps = _lib.GATE_NONE, 1, 1e-10
