@@ -38,18 +38,18 @@ STAGE_NAMES = {0: "k_gdn_wy_fwd", 1: "k_gdn_state_fwd_reg", 4: "k_gdn_state_bwd"
 # sources (kernel_sources_sha16()) at that time, and a build whose sources differ reports traffic = null
 # rather than a stale number.
 CALIB_COPY_BYTES = 256 << 20
-MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237242262, "k_gdn_state_fwd_reg": 1119492165, "k_gdn_state_bwd": 945960857,
-                    "k_gdn_bwd_chunk": 1826536716}
-TRAFFIC_SOURCES_SHA16 = "ccaf947085530fdb"
+MEASURED_TRAFFIC = {"k_gdn_wy_fwd": 237242548, "k_gdn_state_fwd_reg": 1120530337, "k_gdn_state_bwd": 945957881,
+                    "k_gdn_bwd_chunk": 1825838726}
+TRAFFIC_SOURCES_SHA16 = "741aeabd45d2fd45"
 TRAFFIC_SOURCES = ("lmoe_common.hpp", "lmoe_seq.hpp", "lmoe_gdn_wy.hpp", "lmoe_gdn_state.hpp", "lmoe_gdn_state_reg.hpp", "lmoe_gdn_bwd_chunk.hpp",
                    "lmoe_gdn_fwd.hip", "lmoe_gdn_state.hip", "lmoe_gdn_bwd.hip")
 
 
 # HBM bytes per call of the other contract configurations (bench.py --other-configs), same counters and scaling,
 # summed over the kernels of the call; key = configuration number
-OTHER_TRAFFIC = {"1": 2232825, "2": 272914747, "3": 1280815689, "5": 16649364530, "6": 1445168033, "7": 6572069208,
-                 "8": 1510779865}
-OTHER_TRAFFIC_SHA16 = "d77541745afd733e"
+OTHER_TRAFFIC = {"1": 2232824, "2": 272914694, "3": 1279660547, "5": 16651376487, "6": 1444943222, "7": 6580301476,
+                 "8": 1510793999}
+OTHER_TRAFFIC_SHA16 = "9a2741ef41ed699f"
 
 
 def all_sources_sha16():
