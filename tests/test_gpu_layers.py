@@ -36,15 +36,17 @@ def test_layer_matches_the_oracle_chain(cuda, kind, dtype):
     assert y.shape == (T, B, hidden) and y.dtype == dtype
     grads = torch.autograd.grad((y * dy.to(dtype).to(cuda)).sum(), [xd] + list(layer.parameters()))
     torch.cuda.synchronize()
-    # the chain has six roundings to dtype between the projections and the output; the bars are those of the ops
-    tol = 1e-4 if dtype == torch.float32 else 4e-2
+    # the bars of the ops themselves (measured over three seeds: fp32 <= 3.8e-6, bf16 <= 9.7e-3, A_log / dt_bias 1.7e-2)
+    tol = TOL[dtype]
     assert max_abs_rel(y.detach().cpu(), yr.detach()) < tol
     names = ["x"] + list(ref_params)
     for n, gd, gr in zip(names, grads, ref_grads):
         # A_log, dt_bias: H numbers, each the sum of B*T signed per-token terms that cancel to a fraction of their
-        # absolute sum; in bf16 the rounding of every term (dg comes through bf16 q, k, v) does not cancel with it
-        t = 2 * tol if (dtype == torch.bfloat16 and n in ("A_log", "dt_bias")) else tol
-        assert max_abs_rel(gd.cpu(), gr) < t, n
+        # absolute sum; the rounding of every term (in bf16: dg comes through bf16 q, k, v) does not cancel with it:
+        # 4e-5 / 4e-2 for these two (measured: fp32 up to 2.2e-5, bf16 1.7e-2); everything else at the bars of the ops
+        t = (4 if dtype == torch.float32 else 2) * tol if n in ("A_log", "dt_bias") else tol
+        err = max_abs_rel(gd.cpu(), gr)
+        assert err < t, (n, err)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -157,8 +159,12 @@ def test_core_modules_of_the_other_dispatch_branches(cuda, kind, dtype):
     assert y.shape == (T, B, H * D) and y.dtype == dtype
     gd = torch.autograd.grad((y * dy.to(cuda)).sum(), ld + [core.norm_weight])
     torch.cuda.synchronize()
-    # three chained roundings (feature map, op, norm); the normalised basic module divides two rounded sums
-    tol = 5e-5 if dtype == torch.float32 else 4e-2
-    assert max_abs_rel(y.detach().cpu(), yr.detach()) < tol
+    # the bars of the ops; lightning attention in bf16: twice that (its slopes reach e^-8 per token on the last heads,
+    # the outputs of those heads are sums of a few tokens, and the rounding of q and k to bf16 is 3.6e-2 of dq, dk)
+    tol = 2 * TOL[dtype] if (kind.startswith("lightning") and dtype == torch.bfloat16) else TOL[dtype]
+    errs = {"y": max_abs_rel(y.detach().cpu(), yr.detach())}
     for n, a, b in zip(("dq", "dk", "dv", "dw"), gd, gr):
-        assert max_abs_rel(a.cpu(), b) < tol, n
+        errs[n] = max_abs_rel(a.cpu(), b)
+    print(kind, dtype, {n: f"{e:.1e}" for n, e in errs.items()})
+    for n, e in errs.items():
+        assert e < tol, (n, e)
