@@ -105,8 +105,10 @@ def test_based_path_matches_oracle(cuda, kind):
     (o * do.to(cuda)).sum().backward()
     torch.cuda.synchronize()
     assert ht.shape == (B, H, fm_ref(qr).shape[-1], V)
-    # the normaliser q . cumsum(k) is formed in bf16 by torch, as fla does; its rounding dominates the error
-    tol = 3 * TOL[dt]
+    # Taylor features: the bar of the op (the divisor is summed in fp32 inside the kernels; measured <= 7.4e-3 over three
+    # seeds).  ReBased: the weights (q . k)^2 leave the first tokens a divisor that can be tiny, which amplifies the
+    # rounding of q, k to bf16 whatever the kernel does (1.3e-2 on these inputs, more on others): three times the bar
+    tol = TOL[dt] if kind == "taylor" else 3 * TOL[dt]
     assert max_abs_rel(o.detach().cpu(), ref.detach()) < tol
     for a, b in ((qd, qr), (kd, kr), (vd, vr)):
         assert max_abs_rel(a.grad.cpu(), b.grad) < tol
