@@ -69,15 +69,14 @@ def test_gdn_layer_fused_prologue_epilogue_equals_the_unfused_chain(cuda, dtype)
     assert max_abs_rel(outs[0][1].cpu(), outs[1][1].cpu()) < tol
 
 
-@pytest.mark.parametrize("D", [128, 64])
-def test_gdn_mixer_core_equals_prologue_then_op(cuda, D):
+@pytest.mark.parametrize("D,T,B,H", [(128, 200, 2, 3), (64, 200, 2, 3), (128, 1, 1, 1), (64, 65, 3, 2), (128, 64, 1, 2)])
+def test_gdn_mixer_core_equals_prologue_then_op(cuda, D, T, B, H):
     """gdn_mixer_core (q^, k^ written, silu(v) applied where the op stages v, dv written straight into the v block of
     the projection's gradient) against gdn_qkv_prologue followed by chunk_gated_delta_rule: the same output bit for
     bit (the same q^, k^ and the same rounded silu(v) reach the same kernels), the same dg, dbeta and q / k blocks of
     the projection's gradient bit for bit, its v block to the rounding of the element type (one rounding of
     beta dZ silu'(v) instead of two)."""
     import linear_moe_amd as L
-    T, B, H = 200, 2, 3
     bf = torch.bfloat16
     qkv = gen(5250, T, B, H * 3 * D).to(bf).to(cuda)
     g = (-torch.rand(B, T, H, generator=torch.Generator().manual_seed(5251)) * 0.2).to(cuda)
