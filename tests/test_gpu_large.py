@@ -81,3 +81,66 @@ def test_row_kernels_beyond_32_bits(cuda):
         assert torch.equal(gb[-tail:], gs), name
         del xb, yb, dyb, gb
         torch.cuda.empty_cache()
+
+
+def test_gated_norm_and_layer_relayouts_beyond_32_bits(cuda):
+    """The gated output norm and the two kernels that change the layout (the prologue [T, B, H 3D] -> q^, k^, silu(v) as
+    [B, T, H, D]; the epilogue [B, T, H, D] x gate -> [T, B, H D]) on tensors beyond 2^31 elements: the first and the
+    last rows / tokens give inside the large call the bits they give as a call of their own, forward and backward; the
+    weight gradient of the norm, a sum over all rows, against the same sum formed with torch in pieces."""
+    import linear_moe_amd as L
+    if torch.cuda.get_device_properties(0).total_memory < 150 * 2**30:
+        pytest.skip("needs about 60 GB of GPU memory")
+    bf = torch.bfloat16
+    D, R, n = 128, 2**24 + 1024, 512
+    assert R * D > 2**31
+    g_ = torch.Generator(device=cuda).manual_seed(7)
+    rnd = lambda *s: torch.randn(*s, generator=g_, device=cuda, dtype=bf)
+
+    def fwd_bwd(f, args, dy):
+        leaves = [t.detach().clone().requires_grad_(True) for t in args]
+        y = f(*leaves)
+        return (y.detach(),) + torch.autograd.grad(y, leaves, dy)
+
+    x, gate, dy = rnd(R, D), rnd(R, D), rnd(R, D)
+    w = (1 + 0.1 * torch.randn(D, generator=g_, device=cuda)).to(bf)
+    whole = fwd_bwd(lambda a, b: L.rms_norm_swish_gate(a, b, w), (x, gate), dy)
+    for sl in (slice(0, n), slice(R - n, R)):
+        part = fwd_bwd(lambda a, b: L.rms_norm_swish_gate(a, b, w), (x[sl], gate[sl]), dy[sl])
+        torch.cuda.synchronize()
+        for a, b in zip(whole, part):
+            assert torch.equal(a[sl], b), sl
+    del whole
+    wl = w.clone().requires_grad_(True)
+    (dw,) = torch.autograd.grad(L.rms_norm_swish_gate(x, gate, wl), [wl], dy)
+    ref = torch.zeros(D, device=cuda, dtype=torch.float64)
+    for r0 in range(0, R, 2**20):
+        xs, gs, ds = (t[r0:r0 + 2**20].float() for t in (x, gate, dy))
+        ref += (ds * gs * torch.sigmoid(gs) * xs * torch.rsqrt(xs.pow(2).mean(-1, keepdim=True) + 1e-5)).sum(0).double()
+    err = float((dw.double() - ref).abs().max() / ref.abs().max())
+    assert err < 2e-2, err                               # (dw is handed out in bfloat16)
+    del x, gate, dy
+    torch.cuda.empty_cache()
+
+    T, B, H = 2**20 + 64, 3, 2                           # qkv: 2.4e9 elements; the last batch entry ends every tensor
+    assert T * B * H * 3 * D > 2**31
+    pro = lambda t: torch.cat(L.gdn_qkv_prologue(t, H, D), -1)
+    qkv, dqkv = rnd(T, B, H * 3 * D), rnd(B, T, H, 3 * D)
+    whole = fwd_bwd(pro, (qkv,), dqkv)
+    for sl in (slice(0, 64), slice(T - 64, T)):
+        part = fwd_bwd(pro, (qkv[sl],), dqkv[:, sl])
+        torch.cuda.synchronize()
+        assert torch.equal(whole[0][:, sl], part[0]) and torch.equal(whole[1][sl], part[1]), sl
+    del whole, qkv, dqkv
+    torch.cuda.empty_cache()
+
+    T = 2**22 + 64                                       # [B, T, H D]: 3.2e9 elements
+    o, og, dy = rnd(B, T, H, D), rnd(T, B, H * D), rnd(T, B, H * D)
+    whole = fwd_bwd(L.swish_gate_relayout, (o, og), dy)
+    for sl in (slice(0, 64), slice(T - 64, T)):
+        part = fwd_bwd(L.swish_gate_relayout, (o[:, sl], og[sl]), dy[sl])
+        torch.cuda.synchronize()
+        assert torch.equal(whole[0][sl], part[0]) and torch.equal(whole[1][:, sl], part[1]), sl
+        assert torch.equal(whole[2][sl], part[2]), sl
+    del whole, o, og, dy
+    torch.cuda.empty_cache()
