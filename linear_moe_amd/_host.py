@@ -292,6 +292,23 @@ def token_major(B: int, T: int, H: int, D: int, dtype, device) -> torch.Tensor:
     return torch.empty(B, T, H, D, dtype=dtype, device=device)
 
 
+def stash(ctx, call, *extra) -> None:
+    """Hands the tensors ``call`` keeps for its backward (``call.saved``) and ``extra`` over to autograd
+    (``ctx.save_for_backward``).  Autograd then frees them as soon as the node's backward has run -- the per-chunk
+    states of a layer go while the backward sweep passes the layer, not when the whole graph dies --, notices an
+    input that was modified in place between forward and backward, and saved-tensor hooks see them."""
+    ctx.n_stashed = len(call.saved)
+    ctx.save_for_backward(*call.saved, *extra)
+    call.saved = None
+
+
+def unstash(ctx, call):
+    """Gives ``call`` its tensors back for one backward; returns the ``extra`` of ``stash``."""
+    t = ctx.saved_tensors
+    call.saved = tuple(t[:ctx.n_stashed])
+    return t[ctx.n_stashed:]
+
+
 def stream_ptr() -> C.c_void_p:
     return C.c_void_p(torch.cuda.current_stream().cuda_stream)
 

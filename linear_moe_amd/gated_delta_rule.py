@@ -17,7 +17,7 @@ import torch
 from . import _lib
 from .l2norm import l2_norm
 from ._host import (HEAD_DIMS, WIDE_V, seq_plan, _aligned, _check_inputs, _desc, _state_check, base_args, by_head_dim_blocks,
-                    no_tokens, ptr, stream_ptr)
+                    no_tokens, ptr, stash, stream_ptr, unstash)
 
 
 def _scalar_dt(x: torch.Tensor) -> int:
@@ -157,11 +157,16 @@ class _ChunkGatedDeltaRule(torch.autograd.Function):
         o, ht = call.forward(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, head_first,
                              save=any(ctx.needs_input_grad))
         ctx.call = call
+        stash(ctx, call)
         return o, ht
 
     @staticmethod
     def backward(ctx, do, dht):
-        dq, dk, dv, dg, dbeta, dh0 = ctx.call.backward(do, dht)
+        unstash(ctx, ctx.call)
+        try:
+            dq, dk, dv, dg, dbeta, dh0 = ctx.call.backward(do, dht)
+        finally:
+            ctx.call.saved = None
         return dq, dk, dv, dg, dbeta, None, dh0, None, None, None
 
 

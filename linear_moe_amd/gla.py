@@ -14,7 +14,7 @@ import torch
 
 from . import _lib
 from ._host import (HEAD_DIMS, seq_plan, _aligned, _check_inputs, _desc, _state_check, base_args, by_head_dim_blocks,
-                    no_tokens, ptr, stream_ptr)
+                    no_tokens, ptr, stash, stream_ptr, unstash)
 
 
 class GLACall:
@@ -100,11 +100,16 @@ class _ChunkGLA(torch.autograd.Function):
         o, ht = call.forward(q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first,
                              save=any(ctx.needs_input_grad))
         ctx.call, ctx.g_dtype = call, g.dtype
+        stash(ctx, call)
         return o, ht
 
     @staticmethod
     def backward(ctx, do, dht):
-        dq, dk, dv, dg, dh0 = ctx.call.backward(do, dht)
+        unstash(ctx, ctx.call)
+        try:
+            dq, dk, dv, dg, dh0 = ctx.call.backward(do, dht)
+        finally:
+            ctx.call.saved = None
         return dq, dk, dv, dg.to(ctx.g_dtype), None, dh0, None, None, None
 
 

@@ -12,7 +12,7 @@ from __future__ import annotations
 import torch
 
 from . import _lib
-from ._host import stream_ptr
+from ._host import stash, stream_ptr, unstash
 
 
 def _dt(x):
@@ -81,14 +81,14 @@ class _GDNMixerCore(torch.autograd.Function):
         o, _ = call.forward(q, k, v, g, beta, scale, None, False, None, False,
                             save=any(ctx.needs_input_grad[:3]), v_act=True)
         ctx.call = call
-        ctx.save_for_backward(x)
+        stash(ctx, call, x)
         ctx.dims, ctx.eps, ctx.dt, ctx.shape = (T, B, H, D), eps, dt, qkv.shape
         return o
 
     @staticmethod
     def backward(ctx, do):
         T, B, H, D = ctx.dims
-        (x,) = ctx.saved_tensors
+        (x,) = unstash(ctx, ctx.call)
         # the op writes all three blocks of the projection's gradient itself: dv as silu'(v) times its dv, dq and dk
         # through the backward of the L2 norm and of SiLU, applied to its dq, dk tiles on their way out, from the raw
         # rows of the projection
@@ -96,8 +96,11 @@ class _GDNMixerCore(torch.autograd.Function):
         blocks = lambda t: [t.view(T, B, H, 3 * D)[..., i * D:(i + 1) * D].transpose(0, 1) for i in range(3)]
         dxq, dxk, dxv = blocks(dx)
         xq, xk, _ = blocks(x)
-        _, _, _, dg, dbeta, _ = ctx.call.backward(do, None, dv_out=dxv, dq_out=dxq, dk_out=dxk, qk_raw=(xq, xk),
-                                                  qk_eps=ctx.eps)
+        try:
+            _, _, _, dg, dbeta, _ = ctx.call.backward(do, None, dv_out=dxv, dq_out=dxq, dk_out=dxk, qk_raw=(xq, xk),
+                                                      qk_eps=ctx.eps)
+        finally:
+            ctx.call.saved = None
         return dx.view(ctx.shape), dg, dbeta, None, None, None, None
 
 

@@ -14,7 +14,7 @@ import torch
 
 from . import _lib
 from ._host import (HEAD_DIMS, seq_plan, _aligned, _check_inputs, _desc, _state_check, base_args, by_head_dim_blocks,
-                    no_tokens, ptr, stream_ptr)
+                    no_tokens, ptr, stash, stream_ptr, unstash)
 
 
 class SimpleGLACall:
@@ -70,9 +70,9 @@ class SimpleGLACall:
             zs = torch.empty(max(plan.NT, 1), H, K, dtype=torch.float32, device=q.device) if save else None
             a.normalize, a.norm_eps, a.den, a.zs = (2 if emit_den else 1), norm_eps, _desc(den, head_first), ptr(zs)
         _lib.check(lib.lmoe_chunk_simple_gla_fwd(C.byref(a), stream_ptr()), "chunk_simple_gla forward")
-        ctx.saved = (q, k, v, g, h0, hs)
         # (emit_den: den belongs to the caller, the backward does not read it)
-        ctx.norm = None if norm_eps is None else (norm_eps, None if emit_den else den, zs)
+        ctx.saved = (q, k, v, g, h0, hs, None if emit_den else den, zs)
+        ctx.norm_eps = norm_eps
         ctx.emit_den, self.den = emit_den, (den if emit_den else None)
         ctx.fwd_args, ctx.fwd_keep = a, ((o, ht) if self.keep else None)
         ctx.plan, ctx.dims, ctx.head_first, ctx.scale = plan, dims, head_first, scale
@@ -85,7 +85,7 @@ class SimpleGLACall:
         for a call with emit_den (None: zero)."""
         ctx = self
         lib = _lib.load()
-        q, k, v, g, h0, hs = ctx.saved
+        q, k, v, g, h0, hs, den, zs = ctx.saved
         plan, dims, head_first = ctx.plan, ctx.dims, ctx.head_first
         B, T, H, K, V = dims
         do = _aligned(do)
@@ -110,8 +110,8 @@ class SimpleGLACall:
         dhs = torch.empty_like(hs)
         a.dhs = dhs.data_ptr()
         norm_ws = None
-        if ctx.norm is not None:
-            norm_eps, den, zs = ctx.norm
+        if ctx.norm_eps is not None:
+            norm_eps = ctx.norm_eps
             norm_ws = torch.empty(max(plan.NT, 1), H, V // 32, 64 + K, dtype=torch.float32, device=q.device)
             a.norm_eps, a.zs, a.norm_ws = norm_eps, zs.data_ptr(), norm_ws.data_ptr()
             if ctx.emit_den:
@@ -136,14 +136,16 @@ class _ChunkSimpleGLA(torch.autograd.Function):
         o, ht = call.forward(q, k, v, g, scale, initial_state, output_final_state, cu_seqlens, head_first,
                              save=any(ctx.needs_input_grad), norm_eps=norm_eps)
         ctx.call = call
-        if norm_eps is not None:
-            ctx.save_for_backward(o)          # the backward of the normalisation reads the output
+        stash(ctx, call, o if norm_eps is not None else None)    # (the backward of the normalisation reads the output)
         return o, ht
 
     @staticmethod
     def backward(ctx, do, dht):
-        o = ctx.saved_tensors[0] if ctx.saved_tensors else None
-        dq, dk, dv, dg, dh0 = ctx.call.backward(do, dht, o)
+        (o,) = unstash(ctx, ctx.call)
+        try:
+            dq, dk, dv, dg, dh0 = ctx.call.backward(do, dht, o)
+        finally:
+            ctx.call.saved = None
         return dq, dk, dv, dg, None, dh0, None, None, None, None
 
 
@@ -157,13 +159,19 @@ class _ChunkSimpleGLAWithDen(torch.autograd.Function):
                              save=any(ctx.needs_input_grad), emit_den=True)
         ctx.call = call
         den, call.den = call.den, None
+        stash(ctx, call)
         return o, den, ht
 
     @staticmethod
     def backward(ctx, do, dden, dht):
-        if do is None:
-            do = torch.zeros(ctx.call.saved[2].shape, dtype=ctx.call.saved[2].dtype, device=ctx.call.saved[2].device)
-        dq, dk, dv, _, dh0 = ctx.call.backward(do, dht, None, dden)
+        unstash(ctx, ctx.call)
+        try:
+            if do is None:
+                v = ctx.call.saved[2]
+                do = torch.zeros(v.shape, dtype=v.dtype, device=v.device)
+            dq, dk, dv, _, dh0 = ctx.call.backward(do, dht, None, dden)
+        finally:
+            ctx.call.saved = None
         return dq, dk, dv, None, dh0, None, None, None
 
 

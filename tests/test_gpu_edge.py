@@ -325,3 +325,45 @@ def test_the_order_in_which_the_passes_take_the_sequences_does_not_show(cuda, op
     torch.cuda.synchronize()
     for a, b in zip(planned, as_given):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("op", OPS)
+def test_saved_tensors_belong_to_autograd(cuda, op):
+    """What a call keeps for its backward (inputs, per-chunk states, the other intermediates) is handed to autograd:
+    it is freed when the node's backward has run, although the output -- and with it the node -- is still alive; an
+    input modified in place between forward and backward is an error, not a wrong gradient; a second backward works
+    with retain_graph and is refused without."""
+    T, H, K, V = 4096, 4, 128, 128
+    ins = {n: x.to(cuda) for n, x in _inputs(op, T, H, K, V, torch.bfloat16, 3700).items()}
+    do = gen(3711, 1, T, H, V, dtype=torch.bfloat16).to(cuda)
+    names = list(ins)
+
+    def forward():
+        leaves = {n: x.clone().requires_grad_(True) for n, x in ins.items()}
+        work = {n: x * 1 for n, x in leaves.items()}                 # (not leaves: they may be written in place)
+        o, _ = _call(op, work, None, None, True)
+        return leaves, work, o
+
+    torch.cuda.synchronize()
+    m0 = torch.cuda.memory_allocated()
+    leaves, work, o = forward()
+    m1 = torch.cuda.memory_allocated()
+    g1 = torch.autograd.grad(o, [leaves[n] for n in names], do, retain_graph=True)
+    g2 = torch.autograd.grad(o, [leaves[n] for n in names], do)
+    for a, b in zip(g1, g2):
+        assert torch.equal(a, b)
+    with pytest.raises(RuntimeError):
+        torch.autograd.grad(o, [leaves[n] for n in names], do)       # freed by the backward before
+    held = sum(x.numel() * x.element_size() for x in list(leaves.values()) + list(g1) + list(g2)) \
+        + o.numel() * o.element_size()
+    del work
+    torch.cuda.synchronize()
+    m2 = torch.cuda.memory_allocated()
+    states = (T // 64) * H * K * V * 2                               # the per-chunk states alone
+    assert m1 - m0 > held - sum(x.numel() * x.element_size() for x in list(g1) + list(g2)) + states
+    assert m2 - m0 <= held + (1 << 20), (m2 - m0, held)
+
+    leaves, work, o = forward()
+    work["k"].add_(1)
+    with pytest.raises(RuntimeError, match="modified by an inplace operation"):
+        torch.autograd.grad(o, [leaves[n] for n in names], do)
