@@ -272,6 +272,10 @@ def _state_check(x: Optional[torch.Tensor], N, H, K, V, name: str) -> Optional[t
 
 def base_args(q, k, v, head_first: bool, scale: Optional[float], plan: SeqPlan, dims) -> Args:
     B, T, H, K, V = dims
+    if not (q.device == k.device == v.device) or q.device.index != torch.cuda.current_device():
+        # (the kernels go to the current stream of the current device: one process per GPU, as the launchers run it)
+        raise RuntimeError(f"q, k, v must live on the current device cuda:{torch.cuda.current_device()}, got "
+                           f"{q.device}, {k.device}, {v.device}")
     a = Args()
     a.dtype = _DT[q.dtype]
     a.B, a.T, a.H, a.K, a.V = B, T, H, K, V
