@@ -53,7 +53,8 @@ typedef struct lmoe_args {
   int32_t gate;       /* LMOE_GATE_*          */
   int32_t B, T, H, K, V;
   int32_t N;          /* number of sequences: B, or len(cu_seqlens)-1 when packed (then B == 1) */
-  int32_t NT;         /* total number of 64-token chunks over all sequences                    */
+  int32_t NT;         /* total number of 64-token chunks over all sequences: B * ceil(T / 64) for dense
+                       * input (checked), at most ceil(T / 64) + N for packed input (checked)     */
   float scale;
   /* packed variable-length input (all NULL for dense input) -- device int32 arrays */
   const int32_t* cu_seqlens; /* [N+1] token offsets                                   */

@@ -1,6 +1,7 @@
 // C ABI of liblmoe_hip.so (declared in include/lmoe.h): argument validation and kernel dispatch.
 #include <hip/hip_runtime.h>
 #include <stdarg.h>
+#include <stdint.h>
 #include <stdio.h>
 #include <string.h>
 
@@ -31,6 +32,20 @@ int check_common(const lmoe_args* a, const char* op, bool wide_v = false) {
   if (!a->cu_seqlens && a->N != a->B) return fail(-6, "%s: dense input needs N == B", op);
   if (!a->q.ptr || !a->k.ptr || !a->v.ptr) return fail(-7, "%s: q, k, v must not be null", op);
   if (a->H > 65535 || a->N > 65535) return fail(-8, "%s: H and N must be <= 65535", op);
+  // The kernels derive every address from these numbers: a chunk count that does not belong to B and T would send
+  // them past the end of the inputs, rows that are not 16-byte aligned break their 16-byte accesses.
+  const int64_t per_row = ((int64_t)a->T + LMOE_CHUNK - 1) / LMOE_CHUNK;
+  if (!a->cu_seqlens && (int64_t)a->NT != (int64_t)a->B * per_row)
+    return fail(-4, "%s: dense input of B=%d, T=%d has %lld chunks, NT=%d given", op, a->B, a->T,
+                (long long)(a->B * per_row), a->NT);
+  if (a->cu_seqlens && (int64_t)a->NT > per_row + a->N)
+    return fail(-4, "%s: packed input of T=%d, N=%d has at most %lld chunks, NT=%d given", op, a->T, a->N,
+                (long long)(per_row + a->N), a->NT);
+  const int64_t vec = a->dtype == LMOE_BF16 ? 8 : 4;            // elements per 16 bytes
+  const lmoe_tensor* rows[] = {&a->q, &a->k, &a->v, &a->o, &a->d_o, &a->dq, &a->dk, &a->dv, &a->q_raw, &a->k_raw};
+  for (const lmoe_tensor* t : rows)
+    if (t->ptr && (((uintptr_t)t->ptr & 15) || t->sb % vec || t->st % vec || t->sh % vec))
+      return fail(-9, "%s: q, k, v, o and their gradients need 16-byte aligned rows (pointer and strides)", op);
   return 0;
 }
 

@@ -99,6 +99,37 @@ def test_gated_delta_rule_needs_w_and_u_only_where_the_state_pass_reads_them():
                     assert b"w and u must not be null" in lib.lmoe_last_error()
 
 
+def test_chunk_count_and_row_alignment_are_checked_before_any_launch():
+    """The kernels derive every address from B, T, NT and the strides: a chunk count that does not belong to B and T
+    (dense) or exceeds the bound ceil(T / 64) + N (packed), and rows that are not 16-byte aligned, are refused."""
+    from linear_moe_amd import _lib
+    lib = _lib.load()
+    fake = 0x1000                                  # never dereferenced: every call below is refused
+
+    def args(**kw):
+        a = _lib.Args()
+        a.dtype, a.B, a.T, a.H, a.K, a.V, a.N, a.NT = _lib.LMOE_BF16, 2, 130, 1, 64, 64, 2, 6
+        a.scale, a.gate = 1.0, _lib.GATE_NONE
+        for n in ("q", "k", "v", "o"):
+            setattr(a, n, _lib.Tensor4(fake, 130 * 64, 64, 64))
+        for n, x in kw.items():
+            setattr(a, n, x)
+        return a
+
+    for nt in (5, 7, 0):
+        assert lib.lmoe_chunk_simple_gla_fwd(C.byref(args(NT=nt)), None) == -4
+        assert b"has 6 chunks" in lib.lmoe_last_error()
+    packed = dict(B=1, T=260, N=3, cu_seqlens=fake, chunk_map=fake, seq_chunk0=fake)
+    assert lib.lmoe_chunk_simple_gla_fwd(C.byref(args(NT=9, **packed)), None) == -4     # at most 5 + 3
+    assert b"at most 8 chunks" in lib.lmoe_last_error()
+    for bad in (_lib.Tensor4(fake + 2, 130 * 64, 64, 64), _lib.Tensor4(fake, 130 * 64, 68, 64),
+                _lib.Tensor4(fake, 130 * 64 + 4, 64, 64), _lib.Tensor4(fake, 130 * 64, 64, 60)):
+        for name in ("q", "k", "v", "o"):
+            assert lib.lmoe_chunk_simple_gla_fwd(C.byref(args(**{name: bad})), None) == -9, name
+    f32 = args(dtype=_lib.LMOE_F32, v=_lib.Tensor4(fake, 130 * 64, 68, 64))            # 4 elements are 16 bytes
+    assert lib.lmoe_chunk_simple_gla_bwd(C.byref(f32), None) == -11                     # (passes on to the next check)
+
+
 def test_options_outside_flas_signature_are_validated_before_any_launch():
     """V = 256 belongs to the gated delta rule alone (2-byte calls then need tinv); normalize belongs to ungated 2-byte
     calls of chunk_simple_gla and names the buffers it needs; v_act needs 2-byte elements and tinv.  Calls without
